@@ -1,0 +1,195 @@
+/*
+ * ojas_hip.h — C ABI of the MI355X (gfx950) backend for Ojas Engine's quantized-matmul path.
+ *
+ * This is the boundary a Rust `ojas-hip` crate binds with `extern "C"`: plain pointers, sizes and
+ * integer status codes; no C++ types, no exceptions, nothing allocated by the caller is retained
+ * after a call returns.  Each entry names the reference interface it stands in for (paths are
+ * relative to the reference tree).
+ *
+ * Two seams are exported, as in the reference:
+ *   1. the kernel seam  — `Device` + `KernelRuntime` (crates/ojas-core/src/lib.rs:26-40,
+ *      crates/ojas-core/src/kernel.rs:67-81; CUDA implementation
+ *      crates/ojas-cuda/src/device.rs:418-537): families of kernels loaded by name, dispatched
+ *      by canonical entry name with positional buffers then u32 constants;
+ *   2. the op seam      — `CudaSsm::mm(x, &Lin, y, m, accum)`
+ *      (crates/ojas-cuda/src/qwen35.rs:146-201, :644-702) and the MoE expert FFN
+ *      (crates/ojas-cpu/src/cpu_glm.rs:519-597, crates/ojas-cuda/src/kernels/moe.rs:45-125).
+ *
+ * Threading: one HIP stream per device handle; a handle is used from one thread at a time
+ * (the reference's decoder is not Sync either, crates/ojas-core/src/device_fault.rs:19-20).
+ * Every call is asynchronous on that stream unless stated; `ojh_submit` and `ojh_download`
+ * synchronise.
+ *
+ * Errors: every function returns OJH_OK (0) or a negative status; `ojh_last_error()` returns a
+ * thread-local message for the last failure.  Nothing aborts or throws across this boundary.
+ */
+#ifndef OJAS_HIP_H
+#define OJAS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OJH_ABI_VERSION 1
+
+enum {
+    OJH_OK = 0,
+    OJH_ERR_ARG = -1,        /* bad argument / shape the kernel cannot take */
+    OJH_ERR_HIP = -2,        /* a HIP runtime call failed (message has the HIP error) */
+    OJH_ERR_NOT_LOADED = -3, /* kernel or family not loaded: call ojh_ensure_family first */
+    OJH_ERR_UNSUPPORTED = -4,/* format / combination without a kernel */
+    OJH_ERR_BOUNDS = -5,     /* a buffer is too small for what the kernel would touch */
+    OJH_ERR_NO_DEVICE = -6
+};
+
+/* GGUF tensor types handled by this path (crates/ojas-formats/src/gguf.rs:563-591). */
+enum { OJH_Q8_0 = 8, OJH_Q4_K = 12, OJH_Q5_K = 13, OJH_Q6_K = 14 };
+
+/* Element type of an activation buffer handed to ojh_mm. */
+enum { OJH_X_F32 = 0, OJH_X_BF16 = 1, OJH_X_F16 = 2 };
+
+/* Arithmetic contract of a matmul.
+ *   OJH_ACT_Q8K — activations quantized to int8 per 256 (quant_q8k), integer dots: the arithmetic
+ *                 of the CPU reference `matvec_kq` (crates/ojas-cpu/src/cpu_math.rs:1145-1189).
+ *                 Q8_0 weights always take f32 activations, as `dot_q80` does (:971-981).
+ *   OJH_ACT_FLOAT — activations kept in floating point (f32 for the GEMV, rounded to f16 into the
+ *                 MFMA tile for the GEMM): the contract of the reference's GPU kernels
+ *                 (crates/ojas-core/src/quant_src.rs:779-867, crates/ojas-cuda/src/kernels/gemm_q.rs:1-56).
+ *   OJH_ACT_AUTO  — OJH_ACT_Q8K for K-quant GEMV-shaped calls, the MFMA tile above the crossover. */
+enum { OJH_ACT_AUTO = 0, OJH_ACT_Q8K = 1, OJH_ACT_FLOAT = 2 };
+
+typedef struct ojh_device ojh_device; /* one GPU + one stream + loaded families */
+typedef struct ojh_buf ojh_buf;       /* device allocation with a known size */
+typedef struct ojh_lin ojh_lin;       /* a weight matrix W[N,K] in its GGUF block bytes */
+
+/* Mirrors `Caps` (crates/ojas-core/src/kernel.rs:26-41). */
+typedef struct ojh_caps {
+    int32_t tier;            /* 0 = C, 1 = B, 2 = A (matrix units) */
+    int32_t f16_compute;
+    uint32_t simd_width;     /* 64 */
+    int32_t unified_memory;  /* 0 */
+    uint64_t max_buffer;
+    uint32_t compute_units;
+    uint32_t clock_mhz;
+    uint64_t total_memory;
+    char arch[32];           /* "gfx950..." */
+    const char *features;    /* comma-separated: "mfma_bf16,mfma_f16,mfma_i8,dot4_i8,wave64" */
+} ojh_caps;
+
+/* ---- device lifetime ---------------------------------------------------------------------- */
+/* `CudaGpu::new` (crates/ojas-cuda/src/device.rs:91-131). Fails with OJH_ERR_NO_DEVICE when no
+ * gfx950 GPU is visible: there is no CPU fallback behind this library. */
+int ojh_open(int ordinal, ojh_device **out);
+int ojh_close(ojh_device *dev);
+/* `Device::name` (crates/ojas-core/src/lib.rs:31). */
+const char *ojh_name(const ojh_device *dev);
+/* `KernelRuntime::caps` (crates/ojas-core/src/kernel.rs:72). */
+int ojh_caps_get(const ojh_device *dev, ojh_caps *out);
+const char *ojh_last_error(void);
+int ojh_abi_version(void);
+
+/* ---- buffers: `Device::alloc / upload / read` (crates/ojas-core/src/lib.rs:36-39,
+ *      crates/ojas-cuda/src/device.rs:448-476, byte forms :341-389) --------------------------- */
+int ojh_alloc(ojh_device *dev, size_t bytes, ojh_buf **out);
+int ojh_free(ojh_device *dev, ojh_buf *buf);
+/* Wrap device memory owned by someone else (e.g. a tensor of the host framework); not freed. */
+int ojh_wrap(ojh_device *dev, void *device_ptr, size_t bytes, ojh_buf **out);
+size_t ojh_buf_bytes(const ojh_buf *buf);
+void *ojh_buf_ptr(const ojh_buf *buf);
+/* Synchronous with respect to the host buffer: it may be reused as soon as the call returns. */
+int ojh_upload(ojh_device *dev, ojh_buf *dst, size_t dst_off, const void *host, size_t bytes);
+/* Waits for the device stream, then copies. */
+int ojh_download(ojh_device *dev, const ojh_buf *src, size_t src_off, void *host, size_t bytes);
+int ojh_memset0(ojh_device *dev, ojh_buf *dst, size_t off, size_t bytes);
+
+/* ---- kernel seam: `KernelRuntime` (crates/ojas-core/src/kernel.rs:67-81) -------------------- */
+/* Load the family's gfx950 code object (built offline). Families: "dequant", "gemv",
+ * "gemv_q8k", "gemm", "moe".  Idempotent. */
+int ojh_ensure_family(ojh_device *dev, const char *family);
+/* 1 if `name` resolved in a loaded family, 0 otherwise (never an error). */
+int ojh_has_kernel(const ojh_device *dev, const char *name);
+/* The family that defines `name` in this build's manifest, or NULL. */
+const char *ojh_kernel_family(const char *name);
+/* Manifest walk for structural tests: returns the number of kernels; fills name/family/counts
+ * of entry i when i is in range (crates/ojas-core/src/kernel.rs:43-58 `KernelSpec`). */
+int ojh_manifest(int i, const char **name, const char **family, int *n_bufs, int *n_consts);
+/* wave64 launch shape for a kernel at a problem size. The reference's callers carry 32-lane
+ * tables (crates/ojas-core/src/quant_src.rs:83-111); on gfx950 the library owns them. */
+int ojh_launch_shape(const ojh_device *dev, const char *name, uint32_t K, uint32_t N, uint32_t M,
+                     uint32_t grid[3], uint32_t block[3]);
+/* `dispatch(enc, name, bufs, consts, grid, block)`: buffers (with byte offsets) first, then u32
+ * constants, in the kernel's documented order.  Buffer sizes are checked against what the kernel
+ * touches at these constants before anything is launched. */
+int ojh_dispatch(ojh_device *dev, const char *name, int n_bufs, ojh_buf *const *bufs,
+                 const uint64_t *offsets, int n_consts, const uint32_t *consts,
+                 const uint32_t grid[3], const uint32_t block[3]);
+/* `submit(enc)`: wait for everything dispatched so far. */
+int ojh_submit(ojh_device *dev);
+
+/* Event timing on the device's stream (the reference times kernels the same way,
+ * crates/ojas-cuda/tests/prefill_gemm_q.rs:262-283). `ojh_timer_stop` synchronises. */
+int ojh_timer_start(ojh_device *dev);
+int ojh_timer_stop(ojh_device *dev, float *elapsed_ms);
+/* A pool of OJH_MAX_MARKS events for timing individual launches inside a longer region:
+ * `ojh_mark` records event `slot` on the stream; `ojh_mark_elapsed` waits for `b` and returns the
+ * time from `a` to `b`. */
+#define OJH_MAX_MARKS 8192
+int ojh_mark(ojh_device *dev, int slot);
+int ojh_mark_elapsed(ojh_device *dev, int a, int b, float *elapsed_ms);
+
+/* ---- op seam ------------------------------------------------------------------------------ */
+/* `Lin::load` (crates/ojas-cuda/src/qwen35.rs:174-201): keep the tensor in its GGUF block bytes.
+ * `raw` is host memory of n * row_bytes(type, k) bytes and is copied before the call returns. */
+int ojh_lin_create(ojh_device *dev, uint32_t ggml_type, uint32_t n, uint32_t k, const void *raw,
+                   ojh_lin **out);
+/* Same, over block bytes already resident in `raw` at `off` (borrowed, not freed). */
+int ojh_lin_wrap(ojh_device *dev, uint32_t ggml_type, uint32_t n, uint32_t k, ojh_buf *raw,
+                 size_t off, ojh_lin **out);
+int ojh_lin_free(ojh_device *dev, ojh_lin *lin);
+size_t ojh_row_bytes(uint32_t ggml_type, uint32_t k); /* 0 for an unknown type / ragged k */
+
+/* `CudaSsm::mm(x, w, y, m, accum)` (crates/ojas-cuda/src/qwen35.rs:644-702):
+ * y[m][N] (=, +=) x[m][K] . W^T, f32 result.  Chooses GEMV / small-M / MFMA tile / split-K.
+ * `bias` (f32[N]) may be NULL. */
+int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, const ojh_lin *w,
+           ojh_buf *y, size_t y_off, const ojh_buf *bias, uint32_t m, int accum, int act_mode);
+
+/* The same product from activations that are already quantized (`ojh_quant_q8k`): one
+ * quantization feeds every projection that reads the same vector (q/k/v, gate/up), the split the
+ * reference's CUDA path makes between `quantize_q8_1` and `gemv_q80_dp4a`
+ * (crates/ojas-cuda/src/kernels/gemv.rs:37-53, gemv_q8.rs:178-292). K-quant weights only. */
+int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const ojh_lin *w, ojh_buf *y,
+               size_t y_off, const ojh_buf *bias, uint32_t m, int accum);
+
+/* `dequant_to_f16` (crates/ojas-formats/src/gguf.rs:612-1116) on the device: `n_weights`
+ * weights of `raw` -> binary16 bit patterns in `out`. Bit-exact with the reference. */
+int ojh_dequant_f16(ojh_device *dev, uint32_t ggml_type, const ojh_buf *raw, size_t raw_off,
+                    size_t n_weights, ojh_buf *out, size_t out_off);
+
+/* `quant_q8k` (crates/ojas-cpu/src/cpu_math.rs:539-563) for m rows of k activations:
+ * q int8 [m][ceil(k/256)*256], scales f32 [m][ceil(k/256)]. */
+int ojh_quant_q8k(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, uint32_t m,
+                  uint32_t k, ojh_buf *q, ojh_buf *scales);
+
+/* Router: softmax over `n_expert` logits per token, top-`ksel` (lowest index wins ties),
+ * renormalised (crates/ojas-cuda/src/kernels/moe.rs:45-70). idx u32[T][ksel], wgt f32[T][ksel]. */
+int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uint32_t n_expert,
+                  uint32_t ksel, ojh_buf *idx, ojh_buf *wgt);
+
+/* Expert FFN over all (token, slot) assignments, grouped by expert
+ * (crates/ojas-cpu/src/cpu_glm.rs:551-582; per-assignment GPU form
+ * crates/ojas-metal/src/kernels/moe.rs:199-272):
+ *   y[t] (+)= sum_j wgt[t][j] * Wd_e( silu(Wg_e x[t]) * (Wu_e x[t]) ),  e = idx[t][j].
+ * gate/up: n_expert stacked matrices [n_ff][d]; down: n_expert stacked [d][n_ff]. */
+int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint32_t d, uint32_t n_ff,
+                uint32_t n_expert, uint32_t ksel, const ojh_buf *idx, const ojh_buf *wgt,
+                const ojh_lin *gate, const ojh_lin *up, const ojh_lin *down, ojh_buf *y,
+                int accum, int act_mode);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

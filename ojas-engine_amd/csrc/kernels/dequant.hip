@@ -1,0 +1,110 @@
+// Family "dequant": GGUF blocks -> IEEE binary16, bit-exact with the reference decoder
+// (crates/ojas-formats/src/gguf.rs:612-1116; arms :704-709 Q8_0, :1042-1059 Q4_K,
+// :1060-1085 Q5_K, :1086-1108 Q6_K).
+//
+// Bit-exactness rules: every product and difference is a separately rounded f32 operation
+// (__fmul_rn / __fsub_rn, never an FMA), in the reference's association order, followed by one
+// round-to-nearest-even conversion to binary16.  The file is also compiled with
+// -ffp-contract=off.
+//
+// Signature convention: pointers first, then u32 scalars.
+//   dequant_<fmt>_f16(const uchar* w, ushort* out, uint nblocks)
+#include "ojk_common.h"
+
+__device__ __forceinline__ ushort f32_to_f16_bits(float v) {
+    return __half_as_ushort(__float2half_rn(v));
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+dequant_q80_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
+    // one thread per weight
+    size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+    size_t b = i >> 5;
+    if (b >= nblocks) return;
+    const uchar* blk = w + b * Q80_BYTES;
+    float d = f16_bits_to_f32(*(const ushort*)blk);
+    float q = (float)(signed char)blk[2 + (i & 31u)];
+    out[i] = f32_to_f16_bits(__fmul_rn(d, q));
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+dequant_q4k_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
+    // 32 threads per super-block; thread t owns dword t of qs: 4 low-nibble weights of
+    // sub-block 2c and 4 high-nibble weights of sub-block 2c+1, c = t / 8.
+    size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x;
+    size_t b = tid >> 5;
+    if (b >= nblocks) return;
+    uint t = (uint)tid & 31u, c = t >> 3, o = (t & 7u) * 4u;
+    const uchar* blk = w + b * Q4K_BYTES;
+    const uint* hdr = (const uint*)blk;
+    uint dd = hdr[0];
+    float d = f16_bits_to_f32(dd & 0xFFFFu), dmin = f16_bits_to_f32(dd >> 16);
+    uint sc, mn;
+    q4k_scale_min_pair(hdr[1], hdr[2], hdr[3], c, sc, mn);
+    float dl1 = __fmul_rn(d, (float)(sc & 0xFFu)), ml1 = __fmul_rn(dmin, (float)(mn & 0xFFu));
+    float dl2 = __fmul_rn(d, (float)(sc >> 8)), ml2 = __fmul_rn(dmin, (float)(mn >> 8));
+    uint q = hdr[4 + t];
+    ushort* o1 = out + b * 256u + c * 64u + o;
+    ushort* o2 = o1 + 32;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint byte = (q >> (8 * i)) & 0xFFu;
+        o1[i] = f32_to_f16_bits(__fsub_rn(__fmul_rn(dl1, (float)(byte & 0xFu)), ml1));
+        o2[i] = f32_to_f16_bits(__fsub_rn(__fmul_rn(dl2, (float)(byte >> 4)), ml2));
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+dequant_q5k_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
+    // As Q4_K, plus the fifth bit: bit 2c of qh[l] for sub-block 2c, bit 2c+1 for 2c+1.
+    size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x;
+    size_t b = tid >> 5;
+    if (b >= nblocks) return;
+    uint t = (uint)tid & 31u, c = t >> 3, o = (t & 7u) * 4u;
+    const uchar* blk = w + b * Q5K_BYTES;
+    const uint* hdr = (const uint*)blk;
+    uint dd = hdr[0];
+    float d = f16_bits_to_f32(dd & 0xFFFFu), dmin = f16_bits_to_f32(dd >> 16);
+    uint sc, mn;
+    q4k_scale_min_pair(hdr[1], hdr[2], hdr[3], c, sc, mn);
+    float dl1 = __fmul_rn(d, (float)(sc & 0xFFu)), ml1 = __fmul_rn(dmin, (float)(mn & 0xFFu));
+    float dl2 = __fmul_rn(d, (float)(sc >> 8)), ml2 = __fmul_rn(dmin, (float)(mn >> 8));
+    uint qh = hdr[4 + (t & 7u)];  // qh bytes o..o+3
+    uint q = hdr[12 + t];
+    ushort* o1 = out + b * 256u + c * 64u + o;
+    ushort* o2 = o1 + 32;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint byte = (q >> (8 * i)) & 0xFFu;
+        uint hb = (qh >> (8 * i)) & 0xFFu;
+        float h1 = (hb >> (2 * c)) & 1u ? 16.0f : 0.0f;
+        float h2 = (hb >> (2 * c + 1)) & 1u ? 16.0f : 0.0f;
+        o1[i] = f32_to_f16_bits(__fsub_rn(__fmul_rn(dl1, __fadd_rn((float)(byte & 0xFu), h1)), ml1));
+        o2[i] = f32_to_f16_bits(__fsub_rn(__fmul_rn(dl2, __fadd_rn((float)(byte >> 4), h2)), ml2));
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+dequant_q6k_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
+    // 64 threads per super-block: thread (hf, l) decodes weights l, l+32, l+64, l+96 of half hf.
+    // The value is (d * sc) * q, left to right, as the reference writes it.
+    size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x;
+    size_t b = tid >> 6;
+    if (b >= nblocks) return;
+    uint t = (uint)tid & 63u, hf = t >> 5, l = t & 31u, is = l >> 4;
+    const uchar* blk = w + b * Q6K_BYTES;
+    const uchar* ql = blk + hf * 64u;
+    const uchar* qh = blk + 128u + hf * 32u;
+    const signed char* sc = (const signed char*)(blk + 192u + hf * 8u);
+    float d = f16_bits_to_f32(*(const ushort*)(blk + 208u));
+    uint a = ql[l], bq = ql[l + 32u], h = qh[l];
+    int q1 = (int)((a & 0xFu) | ((h & 3u) << 4)) - 32;
+    int q2 = (int)((bq & 0xFu) | (((h >> 2) & 3u) << 4)) - 32;
+    int q3 = (int)((a >> 4) | (((h >> 4) & 3u) << 4)) - 32;
+    int q4 = (int)((bq >> 4) | (((h >> 6) & 3u) << 4)) - 32;
+    ushort* o = out + b * 256u + hf * 128u + l;
+    o[0]  = f32_to_f16_bits(__fmul_rn(__fmul_rn(d, (float)sc[is]), (float)q1));
+    o[32] = f32_to_f16_bits(__fmul_rn(__fmul_rn(d, (float)sc[is + 2]), (float)q2));
+    o[64] = f32_to_f16_bits(__fmul_rn(__fmul_rn(d, (float)sc[is + 4]), (float)q3));
+    o[96] = f32_to_f16_bits(__fmul_rn(__fmul_rn(d, (float)sc[is + 6]), (float)q4));
+}

@@ -1,0 +1,366 @@
+// Family "gemv": fused-dequant matvecs on raw GGUF blocks with f32 activations — the contract
+// of the reference's GPU kernels gemv_nat_<fmt>{,_accum,_bias,_m}
+// (crates/ojas-cuda/src/kernels/nat.rs:69-89; bodies crates/ojas-core/src/quant_src.rs:779-824
+// Q4_K, :833-867 Q6_K, :1028-1057 Q8_0, :1154-1180 batched).
+//
+//   gemv_nat_<fmt>{,_accum}(x, w, y, K, N)        y[n] (=,+=) sum_k W[n,k] x[k]
+//   gemv_nat_<fmt>_bias(x, w, y, bs, K, N)        y[n] = ... + bs[n]
+//   gemv_nat_<fmt>_m(x, w, y, K, N, M, ACC)       x[M][K], y[M][N]
+//
+// wave64 plan, common to the three formats: a group of lanes shares one block, a wave walks
+// several blocks per step, the activation fragment of a step is loaded once and reused across
+// the R rows of the wave.  Scales stay factored: the lane accumulates sum(code * x) per sub-block
+// and applies d*sc (and -dmin*m*sum(x) for Q4_K) once per sub-block.
+#include "ojk_common.h"
+
+enum { ST_SET = 0, ST_ACCUM = 1, ST_BIAS = 2 };
+
+template <int MODE>
+__device__ __forceinline__ void store_row(float* y, const float* bs, uint n, float v) {
+    if (MODE == ST_SET) y[n] = v;
+    else if (MODE == ST_ACCUM) y[n] += v;
+    else y[n] = v + bs[n];
+}
+
+__device__ __forceinline__ float ub0(uint v) { return (float)(v & 0xFFu); }
+__device__ __forceinline__ float ub1(uint v) { return (float)((v >> 8) & 0xFFu); }
+__device__ __forceinline__ float ub2(uint v) { return (float)((v >> 16) & 0xFFu); }
+__device__ __forceinline__ float ub3(uint v) { return (float)(v >> 24); }
+
+// sum of 4 unsigned bytes of `w` times 4 floats
+__device__ __forceinline__ float dot4_ub(uint w, float4 x, float acc) {
+    acc = fmaf(ub0(w), x.x, acc);
+    acc = fmaf(ub1(w), x.y, acc);
+    acc = fmaf(ub2(w), x.z, acc);
+    return fmaf(ub3(w), x.w, acc);
+}
+__device__ __forceinline__ float sum4(float4 v) { return (v.x + v.y) + (v.z + v.w); }
+
+// ------------------------------------------------------------------ Q4_K
+// Lane (g, l) = (lane/8, lane%8): 16 quant bytes l*16.. of super-block g -> 16 weights of
+// sub-block 2c (low nibbles) and 16 of sub-block 2c+1 (high nibbles), c = l/2.
+struct Q4kFragF {
+    float4 xl[4], xh[4];
+    float sl, sh;  // sums of the two 16-float halves (for the -dmin*m term)
+};
+
+__device__ __forceinline__ Q4kFragF q4k_load_frag_f(const float* x, uint sb, uint l) {
+    Q4kFragF f;
+    const float4* p = (const float4*)(x + (size_t)sb * 256u + (l >> 1) * 64u + (l & 1u) * 16u);
+    float sl = 0.0f, sh = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        f.xl[i] = p[i];
+        f.xh[i] = p[8 + i];
+        sl += sum4(f.xl[i]);
+        sh += sum4(f.xh[i]);
+    }
+    f.sl = sl;
+    f.sh = sh;
+    return f;
+}
+
+__device__ __forceinline__ float q4k_lane_dot_f(uint4 hdr, uint4 qs, uint c, const Q4kFragF& f) {
+    const uint M4 = 0x0F0F0F0Fu;
+    float al = dot4_ub(qs.x & M4, f.xl[0], 0.0f);
+    al = dot4_ub(qs.y & M4, f.xl[1], al);
+    al = dot4_ub(qs.z & M4, f.xl[2], al);
+    al = dot4_ub(qs.w & M4, f.xl[3], al);
+    float ah = dot4_ub((qs.x >> 4) & M4, f.xh[0], 0.0f);
+    ah = dot4_ub((qs.y >> 4) & M4, f.xh[1], ah);
+    ah = dot4_ub((qs.z >> 4) & M4, f.xh[2], ah);
+    ah = dot4_ub((qs.w >> 4) & M4, f.xh[3], ah);
+    uint sc, mn;
+    q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
+    float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
+    float pos = (float)(sc & 0xFFu) * al + (float)(sc >> 8) * ah;
+    float neg = (float)(mn & 0xFFu) * f.sl + (float)(mn >> 8) * f.sh;
+    return d * pos - dmin * neg;
+}
+
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_q4k_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                  float* __restrict__ y, const float* __restrict__ bs,
+                                                  uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 >= N) return;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (uint sb = g; sb < nsb; sb += 8u) {
+        uint4 hdr[R], qs[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            uint row = min(row0 + r, N - 1u);
+            const uchar* blk = w + ((size_t)row * nsb + sb) * Q4K_BYTES;
+            hdr[r] = *(const uint4*)blk;
+            qs[r] = *(const uint4*)(blk + 16u + l * 16u);
+        }
+        Q4kFragF f = q4k_load_frag_f(x, sb, l);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += q4k_lane_dot_f(hdr[r], qs[r], c, f);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float t = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, t);
+    }
+}
+
+template <int MT>
+__device__ __forceinline__ void gemv_nat_q4k_m_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                    float* __restrict__ y, uint K, uint N, uint M, uint ACC) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    for (uint m0 = 0; m0 < M; m0 += MT) {
+        float acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; t++) acc[t] = 0.0f;
+        for (uint sb = g; sb < nsb; sb += 8u) {
+            const uchar* blk = w + ((size_t)row * nsb + sb) * Q4K_BYTES;
+            uint4 hdr = *(const uint4*)blk;
+            uint4 qs = *(const uint4*)(blk + 16u + l * 16u);
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                uint m = min(m0 + t, M - 1u);
+                Q4kFragF f = q4k_load_frag_f(x + (size_t)m * K, sb, l);
+                acc[t] += q4k_lane_dot_f(hdr, qs, c, f);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            float s = wave_sum(acc[t]);
+            if (lane == 0 && m0 + t < M) {
+                float* o = y + (size_t)(m0 + t) * N + row;
+                *o = ACC ? *o + s : s;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ Q6_K
+// Lane (g, t) = (lane/16, lane%16): half hf = t/8, weights l0..l0+3 (l0 = 4*(t%8)) of each of the
+// four quarters of that half; one int8 sub-scale per quarter.
+struct Q6kFragF {
+    float4 x[4];
+    float s[4];
+};
+
+__device__ __forceinline__ Q6kFragF q6k_load_frag_f(const float* x, uint sb, uint hf, uint l0) {
+    Q6kFragF f;
+    const float* p = x + (size_t)sb * 256u + hf * 128u + l0;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        f.x[q] = *(const float4*)(p + 32 * q);
+        f.s[q] = sum4(f.x[q]);
+    }
+    return f;
+}
+
+struct Q6kRaw {
+    uint qa, qb, qh, sc4, d16;
+};
+
+__device__ __forceinline__ Q6kRaw q6k_load_raw(const uchar* blk, uint hf, uint l0) {
+    Q6kRaw r;
+    r.qa = *(const u32_a2*)(blk + hf * 64u + l0);
+    r.qb = *(const u32_a2*)(blk + hf * 64u + 32u + l0);
+    r.qh = *(const u32_a2*)(blk + 128u + hf * 32u + l0);
+    u32x2_a2 s = *(const u32x2_a2*)(blk + 192u + hf * 8u);
+    uint is = l0 >> 4;
+    uint a = s.x >> (8u * is), b = s.y >> (8u * is);
+    r.sc4 = (a & 0xFFu) | ((a >> 8) & 0xFF00u) | ((b & 0xFFu) << 16) | ((b << 8) & 0xFF000000u);
+    r.d16 = *(const ushort*)(blk + 208u);
+    return r;
+}
+
+__device__ __forceinline__ float q6k_lane_dot_f(const Q6kRaw& r, const Q6kFragF& f) {
+    const uint M4 = 0x0F0F0F0Fu, H2 = 0x30303030u;
+    uint w0 = (r.qa & M4) | ((r.qh << 4) & H2);
+    uint w1 = (r.qb & M4) | ((r.qh << 2) & H2);
+    uint w2 = ((r.qa >> 4) & M4) | (r.qh & H2);
+    uint w3 = ((r.qb >> 4) & M4) | ((r.qh >> 2) & H2);
+    // sum((code - 32) * x) = sum(code * x) - 32 * sum(x)
+    float t0 = dot4_ub(w0, f.x[0], -32.0f * f.s[0]);
+    float t1 = dot4_ub(w1, f.x[1], -32.0f * f.s[1]);
+    float t2 = dot4_ub(w2, f.x[2], -32.0f * f.s[2]);
+    float t3 = dot4_ub(w3, f.x[3], -32.0f * f.s[3]);
+    float s0 = (float)(signed char)(r.sc4), s1 = (float)(signed char)(r.sc4 >> 8);
+    float s2 = (float)(signed char)(r.sc4 >> 16), s3 = (float)((int)r.sc4 >> 24);
+    return f16_bits_to_f32(r.d16) * ((s0 * t0 + s1 * t1) + (s2 * t2 + s3 * t3));
+}
+
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_q6k_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                  float* __restrict__ y, const float* __restrict__ bs,
+                                                  uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 >= N) return;
+    const uint nsb = K >> 8, g = lane >> 4, t = lane & 15u, hf = t >> 3, l0 = (t & 7u) * 4u;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (uint sb = g; sb < nsb; sb += 4u) {
+        Q6kRaw raw[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            uint row = min(row0 + r, N - 1u);
+            raw[r] = q6k_load_raw(w + ((size_t)row * nsb + sb) * Q6K_BYTES, hf, l0);
+        }
+        Q6kFragF f = q6k_load_frag_f(x, sb, hf, l0);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += q6k_lane_dot_f(raw[r], f);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float s = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, s);
+    }
+}
+
+template <int MT>
+__device__ __forceinline__ void gemv_nat_q6k_m_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                    float* __restrict__ y, uint K, uint N, uint M, uint ACC) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const uint nsb = K >> 8, g = lane >> 4, t = lane & 15u, hf = t >> 3, l0 = (t & 7u) * 4u;
+    for (uint m0 = 0; m0 < M; m0 += MT) {
+        float acc[MT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) acc[i] = 0.0f;
+        for (uint sb = g; sb < nsb; sb += 4u) {
+            Q6kRaw raw = q6k_load_raw(w + ((size_t)row * nsb + sb) * Q6K_BYTES, hf, l0);
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                uint m = min(m0 + i, M - 1u);
+                Q6kFragF f = q6k_load_frag_f(x + (size_t)m * K, sb, hf, l0);
+                acc[i] += q6k_lane_dot_f(raw, f);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float s = wave_sum(acc[i]);
+            if (lane == 0 && m0 + i < M) {
+                float* o = y + (size_t)(m0 + i) * N + row;
+                *o = ACC ? *o + s : s;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ Q8_0
+// Four lanes share a 34-byte block (8 int8 each); a wave walks 16 blocks (512 weights) per step.
+__device__ __forceinline__ float sb0(uint v) { return (float)(signed char)(v); }
+__device__ __forceinline__ float sb1(uint v) { return (float)(signed char)(v >> 8); }
+__device__ __forceinline__ float sb2(uint v) { return (float)(signed char)(v >> 16); }
+__device__ __forceinline__ float sb3(uint v) { return (float)((int)v >> 24); }
+
+__device__ __forceinline__ float q80_lane_dot(uint d16, u32x2_a2 q, float4 x0, float4 x1) {
+    float a = sb0(q.x) * x0.x;
+    a = fmaf(sb1(q.x), x0.y, a);
+    a = fmaf(sb2(q.x), x0.z, a);
+    a = fmaf(sb3(q.x), x0.w, a);
+    a = fmaf(sb0(q.y), x1.x, a);
+    a = fmaf(sb1(q.y), x1.y, a);
+    a = fmaf(sb2(q.y), x1.z, a);
+    a = fmaf(sb3(q.y), x1.w, a);
+    return f16_bits_to_f32(d16) * a;
+}
+
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_q80_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                  float* __restrict__ y, const float* __restrict__ bs,
+                                                  uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 >= N) return;
+    const uint nb = K >> 5, g = lane >> 2, p = lane & 3u;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (uint b = g; b < nb; b += 16u) {
+        uint d16[R];
+        u32x2_a2 q[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            uint row = min(row0 + r, N - 1u);
+            const uchar* blk = w + ((size_t)row * nb + b) * Q80_BYTES;
+            d16[r] = *(const ushort*)blk;
+            q[r] = *(const u32x2_a2*)(blk + 2u + p * 8u);
+        }
+        const float4* xp = (const float4*)(x + (size_t)b * 32u + p * 8u);
+        float4 x0 = xp[0], x1 = xp[1];
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += q80_lane_dot(d16[r], q[r], x0, x1);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float s = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, s);
+    }
+}
+
+template <int MT>
+__device__ __forceinline__ void gemv_nat_q80_m_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                    float* __restrict__ y, uint K, uint N, uint M, uint ACC) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const uint nb = K >> 5, g = lane >> 2, p = lane & 3u;
+    for (uint m0 = 0; m0 < M; m0 += MT) {
+        float acc[MT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) acc[i] = 0.0f;
+        for (uint b = g; b < nb; b += 16u) {
+            const uchar* blk = w + ((size_t)row * nb + b) * Q80_BYTES;
+            uint d16 = *(const ushort*)blk;
+            u32x2_a2 q = *(const u32x2_a2*)(blk + 2u + p * 8u);
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                uint m = min(m0 + i, M - 1u);
+                const float4* xp = (const float4*)(x + (size_t)m * K + (size_t)b * 32u + p * 8u);
+                acc[i] += q80_lane_dot(d16, q, xp[0], xp[1]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float s = wave_sum(acc[i]);
+            if (lane == 0 && m0 + i < M) {
+                float* o = y + (size_t)(m0 + i) * N + row;
+                *o = ACC ? *o + s : s;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ entries
+#define GEMV_NAT_ENTRIES(FMT)                                                                              \
+    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_r1(                                 \
+        const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
+        gemv_nat_##FMT##_body<1, ST_SET>(x, w, y, nullptr, K, N); }                                        \
+    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_r2(                                 \
+        const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
+        gemv_nat_##FMT##_body<2, ST_SET>(x, w, y, nullptr, K, N); }                                        \
+    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT(                                      \
+        const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
+        gemv_nat_##FMT##_body<4, ST_SET>(x, w, y, nullptr, K, N); }                                        \
+    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_accum(                              \
+        const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
+        gemv_nat_##FMT##_body<4, ST_ACCUM>(x, w, y, nullptr, K, N); }                                      \
+    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_bias(                               \
+        const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {                       \
+        gemv_nat_##FMT##_body<4, ST_BIAS>(x, w, y, bs, K, N); }                                            \
+    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_m(                                  \
+        const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {                      \
+        if (M <= 2) gemv_nat_##FMT##_m_body<2>(x, w, y, K, N, M, ACC);                                     \
+        else gemv_nat_##FMT##_m_body<4>(x, w, y, K, N, M, ACC); }
+
+GEMV_NAT_ENTRIES(q80)
+GEMV_NAT_ENTRIES(q4k)
+GEMV_NAT_ENTRIES(q6k)

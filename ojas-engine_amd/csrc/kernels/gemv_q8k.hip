@@ -1,0 +1,334 @@
+// Family "gemv_q8k": the CPU reference's own arithmetic for K-quant rows on the GPU —
+// activations quantized to int8 per 256-superblock ("Q8_K-flavoured"), integer dots against the
+// raw 4/6-bit codes, f32 scale algebra per super-block.
+//
+// Reference: crates/ojas-cpu/src/cpu_math.rs:539-563 (quant_q8k), :609-635 (dot_q4k),
+// :674-722 (dot_q6k), :1145-1189 (matvec_kq).
+//
+//   quantize_q8k{,_bf16}(x, q, scales, K, M)             grid (ceil(K/256), M), block 256
+//   gemv_q8k_<fmt>{,_accum,_bias}(xq, xs, w, y[, bs], K, N)
+//   gemv_q8k_<fmt>_m(xq, xs, w, y, K, N, M, ACC)          y[M][N], one weight pass per MT tokens
+//
+// Integer sums are exact, so  sum_j sc_j*idot_j  and  sum_j m_j*bsum_j  are formed in int32 and
+// converted once; they equal the reference's sequential f32 sums whenever those are exact
+// (always for the min term; for the scale term unless |sum| >= 2^24, where the reference itself
+// rounds).  The per-row f32 accumulation over super-blocks runs in a different order than the
+// reference's (lanes own different super-blocks), which moves the last ulp only.
+#include "ojk_common.h"
+
+// ------------------------------------------------------------------ activation quantizer
+template <bool BF16>
+__device__ __forceinline__ void quantize_q8k_body(const void* __restrict__ xv, signed char* __restrict__ q,
+                                                  float* __restrict__ scales, uint K, uint M) {
+    __shared__ float wmax[4];
+    const uint sb = blockIdx.x, m = blockIdx.y, tid = threadIdx.x;
+    const uint nsb = (K + 255u) >> 8;
+    const uint i = sb * 256u + tid;
+    float v = 0.0f;
+    if (i < K) {
+        if (BF16) v = bf16_bits_to_f32(((const ushort*)xv)[(size_t)m * K + i]);
+        else v = ((const float*)xv)[(size_t)m * K + i];
+    }
+    float a = wave_max(fabsf(v));
+    if ((tid & 63u) == 0) wmax[tid >> 6] = a;
+    __syncthreads();
+    float mx = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+    // scale = amax/127 (1 when the segment is all zero); q = clamp(round_half_away(v * (1/scale)))
+    float scale = mx > 0.0f ? __fdiv_rn(mx, 127.0f) : 1.0f;
+    float inv = __fdiv_rn(1.0f, scale);
+    float r = roundf(__fmul_rn(v, inv));
+    r = fminf(fmaxf(r, -127.0f), 127.0f);
+    // the padded tail of a ragged last segment is written as zero
+    q[((size_t)m * nsb + sb) * 256u + tid] = (signed char)(int)r;
+    if (tid == 0) scales[(size_t)m * nsb + sb] = scale;
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+quantize_q8k(const float* x, signed char* q, float* scales, uint K, uint M) {
+    quantize_q8k_body<false>(x, q, scales, K, M);
+}
+extern "C" __global__ void __launch_bounds__(256)
+quantize_q8k_bf16(const ushort* x, signed char* q, float* scales, uint K, uint M) {
+    quantize_q8k_body<true>(x, q, scales, K, M);
+}
+
+// ------------------------------------------------------------------ store modes
+enum { ST_SET = 0, ST_ACCUM = 1, ST_BIAS = 2 };
+
+template <int MODE>
+__device__ __forceinline__ void store_row(float* y, const float* bs, uint n, float v) {
+    if (MODE == ST_SET) y[n] = v;
+    else if (MODE == ST_ACCUM) y[n] += v;
+    else y[n] = v + bs[n];
+}
+
+__device__ __forceinline__ int bytesum4(uint4 v) {
+    int s = dot4_i8(v.x, 0x01010101u, 0);
+    s = dot4_i8(v.y, 0x01010101u, s);
+    s = dot4_i8(v.z, 0x01010101u, s);
+    return dot4_i8(v.w, 0x01010101u, s);
+}
+
+// ------------------------------------------------------------------ Q4_K
+// Eight lanes share a super-block and a wave walks eight super-blocks (2048 weights) per step.
+// Lane (g, l) = (lane/8, lane%8) owns the 16 quant bytes l*16..l*16+15 of super-block g: 16
+// low-nibble weights of sub-block 2c and 16 high-nibble weights of sub-block 2c+1, c = l/2.  The
+// activation fragment (2 x 16 int8, their sums, the segment scale) is loaded once per step and
+// reused across the R rows of the wave.
+struct Q4kFrag {
+    uint4 xl, xh;  // int8 activations for the low / high nibble halves
+    int bl, bh;    // their sums (the lane's part of bsums)
+    float sx;      // activation scale of the super-block
+};
+
+__device__ __forceinline__ Q4kFrag q4k_load_frag(const signed char* xq, const float* xs, uint sb, uint l) {
+    Q4kFrag f;
+    const signed char* p = xq + (size_t)sb * 256u + (l >> 1) * 64u + (l & 1u) * 16u;
+    f.xl = *(const uint4*)p;
+    f.xh = *(const uint4*)(p + 32);
+    f.bl = bytesum4(f.xl);
+    f.bh = bytesum4(f.xh);
+    f.sx = xs[sb];
+    return f;
+}
+
+// One lane's 32 weights of one super-block against one activation fragment.
+__device__ __forceinline__ float q4k_lane_dot(uint4 hdr, uint4 qs, uint c, const Q4kFrag& f) {
+    const uint M4 = 0x0F0F0F0Fu;
+    int il = dot4_i8(qs.x & M4, f.xl.x, 0);
+    il = dot4_i8(qs.y & M4, f.xl.y, il);
+    il = dot4_i8(qs.z & M4, f.xl.z, il);
+    il = dot4_i8(qs.w & M4, f.xl.w, il);
+    int ih = dot4_i8((qs.x >> 4) & M4, f.xh.x, 0);
+    ih = dot4_i8((qs.y >> 4) & M4, f.xh.y, ih);
+    ih = dot4_i8((qs.z >> 4) & M4, f.xh.z, ih);
+    ih = dot4_i8((qs.w >> 4) & M4, f.xh.w, ih);
+    uint sc, mn;
+    q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
+    int isum = (int)(sc & 0xFFu) * il + (int)(sc >> 8) * ih;
+    int msum = (int)(mn & 0xFFu) * f.bl + (int)(mn >> 8) * f.bh;
+    float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
+    return f.sx * (d * (float)isum - dmin * (float)msum);
+}
+
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_q8k_q4k_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                  const uchar* __restrict__ w, float* __restrict__ y,
+                                                  const float* __restrict__ bs, uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 >= N) return;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (uint sb = g; sb < nsb; sb += 8u) {
+        uint4 hdr[R], qs[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            uint row = min(row0 + r, N - 1u);
+            const uchar* blk = w + ((size_t)row * nsb + sb) * Q4K_BYTES;
+            hdr[r] = *(const uint4*)blk;
+            qs[r] = *(const uint4*)(blk + 16u + l * 16u);
+        }
+        Q4kFrag f = q4k_load_frag(xq, xs, sb, l);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += q4k_lane_dot(hdr[r], qs[r], c, f);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float t = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, t);
+    }
+}
+
+#define GEMV_Q8K_ENTRIES(FMT, BODY)                                                                          \
+    extern "C" __global__ void __launch_bounds__(256) gemv_q8k_##FMT##_r1(                                   \
+        const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N) {                  \
+        BODY<1, ST_SET>(xq, xs, w, y, nullptr, K, N); }                                                      \
+    extern "C" __global__ void __launch_bounds__(256) gemv_q8k_##FMT##_r2(                                   \
+        const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N) {                  \
+        BODY<2, ST_SET>(xq, xs, w, y, nullptr, K, N); }                                                      \
+    extern "C" __global__ void __launch_bounds__(256) gemv_q8k_##FMT(                                        \
+        const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N) {                  \
+        BODY<4, ST_SET>(xq, xs, w, y, nullptr, K, N); }                                                      \
+    extern "C" __global__ void __launch_bounds__(256) gemv_q8k_##FMT##_accum(                                \
+        const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N) {                  \
+        BODY<4, ST_ACCUM>(xq, xs, w, y, nullptr, K, N); }                                                    \
+    extern "C" __global__ void __launch_bounds__(256) gemv_q8k_##FMT##_bias(                                 \
+        const signed char* xq, const float* xs, const uchar* w, float* y, const float* bs, uint K, uint N) { \
+        BODY<4, ST_BIAS>(xq, xs, w, y, bs, K, N); }
+
+GEMV_Q8K_ENTRIES(q4k, gemv_q8k_q4k_body)
+
+// Batched form: y[M][N] (+)= quantized x[M][K] . W^T.  One wave per row; the row's weights are
+// read and unpacked once per tile of MT tokens.
+template <int MT>
+__device__ __forceinline__ void gemv_q8k_q4k_m_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                    const uchar* __restrict__ w, float* __restrict__ y,
+                                                    uint K, uint N, uint M, uint ACC) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    for (uint m0 = 0; m0 < M; m0 += MT) {
+        float acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; t++) acc[t] = 0.0f;
+        for (uint sb = g; sb < nsb; sb += 8u) {
+            const uchar* blk = w + ((size_t)row * nsb + sb) * Q4K_BYTES;
+            uint4 hdr = *(const uint4*)blk;
+            uint4 qs = *(const uint4*)(blk + 16u + l * 16u);
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                uint m = min(m0 + t, M - 1u);
+                Q4kFrag f = q4k_load_frag(xq + (size_t)m * nsb * 256u, xs + (size_t)m * nsb, sb, l);
+                acc[t] += q4k_lane_dot(hdr, qs, c, f);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            float s = wave_sum(acc[t]);
+            if (lane == 0 && m0 + t < M) {
+                float* o = y + (size_t)(m0 + t) * N + row;
+                *o = ACC ? *o + s : s;
+            }
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+gemv_q8k_q4k_m(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    if (M <= 2) gemv_q8k_q4k_m_body<2>(xq, xs, w, y, K, N, M, ACC);
+    else if (M <= 4) gemv_q8k_q4k_m_body<4>(xq, xs, w, y, K, N, M, ACC);
+    else gemv_q8k_q4k_m_body<8>(xq, xs, w, y, K, N, M, ACC);
+}
+
+// ------------------------------------------------------------------ Q6_K
+// Sixteen lanes share a super-block and a wave walks four per step.  Lane (g, t) = (lane/16,
+// lane%16) owns, in half hf = t/8, the four weights l0..l0+3 (l0 = 4*(t%8)) of each of the four
+// quarters: three dwords (two of ql, one of qh) give 16 six-bit codes, each quarter under one
+// int8 sub-scale sc[2q + l0/16].
+struct Q6kFrag {
+    uint x[4];   // 4 int8 activations per quarter
+    int xs[4];   // their sums (for the -32 offset of the codes)
+    float sx;
+};
+
+__device__ __forceinline__ Q6kFrag q6k_load_frag(const signed char* xq, const float* xs, uint sb, uint hf, uint l0) {
+    Q6kFrag f;
+    const signed char* p = xq + (size_t)sb * 256u + hf * 128u + l0;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        f.x[q] = *(const uint*)(p + 32 * q);
+        f.xs[q] = dot4_i8(f.x[q], 0x01010101u, 0);
+    }
+    f.sx = xs[sb];
+    return f;
+}
+
+struct Q6kRaw {
+    uint qa, qb, qh;  // ql[l0..], ql[32+l0..], qh[l0..]
+    uint sc4;         // the lane's four sub-scales, one per byte
+    uint d16;
+};
+
+__device__ __forceinline__ Q6kRaw q6k_load_raw(const uchar* blk, uint hf, uint l0) {
+    Q6kRaw r;
+    r.qa = *(const u32_a2*)(blk + hf * 64u + l0);
+    r.qb = *(const u32_a2*)(blk + hf * 64u + 32u + l0);
+    r.qh = *(const u32_a2*)(blk + 128u + hf * 32u + l0);
+    u32x2_a2 s = *(const u32x2_a2*)(blk + 192u + hf * 8u);
+    // bytes is, is+2, is+4, is+6 of the 8 sub-scales -> one per byte of sc4
+    uint is = l0 >> 4;
+    uint a = s.x >> (8u * is), b = s.y >> (8u * is);
+    r.sc4 = (a & 0xFFu) | ((a >> 8) & 0xFF00u) | ((b & 0xFFu) << 16) | ((b << 8) & 0xFF000000u);
+    r.d16 = *(const ushort*)(blk + 208u);
+    return r;
+}
+
+__device__ __forceinline__ float q6k_lane_dot(const Q6kRaw& r, const Q6kFrag& f) {
+    const uint M4 = 0x0F0F0F0Fu, H2 = 0x30303030u;
+    uint w0 = (r.qa & M4) | ((r.qh << 4) & H2);
+    uint w1 = (r.qb & M4) | ((r.qh << 2) & H2);
+    uint w2 = ((r.qa >> 4) & M4) | (r.qh & H2);
+    uint w3 = ((r.qb >> 4) & M4) | ((r.qh >> 2) & H2);
+    int i0 = dot4_i8(w0, f.x[0], 0) - 32 * f.xs[0];
+    int i1 = dot4_i8(w1, f.x[1], 0) - 32 * f.xs[1];
+    int i2 = dot4_i8(w2, f.x[2], 0) - 32 * f.xs[2];
+    int i3 = dot4_i8(w3, f.x[3], 0) - 32 * f.xs[3];
+    int s0 = (int)(signed char)(r.sc4), s1 = (int)(signed char)(r.sc4 >> 8);
+    int s2 = (int)(signed char)(r.sc4 >> 16), s3 = (int)r.sc4 >> 24;
+    int isum = s0 * i0 + s1 * i1 + s2 * i2 + s3 * i3;
+    return f.sx * f16_bits_to_f32(r.d16) * (float)isum;
+}
+
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_q8k_q6k_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                  const uchar* __restrict__ w, float* __restrict__ y,
+                                                  const float* __restrict__ bs, uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 >= N) return;
+    const uint nsb = K >> 8, g = lane >> 4, t = lane & 15u, hf = t >> 3, l0 = (t & 7u) * 4u;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (uint sb = g; sb < nsb; sb += 4u) {
+        Q6kRaw raw[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            uint row = min(row0 + r, N - 1u);
+            raw[r] = q6k_load_raw(w + ((size_t)row * nsb + sb) * Q6K_BYTES, hf, l0);
+        }
+        Q6kFrag f = q6k_load_frag(xq, xs, sb, hf, l0);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += q6k_lane_dot(raw[r], f);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float s = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, s);
+    }
+}
+
+GEMV_Q8K_ENTRIES(q6k, gemv_q8k_q6k_body)
+
+template <int MT>
+__device__ __forceinline__ void gemv_q8k_q6k_m_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                    const uchar* __restrict__ w, float* __restrict__ y,
+                                                    uint K, uint N, uint M, uint ACC) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const uint nsb = K >> 8, g = lane >> 4, t = lane & 15u, hf = t >> 3, l0 = (t & 7u) * 4u;
+    for (uint m0 = 0; m0 < M; m0 += MT) {
+        float acc[MT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) acc[i] = 0.0f;
+        for (uint sb = g; sb < nsb; sb += 4u) {
+            Q6kRaw raw = q6k_load_raw(w + ((size_t)row * nsb + sb) * Q6K_BYTES, hf, l0);
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                uint m = min(m0 + i, M - 1u);
+                Q6kFrag f = q6k_load_frag(xq + (size_t)m * nsb * 256u, xs + (size_t)m * nsb, sb, hf, l0);
+                acc[i] += q6k_lane_dot(raw, f);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float s = wave_sum(acc[i]);
+            if (lane == 0 && m0 + i < M) {
+                float* o = y + (size_t)(m0 + i) * N + row;
+                *o = ACC ? *o + s : s;
+            }
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+gemv_q8k_q6k_m(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    if (M <= 2) gemv_q8k_q6k_m_body<2>(xq, xs, w, y, K, N, M, ACC);
+    else if (M <= 4) gemv_q8k_q6k_m_body<4>(xq, xs, w, y, K, N, M, ACC);
+    else gemv_q8k_q6k_m_body<8>(xq, xs, w, y, K, N, M, ACC);
+}

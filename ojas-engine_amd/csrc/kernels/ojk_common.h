@@ -1,0 +1,118 @@
+// Device-side helpers shared by every gfx950 kernel family: block-format constants,
+// f16 / bf16 bit conversions, wave64 reductions on DPP, 2-byte-aligned vector loads.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+typedef unsigned int uint;
+typedef unsigned char uchar;
+typedef unsigned short ushort;
+
+#define OJK_WAVE 64
+
+// GGUF block sizes (reference: crates/ojas-formats/src/gguf.rs:563-591).
+#define Q80_BYTES 34u
+#define Q4K_BYTES 144u
+#define Q5K_BYTES 176u
+#define Q6K_BYTES 210u
+
+// Vector types that may sit on a 2-byte boundary: Q8_0 (34 B) and Q6_K (210 B) blocks are only
+// 2-byte aligned inside a row.  gfx950 runs in unaligned-access mode, so these compile to one
+// global_load_dwordxN each.
+struct __attribute__((packed, aligned(2))) u32x4_a2 { uint x, y, z, w; };
+struct __attribute__((packed, aligned(2))) u32x2_a2 { uint x, y; };
+typedef uint __attribute__((aligned(2))) u32_a2;
+
+__device__ __forceinline__ float f16_bits_to_f32(uint bits16) {
+    return __half2float(__ushort_as_half((ushort)bits16));
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint bits16) {
+    return __uint_as_float(bits16 << 16);
+}
+// f32 -> bf16, round to nearest even (NaN kept quiet).
+__device__ __forceinline__ ushort f32_to_bf16_bits(float f) {
+    uint x = __float_as_uint(f);
+    if ((x & 0x7F800000u) == 0x7F800000u && (x & 0x7FFFFFu)) return (ushort)((x >> 16) | 0x40u);
+    x += 0x7FFFu + ((x >> 16) & 1u);
+    return (ushort)(x >> 16);
+}
+
+// ---- DPP cross-lane moves (wave64) --------------------------------------------------------
+#define OJK_DPP_QUAD_XOR1 0xB1   // quad_perm:[1,0,3,2]
+#define OJK_DPP_QUAD_XOR2 0x4E   // quad_perm:[2,3,0,1]
+#define OJK_DPP_ROW_HALF_MIRROR 0x141
+#define OJK_DPP_ROW_MIRROR 0x140
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+
+// Sum over the 16 lanes of a DPP row; every lane of the row ends with the row total.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_f32<OJK_DPP_QUAD_XOR1>(v);
+    v += dpp_f32<OJK_DPP_QUAD_XOR2>(v);
+    v += dpp_f32<OJK_DPP_ROW_HALF_MIRROR>(v);
+    v += dpp_f32<OJK_DPP_ROW_MIRROR>(v);
+    return v;
+}
+// Sum over groups of 8 adjacent lanes; every lane of the group ends with the group total.
+__device__ __forceinline__ float oct_sum(float v) {
+    v += dpp_f32<OJK_DPP_QUAD_XOR1>(v);
+    v += dpp_f32<OJK_DPP_QUAD_XOR2>(v);
+    v += dpp_f32<OJK_DPP_ROW_HALF_MIRROR>(v);
+    return v;
+}
+// Sum over all 64 lanes; the total is returned in every lane (as a wave-uniform value).
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return (a + b) + (c + d);
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_f32<OJK_DPP_QUAD_XOR1>(v));
+    v = fmaxf(v, dpp_f32<OJK_DPP_QUAD_XOR2>(v));
+    v = fmaxf(v, dpp_f32<OJK_DPP_ROW_HALF_MIRROR>(v));
+    v = fmaxf(v, dpp_f32<OJK_DPP_ROW_MIRROR>(v));
+    float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+__device__ __forceinline__ int wave_sum_i32(int v) {
+    v += dpp_i32<OJK_DPP_QUAD_XOR1>(v);
+    v += dpp_i32<OJK_DPP_QUAD_XOR2>(v);
+    v += dpp_i32<OJK_DPP_ROW_HALF_MIRROR>(v);
+    v += dpp_i32<OJK_DPP_ROW_MIRROR>(v);
+    return __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) +
+           __builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48);
+}
+
+// 4 x (i8 * i8) + acc on v_dot4_i32_i8.
+__device__ __forceinline__ int dot4_i8(uint a, uint b, int acc) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, acc, false);
+}
+
+// ---- Q4_K scale / min unpack ---------------------------------------------------------------
+// The 12 scale bytes of a Q4_K / Q5_K super-block as three dwords (s0 = bytes 0..3, s1 = 4..7,
+// s2 = 8..11).  Returns, for the sub-block pair (2c, 2c+1), the two 6-bit scales in bytes 0/1 of
+// `sc` and the two 6-bit mins in bytes 0/1 of `mn`
+// (reference: get_scale_min_k4, crates/ojas-formats/src/gguf.rs:1132-1140).
+__device__ __forceinline__ void q4k_scale_min_pair(uint s0, uint s1, uint s2, uint c, uint& sc, uint& mn) {
+    uint sh = (c & 1u) * 16u;
+    uint y = s0 >> sh, z = s1 >> sh, w = s2 >> sh;
+    uint sc_lo = y & 0x3F3Fu, mn_lo = z & 0x3F3Fu;
+    uint sc_hi = (w & 0x0F0Fu) | ((y >> 2) & 0x3030u);
+    uint mn_hi = ((w >> 4) & 0x0F0Fu) | ((z >> 2) & 0x3030u);
+    sc = c < 2u ? sc_lo : sc_hi;
+    mn = c < 2u ? mn_lo : mn_hi;
+}

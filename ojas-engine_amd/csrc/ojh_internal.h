@@ -1,0 +1,85 @@
+// Internal declarations shared by the host-side translation units of libojas_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/ojas_hip.h"
+
+struct ojh_buf {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+    bool owned = false;
+};
+
+struct ojh_lin {
+    uint32_t type = 0, n = 0, k = 0;
+    size_t row_bytes = 0;
+    ojh_buf *raw = nullptr;  // block bytes
+    size_t off = 0;
+    bool owns_raw = false;
+};
+
+// Scratch the op-level entry points keep per device (quantized activations, MoE staging).
+struct ojh_scratch {
+    ojh_buf *buf = nullptr;
+};
+
+struct ojh_device {
+    int ordinal = 0;
+    hipStream_t stream = nullptr;
+    hipDeviceProp_t prop{};
+    std::string name;
+    std::map<std::string, hipModule_t> modules;      // family -> code object
+    std::map<std::string, hipFunction_t> functions;  // entry name -> function
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::vector<hipEvent_t> marks;  // lazily created, indexed by slot
+    // named scratch buffers, grown on demand
+    std::map<std::string, ojh_buf *> scratch;
+    int gemv_rows_override = 0;  // OJAS_HIP_GEMV_R
+};
+
+// ---- errors ------------------------------------------------------------------------------------
+int ojh_fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+#define OJH_HIP(call)                                                                              \
+    do {                                                                                           \
+        hipError_t e_ = (call);                                                                    \
+        if (e_ != hipSuccess)                                                                      \
+            return ojh_fail(OJH_ERR_HIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_),   \
+                            __FILE__, __LINE__);                                                   \
+    } while (0)
+
+// ---- manifest ----------------------------------------------------------------------------------
+struct ojh_block_format {
+    uint32_t type, bytes, weights;
+    const char *tag;
+};
+const ojh_block_format *ojh_format(uint32_t ggml_type);
+
+// What a kernel touches at given constants. Returns OJH_OK or fails with a message.
+typedef int (*ojh_check_fn)(const struct ojh_kernel_spec *spec, const uint32_t *consts,
+                            const uint32_t grid[3], const uint32_t block[3], size_t need[8],
+                            size_t align[8]);
+typedef int (*ojh_shape_fn)(const struct ojh_kernel_spec *spec, const ojh_device *dev, uint32_t K,
+                            uint32_t N, uint32_t M, uint32_t grid[3], uint32_t block[3]);
+
+struct ojh_kernel_spec {
+    const char *name;
+    const char *family;
+    int n_bufs, n_consts;
+    uint32_t type;       // GGUF type the kernel reads, 0 if none
+    int rows_per_wave;   // for the row-parallel matvecs
+    ojh_check_fn check;
+    ojh_shape_fn shape;
+};
+const std::vector<ojh_kernel_spec> &ojh_manifest_table();
+const ojh_kernel_spec *ojh_find_kernel(const char *name);
+
+// ---- helpers -----------------------------------------------------------------------------------
+int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out);
+int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptrs,
+               const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);

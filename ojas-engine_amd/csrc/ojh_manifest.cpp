@@ -1,0 +1,268 @@
+// Kernel manifest: one row per canonical entry name, with the family (code object) that defines
+// it, its positional signature (buffers first, then u32 constants — the convention the
+// reference enforces in crates/ojas-cuda/tests/conformance.rs:85-109), the bytes each buffer
+// must hold at given constants, and the wave64 launch shape.  The reference keeps the
+// equivalent tables in crates/ojas-core/src/quant_src.rs:83-111 (FORMATS) and :168-193
+// (MOE_FORMATS), and the name -> family registry in crates/ojas-cuda/src/kernels/mod.rs:111-145.
+#include <cstring>
+#include <deque>
+
+#include "ojh_internal.h"
+
+static const ojh_block_format kFormats[] = {
+    {OJH_Q8_0, 34, 32, "q80"},
+    {OJH_Q4_K, 144, 256, "q4k"},
+    {OJH_Q5_K, 176, 256, "q5k"},
+    {OJH_Q6_K, 210, 256, "q6k"},
+};
+
+const ojh_block_format *ojh_format(uint32_t t) {
+    for (const auto &f : kFormats)
+        if (f.type == t) return &f;
+    return nullptr;
+}
+
+size_t ojh_row_bytes(uint32_t ggml_type, uint32_t k) {
+    const ojh_block_format *f = ojh_format(ggml_type);
+    if (!f || k == 0 || k % f->weights) return 0;
+    return (size_t)(k / f->weights) * f->bytes;
+}
+
+// A check fills need[i] = bytes buffer i must hold from its offset, and may lower align[i], the
+// alignment (pointer + offset) must have (16 unless the kernel reads the buffer with narrower
+// loads).
+
+static int check_block(const uint32_t block[3], uint32_t exact) {
+    if (block[1] != 1 || block[2] != 1) return ojh_fail(OJH_ERR_ARG, "block must be [x,1,1]");
+    if (exact) {
+        if (block[0] != exact) return ojh_fail(OJH_ERR_ARG, "block.x must be %u, got %u", exact, block[0]);
+    } else if (block[0] == 0 || block[0] % 64 || block[0] > 256) {
+        return ojh_fail(OJH_ERR_ARG, "block.x must be a multiple of 64 up to 256, got %u", block[0]);
+    }
+    return OJH_OK;
+}
+
+static int check_kn(const ojh_kernel_spec *s, uint32_t K, uint32_t N, const ojh_block_format **fmt) {
+    const ojh_block_format *f = ojh_format(s->type);
+    if (!f) return ojh_fail(OJH_ERR_ARG, "%s: no block format", s->name);
+    if (K == 0 || N == 0 || K % f->weights)
+        return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a positive multiple of %u and N=%u positive",
+                        s->name, K, f->weights, N);
+    *fmt = f;
+    return OJH_OK;
+}
+
+// gemv_nat_<fmt>{,_accum,_bias,_rN}(x, w, y[, bs], K, N)
+static int check_gemv_nat(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                          const uint32_t block[3], size_t need[8], size_t align[8]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], N = c[1];
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if ((rc = check_block(block, 0))) return rc;
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    uint64_t cover = (uint64_t)grid[0] * (block[0] / 64) * s->rows_per_wave;
+    if (cover < N) return ojh_fail(OJH_ERR_ARG, "%s: grid covers %llu rows of N=%u", s->name,
+                                   (unsigned long long)cover, N);
+    need[0] = (size_t)K * 4;
+    need[1] = (size_t)N * (K / f->weights) * f->bytes;
+    need[2] = (size_t)N * 4;
+    if (s->n_bufs == 4) need[3] = (size_t)N * 4;
+    align[1] = f->bytes % 16 ? 2 : 16;
+    align[2] = align[3] = 4;
+    return OJH_OK;
+}
+
+// gemv_q8k_<fmt>{,_accum,_bias,_rN}(xq, xs, w, y[, bs], K, N)
+static int check_gemv_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                          const uint32_t block[3], size_t need[8], size_t align[8]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], N = c[1];
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if ((rc = check_block(block, 0))) return rc;
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    uint64_t cover = (uint64_t)grid[0] * (block[0] / 64) * s->rows_per_wave;
+    if (cover < N) return ojh_fail(OJH_ERR_ARG, "%s: grid covers %llu rows of N=%u", s->name,
+                                   (unsigned long long)cover, N);
+    need[0] = (size_t)K;
+    need[1] = (size_t)(K / 256) * 4;
+    need[2] = (size_t)N * (K / f->weights) * f->bytes;
+    need[3] = (size_t)N * 4;
+    if (s->n_bufs == 5) need[4] = (size_t)N * 4;
+    align[1] = 4;
+    align[2] = f->bytes % 16 ? 2 : 16;
+    align[3] = align[4] = 4;
+    return OJH_OK;
+}
+
+// gemv_nat_<fmt>_m(x, w, y, K, N, M, ACC)
+static int check_gemv_nat_m(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                            const uint32_t block[3], size_t need[8], size_t align[8]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], N = c[1], M = c[2];
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if (M == 0) return ojh_fail(OJH_ERR_ARG, "%s: M must be positive", s->name);
+    if ((rc = check_block(block, 0))) return rc;
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    if ((uint64_t)grid[0] * (block[0] / 64) < N)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover N=%u rows", s->name, N);
+    need[0] = (size_t)M * K * 4;
+    need[1] = (size_t)N * (K / f->weights) * f->bytes;
+    need[2] = (size_t)M * N * 4;
+    align[1] = f->bytes % 16 ? 2 : 16;
+    align[2] = 4;
+    return OJH_OK;
+}
+
+// gemv_q8k_<fmt>_m(xq, xs, w, y, K, N, M, ACC)
+static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                            const uint32_t block[3], size_t need[8], size_t align[8]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], N = c[1], M = c[2];
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if (M == 0) return ojh_fail(OJH_ERR_ARG, "%s: M must be positive", s->name);
+    if ((rc = check_block(block, 0))) return rc;
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    if ((uint64_t)grid[0] * (block[0] / 64) < N)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover N=%u rows", s->name, N);
+    need[0] = (size_t)M * K;
+    need[1] = (size_t)M * (K / 256) * 4;
+    need[2] = (size_t)N * (K / f->weights) * f->bytes;
+    need[3] = (size_t)M * N * 4;
+    align[1] = 4;
+    align[2] = f->bytes % 16 ? 2 : 16;
+    align[3] = 4;
+    return OJH_OK;
+}
+
+// quantize_q8k{,_bf16}(x, q, scales, K, M)
+static int check_quantize(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                          const uint32_t block[3], size_t need[8], size_t align[8]) {
+    uint32_t K = c[0], M = c[1];
+    if (K == 0 || M == 0) return ojh_fail(OJH_ERR_ARG, "%s: K and M must be positive", s->name);
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    uint32_t nsb = (K + 255) / 256;
+    if (grid[0] != nsb || grid[1] != M || grid[2] != 1)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,1]", s->name, nsb, M);
+    size_t esz = strstr(s->name, "bf16") ? 2 : 4;
+    need[0] = (size_t)M * K * esz;
+    need[1] = (size_t)M * nsb * 256;
+    need[2] = (size_t)M * nsb * 4;
+    align[0] = esz;
+    align[2] = 4;
+    return OJH_OK;
+}
+
+// dequant_<fmt>_f16(w, out, nblocks)
+static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                         const uint32_t block[3], size_t need[8], size_t align[8]) {
+    const ojh_block_format *f = ojh_format(s->type);
+    uint32_t nb = c[0];
+    if (!f || nb == 0) return ojh_fail(OJH_ERR_ARG, "%s: nblocks must be positive", s->name);
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    uint32_t tpb = s->type == OJH_Q6_K ? 64 : 32;  // threads per block of the format
+    if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * 256 < (uint64_t)nb * tpb)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover %u blocks", s->name, nb);
+    need[0] = (size_t)nb * f->bytes;
+    need[1] = (size_t)nb * f->weights * 2;
+    align[0] = f->bytes % 16 ? 2 : 16;
+    align[1] = 8;
+    return OJH_OK;
+}
+
+// ---- launch shapes ---------------------------------------------------------------------------
+static int shape_rows(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t,
+                      uint32_t grid[3], uint32_t block[3]) {
+    uint32_t rows_per_block = 4u * (uint32_t)s->rows_per_wave;
+    grid[0] = (N + rows_per_block - 1) / rows_per_block;
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+static int shape_quantize(const ojh_kernel_spec *, const ojh_device *, uint32_t K, uint32_t, uint32_t M,
+                          uint32_t grid[3], uint32_t block[3]) {
+    grid[0] = (K + 255) / 256;
+    grid[1] = M ? M : 1;
+    grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+// dequant: N is the number of blocks
+static int shape_dequant(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t,
+                         uint32_t grid[3], uint32_t block[3]) {
+    uint32_t tpb = s->type == OJH_Q6_K ? 64 : 32;
+    grid[0] = (uint32_t)(((uint64_t)N * tpb + 255) / 256);
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
+static std::vector<ojh_kernel_spec> build_manifest() {
+    std::vector<ojh_kernel_spec> m;
+    // `names` must outlive the table: keep them in a static pool.
+    static std::deque<std::string> pool;
+    auto add = [&](const std::string &name, const char *family, int nb, int nc, uint32_t type, int rpw,
+                   ojh_check_fn chk, ojh_shape_fn shp) {
+        pool.push_back(name);
+        m.push_back({pool.back().c_str(), family, nb, nc, type, rpw, chk, shp});
+    };
+    for (const auto &f : kFormats) {
+        std::string t = f.tag;
+        add("dequant_" + t + "_f16", "dequant", 2, 1, f.type, 0, check_dequant, shape_dequant);
+        if (f.type == OJH_Q5_K) continue;  // Q5_K: decoder only
+        std::string g = "gemv_nat_" + t;
+        add(g, "gemv", 3, 2, f.type, 4, check_gemv_nat, shape_rows);
+        add(g + "_r1", "gemv", 3, 2, f.type, 1, check_gemv_nat, shape_rows);
+        add(g + "_r2", "gemv", 3, 2, f.type, 2, check_gemv_nat, shape_rows);
+        add(g + "_accum", "gemv", 3, 2, f.type, 4, check_gemv_nat, shape_rows);
+        add(g + "_bias", "gemv", 4, 2, f.type, 4, check_gemv_nat, shape_rows);
+        add(g + "_m", "gemv", 3, 4, f.type, 1, check_gemv_nat_m, shape_rows);
+        if (f.type == OJH_Q8_0) continue;  // the CPU path keeps f32 activations for Q8_0
+        std::string q = "gemv_q8k_" + t;
+        add(q, "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
+        add(q + "_r1", "gemv_q8k", 4, 2, f.type, 1, check_gemv_q8k, shape_rows);
+        add(q + "_r2", "gemv_q8k", 4, 2, f.type, 2, check_gemv_q8k, shape_rows);
+        add(q + "_accum", "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
+        add(q + "_bias", "gemv_q8k", 5, 2, f.type, 4, check_gemv_q8k, shape_rows);
+        add(q + "_m", "gemv_q8k", 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
+    }
+    add("quantize_q8k", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
+    add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
+    return m;
+}
+
+const std::vector<ojh_kernel_spec> &ojh_manifest_table() {
+    static const std::vector<ojh_kernel_spec> table = build_manifest();
+    return table;
+}
+
+const ojh_kernel_spec *ojh_find_kernel(const char *name) {
+    if (!name) return nullptr;
+    for (const auto &s : ojh_manifest_table())
+        if (!strcmp(s.name, name)) return &s;
+    return nullptr;
+}
+
+extern "C" const char *ojh_kernel_family(const char *name) {
+    const ojh_kernel_spec *s = ojh_find_kernel(name);
+    return s ? s->family : nullptr;
+}
+
+extern "C" int ojh_manifest(int i, const char **name, const char **family, int *n_bufs, int *n_consts) {
+    const auto &t = ojh_manifest_table();
+    if (i >= 0 && i < (int)t.size()) {
+        if (name) *name = t[i].name;
+        if (family) *family = t[i].family;
+        if (n_bufs) *n_bufs = t[i].n_bufs;
+        if (n_consts) *n_consts = t[i].n_consts;
+    }
+    return (int)t.size();
+}

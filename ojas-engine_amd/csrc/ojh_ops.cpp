@@ -1,0 +1,226 @@
+// Host side of the op seam: weight handles that keep GGUF block bytes in place, and the matmul
+// router that picks a kernel per call — the role `Lin::load` and `CudaSsm::mm` play in the
+// reference (crates/ojas-cuda/src/qwen35.rs:174-201, :644-702; Metal twin
+// crates/ojas-models/src/decoder/dispatch.rs:288-626).
+#include <cstring>
+
+#include "ojh_internal.h"
+
+static int ensure(ojh_device *dev, const char *family) {
+    return dev->modules.count(family) ? OJH_OK : ojh_ensure_family(dev, family);
+}
+
+static int span_ok(const char *what, const ojh_buf *b, size_t off, size_t bytes, size_t align) {
+    if (!b) return ojh_fail(OJH_ERR_ARG, "%s: NULL buffer", what);
+    if (off > b->bytes || bytes > b->bytes - off)
+        return ojh_fail(OJH_ERR_BOUNDS, "%s needs %zu bytes at offset %zu, buffer has %zu", what, bytes, off,
+                        b->bytes);
+    if (((uintptr_t)b->ptr + off) % align)
+        return ojh_fail(OJH_ERR_ARG, "%s (+%zu) must be %zu-byte aligned", what, off, align);
+    return OJH_OK;
+}
+
+static inline void *at(const ojh_buf *b, size_t off) { return (char *)b->ptr + off; }
+
+// ---- Lin ---------------------------------------------------------------------------------------
+static int lin_check(uint32_t type, uint32_t n, uint32_t k, size_t *row_bytes) {
+    const ojh_block_format *f = ojh_format(type);
+    if (!f) return ojh_fail(OJH_ERR_UNSUPPORTED, "GGUF type %u has no kernel on this backend", type);
+    if (!n || !k || k % f->weights)
+        return ojh_fail(OJH_ERR_ARG, "Lin %ux%u: K must be a positive multiple of %u for %s", n, k, f->weights,
+                        f->tag);
+    *row_bytes = (size_t)(k / f->weights) * f->bytes;
+    return OJH_OK;
+}
+
+extern "C" int ojh_lin_create(ojh_device *dev, uint32_t type, uint32_t n, uint32_t k, const void *raw,
+                              ojh_lin **out) {
+    if (!dev || !raw || !out) return ojh_fail(OJH_ERR_ARG, "ojh_lin_create: NULL argument");
+    *out = nullptr;
+    size_t rb;
+    int rc = lin_check(type, n, k, &rb);
+    if (rc) return rc;
+    ojh_buf *buf = nullptr;
+    if ((rc = ojh_alloc(dev, rb * n, &buf))) return rc;
+    if ((rc = ojh_upload(dev, buf, 0, raw, rb * n))) {
+        ojh_free(dev, buf);
+        return rc;
+    }
+    ojh_lin *l = new ojh_lin();
+    l->type = type; l->n = n; l->k = k; l->row_bytes = rb; l->raw = buf; l->off = 0; l->owns_raw = true;
+    *out = l;
+    return OJH_OK;
+}
+
+extern "C" int ojh_lin_wrap(ojh_device *dev, uint32_t type, uint32_t n, uint32_t k, ojh_buf *raw, size_t off,
+                            ojh_lin **out) {
+    if (!dev || !raw || !out) return ojh_fail(OJH_ERR_ARG, "ojh_lin_wrap: NULL argument");
+    *out = nullptr;
+    size_t rb;
+    int rc = lin_check(type, n, k, &rb);
+    if (rc) return rc;
+    const ojh_block_format *f = ojh_format(type);
+    if ((rc = span_ok("ojh_lin_wrap: raw", raw, off, rb * n, f->bytes % 16 ? 2 : 16))) return rc;
+    ojh_lin *l = new ojh_lin();
+    l->type = type; l->n = n; l->k = k; l->row_bytes = rb; l->raw = raw; l->off = off; l->owns_raw = false;
+    *out = l;
+    return OJH_OK;
+}
+
+extern "C" int ojh_lin_free(ojh_device *dev, ojh_lin *lin) {
+    if (!lin) return OJH_OK;
+    int rc = OJH_OK;
+    if (lin->owns_raw) rc = ojh_free(dev, lin->raw);
+    delete lin;
+    return rc;
+}
+
+// ---- dequant -----------------------------------------------------------------------------------
+extern "C" int ojh_dequant_f16(ojh_device *dev, uint32_t type, const ojh_buf *raw, size_t raw_off,
+                               size_t n_weights, ojh_buf *out, size_t out_off) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_dequant_f16: NULL device");
+    const ojh_block_format *f = ojh_format(type);
+    if (!f) return ojh_fail(OJH_ERR_UNSUPPORTED, "GGUF type %u has no decoder on this backend", type);
+    if (!n_weights || n_weights % f->weights)
+        return ojh_fail(OJH_ERR_ARG, "dequant: %zu weights is not a positive multiple of %u", n_weights, f->weights);
+    size_t nb = n_weights / f->weights;
+    if (nb > 0x7FFFFFFFu / 64) return ojh_fail(OJH_ERR_ARG, "dequant: too many blocks in one call (%zu)", nb);
+    int rc;
+    if ((rc = span_ok("dequant: raw", raw, raw_off, nb * f->bytes, f->bytes % 16 ? 2 : 16))) return rc;
+    if ((rc = span_ok("dequant: out", out, out_off, n_weights * 2, 2))) return rc;
+    if ((rc = ensure(dev, "dequant"))) return rc;
+    std::string name = std::string("dequant_") + f->tag + "_f16";
+    uint32_t grid[3], block[3];
+    if ((rc = ojh_launch_shape(dev, name.c_str(), 0, (uint32_t)nb, 0, grid, block))) return rc;
+    return ojh_launch(dev, name.c_str(), {at(raw, raw_off), at(out, out_off)}, {(uint32_t)nb}, grid, block);
+}
+
+// ---- activation quantizer ----------------------------------------------------------------------
+static int quant_q8k_launch(ojh_device *dev, const void *x, int x_dtype, uint32_t m, uint32_t k, void *q,
+                            void *scales) {
+    const char *name = x_dtype == OJH_X_BF16 ? "quantize_q8k_bf16" : "quantize_q8k";
+    uint32_t grid[3] = {(k + 255) / 256, m, 1}, block[3] = {256, 1, 1};
+    return ojh_launch(dev, name, {(void *)x, q, scales}, {k, m}, grid, block);
+}
+
+extern "C" int ojh_quant_q8k(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, uint32_t m,
+                             uint32_t k, ojh_buf *q, ojh_buf *scales) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_quant_q8k: NULL device");
+    if (x_dtype != OJH_X_F32 && x_dtype != OJH_X_BF16)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "quant_q8k takes f32 or bf16 activations");
+    if (!m || !k || m > 65535) return ojh_fail(OJH_ERR_ARG, "quant_q8k: m=%u k=%u out of range", m, k);
+    size_t esz = x_dtype == OJH_X_BF16 ? 2 : 4, nsb = (k + 255) / 256;
+    int rc;
+    if ((rc = span_ok("quant_q8k: x", x, x_off, (size_t)m * k * esz, esz))) return rc;
+    if ((rc = span_ok("quant_q8k: q", q, 0, (size_t)m * nsb * 256, 16))) return rc;
+    if ((rc = span_ok("quant_q8k: scales", scales, 0, (size_t)m * nsb * 4, 4))) return rc;
+    if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+    return quant_q8k_launch(dev, at(x, x_off), x_dtype, m, k, q->ptr, scales->ptr);
+}
+
+// ---- mm ----------------------------------------------------------------------------------------
+// Rows per wave for the row-parallel matvecs: enough waves to put several on every SIMD, while
+// reusing each activation fragment across as many rows as that allows.
+static int pick_rows(const ojh_device *dev, uint32_t n) {
+    if (dev->gemv_rows_override == 1 || dev->gemv_rows_override == 2 || dev->gemv_rows_override == 4)
+        return dev->gemv_rows_override;
+    uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;
+    uint32_t want_waves = cus * 8;  // two per SIMD
+    if (n / 4 >= want_waves) return 4;
+    if (n / 2 >= want_waves) return 2;
+    return 1;
+}
+
+// y (=,+=,+bias) quantized-x . W^T for K-quant weights: the matvec (m = 1) and its batched form.
+static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, const ojh_block_format *f, void *yp,
+                         const ojh_buf *bias, uint32_t m, int accum) {
+    const uint32_t K = w->k, N = w->n;
+    void *wp = at(w->raw, w->off);
+    uint32_t grid[3] = {1, 1, 1}, block[3] = {256, 1, 1};
+    std::string base = std::string("gemv_q8k_") + f->tag;
+    if (m == 1) {
+        int r = (accum || bias) ? 4 : pick_rows(dev, N);
+        std::string name = base + (accum ? "_accum" : bias ? "_bias" : r == 4 ? "" : r == 2 ? "_r2" : "_r1");
+        grid[0] = (N + 4 * r - 1) / (4 * r);
+        std::vector<void *> p = {xq, xs, wp, yp};
+        if (bias) p.push_back(bias->ptr);
+        return ojh_launch(dev, name.c_str(), p, {K, N}, grid, block);
+    }
+    grid[0] = (N + 3) / 4;
+    return ojh_launch(dev, (base + "_m").c_str(), {xq, xs, wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, grid, block);
+}
+
+static int mm_common_checks(const char *who, const ojh_lin *w, ojh_buf *y, size_t y_off, const ojh_buf *bias,
+                            uint32_t m, int accum, const ojh_block_format **fmt) {
+    if (!w) return ojh_fail(OJH_ERR_ARG, "%s: NULL weights", who);
+    if (!m || m > 65535) return ojh_fail(OJH_ERR_ARG, "%s: m=%u out of range", who, m);
+    const ojh_block_format *f = ojh_format(w->type);
+    if (!f) return ojh_fail(OJH_ERR_UNSUPPORTED, "%s: GGUF type %u", who, w->type);
+    if (bias && accum) return ojh_fail(OJH_ERR_UNSUPPORTED, "%s: bias and accum together", who);
+    if (bias && m != 1) return ojh_fail(OJH_ERR_UNSUPPORTED, "%s: bias is a matvec (m=1) epilogue", who);
+    int rc;
+    if ((rc = span_ok("y", y, y_off, (size_t)m * w->n * 4, 4))) return rc;
+    if (bias && (rc = span_ok("bias", bias, 0, (size_t)w->n * 4, 4))) return rc;
+    if ((rc = span_ok("w", w->raw, w->off, w->row_bytes * w->n, f->bytes % 16 ? 2 : 16))) return rc;
+    *fmt = f;
+    return OJH_OK;
+}
+
+extern "C" int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const ojh_lin *w, ojh_buf *y,
+                          size_t y_off, const ojh_buf *bias, uint32_t m, int accum) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_mm_q8k: NULL device");
+    const ojh_block_format *f;
+    int rc = mm_common_checks("ojh_mm_q8k", w, y, y_off, bias, m, accum, &f);
+    if (rc) return rc;
+    if (w->type == OJH_Q8_0)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm_q8k: Q8_0 rows take f32 activations, as dot_q80 does");
+    size_t nsb = w->k / 256;
+    if ((rc = span_ok("xq", xq, 0, (size_t)m * nsb * 256, 16))) return rc;
+    if ((rc = span_ok("xscales", xscales, 0, (size_t)m * nsb * 4, 4))) return rc;
+    if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+    return mm_q8k_launch(dev, xq->ptr, xscales->ptr, w, f, at(y, y_off), bias, m, accum);
+}
+
+extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, const ojh_lin *w, ojh_buf *y,
+                      size_t y_off, const ojh_buf *bias, uint32_t m, int accum, int act_mode) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_mm: NULL device");
+    const ojh_block_format *f;
+    int rc = mm_common_checks("ojh_mm", w, y, y_off, bias, m, accum, &f);
+    if (rc) return rc;
+    if (x_dtype != OJH_X_F32 && x_dtype != OJH_X_BF16)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: activations must be f32 or bf16");
+    const uint32_t K = w->k, N = w->n;
+    size_t esz = x_dtype == OJH_X_BF16 ? 2 : 4;
+    if ((rc = span_ok("ojh_mm: x", x, x_off, (size_t)m * K * esz, 16))) return rc;
+
+    bool q8k = w->type != OJH_Q8_0 && act_mode != OJH_ACT_FLOAT;
+    void *wp = at(w->raw, w->off), *yp = at(y, y_off);
+    uint32_t grid[3] = {1, 1, 1}, block[3] = {256, 1, 1};
+
+    if (q8k) {
+        if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+        size_t nsb = K / 256;
+        ojh_buf *xq, *xs;
+        if ((rc = ojh_scratch_get(dev, "xq", (size_t)m * nsb * 256, &xq))) return rc;
+        if ((rc = ojh_scratch_get(dev, "xs", (size_t)m * nsb * 4, &xs))) return rc;
+        if ((rc = quant_q8k_launch(dev, at(x, x_off), x_dtype, m, K, xq->ptr, xs->ptr))) return rc;
+        return mm_q8k_launch(dev, xq->ptr, xs->ptr, w, f, yp, bias, m, accum);
+    }
+
+    // floating-point activations
+    if (x_dtype != OJH_X_F32)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: the float matvec takes f32 activations");
+    if ((rc = ensure(dev, "gemv"))) return rc;
+    std::string base = std::string("gemv_nat_") + f->tag;
+    if (m == 1) {
+        int r = (accum || bias) ? 4 : pick_rows(dev, N);
+        std::string name = base + (accum ? "_accum" : bias ? "_bias" : r == 4 ? "" : r == 2 ? "_r2" : "_r1");
+        grid[0] = (N + 4 * r - 1) / (4 * r);
+        std::vector<void *> p = {at(x, x_off), wp, yp};
+        if (bias) p.push_back(bias->ptr);
+        return ojh_launch(dev, name.c_str(), p, {K, N}, grid, block);
+    }
+    grid[0] = (N + 3) / 4;
+    return ojh_launch(dev, (base + "_m").c_str(), {at(x, x_off), wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, grid,
+                      block);
+}

@@ -1,0 +1,341 @@
+// Host side of the kernel seam: device lifetime, buffers, family loading (hipModuleLoad of the
+// gfx950 code objects built offline), dispatch by canonical name, event timing.
+// Stands in for `CudaGpu: Device + KernelRuntime` (crates/ojas-cuda/src/device.rs:91-166,
+// :341-537) — same obligations (names resolve in exactly one family, unknown kernel is an error
+// that says "ensure_family first", read synchronises), none of its code.
+#include <dlfcn.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "ojh_internal.h"
+
+static thread_local std::string g_last_error;
+
+int ojh_fail(int code, const char *fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+extern "C" const char *ojh_last_error(void) { return g_last_error.c_str(); }
+extern "C" int ojh_abi_version(void) { return OJH_ABI_VERSION; }
+
+// Directory holding <family>.hsaco: $OJAS_HIP_HSACO_DIR, else "hsaco" beside this library.
+static std::string hsaco_dir() {
+    if (const char *e = getenv("OJAS_HIP_HSACO_DIR")) return e;
+    Dl_info info;
+    if (dladdr((const void *)&ojh_abi_version, &info) && info.dli_fname) {
+        std::string p = info.dli_fname;
+        size_t s = p.find_last_of('/');
+        return (s == std::string::npos ? std::string(".") : p.substr(0, s)) + "/hsaco";
+    }
+    return "hsaco";
+}
+
+extern "C" int ojh_open(int ordinal, ojh_device **out) {
+    if (!out) return ojh_fail(OJH_ERR_ARG, "ojh_open: out is NULL");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0)
+        return ojh_fail(OJH_ERR_NO_DEVICE, "no HIP device visible (%s); this backend has no CPU fallback",
+                        e == hipSuccess ? "count=0" : hipGetErrorString(e));
+    if (ordinal < 0 || ordinal >= count)
+        return ojh_fail(OJH_ERR_ARG, "device ordinal %d out of range (0..%d)", ordinal, count - 1);
+    OJH_HIP(hipSetDevice(ordinal));
+    ojh_device *d = new ojh_device();
+    d->ordinal = ordinal;
+    e = hipGetDeviceProperties(&d->prop, ordinal);
+    if (e != hipSuccess) {
+        delete d;
+        return ojh_fail(OJH_ERR_HIP, "hipGetDeviceProperties: %s", hipGetErrorString(e));
+    }
+    if (strncmp(d->prop.gcnArchName, "gfx950", 6) != 0 && !getenv("OJAS_HIP_ANY_ARCH")) {
+        std::string arch = d->prop.gcnArchName;
+        delete d;
+        return ojh_fail(OJH_ERR_NO_DEVICE, "device %d is %s; the code objects are built for gfx950 only",
+                        ordinal, arch.c_str());
+    }
+    e = hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&d->ev0);
+    if (e == hipSuccess) e = hipEventCreate(&d->ev1);
+    if (e != hipSuccess) {
+        delete d;
+        return ojh_fail(OJH_ERR_HIP, "stream/event creation: %s", hipGetErrorString(e));
+    }
+    d->name = std::string("hip:") + d->prop.name + " (" + d->prop.gcnArchName + ")";
+    if (const char *r = getenv("OJAS_HIP_GEMV_R")) d->gemv_rows_override = atoi(r);
+    *out = d;
+    return OJH_OK;
+}
+
+extern "C" int ojh_close(ojh_device *dev) {
+    if (!dev) return OJH_OK;
+    hipSetDevice(dev->ordinal);
+    hipStreamSynchronize(dev->stream);
+    for (auto &kv : dev->scratch) {
+        if (kv.second) {
+            if (kv.second->owned) hipFree(kv.second->ptr);
+            delete kv.second;
+        }
+    }
+    for (auto &kv : dev->modules) hipModuleUnload(kv.second);
+    for (auto e : dev->marks)
+        if (e) hipEventDestroy(e);
+    if (dev->ev0) hipEventDestroy(dev->ev0);
+    if (dev->ev1) hipEventDestroy(dev->ev1);
+    if (dev->stream) hipStreamDestroy(dev->stream);
+    delete dev;
+    return OJH_OK;
+}
+
+extern "C" const char *ojh_name(const ojh_device *dev) { return dev ? dev->name.c_str() : ""; }
+
+extern "C" int ojh_caps_get(const ojh_device *dev, ojh_caps *out) {
+    if (!dev || !out) return ojh_fail(OJH_ERR_ARG, "ojh_caps_get: NULL argument");
+    memset(out, 0, sizeof *out);
+    out->tier = 2;  // matrix units
+    out->f16_compute = 1;
+    out->simd_width = (uint32_t)dev->prop.warpSize;
+    out->unified_memory = 0;
+    out->max_buffer = dev->prop.totalGlobalMem;
+    out->compute_units = (uint32_t)dev->prop.multiProcessorCount;
+    out->clock_mhz = (uint32_t)(dev->prop.clockRate / 1000);
+    out->total_memory = dev->prop.totalGlobalMem;
+    snprintf(out->arch, sizeof out->arch, "%s", dev->prop.gcnArchName);
+    out->features = "mfma_bf16,mfma_f16,mfma_i8,dot4_i8,wave64,offline_code_objects";
+    return OJH_OK;
+}
+
+// ---- buffers -----------------------------------------------------------------------------------
+extern "C" int ojh_alloc(ojh_device *dev, size_t bytes, ojh_buf **out) {
+    if (!dev || !out) return ojh_fail(OJH_ERR_ARG, "ojh_alloc: NULL argument");
+    *out = nullptr;
+    OJH_HIP(hipSetDevice(dev->ordinal));
+    void *p = nullptr;
+    OJH_HIP(hipMalloc(&p, bytes ? bytes : 1));
+    ojh_buf *b = new ojh_buf();
+    b->ptr = p;
+    b->bytes = bytes;
+    b->owned = true;
+    *out = b;
+    return OJH_OK;
+}
+
+extern "C" int ojh_wrap(ojh_device *dev, void *device_ptr, size_t bytes, ojh_buf **out) {
+    if (!dev || !out || !device_ptr) return ojh_fail(OJH_ERR_ARG, "ojh_wrap: NULL argument");
+    ojh_buf *b = new ojh_buf();
+    b->ptr = device_ptr;
+    b->bytes = bytes;
+    b->owned = false;
+    *out = b;
+    return OJH_OK;
+}
+
+extern "C" int ojh_free(ojh_device *dev, ojh_buf *buf) {
+    if (!buf) return OJH_OK;
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_free: NULL device");
+    if (buf->owned) {
+        // work queued on the stream may still read the buffer
+        OJH_HIP(hipStreamSynchronize(dev->stream));
+        OJH_HIP(hipFree(buf->ptr));
+    }
+    delete buf;
+    return OJH_OK;
+}
+
+extern "C" size_t ojh_buf_bytes(const ojh_buf *buf) { return buf ? buf->bytes : 0; }
+extern "C" void *ojh_buf_ptr(const ojh_buf *buf) { return buf ? buf->ptr : nullptr; }
+
+static int range_ok(const char *what, const ojh_buf *b, size_t off, size_t bytes) {
+    if (!b) return ojh_fail(OJH_ERR_ARG, "%s: NULL buffer", what);
+    if (off > b->bytes || bytes > b->bytes - off)
+        return ojh_fail(OJH_ERR_BOUNDS, "%s: [%zu, +%zu) exceeds the buffer's %zu bytes", what, off, bytes,
+                        b->bytes);
+    return OJH_OK;
+}
+
+extern "C" int ojh_upload(ojh_device *dev, ojh_buf *dst, size_t off, const void *host, size_t bytes) {
+    if (!dev || (!host && bytes)) return ojh_fail(OJH_ERR_ARG, "ojh_upload: NULL argument");
+    int rc = range_ok("ojh_upload", dst, off, bytes);
+    if (rc) return rc;
+    if (!bytes) return OJH_OK;
+    // Ordered after earlier work on the stream; returns when the host buffer has been consumed.
+    OJH_HIP(hipMemcpyAsync((char *)dst->ptr + off, host, bytes, hipMemcpyHostToDevice, dev->stream));
+    OJH_HIP(hipStreamSynchronize(dev->stream));
+    return OJH_OK;
+}
+
+extern "C" int ojh_download(ojh_device *dev, const ojh_buf *src, size_t off, void *host, size_t bytes) {
+    if (!dev || (!host && bytes)) return ojh_fail(OJH_ERR_ARG, "ojh_download: NULL argument");
+    int rc = range_ok("ojh_download", src, off, bytes);
+    if (rc) return rc;
+    if (!bytes) return OJH_OK;
+    OJH_HIP(hipMemcpyAsync(host, (const char *)src->ptr + off, bytes, hipMemcpyDeviceToHost, dev->stream));
+    OJH_HIP(hipStreamSynchronize(dev->stream));
+    return OJH_OK;
+}
+
+extern "C" int ojh_memset0(ojh_device *dev, ojh_buf *dst, size_t off, size_t bytes) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_memset0: NULL device");
+    int rc = range_ok("ojh_memset0", dst, off, bytes);
+    if (rc) return rc;
+    if (!bytes) return OJH_OK;
+    OJH_HIP(hipMemsetAsync((char *)dst->ptr + off, 0, bytes, dev->stream));
+    return OJH_OK;
+}
+
+int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out) {
+    ojh_buf *&slot = dev->scratch[name];
+    if (!slot || slot->bytes < bytes) {
+        if (slot) {
+            int rc = ojh_free(dev, slot);
+            slot = nullptr;
+            if (rc) return rc;
+        }
+        size_t cap = bytes < 4096 ? 4096 : bytes + bytes / 4;
+        int rc = ojh_alloc(dev, cap, &slot);
+        if (rc) return rc;
+    }
+    *out = slot;
+    return OJH_OK;
+}
+
+// ---- families ----------------------------------------------------------------------------------
+extern "C" int ojh_ensure_family(ojh_device *dev, const char *family) {
+    if (!dev || !family) return ojh_fail(OJH_ERR_ARG, "ojh_ensure_family: NULL argument");
+    if (dev->modules.count(family)) return OJH_OK;
+    bool known = false;
+    for (const auto &s : ojh_manifest_table())
+        if (!strcmp(s.family, family)) known = true;
+    if (!known) return ojh_fail(OJH_ERR_UNSUPPORTED, "unknown kernel family '%s'", family);
+    OJH_HIP(hipSetDevice(dev->ordinal));
+    std::string path = hsaco_dir() + "/" + family + ".hsaco";
+    hipModule_t mod = nullptr;
+    hipError_t e = hipModuleLoad(&mod, path.c_str());
+    if (e != hipSuccess)
+        return ojh_fail(OJH_ERR_HIP, "hipModuleLoad(%s): %s — build the code objects first", path.c_str(),
+                        hipGetErrorString(e));
+    // every manifest entry of the family must resolve: a name that drifted is a build error
+    std::map<std::string, hipFunction_t> found;
+    for (const auto &s : ojh_manifest_table()) {
+        if (strcmp(s.family, family)) continue;
+        hipFunction_t fn = nullptr;
+        e = hipModuleGetFunction(&fn, mod, s.name);
+        if (e != hipSuccess) {
+            hipModuleUnload(mod);
+            return ojh_fail(OJH_ERR_HIP, "family '%s' does not define kernel '%s': %s", family, s.name,
+                            hipGetErrorString(e));
+        }
+        found[s.name] = fn;
+    }
+    dev->modules[family] = mod;
+    for (auto &kv : found) dev->functions[kv.first] = kv.second;
+    return OJH_OK;
+}
+
+extern "C" int ojh_has_kernel(const ojh_device *dev, const char *name) {
+    return dev && name && dev->functions.count(name) ? 1 : 0;
+}
+
+extern "C" int ojh_launch_shape(const ojh_device *dev, const char *name, uint32_t K, uint32_t N, uint32_t M,
+                                uint32_t grid[3], uint32_t block[3]) {
+    const ojh_kernel_spec *s = ojh_find_kernel(name);
+    if (!s) return ojh_fail(OJH_ERR_UNSUPPORTED, "unknown kernel '%s'", name ? name : "(null)");
+    if (!grid || !block) return ojh_fail(OJH_ERR_ARG, "ojh_launch_shape: NULL output");
+    return s->shape(s, dev, K, N, M, grid, block);
+}
+
+int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptrs,
+               const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]) {
+    auto it = dev->functions.find(name);
+    if (it == dev->functions.end())
+        return ojh_fail(OJH_ERR_NOT_LOADED, "kernel '%s' not loaded — ensure_family first", name);
+    if (!grid[0] || !grid[1] || !grid[2] || !block[0] || !block[1] || !block[2])
+        return ojh_fail(OJH_ERR_ARG, "%s: empty grid or block", name);
+    std::vector<void *> p = ptrs;
+    std::vector<uint32_t> c = consts;
+    std::vector<void *> args;
+    args.reserve(p.size() + c.size());
+    for (auto &x : p) args.push_back(&x);
+    for (auto &x : c) args.push_back(&x);
+    OJH_HIP(hipModuleLaunchKernel(it->second, grid[0], grid[1], grid[2], block[0], block[1], block[2], 0,
+                                  dev->stream, args.data(), nullptr));
+    return OJH_OK;
+}
+
+extern "C" int ojh_dispatch(ojh_device *dev, const char *name, int n_bufs, ojh_buf *const *bufs,
+                            const uint64_t *offsets, int n_consts, const uint32_t *consts,
+                            const uint32_t grid[3], const uint32_t block[3]) {
+    if (!dev || !name || !grid || !block) return ojh_fail(OJH_ERR_ARG, "ojh_dispatch: NULL argument");
+    const ojh_kernel_spec *s = ojh_find_kernel(name);
+    if (!s) return ojh_fail(OJH_ERR_NOT_LOADED, "kernel '%s' not loaded — ensure_family first", name);
+    if (!dev->functions.count(name))
+        return ojh_fail(OJH_ERR_NOT_LOADED, "kernel '%s' not loaded — ensure_family(\"%s\") first", name,
+                        s->family);
+    if (n_bufs != s->n_bufs || n_consts != s->n_consts)
+        return ojh_fail(OJH_ERR_ARG, "%s takes %d buffers then %d constants, got %d and %d", name, s->n_bufs,
+                        s->n_consts, n_bufs, n_consts);
+    if ((n_bufs && !bufs) || (n_consts && !consts)) return ojh_fail(OJH_ERR_ARG, "%s: NULL argument array", name);
+    size_t need[8] = {0}, align[8];
+    for (auto &a : align) a = 16;
+    int rc = s->check(s, consts, grid, block, need, align);
+    if (rc) return rc;
+    std::vector<void *> ptrs;
+    for (int i = 0; i < n_bufs; i++) {
+        size_t off = offsets ? (size_t)offsets[i] : 0;
+        if (!bufs[i]) return ojh_fail(OJH_ERR_ARG, "%s: buffer %d is NULL", name, i);
+        if (off > bufs[i]->bytes || need[i] > bufs[i]->bytes - off)
+            return ojh_fail(OJH_ERR_BOUNDS, "%s: buffer %d needs %zu bytes at offset %zu, has %zu", name, i,
+                            need[i], off, bufs[i]->bytes);
+        uintptr_t addr = (uintptr_t)bufs[i]->ptr + off;
+        if (addr % align[i])
+            return ojh_fail(OJH_ERR_ARG, "%s: buffer %d (+%zu) must be %zu-byte aligned", name, i, off, align[i]);
+        ptrs.push_back((void *)addr);
+    }
+    return ojh_launch(dev, name, ptrs, std::vector<uint32_t>(consts, consts + n_consts), grid, block);
+}
+
+extern "C" int ojh_submit(ojh_device *dev) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_submit: NULL device");
+    OJH_HIP(hipStreamSynchronize(dev->stream));
+    return OJH_OK;
+}
+
+extern "C" int ojh_timer_start(ojh_device *dev) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_timer_start: NULL device");
+    OJH_HIP(hipEventRecord(dev->ev0, dev->stream));
+    return OJH_OK;
+}
+
+extern "C" int ojh_timer_stop(ojh_device *dev, float *elapsed_ms) {
+    if (!dev || !elapsed_ms) return ojh_fail(OJH_ERR_ARG, "ojh_timer_stop: NULL argument");
+    OJH_HIP(hipEventRecord(dev->ev1, dev->stream));
+    OJH_HIP(hipEventSynchronize(dev->ev1));
+    OJH_HIP(hipEventElapsedTime(elapsed_ms, dev->ev0, dev->ev1));
+    return OJH_OK;
+}
+
+extern "C" int ojh_mark(ojh_device *dev, int slot) {
+    if (!dev || slot < 0 || slot >= OJH_MAX_MARKS) return ojh_fail(OJH_ERR_ARG, "ojh_mark: slot %d out of range", slot);
+    if ((size_t)slot >= dev->marks.size()) dev->marks.resize((size_t)slot + 1, nullptr);
+    if (!dev->marks[slot]) OJH_HIP(hipEventCreate(&dev->marks[slot]));
+    OJH_HIP(hipEventRecord(dev->marks[slot], dev->stream));
+    return OJH_OK;
+}
+
+extern "C" int ojh_mark_elapsed(ojh_device *dev, int a, int b, float *elapsed_ms) {
+    if (!dev || !elapsed_ms) return ojh_fail(OJH_ERR_ARG, "ojh_mark_elapsed: NULL argument");
+    if (a < 0 || b < 0 || (size_t)a >= dev->marks.size() || (size_t)b >= dev->marks.size() || !dev->marks[a] ||
+        !dev->marks[b])
+        return ojh_fail(OJH_ERR_ARG, "ojh_mark_elapsed: slot %d or %d was never recorded", a, b);
+    OJH_HIP(hipEventSynchronize(dev->marks[b]));
+    OJH_HIP(hipEventElapsedTime(elapsed_ms, dev->marks[a], dev->marks[b]));
+    return OJH_OK;
+}

@@ -1,0 +1,354 @@
+"""Host-side mirror of the reference's kernel and op seams over the C ABI of libojas_hip.so.
+
+`HipGpu` has the shape of the reference's `Device` + `KernelRuntime` traits
+(crates/ojas-core/src/lib.rs:26-40, crates/ojas-core/src/kernel.rs:67-81; CUDA implementation
+crates/ojas-cuda/src/device.rs:418-537): `ensure_family`, `has_kernel`, `caps`, `begin`,
+`dispatch(enc, name, bufs, consts, grid, block)`, `submit`, `alloc`, `upload`, `read`.
+`Lin` / `HipGpu.mm` mirror `Lin::load` / `CudaSsm::mm` (crates/ojas-cuda/src/qwen35.rs:174-201,
+:644-702).
+
+Everything here binds the shared library with ctypes; there is no CPU implementation behind it.
+If the library or a GPU is missing the calls raise.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from dataclasses import dataclass
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libojas_hip.so")
+
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+X_F32, X_BF16, X_F16 = 0, 1, 2
+ACT_AUTO, ACT_Q8K, ACT_FLOAT = 0, 1, 2
+
+BLOCK_SHAPE = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
+
+
+class OjasHipError(RuntimeError):
+    def __init__(self, code: int, msg: str):
+        super().__init__(f"[{code}] {msg}")
+        self.code = code
+
+
+class _Caps(C.Structure):
+    _fields_ = [("tier", C.c_int32), ("f16_compute", C.c_int32), ("simd_width", C.c_uint32),
+                ("unified_memory", C.c_int32), ("max_buffer", C.c_uint64), ("compute_units", C.c_uint32),
+                ("clock_mhz", C.c_uint32), ("total_memory", C.c_uint64), ("arch", C.c_char * 32),
+                ("features", C.c_char_p)]
+
+
+@dataclass
+class Caps:
+    """Mirrors `Caps` (crates/ojas-core/src/kernel.rs:26-41)."""
+    tier: str
+    f16_compute: bool
+    simd_width: int
+    unified_memory: bool
+    max_buffer: int
+    compute_units: int
+    clock_mhz: int
+    arch: str
+    features: tuple
+
+    def has(self, feature: str) -> bool:
+        return feature in self.features
+
+
+_lib = None
+
+
+def load_library(path: str | None = None) -> C.CDLL:
+    """Load libojas_hip.so (built offline by build.py) and declare its signatures."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or LIB_PATH
+    if not os.path.exists(p):
+        raise FileNotFoundError(f"{p} is missing: build it with `python ojas-engine_amd/build.py`")
+    L = C.CDLL(p)
+    vp, sz, u32, i32, u64 = C.c_void_p, C.c_size_t, C.c_uint32, C.c_int, C.c_uint64
+    pp = C.POINTER(vp)
+    sig = {
+        "ojh_open": (i32, [i32, pp]),
+        "ojh_close": (i32, [vp]),
+        "ojh_name": (C.c_char_p, [vp]),
+        "ojh_caps_get": (i32, [vp, C.POINTER(_Caps)]),
+        "ojh_last_error": (C.c_char_p, []),
+        "ojh_abi_version": (i32, []),
+        "ojh_alloc": (i32, [vp, sz, pp]),
+        "ojh_free": (i32, [vp, vp]),
+        "ojh_wrap": (i32, [vp, vp, sz, pp]),
+        "ojh_buf_bytes": (sz, [vp]),
+        "ojh_buf_ptr": (vp, [vp]),
+        "ojh_upload": (i32, [vp, vp, sz, vp, sz]),
+        "ojh_download": (i32, [vp, vp, sz, vp, sz]),
+        "ojh_memset0": (i32, [vp, vp, sz, sz]),
+        "ojh_ensure_family": (i32, [vp, C.c_char_p]),
+        "ojh_has_kernel": (i32, [vp, C.c_char_p]),
+        "ojh_kernel_family": (C.c_char_p, [C.c_char_p]),
+        "ojh_manifest": (i32, [i32, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p), C.POINTER(i32), C.POINTER(i32)]),
+        "ojh_launch_shape": (i32, [vp, C.c_char_p, u32, u32, u32, C.POINTER(u32), C.POINTER(u32)]),
+        "ojh_dispatch": (i32, [vp, C.c_char_p, i32, pp, C.POINTER(u64), i32, C.POINTER(u32), C.POINTER(u32),
+                               C.POINTER(u32)]),
+        "ojh_submit": (i32, [vp]),
+        "ojh_timer_start": (i32, [vp]),
+        "ojh_timer_stop": (i32, [vp, C.POINTER(C.c_float)]),
+        "ojh_lin_create": (i32, [vp, u32, u32, u32, vp, pp]),
+        "ojh_lin_wrap": (i32, [vp, u32, u32, u32, vp, sz, pp]),
+        "ojh_lin_free": (i32, [vp, vp]),
+        "ojh_row_bytes": (sz, [u32, u32]),
+        "ojh_mm": (i32, [vp, vp, sz, i32, vp, vp, sz, vp, u32, i32, i32]),
+        "ojh_mm_q8k": (i32, [vp, vp, vp, vp, vp, sz, vp, u32, i32]),
+        "ojh_mark": (i32, [vp, i32]),
+        "ojh_mark_elapsed": (i32, [vp, i32, i32, C.POINTER(C.c_float)]),
+        "ojh_dequant_f16": (i32, [vp, u32, vp, sz, sz, vp, sz]),
+        "ojh_quant_q8k": (i32, [vp, vp, sz, i32, u32, u32, vp, vp]),
+        "ojh_moe_route": (i32, [vp, vp, u32, u32, u32, vp, vp]),
+        "ojh_moe_ffn": (i32, [vp, vp, u32, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp, i32, i32]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+    L._ojh_signatures = sig
+    if path is None:
+        _lib = L
+    return L
+
+
+def manifest() -> list[tuple[str, str, int, int]]:
+    """(name, family, n_bufs, n_consts) of every kernel the library claims. Needs no GPU."""
+    L = load_library()
+    n = L.ojh_manifest(-1, None, None, None, None)
+    out = []
+    for i in range(n):
+        name, fam = C.c_char_p(), C.c_char_p()
+        nb, nc = C.c_int(), C.c_int()
+        L.ojh_manifest(i, C.byref(name), C.byref(fam), C.byref(nb), C.byref(nc))
+        out.append((name.value.decode(), fam.value.decode(), nb.value, nc.value))
+    return out
+
+
+def row_bytes(ty: int, k: int) -> int:
+    bb, wpb = BLOCK_SHAPE[ty]
+    if k % wpb:
+        raise ValueError(f"K={k} is not a multiple of {wpb}")
+    return k // wpb * bb
+
+
+class Buf:
+    """Device buffer. Dropping it frees the memory, as the reference's `CuBuf` does
+    (crates/ojas-cuda/src/device.rs:20-23)."""
+
+    def __init__(self, gpu: "HipGpu", handle: int, nbytes: int):
+        self.gpu, self.handle, self.nbytes = gpu, handle, nbytes
+
+    @property
+    def ptr(self) -> int:
+        return self.gpu._L.ojh_buf_ptr(self.handle) or 0
+
+    def free(self) -> None:
+        if self.handle and self.gpu._dev:
+            self.gpu._check(self.gpu._L.ojh_free(self.gpu._dev, self.handle))
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Enc:
+    """Stand-in for the reference's encoder: this backend has one stream per device, so an
+    encoder is only a marker that ties `dispatch` calls to the `submit` that waits for them."""
+
+    def __init__(self, gpu: "HipGpu"):
+        self.gpu = gpu
+
+
+class Lin:
+    """A weight matrix W[N,K] kept in its GGUF block bytes (crates/ojas-cuda/src/qwen35.rs:146-201)."""
+
+    def __init__(self, gpu: "HipGpu", handle: int, ty: int, n: int, k: int, keep=None):
+        self.gpu, self.handle, self.ty, self.n, self.k = gpu, handle, ty, n, k
+        self._keep = keep  # a wrapped Buf must outlive the handle
+
+    @property
+    def nbytes(self) -> int:
+        return self.n * row_bytes(self.ty, self.k)
+
+    def free(self) -> None:
+        if self.handle and self.gpu._dev:
+            self.gpu._check(self.gpu._L.ojh_lin_free(self.gpu._dev, self.handle))
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class HipGpu:
+    """`Device + KernelRuntime` over the C ABI."""
+
+    def __init__(self, ordinal: int = 0):
+        self._L = load_library()
+        self._dev = None
+        dev = C.c_void_p()
+        self._check(self._L.ojh_open(ordinal, C.byref(dev)))
+        self._dev = dev
+
+    # -- plumbing
+    def _check(self, rc: int) -> None:
+        if rc != 0:
+            raise OjasHipError(rc, (self._L.ojh_last_error() or b"").decode())
+
+    def close(self) -> None:
+        if self._dev:
+            self._L.ojh_close(self._dev)
+            self._dev = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # -- Device
+    def name(self) -> str:
+        return self._L.ojh_name(self._dev).decode()
+
+    def alloc_bytes(self, nbytes: int) -> Buf:
+        h = C.c_void_p()
+        self._check(self._L.ojh_alloc(self._dev, nbytes, C.byref(h)))
+        return Buf(self, h, nbytes)
+
+    def alloc(self, len_f32: int) -> Buf:
+        return self.alloc_bytes(len_f32 * 4)
+
+    def wrap(self, device_ptr: int, nbytes: int) -> Buf:
+        """Borrow device memory owned elsewhere (e.g. a torch tensor's storage)."""
+        h = C.c_void_p()
+        self._check(self._L.ojh_wrap(self._dev, C.c_void_p(device_ptr), nbytes, C.byref(h)))
+        return Buf(self, h, nbytes)
+
+    def upload_bytes(self, data) -> Buf:
+        a = np.ascontiguousarray(data)
+        b = self.alloc_bytes(a.nbytes)
+        self.write_bytes(b, 0, a)
+        return b
+
+    def upload(self, data) -> Buf:
+        return self.upload_bytes(np.ascontiguousarray(data, np.float32))
+
+    def write_bytes(self, buf: Buf, off: int, data) -> None:
+        a = np.ascontiguousarray(data)
+        self._check(self._L.ojh_upload(self._dev, buf.handle, off, C.c_void_p(a.ctypes.data), a.nbytes))
+
+    def read_bytes(self, buf: Buf, off: int, out: np.ndarray) -> np.ndarray:
+        assert out.flags["C_CONTIGUOUS"]
+        self._check(self._L.ojh_download(self._dev, buf.handle, off, C.c_void_p(out.ctypes.data), out.nbytes))
+        return out
+
+    def read(self, buf: Buf, n: int, dtype=np.float32, off: int = 0) -> np.ndarray:
+        return self.read_bytes(buf, off, np.empty(n, dtype))
+
+    def memset0(self, buf: Buf, off: int = 0, nbytes: int | None = None) -> None:
+        self._check(self._L.ojh_memset0(self._dev, buf.handle, off, buf.nbytes - off if nbytes is None else nbytes))
+
+    # -- KernelRuntime
+    def ensure_family(self, family: str) -> None:
+        self._check(self._L.ojh_ensure_family(self._dev, family.encode()))
+
+    def has_kernel(self, name: str) -> bool:
+        return bool(self._L.ojh_has_kernel(self._dev, name.encode()))
+
+    def caps(self) -> Caps:
+        c = _Caps()
+        self._check(self._L.ojh_caps_get(self._dev, C.byref(c)))
+        return Caps(tier="CBA"[c.tier], f16_compute=bool(c.f16_compute), simd_width=c.simd_width,
+                    unified_memory=bool(c.unified_memory), max_buffer=c.max_buffer,
+                    compute_units=c.compute_units, clock_mhz=c.clock_mhz, arch=c.arch.decode(),
+                    features=tuple((c.features or b"").decode().split(",")))
+
+    def begin(self) -> Enc:
+        return Enc(self)
+
+    def launch_shape(self, name: str, K: int, N: int, M: int = 1):
+        g, b = (C.c_uint32 * 3)(), (C.c_uint32 * 3)()
+        self._check(self._L.ojh_launch_shape(self._dev, name.encode(), K, N, M, g, b))
+        return list(g), list(b)
+
+    def dispatch(self, enc: Enc, name: str, bufs, consts, grid, block) -> None:
+        """`bufs` is a list of (Buf, byte_offset); buffers first, then u32 constants."""
+        n = len(bufs)
+        hs = (C.c_void_p * max(n, 1))(*[b.handle for b, _ in bufs])
+        offs = (C.c_uint64 * max(n, 1))(*[o for _, o in bufs])
+        cs = (C.c_uint32 * max(len(consts), 1))(*consts)
+        g, b = (C.c_uint32 * 3)(*grid), (C.c_uint32 * 3)(*block)
+        self._check(self._L.ojh_dispatch(self._dev, name.encode(), n, hs, offs, len(consts), cs, g, b))
+
+    def submit(self, enc: Enc | None = None) -> None:
+        self._check(self._L.ojh_submit(self._dev))
+
+    def timer_start(self) -> None:
+        self._check(self._L.ojh_timer_start(self._dev))
+
+    def timer_stop(self) -> float:
+        ms = C.c_float()
+        self._check(self._L.ojh_timer_stop(self._dev, C.byref(ms)))
+        return ms.value
+
+    # -- op seam
+    def lin(self, ty: int, n: int, k: int, raw) -> Lin:
+        a = np.ascontiguousarray(raw, np.uint8)
+        if a.size != n * row_bytes(ty, k):
+            raise ValueError(f"Lin {n}x{k} of type {ty} needs {n * row_bytes(ty, k)} bytes, got {a.size}")
+        h = C.c_void_p()
+        self._check(self._L.ojh_lin_create(self._dev, ty, n, k, C.c_void_p(a.ctypes.data), C.byref(h)))
+        return Lin(self, h, ty, n, k)
+
+    def lin_wrap(self, ty: int, n: int, k: int, raw: Buf, off: int = 0) -> Lin:
+        h = C.c_void_p()
+        self._check(self._L.ojh_lin_wrap(self._dev, ty, n, k, raw.handle, off, C.byref(h)))
+        return Lin(self, h, ty, n, k, keep=raw)
+
+    def mm(self, x: Buf, w: Lin, y: Buf, m: int = 1, accum: bool = False, *, x_dtype: int = X_F32,
+           act_mode: int = ACT_AUTO, bias: Buf | None = None, x_off: int = 0, y_off: int = 0) -> None:
+        self._check(self._L.ojh_mm(self._dev, x.handle, x_off, x_dtype, w.handle, y.handle, y_off,
+                                   bias.handle if bias else None, m, int(accum), act_mode))
+
+    def mm_q8k(self, xq: Buf, xscales: Buf, w: Lin, y: Buf, m: int = 1, accum: bool = False, *,
+               bias: Buf | None = None, y_off: int = 0) -> None:
+        """Matmul from activations already quantized by `quant_q8k` (shared by several projections)."""
+        self._check(self._L.ojh_mm_q8k(self._dev, xq.handle, xscales.handle, w.handle, y.handle, y_off,
+                                       bias.handle if bias else None, m, int(accum)))
+
+    def mark(self, slot: int) -> None:
+        self._check(self._L.ojh_mark(self._dev, slot))
+
+    def mark_elapsed(self, a: int, b: int) -> float:
+        ms = C.c_float()
+        self._check(self._L.ojh_mark_elapsed(self._dev, a, b, C.byref(ms)))
+        return ms.value
+
+    def dequant_f16(self, ty: int, raw: Buf, n_weights: int, out: Buf, raw_off: int = 0, out_off: int = 0) -> None:
+        self._check(self._L.ojh_dequant_f16(self._dev, ty, raw.handle, raw_off, n_weights, out.handle, out_off))
+
+    def quant_q8k(self, x: Buf, m: int, k: int, q: Buf, scales: Buf, x_dtype: int = X_F32, x_off: int = 0) -> None:
+        self._check(self._L.ojh_quant_q8k(self._dev, x.handle, x_off, x_dtype, m, k, q.handle, scales.handle))
+
+    def moe_route(self, logits: Buf, n_tokens: int, n_expert: int, ksel: int, idx: Buf, wgt: Buf) -> None:
+        self._check(self._L.ojh_moe_route(self._dev, logits.handle, n_tokens, n_expert, ksel, idx.handle, wgt.handle))
+
+    def moe_ffn(self, x: Buf, n_tokens: int, d: int, n_ff: int, n_expert: int, ksel: int, idx: Buf, wgt: Buf,
+                gate: Lin, up: Lin, down: Lin, y: Buf, accum: bool = False, act_mode: int = ACT_AUTO) -> None:
+        self._check(self._L.ojh_moe_ffn(self._dev, x.handle, n_tokens, d, n_ff, n_expert, ksel, idx.handle,
+                                        wgt.handle, gate.handle, up.handle, down.handle, y.handle, int(accum),
+                                        act_mode))

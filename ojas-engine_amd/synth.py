@@ -1,0 +1,178 @@
+"""Seeded synthetic inputs: GGUF block tensors, activations, router logits.
+
+Two kinds of generator live here:
+  * the benchmark configurations' own distributions (uniform codes, |N(0, sigma)| f16 scales,
+    N(0,1) activations), one numpy PCG64 stream per tensor, seeded from (config, tensor) names;
+  * procedures the reference's tests specify in their text, restated so the same bytes can be
+    produced anywhere: `synth::blocks` (crates/ojas-formats/src/synth.rs:29-64), the `tvec` LCG
+    (crates/ojas-cuda/tests/conformance.rs:223-231) and the closed-form Q8_0 rows of
+    crates/ojas-metal/tests/dispatch.rs:357-429 and crates/ojas-formats/tests/rows.rs:13-18.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+BLOCK_SHAPE = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
+
+
+def seed_of(*names) -> int:
+    """FNV-1a-64 of the joined names: one independent stream per (config, tensor)."""
+    h = 0xCBF29CE484222325
+    for b in "/".join(str(n) for n in names).encode():
+        h ^= b
+        h = (h * 0x100000001B3) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+def rng(*names) -> np.random.Generator:
+    return np.random.Generator(np.random.PCG64(seed_of(*names)))
+
+
+def normal_f32(n, *names) -> np.ndarray:
+    return rng(*names).standard_normal(n, dtype=np.float32)
+
+
+def to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """f32 -> bf16 bit patterns, round to nearest even."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    u = u + 0x7FFF + ((u >> 16) & 1)
+    return (u >> 16).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def _f16_abs_normal(g: np.random.Generator, n: int, sigma: float) -> np.ndarray:
+    return np.abs(g.standard_normal(n) * sigma).astype(np.float16).view(np.uint16)
+
+
+# ------------------------------------------------------------------ benchmark distributions
+def q80_weights(n: int, k: int, *names) -> np.ndarray:
+    """Q8_0 rows: per block d = f16(|N(0,0.02)| / 127), 32 int8 codes uniform in [-127, 127]."""
+    g = rng(*names)
+    nb = n * (k // 32)
+    out = np.empty((nb, 34), np.uint8)
+    d = (np.abs(g.standard_normal(nb) * 0.02) / 127.0).astype(np.float16).view(np.uint16)
+    out[:, 0] = d & 0xFF
+    out[:, 1] = d >> 8
+    out[:, 2:] = g.integers(-127, 128, size=(nb, 32), dtype=np.int8).view(np.uint8)
+    return out.reshape(-1)
+
+
+def pack_scales_k4(sc: np.ndarray, mn: np.ndarray) -> np.ndarray:
+    """Inverse of get_scale_min_k4 (crates/ojas-formats/src/gguf.rs:1132-1140): 8 six-bit scales
+    and 8 six-bit mins per super-block -> the 12 packed bytes."""
+    sc = sc.astype(np.uint8)
+    mn = mn.astype(np.uint8)
+    q = np.empty((sc.shape[0], 12), np.uint8)
+    q[:, 0:4] = sc[:, 0:4] | ((sc[:, 4:8] >> 4) << 6)
+    q[:, 4:8] = mn[:, 0:4] | ((mn[:, 4:8] >> 4) << 6)
+    q[:, 8:12] = (sc[:, 4:8] & 0xF) | ((mn[:, 4:8] & 0xF) << 4)
+    return q
+
+
+def q4k_weights(n: int, k: int, *names) -> np.ndarray:
+    """Q4_K rows: d, dmin = f16(|N(0,0.01)|), scales and mins uniform in [0,63], uniform nibbles."""
+    g = rng(*names)
+    nb = n * (k // 256)
+    out = np.empty((nb, 144), np.uint8)
+    hdr = np.empty((nb, 2), np.uint16)
+    hdr[:, 0] = _f16_abs_normal(g, nb, 0.01)
+    hdr[:, 1] = _f16_abs_normal(g, nb, 0.01)
+    out[:, 0:4] = hdr.view(np.uint8).reshape(nb, 4)
+    out[:, 4:16] = pack_scales_k4(g.integers(0, 64, size=(nb, 8), dtype=np.uint8),
+                                  g.integers(0, 64, size=(nb, 8), dtype=np.uint8))
+    out[:, 16:] = g.integers(0, 256, size=(nb, 128), dtype=np.uint8)
+    return out.reshape(-1)
+
+
+def q6k_weights(n: int, k: int, *names) -> np.ndarray:
+    """Q6_K rows: uniform 6-bit codes, int8 sub-scales uniform in [-32,31], d = f16(|N(0,0.01)|)."""
+    g = rng(*names)
+    nb = n * (k // 256)
+    out = np.empty((nb, 210), np.uint8)
+    out[:, 0:192] = g.integers(0, 256, size=(nb, 192), dtype=np.uint8)
+    out[:, 192:208] = g.integers(-32, 32, size=(nb, 16), dtype=np.int8).view(np.uint8)
+    d = _f16_abs_normal(g, nb, 0.01)
+    out[:, 208] = d & 0xFF
+    out[:, 209] = d >> 8
+    return out.reshape(-1)
+
+
+def weights(ty: int, n: int, k: int, *names) -> np.ndarray:
+    return {Q8_0: q80_weights, Q4_K: q4k_weights, Q6_K: q6k_weights}[ty](n, k, *names)
+
+
+# ------------------------------------------------------------------ the reference tests' procedures
+def synth_blocks(ty: int, nb: int) -> np.ndarray:
+    """`synth::blocks(t, nb)`: xorshift64 bytes with the f16 scale fields pinned."""
+    bb, _ = BLOCK_SHAPE[ty]
+    st = 0x2545F4914F6CDD1D
+    mask = 0xFFFFFFFFFFFFFFFF
+    out = np.empty(nb * bb, np.uint8)
+    for i in range(nb * bb):
+        st ^= (st << 13) & mask
+        st ^= st >> 7
+        st ^= (st << 17) & mask
+        out[i] = (st >> 24) & 0xFF
+    blocks = out.reshape(nb, bb)
+    dmin = np.array([0.01], np.float32).astype(np.float16).view(np.uint16)[0]
+    for i in range(nb):
+        d = (np.float32(0.05) + np.float32(i % 7) * np.float32(0.01)).astype(np.float16).view(np.uint16)
+        d = int(d)
+        if ty in (Q4_K, Q5_K):
+            blocks[i, 0], blocks[i, 1] = d & 0xFF, d >> 8
+            blocks[i, 2], blocks[i, 3] = int(dmin) & 0xFF, int(dmin) >> 8
+        elif ty == Q6_K:
+            blocks[i, 208], blocks[i, 209] = d & 0xFF, d >> 8
+        else:
+            blocks[i, 0], blocks[i, 1] = d & 0xFF, d >> 8
+    return out
+
+
+def tvec(n: int, seed: int) -> np.ndarray:
+    """Deterministic vector in [-1, 1) from the reference's test LCG."""
+    a, c = np.uint32(1664525), np.uint32(1013904223)
+    s0 = np.uint32((seed * 2654435761 + 1) & 0xFFFFFFFF)
+    with np.errstate(over="ignore"):
+        A = np.multiply.accumulate(np.full(n, a, np.uint32), dtype=np.uint32)  # a^(i+1)
+        S = np.concatenate(([np.uint32(1)], A[:-1])).astype(np.uint32)  # a^i
+        Csum = np.add.accumulate(S, dtype=np.uint32)                     # sum_{j<=i} a^j
+        s = A * s0 + c * Csum
+    return ((s >> np.uint32(9)).astype(np.float32) / np.float32(1 << 23)) - np.float32(1.0)
+
+
+def q80_rows_closed_form(n: int, k: int):
+    """Q8_0 rows and activations of the reference's `native_q8_matvec_ksplit_matches_cpu`:
+    d = f16(0.003 + ((r+b) mod 7) * 0.001), q = ((17r + 11b + 5j) mod 31) - 15,
+    x_i = ((37 i mod 257) - 128) / 127."""
+    nb = k // 32
+    r = np.arange(n)[:, None, None]
+    b = np.arange(nb)[None, :, None]
+    j = np.arange(32)[None, None, :]
+    q = (((17 * r + 11 * b + 5 * j) % 31) - 15).astype(np.int8)
+    d = (np.float32(0.003) + ((r + b) % 7).astype(np.float32) * np.float32(0.001)).astype(np.float16)
+    out = np.empty((n, nb, 34), np.uint8)
+    dv = d.view(np.uint16).reshape(n, nb)
+    out[:, :, 0] = dv & 0xFF
+    out[:, :, 1] = dv >> 8
+    out[:, :, 2:] = q.view(np.uint8)
+    i = np.arange(k)
+    x = (((37 * i) % 257) - 128).astype(np.float32) / np.float32(127.0)
+    return out.reshape(-1), x
+
+
+def q80_rows_table() -> tuple[np.ndarray, np.ndarray]:
+    """The 3 x 32 Q8_0 table of crates/ojas-formats/tests/rows.rs:13-18 and its exact values:
+    d = 0.25 (r+1), q_j = j - 16 + r."""
+    out = np.empty((3, 34), np.uint8)
+    want = np.empty((3, 32), np.float32)
+    for r in range(3):
+        d = np.array([0.25 * (r + 1)], np.float16)
+        out[r, 0:2] = d.view(np.uint8)
+        q = (np.arange(32) - 16 + r).astype(np.int8)
+        out[r, 2:] = q.view(np.uint8)
+        want[r] = np.float32(d[0]) * q.astype(np.float32)
+    return out.reshape(-1), want

@@ -1,0 +1,710 @@
+/*
+ * TEST INFRASTRUCTURE — CPU restatement of the reference's quantized-matmul arithmetic.
+ * See ojas_oracle.h for what this is, who may use it and how each function is pinned.
+ * Paths in comments are relative to the reference tree.
+ *
+ * Build: gcc -O2 -ffp-contract=off -fno-fast-math (the reference is Rust: one IEEE rounding per
+ * operator, no fused multiply-add).
+ */
+#include "ojas_oracle.h"
+
+#include <math.h>
+#include <pthread.h>
+#include <stdatomic.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ---------------------------------------------------------------- f16 / bf16 */
+
+/* IEEE binary16 -> binary32 (crate half 2.7.1, f16::to_f32; used at gguf.rs:606-608). */
+float ojo_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else { /* subnormal: normalise */
+            int e = -1;
+            do { man <<= 1; e++; } while (!(man & 0x400u));
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3FFu) << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7F800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+/* binary32 -> binary16, round to nearest even (half::f16::from_f32; gguf.rs:602-604). */
+uint16_t ojo_f32_to_f16(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    uint32_t exp = (x >> 23) & 0xFFu;
+    uint32_t man = x & 0x7FFFFFu;
+    if (exp == 0xFF) { /* inf / nan */
+        if (man == 0) return (uint16_t)(sign | 0x7C00u);
+        return (uint16_t)(sign | 0x7C00u | 0x200u | (man >> 13));
+    }
+    int e = (int)exp - 127 + 15;
+    if (e >= 31) return (uint16_t)(sign | 0x7C00u); /* overflow -> inf */
+    if (e <= 0) {
+        if (e < -10) return sign; /* below half the smallest subnormal */
+        man |= 0x800000u;
+        uint32_t shift = (uint32_t)(14 - e);
+        uint32_t hm = man >> shift;
+        uint32_t rem = man & ((1u << shift) - 1u);
+        uint32_t half = 1u << (shift - 1u);
+        if (rem > half || (rem == half && (hm & 1u))) hm++;
+        return (uint16_t)(sign | hm); /* a carry into bit 10 is the smallest normal: correct */
+    }
+    uint32_t hm = man >> 13;
+    uint32_t rem = man & 0x1FFFu;
+    uint16_t out = (uint16_t)(sign | ((uint32_t)e << 10) | hm);
+    if (rem > 0x1000u || (rem == 0x1000u && (hm & 1u))) out++; /* carry may roll into exp / inf */
+    return out;
+}
+
+uint16_t ojo_f32_to_bf16(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    if ((x & 0x7F800000u) == 0x7F800000u && (x & 0x7FFFFFu)) return (uint16_t)((x >> 16) | 0x40u);
+    uint32_t lsb = (x >> 16) & 1u;
+    x += 0x7FFFu + lsb;
+    return (uint16_t)(x >> 16);
+}
+
+float ojo_bf16_to_f32(uint16_t h) {
+    uint32_t x = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &x, 4);
+    return f;
+}
+
+static inline float rdh(const uint8_t *b, size_t i) { /* gguf.rs:606-608 */
+    return ojo_f16_to_f32((uint16_t)(b[i] | (b[i + 1] << 8)));
+}
+
+/* ---------------------------------------------------------------- block shapes, synth */
+
+int ojo_block_shape(uint32_t ty, uint32_t *bytes, uint32_t *weights) { /* synth.rs:12-21 */
+    uint32_t b, w;
+    switch (ty) {
+    case OJO_Q8_0: b = 34; w = 32; break;
+    case OJO_Q4_K: b = 144; w = 256; break;
+    case OJO_Q5_K: b = 176; w = 256; break;
+    case OJO_Q6_K: b = 210; w = 256; break;
+    default: return 0;
+    }
+    if (bytes) *bytes = b;
+    if (weights) *weights = w;
+    return 1;
+}
+
+int ojo_synth_blocks(uint32_t ty, size_t nb, uint8_t *out) { /* synth.rs:29-64 */
+    uint32_t bb;
+    if (!ojo_block_shape(ty, &bb, NULL)) return -1;
+    uint64_t st = 0x2545F4914F6CDD1DULL;
+    for (size_t i = 0; i < nb * bb; i++) {
+        st ^= st << 13; st ^= st >> 7; st ^= st << 17;
+        out[i] = (uint8_t)(st >> 24);
+    }
+    for (size_t i = 0; i < nb; i++) {
+        uint8_t *blk = out + i * bb;
+        uint16_t d = ojo_f32_to_f16(0.05f + (float)(i % 7) * 0.01f);
+        uint16_t dmin = ojo_f32_to_f16(0.01f);
+        switch (ty) {
+        case OJO_Q4_K: case OJO_Q5_K:
+            blk[0] = (uint8_t)d; blk[1] = (uint8_t)(d >> 8);
+            blk[2] = (uint8_t)dmin; blk[3] = (uint8_t)(dmin >> 8);
+            break;
+        case OJO_Q6_K:
+            blk[208] = (uint8_t)d; blk[209] = (uint8_t)(d >> 8);
+            break;
+        default:
+            blk[0] = (uint8_t)d; blk[1] = (uint8_t)(d >> 8);
+        }
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------------- dequant */
+
+/* get_scale_min_k4 (gguf.rs:1132-1140; twin cpu_math.rs:566-574). */
+static inline void scale_min_k4(int j, const uint8_t *q, uint8_t *sc, uint8_t *m) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4));
+        *m = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+int ojo_dequant_to_f16(const uint8_t *b, uint32_t ty, size_t n, uint16_t *out) {
+    uint32_t bb, wpb;
+    if (!ojo_block_shape(ty, &bb, &wpb) || n % wpb) return -1;
+    size_t nblk = n / wpb;
+    for (size_t ib = 0; ib < nblk; ib++) {
+        const uint8_t *blk = b + ib * bb;
+        uint16_t *o = out + ib * wpb;
+        switch (ty) {
+        case OJO_Q8_0: { /* gguf.rs:704-709 */
+            float d = rdh(blk, 0);
+            for (int j = 0; j < 32; j++) o[j] = ojo_f32_to_f16(d * (float)(int8_t)blk[2 + j]);
+        } break;
+        case OJO_Q4_K: { /* gguf.rs:1042-1059 */
+            float d = rdh(blk, 0), dmin = rdh(blk, 2);
+            const uint8_t *sc = blk + 4, *qs = blk + 16;
+            for (int chunk = 0; chunk < 4; chunk++) {
+                uint8_t s1, m1, s2, m2;
+                scale_min_k4(chunk * 2, sc, &s1, &m1);
+                scale_min_k4(chunk * 2 + 1, sc, &s2, &m2);
+                float dl1 = d * (float)s1, ml1 = dmin * (float)m1;
+                float dl2 = d * (float)s2, ml2 = dmin * (float)m2;
+                const uint8_t *q = qs + chunk * 32;
+                for (int l = 0; l < 32; l++) *o++ = ojo_f32_to_f16(dl1 * (float)(q[l] & 0xF) - ml1);
+                for (int l = 0; l < 32; l++) *o++ = ojo_f32_to_f16(dl2 * (float)(q[l] >> 4) - ml2);
+            }
+        } break;
+        case OJO_Q5_K: { /* gguf.rs:1060-1085 */
+            float d = rdh(blk, 0), dmin = rdh(blk, 2);
+            const uint8_t *sc = blk + 4, *qh = blk + 16, *qs = blk + 48;
+            uint8_t u1 = 1, u2 = 2;
+            for (int chunk = 0; chunk < 4; chunk++) {
+                uint8_t s1, m1, s2, m2;
+                scale_min_k4(chunk * 2, sc, &s1, &m1);
+                scale_min_k4(chunk * 2 + 1, sc, &s2, &m2);
+                float dl1 = d * (float)s1, ml1 = dmin * (float)m1;
+                float dl2 = d * (float)s2, ml2 = dmin * (float)m2;
+                const uint8_t *ql = qs + chunk * 32;
+                for (int l = 0; l < 32; l++) {
+                    float hi = (qh[l] & u1) ? 16.0f : 0.0f;
+                    *o++ = ojo_f32_to_f16(dl1 * ((float)(ql[l] & 0xF) + hi) - ml1);
+                }
+                for (int l = 0; l < 32; l++) {
+                    float hi = (qh[l] & u2) ? 16.0f : 0.0f;
+                    *o++ = ojo_f32_to_f16(dl2 * ((float)(ql[l] >> 4) + hi) - ml2);
+                }
+                u1 = (uint8_t)(u1 << 2); u2 = (uint8_t)(u2 << 2);
+            }
+        } break;
+        case OJO_Q6_K: { /* gguf.rs:1086-1108 */
+            float d = rdh(blk, 208);
+            float y[128];
+            for (int hf = 0; hf < 2; hf++) {
+                const uint8_t *ql = blk + hf * 64, *qh = blk + 128 + hf * 32;
+                const int8_t *sc = (const int8_t *)(blk + 192 + hf * 8);
+                for (int l = 0; l < 32; l++) {
+                    int is = l / 16;
+                    int q1 = ((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+                    int q2 = ((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                    int q3 = ((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                    int q4 = ((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+                    /* `d * sc as f32 * q as f32` is left-associative: (d*sc)*q */
+                    y[l]      = d * (float)sc[is]     * (float)q1;
+                    y[l + 32] = d * (float)sc[is + 2] * (float)q2;
+                    y[l + 64] = d * (float)sc[is + 4] * (float)q3;
+                    y[l + 96] = d * (float)sc[is + 6] * (float)q4;
+                }
+                for (int l = 0; l < 128; l++) *o++ = ojo_f32_to_f16(y[l]);
+            }
+        } break;
+        }
+    }
+    return 0;
+}
+
+int ojo_dequant_to_f64(const uint8_t *b, uint32_t ty, size_t n, double *out) {
+    /* Same decoders, exact in double: f16 scale x 6-bit x 6-bit products fit a double
+     * (crates/ojas-models/examples/q6k_gate.rs:60-110 derives its oracle the same way). */
+    uint32_t bb, wpb;
+    if (!ojo_block_shape(ty, &bb, &wpb) || n % wpb) return -1;
+    size_t nblk = n / wpb;
+    for (size_t ib = 0; ib < nblk; ib++) {
+        const uint8_t *blk = b + ib * bb;
+        double *o = out + ib * wpb;
+        switch (ty) {
+        case OJO_Q8_0: {
+            double d = rdh(blk, 0);
+            for (int j = 0; j < 32; j++) o[j] = d * (double)(int8_t)blk[2 + j];
+        } break;
+        case OJO_Q4_K: case OJO_Q5_K: {
+            double d = rdh(blk, 0), dmin = rdh(blk, 2);
+            const uint8_t *sc = blk + 4;
+            const uint8_t *qh = ty == OJO_Q5_K ? blk + 16 : NULL;
+            const uint8_t *qs = ty == OJO_Q5_K ? blk + 48 : blk + 16;
+            for (int chunk = 0; chunk < 4; chunk++) {
+                uint8_t s1, m1, s2, m2;
+                scale_min_k4(chunk * 2, sc, &s1, &m1);
+                scale_min_k4(chunk * 2 + 1, sc, &s2, &m2);
+                const uint8_t *q = qs + chunk * 32;
+                for (int l = 0; l < 32; l++) {
+                    int v = (q[l] & 0xF) + ((qh && (qh[l] & (1 << (2 * chunk)))) ? 16 : 0);
+                    *o++ = d * s1 * v - dmin * m1;
+                }
+                for (int l = 0; l < 32; l++) {
+                    int v = (q[l] >> 4) + ((qh && (qh[l] & (2 << (2 * chunk)))) ? 16 : 0);
+                    *o++ = d * s2 * v - dmin * m2;
+                }
+            }
+        } break;
+        case OJO_Q6_K: {
+            double d = rdh(blk, 208);
+            for (int hf = 0; hf < 2; hf++) {
+                const uint8_t *ql = blk + hf * 64, *qh = blk + 128 + hf * 32;
+                const int8_t *sc = (const int8_t *)(blk + 192 + hf * 8);
+                for (int l = 0; l < 32; l++) {
+                    int is = l / 16;
+                    int q1 = ((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+                    int q2 = ((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                    int q3 = ((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                    int q4 = ((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+                    o[l]      = d * sc[is]     * q1;
+                    o[l + 32] = d * sc[is + 2] * q2;
+                    o[l + 64] = d * sc[is + 4] * q3;
+                    o[l + 96] = d * sc[is + 6] * q4;
+                }
+                o += 128;
+            }
+        } break;
+        }
+    }
+    return 0;
+}
+
+uint64_t ojo_digest_f16(const uint16_t *v, size_t n) { /* quant_formats.rs:20-31 */
+    uint64_t h = 0xcbf29ce484222325ULL;
+    char buf[64];
+    for (size_t i = 0; i < n; i++) {
+        int len = snprintf(buf, sizeof buf, "%.6f", (double)ojo_f16_to_f32(v[i]));
+        for (int c = 0; c < len; c++) {
+            h ^= (uint8_t)buf[c];
+            h *= 0x00000100000001B3ULL;
+        }
+    }
+    return h;
+}
+
+/* ---------------------------------------------------------------- activations */
+
+static inline float clampf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+void ojo_quant_q8k(const float *x, size_t k, float *scales, int8_t *q, int32_t *bsums) {
+    /* cpu_math.rs:545-563. f32::round is round-half-away-from-zero == roundf. */
+    size_t nsb = (k + 255) / 256;
+    memset(q, 0, nsb * 256);
+    memset(bsums, 0, nsb * 8 * sizeof(int32_t));
+    for (size_t sb = 0; sb < nsb; sb++) {
+        size_t lo = sb * 256, hi = lo + 256 < k ? lo + 256 : k;
+        float m = 0.0f;
+        for (size_t i = lo; i < hi; i++) { float a = fabsf(x[i]); if (a > m) m = a; }
+        float scale = m > 0.0f ? m / 127.0f : 1.0f;
+        float inv = 1.0f / scale;
+        scales[sb] = scale;
+        for (size_t i = lo; i < hi; i++) {
+            int8_t qi = (int8_t)clampf(roundf(x[i] * inv), -127.0f, 127.0f);
+            q[i] = qi;
+            bsums[sb * 8 + (i - lo) / 32] += qi;
+        }
+    }
+}
+
+float ojo_quant_row_i8(const float *row, size_t k, int8_t *q) { /* cpu_math.rs:174-179 */
+    float m = 0.0f;
+    for (size_t i = 0; i < k; i++) { float a = fabsf(row[i]); if (a > m) m = a; }
+    float scale = m > 0.0f ? m / 127.0f : 1.0f;
+    float inv = 1.0f / scale;
+    for (size_t i = 0; i < k; i++) q[i] = (int8_t)clampf(roundf(row[i] * inv), -127.0f, 127.0f);
+    return scale;
+}
+
+/* ---------------------------------------------------------------- row dots */
+
+float ojo_dot_q80(const uint8_t *row, const float *x, size_t k) { /* cpu_math.rs:971-981 */
+    float sum = 0.0f;
+    for (size_t b = 0; b < k / 32; b++) {
+        const uint8_t *blk = row + b * 34;
+        const float *xb = x + b * 32;
+        float d = rdh(blk, 0);
+        float acc = 0.0f;
+        for (int j = 0; j < 32; j++) acc += (float)(int8_t)blk[2 + j] * xb[j];
+        sum += d * acc;
+    }
+    return sum;
+}
+
+static inline int32_t idot32(const uint8_t *w, const int8_t *x) { /* cpu_math.rs:583-593 */
+    int32_t s = 0;
+    for (int i = 0; i < 32; i++) s += (int32_t)w[i] * (int32_t)x[i];
+    return s;
+}
+
+float ojo_dot_q4k(const uint8_t *row, size_t k, const float *scales, const int8_t *q,
+                  const int32_t *bsums) { /* cpu_math.rs:609-635 */
+    float total = 0.0f;
+    for (size_t sb = 0; sb < k / 256; sb++) {
+        const uint8_t *blk = row + sb * 144;
+        float d = rdh(blk, 0), dmin = rdh(blk, 2);
+        const uint8_t *sc = blk + 4, *qs = blk + 16;
+        float sx = scales[sb];
+        const int8_t *xq = q + sb * 256;
+        const int32_t *bs = bsums + sb * 8;
+        float sumd = 0.0f, summ = 0.0f;
+        uint8_t lo[32], hi[32];
+        for (int c = 0; c < 4; c++) {
+            const uint8_t *qq = qs + c * 32;
+            for (int l = 0; l < 32; l++) { lo[l] = qq[l] & 0xF; hi[l] = qq[l] >> 4; }
+            uint8_t s1, m1, s2, m2;
+            scale_min_k4(c * 2, sc, &s1, &m1);
+            scale_min_k4(c * 2 + 1, sc, &s2, &m2);
+            sumd += (float)s1 * (float)idot32(lo, xq + c * 64);
+            sumd += (float)s2 * (float)idot32(hi, xq + c * 64 + 32);
+            summ += (float)m1 * (float)bs[c * 2] + (float)m2 * (float)bs[c * 2 + 1];
+        }
+        total += sx * (d * sumd - dmin * summ);
+    }
+    return total;
+}
+
+float ojo_dot_q5k(const uint8_t *row, size_t k, const float *scales, const int8_t *q,
+                  const int32_t *bsums) { /* cpu_math.rs:638-670 */
+    float total = 0.0f;
+    for (size_t sb = 0; sb < k / 256; sb++) {
+        const uint8_t *blk = row + sb * 176;
+        float d = rdh(blk, 0), dmin = rdh(blk, 2);
+        const uint8_t *sc = blk + 4, *qh = blk + 16, *qs = blk + 48;
+        float sx = scales[sb];
+        const int8_t *xq = q + sb * 256;
+        const int32_t *bs = bsums + sb * 8;
+        float sumd = 0.0f, summ = 0.0f;
+        uint8_t lo[32], hi[32];
+        uint8_t u1 = 1, u2 = 2;
+        for (int c = 0; c < 4; c++) {
+            const uint8_t *qq = qs + c * 32;
+            for (int l = 0; l < 32; l++) {
+                lo[l] = (uint8_t)((qq[l] & 0xF) | ((qh[l] & u1) ? 16 : 0));
+                hi[l] = (uint8_t)((qq[l] >> 4) | ((qh[l] & u2) ? 16 : 0));
+            }
+            uint8_t s1, m1, s2, m2;
+            scale_min_k4(c * 2, sc, &s1, &m1);
+            scale_min_k4(c * 2 + 1, sc, &s2, &m2);
+            sumd += (float)s1 * (float)idot32(lo, xq + c * 64);
+            sumd += (float)s2 * (float)idot32(hi, xq + c * 64 + 32);
+            summ += (float)m1 * (float)bs[c * 2] + (float)m2 * (float)bs[c * 2 + 1];
+            u1 = (uint8_t)(u1 << 2); u2 = (uint8_t)(u2 << 2);
+        }
+        total += sx * (d * sumd - dmin * summ);
+    }
+    return total;
+}
+
+float ojo_dot_q6k(const uint8_t *row, size_t k, const float *scales, const int8_t *q,
+                  const int32_t *bsums) { /* cpu_math.rs:674-722 */
+    (void)bsums;
+    float total = 0.0f;
+    uint8_t w[32];
+    for (size_t sb = 0; sb < k / 256; sb++) {
+        const uint8_t *blk = row + sb * 210;
+        float d = rdh(blk, 208);
+        float sx = scales[sb];
+        const int8_t *xq = q + sb * 256;
+        float sum = 0.0f, sub = 0.0f;
+        for (int hf = 0; hf < 2; hf++) {
+            const uint8_t *ql = blk + hf * 64, *qh = blk + 128 + hf * 32;
+            const int8_t *sc = (const int8_t *)(blk + 192 + hf * 8);
+            const int8_t *xh = xq + hf * 128;
+            for (int quarter = 0; quarter < 4; quarter++) {
+                for (int l = 0; l < 32; l++) {
+                    switch (quarter) {
+                    case 0: w[l] = (uint8_t)((ql[l] & 0xF) | ((qh[l] & 3) << 4)); break;
+                    case 1: w[l] = (uint8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)); break;
+                    case 2: w[l] = (uint8_t)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)); break;
+                    default: w[l] = (uint8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4));
+                    }
+                }
+                const int8_t *x32 = xh + quarter * 32;
+                float s0 = (float)sc[quarter * 2], s1 = (float)sc[quarter * 2 + 1];
+                int32_t i0 = 0, i1 = 0, x0 = 0, x1 = 0;
+                for (int l = 0; l < 16; l++) {
+                    i0 += (int32_t)w[l] * x32[l];
+                    x0 += x32[l];
+                    i1 += (int32_t)w[l + 16] * x32[l + 16];
+                    x1 += x32[l + 16];
+                }
+                sum += s0 * (float)i0 + s1 * (float)i1;
+                sub += s0 * (float)x0 + s1 * (float)x1;
+            }
+        }
+        total += sx * d * (sum - 32.0f * sub);
+    }
+    return total;
+}
+
+/* ---------------------------------------------------------------- workers */
+
+typedef void (*row_fn)(void *ctx, size_t row);
+
+struct steal {
+    atomic_size_t next;
+    size_t n, block;
+    row_fn fn;
+    void *ctx;
+};
+
+static void *steal_worker(void *p) {
+    struct steal *s = (struct steal *)p;
+    for (;;) {
+        size_t r0 = atomic_fetch_add_explicit(&s->next, s->block, memory_order_relaxed);
+        if (r0 >= s->n) break;
+        size_t r1 = r0 + s->block < s->n ? r0 + s->block : s->n;
+        for (size_t r = r0; r < r1; r++) s->fn(s->ctx, r);
+    }
+    return NULL;
+}
+
+/* Rows handed out in blocks from one atomic counter, as matvec_kq (cpu_math.rs:1165-1172,
+ * block 8) and matmul (cpu_math.rs:204-216, block 16) do. */
+static void steal_rows(size_t n, size_t block, int threads, row_fn fn, void *ctx) {
+    struct steal s;
+    atomic_init(&s.next, 0);
+    s.n = n; s.block = block; s.fn = fn; s.ctx = ctx;
+    if (threads > (int)n) threads = (int)(n ? n : 1);
+    if (threads <= 1) { steal_worker(&s); return; }
+    pthread_t *th = (pthread_t *)malloc(sizeof(pthread_t) * (size_t)threads);
+    int started = 0;
+    for (int i = 0; i < threads - 1; i++)
+        if (pthread_create(&th[started], NULL, steal_worker, &s) == 0) started++;
+    steal_worker(&s);
+    for (int i = 0; i < started; i++) pthread_join(th[i], NULL);
+    free(th);
+}
+
+/* ---------------------------------------------------------------- matvec_kq */
+
+struct kq_ctx {
+    const uint8_t *raw; uint32_t ty; size_t k, row_bytes;
+    const float *x; const float *scales; const int8_t *q; const int32_t *bsums; float *y;
+};
+
+static void kq_row(void *p, size_t row) {
+    struct kq_ctx *c = (struct kq_ctx *)p;
+    const uint8_t *rb = c->raw + row * c->row_bytes;
+    float v;
+    switch (c->ty) { /* cpu_math.rs:1174-1181 */
+    case OJO_Q4_K: v = ojo_dot_q4k(rb, c->k, c->scales, c->q, c->bsums); break;
+    case OJO_Q5_K: v = ojo_dot_q5k(rb, c->k, c->scales, c->q, c->bsums); break;
+    case OJO_Q8_0: v = ojo_dot_q80(rb, c->x, c->k); break;
+    default:       v = ojo_dot_q6k(rb, c->k, c->scales, c->q, c->bsums);
+    }
+    c->y[row] = v;
+}
+
+int ojo_matvec_kq(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const float *x,
+                  int threads, float *y) { /* cpu_math.rs:1145-1189 */
+    size_t per256;
+    switch (ty) {
+    case OJO_Q4_K: per256 = 144; break;
+    case OJO_Q5_K: per256 = 176; break;
+    case OJO_Q6_K: per256 = 210; break;
+    case OJO_Q8_0: per256 = 272; break;
+    default: return -1;
+    }
+    size_t nsb = (k + 255) / 256;
+    float *scales = (float *)malloc(nsb * sizeof(float));
+    int8_t *q = (int8_t *)malloc(nsb * 256);
+    int32_t *bsums = (int32_t *)malloc(nsb * 8 * sizeof(int32_t));
+    ojo_quant_q8k(x, k, scales, q, bsums); /* done for every type, used by the K-quants */
+    struct kq_ctx c = { raw, ty, k, k / 256 * per256, x, scales, q, bsums, y };
+    if (ty == OJO_Q8_0) c.row_bytes = k / 32 * 34;
+    steal_rows(n, 8, threads, kq_row, &c);
+    free(scales); free(q); free(bsums);
+    return 0;
+}
+
+/* ---------------------------------------------------------------- row-int8 path */
+
+void ojo_q8_rows_from_f16(const uint16_t *w16, size_t n, size_t k, int8_t *q, float *scale) {
+    /* crates/ojas-formats/src/quant.rs:16-39 — note the division by sv, not a reciprocal. */
+    for (size_t r = 0; r < n; r++) {
+        float amax = 0.0f;
+        for (size_t c = 0; c < k; c++) {
+            float a = fabsf(ojo_f16_to_f32(w16[r * k + c]));
+            if (a > amax) amax = a;
+        }
+        float sv = amax > 0.0f ? amax / 127.0f : 1.0f;
+        scale[r] = sv;
+        for (size_t c = 0; c < k; c++)
+            q[r * k + c] = (int8_t)clampf(roundf(ojo_f16_to_f32(w16[r * k + c]) / sv), -127.0f, 127.0f);
+    }
+}
+
+struct q8_ctx {
+    const int8_t *wq; const float *wscale; size_t k, n, m;
+    const int8_t *xq; const float *xs; const float *bias; float *ys;
+};
+
+static void q8_row(void *p, size_t row) { /* cpu_math.rs:217-231, dot_i8 :404-415 */
+    struct q8_ctx *c = (struct q8_ctx *)p;
+    const int8_t *qrow = c->wq + row * c->k;
+    float b = c->bias ? c->bias[row] : 0.0f;
+    float sw = c->wscale[row];
+    for (size_t t = 0; t < c->m; t++) {
+        const int8_t *qx = c->xq + t * c->k;
+        int32_t acc = 0;
+        for (size_t i = 0; i < c->k; i++) acc += (int32_t)qrow[i] * (int32_t)qx[i];
+        c->ys[t * c->n + row] = b + (float)acc * sw * c->xs[t];
+    }
+}
+
+void ojo_matmul_q8(const int8_t *wq, const float *wscale, size_t n, size_t k, const float *xs,
+                   size_t m, const float *bias, int threads, float *ys) { /* cpu_math.rs:187-274 */
+    int8_t *xq = (int8_t *)malloc(m * k);
+    float *sx = (float *)malloc(m * sizeof(float));
+    for (size_t t = 0; t < m; t++) sx[t] = ojo_quant_row_i8(xs + t * k, k, xq + t * k);
+    struct q8_ctx c = { wq, wscale, k, n, m, xq, sx, bias, ys };
+    int nt = (n * k * m < ((size_t)1 << 22)) ? 1 : threads; /* cpu_math.rs:202 */
+    steal_rows(n, 16, nt, q8_row, &c);
+    free(xq); free(sx);
+}
+
+/* ---------------------------------------------------------------- relayout */
+
+void ojo_relayout_q4k_q4l(const uint8_t *w, size_t k, size_t n, uint8_t *nib, uint16_t *qa,
+                          uint16_t *qb) { /* crates/ojas-formats/src/quant.rs:192-222 */
+    size_t nblk = k / 32, nsb = k / 256;
+    for (size_t r = 0; r < n; r++) {
+        for (size_t b = 0; b < nblk; b++) {
+            size_t sb = b >> 3; int j = (int)(b & 7);
+            int g = j >> 1, hi = j & 1;
+            const uint8_t *blk = w + (r * nsb + sb) * 144;
+            float d = rdh(blk, 0), dm = rdh(blk, 2);
+            uint8_t s_, m_;
+            scale_min_k4(j, blk + 4, &s_, &m_);
+            qa[r * nblk + b] = ojo_f32_to_f16(d * (float)s_);
+            qb[r * nblk + b] = ojo_f32_to_f16(-dm * (float)m_);
+            const uint8_t *qq = blk + 16 + g * 32;
+            for (int i = 0; i < 16; i++) {
+                uint8_t a = hi ? qq[2 * i] >> 4 : qq[2 * i] & 15;
+                uint8_t c = hi ? qq[2 * i + 1] >> 4 : qq[2 * i + 1] & 15;
+                nib[r * (k / 2) + b * 16 + i] = (uint8_t)(a | (c << 4));
+            }
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- double-precision reference */
+
+struct ref_ctx {
+    const uint8_t *raw; uint32_t ty; size_t n, k, m, row_bytes; int wmode;
+    const double *xd; double *y;
+};
+
+static void ref_row(void *p, size_t row) {
+    struct ref_ctx *c = (struct ref_ctx *)p;
+    double *w = (double *)malloc(c->k * sizeof(double));
+    const uint8_t *rb = c->raw + row * c->row_bytes;
+    if (c->wmode == 1) {
+        uint16_t *h = (uint16_t *)malloc(c->k * sizeof(uint16_t));
+        ojo_dequant_to_f16(rb, c->ty, c->k, h);
+        for (size_t i = 0; i < c->k; i++) w[i] = ojo_f16_to_f32(h[i]);
+        free(h);
+    } else {
+        ojo_dequant_to_f64(rb, c->ty, c->k, w);
+    }
+    for (size_t t = 0; t < c->m; t++) {
+        const double *x = c->xd + t * c->k;
+        double acc = 0.0;
+        for (size_t i = 0; i < c->k; i++) acc += w[i] * x[i];
+        c->y[t * c->n + row] = acc;
+    }
+    free(w);
+}
+
+int ojo_matmul_ref(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const float *x, size_t m,
+                   int wmode, int xmode, int threads, double *y) {
+    uint32_t bb, wpb;
+    if (!ojo_block_shape(ty, &bb, &wpb) || k % wpb) return -1;
+    double *xd = (double *)malloc(m * k * sizeof(double));
+    for (size_t i = 0; i < m * k; i++) {
+        float v = x[i];
+        if (xmode == 1) v = ojo_f16_to_f32(ojo_f32_to_f16(v));
+        else if (xmode == 2) v = ojo_bf16_to_f32(ojo_f32_to_bf16(v));
+        xd[i] = v;
+    }
+    struct ref_ctx c = { raw, ty, n, k, m, k / wpb * bb, wmode, xd, y };
+    steal_rows(n, 8, threads, ref_row, &c);
+    free(xd);
+    return 0;
+}
+
+/* ---------------------------------------------------------------- MoE */
+
+void ojo_moe_topk(const float *lg, int E, int ksel, uint32_t *idx, float *wgt) {
+    /* crates/ojas-cuda/src/kernels/moe.rs:45-70; crates/ojas-cuda/tests/conformance.rs:385-392 */
+    float *pr = (float *)malloc((size_t)E * sizeof(float));
+    float mx = -3.4028235e38f;
+    for (int e = 0; e < E; e++) if (lg[e] > mx) mx = lg[e];
+    float sum = 0.0f;
+    for (int e = 0; e < E; e++) { pr[e] = expf(lg[e] - mx); sum += pr[e]; }
+    for (int e = 0; e < E; e++) pr[e] = pr[e] / sum;
+    float wsum = 0.0f;
+    for (int j = 0; j < ksel; j++) {
+        float bv = -1.0f; int bi = 0;
+        for (int e = 0; e < E; e++) if (pr[e] > bv) { bv = pr[e]; bi = e; }
+        idx[j] = (uint32_t)bi;
+        wgt[j] = bv;
+        wsum += bv;
+        pr[bi] = -1.0f;
+    }
+    for (int j = 0; j < ksel; j++) wgt[j] = wgt[j] / wsum;
+    free(pr);
+}
+
+static inline float silu(float x) { return x / (1.0f + expf(-x)); } /* cpu_math.rs:486 */
+
+static int matvec_mode(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const float *x,
+                       int mode, int threads, float *y) {
+    if (mode == 0) return ojo_matvec_kq(raw, ty, n, k, x, threads, y);
+    double *yd = (double *)malloc(n * sizeof(double));
+    int rc = ojo_matmul_ref(raw, ty, n, k, x, 1, 0, 0, threads, yd);
+    for (size_t i = 0; i < n; i++) y[i] = (float)yd[i];
+    free(yd);
+    return rc;
+}
+
+int ojo_moe_ffn(const float *x, size_t T, size_t d, size_t n_ff, int n_expert, int ksel,
+                const uint32_t *idx, const float *wgt, const uint8_t *gate, const uint8_t *up,
+                uint32_t ty_gu, const uint8_t *down, uint32_t ty_d, int mode, int threads,
+                float *y) { /* crates/ojas-cpu/src/cpu_glm.rs:551-582 */
+    uint32_t bb_gu, w_gu, bb_d, w_d;
+    if (!ojo_block_shape(ty_gu, &bb_gu, &w_gu) || !ojo_block_shape(ty_d, &bb_d, &w_d)) return -1;
+    if (d % w_gu || n_ff % w_d) return -1;
+    size_t gu_bytes = n_ff * (d / w_gu) * bb_gu;  /* one expert's gate (or up) */
+    size_t dn_bytes = d * (n_ff / w_d) * bb_d;    /* one expert's down */
+    float *gv = (float *)malloc(n_ff * sizeof(float));
+    float *uv = (float *)malloc(n_ff * sizeof(float));
+    float *dv = (float *)malloc(d * sizeof(float));
+    int rc = 0;
+    for (size_t t = 0; t < T && !rc; t++) {
+        const float *xt = x + t * d;
+        for (int j = 0; j < ksel && !rc; j++) {
+            uint32_t e = idx[t * (size_t)ksel + j];
+            if ((int)e >= n_expert) { rc = -2; break; }
+            rc |= matvec_mode(gate + e * gu_bytes, ty_gu, n_ff, d, xt, mode, threads, gv);
+            rc |= matvec_mode(up + e * gu_bytes, ty_gu, n_ff, d, xt, mode, threads, uv);
+            for (size_t i = 0; i < n_ff; i++) gv[i] = silu(gv[i]) * uv[i];
+            rc |= matvec_mode(down + e * dn_bytes, ty_d, d, n_ff, gv, mode, threads, dv);
+            float w = wgt[t * (size_t)ksel + j];
+            for (size_t i = 0; i < d; i++) y[t * d + i] += w * dv[i];
+        }
+    }
+    free(gv); free(uv); free(dv);
+    return rc;
+}

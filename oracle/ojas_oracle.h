@@ -1,0 +1,113 @@
+/*
+ * TEST INFRASTRUCTURE — CPU restatement of the reference's quantized-matmul arithmetic.
+ *
+ * This library is the checker the HIP kernels are compared against.  It is never part of the
+ * shipped product path: only the test-suite, the smoke check and the CPU-baseline leg of the
+ * benchmark may load it.
+ *
+ * Every function cites the reference source (paths relative to the reference tree) whose
+ * arithmetic it restates.  Build with -ffp-contract=off: the reference is Rust, which never
+ * fuses a multiply with an add.
+ *
+ * How each function is pinned (a function without such a check would say "parity unpinned"):
+ *   dequant Q4_K/Q5_K/Q6_K  FNV-1a digests held by crates/ojas-formats/tests/quant_formats.rs:38-40
+ *   dequant Q8_0            closed form of crates/ojas-formats/tests/rows.rs:13-18
+ *   f16 <-> f32             the digests above + exhaustive comparison with IEEE binary16 (numpy)
+ *   quant_q8k               invariants (max|q|=127, bsums, half-away rounding, |x-s*q|<=s/2)
+ *   dot_q80                 f64 dot over the dequantized row, brute force at K=32
+ *   dot_q4k/q5k/q6k         identity dot(row, quant(x)) == sum dequant(row)*(scale*q) in f64,
+ *                           one-hot activations (pins nibble / sub-block order)
+ *   relayout_q4k_q4l        qa*nib+qb == dequant up to the two f16 roundings, one-hot blocks
+ *   moe_topk                softmax + stable sort closed form (numpy)
+ *   moe_ffn                 composition of the above
+ * The f32 association order inside dot_q4k / dot_q6k is pinned by the source text only; it
+ * moves the last ulp, far below the 1e-3 parity bar.
+ */
+#ifndef OJAS_ORACLE_H
+#define OJAS_ORACLE_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GGUF type ids (crates/ojas-formats/src/gguf.rs:563-591). */
+enum { OJO_Q8_0 = 8, OJO_Q4_K = 12, OJO_Q5_K = 13, OJO_Q6_K = 14 };
+
+/* IEEE binary16 <-> binary32, round-to-nearest-even, subnormals kept
+ * (crate half 2.7.1; call sites gguf.rs:602-608). */
+float    ojo_f16_to_f32(uint16_t h);
+uint16_t ojo_f32_to_f16(float f);
+/* bf16 round-to-nearest-even of an f32 (activation rounding of the prefill GEMM). */
+uint16_t ojo_f32_to_bf16(float f);
+float    ojo_bf16_to_f32(uint16_t h);
+
+/* (block bytes, weights per block); returns 0 on unknown type (synth.rs:12-21). */
+int ojo_block_shape(uint32_t ty, uint32_t *bytes, uint32_t *weights);
+
+/* Seeded synthetic blocks (crates/ojas-formats/src/synth.rs:29-64). out: nb*block_bytes. */
+int ojo_synth_blocks(uint32_t ty, size_t nb, uint8_t *out);
+
+/* dequant_to_f16 (gguf.rs:612-1116; arms :704-709, :1042-1059, :1060-1085, :1086-1108).
+ * n = number of weights; out = n binary16 bit patterns. */
+int ojo_dequant_to_f16(const uint8_t *b, uint32_t ty, size_t n, uint16_t *out);
+/* Same decoders evaluated exactly in double (no f32/f16 rounding), as
+ * crates/ojas-models/examples/q6k_gate.rs:60-110 does. */
+int ojo_dequant_to_f64(const uint8_t *b, uint32_t ty, size_t n, double *out);
+
+/* FNV-1a-64 over the ASCII of "%.6f" of every f16 value
+ * (crates/ojas-formats/tests/quant_formats.rs:20-31). */
+uint64_t ojo_digest_f16(const uint16_t *v, size_t n);
+
+/* quant_q8k (crates/ojas-cpu/src/cpu_math.rs:539-563). k need not be a multiple of 256;
+ * q has ceil(k/256)*256 entries, scales ceil(k/256), bsums ceil(k/256)*8. */
+void ojo_quant_q8k(const float *x, size_t k, float *scales, int8_t *q, int32_t *bsums);
+
+/* Row dots (cpu_math.rs:971-981, :609-635, :638-670, :674-722). */
+float ojo_dot_q80(const uint8_t *row, const float *x, size_t k);
+float ojo_dot_q4k(const uint8_t *row, size_t k, const float *scales, const int8_t *q, const int32_t *bsums);
+float ojo_dot_q5k(const uint8_t *row, size_t k, const float *scales, const int8_t *q, const int32_t *bsums);
+float ojo_dot_q6k(const uint8_t *row, size_t k, const float *scales, const int8_t *q, const int32_t *bsums);
+
+/* matvec_kq (cpu_math.rs:1145-1189): 8-row work stealing over `threads` workers. */
+int ojo_matvec_kq(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const float *x,
+                  int threads, float *y);
+
+/* Row-int8 path every dense CPU model runs (cpu_math.rs:174-179, :187-274, :404-415)
+ * and its load-time requantizer (crates/ojas-formats/src/quant.rs:16-39). */
+float ojo_quant_row_i8(const float *row, size_t k, int8_t *q);
+void  ojo_q8_rows_from_f16(const uint16_t *w16, size_t n, size_t k, int8_t *q, float *scale);
+void  ojo_matmul_q8(const int8_t *wq, const float *wscale, size_t n, size_t k,
+                    const float *xs, size_t m, const float *bias, int threads, float *ys);
+
+/* relayout_q4k_q4l (crates/ojas-formats/src/quant.rs:192-222). */
+void ojo_relayout_q4k_q4l(const uint8_t *w, size_t k, size_t n, uint8_t *nib, uint16_t *qa, uint16_t *qb);
+
+/* The GPU-test oracle: y = x * dequant(W)^T accumulated in double
+ * (crates/ojas-cuda/tests/conformance.rs:798-803, tests/prefill_gemm_q.rs:116-130).
+ *   wmode: 0 = weights exact (double), 1 = weights rounded to f16 as dequant_to_f16 stores them
+ *   xmode: 0 = x as given, 1 = x rounded to f16, 2 = x rounded to bf16
+ * x is [m][k] f32, y is [m][n] double. */
+int ojo_matmul_ref(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const float *x, size_t m,
+                   int wmode, int xmode, int threads, double *y);
+
+/* Router: softmax, ksel argmax passes with strict '>', lowest index wins, renormalise
+ * (crates/ojas-cuda/src/kernels/moe.rs:45-70; oracle crates/ojas-cuda/tests/conformance.rs:385-392). */
+void ojo_moe_topk(const float *logits, int n_expert, int ksel, uint32_t *idx, float *wgt);
+
+/* Expert FFN for T tokens (crates/ojas-cpu/src/cpu_glm.rs:551-582; silu cpu_math.rs:486):
+ * for each token t and slot j (in slot order): act = silu(Wg_e x) * (Wu_e x);
+ * y[t] += wgt[t][j] * (Wd_e act).   y must be initialised by the caller.
+ *   mode 0: every matvec is matvec_kq (int8 activations, the CPU path)
+ *   mode 1: every matvec is dequant-in-double dot (the GPU-test convention); y stays f32.
+ * gate/up: [E][n_ff][d] rows of type ty_gu; down: [E][d][n_ff] rows of type ty_d. */
+int ojo_moe_ffn(const float *x, size_t T, size_t d, size_t n_ff, int n_expert, int ksel,
+                const uint32_t *idx, const float *wgt,
+                const uint8_t *gate, const uint8_t *up, uint32_t ty_gu,
+                const uint8_t *down, uint32_t ty_d, int mode, int threads, float *y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

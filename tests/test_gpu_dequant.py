@@ -1,0 +1,66 @@
+"""Device decoders against the CPU oracle: dequantized weights must be bit-exact."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6}
+
+
+def _dequant(gpu, ty, raw, n):
+    rb = gpu.upload_bytes(raw)
+    out = gpu.alloc_bytes(n * 2)
+    gpu.dequant_f16(ty, rb, n, out)
+    return gpu.read(out, n, np.uint16)
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
+def test_reference_digests_on_device(gpu, orc, ty):
+    """The reference's own regression digests (crates/ojas-formats/tests/quant_formats.rs:38-40),
+    computed over what the GPU decoded."""
+    raw = orc.synth_blocks(ty, 40)
+    bits = _dequant(gpu, ty, raw, 10240)
+    assert orc.digest_f16(bits) == DIGESTS[ty]
+
+
+@pytest.mark.parametrize("ty,n,k", [(Q8_0, 37, 4096), (Q4_K, 129, 4096), (Q6_K, 65, 4096), (Q5_K, 16, 1024)])
+def test_bit_exact_on_benchmark_distributions(gpu, orc, pkg, ty, n, k):
+    raw = orc.synth_blocks(ty, n * k // pkg.synth.BLOCK_SHAPE[ty][1]) if ty == Q5_K else \
+        pkg.synth.weights(ty, n, k, "dq", ty)
+    got = _dequant(gpu, ty, raw, n * k)
+    assert np.array_equal(got, orc.dequant_to_f16(raw, ty, n * k))
+
+
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K])
+def test_bit_exact_with_extreme_scales(gpu, orc, pkg, ty):
+    """Subnormal, tiny, huge and negative f16 scales: every rounding path of the decoder."""
+    bb, wpb = pkg.synth.BLOCK_SHAPE[ty]
+    scales = np.array([0x0001, 0x0200, 0x03FF, 0x0400, 0x7BFF, 0x8001, 0xBC00, 0x3555, 0x0000, 0x1234], np.uint16)
+    nb = scales.size * 3
+    raw = orc.synth_blocks(ty, nb).reshape(nb, bb).copy()
+    off = 208 if ty == Q6_K else 0
+    for i in range(nb):
+        raw[i, off:off + 2] = np.array([scales[i % scales.size]], np.uint16).view(np.uint8)
+        if ty in (Q4_K, Q5_K):
+            raw[i, 2:4] = np.array([scales[(i * 7 + 3) % scales.size]], np.uint16).view(np.uint8)
+    raw = raw.reshape(-1)
+    got = _dequant(gpu, ty, raw, nb * wpb)
+    want = orc.dequant_to_f16(raw, ty, nb * wpb)
+    assert np.array_equal(got, want)
+
+
+def test_dequant_through_the_kernel_seam(gpu, orc):
+    """Same decoder reached by name through dispatch, with an offset into a larger buffer."""
+    gpu.ensure_family("dequant")
+    assert gpu.has_kernel("dequant_q4k_f16") and not gpu.has_kernel("dequant_q4k_f32")
+    raw = orc.synth_blocks(Q4_K, 24)
+    pad = 144 * 2
+    rb = gpu.upload_bytes(np.concatenate([np.full(pad, 0xEE, np.uint8), raw]))
+    out = gpu.upload_bytes(np.full(24 * 256 + 16, 0x7777, np.uint16))
+    grid, block = gpu.launch_shape("dequant_q4k_f16", 0, 24)
+    enc = gpu.begin()
+    gpu.dispatch(enc, "dequant_q4k_f16", [(rb, pad), (out, 16)], [24], grid, block)
+    gpu.submit(enc)
+    bits = gpu.read(out, 24 * 256 + 16, np.uint16)
+    assert np.all(bits[:8] == 0x7777) and np.all(bits[-8:] == 0x7777)
+    assert np.array_equal(bits[8:-8], orc.dequant_to_f16(raw, Q4_K, 24 * 256))

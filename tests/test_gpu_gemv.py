@@ -1,0 +1,208 @@
+"""Decode-step matvecs on the GPU against the CPU oracle.
+
+Two contracts, each against its own oracle:
+  * int8-activation kernels (gemv_q8k_*)  vs  matvec_kq, the CPU reference's arithmetic
+    (crates/ojas-cpu/src/cpu_math.rs:1145-1189): max|d| / max|ref| <= 1e-3 required, ~1e-6 seen;
+  * f32-activation kernels (gemv_nat_*)   vs  dequant-in-double dot, the reference's GPU-test
+    oracle (crates/ojas-cuda/tests/conformance.rs:798-823): its bound 2e-3, ours 1e-4.
+"""
+import numpy as np
+import pytest
+
+from conftest import peak_err
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+TAG = {Q8_0: "q80", Q4_K: "q4k", Q6_K: "q6k"}
+TOL_Q8K = 1e-3     # the parity bar against the CPU reference
+TOL_Q8K_SEEN = 2e-5
+TOL_FLOAT = 1e-4   # reference bound is 2e-3
+
+
+def _inputs(pkg, ty, n, k, tag):
+    return pkg.synth.weights(ty, n, k, "gemv", tag, ty, n, k), pkg.synth.normal_f32(k, "gemv", tag, "x", k)
+
+
+def test_quantize_q8k_is_bit_exact(gpu, orc, pkg):
+    for k, m in [(4096, 1), (14336, 3), (300, 2), (256, 1)]:
+        x = pkg.synth.normal_f32(m * k, "q8k", k, m).reshape(m, k)
+        x[0, :7] = [0.5, -0.5, 1.5, -2.5, 0.0, 1e-30, -1e-30]
+        if k >= 512:
+            x[-1, 256:512] = 0.0
+        nsb = (k + 255) // 256
+        xd = gpu.upload(x)
+        q, s = gpu.alloc_bytes(m * nsb * 256), gpu.alloc(m * nsb)
+        gpu.quant_q8k(xd, m, k, q, s)
+        gq = gpu.read(q, m * nsb * 256, np.int8).reshape(m, -1)
+        gs = gpu.read(s, m * nsb).reshape(m, -1)
+        for t in range(m):
+            ws, wq, _ = orc.quant_q8k(x[t])
+            assert np.array_equal(gs[t], ws), (k, t)
+            assert np.array_equal(gq[t], wq), (k, t)
+
+
+def test_quantize_q8k_bf16_input(gpu, orc, pkg):
+    k, m = 4096, 2
+    xb = pkg.synth.to_bf16_bits(pkg.synth.normal_f32(m * k, "q8kb"))
+    xd = gpu.upload_bytes(xb)
+    q, s = gpu.alloc_bytes(m * 16 * 256), gpu.alloc(m * 16)
+    gpu.quant_q8k(xd, m, k, q, s, x_dtype=pkg.X_BF16)
+    xf = pkg.synth.bf16_bits_to_f32(xb).reshape(m, k)
+    gq = gpu.read(q, m * k, np.int8).reshape(m, k)
+    for t in range(m):
+        ws, wq, _ = orc.quant_q8k(xf[t])
+        assert np.array_equal(gq[t], wq)
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+@pytest.mark.parametrize("n,k", [(13, 256), (64, 512), (1024, 4096), (333, 2560), (96, 14336), (4099, 4096)])
+def test_q8k_matvec_matches_cpu_reference(gpu, orc, pkg, ty, n, k):
+    w, x = _inputs(pkg, ty, n, k, "a")
+    lin = gpu.lin(ty, n, k, w)
+    xd, yd = gpu.upload(x), gpu.upload(np.full(n + 2, 12345.0, np.float32))
+    gpu.mm(xd, lin, yd, 1, False, act_mode=pkg.ACT_Q8K, y_off=4)
+    got = gpu.read(yd, n + 2)
+    assert got[0] == 12345.0 and got[-1] == 12345.0, "wrote outside y"
+    want = orc.matvec_kq(w, ty, n, k, x)
+    err = peak_err(got[1:-1], want)
+    assert err <= TOL_Q8K_SEEN <= TOL_Q8K, err
+
+
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("n,k", [(13, 2560), (1024, 4096), (96, 14336), (4099, 4096)])
+def test_float_matvec_matches_dequant_dot(gpu, orc, pkg, ty, n, k):
+    w, x = _inputs(pkg, ty, n, k, "b")
+    lin = gpu.lin(ty, n, k, w)
+    xd, yd = gpu.upload(x), gpu.upload(np.full(n + 2, 12345.0, np.float32))
+    gpu.mm(xd, lin, yd, 1, False, act_mode=pkg.ACT_FLOAT, y_off=4)
+    got = gpu.read(yd, n + 2)
+    assert got[0] == 12345.0 and got[-1] == 12345.0
+    want = orc.matmul_ref(w, ty, n, k, x)[0]
+    assert peak_err(got[1:-1], want) <= TOL_FLOAT
+    # the reference's own oracle rounds each weight to f16 first; its bound is 2e-3
+    want16 = orc.matmul_ref(w, ty, n, k, x, wmode=1)[0]
+    assert peak_err(got[1:-1], want16) <= 2e-3
+
+
+def test_q80_matvec_matches_dot_q80(gpu, orc, pkg):
+    """Config 0: Q8_0 4096x4096 against the CPU path `dot_q80` (f32 activations)."""
+    n = k = 4096
+    w, x = _inputs(pkg, Q8_0, n, k, "c0")
+    lin = gpu.lin(Q8_0, n, k, w)
+    xd, yd = gpu.upload(x), gpu.alloc(n)
+    gpu.mm(xd, lin, yd, 1)
+    want = orc.matvec_kq(w, Q8_0, n, k, x)
+    assert peak_err(gpu.read(yd, n), want) <= 1e-5
+
+
+def test_q80_closed_form_rows_with_guards(gpu, pkg):
+    """crates/ojas-metal/tests/dispatch.rs:357-429: K=2560, N=13, output between sentinels,
+    absolute tolerance 2e-4 against an f64 loop over the same bytes."""
+    n, k = 13, 2560
+    w, x = pkg.synth.q80_rows_closed_form(n, k)
+    blocks = w.reshape(n, k // 32, 34)
+    d = blocks[:, :, 0:2].copy().view(np.float16).astype(np.float64)[:, :, 0]
+    q = blocks[:, :, 2:].view(np.int8).astype(np.float64)
+    want = np.einsum("rb,rbj,bj->r", d, q, x.astype(np.float64).reshape(-1, 32))
+    lin = gpu.lin(Q8_0, n, k, w)
+    yd = gpu.upload(np.full(n + 4, 12345.0, np.float32))
+    gpu.mm(gpu.upload(x), lin, yd, 1, y_off=8)
+    got = gpu.read(yd, n + 4)
+    assert np.all(got[:2] == 12345.0) and np.all(got[-2:] == 12345.0)
+    assert np.max(np.abs(got[2:-2] - want)) < 2e-4
+
+
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("mode", ["float", "q8k"])
+def test_bias_accum_and_batched_variants(gpu, orc, pkg, ty, mode):
+    """The five checks of crates/ojas-models/examples/nat_gemv_gate.rs:36-163: plain, bias
+    (1000 + i), accumulate onto a seeded y, batched M=3 with different rows, batched accumulate."""
+    if ty == Q8_0 and mode == "q8k":
+        pytest.skip("Q8_0 keeps f32 activations in the CPU reference")
+    n, k, m = 200, 1024, 3
+    w = pkg.synth.weights(ty, n, k, "var", ty)
+    xs = pkg.synth.normal_f32(m * k, "var", "x").reshape(m, k)
+    act = pkg.ACT_FLOAT if mode == "float" else pkg.ACT_Q8K
+    if mode == "float":
+        ref = orc.matmul_ref(w, ty, n, k, xs).astype(np.float32)
+        tol = TOL_FLOAT
+    else:
+        ref = np.stack([orc.matvec_kq(w, ty, n, k, xs[t]) for t in range(m)])
+        tol = TOL_Q8K_SEEN
+    lin = gpu.lin(ty, n, k, w)
+    xd = gpu.upload(xs)
+    peak = np.max(np.abs(ref))
+    # bias
+    bias = (1000.0 + np.arange(n)).astype(np.float32)
+    yd = gpu.alloc(n)
+    gpu.mm(xd, lin, yd, 1, act_mode=act, bias=gpu.upload(bias))
+    assert np.max(np.abs(gpu.read(yd, n) - (ref[0] + bias))) <= tol * peak + 1e-3
+    # accumulate
+    y0 = pkg.synth.normal_f32(n, "var", "y0")
+    yd = gpu.upload(y0)
+    gpu.mm(xd, lin, yd, 1, True, act_mode=act)
+    assert np.max(np.abs(gpu.read(yd, n) - (ref[0] + y0))) <= tol * peak + 1e-5
+    # batched, then batched accumulate; nothing written past row M
+    for accum in (False, True):
+        y0 = pkg.synth.normal_f32(m * n, "var", "ym").reshape(m, n) if accum else np.zeros((m, n), np.float32)
+        init = np.concatenate([y0.ravel(), np.full(n, 12345.5, np.float32)])
+        yd = gpu.upload(init)
+        gpu.mm(xd, lin, yd, m, accum, act_mode=act)
+        got = gpu.read(yd, m * n + n)
+        assert np.all(got[m * n:] == 12345.5), "wrote past row M"
+        assert np.max(np.abs(got[:m * n].reshape(m, n) - (ref + y0))) <= tol * peak + 1e-5
+
+
+@pytest.mark.parametrize("m", [1, 2, 4, 5, 8, 16])
+def test_small_m_verify_shapes(gpu, orc, pkg, m):
+    """Speculative-verify widths on a Q6_K head slice with bf16 activations."""
+    n, k = 777, 4096
+    w = pkg.synth.q6k_weights(n, k, "verify", "w")
+    xb = pkg.synth.to_bf16_bits(pkg.synth.normal_f32(m * k, "verify", "x", m))
+    xf = pkg.synth.bf16_bits_to_f32(xb).reshape(m, k)
+    lin = gpu.lin(Q6_K, n, k, w)
+    yd = gpu.alloc(m * n)
+    gpu.mm(gpu.upload_bytes(xb), lin, yd, m, x_dtype=pkg.X_BF16, act_mode=pkg.ACT_Q8K)
+    got = gpu.read(yd, m * n).reshape(m, n)
+    want = np.stack([orc.matvec_kq(w, Q6_K, n, k, xf[t]) for t in range(m)])
+    assert peak_err(got, want) <= TOL_Q8K_SEEN
+
+
+def test_kernel_seam_dispatch_by_name(gpu, orc, pkg):
+    """gemv_nat_q4k through ensure_family / has_kernel / launch_shape / dispatch / submit."""
+    gpu.ensure_family("gemv")
+    n, k = 130, 2048
+    w, x = _inputs(pkg, Q4_K, n, k, "seam")
+    wd, xd, yd = gpu.upload_bytes(w), gpu.upload(x), gpu.alloc(n)
+    for name in ("gemv_nat_q4k", "gemv_nat_q4k_r1", "gemv_nat_q4k_r2"):
+        assert gpu.has_kernel(name)
+        grid, block = gpu.launch_shape(name, k, n)
+        enc = gpu.begin()
+        gpu.memset0(yd)
+        gpu.dispatch(enc, name, [(xd, 0), (wd, 0), (yd, 0)], [k, n], grid, block)
+        gpu.submit(enc)
+        assert peak_err(gpu.read(yd, n), orc.matmul_ref(w, Q4_K, n, k, x)[0]) <= TOL_FLOAT
+
+
+def test_errors_are_reported_not_launched(gpu, pkg):
+    gpu.ensure_family("gemv")
+    n, k = 64, 512
+    wd = gpu.alloc_bytes(n * pkg.row_bytes(Q4_K, k))
+    xd, yd = gpu.alloc(k), gpu.alloc(n)
+    grid, block = gpu.launch_shape("gemv_nat_q4k", k, n)
+    enc = gpu.begin()
+    with pytest.raises(pkg.OjasHipError, match="not loaded"):
+        gpu.dispatch(enc, "gemv_nat_q9k", [(xd, 0), (wd, 0), (yd, 0)], [k, n], grid, block)
+    with pytest.raises(pkg.OjasHipError, match="needs"):   # y too small for N
+        gpu.dispatch(enc, "gemv_nat_q4k", [(xd, 0), (wd, 0), (yd, 0)], [k, n + 1], grid, block)
+    with pytest.raises(pkg.OjasHipError, match="multiple of 256"):
+        gpu.dispatch(enc, "gemv_nat_q4k", [(xd, 0), (wd, 0), (yd, 0)], [k - 32, n], grid, block)
+    with pytest.raises(pkg.OjasHipError, match="covers"):
+        gpu.dispatch(enc, "gemv_nat_q4k", [(xd, 0), (wd, 0), (yd, 0)], [k, n], [1, 1, 1], block)
+    with pytest.raises(pkg.OjasHipError, match="takes 3 buffers"):
+        gpu.dispatch(enc, "gemv_nat_q4k", [(xd, 0), (wd, 0)], [k, n], grid, block)
+    with pytest.raises((pkg.OjasHipError, ValueError)):
+        gpu.lin(Q4_K, 4, 100, np.zeros(4, np.uint8))
+    with pytest.raises(pkg.OjasHipError, match="unknown kernel family"):
+        gpu.ensure_family("attn")
+    gpu.submit(enc)

@@ -1,0 +1,302 @@
+"""Pins the CPU oracle: golden vectors the reference's own tests hold, closed forms, invariants and
+brute force — each chosen so that a dropped term, a wrong index or a transposed nibble fails."""
+import numpy as np
+import pytest
+
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+
+# crates/ojas-formats/tests/quant_formats.rs:38-40
+DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6}
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
+def test_dequant_digest_matches_reference(orc, ty):
+    raw = orc.synth_blocks(ty, 40)
+    bits = orc.dequant_to_f16(raw, ty, 40 * 256)
+    assert bits.size == 10240
+    assert orc.digest_f16(bits) == DIGESTS[ty]
+
+
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K])
+def test_synth_blocks_two_implementations_agree(orc, pkg, ty):
+    assert np.array_equal(orc.synth_blocks(ty, 9), pkg.synth.synth_blocks(ty, 9))
+
+
+def test_f16_to_f32_exhaustive(orc):
+    L = orc.lib()
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([L.ojo_f16_to_f32(int(b)) for b in bits], np.float32)
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.all(np.isnan(got[np.isnan(want)]))
+
+
+def test_f32_to_f16_round_to_nearest_even(orc):
+    L = orc.lib()
+    rng = np.random.default_rng(1)
+    # every f16 value, every midpoint between neighbours, and random f32 across all exponents
+    h = np.arange(0x7C00, dtype=np.uint16).view(np.float16).astype(np.float64)
+    mids = ((h[:-1] + h[1:]) / 2).astype(np.float32)
+    rnd = (rng.standard_normal(20000) * np.exp2(rng.integers(-30, 18, 20000))).astype(np.float32)
+    tiny = (rng.standard_normal(5000) * 2.0 ** -24).astype(np.float32)
+    special = np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e9, -1e9, np.inf, -np.inf, 2.0 ** -25,
+                        2.0 ** -25 * 1.0000001, 2.0 ** -24, 6.1e-5], np.float32)
+    xs = np.concatenate([h.astype(np.float32), mids, -mids, rnd, tiny, special])
+    with np.errstate(over="ignore"):
+        want = xs.astype(np.float16).view(np.uint16)
+    got = np.array([L.ojo_f32_to_f16(float(v)) for v in xs], np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_bf16_rounding(orc, pkg):
+    L = orc.lib()
+    xs = np.random.default_rng(2).standard_normal(4000).astype(np.float32)
+    got = np.array([L.ojo_f32_to_bf16(float(v)) for v in xs], np.uint16)
+    assert np.array_equal(got, pkg.synth.to_bf16_bits(xs))
+    # ties go to even: 1 + 2^-8 is exactly between two bf16 values
+    assert L.ojo_f32_to_bf16(1.0 + 2.0 ** -8) == 0x3F80
+    assert L.ojo_f32_to_bf16(1.0 + 3 * 2.0 ** -8) == 0x3F82
+
+
+def test_q80_table_closed_form(orc, pkg):
+    """crates/ojas-formats/tests/rows.rs:13-18: d = 0.25 (r+1), q_j = j - 16 + r — all exact."""
+    raw, want = pkg.synth.q80_rows_table()
+    got = orc.dequant_to_f16(raw, Q8_0, 96).view(np.float16).astype(np.float32).reshape(3, 32)
+    assert np.array_equal(got, want)
+
+
+def _q4k_block(d, dmin, sc, mn, qs, pkg):
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = np.array([d], np.float16).view(np.uint8)
+    blk[2:4] = np.array([dmin], np.float16).view(np.uint8)
+    blk[4:16] = pkg.synth.pack_scales_k4(np.array([sc]), np.array([mn]))[0]
+    blk[16:] = qs
+    return blk
+
+
+def test_q4k_closed_forms(orc, pkg):
+    # all-zero quants => w = -dmin * m_j, constant per sub-block, in sub-block order
+    mn = np.arange(8) * 7 + 3
+    blk = _q4k_block(0.5, 0.25, np.full(8, 9), mn, np.zeros(128, np.uint8), pkg)
+    w = orc.dequant_to_f16(blk, Q4_K, 256).view(np.float16).astype(np.float32).reshape(8, 32)
+    assert np.array_equal(w, np.repeat((-0.25 * mn).astype(np.float32)[:, None], 32, 1))
+    # sc = 1, m = 0 => w = d * nibble; low nibbles feed sub-block 2c, high nibbles 2c+1
+    qs = np.random.default_rng(3).integers(0, 256, 128, dtype=np.uint8)
+    blk = _q4k_block(2.0, 1.0, np.ones(8), np.zeros(8), qs, pkg)
+    w = orc.dequant_to_f16(blk, Q4_K, 256).view(np.float16).astype(np.float32).reshape(4, 2, 32)
+    q = qs.reshape(4, 32)
+    assert np.array_equal(w[:, 0], 2.0 * (q & 15))
+    assert np.array_equal(w[:, 1], 2.0 * (q >> 4))
+    # scales with the top bits set exercise the j >= 4 packing
+    sc = np.array([1, 2, 3, 4, 63, 48, 33, 17])
+    blk = _q4k_block(1.0, 1.0, sc, sc[::-1].copy(), np.full(128, 0x11, np.uint8), pkg)
+    w = orc.dequant_to_f16(blk, Q4_K, 256).view(np.float16).astype(np.float32).reshape(8, 32)
+    assert np.array_equal(w[:, 0], (sc - sc[::-1]).astype(np.float32))
+
+
+def test_q6k_closed_forms(orc):
+    blk = np.zeros(210, np.uint8)
+    blk[208:210] = np.array([1.0], np.float16).view(np.uint8)
+    blk[192:208] = np.arange(1, 17, dtype=np.int8).view(np.uint8)
+    # code 32 (ql nibble 0, qh bits = 2) decodes to 0
+    blk[0:128] = 0
+    blk[128:192] = 0xAA
+    assert not orc.dequant_to_f16(blk, Q6_K, 256).any()
+    # code 33 => w = d * sc[sub]; sub-scales apply per 16 weights in element order
+    blk[0:128] = 0x11
+    w = orc.dequant_to_f16(blk, Q6_K, 256).view(np.float16).astype(np.float32)
+    assert np.array_equal(w, np.repeat(np.arange(1, 17, dtype=np.float32), 16))
+    # a single byte of ql / qh lands where the layout says
+    blk[0:192] = 0
+    blk[5] = 0xF0           # ql[5] high nibble -> weight 64+5 of the first half
+    blk[128 + 32 + 7] = 0x0C  # qh[7] of the second half, bits 2..3 -> weight 128+32+7
+    w = orc.dequant_to_f64(blk, Q6_K, 256)
+    base = -32.0 * np.repeat(np.arange(1, 17, dtype=np.float64), 16)
+    delta = w - base
+    assert delta[64 + 5] == 15 * 5.0 and delta[128 + 32 + 7] == 48 * 11.0
+    assert np.count_nonzero(delta) == 2
+
+
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K])
+def test_dequant_f64_rounds_to_the_f16_decoder(orc, pkg, ty):
+    raw = orc.synth_blocks(ty, 12)
+    n = 12 * pkg.synth.BLOCK_SHAPE[ty][1]
+    exact = orc.dequant_to_f64(raw, ty, n)
+    f16 = orc.dequant_to_f16(raw, ty, n).view(np.float16).astype(np.float64)
+    # the f16 decoder rounds twice (f32 then f16): within one f16 ulp of the exact value
+    assert np.all(np.abs(f16 - exact) <= np.maximum(np.abs(exact) * 2.0 ** -10, 2.0 ** -24))
+
+
+def test_quant_q8k_invariants(orc):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(1024).astype(np.float32)
+    x[256:512] = 0.0                      # all-zero segment => scale 1, q 0
+    s, q, b = orc.quant_q8k(x)
+    assert s[1] == 1.0 and not q[256:512].any()
+    for sb in (0, 2, 3):
+        seg = x[sb * 256:(sb + 1) * 256]
+        assert s[sb] == np.float32(np.max(np.abs(seg))) / np.float32(127.0)
+        assert np.max(np.abs(q[sb * 256:(sb + 1) * 256])) == 127
+        assert np.all(np.abs(seg - s[sb] * q[sb * 256:(sb + 1) * 256]) <= s[sb] * 0.5000001)
+    assert np.array_equal(b, q.astype(np.int32).reshape(-1, 32).sum(1))
+    # ties round away from zero: amax = 127 makes scale 1, so x = +-2.5 must give +-3
+    x = np.zeros(256, np.float32)
+    x[0], x[1], x[2], x[3] = 127.0, 2.5, -2.5, 0.49999997
+    _, q, _ = orc.quant_q8k(x)
+    assert list(q[:4]) == [127, 3, -3, 0]
+    # ragged tail: K = 300 quantizes the 44-element tail on its own scale, pads with zero
+    x = rng.standard_normal(300).astype(np.float32)
+    s, q, b = orc.quant_q8k(x)
+    assert s.size == 2 and q.size == 512 and not q[300:].any()
+    assert s[1] == np.float32(np.max(np.abs(x[256:]))) / np.float32(127.0)
+
+
+def test_dot_q80_matches_f64_dot(orc, pkg):
+    n, k = 7, 320
+    raw = pkg.synth.q80_weights(n, k, "t", "q80")
+    x = pkg.synth.normal_f32(k, "t", "x")
+    w = orc.dequant_to_f64(raw, Q8_0, n * k).reshape(n, k)
+    want = w @ x.astype(np.float64)
+    got = np.array([orc.dot_q80(raw[r * 340:(r + 1) * 340], x) for r in range(n)])
+    assert np.max(np.abs(got - want)) <= 1e-6 * np.max(np.abs(want))
+    # brute force on one block, in the reference's order: sum = d * (sequential f32 acc)
+    blk = raw[:34]
+    acc = np.float32(0)
+    for j in range(32):
+        acc = np.float32(acc + np.float32(np.int8(blk[2 + j])) * x[j])
+    d = blk[0:2].view(np.float16).astype(np.float32)[0]
+    assert orc.dot_q80(blk, x[:32]) == np.float32(d * acc)
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
+def test_kquant_dot_equals_dequant_dot_on_quantized_activations(orc, pkg, ty):
+    """dot_<fmt>(row, quant_q8k(x)) == sum dequant(row) * (scale * q), evaluated in double."""
+    n, k = 6, 1024
+    bb = pkg.synth.BLOCK_SHAPE[ty][0]
+    raw = orc.synth_blocks(ty, n * k // 256)
+    x = pkg.synth.normal_f32(k, "t", "xk", ty)
+    act = orc.quant_q8k(x)
+    xq = (np.repeat(act[0].astype(np.float64), 256) * act[1].astype(np.float64))
+    w = orc.dequant_to_f64(raw, ty, n * k).reshape(n, k)
+    want = w @ xq
+    rb = k // 256 * bb
+    got = np.array([orc.dot_kq(ty, raw[r * rb:(r + 1) * rb], k, act) for r in range(n)])
+    assert np.max(np.abs(got - want)) <= 2e-6 * np.max(np.abs(want))
+    y = orc.matvec_kq(raw, ty, n, k, x, threads=3)
+    assert np.array_equal(y, got.astype(np.float32))
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
+def test_kquant_dot_one_hot_selects_the_weight(orc, pkg, ty):
+    """x = e_i quantizes to scale 1/127, q_i = 127, so the dot returns w_i: pins element order."""
+    k = 512
+    bb = pkg.synth.BLOCK_SHAPE[ty][0]
+    raw = orc.synth_blocks(ty, 2)
+    w = orc.dequant_to_f64(raw, ty, k)
+    for i in [0, 1, 15, 16, 31, 32, 33, 63, 64, 100, 127, 128, 129, 200, 255, 256, 300, 511]:
+        x = np.zeros(k, np.float32)
+        x[i] = 1.0
+        got = orc.dot_kq(ty, raw[:2 * bb], k, orc.quant_q8k(x))
+        assert abs(got - w[i]) <= 1e-6 * max(abs(w[i]), 1e-3), (ty, i)
+
+
+def test_dot_q4k_brute_force_association(orc, pkg):
+    """One super-block, restated term by term in f32 in the reference's order."""
+    raw = orc.synth_blocks(Q4_K, 1)
+    x = pkg.synth.normal_f32(256, "bf")
+    s, q, b = orc.quant_q8k(x)
+    d, dmin = raw[0:4].view(np.float16).astype(np.float32)
+    sc = raw[4:16]
+    f = np.float32
+    sumd = f(0)
+    summ = f(0)
+    for c in range(4):
+        qq = raw[16 + 32 * c:48 + 32 * c]
+        def sm(j):
+            if j < 4:
+                return sc[j] & 63, sc[j + 4] & 63
+            return (sc[j + 4] & 15) | ((sc[j - 4] >> 6) << 4), (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4)
+        s1, m1 = sm(2 * c)
+        s2, m2 = sm(2 * c + 1)
+        il = int(np.dot((qq & 15).astype(np.int32), q[64 * c:64 * c + 32].astype(np.int32)))
+        ih = int(np.dot((qq >> 4).astype(np.int32), q[64 * c + 32:64 * c + 64].astype(np.int32)))
+        sumd = f(sumd + f(f(s1) * f(il)))
+        sumd = f(sumd + f(f(s2) * f(ih)))
+        summ = f(summ + f(f(f(m1) * f(b[2 * c])) + f(f(m2) * f(b[2 * c + 1]))))
+    want = f(s[0] * f(f(d * sumd) - f(dmin * summ)))
+    assert orc.dot_kq(Q4_K, raw, 256, (s, q, b)) == want
+
+
+def test_relayout_q4k_q4l(orc):
+    n, k = 3, 512
+    raw = orc.synth_blocks(Q4_K, n * k // 256)
+    nib, qa, qb = orc.relayout_q4k_q4l(raw, k, n)
+    lo, hi = nib & 15, nib >> 4
+    codes = np.stack([lo, hi], 1).reshape(n, k)          # element 2i low nibble, 2i+1 high
+    a = np.repeat(qa.view(np.float16).astype(np.float64), 32).reshape(n, k)
+    b = np.repeat(qb.view(np.float16).astype(np.float64), 32).reshape(n, k)
+    w = orc.dequant_to_f64(raw, Q4_K, n * k).reshape(n, k)
+    # qa, qb carry one f16 rounding each
+    assert np.all(np.abs(a * codes + b - w) <= 2.0 ** -10 * (np.abs(a) * 15 + np.abs(b)) + 1e-12)
+    # and the codes are exactly the nibbles in element order (d = 1/sc trick: compare to exact codes)
+    exact = np.empty((n, k), np.int64)
+    blocks = raw.reshape(-1, 144)
+    for i, blk in enumerate(blocks):
+        q = blk[16:].reshape(4, 32)
+        exact.reshape(-1, 256)[i] = np.stack([q & 15, q >> 4], 1).reshape(256)
+    assert np.array_equal(codes, exact)
+
+
+def test_moe_topk_matches_closed_form(orc, pkg):
+    """crates/ojas-cuda/tests/conformance.rs:380-408: E=64, K=8, tvec(64, 51)."""
+    lg = pkg.synth.tvec(64, 51)
+    idx, wgt = orc.moe_topk(lg[None, :], 8)
+    ex = np.exp(lg.astype(np.float64) - lg.max())
+    p = ex / ex.sum()
+    order = sorted(range(64), key=lambda i: (-p[i], i))[:8]
+    assert list(idx[0]) == order
+    assert np.max(np.abs(wgt[0] - p[order] / p[order].sum())) < 1e-6
+    assert abs(float(wgt[0].sum()) - 1.0) < 1e-6
+    # ties resolve to the lowest index
+    idx, _ = orc.moe_topk(np.zeros((1, 16), np.float32), 4)
+    assert list(idx[0]) == [0, 1, 2, 3]
+
+
+def test_matmul_q8_row_int8_path(orc):
+    rng = np.random.default_rng(7)
+    n, k, m = 9, 64, 3
+    w = rng.standard_normal((n, k)).astype(np.float16)
+    wq, ws = orc.q8_rows_from_f16(w.view(np.uint16), n, k)
+    amax = np.abs(w.astype(np.float32)).max(1)
+    assert np.array_equal(ws, amax / np.float32(127.0))
+    assert np.all(np.abs(wq.reshape(n, k)).max(1) == 127)
+    xs = rng.standard_normal((m, k)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    ys = orc.matmul_q8(wq, ws, n, k, xs, bias)
+    for t in range(m):
+        q, s = orc.quant_row_i8(xs[t])
+        acc = wq.reshape(n, k).astype(np.int64) @ q.astype(np.int64)
+        want = bias + acc.astype(np.float32) * ws * np.float32(s)
+        assert np.array_equal(ys[t], want.astype(np.float32))
+
+
+def test_moe_ffn_is_the_composition(orc, pkg):
+    E, d, nff, ksel, T = 4, 256, 256, 2, 3
+    gate = pkg.synth.q4k_weights(E * nff, d, "m", "g")
+    up = pkg.synth.q4k_weights(E * nff, d, "m", "u")
+    down = pkg.synth.q4k_weights(E * d, nff, "m", "d")
+    x = pkg.synth.normal_f32(T * d, "m", "x").reshape(T, d)
+    idx, wgt = orc.moe_topk(pkg.synth.normal_f32(T * E, "m", "lg").reshape(T, E), ksel)
+    y = orc.moe_ffn(x, idx, wgt, gate, up, Q4_K, down, Q4_K, E, nff, mode=0)
+    gb = nff * d // 256 * 144
+    want = np.zeros((T, d), np.float32)
+    for t in range(T):
+        for j in range(ksel):
+            e = int(idx[t, j])
+            g = orc.matvec_kq(gate[e * gb:(e + 1) * gb], Q4_K, nff, d, x[t])
+            u = orc.matvec_kq(up[e * gb:(e + 1) * gb], Q4_K, nff, d, x[t])
+            with np.errstate(over="ignore"):
+                act = (g / (np.float32(1) + np.exp(-g, dtype=np.float32))) * u
+            dv = orc.matvec_kq(down[e * gb:(e + 1) * gb], Q4_K, d, nff, act.astype(np.float32))
+            want[t] += wgt[t, j] * dv
+    assert np.max(np.abs(y - want)) <= 2e-6 * np.max(np.abs(want))
