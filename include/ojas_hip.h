@@ -64,6 +64,7 @@ enum { OJH_ACT_AUTO = 0, OJH_ACT_Q8K = 1, OJH_ACT_FLOAT = 2 };
 typedef struct ojh_device ojh_device; /* one GPU + one stream + loaded families */
 typedef struct ojh_buf ojh_buf;       /* device allocation with a known size */
 typedef struct ojh_lin ojh_lin;       /* a weight matrix W[N,K] in its GGUF block bytes */
+typedef struct ojh_graph ojh_graph;   /* a recorded chain of dispatches, replayable */
 
 /* Mirrors `Caps` (crates/ojas-core/src/kernel.rs:26-41). */
 typedef struct ojh_caps {
@@ -128,6 +129,19 @@ int ojh_dispatch(ojh_device *dev, const char *name, int n_bufs, ojh_buf *const *
                  const uint32_t grid[3], const uint32_t block[3]);
 /* `submit(enc)`: wait for everything dispatched so far. */
 int ojh_submit(ojh_device *dev);
+
+/* Record-and-replay of a chain of dispatches (the reference's encoder is a chain submitted as a
+ * unit, crates/ojas-core/src/kernel.rs:73-80; its `Caps.features` names "cuda_graphs" for the
+ * same purpose, :38-40).  Between begin and end every dispatch / ojh_mm* / ojh_quant_q8k call is
+ * recorded instead of run; calls that synchronise or allocate (alloc, free, upload, download,
+ * submit, a scratch buffer that has to grow) fail with OJH_ERR_ARG — run the chain once eagerly
+ * first.  `ojh_graph_launch` replays the chain on the device's stream with one host call: by
+ * default from a native loop over the recorded launches, or as an instantiated hipGraph when
+ * OJAS_HIP_REPLAY=graph is set in the environment at `ojh_capture_begin`. */
+int ojh_capture_begin(ojh_device *dev);
+int ojh_capture_end(ojh_device *dev, ojh_graph **out);
+int ojh_graph_launch(ojh_device *dev, ojh_graph *graph);
+int ojh_graph_free(ojh_device *dev, ojh_graph *graph);
 
 /* Event timing on the device's stream (the reference times kernels the same way,
  * crates/ojas-cuda/tests/prefill_gemm_q.rs:262-283). `ojh_timer_stop` synchronises. */

@@ -29,6 +29,7 @@ FAMILIES = {
     "dequant": ("dequant.hip", ["-ffp-contract=off"]),
     "gemv": ("gemv.hip", []),
     "gemv_q8k": ("gemv_q8k.hip", []),
+    "glue": ("glue.hip", []),
     "gemm": ("gemm.hip", []),
     "moe": ("moe.hip", []),
 }

@@ -11,7 +11,11 @@
 //   dequant_<fmt>_f16(const uchar* w, ushort* out, uint nblocks)
 #include "ojk_common.h"
 
+// The f32 value is pinned in a register before the conversion: left to itself the compiler folds
+// "multiply, then convert" into one mixed-precision FMA, which rounds once instead of twice and
+// loses the sign of a zero product.
 __device__ __forceinline__ ushort f32_to_f16_bits(float v) {
+    asm volatile("" : "+v"(v));
     return __half_as_ushort(__float2half_rn(v));
 }
 

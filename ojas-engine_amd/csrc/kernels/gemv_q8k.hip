@@ -6,7 +6,10 @@
 // :674-722 (dot_q6k), :1145-1189 (matvec_kq).
 //
 //   quantize_q8k{,_bf16}(x, q, scales, K, M)             grid (ceil(K/256), M), block 256
-//   gemv_q8k_<fmt>{,_accum,_bias}(xq, xs, w, y[, bs], K, N)
+//   gemv_q8k_<fmt>{,_accum,_bias}(xq, xs, w, y[, bs], K, N)   4 rows per wave
+//   gemv_q8k_<fmt>_r1 / _r2 (same arguments)                  1 / 2 rows per wave
+//   gemv_q8k_<fmt>_wide (same arguments)                      2 rows per wave; the entry the op
+//                                                             seam uses for output-head sized N
 //   gemv_q8k_<fmt>_m(xq, xs, w, y, K, N, M, ACC)          y[M][N], one weight pass per MT tokens
 //
 // Integer sums are exact, so  sum_j sc_j*idot_j  and  sum_j m_j*bsum_j  are formed in int32 and
@@ -147,6 +150,9 @@ __device__ __forceinline__ void gemv_q8k_q4k_body(const signed char* __restrict_
         const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N) {                  \
         BODY<1, ST_SET>(xq, xs, w, y, nullptr, K, N); }                                                      \
     extern "C" __global__ void __launch_bounds__(256) gemv_q8k_##FMT##_r2(                                   \
+        const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N) {                  \
+        BODY<2, ST_SET>(xq, xs, w, y, nullptr, K, N); }                                                      \
+    extern "C" __global__ void __launch_bounds__(256) gemv_q8k_##FMT##_wide(                                 \
         const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N) {                  \
         BODY<2, ST_SET>(xq, xs, w, y, nullptr, K, N); }                                                      \
     extern "C" __global__ void __launch_bounds__(256) gemv_q8k_##FMT(                                        \

@@ -1,0 +1,54 @@
+// Family "glue": element-wise helpers around the matmul kernels and two plain streaming kernels
+// used to calibrate bandwidth measurements.
+//
+//   copy_f32_half(x, y, n)   f32 -> f16, round to nearest even  (reference: copy_f32_half,
+//                            crates/ojas-cuda/src/kernels/vision.rs:188-189, run before the
+//                            split-K GEMM entries)
+//   copy_f32_bf16(x, y, n)   f32 -> bf16, round to nearest even
+//   copy_bf16_f32(x, y, n)   bf16 -> f32 (exact)
+//   fill_zero_u32(y, n)      y[i] = 0 for n dwords (a fill kernel, safe inside a captured graph)
+//   stream_copy_u32x4(x, y, n16)  y = x for n16 16-byte units: a copy of known size
+//   stream_read_u32x4(x, y, n16)  reads n16 16-byte units, writes one dword per wave (y: grid*4 dwords)
+#include "ojk_common.h"
+
+extern "C" __global__ void __launch_bounds__(256)
+copy_f32_half(const float* __restrict__ x, ushort* __restrict__ y, uint n) {
+    uint i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) y[i] = __half_as_ushort(__float2half_rn(x[i]));
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+copy_f32_bf16(const float* __restrict__ x, ushort* __restrict__ y, uint n) {
+    uint i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) y[i] = f32_to_bf16_bits(x[i]);
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+copy_bf16_f32(const ushort* __restrict__ x, float* __restrict__ y, uint n) {
+    uint i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) y[i] = bf16_bits_to_f32(x[i]);
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+fill_zero_u32(uint* __restrict__ y, uint n) {
+    uint i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) y[i] = 0u;
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+stream_copy_u32x4(const uint4* __restrict__ x, uint4* __restrict__ y, uint n16) {
+    size_t stride = (size_t)gridDim.x * 256u;
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n16; i += stride) y[i] = x[i];
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+stream_read_u32x4(const uint4* __restrict__ x, uint* __restrict__ y, uint n16) {
+    size_t stride = (size_t)gridDim.x * 256u;
+    uint acc = 0;
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n16; i += stride) {
+        uint4 v = x[i];
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    acc = (uint)wave_sum_i32((int)acc);
+    if ((threadIdx.x & 63u) == 0) y[blockIdx.x * 4u + (threadIdx.x >> 6)] = acc;
+}

@@ -24,6 +24,21 @@ struct ojh_lin {
     bool owns_raw = false;
 };
 
+// One recorded launch.
+struct ojh_command {
+    hipFunction_t fn = nullptr;
+    std::vector<void *> ptrs;
+    std::vector<uint32_t> consts;
+    uint32_t grid[3] = {1, 1, 1}, block[3] = {1, 1, 1};
+};
+
+// A recorded chain: either a command list replayed from a native loop, or an instantiated hipGraph.
+struct ojh_graph {
+    std::vector<ojh_command> list;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
 // Scratch the op-level entry points keep per device (quantized activations, MoE staging).
 struct ojh_scratch {
     ojh_buf *buf = nullptr;
@@ -41,6 +56,9 @@ struct ojh_device {
     // named scratch buffers, grown on demand
     std::map<std::string, ojh_buf *> scratch;
     int gemv_rows_override = 0;  // OJAS_HIP_GEMV_R
+    bool capturing = false;      // between ojh_capture_begin and ojh_capture_end
+    bool capture_hip_graph = false;
+    std::vector<ojh_command> recorded;
 };
 
 // ---- errors ------------------------------------------------------------------------------------

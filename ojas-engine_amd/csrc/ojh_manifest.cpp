@@ -175,7 +175,60 @@ static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint
     return OJH_OK;
 }
 
+// copy_*(x, y, n) / fill_zero_u32(y, n): one thread per element
+static int check_elementwise(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                             const uint32_t block[3], size_t need[8], size_t align[8]) {
+    uint32_t n = c[0];
+    if (!n) return ojh_fail(OJH_ERR_ARG, "%s: n must be positive", s->name);
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * 256 < n)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover %u elements", s->name, n);
+    if (s->n_bufs == 1) {
+        need[0] = (size_t)n * (s->type & 0xFF);
+        align[0] = 4;
+    } else {
+        need[0] = (size_t)n * (s->type >> 8);
+        need[1] = (size_t)n * (s->type & 0xFF);
+        align[0] = s->type >> 8;
+        align[1] = s->type & 0xFF;
+    }
+    return OJH_OK;
+}
+
+// stream_copy_u32x4(x, y, n16) / stream_read_u32x4(x, y, n16): grid-stride over 16-byte units
+static int check_stream(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                        const uint32_t block[3], size_t need[8], size_t align[8]) {
+    (void)align;
+    uint32_t n16 = c[0];
+    if (!n16) return ojh_fail(OJH_ERR_ARG, "%s: n16 must be positive", s->name);
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    need[0] = (size_t)n16 * 16;
+    need[1] = s->type == 1 ? (size_t)grid[0] * 16 : (size_t)n16 * 16;
+    return OJH_OK;
+}
+
 // ---- launch shapes ---------------------------------------------------------------------------
+static int shape_elementwise(const ojh_kernel_spec *, const ojh_device *, uint32_t, uint32_t N, uint32_t,
+                             uint32_t grid[3], uint32_t block[3]) {
+    grid[0] = (N + 255) / 256;  // N = element count
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+static int shape_stream(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t N, uint32_t,
+                        uint32_t grid[3], uint32_t block[3]) {
+    uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
+    uint32_t want = cus * 8u, cover = (N + 255) / 256;  // N = 16-byte units
+    grid[0] = cover < want ? cover : want;
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
 static int shape_rows(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t,
                       uint32_t grid[3], uint32_t block[3]) {
     uint32_t rows_per_block = 4u * (uint32_t)s->rows_per_wave;
@@ -230,12 +283,20 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(q, "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
         add(q + "_r1", "gemv_q8k", 4, 2, f.type, 1, check_gemv_q8k, shape_rows);
         add(q + "_r2", "gemv_q8k", 4, 2, f.type, 2, check_gemv_q8k, shape_rows);
+        add(q + "_wide", "gemv_q8k", 4, 2, f.type, 2, check_gemv_q8k, shape_rows);
         add(q + "_accum", "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
         add(q + "_bias", "gemv_q8k", 5, 2, f.type, 4, check_gemv_q8k, shape_rows);
         add(q + "_m", "gemv_q8k", 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
     }
     add("quantize_q8k", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
+    // glue: `type` carries (input element bytes << 8 | output element bytes)
+    add("copy_f32_half", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);
+    add("copy_f32_bf16", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);
+    add("copy_bf16_f32", "glue", 2, 1, (2u << 8) | 4u, 0, check_elementwise, shape_elementwise);
+    add("fill_zero_u32", "glue", 1, 1, 4u, 0, check_elementwise, shape_elementwise);
+    add("stream_copy_u32x4", "glue", 2, 1, 0, 0, check_stream, shape_stream);
+    add("stream_read_u32x4", "glue", 2, 1, 1, 0, check_stream, shape_stream);
     return m;
 }
 

@@ -125,10 +125,9 @@ static int pick_rows(const ojh_device *dev, uint32_t n) {
     if (dev->gemv_rows_override == 1 || dev->gemv_rows_override == 2 || dev->gemv_rows_override == 4)
         return dev->gemv_rows_override;
     uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;
-    uint32_t want_waves = cus * 8;  // two per SIMD
-    if (n / 4 >= want_waves) return 4;
-    if (n / 2 >= want_waves) return 2;
-    return 1;
+    // Measured on MI355X (Q4_K, K=4096): two rows per wave streams fastest once N gives every CU
+    // several workgroups; four rows per wave loses to it at every size.
+    return n >= cus * 32u ? 2 : 1;
 }
 
 // y (=,+=,+bias) quantized-x . W^T for K-quant weights: the matvec (m = 1) and its batched form.
@@ -140,7 +139,8 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
     std::string base = std::string("gemv_q8k_") + f->tag;
     if (m == 1) {
         int r = (accum || bias) ? 4 : pick_rows(dev, N);
-        std::string name = base + (accum ? "_accum" : bias ? "_bias" : r == 4 ? "" : r == 2 ? "_r2" : "_r1");
+        bool wide = !accum && !bias && r == 2 && N >= 32768u;
+        std::string name = base + (accum ? "_accum" : bias ? "_bias" : wide ? "_wide" : r == 4 ? "" : r == 2 ? "_r2" : "_r1");
         grid[0] = (N + 4 * r - 1) / (4 * r);
         std::vector<void *> p = {xq, xs, wp, yp};
         if (bias) p.push_back(bias->ptr);

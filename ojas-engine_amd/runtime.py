@@ -103,6 +103,10 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_row_bytes": (sz, [u32, u32]),
         "ojh_mm": (i32, [vp, vp, sz, i32, vp, vp, sz, vp, u32, i32, i32]),
         "ojh_mm_q8k": (i32, [vp, vp, vp, vp, vp, sz, vp, u32, i32]),
+        "ojh_capture_begin": (i32, [vp]),
+        "ojh_capture_end": (i32, [vp, pp]),
+        "ojh_graph_launch": (i32, [vp, vp]),
+        "ojh_graph_free": (i32, [vp, vp]),
         "ojh_mark": (i32, [vp, i32]),
         "ojh_mark_elapsed": (i32, [vp, i32, i32, C.POINTER(C.c_float)]),
         "ojh_dequant_f16": (i32, [vp, u32, vp, sz, sz, vp, sz]),
@@ -185,6 +189,27 @@ class Lin:
     def free(self) -> None:
         if self.handle and self.gpu._dev:
             self.gpu._check(self.gpu._L.ojh_lin_free(self.gpu._dev, self.handle))
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Graph:
+    """A recorded chain of dispatches; `launch()` replays it with one host call."""
+
+    def __init__(self, gpu: "HipGpu", handle):
+        self.gpu, self.handle = gpu, handle
+
+    def launch(self) -> None:
+        self.gpu._check(self.gpu._L.ojh_graph_launch(self.gpu._dev, self.handle))
+
+    def free(self) -> None:
+        if self.handle and self.gpu._dev:
+            self.gpu._L.ojh_graph_free(self.gpu._dev, self.handle)
         self.handle = None
 
     def __del__(self):
@@ -329,6 +354,15 @@ class HipGpu:
         """Matmul from activations already quantized by `quant_q8k` (shared by several projections)."""
         self._check(self._L.ojh_mm_q8k(self._dev, xq.handle, xscales.handle, w.handle, y.handle, y_off,
                                        bias.handle if bias else None, m, int(accum)))
+
+    def capture_begin(self) -> None:
+        """Start recording dispatches on the device's stream instead of running them."""
+        self._check(self._L.ojh_capture_begin(self._dev))
+
+    def capture_end(self) -> "Graph":
+        h = C.c_void_p()
+        self._check(self._L.ojh_capture_end(self._dev, C.byref(h)))
+        return Graph(self, h)
 
     def mark(self, slot: int) -> None:
         self._check(self._L.ojh_mark(self._dev, slot))

@@ -194,7 +194,7 @@ def test_errors_are_reported_not_launched(gpu, pkg):
     with pytest.raises(pkg.OjasHipError, match="not loaded"):
         gpu.dispatch(enc, "gemv_nat_q9k", [(xd, 0), (wd, 0), (yd, 0)], [k, n], grid, block)
     with pytest.raises(pkg.OjasHipError, match="needs"):   # y too small for N
-        gpu.dispatch(enc, "gemv_nat_q4k", [(xd, 0), (wd, 0), (yd, 0)], [k, n + 1], grid, block)
+        gpu.dispatch(enc, "gemv_nat_q4k", [(xd, 0), (wd, 0), (yd, 0)], [k, n + 1], [grid[0] + 1, 1, 1], block)
     with pytest.raises(pkg.OjasHipError, match="multiple of 256"):
         gpu.dispatch(enc, "gemv_nat_q4k", [(xd, 0), (wd, 0), (yd, 0)], [k - 32, n], grid, block)
     with pytest.raises(pkg.OjasHipError, match="covers"):
