@@ -6,6 +6,7 @@
 //                            split-K GEMM entries)
 //   copy_f32_bf16(x, y, n)   f32 -> bf16, round to nearest even
 //   copy_bf16_f32(x, y, n)   bf16 -> f32 (exact)
+//   copy_bf16_half(x, y, n)  bf16 -> f16, round to nearest even
 //   fill_zero_u32(y, n)      y[i] = 0 for n dwords (a fill kernel, safe inside a captured graph)
 //   stream_copy_u32x4(x, y, n16)  y = x for n16 16-byte units: a copy of known size
 //   stream_read_u32x4(x, y, n16)  reads n16 16-byte units, writes one dword per wave (y: grid*4 dwords)
@@ -27,6 +28,13 @@ extern "C" __global__ void __launch_bounds__(256)
 copy_bf16_f32(const ushort* __restrict__ x, float* __restrict__ y, uint n) {
     uint i = blockIdx.x * 256u + threadIdx.x;
     if (i < n) y[i] = bf16_bits_to_f32(x[i]);
+}
+
+// bf16 -> f16, round to nearest even (exact for every bf16 value inside f16's normal range)
+extern "C" __global__ void __launch_bounds__(256)
+copy_bf16_half(const ushort* __restrict__ x, ushort* __restrict__ y, uint n) {
+    uint i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) y[i] = __half_as_ushort(__float2half_rn(bf16_bits_to_f32(x[i])));
 }
 
 extern "C" __global__ void __launch_bounds__(256)

@@ -56,6 +56,8 @@ struct ojh_device {
     // named scratch buffers, grown on demand
     std::map<std::string, ojh_buf *> scratch;
     int gemv_rows_override = 0;  // OJAS_HIP_GEMV_R
+    uint32_t gemm_min_m = 32;    // OJAS_HIP_GEMM_MIN_M: rows from which ojh_mm takes the MFMA tile
+    int gemm_split_override = 0; // OJAS_HIP_GEMM_SPLIT
     bool capturing = false;      // between ojh_capture_begin and ojh_capture_end
     bool capture_hip_graph = false;
     std::vector<ojh_command> recorded;

@@ -175,6 +175,46 @@ static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint
     return OJH_OK;
 }
 
+// gemm_mm_<fmt>(xh, w, y, K, N, accum, M) and gemm_mm_<fmt>_sk(xh, w, y, K, N, M, nsplit);
+// `rows_per_wave` = 1 marks the split-K form.
+static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                      const uint32_t block[3], size_t need[8], size_t align[8]) {
+    const ojh_block_format *f;
+    const bool sk = s->rows_per_wave == 1;
+    uint32_t K = c[0], N = c[1], M = sk ? c[2] : c[3], nsplit = sk ? c[3] : 1;
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if (K % 64) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a multiple of 64", s->name, K);
+    if (M == 0 || nsplit == 0) return ojh_fail(OJH_ERR_ARG, "%s: M and nsplit must be positive", s->name);
+    if ((rc = check_block(block, 256))) return rc;
+    if (grid[0] != (N + 127) / 128 || grid[1] != (M + 255) / 256 || grid[2] != nsplit)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, (N + 127) / 128, (M + 255) / 256, nsplit);
+    need[0] = (size_t)M * K * 2;
+    need[1] = (size_t)N * (K / f->weights) * f->bytes;
+    need[2] = (size_t)M * N * 4;
+    align[1] = f->bytes % 16 ? 2 : 16;
+    align[2] = 4;
+    return OJH_OK;
+}
+
+static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
+                      uint32_t grid[3], uint32_t block[3]) {
+    grid[0] = (N + 127) / 128;
+    grid[1] = (M + 255) / 256;
+    grid[2] = 1;
+    if (s->rows_per_wave == 1) {  // split K until every CU has a tile, at least 4 K-steps per slice
+        uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
+        uint32_t tiles = grid[0] * grid[1], steps = K / 64;
+        uint32_t z = tiles ? (cus + tiles - 1) / tiles : 1;
+        if (z > steps / 4) z = steps / 4;
+        if (z > 16) z = 16;
+        grid[2] = z ? z : 1;
+    }
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // copy_*(x, y, n) / fill_zero_u32(y, n): one thread per element
 static int check_elementwise(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                              const uint32_t block[3], size_t need[8], size_t align[8]) {
@@ -290,6 +330,14 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     }
     add("quantize_q8k", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
+    // prefill / verify MFMA tiles: "q8_0" is the reference's spelling for this family
+    for (const auto &f : kFormats) {
+        if (f.type == OJH_Q5_K) continue;
+        std::string g = std::string("gemm_mm_") + (f.type == OJH_Q8_0 ? "q8_0" : f.tag);
+        add(g, "gemm", 3, 4, f.type, 0, check_gemm, shape_gemm);
+        add(g + "_sk", "gemm", 3, 4, f.type, 1, check_gemm, shape_gemm);
+    }
+    add("copy_bf16_half", "glue", 2, 1, (2u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     // glue: `type` carries (input element bytes << 8 | output element bytes)
     add("copy_f32_half", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     add("copy_f32_bf16", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);

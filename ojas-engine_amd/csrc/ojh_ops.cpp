@@ -193,10 +193,36 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     size_t esz = x_dtype == OJH_X_BF16 ? 2 : 4;
     if ((rc = span_ok("ojh_mm: x", x, x_off, (size_t)m * K * esz, 16))) return rc;
 
-    bool q8k = w->type != OJH_Q8_0 && act_mode != OJH_ACT_FLOAT;
     void *wp = at(w->raw, w->off), *yp = at(y, y_off);
     uint32_t grid[3] = {1, 1, 1}, block[3] = {256, 1, 1};
 
+    // Above the crossover the MFMA tile wins over streaming the weights once per few tokens
+    // (the reference switches at 8 rows, crates/ojas-models/src/decoder/dispatch.rs:70-75).
+    if (m >= dev->gemm_min_m && act_mode != OJH_ACT_Q8K && K % 64 == 0 && (uint64_t)m * K < 0x7FFFFFFFull &&
+        (uint64_t)m * N < 0x7FFFFFFFull) {
+        if ((rc = ensure(dev, "glue")) || (rc = ensure(dev, "gemm"))) return rc;
+        ojh_buf *xh;
+        if ((rc = ojh_scratch_get(dev, "xh", (size_t)m * K * 2, &xh))) return rc;
+        uint32_t n_el = m * K, eg[3] = {(n_el + 255) / 256, 1, 1};
+        if ((rc = ojh_launch(dev, x_dtype == OJH_X_BF16 ? "copy_bf16_half" : "copy_f32_half", {at(x, x_off), xh->ptr},
+                             {n_el}, eg, block)))
+            return rc;
+        std::string base = std::string("gemm_mm_") + (w->type == OJH_Q8_0 ? "q8_0" : f->tag);
+        uint32_t sg[3], sb[3];
+        if ((rc = ojh_launch_shape(dev, (base + "_sk").c_str(), K, N, m, sg, sb))) return rc;
+        if (dev->gemm_split_override > 0) sg[2] = (uint32_t)dev->gemm_split_override;
+        if (sg[2] > 1) {
+            if (!accum) {
+                uint32_t n_y = m * N, zg[3] = {(n_y + 255) / 256, 1, 1};
+                if ((rc = ojh_launch(dev, "fill_zero_u32", {yp}, {n_y}, zg, block))) return rc;
+            }
+            return ojh_launch(dev, (base + "_sk").c_str(), {xh->ptr, wp, yp}, {K, N, m, sg[2]}, sg, sb);
+        }
+        sg[2] = 1;
+        return ojh_launch(dev, base.c_str(), {xh->ptr, wp, yp}, {K, N, (uint32_t)(accum != 0), m}, sg, sb);
+    }
+
+    bool q8k = w->type != OJH_Q8_0 && act_mode != OJH_ACT_FLOAT;
     if (q8k) {
         if ((rc = ensure(dev, "gemv_q8k"))) return rc;
         size_t nsb = K / 256;
@@ -207,20 +233,26 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         return mm_q8k_launch(dev, xq->ptr, xs->ptr, w, f, yp, bias, m, accum);
     }
 
-    // floating-point activations
-    if (x_dtype != OJH_X_F32)
-        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: the float matvec takes f32 activations");
+    // floating-point activations: the matvec kernels read f32
+    void *xp = at(x, x_off);
+    if (x_dtype == OJH_X_BF16) {
+        if ((rc = ensure(dev, "glue"))) return rc;
+        ojh_buf *xf;
+        if ((rc = ojh_scratch_get(dev, "xf", (size_t)m * K * 4, &xf))) return rc;
+        uint32_t n_el = m * K, eg[3] = {(n_el + 255) / 256, 1, 1};
+        if ((rc = ojh_launch(dev, "copy_bf16_f32", {xp, xf->ptr}, {n_el}, eg, block))) return rc;
+        xp = xf->ptr;
+    }
     if ((rc = ensure(dev, "gemv"))) return rc;
     std::string base = std::string("gemv_nat_") + f->tag;
     if (m == 1) {
         int r = (accum || bias) ? 4 : pick_rows(dev, N);
         std::string name = base + (accum ? "_accum" : bias ? "_bias" : r == 4 ? "" : r == 2 ? "_r2" : "_r1");
         grid[0] = (N + 4 * r - 1) / (4 * r);
-        std::vector<void *> p = {at(x, x_off), wp, yp};
+        std::vector<void *> p = {xp, wp, yp};
         if (bias) p.push_back(bias->ptr);
         return ojh_launch(dev, name.c_str(), p, {K, N}, grid, block);
     }
     grid[0] = (N + 3) / 4;
-    return ojh_launch(dev, (base + "_m").c_str(), {at(x, x_off), wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, grid,
-                      block);
+    return ojh_launch(dev, (base + "_m").c_str(), {xp, wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, grid, block);
 }

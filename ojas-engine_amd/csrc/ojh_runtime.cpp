@@ -71,6 +71,8 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     }
     d->name = std::string("hip:") + d->prop.name + " (" + d->prop.gcnArchName + ")";
     if (const char *r = getenv("OJAS_HIP_GEMV_R")) d->gemv_rows_override = atoi(r);
+    if (const char *r = getenv("OJAS_HIP_GEMM_MIN_M")) d->gemm_min_m = (uint32_t)atoi(r);
+    if (const char *r = getenv("OJAS_HIP_GEMM_SPLIT")) d->gemm_split_override = atoi(r);
     *out = d;
     return OJH_OK;
 }

@@ -1,0 +1,102 @@
+"""Prefill / verify matmul on the MFMA tile against the CPU oracle.
+
+Oracle: x . dequant(W)^T accumulated in double (crates/ojas-cuda/tests/prefill_gemm_q.rs:116-130),
+once with x rounded to f16 and W as `dequant_to_f16` stores it (what the tile holds: the kernel's
+own error) and once with x and W unrounded.  Metrics and the reference's bounds:
+(max|d| / rms, rms(d) / rms) < (5e-3, 5e-4) against the rounded oracle and < (2e-2, 3e-3) against
+the unrounded one (prefill_gemm_q.rs:288-343).  This tile feeds the MFMA the decoder's exact f16
+bits, so the first pair is held to (2e-5, 5e-6).
+"""
+import numpy as np
+import pytest
+
+from conftest import rms_errs
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+TIGHT = (2e-5, 5e-6)
+
+
+def _run(gpu, pkg, orc, ty, m, k, n, accum=False, x_dtype="f32", split=None):
+    w = pkg.synth.weights(ty, n, k, "gemm", ty, n, k)
+    x = pkg.synth.normal_f32(m * k, "gemm", "x", m, k).reshape(m, k)
+    if x_dtype == "bf16":
+        xb = pkg.synth.to_bf16_bits(x)
+        x = pkg.synth.bf16_bits_to_f32(xb).reshape(m, k)
+        xd = gpu.upload_bytes(xb)
+    else:
+        xd = gpu.upload(x)
+    y0 = pkg.synth.normal_f32(m * n, "gemm", "y0").reshape(m, n) if accum else np.zeros((m, n), np.float32)
+    sent = np.full(n, 12345.5, np.float32)
+    yd = gpu.upload(np.concatenate([y0.ravel(), sent]))
+    lin = gpu.lin(ty, n, k, w)
+    gpu.mm(xd, lin, yd, m, accum, act_mode=pkg.ACT_FLOAT, x_dtype=pkg.X_BF16 if x_dtype == "bf16" else pkg.X_F32)
+    got = gpu.read(yd, m * n + n)
+    assert np.all(got[m * n:] == 12345.5), "wrote past row M"
+    got = got[:m * n].reshape(m, n)
+    want16 = orc.matmul_ref(w, ty, n, k, x, wmode=1, xmode=1) + y0
+    want32 = orc.matmul_ref(w, ty, n, k, x) + y0
+    return rms_errs(got, want16), rms_errs(got, want32)
+
+
+# the reference's sweep: ragged M and N, accumulate, short and long K (prefill_gemm_q.rs:346-380)
+SWEEP = [(64, 256, 128, False), (33, 512, 130, False), (100, 1024, 200, True), (256, 4096, 256, False),
+         (300, 2048, 72, True), (512, 1024, 384, False), (77, 14336, 64, False)]
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("m,k,n,accum", SWEEP)
+def test_gemm_sweep(gpu, orc, pkg, ty, m, k, n, accum):
+    e16, e32 = _run(gpu, pkg, orc, ty, m, k, n, accum)
+    assert e16[0] < TIGHT[0] and e16[1] < TIGHT[1], (e16, "vs the rounded oracle")
+    assert e32[0] < 2e-2 and e32[1] < 3e-3, (e32, "vs the unrounded oracle")
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+def test_gemm_bf16_activations(gpu, orc, pkg, ty):
+    """bf16 activations (the prefill / verify input type) convert to f16 exactly in range."""
+    e16, e32 = _run(gpu, pkg, orc, ty, 128, 2048, 256, x_dtype="bf16")
+    assert e16[0] < TIGHT[0] and e16[1] < TIGHT[1], e16
+    assert e32[0] < 2e-2 and e32[1] < 3e-3, e32
+
+
+def test_split_k_entry_through_the_kernel_seam(gpu, orc, pkg):
+    """gemm_mm_q4k_sk dispatched by name with several K slices; y holds what is accumulated into."""
+    gpu.ensure_family("gemm")
+    gpu.ensure_family("glue")
+    m, k, n = 40, 2048, 200
+    w = pkg.synth.q4k_weights(n, k, "gemmsk", "w")
+    x = pkg.synth.normal_f32(m * k, "gemmsk", "x").reshape(m, k)
+    xh = gpu.upload_bytes(x.astype(np.float16))
+    wd = gpu.upload_bytes(w)
+    want = orc.matmul_ref(w, Q4_K, n, k, x, wmode=1, xmode=1)
+    for nsplit in (1, 3, 8):
+        y0 = pkg.synth.normal_f32(m * n, "gemmsk", "y0", nsplit).reshape(m, n)
+        yd = gpu.upload(y0)
+        enc = gpu.begin()
+        gpu.dispatch(enc, "gemm_mm_q4k_sk", [(xh, 0), (wd, 0), (yd, 0)], [k, n, m, nsplit],
+                     [(n + 127) // 128, (m + 255) // 256, nsplit], [256, 1, 1])
+        gpu.submit(enc)
+        e = rms_errs(gpu.read(yd, m * n).reshape(m, n), want + y0)
+        assert e[0] < 1e-4 and e[1] < 2e-5, (nsplit, e)
+    with pytest.raises(pkg.OjasHipError, match="grid must be"):
+        gpu.dispatch(enc, "gemm_mm_q4k_sk", [(xh, 0), (wd, 0), (yd, 0)], [k, n, m, 2], [2, 1, 1], [256, 1, 1])
+
+
+def test_router_prefers_the_tile_only_above_the_crossover(gpu, orc, pkg):
+    """ACT_AUTO: small M keeps the CPU-reference arithmetic (int8 activations); large M takes the
+    f16 tile.  Both must sit within their own oracle's bound."""
+    n, k = 256, 1024
+    w = pkg.synth.q4k_weights(n, k, "xover", "w")
+    lin = gpu.lin(Q4_K, n, k, w)
+    for m in (4, 64):
+        x = pkg.synth.normal_f32(m * k, "xover", "x", m).reshape(m, k)
+        yd = gpu.alloc(m * n)
+        gpu.mm(gpu.upload(x), lin, yd, m)
+        got = gpu.read(yd, m * n).reshape(m, n)
+        if m < 32:
+            want = np.stack([orc.matvec_kq(w, Q4_K, n, k, x[t]) for t in range(m)])
+            assert np.max(np.abs(got - want)) <= 2e-5 * np.max(np.abs(want))
+        else:
+            e = rms_errs(got, orc.matmul_ref(w, Q4_K, n, k, x, wmode=1, xmode=1))
+            assert e[0] < TIGHT[0] and e[1] < TIGHT[1], e
