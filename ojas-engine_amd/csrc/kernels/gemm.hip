@@ -17,8 +17,8 @@
 // to 144 bytes so 16-byte fragment reads of 16 consecutive rows fall in distinct banks.  Each wave
 // owns 128 x 64 of the tile as 4 x 2 blocks of v_mfma_f32_32x32x16_f16 (A = activations, B =
 // weights, so a D register holds 32 consecutive outputs of one token: coalesced stores).  Global
-// loads for step s+1 are issued before the MFMAs of step s and written to the other LDS stage
-// after them: one barrier per step.
+// loads run three steps ahead in registers and are written to the other LDS stage after the
+// MFMAs of the current step: one barrier per step.
 #include "ojk_common.h"
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -38,18 +38,51 @@ __device__ __forceinline__ uint f16_bits_rn(float v) {
 }
 __device__ __forceinline__ uint pack2(float a, float b) { return f16_bits_rn(a) | (f16_bits_rn(b) << 16); }
 
+// ---- global loads whose issue point the compiler may not move -----------------------------------
+// The compiler sinks ordinary loads down to their first use to save registers, which turns a
+// three-steps-ahead prefetch into load-then-wait.  These loads are opaque to it: they are issued
+// where they are written, and the consumer waits with an explicit s_waitcnt (gm_wait) that also
+// re-defines the destination registers, so nothing that reads them can be scheduled above it.
+// Vector memory operations retire in order, so "at most n outstanding" means every load issued
+// before the last n has landed.
+typedef uint u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4 gm_load16(const void* p) {
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ uint gm_load_u16(const void* p) {
+    uint v;
+    asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ uint gm_load_u8(const void* p) {
+    uint v;
+    asm volatile("global_load_ubyte %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+template <int N>
+__device__ __forceinline__ void gm_wait(u32x4 (&x)[8]) {
+    asm volatile("s_waitcnt vmcnt(%8)"
+                 : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])
+                 : "n"(N)
+                 : "memory");
+}
+
 // ------------------------------------------------------------------ per-format slab loaders
 // A loader owns, for one thread, 32 weights of one row of the 128 x 64 slab: thread t -> row
 // t/2, half h = t%2.  `load` issues the global loads; `store` dequantizes into the LDS row.
 struct LoaderQ4K {
-    uint4 hdr, qs;
+    static constexpr int NL = 2;  // global loads per slab
+    u32x4 hdr, qs;
     uint c;
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(hdr), "+v"(qs)::"memory"); }
     static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * Q4K_BYTES; }
     __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
         const uchar* blk = row + (size_t)(k0 >> 8) * Q4K_BYTES;
         c = (k0 >> 6) & 3u;  // 32-byte chunk of the super-block = sub-blocks 2c, 2c+1
-        hdr = *(const uint4*)blk;
-        qs = *(const uint4*)(blk + 16u + c * 32u + h * 16u);
+        hdr = gm_load16(blk);
+        qs = gm_load16(blk + 16u + c * 32u + h * 16u);
     }
     // 16 low-nibble weights -> slab columns 16h.., 16 high-nibble weights -> columns 32+16h..
     __device__ __forceinline__ void store(uchar* lds_row, uint h) const {
@@ -82,23 +115,28 @@ struct LoaderQ4K {
 };
 
 struct LoaderQ6K {
-    u32x4_a2 qa, qb, qh;
-    uint sc2, d16, hi_half;  // sc2: the two sub-scales (quarters 2j', 2j'+1) of this thread's 16 columns
+    static constexpr int NL = 6;
+    u32x4 qa, qb, qh;
+    uint sca, scb, d16, hi_half;  // sca, scb: the sub-scales of the slab's two quarters for this thread's 16 columns
+    __device__ __forceinline__ void pin() {
+        asm volatile("" : "+v"(qa), "+v"(qb), "+v"(qh), "+v"(sca), "+v"(scb), "+v"(d16)::"memory");
+    }
     static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * Q6K_BYTES; }
     __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
         const uchar* blk = row + (size_t)(k0 >> 8) * Q6K_BYTES;
         uint j = (k0 >> 6) & 3u, hf = j >> 1;  // 64-column slab j of the super-block: half hf, quarters 2(j%2), +1
         hi_half = j & 1u;
-        qa = *(const u32x4_a2*)(blk + hf * 64u + h * 16u);
-        qb = *(const u32x4_a2*)(blk + hf * 64u + 32u + h * 16u);
-        qh = *(const u32x4_a2*)(blk + 128u + hf * 32u + h * 16u);
+        qa = gm_load16(blk + hf * 64u + h * 16u);
+        qb = gm_load16(blk + hf * 64u + 32u + h * 16u);
+        qh = gm_load16(blk + 128u + hf * 32u + h * 16u);
         const uchar* sc = blk + 192u + hf * 8u + (j & 1u) * 4u + h;  // sc[2q + h], q = 2(j%2), 2(j%2)+1
-        sc2 = (uint)sc[0] | ((uint)sc[2] << 8);
-        d16 = *(const ushort*)(blk + 208u);
+        sca = gm_load_u8(sc);
+        scb = gm_load_u8(sc + 2);
+        d16 = gm_load_u16(blk + 208u);
     }
     __device__ __forceinline__ void store(uchar* lds_row, uint h) const {
         float d = f16_bits_to_f32(d16);
-        float s0 = __fmul_rn(d, (float)(signed char)(sc2 & 0xFFu)), s1 = __fmul_rn(d, (float)(signed char)(sc2 >> 8));
+        float s0 = __fmul_rn(d, (float)(signed char)sca), s1 = __fmul_rn(d, (float)(signed char)scb);
         uint a[4] = {qa.x, qa.y, qa.z, qa.w}, b[4] = {qb.x, qb.y, qb.z, qb.w}, hq[4] = {qh.x, qh.y, qh.z, qh.w};
         uint o0[8], o1[8];
         const uint sh_h0 = hi_half ? 4u : 0u, sh_h1 = hi_half ? 6u : 2u, sh_l = hi_half ? 4u : 0u;
@@ -128,14 +166,16 @@ struct LoaderQ6K {
 };
 
 struct LoaderQ80 {
-    u32x4_a2 qa, qb;
+    static constexpr int NL = 3;
+    u32x4 qa, qb;
     uint d16;
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(qa), "+v"(qb), "+v"(d16)::"memory"); }
     static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 5) * Q80_BYTES; }
     __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
         const uchar* blk = row + (size_t)((k0 >> 5) + h) * Q80_BYTES;  // block h of the slab's two
-        d16 = *(const ushort*)blk;
-        qa = *(const u32x4_a2*)(blk + 2u);
-        qb = *(const u32x4_a2*)(blk + 18u);
+        d16 = gm_load_u16(blk);
+        qa = gm_load16(blk + 2u);
+        qb = gm_load16(blk + 18u);
     }
     // block h fills slab columns 32h..32h+31
     __device__ __forceinline__ void store(uchar* lds_row, uint h) const {
@@ -191,56 +231,78 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    uint4 xreg[8];
-    Loader ld;
-    // prologue: first slab into stage 0
-#pragma unroll
-    for (int i = 0; i < 8; i++) xreg[i] = *(const uint4*)(xrow[i] + k_begin);
-    ld.load(wrow, k_begin, wh);
-    {
-        uchar* a = lds;
-        uchar* b = lds + GM_BM * GM_STRIDE;
-#pragma unroll
-        for (int i = 0; i < 8; i++) *(uint4*)(a + (xr + 32u * i) * GM_STRIDE + xc * 2u) = xreg[i];
-        ld.store(b + wr * GM_STRIDE, wh);
-    }
-    __syncthreads();
+    // Three register sets hold the slabs of steps t+1 .. t+3 while step t runs from LDS: loads are
+    // in flight for two whole steps before anyone waits for them (one wave per SIMD cannot lean
+    // on other waves to cover HBM latency).
+    u32x4 xs0[8], xs1[8], xs2[8];
+    Loader ld0, ld1, ld2;
+    const uint nt = (k_end - k_begin) / GM_BK;
 
-    uint stage = 0;
-    for (uint k0 = k_begin; k0 < k_end; k0 += GM_BK) {
-        const bool more = k0 + GM_BK < k_end;
-        if (more) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) xreg[i] = *(const uint4*)(xrow[i] + k0 + GM_BK);
-            ld.load(wrow, k0 + GM_BK, wh);
-        }
-        const uchar* a = lds + stage * GM_STAGE;
-        const uchar* b = a + GM_BM * GM_STRIDE;
-#pragma unroll
-        for (int ks = 0; ks < GM_BK / 16; ks++) {
-            half8 af[4], bf[2];
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                af[i] = *(const half8*)(a + (wm + 32u * i + fr) * GM_STRIDE + (ks * 16u + kg * 8u) * 2u);
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-                bf[j] = *(const half8*)(b + (wn + 32u * j + fr) * GM_STRIDE + (ks * 16u + kg * 8u) * 2u);
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
-        }
-        if (more) {
-            uchar* na = lds + (stage ^ 1u) * GM_STAGE;
-            uchar* nb = na + GM_BM * GM_STRIDE;
-#pragma unroll
-            for (int i = 0; i < 8; i++) *(uint4*)(na + (xr + 32u * i) * GM_STRIDE + xc * 2u) = xreg[i];
-            ld.store(nb + wr * GM_STRIDE, wh);
-        }
-        __syncthreads();
-        stage ^= 1u;
+#define GM_LOAD(XS, LD, T)                                                                       \
+    do {                                                                                         \
+        const uint kk_ = k_begin + (T) * GM_BK;                                                  \
+        _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++) XS[i_] = gm_load16(xrow[i_] + kk_);      \
+        LD.load(wrow, kk_, wh);                                                                  \
+    } while (0)
+#define GM_STORE(XS, LD, STG)                                                                    \
+    do {                                                                                         \
+        uchar* a_ = lds + (STG) * GM_STAGE;                                                      \
+        _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++)                                         \
+            *(u32x4*)(a_ + (xr + 32u * i_) * GM_STRIDE + xc * 2u) = XS[i_];                      \
+        LD.store(a_ + GM_BM * GM_STRIDE + wr * GM_STRIDE, wh);                                   \
+    } while (0)
+#define GM_COMPUTE(STG)                                                                          \
+    do {                                                                                         \
+        const uchar* a_ = lds + (STG) * GM_STAGE;                                                \
+        const uchar* b_ = a_ + GM_BM * GM_STRIDE;                                                \
+        _Pragma("unroll") for (int ks = 0; ks < GM_BK / 16; ks++) {                              \
+            half8 af[4], bf[2];                                                                  \
+            _Pragma("unroll") for (int i = 0; i < 4; i++)                                        \
+                af[i] = *(const half8*)(a_ + (wm + 32u * i + fr) * GM_STRIDE + (ks * 16u + kg * 8u) * 2u); \
+            _Pragma("unroll") for (int j = 0; j < 2; j++)                                        \
+                bf[j] = *(const half8*)(b_ + (wn + 32u * j + fr) * GM_STRIDE + (ks * 16u + kg * 8u) * 2u); \
+            _Pragma("unroll") for (int i = 0; i < 4; i++)                                        \
+                _Pragma("unroll") for (int j = 0; j < 2; j++)                                    \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0); \
+        }                                                                                        \
+    } while (0)
+// step T: refill the set that step T's slab came from, run step T, stage step T+1
+#define GM_STEP(T, XS_FREE, LD_FREE, XS_NEXT, LD_NEXT)                                           \
+    do {                                                                                         \
+        if ((T) + 3u < nt) GM_LOAD(XS_FREE, LD_FREE, (T) + 3u);                                  \
+        GM_COMPUTE((T) & 1u);                                                                    \
+        if ((T) + 1u < nt) {                                                                     \
+            GM_WAIT_FOR(XS_NEXT, LD_NEXT, (T) + 1u);                                             \
+            GM_STORE(XS_NEXT, LD_NEXT, ((T) + 1u) & 1u);                                         \
+        }                                                                                        \
+        __syncthreads();                                                                         \
+    } while (0)
+// wait for the slab of step T: the slabs of steps T+1 and T+2, where they exist, were issued later
+#define GM_WAIT_FOR(XS, LD, T)                                                                   \
+    do {                                                                                         \
+        if ((T) + 2u < nt) gm_wait<2 * LPS>(XS);                                                 \
+        else if ((T) + 1u < nt) gm_wait<LPS>(XS);                                                \
+        else gm_wait<0>(XS);                                                                     \
+        LD.pin();                                                                                \
+    } while (0)
+    constexpr int LPS = 8 + Loader::NL;  // loads per slab
+
+    GM_LOAD(xs0, ld0, 0u);
+    if (nt > 1u) GM_LOAD(xs1, ld1, 1u);
+    if (nt > 2u) GM_LOAD(xs2, ld2, 2u);
+    GM_WAIT_FOR(xs0, ld0, 0u);
+    GM_STORE(xs0, ld0, 0u);
+    __syncthreads();
+    for (uint t = 0; t < nt; t += 3u) {
+        GM_STEP(t, xs0, ld0, xs1, ld1);
+        if (t + 1u < nt) GM_STEP(t + 1u, xs1, ld1, xs2, ld2);
+        if (t + 2u < nt) GM_STEP(t + 2u, xs2, ld2, xs0, ld0);
     }
+#undef GM_LOAD
+#undef GM_STORE
+#undef GM_COMPUTE
+#undef GM_STEP
+#undef GM_WAIT_FOR
 
     // epilogue: D register v of block (i, j) holds row 8*(v/4) + 4*kg + v%4, column fr
 #pragma unroll
