@@ -24,13 +24,14 @@ ARCH = "gfx950"
 DEVICE_FLAGS = ["-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                 "-Wno-unused-command-line-argument"]
 
-# family -> (source, extra flags).  The decoder family must round every operation separately.
+# family -> (source, extra flags).  The decoder family and the GEMM's in-tile decoder must round
+# every operation separately (no fused multiply-add).
 FAMILIES = {
     "dequant": ("dequant.hip", ["-ffp-contract=off"]),
     "gemv": ("gemv.hip", []),
     "gemv_q8k": ("gemv_q8k.hip", []),
     "glue": ("glue.hip", []),
-    "gemm": ("gemm.hip", []),
+    "gemm": ("gemm.hip", ["-ffp-contract=off"]),
     "moe": ("moe.hip", []),
 }
 

@@ -5,24 +5,31 @@
 // the tile, weights dequantized to f16 into the tile, f32 accumulation, f32 y; any M and N (loads
 // clamped, stores masked, nothing written past row M).  Here the dequantized tile holds exactly
 // the bits `dequant_to_f16` produces (crates/ojas-formats/src/gguf.rs:612-1116): every product and
-// difference is rounded on its own, then one round-to-nearest-even to binary16.
+// difference is rounded on its own (the file is compiled with -ffp-contract=off), then one
+// round-to-nearest-even to binary16.
 //
 //   gemm_mm_<fmt>(xh, w, y, K, N, accum, M)        xh: f16 [M][K]; grid [ceil(N/128), ceil(M/256), 1]
 //   gemm_mm_<fmt>_sk(xh, w, y, K, N, M, nsplit)    grid.z = nsplit; adds its K slice into y with
 //                                                  f32 atomics (zero y first for a plain product)
 //
-// CDNA4 plan: one workgroup of 4 waves owns a 256 (tokens) x 128 (outputs) tile and walks K in
-// steps of 64.  Per step the 256 threads stage the activation slab (256 x 64 f16) and dequantize
-// the weight slab (128 rows x one 32-byte chunk of quants = 64 weights each) into LDS, rows padded
-// to 144 bytes so 16-byte fragment reads of 16 consecutive rows fall in distinct banks.  Each wave
+// CDNA4 plan: one workgroup of 4 waves (one per SIMD) owns a 256 (tokens) x 128 (outputs) tile
+// and walks K in steps of 64.  Per step the 256 threads stage the activation slab (256 x 64 f16)
+// and dequantize the weight slab (128 rows x 64 weights, 32 per thread) into LDS, rows padded to
+// 144 bytes so 16-byte fragment reads of 16 consecutive rows fall in distinct banks.  Each wave
 // owns 128 x 64 of the tile as 4 x 2 blocks of v_mfma_f32_32x32x16_f16 (A = activations, B =
-// weights, so a D register holds 32 consecutive outputs of one token: coalesced stores).  Global
-// loads run three steps ahead in registers and are written to the other LDS stage after the
-// MFMAs of the current step: one barrier per step.
+// weights, so a D register holds 32 consecutive outputs of one token: coalesced stores).
+// With one wave per SIMD nothing else hides latency, so the step is a hand-built pipeline:
+//   * global loads run three steps ahead in registers, issued as opaque instructions so the
+//     compiler cannot sink them to their use, and awaited with an explicit s_waitcnt;
+//   * the dequantization of step t+1 (vector ALU) is interleaved with the MFMAs of step t
+//     (sched_group_barrier), its LDS writes go to the other stage, one barrier per step.
 #include "ojk_common.h"
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float2v __attribute__((ext_vector_type(2)));
 typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint u32x4 __attribute__((ext_vector_type(4)));
 
 #define GM_BM 256
 #define GM_BN 128
@@ -30,13 +37,14 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 #define GM_STRIDE 144  // bytes per LDS row: 64 f16 + 16 bytes of padding
 #define GM_STAGE ((GM_BM + GM_BN) * GM_STRIDE)
 
-// f32 -> f16 bits, the value pinned first so that "multiply/subtract, then convert" cannot be
-// folded into one mixed-precision FMA (which would round once and lose the sign of zero).
-__device__ __forceinline__ uint f16_bits_rn(float v) {
-    asm volatile("" : "+v"(v));
-    return (uint)__half_as_ushort(__float2half_rn(v));
+// Two f32 -> packed f16, round to nearest even.  The values are pinned in registers first so that
+// "multiply/subtract, then convert" cannot be folded into a mixed-precision FMA (which would
+// round once instead of twice and lose the sign of a zero product).
+__device__ __forceinline__ uint pack2(float a, float b) {
+    asm volatile("" : "+v"(a), "+v"(b));
+    float2v f = {a, b};
+    return __builtin_bit_cast(uint, __builtin_convertvector(f, half2v));
 }
-__device__ __forceinline__ uint pack2(float a, float b) { return f16_bits_rn(a) | (f16_bits_rn(b) << 16); }
 
 // ---- global loads whose issue point the compiler may not move -----------------------------------
 // The compiler sinks ordinary loads down to their first use to save registers, which turns a
@@ -45,7 +53,6 @@ __device__ __forceinline__ uint pack2(float a, float b) { return f16_bits_rn(a) 
 // re-defines the destination registers, so nothing that reads them can be scheduled above it.
 // Vector memory operations retire in order, so "at most n outstanding" means every load issued
 // before the last n has landed.
-typedef uint u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ u32x4 gm_load16(const void* p) {
     u32x4 v;
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
@@ -71,129 +78,141 @@ __device__ __forceinline__ void gm_wait(u32x4 (&x)[8]) {
 
 // ------------------------------------------------------------------ per-format slab loaders
 // A loader owns, for one thread, 32 weights of one row of the 128 x 64 slab: thread t -> row
-// t/2, half h = t%2.  `load` issues the global loads; `store` dequantizes into the LDS row.
+// t/2, half h = t%2.  `load` issues the global loads (NL of them); after the wait, `prep` unpacks
+// the scales, `part<I>` dequantizes a quarter of the weights (so the work can be spread between
+// MFMAs), `flush` writes the 32 f16 to the LDS row.
 struct LoaderQ4K {
-    static constexpr int NL = 2;  // global loads per slab
+    static constexpr int NL = 2;
     u32x4 hdr, qs;
     uint c;
-    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(hdr), "+v"(qs)::"memory"); }
+    float dl1, ml1, dl2, ml2;
+    uint lo[8], hi[8];
     static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * Q4K_BYTES; }
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(hdr), "+v"(qs)::"memory"); }
     __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
         const uchar* blk = row + (size_t)(k0 >> 8) * Q4K_BYTES;
         c = (k0 >> 6) & 3u;  // 32-byte chunk of the super-block = sub-blocks 2c, 2c+1
         hdr = gm_load16(blk);
         qs = gm_load16(blk + 16u + c * 32u + h * 16u);
     }
-    // 16 low-nibble weights -> slab columns 16h.., 16 high-nibble weights -> columns 32+16h..
-    __device__ __forceinline__ void store(uchar* lds_row, uint h) const {
+    __device__ __forceinline__ void prep() {
         uint sc, mn;
         q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
         float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
-        float dl1 = __fmul_rn(d, (float)(sc & 0xFFu)), ml1 = __fmul_rn(dmin, (float)(mn & 0xFFu));
-        float dl2 = __fmul_rn(d, (float)(sc >> 8)), ml2 = __fmul_rn(dmin, (float)(mn >> 8));
-        uint q[4] = {qs.x, qs.y, qs.z, qs.w};
-        uint lo[8], hi[8];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            uint v = q[i];
-            float a0 = (float)(v & 0xFu), a1 = (float)((v >> 8) & 0xFu), a2 = (float)((v >> 16) & 0xFu),
-                  a3 = (float)((v >> 24) & 0xFu);
-            float b0 = (float)((v >> 4) & 0xFu), b1 = (float)((v >> 12) & 0xFu), b2 = (float)((v >> 20) & 0xFu),
-                  b3 = (float)(v >> 28);
-            lo[2 * i] = pack2(__fsub_rn(__fmul_rn(dl1, a0), ml1), __fsub_rn(__fmul_rn(dl1, a1), ml1));
-            lo[2 * i + 1] = pack2(__fsub_rn(__fmul_rn(dl1, a2), ml1), __fsub_rn(__fmul_rn(dl1, a3), ml1));
-            hi[2 * i] = pack2(__fsub_rn(__fmul_rn(dl2, b0), ml2), __fsub_rn(__fmul_rn(dl2, b1), ml2));
-            hi[2 * i + 1] = pack2(__fsub_rn(__fmul_rn(dl2, b2), ml2), __fsub_rn(__fmul_rn(dl2, b3), ml2));
-        }
-        uint4* p = (uint4*)(lds_row + h * 32u);
-        p[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        p[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
-        uint4* ph = (uint4*)(lds_row + 64u + h * 32u);
-        ph[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-        ph[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+        dl1 = __fmul_rn(d, (float)(sc & 0xFFu));
+        ml1 = __fmul_rn(dmin, (float)(mn & 0xFFu));
+        dl2 = __fmul_rn(d, (float)(sc >> 8));
+        ml2 = __fmul_rn(dmin, (float)(mn >> 8));
+    }
+    template <int I>
+    __device__ __forceinline__ void part() {
+        const uint v = qs[I], l = v & 0x0F0F0F0Fu, u = (v >> 4) & 0x0F0F0F0Fu;
+        float a0 = (float)(l & 0xFFu), a1 = (float)((l >> 8) & 0xFFu), a2 = (float)((l >> 16) & 0xFFu), a3 = (float)(l >> 24);
+        float b0 = (float)(u & 0xFFu), b1 = (float)((u >> 8) & 0xFFu), b2 = (float)((u >> 16) & 0xFFu), b3 = (float)(u >> 24);
+        lo[2 * I] = pack2(__fsub_rn(__fmul_rn(dl1, a0), ml1), __fsub_rn(__fmul_rn(dl1, a1), ml1));
+        lo[2 * I + 1] = pack2(__fsub_rn(__fmul_rn(dl1, a2), ml1), __fsub_rn(__fmul_rn(dl1, a3), ml1));
+        hi[2 * I] = pack2(__fsub_rn(__fmul_rn(dl2, b0), ml2), __fsub_rn(__fmul_rn(dl2, b1), ml2));
+        hi[2 * I + 1] = pack2(__fsub_rn(__fmul_rn(dl2, b2), ml2), __fsub_rn(__fmul_rn(dl2, b3), ml2));
+    }
+    // 16 low-nibble weights -> slab columns 16h.., 16 high-nibble weights -> columns 32+16h..
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* p = (u32x4*)(lds_row + h * 32u);
+        p[0] = (u32x4){lo[0], lo[1], lo[2], lo[3]};
+        p[1] = (u32x4){lo[4], lo[5], lo[6], lo[7]};
+        u32x4* ph = (u32x4*)(lds_row + 64u + h * 32u);
+        ph[0] = (u32x4){hi[0], hi[1], hi[2], hi[3]};
+        ph[1] = (u32x4){hi[4], hi[5], hi[6], hi[7]};
     }
 };
 
+// 64-column slab j of a Q6_K super-block = half hf = j/2, quarters 2(j%2) and 2(j%2)+1: thread half
+// h owns columns 16h..16h+15 of each quarter (ql[16h..], ql[32+16h..], qh[16h..]), one sub-scale
+// per quarter: sc[2q + h].
 struct LoaderQ6K {
     static constexpr int NL = 6;
     u32x4 qa, qb, qh;
-    uint sca, scb, d16, hi_half;  // sca, scb: the sub-scales of the slab's two quarters for this thread's 16 columns
+    uint sca, scb, d16, p;  // p = j%2: which nibble of ql and which bit pairs of qh
+    float s0, s1;
+    uint o0[8], o1[8];
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * Q6K_BYTES; }
     __device__ __forceinline__ void pin() {
         asm volatile("" : "+v"(qa), "+v"(qb), "+v"(qh), "+v"(sca), "+v"(scb), "+v"(d16)::"memory");
     }
-    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * Q6K_BYTES; }
     __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
         const uchar* blk = row + (size_t)(k0 >> 8) * Q6K_BYTES;
-        uint j = (k0 >> 6) & 3u, hf = j >> 1;  // 64-column slab j of the super-block: half hf, quarters 2(j%2), +1
-        hi_half = j & 1u;
+        uint j = (k0 >> 6) & 3u, hf = j >> 1;
+        p = j & 1u;
         qa = gm_load16(blk + hf * 64u + h * 16u);
         qb = gm_load16(blk + hf * 64u + 32u + h * 16u);
         qh = gm_load16(blk + 128u + hf * 32u + h * 16u);
-        const uchar* sc = blk + 192u + hf * 8u + (j & 1u) * 4u + h;  // sc[2q + h], q = 2(j%2), 2(j%2)+1
+        const uchar* sc = blk + 192u + hf * 8u + p * 4u + h;
         sca = gm_load_u8(sc);
         scb = gm_load_u8(sc + 2);
         d16 = gm_load_u16(blk + 208u);
     }
-    __device__ __forceinline__ void store(uchar* lds_row, uint h) const {
+    __device__ __forceinline__ void prep() {
         float d = f16_bits_to_f32(d16);
-        float s0 = __fmul_rn(d, (float)(signed char)sca), s1 = __fmul_rn(d, (float)(signed char)scb);
-        uint a[4] = {qa.x, qa.y, qa.z, qa.w}, b[4] = {qb.x, qb.y, qb.z, qb.w}, hq[4] = {qh.x, qh.y, qh.z, qh.w};
-        uint o0[8], o1[8];
-        const uint sh_h0 = hi_half ? 4u : 0u, sh_h1 = hi_half ? 6u : 2u, sh_l = hi_half ? 4u : 0u;
+        s0 = __fmul_rn(d, (float)(signed char)sca);
+        s1 = __fmul_rn(d, (float)(signed char)scb);
+    }
+    template <int I>
+    __device__ __forceinline__ void part() {
+        // low 4 bits: nibble p of ql; high 2 bits: bits 4p..4p+1 (first quarter) / 4p+2..4p+3 of qh
+        const uint a = (qa[I] >> (4u * p)) & 0x0F0F0F0Fu, b = (qb[I] >> (4u * p)) & 0x0F0F0F0Fu;
+        const uint h = qh[I] >> (4u * p);
+        const uint w0 = a | ((h << 4) & 0x30303030u), w1 = b | ((h << 2) & 0x30303030u);
+        float e0[4], e1[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float w0[4], w1[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                uint av = (a[i] >> (8 * e)) & 0xFFu, bv = (b[i] >> (8 * e)) & 0xFFu, hv = (hq[i] >> (8 * e)) & 0xFFu;
-                int q0 = (int)(((av >> sh_l) & 0xFu) | (((hv >> sh_h0) & 3u) << 4)) - 32;
-                int q1 = (int)(((bv >> sh_l) & 0xFu) | (((hv >> sh_h1) & 3u) << 4)) - 32;
-                w0[e] = __fmul_rn(s0, (float)q0);
-                w1[e] = __fmul_rn(s1, (float)q1);
-            }
-            o0[2 * i] = pack2(w0[0], w0[1]);
-            o0[2 * i + 1] = pack2(w0[2], w0[3]);
-            o1[2 * i] = pack2(w1[0], w1[1]);
-            o1[2 * i + 1] = pack2(w1[2], w1[3]);
+        for (int e = 0; e < 4; e++) {
+            e0[e] = __fmul_rn(s0, (float)((int)((w0 >> (8 * e)) & 0xFFu) - 32));
+            e1[e] = __fmul_rn(s1, (float)((int)((w1 >> (8 * e)) & 0xFFu) - 32));
         }
-        uint4* p = (uint4*)(lds_row + h * 32u);
-        p[0] = make_uint4(o0[0], o0[1], o0[2], o0[3]);
-        p[1] = make_uint4(o0[4], o0[5], o0[6], o0[7]);
-        uint4* ph = (uint4*)(lds_row + 64u + h * 32u);
-        ph[0] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
-        ph[1] = make_uint4(o1[4], o1[5], o1[6], o1[7]);
+        o0[2 * I] = pack2(e0[0], e0[1]);
+        o0[2 * I + 1] = pack2(e0[2], e0[3]);
+        o1[2 * I] = pack2(e1[0], e1[1]);
+        o1[2 * I + 1] = pack2(e1[2], e1[3]);
+    }
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* q = (u32x4*)(lds_row + h * 32u);
+        q[0] = (u32x4){o0[0], o0[1], o0[2], o0[3]};
+        q[1] = (u32x4){o0[4], o0[5], o0[6], o0[7]};
+        u32x4* qh_ = (u32x4*)(lds_row + 64u + h * 32u);
+        qh_[0] = (u32x4){o1[0], o1[1], o1[2], o1[3]};
+        qh_[1] = (u32x4){o1[4], o1[5], o1[6], o1[7]};
     }
 };
 
+// The slab's two Q8_0 blocks: thread half h owns block h = slab columns 32h..32h+31.
 struct LoaderQ80 {
     static constexpr int NL = 3;
     u32x4 qa, qb;
     uint d16;
-    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(qa), "+v"(qb), "+v"(d16)::"memory"); }
+    float d;
+    uint o[16];
     static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 5) * Q80_BYTES; }
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(qa), "+v"(qb), "+v"(d16)::"memory"); }
     __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
-        const uchar* blk = row + (size_t)((k0 >> 5) + h) * Q80_BYTES;  // block h of the slab's two
+        const uchar* blk = row + (size_t)((k0 >> 5) + h) * Q80_BYTES;
         d16 = gm_load_u16(blk);
         qa = gm_load16(blk + 2u);
         qb = gm_load16(blk + 18u);
     }
-    // block h fills slab columns 32h..32h+31
-    __device__ __forceinline__ void store(uchar* lds_row, uint h) const {
-        float d = f16_bits_to_f32(d16);
-        uint q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
-        uint o[16];
+    __device__ __forceinline__ void prep() { d = f16_bits_to_f32(d16); }
+    template <int I>
+    __device__ __forceinline__ void part() {
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            float v0 = __fmul_rn(d, (float)(signed char)(q[i]));
-            float v1 = __fmul_rn(d, (float)(signed char)(q[i] >> 8));
-            float v2 = __fmul_rn(d, (float)(signed char)(q[i] >> 16));
-            float v3 = __fmul_rn(d, (float)((int)q[i] >> 24));
-            o[2 * i] = pack2(v0, v1);
-            o[2 * i + 1] = pack2(v2, v3);
+        for (int s = 0; s < 2; s++) {
+            const uint q = s ? qb[I] : qa[I];
+            float v0 = __fmul_rn(d, (float)(signed char)(q)), v1 = __fmul_rn(d, (float)(signed char)(q >> 8));
+            float v2 = __fmul_rn(d, (float)(signed char)(q >> 16)), v3 = __fmul_rn(d, (float)((int)q >> 24));
+            o[8 * s + 2 * I] = pack2(v0, v1);
+            o[8 * s + 2 * I + 1] = pack2(v2, v3);
         }
-        uint4* p = (uint4*)(lds_row + h * 64u);
+    }
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* q = (u32x4*)(lds_row + h * 64u);
 #pragma unroll
-        for (int i = 0; i < 4; i++) p[i] = make_uint4(o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]);
+        for (int i = 0; i < 4; i++) q[i] = (u32x4){o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
     }
 };
 
@@ -219,10 +238,14 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
     const ushort* xrow[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) xrow[i] = xh + (size_t)min(m0 + xr + 32u * i, M - 1u) * K + xc;
+    const uint x_lds = xr * GM_STRIDE + xc * 2u;                   // + i * 32 rows
+    const uint w_lds = GM_BM * GM_STRIDE + wr * GM_STRIDE;
 
     // wave tile: 128 (m) x 64 (n)
     const uint wm = (wave >> 1) * 128u, wn = (wave & 1u) * 64u;
     const uint fr = lane & 31u, kg = lane >> 5;
+    const uint a_lds = (wm + fr) * GM_STRIDE + kg * 16u;           // + i * 32 rows, + ks * 32 bytes
+    const uint b_lds = GM_BM * GM_STRIDE + (wn + fr) * GM_STRIDE + kg * 16u;
     float16v acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; i++)
@@ -231,51 +254,16 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    // Three register sets hold the slabs of steps t+1 .. t+3 while step t runs from LDS: loads are
-    // in flight for two whole steps before anyone waits for them (one wave per SIMD cannot lean
-    // on other waves to cover HBM latency).
     u32x4 xs0[8], xs1[8], xs2[8];
     Loader ld0, ld1, ld2;
     const uint nt = (k_end - k_begin) / GM_BK;
+    constexpr int LPS = 8 + Loader::NL;  // loads per slab
 
 #define GM_LOAD(XS, LD, T)                                                                       \
     do {                                                                                         \
         const uint kk_ = k_begin + (T) * GM_BK;                                                  \
         _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++) XS[i_] = gm_load16(xrow[i_] + kk_);      \
         LD.load(wrow, kk_, wh);                                                                  \
-    } while (0)
-#define GM_STORE(XS, LD, STG)                                                                    \
-    do {                                                                                         \
-        uchar* a_ = lds + (STG) * GM_STAGE;                                                      \
-        _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++)                                         \
-            *(u32x4*)(a_ + (xr + 32u * i_) * GM_STRIDE + xc * 2u) = XS[i_];                      \
-        LD.store(a_ + GM_BM * GM_STRIDE + wr * GM_STRIDE, wh);                                   \
-    } while (0)
-#define GM_COMPUTE(STG)                                                                          \
-    do {                                                                                         \
-        const uchar* a_ = lds + (STG) * GM_STAGE;                                                \
-        const uchar* b_ = a_ + GM_BM * GM_STRIDE;                                                \
-        _Pragma("unroll") for (int ks = 0; ks < GM_BK / 16; ks++) {                              \
-            half8 af[4], bf[2];                                                                  \
-            _Pragma("unroll") for (int i = 0; i < 4; i++)                                        \
-                af[i] = *(const half8*)(a_ + (wm + 32u * i + fr) * GM_STRIDE + (ks * 16u + kg * 8u) * 2u); \
-            _Pragma("unroll") for (int j = 0; j < 2; j++)                                        \
-                bf[j] = *(const half8*)(b_ + (wn + 32u * j + fr) * GM_STRIDE + (ks * 16u + kg * 8u) * 2u); \
-            _Pragma("unroll") for (int i = 0; i < 4; i++)                                        \
-                _Pragma("unroll") for (int j = 0; j < 2; j++)                                    \
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0); \
-        }                                                                                        \
-    } while (0)
-// step T: refill the set that step T's slab came from, run step T, stage step T+1
-#define GM_STEP(T, XS_FREE, LD_FREE, XS_NEXT, LD_NEXT)                                           \
-    do {                                                                                         \
-        if ((T) + 3u < nt) GM_LOAD(XS_FREE, LD_FREE, (T) + 3u);                                  \
-        GM_COMPUTE((T) & 1u);                                                                    \
-        if ((T) + 1u < nt) {                                                                     \
-            GM_WAIT_FOR(XS_NEXT, LD_NEXT, (T) + 1u);                                             \
-            GM_STORE(XS_NEXT, LD_NEXT, ((T) + 1u) & 1u);                                         \
-        }                                                                                        \
-        __syncthreads();                                                                         \
     } while (0)
 // wait for the slab of step T: the slabs of steps T+1 and T+2, where they exist, were issued later
 #define GM_WAIT_FOR(XS, LD, T)                                                                   \
@@ -285,24 +273,108 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
         else gm_wait<0>(XS);                                                                     \
         LD.pin();                                                                                \
     } while (0)
-    constexpr int LPS = 8 + Loader::NL;  // loads per slab
+#define GM_STORE_X(XS, STG)                                                                      \
+    do {                                                                                         \
+        uchar* a_ = lds + (STG) * GM_STAGE + x_lds;                                              \
+        _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++) *(u32x4*)(a_ + i_ * 32u * GM_STRIDE) = XS[i_]; \
+    } while (0)
+// fragments of K sub-step KS of stage STG into registers AF/BF; the MFMAs that consume them
+#define GM_READ(STG, KS, AF, BF)                                                                 \
+    do {                                                                                         \
+        const uchar* s_ = lds + (STG) * GM_STAGE;                                                \
+        _Pragma("unroll") for (int i = 0; i < 4; i++)                                            \
+            AF[i] = *(const half8*)(s_ + a_lds + i * 32u * GM_STRIDE + (KS) * 32u);              \
+        _Pragma("unroll") for (int j = 0; j < 2; j++)                                            \
+            BF[j] = *(const half8*)(s_ + b_lds + j * 32u * GM_STRIDE + (KS) * 32u);              \
+    } while (0)
+#define GM_MMA(AF, BF)                                                                           \
+    do {                                                                                         \
+        _Pragma("unroll") for (int i = 0; i < 4; i++)                                            \
+            _Pragma("unroll") for (int j = 0; j < 2; j++)                                        \
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(AF[i], BF[j], acc[i][j], 0, 0, 0); \
+    } while (0)
+#define GM_MFMA(STG, KS)                                                                         \
+    do {                                                                                         \
+        half8 af_[4], bf_[2];                                                                    \
+        GM_READ(STG, KS, af_, bf_);                                                              \
+        GM_MMA(af_, bf_);                                                                        \
+    } while (0)
+// interleave: one MFMA, one LDS read (the next sub-step's fragments), a few vector-ALU
+// instructions (the next step's dequantization) — eight times
+#define GM_MIX()                                                                                 \
+    do {                                                                                         \
+        _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {                                       \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                   \
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                   \
+            __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);                                   \
+        }                                                                                        \
+    } while (0)
+// Interior step T (steps T+1 .. T+3 exist): no branches, so MFMAs and dequantization share one
+// scheduling region.  Fragments are read one sub-step ahead of the MFMAs that use them.
+#define GM_STEP_FULL(T, XS_FREE, LD_FREE, XS_NEXT, LD_NEXT)                                      \
+    do {                                                                                         \
+        const uint cur_ = (T) & 1u, nxt_ = cur_ ^ 1u;                                            \
+        half8 afA[4], bfA[2], afB[4], bfB[2];                                                    \
+        GM_READ(cur_, 0, afA, bfA);                                                              \
+        GM_LOAD(XS_FREE, LD_FREE, (T) + 3u);                                                     \
+        gm_wait<2 * LPS>(XS_NEXT);                                                               \
+        LD_NEXT.pin();                                                                           \
+        LD_NEXT.prep();                                                                          \
+        GM_READ(cur_, 1, afB, bfB); GM_MMA(afA, bfA); LD_NEXT.template part<0>(); GM_MIX();      \
+        GM_READ(cur_, 2, afA, bfA); GM_MMA(afB, bfB); LD_NEXT.template part<1>(); GM_MIX();      \
+        GM_READ(cur_, 3, afB, bfB); GM_MMA(afA, bfA); LD_NEXT.template part<2>(); GM_MIX();      \
+        GM_MMA(afB, bfB); LD_NEXT.template part<3>(); GM_MIX();                                  \
+        GM_STORE_X(XS_NEXT, nxt_);                                                               \
+        LD_NEXT.flush(lds + nxt_ * GM_STAGE + w_lds, wh);                                        \
+        __syncthreads();                                                                         \
+    } while (0)
+// Guarded step for the head and tail of the K range.
+#define GM_STEP_ANY(T, XS_FREE, LD_FREE, XS_NEXT, LD_NEXT)                                       \
+    do {                                                                                         \
+        if ((T) + 3u < nt) GM_LOAD(XS_FREE, LD_FREE, (T) + 3u);                                  \
+        const uint cur_ = (T) & 1u, nxt_ = cur_ ^ 1u;                                            \
+        GM_MFMA(cur_, 0); GM_MFMA(cur_, 1); GM_MFMA(cur_, 2); GM_MFMA(cur_, 3);                  \
+        if ((T) + 1u < nt) {                                                                     \
+            GM_WAIT_FOR(XS_NEXT, LD_NEXT, (T) + 1u);                                             \
+            LD_NEXT.prep();                                                                      \
+            LD_NEXT.template part<0>(); LD_NEXT.template part<1>();                              \
+            LD_NEXT.template part<2>(); LD_NEXT.template part<3>();                              \
+            GM_STORE_X(XS_NEXT, nxt_);                                                           \
+            LD_NEXT.flush(lds + nxt_ * GM_STAGE + w_lds, wh);                                    \
+        }                                                                                        \
+        __syncthreads();                                                                         \
+    } while (0)
 
     GM_LOAD(xs0, ld0, 0u);
     if (nt > 1u) GM_LOAD(xs1, ld1, 1u);
     if (nt > 2u) GM_LOAD(xs2, ld2, 2u);
     GM_WAIT_FOR(xs0, ld0, 0u);
-    GM_STORE(xs0, ld0, 0u);
+    ld0.prep();
+    ld0.template part<0>(); ld0.template part<1>(); ld0.template part<2>(); ld0.template part<3>();
+    GM_STORE_X(xs0, 0u);
+    ld0.flush(lds + w_lds, wh);
     __syncthreads();
-    for (uint t = 0; t < nt; t += 3u) {
-        GM_STEP(t, xs0, ld0, xs1, ld1);
-        if (t + 1u < nt) GM_STEP(t + 1u, xs1, ld1, xs2, ld2);
-        if (t + 2u < nt) GM_STEP(t + 2u, xs2, ld2, xs0, ld0);
+
+    uint t = 0;
+    for (; t + 6u <= nt; t += 3u) {  // steps t, t+1, t+2 all have three successors
+        GM_STEP_FULL(t, xs0, ld0, xs1, ld1);
+        GM_STEP_FULL(t + 1u, xs1, ld1, xs2, ld2);
+        GM_STEP_FULL(t + 2u, xs2, ld2, xs0, ld0);
+    }
+    for (; t < nt; t += 3u) {
+        GM_STEP_ANY(t, xs0, ld0, xs1, ld1);
+        if (t + 1u < nt) GM_STEP_ANY(t + 1u, xs1, ld1, xs2, ld2);
+        if (t + 2u < nt) GM_STEP_ANY(t + 2u, xs2, ld2, xs0, ld0);
     }
 #undef GM_LOAD
-#undef GM_STORE
-#undef GM_COMPUTE
-#undef GM_STEP
 #undef GM_WAIT_FOR
+#undef GM_STORE_X
+#undef GM_MFMA
+#undef GM_READ
+#undef GM_MMA
+#undef GM_MIX
+#undef GM_STEP_FULL
+#undef GM_STEP_ANY
 
     // epilogue: D register v of block (i, j) holds row 8*(v/4) + 4*kg + v%4, column fr
 #pragma unroll

@@ -60,6 +60,32 @@ def test_gemm_bf16_activations(gpu, orc, pkg, ty):
     assert e32[0] < 2e-2 and e32[1] < 3e-3, e32
 
 
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
+def test_tile_holds_the_reference_decoders_bits(gpu, orc, pkg, ty):
+    """One-hot activations read the tile back: y[m][n] must be dequant_to_f16(W)[n][m] exactly,
+    for every weight of two super-blocks per row and for extreme scales."""
+    k, n = 512, 160
+    bb, wpb = pkg.synth.BLOCK_SHAPE[ty]
+    raw = orc.synth_blocks(ty, n * k // wpb).reshape(-1, bb).copy()
+    scales = np.array([0x0001, 0x03FF, 0x0400, 0x8001, 0xBC00, 0x3555, 0x1234, 0x2E66], np.uint16)
+    off = 208 if ty == Q6_K else 0
+    for i in range(raw.shape[0]):
+        raw[i, off:off + 2] = scales[i % 8:i % 8 + 1].view(np.uint8)
+        if ty == Q4_K:
+            raw[i, 2:4] = scales[(i * 3 + 1) % 8:(i * 3 + 1) % 8 + 1].view(np.uint8)
+    raw = raw.reshape(-1)
+    want = orc.dequant_to_f16(raw, ty, n * k).view(np.float16).astype(np.float32).reshape(n, k)
+    lin = gpu.lin(ty, n, k, raw)
+    x = np.eye(k, dtype=np.float32)
+    yd = gpu.alloc(k * n)
+    gpu.mm(gpu.upload(x), lin, yd, k, act_mode=pkg.ACT_FLOAT)
+    got = gpu.read(yd, k * n).reshape(k, n)
+    # value equality: a -0 weight reads back as +0 through the accumulator, every other bit must match
+    assert np.array_equal(got, want.T)
+    nz = want.T != 0
+    assert np.array_equal(got.view(np.uint32)[nz], want.T.copy().view(np.uint32)[nz])
+
+
 def test_split_k_entry_through_the_kernel_seam(gpu, orc, pkg):
     """gemm_mm_q4k_sk dispatched by name with several K slices; y holds what is accumulated into."""
     gpu.ensure_family("gemm")
