@@ -1,0 +1,257 @@
+// Family "moe": router and grouped expert FFN on raw Q4_K expert tensors.
+//
+// Semantics (reference: router crates/ojas-cuda/src/kernels/moe.rs:45-70; expert FFN
+// crates/ojas-cpu/src/cpu_glm.rs:551-582, batched per-assignment GPU form
+// crates/ojas-metal/src/kernels/moe.rs:199-272):
+//   idx, wgt = top-KSEL of softmax(logits), lowest index wins ties, weights renormalised
+//   for every assignment a = (token t, slot j), e = idx[a]:
+//       act[a] = silu(Wg_e x_t) * (Wu_e x_t);   dv[a] = Wd_e act[a]
+//   y[t] (+)= sum_j wgt[t][j] * dv[t*KSEL + j]           (slot order, f32)
+// with every matvec in the CPU reference's arithmetic (activations quantized per 256 by quant_q8k,
+// integer dots, crates/ojas-cpu/src/cpu_math.rs:539-635).
+//
+// The reference launches one workgroup column per assignment and leans on the cache for experts
+// shared by several tokens.  Here assignments are grouped by expert first (moe_group: counting
+// sort -> per-expert offsets + assignment list), and one launch per projection walks the
+// experts: a wave loads its rows of expert e once into registers and runs them against every
+// token routed to e, so an expert's bytes cross HBM once however many tokens chose it.
+//
+//   moe_topk(lg, idx, wgt, E, KSEL)                          one token, 1 x 64 threads
+//   moe_topk_m(lg, idx, wgt, E, KSEL)                        grid = tokens
+//   moe_group(idx, counts, offsets, list, NA, E)             1 x 256 threads; NA = tokens*KSEL
+//   moe_gu_q4k_m(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA)   grid (ceil(N/8), E)
+//   moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)            grid (ceil(N/16), E)
+//   moe_combine(dv, wgt, y, T, KSEL, D, ACC)                 grid ceil(T*D/256)
+#include "ojk_common.h"
+#include "ojk_q4k_dot.h"
+
+// ------------------------------------------------------------------ router
+__device__ __forceinline__ void moe_topk_body(const float* __restrict__ lg, uint* __restrict__ idx,
+                                              float* __restrict__ wgt, uint E, uint KSEL) {
+    // one wave per token; lane l owns experts l, l+64, ... (E <= 1024)
+    const uint lane = threadIdx.x & 63u;
+    float p[16];
+    float mx = -3.4028235e38f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        uint e = lane + 64u * i;
+        p[i] = e < E ? lg[e] : -3.4028235e38f;
+        mx = fmaxf(mx, p[i]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        uint e = lane + 64u * i;
+        p[i] = e < E ? expf(p[i] - mx) : -1.0f;
+        if (e < E) sum += p[i];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+        if (lane + 64u * i < E) p[i] = p[i] / sum;
+    float wsum = 0.0f, mine = 0.0f;
+    uint mine_idx = 0;
+    for (uint j = 0; j < KSEL; j++) {
+        float bv = -1.0f;
+        uint bi = 0xFFFFFFFFu;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {  // ascending expert index within the lane: '>' keeps the lowest
+            if (p[i] > bv) { bv = p[i]; bi = lane + 64u * i; }
+        }
+        float m2 = wave_max(bv);
+        // lowest index among the lanes holding the maximum
+        uint cand = (bv == m2) ? bi : 0xFFFFFFFFu;
+        cand = min(cand, (uint)dpp_i32<OJK_DPP_QUAD_XOR1>((int)cand));
+        cand = min(cand, (uint)dpp_i32<OJK_DPP_QUAD_XOR2>((int)cand));
+        cand = min(cand, (uint)dpp_i32<OJK_DPP_ROW_HALF_MIRROR>((int)cand));
+        cand = min(cand, (uint)dpp_i32<OJK_DPP_ROW_MIRROR>((int)cand));
+        uint c0 = (uint)__builtin_amdgcn_readlane((int)cand, 0), c1 = (uint)__builtin_amdgcn_readlane((int)cand, 16);
+        uint c2 = (uint)__builtin_amdgcn_readlane((int)cand, 32), c3 = (uint)__builtin_amdgcn_readlane((int)cand, 48);
+        uint win = min(min(c0, c1), min(c2, c3));
+        wsum += m2;
+        if (lane == j) { mine = m2; mine_idx = win; }
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            if (lane + 64u * i == win) p[i] = -1.0f;
+    }
+    if (lane < KSEL) {
+        idx[lane] = mine_idx;
+        wgt[lane] = mine / wsum;
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(64)
+moe_topk(const float* lg, uint* idx, float* wgt, uint E, uint KSEL) {
+    moe_topk_body(lg, idx, wgt, E, KSEL);
+}
+extern "C" __global__ void __launch_bounds__(64)
+moe_topk_m(const float* lg, uint* idx, float* wgt, uint E, uint KSEL) {
+    const size_t t = blockIdx.x;
+    moe_topk_body(lg + t * E, idx + t * KSEL, wgt + t * KSEL, E, KSEL);
+}
+
+// ------------------------------------------------------------------ grouping
+// Counting sort of the NA assignments by expert: counts[E], offsets[E+1], list[NA] (assignment
+// ids, expert-major; the order inside an expert's group is arbitrary and has no effect on the
+// results, which are stored per assignment).  One workgroup; E <= 1024.
+extern "C" __global__ void __launch_bounds__(256)
+moe_group(const uint* __restrict__ idx, uint* __restrict__ counts, uint* __restrict__ offsets,
+          uint* __restrict__ list, uint NA, uint E) {
+    __shared__ uint cnt[1024];
+    __shared__ uint off[1025];
+    const uint tid = threadIdx.x;
+    for (uint e = tid; e < E; e += 256u) cnt[e] = 0u;
+    __syncthreads();
+    for (uint a = tid; a < NA; a += 256u) {
+        uint e = idx[a];
+        if (e < E) atomicAdd(&cnt[e], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint run = 0;
+        for (uint e = 0; e < E; e++) { off[e] = run; run += cnt[e]; }
+        off[E] = run;
+    }
+    __syncthreads();
+    for (uint e = tid; e <= E; e += 256u) {
+        offsets[e] = off[e];
+        if (e < E) counts[e] = cnt[e];
+    }
+    for (uint e = tid; e < E; e += 256u) cnt[e] = 0u;  // reused as the per-expert cursor
+    __syncthreads();
+    for (uint a = tid; a < NA; a += 256u) {
+        uint e = idx[a];
+        if (e < E) list[off[e] + atomicAdd(&cnt[e], 1u)] = a;
+    }
+}
+
+// ------------------------------------------------------------------ grouped gate / up
+// Block (rb, e): 4 waves x 2 rows = 8 rows of expert e's gate and up.  K must be a multiple of
+// 256; a wave walks K in steps of 8 super-blocks (one step for the usual hidden sizes).
+extern "C" __global__ void __launch_bounds__(256)
+moe_gu_q4k_m(const signed char* __restrict__ xq, const float* __restrict__ xs, const uchar* __restrict__ wg,
+             const uchar* __restrict__ wu, float* __restrict__ act, const uint* __restrict__ offsets,
+             const uint* __restrict__ list, uint K, uint N, uint KSEL, uint NA) {
+    const uint e = blockIdx.y;
+    const uint a0 = min(offsets[e], NA), a1 = min(offsets[e + 1], NA);
+    if (a0 >= a1) return;
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 2u;
+    if (row0 >= N) return;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    const size_t rb = (size_t)nsb * Q4K_BYTES;
+    const uchar* g0 = wg + ((size_t)e * N + row0) * rb;
+    const uchar* u0 = wu + ((size_t)e * N + row0) * rb;
+    const bool two = row0 + 1u < N;
+    const size_t r1 = two ? rb : 0;
+    if (nsb <= 8u) {
+        // the whole row fits one step: weights stay in registers across the expert's tokens
+        const bool on = g < nsb;
+        const size_t o = (size_t)(on ? g : 0u) * Q4K_BYTES;
+        uint4 hg0 = *(const uint4*)(g0 + o), qg0 = *(const uint4*)(g0 + o + 16u + l * 16u);
+        uint4 hg1 = *(const uint4*)(g0 + r1 + o), qg1 = *(const uint4*)(g0 + r1 + o + 16u + l * 16u);
+        uint4 hu0 = *(const uint4*)(u0 + o), qu0 = *(const uint4*)(u0 + o + 16u + l * 16u);
+        uint4 hu1 = *(const uint4*)(u0 + r1 + o), qu1 = *(const uint4*)(u0 + r1 + o + 16u + l * 16u);
+        for (uint i = a0; i < a1; i++) {
+            const uint a = min(list[i], NA - 1u), t = a / KSEL;
+            Q4kFrag f = q4k_load_frag(xq + (size_t)t * nsb * 256u, xs + (size_t)t * nsb, on ? g : 0u, l);
+            float vg0 = on ? q4k_lane_dot(hg0, qg0, c, f) : 0.0f, vg1 = on ? q4k_lane_dot(hg1, qg1, c, f) : 0.0f;
+            float vu0 = on ? q4k_lane_dot(hu0, qu0, c, f) : 0.0f, vu1 = on ? q4k_lane_dot(hu1, qu1, c, f) : 0.0f;
+            vg0 = wave_sum(vg0); vg1 = wave_sum(vg1); vu0 = wave_sum(vu0); vu1 = wave_sum(vu1);
+            if (lane == 0) {
+                float* o_ = act + (size_t)a * N + row0;
+                o_[0] = (vg0 / (1.0f + expf(-vg0))) * vu0;
+                if (two) o_[1] = (vg1 / (1.0f + expf(-vg1))) * vu1;
+            }
+        }
+    } else {
+        for (uint i = a0; i < a1; i++) {
+            const uint a = min(list[i], NA - 1u), t = a / KSEL;
+            float vg0 = 0.0f, vg1 = 0.0f, vu0 = 0.0f, vu1 = 0.0f;
+            for (uint sb = g; sb < nsb; sb += 8u) {
+                const size_t o = (size_t)sb * Q4K_BYTES;
+                Q4kFrag f = q4k_load_frag(xq + (size_t)t * nsb * 256u, xs + (size_t)t * nsb, sb, l);
+                vg0 += q4k_lane_dot(*(const uint4*)(g0 + o), *(const uint4*)(g0 + o + 16u + l * 16u), c, f);
+                vg1 += q4k_lane_dot(*(const uint4*)(g0 + r1 + o), *(const uint4*)(g0 + r1 + o + 16u + l * 16u), c, f);
+                vu0 += q4k_lane_dot(*(const uint4*)(u0 + o), *(const uint4*)(u0 + o + 16u + l * 16u), c, f);
+                vu1 += q4k_lane_dot(*(const uint4*)(u0 + r1 + o), *(const uint4*)(u0 + r1 + o + 16u + l * 16u), c, f);
+            }
+            vg0 = wave_sum(vg0); vg1 = wave_sum(vg1); vu0 = wave_sum(vu0); vu1 = wave_sum(vu1);
+            if (lane == 0) {
+                float* o_ = act + (size_t)a * N + row0;
+                o_[0] = (vg0 / (1.0f + expf(-vg0))) * vu0;
+                if (two) o_[1] = (vg1 / (1.0f + expf(-vg1))) * vu1;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ grouped down
+// Block (rb, e): 4 waves x 4 rows = 16 rows of expert e's down projection, against the quantized
+// act of every assignment routed to e.  dv[a][n] holds the unweighted result.
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q4k_m(const signed char* __restrict__ aq, const float* __restrict__ as_, const uchar* __restrict__ wd,
+               float* __restrict__ dv, const uint* __restrict__ offsets, const uint* __restrict__ list,
+               uint K, uint N, uint NA) {
+    const uint e = blockIdx.y;
+    const uint a0 = min(offsets[e], NA), a1 = min(offsets[e + 1], NA);
+    if (a0 >= a1) return;
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 4u;
+    if (row0 >= N) return;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    const size_t rb = (size_t)nsb * Q4K_BYTES;
+    const uchar* w0 = wd + ((size_t)e * N + row0) * rb;
+    if (nsb <= 8u) {
+        const bool on = g < nsb;
+        const size_t o = (size_t)(on ? g : 0u) * Q4K_BYTES;
+        uint4 h[4], q[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const size_t ro = (size_t)min((uint)r, N - 1u - row0) * rb;
+            h[r] = *(const uint4*)(w0 + ro + o);
+            q[r] = *(const uint4*)(w0 + ro + o + 16u + l * 16u);
+        }
+        for (uint i = a0; i < a1; i++) {
+            const uint a = min(list[i], NA - 1u);
+            Q4kFrag f = q4k_load_frag(aq + (size_t)a * nsb * 256u, as_ + (size_t)a * nsb, on ? g : 0u, l);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float v = wave_sum(on ? q4k_lane_dot(h[r], q[r], c, f) : 0.0f);
+                if (lane == 0 && row0 + r < N) dv[(size_t)a * N + row0 + r] = v;
+            }
+        }
+    } else {
+        for (uint i = a0; i < a1; i++) {
+            const uint a = min(list[i], NA - 1u);
+            float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (uint sb = g; sb < nsb; sb += 8u) {
+                Q4kFrag f = q4k_load_frag(aq + (size_t)a * nsb * 256u, as_ + (size_t)a * nsb, sb, l);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const uchar* blk = w0 + (size_t)min((uint)r, N - 1u - row0) * rb + (size_t)sb * Q4K_BYTES;
+                    v[r] += q4k_lane_dot(*(const uint4*)blk, *(const uint4*)(blk + 16u + l * 16u), c, f);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float s = wave_sum(v[r]);
+                if (lane == 0 && row0 + r < N) dv[(size_t)a * N + row0 + r] = s;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ combine
+// y[t][i] (=, +=) sum_j wgt[t][j] * dv[t*KSEL + j][i], slots in order.
+extern "C" __global__ void __launch_bounds__(256)
+moe_combine(const float* __restrict__ dv, const float* __restrict__ wgt, float* __restrict__ y,
+            uint T, uint KSEL, uint D, uint ACC) {
+    const size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+    if (i >= (size_t)T * D) return;
+    const uint t = (uint)(i / D), col = (uint)(i % D);
+    float acc = ACC ? y[i] : 0.0f;
+    for (uint j = 0; j < KSEL; j++) acc += wgt[(size_t)t * KSEL + j] * dv[((size_t)t * KSEL + j) * D + col];
+    y[i] = acc;
+}

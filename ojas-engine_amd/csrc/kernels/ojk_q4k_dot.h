@@ -1,0 +1,53 @@
+// The lane-level Q4_K x int8 dot shared by the decode matvecs and the MoE expert kernels:
+// the arithmetic of the CPU reference's dot_q4k (crates/ojas-cpu/src/cpu_math.rs:609-635) for the
+// 32 weights one lane owns.
+#pragma once
+#include "ojk_common.h"
+
+__device__ __forceinline__ int bytesum4(uint4 v) {
+    int s = dot4_i8(v.x, 0x01010101u, 0);
+    s = dot4_i8(v.y, 0x01010101u, s);
+    s = dot4_i8(v.z, 0x01010101u, s);
+    return dot4_i8(v.w, 0x01010101u, s);
+}
+
+// Eight lanes share a super-block and a wave walks eight super-blocks (2048 weights) per step.
+// Lane (g, l) = (lane/8, lane%8) owns the 16 quant bytes l*16..l*16+15 of super-block g: 16
+// low-nibble weights of sub-block 2c and 16 high-nibble weights of sub-block 2c+1, c = l/2.  The
+// activation fragment (2 x 16 int8, their sums, the segment scale) is loaded once per step and
+// reused across the R rows of the wave.
+struct Q4kFrag {
+    uint4 xl, xh;  // int8 activations for the low / high nibble halves
+    int bl, bh;    // their sums (the lane's part of bsums)
+    float sx;      // activation scale of the super-block
+};
+
+__device__ __forceinline__ Q4kFrag q4k_load_frag(const signed char* xq, const float* xs, uint sb, uint l) {
+    Q4kFrag f;
+    const signed char* p = xq + (size_t)sb * 256u + (l >> 1) * 64u + (l & 1u) * 16u;
+    f.xl = *(const uint4*)p;
+    f.xh = *(const uint4*)(p + 32);
+    f.bl = bytesum4(f.xl);
+    f.bh = bytesum4(f.xh);
+    f.sx = xs[sb];
+    return f;
+}
+
+// One lane's 32 weights of one super-block against one activation fragment.
+__device__ __forceinline__ float q4k_lane_dot(uint4 hdr, uint4 qs, uint c, const Q4kFrag& f) {
+    const uint M4 = 0x0F0F0F0Fu;
+    int il = dot4_i8(qs.x & M4, f.xl.x, 0);
+    il = dot4_i8(qs.y & M4, f.xl.y, il);
+    il = dot4_i8(qs.z & M4, f.xl.z, il);
+    il = dot4_i8(qs.w & M4, f.xl.w, il);
+    int ih = dot4_i8((qs.x >> 4) & M4, f.xh.x, 0);
+    ih = dot4_i8((qs.y >> 4) & M4, f.xh.y, ih);
+    ih = dot4_i8((qs.z >> 4) & M4, f.xh.z, ih);
+    ih = dot4_i8((qs.w >> 4) & M4, f.xh.w, ih);
+    uint sc, mn;
+    q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
+    int isum = (int)(sc & 0xFFu) * il + (int)(sc >> 8) * ih;
+    int msum = (int)(mn & 0xFFu) * f.bl + (int)(mn >> 8) * f.bh;
+    float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
+    return f.sx * (d * (float)isum - dmin * (float)msum);
+}

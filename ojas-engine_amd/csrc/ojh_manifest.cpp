@@ -215,6 +215,98 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
     return OJH_OK;
 }
 
+// The MoE family; the number of tokens of the batched entries is read off the grid.
+//   0 moe_topk(lg, idx, wgt, E, KSEL)            1 moe_topk_m(same)              grid [T,1,1] x 64
+//   2 moe_group(idx, counts, offsets, list, NA, E)                                grid [1,1,1] x 256
+//   3 moe_gu_q4k_m(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA)            grid [ceil(N/8), E, 1]
+//   4 moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)                     grid [ceil(N/16), E, 1]
+//   5 moe_combine(dv, wgt, y, T, KSEL, D, ACC)                                    grid [ceil(T*D/256),1,1]
+static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                     const uint32_t block[3], size_t need[8], size_t align[8]) {
+    int rc;
+    for (int i = 0; i < 8; i++) align[i] = 4;
+    switch (s->rows_per_wave) {
+    case 0: case 1: {
+        uint32_t E = c[0], KS = c[1], T = grid[0];
+        if ((rc = check_block(block, 64))) return rc;
+        if (!E || E > 1024 || !KS || KS > E || KS > 64) return ojh_fail(OJH_ERR_ARG, "%s: E=%u KSEL=%u out of range", s->name, E, KS);
+        if (grid[1] != 1 || grid[2] != 1 || (s->rows_per_wave == 0 && T != 1))
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [tokens,1,1]", s->name);
+        need[0] = (size_t)T * E * 4;
+        need[1] = need[2] = (size_t)T * KS * 4;
+        return OJH_OK;
+    }
+    case 2: {
+        uint32_t NA = c[0], E = c[1];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!NA || !E || E > 1024) return ojh_fail(OJH_ERR_ARG, "%s: NA=%u E=%u out of range", s->name, NA, E);
+        if (grid[0] != 1 || grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1,1,1]", s->name);
+        need[0] = need[3] = (size_t)NA * 4;
+        need[1] = (size_t)E * 4;
+        need[2] = (size_t)(E + 1) * 4;
+        return OJH_OK;
+    }
+    case 3: {
+        uint32_t K = c[0], N = c[1], KS = c[2], NA = c[3], E = grid[1];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!K || K % 256 || !N || !KS || !NA || NA % KS) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u KSEL=%u NA=%u", s->name, K, N, KS, NA);
+        if (grid[0] != (N + 7) / 8 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/8), E, 1]", s->name);
+        size_t rb = (size_t)(K / 256) * 144;
+        need[0] = (size_t)(NA / KS) * K;
+        need[1] = (size_t)(NA / KS) * (K / 256) * 4;
+        need[2] = need[3] = (size_t)E * N * rb;
+        need[4] = (size_t)NA * N * 4;
+        need[5] = (size_t)(E + 1) * 4;
+        need[6] = (size_t)NA * 4;
+        align[0] = align[2] = align[3] = 16;
+        return OJH_OK;
+    }
+    case 4: {
+        uint32_t K = c[0], N = c[1], NA = c[2], E = grid[1];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!K || K % 256 || !N || !NA) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u NA=%u", s->name, K, N, NA);
+        if (grid[0] != (N + 15) / 16 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/16), E, 1]", s->name);
+        need[0] = (size_t)NA * K;
+        need[1] = (size_t)NA * (K / 256) * 4;
+        need[2] = (size_t)E * N * (K / 256) * 144;
+        need[3] = (size_t)NA * N * 4;
+        need[4] = (size_t)(E + 1) * 4;
+        need[5] = (size_t)NA * 4;
+        align[0] = align[2] = 16;
+        return OJH_OK;
+    }
+    default: {
+        uint32_t T = c[0], KS = c[1], D = c[2];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!T || !KS || !D) return ojh_fail(OJH_ERR_ARG, "%s: T=%u KSEL=%u D=%u", s->name, T, KS, D);
+        if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * 256 < (uint64_t)T * D)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover %u x %u outputs", s->name, T, D);
+        need[0] = (size_t)T * KS * D * 4;
+        need[1] = (size_t)T * KS * 4;
+        need[2] = (size_t)T * D * 4;
+        return OJH_OK;
+    }
+    }
+}
+
+// K, N as named by the kernel; M = tokens (topk, combine) or assignments (group)
+static int shape_moe(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, uint32_t N, uint32_t M,
+                     uint32_t grid[3], uint32_t block[3]) {
+    (void)K;
+    grid[0] = grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    switch (s->rows_per_wave) {
+    case 0: block[0] = 64; break;
+    case 1: block[0] = 64; grid[0] = M ? M : 1; break;
+    case 2: break;
+    case 3: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = experts
+    case 4: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
+    default: grid[0] = (uint32_t)(((uint64_t)M * N + 255) / 256); break;  // N = D, M = tokens
+    }
+    return OJH_OK;
+}
+
 // copy_*(x, y, n) / fill_zero_u32(y, n): one thread per element
 static int check_elementwise(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                              const uint32_t block[3], size_t need[8], size_t align[8]) {
@@ -337,6 +429,13 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g, "gemm", 3, 4, f.type, 0, check_gemm, shape_gemm);
         add(g + "_sk", "gemm", 3, 4, f.type, 1, check_gemm, shape_gemm);
     }
+    // MoE: `rows_per_wave` selects the kernel inside check_moe / shape_moe
+    add("moe_topk", "moe", 3, 2, 0, 0, check_moe, shape_moe);
+    add("moe_topk_m", "moe", 3, 2, 0, 1, check_moe, shape_moe);
+    add("moe_group", "moe", 4, 2, 0, 2, check_moe, shape_moe);
+    add("moe_gu_q4k_m", "moe", 7, 4, OJH_Q4_K, 3, check_moe, shape_moe);
+    add("moe_down_q4k_m", "moe", 6, 3, OJH_Q4_K, 4, check_moe, shape_moe);
+    add("moe_combine", "moe", 3, 4, 0, 5, check_moe, shape_moe);
     add("copy_bf16_half", "glue", 2, 1, (2u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     // glue: `type` carries (input element bytes << 8 | output element bytes)
     add("copy_f32_half", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);

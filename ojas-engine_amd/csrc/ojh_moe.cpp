@@ -1,12 +1,109 @@
-// MoE op seam: router and grouped expert FFN.
+// MoE op seam: router and grouped expert FFN (the host side of the "moe" kernel family).
+// Stands in for the reference's MoE layer drivers (decode crates/ojas-models/src/decoder/
+// graph_decode.rs:441-499, prefill graph_chunk.rs:564-628; CPU crates/ojas-cpu/src/cpu_glm.rs:519-597):
+// router -> group assignments by expert -> gate/up (+SiLU*mul) -> quantize -> down -> weighted sum.
 #include "ojh_internal.h"
 
-extern "C" int ojh_moe_route(ojh_device *, const ojh_buf *, uint32_t, uint32_t, uint32_t, ojh_buf *, ojh_buf *) {
-    return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_moe_route: not built yet");
+static int ensure(ojh_device *dev, const char *family) {
+    return dev->modules.count(family) ? OJH_OK : ojh_ensure_family(dev, family);
 }
 
-extern "C" int ojh_moe_ffn(ojh_device *, const ojh_buf *, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t,
-                           const ojh_buf *, const ojh_buf *, const ojh_lin *, const ojh_lin *, const ojh_lin *,
-                           ojh_buf *, int, int) {
-    return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_moe_ffn: not built yet");
+static int span(const char *what, const ojh_buf *b, size_t bytes, size_t align) {
+    if (!b) return ojh_fail(OJH_ERR_ARG, "%s: NULL buffer", what);
+    if (bytes > b->bytes) return ojh_fail(OJH_ERR_BOUNDS, "%s needs %zu bytes, buffer has %zu", what, bytes, b->bytes);
+    if ((uintptr_t)b->ptr % align) return ojh_fail(OJH_ERR_ARG, "%s must be %zu-byte aligned", what, align);
+    return OJH_OK;
+}
+
+extern "C" int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uint32_t n_expert,
+                             uint32_t ksel, ojh_buf *idx, ojh_buf *wgt) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_moe_route: NULL device");
+    if (!n_tokens || !n_expert || n_expert > 1024 || !ksel || ksel > n_expert || ksel > 64)
+        return ojh_fail(OJH_ERR_ARG, "moe_route: tokens=%u experts=%u (<= 1024) ksel=%u (<= 64, <= experts)", n_tokens,
+                        n_expert, ksel);
+    int rc;
+    if ((rc = span("moe_route: logits", logits, (size_t)n_tokens * n_expert * 4, 4))) return rc;
+    if ((rc = span("moe_route: idx", idx, (size_t)n_tokens * ksel * 4, 4))) return rc;
+    if ((rc = span("moe_route: wgt", wgt, (size_t)n_tokens * ksel * 4, 4))) return rc;
+    if ((rc = ensure(dev, "moe"))) return rc;
+    uint32_t grid[3] = {n_tokens, 1, 1}, block[3] = {64, 1, 1};
+    return ojh_launch(dev, "moe_topk_m", {logits->ptr, idx->ptr, wgt->ptr}, {n_expert, ksel}, grid, block);
+}
+
+extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32_t d, uint32_t n_ff, uint32_t E,
+                           uint32_t ksel, const ojh_buf *idx, const ojh_buf *wgt, const ojh_lin *gate,
+                           const ojh_lin *up, const ojh_lin *down, ojh_buf *y, int accum, int act_mode) {
+    if (!dev || !gate || !up || !down) return ojh_fail(OJH_ERR_ARG, "ojh_moe_ffn: NULL argument");
+    if (act_mode == OJH_ACT_FLOAT)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_moe_ffn: only the quantized-activation contract (OJH_ACT_Q8K) is built");
+    if (!T || !E || E > 1024 || !ksel || ksel > E || T > 65535u / ksel)
+        return ojh_fail(OJH_ERR_ARG, "moe_ffn: tokens=%u experts=%u ksel=%u out of range", T, E, ksel);
+    if (gate->type != OJH_Q4_K || up->type != OJH_Q4_K || down->type != OJH_Q4_K)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: expert tensors must be Q4_K (gate %u, up %u, down %u)", gate->type,
+                        up->type, down->type);
+    if (d % 256 || n_ff % 256) return ojh_fail(OJH_ERR_ARG, "moe_ffn: d=%u and n_ff=%u must be multiples of 256", d, n_ff);
+    if (gate->k != d || up->k != d || gate->n != (uint64_t)E * n_ff || up->n != gate->n || down->k != n_ff ||
+        down->n != (uint64_t)E * d)
+        return ojh_fail(OJH_ERR_ARG, "moe_ffn: expert tensor shapes do not match E=%u d=%u n_ff=%u", E, d, n_ff);
+    const uint32_t NA = T * ksel;
+    int rc;
+    if ((rc = span("moe_ffn: x", x, (size_t)T * d * 4, 16))) return rc;
+    if ((rc = span("moe_ffn: idx", idx, (size_t)NA * 4, 4))) return rc;
+    if ((rc = span("moe_ffn: wgt", wgt, (size_t)NA * 4, 4))) return rc;
+    if ((rc = span("moe_ffn: y", y, (size_t)T * d * 4, 4))) return rc;
+    if ((rc = ensure(dev, "moe")) || (rc = ensure(dev, "gemv_q8k"))) return rc;
+
+    const uint32_t nsb_d = d / 256, nsb_f = n_ff / 256;
+    ojh_buf *xq, *xs, *act, *aq, *as_, *dv, *grp;
+    if ((rc = ojh_scratch_get(dev, "moe_xq", (size_t)T * d, &xq))) return rc;
+    if ((rc = ojh_scratch_get(dev, "moe_xs", (size_t)T * nsb_d * 4, &xs))) return rc;
+    if ((rc = ojh_scratch_get(dev, "moe_act", (size_t)NA * n_ff * 4, &act))) return rc;
+    if ((rc = ojh_scratch_get(dev, "moe_aq", (size_t)NA * n_ff, &aq))) return rc;
+    if ((rc = ojh_scratch_get(dev, "moe_as", (size_t)NA * nsb_f * 4, &as_))) return rc;
+    if ((rc = ojh_scratch_get(dev, "moe_dv", (size_t)NA * d * 4, &dv))) return rc;
+    // counts[E] | offsets[E+1] | list[NA]
+    if ((rc = ojh_scratch_get(dev, "moe_grp", ((size_t)2 * E + 1 + NA) * 4, &grp))) return rc;
+    uint32_t *counts = (uint32_t *)grp->ptr, *offsets = counts + E, *list = offsets + E + 1;
+
+    uint32_t b256[3] = {256, 1, 1};
+    // 1. quantize the tokens once
+    {
+        uint32_t g[3] = {nsb_d, T, 1};
+        if ((rc = ojh_launch(dev, "quantize_q8k", {x->ptr, xq->ptr, xs->ptr}, {d, T}, g, b256))) return rc;
+    }
+    // 2. group the (token, slot) assignments by expert
+    {
+        uint32_t g[3] = {1, 1, 1};
+        if ((rc = ojh_launch(dev, "moe_group", {idx->ptr, counts, offsets, list}, {NA, E}, g, b256))) return rc;
+    }
+    // 3. gate/up + SiLU*mul, one launch over all experts
+    {
+        uint32_t g[3] = {(n_ff + 7) / 8, E, 1};
+        if ((rc = ojh_launch(dev, "moe_gu_q4k_m",
+                             {xq->ptr, xs->ptr, (char *)gate->raw->ptr + gate->off, (char *)up->raw->ptr + up->off, act->ptr,
+                              offsets, list},
+                             {d, n_ff, ksel, NA}, g, b256)))
+            return rc;
+    }
+    // 4. quantize every assignment's activation (the CPU path quantizes `act` inside matvec_kq)
+    {
+        uint32_t g[3] = {nsb_f, NA, 1};
+        if ((rc = ojh_launch(dev, "quantize_q8k", {act->ptr, aq->ptr, as_->ptr}, {n_ff, NA}, g, b256))) return rc;
+    }
+    // 5. down, one launch over all experts
+    {
+        uint32_t g[3] = {(d + 15) / 16, E, 1};
+        if ((rc = ojh_launch(dev, "moe_down_q4k_m",
+                             {aq->ptr, as_->ptr, (char *)down->raw->ptr + down->off, dv->ptr, offsets, list},
+                             {n_ff, d, NA}, g, b256)))
+            return rc;
+    }
+    // 6. router-weighted sum over slots, in slot order
+    {
+        uint64_t n = (uint64_t)T * d;
+        uint32_t g[3] = {(uint32_t)((n + 255) / 256), 1, 1};
+        if ((rc = ojh_launch(dev, "moe_combine", {dv->ptr, wgt->ptr, y->ptr}, {T, ksel, d, (uint32_t)(accum != 0)}, g, b256)))
+            return rc;
+    }
+    return OJH_OK;
 }

@@ -1,0 +1,124 @@
+"""MoE router and grouped expert FFN on the GPU against the CPU oracle.
+
+Router: indices must match exactly and weights within 1e-5, the reference's own bounds
+(crates/ojas-cuda/tests/conformance.rs:380-408).  Expert FFN: against the composition of the CPU
+path's matvecs (crates/ojas-cpu/src/cpu_glm.rs:551-582 over matvec_kq), peak-normalised error
+<= 1e-3 required.  The activation of every assignment is re-quantized to int8 before the down
+projection, so a last-ulp difference upstream can flip one int8 code; 3e-4 is what that costs at
+most in these cases.
+"""
+import numpy as np
+import pytest
+
+from conftest import peak_err
+
+pytestmark = pytest.mark.gpu
+Q4_K = 12
+TOL = 1e-3
+TOL_SEEN = 3e-4
+
+
+def _route(gpu, logits, ksel):
+    T, E = logits.shape
+    ld = gpu.upload(logits)
+    idx, wgt = gpu.alloc_bytes(T * ksel * 4), gpu.alloc(T * ksel)
+    gpu.moe_route(ld, T, E, ksel, idx, wgt)
+    return gpu.read(idx, T * ksel, np.uint32).reshape(T, ksel), gpu.read(wgt, T * ksel).reshape(T, ksel), idx, wgt
+
+
+def test_router_reference_case(gpu, orc, pkg):
+    """E=64, KSEL=8, logits = tvec(64, 51): the reference's known-answer procedure."""
+    lg = pkg.synth.tvec(64, 51)[None, :]
+    gi, gw, _, _ = _route(gpu, lg, 8)
+    wi, ww = orc.moe_topk(lg, 8)
+    assert np.array_equal(gi, wi)
+    assert np.max(np.abs(gw - ww)) < 1e-5
+    # through the kernel seam, single-token entry
+    gpu.ensure_family("moe")
+    ld, idx, wgt = gpu.upload(lg), gpu.alloc_bytes(32), gpu.alloc(8)
+    grid, block = gpu.launch_shape("moe_topk", 0, 0, 1)
+    gpu.dispatch(gpu.begin(), "moe_topk", [(ld, 0), (idx, 0), (wgt, 0)], [64, 8], grid, block)
+    assert np.array_equal(gpu.read(idx, 8, np.uint32), wi[0])
+
+
+@pytest.mark.parametrize("T,E,ksel", [(1, 128, 8), (16, 128, 8), (256, 128, 8), (5, 1000, 6), (3, 7, 7)])
+def test_router_matches_oracle(gpu, orc, pkg, T, E, ksel):
+    lg = pkg.synth.normal_f32(T * E, "moe", "logits", T, E).reshape(T, E)
+    gi, gw, _, _ = _route(gpu, lg, ksel)
+    wi, ww = orc.moe_topk(lg, ksel)
+    assert np.array_equal(gi, wi)
+    assert np.max(np.abs(gw - ww)) < 1e-5
+    assert np.allclose(gw.sum(1), 1.0, atol=1e-5)
+
+
+def test_router_ties_take_the_lowest_index(gpu):
+    lg = np.zeros((2, 128), np.float32)
+    lg[1, 70] = lg[1, 3] = lg[1, 127] = 1.0
+    gi, _, _, _ = _route(gpu, lg, 4)
+    assert list(gi[0]) == [0, 1, 2, 3]
+    assert list(gi[1]) == [3, 70, 127, 0]
+
+
+def _experts(pkg, E, d, nff, tag):
+    gate = pkg.synth.q4k_weights(E * nff, d, "moe", tag, "gate")
+    up = pkg.synth.q4k_weights(E * nff, d, "moe", tag, "up")
+    down = pkg.synth.q4k_weights(E * d, nff, "moe", tag, "down")
+    return gate, up, down
+
+
+@pytest.mark.parametrize("T,E,ksel,d,nff,accum", [(1, 8, 2, 256, 256, False), (7, 16, 4, 512, 256, True),
+                                                   (33, 8, 8, 1024, 768, False), (4, 4, 1, 2304, 512, False)])
+def test_expert_ffn_matches_cpu_path(gpu, orc, pkg, T, E, ksel, d, nff, accum):
+    gate, up, down = _experts(pkg, E, d, nff, (E, d, nff))
+    x = pkg.synth.normal_f32(T * d, "moe", "x", T, d).reshape(T, d)
+    lg = pkg.synth.normal_f32(T * E, "moe", "lg", T, E).reshape(T, E)
+    gi, gw, idx_d, wgt_d = _route(gpu, lg, ksel)
+    y0 = pkg.synth.normal_f32(T * d, "moe", "y0").reshape(T, d) if accum else np.zeros((T, d), np.float32)
+    yd = gpu.upload(np.concatenate([y0.ravel(), np.full(d, 12345.5, np.float32)]))
+    lg_, lu_, ld_ = gpu.lin(Q4_K, E * nff, d, gate), gpu.lin(Q4_K, E * nff, d, up), gpu.lin(Q4_K, E * d, nff, down)
+    gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, accum=accum, act_mode=pkg.ACT_Q8K)
+    got = gpu.read(yd, T * d + d)
+    assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
+    want = orc.moe_ffn(x, gi, gw, gate, up, Q4_K, down, Q4_K, E, nff, mode=0, y0=y0)
+    err = peak_err(got[:T * d].reshape(T, d) - y0, want - y0)
+    assert err <= TOL_SEEN <= TOL, err
+
+
+def test_expert_ffn_at_the_benchmark_shape(gpu, orc, pkg):
+    """128 experts, top-8, hidden 2048, expert FFN 768: T = 1 and 16 against the CPU path in full,
+    T = 256 against the CPU path on sampled tokens and against the T = 1 launches of the same
+    tokens (a token's result cannot depend on who else is in the batch)."""
+    E, ksel, d, nff = 128, 8, 2048, 768
+    gate, up, down = _experts(pkg, E, d, nff, "bench")
+    lg_, lu_, ld_ = gpu.lin(Q4_K, E * nff, d, gate), gpu.lin(Q4_K, E * nff, d, up), gpu.lin(Q4_K, E * d, nff, down)
+    for T in (1, 16, 256):
+        x = pkg.synth.normal_f32(T * d, "moe", "bx", T).reshape(T, d)
+        lg = pkg.synth.normal_f32(T * E, "moe", "blg", T).reshape(T, E)
+        gi, gw, idx_d, wgt_d = _route(gpu, lg, ksel)
+        yd = gpu.alloc(T * d)
+        gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd)
+        got = gpu.read(yd, T * d).reshape(T, d)
+        sample = range(T) if T <= 16 else [0, 17, 100, 255]
+        for t in sample:
+            want = orc.moe_ffn(x[t:t + 1], gi[t:t + 1], gw[t:t + 1], gate, up, Q4_K, down, Q4_K, E, nff, mode=0)
+            assert peak_err(got[t], want[0]) <= TOL_SEEN, (T, t)
+        if T == 256:
+            for t in (3, 200):
+                y1 = gpu.alloc(d)
+                i1, w1 = gpu.upload_bytes(gi[t]), gpu.upload(gw[t])
+                gpu.moe_ffn(gpu.upload(x[t]), 1, d, nff, E, ksel, i1, w1, lg_, lu_, ld_, y1)
+                assert np.array_equal(gpu.read(y1, d), got[t])
+
+
+def test_expert_ffn_rejects_what_it_cannot_run(gpu, pkg):
+    E, d, nff = 4, 256, 256
+    gate, up, down = _experts(pkg, E, d, nff, "err")
+    lg_, lu_, ld_ = gpu.lin(Q4_K, E * nff, d, gate), gpu.lin(Q4_K, E * nff, d, up), gpu.lin(Q4_K, E * d, nff, down)
+    x, y = gpu.alloc(d), gpu.alloc(d)
+    idx, wgt = gpu.upload_bytes(np.array([1, 2], np.uint32)), gpu.upload(np.array([0.5, 0.5], np.float32))
+    with pytest.raises(pkg.OjasHipError, match="shapes do not match"):
+        gpu.moe_ffn(x, 1, d, nff, E + 1, 2, idx, wgt, lg_, lu_, ld_, y)
+    with pytest.raises(pkg.OjasHipError, match="quantized-activation"):
+        gpu.moe_ffn(x, 1, d, nff, E, 2, idx, wgt, lg_, lu_, ld_, y, act_mode=pkg.ACT_FLOAT)
+    with pytest.raises(pkg.OjasHipError, match="needs"):
+        gpu.moe_ffn(x, 2, d, nff, E, 2, idx, wgt, lg_, lu_, ld_, y)
