@@ -176,9 +176,86 @@ def main() -> int:
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(host, dims)
+    if not args.no_extra:
+        # free the decode sets first: the secondary shapes bring their own tensors
+        graphs.clear()
+        lin_q = sets[0]["gate"], sets[0]["down"]
+        result["extra"] = extras(gpu, pkg, lin_q)
     print(json.dumps(result))
     gpu.close()
     return 0
+
+
+def _time(gpu, fn, reps: int, warm: int = 3) -> float:
+    """Average microseconds per call of `fn(i)` over `reps` calls, events on the launching stream."""
+    for i in range(warm):
+        fn(i)
+    gpu.timer_start()
+    for i in range(reps):
+        fn(i)
+    return gpu.timer_stop() / reps * 1e3
+
+
+def extras(gpu, pkg, lin_q) -> dict:
+    """Secondary configurations: prefill GEMM, Q8_0 matvec, MoE grouped FFN, Q6_K head verify."""
+    synth = pkg.synth
+    out = {}
+    # ---- prefill dequant-GEMM, Q4_K gate/up (14336x4096) and down (4096x14336), f16 MFMA tile
+    gemm = {}
+    for name, lin in zip(("gate_up_14336x4096", "down_4096x14336"), lin_q):
+        n, k = lin.n, lin.k
+        for m in (128, 512, 2048):
+            xb = gpu.upload_bytes(synth.to_bf16_bits(synth.normal_f32(m * k, "bench", "gemm_x", m, k)))
+            y = gpu.alloc(m * n)
+            us = _time(gpu, lambda i: gpu.mm(xb, lin, y, m, x_dtype=pkg.X_BF16, act_mode=pkg.ACT_FLOAT), 20, 5)
+            tf = 2.0 * m * n * k / us / 1e6
+            gemm[f"{name}_M{m}"] = {"us": round(us, 1), "tflops": round(tf, 1), "mfma_frac": round(tf / 2500.0, 4)}
+    out["prefill_gemm_q4k"] = {"activations": "bf16 N(0,1), converted to f16 into the tile", "accumulate": "f32",
+                               "tile": "v_mfma_f32_32x32x16_f16, weights = dequant_to_f16 bits",
+                               "peak_tflops": 2500.0, "timed": "conversion + zero fill (split-K) + tile", **gemm}
+    # ---- config 0: Q8_0 matvec 4096x4096, f32 activations (dot_q80 contract)
+    n = k = 4096
+    wq8 = [gpu.lin(pkg.Q8_0, n, k, synth.q80_weights(n, k, "bench", "q80")) for _ in range(16)]
+    x, y = gpu.upload(synth.normal_f32(k, "bench", "q80x")), gpu.alloc(n)
+    us = _time(gpu, lambda i: gpu.mm(x, wq8[i % 16], y), 64, 16)
+    b = n * (k // 32) * 34 + 4 * k + 4 * n
+    out["q80_gemv_4096x4096"] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
+    del wq8
+    # ---- MoE: 128 experts, top-8, hidden 2048, expert FFN 768, Q4_K; tokens 1 / 16 / 256
+    E, ksel, d, nff = 128, 8, 2048, 768
+    gate = gpu.lin(pkg.Q4_K, E * nff, d, synth.q4k_weights(E * nff, d, "bench", "moe_gate"))
+    up = gpu.lin(pkg.Q4_K, E * nff, d, synth.q4k_weights(E * nff, d, "bench", "moe_up"))
+    down = gpu.lin(pkg.Q4_K, E * d, nff, synth.q4k_weights(E * d, nff, "bench", "moe_down"))
+    moe = {}
+    for T in (1, 16, 256):
+        lg = gpu.upload(synth.normal_f32(T * E, "bench", "moe_lg", T))
+        xt, yt = gpu.upload(synth.normal_f32(T * d, "bench", "moe_x", T)), gpu.alloc(T * d)
+        idx, wgt = gpu.alloc_bytes(T * ksel * 4), gpu.alloc(T * ksel)
+
+        def layer(i):
+            gpu.moe_route(lg, T, E, ksel, idx, wgt)
+            gpu.moe_ffn(xt, T, d, nff, E, ksel, idx, wgt, gate, up, down, yt)
+        us = _time(gpu, layer, 20, 3)
+        distinct = len(np.unique(gpu.read(idx, T * ksel, np.uint32)))
+        b = distinct * 3 * nff * (d // 256) * 144 + T * d * 8
+        fl = 2.0 * T * ksel * 3 * nff * d
+        moe[f"T{T}"] = {"us": round(us, 1), "distinct_experts": distinct, "gbs": round(b / us / 1e3, 1),
+                        "tflops": round(fl / us / 1e6, 2)}
+    out["moe_ffn_q4k_128x_top8"] = {"timed": "router + quantize + group + gate/up + quantize + down + combine", **moe}
+    del gate, up, down
+    # ---- speculative verify on a Q6_K output head 151936 x 4096, bf16 activations
+    n, k = 151936, 4096
+    head = gpu.lin(pkg.Q6_K, n, k, synth.q6k_weights(n, k, "bench", "q6k_head"))
+    ver = {}
+    for m in (1, 2, 4, 8, 16):
+        xb = gpu.upload_bytes(synth.to_bf16_bits(synth.normal_f32(m * k, "bench", "ver_x", m)))
+        y = gpu.alloc(m * n)
+        us = _time(gpu, lambda i: gpu.mm(xb, head, y, m, x_dtype=pkg.X_BF16), 10, 2)
+        b = n * (k // 256) * 210 + m * (2 * k + 4 * n)
+        ver[f"M{m}"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4),
+                        "tflops": round(2.0 * m * n * k / us / 1e6, 2)}
+    out["verify_q6k_head_151936x4096"] = {"activations": "bf16, quantized per 256 (quant_q8k)", **ver}
+    return out
 
 
 def cpu_baseline(host, dims) -> dict:

@@ -205,7 +205,7 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
     if (s->rows_per_wave == 1) {  // split K until every CU has a tile, at least 4 K-steps per slice
         uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
         uint32_t tiles = grid[0] * grid[1], steps = K / 64;
-        uint32_t z = tiles ? (cus + tiles - 1) / tiles : 1;
+        uint32_t z = tiles ? cus / tiles : 1;  // floor: 224 tiles on 256 CUs are better left whole
         if (z > steps / 4) z = steps / 4;
         if (z > 16) z = 16;
         grid[2] = z ? z : 1;
