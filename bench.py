@@ -4,9 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 One step = one decode token's worth of Q4_K projections of a Llama-3-8B-shaped model through the
-C ABI: the activation vector of each stage is quantized once (quant_q8k) and feeds the matvecs that
-read it — q/k/v, o, gate/up, down, output head — 5 quantizations and 8 matvecs, all reading
-weights from HBM (the step's 418 MB exceed the 256 MB last-level cache and the weight sets rotate).
+C ABI — q, k, v, o, gate, up, down, output head: 8 matvecs in the CPU reference's arithmetic, the
+activation vector of each of the 5 stages quantized once per 256 (quant_q8k) and shared by the
+projections that read it, all reading weights from HBM (the step's 418 MB exceed the 256 MB last-level cache and the weight sets rotate).
 Prints ONE JSON line: whole-step GB/s of algorithmic bytes, the roofline of the dominant kernel
 (timed per launch with events on the launching stream), the CPU oracle timed on the host cores,
 and secondary figures (prefill GEMM, MoE, verify) under "extra".
@@ -48,6 +48,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--copies", type=int, default=2, help="rotating weight sets")
     ap.add_argument("--eager", action="store_true", help="issue every launch from the host instead of replaying a recorded step")
+    ap.add_argument("--fused-quant", action="store_true",
+                    help="quantize x inside every matvec launch (8 launches per step) instead of once per "
+                         "stage in a launch of its own (5 + 8 launches); measured slower")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
     args = ap.parse_args()
@@ -75,14 +78,23 @@ def main() -> int:
     step_bytes = sum(algorithmic_bytes(n, k) for _, n, k in SHAPES)
     dom = "head"  # the launch that dominates the step: 295.5 MB of its 418 MB
 
+    def one(st: str, lin, y) -> None:
+        """One projection from the f32 stage input: by default a single launch that quantizes x
+        in-kernel; with --split-quant, from the stage's separately quantized copy."""
+        if (not args.fused_quant):
+            gpu.mm_q8k(xq[st], xsc[st], lin, y)
+        else:
+            gpu.mm(xs[st], lin, y, 1, act_mode=pkg.ACT_Q8K)
+
     def step(i: int) -> None:
         w = sets[i % args.copies]
         for st, k, names in STAGES:
-            gpu.quant_q8k(xs[st], 1, k, xq[st], xsc[st])
+            if (not args.fused_quant):
+                gpu.quant_q8k(xs[st], 1, k, xq[st], xsc[st])
             for name in names:
-                gpu.mm_q8k(xq[st], xsc[st], w[name], ys[name])
+                one(st, w[name], ys[name])
 
-    # The 13 launches of a step are recorded once per weight set and replayed with one host call,
+    # The launches of a step are recorded once per weight set and replayed with one host call,
     # so the host's per-call cost (here: Python) stays out of the device timeline.
     for i in range(args.copies):
         step(i)
@@ -120,11 +132,13 @@ def main() -> int:
     dn, dk = dims[dom]
     dom_bytes = algorithmic_bytes(dn, dk)
     dom_reps = max(args.steps, 20)
+    for st, k, _ in STAGES:  # the split form reads these
+        gpu.quant_q8k(xs[st], 1, k, xq[st], xsc[st])
     for i in range(3):
-        gpu.mm_q8k(xq["x_head"], xsc["x_head"], sets[i % args.copies][dom], ys[dom])
+        one("x_head", sets[i % args.copies][dom], ys[dom])
     gpu.timer_start()
     for i in range(dom_reps):
-        gpu.mm_q8k(xq["x_head"], xsc["x_head"], sets[i % args.copies][dom], ys[dom])
+        one("x_head", sets[i % args.copies][dom], ys[dom])
     dom_avg_ms = gpu.timer_stop() / dom_reps
     achieved = dom_bytes / (dom_avg_ms * 1e-3) / 1e9
 
@@ -134,10 +148,10 @@ def main() -> int:
     for name, n, k in SHAPES:
         st = next(s for s, _, names in STAGES if name in names)
         for i in range(3):
-            gpu.mm_q8k(xq[st], xsc[st], sets[i % args.copies][name], ys[name])
+            one(st, sets[i % args.copies][name], ys[name])
         gpu.timer_start()
         for i in range(reps):
-            gpu.mm_q8k(xq[st], xsc[st], sets[i % args.copies][name], ys[name])
+            one(st, sets[i % args.copies][name], ys[name])
         us = gpu.timer_stop() / reps * 1e3
         b = algorithmic_bytes(n, k)
         per_shape[name] = {"n": n, "k": k, "us": round(us, 2), "gbs": round(b / us / 1e3, 1),
@@ -160,12 +174,13 @@ def main() -> int:
                                "(q,k,v,o 4096; gate,up 14336x4096; down 4096x14336; head 128256x4096), "
                                "f32 activations N(0,1) quantized once per stage, weights in HBM",
                    "bytes_per_step": step_bytes, "weight_sets": args.copies,
-                   "launches_per_step": "5 quantize_q8k + 8 gemv_q8k_q4k*",
+                   "launches_per_step": "5 quantize_q8k + 8 gemv_q8k_q4k*" if (not args.fused_quant) else
+                                        "8 gemv_fq8k_q4k* (activation quantizer folded into each launch)",
                    "submission": "eager, one host call per launch" if args.eager else
                                  "recorded step replayed from the library (%s)" % os.environ.get("OJAS_HIP_REPLAY", "list")},
         "hbm_frac": round(value / HBM_PEAK_GBS, 4),
         "host_ms_per_step": round(host_ms / args.steps, 5),
-        "roofline": {"bound": "hbm", "kernel": "gemv_q8k_q4k_wide", "launch": f"head {dn}x{dk}",
+        "roofline": {"bound": "hbm", "kernel": "gemv_q8k_q4k_wide" if (not args.fused_quant) else "gemv_fq8k_q4k_wide", "launch": f"head {dn}x{dk}",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_avg_ms * 1e3, 2)},

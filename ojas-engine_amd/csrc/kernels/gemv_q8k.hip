@@ -120,6 +120,101 @@ __device__ __forceinline__ void gemv_q8k_q4k_body(const signed char* __restrict_
 
 GEMV_Q8K_ENTRIES(q4k, gemv_q8k_q4k_body)
 
+// ---- the same matvec with the activation quantizer folded in ---------------------------------
+//   gemv_fq8k_q4k_{r1,r2,wide}(x, w, y, K, N, NRB)      x: f32[K], K <= 16384
+// A decode step is a chain of few-microsecond launches, each costing a dispatch and a DRAM round
+// trip; quantizing in a launch of its own doubles that chain.  Here every workgroup quantizes x
+// itself into LDS — the same arithmetic as quantize_q8k, so results are bit-identical to the
+// two-launch form — after its first weight loads are already in flight, so the quantization
+// hides under their latency; it then walks NRB rows (a multiple of 4R, chosen by the host so
+// that the repeated quantization stays a small share of the work).  LDS segments are 288 bytes
+// apart: the 16-byte fragment reads of 16 consecutive lanes then fall in distinct banks.
+#define FQ_SEG 288u
+#define FQ_MAX_K 16384u
+
+template <int R>
+__device__ __forceinline__ void gemv_fq8k_q4k_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                   float* __restrict__ y, uint K, uint N, uint NRB) {
+    __shared__ __attribute__((aligned(16))) signed char sx[(FQ_MAX_K / 256u) * FQ_SEG];
+    __shared__ float ss[FQ_MAX_K / 256u];
+    const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    const uint row_end = min((blockIdx.x + 1u) * NRB, N);
+    uint row0 = blockIdx.x * NRB + wave * R;
+    // first step's weights: issued before anything else
+    uint4 hdr[R], qs[R];
+    {
+        const uint sb = min(g, nsb - 1u);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            uint row = min(row0 + r, N - 1u);
+            const uchar* blk = w + ((size_t)row * nsb + sb) * Q4K_BYTES;
+            hdr[r] = *(const uint4*)blk;
+            qs[r] = *(const uint4*)(blk + 16u + l * 16u);
+        }
+    }
+    // quantize x: wave `wave` owns segments wave, wave+4, ...; a lane holds 4 consecutive values
+    for (uint seg = wave; seg < nsb; seg += 4u) {
+        float4 v = *(const float4*)(x + (size_t)seg * 256u + lane * 4u);
+        float a = wave_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        float scale = a > 0.0f ? __fdiv_rn(a, 127.0f) : 1.0f;
+        float inv = __fdiv_rn(1.0f, scale);
+        int q0 = (int)fminf(fmaxf(roundf(__fmul_rn(v.x, inv)), -127.0f), 127.0f);
+        int q1 = (int)fminf(fmaxf(roundf(__fmul_rn(v.y, inv)), -127.0f), 127.0f);
+        int q2 = (int)fminf(fmaxf(roundf(__fmul_rn(v.z, inv)), -127.0f), 127.0f);
+        int q3 = (int)fminf(fmaxf(roundf(__fmul_rn(v.w, inv)), -127.0f), 127.0f);
+        *(uint*)(sx + seg * FQ_SEG + lane * 4u) =
+            (uint)(q0 & 0xFF) | ((uint)(q1 & 0xFF) << 8) | ((uint)(q2 & 0xFF) << 16) | ((uint)(q3 & 0xFF) << 24);
+        if (lane == 0) ss[seg] = scale;
+    }
+    __syncthreads();
+    bool first = true;
+    for (; row0 < row_end; row0 += 4u * R) {
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = 0.0f;
+        for (uint sb = g; sb < nsb; sb += 8u) {
+            if (!(first && sb == g)) {
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    uint row = min(row0 + r, N - 1u);
+                    const uchar* blk = w + ((size_t)row * nsb + sb) * Q4K_BYTES;
+                    hdr[r] = *(const uint4*)blk;
+                    qs[r] = *(const uint4*)(blk + 16u + l * 16u);
+                }
+            }
+            Q4kFrag f;
+            const signed char* p = sx + sb * FQ_SEG + c * 64u + (l & 1u) * 16u;
+            f.xl = *(const uint4*)p;
+            f.xh = *(const uint4*)(p + 32);
+            f.bl = bytesum4(f.xl);
+            f.bh = bytesum4(f.xh);
+            f.sx = ss[sb];
+#pragma unroll
+            for (int r = 0; r < R; r++) acc[r] += q4k_lane_dot(hdr[r], qs[r], c, f);
+        }
+        first = false;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float t = wave_sum(acc[r]);
+            if (lane == 0 && row0 + r < row_end) y[row0 + r] = t;
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+gemv_fq8k_q4k_r1(const float* x, const uchar* w, float* y, uint K, uint N, uint NRB) {
+    gemv_fq8k_q4k_body<1>(x, w, y, K, N, NRB);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemv_fq8k_q4k_r2(const float* x, const uchar* w, float* y, uint K, uint N, uint NRB) {
+    gemv_fq8k_q4k_body<2>(x, w, y, K, N, NRB);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemv_fq8k_q4k_wide(const float* x, const uchar* w, float* y, uint K, uint N, uint NRB) {
+    gemv_fq8k_q4k_body<2>(x, w, y, K, N, NRB);
+}
+
 // Batched form: y[M][N] (+)= quantized x[M][K] . W^T.  One wave per row; the row's weights are
 // read and unpacked once per tile of MT tokens.
 template <int MT>

@@ -96,6 +96,27 @@ static int check_gemv_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uin
     return OJH_OK;
 }
 
+// gemv_fq8k_<fmt>_{r1,r2,wide}(x, w, y, K, N, NRB): quantizer folded in; 4 waves per block,
+// K <= 16384, NRB rows per block (a multiple of 4 * rows per wave)
+static int check_gemv_fq8k(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                           const uint32_t block[3], size_t need[8], size_t align[8]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], N = c[1], NRB = c[2];
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if ((rc = check_block(block, 256))) return rc;
+    if (K > 16384) return ojh_fail(OJH_ERR_ARG, "%s: K=%u exceeds 16384", s->name, K);
+    uint32_t unit = 4u * (uint32_t)s->rows_per_wave;
+    if (!NRB || NRB % unit) return ojh_fail(OJH_ERR_ARG, "%s: NRB=%u must be a positive multiple of %u", s->name, NRB, unit);
+    if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * NRB < N)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid x NRB does not cover N=%u rows", s->name, N);
+    need[0] = (size_t)K * 4;
+    need[1] = (size_t)N * (K / f->weights) * f->bytes;
+    need[2] = (size_t)N * 4;
+    align[2] = 4;
+    return OJH_OK;
+}
+
 // gemv_nat_<fmt>_m(x, w, y, K, N, M, ACC)
 static int check_gemv_nat_m(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                             const uint32_t block[3], size_t need[8], size_t align[8]) {
@@ -419,6 +440,12 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(q + "_accum", "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
         add(q + "_bias", "gemv_q8k", 5, 2, f.type, 4, check_gemv_q8k, shape_rows);
         add(q + "_m", "gemv_q8k", 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
+        if (f.type == OJH_Q4_K) {
+            std::string fq = "gemv_fq8k_" + t;
+            add(fq + "_r1", "gemv_q8k", 3, 3, f.type, 1, check_gemv_fq8k, shape_rows);
+            add(fq + "_r2", "gemv_q8k", 3, 3, f.type, 2, check_gemv_fq8k, shape_rows);
+            add(fq + "_wide", "gemv_q8k", 3, 3, f.type, 2, check_gemv_fq8k, shape_rows);
+        }
     }
     add("quantize_q8k", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);

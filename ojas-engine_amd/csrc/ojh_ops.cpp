@@ -223,6 +223,24 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     }
 
     bool q8k = w->type != OJH_Q8_0 && act_mode != OJH_ACT_FLOAT;
+    // Opt-in: one token, f32 in, plain store through the launch that quantizes x itself
+    // (bit-identical results).  Measured slower than quantize + matvec at every decode shape on
+    // MI355X — each block repeats the quantization and reads x through LDS — so it is off by default.
+    if (q8k && m == 1 && !accum && !bias && x_dtype == OJH_X_F32 && w->type == OJH_Q4_K && K <= 16384 &&
+        dev->fused_quant) {
+        if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+        int r = pick_rows(dev, N);
+        if (r > 2) r = 2;
+        const char *name = (r == 2 && N >= 32768u) ? "gemv_fq8k_q4k_wide" : r == 2 ? "gemv_fq8k_q4k_r2" : "gemv_fq8k_q4k_r1";
+        // rows per block: every block re-quantizes x, so give it enough rows that this stays a
+        // small share, but keep several blocks per CU
+        uint32_t unit = 4u * (uint32_t)r, cus = (uint32_t)dev->prop.multiProcessorCount;
+        uint32_t nrb = (N + cus * dev->fq_blocks_per_cu - 1) / (cus * dev->fq_blocks_per_cu);
+        nrb = ((nrb + unit - 1) / unit) * unit;
+        if (nrb < unit) nrb = unit;
+        grid[0] = (N + nrb - 1) / nrb;
+        return ojh_launch(dev, name, {at(x, x_off), wp, yp}, {K, N, nrb}, grid, block);
+    }
     if (q8k) {
         if ((rc = ensure(dev, "gemv_q8k"))) return rc;
         size_t nsb = K / 256;

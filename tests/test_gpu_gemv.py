@@ -206,3 +206,23 @@ def test_errors_are_reported_not_launched(gpu, pkg):
     with pytest.raises(pkg.OjasHipError, match="unknown kernel family"):
         gpu.ensure_family("attn")
     gpu.submit(enc)
+
+
+@pytest.mark.parametrize("n,k", [(1024, 4096), (4099, 4096), (96, 14336), (13, 256), (40000, 512)])
+def test_fused_quantizer_is_bit_identical_to_the_two_launch_form(gpu, orc, pkg, n, k):
+    """gemv_fq8k_q4k_* (one launch, x quantized in-kernel) == ojh_quant_q8k + ojh_mm_q8k, bit for bit."""
+    w, x = _inputs(pkg, Q4_K, n, k, "fq")
+    x[:5] = [0.5, -2.5, 0.0, 1e-30, 3.0]
+    lin = gpu.lin(Q4_K, n, k, w)
+    wd = gpu.upload_bytes(w)
+    xd, y1, y2 = gpu.upload(x), gpu.alloc(n), gpu.alloc(n)
+    xq, xs = gpu.alloc_bytes(k), gpu.alloc(k // 256)
+    gpu.ensure_family("gemv_q8k")
+    nrb = 24 if n > 100 else 8
+    gpu.dispatch(gpu.begin(), "gemv_fq8k_q4k_r2", [(xd, 0), (wd, 0), (y1, 0)], [k, n, nrb], [(n + nrb - 1) // nrb, 1, 1],
+                 [256, 1, 1])
+    gpu.quant_q8k(xd, 1, k, xq, xs)
+    gpu.mm_q8k(xq, xs, lin, y2)
+    a, b = gpu.read(y1, n), gpu.read(y2, n)
+    assert np.array_equal(a, b)
+    assert peak_err(a, orc.matvec_kq(w, Q4_K, n, k, x)) <= TOL_Q8K_SEEN
