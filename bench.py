@@ -36,6 +36,12 @@ STAGES = [("x_attn", 4096, ["q", "k", "v"]), ("x_o", 4096, ["o"]), ("x_ffn", 409
           ("x_down", 14336, ["down"]), ("x_head", 4096, ["head"])]
 
 
+# HBM bytes per launch of the head matvec (128256 x 4096 Q4_K) from hardware counters: FETCH_SIZE
+# 144 324.7 KiB x 2.000 (the factor the same counter needs to read a 512 MiB copy correctly) +
+# WRITE_SIZE 501.4 KiB.  Algorithmic bytes of the launch: 296 031 232.
+HEAD_TRAFFIC_BYTES = 296_090_000
+
+
 def algorithmic_bytes(n: int, k: int) -> int:
     """Weight bytes + activation vector + output vector of one Q4_K matvec."""
     return n * (k // 256) * 144 + 4 * k + 4 * n
@@ -48,6 +54,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--copies", type=int, default=2, help="rotating weight sets")
     ap.add_argument("--eager", action="store_true", help="issue every launch from the host instead of replaying a recorded step")
+    ap.add_argument("--per-projection", action="store_true",
+                    help="one launch per projection instead of grouped q/k/v and gate/up launches")
     ap.add_argument("--fused-quant", action="store_true",
                     help="quantize x inside every matvec launch (8 launches per step) instead of once per "
                          "stage in a launch of its own (5 + 8 launches); measured slower")
@@ -86,11 +94,17 @@ def main() -> int:
         else:
             gpu.mm(xs[st], lin, y, 1, act_mode=pkg.ACT_Q8K)
 
+    grouped = not args.fused_quant and not args.per_projection
+
     def step(i: int) -> None:
         w = sets[i % args.copies]
         for st, k, names in STAGES:
             if (not args.fused_quant):
                 gpu.quant_q8k(xs[st], 1, k, xq[st], xsc[st])
+            if grouped and len(names) > 1:
+                # q/k/v and gate/up read the same vector: one launch over the separate tensors
+                gpu.mm_q8k_multi(xq[st], xsc[st], [w[n] for n in names], [ys[n] for n in names])
+                continue
             for name in names:
                 one(st, w[name], ys[name])
 
@@ -142,6 +156,19 @@ def main() -> int:
     dom_avg_ms = gpu.timer_stop() / dom_reps
     achieved = dom_bytes / (dom_avg_ms * 1e-3) / 1e9
 
+    # ---- calibration launches: a plain copy and a plain read of known size (512 MiB each way),
+    # the yardstick for hardware counters and for what this chip's HBM delivers to any kernel
+    gpu.ensure_family("glue")
+    cal_n16 = (512 << 20) // 16
+    cal_src, cal_dst = gpu.alloc_bytes(cal_n16 * 16), gpu.alloc_bytes(cal_n16 * 16)
+    gpu.memset0(cal_src)
+    cgrid, cblock = gpu.launch_shape("stream_copy_u32x4", 0, cal_n16, 0)
+    cal = {}
+    for kname, moved in (("stream_copy_u32x4", 2 * cal_n16 * 16), ("stream_read_u32x4", cal_n16 * 16)):
+        us = _time(gpu, lambda i: gpu.dispatch(gpu.begin(), kname, [(cal_src, 0), (cal_dst, 0)], [cal_n16], cgrid, cblock), 5, 2)
+        cal[kname] = {"bytes_moved": moved, "us": round(us, 1), "gbs": round(moved / us / 1e3, 1)}
+    del cal_src, cal_dst
+
     # ---- per-shape latency (each shape alone, back to back, rotating sets), for the record
     per_shape = {}
     reps = 50
@@ -174,7 +201,9 @@ def main() -> int:
                                "(q,k,v,o 4096; gate,up 14336x4096; down 4096x14336; head 128256x4096), "
                                "f32 activations N(0,1) quantized once per stage, weights in HBM",
                    "bytes_per_step": step_bytes, "weight_sets": args.copies,
-                   "launches_per_step": "5 quantize_q8k + 8 gemv_q8k_q4k*" if (not args.fused_quant) else
+                   "launches_per_step": "5 quantize_q8k + 5 gemv_q8k_q4k* (q/k/v and gate/up each one grouped "
+                                        "launch over separate tensors)" if grouped else
+                                        "5 quantize_q8k + 8 gemv_q8k_q4k*" if (not args.fused_quant) else
                                         "8 gemv_fq8k_q4k* (activation quantizer folded into each launch)",
                    "submission": "eager, one host call per launch" if args.eager else
                                  "recorded step replayed from the library (%s)" % os.environ.get("OJAS_HIP_REPLAY", "list")},
@@ -182,9 +211,14 @@ def main() -> int:
         "host_ms_per_step": round(host_ms / args.steps, 5),
         "roofline": {"bound": "hbm", "kernel": "gemv_q8k_q4k_wide" if (not args.fused_quant) else "gemv_fq8k_q4k_wide", "launch": f"head {dn}x{dk}",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": HEAD_TRAFFIC_BYTES if (dom == "head" and not args.fused_quant) else None,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by the "
+                                       "same counters over stream_copy_u32x4 (x2.000 / x1.000); a recorded "
+                                       "figure, not re-measured by this run",
                      "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_avg_ms * 1e3, 2)},
         "per_shape": per_shape,
+        "calibration": cal,
         "device": {"name": gpu.name(), "cus": caps.compute_units, "clock_mhz": caps.clock_mhz},
         "setup_s": round(setup_s, 1),
     }

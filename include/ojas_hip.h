@@ -178,6 +178,15 @@ int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, const o
 int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const ojh_lin *w, ojh_buf *y,
                size_t y_off, const ojh_buf *bias, uint32_t m, int accum);
 
+/* One to four projections of the same quantized vector in ONE launch: ys[i] = xq . ws[i]^T, each
+ * Lin its own allocation, all with the same K.  The reference's fused q/k/v and gate/up launches
+ * (`qkv_q80_dp4a`, `ffn_gu_q80_dp4a`: crates/ojas-core/src/kernels/gemv_q8.rs:229-260) take one
+ * pointer per projection in the same way.  Results are bit-identical to `count` calls of
+ * `ojh_mm_q8k`; formats without a grouped kernel (Q5_K, Q6_K) run as that many launches.
+ * `y_offs` (bytes) may be NULL. */
+int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, int count,
+                     const ojh_lin *const *ws, ojh_buf *const *ys, const size_t *y_offs);
+
 /* `dequant_to_f16` (crates/ojas-formats/src/gguf.rs:612-1116) on the device: `n_weights`
  * weights of `raw` -> binary16 bit patterns in `out`. Bit-exact with the reference. */
 int ojh_dequant_f16(ojh_device *dev, uint32_t ggml_type, const ojh_buf *raw, size_t raw_off,

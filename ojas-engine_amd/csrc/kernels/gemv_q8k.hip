@@ -120,6 +120,76 @@ __device__ __forceinline__ void gemv_q8k_q4k_body(const signed char* __restrict_
 
 GEMV_Q8K_ENTRIES(q4k, gemv_q8k_q4k_body)
 
+// ---- several projections of one activation in one launch -------------------------------------
+//   gemv_q8k_q4k_x4_{r1,r2}(xq, xs, w0, w1, w2, w3, y0, y1, y2, y3, K, E0, E1, E2, E3)
+// Up to four weight tensors (separate allocations, all K wide) share the quantized activation:
+// global row r belongs to tensor i when E(i-1) <= r < E(i), E being the running row totals.
+// The counterpart of the reference's fused q/k/v and gate/up launches
+// (crates/ojas-core/src/kernels/gemv_q8.rs:229-260), which likewise take one pointer per
+// projection.  Each row runs exactly the single-tensor arithmetic, so results are bit-identical
+// to separate launches; what is saved is a dispatch and a DRAM round trip per projection.
+struct X4Row {
+    const uchar* w;
+    float* y;
+};
+
+template <int R>
+__device__ __forceinline__ void gemv_q8k_q4k_x4_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                     const uchar* w0, const uchar* w1, const uchar* w2,
+                                                     const uchar* w3, float* y0, float* y1, float* y2, float* y3,
+                                                     uint K, uint E0, uint E1, uint E2, uint E3) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 >= E3) return;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    X4Row rw[R];
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const uint gr = min(row0 + r, E3 - 1u);
+        const uchar* w;
+        float* y;
+        uint lr;
+        if (gr < E0) { w = w0; y = y0; lr = gr; }
+        else if (gr < E1) { w = w1; y = y1; lr = gr - E0; }
+        else if (gr < E2) { w = w2; y = y2; lr = gr - E1; }
+        else { w = w3; y = y3; lr = gr - E2; }
+        rw[r].w = w + (size_t)lr * nsb * Q4K_BYTES;
+        rw[r].y = y + lr;
+        acc[r] = 0.0f;
+    }
+    for (uint sb = g; sb < nsb; sb += 8u) {
+        uint4 hdr[R], qs[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uchar* blk = rw[r].w + (size_t)sb * Q4K_BYTES;
+            hdr[r] = *(const uint4*)blk;
+            qs[r] = *(const uint4*)(blk + 16u + l * 16u);
+        }
+        Q4kFrag f = q4k_load_frag(xq, xs, sb, l);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += q4k_lane_dot(hdr[r], qs[r], c, f);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float t = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < E3) *rw[r].y = t;
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+gemv_q8k_q4k_x4_r1(const signed char* xq, const float* xs, const uchar* w0, const uchar* w1, const uchar* w2,
+                   const uchar* w3, float* y0, float* y1, float* y2, float* y3, uint K, uint E0, uint E1, uint E2,
+                   uint E3) {
+    gemv_q8k_q4k_x4_body<1>(xq, xs, w0, w1, w2, w3, y0, y1, y2, y3, K, E0, E1, E2, E3);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemv_q8k_q4k_x4_r2(const signed char* xq, const float* xs, const uchar* w0, const uchar* w1, const uchar* w2,
+                   const uchar* w3, float* y0, float* y1, float* y2, float* y3, uint K, uint E0, uint E1, uint E2,
+                   uint E3) {
+    gemv_q8k_q4k_x4_body<2>(xq, xs, w0, w1, w2, w3, y0, y1, y2, y3, K, E0, E1, E2, E3);
+}
+
 // ---- the same matvec with the activation quantizer folded in ---------------------------------
 //   gemv_fq8k_q4k_{r1,r2,wide}(x, w, y, K, N, NRB)      x: f32[K], K <= 16384
 // A decode step is a chain of few-microsecond launches, each costing a dispatch and a DRAM round

@@ -84,8 +84,8 @@ const ojh_block_format *ojh_format(uint32_t ggml_type);
 
 // What a kernel touches at given constants. Returns OJH_OK or fails with a message.
 typedef int (*ojh_check_fn)(const struct ojh_kernel_spec *spec, const uint32_t *consts,
-                            const uint32_t grid[3], const uint32_t block[3], size_t need[8],
-                            size_t align[8]);
+                            const uint32_t grid[3], const uint32_t block[3], size_t need[16],
+                            size_t align[16]);
 typedef int (*ojh_shape_fn)(const struct ojh_kernel_spec *spec, const ojh_device *dev, uint32_t K,
                             uint32_t N, uint32_t M, uint32_t grid[3], uint32_t block[3]);
 

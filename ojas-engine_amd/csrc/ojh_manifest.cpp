@@ -54,7 +54,7 @@ static int check_kn(const ojh_kernel_spec *s, uint32_t K, uint32_t N, const ojh_
 
 // gemv_nat_<fmt>{,_accum,_bias,_rN}(x, w, y[, bs], K, N)
 static int check_gemv_nat(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                          const uint32_t block[3], size_t need[8], size_t align[8]) {
+                          const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f;
     uint32_t K = c[0], N = c[1];
     int rc = check_kn(s, K, N, &f);
@@ -75,7 +75,7 @@ static int check_gemv_nat(const ojh_kernel_spec *s, const uint32_t *c, const uin
 
 // gemv_q8k_<fmt>{,_accum,_bias,_rN}(xq, xs, w, y[, bs], K, N)
 static int check_gemv_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                          const uint32_t block[3], size_t need[8], size_t align[8]) {
+                          const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f;
     uint32_t K = c[0], N = c[1];
     int rc = check_kn(s, K, N, &f);
@@ -96,10 +96,38 @@ static int check_gemv_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uin
     return OJH_OK;
 }
 
+// gemv_q8k_<fmt>_x4_{r1,r2}(xq, xs, w0..w3, y0..y3, K, E0..E3): up to four tensors, one activation;
+// E are running row totals (non-decreasing; a tensor with no rows still needs a valid pointer)
+static int check_gemv_q8k_x4(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                             const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], E[4] = {c[1], c[2], c[3], c[4]};
+    int rc = check_kn(s, K, E[3], &f);
+    if (rc) return rc;
+    if ((rc = check_block(block, 0))) return rc;
+    if (E[0] > E[1] || E[1] > E[2] || E[2] > E[3])
+        return ojh_fail(OJH_ERR_ARG, "%s: row totals %u,%u,%u,%u must not decrease", s->name, E[0], E[1], E[2], E[3]);
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    uint64_t cover = (uint64_t)grid[0] * (block[0] / 64) * s->rows_per_wave;
+    if (cover < E[3]) return ojh_fail(OJH_ERR_ARG, "%s: grid covers %llu rows of N=%u", s->name,
+                                      (unsigned long long)cover, E[3]);
+    need[0] = (size_t)K;
+    need[1] = (size_t)(K / 256) * 4;
+    align[1] = 4;
+    for (int i = 0; i < 4; i++) {
+        size_t rows = E[i] - (i ? E[i - 1] : 0);
+        need[2 + i] = rows * (K / f->weights) * f->bytes;
+        need[6 + i] = rows * 4;
+        align[2 + i] = f->bytes % 16 ? 2 : 16;
+        align[6 + i] = 4;
+    }
+    return OJH_OK;
+}
+
 // gemv_fq8k_<fmt>_{r1,r2,wide}(x, w, y, K, N, NRB): quantizer folded in; 4 waves per block,
 // K <= 16384, NRB rows per block (a multiple of 4 * rows per wave)
 static int check_gemv_fq8k(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                           const uint32_t block[3], size_t need[8], size_t align[8]) {
+                           const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f;
     uint32_t K = c[0], N = c[1], NRB = c[2];
     int rc = check_kn(s, K, N, &f);
@@ -119,7 +147,7 @@ static int check_gemv_fq8k(const ojh_kernel_spec *s, const uint32_t *c, const ui
 
 // gemv_nat_<fmt>_m(x, w, y, K, N, M, ACC)
 static int check_gemv_nat_m(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                            const uint32_t block[3], size_t need[8], size_t align[8]) {
+                            const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f;
     uint32_t K = c[0], N = c[1], M = c[2];
     int rc = check_kn(s, K, N, &f);
@@ -139,7 +167,7 @@ static int check_gemv_nat_m(const ojh_kernel_spec *s, const uint32_t *c, const u
 
 // gemv_q8k_<fmt>_m(xq, xs, w, y, K, N, M, ACC)
 static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                            const uint32_t block[3], size_t need[8], size_t align[8]) {
+                            const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f;
     uint32_t K = c[0], N = c[1], M = c[2];
     int rc = check_kn(s, K, N, &f);
@@ -161,7 +189,7 @@ static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const u
 
 // quantize_q8k{,_bf16}(x, q, scales, K, M)
 static int check_quantize(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                          const uint32_t block[3], size_t need[8], size_t align[8]) {
+                          const uint32_t block[3], size_t need[16], size_t align[16]) {
     uint32_t K = c[0], M = c[1];
     if (K == 0 || M == 0) return ojh_fail(OJH_ERR_ARG, "%s: K and M must be positive", s->name);
     int rc = check_block(block, 256);
@@ -180,7 +208,7 @@ static int check_quantize(const ojh_kernel_spec *s, const uint32_t *c, const uin
 
 // dequant_<fmt>_f16(w, out, nblocks)
 static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                         const uint32_t block[3], size_t need[8], size_t align[8]) {
+                         const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f = ojh_format(s->type);
     uint32_t nb = c[0];
     if (!f || nb == 0) return ojh_fail(OJH_ERR_ARG, "%s: nblocks must be positive", s->name);
@@ -199,7 +227,7 @@ static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint
 // gemm_mm_<fmt>(xh, w, y, K, N, accum, M) and gemm_mm_<fmt>_sk(xh, w, y, K, N, M, nsplit);
 // `rows_per_wave` = 1 marks the split-K form.
 static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                      const uint32_t block[3], size_t need[8], size_t align[8]) {
+                      const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f;
     const bool sk = s->rows_per_wave == 1;
     uint32_t K = c[0], N = c[1], M = sk ? c[2] : c[3], nsplit = sk ? c[3] : 1;
@@ -243,7 +271,7 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
 //   4 moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)                     grid [ceil(N/16), E, 1]
 //   5 moe_combine(dv, wgt, y, T, KSEL, D, ACC)                                    grid [ceil(T*D/256),1,1]
 static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                     const uint32_t block[3], size_t need[8], size_t align[8]) {
+                     const uint32_t block[3], size_t need[16], size_t align[16]) {
     int rc;
     for (int i = 0; i < 8; i++) align[i] = 4;
     switch (s->rows_per_wave) {
@@ -330,7 +358,7 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, u
 
 // copy_*(x, y, n) / fill_zero_u32(y, n): one thread per element
 static int check_elementwise(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                             const uint32_t block[3], size_t need[8], size_t align[8]) {
+                             const uint32_t block[3], size_t need[16], size_t align[16]) {
     uint32_t n = c[0];
     if (!n) return ojh_fail(OJH_ERR_ARG, "%s: n must be positive", s->name);
     int rc = check_block(block, 256);
@@ -351,7 +379,7 @@ static int check_elementwise(const ojh_kernel_spec *s, const uint32_t *c, const 
 
 // stream_copy_u32x4(x, y, n16) / stream_read_u32x4(x, y, n16): grid-stride over 16-byte units
 static int check_stream(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
-                        const uint32_t block[3], size_t need[8], size_t align[8]) {
+                        const uint32_t block[3], size_t need[16], size_t align[16]) {
     (void)align;
     uint32_t n16 = c[0];
     if (!n16) return ojh_fail(OJH_ERR_ARG, "%s: n16 must be positive", s->name);
@@ -442,6 +470,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(q + "_m", "gemv_q8k", 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
         if (f.type == OJH_Q4_K) {
             std::string fq = "gemv_fq8k_" + t;
+            add(q + "_x4_r1", "gemv_q8k", 10, 5, f.type, 1, check_gemv_q8k_x4, shape_rows);
+            add(q + "_x4_r2", "gemv_q8k", 10, 5, f.type, 2, check_gemv_q8k_x4, shape_rows);
             add(fq + "_r1", "gemv_q8k", 3, 3, f.type, 1, check_gemv_fq8k, shape_rows);
             add(fq + "_r2", "gemv_q8k", 3, 3, f.type, 2, check_gemv_fq8k, shape_rows);
             add(fq + "_wide", "gemv_q8k", 3, 3, f.type, 2, check_gemv_fq8k, shape_rows);

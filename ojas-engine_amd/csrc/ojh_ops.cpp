@@ -181,6 +181,55 @@ extern "C" int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xsc
     return mm_q8k_launch(dev, xq->ptr, xscales->ptr, w, f, at(y, y_off), bias, m, accum);
 }
 
+extern "C" int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, int count,
+                                const ojh_lin *const *ws, ojh_buf *const *ys, const size_t *y_offs) {
+    if (!dev || !ws || !ys) return ojh_fail(OJH_ERR_ARG, "ojh_mm_q8k_multi: NULL argument");
+    if (count < 1 || count > 4) return ojh_fail(OJH_ERR_ARG, "ojh_mm_q8k_multi: count=%d, takes 1 to 4 projections", count);
+    int rc;
+    bool grouped = true;
+    uint64_t total = 0;
+    for (int i = 0; i < count; i++) {
+        const ojh_block_format *fi;
+        if ((rc = mm_common_checks("ojh_mm_q8k_multi", ws[i], ys[i], y_offs ? y_offs[i] : 0, nullptr, 1, 0, &fi))) return rc;
+        if (ws[i]->type == OJH_Q8_0)
+            return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm_q8k_multi: Q8_0 rows take f32 activations, as dot_q80 does");
+        if (ws[i]->k != ws[0]->k)
+            return ojh_fail(OJH_ERR_ARG, "ojh_mm_q8k_multi: projection %d has K=%u, the first has K=%u", i, ws[i]->k, ws[0]->k);
+        if (ws[i]->type != OJH_Q4_K) grouped = false;
+        total += ws[i]->n;
+    }
+    if (total > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "ojh_mm_q8k_multi: too many rows");
+    size_t nsb = ws[0]->k / 256;
+    if ((rc = span_ok("xq", xq, 0, nsb * 256, 16))) return rc;
+    if ((rc = span_ok("xscales", xscales, 0, nsb * 4, 4))) return rc;
+    if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+    if (!grouped || count == 1) {   // formats without a grouped entry: one launch per projection
+        for (int i = 0; i < count; i++) {
+            const ojh_block_format *fi = ojh_format(ws[i]->type);
+            if ((rc = mm_q8k_launch(dev, xq->ptr, xscales->ptr, ws[i], fi, at(ys[i], y_offs ? y_offs[i] : 0), nullptr, 1, 0)))
+                return rc;
+        }
+        return OJH_OK;
+    }
+    std::vector<void *> p = {xq->ptr, xscales->ptr};
+    uint32_t ends[4], run = 0;
+    for (int i = 0; i < 4; i++) {
+        int j = i < count ? i : count - 1;
+        p.push_back(at(ws[j]->raw, ws[j]->off));
+        if (i < count) run += ws[i]->n;
+        ends[i] = run;
+    }
+    for (int i = 0; i < 4; i++) {
+        int j = i < count ? i : count - 1;
+        p.push_back(at(ys[j], y_offs ? y_offs[j] : 0));
+    }
+    int r = pick_rows(dev, run);
+    if (r == 4) r = 2;
+    uint32_t grid[3] = {(run + 4 * r - 1) / (4 * r), 1, 1}, block[3] = {256, 1, 1};
+    return ojh_launch(dev, r == 2 ? "gemv_q8k_q4k_x4_r2" : "gemv_q8k_q4k_x4_r1", p,
+                      {ws[0]->k, ends[0], ends[1], ends[2], ends[3]}, grid, block);
+}
+
 extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, const ojh_lin *w, ojh_buf *y,
                       size_t y_off, const ojh_buf *bias, uint32_t m, int accum, int act_mode) {
     if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_mm: NULL device");

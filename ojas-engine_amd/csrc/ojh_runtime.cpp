@@ -306,7 +306,7 @@ extern "C" int ojh_dispatch(ojh_device *dev, const char *name, int n_bufs, ojh_b
         return ojh_fail(OJH_ERR_ARG, "%s takes %d buffers then %d constants, got %d and %d", name, s->n_bufs,
                         s->n_consts, n_bufs, n_consts);
     if ((n_bufs && !bufs) || (n_consts && !consts)) return ojh_fail(OJH_ERR_ARG, "%s: NULL argument array", name);
-    size_t need[8] = {0}, align[8];
+    size_t need[16] = {0}, align[16];
     for (auto &a : align) a = 16;
     int rc = s->check(s, consts, grid, block, need, align);
     if (rc) return rc;

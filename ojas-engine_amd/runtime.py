@@ -103,6 +103,7 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_row_bytes": (sz, [u32, u32]),
         "ojh_mm": (i32, [vp, vp, sz, i32, vp, vp, sz, vp, u32, i32, i32]),
         "ojh_mm_q8k": (i32, [vp, vp, vp, vp, vp, sz, vp, u32, i32]),
+        "ojh_mm_q8k_multi": (i32, [vp, vp, vp, i32, vp, vp, vp]),
         "ojh_capture_begin": (i32, [vp]),
         "ojh_capture_end": (i32, [vp, pp]),
         "ojh_graph_launch": (i32, [vp, vp]),
@@ -354,6 +355,16 @@ class HipGpu:
         """Matmul from activations already quantized by `quant_q8k` (shared by several projections)."""
         self._check(self._L.ojh_mm_q8k(self._dev, xq.handle, xscales.handle, w.handle, y.handle, y_off,
                                        bias.handle if bias else None, m, int(accum)))
+
+    def mm_q8k_multi(self, xq: Buf, xscales: Buf, ws: list, ys: list, y_offs: list | None = None) -> None:
+        """Up to four projections of one quantized vector in one launch (fused q/k/v, gate/up)."""
+        n = len(ws)
+        if n != len(ys) or (y_offs is not None and len(y_offs) != n):
+            raise ValueError("mm_q8k_multi: ws, ys and y_offs must have the same length")
+        wa = (C.c_void_p * n)(*[w.handle for w in ws])
+        ya = (C.c_void_p * n)(*[y.handle for y in ys])
+        oa = (C.c_size_t * n)(*y_offs) if y_offs is not None else None
+        self._check(self._L.ojh_mm_q8k_multi(self._dev, xq.handle, xscales.handle, n, wa, ya, oa))
 
     def capture_begin(self) -> None:
         """Start recording dispatches on the device's stream instead of running them."""

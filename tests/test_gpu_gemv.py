@@ -226,3 +226,46 @@ def test_fused_quantizer_is_bit_identical_to_the_two_launch_form(gpu, orc, pkg, 
     a, b = gpu.read(y1, n), gpu.read(y2, n)
     assert np.array_equal(a, b)
     assert peak_err(a, orc.matvec_kq(w, Q4_K, n, k, x)) <= TOL_Q8K_SEEN
+
+
+@pytest.mark.parametrize("ns,k", [((4096, 1024, 1024), 4096), ((14336, 14336), 4096), ((13, 1, 7, 2), 512),
+                                  ((5, 300), 2560), ((33,), 256)])
+def test_grouped_projections_equal_separate_launches(gpu, orc, pkg, ns, k):
+    """ojh_mm_q8k_multi: q/k/v (or gate/up) as separate tensors in one launch; every output must equal
+    the single-tensor launch bit for bit, sit within the parity bar of matvec_kq, and no output may
+    be written past its N rows (odd row counts make a wave straddle two tensors)."""
+    x = pkg.synth.normal_f32(k, "multi", "x", k)
+    ws = [pkg.synth.q4k_weights(n, k, "multi", i, n, k) for i, n in enumerate(ns)]
+    lins = [gpu.lin(Q4_K, n, k, w) for n, w in zip(ns, ws)]
+    xq, xs = gpu.alloc_bytes(k), gpu.alloc(k // 256)
+    gpu.quant_q8k(gpu.upload(x), 1, k, xq, xs)
+    guard = np.float32(-7.25)
+    ys = [gpu.upload(np.full(n + 4, guard, np.float32)) for n in ns]
+    gpu.mm_q8k_multi(xq, xs, lins, ys)
+    for n, w, lin, y in zip(ns, ws, lins, ys):
+        got = gpu.read(y, n + 4)
+        assert np.all(got[n:] == guard)
+        y1 = gpu.alloc(n)
+        gpu.mm_q8k(xq, xs, lin, y1)
+        assert np.array_equal(got[:n], gpu.read(y1, n))
+        assert peak_err(got[:n], orc.matvec_kq(w, Q4_K, n, k, x)) <= TOL_Q8K_SEEN
+
+
+def test_grouped_projections_other_formats_and_errors(gpu, orc, pkg):
+    k = 512
+    x = pkg.synth.normal_f32(k, "multi", "x6", k)
+    w4, w6 = pkg.synth.q4k_weights(40, k, "multi", "a"), pkg.synth.q6k_weights(24, k, "multi", "b")
+    l4, l6 = gpu.lin(Q4_K, 40, k, w4), gpu.lin(Q6_K, 24, k, w6)
+    xq, xs = gpu.alloc_bytes(k), gpu.alloc(k // 256)
+    gpu.quant_q8k(gpu.upload(x), 1, k, xq, xs)
+    y4, y6 = gpu.alloc(40), gpu.alloc(24)
+    gpu.mm_q8k_multi(xq, xs, [l4, l6], [y4, y6])      # mixed formats: one launch each
+    assert peak_err(gpu.read(y4, 40), orc.matvec_kq(w4, Q4_K, 40, k, x)) <= TOL_Q8K_SEEN
+    assert peak_err(gpu.read(y6, 24), orc.matvec_kq(w6, Q6_K, 24, k, x)) <= TOL_Q8K_SEEN
+    other = gpu.lin(Q4_K, 8, 256, pkg.synth.q4k_weights(8, 256, "multi", "c"))
+    with pytest.raises(pkg.OjasHipError, match="has K="):
+        gpu.mm_q8k_multi(xq, xs, [l4, other], [y4, y6])
+    with pytest.raises(pkg.OjasHipError, match="1 to 4"):
+        gpu.mm_q8k_multi(xq, xs, [l4] * 5, [y4] * 5)
+    with pytest.raises(pkg.OjasHipError, match="needs"):
+        gpu.mm_q8k_multi(xq, xs, [l4, l4], [y4, y6])
