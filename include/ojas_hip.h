@@ -58,8 +58,14 @@ enum { OJH_X_F32 = 0, OJH_X_BF16 = 1, OJH_X_F16 = 2 };
  *   OJH_ACT_FLOAT — activations kept in floating point (f32 for the GEMV, rounded to f16 into the
  *                 MFMA tile for the GEMM): the contract of the reference's GPU kernels
  *                 (crates/ojas-core/src/quant_src.rs:779-867, crates/ojas-cuda/src/kernels/gemm_q.rs:1-56).
- *   OJH_ACT_AUTO  — OJH_ACT_Q8K for K-quant GEMV-shaped calls, the MFMA tile above the crossover. */
-enum { OJH_ACT_AUTO = 0, OJH_ACT_Q8K = 1, OJH_ACT_FLOAT = 2 };
+ *                 In the tile a Q4_K weight is the binary16 fma qa*q + qb with qa = f16(d*sc),
+ *                 qb = f16(-dmin*m): the bits the reference's `gemm_mm_q4l` multiplies
+ *                 (gemm_q.rs:104-140 over crates/ojas-formats/src/quant.rs:187-222); Q6_K and Q8_0
+ *                 weights are the bits of `dequant_to_f16`.
+ *   OJH_ACT_FLOAT_EXACT — as OJH_ACT_FLOAT, but a Q4_K weight too enters the tile as the bits of
+ *                 `dequant_to_f16` (crates/ojas-formats/src/gguf.rs:612-1116); a slower tile.
+ *   OJH_ACT_AUTO  — OJH_ACT_Q8K for K-quant GEMV-shaped calls, OJH_ACT_FLOAT above the crossover. */
+enum { OJH_ACT_AUTO = 0, OJH_ACT_Q8K = 1, OJH_ACT_FLOAT = 2, OJH_ACT_FLOAT_EXACT = 3 };
 
 typedef struct ojh_device ojh_device; /* one GPU + one stream + loaded families */
 typedef struct ojh_buf ojh_buf;       /* device allocation with a known size */

@@ -32,6 +32,7 @@ FAMILIES = {
     "gemv_q8k": ("gemv_q8k.hip", []),
     "glue": ("glue.hip", []),
     "gemm": ("gemm.hip", ["-ffp-contract=off"]),
+    "gemm_xl": ("gemm_xl.hip", ["-ffp-contract=off"]),
     "moe": ("moe.hip", []),
 }
 

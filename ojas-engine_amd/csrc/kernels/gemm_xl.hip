@@ -1,0 +1,291 @@
+// Family "gemm_xl": the prefill matmul  y[M,N] (+)= x[M,K] . W^T  on raw Q4_K blocks with the
+// arithmetic of the reference's GPU prefill kernel `gemm_mm_q4l`
+// (crates/ojas-cuda/src/kernels/gemm_q.rs:104-140 over crates/ojas-formats/src/quant.rs:187-222):
+// per 32-weight sub-block  qa = f16(d*sc),  qb = f16(-dmin*m),  and every weight enters the tile as
+// the f16 fused multiply-add  qa*q + qb  (one rounding).  The reference computes qa / qb in a
+// load-time relayout pass; here they are formed in the kernel from the raw super-block header, so
+// the weights stay in the file's layout.  Activations are f16 [M][K], accumulation is f32.
+//
+//   gemm_mm_q4kl{,_m128}(xh, w, y, K, N, accum, M)        grid [ceil(N/256), ceil(M/BM), 1]
+//   gemm_mm_q4kl{,_m128}_sk(xh, w, y, K, N, M, nsplit)    grid.z = nsplit; f32 atomic adds into y
+//   (BM = 256 tokens per tile, 128 for the _m128 entries)
+//
+// CDNA4 plan.  One workgroup of 4 waves (one per SIMD) owns BM x 256 outputs and walks K in steps
+// of 64; a wave owns (BM/2) x 128 as (BM/64) x 4 blocks of v_mfma_f32_32x32x16_f16, 256
+// accumulator registers at BM = 256.  What bounds such a tile on this chip is LDS bandwidth
+// (128 bytes per clock per CU, shared by the four SIMDs) and vector-ALU issue, not the matrix
+// pipe, so the design spends as little of either as it can:
+//   * a wave tile of 128 x 128 reads 512 LDS bytes per MFMA (a 128 x 64 wave tile reads 768);
+//   * activations go from global memory straight into LDS (global_load_lds_dwordx4), never
+//     through registers; rows are 128 bytes, and the 16-byte chunk c of row r sits in slot
+//     c ^ ((r >> 1) & 7), applied on the global side of the copy: LDS has 64 four-byte banks, two
+//     rows span them once, so 16 consecutive rows reading the same chunk touch every bank
+//     exactly once and a 128-bit fragment read runs at the full 256 bytes per clock, unpadded;
+//   * a nibble becomes the f16 1024 + q by or-ing it into 0x6400; subtracting 1024 and one packed
+//     fma per pair of weights finish the job: about 2 vector instructions per weight;
+//   * the raw weight bytes take the same road (a thread's 48 bytes per step: super-block header
+//     and one 32-byte chunk), two steps ahead, and are read back from LDS by the thread that
+//     dequantizes them: no asynchronous load ever targets a register, so there is nothing the
+//     compiler could copy or sink before it has landed; the copies are awaited with s_waitcnt.
+#include "ojk_common.h"
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint u32x4 __attribute__((ext_vector_type(4)));
+
+#define GX_BN 256u
+#define GX_BK 64u
+#define GX_ROW 128u                   // bytes per LDS row: 64 f16
+#define GX_WSTAGE (GX_BN * GX_ROW)    // 32 KB
+#define GX_RAW (GX_BN * 48u)           // raw bytes of a weight slab: 16 (header) + 32 (chunk) per row
+
+// 16 bytes per lane from `base + voff` to LDS at `lds_addr + 16 * lane` (base and lds_addr uniform).
+__device__ __forceinline__ void gx_load_lds16(const void* base, uint voff, uint lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(base), "s"(lds_addr)
+                 : "memory");
+}
+template <int N>
+__device__ __forceinline__ void gx_wait() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// One thread's share of a weight slab: 64 weights of one row = one 32-byte chunk c of a Q4_K
+// super-block (low nibbles: sub-block 2c, high nibbles: sub-block 2c+1) plus the header.
+struct GxQ4K {
+    u32x4 hdr, q0, q1;
+    uint c;
+    half2v a_lo, c_lo, a_hi, c_hi;
+    // from the raw staging slot: header, then the two halves of the chunk (4 KB apart per part)
+    __device__ __forceinline__ void read(const uchar* raw, uint chunk) {
+        c = chunk;
+        hdr = *(const u32x4*)raw;
+        q0 = *(const u32x4*)(raw + 4096u);
+        q1 = *(const u32x4*)(raw + 8192u);
+    }
+    __device__ __forceinline__ void prep() {
+        uint sc, mn;
+        q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
+        const float d = f16_bits_to_f32(hdr.x & 0xFFFFu), ndm = -f16_bits_to_f32(hdr.x >> 16);
+        // products of an f16 and a 6-bit integer are exact in f32: one rounding, to f16
+        // (pinned, so that a product of zero keeps its sign through the conversion)
+        float p1 = d * (float)(sc & 0xFFu), r1 = ndm * (float)(mn & 0xFFu);
+        float p2 = d * (float)(sc >> 8), r2 = ndm * (float)(mn >> 8);
+        asm volatile("" : "+v"(p1), "+v"(r1), "+v"(p2), "+v"(r2));
+        const _Float16 a1 = (_Float16)p1, b1 = (_Float16)r1, a2 = (_Float16)p2, b2 = (_Float16)r2;
+        a_lo = (half2v){a1, a1};
+        c_lo = (half2v){b1, b1};
+        a_hi = (half2v){a2, a2};
+        c_hi = (half2v){b2, b2};
+    }
+    static __device__ __forceinline__ uint fma2(uint bits, half2v a, half2v c) {
+        const half2v k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+        half2v q = __builtin_bit_cast(half2v, bits) - k1024;
+        return __builtin_bit_cast(uint, __builtin_elementwise_fma(q, a, c));
+    }
+    // dword I (0..7) of the chunk: bytes 4I..4I+3 -> columns 4I..4I+3 (low) and 32+4I.. (high)
+    template <int I>
+    __device__ __forceinline__ void part(uint (&lo)[2], uint (&hi)[2]) const {
+        const uint v = I < 4 ? q0[I & 3] : q1[I & 3];
+        const uint p0 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u);  // bytes (b0, 0, b1, 0)
+        const uint p1 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u);  // bytes (b2, 0, b3, 0)
+        lo[0] = fma2((p0 & 0x000F000Fu) | 0x64006400u, a_lo, c_lo);
+        lo[1] = fma2((p1 & 0x000F000Fu) | 0x64006400u, a_lo, c_lo);
+        hi[0] = fma2(((p0 >> 4) & 0x000F000Fu) | 0x64006400u, a_hi, c_hi);
+        hi[1] = fma2(((p1 >> 4) & 0x000F000Fu) | 0x64006400u, a_hi, c_hi);
+    }
+};
+
+// MI = 32-row blocks per wave along M: the tile is (64 MI) x 256.
+template <int MI, bool SPLITK>
+__device__ __forceinline__ void gemm_xl_body(const ushort* __restrict__ xh, const uchar* __restrict__ w,
+                                             float* __restrict__ y, uint K, uint N, uint accum, uint M, uint nsplit) {
+    constexpr uint BM = 64u * MI;
+    constexpr uint XSTAGE = BM * GX_ROW;
+    constexpr int XL = MI * 2;  // LDS-direct loads per wave and slab
+    __shared__ __attribute__((aligned(1024))) uchar lds[2 * XSTAGE + 2 * GX_WSTAGE + 2 * GX_RAW];
+    const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint n0 = blockIdx.x * GX_BN, m0 = blockIdx.y * BM;
+    uint k_begin = 0, k_end = K;
+    if (SPLITK) {
+        uint steps = K / GX_BK, per = (steps + nsplit - 1) / nsplit;
+        k_begin = min(blockIdx.z * per, steps) * GX_BK;
+        k_end = min((blockIdx.z + 1) * per, steps) * GX_BK;
+        if (k_begin >= k_end) return;
+    }
+    const uint nt = (k_end - k_begin) / GX_BK;
+    const uint lds0 = (uint)(size_t)(__attribute__((address_space(3))) uchar*)lds;
+
+    // activation slab: wave `wave`, copy i moves rows (wave*XL + i)*8 .. +7; lane -> row lane/8,
+    // slot lane%8, which holds source chunk (lane%8) ^ ((row/2)%8)
+    uint xoff[XL];
+#pragma unroll
+    for (int i = 0; i < XL; i++) {
+        const uint r = (wave * XL + i) * 8u + (lane >> 3);
+        const uint m = min(m0 + r, M - 1u);
+        xoff[i] = m * K * 2u + (((lane & 7u) ^ ((r >> 1) & 7u)) << 4);
+    }
+    // (wave-uniform by construction; readfirstlane tells the compiler so)
+    const uint x_lds = lds0 + (uint)__builtin_amdgcn_readfirstlane((int)wave) * XL * 1024u;  // + stage * XSTAGE + i * 1024
+    // weight slab: thread -> row tid, all 64 columns.  Raw bytes: three 4 KB parts per staging
+    // slot (headers, first and second half of the chunk), a thread's 16 bytes at 16 * tid.
+    const uint wrow_off = min(n0 + tid, N - 1u) * ((K >> 8) * Q4K_BYTES);
+    const uint raw_off = 2u * XSTAGE + 2u * GX_WSTAGE;
+    const uint raw_lds = lds0 + raw_off + (uint)__builtin_amdgcn_readfirstlane((int)wave) * 1024u;  // + slot * GX_RAW + part * 4096
+    const uchar* const raw_rd = lds + raw_off + tid * 16u;                                          // + slot * GX_RAW + part * 4096
+    uchar* const w_lds = lds + 2u * XSTAGE + tid * GX_ROW;  // + stage * GX_WSTAGE + slot * 16
+    const uint wsw = (tid >> 1) & 7u;
+
+    // wave tile: rows wy*32*MI.., columns wx*128..
+    const uint wy = wave >> 1, wx = wave & 1u;
+    const uint fr = lane & 31u, kg = lane >> 5, sw = (fr >> 1) & 7u;
+    const uint a_lds = (wy * 32u * MI + fr) * GX_ROW;
+    const uint b_lds = 2u * XSTAGE + (wx * 128u + fr) * GX_ROW;
+    float16v acc[MI][4];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    GxQ4K ld;
+    const uchar* xbase = (const uchar*)xh;
+    const uint last = nt - 1u;
+
+// Requests past the last slab are clamped onto it: every step is then the same straight-line
+// code (the surplus slab is fetched and dequantized into a stage nobody reads again).
+#define GX_LOAD_X(T)                                                                             \
+    do {                                                                                         \
+        const uchar* b_ = xbase + (size_t)(k_begin + min((T), last) * GX_BK) * 2u;               \
+        const uint s_ = x_lds + ((T) & 1u) * XSTAGE;                                             \
+        _Pragma("unroll") for (int i_ = 0; i_ < XL; i_++) gx_load_lds16(b_, xoff[i_], s_ + i_ * 1024u); \
+    } while (0)
+#define GX_LOAD_W(T)                                                                             \
+    do {                                                                                         \
+        const uint k0_ = k_begin + min((T), last) * GX_BK;                                       \
+        const uchar* b_ = w + (size_t)(k0_ >> 8) * Q4K_BYTES;                                    \
+        const uchar* q_ = b_ + 16u + ((k0_ >> 6) & 3u) * 32u;                                    \
+        const uint s_ = raw_lds + ((T) & 1u) * GX_RAW;                                           \
+        gx_load_lds16(b_, wrow_off, s_);                                                         \
+        gx_load_lds16(q_, wrow_off, s_ + 4096u);                                                 \
+        gx_load_lds16(q_ + 16u, wrow_off, s_ + 8192u);                                           \
+    } while (0)
+#define GX_READ_W(T) ld.read(raw_rd + ((T) & 1u) * GX_RAW, ((k_begin >> 6) + min((T), last)) & 3u)
+// dequantize dwords 2P, 2P+1 of the chunk and write slots P (low nibbles) and 4+P (high)
+#define GX_DEQ(LD, STG, P)                                                                       \
+    do {                                                                                         \
+        uint l0_[2], h0_[2], l1_[2], h1_[2];                                                     \
+        LD.template part<2 * (P)>(l0_, h0_);                                                     \
+        LD.template part<2 * (P) + 1>(l1_, h1_);                                                 \
+        uchar* r_ = w_lds + (STG) * GX_WSTAGE;                                                   \
+        *(u32x4*)(r_ + ((((uint)(P)) ^ wsw) << 4)) = (u32x4){l0_[0], l0_[1], l1_[0], l1_[1]};    \
+        *(u32x4*)(r_ + (((4u + (P)) ^ wsw) << 4)) = (u32x4){h0_[0], h0_[1], h1_[0], h1_[1]};     \
+    } while (0)
+#define GX_READ(STG, KS, AF, BF)                                                                 \
+    do {                                                                                         \
+        const uint o_ = (((2u * (KS) + kg) ^ sw) << 4);                                          \
+        const uchar* xa_ = lds + (STG) * XSTAGE + a_lds + o_;                                    \
+        const uchar* wb_ = lds + (STG) * GX_WSTAGE + b_lds + o_;                                 \
+        _Pragma("unroll") for (int i = 0; i < MI; i++) AF[i] = *(const half8*)(xa_ + i * 32u * GX_ROW); \
+        _Pragma("unroll") for (int j = 0; j < 4; j++) BF[j] = *(const half8*)(wb_ + j * 32u * GX_ROW);  \
+    } while (0)
+#define GX_MMA(AF, BF)                                                                           \
+    do {                                                                                         \
+        _Pragma("unroll") for (int i = 0; i < MI; i++)                                           \
+            _Pragma("unroll") for (int j = 0; j < 4; j++)                                        \
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(AF[i], BF[j], acc[i][j], 0, 0, 0); \
+    } while (0)
+// One K sub-step's worth of interleaving: 4 MI MFMAs.  The LDS reads (the next sub-step's
+// fragments) go out in pairs behind the first MFMAs so that their data is back long before the
+// sub-step ends; the dequantization's vector-ALU instructions fill the gaps after every MFMA; the
+// two LDS writes of the dequantized chunk come last.
+#define GX_MIX()                                                                                 \
+    do {                                                                                         \
+        _Pragma("unroll") for (int g_ = 0; g_ < 4 * MI; g_++) {                                  \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                   \
+            if (g_ < (MI + 4 + 1) / 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);        \
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                                   \
+        }                                                                                        \
+        __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);                                       \
+    } while (0)
+// Step T: the raw weights of slab T+1 (landed during step T-1) come out of their staging slot,
+// the activations of slab T+1 and the raw weights of slab T+2 are requested, and slab T+1 is
+// dequantized between the MFMAs of slab T.  Everything requested has landed at the barrier.
+#define GX_STEP(T)                                                                               \
+    do {                                                                                         \
+        const uint cur_ = (T) & 1u, nxt_ = cur_ ^ 1u;                                            \
+        half8 afA[MI], bfA[4], afB[MI], bfB[4];                                                  \
+        GX_READ(cur_, 0, afA, bfA);                                                              \
+        GX_READ_W((T) + 1u);                                                                     \
+        GX_LOAD_X((T) + 1u);                                                                     \
+        GX_LOAD_W((T) + 2u);                                                                     \
+        ld.prep();                                                                               \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+        GX_READ(cur_, 1, afB, bfB); GX_MMA(afA, bfA); GX_DEQ(ld, nxt_, 0); GX_MIX();             \
+        GX_READ(cur_, 2, afA, bfA); GX_MMA(afB, bfB); GX_DEQ(ld, nxt_, 1); GX_MIX();             \
+        GX_READ(cur_, 3, afB, bfB); GX_MMA(afA, bfA); GX_DEQ(ld, nxt_, 2); GX_MIX();             \
+        GX_MMA(afB, bfB); GX_DEQ(ld, nxt_, 3); GX_MIX();                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+        gx_wait<0>();                                                                            \
+        __syncthreads();                                                                         \
+    } while (0)
+
+    // prologue: slab 0 in place, the raw weights of slab 1 staged
+    GX_LOAD_X(0u);
+    GX_LOAD_W(0u);
+    GX_LOAD_W(1u);
+    gx_wait<0>();
+    GX_READ_W(0u);
+    ld.prep();
+    GX_DEQ(ld, 0u, 0); GX_DEQ(ld, 0u, 1); GX_DEQ(ld, 0u, 2); GX_DEQ(ld, 0u, 3);
+    __syncthreads();
+
+    for (uint t = 0; t < nt; t++) GX_STEP(t);
+#undef GX_READ_W
+#undef GX_LOAD_X
+#undef GX_LOAD_W
+#undef GX_DEQ
+#undef GX_READ
+#undef GX_MMA
+#undef GX_MIX
+#undef GX_STEP
+
+    // epilogue: D register v of block (i, j) holds token row 8*(v/4) + 4*kg + v%4, output fr
+#pragma unroll
+    for (int i = 0; i < MI; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint n = n0 + wx * 128u + 32u * j + fr;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const uint m = m0 + wy * 32u * MI + 32u * i + 8u * (v >> 2) + 4u * kg + (v & 3u);
+                if (m < M && n < N) {
+                    float* o = y + (size_t)m * N + n;
+                    if (SPLITK) atomicAdd(o, acc[i][j][v]);
+                    else *o = accum ? *o + acc[i][j][v] : acc[i][j][v];
+                }
+            }
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+gemm_mm_q4kl(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
+    gemm_xl_body<4, false>(xh, w, y, K, N, accum, M, 1u);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemm_mm_q4kl_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
+    gemm_xl_body<4, true>(xh, w, y, K, N, 1u, M, nsplit);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemm_mm_q4kl_m128(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
+    gemm_xl_body<2, false>(xh, w, y, K, N, accum, M, 1u);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemm_mm_q4kl_m128_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
+    gemm_xl_body<2, true>(xh, w, y, K, N, 1u, M, nsplit);
+}

@@ -226,18 +226,33 @@ static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint
 
 // gemm_mm_<fmt>(xh, w, y, K, N, accum, M) and gemm_mm_<fmt>_sk(xh, w, y, K, N, M, nsplit);
 // `rows_per_wave` = 1 marks the split-K form.
+// `rows_per_wave` carries the variant: bit 0 = split-K entry; 0/1 the 256 x 128 tile of family
+// "gemm", 2/3 the 256 x 256 tile and 4/5 the 128 x 256 tile of family "gemm_xl".
+static void gemm_tile(const ojh_kernel_spec *s, uint32_t *bm, uint32_t *bn, bool *sk) {
+    *sk = s->rows_per_wave & 1;
+    *bn = s->rows_per_wave >= 2 ? 256 : 128;
+    *bm = s->rows_per_wave >= 4 ? 128 : 256;
+}
+
 static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                       const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f;
-    const bool sk = s->rows_per_wave == 1;
+    bool sk;
+    uint32_t bm, bn;
+    gemm_tile(s, &bm, &bn, &sk);
     uint32_t K = c[0], N = c[1], M = sk ? c[2] : c[3], nsplit = sk ? c[3] : 1;
     int rc = check_kn(s, K, N, &f);
     if (rc) return rc;
     if (K % 64) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a multiple of 64", s->name, K);
     if (M == 0 || nsplit == 0) return ojh_fail(OJH_ERR_ARG, "%s: M and nsplit must be positive", s->name);
     if ((rc = check_block(block, 256))) return rc;
-    if (grid[0] != (N + 127) / 128 || grid[1] != (M + 255) / 256 || grid[2] != nsplit)
-        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, (N + 127) / 128, (M + 255) / 256, nsplit);
+    if (grid[0] != (N + bn - 1) / bn || grid[1] != (M + bm - 1) / bm || grid[2] != nsplit)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, (N + bn - 1) / bn, (M + bm - 1) / bm, nsplit);
+    // the 256-wide tiles address activations with 32-bit byte offsets
+    if (bn == 256 && (uint64_t)M * K * 2 > 0xFFFFFFFFull)
+        return ojh_fail(OJH_ERR_ARG, "%s: M*K=%llu exceeds 2^31 activations", s->name, (unsigned long long)M * K);
+    if (bn == 256 && (uint64_t)N * (K / f->weights) * f->bytes > 0xFFFFFFFFull)
+        return ojh_fail(OJH_ERR_ARG, "%s: the weight tensor exceeds 4 GiB", s->name);
     need[0] = (size_t)M * K * 2;
     need[1] = (size_t)N * (K / f->weights) * f->bytes;
     need[2] = (size_t)M * N * 4;
@@ -248,10 +263,13 @@ static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_
 
 static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
                       uint32_t grid[3], uint32_t block[3]) {
-    grid[0] = (N + 127) / 128;
-    grid[1] = (M + 255) / 256;
+    bool sk;
+    uint32_t bm, bn;
+    gemm_tile(s, &bm, &bn, &sk);
+    grid[0] = (N + bn - 1) / bn;
+    grid[1] = (M + bm - 1) / bm;
     grid[2] = 1;
-    if (s->rows_per_wave == 1) {  // split K until every CU has a tile, at least 4 K-steps per slice
+    if (sk) {  // split K until every CU has a tile, at least 4 K-steps per slice
         uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
         uint32_t tiles = grid[0] * grid[1], steps = K / 64;
         uint32_t z = tiles ? cus / tiles : 1;  // floor: 224 tiles on 256 CUs are better left whole
@@ -486,6 +504,11 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g, "gemm", 3, 4, f.type, 0, check_gemm, shape_gemm);
         add(g + "_sk", "gemm", 3, 4, f.type, 1, check_gemm, shape_gemm);
     }
+    // Q4_K with the arithmetic of the reference's `gemm_mm_q4l` (f16 qa*q + qb), 256-wide tiles
+    add("gemm_mm_q4kl", "gemm_xl", 3, 4, OJH_Q4_K, 2, check_gemm, shape_gemm);
+    add("gemm_mm_q4kl_sk", "gemm_xl", 3, 4, OJH_Q4_K, 3, check_gemm, shape_gemm);
+    add("gemm_mm_q4kl_m128", "gemm_xl", 3, 4, OJH_Q4_K, 4, check_gemm, shape_gemm);
+    add("gemm_mm_q4kl_m128_sk", "gemm_xl", 3, 4, OJH_Q4_K, 5, check_gemm, shape_gemm);
     // MoE: `rows_per_wave` selects the kernel inside check_moe / shape_moe
     add("moe_topk", "moe", 3, 2, 0, 0, check_moe, shape_moe);
     add("moe_topk_m", "moe", 3, 2, 0, 1, check_moe, shape_moe);

@@ -249,7 +249,11 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     // (the reference switches at 8 rows, crates/ojas-models/src/decoder/dispatch.rs:70-75).
     if (m >= dev->gemm_min_m && act_mode != OJH_ACT_Q8K && K % 64 == 0 && (uint64_t)m * K < 0x7FFFFFFFull &&
         (uint64_t)m * N < 0x7FFFFFFFull) {
-        if ((rc = ensure(dev, "glue")) || (rc = ensure(dev, "gemm"))) return rc;
+        // Q4_K takes the 256-wide tile with the reference GPU kernel's arithmetic (f16 qa*q + qb)
+        // unless the tile that reproduces dequant_to_f16 bit for bit is asked for.
+        const bool xl = w->type == OJH_Q4_K && !dev->gemm_exact && act_mode != OJH_ACT_FLOAT_EXACT &&
+                        (uint64_t)w->row_bytes * N <= 0xFFFFFFFFull;  // 32-bit row offsets in that tile
+        if ((rc = ensure(dev, "glue")) || (rc = ensure(dev, xl ? "gemm_xl" : "gemm"))) return rc;
         ojh_buf *xh;
         if ((rc = ojh_scratch_get(dev, "xh", (size_t)m * K * 2, &xh))) return rc;
         uint32_t n_el = m * K, eg[3] = {(n_el + 255) / 256, 1, 1};
@@ -257,6 +261,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
                              {n_el}, eg, block)))
             return rc;
         std::string base = std::string("gemm_mm_") + (w->type == OJH_Q8_0 ? "q8_0" : f->tag);
+        if (xl) base = m > 128 ? "gemm_mm_q4kl" : "gemm_mm_q4kl_m128";
         uint32_t sg[3], sb[3];
         if ((rc = ojh_launch_shape(dev, (base + "_sk").c_str(), K, N, m, sg, sb))) return rc;
         if (dev->gemm_split_override > 0) sg[2] = (uint32_t)dev->gemm_split_override;
@@ -271,7 +276,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         return ojh_launch(dev, base.c_str(), {xh->ptr, wp, yp}, {K, N, (uint32_t)(accum != 0), m}, sg, sb);
     }
 
-    bool q8k = w->type != OJH_Q8_0 && act_mode != OJH_ACT_FLOAT;
+    bool q8k = w->type != OJH_Q8_0 && act_mode != OJH_ACT_FLOAT && act_mode != OJH_ACT_FLOAT_EXACT;
     // Opt-in: one token, f32 in, plain store through the launch that quantizes x itself
     // (bit-identical results).  Measured slower than quantize + matvec at every decode shape on
     // MI355X — each block repeats the quantization and reads x through LDS — so it is off by default.

@@ -599,6 +599,43 @@ void ojo_relayout_q4k_q4l(const uint8_t *w, size_t k, size_t n, uint8_t *nib, ui
     }
 }
 
+/* double -> binary16, round to nearest even, directly (no intermediate f32 rounding) */
+static uint16_t f64_to_f16(double v) {
+    uint16_t h = ojo_f32_to_f16((float)v);
+    uint16_t sign = h & 0x8000u, mag = h & 0x7FFFu;
+    if (mag >= 0x7C00u || v != v) return h;
+    double a = v < 0 ? -v : v, best = -1.0;
+    uint16_t pick = mag;
+    for (int dlt = -1; dlt <= 1; dlt++) {
+        int c = (int)mag + dlt;
+        if (c < 0 || c >= 0x7C00) continue;
+        double cv = (double)ojo_f16_to_f32((uint16_t)c), e = cv > a ? cv - a : a - cv;
+        if (best < 0 || e < best || (e == best && !(c & 1))) { best = e; pick = (uint16_t)c; }
+    }
+    return (uint16_t)(sign | pick);
+}
+
+void ojo_q4l_weights_f16(const uint8_t *w, size_t k, size_t n, uint16_t *out) {
+    /* What the reference's GPU prefill kernel puts in its tile for a Q4L weight
+     * (crates/ojas-cuda/src/kernels/gemm_q.rs:104-140): q as a half, then one fused multiply-add
+     * qa*q + qb in binary16 — the exact value rounded once.  qa*q + qb is exact in double
+     * (11-bit x 4-bit product plus an 11-bit addend within the binary16 exponent range). */
+    size_t nblk = k / 32;
+    uint8_t *nib = (uint8_t *)malloc(n * k / 2);
+    uint16_t *qa = (uint16_t *)malloc(n * nblk * 2), *qb = (uint16_t *)malloc(n * nblk * 2);
+    ojo_relayout_q4k_q4l(w, k, n, nib, qa, qb);
+    for (size_t r = 0; r < n; r++)
+        for (size_t b = 0; b < nblk; b++) {
+            double a = (double)ojo_f16_to_f32(qa[r * nblk + b]), c = (double)ojo_f16_to_f32(qb[r * nblk + b]);
+            for (int i = 0; i < 16; i++) {
+                uint8_t v = nib[r * (k / 2) + b * 16 + i];
+                out[r * k + b * 32 + 2 * i] = f64_to_f16(a * (double)(v & 15) + c);
+                out[r * k + b * 32 + 2 * i + 1] = f64_to_f16(a * (double)(v >> 4) + c);
+            }
+        }
+    free(nib); free(qa); free(qb);
+}
+
 /* ---------------------------------------------------------------- double-precision reference */
 
 struct ref_ctx {
@@ -610,9 +647,10 @@ static void ref_row(void *p, size_t row) {
     struct ref_ctx *c = (struct ref_ctx *)p;
     double *w = (double *)malloc(c->k * sizeof(double));
     const uint8_t *rb = c->raw + row * c->row_bytes;
-    if (c->wmode == 1) {
+    if (c->wmode == 1 || c->wmode == 2) {
         uint16_t *h = (uint16_t *)malloc(c->k * sizeof(uint16_t));
-        ojo_dequant_to_f16(rb, c->ty, c->k, h);
+        if (c->wmode == 2) ojo_q4l_weights_f16(rb, c->k, 1, h);
+        else ojo_dequant_to_f16(rb, c->ty, c->k, h);
         for (size_t i = 0; i < c->k; i++) w[i] = ojo_f16_to_f32(h[i]);
         free(h);
     } else {
@@ -631,6 +669,7 @@ int ojo_matmul_ref(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const fl
                    int wmode, int xmode, int threads, double *y) {
     uint32_t bb, wpb;
     if (!ojo_block_shape(ty, &bb, &wpb) || k % wpb) return -1;
+    if (wmode == 2 && ty != 12) return -1; /* the Q4L arithmetic exists for Q4_K only */
     double *xd = (double *)malloc(m * k * sizeof(double));
     for (size_t i = 0; i < m * k; i++) {
         float v = x[i];

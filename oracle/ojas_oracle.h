@@ -84,9 +84,15 @@ void  ojo_matmul_q8(const int8_t *wq, const float *wscale, size_t n, size_t k,
 /* relayout_q4k_q4l (crates/ojas-formats/src/quant.rs:192-222). */
 void ojo_relayout_q4k_q4l(const uint8_t *w, size_t k, size_t n, uint8_t *nib, uint16_t *qa, uint16_t *qb);
 
+/* The f16 weights the reference's GPU prefill kernel multiplies for Q4_K tensors relaid to Q4L:
+ * binary16 fma(qa, q, qb) per weight (crates/ojas-cuda/src/kernels/gemm_q.rs:104-140 over the
+ * relayout above).  `out` is [n][k] binary16 bit patterns in the tensor's own weight order. */
+void ojo_q4l_weights_f16(const uint8_t *w, size_t k, size_t n, uint16_t *out);
+
 /* The GPU-test oracle: y = x * dequant(W)^T accumulated in double
  * (crates/ojas-cuda/tests/conformance.rs:798-803, tests/prefill_gemm_q.rs:116-130).
- *   wmode: 0 = weights exact (double), 1 = weights rounded to f16 as dequant_to_f16 stores them
+ *   wmode: 0 = weights exact (double), 1 = weights rounded to f16 as dequant_to_f16 stores them,
+ *          2 = Q4_K weights as the Q4L GPU kernel forms them (ojo_q4l_weights_f16)
  *   xmode: 0 = x as given, 1 = x rounded to f16, 2 = x rounded to bf16
  * x is [m][k] f32, y is [m][n] double. */
 int ojo_matmul_ref(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const float *x, size_t m,

@@ -65,6 +65,8 @@ def lib() -> C.CDLL:
         L.ojo_matmul_q8.argtypes = [vp, vp, sz, sz, vp, sz, vp, i32, vp]
         L.ojo_relayout_q4k_q4l.restype = None
         L.ojo_relayout_q4k_q4l.argtypes = [vp, sz, sz, vp, vp, vp]
+        L.ojo_q4l_weights_f16.restype = None
+        L.ojo_q4l_weights_f16.argtypes = [vp, sz, sz, vp]
         L.ojo_matmul_ref.argtypes = [vp, u32, sz, sz, vp, sz, i32, i32, i32, vp]
         L.ojo_moe_topk.restype = None
         L.ojo_moe_topk.argtypes = [vp, i32, i32, vp, vp]
@@ -188,8 +190,17 @@ def relayout_q4k_q4l(w: np.ndarray, k: int, n: int):
     return nib, qa, qb
 
 
+def q4l_weights_f16(w: np.ndarray, k: int, n: int) -> np.ndarray:
+    """binary16 bit patterns [n*k] of fma(qa, q, qb): the Q4L GPU kernel's in-tile weights."""
+    w = np.ascontiguousarray(w, np.uint8)
+    assert w.size == n * k // 256 * 144
+    out = np.empty(n * k, np.uint16)
+    lib().ojo_q4l_weights_f16(_p(w), k, n, _p(out))
+    return out
+
+
 def matmul_ref(raw, ty, n, k, x, wmode: int = 0, xmode: int = 0, threads: int = 8) -> np.ndarray:
-    """y[m][n] in float64; wmode 0 exact / 1 f16-rounded weights; xmode 0 / 1 f16 / 2 bf16."""
+    """y[m][n] in float64; wmode 0 exact / 1 f16-rounded weights / 2 Q4L kernel weights; xmode 0 / 1 f16 / 2 bf16."""
     raw = np.ascontiguousarray(raw, np.uint8)
     x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
     m = x.shape[0]

@@ -1,11 +1,15 @@
-"""Prefill / verify matmul on the MFMA tile against the CPU oracle.
+"""Prefill / verify matmul on the MFMA tiles against the CPU oracle.
 
-Oracle: x . dequant(W)^T accumulated in double (crates/ojas-cuda/tests/prefill_gemm_q.rs:116-130),
-once with x rounded to f16 and W as `dequant_to_f16` stores it (what the tile holds: the kernel's
-own error) and once with x and W unrounded.  Metrics and the reference's bounds:
+Oracle: x . W^T accumulated in double (crates/ojas-cuda/tests/prefill_gemm_q.rs:116-130), once
+with x rounded to f16 and W as the f16 bits the tile is specified to hold (the kernel's own
+error) and once with x and W unrounded.  Metrics and the reference's bounds:
 (max|d| / rms, rms(d) / rms) < (5e-3, 5e-4) against the rounded oracle and < (2e-2, 3e-3) against
-the unrounded one (prefill_gemm_q.rs:288-343).  This tile feeds the MFMA the decoder's exact f16
-bits, so the first pair is held to (2e-5, 5e-6).
+the unrounded one (prefill_gemm_q.rs:288-343).  Every tile here feeds the MFMA exactly the
+specified f16 bits, so the first pair is held to (2e-5, 5e-6).
+
+The specified bits: `dequant_to_f16` for Q6_K, Q8_0 and for Q4_K under ACT_FLOAT_EXACT ("x4"
+below); for Q4_K under ACT_FLOAT the binary16 fma qa*q + qb of the reference's `gemm_mm_q4l`
+(crates/ojas-cuda/src/kernels/gemm_q.rs:104-140), oracle weight mode 2.
 """
 import numpy as np
 import pytest
@@ -14,10 +18,19 @@ from conftest import rms_errs
 
 pytestmark = pytest.mark.gpu
 Q8_0, Q4_K, Q6_K = 8, 12, 14
+X4 = "q4k-exact"   # Q4_K through the tile that holds dequant_to_f16 bits
 TIGHT = (2e-5, 5e-6)
 
 
+def _mode(pkg, ty):
+    """(GGUF type, act_mode, oracle weight mode) of a test case label."""
+    if ty == X4:
+        return Q4_K, pkg.ACT_FLOAT_EXACT, 1
+    return ty, pkg.ACT_FLOAT, 2 if ty == Q4_K else 1
+
+
 def _run(gpu, pkg, orc, ty, m, k, n, accum=False, x_dtype="f32", split=None):
+    ty, act, wmode = _mode(pkg, ty)
     w = pkg.synth.weights(ty, n, k, "gemm", ty, n, k)
     x = pkg.synth.normal_f32(m * k, "gemm", "x", m, k).reshape(m, k)
     if x_dtype == "bf16":
@@ -30,21 +43,22 @@ def _run(gpu, pkg, orc, ty, m, k, n, accum=False, x_dtype="f32", split=None):
     sent = np.full(n, 12345.5, np.float32)
     yd = gpu.upload(np.concatenate([y0.ravel(), sent]))
     lin = gpu.lin(ty, n, k, w)
-    gpu.mm(xd, lin, yd, m, accum, act_mode=pkg.ACT_FLOAT, x_dtype=pkg.X_BF16 if x_dtype == "bf16" else pkg.X_F32)
+    gpu.mm(xd, lin, yd, m, accum, act_mode=act, x_dtype=pkg.X_BF16 if x_dtype == "bf16" else pkg.X_F32)
     got = gpu.read(yd, m * n + n)
     assert np.all(got[m * n:] == 12345.5), "wrote past row M"
     got = got[:m * n].reshape(m, n)
-    want16 = orc.matmul_ref(w, ty, n, k, x, wmode=1, xmode=1) + y0
+    want16 = orc.matmul_ref(w, ty, n, k, x, wmode=wmode, xmode=1) + y0
     want32 = orc.matmul_ref(w, ty, n, k, x) + y0
     return rms_errs(got, want16), rms_errs(got, want32)
 
 
 # the reference's sweep: ragged M and N, accumulate, short and long K (prefill_gemm_q.rs:346-380)
 SWEEP = [(64, 256, 128, False), (33, 512, 130, False), (100, 1024, 200, True), (256, 4096, 256, False),
-         (300, 2048, 72, True), (512, 1024, 384, False), (77, 14336, 64, False)]
+         (300, 2048, 72, True), (512, 1024, 384, False), (77, 14336, 64, False), (129, 768, 513, False),
+         (700, 768, 300, True)]
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("ty", [Q4_K, X4, Q6_K, Q8_0])
 @pytest.mark.parametrize("m,k,n,accum", SWEEP)
 def test_gemm_sweep(gpu, orc, pkg, ty, m, k, n, accum):
     e16, e32 = _run(gpu, pkg, orc, ty, m, k, n, accum)
@@ -52,7 +66,7 @@ def test_gemm_sweep(gpu, orc, pkg, ty, m, k, n, accum):
     assert e32[0] < 2e-2 and e32[1] < 3e-3, (e32, "vs the unrounded oracle")
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q4_K, X4, Q6_K])
 def test_gemm_bf16_activations(gpu, orc, pkg, ty):
     """bf16 activations (the prefill / verify input type) convert to f16 exactly in range."""
     e16, e32 = _run(gpu, pkg, orc, ty, 128, 2048, 256, x_dtype="bf16")
@@ -60,11 +74,12 @@ def test_gemm_bf16_activations(gpu, orc, pkg, ty):
     assert e32[0] < 2e-2 and e32[1] < 3e-3, e32
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("ty", [Q4_K, X4, Q6_K, Q8_0])
 def test_tile_holds_the_reference_decoders_bits(gpu, orc, pkg, ty):
-    """One-hot activations read the tile back: y[m][n] must be dequant_to_f16(W)[n][m] exactly,
-    for every weight of two super-blocks per row and for extreme scales."""
+    """One-hot activations read the tile back: y[m][n] must be the specified f16 weight [n][m]
+    exactly, for every weight of two super-blocks per row and for extreme scales."""
     k, n = 512, 160
+    ty, act, wmode = _mode(pkg, ty)
     bb, wpb = pkg.synth.BLOCK_SHAPE[ty]
     raw = orc.synth_blocks(ty, n * k // wpb).reshape(-1, bb).copy()
     scales = np.array([0x0001, 0x03FF, 0x0400, 0x8001, 0xBC00, 0x3555, 0x1234, 0x2E66], np.uint16)
@@ -74,11 +89,12 @@ def test_tile_holds_the_reference_decoders_bits(gpu, orc, pkg, ty):
         if ty == Q4_K:
             raw[i, 2:4] = scales[(i * 3 + 1) % 8:(i * 3 + 1) % 8 + 1].view(np.uint8)
     raw = raw.reshape(-1)
-    want = orc.dequant_to_f16(raw, ty, n * k).view(np.float16).astype(np.float32).reshape(n, k)
+    bits = orc.q4l_weights_f16(raw, k, n) if wmode == 2 else orc.dequant_to_f16(raw, ty, n * k)
+    want = bits.view(np.float16).astype(np.float32).reshape(n, k)
     lin = gpu.lin(ty, n, k, raw)
     x = np.eye(k, dtype=np.float32)
     yd = gpu.alloc(k * n)
-    gpu.mm(gpu.upload(x), lin, yd, k, act_mode=pkg.ACT_FLOAT)
+    gpu.mm(gpu.upload(x), lin, yd, k, act_mode=act)
     got = gpu.read(yd, k * n).reshape(k, n)
     # value equality: a -0 weight reads back as +0 through the accumulator, every other bit must match
     assert np.array_equal(got, want.T)
@@ -86,27 +102,30 @@ def test_tile_holds_the_reference_decoders_bits(gpu, orc, pkg, ty):
     assert np.array_equal(got.view(np.uint32)[nz], want.T.copy().view(np.uint32)[nz])
 
 
-def test_split_k_entry_through_the_kernel_seam(gpu, orc, pkg):
-    """gemm_mm_q4k_sk dispatched by name with several K slices; y holds what is accumulated into."""
-    gpu.ensure_family("gemm")
+@pytest.mark.parametrize("kernel,family,bm,bn,wmode", [("gemm_mm_q4k_sk", "gemm", 256, 128, 1),
+                                                       ("gemm_mm_q4kl_sk", "gemm_xl", 256, 256, 2),
+                                                       ("gemm_mm_q4kl_m128_sk", "gemm_xl", 128, 256, 2)])
+def test_split_k_entry_through_the_kernel_seam(gpu, orc, pkg, kernel, family, bm, bn, wmode):
+    """Split-K entries dispatched by name with several K slices; y holds what is accumulated into."""
+    gpu.ensure_family(family)
     gpu.ensure_family("glue")
-    m, k, n = 40, 2048, 200
+    m, k, n = 140, 2048, 300
     w = pkg.synth.q4k_weights(n, k, "gemmsk", "w")
     x = pkg.synth.normal_f32(m * k, "gemmsk", "x").reshape(m, k)
     xh = gpu.upload_bytes(x.astype(np.float16))
     wd = gpu.upload_bytes(w)
-    want = orc.matmul_ref(w, Q4_K, n, k, x, wmode=1, xmode=1)
+    want = orc.matmul_ref(w, Q4_K, n, k, x, wmode=wmode, xmode=1)
     for nsplit in (1, 3, 8):
         y0 = pkg.synth.normal_f32(m * n, "gemmsk", "y0", nsplit).reshape(m, n)
         yd = gpu.upload(y0)
         enc = gpu.begin()
-        gpu.dispatch(enc, "gemm_mm_q4k_sk", [(xh, 0), (wd, 0), (yd, 0)], [k, n, m, nsplit],
-                     [(n + 127) // 128, (m + 255) // 256, nsplit], [256, 1, 1])
+        gpu.dispatch(enc, kernel, [(xh, 0), (wd, 0), (yd, 0)], [k, n, m, nsplit],
+                     [(n + bn - 1) // bn, (m + bm - 1) // bm, nsplit], [256, 1, 1])
         gpu.submit(enc)
         e = rms_errs(gpu.read(yd, m * n).reshape(m, n), want + y0)
         assert e[0] < 1e-4 and e[1] < 2e-5, (nsplit, e)
     with pytest.raises(pkg.OjasHipError, match="grid must be"):
-        gpu.dispatch(enc, "gemm_mm_q4k_sk", [(xh, 0), (wd, 0), (yd, 0)], [k, n, m, 2], [2, 1, 1], [256, 1, 1])
+        gpu.dispatch(enc, kernel, [(xh, 0), (wd, 0), (yd, 0)], [k, n, m, 2], [3, 1, 1], [256, 1, 1])
 
 
 def test_router_prefers_the_tile_only_above_the_crossover(gpu, orc, pkg):
@@ -124,5 +143,5 @@ def test_router_prefers_the_tile_only_above_the_crossover(gpu, orc, pkg):
             want = np.stack([orc.matvec_kq(w, Q4_K, n, k, x[t]) for t in range(m)])
             assert np.max(np.abs(got - want)) <= 2e-5 * np.max(np.abs(want))
         else:
-            e = rms_errs(got, orc.matmul_ref(w, Q4_K, n, k, x, wmode=1, xmode=1))
+            e = rms_errs(got, orc.matmul_ref(w, Q4_K, n, k, x, wmode=2, xmode=1))
             assert e[0] < TIGHT[0] and e[1] < TIGHT[1], e

@@ -247,6 +247,28 @@ def test_relayout_q4k_q4l(orc):
     assert np.array_equal(codes, exact)
 
 
+def test_q4l_kernel_weights_round_once(orc):
+    """ojo_q4l_weights_f16 = binary16(qa*q + qb) with ONE rounding (the half fma of
+    crates/ojas-cuda/src/kernels/gemm_q.rs:112-121), checked against numpy's correctly rounded
+    float64 -> float16 conversion of the exact value; a conversion through f32 first would
+    double-round and fail this on ties."""
+    n, k = 16, 1024
+    raw = orc.synth_blocks(Q4_K, n * k // 256)
+    nib, qa, qb = orc.relayout_q4k_q4l(raw, k, n)
+    codes = np.stack([nib & 15, nib >> 4], 1).reshape(n, k).astype(np.float64)
+    a = np.repeat(qa.view(np.float16).astype(np.float64), 32).reshape(n, k)
+    b = np.repeat(qb.view(np.float16).astype(np.float64), 32).reshape(n, k)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = (a * codes + b).astype(np.float16).reshape(-1)
+    got = orc.q4l_weights_f16(raw, k, n).view(np.float16)
+    ok = np.isfinite(want)
+    assert ok.sum() > 0.9 * want.size
+    assert np.array_equal(got.view(np.uint16)[ok], want.view(np.uint16)[ok])
+    # and against the dequantized tensor: one extra f16 rounding of each scale, nothing more
+    w = orc.dequant_to_f64(raw, Q4_K, n * k)
+    assert np.all(np.abs(got.astype(np.float64)[ok] - w[ok]) <= 2.0 ** -9 * (np.abs(a.reshape(-1)[ok]) * 15 + np.abs(b.reshape(-1)[ok])) + 1e-12)
+
+
 def test_moe_topk_matches_closed_form(orc, pkg):
     """crates/ojas-cuda/tests/conformance.rs:380-408: E=64, K=8, tvec(64, 51)."""
     lg = pkg.synth.tvec(64, 51)
