@@ -86,16 +86,24 @@ struct GxQ4K {
         half2v q = __builtin_bit_cast(half2v, bits) - k1024;
         return __builtin_bit_cast(uint, __builtin_elementwise_fma(q, a, c));
     }
+    // (x & 0x000F000F) | 0x64006400 in one instruction: two nibbles as the halves 1024 + q.
+    // (The mask travels in a scalar register, the magic in a vector register: a VOP3 instruction
+    // of this target reads one scalar operand.)
+    static __device__ __forceinline__ uint nib2h(uint x, uint magic) {
+        uint r;
+        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(0x000F000Fu), "v"(magic));
+        return r;
+    }
     // dword I (0..7) of the chunk: bytes 4I..4I+3 -> columns 4I..4I+3 (low) and 32+4I.. (high)
     template <int I>
-    __device__ __forceinline__ void part(uint (&lo)[2], uint (&hi)[2]) const {
+    __device__ __forceinline__ void part(uint (&lo)[2], uint (&hi)[2], uint magic) const {
         const uint v = I < 4 ? q0[I & 3] : q1[I & 3];
         const uint p0 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u);  // bytes (b0, 0, b1, 0)
         const uint p1 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u);  // bytes (b2, 0, b3, 0)
-        lo[0] = fma2((p0 & 0x000F000Fu) | 0x64006400u, a_lo, c_lo);
-        lo[1] = fma2((p1 & 0x000F000Fu) | 0x64006400u, a_lo, c_lo);
-        hi[0] = fma2(((p0 >> 4) & 0x000F000Fu) | 0x64006400u, a_hi, c_hi);
-        hi[1] = fma2(((p1 >> 4) & 0x000F000Fu) | 0x64006400u, a_hi, c_hi);
+        lo[0] = fma2(nib2h(p0, magic), a_lo, c_lo);
+        lo[1] = fma2(nib2h(p1, magic), a_lo, c_lo);
+        hi[0] = fma2(nib2h(p0 >> 4, magic), a_hi, c_hi);
+        hi[1] = fma2(nib2h(p1 >> 4, magic), a_hi, c_hi);
     }
 };
 
@@ -153,37 +161,35 @@ __device__ __forceinline__ void gemm_xl_body(const ushort* __restrict__ xh, cons
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     GxQ4K ld;
+    uint magic = 0x64006400u;
+    asm volatile("" : "+v"(magic));  // kept in a register: see nib2h
     const uchar* xbase = (const uchar*)xh;
     const uint last = nt - 1u;
 
 // Requests past the last slab are clamped onto it: every step is then the same straight-line
 // code (the surplus slab is fetched and dequantized into a stage nobody reads again).
-#define GX_LOAD_X(T)                                                                             \
+// copy I of the XL + 3 that bring in slab TX's activations (I < XL) and slab TW's raw weights
+#define GX_COPY(I, TX, TW)                                                                       \
     do {                                                                                         \
-        const uchar* b_ = xbase + (size_t)(k_begin + min((T), last) * GX_BK) * 2u;               \
-        const uint s_ = x_lds + ((T) & 1u) * XSTAGE;                                             \
-        _Pragma("unroll") for (int i_ = 0; i_ < XL; i_++) gx_load_lds16(b_, xoff[i_], s_ + i_ * 1024u); \
-    } while (0)
-#define GX_LOAD_W(T)                                                                             \
-    do {                                                                                         \
-        const uint k0_ = k_begin + min((T), last) * GX_BK;                                       \
-        const uchar* b_ = w + (size_t)(k0_ >> 8) * Q4K_BYTES;                                    \
-        const uchar* q_ = b_ + 16u + ((k0_ >> 6) & 3u) * 32u;                                    \
-        const uint s_ = raw_lds + ((T) & 1u) * GX_RAW;                                           \
-        gx_load_lds16(b_, wrow_off, s_);                                                         \
-        gx_load_lds16(q_, wrow_off, s_ + 4096u);                                                 \
-        gx_load_lds16(q_ + 16u, wrow_off, s_ + 8192u);                                           \
+        if ((I) < XL) {                                                                          \
+            const uchar* b_ = xbase + (size_t)(k_begin + min((TX), last) * GX_BK) * 2u;          \
+            gx_load_lds16(b_, xoff[(I) < XL ? (I) : 0], x_lds + ((TX) & 1u) * XSTAGE + (I) * 1024u); \
+        } else {                                                                                 \
+            const uint k0_ = k_begin + min((TW), last) * GX_BK;                                  \
+            const uchar* b_ = w + (size_t)(k0_ >> 8) * Q4K_BYTES;                                \
+            if ((I) > XL) b_ += ((k0_ >> 6) & 3u) * 32u + 16u * ((I) - XL);                      \
+            gx_load_lds16(b_, wrow_off, raw_lds + ((TW) & 1u) * GX_RAW + ((I) - XL) * 4096u);    \
+        }                                                                                        \
     } while (0)
 #define GX_READ_W(T) ld.read(raw_rd + ((T) & 1u) * GX_RAW, ((k_begin >> 6) + min((T), last)) & 3u)
-// dequantize dwords 2P, 2P+1 of the chunk and write slots P (low nibbles) and 4+P (high)
-#define GX_DEQ(LD, STG, P)                                                                       \
+// dequantize dword I of the chunk into OUT (two low-nibble, two high-nibble pairs)
+#define GX_PART(I, LO, HI) ld.template part<I>(LO, HI, magic)
+// write slots P (low nibbles) and 4+P (high) of the thread's row from the pairs of dwords 2P, 2P+1
+#define GX_PUT(STG, P, L0, H0, L1, H1)                                                           \
     do {                                                                                         \
-        uint l0_[2], h0_[2], l1_[2], h1_[2];                                                     \
-        LD.template part<2 * (P)>(l0_, h0_);                                                     \
-        LD.template part<2 * (P) + 1>(l1_, h1_);                                                 \
         uchar* r_ = w_lds + (STG) * GX_WSTAGE;                                                   \
-        *(u32x4*)(r_ + ((((uint)(P)) ^ wsw) << 4)) = (u32x4){l0_[0], l0_[1], l1_[0], l1_[1]};    \
-        *(u32x4*)(r_ + (((4u + (P)) ^ wsw) << 4)) = (u32x4){h0_[0], h0_[1], h1_[0], h1_[1]};     \
+        *(u32x4*)(r_ + ((((uint)(P)) ^ wsw) << 4)) = (u32x4){L0[0], L0[1], L1[0], L1[1]};        \
+        *(u32x4*)(r_ + (((4u + (P)) ^ wsw) << 4)) = (u32x4){H0[0], H0[1], H1[0], H1[1]};         \
     } while (0)
 #define GX_READ(STG, KS, AF, BF)                                                                 \
     do {                                                                                         \
@@ -193,63 +199,101 @@ __device__ __forceinline__ void gemm_xl_body(const ushort* __restrict__ xh, cons
         _Pragma("unroll") for (int i = 0; i < MI; i++) AF[i] = *(const half8*)(xa_ + i * 32u * GX_ROW); \
         _Pragma("unroll") for (int j = 0; j < 4; j++) BF[j] = *(const half8*)(wb_ + j * 32u * GX_ROW);  \
     } while (0)
+#define GX_MMA1(Q, AF, BF)                                                                       \
+    acc[(Q) >> 2][(Q) & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(AF[(Q) >> 2], BF[(Q) & 3], acc[(Q) >> 2][(Q) & 3], 0, 0, 0)
 #define GX_MMA(AF, BF)                                                                           \
     do {                                                                                         \
-        _Pragma("unroll") for (int i = 0; i < MI; i++)                                           \
-            _Pragma("unroll") for (int j = 0; j < 4; j++)                                        \
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(AF[i], BF[j], acc[i][j], 0, 0, 0); \
+        _Pragma("unroll") for (int q_ = 0; q_ < 4 * MI; q_++) GX_MMA1(q_, AF, BF);               \
     } while (0)
 // One K sub-step's worth of interleaving: 4 MI MFMAs.  The LDS reads (the next sub-step's
 // fragments) go out in pairs behind the first MFMAs so that their data is back long before the
-// sub-step ends; the dequantization's vector-ALU instructions fill the gaps after every MFMA; the
-// two LDS writes of the dequantized chunk come last.
-#define GX_MIX()                                                                                 \
+// sub-step ends; NV vector-ALU instructions of the dequantization follow every MFMA; the LDS
+// writes of the finished chunks come last.
+#define GX_MIX(NV, NW)                                                                           \
     do {                                                                                         \
         _Pragma("unroll") for (int g_ = 0; g_ < 4 * MI; g_++) {                                  \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                   \
             if (g_ < (MI + 4 + 1) / 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);        \
-            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                                   \
+            __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);                                  \
         }                                                                                        \
-        __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);                                       \
+        __builtin_amdgcn_sched_group_barrier(0x200, NW, 0);                                      \
     } while (0)
-// Step T: the raw weights of slab T+1 (landed during step T-1) come out of their staging slot,
-// the activations of slab T+1 and the raw weights of slab T+2 are requested, and slab T+1 is
-// dequantized between the MFMAs of slab T.  Everything requested has landed at the barrier.
+// Step T, entered with the fragments of its first K sub-step in afA / bfA and the raw weights of
+// slab T+1 unpacked in `ld`.  Sub-steps 0..2 carry the dequantization of slab T+1; then every
+// wave waits for its copies and meets the others (slab T+1 complete in LDS, slab T's stages
+// free); sub-step 3 — its fragments already in registers — covers what must follow the
+// barrier: the first fragments of slab T+1, the raw weights of slab T+2 out of their slot, and
+// the requests for slab T+2's activations and slab T+3's raw weights, one between two MFMAs.
 #define GX_STEP(T)                                                                               \
     do {                                                                                         \
         const uint cur_ = (T) & 1u, nxt_ = cur_ ^ 1u;                                            \
-        half8 afA[MI], bfA[4], afB[MI], bfB[4];                                                  \
-        GX_READ(cur_, 0, afA, bfA);                                                              \
-        GX_READ_W((T) + 1u);                                                                     \
-        GX_LOAD_X((T) + 1u);                                                                     \
-        GX_LOAD_W((T) + 2u);                                                                     \
-        ld.prep();                                                                               \
+        uint l0_[2], h0_[2], l1_[2], h1_[2], l2_[2], h2_[2];                                     \
         __builtin_amdgcn_sched_barrier(0);                                                       \
-        GX_READ(cur_, 1, afB, bfB); GX_MMA(afA, bfA); GX_DEQ(ld, nxt_, 0); GX_MIX();             \
-        GX_READ(cur_, 2, afA, bfA); GX_MMA(afB, bfB); GX_DEQ(ld, nxt_, 1); GX_MIX();             \
-        GX_READ(cur_, 3, afB, bfB); GX_MMA(afA, bfA); GX_DEQ(ld, nxt_, 2); GX_MIX();             \
-        GX_MMA(afB, bfB); GX_DEQ(ld, nxt_, 3); GX_MIX();                                         \
+        GX_READ(cur_, 1, afB, bfB); GX_MMA(afA, bfA);                                            \
+        GX_PART(0, l0_, h0_); GX_PART(1, l1_, h1_); GX_PUT(nxt_, 0, l0_, h0_, l1_, h1_); GX_PART(2, l2_, h2_); \
+        GX_MIX(5, 2);                                                                            \
+        GX_READ(cur_, 2, afA, bfA); GX_MMA(afB, bfB);                                            \
+        GX_PART(3, l0_, h0_); GX_PUT(nxt_, 1, l2_, h2_, l0_, h0_);                               \
+        GX_PART(4, l1_, h1_); GX_PART(5, l2_, h2_); GX_PUT(nxt_, 2, l1_, h1_, l2_, h2_);         \
+        GX_MIX(5, 4);                                                                            \
+        GX_READ(cur_, 3, afB, bfB); GX_MMA(afA, bfA);                                            \
+        GX_PART(6, l0_, h0_); GX_PART(7, l1_, h1_); GX_PUT(nxt_, 3, l0_, h0_, l1_, h1_);         \
+        GX_MIX(4, 2);                                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                       \
         gx_wait<0>();                                                                            \
         __syncthreads();                                                                         \
+        GX_READ(nxt_, 0, afA, bfA);                                                              \
+        GX_READ_W((T) + 2u);                                                                     \
+        GX_MMA1(0, afB, bfB);                                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+        _Pragma("unroll") for (int q_ = 1; q_ < 4 * MI; q_++) {                                  \
+            if (q_ - 1 < XL + 3) {                                                               \
+                GX_COPY(q_ - 1, (T) + 2u, (T) + 3u);                                             \
+                GX_MMA1(q_, afB, bfB);                                                           \
+                __builtin_amdgcn_sched_barrier(0);                                               \
+            } else {                                                                             \
+                GX_MMA1(q_, afB, bfB);                                                           \
+            }                                                                                    \
+        }                                                                                        \
+        if (XL + 3 > 4 * MI - 1) {                                                               \
+            _Pragma("unroll") for (int c_ = 4 * MI - 1; c_ < XL + 3; c_++) GX_COPY(c_, (T) + 2u, (T) + 3u); \
+        }                                                                                        \
+        ld.prep();                                                                               \
+        _Pragma("unroll") for (int g_ = 0; g_ < 4 * MI; g_++) {                                  \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                   \
+            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);                                  \
+        }                                                                                        \
     } while (0)
 
-    // prologue: slab 0 in place, the raw weights of slab 1 staged
-    GX_LOAD_X(0u);
-    GX_LOAD_W(0u);
-    GX_LOAD_W(1u);
+    // prologue: slab 0 in place; then the state a step expects on entry
+    half8 afA[MI], bfA[4], afB[MI], bfB[4];
+    _Pragma("unroll") for (int c_ = 0; c_ < XL + 3; c_++) GX_COPY(c_, 0u, 0u);
     gx_wait<0>();
     GX_READ_W(0u);
     ld.prep();
-    GX_DEQ(ld, 0u, 0); GX_DEQ(ld, 0u, 1); GX_DEQ(ld, 0u, 2); GX_DEQ(ld, 0u, 3);
+    {
+        uint l0_[2], h0_[2], l1_[2], h1_[2];
+        GX_PART(0, l0_, h0_); GX_PART(1, l1_, h1_); GX_PUT(0u, 0, l0_, h0_, l1_, h1_);
+        GX_PART(2, l0_, h0_); GX_PART(3, l1_, h1_); GX_PUT(0u, 1, l0_, h0_, l1_, h1_);
+        GX_PART(4, l0_, h0_); GX_PART(5, l1_, h1_); GX_PUT(0u, 2, l0_, h0_, l1_, h1_);
+        GX_PART(6, l0_, h0_); GX_PART(7, l1_, h1_); GX_PUT(0u, 3, l0_, h0_, l1_, h1_);
+    }
+    _Pragma("unroll") for (int c_ = XL; c_ < XL + 3; c_++) GX_COPY(c_, 0u, 1u);
+    gx_wait<0>();
     __syncthreads();
+    GX_READ(0u, 0, afA, bfA);
+    GX_READ_W(1u);
+    _Pragma("unroll") for (int c_ = 0; c_ < XL + 3; c_++) GX_COPY(c_, 1u, 2u);
+    ld.prep();
 
     for (uint t = 0; t < nt; t++) GX_STEP(t);
+    gx_wait<0>();
 #undef GX_READ_W
-#undef GX_LOAD_X
-#undef GX_LOAD_W
-#undef GX_DEQ
+#undef GX_COPY
+#undef GX_PART
+#undef GX_PUT
 #undef GX_READ
+#undef GX_MMA1
 #undef GX_MMA
 #undef GX_MIX
 #undef GX_STEP

@@ -261,7 +261,15 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
                              {n_el}, eg, block)))
             return rc;
         std::string base = std::string("gemm_mm_") + (w->type == OJH_Q8_0 ? "q8_0" : f->tag);
-        if (xl) base = m > 128 ? "gemm_mm_q4kl" : "gemm_mm_q4kl_m128";
+        if (xl) {
+            // 256-token tiles when they give every CU a tile, or half of them with a K long enough
+            // to split in two without the slices' fixed costs showing (measured on MI355X);
+            // 128-token tiles, which dequantize every weight for half as many MFMAs, otherwise.
+            uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;
+            uint32_t t256 = ((N + 255) / 256) * ((m + 255) / 256);
+            bool tall = m > 128 && (t256 >= cus || (2 * t256 >= cus && K >= 8192));
+            base = tall ? "gemm_mm_q4kl" : "gemm_mm_q4kl_m128";
+        }
         uint32_t sg[3], sb[3];
         if ((rc = ojh_launch_shape(dev, (base + "_sk").c_str(), K, N, m, sg, sb))) return rc;
         if (dev->gemm_split_override > 0) sg[2] = (uint32_t)dev->gemm_split_override;
