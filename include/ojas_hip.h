@@ -193,6 +193,18 @@ int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const
 int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, int count,
                      const ojh_lin *const *ws, ojh_buf *const *ys, const size_t *y_offs);
 
+/* The row-int8 representation of the reference's CPU models (`W::Q8`,
+ * crates/ojas-cpu/src/cpu_math.rs:14-23).  `ojh_q8rows_from_f16` is the load-time requantization
+ * `q8_rows_from_f16` (crates/ojas-formats/src/quant.rs:16-39): binary16 weights [n][k] -> int8
+ * [n][k] + one f32 scale per row.  `ojh_matmul_q8` is `matmul(w, xs, m)` (cpu_math.rs:187-289):
+ * every row of x (f32 [m][k]) quantized per whole vector (`quant_row_i8`, :174-179), integer
+ * dots, y[m][n] = bias + acc*sw*sx rounded operation by operation — bit-identical to the CPU
+ * path.  `bias` (f32[n]) may be NULL.  K must be a multiple of 16. */
+int ojh_q8rows_from_f16(ojh_device *dev, const ojh_buf *w16, size_t w_off, uint32_t n, uint32_t k,
+                        ojh_buf *q, ojh_buf *scale);
+int ojh_matmul_q8(ojh_device *dev, const ojh_buf *x, size_t x_off, const ojh_buf *wq, const ojh_buf *wscale,
+                  const ojh_buf *bias, ojh_buf *y, size_t y_off, uint32_t n, uint32_t k, uint32_t m);
+
 /* `dequant_to_f16` (crates/ojas-formats/src/gguf.rs:612-1116) on the device: `n_weights`
  * weights of `raw` -> binary16 bit patterns in `out`. Bit-exact with the reference. */
 int ojh_dequant_f16(ojh_device *dev, uint32_t ggml_type, const ojh_buf *raw, size_t raw_off,

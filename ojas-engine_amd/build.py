@@ -34,6 +34,7 @@ FAMILIES = {
     "gemm": ("gemm.hip", ["-ffp-contract=off"]),
     "gemm_xl": ("gemm_xl.hip", ["-ffp-contract=off"]),
     "moe": ("moe.hip", []),
+    "rowq8": ("rowq8.hip", ["-ffp-contract=off"]),
 }
 
 HOST_SOURCES = ["ojh_runtime.cpp", "ojh_manifest.cpp", "ojh_ops.cpp", "ojh_moe.cpp"]

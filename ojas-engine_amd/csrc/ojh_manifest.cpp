@@ -206,6 +206,48 @@ static int check_quantize(const ojh_kernel_spec *s, const uint32_t *c, const uin
     return OJH_OK;
 }
 
+// The row-int8 family; `rows_per_wave` selects the entry:
+//   0 rows_q8_from_f16(w16, q, scale, K, N)   1 quant_rows_i8(x, q, scale, K, M)       grid [rows,1,1]
+//   2 matmul_q8row(xq, sx, wq, sw, y, K, N, M)   3 matmul_q8row_bias(.., y, bs, K, N, M)  grid [ceil(N/4),1,1]
+static int check_rowq8(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                       const uint32_t block[3], size_t need[16], size_t align[16]) {
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    uint32_t K = c[0], R = c[1];
+    if (!K || !R) return ojh_fail(OJH_ERR_ARG, "%s: K and the row count must be positive", s->name);
+    if (s->rows_per_wave < 2) {
+        if (grid[0] != R) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,1,1]", s->name, R);
+        size_t esz = s->rows_per_wave == 0 ? 2 : 4;
+        need[0] = (size_t)R * K * esz;
+        need[1] = (size_t)R * K;
+        need[2] = (size_t)R * 4;
+        align[0] = esz;
+        align[1] = 1;
+        align[2] = 4;
+        return OJH_OK;
+    }
+    uint32_t N = R, M = c[2];
+    if (!M || K % 16) return ojh_fail(OJH_ERR_ARG, "%s: M must be positive and K=%u a multiple of 16", s->name, K);
+    if ((uint64_t)grid[0] * 4 < N) return ojh_fail(OJH_ERR_ARG, "%s: grid covers %u rows of N=%u", s->name, grid[0] * 4, N);
+    need[0] = (size_t)M * K;
+    need[1] = (size_t)M * 4;
+    need[2] = (size_t)N * K;
+    need[3] = (size_t)N * 4;
+    need[4] = (size_t)M * N * 4;
+    if (s->n_bufs == 6) need[5] = (size_t)N * 4;
+    align[1] = align[3] = align[4] = align[5] = 4;
+    return OJH_OK;
+}
+static int shape_rowq8(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t M,
+                       uint32_t grid[3], uint32_t block[3]) {
+    grid[0] = s->rows_per_wave == 0 ? N : s->rows_per_wave == 1 ? M : (N + 3) / 4;
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // dequant_<fmt>_f16(w, out, nblocks)
 static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                          const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -495,6 +537,10 @@ static std::vector<ojh_kernel_spec> build_manifest() {
             add(fq + "_wide", "gemv_q8k", 3, 3, f.type, 2, check_gemv_fq8k, shape_rows);
         }
     }
+    add("rows_q8_from_f16", "rowq8", 3, 2, 0, 0, check_rowq8, shape_rowq8);
+    add("quant_rows_i8", "rowq8", 3, 2, 0, 1, check_rowq8, shape_rowq8);
+    add("matmul_q8row", "rowq8", 5, 3, 0, 2, check_rowq8, shape_rowq8);
+    add("matmul_q8row_bias", "rowq8", 6, 3, 0, 3, check_rowq8, shape_rowq8);
     add("quantize_q8k", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     // prefill / verify MFMA tiles: "q8_0" is the reference's spelling for this family

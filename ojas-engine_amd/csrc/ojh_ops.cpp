@@ -336,3 +336,40 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     grid[0] = (N + 3) / 4;
     return ojh_launch(dev, (base + "_m").c_str(), {xp, wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, grid, block);
 }
+
+// ---- row-int8 path -------------------------------------------------------------------------------
+extern "C" int ojh_q8rows_from_f16(ojh_device *dev, const ojh_buf *w16, size_t w_off, uint32_t n, uint32_t k,
+                                   ojh_buf *q, ojh_buf *scale) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_q8rows_from_f16: NULL device");
+    if (!n || !k) return ojh_fail(OJH_ERR_ARG, "ojh_q8rows_from_f16: n=%u k=%u", n, k);
+    int rc;
+    if ((rc = span_ok("q8rows: w16", w16, w_off, (size_t)n * k * 2, 2))) return rc;
+    if ((rc = span_ok("q8rows: q", q, 0, (size_t)n * k, 16))) return rc;
+    if ((rc = span_ok("q8rows: scale", scale, 0, (size_t)n * 4, 4))) return rc;
+    if ((rc = ensure(dev, "rowq8"))) return rc;
+    uint32_t grid[3] = {n, 1, 1}, block[3] = {256, 1, 1};
+    return ojh_launch(dev, "rows_q8_from_f16", {at(w16, w_off), q->ptr, scale->ptr}, {k, n}, grid, block);
+}
+
+extern "C" int ojh_matmul_q8(ojh_device *dev, const ojh_buf *x, size_t x_off, const ojh_buf *wq, const ojh_buf *wscale,
+                             const ojh_buf *bias, ojh_buf *y, size_t y_off, uint32_t n, uint32_t k, uint32_t m) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_matmul_q8: NULL device");
+    if (!n || !k || !m || m > 65535) return ojh_fail(OJH_ERR_ARG, "ojh_matmul_q8: n=%u k=%u m=%u out of range", n, k, m);
+    if (k % 16) return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_matmul_q8: K=%u must be a multiple of 16", k);
+    int rc;
+    if ((rc = span_ok("matmul_q8: x", x, x_off, (size_t)m * k * 4, 4))) return rc;
+    if ((rc = span_ok("matmul_q8: wq", wq, 0, (size_t)n * k, 16))) return rc;
+    if ((rc = span_ok("matmul_q8: wscale", wscale, 0, (size_t)n * 4, 4))) return rc;
+    if (bias && (rc = span_ok("matmul_q8: bias", bias, 0, (size_t)n * 4, 4))) return rc;
+    if ((rc = span_ok("matmul_q8: y", y, y_off, (size_t)m * n * 4, 4))) return rc;
+    if ((rc = ensure(dev, "rowq8"))) return rc;
+    ojh_buf *xq, *sx;
+    if ((rc = ojh_scratch_get(dev, "q8_xq", (size_t)m * k, &xq))) return rc;
+    if ((rc = ojh_scratch_get(dev, "q8_sx", (size_t)m * 4, &sx))) return rc;
+    uint32_t block[3] = {256, 1, 1}, gq[3] = {m, 1, 1}, gm[3] = {(n + 3) / 4, 1, 1};
+    if ((rc = ojh_launch(dev, "quant_rows_i8", {at(x, x_off), xq->ptr, sx->ptr}, {k, m}, gq, block))) return rc;
+    if (bias)
+        return ojh_launch(dev, "matmul_q8row_bias", {xq->ptr, sx->ptr, wq->ptr, wscale->ptr, at(y, y_off), bias->ptr},
+                          {k, n, m}, gm, block);
+    return ojh_launch(dev, "matmul_q8row", {xq->ptr, sx->ptr, wq->ptr, wscale->ptr, at(y, y_off)}, {k, n, m}, gm, block);
+}

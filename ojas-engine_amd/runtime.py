@@ -104,6 +104,8 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_mm": (i32, [vp, vp, sz, i32, vp, vp, sz, vp, u32, i32, i32]),
         "ojh_mm_q8k": (i32, [vp, vp, vp, vp, vp, sz, vp, u32, i32]),
         "ojh_mm_q8k_multi": (i32, [vp, vp, vp, i32, vp, vp, vp]),
+        "ojh_q8rows_from_f16": (i32, [vp, vp, sz, u32, u32, vp, vp]),
+        "ojh_matmul_q8": (i32, [vp, vp, sz, vp, vp, vp, vp, sz, u32, u32, u32]),
         "ojh_capture_begin": (i32, [vp]),
         "ojh_capture_end": (i32, [vp, pp]),
         "ojh_graph_launch": (i32, [vp, vp]),
@@ -365,6 +367,16 @@ class HipGpu:
         ya = (C.c_void_p * n)(*[y.handle for y in ys])
         oa = (C.c_size_t * n)(*y_offs) if y_offs is not None else None
         self._check(self._L.ojh_mm_q8k_multi(self._dev, xq.handle, xscales.handle, n, wa, ya, oa))
+
+    def q8rows_from_f16(self, w16: Buf, n: int, k: int, q: Buf, scale: Buf, w_off: int = 0) -> None:
+        """Load-time requantization of f16 weights [n][k] to int8 rows + per-row f32 scales."""
+        self._check(self._L.ojh_q8rows_from_f16(self._dev, w16.handle, w_off, n, k, q.handle, scale.handle))
+
+    def matmul_q8(self, x: Buf, wq: Buf, wscale: Buf, y: Buf, n: int, k: int, m: int = 1, *,
+                  bias: Buf | None = None, x_off: int = 0, y_off: int = 0) -> None:
+        """The CPU models' row-int8 matmul: y[m][n] = bias + (qx . qw) * sw * sx."""
+        self._check(self._L.ojh_matmul_q8(self._dev, x.handle, x_off, wq.handle, wscale.handle,
+                                          bias.handle if bias else None, y.handle, y_off, n, k, m))
 
     def capture_begin(self) -> None:
         """Start recording dispatches on the device's stream instead of running them."""
