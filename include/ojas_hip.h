@@ -193,6 +193,13 @@ int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const
 int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, int count,
                      const ojh_lin *const *ws, ojh_buf *const *ys, const size_t *y_offs);
 
+/* `relayout_q4k_q4l` (crates/ojas-formats/src/quant.rs:192-222) on the device: n rows of k Q4_K
+ * weights -> nibble pairs `nib` [n*k/2], f16 `qa` = d*sc and `qb` = -dmin*m per 32 weights
+ * [n*k/32 each].  Bit-exact with the reference.  The library's own prefill GEMM does not need
+ * it (it forms qa / qb in the tile from the raw blocks); it serves callers that keep Q4L. */
+int ojh_relayout_q4k_q4l(ojh_device *dev, const ojh_buf *raw, size_t raw_off, uint32_t n, uint32_t k,
+                         ojh_buf *nib, ojh_buf *qa, ojh_buf *qb);
+
 /* The row-int8 representation of the reference's CPU models (`W::Q8`,
  * crates/ojas-cpu/src/cpu_math.rs:14-23).  `ojh_q8rows_from_f16` is the load-time requantization
  * `q8_rows_from_f16` (crates/ojas-formats/src/quant.rs:16-39): binary16 weights [n][k] -> int8

@@ -112,3 +112,36 @@ dequant_q6k_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblo
     o[64] = f32_to_f16_bits(__fmul_rn(__fmul_rn(d, (float)sc[is + 4]), (float)q3));
     o[96] = f32_to_f16_bits(__fmul_rn(__fmul_rn(d, (float)sc[is + 6]), (float)q4));
 }
+
+// relayout_q4k_q4l(w, nib, qa, qb, nblocks): Q4_K super-blocks -> the Q4L side arrays of the
+// reference's prefill GEMM (crates/ojas-formats/src/quant.rs:192-222): per 32-weight block j of
+// a super-block, qa = f16(d*sc_j), qb = f16(-dmin*m_j), and 16 bytes holding weights (2i, 2i+1)
+// of the block as (low, high) nibble.  Rows are whole super-blocks, so the arrays are indexed
+// by the running super-block number.  One thread per 32-weight block.
+extern "C" __global__ void __launch_bounds__(256)
+relayout_q4k_q4l(const uchar* __restrict__ w, uchar* __restrict__ nib, ushort* __restrict__ qa,
+                 ushort* __restrict__ qb, uint nblocks) {
+    size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x;
+    size_t b = tid >> 3;
+    if (b >= nblocks) return;
+    const uint j = (uint)tid & 7u, c = j >> 1, hi = j & 1u;
+    const uchar* blk = w + b * Q4K_BYTES;
+    const uint* hdr = (const uint*)blk;
+    const uint dd = hdr[0];
+    const float d = f16_bits_to_f32(dd & 0xFFFFu), ndm = -f16_bits_to_f32(dd >> 16);
+    uint sc, mn;
+    q4k_scale_min_pair(hdr[1], hdr[2], hdr[3], c, sc, mn);
+    const uint s_ = hi ? sc >> 8 : sc & 0xFFu, m_ = hi ? mn >> 8 : mn & 0xFFu;
+    qa[tid] = f32_to_f16_bits(__fmul_rn(d, (float)s_));
+    qb[tid] = f32_to_f16_bits(__fmul_rn(ndm, (float)m_));
+    const uint* qq = hdr + 4 + c * 8u;   // the chunk's 32 bytes
+    uint out[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {        // 8 source bytes -> 4 packed bytes
+        uint a = qq[2 * i] >> (4u * hi), e = qq[2 * i + 1] >> (4u * hi);
+        uint p0 = (a & 0xFu) | (((a >> 8) & 0xFu) << 4), p1 = ((a >> 16) & 0xFu) | (((a >> 24) & 0xFu) << 4);
+        uint p2 = (e & 0xFu) | (((e >> 8) & 0xFu) << 4), p3 = ((e >> 16) & 0xFu) | (((e >> 24) & 0xFu) << 4);
+        out[i] = p0 | (p1 << 8) | (p2 << 16) | (p3 << 24);
+    }
+    *(uint4*)(nib + tid * 16u) = make_uint4(out[0], out[1], out[2], out[3]);
+}

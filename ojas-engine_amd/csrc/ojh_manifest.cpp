@@ -248,6 +248,30 @@ static int shape_rowq8(const ojh_kernel_spec *s, const ojh_device *, uint32_t, u
     return OJH_OK;
 }
 
+// relayout_q4k_q4l(w, nib, qa, qb, nblocks): 8 threads per super-block
+static int check_relayout(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                          const uint32_t block[3], size_t need[16], size_t align[16]) {
+    uint32_t nb = c[0];
+    if (!nb || nb > 0x0FFFFFFFu) return ojh_fail(OJH_ERR_ARG, "%s: nblocks=%u out of range", s->name, nb);
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * 32 < nb)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must cover %u super-blocks, 32 per workgroup", s->name, nb);
+    need[0] = (size_t)nb * 144;
+    need[1] = (size_t)nb * 128;
+    need[2] = need[3] = (size_t)nb * 16;
+    align[2] = align[3] = 2;
+    return OJH_OK;
+}
+static int shape_relayout(const ojh_kernel_spec *, const ojh_device *, uint32_t, uint32_t N, uint32_t,
+                          uint32_t grid[3], uint32_t block[3]) {
+    grid[0] = (N + 31) / 32;  // N = super-blocks
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // dequant_<fmt>_f16(w, out, nblocks)
 static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                          const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -537,6 +561,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
             add(fq + "_wide", "gemv_q8k", 3, 3, f.type, 2, check_gemv_fq8k, shape_rows);
         }
     }
+    add("relayout_q4k_q4l", "dequant", 4, 1, OJH_Q4_K, 0, check_relayout, shape_relayout);
     add("rows_q8_from_f16", "rowq8", 3, 2, 0, 0, check_rowq8, shape_rowq8);
     add("quant_rows_i8", "rowq8", 3, 2, 0, 1, check_rowq8, shape_rowq8);
     add("matmul_q8row", "rowq8", 5, 3, 0, 2, check_rowq8, shape_rowq8);

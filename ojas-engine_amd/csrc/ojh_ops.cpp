@@ -95,6 +95,22 @@ extern "C" int ojh_dequant_f16(ojh_device *dev, uint32_t type, const ojh_buf *ra
     return ojh_launch(dev, name.c_str(), {at(raw, raw_off), at(out, out_off)}, {(uint32_t)nb}, grid, block);
 }
 
+extern "C" int ojh_relayout_q4k_q4l(ojh_device *dev, const ojh_buf *raw, size_t raw_off, uint32_t n, uint32_t k,
+                                    ojh_buf *nib, ojh_buf *qa, ojh_buf *qb) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_relayout_q4k_q4l: NULL device");
+    if (!n || !k || k % 256) return ojh_fail(OJH_ERR_ARG, "relayout_q4k_q4l: %u rows of %u weights (K must be a multiple of 256)", n, k);
+    size_t nb = (size_t)n * (k / 256);
+    if (nb > 0x0FFFFFFFu) return ojh_fail(OJH_ERR_ARG, "relayout_q4k_q4l: too many super-blocks (%zu)", nb);
+    int rc;
+    if ((rc = span_ok("relayout: raw", raw, raw_off, nb * 144, 16))) return rc;
+    if ((rc = span_ok("relayout: nib", nib, 0, nb * 128, 16))) return rc;
+    if ((rc = span_ok("relayout: qa", qa, 0, nb * 16, 2))) return rc;
+    if ((rc = span_ok("relayout: qb", qb, 0, nb * 16, 2))) return rc;
+    if ((rc = ensure(dev, "dequant"))) return rc;
+    uint32_t grid[3] = {(uint32_t)((nb + 31) / 32), 1, 1}, block[3] = {256, 1, 1};
+    return ojh_launch(dev, "relayout_q4k_q4l", {at(raw, raw_off), nib->ptr, qa->ptr, qb->ptr}, {(uint32_t)nb}, grid, block);
+}
+
 // ---- activation quantizer ----------------------------------------------------------------------
 static int quant_q8k_launch(ojh_device *dev, const void *x, int x_dtype, uint32_t m, uint32_t k, void *q,
                             void *scales) {

@@ -104,6 +104,7 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_mm": (i32, [vp, vp, sz, i32, vp, vp, sz, vp, u32, i32, i32]),
         "ojh_mm_q8k": (i32, [vp, vp, vp, vp, vp, sz, vp, u32, i32]),
         "ojh_mm_q8k_multi": (i32, [vp, vp, vp, i32, vp, vp, vp]),
+        "ojh_relayout_q4k_q4l": (i32, [vp, vp, sz, u32, u32, vp, vp, vp]),
         "ojh_q8rows_from_f16": (i32, [vp, vp, sz, u32, u32, vp, vp]),
         "ojh_matmul_q8": (i32, [vp, vp, sz, vp, vp, vp, vp, sz, u32, u32, u32]),
         "ojh_capture_begin": (i32, [vp]),
@@ -367,6 +368,10 @@ class HipGpu:
         ya = (C.c_void_p * n)(*[y.handle for y in ys])
         oa = (C.c_size_t * n)(*y_offs) if y_offs is not None else None
         self._check(self._L.ojh_mm_q8k_multi(self._dev, xq.handle, xscales.handle, n, wa, ya, oa))
+
+    def relayout_q4k_q4l(self, raw: Buf, n: int, k: int, nib: Buf, qa: Buf, qb: Buf, raw_off: int = 0) -> None:
+        """Q4_K blocks -> the Q4L arrays (nibble pairs, f16 qa / qb per 32 weights)."""
+        self._check(self._L.ojh_relayout_q4k_q4l(self._dev, raw.handle, raw_off, n, k, nib.handle, qa.handle, qb.handle))
 
     def q8rows_from_f16(self, w16: Buf, n: int, k: int, q: Buf, scale: Buf, w_off: int = 0) -> None:
         """Load-time requantization of f16 weights [n][k] to int8 rows + per-row f32 scales."""

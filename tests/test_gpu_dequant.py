@@ -64,3 +64,21 @@ def test_dequant_through_the_kernel_seam(gpu, orc):
     bits = gpu.read(out, 24 * 256 + 16, np.uint16)
     assert np.all(bits[:8] == 0x7777) and np.all(bits[-8:] == 0x7777)
     assert np.array_equal(bits[8:-8], orc.dequant_to_f16(raw, Q4_K, 24 * 256))
+
+
+def test_relayout_q4k_q4l_is_bit_exact(gpu, orc, pkg):
+    """crates/ojas-formats/src/quant.rs:192-222 on the device: nibble pairs, qa, qb all equal to the
+    CPU restatement (which the oracle tests pin against the decoder), including extreme scales."""
+    n, k = 37, 1024
+    raw = orc.synth_blocks(12, n * k // 256).reshape(-1, 144).copy()
+    probes = np.array([0x0001, 0x03FF, 0x0400, 0x8001, 0xBC00, 0x3555, 0x7BFF, 0x0000], np.uint16)
+    for i in range(raw.shape[0]):
+        raw[i, 0:2] = probes[i % 8:i % 8 + 1].view(np.uint8)
+        raw[i, 2:4] = probes[(3 * i + 1) % 8:(3 * i + 1) % 8 + 1].view(np.uint8)
+    raw = raw.reshape(-1)
+    nib, qa, qb = gpu.alloc_bytes(n * k // 2), gpu.alloc_bytes(n * k // 16), gpu.alloc_bytes(n * k // 16)
+    gpu.relayout_q4k_q4l(gpu.upload_bytes(raw), n, k, nib, qa, qb)
+    wn, wa, wb = orc.relayout_q4k_q4l(raw, k, n)
+    assert np.array_equal(gpu.read(nib, n * k // 2, np.uint8), wn)
+    assert np.array_equal(gpu.read(qa, n * k // 32, np.uint16), wa)
+    assert np.array_equal(gpu.read(qb, n * k // 32, np.uint16), wb)
