@@ -440,15 +440,14 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, u
     return OJH_OK;
 }
 
-// copy_*(x, y, n) / fill_zero_u32(y, n): one thread per element
+// copy_*(x, y, n) / fill_zero_u32(y, n): grid-stride, any positive grid of 256-thread blocks
 static int check_elementwise(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                              const uint32_t block[3], size_t need[16], size_t align[16]) {
     uint32_t n = c[0];
     if (!n) return ojh_fail(OJH_ERR_ARG, "%s: n must be positive", s->name);
     int rc = check_block(block, 256);
     if (rc) return rc;
-    if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * 256 < n)
-        return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover %u elements", s->name, n);
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
     if (s->n_bufs == 1) {
         need[0] = (size_t)n * (s->type & 0xFF);
         align[0] = 4;
@@ -478,7 +477,8 @@ static int check_stream(const ojh_kernel_spec *s, const uint32_t *c, const uint3
 // ---- launch shapes ---------------------------------------------------------------------------
 static int shape_elementwise(const ojh_kernel_spec *, const ojh_device *, uint32_t, uint32_t N, uint32_t,
                              uint32_t grid[3], uint32_t block[3]) {
-    grid[0] = (N + 255) / 256;  // N = element count
+    grid[0] = (N / 8 + 255) / 256;  // N = element count; a thread takes 8 elements per trip
+    if (!grid[0]) grid[0] = 1;
     grid[1] = grid[2] = 1;
     block[0] = 256;
     block[1] = block[2] = 1;

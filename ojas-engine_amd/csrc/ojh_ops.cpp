@@ -272,7 +272,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         if ((rc = ensure(dev, "glue")) || (rc = ensure(dev, xl ? "gemm_xl" : "gemm"))) return rc;
         ojh_buf *xh;
         if ((rc = ojh_scratch_get(dev, "xh", (size_t)m * K * 2, &xh))) return rc;
-        uint32_t n_el = m * K, eg[3] = {(n_el + 255) / 256, 1, 1};
+        uint32_t n_el = m * K, eg[3] = {(n_el / 8 + 255) / 256 + 1, 1, 1};
         if ((rc = ojh_launch(dev, x_dtype == OJH_X_BF16 ? "copy_bf16_half" : "copy_f32_half", {at(x, x_off), xh->ptr},
                              {n_el}, eg, block)))
             return rc;
@@ -291,7 +291,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         if (dev->gemm_split_override > 0) sg[2] = (uint32_t)dev->gemm_split_override;
         if (sg[2] > 1) {
             if (!accum) {
-                uint32_t n_y = m * N, zg[3] = {(n_y + 255) / 256, 1, 1};
+                uint32_t n_y = m * N, zg[3] = {(n_y / 4 + 255) / 256 + 1, 1, 1};
                 if ((rc = ojh_launch(dev, "fill_zero_u32", {yp}, {n_y}, zg, block))) return rc;
             }
             return ojh_launch(dev, (base + "_sk").c_str(), {xh->ptr, wp, yp}, {K, N, m, sg[2]}, sg, sb);
@@ -335,7 +335,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         if ((rc = ensure(dev, "glue"))) return rc;
         ojh_buf *xf;
         if ((rc = ojh_scratch_get(dev, "xf", (size_t)m * K * 4, &xf))) return rc;
-        uint32_t n_el = m * K, eg[3] = {(n_el + 255) / 256, 1, 1};
+        uint32_t n_el = m * K, eg[3] = {(n_el / 8 + 255) / 256 + 1, 1, 1};
         if ((rc = ojh_launch(dev, "copy_bf16_f32", {xp, xf->ptr}, {n_el}, eg, block))) return rc;
         xp = xf->ptr;
     }
