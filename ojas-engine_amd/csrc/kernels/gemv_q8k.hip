@@ -329,61 +329,81 @@ gemv_q8k_q4k_m(const signed char* xq, const float* xs, const uchar* w, float* y,
 }
 
 // ------------------------------------------------------------------ Q6_K
-// Sixteen lanes share a super-block and a wave walks four per step.  Lane (g, t) = (lane/16,
-// lane%16) owns, in half hf = t/8, the four weights l0..l0+3 (l0 = 4*(t%8)) of each of the four
-// quarters: three dwords (two of ql, one of qh) give 16 six-bit codes, each quarter under one
-// int8 sub-scale sc[2q + l0/16].
-struct Q6kFrag {
-    uint x[4];   // 4 int8 activations per quarter
-    int xs[4];   // their sums (for the -32 offset of the codes)
+// Four lanes share a super-block and a wave walks sixteen per step.  Lane u = lane % 4 owns, in
+// half hf = u / 2, the sixteen positions l0..l0+15 (l0 = 16 (u % 2)) of each of the four
+// quarters: three 16-byte loads (two of ql, one of qh) give 64 six-bit codes, each quarter
+// under one int8 sub-scale sc[8 hf + 2 q + u % 2].
+struct Q6kX {          // a lane's share of the activations of one super-block
+    uint4 x[4];        // 16 int8 per quarter
+    int xs[4];         // their sums (for the -32 offset of the codes)
     float sx;
 };
 
-__device__ __forceinline__ Q6kFrag q6k_load_frag(const signed char* xq, const float* xs, uint sb, uint hf, uint l0) {
-    Q6kFrag f;
+__device__ __forceinline__ Q6kX q6k_load_x(const signed char* xq, const float* xs, uint sb, uint hf, uint l0) {
+    Q6kX f;
     const signed char* p = xq + (size_t)sb * 256u + hf * 128u + l0;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        f.x[q] = *(const uint*)(p + 32 * q);
-        f.xs[q] = dot4_i8(f.x[q], 0x01010101u, 0);
+        f.x[q] = *(const uint4*)(p + 32 * q);
+        int t = dot4_i8(f.x[q].x, 0x01010101u, 0);
+        t = dot4_i8(f.x[q].y, 0x01010101u, t);
+        t = dot4_i8(f.x[q].z, 0x01010101u, t);
+        f.xs[q] = dot4_i8(f.x[q].w, 0x01010101u, t);
     }
     f.sx = xs[sb];
     return f;
 }
 
-struct Q6kRaw {
-    uint qa, qb, qh;  // ql[l0..], ql[32+l0..], qh[l0..]
-    uint sc4;         // the lane's four sub-scales, one per byte
+struct Q6kW {          // a lane's share of one super-block of one row
+    u32x4_a2 qa, qb, qh;  // ql[l0..], ql[32 + l0..], qh[l0..] of the lane's half
+    uint sc4;          // the four sub-scales, one per byte
     uint d16;
 };
 
-__device__ __forceinline__ Q6kRaw q6k_load_raw(const uchar* blk, uint hf, uint l0) {
-    Q6kRaw r;
-    r.qa = *(const u32_a2*)(blk + hf * 64u + l0);
-    r.qb = *(const u32_a2*)(blk + hf * 64u + 32u + l0);
-    r.qh = *(const u32_a2*)(blk + 128u + hf * 32u + l0);
+__device__ __forceinline__ Q6kW q6k_load_w(const uchar* blk, uint hf, uint l0) {
+    Q6kW r;
+    r.qa = *(const u32x4_a2*)(blk + hf * 64u + l0);
+    r.qb = *(const u32x4_a2*)(blk + hf * 64u + 32u + l0);
+    r.qh = *(const u32x4_a2*)(blk + 128u + hf * 32u + l0);
     u32x2_a2 s = *(const u32x2_a2*)(blk + 192u + hf * 8u);
-    // bytes is, is+2, is+4, is+6 of the 8 sub-scales -> one per byte of sc4
-    uint is = l0 >> 4;
-    uint a = s.x >> (8u * is), b = s.y >> (8u * is);
+    // bytes is, is+2, is+4, is+6 of the half's 8 sub-scales -> one per byte of sc4
+    const uint is = l0 >> 4;
+    const uint a = s.x >> (8u * is), b = s.y >> (8u * is);
     r.sc4 = (a & 0xFFu) | ((a >> 8) & 0xFF00u) | ((b & 0xFFu) << 16) | ((b << 8) & 0xFF000000u);
     r.d16 = *(const ushort*)(blk + 208u);
     return r;
 }
 
-__device__ __forceinline__ float q6k_lane_dot(const Q6kRaw& r, const Q6kFrag& f) {
+// the 16 codes (0..63) of quarter Q as four dwords
+template <int Q>
+__device__ __forceinline__ void q6k_codes(const Q6kW& r, uint (&w)[4]) {
     const uint M4 = 0x0F0F0F0Fu, H2 = 0x30303030u;
-    uint w0 = (r.qa & M4) | ((r.qh << 4) & H2);
-    uint w1 = (r.qb & M4) | ((r.qh << 2) & H2);
-    uint w2 = ((r.qa >> 4) & M4) | (r.qh & H2);
-    uint w3 = ((r.qb >> 4) & M4) | ((r.qh >> 2) & H2);
-    int i0 = dot4_i8(w0, f.x[0], 0) - 32 * f.xs[0];
-    int i1 = dot4_i8(w1, f.x[1], 0) - 32 * f.xs[1];
-    int i2 = dot4_i8(w2, f.x[2], 0) - 32 * f.xs[2];
-    int i3 = dot4_i8(w3, f.x[3], 0) - 32 * f.xs[3];
-    int s0 = (int)(signed char)(r.sc4), s1 = (int)(signed char)(r.sc4 >> 8);
-    int s2 = (int)(signed char)(r.sc4 >> 16), s3 = (int)r.sc4 >> 24;
-    int isum = s0 * i0 + s1 * i1 + s2 * i2 + s3 * i3;
+    const uint ql[4] = {Q & 1 ? r.qb.x : r.qa.x, Q & 1 ? r.qb.y : r.qa.y, Q & 1 ? r.qb.z : r.qa.z, Q & 1 ? r.qb.w : r.qa.w};
+    const uint qh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint lo = Q < 2 ? ql[j] & M4 : (ql[j] >> 4) & M4;
+        const uint hi = Q == 0 ? (qh[j] << 4) & H2 : Q == 1 ? (qh[j] << 2) & H2 : Q == 2 ? qh[j] & H2 : (qh[j] >> 2) & H2;
+        w[j] = lo | hi;
+    }
+}
+
+__device__ __forceinline__ int dot16(const uint (&w)[4], const uint4& x) {
+    int t = dot4_i8(w[0], x.x, 0);
+    t = dot4_i8(w[1], x.y, t);
+    t = dot4_i8(w[2], x.z, t);
+    return dot4_i8(w[3], x.w, t);
+}
+
+__device__ __forceinline__ float q6k_lane_dot(const Q6kW& r, const Q6kX& f) {
+    uint w[4];
+    q6k_codes<0>(r, w); const int i0 = dot16(w, f.x[0]) - 32 * f.xs[0];
+    q6k_codes<1>(r, w); const int i1 = dot16(w, f.x[1]) - 32 * f.xs[1];
+    q6k_codes<2>(r, w); const int i2 = dot16(w, f.x[2]) - 32 * f.xs[2];
+    q6k_codes<3>(r, w); const int i3 = dot16(w, f.x[3]) - 32 * f.xs[3];
+    const int s0 = (int)(signed char)(r.sc4), s1 = (int)(signed char)(r.sc4 >> 8);
+    const int s2 = (int)(signed char)(r.sc4 >> 16), s3 = (int)r.sc4 >> 24;
+    const int isum = s0 * i0 + s1 * i1 + s2 * i2 + s3 * i3;
     return f.sx * f16_bits_to_f32(r.d16) * (float)isum;
 }
 
@@ -394,18 +414,18 @@ __device__ __forceinline__ void gemv_q8k_q6k_body(const signed char* __restrict_
     const uint lane = threadIdx.x & 63u;
     const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
     if (row0 >= N) return;
-    const uint nsb = K >> 8, g = lane >> 4, t = lane & 15u, hf = t >> 3, l0 = (t & 7u) * 4u;
+    const uint nsb = K >> 8, g = lane >> 2, hf = (lane >> 1) & 1u, l0 = (lane & 1u) * 16u;
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.0f;
-    for (uint sb = g; sb < nsb; sb += 4u) {
-        Q6kRaw raw[R];
+    for (uint sb = g; sb < nsb; sb += 16u) {
+        Q6kW raw[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
             uint row = min(row0 + r, N - 1u);
-            raw[r] = q6k_load_raw(w + ((size_t)row * nsb + sb) * Q6K_BYTES, hf, l0);
+            raw[r] = q6k_load_w(w + ((size_t)row * nsb + sb) * Q6K_BYTES, hf, l0);
         }
-        Q6kFrag f = q6k_load_frag(xq, xs, sb, hf, l0);
+        Q6kX f = q6k_load_x(xq, xs, sb, hf, l0);
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] += q6k_lane_dot(raw[r], f);
     }
@@ -425,17 +445,17 @@ __device__ __forceinline__ void gemv_q8k_q6k_m_body(const signed char* __restric
     const uint lane = threadIdx.x & 63u;
     const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= N) return;
-    const uint nsb = K >> 8, g = lane >> 4, t = lane & 15u, hf = t >> 3, l0 = (t & 7u) * 4u;
+    const uint nsb = K >> 8, g = lane >> 2, hf = (lane >> 1) & 1u, l0 = (lane & 1u) * 16u;
     for (uint m0 = 0; m0 < M; m0 += MT) {
         float acc[MT];
 #pragma unroll
         for (int i = 0; i < MT; i++) acc[i] = 0.0f;
-        for (uint sb = g; sb < nsb; sb += 4u) {
-            Q6kRaw raw = q6k_load_raw(w + ((size_t)row * nsb + sb) * Q6K_BYTES, hf, l0);
+        for (uint sb = g; sb < nsb; sb += 16u) {
+            Q6kW raw = q6k_load_w(w + ((size_t)row * nsb + sb) * Q6K_BYTES, hf, l0);
 #pragma unroll
             for (int i = 0; i < MT; i++) {
                 uint m = min(m0 + i, M - 1u);
-                Q6kFrag f = q6k_load_frag(xq + (size_t)m * nsb * 256u, xs + (size_t)m * nsb, sb, hf, l0);
+                Q6kX f = q6k_load_x(xq + (size_t)m * nsb * 256u, xs + (size_t)m * nsb, sb, hf, l0);
                 acc[i] += q6k_lane_dot(raw, f);
             }
         }
@@ -455,4 +475,105 @@ gemv_q8k_q6k_m(const signed char* xq, const float* xs, const uchar* w, float* y,
     if (M <= 2) gemv_q8k_q6k_m_body<2>(xq, xs, w, y, K, N, M, ACC);
     else if (M <= 4) gemv_q8k_q6k_m_body<4>(xq, xs, w, y, K, N, M, ACC);
     else gemv_q8k_q6k_m_body<8>(xq, xs, w, y, K, N, M, ACC);
+}
+
+// Few tokens against a long tensor (speculative verify on the output head): the quantized
+// activations of all M <= 16 tokens are staged once per workgroup in LDS, laid out so that the 64
+// lanes of a wave read 64 consecutive 16-byte pieces per (token, step, quarter); a wave then
+// walks rows grid-stride, turns a row's codes into signed bytes once (w - 32: flip bit 5, then
+// copy the flipped bit into bits 6 and 7) and runs plain int8 dots against every token.
+//   gemv_q8k_q6k_mx(xq, xs, w, y, K, N, M, ACC)    M <= 16, M * ceil(K/4096) <= 19 (80 KB of LDS,
+//                                                  two workgroups per CU); any grid of 256-thread blocks
+#define Q6K_MX_LDS 81920u
+template <int MT>
+__device__ __forceinline__ void gemv_q8k_q6k_mx_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                     const uchar* __restrict__ w, float* __restrict__ y,
+                                                     uint K, uint N, uint M, uint ACC, uchar* lds) {
+    const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint nsb = K >> 8, nstep = (nsb + 15u) >> 4;
+    // LDS: token t, step s, quarter q, lane -> 16 bytes at ((t * nstep + s) * 4 + q) * 1024 + lane * 16;
+    // then the scales, token-major, one float per super-block (zero beyond nsb)
+    const uint xbytes = M * nstep * 4096u;
+    float* lsx = (float*)(lds + xbytes);
+    for (uint i = tid; i < M * nstep * 256u; i += 256u) {   // one 16-byte piece per trip
+        const uint ln = i & 63u, q = (i >> 6) & 3u, ts = i >> 8, s = ts % nstep, t = ts / nstep;
+        const uint sb = s * 16u + (ln >> 2);
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (sb < nsb) v = *(const uint4*)(xq + (size_t)t * nsb * 256u + sb * 256u + ((ln >> 1) & 1u) * 128u + q * 32u + (ln & 1u) * 16u);
+        *(uint4*)(lds + (size_t)i * 16u) = v;
+    }
+    for (uint i = tid; i < M * nstep * 16u; i += 256u) {
+        const uint sb = i % (nstep * 16u), t = i / (nstep * 16u);
+        lsx[i] = sb < nsb ? xs[(size_t)t * nsb + sb] : 0.0f;
+    }
+    __syncthreads();
+    const uint g = lane >> 2, hf = (lane >> 1) & 1u, l0 = (lane & 1u) * 16u;
+    constexpr int R = 2;   // rows per wave and trip: twice the loads in flight, half the LDS reads per row
+    for (uint row0 = (blockIdx.x * 4u + wave) * R; row0 < N; row0 += gridDim.x * 4u * R) {
+        float acc[R][MT];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++) acc[r][t] = 0.0f;
+        for (uint s = 0; s < nstep; s++) {
+            const uint sb = min(s * 16u + g, nsb - 1u);   // lanes past the row's end re-read its last block against zero scales
+            Q6kW raw[R];
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                raw[r] = q6k_load_w(w + ((size_t)min(row0 + r, N - 1u) * nsb + sb) * Q6K_BYTES, hf, l0);
+            uint c[R][4][4];
+            int sc[R][4];
+            float d[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                q6k_codes<0>(raw[r], c[r][0]); q6k_codes<1>(raw[r], c[r][1]);
+                q6k_codes<2>(raw[r], c[r][2]); q6k_codes<3>(raw[r], c[r][3]);
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const uint x = c[r][q][j] ^ 0x20202020u, m = x & 0x20202020u;
+                        c[r][q][j] = x | (m << 1) | (m << 2);
+                    }
+                sc[r][0] = (int)(signed char)(raw[r].sc4); sc[r][1] = (int)(signed char)(raw[r].sc4 >> 8);
+                sc[r][2] = (int)(signed char)(raw[r].sc4 >> 16); sc[r][3] = (int)raw[r].sc4 >> 24;
+                d[r] = f16_bits_to_f32(raw[r].d16);
+            }
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                if (t < (int)M) {
+                    const uchar* px = lds + ((size_t)(t * nstep + s) * 4u) * 1024u + lane * 16u;
+                    const uint4 x0 = *(const uint4*)px, x1 = *(const uint4*)(px + 1024);
+                    const uint4 x2 = *(const uint4*)(px + 2048), x3 = *(const uint4*)(px + 3072);
+                    const float sx = lsx[(t * nstep + s) * 16u + g];
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const int isum = sc[r][0] * dot16(c[r][0], x0) + sc[r][1] * dot16(c[r][1], x1) +
+                                         sc[r][2] * dot16(c[r][2], x2) + sc[r][3] * dot16(c[r][3], x3);
+                        acc[r][t] += sx * d[r] * (float)isum;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                if (t < (int)M) {
+                    const float sum = wave_sum(acc[r][t]);
+                    if (lane == 0 && row0 + r < N) {
+                        float* o = y + (size_t)t * N + row0 + r;
+                        *o = ACC ? *o + sum : sum;
+                    }
+                }
+            }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+gemv_q8k_q6k_mx(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    __shared__ __attribute__((aligned(16))) uchar lds_mx[Q6K_MX_LDS];
+    if (M <= 4) gemv_q8k_q6k_mx_body<4>(xq, xs, w, y, K, N, M, ACC, lds_mx);
+    else if (M <= 8) gemv_q8k_q6k_mx_body<8>(xq, xs, w, y, K, N, M, ACC, lds_mx);
+    else gemv_q8k_q6k_mx_body<16>(xq, xs, w, y, K, N, M, ACC, lds_mx);
 }

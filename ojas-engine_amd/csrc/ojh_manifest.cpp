@@ -173,10 +173,16 @@ static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     int rc = check_kn(s, K, N, &f);
     if (rc) return rc;
     if (M == 0) return ojh_fail(OJH_ERR_ARG, "%s: M must be positive", s->name);
-    if ((rc = check_block(block, 0))) return rc;
+    const bool mx = s->rows_per_wave == 0;   // the LDS-staged, grid-stride entry
+    if ((rc = check_block(block, mx ? 256 : 0))) return rc;
     if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
-    if ((uint64_t)grid[0] * (block[0] / 64) < N)
+    if (mx) {
+        if (M > 16 || (uint64_t)M * ((K + 4095) / 4096) > 19)
+            return ojh_fail(OJH_ERR_ARG, "%s: M=%u tokens of K=%u do not fit its 80 KB of LDS (M <= 16, M*ceil(K/4096) <= 19)",
+                            s->name, M, K);
+    } else if ((uint64_t)grid[0] * (block[0] / 64) < N) {
         return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover N=%u rows", s->name, N);
+    }
     need[0] = (size_t)M * K;
     need[1] = (size_t)M * (K / 256) * 4;
     need[2] = (size_t)N * (K / f->weights) * f->bytes;
@@ -494,6 +500,15 @@ static int shape_stream(const ojh_kernel_spec *, const ojh_device *dev, uint32_t
     block[1] = block[2] = 1;
     return OJH_OK;
 }
+static int shape_mx(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t N, uint32_t,
+                    uint32_t grid[3], uint32_t block[3]) {
+    uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, cover = (N + 7) / 8;
+    grid[0] = cover < 2 * cus ? cover : 2 * cus;   // two resident workgroups per CU, rows grid-stride
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
 static int shape_rows(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t,
                       uint32_t grid[3], uint32_t block[3]) {
     uint32_t rows_per_block = 4u * (uint32_t)s->rows_per_wave;
@@ -552,6 +567,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(q + "_accum", "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
         add(q + "_bias", "gemv_q8k", 5, 2, f.type, 4, check_gemv_q8k, shape_rows);
         add(q + "_m", "gemv_q8k", 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
+        if (f.type == OJH_Q6_K) add(q + "_mx", "gemv_q8k", 4, 4, f.type, 0, check_gemv_q8k_m, shape_mx);
         if (f.type == OJH_Q4_K) {
             std::string fq = "gemv_fq8k_" + t;
             add(q + "_x4_r1", "gemv_q8k", 10, 5, f.type, 1, check_gemv_q8k_x4, shape_rows);

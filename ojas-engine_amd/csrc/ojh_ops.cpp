@@ -162,6 +162,13 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
         if (bias) p.push_back(bias->ptr);
         return ojh_launch(dev, name.c_str(), p, {K, N}, grid, block);
     }
+    // few tokens on Q6_K rows: activations staged in LDS once per workgroup, rows grid-stride
+    if (w->type == OJH_Q6_K && m <= 16 && (uint64_t)m * ((K + 4095) / 4096) <= 19) {
+        uint32_t sg[3], sb[3];
+        int rc = ojh_launch_shape(dev, "gemv_q8k_q6k_mx", K, N, m, sg, sb);
+        if (rc) return rc;
+        return ojh_launch(dev, "gemv_q8k_q6k_mx", {xq, xs, wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, sg, sb);
+    }
     grid[0] = (N + 3) / 4;
     return ojh_launch(dev, (base + "_m").c_str(), {xq, xs, wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, grid, block);
 }

@@ -269,3 +269,35 @@ def test_grouped_projections_other_formats_and_errors(gpu, orc, pkg):
         gpu.mm_q8k_multi(xq, xs, [l4] * 5, [y4] * 5)
     with pytest.raises(pkg.OjasHipError, match="needs"):
         gpu.mm_q8k_multi(xq, xs, [l4, l4], [y4, y6])
+
+
+@pytest.mark.parametrize("m,n,k,accum", [(3, 50, 256, False), (4, 130, 14336, True), (16, 301, 4096, False),
+                                         (9, 64, 2560, True), (17, 40, 4096, False), (5, 33, 16384, False)])
+def test_q6k_few_tokens_staged_and_streamed_forms_agree(gpu, orc, pkg, m, n, k, accum):
+    """Q6_K rows against a few tokens: the router's choice (activations staged in LDS when they fit,
+    the streamed `_m` entry otherwise) within the parity bar of matvec_kq, ragged super-block
+    counts and accumulate included; where both forms apply they must agree bit for bit in the
+    integer part, i.e. to the last-ulp association of the f32 sums."""
+    w = pkg.synth.q6k_weights(n, k, "mx", n, k)
+    x = pkg.synth.normal_f32(m * k, "mx", "x", m, k).reshape(m, k)
+    lin = gpu.lin(Q6_K, n, k, w)
+    y0 = pkg.synth.normal_f32(m * n, "mx", "y0").reshape(m, n) if accum else np.zeros((m, n), np.float32)
+    yd = gpu.upload(np.concatenate([y0.ravel(), np.full(8, 4242.5, np.float32)]))
+    gpu.mm(gpu.upload(x), lin, yd, m, accum, act_mode=pkg.ACT_Q8K)
+    got = gpu.read(yd, m * n + 8)
+    assert np.all(got[m * n:] == 4242.5)
+    want = np.stack([orc.matvec_kq(w, Q6_K, n, k, x[t]) for t in range(m)])
+    assert peak_err(got[:m * n].reshape(m, n) - y0, want) <= TOL_Q8K_SEEN
+    # the streamed entry by name on the same quantized activations
+    gpu.ensure_family("gemv_q8k")
+    nsb = k // 256
+    xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
+    gpu.quant_q8k(gpu.upload(x), m, k, xq, xs)
+    y2 = gpu.upload(y0)
+    gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_m", [(xq, 0), (xs, 0), (gpu.upload_bytes(w), 0), (y2, 0)],
+                 [k, n, m, int(accum)], [(n + 3) // 4, 1, 1], [256, 1, 1])
+    assert peak_err(gpu.read(y2, m * n).reshape(m, n) - y0, got[:m * n].reshape(m, n) - y0) <= 2e-6
+    if m > 16:
+        with pytest.raises(pkg.OjasHipError, match="do not fit"):
+            gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_mx", [(xq, 0), (xs, 0), (gpu.upload_bytes(w), 0), (y2, 0)],
+                         [k, n, m, 0], [8, 1, 1], [256, 1, 1])
