@@ -22,6 +22,8 @@
 //   moe_gu_q4k_m(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA)   grid (ceil(N/8), E)
 //   moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)            grid (ceil(N/16), E)
 //   moe_combine(dv, wgt, y, T, KSEL, D, ACC)                 grid ceil(T*D/256)
+//   moe_gu_q4k_mm / moe_down_q4k_mm (same arguments as the _m entries)
+//                                                            grid (ceil(N/16), E): the int8 matrix-core form
 #include "ojk_common.h"
 #include "ojk_q4k_dot.h"
 
@@ -239,6 +241,202 @@ moe_down_q4k_m(const signed char* __restrict__ aq, const float* __restrict__ as_
                 float s = wave_sum(v[r]);
                 if (lane == 0 && row0 + r < N) dv[(size_t)a * N + row0 + r] = s;
             }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ grouped products on the matrix cores
+// A workgroup owns 16 rows of expert e and walks the expert's assignments 16 at a time.  Per 32-weight
+// sub-block one v_mfma_i32_16x16x32_i8 multiplies the tile of quantized activations (A: lane
+// (m, kg) = (lane % 16, lane / 16) holds bytes 8 kg .. 8 kg + 7 of token m) with the sub-block's
+// 4-bit codes as bytes (B: lane (n, kg) holds the same bytes of row n); D register v of lane
+// (n, kg) is the integer dot of token 4 kg + v with row n.  A second MFMA against a tile of ones
+// gives every lane the activations' sub-block sums in the same layout, so the scale algebra
+//     sum_sb sx[t][sb] * sum_j ( d sc_j * idot_j  -  dmin m_j * bsum_j )
+// needs no cross-lane traffic: per MFMA four converts and four FMAs with lane-constant scales
+// (about a fifth of the vector instructions of the integer-dot form).  A token's result does not
+// depend on which other tokens share its tile.
+typedef int int4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ long pack2(uint lo, uint hi) { return (long)(((unsigned long)hi << 32) | lo); }
+
+// acc[w][v] += sx[v] * sum_j (a_j * idot_j[v] - b_j * bsum_j[v]) for one super-block of NW weight
+// tensors sharing the activations.  `xsb` points at the lane's 8 bytes of sub-block 0 (sub-block j
+// 32 bytes further); `wblk[w]` at the lane's row inside a wave-private LDS copy of the 16 x 144-byte
+// tile.
+template <int NW>
+__device__ __forceinline__ void mm_superblock(const signed char* xsb, const uchar* const (&wblk)[NW], uint kg,
+                                              const float (&sx)[4], float (&acc)[NW][4]) {
+    float tmp[NW][4], d[NW], dmin[NW];
+    uint s0[NW], s1[NW], s2[NW];
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+        const uint4 hdr = *(const uint4*)wblk[w];
+        d[w] = f16_bits_to_f32(hdr.x & 0xFFFFu);
+        dmin[w] = f16_bits_to_f32(hdr.x >> 16);
+        s0[w] = hdr.y; s1[w] = hdr.z; s2[w] = hdr.w;
+#pragma unroll
+        for (int v = 0; v < 4; v++) tmp[w][v] = 0.0f;
+    }
+    const long ones = 0x0101010101010101L;
+    const int4v zero = {0, 0, 0, 0};
+    // (kept rolled: unrolled, the compiler holds every scale and code of the super-block at once,
+    // occupancy drops, and the kernel measured slower)
+#pragma unroll 1
+    for (uint c = 0; c < 4u; c++) {
+        const uint2 x0 = *(const uint2*)(xsb + c * 64u), x1 = *(const uint2*)(xsb + c * 64u + 32u);
+        const long A0 = pack2(x0.x, x0.y), A1 = pack2(x1.x, x1.y);
+        const int4v b0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(A0, ones, zero, 0, 0, 0);
+        const int4v b1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(A1, ones, zero, 0, 0, 0);
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            uint sc, mn;
+            q4k_scale_min_pair(s0[w], s1[w], s2[w], c, sc, mn);
+            const float a_lo = d[w] * (float)(sc & 0xFFu), a_hi = d[w] * (float)(sc >> 8);
+            const float m_lo = dmin[w] * (float)(mn & 0xFFu), m_hi = dmin[w] * (float)(mn >> 8);
+            const uint2 q = *(const uint2*)(wblk[w] + 16u + c * 32u + 8u * kg);
+            const int4v dl = __builtin_amdgcn_mfma_i32_16x16x32_i8(A0, pack2(q.x & 0x0F0F0F0Fu, q.y & 0x0F0F0F0Fu), zero, 0, 0, 0);
+            const int4v dh = __builtin_amdgcn_mfma_i32_16x16x32_i8(A1, pack2((q.x >> 4) & 0x0F0F0F0Fu, (q.y >> 4) & 0x0F0F0F0Fu), zero, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                tmp[w][v] += a_lo * (float)dl[v] - m_lo * (float)b0[v];
+                tmp[w][v] += a_hi * (float)dh[v] - m_hi * (float)b1[v];
+            }
+        }
+    }
+#pragma unroll
+    for (int w = 0; w < NW; w++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[w][v] += sx[v] * tmp[w][v];
+}
+
+// Copy the super-block `sb` of 16 consecutive rows (144 bytes each, `rb` apart, rows past `nrows`
+// clamped) into the wave's LDS tile with 16-byte pieces, 64 lanes side by side: the loads are
+// contiguous per row instead of 8 bytes per lane and row.
+__device__ __forceinline__ void mm_stage_tile(const uchar* w_row0, size_t rb, uint nrows, uint sb, uchar* tile, uint lane) {
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+        const uint p = lane + 64u * i;
+        if (p < 144u) {
+            const uint r = p / 9u, c = p - r * 9u;
+            *(uint4*)(tile + p * 16u) = *(const uint4*)(w_row0 + (size_t)min(r, nrows - 1u) * rb + (size_t)sb * Q4K_BYTES + c * 16u);
+        }
+    }
+}
+
+// Workgroup = one 16-row tile of expert e; its four waves split the super-blocks of K between
+// them (wave w takes w, w + 4, ...) and their partial sums meet in LDS, added in wave order.
+template <int NW>
+__device__ __forceinline__ void mm_reduce(float (&acc)[NW][4], float* red, uint wave, uint lane) {
+    // red: [3 waves][NW * 4][64 lanes]
+    if (wave > 0) {
+#pragma unroll
+        for (int w = 0; w < NW; w++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) red[((wave - 1u) * (NW * 4) + w * 4 + v) * 64u + lane] = acc[w][v];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int k = 0; k < 3; k++)
+#pragma unroll
+            for (int w = 0; w < NW; w++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) acc[w][v] += red[(k * (NW * 4) + w * 4 + v) * 64u + lane];
+    }
+    __syncthreads();
+}
+
+// (four waves per SIMD: latency of the dependent list -> activation -> weight loads is hidden by occupancy)
+extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8)))
+moe_gu_q4k_mm(const signed char* __restrict__ xq, const float* __restrict__ xs, const uchar* __restrict__ wg,
+              const uchar* __restrict__ wu, float* __restrict__ act, const uint* __restrict__ offsets,
+              const uint* __restrict__ list, uint K, uint N, uint KSEL, uint NA) {
+    __shared__ float red[3 * 8 * 64];
+    __shared__ __attribute__((aligned(16))) uchar tiles[4][2][16 * Q4K_BYTES];
+    const uint e = blockIdx.y;
+    const uint a0 = min(offsets[e], NA), a1 = min(offsets[e + 1], NA);
+    if (a0 >= a1) return;
+    const uint lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, n = lane & 15u, kg = lane >> 4;
+    const uint row0 = blockIdx.x * 16u;
+    const uint nsb = K >> 8;
+    const size_t rb = (size_t)nsb * Q4K_BYTES;
+    const uchar* gw = wg + ((size_t)e * N + row0) * rb;
+    const uchar* uw = wu + ((size_t)e * N + row0) * rb;
+    const uint nrows = min(16u, N - row0);
+    for (uint tt = a0; tt < a1; tt += 16u) {
+        // activations: lane's token for the A operand, and the four tokens of its D registers
+        const uint ta = min(list[min(tt + n, a1 - 1u)], NA - 1u) / KSEL;
+        const signed char* xrow = xq + (size_t)ta * K + 8u * kg;
+        uint av[4], tv[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            av[v] = min(list[min(tt + 4u * kg + v, a1 - 1u)], NA - 1u);
+            tv[v] = av[v] / KSEL;
+        }
+        float acc[2][4];
+#pragma unroll
+        for (int w = 0; w < 2; w++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[w][v] = 0.0f;
+#pragma unroll 1
+        for (uint sb = wave; sb < nsb; sb += 4u) {
+            float sx[4];
+#pragma unroll
+            for (int v = 0; v < 4; v++) sx[v] = xs[(size_t)tv[v] * nsb + sb];
+            mm_stage_tile(gw, rb, nrows, sb, tiles[wave][0], lane);
+            mm_stage_tile(uw, rb, nrows, sb, tiles[wave][1], lane);
+            const uchar* const wb[2] = {tiles[wave][0] + n * Q4K_BYTES, tiles[wave][1] + n * Q4K_BYTES};
+            mm_superblock<2>(xrow + sb * 256u, wb, kg, sx, acc);
+        }
+        mm_reduce<2>(acc, red, wave, lane);
+        if (wave == 0 && row0 + n < N) {
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                if (tt + 4u * kg + v < a1) {
+                    const float g = acc[0][v];
+                    act[(size_t)av[v] * N + row0 + n] = (g / (1.0f + expf(-g))) * acc[1][v];
+                }
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8)))
+moe_down_q4k_mm(const signed char* __restrict__ aq, const float* __restrict__ as_, const uchar* __restrict__ wd,
+                float* __restrict__ dv, const uint* __restrict__ offsets, const uint* __restrict__ list,
+                uint K, uint N, uint NA) {
+    __shared__ float red[3 * 4 * 64];
+    __shared__ __attribute__((aligned(16))) uchar tiles[4][16 * Q4K_BYTES];
+    const uint e = blockIdx.y;
+    const uint a0 = min(offsets[e], NA), a1 = min(offsets[e + 1], NA);
+    if (a0 >= a1) return;
+    const uint lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, n = lane & 15u, kg = lane >> 4;
+    const uint row0 = blockIdx.x * 16u;
+    const uint nsb = K >> 8;
+    const size_t rb = (size_t)nsb * Q4K_BYTES;
+    const uchar* dw = wd + ((size_t)e * N + row0) * rb;
+    const uint nrows = min(16u, N - row0);
+    for (uint tt = a0; tt < a1; tt += 16u) {
+        const uint aa = min(list[min(tt + n, a1 - 1u)], NA - 1u);
+        const signed char* xrow = aq + (size_t)aa * K + 8u * kg;
+        uint av[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) av[v] = min(list[min(tt + 4u * kg + v, a1 - 1u)], NA - 1u);
+        float acc[1][4] = {{0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll 1
+        for (uint sb = wave; sb < nsb; sb += 4u) {
+            float sx[4];
+#pragma unroll
+            for (int v = 0; v < 4; v++) sx[v] = as_[(size_t)av[v] * nsb + sb];
+            mm_stage_tile(dw, rb, nrows, sb, tiles[wave], lane);
+            const uchar* const wb[1] = {tiles[wave] + n * Q4K_BYTES};
+            mm_superblock<1>(xrow + sb * 256u, wb, kg, sx, acc);
+        }
+        mm_reduce<1>(acc, red, wave, lane);
+        if (wave == 0 && row0 + n < N) {
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                if (tt + 4u * kg + v < a1) dv[(size_t)av[v] * N + row0 + n] = acc[0][v];
         }
     }
 }

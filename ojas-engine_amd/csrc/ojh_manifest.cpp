@@ -360,6 +360,7 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
 //   3 moe_gu_q4k_m(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA)            grid [ceil(N/8), E, 1]
 //   4 moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)                     grid [ceil(N/16), E, 1]
 //   5 moe_combine(dv, wgt, y, T, KSEL, D, ACC)                                    grid [ceil(T*D/256),1,1]
+//   6 moe_gu_q4k_mm, 7 moe_down_q4k_mm: the arguments of 3 and 4, grid [ceil(N/16), E, 1]
 static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                      const uint32_t block[3], size_t need[16], size_t align[16]) {
     int rc;
@@ -385,11 +386,13 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         need[2] = (size_t)(E + 1) * 4;
         return OJH_OK;
     }
-    case 3: {
+    case 3: case 6: {
         uint32_t K = c[0], N = c[1], KS = c[2], NA = c[3], E = grid[1];
+        const uint32_t per = s->rows_per_wave == 3 ? 8 : 16;   // rows per workgroup
         if ((rc = check_block(block, 256))) return rc;
         if (!K || K % 256 || !N || !KS || !NA || NA % KS) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u KSEL=%u NA=%u", s->name, K, N, KS, NA);
-        if (grid[0] != (N + 7) / 8 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/8), E, 1]", s->name);
+        if (grid[0] != (N + per - 1) / per || grid[2] != 1)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/%u), E, 1]", s->name, per);
         size_t rb = (size_t)(K / 256) * 144;
         need[0] = (size_t)(NA / KS) * K;
         need[1] = (size_t)(NA / KS) * (K / 256) * 4;
@@ -400,11 +403,13 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         align[0] = align[2] = align[3] = 16;
         return OJH_OK;
     }
-    case 4: {
+    case 4: case 7: {
         uint32_t K = c[0], N = c[1], NA = c[2], E = grid[1];
+        const uint32_t per = 16;
         if ((rc = check_block(block, 256))) return rc;
         if (!K || K % 256 || !N || !NA) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u NA=%u", s->name, K, N, NA);
-        if (grid[0] != (N + 15) / 16 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/16), E, 1]", s->name);
+        if (grid[0] != (N + per - 1) / per || grid[2] != 1)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/%u), E, 1]", s->name, per);
         need[0] = (size_t)NA * K;
         need[1] = (size_t)NA * (K / 256) * 4;
         need[2] = (size_t)E * N * (K / 256) * 144;
@@ -441,6 +446,7 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, u
     case 2: break;
     case 3: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = experts
     case 4: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
+    case 6: case 7: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;
     default: grid[0] = (uint32_t)(((uint64_t)M * N + 255) / 256); break;  // N = D, M = tokens
     }
     return OJH_OK;
@@ -603,6 +609,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("moe_gu_q4k_m", "moe", 7, 4, OJH_Q4_K, 3, check_moe, shape_moe);
     add("moe_down_q4k_m", "moe", 6, 3, OJH_Q4_K, 4, check_moe, shape_moe);
     add("moe_combine", "moe", 3, 4, 0, 5, check_moe, shape_moe);
+    add("moe_gu_q4k_mm", "moe", 7, 4, OJH_Q4_K, 6, check_moe, shape_moe);
+    add("moe_down_q4k_mm", "moe", 6, 3, OJH_Q4_K, 7, check_moe, shape_moe);
     add("copy_bf16_half", "glue", 2, 1, (2u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     // glue: `type` carries (input element bytes << 8 | output element bytes)
     add("copy_f32_half", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);

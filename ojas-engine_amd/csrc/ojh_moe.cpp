@@ -66,6 +66,10 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     uint32_t *counts = (uint32_t *)grp->ptr, *offsets = counts + E, *list = offsets + E + 1;
 
     uint32_t b256[3] = {256, 1, 1};
+    // Expert products: on the matrix cores once experts see a few tokens each (measured crossover on
+    // MI355X: ~2 assignments per expert), on integer dots below that, where the launch is a pure
+    // stream of weight rows.  The two forms round their f32 sums in different orders (last ulp).
+    const bool mm = dev->moe_mode == 1 || (dev->moe_mode == 0 && NA >= 2 * E);
     // 1. quantize the tokens once
     {
         uint32_t g[3] = {nsb_d, T, 1};
@@ -78,8 +82,8 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     }
     // 3. gate/up + SiLU*mul, one launch over all experts
     {
-        uint32_t g[3] = {(n_ff + 7) / 8, E, 1};
-        if ((rc = ojh_launch(dev, "moe_gu_q4k_m",
+        uint32_t g[3] = {mm ? (n_ff + 15) / 16 : (n_ff + 7) / 8, E, 1};
+        if ((rc = ojh_launch(dev, mm ? "moe_gu_q4k_mm" : "moe_gu_q4k_m",
                              {xq->ptr, xs->ptr, (char *)gate->raw->ptr + gate->off, (char *)up->raw->ptr + up->off, act->ptr,
                               offsets, list},
                              {d, n_ff, ksel, NA}, g, b256)))
@@ -93,7 +97,7 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     // 5. down, one launch over all experts
     {
         uint32_t g[3] = {(d + 15) / 16, E, 1};
-        if ((rc = ojh_launch(dev, "moe_down_q4k_m",
+        if ((rc = ojh_launch(dev, mm ? "moe_down_q4k_mm" : "moe_down_q4k_m",
                              {aq->ptr, as_->ptr, (char *)down->raw->ptr + down->off, dv->ptr, offsets, list},
                              {n_ff, d, NA}, g, b256)))
             return rc;
