@@ -271,6 +271,32 @@ def extras(gpu, pkg, lin_q) -> dict:
     b = n * (k // 32) * 34 + 4 * k + 4 * n
     out["q80_gemv_4096x4096"] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
     del wq8
+    # ---- one FFN block of a decode layer with the fused epilogues: rmsnorm+quantize, gate/up+SiLU,
+    # quantize, down accumulated onto the residual (4 launches, recorded and replayed)
+    d, nff = 4096, 14336
+    blocks = []
+    for c in range(4):
+        blocks.append((gpu.lin(pkg.Q4_K, nff, d, synth.q4k_weights(nff, d, "bench", "ffn_g", c)),
+                       gpu.lin(pkg.Q4_K, nff, d, synth.q4k_weights(nff, d, "bench", "ffn_u", c)),
+                       gpu.lin(pkg.Q4_K, d, nff, synth.q4k_weights(d, nff, "bench", "ffn_d", c))))
+    xr = gpu.upload(synth.normal_f32(d, "bench", "ffn_x"))
+    gm = gpu.upload(np.ones(d, np.float32))
+    xq_, xs_ = gpu.alloc_bytes(d), gpu.alloc(d // 256)
+    aq_, as__ = gpu.alloc_bytes(nff), gpu.alloc(nff // 256)
+    act_ = gpu.alloc(nff)
+    graphs = []
+    for g_, u_, d_ in blocks:
+        gpu.capture_begin()
+        gpu.rmsnorm_quant_q8k(xr, gm, 1e-5, 1, d, xq_, xs_)
+        gpu.ffn_gu_q8k(xq_, xs_, g_, u_, act_)
+        gpu.quant_q8k(act_, 1, nff, aq_, as__)
+        gpu.mm_q8k(aq_, as__, d_, xr, accum=True)
+        graphs.append(gpu.capture_end())
+    us = _time(gpu, lambda i: graphs[i % 4].launch(), 40, 8)
+    b = 3 * nff * (d // 256) * 144
+    out["ffn_block_q4k_14336x4096"] = {"launches": "rmsnorm_q8k, ffn_gu_q8k_q4k, quantize_q8k, gemv_q8k_q4k_accum",
+                                       "us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
+    del blocks, graphs
     # ---- MoE: 128 experts, top-8, hidden 2048, expert FFN 768, Q4_K; tokens 1 / 16 / 256
     E, ksel, d, nff = 128, 8, 2048, 768
     gate = gpu.lin(pkg.Q4_K, E * nff, d, synth.q4k_weights(E * nff, d, "bench", "moe_gate"))

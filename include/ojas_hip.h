@@ -193,6 +193,19 @@ int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const
 int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, int count,
                      const ojh_lin *const *ws, ojh_buf *const *ys, const size_t *y_offs);
 
+/* Decode-layer epilogues around the matvec (the reference fuses the same steps on its GPU path:
+ * `rmsnorm_q8` / `quantize_q8_1` and `ffn_gu_q80_dp4a`, crates/ojas-cuda/src/kernels/gemv.rs:37-53,
+ * gemv_q8.rs:246-260).
+ *   ojh_rmsnorm_quant_q8k: per row of x (f32 [m][k], k <= 16384), xn = x * rsqrt(mean(x^2) + eps) * gamma
+ *     (`rmsnorm`, crates/ojas-cpu/src/cpu_math.rs:456-460) quantized as `quant_q8k` does, in one
+ *     launch; `xn` (f32 [m][k]) may be NULL when only the quantized form is needed.
+ *   ojh_ffn_gu_q8k: out[n] = act(gate[n] . x) * (up[n] . x) from one quantized vector; act 0 = SiLU
+ *     (cpu_math.rs:486), 1 = GELU tanh form (:497-501).  Q4_K tensors of equal shape. */
+int ojh_rmsnorm_quant_q8k(ojh_device *dev, const ojh_buf *x, size_t x_off, const ojh_buf *gamma, float eps,
+                          uint32_t m, uint32_t k, ojh_buf *q, ojh_buf *scales, ojh_buf *xn);
+int ojh_ffn_gu_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const ojh_lin *gate,
+                   const ojh_lin *up, ojh_buf *out, size_t out_off, int act);
+
 /* `relayout_q4k_q4l` (crates/ojas-formats/src/quant.rs:192-222) on the device: n rows of k Q4_K
  * weights -> nibble pairs `nib` [n*k/2], f16 `qa` = d*sc and `qb` = -dmin*m per 32 weights
  * [n*k/32 each].  Bit-exact with the reference.  The library's own prefill GEMM does not need

@@ -6,7 +6,8 @@
 // :674-722 (dot_q6k), :1145-1189 (matvec_kq).
 //
 //   quantize_q8k{,_bf16}(x, q, scales, K, M)             grid (ceil(K/256), M), block 256
-//   gemv_q8k_<fmt>{,_accum,_bias}(xq, xs, w, y[, bs], K, N)   4 rows per wave
+//   gemv_q8k_<fmt>(xq, xs, w, y, K, N)                        4 rows per wave
+//   gemv_q8k_<fmt>{_accum,_bias}(xq, xs, w, y[, bs], K, N)    1 row per wave (residual-sized N)
 //   gemv_q8k_<fmt>_r1 / _r2 (same arguments)                  1 / 2 rows per wave
 //   gemv_q8k_<fmt>_wide (same arguments)                      2 rows per wave; the entry the op
 //                                                             seam uses for output-head sized N
@@ -113,10 +114,10 @@ __device__ __forceinline__ void gemv_q8k_q4k_body(const signed char* __restrict_
         BODY<4, ST_SET>(xq, xs, w, y, nullptr, K, N); }                                                      \
     extern "C" __global__ void __launch_bounds__(256) gemv_q8k_##FMT##_accum(                                \
         const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N) {                  \
-        BODY<4, ST_ACCUM>(xq, xs, w, y, nullptr, K, N); }                                                    \
+        BODY<1, ST_ACCUM>(xq, xs, w, y, nullptr, K, N); }                                                    \
     extern "C" __global__ void __launch_bounds__(256) gemv_q8k_##FMT##_bias(                                 \
         const signed char* xq, const float* xs, const uchar* w, float* y, const float* bs, uint K, uint N) { \
-        BODY<4, ST_BIAS>(xq, xs, w, y, bs, K, N); }
+        BODY<1, ST_BIAS>(xq, xs, w, y, bs, K, N); }
 
 GEMV_Q8K_ENTRIES(q4k, gemv_q8k_q4k_body)
 
@@ -188,6 +189,116 @@ gemv_q8k_q4k_x4_r2(const signed char* xq, const float* xs, const uchar* w0, cons
                    const uchar* w3, float* y0, float* y1, float* y2, float* y3, uint K, uint E0, uint E1, uint E2,
                    uint E3) {
     gemv_q8k_q4k_x4_body<2>(xq, xs, w0, w1, w2, w3, y0, y1, y2, y3, K, E0, E1, E2, E3);
+}
+
+// ---- gate and up projections with the activation function in one launch -----------------------
+//   ffn_gu_q8k_q4k(xq, xs, wg, wu, out, K, N, ACT)     out[n] = act(Wg[n] . x) * (Wu[n] . x)
+// ACT 0 = SiLU  g / (1 + exp(-g))  (crates/ojas-cpu/src/cpu_math.rs:486), 1 = GELU, tanh form
+// (:497-501).  The reference's decode path fuses the same three steps
+// (`ffn_gu_q80_dp4a`, crates/ojas-cuda/src/kernels/gemv_q8.rs:246-260); each dot is the
+// single-tensor arithmetic of gemv_q8k_q4k.
+__device__ __forceinline__ float ffn_act(float g, uint act) {
+    if (act == 1u) {
+        const float c = 0.7978845608028654f, a = 0.044715f;
+        return 0.5f * g * (1.0f + tanhf(c * g * (1.0f + a * g * g)));
+    }
+    return g / (1.0f + expf(-g));
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+ffn_gu_q8k_q4k(const signed char* __restrict__ xq, const float* __restrict__ xs, const uchar* __restrict__ wg,
+               const uchar* __restrict__ wu, float* __restrict__ out, uint K, uint N, uint ACT) {
+    constexpr int R = 1;   // one row per wave (two weight streams): K is short, so more, lighter waves win
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 >= N) return;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    float ag[R], au[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) ag[r] = au[r] = 0.0f;
+    for (uint sb = g; sb < nsb; sb += 8u) {
+        uint4 hg[R], qg[R], hu[R], qu[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const size_t o = ((size_t)min(row0 + r, N - 1u) * nsb + sb) * Q4K_BYTES;
+            hg[r] = *(const uint4*)(wg + o); qg[r] = *(const uint4*)(wg + o + 16u + l * 16u);
+            hu[r] = *(const uint4*)(wu + o); qu[r] = *(const uint4*)(wu + o + 16u + l * 16u);
+        }
+        Q4kFrag f = q4k_load_frag(xq, xs, sb, l);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            ag[r] += q4k_lane_dot(hg[r], qg[r], c, f);
+            au[r] += q4k_lane_dot(hu[r], qu[r], c, f);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const float sg = wave_sum(ag[r]), su = wave_sum(au[r]);
+        if (lane == 0 && row0 + r < N) out[row0 + r] = ffn_act(sg, ACT) * su;
+    }
+}
+
+// ---- RMS norm and activation quantizer in one launch --------------------------------------------
+//   rmsnorm_q8k(x, gamma, q, scales, xn, K, M, EPS_BITS, WRITE_XN)    grid M, block 256, K <= 16384
+// xn = x * (1 / sqrt(mean(x^2) + eps)) * gamma  (crates/ojas-cpu/src/cpu_math.rs:456-460), then
+// quant_q8k(xn) (:539-563) without a trip through memory: a decode layer's projections read the
+// normalized vector only through its quantized form.  The mean of squares is summed in f64 and
+// rounded once; the reference sums in f32 in index order, so `inv` may differ in its last bit.
+extern "C" __global__ void __launch_bounds__(256)
+rmsnorm_q8k(const float* __restrict__ x, const float* __restrict__ gamma, signed char* __restrict__ q,
+            float* __restrict__ scales, float* __restrict__ xn, uint K, uint M, uint EPS_BITS, uint WRITE_XN) {
+    __shared__ double part[4];
+    const uint m = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint nsb = (K + 255u) >> 8;
+    const float* row = x + (size_t)m * K;
+    const bool vec = (K & 3u) == 0 && (((size_t)row | (size_t)gamma) & 15u) == 0;   // 128-bit loads
+    // wave w owns segments w, w + 4, ...; a lane holds 4 consecutive values of each
+    auto load4 = [&](const float* p, uint i0, float (&o)[4]) {
+        if (vec && i0 + 3u < K) {
+            const float4 t = *(const float4*)(p + i0);
+            o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = i0 + e < K ? p[i0 + e] : 0.0f;
+        }
+    };
+    double ss = 0.0;
+    for (uint seg = wave; seg < nsb; seg += 4u) {
+        float v[4];
+        load4(row, seg * 256u + lane * 4u, v);
+#pragma unroll
+        for (int e = 0; e < 4; e++) ss += (double)v[e] * (double)v[e];
+    }
+    // wave reduction in f64 through two 32-bit halves
+    for (int off = 32; off > 0; off >>= 1) {
+        const long b = __double_as_longlong(ss);
+        const int lo = __shfl_xor((int)b, off), hi = __shfl_xor((int)(b >> 32), off);
+        ss += __longlong_as_double(((long)hi << 32) | (unsigned int)lo);
+    }
+    if (lane == 0) part[wave] = ss;
+    __syncthreads();
+    const float mean = (float)(((part[0] + part[1]) + (part[2] + part[3])) / (double)K);
+    const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(mean, __uint_as_float(EPS_BITS))));
+    for (uint seg = wave; seg < nsb; seg += 4u) {
+        const uint i0 = seg * 256u + lane * 4u;
+        float v[4], gm[4], t[4];
+        load4(row, i0, v);      // second read: from the cache
+        load4(gamma, i0, gm);
+#pragma unroll
+        for (int e = 0; e < 4; e++) t[e] = i0 + e < K ? __fmul_rn(__fmul_rn(v[e], inv), gm[e]) : 0.0f;
+        const float a = wave_max(fmaxf(fmaxf(fabsf(t[0]), fabsf(t[1])), fmaxf(fabsf(t[2]), fabsf(t[3]))));
+        const float scale = a > 0.0f ? __fdiv_rn(a, 127.0f) : 1.0f;
+        const float is = __fdiv_rn(1.0f, scale);
+        uint packed = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int qi = (int)fminf(fmaxf(roundf(__fmul_rn(t[e], is)), -127.0f), 127.0f);
+            packed |= (uint)(qi & 0xFF) << (8 * e);
+            if (WRITE_XN && i0 + e < K) xn[(size_t)m * K + i0 + e] = t[e];
+        }
+        *(uint*)(q + ((size_t)m * nsb + seg) * 256u + lane * 4u) = packed;
+        if (lane == 0) scales[(size_t)m * nsb + seg] = scale;
+    }
 }
 
 // ---- the same matvec with the activation quantizer folded in ---------------------------------

@@ -124,6 +124,51 @@ static int check_gemv_q8k_x4(const ojh_kernel_spec *s, const uint32_t *c, const 
     return OJH_OK;
 }
 
+// ffn_gu_q8k_<fmt>(xq, xs, wg, wu, out, K, N, ACT): one wave per row
+static int check_ffn_gu(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                        const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], N = c[1], ACT = c[2];
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if (ACT > 1) return ojh_fail(OJH_ERR_ARG, "%s: ACT=%u (0 = SiLU, 1 = GELU)", s->name, ACT);
+    if ((rc = check_block(block, 0))) return rc;
+    if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * (block[0] / 64) * s->rows_per_wave < N)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover N=%u rows", s->name, N);
+    need[0] = (size_t)K;
+    need[1] = (size_t)(K / 256) * 4;
+    need[2] = need[3] = (size_t)N * (K / f->weights) * f->bytes;
+    need[4] = (size_t)N * 4;
+    align[1] = align[4] = 4;
+    return OJH_OK;
+}
+
+// rmsnorm_q8k(x, gamma, q, scales, xn, K, M, EPS_BITS, WRITE_XN): grid [M,1,1] x 256
+static int check_rmsnorm_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                             const uint32_t block[3], size_t need[16], size_t align[16]) {
+    uint32_t K = c[0], M = c[1], WR = c[3];
+    if (!K || !M || K > 16384) return ojh_fail(OJH_ERR_ARG, "%s: K=%u (1..16384) M=%u", s->name, K, M);
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (grid[0] != M || grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,1,1]", s->name, M);
+    uint32_t nsb = (K + 255) / 256;
+    need[0] = (size_t)M * K * 4;
+    need[1] = (size_t)K * 4;
+    need[2] = (size_t)M * nsb * 256;
+    need[3] = (size_t)M * nsb * 4;
+    need[4] = WR ? (size_t)M * K * 4 : 0;
+    align[0] = align[1] = align[3] = align[4] = 4;
+    return OJH_OK;
+}
+static int shape_rmsnorm(const ojh_kernel_spec *, const ojh_device *, uint32_t, uint32_t, uint32_t M,
+                         uint32_t grid[3], uint32_t block[3]) {
+    grid[0] = M ? M : 1;
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // gemv_fq8k_<fmt>_{r1,r2,wide}(x, w, y, K, N, NRB): quantizer folded in; 4 waves per block,
 // K <= 16384, NRB rows per block (a multiple of 4 * rows per wave)
 static int check_gemv_fq8k(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
@@ -570,8 +615,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(q + "_r1", "gemv_q8k", 4, 2, f.type, 1, check_gemv_q8k, shape_rows);
         add(q + "_r2", "gemv_q8k", 4, 2, f.type, 2, check_gemv_q8k, shape_rows);
         add(q + "_wide", "gemv_q8k", 4, 2, f.type, 2, check_gemv_q8k, shape_rows);
-        add(q + "_accum", "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
-        add(q + "_bias", "gemv_q8k", 5, 2, f.type, 4, check_gemv_q8k, shape_rows);
+        add(q + "_accum", "gemv_q8k", 4, 2, f.type, 1, check_gemv_q8k, shape_rows);
+        add(q + "_bias", "gemv_q8k", 5, 2, f.type, 1, check_gemv_q8k, shape_rows);
         add(q + "_m", "gemv_q8k", 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
         if (f.type == OJH_Q6_K) add(q + "_mx", "gemv_q8k", 4, 4, f.type, 0, check_gemv_q8k_m, shape_mx);
         if (f.type == OJH_Q4_K) {
@@ -588,6 +633,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("quant_rows_i8", "rowq8", 3, 2, 0, 1, check_rowq8, shape_rowq8);
     add("matmul_q8row", "rowq8", 5, 3, 0, 2, check_rowq8, shape_rowq8);
     add("matmul_q8row_bias", "rowq8", 6, 3, 0, 3, check_rowq8, shape_rowq8);
+    add("ffn_gu_q8k_q4k", "gemv_q8k", 5, 3, OJH_Q4_K, 1, check_ffn_gu, shape_rows);
+    add("rmsnorm_q8k", "gemv_q8k", 5, 4, 0, 0, check_rmsnorm_q8k, shape_rmsnorm);
     add("quantize_q8k", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     // prefill / verify MFMA tiles: "q8_0" is the reference's spelling for this family

@@ -154,7 +154,7 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
     uint32_t grid[3] = {1, 1, 1}, block[3] = {256, 1, 1};
     std::string base = std::string("gemv_q8k_") + f->tag;
     if (m == 1) {
-        int r = (accum || bias) ? 4 : pick_rows(dev, N);
+        int r = (accum || bias) ? 1 : pick_rows(dev, N);
         bool wide = !accum && !bias && r == 2 && N >= 32768u;
         std::string name = base + (accum ? "_accum" : bias ? "_bias" : wide ? "_wide" : r == 4 ? "" : r == 2 ? "_r2" : "_r1");
         grid[0] = (N + 4 * r - 1) / (4 * r);
@@ -395,4 +395,46 @@ extern "C" int ojh_matmul_q8(ojh_device *dev, const ojh_buf *x, size_t x_off, co
         return ojh_launch(dev, "matmul_q8row_bias", {xq->ptr, sx->ptr, wq->ptr, wscale->ptr, at(y, y_off), bias->ptr},
                           {k, n, m}, gm, block);
     return ojh_launch(dev, "matmul_q8row", {xq->ptr, sx->ptr, wq->ptr, wscale->ptr, at(y, y_off)}, {k, n, m}, gm, block);
+}
+
+// ---- decode-layer epilogues around the matvec ----------------------------------------------------
+extern "C" int ojh_rmsnorm_quant_q8k(ojh_device *dev, const ojh_buf *x, size_t x_off, const ojh_buf *gamma, float eps,
+                                     uint32_t m, uint32_t k, ojh_buf *q, ojh_buf *scales, ojh_buf *xn) {
+    if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_rmsnorm_quant_q8k: NULL device");
+    if (!m || !k || k > 16384 || m > 65535) return ojh_fail(OJH_ERR_ARG, "rmsnorm_quant_q8k: m=%u k=%u out of range (k <= 16384)", m, k);
+    size_t nsb = (k + 255) / 256;
+    int rc;
+    if ((rc = span_ok("rmsnorm_quant_q8k: x", x, x_off, (size_t)m * k * 4, 4))) return rc;
+    if ((rc = span_ok("rmsnorm_quant_q8k: gamma", gamma, 0, (size_t)k * 4, 4))) return rc;
+    if ((rc = span_ok("rmsnorm_quant_q8k: q", q, 0, (size_t)m * nsb * 256, 16))) return rc;
+    if ((rc = span_ok("rmsnorm_quant_q8k: scales", scales, 0, (size_t)m * nsb * 4, 4))) return rc;
+    if (xn && (rc = span_ok("rmsnorm_quant_q8k: xn", xn, 0, (size_t)m * k * 4, 4))) return rc;
+    if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+    uint32_t eps_bits;
+    memcpy(&eps_bits, &eps, 4);
+    uint32_t grid[3] = {m, 1, 1}, block[3] = {256, 1, 1};
+    return ojh_launch(dev, "rmsnorm_q8k", {at(x, x_off), gamma->ptr, q->ptr, scales->ptr, xn ? xn->ptr : q->ptr},
+                      {k, m, eps_bits, (uint32_t)(xn != nullptr)}, grid, block);
+}
+
+extern "C" int ojh_ffn_gu_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const ojh_lin *gate,
+                              const ojh_lin *up, ojh_buf *out, size_t out_off, int act) {
+    if (!dev || !gate || !up) return ojh_fail(OJH_ERR_ARG, "ojh_ffn_gu_q8k: NULL argument");
+    if (gate->type != OJH_Q4_K || up->type != OJH_Q4_K)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_ffn_gu_q8k: gate and up must be Q4_K (got %u, %u)", gate->type, up->type);
+    if (gate->n != up->n || gate->k != up->k)
+        return ojh_fail(OJH_ERR_ARG, "ojh_ffn_gu_q8k: gate is %ux%u, up is %ux%u", gate->n, gate->k, up->n, up->k);
+    if (act != 0 && act != 1) return ojh_fail(OJH_ERR_ARG, "ojh_ffn_gu_q8k: act=%d (0 = SiLU, 1 = GELU)", act);
+    const uint32_t N = gate->n, K = gate->k;
+    size_t nsb = K / 256;
+    int rc;
+    if ((rc = span_ok("ffn_gu: xq", xq, 0, nsb * 256, 16))) return rc;
+    if ((rc = span_ok("ffn_gu: xscales", xscales, 0, nsb * 4, 4))) return rc;
+    if ((rc = span_ok("ffn_gu: out", out, out_off, (size_t)N * 4, 4))) return rc;
+    if ((rc = span_ok("ffn_gu: gate", gate->raw, gate->off, gate->row_bytes * N, 16))) return rc;
+    if ((rc = span_ok("ffn_gu: up", up->raw, up->off, up->row_bytes * N, 16))) return rc;
+    if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+    uint32_t grid[3] = {(N + 3) / 4, 1, 1}, block[3] = {256, 1, 1};
+    return ojh_launch(dev, "ffn_gu_q8k_q4k", {xq->ptr, xscales->ptr, at(gate->raw, gate->off), at(up->raw, up->off), at(out, out_off)},
+                      {K, N, (uint32_t)act}, grid, block);
 }

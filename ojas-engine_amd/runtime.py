@@ -104,6 +104,8 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_mm": (i32, [vp, vp, sz, i32, vp, vp, sz, vp, u32, i32, i32]),
         "ojh_mm_q8k": (i32, [vp, vp, vp, vp, vp, sz, vp, u32, i32]),
         "ojh_mm_q8k_multi": (i32, [vp, vp, vp, i32, vp, vp, vp]),
+        "ojh_rmsnorm_quant_q8k": (i32, [vp, vp, sz, vp, C.c_float, u32, u32, vp, vp, vp]),
+        "ojh_ffn_gu_q8k": (i32, [vp, vp, vp, vp, vp, vp, sz, i32]),
         "ojh_relayout_q4k_q4l": (i32, [vp, vp, sz, u32, u32, vp, vp, vp]),
         "ojh_q8rows_from_f16": (i32, [vp, vp, sz, u32, u32, vp, vp]),
         "ojh_matmul_q8": (i32, [vp, vp, sz, vp, vp, vp, vp, sz, u32, u32, u32]),
@@ -368,6 +370,17 @@ class HipGpu:
         ya = (C.c_void_p * n)(*[y.handle for y in ys])
         oa = (C.c_size_t * n)(*y_offs) if y_offs is not None else None
         self._check(self._L.ojh_mm_q8k_multi(self._dev, xq.handle, xscales.handle, n, wa, ya, oa))
+
+    def rmsnorm_quant_q8k(self, x: Buf, gamma: Buf, eps: float, m: int, k: int, q: Buf, scales: Buf,
+                          xn: Buf | None = None, x_off: int = 0) -> None:
+        """RMS norm + quant_q8k in one launch (xn optional f32 copy of the normalized rows)."""
+        self._check(self._L.ojh_rmsnorm_quant_q8k(self._dev, x.handle, x_off, gamma.handle, eps, m, k, q.handle,
+                                                  scales.handle, xn.handle if xn else None))
+
+    def ffn_gu_q8k(self, xq: Buf, xscales: Buf, gate: Lin, up: Lin, out: Buf, act: int = 0, out_off: int = 0) -> None:
+        """out = act(gate . x) * (up . x) in one launch (act 0 SiLU, 1 GELU)."""
+        self._check(self._L.ojh_ffn_gu_q8k(self._dev, xq.handle, xscales.handle, gate.handle, up.handle, out.handle,
+                                           out_off, act))
 
     def relayout_q4k_q4l(self, raw: Buf, n: int, k: int, nib: Buf, qa: Buf, qb: Buf, raw_off: int = 0) -> None:
         """Q4_K blocks -> the Q4L arrays (nibble pairs, f16 qa / qb per 32 weights)."""

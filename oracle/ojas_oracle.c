@@ -683,6 +683,27 @@ int ojo_matmul_ref(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const fl
     return 0;
 }
 
+/* ---------------------------------------------------------------- decode-layer glue */
+
+void ojo_rmsnorm(const float *x, const float *w, size_t k, float eps, float *y) {
+    /* crates/ojas-cpu/src/cpu_math.rs:456-460: f32 sum of squares in index order, / len,
+     * inv = 1 / sqrt(ss + eps), y = (x * inv) * w */
+    float ss = 0.0f;
+    for (size_t i = 0; i < k; i++) ss += x[i] * x[i];
+    ss = ss / (float)k;
+    float inv = 1.0f / sqrtf(ss + eps);
+    for (size_t i = 0; i < k; i++) y[i] = x[i] * inv * w[i];
+}
+
+float ojo_ffn_act(float g, int act) {
+    /* act 0: silu, cpu_math.rs:486; act 1: gelu (tanh form), cpu_math.rs:497-501 */
+    if (act == 1) {
+        const float c = 0.7978845608028654f, a = 0.044715f;
+        return 0.5f * g * (1.0f + tanhf(c * g * (1.0f + a * g * g)));
+    }
+    return g / (1.0f + expf(-g));
+}
+
 /* ---------------------------------------------------------------- MoE */
 
 void ojo_moe_topk(const float *lg, int E, int ksel, uint32_t *idx, float *wgt) {

@@ -98,6 +98,11 @@ void ojo_q4l_weights_f16(const uint8_t *w, size_t k, size_t n, uint16_t *out);
 int ojo_matmul_ref(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const float *x, size_t m,
                    int wmode, int xmode, int threads, double *y);
 
+/* rmsnorm (crates/ojas-cpu/src/cpu_math.rs:456-460) and the FFN activation functions
+ * (silu :486, gelu tanh form :497-501). */
+void  ojo_rmsnorm(const float *x, const float *w, size_t k, float eps, float *y);
+float ojo_ffn_act(float g, int act);
+
 /* Router: softmax, ksel argmax passes with strict '>', lowest index wins, renormalise
  * (crates/ojas-cuda/src/kernels/moe.rs:45-70; oracle crates/ojas-cuda/tests/conformance.rs:385-392). */
 void ojo_moe_topk(const float *logits, int n_expert, int ksel, uint32_t *idx, float *wgt);

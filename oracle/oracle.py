@@ -68,6 +68,10 @@ def lib() -> C.CDLL:
         L.ojo_q4l_weights_f16.restype = None
         L.ojo_q4l_weights_f16.argtypes = [vp, sz, sz, vp]
         L.ojo_matmul_ref.argtypes = [vp, u32, sz, sz, vp, sz, i32, i32, i32, vp]
+        L.ojo_rmsnorm.restype = None
+        L.ojo_rmsnorm.argtypes = [vp, vp, sz, C.c_float, vp]
+        L.ojo_ffn_act.restype = C.c_float
+        L.ojo_ffn_act.argtypes = [C.c_float, i32]
         L.ojo_moe_topk.restype = None
         L.ojo_moe_topk.argtypes = [vp, i32, i32, vp, vp]
         L.ojo_moe_ffn.argtypes = [vp, sz, sz, sz, i32, i32, vp, vp, vp, vp, u32, vp, u32, i32, i32, vp]
@@ -208,6 +212,19 @@ def matmul_ref(raw, ty, n, k, x, wmode: int = 0, xmode: int = 0, threads: int = 
     y = np.empty((m, n), np.float64)
     assert lib().ojo_matmul_ref(_p(raw), ty, n, k, _p(x), m, wmode, xmode, threads, _p(y)) == 0
     return y
+
+
+def rmsnorm(x: np.ndarray, w: np.ndarray, eps: float) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    y = np.empty_like(x)
+    lib().ojo_rmsnorm(_p(x), _p(w), x.size, eps, _p(y))
+    return y
+
+
+def ffn_act(g: np.ndarray, act: int = 0) -> np.ndarray:
+    g = np.ascontiguousarray(g, np.float32)
+    return np.array([lib().ojo_ffn_act(float(v), act) for v in g.ravel()], np.float32).reshape(g.shape)
 
 
 def moe_topk(logits: np.ndarray, ksel: int):

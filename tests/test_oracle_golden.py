@@ -322,3 +322,20 @@ def test_moe_ffn_is_the_composition(orc, pkg):
             dv = orc.matvec_kq(down[e * gb:(e + 1) * gb], Q4_K, d, nff, act.astype(np.float32))
             want[t] += wgt[t, j] * dv
     assert np.max(np.abs(y - want)) <= 2e-6 * np.max(np.abs(want))
+
+
+def test_rmsnorm_and_activations_closed_forms(orc):
+    """rmsnorm (crates/ojas-cpu/src/cpu_math.rs:456-460) and the FFN activations (:486, :497-501)
+    against their textbook forms in float64."""
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(777).astype(np.float32) * 2.5
+    w = (1.0 + 0.2 * rng.standard_normal(777)).astype(np.float32)
+    got = orc.rmsnorm(x, w, 1e-5)
+    want = x.astype(np.float64) / np.sqrt(np.mean(x.astype(np.float64) ** 2) + 1e-5) * w
+    assert np.max(np.abs(got - want)) <= 5e-7 * np.max(np.abs(want))
+    assert np.allclose(orc.rmsnorm(np.full(64, 3.0, np.float32), np.ones(64, np.float32), 0.0), 1.0, atol=1e-7)
+    g = np.array([-20.0, -3.0, -0.5, 0.0, 0.5, 3.0, 20.0], np.float32)
+    g64 = g.astype(np.float64)
+    assert np.allclose(orc.ffn_act(g, 0), g64 / (1.0 + np.exp(-g64)), rtol=1e-6, atol=1e-12)
+    gelu = 0.5 * g64 * (1.0 + np.tanh(0.7978845608028654 * g64 * (1.0 + 0.044715 * g64 * g64)))
+    assert np.allclose(orc.ffn_act(g, 1), gelu, rtol=2e-6, atol=1e-7)
