@@ -67,6 +67,7 @@ enum { OJH_X_F32 = 0, OJH_X_BF16 = 1, OJH_X_F16 = 2 };
  *   OJH_ACT_AUTO  — OJH_ACT_Q8K for K-quant GEMV-shaped calls, OJH_ACT_FLOAT above the crossover. */
 enum { OJH_ACT_AUTO = 0, OJH_ACT_Q8K = 1, OJH_ACT_FLOAT = 2, OJH_ACT_FLOAT_EXACT = 3 };
 
+typedef struct ojh_gguf ojh_gguf;     /* an open GGUF file: metadata + tensor index */
 typedef struct ojh_device ojh_device; /* one GPU + one stream + loaded families */
 typedef struct ojh_buf ojh_buf;       /* device allocation with a known size */
 typedef struct ojh_lin ojh_lin;       /* a weight matrix W[N,K] in its GGUF block bytes */
@@ -249,6 +250,29 @@ int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint32_t d
                 uint32_t n_expert, uint32_t ksel, const ojh_buf *idx, const ojh_buf *wgt,
                 const ojh_lin *gate, const ojh_lin *up, const ojh_lin *down, ojh_buf *y,
                 int accum, int act_mode);
+
+/* ---- GGUF files -> device (no GPU needed for the reader itself) --------------------------------
+ * `Gguf::open` / `tensor_meta` / `read_tensor_raw` (crates/ojas-formats/src/gguf.rs:100-206, 297-339,
+ * 440-452, 551-556): versions 2 and 3, the reference's header limits, `general.alignment`, extents
+ * validated against the file length.  Split models (split.count > 1) are refused.
+ * `ojh_gguf_tensor_meta`: dims padded with 1 to four entries; `bytes` is 0 for a type whose on-disk
+ * size this reader does not know (`stored_bytes`, gguf.rs:563-591). */
+int ojh_gguf_open(const char *path, ojh_gguf **out);
+int ojh_gguf_close(ojh_gguf *g);
+int ojh_gguf_tensor_count(const ojh_gguf *g);
+const char *ojh_gguf_tensor_name(const ojh_gguf *g, int i);
+int ojh_gguf_tensor_meta(const ojh_gguf *g, const char *name, uint32_t *ggml_type, uint32_t *n_dims,
+                         uint64_t dims[4], uint64_t *file_offset, uint64_t *bytes);
+int ojh_gguf_meta_u64(const ojh_gguf *g, const char *key, uint64_t *out);
+int ojh_gguf_meta_str(const ojh_gguf *g, const char *key, char *out, size_t cap);
+int ojh_gguf_read_raw(ojh_gguf *g, const char *name, void *dst, uint64_t cap);
+
+/* `Lin::load` (crates/ojas-cuda/src/qwen35.rs:174-201): the named tensors, which must share K
+ * (dims[0]) and the GGUF type, stacked along N into one device allocation in the file's own
+ * block bytes (Q8_0 / Q4_K / Q6_K with K a whole number of blocks; anything else is refused —
+ * the reference dequantizes such groups to f16, which is outside this library).  The file is
+ * streamed through a pinned staging buffer; no host copy of the tensor is kept. */
+int ojh_lin_load(ojh_device *dev, ojh_gguf *g, const char *const *names, int count, ojh_lin **out);
 
 #ifdef __cplusplus
 }

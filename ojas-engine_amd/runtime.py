@@ -104,6 +104,15 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_mm": (i32, [vp, vp, sz, i32, vp, vp, sz, vp, u32, i32, i32]),
         "ojh_mm_q8k": (i32, [vp, vp, vp, vp, vp, sz, vp, u32, i32]),
         "ojh_mm_q8k_multi": (i32, [vp, vp, vp, i32, vp, vp, vp]),
+        "ojh_gguf_open": (i32, [C.c_char_p, vp]),
+        "ojh_gguf_close": (i32, [vp]),
+        "ojh_gguf_tensor_count": (i32, [vp]),
+        "ojh_gguf_tensor_name": (C.c_char_p, [vp, i32]),
+        "ojh_gguf_tensor_meta": (i32, [vp, C.c_char_p, vp, vp, vp, vp, vp]),
+        "ojh_gguf_meta_u64": (i32, [vp, C.c_char_p, vp]),
+        "ojh_gguf_meta_str": (i32, [vp, C.c_char_p, vp, sz]),
+        "ojh_gguf_read_raw": (i32, [vp, C.c_char_p, vp, C.c_uint64]),
+        "ojh_lin_load": (i32, [vp, vp, vp, i32, vp]),
         "ojh_rmsnorm_quant_q8k": (i32, [vp, vp, sz, vp, C.c_float, u32, u32, vp, vp, vp]),
         "ojh_ffn_gu_q8k": (i32, [vp, vp, vp, vp, vp, vp, sz, i32]),
         "ojh_relayout_q4k_q4l": (i32, [vp, vp, sz, u32, u32, vp, vp, vp]),
@@ -128,6 +137,63 @@ def load_library(path: str | None = None) -> C.CDLL:
     if path is None:
         _lib = L
     return L
+
+
+class Gguf:
+    """An open GGUF file (metadata + tensor index), the shape of the reference's `Gguf`
+    (crates/ojas-formats/src/gguf.rs:297-339, 440-452, 551-556).  Needs no GPU."""
+
+    def __init__(self, path: str):
+        self._L = load_library()
+        h = C.c_void_p()
+        rc = self._L.ojh_gguf_open(os.fsencode(path), C.byref(h))
+        if rc:
+            raise OjasHipError(rc, self._L.ojh_last_error().decode())
+        self.handle = h
+
+    def _check(self, rc: int) -> None:
+        if rc:
+            raise OjasHipError(rc, self._L.ojh_last_error().decode())
+
+    def close(self) -> None:
+        if self.handle:
+            self._L.ojh_gguf_close(self.handle)
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def tensor_names(self) -> list[str]:
+        return [self._L.ojh_gguf_tensor_name(self.handle, i).decode() for i in range(self._L.ojh_gguf_tensor_count(self.handle))]
+
+    def tensor_meta(self, name: str):
+        """(dims, ggml_type, absolute file offset, raw byte length)."""
+        ty, nd, off, nb = C.c_uint32(), C.c_uint32(), C.c_uint64(), C.c_uint64()
+        dims = (C.c_uint64 * 4)()
+        self._check(self._L.ojh_gguf_tensor_meta(self.handle, name.encode(), C.byref(ty), C.byref(nd), dims, C.byref(off), C.byref(nb)))
+        return list(dims[:nd.value]), ty.value, off.value, nb.value
+
+    def meta_u64(self, key: str) -> int:
+        v = C.c_uint64()
+        self._check(self._L.ojh_gguf_meta_u64(self.handle, key.encode(), C.byref(v)))
+        return v.value
+
+    def meta_str(self, key: str) -> str:
+        buf = C.create_string_buffer(4096)
+        self._check(self._L.ojh_gguf_meta_str(self.handle, key.encode(), buf, 4096))
+        return buf.value.decode()
+
+    def read_tensor_raw(self, name: str):
+        """(dims, ggml_type, bytes) — `read_tensor_raw`."""
+        dims, ty, _, nb = self.tensor_meta(name)
+        if nb == 0:
+            raise OjasHipError(4, f"read_tensor_raw: unsupported GGUF type {ty}")
+        out = np.empty(nb, np.uint8)
+        self._check(self._L.ojh_gguf_read_raw(self.handle, name.encode(), C.c_void_p(out.ctypes.data), nb))
+        return dims, ty, out
 
 
 def manifest() -> list[tuple[str, str, int, int]]:
@@ -349,6 +415,15 @@ class HipGpu:
         h = C.c_void_p()
         self._check(self._L.ojh_lin_wrap(self._dev, ty, n, k, raw.handle, off, C.byref(h)))
         return Lin(self, h, ty, n, k, keep=raw)
+
+    def lin_load(self, g: Gguf, names: list[str]) -> Lin:
+        """`Lin::load`: the named tensors stacked along N, kept in the file's block bytes."""
+        arr = (C.c_char_p * len(names))(*[n.encode() for n in names])
+        h = C.c_void_p()
+        self._check(self._L.ojh_lin_load(self._dev, g.handle, arr, len(names), C.byref(h)))
+        n = sum((g.tensor_meta(nm)[0] + [1])[1] for nm in names)
+        dims, ty, _, _ = g.tensor_meta(names[0])
+        return Lin(self, h, ty, n, dims[0])
 
     def mm(self, x: Buf, w: Lin, y: Buf, m: int = 1, accum: bool = False, *, x_dtype: int = X_F32,
            act_mode: int = ACT_AUTO, bias: Buf | None = None, x_off: int = 0, y_off: int = 0) -> None:
