@@ -121,6 +121,112 @@ __device__ __forceinline__ void gemv_q8k_q4k_body(const signed char* __restrict_
 
 GEMV_Q8K_ENTRIES(q4k, gemv_q8k_q4k_body)
 
+// ------------------------------------------------------------------ Q5_K
+// The Q4_K lane map on 176-byte super-blocks: {f16 d, f16 dmin, scales[12], qh[32], qs[128]}.
+// The fifth bit of weight l of sub-block j is bit j of qh[l] (crates/ojas-cpu/src/cpu_math.rs:638-670),
+// so a lane adds 16 * dot(bit plane, x) to each of its two nibble dots: the 16 qh bytes it needs
+// are those at the positions of its 16 quant bytes within the 32-byte chunk.
+__device__ __forceinline__ float q5k_lane_dot(uint4 hdr, uint4 qs, uint4 qh, uint c, const Q4kFrag& f) {
+    const uint M4 = 0x0F0F0F0Fu, B1 = 0x01010101u;
+    const uint sl = 2u * c, sh = 2u * c + 1u;
+    int il = dot4_i8(qs.x & M4, f.xl.x, 0);
+    il = dot4_i8(qs.y & M4, f.xl.y, il);
+    il = dot4_i8(qs.z & M4, f.xl.z, il);
+    il = dot4_i8(qs.w & M4, f.xl.w, il);
+    int bl = dot4_i8((qh.x >> sl) & B1, f.xl.x, 0);
+    bl = dot4_i8((qh.y >> sl) & B1, f.xl.y, bl);
+    bl = dot4_i8((qh.z >> sl) & B1, f.xl.z, bl);
+    bl = dot4_i8((qh.w >> sl) & B1, f.xl.w, bl);
+    int ih = dot4_i8((qs.x >> 4) & M4, f.xh.x, 0);
+    ih = dot4_i8((qs.y >> 4) & M4, f.xh.y, ih);
+    ih = dot4_i8((qs.z >> 4) & M4, f.xh.z, ih);
+    ih = dot4_i8((qs.w >> 4) & M4, f.xh.w, ih);
+    int bh = dot4_i8((qh.x >> sh) & B1, f.xh.x, 0);
+    bh = dot4_i8((qh.y >> sh) & B1, f.xh.y, bh);
+    bh = dot4_i8((qh.z >> sh) & B1, f.xh.z, bh);
+    bh = dot4_i8((qh.w >> sh) & B1, f.xh.w, bh);
+    uint sc, mn;
+    q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
+    const int isum = (int)(sc & 0xFFu) * (il + 16 * bl) + (int)(sc >> 8) * (ih + 16 * bh);
+    const int msum = (int)(mn & 0xFFu) * f.bl + (int)(mn >> 8) * f.bh;
+    const float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
+    return f.sx * (d * (float)isum - dmin * (float)msum);
+}
+
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_q8k_q5k_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                  const uchar* __restrict__ w, float* __restrict__ y,
+                                                  const float* __restrict__ bs, uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 >= N) return;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (uint sb = g; sb < nsb; sb += 8u) {
+        uint4 hdr[R], qs[R], qh[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uchar* blk = w + ((size_t)min(row0 + r, N - 1u) * nsb + sb) * Q5K_BYTES;
+            hdr[r] = *(const uint4*)blk;
+            qh[r] = *(const uint4*)(blk + 16u + (l & 1u) * 16u);
+            qs[r] = *(const uint4*)(blk + 48u + l * 16u);
+        }
+        Q4kFrag f = q4k_load_frag(xq, xs, sb, l);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += q5k_lane_dot(hdr[r], qs[r], qh[r], c, f);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float t = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, t);
+    }
+}
+
+GEMV_Q8K_ENTRIES(q5k, gemv_q8k_q5k_body)
+
+template <int MT>
+__device__ __forceinline__ void gemv_q8k_q5k_m_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                    const uchar* __restrict__ w, float* __restrict__ y,
+                                                    uint K, uint N, uint M, uint ACC) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    for (uint m0 = 0; m0 < M; m0 += MT) {
+        float acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; t++) acc[t] = 0.0f;
+        for (uint sb = g; sb < nsb; sb += 8u) {
+            const uchar* blk = w + ((size_t)row * nsb + sb) * Q5K_BYTES;
+            const uint4 hdr = *(const uint4*)blk, qh = *(const uint4*)(blk + 16u + (l & 1u) * 16u);
+            const uint4 qs = *(const uint4*)(blk + 48u + l * 16u);
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                uint m = min(m0 + t, M - 1u);
+                Q4kFrag f = q4k_load_frag(xq + (size_t)m * nsb * 256u, xs + (size_t)m * nsb, sb, l);
+                acc[t] += q5k_lane_dot(hdr, qs, qh, c, f);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            float s = wave_sum(acc[t]);
+            if (lane == 0 && m0 + t < M) {
+                float* o = y + (size_t)(m0 + t) * N + row;
+                *o = ACC ? *o + s : s;
+            }
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+gemv_q8k_q5k_m(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    if (M <= 2) gemv_q8k_q5k_m_body<2>(xq, xs, w, y, K, N, M, ACC);
+    else if (M <= 4) gemv_q8k_q5k_m_body<4>(xq, xs, w, y, K, N, M, ACC);
+    else gemv_q8k_q5k_m_body<8>(xq, xs, w, y, K, N, M, ACC);
+}
+
 // ---- several projections of one activation in one launch -------------------------------------
 //   gemv_q8k_q4k_x4_{r1,r2}(xq, xs, w0, w1, w2, w3, y0, y1, y2, y3, K, E0, E1, E2, E3)
 // Up to four weight tensors (separate allocations, all K wide) share the quantized activation:

@@ -268,6 +268,14 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     void *wp = at(w->raw, w->off), *yp = at(y, y_off);
     uint32_t grid[3] = {1, 1, 1}, block[3] = {256, 1, 1};
 
+    // Q5_K has the CPU path's arithmetic only (dot_q5k over int8 activations); no floating-point
+    // matvec and no MFMA tile read it, at any token count.
+    if (w->type == OJH_Q5_K) {
+        if (act_mode == OJH_ACT_FLOAT || act_mode == OJH_ACT_FLOAT_EXACT)
+            return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: Q5_K rows take int8 activations only (OJH_ACT_Q8K or OJH_ACT_AUTO)");
+        act_mode = OJH_ACT_Q8K;
+    }
+
     // Above the crossover the MFMA tile wins over streaming the weights once per few tokens
     // (the reference switches at 8 rows, crates/ojas-models/src/decoder/dispatch.rs:70-75).
     if (m >= dev->gemm_min_m && act_mode != OJH_ACT_Q8K && K % 64 == 0 && (uint64_t)m * K < 0x7FFFFFFFull &&

@@ -88,6 +88,21 @@ def q4k_weights(n: int, k: int, *names) -> np.ndarray:
     return out.reshape(-1)
 
 
+def q5k_weights(n: int, k: int, *names) -> np.ndarray:
+    """Q5_K rows: the Q4_K header, 32 bytes of fifth bits, 128 bytes of nibbles, all uniform."""
+    g = rng(*names)
+    nb = n * (k // 256)
+    out = np.empty((nb, 176), np.uint8)
+    hdr = np.empty((nb, 2), np.uint16)
+    hdr[:, 0] = _f16_abs_normal(g, nb, 0.01)
+    hdr[:, 1] = _f16_abs_normal(g, nb, 0.01)
+    out[:, 0:4] = hdr.view(np.uint8).reshape(nb, 4)
+    out[:, 4:16] = pack_scales_k4(g.integers(0, 64, size=(nb, 8), dtype=np.uint8),
+                                  g.integers(0, 64, size=(nb, 8), dtype=np.uint8))
+    out[:, 16:] = g.integers(0, 256, size=(nb, 160), dtype=np.uint8)
+    return out.reshape(-1)
+
+
 def q6k_weights(n: int, k: int, *names) -> np.ndarray:
     """Q6_K rows: uniform 6-bit codes, int8 sub-scales uniform in [-32,31], d = f16(|N(0,0.01)|)."""
     g = rng(*names)
@@ -102,7 +117,7 @@ def q6k_weights(n: int, k: int, *names) -> np.ndarray:
 
 
 def weights(ty: int, n: int, k: int, *names) -> np.ndarray:
-    return {Q8_0: q80_weights, Q4_K: q4k_weights, Q6_K: q6k_weights}[ty](n, k, *names)
+    return {Q8_0: q80_weights, Q4_K: q4k_weights, Q5_K: q5k_weights, Q6_K: q6k_weights}[ty](n, k, *names)
 
 
 # ------------------------------------------------------------------ the reference tests' procedures

@@ -12,8 +12,8 @@ import pytest
 from conftest import peak_err
 
 pytestmark = pytest.mark.gpu
-Q8_0, Q4_K, Q6_K = 8, 12, 14
-TAG = {Q8_0: "q80", Q4_K: "q4k", Q6_K: "q6k"}
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+TAG = {Q8_0: "q80", Q4_K: "q4k", Q5_K: "q5k", Q6_K: "q6k"}
 TOL_Q8K = 1e-3     # the parity bar against the CPU reference
 TOL_Q8K_SEEN = 2e-5
 TOL_FLOAT = 1e-4   # reference bound is 2e-3
@@ -54,7 +54,7 @@ def test_quantize_q8k_bf16_input(gpu, orc, pkg):
         assert np.array_equal(gq[t], wq)
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("n,k", [(13, 256), (64, 512), (1024, 4096), (333, 2560), (96, 14336), (4099, 4096)])
 def test_q8k_matvec_matches_cpu_reference(gpu, orc, pkg, ty, n, k):
     w, x = _inputs(pkg, ty, n, k, "a")
@@ -112,13 +112,15 @@ def test_q80_closed_form_rows_with_guards(gpu, pkg):
     assert np.max(np.abs(got[2:-2] - want)) < 2e-4
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("mode", ["float", "q8k"])
 def test_bias_accum_and_batched_variants(gpu, orc, pkg, ty, mode):
     """The five checks of crates/ojas-models/examples/nat_gemv_gate.rs:36-163: plain, bias
     (1000 + i), accumulate onto a seeded y, batched M=3 with different rows, batched accumulate."""
     if ty == Q8_0 and mode == "q8k":
         pytest.skip("Q8_0 keeps f32 activations in the CPU reference")
+    if ty == Q5_K and mode == "float":
+        pytest.skip("Q5_K has the int8-activation matvec only")
     n, k, m = 200, 1024, 3
     w = pkg.synth.weights(ty, n, k, "var", ty)
     xs = pkg.synth.normal_f32(m * k, "var", "x").reshape(m, k)
@@ -301,3 +303,26 @@ def test_q6k_few_tokens_staged_and_streamed_forms_agree(gpu, orc, pkg, m, n, k, 
         with pytest.raises(pkg.OjasHipError, match="do not fit"):
             gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_mx", [(xq, 0), (xs, 0), (gpu.upload_bytes(w), 0), (y2, 0)],
                          [k, n, m, 0], [8, 1, 1], [256, 1, 1])
+
+
+def test_q5k_takes_the_int8_path_at_every_token_count(gpu, orc, pkg):
+    """Q5_K has dot_q5k's arithmetic (crates/ojas-cpu/src/cpu_math.rs:638-670) and nothing else:
+    AUTO resolves to it for one token and for a prefill-sized batch alike, a floating-point
+    contract is refused, and the wide-row form (N >= 32768) agrees with the oracle too."""
+    n, k = 300, 1024
+    w = pkg.synth.weights(Q5_K, n, k, "q5k", "any-m")
+    lin = gpu.lin(Q5_K, n, k, w)
+    for m in (1, 9, 40):
+        xs = pkg.synth.normal_f32(m * k, "q5k", "x", m).reshape(m, k)
+        yd = gpu.alloc(m * n)
+        gpu.mm(gpu.upload(xs), lin, yd, m, act_mode=pkg.ACT_AUTO)
+        want = np.stack([orc.matvec_kq(w, Q5_K, n, k, xs[t]) for t in range(m)])
+        assert peak_err(gpu.read(yd, m * n).reshape(m, n), want) <= TOL_Q8K_SEEN
+    for act in (pkg.ACT_FLOAT, pkg.ACT_FLOAT_EXACT):
+        with pytest.raises(pkg.OjasHipError):
+            gpu.mm(gpu.upload(xs), lin, yd, 1, act_mode=act)
+    n, k = 33000, 256
+    w, x = _inputs(pkg, Q5_K, n, k, "wide")
+    yd = gpu.alloc(n)
+    gpu.mm(gpu.upload(x), gpu.lin(Q5_K, n, k, w), yd, 1, act_mode=pkg.ACT_Q8K)
+    assert peak_err(gpu.read(yd, n), orc.matvec_kq(w, Q5_K, n, k, x)) <= TOL_Q8K_SEEN
