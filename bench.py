@@ -317,7 +317,7 @@ def extras(gpu, pkg, lin_q) -> dict:
         fl = 2.0 * T * ksel * 3 * nff * d
         moe[f"T{T}"] = {"us": round(us, 1), "distinct_experts": distinct, "gbs": round(b / us / 1e3, 1),
                         "tflops": round(fl / us / 1e6, 2)}
-    out["moe_ffn_q4k_128x_top8"] = {"timed": "router + quantize + group + gate/up + quantize + down + combine", **moe}
+    out["moe_ffn_q4k_128x_top8"] = {"timed": "router + expert FFN (T <= 8: gate/up and down launches addressed by assignment; above: quantize, group, gate/up, quantize, down, combine)", **moe}
     del gate, up, down
     # ---- speculative verify on a Q6_K output head 151936 x 4096, bf16 activations
     n, k = 151936, 4096

@@ -22,20 +22,23 @@
 //   moe_gu_q4k_m(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA)   grid (ceil(N/8), E)
 //   moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)            grid (ceil(N/16), E)
 //   moe_combine(dv, wgt, y, T, KSEL, D, ACC)                 grid ceil(T*D/256)
+//   moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)   grid (ceil(N/8), NA): few tokens, f32 in
+//   moe_down_q4k_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)  grid (ceil(N/8), T): down + weighted sum
 //   moe_gu_q4k_mm / moe_down_q4k_mm (same arguments as the _m entries)
 //                                                            grid (ceil(N/16), E): the int8 matrix-core form
 #include "ojk_common.h"
 #include "ojk_q4k_dot.h"
 
 // ------------------------------------------------------------------ router
-__device__ __forceinline__ void moe_topk_body(const float* __restrict__ lg, uint* __restrict__ idx,
-                                              float* __restrict__ wgt, uint E, uint KSEL) {
-    // one wave per token; lane l owns experts l, l+64, ... (E <= 1024)
+template <int NI>
+__device__ __forceinline__ void moe_topk_lanes(const float* __restrict__ lg, uint* __restrict__ idx,
+                                               float* __restrict__ wgt, uint E, uint KSEL) {
+    // one wave per token; lane l owns experts l, l+64, ... (E <= 64 NI)
     const uint lane = threadIdx.x & 63u;
-    float p[16];
+    float p[NI];
     float mx = -3.4028235e38f;
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
+    for (int i = 0; i < NI; i++) {
         uint e = lane + 64u * i;
         p[i] = e < E ? lg[e] : -3.4028235e38f;
         mx = fmaxf(mx, p[i]);
@@ -43,14 +46,14 @@ __device__ __forceinline__ void moe_topk_body(const float* __restrict__ lg, uint
     mx = wave_max(mx);
     float sum = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
+    for (int i = 0; i < NI; i++) {
         uint e = lane + 64u * i;
         p[i] = e < E ? expf(p[i] - mx) : -1.0f;
         if (e < E) sum += p[i];
     }
     sum = wave_sum(sum);
 #pragma unroll
-    for (int i = 0; i < 16; i++)
+    for (int i = 0; i < NI; i++)
         if (lane + 64u * i < E) p[i] = p[i] / sum;
     float wsum = 0.0f, mine = 0.0f;
     uint mine_idx = 0;
@@ -58,7 +61,7 @@ __device__ __forceinline__ void moe_topk_body(const float* __restrict__ lg, uint
         float bv = -1.0f;
         uint bi = 0xFFFFFFFFu;
 #pragma unroll
-        for (int i = 0; i < 16; i++) {  // ascending expert index within the lane: '>' keeps the lowest
+        for (int i = 0; i < NI; i++) {  // ascending expert index within the lane: '>' keeps the lowest
             if (p[i] > bv) { bv = p[i]; bi = lane + 64u * i; }
         }
         float m2 = wave_max(bv);
@@ -74,13 +77,20 @@ __device__ __forceinline__ void moe_topk_body(const float* __restrict__ lg, uint
         wsum += m2;
         if (lane == j) { mine = m2; mine_idx = win; }
 #pragma unroll
-        for (int i = 0; i < 16; i++)
+        for (int i = 0; i < NI; i++)
             if (lane + 64u * i == win) p[i] = -1.0f;
     }
     if (lane < KSEL) {
         idx[lane] = mine_idx;
         wgt[lane] = mine / wsum;
     }
+}
+
+__device__ __forceinline__ void moe_topk_body(const float* __restrict__ lg, uint* __restrict__ idx,
+                                              float* __restrict__ wgt, uint E, uint KSEL) {
+    if (E <= 128u) moe_topk_lanes<2>(lg, idx, wgt, E, KSEL);
+    else if (E <= 256u) moe_topk_lanes<4>(lg, idx, wgt, E, KSEL);
+    else moe_topk_lanes<16>(lg, idx, wgt, E, KSEL);
 }
 
 extern "C" __global__ void __launch_bounds__(64)
@@ -242,6 +252,155 @@ moe_down_q4k_m(const signed char* __restrict__ aq, const float* __restrict__ as_
                 if (lane == 0 && row0 + r < N) dv[(size_t)a * N + row0 + r] = s;
             }
         }
+    }
+}
+
+// ------------------------------------------------------------------ decode: a few tokens, two launches
+// With one or a few tokens almost every assignment has its expert to itself, so grouping buys
+// nothing and the six launches of the grouped pipeline cost more than the bytes.  Here a workgroup
+// is addressed by assignment (gate/up) or by token (down), quantizes the activations it needs into
+// LDS itself, and the down projection owns all KSEL slots of its rows, so the router-weighted sum
+// happens in the same launch, in slot order.  The arithmetic is that of the grouped integer-dot
+// kernels step for step: results are bit-identical.
+#define MOE_DEC_GU_K 8192u      // longest row of gate/up the decode form stages (bytes of int8 in LDS)
+#define MOE_DEC_DOWN_ACT 32768u // most KSEL * K int8 activations the down launch stages
+
+// All 256 threads: quantize n (a multiple of 256) f32 values into q (int8) and s (one scale per
+// 256 values) with quant_q8k's rule (crates/ojas-cpu/src/cpu_math.rs:539-563), the operations of
+// the quantize_q8k kernel.  A thread owns 8 consecutive values, 32 lanes side by side a segment.
+__device__ __forceinline__ void block_quant_q8k(const float* __restrict__ x, uint n, signed char* q, float* s) {
+    for (uint base = threadIdx.x * 8u; base < n; base += 2048u) {
+        const float4 a = *(const float4*)(x + base), b = *(const float4*)(x + base + 4u);
+        float m = fmaxf(amax4(a), amax4(b));
+        m = fmaxf(m, dpp_f32<OJK_DPP_QUAD_XOR1>(m));
+        m = fmaxf(m, dpp_f32<OJK_DPP_QUAD_XOR2>(m));
+        m = fmaxf(m, dpp_f32<OJK_DPP_ROW_HALF_MIRROR>(m));
+        m = fmaxf(m, dpp_f32<OJK_DPP_ROW_MIRROR>(m));
+        m = fmaxf(m, __shfl_xor(m, 16, 64));
+        const float scale = m > 0.0f ? __fdiv_rn(m, 127.0f) : 1.0f;
+        const float inv = __fdiv_rn(1.0f, scale);
+        *(uint2*)(q + base) = make_uint2(q8k_pack4(a, inv), q8k_pack4(b, inv));
+        if ((threadIdx.x & 31u) == 0) s[base >> 8] = scale;
+    }
+}
+
+// Block (rb, a): 4 waves x 2 rows of gate and up of expert idx[a] against token a / KSEL.
+extern "C" __global__ void __launch_bounds__(256)
+moe_gu_q4k_dec(const float* __restrict__ x, const uchar* __restrict__ wg, const uchar* __restrict__ wu,
+               float* __restrict__ act, const uint* __restrict__ idx, uint K, uint N, uint KSEL, uint NA, uint E) {
+    __shared__ __align__(16) signed char xq[MOE_DEC_GU_K];
+    __shared__ float xs[MOE_DEC_GU_K / 256u];
+    const uint a = blockIdx.y;
+    const uint e = min(idx[a], E - 1u), t = a / KSEL;
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = min((blockIdx.x * 4u + (threadIdx.x >> 6)) * 2u, N - 1u);   // surplus waves repeat the last row
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    const size_t rb = (size_t)nsb * Q4K_BYTES;
+    const uchar* g0 = wg + ((size_t)e * N + row0) * rb;
+    const uchar* u0 = wu + ((size_t)e * N + row0) * rb;
+    const bool two = row0 + 1u < N;
+    const size_t r1 = two ? rb : 0;
+    // the first step's weights are on their way while the activations are quantized
+    const size_t o0 = (size_t)min(g, nsb - 1u) * Q4K_BYTES, q0 = o0 + 16u + l * 16u;
+    uint4 hg0 = *(const uint4*)(g0 + o0), qg0 = *(const uint4*)(g0 + q0);
+    uint4 hg1 = *(const uint4*)(g0 + r1 + o0), qg1 = *(const uint4*)(g0 + r1 + q0);
+    uint4 hu0 = *(const uint4*)(u0 + o0), qu0 = *(const uint4*)(u0 + q0);
+    uint4 hu1 = *(const uint4*)(u0 + r1 + o0), qu1 = *(const uint4*)(u0 + r1 + q0);
+    block_quant_q8k(x + (size_t)t * K, K, xq, xs);
+    __syncthreads();
+    float vg0 = 0.0f, vg1 = 0.0f, vu0 = 0.0f, vu1 = 0.0f;
+    for (uint sb = g; sb < nsb; sb += 8u) {
+        const Q4kFrag f = q4k_load_frag(xq, xs, sb, l);
+        vg0 += q4k_lane_dot(hg0, qg0, c, f);
+        vg1 += q4k_lane_dot(hg1, qg1, c, f);
+        vu0 += q4k_lane_dot(hu0, qu0, c, f);
+        vu1 += q4k_lane_dot(hu1, qu1, c, f);
+        if (sb + 8u < nsb) {
+            const size_t o = (size_t)(sb + 8u) * Q4K_BYTES, oq = o + 16u + l * 16u;
+            hg0 = *(const uint4*)(g0 + o); qg0 = *(const uint4*)(g0 + oq);
+            hg1 = *(const uint4*)(g0 + r1 + o); qg1 = *(const uint4*)(g0 + r1 + oq);
+            hu0 = *(const uint4*)(u0 + o); qu0 = *(const uint4*)(u0 + oq);
+            hu1 = *(const uint4*)(u0 + r1 + o); qu1 = *(const uint4*)(u0 + r1 + oq);
+        }
+    }
+    vg0 = wave_sum(vg0); vg1 = wave_sum(vg1); vu0 = wave_sum(vu0); vu1 = wave_sum(vu1);
+    if (lane == 0) {
+        float* o_ = act + (size_t)a * N + row0;
+        o_[0] = (vg0 / (1.0f + expf(-vg0))) * vu0;
+        if (two) o_[1] = (vg1 / (1.0f + expf(-vg1))) * vu1;
+    }
+}
+
+// Block (rb, t): 8 rows of the down projection for every slot of token t, 2 rows per wave.  The
+// workgroup quantizes the token's KSEL act vectors into LDS.  An expert's row is short (K / 256 <= 8
+// super-blocks, three at the usual 768), so a wave's eight lane groups take (slot, super-block)
+// pairs side by side instead of one slot at a time: group sums go through LDS, lane j rebuilds
+// slot j's dot with the association of wave_sum, and the slots are added in order,
+//     y[t][row] (=, +=) sum_j wgt[t][j] * (Wd_{idx[t][j]} act[t][j])[row].
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q4k_dec(const float* __restrict__ act, const uchar* __restrict__ wd, const uint* __restrict__ idx,
+                 const float* __restrict__ wgt, float* __restrict__ y, uint K, uint N, uint KSEL, uint E, uint ACC) {
+    __shared__ __align__(16) signed char aq[MOE_DEC_DOWN_ACT];
+    __shared__ float as_[MOE_DEC_DOWN_ACT / 256u];
+    __shared__ uint s_idx[64];
+    __shared__ __align__(16) float part[4][2][64][8];   // [wave][row][slot][super-block] group sums
+    const uint t = blockIdx.y, lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint row0 = min(blockIdx.x * 8u + wave * 2u, N - 1u);   // surplus waves repeat the last row
+    const bool two = row0 + 1u < N;
+    const uint nsb = K >> 8, G = lane >> 3, l = lane & 7u, c = l >> 1;
+    const size_t rb = (size_t)nsb * Q4K_BYTES, r1 = two ? rb : 0;
+    const uint* ti = idx + (size_t)t * KSEL;
+    const uint U = KSEL * nsb;
+    // the first pass's weights are on their way while the activations are quantized
+    uint u = min(G, U - 1u), j = u / nsb, sb = u - j * nsb;
+    const uchar* w = wd + (((size_t)min(ti[j], E - 1u) * N + row0) * nsb + sb) * Q4K_BYTES;
+    uint4 h0 = *(const uint4*)w, p0 = *(const uint4*)(w + 16u + l * 16u);
+    uint4 h1 = *(const uint4*)(w + r1), p1 = *(const uint4*)(w + r1 + 16u + l * 16u);
+    if (threadIdx.x < KSEL) s_idx[threadIdx.x] = min(ti[threadIdx.x], E - 1u);
+    block_quant_q8k(act + (size_t)t * KSEL * K, KSEL * K, aq, as_);
+    __syncthreads();
+    for (uint u0 = 0; u0 < U; u0 += 8u) {
+        const bool on = u0 + G < U;
+        const uint un = min(u0 + 8u + G, U - 1u), jn = un / nsb, sbn = un - jn * nsb;
+        const uchar* wn = wd + (((size_t)s_idx[jn] * N + row0) * nsb + sbn) * Q4K_BYTES;
+        const uint4 nh0 = *(const uint4*)wn, np0 = *(const uint4*)(wn + 16u + l * 16u);
+        const uint4 nh1 = *(const uint4*)(wn + r1), np1 = *(const uint4*)(wn + r1 + 16u + l * 16u);
+        const Q4kFrag f = q4k_load_frag(aq + (size_t)j * K, as_ + (size_t)j * nsb, sb, l);
+        const float v0 = oct_sum(q4k_lane_dot(h0, p0, c, f)), v1 = oct_sum(q4k_lane_dot(h1, p1, c, f));
+        if (on && l == 0) {
+            part[wave][0][j][sb] = v0;
+            part[wave][1][j][sb] = v1;
+        }
+        j = jn; sb = sbn; h0 = nh0; p0 = np0; h1 = nh1; p1 = np1;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // lane j: slot j's two dots, summed like wave_sum sums the eight groups of a wave
+    float d0 = 0.0f, d1 = 0.0f;
+    if (lane < KSEL) {
+        float s0[8], s1[8];
+#pragma unroll
+        for (uint k = 0; k < 8; k++) {
+            s0[k] = k < nsb ? part[wave][0][lane][k] : 0.0f;
+            s1[k] = k < nsb ? part[wave][1][lane][k] : 0.0f;
+        }
+        d0 = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s0[4] + s0[5]) + (s0[6] + s0[7]));
+        d1 = ((s1[0] + s1[1]) + (s1[2] + s1[3])) + ((s1[4] + s1[5]) + (s1[6] + s1[7]));
+    }
+    float acc0 = 0.0f, acc1 = 0.0f;
+    if (ACC) {
+        acc0 = y[(size_t)t * N + row0];
+        acc1 = y[(size_t)t * N + row0 + (two ? 1u : 0u)];
+    }
+    for (uint k = 0; k < KSEL; k++) {
+        const float wk = wgt[(size_t)t * KSEL + k];
+        acc0 += wk * __int_as_float(__builtin_amdgcn_readlane(__float_as_int(d0), k));
+        acc1 += wk * __int_as_float(__builtin_amdgcn_readlane(__float_as_int(d1), k));
+    }
+    if (lane == 0) {
+        y[(size_t)t * N + row0] = acc0;
+        if (two) y[(size_t)t * N + row0 + 1u] = acc1;
     }
 }
 

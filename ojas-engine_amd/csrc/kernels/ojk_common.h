@@ -53,8 +53,17 @@ __device__ __forceinline__ int dpp_i32(int v) {
     return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
 }
 
+// The sums below start from a rounded value: without the empty asm the compiler contracts a
+// product feeding the first step into fma(a, b, neighbour's product), which rounds differently
+// from lane to lane and from one call site to the next.
+__device__ __forceinline__ float rounded(float v) {
+    asm("" : "+v"(v));
+    return v;
+}
+
 // Sum over the 16 lanes of a DPP row; every lane of the row ends with the row total.
 __device__ __forceinline__ float row16_sum(float v) {
+    v = rounded(v);
     v += dpp_f32<OJK_DPP_QUAD_XOR1>(v);
     v += dpp_f32<OJK_DPP_QUAD_XOR2>(v);
     v += dpp_f32<OJK_DPP_ROW_HALF_MIRROR>(v);
@@ -63,6 +72,7 @@ __device__ __forceinline__ float row16_sum(float v) {
 }
 // Sum over groups of 8 adjacent lanes; every lane of the group ends with the group total.
 __device__ __forceinline__ float oct_sum(float v) {
+    v = rounded(v);
     v += dpp_f32<OJK_DPP_QUAD_XOR1>(v);
     v += dpp_f32<OJK_DPP_QUAD_XOR2>(v);
     v += dpp_f32<OJK_DPP_ROW_HALF_MIRROR>(v);

@@ -33,6 +33,42 @@ __device__ __forceinline__ Q4kFrag q4k_load_frag(const signed char* xq, const fl
     return f;
 }
 
+// The same fragment straight from f32 activations: the eight lanes of a group hold the 256 values
+// of super-block `sb` between them, so the segment's quantizer (scale = amax/127, 1 if all zero;
+// q = clamp(round_half_away(v * (1/scale))), crates/ojas-cpu/src/cpu_math.rs:539-563) needs one
+// maximum over the group and nothing outside registers.  Same operations as the quantize_q8k
+// kernel, hence the same bytes.
+__device__ __forceinline__ uint q8k_pack4(float4 v, float inv) {
+    float a = fminf(fmaxf(roundf(__fmul_rn(v.x, inv)), -127.0f), 127.0f);
+    float b = fminf(fmaxf(roundf(__fmul_rn(v.y, inv)), -127.0f), 127.0f);
+    float c = fminf(fmaxf(roundf(__fmul_rn(v.z, inv)), -127.0f), 127.0f);
+    float d = fminf(fmaxf(roundf(__fmul_rn(v.w, inv)), -127.0f), 127.0f);
+    return ((uint)(int)a & 0xFFu) | (((uint)(int)b & 0xFFu) << 8) | (((uint)(int)c & 0xFFu) << 16) | ((uint)(int)d << 24);
+}
+
+__device__ __forceinline__ float amax4(float4 v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); }
+
+__device__ __forceinline__ Q4kFrag q4k_quant_frag(const float* x, uint sb, uint l) {
+    const float4* p = (const float4*)(x + (size_t)sb * 256u + (l >> 1) * 64u + (l & 1u) * 16u);
+    float4 lo[4], hi[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { lo[i] = p[i]; hi[i] = p[8 + i]; }
+    float a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) a = fmaxf(a, fmaxf(amax4(lo[i]), amax4(hi[i])));
+    a = fmaxf(a, dpp_f32<OJK_DPP_QUAD_XOR1>(a));
+    a = fmaxf(a, dpp_f32<OJK_DPP_QUAD_XOR2>(a));
+    a = fmaxf(a, dpp_f32<OJK_DPP_ROW_HALF_MIRROR>(a));
+    Q4kFrag f;
+    f.sx = a > 0.0f ? __fdiv_rn(a, 127.0f) : 1.0f;
+    const float inv = __fdiv_rn(1.0f, f.sx);
+    f.xl = make_uint4(q8k_pack4(lo[0], inv), q8k_pack4(lo[1], inv), q8k_pack4(lo[2], inv), q8k_pack4(lo[3], inv));
+    f.xh = make_uint4(q8k_pack4(hi[0], inv), q8k_pack4(hi[1], inv), q8k_pack4(hi[2], inv), q8k_pack4(hi[3], inv));
+    f.bl = bytesum4(f.xl);
+    f.bh = bytesum4(f.xh);
+    return f;
+}
+
 // One lane's 32 weights of one super-block against one activation fragment.
 __device__ __forceinline__ float q4k_lane_dot(uint4 hdr, uint4 qs, uint c, const Q4kFrag& f) {
     const uint M4 = 0x0F0F0F0Fu;

@@ -58,7 +58,9 @@ struct ojh_device {
     int gemv_rows_override = 0;  // OJAS_HIP_GEMV_R
     uint32_t gemm_min_m = 32;    // OJAS_HIP_GEMM_MIN_M: rows from which ojh_mm takes the MFMA tile
     int gemm_split_override = 0; // OJAS_HIP_GEMM_SPLIT
-    int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = integer dots always
+    int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
+                                 // 3 = per-assignment decode form always
+    uint32_t moe_dec_tokens = 8; // OJAS_HIP_MOE_DEC_TOKENS: the decode form serves up to this many tokens
     bool gemm_exact = false;     // OJAS_HIP_GEMM_EXACT: Q4_K prefill through the tile that holds dequant_to_f16 bits
     bool fused_quant = false;    // OJAS_HIP_FUSED_QUANT=1: ojh_mm (m = 1, Q4_K) quantizes x inside the matvec launch
     uint32_t fq_blocks_per_cu = 8; // OJAS_HIP_FQ_BLOCKS: blocks per CU the fused-quantizer matvec aims for

@@ -406,6 +406,8 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
 //   4 moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)                     grid [ceil(N/16), E, 1]
 //   5 moe_combine(dv, wgt, y, T, KSEL, D, ACC)                                    grid [ceil(T*D/256),1,1]
 //   6 moe_gu_q4k_mm, 7 moe_down_q4k_mm: the arguments of 3 and 4, grid [ceil(N/16), E, 1]
+//   8 moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)                      grid [ceil(N/8), NA, 1]
+//   9 moe_down_q4k_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)                  grid [ceil(N/8), T, 1]
 static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                      const uint32_t block[3], size_t need[16], size_t align[16]) {
     int rc;
@@ -464,6 +466,35 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         align[0] = align[2] = 16;
         return OJH_OK;
     }
+    case 8: {   // moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)
+        uint32_t K = c[0], N = c[1], KS = c[2], NA = c[3], E = c[4];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!K || K % 256 || !N || !KS || !NA || NA % KS || !E) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u KSEL=%u NA=%u E=%u", s->name, K, N, KS, NA, E);
+        if (K > 8192) return ojh_fail(OJH_ERR_UNSUPPORTED, "%s: K=%u exceeds the 8192 activations staged in LDS", s->name, K);
+        if (grid[0] != (N + 7) / 8 || grid[1] != NA || grid[2] != 1)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/8), NA, 1]", s->name);
+        need[0] = (size_t)(NA / KS) * K * 4;
+        need[1] = need[2] = (size_t)E * N * (K / 256) * 144;
+        need[3] = (size_t)NA * N * 4;
+        need[4] = (size_t)NA * 4;
+        align[0] = align[1] = align[2] = 16;
+        return OJH_OK;
+    }
+    case 9: {   // moe_down_q4k_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)
+        uint32_t K = c[0], N = c[1], KS = c[2], E = c[3], T = grid[1];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!K || K % 256 || !N || !KS || KS > 64 || !E) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u KSEL=%u (<= 64) E=%u", s->name, K, N, KS, E);
+        if (K > 2048) return ojh_fail(OJH_ERR_UNSUPPORTED, "%s: K=%u exceeds the 2048 (eight super-blocks) a wave takes side by side", s->name, K);
+        if ((uint64_t)KS * K > 32768) return ojh_fail(OJH_ERR_UNSUPPORTED, "%s: KSEL * K = %llu activations exceed the 32768 staged in LDS", s->name, (unsigned long long)KS * K);
+        if (grid[0] != (N + 7) / 8 || !T || grid[2] != 1)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/8), tokens, 1]", s->name);
+        need[0] = (size_t)T * KS * K * 4;
+        need[1] = (size_t)E * N * (K / 256) * 144;
+        need[2] = need[3] = (size_t)T * KS * 4;
+        need[4] = (size_t)T * N * 4;
+        align[0] = align[1] = 16;
+        return OJH_OK;
+    }
     default: {
         uint32_t T = c[0], KS = c[1], D = c[2];
         if ((rc = check_block(block, 256))) return rc;
@@ -492,6 +523,8 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, u
     case 3: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = experts
     case 4: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
     case 6: case 7: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;
+    case 8: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = assignments
+    case 9: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = tokens
     default: grid[0] = (uint32_t)(((uint64_t)M * N + 255) / 256); break;  // N = D, M = tokens
     }
     return OJH_OK;
@@ -668,6 +701,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("moe_combine", "moe", 3, 4, 0, 5, check_moe, shape_moe);
     add("moe_gu_q4k_mm", "moe", 7, 4, OJH_Q4_K, 6, check_moe, shape_moe);
     add("moe_down_q4k_mm", "moe", 6, 3, OJH_Q4_K, 7, check_moe, shape_moe);
+    add("moe_gu_q4k_dec", "moe", 5, 5, OJH_Q4_K, 8, check_moe, shape_moe);
+    add("moe_down_q4k_dec", "moe", 5, 5, OJH_Q4_K, 9, check_moe, shape_moe);
     add("copy_bf16_half", "glue", 2, 1, (2u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     // glue: `type` carries (input element bytes << 8 | output element bytes)
     add("copy_f32_half", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);

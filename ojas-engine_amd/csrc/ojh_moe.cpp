@@ -54,6 +54,25 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     if ((rc = ensure(dev, "moe")) || (rc = ensure(dev, "gemv_q8k"))) return rc;
 
     const uint32_t nsb_d = d / 256, nsb_f = n_ff / 256;
+    uint32_t b256[3] = {256, 1, 1};
+    // A few tokens: two launches addressed by assignment, activations quantized in registers,
+    // weighted sum inside the down launch (bit-identical to the grouped integer-dot pipeline).
+    // Measured on MI355X the grouped pipeline takes over once tokens start sharing experts.
+    const bool dec_fits = d <= 8192 && n_ff <= 2048 && (uint64_t)ksel * n_ff <= 32768;   // what the two launches stage in LDS
+    if (dev->moe_mode == 3 || (dev->moe_mode == 0 && T <= dev->moe_dec_tokens && dec_fits)) {
+        if (!dec_fits)
+            return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: the decode form serves d <= 8192, n_ff <= 2048 and ksel * n_ff <= 32768");
+        ojh_buf *act;
+        if ((rc = ojh_scratch_get(dev, "moe_act", (size_t)NA * n_ff * 4, &act))) return rc;
+        uint32_t g1[3] = {(n_ff + 7) / 8, NA, 1};
+        if ((rc = ojh_launch(dev, "moe_gu_q4k_dec",
+                             {x->ptr, (char *)gate->raw->ptr + gate->off, (char *)up->raw->ptr + up->off, act->ptr, idx->ptr},
+                             {d, n_ff, ksel, NA, E}, g1, b256)))
+            return rc;
+        uint32_t g2[3] = {(d + 7) / 8, T, 1};
+        return ojh_launch(dev, "moe_down_q4k_dec", {act->ptr, (char *)down->raw->ptr + down->off, idx->ptr, wgt->ptr, y->ptr},
+                          {n_ff, d, ksel, E, (uint32_t)(accum != 0)}, g2, b256);
+    }
     ojh_buf *xq, *xs, *act, *aq, *as_, *dv, *grp;
     if ((rc = ojh_scratch_get(dev, "moe_xq", (size_t)T * d, &xq))) return rc;
     if ((rc = ojh_scratch_get(dev, "moe_xs", (size_t)T * nsb_d * 4, &xs))) return rc;
@@ -65,7 +84,6 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     if ((rc = ojh_scratch_get(dev, "moe_grp", ((size_t)2 * E + 1 + NA) * 4, &grp))) return rc;
     uint32_t *counts = (uint32_t *)grp->ptr, *offsets = counts + E, *list = offsets + E + 1;
 
-    uint32_t b256[3] = {256, 1, 1};
     // Expert products: on the matrix cores once experts see a few tokens each (measured crossover on
     // MI355X: ~2 assignments per expert), on integer dots below that, where the launch is a pure
     // stream of weight rows.  The two forms round their f32 sums in different orders (last ulp).

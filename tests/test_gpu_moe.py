@@ -117,6 +117,35 @@ def test_expert_ffn_at_the_benchmark_shape(gpu, orc, pkg):
             assert np.array_equal(gpu.read(y2, T * d).reshape(T, d), got[perm])
 
 
+@pytest.mark.parametrize("T,E,ksel,d,nff,accum", [(1, 128, 8, 2048, 768, False), (3, 16, 5, 2304, 512, True),
+                                                   (4, 8, 8, 768, 256, False), (2, 70, 64, 256, 256, False)])
+def test_decode_form_is_bit_identical_to_the_grouped_integer_dots(gpu, pkg, monkeypatch, T, E, ksel, d, nff, accum):
+    """Few tokens run as two launches addressed by assignment (activations quantized in registers,
+    weighted sum inside the down launch); the same arithmetic step for step as quantize -> group ->
+    gate/up -> quantize -> down -> combine, so the same bits, including accumulate onto y."""
+    gate, up, down = _experts(pkg, E, d, nff, ("dec", E, d, nff))
+    x = pkg.synth.normal_f32(T * d, "moe", "dx", T, d).reshape(T, d)
+    x[0, :256] = 0.0                                    # an all-zero segment: scale 1
+    lg = pkg.synth.normal_f32(T * E, "moe", "dlg", T, E).reshape(T, E)
+    gi, gw, _, _ = _route(gpu, lg, ksel)
+    y0 = pkg.synth.normal_f32(T * d, "moe", "dy0").reshape(T, d)
+    outs = []
+    for mode in ("3", "2"):
+        monkeypatch.setenv("OJAS_HIP_MOE", mode)
+        g = pkg.HipGpu(0)
+        try:
+            lg_, lu_, ld_ = g.lin(Q4_K, E * nff, d, gate), g.lin(Q4_K, E * nff, d, up), g.lin(Q4_K, E * d, nff, down)
+            yd = g.upload(np.concatenate([y0.ravel(), np.full(d, 12345.5, np.float32)]))
+            g.moe_ffn(g.upload(x), T, d, nff, E, ksel, g.upload_bytes(gi), g.upload(gw), lg_, lu_, ld_, yd, accum=accum)
+            got = g.read(yd, T * d + d)
+            assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
+            outs.append(got[:T * d].copy())
+        finally:
+            g.close()
+    assert np.array_equal(outs[0], outs[1])
+    assert np.all(np.isfinite(outs[0])) and np.any(outs[0] != (y0.ravel() if accum else 0.0))
+
+
 def test_expert_ffn_rejects_what_it_cannot_run(gpu, pkg):
     E, d, nff = 4, 256, 256
     gate, up, down = _experts(pkg, E, d, nff, "err")
