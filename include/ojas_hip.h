@@ -245,7 +245,13 @@ int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uin
  * (crates/ojas-cpu/src/cpu_glm.rs:551-582; per-assignment GPU form
  * crates/ojas-metal/src/kernels/moe.rs:199-272):
  *   y[t] (+)= sum_j wgt[t][j] * Wd_e( silu(Wg_e x[t]) * (Wu_e x[t]) ),  e = idx[t][j].
- * gate/up: n_expert stacked matrices [n_ff][d]; down: n_expert stacked [d][n_ff]. */
+ * gate/up: n_expert stacked matrices [n_ff][d]; down: n_expert stacked [d][n_ff].
+ * Expert indices must be below n_expert (one that is not never reads outside the tensors; what
+ * it contributes is unspecified). Up to 8 tokens run as two launches addressed
+ * by assignment (bit-identical to the grouped integer-dot pipeline); larger batches are grouped
+ * by expert, on int8 MFMA from two assignments per expert (sums associate differently there:
+ * last ulps). Environment: OJAS_HIP_MOE = 1 / 2 / 3 forces MFMA / grouped dots / the decode
+ * form, OJAS_HIP_MOE_DEC_TOKENS moves the 8. */
 int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint32_t d, uint32_t n_ff,
                 uint32_t n_expert, uint32_t ksel, const ojh_buf *idx, const ojh_buf *wgt,
                 const ojh_lin *gate, const ojh_lin *up, const ojh_lin *down, ojh_buf *y,
