@@ -339,6 +339,143 @@ __device__ __forceinline__ void gemv_nat_q80_m_body(const float* __restrict__ x,
     }
 }
 
+// ------------------------------------------------------------------ Q8_0, rows staged through LDS
+//   gemv_nat_q80_lds{,_accum}(x, w, y, K, N, KC)   gemv_nat_q80_lds_bias(x, w, y, bs, K, N, KC)
+// 34-byte blocks defeat wide per-lane loads, and f32 activations are four bytes per weight byte
+// if they come through the cache every time.  Here a wave keeps its activations in registers
+// for the whole launch and has its rows copied into LDS by the memory system itself:
+//   * K is cut into KC (1, 2 or 4) chunks of CB = K / 32 / KC <= 128 blocks; wave w of the
+//     workgroup owns chunk w % KC of row slot w / KC (4 / KC rows per workgroup step);
+//   * lane l holds the 64 activations of blocks 2l and 2l + 1 of its chunk (lanes past CB / 2 idle);
+//   * a row's chunk (CB * 34 bytes, a multiple of 16) goes global -> LDS with
+//     global_load_lds_dwordx4, 1 KB per instruction and perfectly coalesced, the next row in
+//     flight while one is consumed (deeper queues and more resident waves measured slower);
+//   * the lane reads its 68 bytes back as 17 dwords (stride 17 banks: conflict-free) and runs
+//     dot_q80's arithmetic: per block sum_j (float)q_j x_j, times d, added up
+//     (crates/ojas-cpu/src/cpu_math.rs:971-981);
+//   * chunks of a row meet in LDS and are added in chunk order.
+// Rows are grid-stride; every wave of a workgroup runs the same number of steps (surplus rows are
+// clamped and not stored), so the workgroup barriers line up.
+#define Q80L_CHUNK 4352u   // 128 blocks
+#define Q80L_DEPTH 2u
+
+__device__ __forceinline__ void q80l_load_lds16(const void* base, uint voff, uint lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(base), "s"(lds_addr)
+                 : "memory");
+}
+// wait until at most `n` (0 .. 10) vector loads are outstanding
+__device__ __forceinline__ void q80l_wait(uint n) {
+    switch (n) {
+    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+    case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+    case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+    case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+    case 9: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
+    case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+    case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+    case 15: asm volatile("s_waitcnt vmcnt(15)" ::: "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+}
+
+__device__ __forceinline__ float q80l_dot4(uint v, float a, float x0, float x1, float x2, float x3) {
+    a = fmaf(sb0(v), x0, a);
+    a = fmaf(sb1(v), x1, a);
+    a = fmaf(sb2(v), x2, a);
+    return fmaf(sb3(v), x3, a);
+}
+
+template <int MODE>
+__device__ __forceinline__ void gemv_nat_q80_lds_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                      float* __restrict__ y, const float* __restrict__ bs,
+                                                      uint K, uint N, uint KC) {
+    __shared__ __attribute__((aligned(16))) uchar stage[4u * Q80L_DEPTH * Q80L_CHUNK];
+    __shared__ float part[2][4];
+    const uint lane = threadIdx.x & 63u;
+    const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint nb = K >> 5, CB = nb / KC, chunk = wave % KC, slot = wave / KC, RPB = 4u / KC;
+    const uint chunk_bytes = CB * Q80_BYTES, n16 = chunk_bytes >> 4, NI = (n16 + 63u) >> 6;
+    const size_t row_bytes = (size_t)nb * Q80_BYTES;
+    const bool on = 2u * lane < CB;
+    const uint lds0 = (uint)(size_t)(__attribute__((address_space(3))) uchar*)stage + wave * (Q80L_DEPTH * Q80L_CHUNK);
+    const uchar* mine = stage + wave * (Q80L_DEPTH * Q80L_CHUNK) + lane * 68u;
+    const uint steps = (N + RPB - 1u) / RPB;                        // workgroup steps in the launch
+    const uint my_steps = blockIdx.x < steps ? (steps - blockIdx.x + gridDim.x - 1u) / gridDim.x : 0u;
+    // row of step k: (blockIdx.x + k * gridDim.x) * RPB + slot, clamped
+    auto issue = [&](uint k) {
+        const uint row = min((blockIdx.x + k * gridDim.x) * RPB + slot, N - 1u);
+        const uchar* base = w + (size_t)row * row_bytes + (size_t)chunk * chunk_bytes;
+        const uint dst = lds0 + (k % Q80L_DEPTH) * Q80L_CHUNK;
+        for (uint i = 0; i < NI; i++)
+            if (i * 64u + lane < n16) q80l_load_lds16(base, (i * 64u + lane) << 4, dst + i * 1024u);
+    };
+    // the wave's activations: blocks 2l, 2l+1 of its chunk
+    float xr[64];
+    {
+        const float4* xp = (const float4*)(x + ((size_t)chunk * CB + (on ? 2u * lane : 0u)) * 32u);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float4 v = xp[i];
+            xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
+        }
+    }
+    // the activation loads above are older than every row copy, so counting copies alone is safe
+    for (uint k = 0; k + 1u < Q80L_DEPTH; k++)
+        if (k < my_steps) issue(k);
+    for (uint k = 0; k < my_steps; k++) {
+        if (k + Q80L_DEPTH - 1u < my_steps) issue(k + Q80L_DEPTH - 1u);
+        q80l_wait(min(my_steps - 1u - k, Q80L_DEPTH - 1u) * NI);
+        const uint* p = (const uint*)(mine + (k % Q80L_DEPTH) * Q80L_CHUNK);
+        uint d[17];
+#pragma unroll
+        for (int i = 0; i < 17; i++) d[i] = p[i];
+        // block 2l: scale in the low half of dword 0, quants at bytes 2 .. 33
+        float s0 = fmaf(sb2(d[0]), xr[0], 0.0f);
+        s0 = fmaf(sb3(d[0]), xr[1], s0);
+#pragma unroll
+        for (int j = 1; j < 8; j++) s0 = q80l_dot4(d[j], s0, xr[4 * j - 2], xr[4 * j - 1], xr[4 * j], xr[4 * j + 1]);
+        s0 = fmaf(sb0(d[8]), xr[30], s0);
+        s0 = fmaf(sb1(d[8]), xr[31], s0);
+        // block 2l+1: scale in the high half of dword 8, quants in dwords 9 .. 16
+        float s1 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) s1 = q80l_dot4(d[9 + j], s1, xr[32 + 4 * j], xr[33 + 4 * j], xr[34 + 4 * j], xr[35 + 4 * j]);
+        float v = on ? f16_bits_to_f32(d[0] & 0xFFFFu) * s0 + f16_bits_to_f32(d[8] >> 16) * s1 : 0.0f;
+        v = wave_sum(v);
+        const uint row = (blockIdx.x + k * gridDim.x) * RPB + slot;
+        if (KC == 1u) {
+            if (lane == 0 && row < N) store_row<MODE>(y, bs, row, v);
+        } else {
+            if (lane == 0) part[k & 1u][wave] = v;
+            __syncthreads();
+            if (lane == 0 && chunk == 0u && row < N) {
+                float t = part[k & 1u][wave];
+                for (uint c = 1; c < KC; c++) t += part[k & 1u][wave + c];
+                store_row<MODE>(y, bs, row, t);
+            }
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+gemv_nat_q80_lds(const float* x, const uchar* w, float* y, uint K, uint N, uint KC) {
+    gemv_nat_q80_lds_body<ST_SET>(x, w, y, nullptr, K, N, KC);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemv_nat_q80_lds_accum(const float* x, const uchar* w, float* y, uint K, uint N, uint KC) {
+    gemv_nat_q80_lds_body<ST_ACCUM>(x, w, y, nullptr, K, N, KC);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemv_nat_q80_lds_bias(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N, uint KC) {
+    gemv_nat_q80_lds_body<ST_BIAS>(x, w, y, bs, K, N, KC);
+}
+
 // ------------------------------------------------------------------ entries
 #define GEMV_NAT_ENTRIES(FMT)                                                                              \
     extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_r1(                                 \

@@ -58,6 +58,9 @@ struct ojh_device {
     int gemv_rows_override = 0;  // OJAS_HIP_GEMV_R
     uint32_t gemm_min_m = 32;    // OJAS_HIP_GEMM_MIN_M: rows from which ojh_mm takes the MFMA tile
     int gemm_split_override = 0; // OJAS_HIP_GEMM_SPLIT
+    int q80_lds = 1;             // OJAS_HIP_Q80_LDS: 0 = never take the LDS-staged Q8_0 matvec
+    uint32_t q80_lds_min_n = 16384; // OJAS_HIP_Q80_LDS_MIN_N: rows from which it is taken (measured crossover)
+    uint32_t q80_lds_bpc = 3;       // OJAS_HIP_Q80_LDS_BPC: workgroups per CU its grid is sized for (35 KB of LDS each; 3 measured best)
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
                                  // 3 = per-assignment decode form always
     uint32_t moe_dec_tokens = 8; // OJAS_HIP_MOE_DEC_TOKENS: the decode form serves up to this many tokens
@@ -109,3 +112,4 @@ const ojh_kernel_spec *ojh_find_kernel(const char *name);
 int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out);
 int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptrs,
                const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);
+uint32_t ojh_q80_lds_kc(uint32_t K);   // chunks of K for gemv_nat_q80_lds, 0 if none (ojh_manifest.cpp)

@@ -73,6 +73,50 @@ static int check_gemv_nat(const ojh_kernel_spec *s, const uint32_t *c, const uin
     return OJH_OK;
 }
 
+// The LDS-staged Q8_0 matvec cuts K into KC chunks of K / 32 / KC blocks: the smallest KC of 1, 2, 4
+// whose chunk is at most 128 blocks and a multiple of 8 blocks (16-byte copy units); 0 if none.
+uint32_t ojh_q80_lds_kc(uint32_t K) {
+    if (!K || K % 256) return 0;
+    const uint32_t nb = K / 32;
+    for (uint32_t kc = 1; kc <= 4; kc *= 2)
+        if (nb % kc == 0 && nb / kc <= 128 && (nb / kc) % 8 == 0) return kc;
+    return 0;
+}
+
+// gemv_nat_q80_lds{,_accum,_bias}(x, w, y[, bs], K, N, KC): rows grid-stride, 4 / KC per workgroup step
+static int check_gemv_q80_lds(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                              const uint32_t block[3], size_t need[16], size_t align[16]) {
+    uint32_t K = c[0], N = c[1], KC = c[2];
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (!N) return ojh_fail(OJH_ERR_ARG, "%s: N must be positive", s->name);
+    const uint32_t want = ojh_q80_lds_kc(K);
+    if (!want) return ojh_fail(OJH_ERR_UNSUPPORTED, "%s: K=%u has no chunking of 1, 2 or 4 pieces of <= 128 blocks in 16-byte units", s->name, K);
+    if (KC != want) return ojh_fail(OJH_ERR_ARG, "%s: KC=%u, K=%u takes KC=%u", s->name, KC, K, want);
+    if (!grid[0] || grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1], x > 0", s->name);
+    need[0] = (size_t)K * 4;
+    need[1] = (size_t)N * (K / 32) * 34;
+    need[2] = (size_t)N * 4;
+    if (s->n_bufs == 4) need[3] = (size_t)N * 4;
+    align[0] = align[1] = 16;
+    align[2] = align[3] = 4;
+    return OJH_OK;
+}
+// three workgroups per CU (measured best; four would fit), steps spread evenly
+static int shape_q80_lds(const ojh_kernel_spec *, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t,
+                         uint32_t grid[3], uint32_t block[3]) {
+    uint32_t kc = ojh_q80_lds_kc(K);
+    if (!kc) return ojh_fail(OJH_ERR_UNSUPPORTED, "gemv_nat_q80_lds: K=%u cannot be chunked", K);
+    uint32_t steps = (N + 4 / kc - 1) / (4 / kc);
+    uint32_t resident = (uint32_t)dev->prop.multiProcessorCount * dev->q80_lds_bpc;
+    uint32_t rounds = (steps + resident - 1) / resident;
+    grid[0] = (steps + rounds - 1) / rounds;
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // gemv_q8k_<fmt>{,_accum,_bias,_rN}(xq, xs, w, y[, bs], K, N)
 static int check_gemv_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                           const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -652,7 +696,12 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g + "_accum", "gemv", 3, 2, f.type, 4, check_gemv_nat, shape_rows);
         add(g + "_bias", "gemv", 4, 2, f.type, 4, check_gemv_nat, shape_rows);
         add(g + "_m", "gemv", 3, 4, f.type, 1, check_gemv_nat_m, shape_rows);
-        if (f.type == OJH_Q8_0) continue;  // the CPU path keeps f32 activations for Q8_0
+        if (f.type == OJH_Q8_0) {
+            add(g + "_lds", "gemv", 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
+            add(g + "_lds_accum", "gemv", 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
+            add(g + "_lds_bias", "gemv", 4, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
+            continue;  // the CPU path keeps f32 activations for Q8_0
+        }
         std::string q = "gemv_q8k_" + t;
         add(q, "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
         add(q + "_r1", "gemv_q8k", 4, 2, f.type, 1, check_gemv_q8k, shape_rows);

@@ -356,6 +356,17 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     }
     if ((rc = ensure(dev, "gemv"))) return rc;
     std::string base = std::string("gemv_nat_") + f->tag;
+    // Q8_0 rows from a few thousand up: activations in registers, rows copied into LDS by the
+    // memory system (needs 16-byte aligned rows and a K that chunks)
+    if (m == 1 && w->type == OJH_Q8_0 && dev->q80_lds && N >= dev->q80_lds_min_n && ojh_q80_lds_kc(K) &&
+        (uintptr_t)wp % 16 == 0 && (uintptr_t)xp % 16 == 0) {
+        uint32_t sg[3], sb[3];
+        if ((rc = ojh_launch_shape(dev, "gemv_nat_q80_lds", K, N, 1, sg, sb))) return rc;
+        std::vector<void *> p = {xp, wp, yp};
+        if (bias) p.push_back(bias->ptr);
+        return ojh_launch(dev, accum ? "gemv_nat_q80_lds_accum" : bias ? "gemv_nat_q80_lds_bias" : "gemv_nat_q80_lds", p,
+                          {K, N, ojh_q80_lds_kc(K)}, sg, sb);
+    }
     if (m == 1) {
         int r = (accum || bias) ? 4 : pick_rows(dev, N);
         std::string name = base + (accum ? "_accum" : bias ? "_bias" : r == 4 ? "" : r == 2 ? "_r2" : "_r1");

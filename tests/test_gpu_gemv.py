@@ -326,3 +326,39 @@ def test_q5k_takes_the_int8_path_at_every_token_count(gpu, orc, pkg):
     yd = gpu.alloc(n)
     gpu.mm(gpu.upload(x), gpu.lin(Q5_K, n, k, w), yd, 1, act_mode=pkg.ACT_Q8K)
     assert peak_err(gpu.read(yd, n), orc.matvec_kq(w, Q5_K, n, k, x)) <= TOL_Q8K_SEEN
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (4099, 4096), (2049, 8192), (2050, 14336), (3000, 2560), (5, 256),
+                                 (1, 4096), (7, 14336), (70000, 256)])
+def test_q80_rows_staged_through_lds(pkg, orc, monkeypatch, n, k):
+    """The Q8_0 matvec that keeps activations in registers and has rows copied into LDS: one, two
+    and four K chunks, partly filled chunks (K = 2560, 14336), row counts that leave surplus waves
+    and surplus steps, bias and accumulate — against dot_q80 and against the streaming kernel."""
+    w, x = _inputs(pkg, Q8_0, n, k, "lds")
+    bias = (1000.0 + np.arange(n)).astype(np.float32)
+    y0 = pkg.synth.normal_f32(n, "lds", "y0", n)
+    want = orc.matvec_kq(w, Q8_0, n, k, x)
+    outs = {}
+    for lds in ("1", "0"):
+        monkeypatch.setenv("OJAS_HIP_Q80_LDS", lds)
+        monkeypatch.setenv("OJAS_HIP_Q80_LDS_MIN_N", "1")
+        g = pkg.HipGpu(0)
+        try:
+            lin, xd = g.lin(Q8_0, n, k, w), g.upload(x)
+            yd = g.upload(np.full(n + 2, 12345.0, np.float32))
+            g.mm(xd, lin, yd, 1, y_off=4)
+            got = g.read(yd, n + 2)
+            assert got[0] == 12345.0 and got[-1] == 12345.0, "wrote outside y"
+            yb, ya = g.alloc(n), g.upload(y0)
+            g.mm(xd, lin, yb, 1, bias=g.upload(bias))
+            g.mm(xd, lin, ya, 1, True)
+            outs[lds] = (got[1:-1].copy(), g.read(yb, n), g.read(ya, n))
+        finally:
+            g.close()
+    peak = np.max(np.abs(want))
+    for lds in ("1", "0"):
+        plain, with_bias, onto = outs[lds]
+        assert peak_err(plain, want) <= 1e-5, lds
+        assert np.max(np.abs(with_bias - (want + bias))) <= 1e-5 * peak + 1e-3, lds
+        assert np.max(np.abs(onto - (want + y0))) <= 1e-5 * peak + 1e-5, lds
+    assert peak_err(outs["1"][0], outs["0"][0]) <= 2e-6
