@@ -794,3 +794,168 @@ gemv_q8k_q6k_mx(const signed char* xq, const float* xs, const uchar* w, float* y
     else if (M <= 8) gemv_q8k_q6k_mx_body<8>(xq, xs, w, y, K, N, M, ACC, lds_mx);
     else gemv_q8k_q6k_mx_body<16>(xq, xs, w, y, K, N, M, ACC, lds_mx);
 }
+
+// ---- Q6_K against up to 16 tokens on the int8 matrix cores ------------------------------------
+//   gemv_q8k_q6k_mf(xq, xs, w, y, K, N, M, ACC)    M <= 16, MT (K + 32) + K / 4 <= 69632 (MT = 8 or 16)
+// The verify head reads 510 MB of weights whatever the token count; with integer dots the work
+// per row grows with M and the launch turns compute-bound from M = 4.  Here a wave owns 16 rows
+// and runs them against 8 tokens at a time with v_mfma_i32_16x16x32_i8:
+//   * B (weights): lane (n, kg) = (lane % 16, lane / 16) builds, for each of the eight 32-weight
+//     quarters of a super-block, the signed codes q - 32 of positions 8 kg .. 8 kg + 7 of row n;
+//   * a quarter holds two 16-weight groups with their own int8 scale, and an MFMA sums over all
+//     32 positions.  So the 16 token rows of A are 8 tokens twice: rows 0-7 carry only positions
+//     0-15 (lanes kg < 2), rows 8-15 only positions 16-31 (lanes kg >= 2); the other lanes hold
+//     zeros for good.  D then has a token's two group dots in different rows, each multiplied by
+//     its own scale with one integer multiply-add; the two halves meet once per 16-row tile;
+//   * activations wait in LDS, token rows 32 bytes longer than K so that the 32 live lanes of an
+//     8-byte read fall in 64 distinct banks.
+// Per super-block and lane the arithmetic is dot_q6k's: sx * d * sum_g scale_g * idot_g, integer
+// sums exact (crates/ojas-cpu/src/cpu_math.rs:674-722).
+typedef int q6k_i4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ long q6k_signed8(uint ql0, uint ql1, uint qh0, uint qh1, int Q) {
+    const uint M4 = 0x0F0F0F0Fu, H2 = 0x30303030u;
+    const uint lo0 = Q < 2 ? ql0 & M4 : (ql0 >> 4) & M4, lo1 = Q < 2 ? ql1 & M4 : (ql1 >> 4) & M4;
+    const uint hi0 = Q == 0 ? (qh0 << 4) & H2 : Q == 1 ? (qh0 << 2) & H2 : Q == 2 ? qh0 & H2 : (qh0 >> 2) & H2;
+    const uint hi1 = Q == 0 ? (qh1 << 4) & H2 : Q == 1 ? (qh1 << 2) & H2 : Q == 2 ? qh1 & H2 : (qh1 >> 2) & H2;
+    // code in 0..63 -> code - 32 as int8, bytewise: + 96 cannot carry, the flip of bit 7 subtracts 128
+    const uint c0 = ((lo0 | hi0) + 0x60606060u) ^ 0x80808080u, c1 = ((lo1 | hi1) + 0x60606060u) ^ 0x80808080u;
+    return (long)(((unsigned long)c1 << 32) | c0);
+}
+
+struct Q6kMfW {          // lane (n, kg): its bytes of one super-block of row n
+    u32x2_a2 la[2], lb[2], qh[2];   // per half: ql[8 kg ..], ql[32 + 8 kg ..], qh[8 kg ..]
+    u32x4_a2 sc;
+    uint d16;
+};
+// A super-block is 210 bytes, so a lane's 8-byte pieces sit at even or odd multiples of two
+// bytes.  With sixteen rows per load instruction, 8-byte loads that are not dword aligned cost
+// the memory pipeline more than their size (measured: 217 -> 161 us for this kernel); these read
+// the three aligned dwords around a piece and shift (sh = 0 or 16 bits, v_alignbit).  The
+// streaming kernels' 16-byte pieces measured the other way round and stay unaligned loads.
+__device__ __forceinline__ u32x2_a2 q6k_ld8(const uchar* a4, uint sh) {   // a4: piece address rounded down to 4
+    const uint* p = (const uint*)a4;
+    const uint d0 = p[0], d1 = p[1], d2 = p[2];
+    u32x2_a2 r;
+    r.x = __builtin_amdgcn_alignbit(d1, d0, sh);
+    r.y = __builtin_amdgcn_alignbit(d2, d1, sh);
+    return r;
+}
+__device__ __forceinline__ Q6kMfW q6k_mf_load(const uchar* blk, uint kg) {
+    Q6kMfW r;
+    const uint sh = ((uint)(size_t)blk & 2u) << 3;
+    const uchar* b4 = blk - ((size_t)blk & 2u);
+#pragma unroll
+    for (int hf = 0; hf < 2; hf++) {
+        r.la[hf] = q6k_ld8(b4 + 64u * hf + 8u * kg, sh);
+        r.lb[hf] = q6k_ld8(b4 + 64u * hf + 32u + 8u * kg, sh);
+        r.qh[hf] = q6k_ld8(b4 + 128u + 32u * hf + 8u * kg, sh);
+    }
+    const uint* ps = (const uint*)(b4 + 192u);
+    const uint s0 = ps[0], s1 = ps[1], s2 = ps[2], s3 = ps[3], s4 = ps[4];   // scales, d and up to two bytes more
+    r.sc.x = __builtin_amdgcn_alignbit(s1, s0, sh);
+    r.sc.y = __builtin_amdgcn_alignbit(s2, s1, sh);
+    r.sc.z = __builtin_amdgcn_alignbit(s3, s2, sh);
+    r.sc.w = __builtin_amdgcn_alignbit(s4, s3, sh);
+    r.d16 = (s4 >> sh) & 0xFFFFu;
+    return r;
+}
+
+template <int P>   // P passes of 8 tokens
+__device__ __forceinline__ void gemv_q8k_q6k_mf_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                     const uchar* __restrict__ w, float* __restrict__ y,
+                                                     uint K, uint N, uint M, uint ACC, uchar* lds) {
+    const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint nsb = K >> 8, S = K + 32u;
+    float* lsx = (float*)(lds + (size_t)(8 * P) * S);       // [sb][16] token scales
+    // stage the tokens (rows past M are zero) and their scales
+    const uint per_row = K >> 4;
+    for (uint i = tid; i < (uint)(8 * P) * per_row; i += blockDim.x) {
+        const uint t = i / per_row, o = (i - t * per_row) << 4;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (t < M) v = *(const uint4*)(xq + (size_t)t * K + o);
+        *(uint4*)(lds + (size_t)t * S + o) = v;
+    }
+    for (uint i = tid; i < nsb * 16u; i += blockDim.x) {
+        const uint sb = i >> 4, t = i & 15u;
+        lsx[i] = t < M ? xs[(size_t)t * nsb + sb] : 0.0f;
+    }
+    __syncthreads();
+    const uint n = lane & 15u, kg = lane >> 4;
+    const bool live = (n < 8u) == (kg < 2u);       // this lane's A rows carry its positions
+    const uint h = kg >> 1;                        // which 16-weight group of a quarter its D rows hold
+    const uchar* xa = lds + (size_t)(n & 7u) * S + 8u * kg;
+    const uint tiles = (N + 15u) >> 4;
+    const uint nwave = blockDim.x >> 6;
+    for (uint tile = blockIdx.x * nwave + wave; tile < tiles; tile += gridDim.x * nwave) {
+        const uint row = min(tile * 16u + n, N - 1u);
+        const uchar* wr = w + (size_t)row * nsb * Q6K_BYTES;
+        float acc[P][4];
+#pragma unroll
+        for (int p = 0; p < P; p++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[p][v] = 0.0f;
+        // two super-blocks ahead: a wave has ~8 KB on its way, which is what eight waves per CU need
+        Q6kMfW cur = q6k_mf_load(wr, kg), nx = q6k_mf_load(wr + (size_t)min(1u, nsb - 1u) * Q6K_BYTES, kg);
+        for (uint sb = 0; sb < nsb; sb++) {
+            const Q6kMfW nx2 = q6k_mf_load(wr + (size_t)min(sb + 2u, nsb - 1u) * Q6K_BYTES, kg);
+            int isum[P][4];
+#pragma unroll
+            for (int p = 0; p < P; p++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) isum[p][v] = 0;
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {
+                // scales 8 hf + 2 q + h, q = 0..3: bytes h, 2 + h of the half's two dwords
+                const uint s_lo = (hf ? cur.sc.z : cur.sc.x) >> (8u * h), s_hi = (hf ? cur.sc.w : cur.sc.y) >> (8u * h);
+                const int scl[4] = {(int)(signed char)s_lo, (int)(signed char)(s_lo >> 16), (int)(signed char)s_hi,
+                                    (int)(signed char)(s_hi >> 16)};
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const u32x2_a2 ql = (q & 1) ? cur.lb[hf] : cur.la[hf];
+                    const long B = q6k_signed8(ql.x, ql.y, cur.qh[hf].x, cur.qh[hf].y, q);
+#pragma unroll
+                    for (int p = 0; p < P; p++) {
+                        long A = 0;
+                        if (live) A = *(const long*)(xa + (size_t)(8 * p) * S + sb * 256u + 128u * hf + 32u * q);
+                        const q6k_i4 zero = {0, 0, 0, 0};
+                        const q6k_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B, zero, 0, 0, 0);
+#pragma unroll
+                        for (int v = 0; v < 4; v++) isum[p][v] += __mul24(scl[q], D[v]);
+                    }
+                }
+            }
+            const float d = f16_bits_to_f32(cur.d16);
+#pragma unroll
+            for (int p = 0; p < P; p++) {
+                const float4 sx = *(const float4*)(lsx + sb * 16u + 8u * p + 4u * (kg & 1u));
+                acc[p][0] += sx.x * d * (float)isum[p][0];
+                acc[p][1] += sx.y * d * (float)isum[p][1];
+                acc[p][2] += sx.z * d * (float)isum[p][2];
+                acc[p][3] += sx.w * d * (float)isum[p][3];
+            }
+            cur = nx;
+            nx = nx2;
+        }
+        // D rows 4 kg + v: token 4 (kg & 1) + v, first group in lanes kg < 2, second in kg >= 2
+#pragma unroll
+        for (int p = 0; p < P; p++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float tot = acc[p][v] + __shfl_xor(acc[p][v], 32, 64);
+                const uint t = 8u * p + 4u * kg + v;
+                if (kg < 2u && t < M && tile * 16u + n < N) {
+                    float* o = y + (size_t)t * N + tile * 16u + n;
+                    *o = ACC ? *o + tot : tot;
+                }
+            }
+    }
+}
+
+#define Q6K_MF_LDS 69632u    // 16 tokens of K = 4096: two workgroups per CU
+extern "C" __global__ void __launch_bounds__(256)
+gemv_q8k_q6k_mf(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    __shared__ __attribute__((aligned(16))) uchar lds_mf[Q6K_MF_LDS];
+    if (M <= 8) gemv_q8k_q6k_mf_body<1>(xq, xs, w, y, K, N, M, ACC, lds_mf);
+    else gemv_q8k_q6k_mf_body<2>(xq, xs, w, y, K, N, M, ACC, lds_mf);
+}

@@ -162,6 +162,17 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
         if (bias) p.push_back(bias->ptr);
         return ojh_launch(dev, name.c_str(), p, {K, N}, grid, block);
     }
+    // a handful of tokens on Q6_K rows: the int8 matrix cores, 8 tokens per pass
+    const size_t w_bytes = w->row_bytes * N;
+    const bool dwords_ok = (uintptr_t)wp % 4 == 0 && (w_bytes % 4 == 0 || w->off + w_bytes + 2 <= w->raw->bytes);
+    if (w->type == OJH_Q6_K && m >= dev->q6k_mf_min_m && m <= 16 && dwords_ok) {
+        if ((uint64_t)(m <= 8 ? 8 : 16) * (K + 32) + K / 4 <= 69632) {
+            uint32_t sg[3], sb[3];
+            int rc = ojh_launch_shape(dev, "gemv_q8k_q6k_mf", K, N, m, sg, sb);
+            if (rc) return rc;
+            return ojh_launch(dev, "gemv_q8k_q6k_mf", {xq, xs, wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, sg, sb);
+        }
+    }
     // few tokens on Q6_K rows: activations staged in LDS once per workgroup, rows grid-stride
     if (w->type == OJH_Q6_K && m <= 16 && (uint64_t)m * ((K + 4095) / 4096) <= 19) {
         uint32_t sg[3], sb[3];

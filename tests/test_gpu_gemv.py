@@ -362,3 +362,38 @@ def test_q80_rows_staged_through_lds(pkg, orc, monkeypatch, n, k):
         assert np.max(np.abs(with_bias - (want + bias))) <= 1e-5 * peak + 1e-3, lds
         assert np.max(np.abs(onto - (want + y0))) <= 1e-5 * peak + 1e-5, lds
     assert peak_err(outs["1"][0], outs["0"][0]) <= 2e-6
+
+
+@pytest.mark.parametrize("m,n,k,accum", [(4, 50, 256, False), (8, 130, 4096, True), (9, 301, 4096, False),
+                                         (16, 1000, 4096, False), (16, 17, 512, True), (12, 4099, 2560, False),
+                                         (6, 64, 7168, False)])
+def test_q6k_tokens_on_the_int8_matrix_cores(gpu, orc, pkg, m, n, k, accum):
+    """5 to 16 tokens against Q6_K rows: `gemv_q8k_q6k_mf` by name and through the router, against
+    matvec_kq per token and against the LDS-staged integer-dot entry on the same quantized
+    activations (same integer sums; the f32 sums associate differently)."""
+    w = pkg.synth.q6k_weights(n, k, "mf", n, k)
+    x = pkg.synth.normal_f32(m * k, "mf", "x", m, k).reshape(m, k)
+    x[0, :256] = 0.0
+    y0 = pkg.synth.normal_f32(m * n, "mf", "y0").reshape(m, n) if accum else np.zeros((m, n), np.float32)
+    want = np.stack([orc.matvec_kq(w, Q6_K, n, k, x[t]) for t in range(m)])
+    lin = gpu.lin(Q6_K, n, k, w)
+    yd = gpu.upload(np.concatenate([y0.ravel(), np.full(8, 4242.5, np.float32)]))
+    gpu.mm(gpu.upload(x), lin, yd, m, accum, act_mode=pkg.ACT_Q8K)
+    got = gpu.read(yd, m * n + 8)
+    assert np.all(got[m * n:] == 4242.5), "wrote past the last token"
+    assert peak_err(got[:m * n].reshape(m, n) - y0, want) <= TOL_Q8K_SEEN
+    gpu.ensure_family("gemv_q8k")
+    nsb = k // 256
+    xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
+    gpu.quant_q8k(gpu.upload(x), m, k, xq, xs)
+    wd = gpu.upload_bytes(w)
+    outs = []
+    for name in ("gemv_q8k_q6k_mf", "gemv_q8k_q6k_mx"):
+        grid, block = gpu.launch_shape(name, k, n, m)
+        y2 = gpu.upload(y0)
+        gpu.dispatch(gpu.begin(), name, [(xq, 0), (xs, 0), (wd, 0), (y2, 0)], [k, n, m, int(accum)], grid, block)
+        outs.append(gpu.read(y2, m * n).reshape(m, n) - y0)
+    assert peak_err(outs[0], want) <= TOL_Q8K_SEEN
+    assert peak_err(outs[0], outs[1]) <= 2e-6
+    with pytest.raises(pkg.OjasHipError, match="do not fit"):
+        gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_mf", [(xq, 0), (xs, 0), (wd, 0), (y2, 0)], [k, n, 17, 0], [8, 1, 1], [256, 1, 1])
