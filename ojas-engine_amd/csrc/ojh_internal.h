@@ -60,7 +60,7 @@ struct ojh_device {
     int gemm_split_override = 0; // OJAS_HIP_GEMM_SPLIT
     int q80_lds = 1;             // OJAS_HIP_Q80_LDS: 0 = never take the LDS-staged Q8_0 matvec
     uint32_t q80_lds_min_n = 16384; // OJAS_HIP_Q80_LDS_MIN_N: rows from which it is taken (measured crossover)
-    uint32_t q80_lds_bpc = 3;       // OJAS_HIP_Q80_LDS_BPC: workgroups per CU its grid is sized for (35 KB of LDS each; 3 measured best)
+    uint32_t q80_lds_bpc = 0;       // OJAS_HIP_Q80_LDS_BPC: workgroups per CU its grid is sized for (0: 2 or 3 by K chunking)
     uint32_t q6k_mf_min_m = 4;   // OJAS_HIP_Q6K_MF_MIN_M: tokens from which Q6_K rows go to the int8 matrix cores
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
                                  // 3 = per-assignment decode form always

@@ -76,7 +76,7 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_GEMM_EXACT")) d->gemm_exact = atoi(r) != 0;
     if (const char *r = getenv("OJAS_HIP_Q80_LDS")) d->q80_lds = atoi(r);
     if (const char *r = getenv("OJAS_HIP_Q80_LDS_MIN_N")) d->q80_lds_min_n = (uint32_t)atoi(r);
-    if (const char *r = getenv("OJAS_HIP_Q80_LDS_BPC")) d->q80_lds_bpc = (uint32_t)std::max(1, atoi(r));
+    if (const char *r = getenv("OJAS_HIP_Q80_LDS_BPC")) d->q80_lds_bpc = (uint32_t)std::max(0, atoi(r));
     if (const char *r = getenv("OJAS_HIP_Q6K_MF_MIN_M")) d->q6k_mf_min_m = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE")) d->moe_mode = atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE_DEC_TOKENS")) d->moe_dec_tokens = (uint32_t)atoi(r);
