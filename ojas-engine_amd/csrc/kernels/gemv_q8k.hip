@@ -655,6 +655,52 @@ __device__ __forceinline__ void gemv_q8k_q6k_body(const signed char* __restrict_
 
 GEMV_Q8K_ENTRIES(q6k, gemv_q8k_q6k_body)
 
+// Tall matrices (an output head): rows grid-stride, the wave's share of the quantized activations
+// loaded once and kept in registers (21 per 4096 of K), so the per-row traffic through the vector
+// memory path is the row's own bytes only (head 151936 x 4096: 104 -> 93 us; the same form of the
+// Q4_K kernel, whose activation fragment is a third the size, measured 5 % slower than one wave
+// per two rows and is not built).
+//   gemv_q8k_q6k_px(xq, xs, w, y, K, N)     K <= 8192; any grid of 256-thread workgroups
+template <int NS>
+__device__ __forceinline__ void gemv_q8k_q6k_px_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                     const uchar* __restrict__ w, float* __restrict__ y, uint K, uint N) {
+    constexpr int R = 2;
+    const uint lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint nsb = K >> 8, g = lane >> 2, hf = (lane >> 1) & 1u, l0 = (lane & 1u) * 16u;
+    Q6kX f[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const uint sb = (uint)s * 16u + g;
+        f[s] = q6k_load_x(xq, xs, min(sb, nsb - 1u), hf, l0);
+        if (sb >= nsb) f[s].sx = 0.0f;            // lanes past the row's end contribute nothing
+    }
+    for (uint row0 = (blockIdx.x * 4u + wave) * R; row0 < N; row0 += gridDim.x * 4u * R) {
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const uint sb = min((uint)s * 16u + g, nsb - 1u);
+            Q6kW raw[R];
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                raw[r] = q6k_load_w(w + ((size_t)min(row0 + r, N - 1u) * nsb + sb) * Q6K_BYTES, hf, l0);
+#pragma unroll
+            for (int r = 0; r < R; r++) acc[r] += q6k_lane_dot(raw[r], f[s]);
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const float t = wave_sum(acc[r]);
+            if (lane == 0 && row0 + r < N) y[row0 + r] = t;
+        }
+    }
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemv_q8k_q6k_px(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N) {
+    if (K <= 4096u) gemv_q8k_q6k_px_body<1>(xq, xs, w, y, K, N);
+    else gemv_q8k_q6k_px_body<2>(xq, xs, w, y, K, N);
+}
+
 template <int MT>
 __device__ __forceinline__ void gemv_q8k_q6k_m_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
                                                     const uchar* __restrict__ w, float* __restrict__ y,

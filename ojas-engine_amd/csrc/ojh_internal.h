@@ -62,6 +62,8 @@ struct ojh_device {
     uint32_t q80_lds_min_n = 16384; // OJAS_HIP_Q80_LDS_MIN_N: rows from which it is taken (measured crossover)
     uint32_t q80_lds_bpc = 0;       // OJAS_HIP_Q80_LDS_BPC: workgroups per CU its grid is sized for (0: 2 or 3 by K chunking)
     uint32_t q6k_mf_min_m = 4;   // OJAS_HIP_Q6K_MF_MIN_M: tokens from which Q6_K rows go to the int8 matrix cores
+    uint32_t px_bpc = 0;         // OJAS_HIP_PX_BPC: workgroups per CU for the grid-stride head matvec (0: 8)
+    int px = 1;                  // OJAS_HIP_PX: 0 = never take it
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
                                  // 3 = per-assignment decode form always
     uint32_t moe_dec_tokens = 8; // OJAS_HIP_MOE_DEC_TOKENS: the decode form serves up to this many tokens

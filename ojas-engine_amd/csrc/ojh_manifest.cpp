@@ -118,6 +118,36 @@ static int shape_q80_lds(const ojh_kernel_spec *, const ojh_device *dev, uint32_
     return OJH_OK;
 }
 
+// gemv_q8k_q6k_px(xq, xs, w, y, K, N): rows grid-stride, activations in registers (K <= 8192)
+static int check_gemv_q8k_px(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                             const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], N = c[1];
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if ((rc = check_block(block, 256))) return rc;
+    if (K > 8192) return ojh_fail(OJH_ERR_UNSUPPORTED, "%s: K=%u exceeds the 8192 activations a wave keeps in registers", s->name, K);
+    if (!grid[0] || grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1], x > 0", s->name);
+    need[0] = (size_t)K;
+    need[1] = (size_t)(K / 256) * 4;
+    need[2] = (size_t)N * (K / f->weights) * f->bytes;
+    need[3] = (size_t)N * 4;
+    align[1] = 4;
+    align[2] = f->bytes % 16 ? 2 : 16;
+    align[3] = 4;
+    return OJH_OK;
+}
+static int shape_px(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t N, uint32_t,
+                    uint32_t grid[3], uint32_t block[3]) {
+    uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, cover = (N + 7) / 8;
+    uint32_t bpc = dev && dev->px_bpc ? dev->px_bpc : 8u;
+    grid[0] = cover < bpc * cus ? cover : bpc * cus;   // a whole multiple of the CU count
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // gemv_q8k_<fmt>{,_accum,_bias,_rN}(xq, xs, w, y[, bs], K, N)
 static int check_gemv_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                           const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -734,6 +764,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(q + "_m", "gemv_q8k", 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
         if (f.type == OJH_Q6_K) add(q + "_mx", "gemv_q8k", 4, 4, f.type, 0, check_gemv_q8k_m, shape_mx);
         if (f.type == OJH_Q6_K) add(q + "_mf", "gemv_q8k", 4, 4, f.type, -1, check_gemv_q8k_m, shape_mf);
+        if (f.type == OJH_Q6_K) add(q + "_px", "gemv_q8k", 4, 2, f.type, 2, check_gemv_q8k_px, shape_px);
         if (f.type == OJH_Q4_K) {
             std::string fq = "gemv_fq8k_" + t;
             add(q + "_x4_r1", "gemv_q8k", 10, 5, f.type, 1, check_gemv_q8k_x4, shape_rows);

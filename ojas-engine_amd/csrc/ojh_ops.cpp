@@ -153,6 +153,14 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
     void *wp = at(w->raw, w->off);
     uint32_t grid[3] = {1, 1, 1}, block[3] = {256, 1, 1};
     std::string base = std::string("gemv_q8k_") + f->tag;
+    // an output head: rows grid-stride, activations in registers
+    if (m == 1 && w->type == OJH_Q6_K && dev->px && !accum && !bias && N >= 32768u && K <= 8192u) {
+        uint32_t sg[3], sb[3];
+        const std::string name = base + "_px";
+        int rc = ojh_launch_shape(dev, name.c_str(), K, N, 1, sg, sb);
+        if (rc) return rc;
+        return ojh_launch(dev, name.c_str(), {xq, xs, wp, yp}, {K, N}, sg, sb);
+    }
     if (m == 1) {
         int r = (accum || bias) ? 1 : pick_rows(dev, N);
         bool wide = !accum && !bias && r == 2 && N >= 32768u;

@@ -397,3 +397,30 @@ def test_q6k_tokens_on_the_int8_matrix_cores(gpu, orc, pkg, m, n, k, accum):
     assert peak_err(outs[0], outs[1]) <= 2e-6
     with pytest.raises(pkg.OjasHipError, match="do not fit"):
         gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_mf", [(xq, 0), (xs, 0), (wd, 0), (y2, 0)], [k, n, 17, 0], [8, 1, 1], [256, 1, 1])
+
+
+@pytest.mark.parametrize("n,k", [(33000, 256), (40001, 2560), (32768, 8192)])
+def test_q6k_head_form_keeps_activations_in_registers(gpu, orc, pkg, n, k):
+    """From 32768 rows a Q6_K matvec runs grid-stride with the activations in registers: the lane
+    arithmetic of the row-per-wave kernel, so the same bits, checked by name against `_r2`, and the
+    oracle's values; partly filled steps (K = 256, 2560), two steps (K = 8192), odd row counts."""
+    w, x = _inputs(pkg, Q6_K, n, k, "px")
+    lin = gpu.lin(Q6_K, n, k, w)
+    yd = gpu.upload(np.full(n + 2, 12345.0, np.float32))
+    gpu.mm(gpu.upload(x), lin, yd, 1, act_mode=pkg.ACT_Q8K, y_off=4)
+    got = gpu.read(yd, n + 2)
+    assert got[0] == 12345.0 and got[-1] == 12345.0, "wrote outside y"
+    assert peak_err(got[1:-1], orc.matvec_kq(w, Q6_K, n, k, x)) <= TOL_Q8K_SEEN
+    gpu.ensure_family("gemv_q8k")
+    xq, xs = gpu.alloc_bytes(k), gpu.alloc(k // 256)
+    gpu.quant_q8k(gpu.upload(x), 1, k, xq, xs)
+    wd = gpu.upload_bytes(w)
+    outs = []
+    for name in ("gemv_q8k_q6k_px", "gemv_q8k_q6k_r2"):
+        grid, block = gpu.launch_shape(name, k, n, 1)
+        y2 = gpu.alloc(n)
+        gpu.dispatch(gpu.begin(), name, [(xq, 0), (xs, 0), (wd, 0), (y2, 0)], [k, n], grid, block)
+        outs.append(gpu.read(y2, n))
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], got[1:-1])
+    with pytest.raises(pkg.OjasHipError, match="8192"):
+        gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_px", [(xq, 0), (xs, 0), (wd, 0), (y2, 0)], [16384, n, 0][:2], [8, 1, 1], [256, 1, 1])
