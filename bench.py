@@ -271,6 +271,14 @@ def extras(gpu, pkg, lin_q) -> dict:
     b = n * (k // 32) * 34 + 4 * k + 4 * n
     out["q80_gemv_4096x4096"] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
     del wq8
+    # the same contract on a tall matrix (rows staged through LDS, activations in registers)
+    n = 128256
+    wq8 = [gpu.lin(pkg.Q8_0, n, k, synth.q80_weights(n, k, "bench", "q80_head")) for _ in range(2)]
+    y = gpu.alloc(n)
+    us = _time(gpu, lambda i: gpu.mm(x, wq8[i % 2], y), 20, 3)
+    b = n * (k // 32) * 34 + 4 * k + 4 * n
+    out["q80_gemv_128256x4096"] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
+    del wq8
     # ---- one FFN block of a decode layer with the fused epilogues: rmsnorm+quantize, gate/up+SiLU,
     # quantize, down accumulated onto the residual (4 launches, recorded and replayed)
     d, nff = 4096, 14336
@@ -330,7 +338,8 @@ def extras(gpu, pkg, lin_q) -> dict:
         b = n * (k // 256) * 210 + m * (2 * k + 4 * n)
         ver[f"M{m}"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4),
                         "tflops": round(2.0 * m * n * k / us / 1e6, 2)}
-    out["verify_q6k_head_151936x4096"] = {"activations": "bf16, quantized per 256 (quant_q8k)", **ver}
+    out["verify_q6k_head_151936x4096"] = {"activations": "bf16, quantized per 256 (quant_q8k)",
+                                          "kernels": "M1 gemv_q8k_q6k_px, M2 gemv_q8k_q6k_mx, M4-16 gemv_q8k_q6k_mf (int8 MFMA)", **ver}
     return out
 
 
