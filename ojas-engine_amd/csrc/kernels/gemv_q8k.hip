@@ -66,6 +66,16 @@ __device__ __forceinline__ void store_row(float* y, const float* bs, uint n, flo
     else if (MODE == ST_ACCUM) y[n] += v;
     else y[n] = v + bs[n];
 }
+// The value an accumulate / bias store adds, fetched when the wave starts instead of after its
+// last reduction (a dependent load at the tail of every wave otherwise).
+template <int MODE>
+__device__ __forceinline__ float store_addend(const float* y, const float* bs, uint n) {
+    return MODE == ST_ACCUM ? y[n] : MODE == ST_BIAS ? bs[n] : 0.0f;
+}
+template <int MODE>
+__device__ __forceinline__ void store_row_with(float* y, uint n, float v, float addend) {
+    y[n] = MODE == ST_SET ? v : MODE == ST_ACCUM ? addend + v : v + addend;
+}
 
 // ------------------------------------------------------------------ Q4_K (lane dot: ojk_q4k_dot.h)
 template <int R, int MODE>
@@ -76,9 +86,12 @@ __device__ __forceinline__ void gemv_q8k_q4k_body(const signed char* __restrict_
     const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
     if (row0 >= N) return;
     const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
-    float acc[R];
+    float acc[R], add[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.0f;
+        add[r] = store_addend<MODE>(y, bs, min(row0 + r, N - 1u));
+    }
     for (uint sb = g; sb < nsb; sb += 8u) {
         uint4 hdr[R], qs[R];
 #pragma unroll
@@ -95,7 +108,7 @@ __device__ __forceinline__ void gemv_q8k_q4k_body(const signed char* __restrict_
 #pragma unroll
     for (int r = 0; r < R; r++) {
         float t = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, t);
+        if (lane == 0 && row0 + r < N) store_row_with<MODE>(y, row0 + r, t, add[r]);
     }
 }
 
@@ -161,9 +174,12 @@ __device__ __forceinline__ void gemv_q8k_q5k_body(const signed char* __restrict_
     const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
     if (row0 >= N) return;
     const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
-    float acc[R];
+    float acc[R], add[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.0f;
+        add[r] = store_addend<MODE>(y, bs, min(row0 + r, N - 1u));
+    }
     for (uint sb = g; sb < nsb; sb += 8u) {
         uint4 hdr[R], qs[R], qh[R];
 #pragma unroll
@@ -180,7 +196,7 @@ __device__ __forceinline__ void gemv_q8k_q5k_body(const signed char* __restrict_
 #pragma unroll
     for (int r = 0; r < R; r++) {
         float t = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, t);
+        if (lane == 0 && row0 + r < N) store_row_with<MODE>(y, row0 + r, t, add[r]);
     }
 }
 
@@ -368,12 +384,28 @@ rmsnorm_q8k(const float* __restrict__ x, const float* __restrict__ gamma, signed
             for (int e = 0; e < 4; e++) o[e] = i0 + e < K ? p[i0 + e] : 0.0f;
         }
     };
+    // up to 4096 values the row and gamma stay in registers between the two passes
+    const bool keep = nsb <= 16u;
+    float kv[4][4], kg[4][4];
     double ss = 0.0;
-    for (uint seg = wave; seg < nsb; seg += 4u) {
-        float v[4];
-        load4(row, seg * 256u + lane * 4u, v);
+    if (keep) {
 #pragma unroll
-        for (int e = 0; e < 4; e++) ss += (double)v[e] * (double)v[e];
+        for (int j = 0; j < 4; j++) {
+            const uint i0 = (wave + 4u * j) * 256u + lane * 4u;
+            load4(row, i0, kv[j]);        // past the row: zeros
+            load4(gamma, i0, kg[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) ss += (double)kv[j][e] * (double)kv[j][e];
+    } else {
+        for (uint seg = wave; seg < nsb; seg += 4u) {
+            float v[4];
+            load4(row, seg * 256u + lane * 4u, v);
+#pragma unroll
+            for (int e = 0; e < 4; e++) ss += (double)v[e] * (double)v[e];
+        }
     }
     // wave reduction in f64 through two 32-bit halves
     for (int off = 32; off > 0; off >>= 1) {
@@ -385,11 +417,19 @@ rmsnorm_q8k(const float* __restrict__ x, const float* __restrict__ gamma, signed
     __syncthreads();
     const float mean = (float)(((part[0] + part[1]) + (part[2] + part[3])) / (double)K);
     const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(mean, __uint_as_float(EPS_BITS))));
-    for (uint seg = wave; seg < nsb; seg += 4u) {
+    for (uint seg = wave, j = 0; seg < nsb; seg += 4u, j++) {
         const uint i0 = seg * 256u + lane * 4u;
         float v[4], gm[4], t[4];
-        load4(row, i0, v);      // second read: from the cache
-        load4(gamma, i0, gm);
+        if (keep) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                v[e] = j == 0 ? kv[0][e] : j == 1 ? kv[1][e] : j == 2 ? kv[2][e] : kv[3][e];
+                gm[e] = j == 0 ? kg[0][e] : j == 1 ? kg[1][e] : j == 2 ? kg[2][e] : kg[3][e];
+            }
+        } else {
+            load4(row, i0, v);      // second read: from the cache
+            load4(gamma, i0, gm);
+        }
 #pragma unroll
         for (int e = 0; e < 4; e++) t[e] = i0 + e < K ? __fmul_rn(__fmul_rn(v[e], inv), gm[e]) : 0.0f;
         const float a = wave_max(fmaxf(fmaxf(fabsf(t[0]), fabsf(t[1])), fmaxf(fabsf(t[2]), fabsf(t[3]))));
@@ -632,9 +672,12 @@ __device__ __forceinline__ void gemv_q8k_q6k_body(const signed char* __restrict_
     const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
     if (row0 >= N) return;
     const uint nsb = K >> 8, g = lane >> 2, hf = (lane >> 1) & 1u, l0 = (lane & 1u) * 16u;
-    float acc[R];
+    float acc[R], add[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.0f;
+        add[r] = store_addend<MODE>(y, bs, min(row0 + r, N - 1u));
+    }
     for (uint sb = g; sb < nsb; sb += 16u) {
         Q6kW raw[R];
 #pragma unroll
@@ -649,7 +692,7 @@ __device__ __forceinline__ void gemv_q8k_q6k_body(const signed char* __restrict_
 #pragma unroll
     for (int r = 0; r < R; r++) {
         float s = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, s);
+        if (lane == 0 && row0 + r < N) store_row_with<MODE>(y, row0 + r, s, add[r]);
     }
 }
 
