@@ -411,9 +411,10 @@ moe_down_q4k_dec(const float* __restrict__ act, const uchar* __restrict__ wd, co
 // 4-bit codes as bytes (B: lane (n, kg) holds the same bytes of row n); D register v of lane
 // (n, kg) is the integer dot of token 4 kg + v with row n.  A second MFMA against a tile of ones
 // gives every lane the activations' sub-block sums in the same layout, so the scale algebra
-//     sum_sb sx[t][sb] * sum_j ( d sc_j * idot_j  -  dmin m_j * bsum_j )
-// needs no cross-lane traffic: per MFMA four converts and four FMAs with lane-constant scales
-// (about a fifth of the vector instructions of the integer-dot form).  A token's result does not
+//     sum_sb sx[t][sb] * ( d * sum_j sc_j * idot_j  -  dmin * sum_j m_j * bsum_j )
+// needs no cross-lane traffic: per MFMA result register one integer multiply-add with a
+// lane-constant 6-bit scale (the sums over j are exact in int32: |.| < 2^25), and per super-block
+// two converts and three FMAs, the form of dot_q4k itself (crates/ojas-cpu/src/cpu_math.rs:609-635).  A token's result does not
 // depend on which other tokens share its tile.
 typedef int int4v __attribute__((ext_vector_type(4)));
 
@@ -426,7 +427,10 @@ __device__ __forceinline__ long pack2(uint lo, uint hi) { return (long)(((unsign
 template <int NW>
 __device__ __forceinline__ void mm_superblock(const signed char* xsb, const uchar* const (&wblk)[NW], uint kg,
                                               const float (&sx)[4], float (&acc)[NW][4]) {
-    float tmp[NW][4], d[NW], dmin[NW];
+    // integer partial sums are exact, so sum_j sc_j * idot_j and sum_j m_j * bsum_j are formed in
+    // int32 (one v_mad_i32_i24 per MFMA result register) and converted once per super-block
+    int isum[NW][4], msum[NW][4];
+    float d[NW], dmin[NW];
     uint s0[NW], s1[NW], s2[NW];
 #pragma unroll
     for (int w = 0; w < NW; w++) {
@@ -435,7 +439,7 @@ __device__ __forceinline__ void mm_superblock(const signed char* xsb, const ucha
         dmin[w] = f16_bits_to_f32(hdr.x >> 16);
         s0[w] = hdr.y; s1[w] = hdr.z; s2[w] = hdr.w;
 #pragma unroll
-        for (int v = 0; v < 4; v++) tmp[w][v] = 0.0f;
+        for (int v = 0; v < 4; v++) { isum[w][v] = 0; msum[w][v] = 0; }
     }
     const long ones = 0x0101010101010101L;
     const int4v zero = {0, 0, 0, 0};
@@ -451,22 +455,21 @@ __device__ __forceinline__ void mm_superblock(const signed char* xsb, const ucha
         for (int w = 0; w < NW; w++) {
             uint sc, mn;
             q4k_scale_min_pair(s0[w], s1[w], s2[w], c, sc, mn);
-            const float a_lo = d[w] * (float)(sc & 0xFFu), a_hi = d[w] * (float)(sc >> 8);
-            const float m_lo = dmin[w] * (float)(mn & 0xFFu), m_hi = dmin[w] * (float)(mn >> 8);
+            const int sc_lo = (int)(sc & 0xFFu), sc_hi = (int)(sc >> 8), m_lo = (int)(mn & 0xFFu), m_hi = (int)(mn >> 8);
             const uint2 q = *(const uint2*)(wblk[w] + 16u + c * 32u + 8u * kg);
             const int4v dl = __builtin_amdgcn_mfma_i32_16x16x32_i8(A0, pack2(q.x & 0x0F0F0F0Fu, q.y & 0x0F0F0F0Fu), zero, 0, 0, 0);
             const int4v dh = __builtin_amdgcn_mfma_i32_16x16x32_i8(A1, pack2((q.x >> 4) & 0x0F0F0F0Fu, (q.y >> 4) & 0x0F0F0F0Fu), zero, 0, 0, 0);
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                tmp[w][v] += a_lo * (float)dl[v] - m_lo * (float)b0[v];
-                tmp[w][v] += a_hi * (float)dh[v] - m_hi * (float)b1[v];
+                isum[w][v] += __mul24(sc_lo, dl[v]) + __mul24(sc_hi, dh[v]);
+                msum[w][v] += __mul24(m_lo, b0[v]) + __mul24(m_hi, b1[v]);
             }
         }
     }
 #pragma unroll
     for (int w = 0; w < NW; w++)
 #pragma unroll
-        for (int v = 0; v < 4; v++) acc[w][v] += sx[v] * tmp[w][v];
+        for (int v = 0; v < 4; v++) acc[w][v] += sx[v] * (d[w] * (float)isum[w][v] - dmin[w] * (float)msum[w][v]);
 }
 
 // Copy the super-block `sb` of 16 consecutive rows (144 bytes each, `rb` apart, rows past `nrows`
