@@ -139,33 +139,6 @@ GEMV_Q8K_ENTRIES(q4k, gemv_q8k_q4k_body)
 // The fifth bit of weight l of sub-block j is bit j of qh[l] (crates/ojas-cpu/src/cpu_math.rs:638-670),
 // so a lane adds 16 * dot(bit plane, x) to each of its two nibble dots: the 16 qh bytes it needs
 // are those at the positions of its 16 quant bytes within the 32-byte chunk.
-__device__ __forceinline__ float q5k_lane_dot(uint4 hdr, uint4 qs, uint4 qh, uint c, const Q4kFrag& f) {
-    const uint M4 = 0x0F0F0F0Fu, B1 = 0x01010101u;
-    const uint sl = 2u * c, sh = 2u * c + 1u;
-    int il = dot4_i8(qs.x & M4, f.xl.x, 0);
-    il = dot4_i8(qs.y & M4, f.xl.y, il);
-    il = dot4_i8(qs.z & M4, f.xl.z, il);
-    il = dot4_i8(qs.w & M4, f.xl.w, il);
-    int bl = dot4_i8((qh.x >> sl) & B1, f.xl.x, 0);
-    bl = dot4_i8((qh.y >> sl) & B1, f.xl.y, bl);
-    bl = dot4_i8((qh.z >> sl) & B1, f.xl.z, bl);
-    bl = dot4_i8((qh.w >> sl) & B1, f.xl.w, bl);
-    int ih = dot4_i8((qs.x >> 4) & M4, f.xh.x, 0);
-    ih = dot4_i8((qs.y >> 4) & M4, f.xh.y, ih);
-    ih = dot4_i8((qs.z >> 4) & M4, f.xh.z, ih);
-    ih = dot4_i8((qs.w >> 4) & M4, f.xh.w, ih);
-    int bh = dot4_i8((qh.x >> sh) & B1, f.xh.x, 0);
-    bh = dot4_i8((qh.y >> sh) & B1, f.xh.y, bh);
-    bh = dot4_i8((qh.z >> sh) & B1, f.xh.z, bh);
-    bh = dot4_i8((qh.w >> sh) & B1, f.xh.w, bh);
-    uint sc, mn;
-    q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
-    const int isum = (int)(sc & 0xFFu) * (il + 16 * bl) + (int)(sc >> 8) * (ih + 16 * bh);
-    const int msum = (int)(mn & 0xFFu) * f.bl + (int)(mn >> 8) * f.bh;
-    const float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
-    return f.sx * (d * (float)isum - dmin * (float)msum);
-}
-
 template <int R, int MODE>
 __device__ __forceinline__ void gemv_q8k_q5k_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
                                                   const uchar* __restrict__ w, float* __restrict__ y,

@@ -20,10 +20,10 @@
 //   moe_topk_m(lg, idx, wgt, E, KSEL)                        grid = tokens
 //   moe_group(idx, counts, offsets, list, NA, E)             1 x 256 threads; NA = tokens*KSEL
 //   moe_gu_q4k_m(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA)   grid (ceil(N/8), E)
-//   moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)            grid (ceil(N/16), E)
+//   moe_down_{q4k,q5k}_m(aq, as, wd, dv, offsets, list, K, N, NA)      grid (ceil(N/16), E)
 //   moe_combine(dv, wgt, y, T, KSEL, D, ACC)                 grid ceil(T*D/256)
 //   moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)   grid (ceil(N/8), NA): few tokens, f32 in
-//   moe_down_q4k_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)  grid (ceil(N/8), T): down + weighted sum
+//   moe_down_{q4k,q5k}_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)  grid (ceil(N/8), T): down + weighted sum
 //   moe_gu_q4k_mm / moe_down_q4k_mm (same arguments as the _m entries)
 //                                                            grid (ceil(N/16), E): the int8 matrix-core form
 #include "ojk_common.h"
@@ -202,10 +202,11 @@ moe_gu_q4k_m(const signed char* __restrict__ xq, const float* __restrict__ xs, c
 // ------------------------------------------------------------------ grouped down
 // Block (rb, e): 4 waves x 4 rows = 16 rows of expert e's down projection, against the quantized
 // act of every assignment routed to e.  dv[a][n] holds the unweighted result.
-extern "C" __global__ void __launch_bounds__(256)
-moe_down_q4k_m(const signed char* __restrict__ aq, const float* __restrict__ as_, const uchar* __restrict__ wd,
-               float* __restrict__ dv, const uint* __restrict__ offsets, const uint* __restrict__ list,
-               uint K, uint N, uint NA) {
+template <class W>
+__device__ __forceinline__ void moe_down_m_body(const signed char* __restrict__ aq, const float* __restrict__ as_,
+                                                const uchar* __restrict__ wd, float* __restrict__ dv,
+                                                const uint* __restrict__ offsets, const uint* __restrict__ list,
+                                                uint K, uint N, uint NA) {
     const uint e = blockIdx.y;
     const uint a0 = min(offsets[e], NA), a1 = min(offsets[e + 1], NA);
     if (a0 >= a1) return;
@@ -213,24 +214,20 @@ moe_down_q4k_m(const signed char* __restrict__ aq, const float* __restrict__ as_
     const uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 4u;
     if (row0 >= N) return;
     const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
-    const size_t rb = (size_t)nsb * Q4K_BYTES;
+    const size_t rb = (size_t)nsb * W::BYTES;
     const uchar* w0 = wd + ((size_t)e * N + row0) * rb;
     if (nsb <= 8u) {
         const bool on = g < nsb;
-        const size_t o = (size_t)(on ? g : 0u) * Q4K_BYTES;
-        uint4 h[4], q[4];
+        const size_t o = (size_t)(on ? g : 0u) * W::BYTES;
+        W wr[4];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const size_t ro = (size_t)min((uint)r, N - 1u - row0) * rb;
-            h[r] = *(const uint4*)(w0 + ro + o);
-            q[r] = *(const uint4*)(w0 + ro + o + 16u + l * 16u);
-        }
+        for (int r = 0; r < 4; r++) wr[r].load(w0 + (size_t)min((uint)r, N - 1u - row0) * rb + o, l);
         for (uint i = a0; i < a1; i++) {
             const uint a = min(list[i], NA - 1u);
             Q4kFrag f = q4k_load_frag(aq + (size_t)a * nsb * 256u, as_ + (size_t)a * nsb, on ? g : 0u, l);
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                float v = wave_sum(on ? q4k_lane_dot(h[r], q[r], c, f) : 0.0f);
+                float v = wave_sum(on ? wr[r].dot(c, f) : 0.0f);
                 if (lane == 0 && row0 + r < N) dv[(size_t)a * N + row0 + r] = v;
             }
         }
@@ -242,8 +239,9 @@ moe_down_q4k_m(const signed char* __restrict__ aq, const float* __restrict__ as_
                 Q4kFrag f = q4k_load_frag(aq + (size_t)a * nsb * 256u, as_ + (size_t)a * nsb, sb, l);
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const uchar* blk = w0 + (size_t)min((uint)r, N - 1u - row0) * rb + (size_t)sb * Q4K_BYTES;
-                    v[r] += q4k_lane_dot(*(const uint4*)blk, *(const uint4*)(blk + 16u + l * 16u), c, f);
+                    W wr;
+                    wr.load(w0 + (size_t)min((uint)r, N - 1u - row0) * rb + (size_t)sb * W::BYTES, l);
+                    v[r] += wr.dot(c, f);
                 }
             }
 #pragma unroll
@@ -253,6 +251,17 @@ moe_down_q4k_m(const signed char* __restrict__ aq, const float* __restrict__ as_
             }
         }
     }
+}
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q4k_m(const signed char* aq, const float* as_, const uchar* wd, float* dv, const uint* offsets,
+               const uint* list, uint K, uint N, uint NA) {
+    moe_down_m_body<W4k>(aq, as_, wd, dv, offsets, list, K, N, NA);
+}
+// the same over Q5_K rows (an expert's down tensor is often kept a step finer than gate / up)
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q5k_m(const signed char* aq, const float* as_, const uchar* wd, float* dv, const uint* offsets,
+               const uint* list, uint K, uint N, uint NA) {
+    moe_down_m_body<W5k>(aq, as_, wd, dv, offsets, list, K, N, NA);
 }
 
 // ------------------------------------------------------------------ decode: a few tokens, two launches
@@ -337,9 +346,10 @@ moe_gu_q4k_dec(const float* __restrict__ x, const uchar* __restrict__ wg, const 
 // pairs side by side instead of one slot at a time: group sums go through LDS, lane j rebuilds
 // slot j's dot with the association of wave_sum, and the slots are added in order,
 //     y[t][row] (=, +=) sum_j wgt[t][j] * (Wd_{idx[t][j]} act[t][j])[row].
-extern "C" __global__ void __launch_bounds__(256)
-moe_down_q4k_dec(const float* __restrict__ act, const uchar* __restrict__ wd, const uint* __restrict__ idx,
-                 const float* __restrict__ wgt, float* __restrict__ y, uint K, uint N, uint KSEL, uint E, uint ACC) {
+template <class W>
+__device__ __forceinline__ void moe_down_dec_body(const float* __restrict__ act, const uchar* __restrict__ wd,
+                                                  const uint* __restrict__ idx, const float* __restrict__ wgt,
+                                                  float* __restrict__ y, uint K, uint N, uint KSEL, uint E, uint ACC) {
     __shared__ __align__(16) signed char aq[MOE_DEC_DOWN_ACT];
     __shared__ float as_[MOE_DEC_DOWN_ACT / 256u];
     __shared__ uint s_idx[64];
@@ -348,30 +358,32 @@ moe_down_q4k_dec(const float* __restrict__ act, const uchar* __restrict__ wd, co
     const uint row0 = min(blockIdx.x * 8u + wave * 2u, N - 1u);   // surplus waves repeat the last row
     const bool two = row0 + 1u < N;
     const uint nsb = K >> 8, G = lane >> 3, l = lane & 7u, c = l >> 1;
-    const size_t rb = (size_t)nsb * Q4K_BYTES, r1 = two ? rb : 0;
+    const size_t rb = (size_t)nsb * W::BYTES, r1 = two ? rb : 0;
     const uint* ti = idx + (size_t)t * KSEL;
     const uint U = KSEL * nsb;
     // the first pass's weights are on their way while the activations are quantized
     uint u = min(G, U - 1u), j = u / nsb, sb = u - j * nsb;
-    const uchar* w = wd + (((size_t)min(ti[j], E - 1u) * N + row0) * nsb + sb) * Q4K_BYTES;
-    uint4 h0 = *(const uint4*)w, p0 = *(const uint4*)(w + 16u + l * 16u);
-    uint4 h1 = *(const uint4*)(w + r1), p1 = *(const uint4*)(w + r1 + 16u + l * 16u);
+    const uchar* w = wd + (((size_t)min(ti[j], E - 1u) * N + row0) * nsb + sb) * W::BYTES;
+    W w0, w1;
+    w0.load(w, l);
+    w1.load(w + r1, l);
     if (threadIdx.x < KSEL) s_idx[threadIdx.x] = min(ti[threadIdx.x], E - 1u);
     block_quant_q8k(act + (size_t)t * KSEL * K, KSEL * K, aq, as_);
     __syncthreads();
     for (uint u0 = 0; u0 < U; u0 += 8u) {
         const bool on = u0 + G < U;
         const uint un = min(u0 + 8u + G, U - 1u), jn = un / nsb, sbn = un - jn * nsb;
-        const uchar* wn = wd + (((size_t)s_idx[jn] * N + row0) * nsb + sbn) * Q4K_BYTES;
-        const uint4 nh0 = *(const uint4*)wn, np0 = *(const uint4*)(wn + 16u + l * 16u);
-        const uint4 nh1 = *(const uint4*)(wn + r1), np1 = *(const uint4*)(wn + r1 + 16u + l * 16u);
+        const uchar* wn = wd + (((size_t)s_idx[jn] * N + row0) * nsb + sbn) * W::BYTES;
+        W n0, n1;
+        n0.load(wn, l);
+        n1.load(wn + r1, l);
         const Q4kFrag f = q4k_load_frag(aq + (size_t)j * K, as_ + (size_t)j * nsb, sb, l);
-        const float v0 = oct_sum(q4k_lane_dot(h0, p0, c, f)), v1 = oct_sum(q4k_lane_dot(h1, p1, c, f));
+        const float v0 = oct_sum(w0.dot(c, f)), v1 = oct_sum(w1.dot(c, f));
         if (on && l == 0) {
             part[wave][0][j][sb] = v0;
             part[wave][1][j][sb] = v1;
         }
-        j = jn; sb = sbn; h0 = nh0; p0 = np0; h1 = nh1; p1 = np1;
+        j = jn; sb = sbn; w0 = n0; w1 = n1;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -402,6 +414,16 @@ moe_down_q4k_dec(const float* __restrict__ act, const uchar* __restrict__ wd, co
         y[(size_t)t * N + row0] = acc0;
         if (two) y[(size_t)t * N + row0 + 1u] = acc1;
     }
+}
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q4k_dec(const float* act, const uchar* wd, const uint* idx, const float* wgt, float* y, uint K, uint N,
+                 uint KSEL, uint E, uint ACC) {
+    moe_down_dec_body<W4k>(act, wd, idx, wgt, y, K, N, KSEL, E, ACC);
+}
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q5k_dec(const float* act, const uchar* wd, const uint* idx, const float* wgt, float* y, uint K, uint N,
+                 uint KSEL, uint E, uint ACC) {
+    moe_down_dec_body<W5k>(act, wd, idx, wgt, y, K, N, KSEL, E, ACC);
 }
 
 // ------------------------------------------------------------------ grouped products on the matrix cores

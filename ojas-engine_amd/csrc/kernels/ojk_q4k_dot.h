@@ -87,3 +87,54 @@ __device__ __forceinline__ float q4k_lane_dot(uint4 hdr, uint4 qs, uint c, const
     float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
     return f.sx * (d * (float)isum - dmin * (float)msum);
 }
+
+// Q5_K: the same 32 weights with their fifth bits.  Bit j of qh[l] belongs to weight l of
+// sub-block j (crates/ojas-cpu/src/cpu_math.rs:638-670); `qh` holds the 16 bytes at the positions
+// of the lane's 16 quant bytes.
+__device__ __forceinline__ float q5k_lane_dot(uint4 hdr, uint4 qs, uint4 qh, uint c, const Q4kFrag& f) {
+    const uint M4 = 0x0F0F0F0Fu, B1 = 0x01010101u;
+    const uint sl = 2u * c, sh = 2u * c + 1u;
+    int il = dot4_i8(qs.x & M4, f.xl.x, 0);
+    il = dot4_i8(qs.y & M4, f.xl.y, il);
+    il = dot4_i8(qs.z & M4, f.xl.z, il);
+    il = dot4_i8(qs.w & M4, f.xl.w, il);
+    int bl = dot4_i8((qh.x >> sl) & B1, f.xl.x, 0);
+    bl = dot4_i8((qh.y >> sl) & B1, f.xl.y, bl);
+    bl = dot4_i8((qh.z >> sl) & B1, f.xl.z, bl);
+    bl = dot4_i8((qh.w >> sl) & B1, f.xl.w, bl);
+    int ih = dot4_i8((qs.x >> 4) & M4, f.xh.x, 0);
+    ih = dot4_i8((qs.y >> 4) & M4, f.xh.y, ih);
+    ih = dot4_i8((qs.z >> 4) & M4, f.xh.z, ih);
+    ih = dot4_i8((qs.w >> 4) & M4, f.xh.w, ih);
+    int bh = dot4_i8((qh.x >> sh) & B1, f.xh.x, 0);
+    bh = dot4_i8((qh.y >> sh) & B1, f.xh.y, bh);
+    bh = dot4_i8((qh.z >> sh) & B1, f.xh.z, bh);
+    bh = dot4_i8((qh.w >> sh) & B1, f.xh.w, bh);
+    uint sc, mn;
+    q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
+    const int isum = (int)(sc & 0xFFu) * (il + 16 * bl) + (int)(sc >> 8) * (ih + 16 * bh);
+    const int msum = (int)(mn & 0xFFu) * f.bl + (int)(mn >> 8) * f.bh;
+    const float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
+    return f.sx * (d * (float)isum - dmin * (float)msum);
+}
+
+// A lane's bytes of one super-block of one row, by format: what the MoE kernels are written over.
+struct W4k {
+    static constexpr uint BYTES = Q4K_BYTES;
+    uint4 h, q;
+    __device__ __forceinline__ void load(const uchar* blk, uint l) {
+        h = *(const uint4*)blk;
+        q = *(const uint4*)(blk + 16u + l * 16u);
+    }
+    __device__ __forceinline__ float dot(uint c, const Q4kFrag& f) const { return q4k_lane_dot(h, q, c, f); }
+};
+struct W5k {
+    static constexpr uint BYTES = Q5K_BYTES;
+    uint4 h, q, qh;
+    __device__ __forceinline__ void load(const uchar* blk, uint l) {
+        h = *(const uint4*)blk;
+        qh = *(const uint4*)(blk + 16u + (l & 1u) * 16u);
+        q = *(const uint4*)(blk + 48u + l * 16u);
+    }
+    __device__ __forceinline__ float dot(uint c, const Q4kFrag& f) const { return q5k_lane_dot(h, q, qh, c, f); }
+};

@@ -544,7 +544,7 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
             return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/%u), E, 1]", s->name, per);
         need[0] = (size_t)NA * K;
         need[1] = (size_t)NA * (K / 256) * 4;
-        need[2] = (size_t)E * N * (K / 256) * 144;
+        need[2] = (size_t)E * N * (K / 256) * ojh_format(s->type)->bytes;
         need[3] = (size_t)NA * N * 4;
         need[4] = (size_t)(E + 1) * 4;
         need[5] = (size_t)NA * 4;
@@ -574,7 +574,7 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         if (grid[0] != (N + 7) / 8 || !T || grid[2] != 1)
             return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/8), tokens, 1]", s->name);
         need[0] = (size_t)T * KS * K * 4;
-        need[1] = (size_t)E * N * (K / 256) * 144;
+        need[1] = (size_t)E * N * (K / 256) * ojh_format(s->type)->bytes;
         need[2] = need[3] = (size_t)T * KS * 4;
         need[4] = (size_t)T * N * 4;
         align[0] = align[1] = 16;
@@ -806,6 +806,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("moe_down_q4k_mm", "moe", 6, 3, OJH_Q4_K, 7, check_moe, shape_moe);
     add("moe_gu_q4k_dec", "moe", 5, 5, OJH_Q4_K, 8, check_moe, shape_moe);
     add("moe_down_q4k_dec", "moe", 5, 5, OJH_Q4_K, 9, check_moe, shape_moe);
+    add("moe_down_q5k_m", "moe", 6, 3, OJH_Q5_K, 4, check_moe, shape_moe);
+    add("moe_down_q5k_dec", "moe", 5, 5, OJH_Q5_K, 9, check_moe, shape_moe);
     add("copy_bf16_half", "glue", 2, 1, (2u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     // glue: `type` carries (input element bytes << 8 | output element bytes)
     add("copy_f32_half", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);
