@@ -257,6 +257,17 @@ int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint32_t d
                 const ojh_lin *gate, const ojh_lin *up, const ojh_lin *down, ojh_buf *y,
                 int accum, int act_mode);
 
+/* The same over streamed experts: the matrices of assignment a = (token, slot) start at byte
+ * offset off_*[a] (u64, 16-byte aligned) of their arena, wherever the caller's expert cache put
+ * them (crates/ojas-cuda/src/kernels/moe.rs:133-174 `moe_{gu,down}_*_slots`,
+ * crates/ojas-cuda/src/expert_cache.rs). Q4_K experts, the two-launch form at any token count;
+ * d <= 8192, n_ff <= 2048, ksel <= 64, ksel * n_ff <= 32768. An offset at which a whole expert
+ * does not fit is clamped to the last one at which it does. */
+int ojh_moe_ffn_slots(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint32_t d, uint32_t n_ff,
+                      uint32_t ksel, const ojh_buf *arena_gate, const ojh_buf *off_gate,
+                      const ojh_buf *arena_up, const ojh_buf *off_up, const ojh_buf *arena_down,
+                      const ojh_buf *off_down, const ojh_buf *wgt, ojh_buf *y, int accum);
+
 /* ---- GGUF files -> device (no GPU needed for the reader itself) --------------------------------
  * `Gguf::open` / `tensor_meta` / `read_tensor_raw` (crates/ojas-formats/src/gguf.rs:100-206, 297-339,
  * 440-452, 551-556): versions 2 and 3, the reference's header limits, `general.alignment`, extents

@@ -24,6 +24,8 @@
 //   moe_combine(dv, wgt, y, T, KSEL, D, ACC)                 grid ceil(T*D/256)
 //   moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)   grid (ceil(N/8), NA): few tokens, f32 in
 //   moe_down_{q4k,q5k}_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)  grid (ceil(N/8), T): down + weighted sum
+//   moe_gu_q4k_slots(x, arena_g, arena_u, act, off_g, off_u, K, N, KSEL, NA, LIM_G, LIM_U)   the decode form over
+//   moe_down_q4k_slots(act, arena, off_d, wgt, y, K, N, KSEL, LIM, ACC)                     streamed experts (u64 byte offsets)
 //   moe_gu_q4k_mm / moe_down_q4k_mm (same arguments as the _m entries)
 //                                                            grid (ceil(N/16), E): the int8 matrix-core form
 #include "ojk_common.h"
@@ -293,20 +295,34 @@ __device__ __forceinline__ void block_quant_q8k(const float* __restrict__ x, uin
     }
 }
 
-// Block (rb, a): 4 waves x 2 rows of gate and up of expert idx[a] against token a / KSEL.
-extern "C" __global__ void __launch_bounds__(256)
-moe_gu_q4k_dec(const float* __restrict__ x, const uchar* __restrict__ wg, const uchar* __restrict__ wu,
-               float* __restrict__ act, const uint* __restrict__ idx, uint K, uint N, uint KSEL, uint NA, uint E) {
+// Where an assignment's expert starts, in bytes from the tensor (or arena) base.  Resident experts
+// are indexed (idx[a] * N rows); streamed experts sit wherever the host's cache put them and come
+// as one byte offset per assignment (the reference's `_slots` kernels,
+// crates/ojas-cuda/src/kernels/moe.rs:133-174).  Offsets are rounded down to 16 bytes and clamped
+// to `lim256` * 256, the last offset at which a whole expert still fits.
+__device__ __forceinline__ size_t expert_base(const void* sel, uint a, bool slots, uint e_or_lim, size_t expert_bytes) {
+    if (slots) {
+        const size_t o = (size_t)((const unsigned long*)sel)[a] & ~(size_t)15;
+        return min(o, (size_t)e_or_lim * 256u);
+    }
+    return (size_t)min(((const uint*)sel)[a], e_or_lim - 1u) * expert_bytes;
+}
+
+// Block (rb, a): 4 waves x 2 rows of gate and up of assignment a's expert against token a / KSEL.
+template <bool SLOTS>
+__device__ __forceinline__ void moe_gu_dec_body(const float* __restrict__ x, const uchar* __restrict__ wg,
+                                                const uchar* __restrict__ wu, float* __restrict__ act,
+                                                const void* __restrict__ sel_g, const void* __restrict__ sel_u,
+                                                uint K, uint N, uint KSEL, uint EG, uint EU) {
     __shared__ __align__(16) signed char xq[MOE_DEC_GU_K];
     __shared__ float xs[MOE_DEC_GU_K / 256u];
-    const uint a = blockIdx.y;
-    const uint e = min(idx[a], E - 1u), t = a / KSEL;
+    const uint a = blockIdx.y, t = a / KSEL;
     const uint lane = threadIdx.x & 63u;
     const uint row0 = min((blockIdx.x * 4u + (threadIdx.x >> 6)) * 2u, N - 1u);   // surplus waves repeat the last row
     const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
     const size_t rb = (size_t)nsb * Q4K_BYTES;
-    const uchar* g0 = wg + ((size_t)e * N + row0) * rb;
-    const uchar* u0 = wu + ((size_t)e * N + row0) * rb;
+    const uchar* g0 = wg + expert_base(sel_g, a, SLOTS, EG, (size_t)N * rb) + (size_t)row0 * rb;
+    const uchar* u0 = wu + expert_base(sel_u, a, SLOTS, EU, (size_t)N * rb) + (size_t)row0 * rb;
     const bool two = row0 + 1u < N;
     const size_t r1 = two ? rb : 0;
     // the first step's weights are on their way while the activations are quantized
@@ -339,6 +355,16 @@ moe_gu_q4k_dec(const float* __restrict__ x, const uchar* __restrict__ wg, const 
         if (two) o_[1] = (vg1 / (1.0f + expf(-vg1))) * vu1;
     }
 }
+extern "C" __global__ void __launch_bounds__(256)
+moe_gu_q4k_dec(const float* x, const uchar* wg, const uchar* wu, float* act, const uint* idx, uint K, uint N, uint KSEL,
+               uint NA, uint E) {
+    moe_gu_dec_body<false>(x, wg, wu, act, idx, idx, K, N, KSEL, E, E);
+}
+extern "C" __global__ void __launch_bounds__(256)
+moe_gu_q4k_slots(const float* x, const uchar* arena_g, const uchar* arena_u, float* act, const unsigned long* off_g,
+                 const unsigned long* off_u, uint K, uint N, uint KSEL, uint NA, uint LIM_G, uint LIM_U) {
+    moe_gu_dec_body<true>(x, arena_g, arena_u, act, off_g, off_u, K, N, KSEL, LIM_G, LIM_U);
+}
 
 // Block (rb, t): 8 rows of the down projection for every slot of token t, 2 rows per wave.  The
 // workgroup quantizes the token's KSEL act vectors into LDS.  An expert's row is short (K / 256 <= 8
@@ -346,34 +372,33 @@ moe_gu_q4k_dec(const float* __restrict__ x, const uchar* __restrict__ wg, const 
 // pairs side by side instead of one slot at a time: group sums go through LDS, lane j rebuilds
 // slot j's dot with the association of wave_sum, and the slots are added in order,
 //     y[t][row] (=, +=) sum_j wgt[t][j] * (Wd_{idx[t][j]} act[t][j])[row].
-template <class W>
+template <class W, bool SLOTS>
 __device__ __forceinline__ void moe_down_dec_body(const float* __restrict__ act, const uchar* __restrict__ wd,
-                                                  const uint* __restrict__ idx, const float* __restrict__ wgt,
+                                                  const void* __restrict__ sel, const float* __restrict__ wgt,
                                                   float* __restrict__ y, uint K, uint N, uint KSEL, uint E, uint ACC) {
     __shared__ __align__(16) signed char aq[MOE_DEC_DOWN_ACT];
     __shared__ float as_[MOE_DEC_DOWN_ACT / 256u];
-    __shared__ uint s_idx[64];
+    __shared__ size_t s_base[64];
     __shared__ __align__(16) float part[4][2][64][8];   // [wave][row][slot][super-block] group sums
     const uint t = blockIdx.y, lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint row0 = min(blockIdx.x * 8u + wave * 2u, N - 1u);   // surplus waves repeat the last row
     const bool two = row0 + 1u < N;
     const uint nsb = K >> 8, G = lane >> 3, l = lane & 7u, c = l >> 1;
     const size_t rb = (size_t)nsb * W::BYTES, r1 = two ? rb : 0;
-    const uint* ti = idx + (size_t)t * KSEL;
     const uint U = KSEL * nsb;
     // the first pass's weights are on their way while the activations are quantized
     uint u = min(G, U - 1u), j = u / nsb, sb = u - j * nsb;
-    const uchar* w = wd + (((size_t)min(ti[j], E - 1u) * N + row0) * nsb + sb) * W::BYTES;
+    const uchar* w = wd + expert_base(sel, t * KSEL + j, SLOTS, E, (size_t)N * rb) + ((size_t)row0 * nsb + sb) * W::BYTES;
     W w0, w1;
     w0.load(w, l);
     w1.load(w + r1, l);
-    if (threadIdx.x < KSEL) s_idx[threadIdx.x] = min(ti[threadIdx.x], E - 1u);
+    if (threadIdx.x < KSEL) s_base[threadIdx.x] = expert_base(sel, t * KSEL + threadIdx.x, SLOTS, E, (size_t)N * rb);
     block_quant_q8k(act + (size_t)t * KSEL * K, KSEL * K, aq, as_);
     __syncthreads();
     for (uint u0 = 0; u0 < U; u0 += 8u) {
         const bool on = u0 + G < U;
         const uint un = min(u0 + 8u + G, U - 1u), jn = un / nsb, sbn = un - jn * nsb;
-        const uchar* wn = wd + (((size_t)s_idx[jn] * N + row0) * nsb + sbn) * W::BYTES;
+        const uchar* wn = wd + s_base[jn] + ((size_t)row0 * nsb + sbn) * W::BYTES;
         W n0, n1;
         n0.load(wn, l);
         n1.load(wn + r1, l);
@@ -418,12 +443,17 @@ __device__ __forceinline__ void moe_down_dec_body(const float* __restrict__ act,
 extern "C" __global__ void __launch_bounds__(256)
 moe_down_q4k_dec(const float* act, const uchar* wd, const uint* idx, const float* wgt, float* y, uint K, uint N,
                  uint KSEL, uint E, uint ACC) {
-    moe_down_dec_body<W4k>(act, wd, idx, wgt, y, K, N, KSEL, E, ACC);
+    moe_down_dec_body<W4k, false>(act, wd, idx, wgt, y, K, N, KSEL, E, ACC);
+}
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q4k_slots(const float* act, const uchar* arena, const unsigned long* off_d, const float* wgt, float* y, uint K,
+                   uint N, uint KSEL, uint LIM, uint ACC) {
+    moe_down_dec_body<W4k, true>(act, arena, off_d, wgt, y, K, N, KSEL, LIM, ACC);
 }
 extern "C" __global__ void __launch_bounds__(256)
 moe_down_q5k_dec(const float* act, const uchar* wd, const uint* idx, const float* wgt, float* y, uint K, uint N,
                  uint KSEL, uint E, uint ACC) {
-    moe_down_dec_body<W5k>(act, wd, idx, wgt, y, K, N, KSEL, E, ACC);
+    moe_down_dec_body<W5k, false>(act, wd, idx, wgt, y, K, N, KSEL, E, ACC);
 }
 
 // ------------------------------------------------------------------ grouped products on the matrix cores

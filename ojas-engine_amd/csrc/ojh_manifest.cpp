@@ -493,6 +493,8 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
 //   6 moe_gu_q4k_mm, 7 moe_down_q4k_mm: the arguments of 3 and 4, grid [ceil(N/16), E, 1]
 //   8 moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)                      grid [ceil(N/8), NA, 1]
 //   9 moe_down_q4k_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)                  grid [ceil(N/8), T, 1]
+//  10 moe_gu_q4k_slots, 11 moe_down_q4k_slots: 8 and 9 with a u64 byte offset per assignment into an arena
+//     and LIM * 256 = the last offset at which an expert still fits, in place of idx and E
 static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                      const uint32_t block[3], size_t need[16], size_t align[16]) {
     int rc;
@@ -580,6 +582,38 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         align[0] = align[1] = 16;
         return OJH_OK;
     }
+    case 10: {  // moe_gu_q4k_slots(x, arena_g, arena_u, act, off_g, off_u, K, N, KSEL, NA, LIM_G, LIM_U)
+        uint32_t K = c[0], N = c[1], KS = c[2], NA = c[3];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!K || K % 256 || K > 8192 || !N || !KS || !NA || NA % KS) return ojh_fail(OJH_ERR_ARG, "%s: K=%u (<= 8192) N=%u KSEL=%u NA=%u", s->name, K, N, KS, NA);
+        if (grid[0] != (N + 7) / 8 || grid[1] != NA || grid[2] != 1)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/8), NA, 1]", s->name);
+        const size_t eb = (size_t)N * (K / 256) * 144;
+        need[0] = (size_t)(NA / KS) * K * 4;
+        need[1] = (size_t)c[4] * 256 + eb;
+        need[2] = (size_t)c[5] * 256 + eb;
+        need[3] = (size_t)NA * N * 4;
+        need[4] = need[5] = (size_t)NA * 8;
+        align[0] = align[1] = align[2] = 16;
+        align[4] = align[5] = 8;
+        return OJH_OK;
+    }
+    case 11: {  // moe_down_q4k_slots(act, arena, off_d, wgt, y, K, N, KSEL, LIM, ACC)
+        uint32_t K = c[0], N = c[1], KS = c[2], T = grid[1];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!K || K % 256 || K > 2048 || !N || !KS || KS > 64 || (uint64_t)KS * K > 32768)
+            return ojh_fail(OJH_ERR_ARG, "%s: K=%u (<= 2048) N=%u KSEL=%u (<= 64, KSEL * K <= 32768)", s->name, K, N, KS);
+        if (grid[0] != (N + 7) / 8 || !T || grid[2] != 1)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/8), tokens, 1]", s->name);
+        need[0] = (size_t)T * KS * K * 4;
+        need[1] = (size_t)c[3] * 256 + (size_t)N * (K / 256) * 144;
+        need[2] = (size_t)T * KS * 8;
+        need[3] = (size_t)T * KS * 4;
+        need[4] = (size_t)T * N * 4;
+        align[0] = align[1] = 16;
+        align[2] = 8;
+        return OJH_OK;
+    }
     default: {
         uint32_t T = c[0], KS = c[1], D = c[2];
         if ((rc = check_block(block, 256))) return rc;
@@ -608,8 +642,8 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, u
     case 3: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = experts
     case 4: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
     case 6: case 7: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;
-    case 8: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = assignments
-    case 9: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = tokens
+    case 8: case 10: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = assignments
+    case 9: case 11: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = tokens
     default: grid[0] = (uint32_t)(((uint64_t)M * N + 255) / 256); break;  // N = D, M = tokens
     }
     return OJH_OK;
@@ -806,6 +840,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("moe_down_q4k_mm", "moe", 6, 3, OJH_Q4_K, 7, check_moe, shape_moe);
     add("moe_gu_q4k_dec", "moe", 5, 5, OJH_Q4_K, 8, check_moe, shape_moe);
     add("moe_down_q4k_dec", "moe", 5, 5, OJH_Q4_K, 9, check_moe, shape_moe);
+    add("moe_gu_q4k_slots", "moe", 6, 6, OJH_Q4_K, 10, check_moe, shape_moe);
+    add("moe_down_q4k_slots", "moe", 5, 5, OJH_Q4_K, 11, check_moe, shape_moe);
     add("moe_down_q5k_m", "moe", 6, 3, OJH_Q5_K, 4, check_moe, shape_moe);
     add("moe_down_q5k_dec", "moe", 5, 5, OJH_Q5_K, 9, check_moe, shape_moe);
     add("copy_bf16_half", "glue", 2, 1, (2u << 8) | 2u, 0, check_elementwise, shape_elementwise);

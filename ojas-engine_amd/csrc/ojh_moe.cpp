@@ -131,3 +131,40 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     }
     return OJH_OK;
 }
+
+// The decode form over streamed experts: every assignment's gate, up and down matrices sit at a
+// byte offset of their arena (the reference's expert cache hands out slots,
+// crates/ojas-cuda/src/expert_cache.rs; kernels crates/ojas-cuda/src/kernels/moe.rs:133-174).
+extern "C" int ojh_moe_ffn_slots(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32_t d, uint32_t n_ff, uint32_t ksel,
+                                 const ojh_buf *arena_gate, const ojh_buf *off_gate, const ojh_buf *arena_up,
+                                 const ojh_buf *off_up, const ojh_buf *arena_down, const ojh_buf *off_down,
+                                 const ojh_buf *wgt, ojh_buf *y, int accum) {
+    if (!dev || !arena_gate || !arena_up || !arena_down) return ojh_fail(OJH_ERR_ARG, "ojh_moe_ffn_slots: NULL argument");
+    if (!T || !ksel || ksel > 64 || T > 65535u / ksel)
+        return ojh_fail(OJH_ERR_ARG, "moe_ffn_slots: tokens=%u ksel=%u out of range (ksel <= 64, tokens * ksel <= 65535)", T, ksel);
+    if (!d || !n_ff || d % 256 || n_ff % 256 || d > 8192 || n_ff > 2048 || (uint64_t)ksel * n_ff > 32768)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn_slots: d=%u (multiple of 256, <= 8192), n_ff=%u (<= 2048), ksel * n_ff <= 32768", d, n_ff);
+    const uint32_t NA = T * ksel;
+    const size_t gu_bytes = (size_t)n_ff * (d / 256) * 144, dn_bytes = (size_t)d * (n_ff / 256) * 144;
+    int rc;
+    if ((rc = span("moe_ffn_slots: x", x, (size_t)T * d * 4, 16))) return rc;
+    if ((rc = span("moe_ffn_slots: gate arena", arena_gate, gu_bytes, 16))) return rc;
+    if ((rc = span("moe_ffn_slots: up arena", arena_up, gu_bytes, 16))) return rc;
+    if ((rc = span("moe_ffn_slots: down arena", arena_down, dn_bytes, 16))) return rc;
+    if ((rc = span("moe_ffn_slots: gate offsets", off_gate, (size_t)NA * 8, 8))) return rc;
+    if ((rc = span("moe_ffn_slots: up offsets", off_up, (size_t)NA * 8, 8))) return rc;
+    if ((rc = span("moe_ffn_slots: down offsets", off_down, (size_t)NA * 8, 8))) return rc;
+    if ((rc = span("moe_ffn_slots: wgt", wgt, (size_t)NA * 4, 4))) return rc;
+    if ((rc = span("moe_ffn_slots: y", y, (size_t)T * d * 4, 4))) return rc;
+    if ((rc = ensure(dev, "moe"))) return rc;
+    // the last 256-byte step at which a whole expert still fits: offsets beyond it are clamped
+    auto lim = [](const ojh_buf *a, size_t e) { return (uint32_t)std::min<size_t>((a->bytes - e) / 256, 0xFFFFFFFFu); };
+    ojh_buf *act;
+    if ((rc = ojh_scratch_get(dev, "moe_act", (size_t)NA * n_ff * 4, &act))) return rc;
+    uint32_t b256[3] = {256, 1, 1}, g1[3] = {(n_ff + 7) / 8, NA, 1}, g2[3] = {(d + 7) / 8, T, 1};
+    if ((rc = ojh_launch(dev, "moe_gu_q4k_slots", {x->ptr, arena_gate->ptr, arena_up->ptr, act->ptr, off_gate->ptr, off_up->ptr},
+                         {d, n_ff, ksel, NA, lim(arena_gate, gu_bytes), lim(arena_up, gu_bytes)}, g1, b256)))
+        return rc;
+    return ojh_launch(dev, "moe_down_q4k_slots", {act->ptr, arena_down->ptr, off_down->ptr, wgt->ptr, y->ptr},
+                      {n_ff, d, ksel, lim(arena_down, dn_bytes), (uint32_t)(accum != 0)}, g2, b256);
+}

@@ -128,6 +128,7 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_quant_q8k": (i32, [vp, vp, sz, i32, u32, u32, vp, vp]),
         "ojh_moe_route": (i32, [vp, vp, u32, u32, u32, vp, vp]),
         "ojh_moe_ffn": (i32, [vp, vp, u32, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp, i32, i32]),
+        "ojh_moe_ffn_slots": (i32, [vp, vp, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp, vp, vp, i32]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -496,6 +497,14 @@ class HipGpu:
 
     def moe_route(self, logits: Buf, n_tokens: int, n_expert: int, ksel: int, idx: Buf, wgt: Buf) -> None:
         self._check(self._L.ojh_moe_route(self._dev, logits.handle, n_tokens, n_expert, ksel, idx.handle, wgt.handle))
+
+    def moe_ffn_slots(self, x: Buf, n_tokens: int, d: int, n_ff: int, ksel: int, arena_gate: Buf, off_gate: Buf,
+                      arena_up: Buf, off_up: Buf, arena_down: Buf, off_down: Buf, wgt: Buf, y: Buf,
+                      accum: bool = False) -> None:
+        """Expert FFN over streamed experts: u64 byte offsets per (token, slot) into three arenas."""
+        self._check(self._L.ojh_moe_ffn_slots(self._dev, x.handle, n_tokens, d, n_ff, ksel, arena_gate.handle,
+                                              off_gate.handle, arena_up.handle, off_up.handle, arena_down.handle,
+                                              off_down.handle, wgt.handle, y.handle, int(accum)))
 
     def moe_ffn(self, x: Buf, n_tokens: int, d: int, n_ff: int, n_expert: int, ksel: int, idx: Buf, wgt: Buf,
                 gate: Lin, up: Lin, down: Lin, y: Buf, accum: bool = False, act_mode: int = ACT_AUTO) -> None:

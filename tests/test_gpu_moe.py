@@ -167,6 +167,60 @@ def test_expert_ffn_with_q5k_down_tensors(gpu, orc, pkg, T, E, ksel, d, nff):
     assert peak_err(got[:T * d].reshape(T, d), want) <= TOL
 
 
+@pytest.mark.parametrize("T,E,ksel,d,nff,accum", [(1, 128, 8, 2048, 768, False), (3, 16, 5, 2304, 512, True),
+                                                   (9, 6, 2, 256, 256, False)])
+def test_streamed_experts_by_slot_offsets(gpu, pkg, T, E, ksel, d, nff, accum):
+    """Experts scattered over an arena in cache-slot order, addressed by one byte offset per
+    assignment (crates/ojas-cuda/src/kernels/moe.rs:133-174): the same bits as the resident,
+    index-addressed decode form on the same experts; an offset past the arena is clamped, not read."""
+    gate, up, down = _experts(pkg, E, d, nff, ("slots", E, d, nff))
+    x = pkg.synth.normal_f32(T * d, "moe", "sx", T, d).reshape(T, d)
+    lg = pkg.synth.normal_f32(T * E, "moe", "slg", T, E).reshape(T, E)
+    gi, gw, idx_d, wgt_d = _route(gpu, lg, ksel)
+    y0 = pkg.synth.normal_f32(T * d, "moe", "sy0").reshape(T, d)
+    monkey = pytest.MonkeyPatch()
+    monkey.setenv("OJAS_HIP_MOE", "3")
+    g = pkg.HipGpu(0)
+    try:
+        lg_, lu_, ld_ = g.lin(Q4_K, E * nff, d, gate), g.lin(Q4_K, E * nff, d, up), g.lin(Q4_K, E * d, nff, down)
+        yr = g.upload(y0)
+        g.moe_ffn(g.upload(x), T, d, nff, E, ksel, g.upload_bytes(gi), g.upload(gw), lg_, lu_, ld_, yr, accum=accum)
+        want = g.read(yr, T * d)
+    finally:
+        g.close()
+        monkey.undo()
+    # an arena per tensor: the experts in a shuffled slot order, 4 KiB of padding in front
+    eb_gu, eb_d = nff * (d // 256) * 144, d * (nff // 256) * 144
+    perm = pkg.synth.rng("slots", E).permutation(E)
+    slot_of = np.empty(E, np.int64)
+    slot_of[perm] = np.arange(E)
+    pad = 4096
+
+    def arena(raw, eb):
+        a = np.zeros(pad + E * eb, np.uint8)
+        for s_, e in enumerate(perm):
+            a[pad + s_ * eb:pad + (s_ + 1) * eb] = raw[e * eb:(e + 1) * eb]
+        return a
+    ag, au, ad = gpu.upload_bytes(arena(gate, eb_gu)), gpu.upload_bytes(arena(up, eb_gu)), gpu.upload_bytes(arena(down, eb_d))
+    sel = np.asarray(gi, np.int64).reshape(-1)
+    og = (pad + slot_of[sel] * eb_gu).astype(np.uint64)
+    od = (pad + slot_of[sel] * eb_d).astype(np.uint64)
+    yd = gpu.upload(np.concatenate([y0.ravel(), np.full(d, 12345.5, np.float32)]))
+    gpu.moe_ffn_slots(gpu.upload(x), T, d, nff, ksel, ag, gpu.upload_bytes(og), au, gpu.upload_bytes(og), ad,
+                      gpu.upload_bytes(od), wgt_d, yd, accum=accum)
+    got = gpu.read(yd, T * d + d)
+    assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
+    assert np.array_equal(got[:T * d], want)
+    # offsets far outside the arenas: clamped to the last slot, the launch completes
+    bad = np.full(T * ksel, 1 << 40, np.uint64)
+    gpu.moe_ffn_slots(gpu.upload(x), T, d, nff, ksel, ag, gpu.upload_bytes(bad), au, gpu.upload_bytes(bad), ad,
+                      gpu.upload_bytes(bad), wgt_d, yd)
+    assert np.all(np.isfinite(gpu.read(yd, T * d)))
+    with pytest.raises(pkg.OjasHipError, match="needs"):
+        gpu.moe_ffn_slots(gpu.upload(x), T, d, nff, ksel, ag, gpu.upload_bytes(og[:-1]), au, gpu.upload_bytes(og), ad,
+                          gpu.upload_bytes(od), wgt_d, yd)
+
+
 def test_expert_ffn_rejects_what_it_cannot_run(gpu, pkg):
     E, d, nff = 4, 256, 256
     gate, up, down = _experts(pkg, E, d, nff, "err")
