@@ -33,6 +33,7 @@ FAMILIES = {
     "glue": ("glue.hip", []),
     "gemm": ("gemm.hip", ["-ffp-contract=off"]),
     "gemm_xl": ("gemm_xl.hip", ["-ffp-contract=off"]),
+    "gemm_q8k": ("gemm_q8k.hip", []),
     "moe": ("moe.hip", []),
     "rowq8": ("rowq8.hip", ["-ffp-contract=off"]),
 }

@@ -1,0 +1,216 @@
+// Family "gemm_q8k": Q4_K rows against a batch of tokens on the int8 matrix cores, in the CPU
+// reference's arithmetic — activations quantized per 256 by quant_q8k, integer dots per 32-weight
+// sub-block, the scale algebra of dot_q4k (crates/ojas-cpu/src/cpu_math.rs:539-635):
+//     y[t][n] (=, +=) sum_sb sx[t][sb] * ( d * sum_j sc_j * idot_j  -  dmin * sum_j m_j * bsum_j ).
+// This is what serves speculative verify (2-16 tokens on every projection) and prefill chunks
+// with results within the parity bar of the CPU path, which an f16 tile cannot give.
+//
+//   gemm_q8k_q4k_mf(xq, xs, w, y, K, N, M, ACC, RW)      block 256, grid [x <= ceil(N / (16 RW)), ceil(M / 64), 1]
+//
+// v_mfma_i32_16x16x32_i8 multiplies 16 tokens x 16 rows over one sub-block:
+//   A: lane (m, kg) = (lane % 16, lane / 16) holds int8 positions 8 kg .. 8 kg + 7 of token m;
+//   B: lane (n, kg) the 4-bit codes of the same positions of row n, as bytes;
+//   D: register v of lane (n, kg) = idot of token 4 kg + v with row n.
+// The row is lane-constant in D, so a sub-block's 6-bit scale enters with one v_mad_i32_i24 per D
+// register (the sum over the eight sub-blocks is exact in int32).  The min term
+// sum_j m_j * bsum_j is itself a small product over j: the workgroup splits every bsum (|.| <= 4064)
+// into 64 hi + lo with both parts in int8 while it stages the tokens, and two more MFMAs per
+// super-block (the row's eight mins as B in the first eight positions) give sum_j m_j lo_j and
+// sum_j m_j hi_j for all 16 x 16 outputs at once.  A super-block ends with two converts and
+// three FMAs per output.
+//
+// A workgroup owns 16 RW rows (RW = 1, 2 or 4 row tiles) and up to 64 tokens (P = 1, 2 or 4 passes of
+// 16; eight passes do not fit the register file); its four waves are RW row tiles x KW = 4 / RW slices of the super-blocks.  Tokens wait in
+// LDS, chunk by chunk of K (as many super-blocks as fit 76 KB for the workgroup's tokens: 256 bytes,
+// a scale and 16 bytes of split sums per token and super-block), rows 32 bytes longer than the
+// chunk so that an 8-byte read of 64 lanes spreads over all banks.
+// K-slices meet in LDS in wave order.
+#include "ojk_common.h"
+
+typedef int gq_i4 __attribute__((ext_vector_type(4)));
+#define GQ_LDS 77824u
+
+__device__ __forceinline__ long gq_pack(uint lo, uint hi) { return (long)(((unsigned long)hi << 32) | lo); }
+
+struct GqW {            // lane (n, kg): its bytes of one super-block of row n
+    uint4 hdr;          // d, dmin, the 12 scale bytes
+    uint2 q[4];         // codes of positions 8 kg .. 8 kg + 7 of each 64-weight chunk (low | high nibbles)
+};
+__device__ __forceinline__ GqW gq_load(const uchar* blk, uint kg) {
+    GqW r;
+    r.hdr = *(const uint4*)blk;
+#pragma unroll
+    for (int c = 0; c < 4; c++) r.q[c] = *(const uint2*)(blk + 16u + 32u * c + 8u * kg);
+    return r;
+}
+
+template <int P>
+__device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                     const uchar* __restrict__ w, float* __restrict__ y,
+                                                     uint K, uint N, uint M, uint ACC, uint RW, uchar* lds) {
+    const uint tid = threadIdx.x, lane = tid & 63u;
+    const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint nsb = K >> 8, KW = 4u / RW, rt = wave / KW, kw = wave % KW;
+    const uint BM = 16u * P, t0 = blockIdx.y * 64u;
+    // LDS: [reduction buffer: 4 waves x P x 4 x 64 floats] [tokens] [token scales] [split bsums].
+    // Chunk of K staged at a time: BM * (KC + 32) + (KC / 256) * BM * 20 bytes, a whole multiple of
+    // KW super-blocks so that a wave's slice continues from chunk to chunk (the host picks RW so
+    // that at least KW fit).  When the whole K fits, the tokens are staged once and the workgroup
+    // walks row tiles blockIdx.x, blockIdx.x + gridDim.x, ...
+    float* red = (float*)lds;
+    uchar* tok = lds + 4096u * P;
+    const uint fit = ((GQ_LDS - 4096u * P) / BM - 32u) / 276u;
+    const bool whole = nsb <= fit;
+    const uint csb = whole ? nsb : fit / KW * KW;                // super-blocks per chunk
+    const uint S = csb * 256u + 32u;
+    float* lsx = (float*)(tok + (size_t)BM * S);                 // [csb][BM] token scales
+    uchar* lbq = (uchar*)(lsx + csb * BM);                       // [csb][BM][16]: lo_0..7, hi_0..7 of the bsums
+    const uint n = lane & 15u, kg = lane >> 4;
+    const uchar* xa = tok + (size_t)n * S + 8u * kg;
+    const gq_i4 zero = {0, 0, 0, 0};
+    const uint ntiles = (N + 16u * RW - 1u) / (16u * RW);
+    for (uint tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const uint row = min((tile * RW + rt) * 16u + n, N - 1u);
+        const uchar* wr = w + (size_t)row * nsb * Q4K_BYTES;
+        float acc[P][4];
+#pragma unroll
+        for (int p = 0; p < P; p++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[p][v] = 0.0f;
+        GqW cur = gq_load(wr + (size_t)min(kw, nsb - 1u) * Q4K_BYTES, kg);
+        for (uint sb0 = 0; sb0 < nsb; sb0 += csb) {
+            const uint cn = min(csb, nsb - sb0);                 // super-blocks in this chunk
+            if (!whole || tile == blockIdx.x) {
+                if (sb0 || tile != blockIdx.x) __syncthreads();  // everyone is done with the previous chunk
+                // stage tokens t0 .. t0 + BM - 1 (zeros past M): a thread keeps one 16-byte column of the
+                // chunk and walks the tokens eight loads at a time (one wait per eight, not per load)
+                const uint per_row = cn * 16u, lpr = min(per_row, 256u), rpp = 256u / lpr;
+                const uint c0 = tid % lpr, ts = tid / lpr;
+                if (ts < rpp) {
+                    for (uint c = c0; c < per_row; c += lpr) {
+                        const signed char* src = xq + (size_t)t0 * K + (size_t)sb0 * 256u + (size_t)c * 16u;
+                        for (uint tb = ts; tb < BM; tb += 8u * rpp) {
+                            uint4 v[8];
+#pragma unroll
+                            for (int u = 0; u < 8; u++) {
+                                const uint t = tb + (uint)u * rpp;
+                                v[u] = make_uint4(0u, 0u, 0u, 0u);
+                                if (t < BM && t0 + t < M) v[u] = *(const uint4*)(src + (size_t)t * K);
+                            }
+#pragma unroll
+                            for (int u = 0; u < 8; u++) {
+                                const uint t = tb + (uint)u * rpp;
+                                if (t < BM) *(uint4*)(tok + (size_t)t * S + (size_t)c * 16u) = v[u];
+                            }
+                        }
+                    }
+                }
+                for (uint i = tid; i < cn * BM; i += 256u) {
+                    const uint s = i / BM, t = i - s * BM;
+                    lsx[i] = t0 + t < M ? xs[(size_t)(t0 + t) * nsb + sb0 + s] : 0.0f;
+                }
+                __syncthreads();
+                // bsum of every (token, sub-block) of the chunk, split into int8 parts: 64 * hi + lo
+                for (uint i = tid; i < cn * BM * 8u; i += 256u) {
+                    const uint jj = i & 7u, t = (i >> 3) % BM, s = i / (8u * BM);
+                    const uint4* px = (const uint4*)(tok + (size_t)t * S + s * 256u + jj * 32u);
+                    const uint4 a = px[0], b = px[1];
+                    int bs = dot4_i8(a.x, 0x01010101u, 0);
+                    bs = dot4_i8(a.y, 0x01010101u, bs); bs = dot4_i8(a.z, 0x01010101u, bs); bs = dot4_i8(a.w, 0x01010101u, bs);
+                    bs = dot4_i8(b.x, 0x01010101u, bs); bs = dot4_i8(b.y, 0x01010101u, bs);
+                    bs = dot4_i8(b.z, 0x01010101u, bs); bs = dot4_i8(b.w, 0x01010101u, bs);
+                    uchar* o = lbq + ((size_t)s * BM + t) * 16u;
+                    o[jj] = (uchar)(bs & 63);
+                    o[8u + jj] = (uchar)(bs >> 6);
+                }
+                __syncthreads();
+            }
+            for (uint s = kw; s < cn; s += KW) {
+                // the next super-block of this wave's slice (in this chunk or the next) is on its way
+                const uint nxt = s + KW < cn ? sb0 + s + KW : sb0 + csb + kw;
+                const GqW nx = gq_load(wr + (size_t)min(nxt, nsb - 1u) * Q4K_BYTES, kg);
+                const float d = f16_bits_to_f32(cur.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
+                int sc[8];
+                long B[8], Bm = 0;
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    uint a, b;
+                    q4k_scale_min_pair(cur.hdr.y, cur.hdr.z, cur.hdr.w, (uint)c, a, b);
+                    sc[2 * c] = (int)(a & 0xFFu); sc[2 * c + 1] = (int)(a >> 8);
+                    Bm |= (long)(unsigned long)(b & 0xFFFFu) << (16 * c);    // mins 2c, 2c + 1 -> bytes 2c, 2c + 1
+                    B[2 * c] = gq_pack(cur.q[c].x & 0x0F0F0F0Fu, cur.q[c].y & 0x0F0F0F0Fu);
+                    B[2 * c + 1] = gq_pack((cur.q[c].x >> 4) & 0x0F0F0F0Fu, (cur.q[c].y >> 4) & 0x0F0F0F0Fu);
+                }
+                if (kg != 0u) Bm = 0;                                        // only positions 0..7 carry mins
+#pragma unroll
+                for (int p = 0; p < P; p++) {
+                    int isum[4] = {0, 0, 0, 0};
+                    const uchar* xp = xa + (size_t)(16 * p) * S + s * 256u;
+#pragma unroll
+                    for (int jj = 0; jj < 8; jj++) {
+                        const long A = *(const long*)(xp + 32 * jj);
+                        const gq_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B[jj], zero, 0, 0, 0);
+#pragma unroll
+                        for (int v = 0; v < 4; v++) isum[v] += __mul24(sc[jj], D[v]);
+                    }
+                    // token n of this pass: its eight lo parts, then its eight hi parts (lanes kg = 0 only)
+                    const uchar* pq = lbq + ((size_t)s * BM + 16u * p + n) * 16u;
+                    long Alo = 0, Ahi = 0;
+                    if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
+                    const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
+                    const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
+                    const float4 sx = *(const float4*)(lsx + s * BM + 16u * p + 4u * kg);
+                    acc[p][0] += sx.x * (d * (float)isum[0] - dmin * (float)(64 * Dhi[0] + Dlo[0]));
+                    acc[p][1] += sx.y * (d * (float)isum[1] - dmin * (float)(64 * Dhi[1] + Dlo[1]));
+                    acc[p][2] += sx.z * (d * (float)isum[2] - dmin * (float)(64 * Dhi[2] + Dlo[2]));
+                    acc[p][3] += sx.w * (d * (float)isum[3] - dmin * (float)(64 * Dhi[3] + Dlo[3]));
+                }
+                cur = nx;
+            }
+        }
+        // K-slices of a row tile meet in LDS, added in slice order
+        if (KW > 1u) {
+#pragma unroll
+            for (int p = 0; p < P; p++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) red[((wave * P + p) * 4 + v) * 64u + lane] = acc[p][v];
+            __syncthreads();
+            if (kw == 0u) {
+#pragma unroll
+                for (int p = 0; p < P; p++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        float t = acc[p][v];
+                        for (uint k2 = 1; k2 < KW; k2++) t += red[(((wave + k2) * P + p) * 4 + v) * 64u + lane];
+                        acc[p][v] = t;
+                    }
+            }
+            __syncthreads();                                     // before the next tile writes `red`
+        }
+        if (kw == 0u) {
+            const uint r_out = (tile * RW + rt) * 16u + n;
+#pragma unroll
+            for (int p = 0; p < P; p++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const uint t = t0 + 16u * p + 4u * kg + v;
+                    if (t < M && r_out < N) {
+                        float* o = y + (size_t)t * N + r_out;
+                        *o = ACC ? *o + acc[p][v] : acc[p][v];
+                    }
+                }
+        }
+    }
+}
+
+// (at least two waves per SIMD: with a register budget of 256 the matrix-core results are written
+// to ordinary registers instead of the accumulation file, which saves a move per result)
+extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8)))
+gemm_q8k_q4k_mf(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC,
+                uint RW) {
+    __shared__ __attribute__((aligned(16))) uchar lds_gq[GQ_LDS];
+    const uint left = M - min(M, blockIdx.y * 64u);              // tokens of this workgroup's tile
+    if (left <= 16u) gemm_q8k_q4k_mf_body<1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
+    else if (left <= 32u) gemm_q8k_q4k_mf_body<2>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
+    else gemm_q8k_q4k_mf_body<4>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
+}

@@ -64,6 +64,7 @@ struct ojh_device {
     uint32_t q6k_mf_min_m = 4;   // OJAS_HIP_Q6K_MF_MIN_M: tokens from which Q6_K rows go to the int8 matrix cores
     uint32_t px_bpc = 0;         // OJAS_HIP_PX_BPC: workgroups per CU for the grid-stride head matvec (0: 8)
     int px = 1;                  // OJAS_HIP_PX: 0 = never take it
+    uint32_t q4k_mf_min_m = 5;   // OJAS_HIP_Q4K_MF_MIN_M: tokens from which Q4_K rows go to the int8 matrix cores
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
                                  // 3 = per-assignment decode form always
     uint32_t moe_dec_tokens = 8; // OJAS_HIP_MOE_DEC_TOKENS: the decode form serves up to this many tokens
@@ -115,4 +116,5 @@ const ojh_kernel_spec *ojh_find_kernel(const char *name);
 int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out);
 int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptrs,
                const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);
+uint32_t ojh_gemm_q8k_rw(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M);   // row tiles per workgroup of gemm_q8k_q4k_mf
 uint32_t ojh_q80_lds_kc(uint32_t K);   // chunks of K for gemv_nat_q80_lds, 0 if none (ojh_manifest.cpp)

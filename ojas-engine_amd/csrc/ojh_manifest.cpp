@@ -118,6 +118,64 @@ static int shape_q80_lds(const ojh_kernel_spec *, const ojh_device *dev, uint32_
     return OJH_OK;
 }
 
+// gemm_q8k_q4k_mf(xq, xs, w, y, K, N, M, ACC, RW): 16 RW rows x up to 64 tokens per workgroup.
+// The tokens of a workgroup wait in 76 KB of LDS chunk by chunk of K; a chunk must hold at least
+// 4 / RW super-blocks (the waves that split K).
+uint32_t ojh_gemm_q8k_fit(uint32_t M) {   // super-blocks of K that fit for the largest token tile of M tokens
+    uint32_t left = M > 64 ? 64 : M, bm = left <= 16 ? 16 : left <= 32 ? 32 : 64;
+    return ((77824 - 256 * bm) / bm - 32) / 276;   // 4 KB of reduction buffer per 16 tokens come first
+}
+static int check_gemm_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                          const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], N = c[1], M = c[2], RW = c[4];
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if ((rc = check_block(block, 256))) return rc;
+    if (!M || M > 65535) return ojh_fail(OJH_ERR_ARG, "%s: M=%u out of range", s->name, M);
+    if (RW != 1 && RW != 2 && RW != 4) return ojh_fail(OJH_ERR_ARG, "%s: RW=%u must be 1, 2 or 4", s->name, RW);
+    if (K / 256 > ojh_gemm_q8k_fit(M) && ojh_gemm_q8k_fit(M) < 4 / RW)
+        return ojh_fail(OJH_ERR_ARG, "%s: RW=%u leaves %u waves on K but only %u super-blocks of %u tokens fit in LDS", s->name,
+                        RW, 4 / RW, ojh_gemm_q8k_fit(M), M > 64 ? 64 : M);
+    if (!grid[0] || grid[0] > (N + 16 * RW - 1) / (16 * RW) || grid[1] != (M + 63) / 64 || grid[2] != 1)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N / (16 RW)), ceil(M / 64), 1]", s->name);
+    need[0] = (size_t)M * K;
+    need[1] = (size_t)M * (K / 256) * 4;
+    need[2] = (size_t)N * (K / 256) * 144;
+    need[3] = (size_t)M * N * 4;
+    align[1] = 4;
+    align[3] = 4;
+    return OJH_OK;
+}
+// row tiles per workgroup: as many as still give every CU a workgroup and a half (more rows per workgroup
+// spread the staging of the tokens over more work; measured on 14336 x 4096 and 4096 x 4096), at least
+// what the LDS chunk asks for
+uint32_t ojh_gemm_q8k_rw(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M) {
+    const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, fit = ojh_gemm_q8k_fit(M);
+    const uint32_t rw_min = K / 256 <= fit || fit >= 4 ? 1 : fit >= 2 ? 2 : 4;
+    const uint64_t tiles_m = (M + 63) / 64;
+    uint32_t rw = 4;
+    while (rw > rw_min && (uint64_t)((N + 16 * rw - 1) / (16 * rw)) * tiles_m * 2 < 3ull * cus) rw /= 2;
+    return rw;
+}
+static int shape_gemm_q8k(const ojh_kernel_spec *, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
+                          uint32_t grid[3], uint32_t block[3]) {
+    if (!M) M = 1;
+    const uint32_t rw = ojh_gemm_q8k_rw(dev, K, N, M);
+    grid[0] = (N + 16 * rw - 1) / (16 * rw);
+    grid[1] = (M + 63) / 64;
+    // the whole K staged once: row tiles grid-stride over two workgroups per CU
+    const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
+    if (K / 256 <= ojh_gemm_q8k_fit(M) && grid[0] * grid[1] > 2 * cus) {
+        uint32_t gx = 2 * cus / grid[1];
+        grid[0] = gx ? gx : 1;
+    }
+    grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // gemv_q8k_q6k_px(xq, xs, w, y, K, N): rows grid-stride, activations in registers (K <= 8192)
 static int check_gemv_q8k_px(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                              const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -808,6 +866,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
             add(fq + "_wide", "gemv_q8k", 3, 3, f.type, 2, check_gemv_fq8k, shape_rows);
         }
     }
+    add("gemm_q8k_q4k_mf", "gemm_q8k", 4, 5, OJH_Q4_K, 1, check_gemm_q8k, shape_gemm_q8k);
     add("relayout_q4k_q4l", "dequant", 4, 1, OJH_Q4_K, 0, check_relayout, shape_relayout);
     add("rows_q8_from_f16", "rowq8", 3, 2, 0, 0, check_rowq8, shape_rowq8);
     add("quant_rows_i8", "rowq8", 3, 2, 0, 1, check_rowq8, shape_rowq8);

@@ -171,6 +171,15 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
         return ojh_launch(dev, name.c_str(), p, {K, N}, grid, block);
     }
     // a handful of tokens on Q6_K rows: the int8 matrix cores, 8 tokens per pass
+    // Q4_K rows against several tokens: the int8 matrix cores
+    if (w->type == OJH_Q4_K && m >= dev->q4k_mf_min_m) {
+        int rc = ensure(dev, "gemm_q8k");
+        if (rc) return rc;
+        uint32_t sg[3], sb[3];
+        if ((rc = ojh_launch_shape(dev, "gemm_q8k_q4k_mf", K, N, m, sg, sb))) return rc;
+        return ojh_launch(dev, "gemm_q8k_q4k_mf", {xq, xs, wp, yp},
+                          {K, N, m, (uint32_t)(accum != 0), ojh_gemm_q8k_rw(dev, K, N, m)}, sg, sb);
+    }
     const size_t w_bytes = w->row_bytes * N;
     const bool dwords_ok = (uintptr_t)wp % 4 == 0 && (w_bytes % 4 == 0 || w->off + w_bytes + 2 <= w->raw->bytes);
     if (w->type == OJH_Q6_K && m >= dev->q6k_mf_min_m && m <= 16 && dwords_ok) {

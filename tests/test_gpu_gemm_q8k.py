@@ -1,0 +1,85 @@
+"""Q4_K rows against batches of tokens on the int8 matrix cores (`gemm_q8k_q4k_mf`): the CPU
+reference's arithmetic at verify and prefill sizes — every token against matvec_kq
+(crates/ojas-cpu/src/cpu_math.rs:1145-1189), the same bar as the one-token kernels."""
+import numpy as np
+import pytest
+
+from conftest import peak_err
+
+pytestmark = pytest.mark.gpu
+Q4_K = 12
+TOL_SEEN = 2e-5
+
+
+def _case(pkg, m, n, k, tag):
+    w = pkg.synth.q4k_weights(n, k, "gq", tag, n, k)
+    x = pkg.synth.normal_f32(m * k, "gq", tag, "x", m, k).reshape(m, k)
+    x[0, :256] = 0.0                      # an all-zero segment: scale 1
+    return w, x
+
+
+@pytest.mark.parametrize("m,n,k,accum", [(2, 50, 256, False), (16, 130, 4096, True), (17, 333, 2560, False),
+                                         (40, 64, 14336, True), (128, 100, 1024, False), (129, 300, 512, False),
+                                         (300, 40, 4096, True), (8, 4099, 4096, False), (64, 17, 8192, False)])
+def test_router_path_matches_the_cpu_reference(gpu, orc, pkg, m, n, k, accum):
+    w, x = _case(pkg, m, n, k, "a")
+    lin = gpu.lin(Q4_K, n, k, w)
+    y0 = pkg.synth.normal_f32(m * n, "gq", "y0", m, n).reshape(m, n) if accum else np.zeros((m, n), np.float32)
+    yd = gpu.upload(np.concatenate([y0.ravel(), np.full(n, 4242.5, np.float32)]))
+    gpu.mm(gpu.upload(x), lin, yd, m, accum, act_mode=pkg.ACT_Q8K)
+    got = gpu.read(yd, m * n + n)
+    assert np.all(got[m * n:] == 4242.5), "wrote past the last token"
+    want = np.stack([orc.matvec_kq(w, Q4_K, n, k, x[t]) for t in range(m)])
+    assert peak_err(got[:m * n].reshape(m, n) - y0, want) <= TOL_SEEN
+
+
+@pytest.mark.parametrize("m,n,k", [(5, 70, 4096), (33, 200, 2048), (100, 48, 14336), (128, 64, 512)])
+def test_every_row_tiling_and_the_integer_dot_kernel_agree(gpu, orc, pkg, m, n, k):
+    """By name: RW = 1, 2, 4 row tiles per workgroup (4, 2, 1 waves on K) where the tokens' chunk
+    allows it, and `gemv_q8k_q4k_m` on the same quantized activations.  Integer sums are exact in
+    all of them; the f32 sums over super-blocks associate differently."""
+    w, x = _case(pkg, m, n, k, "b")
+    gpu.ensure_family("gemm_q8k")
+    gpu.ensure_family("gemv_q8k")
+    nsb = k // 256
+    xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
+    gpu.quant_q8k(gpu.upload(x), m, k, xq, xs)
+    wd = gpu.upload_bytes(w)
+    want = np.stack([orc.matvec_kq(w, Q4_K, n, k, x[t]) for t in range(m)])
+    y = gpu.alloc(m * n)
+    gpu.dispatch(gpu.begin(), "gemv_q8k_q4k_m", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0],
+                 [(n + 3) // 4, 1, 1], [256, 1, 1])
+    dots = gpu.read(y, m * n).reshape(m, n)
+    ran = 0
+    for rw in (1, 2, 4):
+        grid = [(n + 16 * rw - 1) // (16 * rw), (m + 63) // 64, 1]
+        y = gpu.upload(np.full(m * n, 7.0, np.float32))
+        try:
+            gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0, rw], grid,
+                         [256, 1, 1])
+        except pkg.OjasHipError as e:
+            assert "super-blocks" in str(e)            # the chunk is too short for that many waves on K
+            continue
+        got = gpu.read(y, m * n).reshape(m, n)
+        assert peak_err(got, want) <= TOL_SEEN, rw
+        assert peak_err(got, dots) <= 2e-6, rw
+        ran += 1
+    assert ran >= 1
+    with pytest.raises(pkg.OjasHipError, match="RW"):
+        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0, 3],
+                     [(n + 47) // 48, (m + 63) // 64, 1], [256, 1, 1])
+    with pytest.raises(pkg.OjasHipError, match="grid"):
+        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0, 4], [100000, 1, 1],
+                     [256, 1, 1])
+
+
+def test_a_token_does_not_depend_on_its_batch(gpu, pkg):
+    """The same tokens rolled by 37 positions: every output bit for bit, moved."""
+    m, n, k = 200, 512, 4096
+    w, x = _case(pkg, m, n, k, "c")
+    lin = gpu.lin(Q4_K, n, k, w)
+    y1, y2 = gpu.alloc(m * n), gpu.alloc(m * n)
+    gpu.mm(gpu.upload(x), lin, y1, m, act_mode=pkg.ACT_Q8K)
+    perm = np.roll(np.arange(m), 37)
+    gpu.mm(gpu.upload(x[perm].copy()), lin, y2, m, act_mode=pkg.ACT_Q8K)
+    assert np.array_equal(gpu.read(y2, m * n).reshape(m, n), gpu.read(y1, m * n).reshape(m, n)[perm])
