@@ -182,12 +182,23 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
     }
     const size_t w_bytes = w->row_bytes * N;
     const bool dwords_ok = (uintptr_t)wp % 4 == 0 && (w_bytes % 4 == 0 || w->off + w_bytes + 2 <= w->raw->bytes);
-    if (w->type == OJH_Q6_K && m >= dev->q6k_mf_min_m && m <= 16 && dwords_ok) {
+    // (up to 64 tokens as launches of 16: each streams the rows once, which the per-token loop of the
+    // general entry does sixteen times over)
+    if (w->type == OJH_Q6_K && m >= dev->q6k_mf_min_m && m <= 64 && dwords_ok) {
         if ((uint64_t)(m <= 8 ? 8 : 16) * (K + 32) + K / 4 <= 69632) {
-            uint32_t sg[3], sb[3];
-            int rc = ojh_launch_shape(dev, "gemv_q8k_q6k_mf", K, N, m, sg, sb);
-            if (rc) return rc;
-            return ojh_launch(dev, "gemv_q8k_q6k_mf", {xq, xs, wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, sg, sb);
+            const size_t nsb = K / 256;
+            for (uint32_t t0 = 0; t0 < m; t0 += 16) {
+                const uint32_t mc = m - t0 < 16 ? m - t0 : 16;
+                uint32_t sg[3], sb[3];
+                int rc = ojh_launch_shape(dev, "gemv_q8k_q6k_mf", K, N, mc, sg, sb);
+                if (rc) return rc;
+                if ((rc = ojh_launch(dev, "gemv_q8k_q6k_mf",
+                                     {(char *)xq + (size_t)t0 * nsb * 256, (char *)xs + (size_t)t0 * nsb * 4, wp,
+                                      (char *)yp + (size_t)t0 * N * 4},
+                                     {K, N, mc, (uint32_t)(accum != 0)}, sg, sb)))
+                    return rc;
+            }
+            return OJH_OK;
         }
     }
     // few tokens on Q6_K rows: activations staged in LDS once per workgroup, rows grid-stride

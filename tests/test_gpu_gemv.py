@@ -366,7 +366,7 @@ def test_q80_rows_staged_through_lds(pkg, orc, monkeypatch, n, k):
 
 @pytest.mark.parametrize("m,n,k,accum", [(4, 50, 256, False), (8, 130, 4096, True), (9, 301, 4096, False),
                                          (16, 1000, 4096, False), (16, 17, 512, True), (12, 4099, 2560, False),
-                                         (6, 64, 7168, False)])
+                                         (6, 64, 7168, False), (40, 300, 4096, True), (64, 33, 1024, False)])
 def test_q6k_tokens_on_the_int8_matrix_cores(gpu, orc, pkg, m, n, k, accum):
     """5 to 16 tokens against Q6_K rows: `gemv_q8k_q6k_mf` by name and through the router, against
     matvec_kq per token and against the LDS-staged integer-dot entry on the same quantized
@@ -382,6 +382,8 @@ def test_q6k_tokens_on_the_int8_matrix_cores(gpu, orc, pkg, m, n, k, accum):
     got = gpu.read(yd, m * n + 8)
     assert np.all(got[m * n:] == 4242.5), "wrote past the last token"
     assert peak_err(got[:m * n].reshape(m, n) - y0, want) <= TOL_Q8K_SEEN
+    if m > 16:
+        return          # the router ran it as launches of 16 tokens; the entries themselves take at most 16
     gpu.ensure_family("gemv_q8k")
     nsb = k // 256
     xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
