@@ -172,7 +172,8 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
     }
     // a handful of tokens on Q6_K rows: the int8 matrix cores, 8 tokens per pass
     // Q4_K rows against several tokens: the int8 matrix cores
-    if (w->type == OJH_Q4_K && m >= dev->q4k_mf_min_m) {
+    // (from 5 tokens; from 3 on an output head, where the per-token loop of the dot kernel costs most)
+    if (w->type == OJH_Q4_K && (m >= dev->q4k_mf_min_m || (m >= 3 && m + 2 >= dev->q4k_mf_min_m && N >= 32768u))) {
         int rc = ensure(dev, "gemm_q8k");
         if (rc) return rc;
         uint32_t sg[3], sb[3];
