@@ -263,6 +263,19 @@ def extras(gpu, pkg, lin_q) -> dict:
                                "tile": "v_mfma_f32_32x32x16_f16, 256x256 outputs per workgroup (128x256 when that fills more CUs); "
                                        "weights = binary16 fma(qa, q, qb), the bits of the reference's gemm_mm_q4l",
                                "peak_tflops": 2500.0, "timed": "conversion + zero fill (split-K) + tile", **gemm}
+    # ---- the same two matrices in the CPU path's arithmetic (quant_q8k activations, int8 MFMA), f32 in
+    i8 = {}
+    for name, lin in zip(("gate_up_14336x4096", "down_4096x14336"), lin_q):
+        n, k = lin.n, lin.k
+        for m in (8, 16, 128, 512):
+            xf = gpu.upload(synth.normal_f32(m * k, "bench", "i8_x", m, k))
+            y = gpu.alloc(m * n)
+            us = _time(gpu, lambda i: gpu.mm(xf, lin, y, m, act_mode=pkg.ACT_Q8K), 20, 5)
+            i8[f"{name}_M{m}"] = {"us": round(us, 1), "tops": round(2.0 * m * n * k / us / 1e6, 1),
+                                  "weight_gbs": round(n * (k // 256) * 144 / us / 1e3, 1)}
+    out["verify_prefill_q4k_int8"] = {"arithmetic": "quant_q8k activations, int8 x u4 dots on v_mfma_i32_16x16x32_i8, "
+                                                    "the CPU reference's scale algebra (gemm_q8k_q4k_mf)",
+                                      "timed": "quantize_q8k + gemm_q8k_q4k_mf", **i8}
     # ---- config 0: Q8_0 matvec 4096x4096, f32 activations (dot_q80 contract)
     n = k = 4096
     wq8 = [gpu.lin(pkg.Q8_0, n, k, synth.q80_weights(n, k, "bench", "q80")) for _ in range(16)]
