@@ -5,7 +5,7 @@
 // This is what serves speculative verify (2-16 tokens on every projection) and prefill chunks
 // with results within the parity bar of the CPU path, which an f16 tile cannot give.
 //
-//   gemm_q8k_q4k_mf(xq, xs, w, y, K, N, M, ACC, RW)      block 256, grid [x <= ceil(N / (16 RW)), ceil(M / 64), 1]
+//   gemm_q8k_q4k_mf(xq, xs, w, y, K, N, M, ACC, RW, RT)   block 256, grid [x <= ceil(N / (16 RW RT)), ceil(M / 64), 1]
 //
 // v_mfma_i32_16x16x32_i8 multiplies 16 tokens x 16 rows over one sub-block:
 //   A: lane (m, kg) = (lane % 16, lane / 16) holds int8 positions 8 kg .. 8 kg + 7 of token m;
@@ -19,7 +19,8 @@
 // sum_j m_j hi_j for all 16 x 16 outputs at once.  A super-block ends with two converts and
 // three FMAs per output.
 //
-// A workgroup owns 16 RW rows (RW = 1, 2 or 4 row tiles) and up to 64 tokens (P = 1, 2 or 4 passes of
+// A workgroup owns 16 RW RT rows (RW = 1, 2 or 4 row tiles side by side, each wave RT of them one after
+// the other per staged chunk; only RT = 1 is built) and up to 64 tokens (P = 1, 2 or 4 passes of
 // 16; eight passes do not fit the register file); its four waves are RW row tiles x KW = 4 / RW slices of the super-blocks.  Tokens wait in
 // LDS, chunk by chunk of K (as many super-blocks as fit 76 KB for the workgroup's tokens: 256 bytes,
 // a scale and 16 bytes of split sums per token and super-block), rows 32 bytes longer than the
@@ -44,7 +45,7 @@ __device__ __forceinline__ GqW gq_load(const uchar* blk, uint kg) {
     return r;
 }
 
-template <int P>
+template <int P, int RT>
 __device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
                                                      const uchar* __restrict__ w, float* __restrict__ y,
                                                      uint K, uint N, uint M, uint ACC, uint RW, uchar* lds) {
@@ -52,14 +53,14 @@ __device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restri
     const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint nsb = K >> 8, KW = 4u / RW, rt = wave / KW, kw = wave % KW;
     const uint BM = 16u * P, t0 = blockIdx.y * 64u;
-    // LDS: [reduction buffer: 4 waves x P x 4 x 64 floats] [tokens] [token scales] [split bsums].
+    // LDS: [reduction buffer: 4 waves x RT x P x 4 x 64 floats] [tokens] [token scales] [split bsums].
     // Chunk of K staged at a time: BM * (KC + 32) + (KC / 256) * BM * 20 bytes, a whole multiple of
     // KW super-blocks so that a wave's slice continues from chunk to chunk (the host picks RW so
     // that at least KW fit).  When the whole K fits, the tokens are staged once and the workgroup
-    // walks row tiles blockIdx.x, blockIdx.x + gridDim.x, ...
+    // walks row groups blockIdx.x, blockIdx.x + gridDim.x, ...
     float* red = (float*)lds;
-    uchar* tok = lds + 4096u * P;
-    const uint fit = ((GQ_LDS - 4096u * P) / BM - 32u) / 276u;
+    uchar* tok = lds + 4096u * P * (KW > 1u ? RT : 0u);
+    const uint fit = ((GQ_LDS - 4096u * P * (KW > 1u ? RT : 0u)) / BM - 32u) / 276u;
     const bool whole = nsb <= fit;
     const uint csb = whole ? nsb : fit / KW * KW;                // super-blocks per chunk
     const uint S = csb * 256u + 32u;
@@ -68,20 +69,26 @@ __device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restri
     const uint n = lane & 15u, kg = lane >> 4;
     const uchar* xa = tok + (size_t)n * S + 8u * kg;
     const gq_i4 zero = {0, 0, 0, 0};
-    const uint ntiles = (N + 16u * RW - 1u) / (16u * RW);
-    for (uint tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const uint row = min((tile * RW + rt) * 16u + n, N - 1u);
-        const uchar* wr = w + (size_t)row * nsb * Q4K_BYTES;
-        float acc[P][4];
+    const uint ngroups = (N + 16u * RW * RT - 1u) / (16u * RW * RT);
+    const size_t rtb = (size_t)16u * RW * nsb * Q4K_BYTES;       // bytes from a row tile of this wave to its next
+    for (uint grp = blockIdx.x; grp < ngroups; grp += gridDim.x) {
+        // this wave's row tiles: (grp * RT + q) * RW + rt, q = 0 .. RT - 1 (rows past N clamped per tile)
+        const uint tile0 = grp * RT * RW + rt;
+        uint rowq[RT];
 #pragma unroll
-        for (int p = 0; p < P; p++)
+        for (int q = 0; q < RT; q++) rowq[q] = min((tile0 + (uint)q * RW) * 16u + n, N - 1u);
+        float acc[RT][P][4];
 #pragma unroll
-            for (int v = 0; v < 4; v++) acc[p][v] = 0.0f;
-        GqW cur = gq_load(wr + (size_t)min(kw, nsb - 1u) * Q4K_BYTES, kg);
+        for (int q = 0; q < RT; q++)
+#pragma unroll
+            for (int p = 0; p < P; p++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) acc[q][p][v] = 0.0f;
+        GqW cur = gq_load(w + ((size_t)rowq[0] * nsb + min(kw, nsb - 1u)) * Q4K_BYTES, kg);
         for (uint sb0 = 0; sb0 < nsb; sb0 += csb) {
             const uint cn = min(csb, nsb - sb0);                 // super-blocks in this chunk
-            if (!whole || tile == blockIdx.x) {
-                if (sb0 || tile != blockIdx.x) __syncthreads();  // everyone is done with the previous chunk
+            if (!whole || grp == blockIdx.x) {
+                if (sb0 || grp != blockIdx.x) __syncthreads();   // everyone is done with the previous chunk
                 // stage tokens t0 .. t0 + BM - 1 (zeros past M): a thread keeps one 16-byte column of the
                 // chunk and walks the tokens eight loads at a time (one wait per eight, not per load)
                 const uint per_row = cn * 16u, lpr = min(per_row, 256u), rpp = 256u / lpr;
@@ -126,91 +133,114 @@ __device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restri
                 __syncthreads();
             }
             for (uint s = kw; s < cn; s += KW) {
-                // the next super-block of this wave's slice (in this chunk or the next) is on its way
-                const uint nxt = s + KW < cn ? sb0 + s + KW : sb0 + csb + kw;
-                const GqW nx = gq_load(wr + (size_t)min(nxt, nsb - 1u) * Q4K_BYTES, kg);
-                const float d = f16_bits_to_f32(cur.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
-                int sc[8];
-                long B[8], Bm = 0;
+                const uint nxt = s + KW < cn ? sb0 + s + KW : sb0 + csb + kw;   // this slice's next super-block
 #pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    uint a, b;
-                    q4k_scale_min_pair(cur.hdr.y, cur.hdr.z, cur.hdr.w, (uint)c, a, b);
-                    sc[2 * c] = (int)(a & 0xFFu); sc[2 * c + 1] = (int)(a >> 8);
-                    Bm |= (long)(unsigned long)(b & 0xFFFFu) << (16 * c);    // mins 2c, 2c + 1 -> bytes 2c, 2c + 1
-                    B[2 * c] = gq_pack(cur.q[c].x & 0x0F0F0F0Fu, cur.q[c].y & 0x0F0F0F0Fu);
-                    B[2 * c + 1] = gq_pack((cur.q[c].x >> 4) & 0x0F0F0F0Fu, (cur.q[c].y >> 4) & 0x0F0F0F0Fu);
-                }
-                if (kg != 0u) Bm = 0;                                        // only positions 0..7 carry mins
+                for (int q = 0; q < RT; q++) {
+                    // the next (row tile, super-block) of this wave is on its way
+                    const GqW nx = q + 1 < RT
+                        ? gq_load(w + ((size_t)rowq[q + 1 < RT ? q + 1 : 0] * nsb + sb0 + s) * Q4K_BYTES, kg)
+                        : gq_load(w + ((size_t)rowq[0] * nsb + min(nxt, nsb - 1u)) * Q4K_BYTES, kg);
+                    const float d = f16_bits_to_f32(cur.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
+                    int sc[8];
+                    long B[8], Bm = 0;
 #pragma unroll
-                for (int p = 0; p < P; p++) {
-                    int isum[4] = {0, 0, 0, 0};
-                    const uchar* xp = xa + (size_t)(16 * p) * S + s * 256u;
-#pragma unroll
-                    for (int jj = 0; jj < 8; jj++) {
-                        const long A = *(const long*)(xp + 32 * jj);
-                        const gq_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B[jj], zero, 0, 0, 0);
-#pragma unroll
-                        for (int v = 0; v < 4; v++) isum[v] += __mul24(sc[jj], D[v]);
+                    for (int c = 0; c < 4; c++) {
+                        uint a, b;
+                        q4k_scale_min_pair(cur.hdr.y, cur.hdr.z, cur.hdr.w, (uint)c, a, b);
+                        sc[2 * c] = (int)(a & 0xFFu); sc[2 * c + 1] = (int)(a >> 8);
+                        Bm |= (long)(unsigned long)(b & 0xFFFFu) << (16 * c);    // mins 2c, 2c + 1 -> bytes 2c, 2c + 1
+                        B[2 * c] = gq_pack(cur.q[c].x & 0x0F0F0F0Fu, cur.q[c].y & 0x0F0F0F0Fu);
+                        B[2 * c + 1] = gq_pack((cur.q[c].x >> 4) & 0x0F0F0F0Fu, (cur.q[c].y >> 4) & 0x0F0F0F0Fu);
                     }
-                    // token n of this pass: its eight lo parts, then its eight hi parts (lanes kg = 0 only)
-                    const uchar* pq = lbq + ((size_t)s * BM + 16u * p + n) * 16u;
-                    long Alo = 0, Ahi = 0;
-                    if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
-                    const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
-                    const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
-                    const float4 sx = *(const float4*)(lsx + s * BM + 16u * p + 4u * kg);
-                    acc[p][0] += sx.x * (d * (float)isum[0] - dmin * (float)(64 * Dhi[0] + Dlo[0]));
-                    acc[p][1] += sx.y * (d * (float)isum[1] - dmin * (float)(64 * Dhi[1] + Dlo[1]));
-                    acc[p][2] += sx.z * (d * (float)isum[2] - dmin * (float)(64 * Dhi[2] + Dlo[2]));
-                    acc[p][3] += sx.w * (d * (float)isum[3] - dmin * (float)(64 * Dhi[3] + Dlo[3]));
+                    if (kg != 0u) Bm = 0;                                        // only positions 0..7 carry mins
+#pragma unroll
+                    for (int p = 0; p < P; p++) {
+                        int isum[4] = {0, 0, 0, 0};
+                        const uchar* xp = xa + (size_t)(16 * p) * S + s * 256u;
+#pragma unroll
+                        for (int jj = 0; jj < 8; jj++) {
+                            const long A = *(const long*)(xp + 32 * jj);
+                            const gq_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B[jj], zero, 0, 0, 0);
+#pragma unroll
+                            for (int v = 0; v < 4; v++) isum[v] += __mul24(sc[jj], D[v]);
+                        }
+                        // token n of this pass: its eight lo parts, then its eight hi parts (lanes kg = 0 only)
+                        const uchar* pq = lbq + ((size_t)s * BM + 16u * p + n) * 16u;
+                        long Alo = 0, Ahi = 0;
+                        if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
+                        const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
+                        const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
+                        const float4 sx = *(const float4*)(lsx + s * BM + 16u * p + 4u * kg);
+                        acc[q][p][0] += sx.x * (d * (float)isum[0] - dmin * (float)(64 * Dhi[0] + Dlo[0]));
+                        acc[q][p][1] += sx.y * (d * (float)isum[1] - dmin * (float)(64 * Dhi[1] + Dlo[1]));
+                        acc[q][p][2] += sx.z * (d * (float)isum[2] - dmin * (float)(64 * Dhi[2] + Dlo[2]));
+                        acc[q][p][3] += sx.w * (d * (float)isum[3] - dmin * (float)(64 * Dhi[3] + Dlo[3]));
+                        // (keeps the passes apart: let loose, the scheduler hoists every pass's reads and
+                        // products to the front and the kernel spills)
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    cur = nx;
+                    // the tokens are read from LDS again for the next row tile: kept in registers across
+                    // row tiles (which the compiler would do) they cost 96 registers and the kernel spills
+                    if (RT > 1) asm volatile("" ::: "memory");
                 }
-                cur = nx;
             }
         }
         // K-slices of a row tile meet in LDS, added in slice order
         if (KW > 1u) {
 #pragma unroll
-            for (int p = 0; p < P; p++)
+            for (int q = 0; q < RT; q++)
 #pragma unroll
-                for (int v = 0; v < 4; v++) red[((wave * P + p) * 4 + v) * 64u + lane] = acc[p][v];
+                for (int p = 0; p < P; p++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) red[(((wave * RT + q) * P + p) * 4 + v) * 64u + lane] = acc[q][p][v];
             __syncthreads();
             if (kw == 0u) {
+#pragma unroll
+                for (int q = 0; q < RT; q++)
+#pragma unroll
+                    for (int p = 0; p < P; p++)
+#pragma unroll
+                        for (int v = 0; v < 4; v++) {
+                            float t = acc[q][p][v];
+                            for (uint k2 = 1; k2 < KW; k2++) t += red[((((wave + k2) * RT + q) * P + p) * 4 + v) * 64u + lane];
+                            acc[q][p][v] = t;
+                        }
+            }
+            __syncthreads();                                     // before the next group writes `red`
+        }
+        if (kw == 0u) {
+#pragma unroll
+            for (int q = 0; q < RT; q++) {
+                const uint r_out = (tile0 + (uint)q * RW) * 16u + n;
 #pragma unroll
                 for (int p = 0; p < P; p++)
 #pragma unroll
                     for (int v = 0; v < 4; v++) {
-                        float t = acc[p][v];
-                        for (uint k2 = 1; k2 < KW; k2++) t += red[(((wave + k2) * P + p) * 4 + v) * 64u + lane];
-                        acc[p][v] = t;
+                        const uint t = t0 + 16u * p + 4u * kg + v;
+                        if (t < M && r_out < N) {
+                            float* o = y + (size_t)t * N + r_out;
+                            *o = ACC ? *o + acc[q][p][v] : acc[q][p][v];
+                        }
                     }
             }
-            __syncthreads();                                     // before the next tile writes `red`
-        }
-        if (kw == 0u) {
-            const uint r_out = (tile * RW + rt) * 16u + n;
-#pragma unroll
-            for (int p = 0; p < P; p++)
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    const uint t = t0 + 16u * p + 4u * kg + v;
-                    if (t < M && r_out < N) {
-                        float* o = y + (size_t)t * N + r_out;
-                        *o = ACC ? *o + acc[p][v] : acc[p][v];
-                    }
-                }
         }
     }
 }
 
+// (Only RT = 1 is built.  With four row tiles per wave a staged chunk of tokens would serve 256 rows,
+// which is what a batch of hundreds of tokens needs — at 64 rows per workgroup the re-staging of the
+// tokens is the larger stream — but that instance needs more than 256 registers as compiled, spills and
+// runs ten times slower.)
 // (at least two waves per SIMD: with a register budget of 256 the matrix-core results are written
 // to ordinary registers instead of the accumulation file, which saves a move per result)
 extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8)))
 gemm_q8k_q4k_mf(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC,
-                uint RW) {
+                uint RW, uint RT) {
     __shared__ __attribute__((aligned(16))) uchar lds_gq[GQ_LDS];
     const uint left = M - min(M, blockIdx.y * 64u);              // tokens of this workgroup's tile
-    if (left <= 16u) gemm_q8k_q4k_mf_body<1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
-    else if (left <= 32u) gemm_q8k_q4k_mf_body<2>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
-    else gemm_q8k_q4k_mf_body<4>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
+    (void)RT;                                                    // only one row tile per wave is built
+    if (left <= 16u) gemm_q8k_q4k_mf_body<1, 1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
+    else if (left <= 32u) gemm_q8k_q4k_mf_body<2, 1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
+    else gemm_q8k_q4k_mf_body<4, 1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
 }

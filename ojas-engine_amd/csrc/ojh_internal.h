@@ -116,5 +116,5 @@ const ojh_kernel_spec *ojh_find_kernel(const char *name);
 int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out);
 int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptrs,
                const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);
-uint32_t ojh_gemm_q8k_rw(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M);   // row tiles per workgroup of gemm_q8k_q4k_mf
+void ojh_gemm_q8k_tiles(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M, uint32_t *rw, uint32_t *rt);   // row tiles per workgroup / per wave of gemm_q8k_q4k_mf
 uint32_t ojh_q80_lds_kc(uint32_t K);   // chunks of K for gemv_nat_q80_lds, 0 if none (ojh_manifest.cpp)

@@ -118,27 +118,31 @@ static int shape_q80_lds(const ojh_kernel_spec *, const ojh_device *dev, uint32_
     return OJH_OK;
 }
 
-// gemm_q8k_q4k_mf(xq, xs, w, y, K, N, M, ACC, RW): 16 RW rows x up to 64 tokens per workgroup.
+// gemm_q8k_q4k_mf(xq, xs, w, y, K, N, M, ACC, RW, RT): 16 RW RT rows x up to 64 tokens per workgroup.
 // The tokens of a workgroup wait in 76 KB of LDS chunk by chunk of K; a chunk must hold at least
-// 4 / RW super-blocks (the waves that split K).
-uint32_t ojh_gemm_q8k_fit(uint32_t M) {   // super-blocks of K that fit for the largest token tile of M tokens
+// 4 / RW super-blocks (the waves that split K).  RT (row tiles per wave) must be 1.
+uint32_t ojh_gemm_q8k_fit(uint32_t M, uint32_t RW, uint32_t RT) {   // super-blocks of K that fit for the largest token tile
     uint32_t left = M > 64 ? 64 : M, bm = left <= 16 ? 16 : left <= 32 ? 32 : 64;
-    return ((77824 - 256 * bm) / bm - 32) / 276;   // 4 KB of reduction buffer per 16 tokens come first
+    uint32_t red = RW < 4 ? 256 * bm * RT : 0;     // the K-slices' reduction buffer comes first
+    return ((77824 - red) / bm - 32) / 276;
 }
 static int check_gemm_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                           const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f;
-    uint32_t K = c[0], N = c[1], M = c[2], RW = c[4];
+    uint32_t K = c[0], N = c[1], M = c[2], RW = c[4], RT = c[5];
     int rc = check_kn(s, K, N, &f);
     if (rc) return rc;
     if ((rc = check_block(block, 256))) return rc;
     if (!M || M > 65535) return ojh_fail(OJH_ERR_ARG, "%s: M=%u out of range", s->name, M);
     if (RW != 1 && RW != 2 && RW != 4) return ojh_fail(OJH_ERR_ARG, "%s: RW=%u must be 1, 2 or 4", s->name, RW);
-    if (K / 256 > ojh_gemm_q8k_fit(M) && ojh_gemm_q8k_fit(M) < 4 / RW)
+    if (RT != 1) return ojh_fail(OJH_ERR_ARG, "%s: RT=%u: only one row tile per wave is built", s->name, RT);
+    const uint32_t fit = ojh_gemm_q8k_fit(M, RW, RT);
+    if (K / 256 > fit && fit < 4 / RW)
         return ojh_fail(OJH_ERR_ARG, "%s: RW=%u leaves %u waves on K but only %u super-blocks of %u tokens fit in LDS", s->name,
-                        RW, 4 / RW, ojh_gemm_q8k_fit(M), M > 64 ? 64 : M);
-    if (!grid[0] || grid[0] > (N + 16 * RW - 1) / (16 * RW) || grid[1] != (M + 63) / 64 || grid[2] != 1)
-        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N / (16 RW)), ceil(M / 64), 1]", s->name);
+                        RW, 4 / RW, fit, M > 64 ? 64 : M);
+    const uint32_t groups = (N + 16 * RW * RT - 1) / (16 * RW * RT);
+    if (!grid[0] || grid[0] > groups || grid[1] != (M + 63) / 64 || grid[2] != 1)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N / (16 RW RT)), ceil(M / 64), 1]", s->name);
     need[0] = (size_t)M * K;
     need[1] = (size_t)M * (K / 256) * 4;
     need[2] = (size_t)N * (K / 256) * 144;
@@ -147,30 +151,39 @@ static int check_gemm_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uin
     align[3] = 4;
     return OJH_OK;
 }
-// row tiles per workgroup: as many as still give every CU a workgroup and a half (more rows per workgroup
-// spread the staging of the tokens over more work; measured on 14336 x 4096 and 4096 x 4096), at least
-// what the LDS chunk asks for
-uint32_t ojh_gemm_q8k_rw(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M) {
-    const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, fit = ojh_gemm_q8k_fit(M);
-    const uint32_t rw_min = K / 256 <= fit || fit >= 4 ? 1 : fit >= 2 ? 2 : 4;
+// Row tiles per workgroup (RW side by side, RT = 1 per wave): as many side by side as still give every CU a
+// workgroup and a half (measured on 14336 x 4096 and 4096 x 4096), at least what the LDS chunk asks for.
+void ojh_gemm_q8k_tiles(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M, uint32_t *rw_out, uint32_t *rt_out) {
+    const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
     const uint64_t tiles_m = (M + 63) / 64;
     uint32_t rw = 4;
-    while (rw > rw_min && (uint64_t)((N + 16 * rw - 1) / (16 * rw)) * tiles_m * 2 < 3ull * cus) rw /= 2;
-    return rw;
+    for (;;) {
+        const uint32_t fit = ojh_gemm_q8k_fit(M, rw, 1);
+        const bool ok = K / 256 <= fit || fit >= 4 / rw;
+        const bool enough = (uint64_t)((N + 16 * rw - 1) / (16 * rw)) * tiles_m * 2 >= 3ull * cus;
+        if (rw == 1 || (ok && enough)) break;
+        // fewer rows per workgroup only if the chunk still feeds the extra waves on K
+        const uint32_t fit2 = ojh_gemm_q8k_fit(M, rw / 2, 1);
+        if (!(K / 256 <= fit2 || fit2 >= 4 / (rw / 2))) break;
+        rw /= 2;
+    }
+    *rw_out = rw;
+    *rt_out = 1;
 }
 static int shape_gemm_q8k(const ojh_kernel_spec *, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
                           uint32_t grid[3], uint32_t block[3]) {
     if (!M) M = 1;
-    const uint32_t rw = ojh_gemm_q8k_rw(dev, K, N, M);
-    grid[0] = (N + 16 * rw - 1) / (16 * rw);
+    uint32_t rw, rt;
+    ojh_gemm_q8k_tiles(dev, K, N, M, &rw, &rt);
+    grid[0] = (N + 16 * rw * rt - 1) / (16 * rw * rt);
     grid[1] = (M + 63) / 64;
-    // the whole K staged once: row tiles grid-stride over two workgroups per CU
+    grid[2] = 1;
+    // the whole K staged once: row groups grid-stride over two workgroups per CU
     const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
-    if (K / 256 <= ojh_gemm_q8k_fit(M) && grid[0] * grid[1] > 2 * cus) {
+    if (K / 256 <= ojh_gemm_q8k_fit(M, rw, rt) && grid[0] * grid[1] > 2 * cus) {
         uint32_t gx = 2 * cus / grid[1];
         grid[0] = gx ? gx : 1;
     }
-    grid[2] = 1;
     block[0] = 256;
     block[1] = block[2] = 1;
     return OJH_OK;
@@ -866,7 +879,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
             add(fq + "_wide", "gemv_q8k", 3, 3, f.type, 2, check_gemv_fq8k, shape_rows);
         }
     }
-    add("gemm_q8k_q4k_mf", "gemm_q8k", 4, 5, OJH_Q4_K, 1, check_gemm_q8k, shape_gemm_q8k);
+    add("gemm_q8k_q4k_mf", "gemm_q8k", 4, 6, OJH_Q4_K, 1, check_gemm_q8k, shape_gemm_q8k);
     add("relayout_q4k_q4l", "dequant", 4, 1, OJH_Q4_K, 0, check_relayout, shape_relayout);
     add("rows_q8_from_f16", "rowq8", 3, 2, 0, 0, check_rowq8, shape_rowq8);
     add("quant_rows_i8", "rowq8", 3, 2, 0, 1, check_rowq8, shape_rowq8);

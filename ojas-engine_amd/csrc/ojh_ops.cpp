@@ -178,8 +178,9 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
         if (rc) return rc;
         uint32_t sg[3], sb[3];
         if ((rc = ojh_launch_shape(dev, "gemm_q8k_q4k_mf", K, N, m, sg, sb))) return rc;
-        return ojh_launch(dev, "gemm_q8k_q4k_mf", {xq, xs, wp, yp},
-                          {K, N, m, (uint32_t)(accum != 0), ojh_gemm_q8k_rw(dev, K, N, m)}, sg, sb);
+        uint32_t rw, rt;
+        ojh_gemm_q8k_tiles(dev, K, N, m, &rw, &rt);
+        return ojh_launch(dev, "gemm_q8k_q4k_mf", {xq, xs, wp, yp}, {K, N, m, (uint32_t)(accum != 0), rw, rt}, sg, sb);
     }
     const size_t w_bytes = w->row_bytes * N;
     const bool dwords_ok = (uintptr_t)wp % 4 == 0 && (w_bytes % 4 == 0 || w->off + w_bytes + 2 <= w->raw->bytes);

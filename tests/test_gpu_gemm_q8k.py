@@ -20,7 +20,8 @@ def _case(pkg, m, n, k, tag):
 
 @pytest.mark.parametrize("m,n,k,accum", [(2, 50, 256, False), (16, 130, 4096, True), (17, 333, 2560, False),
                                          (40, 64, 14336, True), (128, 100, 1024, False), (129, 300, 512, False),
-                                         (300, 40, 4096, True), (8, 4099, 4096, False), (64, 17, 8192, False)])
+                                         (300, 40, 4096, True), (8, 4099, 4096, False), (64, 17, 8192, False),
+                                         (130, 6200, 512, True)])
 def test_router_path_matches_the_cpu_reference(gpu, orc, pkg, m, n, k, accum):
     w, x = _case(pkg, m, n, k, "a")
     lin = gpu.lin(Q4_K, n, k, w)
@@ -55,7 +56,7 @@ def test_every_row_tiling_and_the_integer_dot_kernel_agree(gpu, orc, pkg, m, n, 
         grid = [(n + 16 * rw - 1) // (16 * rw), (m + 63) // 64, 1]
         y = gpu.upload(np.full(m * n, 7.0, np.float32))
         try:
-            gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0, rw], grid,
+            gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0, rw, 1], grid,
                          [256, 1, 1])
         except pkg.OjasHipError as e:
             assert "super-blocks" in str(e)            # the chunk is too short for that many waves on K
@@ -65,11 +66,14 @@ def test_every_row_tiling_and_the_integer_dot_kernel_agree(gpu, orc, pkg, m, n, 
         assert peak_err(got, dots) <= 2e-6, rw
         ran += 1
     assert ran >= 1
+    with pytest.raises(pkg.OjasHipError, match="RT"):
+        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0, 4, 4],
+                     [(n + 255) // 256, (m + 63) // 64, 1], [256, 1, 1])
     with pytest.raises(pkg.OjasHipError, match="RW"):
-        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0, 3],
+        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0, 3, 1],
                      [(n + 47) // 48, (m + 63) // 64, 1], [256, 1, 1])
     with pytest.raises(pkg.OjasHipError, match="grid"):
-        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0, 4], [100000, 1, 1],
+        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y, 0)], [k, n, m, 0, 4, 1], [100000, 1, 1],
                      [256, 1, 1])
 
 
