@@ -20,7 +20,7 @@
 //   moe_topk_m(lg, idx, wgt, E, KSEL)                        grid = tokens
 //   moe_group(idx, counts, offsets, list, NA, E)             1 x 256 threads; NA = tokens*KSEL
 //   moe_gu_q4k_m(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA)   grid (ceil(N/8), E)
-//   moe_down_{q4k,q5k}_m(aq, as, wd, dv, offsets, list, K, N, NA)      grid (ceil(N/16), E)
+//   moe_down_{q4k,q5k}_m(aq, as, wd, dv, offsets, list, K, N, NA)      grid (ceil(N/16), E); ceil(N/32) for K <= 1024
 //   moe_combine(dv, wgt, y, T, KSEL, D, ACC)                 grid ceil(T*D/256)
 //   moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)   grid (ceil(N/8), NA): few tokens, f32 in
 //   moe_down_{q4k,q5k}_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)  grid (ceil(N/8), T): down + weighted sum
@@ -213,10 +213,36 @@ __device__ __forceinline__ void moe_down_m_body(const signed char* __restrict__ 
     const uint a0 = min(offsets[e], NA), a1 = min(offsets[e + 1], NA);
     if (a0 >= a1) return;
     const uint lane = threadIdx.x & 63u;
-    const uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 4u;
-    if (row0 >= N) return;
     const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
     const size_t rb = (size_t)nsb * W::BYTES;
+    if (nsb <= 4u) {
+        // A short row (an expert's down projection: 768 = 3 super-blocks) leaves most of a wave idle in
+        // the layout below.  Here the wave's halves take different rows: 8 rows per wave, 32 per
+        // workgroup, and a half's two 16-lane sums are added as wave_sum adds them.
+        const uint hf = lane >> 5, G = g & 3u;
+        const uint rowh = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 8u + hf * 4u;     // this half's first row
+        const bool on = G < nsb;
+        const uchar* wh = wd + ((size_t)e * N + min(rowh, N - 1u)) * rb + (size_t)(on ? G : 0u) * W::BYTES;
+        W wr[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) wr[r].load(wh + (size_t)min((uint)r, N - 1u - min(rowh, N - 1u)) * rb, l);
+        for (uint i = a0; i < a1; i++) {
+            const uint a = min(list[i], NA - 1u);
+            Q4kFrag f = q4k_load_frag(aq + (size_t)a * nsb * 256u, as_ + (size_t)a * nsb, on ? G : 0u, l);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float v = row16_sum(on ? wr[r].dot(c, f) : 0.0f);
+                const float s0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)) +
+                                 __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+                const float s1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32)) +
+                                 __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+                if ((lane & 31u) == 0 && rowh + r < N) dv[(size_t)a * N + rowh + r] = hf ? s1 : s0;
+            }
+        }
+        return;
+    }
+    const uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 4u;
+    if (row0 >= N) return;
     const uchar* w0 = wd + ((size_t)e * N + row0) * rb;
     if (nsb <= 8u) {
         const bool on = g < nsb;

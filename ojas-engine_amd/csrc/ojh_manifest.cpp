@@ -559,7 +559,7 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
 //   0 moe_topk(lg, idx, wgt, E, KSEL)            1 moe_topk_m(same)              grid [T,1,1] x 64
 //   2 moe_group(idx, counts, offsets, list, NA, E)                                grid [1,1,1] x 256
 //   3 moe_gu_q4k_m(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA)            grid [ceil(N/8), E, 1]
-//   4 moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)                     grid [ceil(N/16), E, 1]
+//   4 moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)                     grid [ceil(N/16), E, 1]; ceil(N/32) for K <= 1024
 //   5 moe_combine(dv, wgt, y, T, KSEL, D, ACC)                                    grid [ceil(T*D/256),1,1]
 //   6 moe_gu_q4k_mm, 7 moe_down_q4k_mm: the arguments of 3 and 4, grid [ceil(N/16), E, 1]
 //   8 moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)                      grid [ceil(N/8), NA, 1]
@@ -610,7 +610,7 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
     }
     case 4: case 7: {
         uint32_t K = c[0], N = c[1], NA = c[2], E = grid[1];
-        const uint32_t per = 16;
+        const uint32_t per = s->rows_per_wave == 4 && K <= 1024 ? 32 : 16;   // short rows: two row sets per wave
         if ((rc = check_block(block, 256))) return rc;
         if (!K || K % 256 || !N || !NA) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u NA=%u", s->name, K, N, NA);
         if (grid[0] != (N + per - 1) / per || grid[2] != 1)
@@ -702,7 +702,6 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
 // K, N as named by the kernel; M = tokens (topk, combine) or assignments (group)
 static int shape_moe(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, uint32_t N, uint32_t M,
                      uint32_t grid[3], uint32_t block[3]) {
-    (void)K;
     grid[0] = grid[1] = grid[2] = 1;
     block[0] = 256;
     block[1] = block[2] = 1;
@@ -711,7 +710,7 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, u
     case 1: block[0] = 64; grid[0] = M ? M : 1; break;
     case 2: break;
     case 3: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = experts
-    case 4: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
+    case 4: grid[0] = K <= 1024 ? (N + 31) / 32 : (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
     case 6: case 7: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;
     case 8: case 10: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = assignments
     case 9: case 11: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = tokens

@@ -86,9 +86,9 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     uint32_t *counts = (uint32_t *)grp->ptr, *offsets = counts + E, *list = offsets + E + 1;
 
     // Expert products: on the matrix cores once experts see a few tokens each (measured crossover on
-    // MI355X: ~2 assignments per expert), on integer dots below that, where the launch is a pure
+    // MI355X: ~4 assignments per expert), on integer dots below that, where the launch is a pure
     // stream of weight rows.  The two forms round their f32 sums in different orders (last ulp).
-    const bool mm = dev->moe_mode == 1 || (dev->moe_mode == 0 && NA >= 2 * E);
+    const bool mm = dev->moe_mode == 1 || (dev->moe_mode == 0 && NA >= 4 * E);
     // 1. quantize the tokens once
     {
         uint32_t g[3] = {nsb_d, T, 1};
@@ -115,7 +115,8 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     }
     // 5. down, one launch over all experts
     {
-        uint32_t g[3] = {(d + 15) / 16, E, 1};
+        const bool dots = down5 || !mm;
+        uint32_t g[3] = {dots && n_ff <= 1024 ? (d + 31) / 32 : (d + 15) / 16, E, 1};
         // (Q5_K rows have no matrix-core form: they stay on integer dots at every batch size)
         if ((rc = ojh_launch(dev, down5 ? "moe_down_q5k_m" : mm ? "moe_down_q4k_mm" : "moe_down_q4k_m",
                              {aq->ptr, as_->ptr, (char *)down->raw->ptr + down->off, dv->ptr, offsets, list},
