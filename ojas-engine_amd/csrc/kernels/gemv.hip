@@ -359,31 +359,6 @@ __device__ __forceinline__ void gemv_nat_q80_m_body(const float* __restrict__ x,
 #define Q80L_CHUNK 4352u   // 128 blocks
 #define Q80L_DEPTH 2u
 
-__device__ __forceinline__ void q80l_load_lds16(const void* base, uint voff, uint lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(voff), "s"(base), "s"(lds_addr)
-                 : "memory");
-}
-// wait until at most `n` (0 .. 10) vector loads are outstanding
-__device__ __forceinline__ void q80l_wait(uint n) {
-    switch (n) {
-    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-    case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
-    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
-    case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
-    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-    case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
-    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
-    case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-    case 9: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
-    case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
-    case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
-    case 15: asm volatile("s_waitcnt vmcnt(15)" ::: "memory"); break;
-    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-    }
-}
-
 __device__ __forceinline__ float q80l_dot4(uint v, float a, float x0, float x1, float x2, float x3) {
     a = fmaf(sb0(v), x0, a);
     a = fmaf(sb1(v), x1, a);
@@ -413,7 +388,7 @@ __device__ __forceinline__ void gemv_nat_q80_lds_body(const float* __restrict__ 
         const uchar* base = w + (size_t)row * row_bytes + (size_t)chunk * chunk_bytes;
         const uint dst = lds0 + (k % Q80L_DEPTH) * Q80L_CHUNK;
         for (uint i = 0; i < NI; i++)
-            if (i * 64u + lane < n16) q80l_load_lds16(base, (i * 64u + lane) << 4, dst + i * 1024u);
+            if (i * 64u + lane < n16) lds_dma16(base, (i * 64u + lane) << 4, dst + i * 1024u);
     };
     // the wave's activations: blocks 2l, 2l+1 of its chunk
     float xr[64];
@@ -430,7 +405,7 @@ __device__ __forceinline__ void gemv_nat_q80_lds_body(const float* __restrict__ 
         if (k < my_steps) issue(k);
     for (uint k = 0; k < my_steps; k++) {
         if (k + Q80L_DEPTH - 1u < my_steps) issue(k + Q80L_DEPTH - 1u);
-        q80l_wait(min(my_steps - 1u - k, Q80L_DEPTH - 1u) * NI);
+        vm_wait(min(my_steps - 1u - k, Q80L_DEPTH - 1u) * NI);
         const uint* p = (const uint*)(mine + (k % Q80L_DEPTH) * Q80L_CHUNK);
         uint d[17];
 #pragma unroll

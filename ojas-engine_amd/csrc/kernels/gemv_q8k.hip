@@ -858,7 +858,7 @@ gemv_q8k_q6k_mx(const signed char* xq, const float* xs, const uchar* w, float* y
 }
 
 // ---- Q6_K against up to 16 tokens on the int8 matrix cores ------------------------------------
-//   gemv_q8k_q6k_mf(xq, xs, w, y, K, N, M, ACC)    M <= 16, MT (K + 32) + K / 4 <= 69632 (MT = 8 or 16)
+//   gemv_q8k_q6k_mf(xq, xs, w, y, K, N, M, ACC)    M <= 16, MT (K + 32) + K / 4 + 256 <= 69632 (MT = 8 or 16)
 // The verify head reads 510 MB of weights whatever the token count; with integer dots the work
 // per row grows with M and the launch turns compute-bound from M = 4.  Here a wave owns 16 rows
 // and runs them against 8 tokens at a time with v_mfma_i32_16x16x32_i8:
@@ -866,8 +866,8 @@ gemv_q8k_q6k_mx(const signed char* xq, const float* xs, const uchar* w, float* y
 //     quarters of a super-block, the signed codes q - 32 of positions 8 kg .. 8 kg + 7 of row n;
 //   * a quarter holds two 16-weight groups with their own int8 scale, and an MFMA sums over all
 //     32 positions.  So the 16 token rows of A are 8 tokens twice: rows 0-7 carry only positions
-//     0-15 (lanes kg < 2), rows 8-15 only positions 16-31 (lanes kg >= 2); the other lanes hold
-//     zeros for good.  D then has a token's two group dots in different rows, each multiplied by
+//     0-15 (lanes kg < 2), rows 8-15 only positions 16-31 (lanes kg >= 2); the other lanes read
+//     zeros (from one 256-byte LDS region, so no lane is switched off around the reads).  D then has a token's two group dots in different rows, each multiplied by
 //     its own scale with one integer multiply-add; the two halves meet once per 16-row tile;
 //   * activations wait in LDS, token rows 32 bytes longer than K so that the 32 live lanes of an
 //     8-byte read fall in 64 distinct banks.
@@ -923,6 +923,49 @@ __device__ __forceinline__ Q6kMfW q6k_mf_load(const uchar* blk, uint kg) {
     return r;
 }
 
+// One super-block of a 16-row tile against P passes of 8 tokens: acc += sx * d * sum_g scale_g * idot_g.
+// xp[p]: the lane's 8 bytes of pass p's token row at this super-block (row n % 8, byte 8 kg) if its A
+// rows carry its positions, else 256 bytes of zeros; sx: the super-block's 16 token scales.
+template <int P>
+__device__ __forceinline__ void q6k_mf_superblock(const Q6kMfW& cur, const uchar* const (&xp)[P], uint kg, const float* sx16,
+                                                  float (&acc)[P][4]) {
+    const uint h = kg >> 1;                        // which 16-weight group of a quarter the lane's D rows hold
+    int isum[P][4];
+#pragma unroll
+    for (int p = 0; p < P; p++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) isum[p][v] = 0;
+#pragma unroll
+    for (int hf = 0; hf < 2; hf++) {
+        // scales 8 hf + 2 q + h, q = 0..3: bytes h, 2 + h of the half's two dwords
+        const uint s_lo = (hf ? cur.sc.z : cur.sc.x) >> (8u * h), s_hi = (hf ? cur.sc.w : cur.sc.y) >> (8u * h);
+        const int scl[4] = {(int)(signed char)s_lo, (int)(signed char)(s_lo >> 16), (int)(signed char)s_hi,
+                            (int)(signed char)(s_hi >> 16)};
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const u32x2_a2 ql = (q & 1) ? cur.lb[hf] : cur.la[hf];
+            const long B = q6k_signed8(ql.x, ql.y, cur.qh[hf].x, cur.qh[hf].y, q);
+#pragma unroll
+            for (int p = 0; p < P; p++) {
+                const long A = *(const long*)(xp[p] + 128u * hf + 32u * q);
+                const q6k_i4 zero = {0, 0, 0, 0};
+                const q6k_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B, zero, 0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < 4; v++) isum[p][v] += __mul24(scl[q], D[v]);
+            }
+        }
+    }
+    const float d = f16_bits_to_f32(cur.d16);
+#pragma unroll
+    for (int p = 0; p < P; p++) {
+        const float4 sx = *(const float4*)(sx16 + 8u * p + 4u * (kg & 1u));
+        acc[p][0] += sx.x * d * (float)isum[p][0];
+        acc[p][1] += sx.y * d * (float)isum[p][1];
+        acc[p][2] += sx.z * d * (float)isum[p][2];
+        acc[p][3] += sx.w * d * (float)isum[p][3];
+    }
+}
+
 template <int P>   // P passes of 8 tokens
 __device__ __forceinline__ void gemv_q8k_q6k_mf_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
                                                      const uchar* __restrict__ w, float* __restrict__ y,
@@ -930,6 +973,8 @@ __device__ __forceinline__ void gemv_q8k_q6k_mf_body(const signed char* __restri
     const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint nsb = K >> 8, S = K + 32u;
     float* lsx = (float*)(lds + (size_t)(8 * P) * S);       // [sb][16] token scales
+    uchar* zeros = (uchar*)(lsx + nsb * 16u);               // 256 bytes the idle half of the A lanes reads
+    if (tid < 64u) ((uint*)zeros)[tid] = 0u;
     // stage the tokens (rows past M are zero) and their scales
     const uint per_row = K >> 4;
     for (uint i = tid; i < (uint)(8 * P) * per_row; i += blockDim.x) {
@@ -945,8 +990,8 @@ __device__ __forceinline__ void gemv_q8k_q6k_mf_body(const signed char* __restri
     __syncthreads();
     const uint n = lane & 15u, kg = lane >> 4;
     const bool live = (n < 8u) == (kg < 2u);       // this lane's A rows carry its positions
-    const uint h = kg >> 1;                        // which 16-weight group of a quarter its D rows hold
-    const uchar* xa = lds + (size_t)(n & 7u) * S + 8u * kg;
+    const uchar* xa = live ? lds + (size_t)(n & 7u) * S + 8u * kg : zeros + 8u * kg;
+    const uint xstep = live ? 256u : 0u, xpass = live ? 8u * S : 0u;
     const uint tiles = (N + 15u) >> 4;
     const uint nwave = blockDim.x >> 6;
     for (uint tile = blockIdx.x * nwave + wave; tile < tiles; tile += gridDim.x * nwave) {
@@ -961,41 +1006,10 @@ __device__ __forceinline__ void gemv_q8k_q6k_mf_body(const signed char* __restri
         Q6kMfW cur = q6k_mf_load(wr, kg), nx = q6k_mf_load(wr + (size_t)min(1u, nsb - 1u) * Q6K_BYTES, kg);
         for (uint sb = 0; sb < nsb; sb++) {
             const Q6kMfW nx2 = q6k_mf_load(wr + (size_t)min(sb + 2u, nsb - 1u) * Q6K_BYTES, kg);
-            int isum[P][4];
+            const uchar* xp[P];
 #pragma unroll
-            for (int p = 0; p < P; p++)
-#pragma unroll
-                for (int v = 0; v < 4; v++) isum[p][v] = 0;
-#pragma unroll
-            for (int hf = 0; hf < 2; hf++) {
-                // scales 8 hf + 2 q + h, q = 0..3: bytes h, 2 + h of the half's two dwords
-                const uint s_lo = (hf ? cur.sc.z : cur.sc.x) >> (8u * h), s_hi = (hf ? cur.sc.w : cur.sc.y) >> (8u * h);
-                const int scl[4] = {(int)(signed char)s_lo, (int)(signed char)(s_lo >> 16), (int)(signed char)s_hi,
-                                    (int)(signed char)(s_hi >> 16)};
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const u32x2_a2 ql = (q & 1) ? cur.lb[hf] : cur.la[hf];
-                    const long B = q6k_signed8(ql.x, ql.y, cur.qh[hf].x, cur.qh[hf].y, q);
-#pragma unroll
-                    for (int p = 0; p < P; p++) {
-                        long A = 0;
-                        if (live) A = *(const long*)(xa + (size_t)(8 * p) * S + sb * 256u + 128u * hf + 32u * q);
-                        const q6k_i4 zero = {0, 0, 0, 0};
-                        const q6k_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B, zero, 0, 0, 0);
-#pragma unroll
-                        for (int v = 0; v < 4; v++) isum[p][v] += __mul24(scl[q], D[v]);
-                    }
-                }
-            }
-            const float d = f16_bits_to_f32(cur.d16);
-#pragma unroll
-            for (int p = 0; p < P; p++) {
-                const float4 sx = *(const float4*)(lsx + sb * 16u + 8u * p + 4u * (kg & 1u));
-                acc[p][0] += sx.x * d * (float)isum[p][0];
-                acc[p][1] += sx.y * d * (float)isum[p][1];
-                acc[p][2] += sx.z * d * (float)isum[p][2];
-                acc[p][3] += sx.w * d * (float)isum[p][3];
-            }
+            for (int p = 0; p < P; p++) xp[p] = xa + sb * xstep + p * xpass;
+            q6k_mf_superblock<P>(cur, xp, kg, lsx + sb * 16u, acc);
             cur = nx;
             nx = nx2;
         }
@@ -1020,4 +1034,134 @@ gemv_q8k_q6k_mf(const signed char* xq, const float* xs, const uchar* w, float* y
     __shared__ __attribute__((aligned(16))) uchar lds_mf[Q6K_MF_LDS];
     if (M <= 8) gemv_q8k_q6k_mf_body<1>(xq, xs, w, y, K, N, M, ACC, lds_mf);
     else gemv_q8k_q6k_mf_body<2>(xq, xs, w, y, K, N, M, ACC, lds_mf);
+}
+
+// ---- the same tile with the weights copied through LDS ----------------------------------------
+//   gemv_q8k_q6k_ml(xq, xs, w, y, K, N, M, ACC)    M <= 16, 512 threads, rows within 4 GiB,
+//       8 (K + 32) + K / 4 + 101632 <= 163840 (M <= 8)   16 (K + 32) + K / 4 + 67840 <= 163840 (M > 8)
+// gemv_q8k_q6k_mf is bound by its loads: 8-byte pieces of sixteen rows a row apart, three aligned
+// dwords fetched and shifted for each.  Here the memory system copies them: one
+// global_load_lds_dwordx4 moves four super-blocks (rows 4 i .. 4 i + 3 of the tile at one k),
+// fourteen lanes each, into 224-byte LDS slots, so every piece a lane then reads is 8-byte aligned
+// in LDS whatever its alignment in memory.  A super-block is 210 bytes: the fourteenth lane copies
+// its last 16 bytes (194 .. 209) rather than 208 .. 223, so nothing is read past the row and the
+// f16 scale sits at slot byte 222.  Each wave owns a ring of D units (one unit = the wave's 16 rows
+// at one super-block, four copies) and walks its tiles as one stream of units, D - 1 copies ahead
+// across tile borders; waves never wait for each other after the tokens are staged.
+// Slots of copy i start at 1024 i + 128 (i & 1): the sixteen rows then spread over all 64 banks.
+#define Q6K_ML_SLOT 224u
+#define Q6K_ML_UNIT 4224u
+#define Q6K_ML_LDS 163840u
+
+template <int P, int D>
+__device__ __forceinline__ void gemv_q8k_q6k_ml_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                     const uchar* __restrict__ w, float* __restrict__ y,
+                                                     uint K, uint N, uint M, uint ACC, uchar* lds, uint lds_addr) {
+    const uint tid = threadIdx.x, lane = tid & 63u;
+    const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint nsb = K >> 8, S = K + 32u;
+    const uint o_lsx = (uint)(8 * P) * S, o_zero = o_lsx + nsb * 64u, o_ring = o_zero + 256u + wave * ((uint)D * Q6K_ML_UNIT);
+    float* lsx = (float*)(lds + o_lsx);            // [sb][16] token scales
+    if (tid < 64u) ((uint*)(lds + o_zero))[tid] = 0u;   // what the idle half of the A lanes reads
+    const uint per_row = K >> 4;
+    for (uint i = tid; i < (uint)(8 * P) * per_row; i += blockDim.x) {
+        const uint t = i / per_row, o = (i - t * per_row) << 4;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (t < M) v = *(const uint4*)(xq + (size_t)t * K + o);
+        *(uint4*)(lds + (size_t)t * S + o) = v;
+    }
+    for (uint i = tid; i < nsb * 16u; i += blockDim.x) {
+        const uint sb = i >> 4, t = i & 15u;
+        lsx[i] = t < M ? xs[(size_t)t * nsb + sb] : 0.0f;
+    }
+    __syncthreads();                               // the only barrier; these loads are older than every copy
+    // wave ids interleave over the workgroups, so each CU gets its share of the waves with one tile more
+    const uint tiles = (N + 15u) >> 4, stride = gridDim.x * (blockDim.x >> 6), first = wave * gridDim.x + blockIdx.x;
+    const uint my_tiles = first < tiles ? (tiles - first + stride - 1u) / stride : 0u;
+    const uint total = my_tiles * nsb;             // units this wave walks
+    const uint row_bytes = nsb * Q6K_BYTES;
+    // the copy stream: lane -> slot cq of a copy, piece cpc of the slot
+    const uint cq = lane / 14u, cpc = lane - cq * 14u;
+    const bool con = lane < 56u;
+    const uint pc_off = cpc < 13u ? cpc * 16u : Q6K_BYTES - 16u;
+    uint i_off[4], iu = 0u, i_sb = 0u, i_tile = first, i_slot = 0u;
+    auto issue_next = [&]() {
+        if (i_sb == 0u) {
+#pragma unroll
+            for (uint i = 0; i < 4u; i++) i_off[i] = min(i_tile * 16u + 4u * i + cq, N - 1u) * row_bytes + pc_off;
+        }
+        const uint dst = lds_addr + o_ring + i_slot * Q6K_ML_UNIT;
+        if (con) {
+#pragma unroll
+            for (uint i = 0; i < 4u; i++) lds_dma16(w, i_off[i] + i_sb * Q6K_BYTES, dst + i * 1024u + (i & 1u) * 128u);
+        }
+        iu++;
+        i_slot = i_slot + 1u == (uint)D ? 0u : i_slot + 1u;
+        if (++i_sb == nsb) {
+            i_sb = 0u;
+            i_tile += stride;
+        }
+    };
+    for (uint k = 0; k + 1u < (uint)D; k++)
+        if (iu < total) issue_next();
+    const uint n = lane & 15u, kg = lane >> 4;
+    const bool live = (n < 8u) == (kg < 2u);
+    const uchar* xa = live ? lds + (size_t)(n & 7u) * S + 8u * kg : lds + o_zero + 8u * kg;
+    const uint xstep = live ? 256u : 0u, xpass = live ? 8u * S : 0u;
+    const uchar* rd = lds + o_ring + (n >> 2) * 1024u + ((n >> 2) & 1u) * 128u + (n & 3u) * Q6K_ML_SLOT;
+    float acc[P][4];
+#pragma unroll
+    for (int p = 0; p < P; p++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[p][v] = 0.0f;
+    uint c_sb = 0u, c_tile = first, c_slot = 0u;
+    for (uint u = 0; u < total; u++) {
+        if (iu < total) issue_next();              // unit u + D - 1, into the slot read during unit u - 1
+        vm_wait(min(total - 1u - u, (uint)D - 1u) * 4u);
+        const uchar* blk = rd + c_slot * Q6K_ML_UNIT;
+        c_slot = c_slot + 1u == (uint)D ? 0u : c_slot + 1u;
+        Q6kMfW cur;
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            const uint2 a = *(const uint2*)(blk + 64u * hf + 8u * kg), b = *(const uint2*)(blk + 64u * hf + 32u + 8u * kg),
+                        h = *(const uint2*)(blk + 128u + 32u * hf + 8u * kg);
+            cur.la[hf].x = a.x; cur.la[hf].y = a.y;
+            cur.lb[hf].x = b.x; cur.lb[hf].y = b.y;
+            cur.qh[hf].x = h.x; cur.qh[hf].y = h.y;
+        }
+        {
+            const uint4 sc = *(const uint4*)(blk + 192u);
+            cur.sc.x = sc.x; cur.sc.y = sc.y; cur.sc.z = sc.z; cur.sc.w = sc.w;
+            cur.d16 = *(const ushort*)(blk + Q6K_ML_SLOT - 2u);
+        }
+        const uchar* xp[P];
+#pragma unroll
+        for (int p = 0; p < P; p++) xp[p] = xa + c_sb * xstep + p * xpass;
+        q6k_mf_superblock<P>(cur, xp, kg, lsx + c_sb * 16u, acc);
+        if (++c_sb == nsb) {
+            // D rows 4 kg + v: token 4 (kg & 1) + v, first group in lanes kg < 2, second in kg >= 2
+#pragma unroll
+            for (int p = 0; p < P; p++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const float tot = acc[p][v] + __shfl_xor(acc[p][v], 32, 64);
+                    const uint t = 8u * p + 4u * kg + v;
+                    if (kg < 2u && t < M && c_tile * 16u + n < N) {
+                        float* o = y + (size_t)t * N + c_tile * 16u + n;
+                        *o = ACC ? *o + tot : tot;
+                    }
+                    acc[p][v] = 0.0f;
+                }
+            c_sb = 0u;
+            c_tile += stride;
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(512)
+gemv_q8k_q6k_ml(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    __shared__ __attribute__((aligned(16))) uchar lds_ml[Q6K_ML_LDS];
+    const uint lds_addr = (uint)(size_t)(__attribute__((address_space(3))) uchar*)lds_ml;
+    if (M <= 8) gemv_q8k_q6k_ml_body<1, 3>(xq, xs, w, y, K, N, M, ACC, lds_ml, lds_addr);
+    else gemv_q8k_q6k_ml_body<2, 2>(xq, xs, w, y, K, N, M, ACC, lds_ml, lds_addr);
 }

@@ -126,3 +126,34 @@ __device__ __forceinline__ void q4k_scale_min_pair(uint s0, uint s1, uint s2, ui
     sc = c < 2u ? sc_lo : sc_hi;
     mn = c < 2u ? mn_lo : mn_hi;
 }
+
+// ---- global -> LDS copies by the memory system ------------------------------------------------
+// One instruction moves 16 bytes per lane from base + voff to LDS bytes lds_addr + 16 lane .. (1 KB
+// per wave, contiguous in LDS whatever the global addresses; lds_addr is the same in every lane).
+// Completion is counted by vmcnt.
+__device__ __forceinline__ void lds_dma16(const void* base, uint voff, uint lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(base), "s"(__builtin_amdgcn_readfirstlane((int)lds_addr))
+                 : "memory");
+}
+// wait until at most `n` vector memory operations are outstanding (a count not listed waits for all)
+__device__ __forceinline__ void vm_wait(uint n) {
+    switch (n) {
+    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+    case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+    case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+    case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+    case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+    case 9: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
+    case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+    case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+    case 15: asm volatile("s_waitcnt vmcnt(15)" ::: "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+}
+

@@ -356,6 +356,12 @@ static int check_gemv_nat_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     return OJH_OK;
 }
 
+// LDS of gemv_q8k_q6k_ml: token rows, their scales, eight waves' copy rings (3 units deep up to 8 tokens, 2 beyond)
+uint64_t ojh_q6k_ml_lds(uint32_t K, uint32_t M) {
+    const uint64_t p = M <= 8 ? 1 : 2;
+    return 8 * p * ((uint64_t)K + 32) + K / 4 + 256 + 8 * (p == 1 ? 3 : 2) * 4224;
+}
+
 // gemv_q8k_<fmt>_m(xq, xs, w, y, K, N, M, ACC)
 static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                             const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -365,14 +371,25 @@ static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     if (rc) return rc;
     if (M == 0) return ojh_fail(OJH_ERR_ARG, "%s: M must be positive", s->name);
     const bool mx = s->rows_per_wave == 0;   // the LDS-staged, grid-stride entry
-    const bool mf = s->rows_per_wave < 0;    // the same on the int8 matrix cores
-    if ((rc = check_block(block, mx || mf ? 256 : 0))) return rc;
+    const bool mf = s->rows_per_wave == -1;  // the same on the int8 matrix cores
+    const bool ml = s->rows_per_wave == -2;  // ... with the rows copied through LDS
+    if (ml) {   // one to eight waves, each with its own copy ring
+        if (block[1] != 1 || block[2] != 1 || !block[0] || block[0] % 64 || block[0] > 512)
+            return ojh_fail(OJH_ERR_ARG, "%s: block must be [64 .. 512 in whole waves,1,1], got [%u,%u,%u]", s->name, block[0], block[1], block[2]);
+    } else if ((rc = check_block(block, mx || mf ? 256 : 0))) return rc;
     if (grid[1] != 1 || grid[2] != 1 || !grid[0]) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1], x > 0", s->name);
     if (mf) {
-        const uint64_t lds = (uint64_t)(M <= 8 ? 8 : 16) * (K + 32) + K / 4;
+        const uint64_t lds = (uint64_t)(M <= 8 ? 8 : 16) * (K + 32) + K / 4 + 256;
         if (M > 16 || lds > 69632)
             return ojh_fail(OJH_ERR_ARG, "%s: M=%u tokens of K=%u do not fit its 68 KB of LDS (M <= 16, %llu bytes needed)",
                             s->name, M, K, (unsigned long long)lds);
+    } else if (ml) {
+        const uint64_t lds = ojh_q6k_ml_lds(K, M);
+        if (M > 16 || lds > 163840)
+            return ojh_fail(OJH_ERR_ARG, "%s: M=%u tokens of K=%u do not fit its 160 KB of LDS (M <= 16, %llu bytes needed)",
+                            s->name, M, K, (unsigned long long)lds);
+        if ((uint64_t)N * (K / 256) * 210 > 0xFFFFFFFFull)
+            return ojh_fail(OJH_ERR_ARG, "%s: %u rows of K=%u pass 4 GiB, the reach of its 32-bit row offsets", s->name, N, K);
     } else if (mx) {
         if (M > 16 || (uint64_t)M * ((K + 4095) / 4096) > 19)
             return ojh_fail(OJH_ERR_ARG, "%s: M=%u tokens of K=%u do not fit its 80 KB of LDS (M <= 16, M*ceil(K/4096) <= 19)",
@@ -793,6 +810,16 @@ static int shape_mf(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, ui
     block[1] = block[2] = 1;
     return OJH_OK;
 }
+// one 512-thread workgroup per CU (all of its LDS), 16-row tiles grid-stride over the waves
+static int shape_ml(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t N, uint32_t,
+                    uint32_t grid[3], uint32_t block[3]) {
+    uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, wgs = (N + 127) / 128;
+    grid[0] = wgs < cus ? wgs : cus;
+    grid[1] = grid[2] = 1;
+    block[0] = 512;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
 static int shape_rows(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t,
                       uint32_t grid[3], uint32_t block[3]) {
     uint32_t rows_per_block = 4u * (uint32_t)s->rows_per_wave;
@@ -868,6 +895,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(q + "_m", "gemv_q8k", 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
         if (f.type == OJH_Q6_K) add(q + "_mx", "gemv_q8k", 4, 4, f.type, 0, check_gemv_q8k_m, shape_mx);
         if (f.type == OJH_Q6_K) add(q + "_mf", "gemv_q8k", 4, 4, f.type, -1, check_gemv_q8k_m, shape_mf);
+        if (f.type == OJH_Q6_K) add(q + "_ml", "gemv_q8k", 4, 4, f.type, -2, check_gemv_q8k_m, shape_ml);
         if (f.type == OJH_Q6_K) add(q + "_px", "gemv_q8k", 4, 2, f.type, 2, check_gemv_q8k_px, shape_px);
         if (f.type == OJH_Q4_K) {
             std::string fq = "gemv_fq8k_" + t;

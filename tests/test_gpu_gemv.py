@@ -401,6 +401,42 @@ def test_q6k_tokens_on_the_int8_matrix_cores(gpu, orc, pkg, m, n, k, accum):
         gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_mf", [(xq, 0), (xs, 0), (wd, 0), (y2, 0)], [k, n, 17, 0], [8, 1, 1], [256, 1, 1])
 
 
+@pytest.mark.parametrize("m,n,k,accum,grid_x", [(4, 50, 256, False, None), (8, 130, 4096, True, 3), (9, 301, 4096, False, 2),
+                                                (16, 1000, 4096, False, 7), (16, 17, 512, True, None),
+                                                (3, 4099, 2560, False, None), (8, 77, 7168, True, 1), (12, 333, 5632, False, 1)])
+def test_q6k_tokens_with_rows_copied_through_lds(gpu, orc, pkg, m, n, k, accum, grid_x):
+    """`gemv_q8k_q6k_ml`: the matrix-core tile with each wave's rows copied global -> LDS a
+    super-block at a time.  Against matvec_kq per token and, bit for bit, the direct-load entry on
+    the same quantized activations (the same arithmetic on the same bytes).  Small grids make a
+    wave walk many tiles, so its copy ring wraps and runs ahead across tile borders; the last rows
+    of the weights end exactly at the end of their buffer."""
+    w = pkg.synth.q6k_weights(n, k, "ml", n, k)
+    x = pkg.synth.normal_f32(m * k, "ml", "x", m, k).reshape(m, k)
+    y0 = pkg.synth.normal_f32(m * n, "ml", "y0").reshape(m, n) if accum else np.zeros((m, n), np.float32)
+    want = np.stack([orc.matvec_kq(w, Q6_K, n, k, x[t]) for t in range(m)])
+    gpu.ensure_family("gemv_q8k")
+    nsb = k // 256
+    xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
+    gpu.quant_q8k(gpu.upload(x), m, k, xq, xs)
+    wd = gpu.upload_bytes(w)
+    outs = {}
+    mf_fits = (8 if m <= 8 else 16) * (k + 32) + k // 4 + 256 <= 69632
+    for name in ("gemv_q8k_q6k_ml", "gemv_q8k_q6k_mf") if mf_fits else ("gemv_q8k_q6k_ml",):
+        grid, block = gpu.launch_shape(name, k, n, m)
+        if grid_x and name.endswith("ml"):
+            grid = [grid_x, 1, 1]
+        yd = gpu.upload(np.concatenate([y0.ravel(), np.full(8, 4242.5, np.float32)]))
+        gpu.dispatch(gpu.begin(), name, [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], [k, n, m, int(accum)], grid, block)
+        got = gpu.read(yd, m * n + 8)
+        assert np.all(got[m * n:] == 4242.5), "wrote past the last token"
+        outs[name] = got[:m * n].reshape(m, n) - y0
+    assert peak_err(outs["gemv_q8k_q6k_ml"], want) <= TOL_Q8K_SEEN
+    if mf_fits:
+        assert np.array_equal(outs["gemv_q8k_q6k_ml"], outs["gemv_q8k_q6k_mf"])
+    with pytest.raises(pkg.OjasHipError, match="do not fit"):
+        gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_ml", [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], [k, n, 17, 0], [8, 1, 1], [512, 1, 1])
+
+
 @pytest.mark.parametrize("n,k", [(33000, 256), (40001, 2560), (32768, 8192)])
 def test_q6k_head_form_keeps_activations_in_registers(gpu, orc, pkg, n, k):
     """From 32768 rows a Q6_K matvec runs grid-stride with the activations in registers: the lane
