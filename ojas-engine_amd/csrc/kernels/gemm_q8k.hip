@@ -244,3 +244,149 @@ gemm_q8k_q4k_mf(const signed char* xq, const float* xs, const uchar* w, float* y
     else if (left <= 32u) gemm_q8k_q4k_mf_body<2, 1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
     else gemm_q8k_q4k_mf_body<4, 1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
 }
+
+// ---- up to 16 tokens, rows copied through LDS --------------------------------------------------
+//   gemm_q8k_q4k_ml(xq, xs, w, y, K, N, M, ACC)   M <= 16, block 64 .. 512, w 16-byte aligned, rows within 4 GiB,
+//                                                 16 (K + 32) + 5 K / 4 + 73728 <= 163840
+// On a long matrix (an output head) and few tokens gemm_q8k_q4k_mf is bound by the address
+// path of its loads (8-byte pieces of sixteen rows 144 K / 256 bytes apart: the unit that walks
+// them is busy 85 % of the launch).  Here the memory system copies the rows instead: a wave owns
+// 16-row tiles and a ring of four units in LDS (one unit = its 16 rows at one super-block,
+// 2304 bytes, three global_load_lds_dwordx4 of nine lanes per row), walks its tiles as one stream
+// of units with the copies three units ahead across tile borders, and never waits for another
+// wave once the tokens are staged.  Rows land 144 bytes apart: 36 n mod 64 is a different multiple
+// of four for each of the sixteen rows, so header and code reads spread evenly over the banks.
+// The arithmetic per super-block is gemm_q8k_q4k_mf's; super-blocks are added in order (its
+// RW = 4 form: the same bits).
+#define GQL_UNIT 2304u
+#define GQL_DEPTH 4u
+#define GQL_LDS 163840u
+
+extern "C" __global__ void __launch_bounds__(512)
+gemm_q8k_q4k_ml(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    __shared__ __attribute__((aligned(16))) uchar lds[GQL_LDS];
+    const uint lds_addr = (uint)(size_t)(__attribute__((address_space(3))) uchar*)lds;
+    const uint tid = threadIdx.x, lane = tid & 63u;
+    const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint nsb = K >> 8, S = K + 32u;
+    const uint o_lsx = 16u * S, o_lbq = o_lsx + nsb * 64u, o_ring = o_lbq + nsb * 256u + wave * (GQL_DEPTH * GQL_UNIT);
+    float* lsx = (float*)(lds + o_lsx);            // [sb][16] token scales
+    uchar* lbq = lds + o_lbq;                      // [sb][16][16]: lo_0..7, hi_0..7 of the bsums
+    const uint per_row = K >> 4;
+    for (uint i = tid; i < 16u * per_row; i += blockDim.x) {
+        const uint t = i / per_row, o = (i - t * per_row) << 4;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (t < M) v = *(const uint4*)(xq + (size_t)t * K + o);
+        *(uint4*)(lds + (size_t)t * S + o) = v;
+    }
+    for (uint i = tid; i < nsb * 16u; i += blockDim.x) {
+        const uint sb = i >> 4, t = i & 15u;
+        lsx[i] = t < M ? xs[(size_t)t * nsb + sb] : 0.0f;
+    }
+    __syncthreads();
+    // bsum of every (token, sub-block), split into int8 parts: 64 * hi + lo
+    for (uint i = tid; i < nsb * 128u; i += blockDim.x) {
+        const uint jj = i & 7u, t = (i >> 3) & 15u, s = i >> 7;
+        const uint4* px = (const uint4*)(lds + (size_t)t * S + s * 256u + jj * 32u);
+        const uint4 a = px[0], b = px[1];
+        int bs = dot4_i8(a.x, 0x01010101u, 0);
+        bs = dot4_i8(a.y, 0x01010101u, bs); bs = dot4_i8(a.z, 0x01010101u, bs); bs = dot4_i8(a.w, 0x01010101u, bs);
+        bs = dot4_i8(b.x, 0x01010101u, bs); bs = dot4_i8(b.y, 0x01010101u, bs);
+        bs = dot4_i8(b.z, 0x01010101u, bs); bs = dot4_i8(b.w, 0x01010101u, bs);
+        uchar* o = lbq + ((size_t)s * 16u + t) * 16u;
+        o[jj] = (uchar)(bs & 63);
+        o[8u + jj] = (uchar)(bs >> 6);
+    }
+    __syncthreads();                               // the last barrier; every load so far is older than the copies
+    // wave ids interleave over the workgroups, so each CU gets its share of the waves with one tile more
+    const uint tiles = (N + 15u) >> 4, stride = gridDim.x * (blockDim.x >> 6), first = wave * gridDim.x + blockIdx.x;
+    const uint my_tiles = first < tiles ? (tiles - first + stride - 1u) / stride : 0u;
+    const uint total = my_tiles * nsb;             // units this wave walks
+    const uint row_bytes = nsb * Q4K_BYTES;
+    // the copy stream: nine lanes per row, seven rows per copy (rows 14 and 15 in the third)
+    const uint cq = lane / 9u, cpc = lane - cq * 9u;
+    uint i_off[3], iu = 0u, i_sb = 0u, i_tile = first, i_slot = 0u;
+    auto issue_next = [&]() {
+        if (i_sb == 0u) {
+#pragma unroll
+            for (uint i = 0; i < 3u; i++) i_off[i] = min(i_tile * 16u + min(7u * i + cq, 15u), N - 1u) * row_bytes + cpc * 16u;
+        }
+        const uint dst = lds_addr + o_ring + i_slot * GQL_UNIT;
+        if (lane < 63u) {
+            lds_dma16(w, i_off[0] + i_sb * Q4K_BYTES, dst);
+            lds_dma16(w, i_off[1] + i_sb * Q4K_BYTES, dst + 1008u);
+        }
+        if (lane < 18u) lds_dma16(w, i_off[2] + i_sb * Q4K_BYTES, dst + 2016u);
+        iu++;
+        i_slot = i_slot + 1u == GQL_DEPTH ? 0u : i_slot + 1u;
+        if (++i_sb == nsb) {
+            i_sb = 0u;
+            i_tile += stride;
+        }
+    };
+    for (uint k = 0; k + 1u < GQL_DEPTH; k++)
+        if (iu < total) issue_next();
+    const uint n = lane & 15u, kg = lane >> 4;
+    const uchar* xa = lds + (size_t)n * S + 8u * kg;
+    const uchar* rd = lds + o_ring + n * Q4K_BYTES;
+    const gq_i4 zero = {0, 0, 0, 0};
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    uint c_sb = 0u, c_tile = first, c_slot = 0u;
+    for (uint u = 0; u < total; u++) {
+        if (iu < total) issue_next();              // unit u + 3, into the slot read during unit u - 1
+        vm_wait(min(total - 1u - u, GQL_DEPTH - 1u) * 3u);
+        const uchar* blk = rd + c_slot * GQL_UNIT;
+        c_slot = c_slot + 1u == GQL_DEPTH ? 0u : c_slot + 1u;
+        GqW cur;
+        cur.hdr = *(const uint4*)blk;
+#pragma unroll
+        for (int c = 0; c < 4; c++) cur.q[c] = *(const uint2*)(blk + 16u + 32u * c + 8u * kg);
+        const float d = f16_bits_to_f32(cur.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
+        int sc[8];
+        long B[8], Bm = 0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            uint a, b;
+            q4k_scale_min_pair(cur.hdr.y, cur.hdr.z, cur.hdr.w, (uint)c, a, b);
+            sc[2 * c] = (int)(a & 0xFFu); sc[2 * c + 1] = (int)(a >> 8);
+            Bm |= (long)(unsigned long)(b & 0xFFFFu) << (16 * c);    // mins 2c, 2c + 1 -> bytes 2c, 2c + 1
+            B[2 * c] = gq_pack(cur.q[c].x & 0x0F0F0F0Fu, cur.q[c].y & 0x0F0F0F0Fu);
+            B[2 * c + 1] = gq_pack((cur.q[c].x >> 4) & 0x0F0F0F0Fu, (cur.q[c].y >> 4) & 0x0F0F0F0Fu);
+        }
+        if (kg != 0u) Bm = 0;                                        // only positions 0..7 carry mins
+        int isum[4] = {0, 0, 0, 0};
+        const uchar* xp = xa + c_sb * 256u;
+#pragma unroll
+        for (int jj = 0; jj < 8; jj++) {
+            const long A = *(const long*)(xp + 32 * jj);
+            const gq_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B[jj], zero, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 4; v++) isum[v] += __mul24(sc[jj], D[v]);
+        }
+        // token n: its eight lo parts, then its eight hi parts (lanes kg = 0 only)
+        const uchar* pq = lbq + ((size_t)c_sb * 16u + n) * 16u;
+        long Alo = 0, Ahi = 0;
+        if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
+        const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
+        const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
+        const float4 sx = *(const float4*)(lsx + c_sb * 16u + 4u * kg);
+        acc[0] += sx.x * (d * (float)isum[0] - dmin * (float)(64 * Dhi[0] + Dlo[0]));
+        acc[1] += sx.y * (d * (float)isum[1] - dmin * (float)(64 * Dhi[1] + Dlo[1]));
+        acc[2] += sx.z * (d * (float)isum[2] - dmin * (float)(64 * Dhi[2] + Dlo[2]));
+        acc[3] += sx.w * (d * (float)isum[3] - dmin * (float)(64 * Dhi[3] + Dlo[3]));
+        if (++c_sb == nsb) {
+            const uint r_out = c_tile * 16u + n;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const uint t = 4u * kg + v;
+                if (t < M && r_out < N) {
+                    float* o = y + (size_t)t * N + r_out;
+                    *o = ACC ? *o + acc[v] : acc[v];
+                }
+                acc[v] = 0.0f;
+            }
+            c_sb = 0u;
+            c_tile += stride;
+        }
+    }
+}

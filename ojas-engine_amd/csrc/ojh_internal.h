@@ -66,6 +66,7 @@ struct ojh_device {
     int q6k_ml = 1;              // OJAS_HIP_Q6K_ML: 0 = keep those rows on direct loads (gemv_q8k_q6k_mf)
     uint32_t px_bpc = 0;         // OJAS_HIP_PX_BPC: workgroups per CU for the grid-stride head matvec (0: 8)
     int px = 1;                  // OJAS_HIP_PX: 0 = never take it
+    uint32_t q4k_ml_min_m = 2;   // OJAS_HIP_Q4K_ML_MIN_M: tokens from which long Q4_K matrices (32768 rows or more) take the LDS-copy form (0: never)
     uint32_t q4k_mf_min_m = 5;   // OJAS_HIP_Q4K_MF_MIN_M: tokens from which Q4_K rows go to the int8 matrix cores
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
                                  // 3 = per-assignment decode form always
@@ -119,5 +120,6 @@ int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **o
 int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptrs,
                const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);
 void ojh_gemm_q8k_tiles(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M, uint32_t *rw, uint32_t *rt);   // row tiles per workgroup / per wave of gemm_q8k_q4k_mf
+uint64_t ojh_gemm_q8k_ml_lds(uint32_t K);           // LDS bytes of gemm_q8k_q4k_ml (ojh_manifest.cpp)
 uint64_t ojh_q6k_ml_lds(uint32_t K, uint32_t M);   // LDS bytes of gemv_q8k_q6k_ml (ojh_manifest.cpp)
 uint32_t ojh_q80_lds_kc(uint32_t K);   // chunks of K for gemv_nat_q80_lds, 0 if none (ojh_manifest.cpp)

@@ -78,6 +78,7 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_Q80_LDS_MIN_N")) d->q80_lds_min_n = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_Q80_LDS_BPC")) d->q80_lds_bpc = (uint32_t)std::max(0, atoi(r));
     if (const char *r = getenv("OJAS_HIP_Q6K_MF_MIN_M")) d->q6k_mf_min_m = (uint32_t)atoi(r);
+    if (const char *r = getenv("OJAS_HIP_Q4K_ML_MIN_M")) d->q4k_ml_min_m = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_Q6K_ML")) d->q6k_ml = atoi(r);
     if (const char *r = getenv("OJAS_HIP_Q6K_ML_MIN_M")) d->q6k_ml_min_m = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_PX_BPC")) d->px_bpc = (uint32_t)std::max(0, atoi(r));

@@ -77,6 +77,41 @@ def test_every_row_tiling_and_the_integer_dot_kernel_agree(gpu, orc, pkg, m, n, 
                      [256, 1, 1])
 
 
+@pytest.mark.parametrize("m,n,k,accum,grid_x,block_x", [(2, 50, 256, False, None, 512), (16, 130, 4096, True, 3, 512),
+                                                        (9, 301, 4096, False, 2, 256), (16, 1000, 5120, False, 7, 512),
+                                                        (1, 17, 512, True, None, 64), (5, 4099, 2560, False, None, 512),
+                                                        (8, 77, 1024, True, 1, 128)])
+def test_rows_copied_through_lds_by_name(gpu, orc, pkg, m, n, k, accum, grid_x, block_x):
+    """`gemm_q8k_q4k_ml`, up to 16 tokens: against matvec_kq per token and, bit for bit, against
+    `gemm_q8k_q4k_mf` with four row tiles per workgroup (no wave splits K there either, so the same
+    sums in the same order).  Small grids make a wave walk many tiles: its copy ring wraps and runs
+    ahead across tile borders; the last row ends exactly at the end of the weight buffer."""
+    w, x = _case(pkg, m, n, k, "ml")
+    y0 = pkg.synth.normal_f32(m * n, "gq", "ml-y0", m, n).reshape(m, n) if accum else np.zeros((m, n), np.float32)
+    want = np.stack([orc.matvec_kq(w, Q4_K, n, k, x[t]) for t in range(m)])
+    gpu.ensure_family("gemm_q8k")
+    nsb = k // 256
+    xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
+    gpu.quant_q8k(gpu.upload(x), m, k, xq, xs)
+    wd = gpu.upload_bytes(w)
+    grid, block = gpu.launch_shape("gemm_q8k_q4k_ml", k, n, m)
+    assert block == [512, 1, 1]
+    grid, block = [grid_x or grid[0], 1, 1], [block_x, 1, 1]
+    yd = gpu.upload(np.concatenate([y0.ravel(), np.full(8, 4242.5, np.float32)]))
+    gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_ml", [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], [k, n, m, int(accum)], grid, block)
+    got = gpu.read(yd, m * n + 8)
+    assert np.all(got[m * n:] == 4242.5), "wrote past the last token"
+    got = got[:m * n].reshape(m, n) - y0
+    assert peak_err(got, want) <= TOL_SEEN
+    y2 = gpu.upload(y0)
+    gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (y2, 0)], [k, n, m, int(accum), 4, 1],
+                 [(n + 63) // 64, 1, 1], [256, 1, 1])
+    assert np.array_equal(got, gpu.read(y2, m * n).reshape(m, n) - y0)
+    for consts, what in (([k, n, 17, 0], "do not fit"), ([8192, n, 4, 0], "do not fit")):
+        with pytest.raises(pkg.OjasHipError, match=what):
+            gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_ml", [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], consts, [8, 1, 1], [512, 1, 1])
+
+
 def test_a_token_does_not_depend_on_its_batch(gpu, pkg):
     """The same tokens rolled by 37 positions: every output bit for bit, moved."""
     m, n, k = 200, 512, 4096
