@@ -923,6 +923,27 @@ __device__ __forceinline__ Q6kMfW q6k_mf_load(const uchar* blk, uint kg) {
     return r;
 }
 
+// Token rows 0 .. rows - 1 (K int8 each, zeros from row M on) into LDS rows S bytes apart: 16 bytes per
+// thread and step, eight loads in flight before the first store (one load, one store, one wait per
+// step is a chain of cache latencies: fourteen of them for 8 tokens of K = 14336 and 512 threads).
+__device__ __forceinline__ void q8k_stage_tokens(uchar* lds, const signed char* __restrict__ xq, uint K, uint S, uint M, uint rows) {
+    const uint per_row = K >> 4, total = rows * per_row, nt = blockDim.x;
+    for (uint i0 = threadIdx.x; i0 < total; i0 += 8u * nt) {
+        uint4 v[8];
+        uint dst[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const uint i = i0 + (uint)u * nt, t = i / per_row, o = (i - t * per_row) << 4;
+            v[u] = make_uint4(0u, 0u, 0u, 0u);
+            dst[u] = t * S + o;
+            if (i < total && t < M) v[u] = *(const uint4*)(xq + (size_t)t * K + o);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (i0 + (uint)u * nt < total) *(uint4*)(lds + dst[u]) = v[u];
+    }
+}
+
 // One super-block of a 16-row tile against P passes of 8 tokens: acc += sx * d * sum_g scale_g * idot_g.
 // xp[p]: the lane's 8 bytes of pass p's token row at this super-block (row n % 8, byte 8 kg) if its A
 // rows carry its positions, else 256 bytes of zeros; sx: the super-block's 16 token scales.
@@ -976,13 +997,7 @@ __device__ __forceinline__ void gemv_q8k_q6k_mf_body(const signed char* __restri
     uchar* zeros = (uchar*)(lsx + nsb * 16u);               // 256 bytes the idle half of the A lanes reads
     if (tid < 64u) ((uint*)zeros)[tid] = 0u;
     // stage the tokens (rows past M are zero) and their scales
-    const uint per_row = K >> 4;
-    for (uint i = tid; i < (uint)(8 * P) * per_row; i += blockDim.x) {
-        const uint t = i / per_row, o = (i - t * per_row) << 4;
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (t < M) v = *(const uint4*)(xq + (size_t)t * K + o);
-        *(uint4*)(lds + (size_t)t * S + o) = v;
-    }
+    q8k_stage_tokens(lds, xq, K, S, M, (uint)(8 * P));
     for (uint i = tid; i < nsb * 16u; i += blockDim.x) {
         const uint sb = i >> 4, t = i & 15u;
         lsx[i] = t < M ? xs[(size_t)t * nsb + sb] : 0.0f;
@@ -1036,6 +1051,83 @@ gemv_q8k_q6k_mf(const signed char* xq, const float* xs, const uchar* w, float* y
     else gemv_q8k_q6k_mf_body<2>(xq, xs, w, y, K, N, M, ACC, lds_mf);
 }
 
+// ---- the same tile on few rows: its super-blocks split over the workgroup's waves --------------
+//   gemv_q8k_q6k_mk(xq, xs, w, y, K, N, M, ACC)   M <= 16, block 512, 8 P (K + 32) + K / 4 + 256 + 4096 P <= 163840
+// A projection of a few thousand rows has fewer 16-row tiles than the GPU has waves, and a wave
+// that walks a whole row of K = 14336 alone is a chain of 56 dependent steps.  Here a workgroup
+// owns a tile: wave w takes super-blocks w, w + 8, ...; the eight partial sums meet in LDS and are
+// added in wave order.  All of LDS belongs to the one workgroup of a CU, so 8 tokens of K up to
+// 18000 (16 of K up to 9000) wait there whole.
+#define Q6K_MK_LDS 163840u
+template <int P>
+__device__ __forceinline__ void gemv_q8k_q6k_mk_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                     const uchar* __restrict__ w, float* __restrict__ y,
+                                                     uint K, uint N, uint M, uint ACC, uchar* lds) {
+    const uint tid = threadIdx.x, lane = tid & 63u;
+    const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6)), nw = blockDim.x >> 6;
+    const uint nsb = K >> 8, S = K + 32u;
+    float* lsx = (float*)(lds + (size_t)(8 * P) * S);       // [sb][16] token scales
+    uchar* zeros = (uchar*)(lsx + nsb * 16u);               // 256 bytes the idle half of the A lanes reads
+    float* red = (float*)(zeros + 256u);                    // [wave][4 P][32]
+    if (tid < 64u) ((uint*)zeros)[tid] = 0u;
+    q8k_stage_tokens(lds, xq, K, S, M, (uint)(8 * P));
+    for (uint i = tid; i < nsb * 16u; i += blockDim.x) {
+        const uint sb = i >> 4, t = i & 15u;
+        lsx[i] = t < M ? xs[(size_t)t * nsb + sb] : 0.0f;
+    }
+    __syncthreads();
+    const uint n = lane & 15u, kg = lane >> 4;
+    const bool live = (n < 8u) == (kg < 2u);
+    const uchar* xa = live ? lds + (size_t)(n & 7u) * S + 8u * kg : zeros + 8u * kg;
+    const uint xstep = live ? 256u : 0u, xpass = live ? 8u * S : 0u;
+    const uint tiles = (N + 15u) >> 4;
+    for (uint tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const uint row = min(tile * 16u + n, N - 1u);
+        const uchar* wr = w + (size_t)row * nsb * Q6K_BYTES;
+        float acc[P][4];
+#pragma unroll
+        for (int p = 0; p < P; p++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[p][v] = 0.0f;
+        Q6kMfW cur = q6k_mf_load(wr + (size_t)min(wave, nsb - 1u) * Q6K_BYTES, kg);
+        for (uint sb = wave; sb < nsb; sb += nw) {
+            const Q6kMfW nx = q6k_mf_load(wr + (size_t)min(sb + nw, nsb - 1u) * Q6K_BYTES, kg);
+            const uchar* xp[P];
+#pragma unroll
+            for (int p = 0; p < P; p++) xp[p] = xa + sb * xstep + p * xpass;
+            q6k_mf_superblock<P>(cur, xp, kg, lsx + sb * 16u, acc);
+            cur = nx;
+        }
+        // D rows 4 kg + v: token 4 (kg & 1) + v, first group in lanes kg < 2, second in kg >= 2
+#pragma unroll
+        for (int p = 0; p < P; p++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float tot = acc[p][v] + __shfl_xor(acc[p][v], 32, 64);
+                if (lane < 32u) red[(wave * (uint)(4 * P) + (uint)(4 * p + v)) * 32u + lane] = tot;
+            }
+        __syncthreads();
+        if (tid < (uint)(128 * P)) {
+            const uint l32 = tid & 31u, pv = tid >> 5;
+            float sum = red[pv * 32u + l32];
+            for (uint w8 = 1; w8 < nw; w8++) sum += red[(w8 * (uint)(4 * P) + pv) * 32u + l32];
+            const uint nn = l32 & 15u, t = 8u * (pv >> 2) + 4u * (l32 >> 4) + (pv & 3u);
+            if (t < M && tile * 16u + nn < N) {
+                float* o = y + (size_t)t * N + tile * 16u + nn;
+                *o = ACC ? *o + sum : sum;
+            }
+        }
+        __syncthreads();                                    // before the next tile's partial sums
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(512)
+gemv_q8k_q6k_mk(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    __shared__ __attribute__((aligned(16))) uchar lds_mk[Q6K_MK_LDS];
+    if (M <= 8) gemv_q8k_q6k_mk_body<1>(xq, xs, w, y, K, N, M, ACC, lds_mk);
+    else gemv_q8k_q6k_mk_body<2>(xq, xs, w, y, K, N, M, ACC, lds_mk);
+}
+
 // ---- the same tile with the weights copied through LDS ----------------------------------------
 //   gemv_q8k_q6k_ml(xq, xs, w, y, K, N, M, ACC)    M <= 16, 512 threads, rows within 4 GiB,
 //       8 (K + 32) + K / 4 + 101632 <= 163840 (M <= 8)   16 (K + 32) + K / 4 + 67840 <= 163840 (M > 8)
@@ -1063,13 +1155,7 @@ __device__ __forceinline__ void gemv_q8k_q6k_ml_body(const signed char* __restri
     const uint o_lsx = (uint)(8 * P) * S, o_zero = o_lsx + nsb * 64u, o_ring = o_zero + 256u + wave * ((uint)D * Q6K_ML_UNIT);
     float* lsx = (float*)(lds + o_lsx);            // [sb][16] token scales
     if (tid < 64u) ((uint*)(lds + o_zero))[tid] = 0u;   // what the idle half of the A lanes reads
-    const uint per_row = K >> 4;
-    for (uint i = tid; i < (uint)(8 * P) * per_row; i += blockDim.x) {
-        const uint t = i / per_row, o = (i - t * per_row) << 4;
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (t < M) v = *(const uint4*)(xq + (size_t)t * K + o);
-        *(uint4*)(lds + (size_t)t * S + o) = v;
-    }
+    q8k_stage_tokens(lds, xq, K, S, M, (uint)(8 * P));
     for (uint i = tid; i < nsb * 16u; i += blockDim.x) {
         const uint sb = i >> 4, t = i & 15u;
         lsx[i] = t < M ? xs[(size_t)t * nsb + sb] : 0.0f;

@@ -61,7 +61,7 @@ struct ojh_device {
     int q80_lds = 1;             // OJAS_HIP_Q80_LDS: 0 = never take the LDS-staged Q8_0 matvec
     uint32_t q80_lds_min_n = 16384; // OJAS_HIP_Q80_LDS_MIN_N: rows from which it is taken (measured crossover)
     uint32_t q80_lds_bpc = 0;       // OJAS_HIP_Q80_LDS_BPC: workgroups per CU its grid is sized for (0: 2 or 3 by K chunking)
-    uint32_t q6k_mf_min_m = 8;   // OJAS_HIP_Q6K_MF_MIN_M: tokens from which Q6_K rows (8192 or more) go to the int8 matrix cores
+    uint32_t q6k_mf_min_m = 5;   // OJAS_HIP_Q6K_MF_MIN_M: tokens from which Q6_K rows (fewer than 32768) go to the int8 matrix cores
     uint32_t q6k_ml_min_m = 2;   // OJAS_HIP_Q6K_ML_MIN_M: ... with the rows copied through LDS (32768 rows or more)
     int q6k_ml = 1;              // OJAS_HIP_Q6K_ML: 0 = keep those rows on direct loads (gemv_q8k_q6k_mf)
     uint32_t px_bpc = 0;         // OJAS_HIP_PX_BPC: workgroups per CU for the grid-stride head matvec (0: 8)
@@ -121,5 +121,6 @@ int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptr
                const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);
 void ojh_gemm_q8k_tiles(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M, uint32_t *rw, uint32_t *rt);   // row tiles per workgroup / per wave of gemm_q8k_q4k_mf
 uint64_t ojh_gemm_q8k_ml_lds(uint32_t K);           // LDS bytes of gemm_q8k_q4k_ml (ojh_manifest.cpp)
+uint64_t ojh_q6k_mk_lds(uint32_t K, uint32_t M);   // LDS bytes of gemv_q8k_q6k_mk (ojh_manifest.cpp)
 uint64_t ojh_q6k_ml_lds(uint32_t K, uint32_t M);   // LDS bytes of gemv_q8k_q6k_ml (ojh_manifest.cpp)
 uint32_t ojh_q80_lds_kc(uint32_t K);   // chunks of K for gemv_nat_q80_lds, 0 if none (ojh_manifest.cpp)

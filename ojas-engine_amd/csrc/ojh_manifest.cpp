@@ -189,6 +189,16 @@ static int shape_gemm_q8k(const ojh_kernel_spec *, const ojh_device *dev, uint32
     return OJH_OK;
 }
 
+// one 512-thread workgroup per CU (all of its LDS), a 16-row tile per workgroup step
+static int shape_mk(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t N, uint32_t,
+                    uint32_t grid[3], uint32_t block[3]) {
+    uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, tiles = (N + 15) / 16;
+    grid[0] = tiles < cus ? tiles : cus;
+    grid[1] = grid[2] = 1;
+    block[0] = 512;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
 // one 512-thread workgroup per CU (all of its LDS), 16-row tiles grid-stride over the waves
 static int shape_ml(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t N, uint32_t,
                     uint32_t grid[3], uint32_t block[3]) {
@@ -394,6 +404,11 @@ static int check_gemv_nat_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     return OJH_OK;
 }
 
+// LDS of gemv_q8k_q6k_mk: token rows, their scales, a zero region, eight waves' partial sums
+uint64_t ojh_q6k_mk_lds(uint32_t K, uint32_t M) {
+    const uint64_t p = M <= 8 ? 1 : 2;
+    return 8 * p * ((uint64_t)K + 32) + K / 4 + 256 + 4096 * p;
+}
 // LDS of gemv_q8k_q6k_ml: token rows, their scales, eight waves' copy rings (3 units deep up to 8 tokens, 2 beyond)
 uint64_t ojh_q6k_ml_lds(uint32_t K, uint32_t M) {
     const uint64_t p = M <= 8 ? 1 : 2;
@@ -411,12 +426,18 @@ static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     const bool mx = s->rows_per_wave == 0;   // the LDS-staged, grid-stride entry
     const bool mf = s->rows_per_wave == -1;  // the same on the int8 matrix cores
     const bool ml = s->rows_per_wave == -2;  // ... with the rows copied through LDS
+    const bool mk = s->rows_per_wave == -3;  // ... with a tile's super-blocks split over eight waves
     if (ml) {   // one to eight waves, each with its own copy ring
         if (block[1] != 1 || block[2] != 1 || !block[0] || block[0] % 64 || block[0] > 512)
             return ojh_fail(OJH_ERR_ARG, "%s: block must be [64 .. 512 in whole waves,1,1], got [%u,%u,%u]", s->name, block[0], block[1], block[2]);
-    } else if ((rc = check_block(block, mx || mf ? 256 : 0))) return rc;
+    } else if ((rc = check_block(block, mk ? 512 : mx || mf ? 256 : 0))) return rc;
     if (grid[1] != 1 || grid[2] != 1 || !grid[0]) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1], x > 0", s->name);
-    if (mf) {
+    if (mk) {
+        const uint64_t lds = ojh_q6k_mk_lds(K, M);
+        if (M > 16 || lds > 163840)
+            return ojh_fail(OJH_ERR_ARG, "%s: M=%u tokens of K=%u do not fit its 160 KB of LDS (M <= 16, %llu bytes needed)",
+                            s->name, M, K, (unsigned long long)lds);
+    } else if (mf) {
         const uint64_t lds = (uint64_t)(M <= 8 ? 8 : 16) * (K + 32) + K / 4 + 256;
         if (M > 16 || lds > 69632)
             return ojh_fail(OJH_ERR_ARG, "%s: M=%u tokens of K=%u do not fit its 68 KB of LDS (M <= 16, %llu bytes needed)",
@@ -442,7 +463,7 @@ static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     align[1] = 4;
     align[2] = f->bytes % 16 ? 2 : 16;
     align[3] = 4;
-    if (mf) {                 // whole aligned dwords around every piece: the last one may end 2 bytes on
+    if (mf || mk) {           // whole aligned dwords around every piece: the last one may end 2 bytes on
         need[2] = (need[2] + 3) & ~(size_t)3;
         align[2] = 4;
     }
@@ -924,6 +945,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         if (f.type == OJH_Q6_K) add(q + "_mx", "gemv_q8k", 4, 4, f.type, 0, check_gemv_q8k_m, shape_mx);
         if (f.type == OJH_Q6_K) add(q + "_mf", "gemv_q8k", 4, 4, f.type, -1, check_gemv_q8k_m, shape_mf);
         if (f.type == OJH_Q6_K) add(q + "_ml", "gemv_q8k", 4, 4, f.type, -2, check_gemv_q8k_m, shape_ml);
+        if (f.type == OJH_Q6_K) add(q + "_mk", "gemv_q8k", 4, 4, f.type, -3, check_gemv_q8k_m, shape_mk);
         if (f.type == OJH_Q6_K) add(q + "_px", "gemv_q8k", 4, 2, f.type, 2, check_gemv_q8k_px, shape_px);
         if (f.type == OJH_Q4_K) {
             std::string fq = "gemv_fq8k_" + t;

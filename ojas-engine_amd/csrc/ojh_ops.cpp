@@ -193,24 +193,41 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
     }
     const size_t w_bytes = w->row_bytes * N;
     const bool dwords_ok = (uintptr_t)wp % 4 == 0 && (w_bytes % 4 == 0 || w->off + w_bytes + 2 <= w->raw->bytes);
-    // Q6_K rows against 2 .. 64 tokens on the int8 matrix cores (beyond 16 tokens as launches of 16:
+    // Q6_K rows against 2 .. 64 tokens on the int8 matrix cores (beyond 16 tokens as launches of 16 or 8:
     // each streams the rows once, which the per-token loop of the general entry does sixteen times
-    // over).  A wave walks a 16-row tile from end to end, so these want many tiles: measured on K = 4096,
-    //   rows copied through LDS (8 waves per CU busy from 32768 rows): ahead from 2 tokens there;
-    //   direct loads: ahead of the integer-dot entry from 8 tokens and 8192 rows;
-    //   the integer-dot entry (next) everywhere else it fits.
+    // over).  Three shapes of the same tile arithmetic, picked by what was measured on K = 4096 and 14336:
+    //   many rows (eight tiles per CU and wave, 32768 rows on this GPU): a wave per tile, rows copied
+    //     through LDS, ahead of everything from 2 tokens;
+    //   few rows (up to two tiles per CU, 8192 rows): a workgroup per tile, its waves splitting K, ahead of
+    //     the integer-dot entry from 5 tokens (from 3 when K is long) and the only one that holds 8 tokens
+    //     of K = 14336;
+    //   between: a wave per tile with direct loads, ahead of the integer-dot entry from 5 tokens.
     if (w->type == OJH_Q6_K && m >= 2 && m <= 64) {
         const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount, tiles = (N + 15) / 16;
-        const bool ml_fits = dev->q6k_ml && (uint64_t)w_bytes <= 0xFFFFFFFFull && ojh_q6k_ml_lds(K, m <= 8 ? m : 16) <= 163840;
+        const uint32_t mc16 = m <= 8 ? m : 16;
+        const bool ml_fits = dev->q6k_ml && (uint64_t)w_bytes <= 0xFFFFFFFFull && ojh_q6k_ml_lds(K, mc16) <= 163840;
         const bool mf_fits = dwords_ok && (uint64_t)(m <= 8 ? 8 : 16) * (K + 32) + K / 4 + 256 <= 69632;
+        const bool mk16 = dwords_ok && ojh_q6k_mk_lds(K, mc16) <= 163840, mk8 = dwords_ok && ojh_q6k_mk_lds(K, 8) <= 163840;
         const bool mx_fits = m <= 16 && (uint64_t)m * ((K + 4095) / 4096) <= 19;
         const char *entry = nullptr;
-        if (ml_fits && m >= dev->q6k_ml_min_m && (tiles >= 8 * cus || (!mx_fits && !mf_fits))) entry = "gemv_q8k_q6k_ml";
-        else if (mf_fits && ((m >= dev->q6k_mf_min_m && N >= 8192) || !mx_fits)) entry = "gemv_q8k_q6k_mf";
+        uint32_t step = 16;
+        if (ml_fits && m >= dev->q6k_ml_min_m && tiles >= 8 * cus) {
+            entry = "gemv_q8k_q6k_ml";
+        } else if (tiles <= 2 * cus && (mk16 || mk8) && (m >= dev->q6k_mf_min_m || (m >= 3 && K > 8192) || !mx_fits)) {
+            entry = "gemv_q8k_q6k_mk";
+            step = mk16 ? 16 : 8;
+        } else if (mf_fits && (m >= dev->q6k_mf_min_m || !mx_fits)) {
+            entry = "gemv_q8k_q6k_mf";
+        } else if (!mx_fits && (mk16 || mk8)) {
+            entry = "gemv_q8k_q6k_mk";
+            step = mk16 ? 16 : 8;
+        } else if (!mx_fits && ml_fits) {
+            entry = "gemv_q8k_q6k_ml";
+        }
         if (entry) {
             const size_t nsb = K / 256;
-            for (uint32_t t0 = 0; t0 < m; t0 += 16) {
-                const uint32_t mc = m - t0 < 16 ? m - t0 : 16;
+            for (uint32_t t0 = 0; t0 < m; t0 += step) {
+                const uint32_t mc = m - t0 < step ? m - t0 : step;
                 uint32_t sg[3], sb[3];
                 int rc = ojh_launch_shape(dev, entry, K, N, mc, sg, sb);
                 if (rc) return rc;

@@ -437,6 +437,40 @@ def test_q6k_tokens_with_rows_copied_through_lds(gpu, orc, pkg, m, n, k, accum, 
         gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_ml", [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], [k, n, 17, 0], [8, 1, 1], [512, 1, 1])
 
 
+@pytest.mark.parametrize("m,n,k,accum,grid_x", [(4, 50, 256, False, None), (8, 130, 4096, True, 3), (9, 301, 4096, False, None),
+                                                (16, 100, 8192, False, 2), (8, 33, 14336, True, None), (3, 4099, 2560, False, None)])
+def test_q6k_tokens_with_k_split_over_the_waves(gpu, orc, pkg, m, n, k, accum, grid_x):
+    """`gemv_q8k_q6k_mk`: a workgroup per 16-row tile, super-blocks dealt to its eight waves, partial
+    sums added in wave order.  Against matvec_kq per token; the router takes it for few rows."""
+    w = pkg.synth.q6k_weights(n, k, "mk", n, k)
+    x = pkg.synth.normal_f32(m * k, "mk", "x", m, k).reshape(m, k)
+    y0 = pkg.synth.normal_f32(m * n, "mk", "y0").reshape(m, n) if accum else np.zeros((m, n), np.float32)
+    want = np.stack([orc.matvec_kq(w, Q6_K, n, k, x[t]) for t in range(m)])
+    gpu.ensure_family("gemv_q8k")
+    nsb = k // 256
+    xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
+    gpu.quant_q8k(gpu.upload(x), m, k, xq, xs)
+    wd = gpu.upload_bytes(w)
+    grid, block = gpu.launch_shape("gemv_q8k_q6k_mk", k, n, m)
+    if grid_x:
+        grid = [grid_x, 1, 1]
+    yd = gpu.upload(np.concatenate([y0.ravel(), np.full(8, 4242.5, np.float32)]))
+    gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_mk", [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], [k, n, m, int(accum)], grid, block)
+    got = gpu.read(yd, m * n + 8)
+    assert np.all(got[m * n:] == 4242.5), "wrote past the last token"
+    assert peak_err(got[:m * n].reshape(m, n) - y0, want) <= TOL_Q8K_SEEN
+    # through the router (few rows: this entry from 5 tokens, or 3 of a long K), in chunks where 16 tokens do not fit
+    lin = gpu.lin(Q6_K, n, k, w)
+    for mm in (m, 2 * m + 1):
+        xx = np.concatenate([x, x[::-1], x[:1]])[:mm]
+        yr = gpu.alloc(mm * n)
+        gpu.mm(gpu.upload(xx), lin, yr, mm, act_mode=pkg.ACT_Q8K)
+        wantr = np.stack([orc.matvec_kq(w, Q6_K, n, k, xx[t]) for t in range(mm)])
+        assert peak_err(gpu.read(yr, mm * n).reshape(mm, n), wantr) <= TOL_Q8K_SEEN, mm
+    with pytest.raises(pkg.OjasHipError, match="do not fit"):
+        gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_mk", [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], [k, n, 17, 0], [8, 1, 1], [512, 1, 1])
+
+
 @pytest.mark.parametrize("n,k", [(33000, 256), (40001, 2560), (32768, 8192)])
 def test_q6k_head_form_keeps_activations_in_registers(gpu, orc, pkg, n, k):
     """From 32768 rows a Q6_K matvec runs grid-stride with the activations in registers: the lane
