@@ -245,9 +245,91 @@ gemm_q8k_q4k_mf(const signed char* xq, const float* xs, const uchar* w, float* y
     else gemm_q8k_q4k_mf_body<4, 1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
 }
 
+// One super-block of a 16-row tile against one pass of 16 tokens:
+//   acc[v] += sx * (d * sum_j sc_j idot_j - dmin * sum_j m_j bsum_j)   for token 4 kg + v, row n.
+// xp: the lane's 8 bytes of token n at this super-block (byte 8 kg); pq: token n's split sums
+// (eight lo parts, eight hi parts); sx16: the super-block's 16 token scales.
+__device__ __forceinline__ void gq_superblock(const GqW& cur, const uchar* xp, const uchar* pq, const float* sx16, uint kg,
+                                              float (&acc)[4]) {
+    const gq_i4 zero = {0, 0, 0, 0};
+    const float d = f16_bits_to_f32(cur.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
+    int sc[8];
+    long B[8], Bm = 0;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        uint a, b;
+        q4k_scale_min_pair(cur.hdr.y, cur.hdr.z, cur.hdr.w, (uint)c, a, b);
+        sc[2 * c] = (int)(a & 0xFFu); sc[2 * c + 1] = (int)(a >> 8);
+        Bm |= (long)(unsigned long)(b & 0xFFFFu) << (16 * c);    // mins 2c, 2c + 1 -> bytes 2c, 2c + 1
+        B[2 * c] = gq_pack(cur.q[c].x & 0x0F0F0F0Fu, cur.q[c].y & 0x0F0F0F0Fu);
+        B[2 * c + 1] = gq_pack((cur.q[c].x >> 4) & 0x0F0F0F0Fu, (cur.q[c].y >> 4) & 0x0F0F0F0Fu);
+    }
+    if (kg != 0u) Bm = 0;                                        // only positions 0..7 carry mins
+    int isum[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++) {
+        const long A = *(const long*)(xp + 32 * jj);
+        const gq_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B[jj], zero, 0, 0, 0);
+#pragma unroll
+        for (int v = 0; v < 4; v++) isum[v] += __mul24(sc[jj], D[v]);
+    }
+    long Alo = 0, Ahi = 0;
+    if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
+    const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
+    const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
+    const float4 sx = *(const float4*)(sx16 + 4u * kg);
+    acc[0] += sx.x * (d * (float)isum[0] - dmin * (float)(64 * Dhi[0] + Dlo[0]));
+    acc[1] += sx.y * (d * (float)isum[1] - dmin * (float)(64 * Dhi[1] + Dlo[1]));
+    acc[2] += sx.z * (d * (float)isum[2] - dmin * (float)(64 * Dhi[2] + Dlo[2]));
+    acc[3] += sx.w * (d * (float)isum[3] - dmin * (float)(64 * Dhi[3] + Dlo[3]));
+}
+
+// What the two entries below stage once per workgroup: token rows 0 .. M - 1 (S bytes apart, eight
+// loads in flight per thread), scales [sb][16] and split sums [sb][16][16] (zero from token M on).
+__device__ __forceinline__ void gq_stage16(uchar* lds, float* lsx, uchar* lbq, const signed char* __restrict__ xq,
+                                           const float* __restrict__ xs, uint K, uint S, uint M) {
+    const uint nsb = K >> 8, per_row = K >> 4, total = M * per_row, nt = blockDim.x, tid = threadIdx.x;
+    for (uint i0 = tid; i0 < total; i0 += 8u * nt) {
+        uint4 v[8];
+        uint dst[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const uint i = i0 + (uint)u * nt, t = i / per_row, o = (i - t * per_row) << 4;
+            v[u] = make_uint4(0u, 0u, 0u, 0u);
+            dst[u] = t * S + o;
+            if (i < total) v[u] = *(const uint4*)(xq + (size_t)t * K + o);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (i0 + (uint)u * nt < total) *(uint4*)(lds + dst[u]) = v[u];
+    }
+    for (uint i = tid; i < nsb * 16u; i += nt) {
+        const uint sb = i >> 4, t = i & 15u;
+        lsx[i] = t < M ? xs[(size_t)t * nsb + sb] : 0.0f;
+    }
+    __syncthreads();
+    // bsum of every (token, sub-block), split into int8 parts: 64 * hi + lo
+    for (uint i = tid; i < nsb * 128u; i += nt) {
+        const uint jj = i & 7u, t = (i >> 3) & 15u, s = i >> 7;
+        int bs = 0;
+        if (t < M) {
+            const uint4* px = (const uint4*)(lds + (size_t)t * S + s * 256u + jj * 32u);
+            const uint4 a = px[0], b = px[1];
+            bs = dot4_i8(a.x, 0x01010101u, 0);
+            bs = dot4_i8(a.y, 0x01010101u, bs); bs = dot4_i8(a.z, 0x01010101u, bs); bs = dot4_i8(a.w, 0x01010101u, bs);
+            bs = dot4_i8(b.x, 0x01010101u, bs); bs = dot4_i8(b.y, 0x01010101u, bs);
+            bs = dot4_i8(b.z, 0x01010101u, bs); bs = dot4_i8(b.w, 0x01010101u, bs);
+        }
+        uchar* o = lbq + ((size_t)s * 16u + t) * 16u;
+        o[jj] = (uchar)(bs & 63);
+        o[8u + jj] = (uchar)(bs >> 6);
+    }
+    __syncthreads();
+}
+
 // ---- up to 16 tokens, rows copied through LDS --------------------------------------------------
 //   gemm_q8k_q4k_ml(xq, xs, w, y, K, N, M, ACC)   M <= 16, block 64 .. 512, w 16-byte aligned, rows within 4 GiB,
-//                                                 16 (K + 32) + 5 K / 4 + 73728 <= 163840
+//                                                 16 (K + 32) + 5 K / 4 + 256 + 73728 <= 163840
 // On a long matrix (an output head) and few tokens gemm_q8k_q4k_mf is bound by the address
 // path of its loads (8-byte pieces of sixteen rows 144 K / 256 bytes apart: the unit that walks
 // them is busy 85 % of the launch).  Here the memory system copies the rows instead: a wave owns
@@ -269,35 +351,12 @@ gemm_q8k_q4k_ml(const signed char* xq, const float* xs, const uchar* w, float* y
     const uint tid = threadIdx.x, lane = tid & 63u;
     const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint nsb = K >> 8, S = K + 32u;
-    const uint o_lsx = 16u * S, o_lbq = o_lsx + nsb * 64u, o_ring = o_lbq + nsb * 256u + wave * (GQL_DEPTH * GQL_UNIT);
+    const uint o_lsx = 16u * S, o_lbq = o_lsx + nsb * 64u, o_zero = o_lbq + nsb * 256u;
+    const uint o_ring = o_zero + 256u + wave * (GQL_DEPTH * GQL_UNIT);
     float* lsx = (float*)(lds + o_lsx);            // [sb][16] token scales
     uchar* lbq = lds + o_lbq;                      // [sb][16][16]: lo_0..7, hi_0..7 of the bsums
-    const uint per_row = K >> 4;
-    for (uint i = tid; i < 16u * per_row; i += blockDim.x) {
-        const uint t = i / per_row, o = (i - t * per_row) << 4;
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (t < M) v = *(const uint4*)(xq + (size_t)t * K + o);
-        *(uint4*)(lds + (size_t)t * S + o) = v;
-    }
-    for (uint i = tid; i < nsb * 16u; i += blockDim.x) {
-        const uint sb = i >> 4, t = i & 15u;
-        lsx[i] = t < M ? xs[(size_t)t * nsb + sb] : 0.0f;
-    }
-    __syncthreads();
-    // bsum of every (token, sub-block), split into int8 parts: 64 * hi + lo
-    for (uint i = tid; i < nsb * 128u; i += blockDim.x) {
-        const uint jj = i & 7u, t = (i >> 3) & 15u, s = i >> 7;
-        const uint4* px = (const uint4*)(lds + (size_t)t * S + s * 256u + jj * 32u);
-        const uint4 a = px[0], b = px[1];
-        int bs = dot4_i8(a.x, 0x01010101u, 0);
-        bs = dot4_i8(a.y, 0x01010101u, bs); bs = dot4_i8(a.z, 0x01010101u, bs); bs = dot4_i8(a.w, 0x01010101u, bs);
-        bs = dot4_i8(b.x, 0x01010101u, bs); bs = dot4_i8(b.y, 0x01010101u, bs);
-        bs = dot4_i8(b.z, 0x01010101u, bs); bs = dot4_i8(b.w, 0x01010101u, bs);
-        uchar* o = lbq + ((size_t)s * 16u + t) * 16u;
-        o[jj] = (uchar)(bs & 63);
-        o[8u + jj] = (uchar)(bs >> 6);
-    }
-    __syncthreads();                               // the last barrier; every load so far is older than the copies
+    if (tid < 64u) ((uint*)(lds + o_zero))[tid] = 0u;   // what the A lanes of tokens past M read
+    gq_stage16(lds, lsx, lbq, xq, xs, K, S, M);    // (its last barrier: every load so far is older than the copies)
     // wave ids interleave over the workgroups, so each CU gets its share of the waves with one tile more
     const uint tiles = (N + 15u) >> 4, stride = gridDim.x * (blockDim.x >> 6), first = wave * gridDim.x + blockIdx.x;
     const uint my_tiles = first < tiles ? (tiles - first + stride - 1u) / stride : 0u;
@@ -327,9 +386,9 @@ gemm_q8k_q4k_ml(const signed char* xq, const float* xs, const uchar* w, float* y
     for (uint k = 0; k + 1u < GQL_DEPTH; k++)
         if (iu < total) issue_next();
     const uint n = lane & 15u, kg = lane >> 4;
-    const uchar* xa = lds + (size_t)n * S + 8u * kg;
+    const uchar* xa = n < M ? lds + (size_t)n * S + 8u * kg : lds + o_zero + 8u * kg;
+    const uint xstep = n < M ? 256u : 0u;
     const uchar* rd = lds + o_ring + n * Q4K_BYTES;
-    const gq_i4 zero = {0, 0, 0, 0};
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     uint c_sb = 0u, c_tile = first, c_slot = 0u;
     for (uint u = 0; u < total; u++) {
@@ -341,39 +400,7 @@ gemm_q8k_q4k_ml(const signed char* xq, const float* xs, const uchar* w, float* y
         cur.hdr = *(const uint4*)blk;
 #pragma unroll
         for (int c = 0; c < 4; c++) cur.q[c] = *(const uint2*)(blk + 16u + 32u * c + 8u * kg);
-        const float d = f16_bits_to_f32(cur.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
-        int sc[8];
-        long B[8], Bm = 0;
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            uint a, b;
-            q4k_scale_min_pair(cur.hdr.y, cur.hdr.z, cur.hdr.w, (uint)c, a, b);
-            sc[2 * c] = (int)(a & 0xFFu); sc[2 * c + 1] = (int)(a >> 8);
-            Bm |= (long)(unsigned long)(b & 0xFFFFu) << (16 * c);    // mins 2c, 2c + 1 -> bytes 2c, 2c + 1
-            B[2 * c] = gq_pack(cur.q[c].x & 0x0F0F0F0Fu, cur.q[c].y & 0x0F0F0F0Fu);
-            B[2 * c + 1] = gq_pack((cur.q[c].x >> 4) & 0x0F0F0F0Fu, (cur.q[c].y >> 4) & 0x0F0F0F0Fu);
-        }
-        if (kg != 0u) Bm = 0;                                        // only positions 0..7 carry mins
-        int isum[4] = {0, 0, 0, 0};
-        const uchar* xp = xa + c_sb * 256u;
-#pragma unroll
-        for (int jj = 0; jj < 8; jj++) {
-            const long A = *(const long*)(xp + 32 * jj);
-            const gq_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B[jj], zero, 0, 0, 0);
-#pragma unroll
-            for (int v = 0; v < 4; v++) isum[v] += __mul24(sc[jj], D[v]);
-        }
-        // token n: its eight lo parts, then its eight hi parts (lanes kg = 0 only)
-        const uchar* pq = lbq + ((size_t)c_sb * 16u + n) * 16u;
-        long Alo = 0, Ahi = 0;
-        if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
-        const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
-        const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
-        const float4 sx = *(const float4*)(lsx + c_sb * 16u + 4u * kg);
-        acc[0] += sx.x * (d * (float)isum[0] - dmin * (float)(64 * Dhi[0] + Dlo[0]));
-        acc[1] += sx.y * (d * (float)isum[1] - dmin * (float)(64 * Dhi[1] + Dlo[1]));
-        acc[2] += sx.z * (d * (float)isum[2] - dmin * (float)(64 * Dhi[2] + Dlo[2]));
-        acc[3] += sx.w * (d * (float)isum[3] - dmin * (float)(64 * Dhi[3] + Dlo[3]));
+        gq_superblock(cur, xa + c_sb * xstep, lbq + ((size_t)c_sb * 16u + n) * 16u, lsx + c_sb * 16u, kg, acc);
         if (++c_sb == nsb) {
             const uint r_out = c_tile * 16u + n;
 #pragma unroll
@@ -388,5 +415,56 @@ gemm_q8k_q4k_ml(const signed char* xq, const float* xs, const uchar* w, float* y
             c_sb = 0u;
             c_tile += stride;
         }
+    }
+}
+
+// ---- up to 16 tokens on few rows: a tile's super-blocks split over the workgroup's waves --------
+//   gemm_q8k_q4k_mk(xq, xs, w, y, K, N, M, ACC)   M <= 16, block 512, M (K + 32) + 5 K / 4 + 256 + 8192 <= 163840
+// A projection of a few thousand rows has fewer 16-row tiles than the GPU has waves.  Here a
+// workgroup owns a tile (tiles grid-stride): wave w takes super-blocks w, w + 8, ... against all the
+// tokens, and the eight partial sums meet in LDS, added in wave order.  The whole of LDS belongs to
+// the one workgroup of a CU, so the M tokens wait there whole (8 tokens of K = 14336); token rows
+// past M are one shared block of zeros.
+extern "C" __global__ void __launch_bounds__(512)
+gemm_q8k_q4k_mk(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    __shared__ __attribute__((aligned(16))) uchar lds[GQL_LDS];
+    const uint tid = threadIdx.x, lane = tid & 63u;
+    const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6)), nw = blockDim.x >> 6;
+    const uint nsb = K >> 8, S = K + 32u;
+    const uint o_lsx = M * S, o_lbq = o_lsx + nsb * 64u, o_zero = o_lbq + nsb * 256u, o_red = o_zero + 256u;
+    float* lsx = (float*)(lds + o_lsx);            // [sb][16] token scales
+    uchar* lbq = lds + o_lbq;                      // [sb][16][16]: lo_0..7, hi_0..7 of the bsums
+    float* red = (float*)(lds + o_red);            // [wave][4][64]
+    if (tid < 64u) ((uint*)(lds + o_zero))[tid] = 0u;
+    gq_stage16(lds, lsx, lbq, xq, xs, K, S, M);
+    const uint n = lane & 15u, kg = lane >> 4;
+    const uchar* xa = n < M ? lds + (size_t)n * S + 8u * kg : lds + o_zero + 8u * kg;
+    const uint xstep = n < M ? 256u : 0u;
+    const uint tiles = (N + 15u) >> 4;
+    for (uint tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const uint row = min(tile * 16u + n, N - 1u);
+        const uchar* wr = w + (size_t)row * nsb * Q4K_BYTES;
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        // (one super-block ahead; two ahead, and loads skipped rather than clamped past the slice, measured the same)
+        GqW cur = gq_load(wr + (size_t)min(wave, nsb - 1u) * Q4K_BYTES, kg);
+        for (uint sb = wave; sb < nsb; sb += nw) {
+            const GqW nx = gq_load(wr + (size_t)min(sb + nw, nsb - 1u) * Q4K_BYTES, kg);
+            gq_superblock(cur, xa + sb * xstep, lbq + ((size_t)sb * 16u + n) * 16u, lsx + sb * 16u, kg, acc);
+            cur = nx;
+        }
+#pragma unroll
+        for (int v = 0; v < 4; v++) red[(wave * 4u + (uint)v) * 64u + lane] = acc[v];
+        __syncthreads();
+        if (tid < 256u) {
+            const uint l = tid & 63u, v = tid >> 6;
+            float sum = red[v * 64u + l];
+            for (uint w8 = 1; w8 < nw; w8++) sum += red[(w8 * 4u + v) * 64u + l];
+            const uint t = 4u * (l >> 4) + v, r_out = tile * 16u + (l & 15u);
+            if (t < M && r_out < N) {
+                float* o = y + (size_t)t * N + r_out;
+                *o = ACC ? *o + sum : sum;
+            }
+        }
+        __syncthreads();                           // before the next tile's partial sums
     }
 }

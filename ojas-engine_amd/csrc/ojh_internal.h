@@ -120,6 +120,7 @@ int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **o
 int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptrs,
                const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);
 void ojh_gemm_q8k_tiles(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M, uint32_t *rw, uint32_t *rt);   // row tiles per workgroup / per wave of gemm_q8k_q4k_mf
+uint64_t ojh_gemm_q8k_mk_lds(uint32_t K, uint32_t M);   // LDS bytes of gemm_q8k_q4k_mk (ojh_manifest.cpp)
 uint64_t ojh_gemm_q8k_ml_lds(uint32_t K);           // LDS bytes of gemm_q8k_q4k_ml (ojh_manifest.cpp)
 uint64_t ojh_q6k_mk_lds(uint32_t K, uint32_t M);   // LDS bytes of gemv_q8k_q6k_mk (ojh_manifest.cpp)
 uint64_t ojh_q6k_ml_lds(uint32_t K, uint32_t M);   // LDS bytes of gemv_q8k_q6k_ml (ojh_manifest.cpp)

@@ -211,20 +211,24 @@ static int shape_ml(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, ui
 }
 // gemm_q8k_q4k_ml(xq, xs, w, y, K, N, M, ACC): up to 16 tokens, each wave's rows copied through its own LDS ring.
 // LDS: 16 token rows, their scales and split sums, eight rings of four 2304-byte units.
-uint64_t ojh_gemm_q8k_ml_lds(uint32_t K) { return 16 * ((uint64_t)K + 32) + K / 4 + K + 8 * 4 * 2304; }
+uint64_t ojh_gemm_q8k_ml_lds(uint32_t K) { return 16 * ((uint64_t)K + 32) + K / 4 + K + 256 + 8 * 4 * 2304; }
+// gemm_q8k_q4k_mk: M token rows, scales, split sums, a zero block, eight waves' partial sums
+uint64_t ojh_gemm_q8k_mk_lds(uint32_t K, uint32_t M) { return (uint64_t)M * ((uint64_t)K + 32) + K / 4 + K + 256 + 8192; }
 static int check_gemm_q8k_ml(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                              const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f;
     uint32_t K = c[0], N = c[1], M = c[2];
     int rc = check_kn(s, K, N, &f);
     if (rc) return rc;
-    if (block[1] != 1 || block[2] != 1 || !block[0] || block[0] % 64 || block[0] > 512)
-        return ojh_fail(OJH_ERR_ARG, "%s: block must be [64 .. 512 in whole waves,1,1], got [%u,%u,%u]", s->name, block[0], block[1], block[2]);
+    const bool mk = s->rows_per_wave == 2;      // gemm_q8k_q4k_mk: a tile per workgroup, K split over its eight waves
+    if (mk ? (rc = check_block(block, 512)) != 0 : block[1] != 1 || block[2] != 1 || !block[0] || block[0] % 64 || block[0] > 512)
+        return mk ? rc : ojh_fail(OJH_ERR_ARG, "%s: block must be [64 .. 512 in whole waves,1,1], got [%u,%u,%u]", s->name, block[0], block[1], block[2]);
     if (grid[1] != 1 || grid[2] != 1 || !grid[0]) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1], x > 0", s->name);
-    if (!M || M > 16 || ojh_gemm_q8k_ml_lds(K) > 163840)
+    const uint64_t lds = mk ? ojh_gemm_q8k_mk_lds(K, M) : ojh_gemm_q8k_ml_lds(K);
+    if (!M || M > 16 || lds > 163840)
         return ojh_fail(OJH_ERR_ARG, "%s: M=%u tokens of K=%u do not fit its 160 KB of LDS (1 <= M <= 16, %llu bytes needed)", s->name,
-                        M, K, (unsigned long long)ojh_gemm_q8k_ml_lds(K));
-    if ((uint64_t)N * (K / 256) * 144 > 0xFFFFFFFFull)
+                        M, K, (unsigned long long)lds);
+    if (!mk && (uint64_t)N * (K / 256) * 144 > 0xFFFFFFFFull)
         return ojh_fail(OJH_ERR_ARG, "%s: %u rows of K=%u pass 4 GiB, the reach of its 32-bit row offsets", s->name, N, K);
     need[0] = (size_t)M * K;
     need[1] = (size_t)M * (K / 256) * 4;
@@ -958,6 +962,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     }
     add("gemm_q8k_q4k_mf", "gemm_q8k", 4, 6, OJH_Q4_K, 1, check_gemm_q8k, shape_gemm_q8k);
     add("gemm_q8k_q4k_ml", "gemm_q8k", 4, 4, OJH_Q4_K, 1, check_gemm_q8k_ml, shape_ml);
+    add("gemm_q8k_q4k_mk", "gemm_q8k", 4, 4, OJH_Q4_K, 2, check_gemm_q8k_ml, shape_mk);
     add("relayout_q4k_q4l", "dequant", 4, 1, OJH_Q4_K, 0, check_relayout, shape_relayout);
     add("rows_q8_from_f16", "rowq8", 3, 2, 0, 0, check_rowq8, shape_rowq8);
     add("quant_rows_i8", "rowq8", 3, 2, 0, 1, check_rowq8, shape_rowq8);

@@ -112,6 +112,32 @@ def test_rows_copied_through_lds_by_name(gpu, orc, pkg, m, n, k, accum, grid_x, 
             gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_ml", [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], consts, [8, 1, 1], [512, 1, 1])
 
 
+@pytest.mark.parametrize("m,n,k,accum,grid_x", [(2, 50, 256, False, None), (16, 130, 4096, True, 3), (9, 301, 14336, False, None),
+                                                (16, 100, 8192, False, 2), (5, 4099, 2560, True, None)])
+def test_k_split_over_the_waves_by_name(gpu, orc, pkg, m, n, k, accum, grid_x):
+    """`gemm_q8k_q4k_mk`: a workgroup per 16-row tile, super-blocks dealt to its eight waves, partial
+    sums added in wave order; token rows past M are a shared block of zeros."""
+    w, x = _case(pkg, m, n, k, "mk")
+    y0 = pkg.synth.normal_f32(m * n, "gq", "mk-y0", m, n).reshape(m, n) if accum else np.zeros((m, n), np.float32)
+    want = np.stack([orc.matvec_kq(w, Q4_K, n, k, x[t]) for t in range(m)])
+    gpu.ensure_family("gemm_q8k")
+    nsb = k // 256
+    xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
+    gpu.quant_q8k(gpu.upload(x), m, k, xq, xs)
+    wd = gpu.upload_bytes(w)
+    grid, block = gpu.launch_shape("gemm_q8k_q4k_mk", k, n, m)
+    grid = [grid_x or grid[0], 1, 1]
+    yd = gpu.upload(np.concatenate([y0.ravel(), np.full(8, 4242.5, np.float32)]))
+    gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mk", [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], [k, n, m, int(accum)], grid, block)
+    got = gpu.read(yd, m * n + 8)
+    assert np.all(got[m * n:] == 4242.5), "wrote past the last token"
+    assert peak_err(got[:m * n].reshape(m, n) - y0, want) <= TOL_SEEN
+    with pytest.raises(pkg.OjasHipError, match="do not fit"):
+        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mk", [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], [14336, n, 12, 0], [8, 1, 1], [512, 1, 1])
+    with pytest.raises(pkg.OjasHipError, match="block"):
+        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mk", [(xq, 0), (xs, 0), (wd, 0), (yd, 0)], [k, n, m, 0], [8, 1, 1], [256, 1, 1])
+
+
 def test_a_token_does_not_depend_on_its_batch(gpu, pkg):
     """The same tokens rolled by 37 positions: every output bit for bit, moved."""
     m, n, k = 200, 512, 4096
