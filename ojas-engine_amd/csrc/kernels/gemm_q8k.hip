@@ -27,23 +27,9 @@
 // chunk so that an 8-byte read of 64 lanes spreads over all banks.
 // K-slices meet in LDS in wave order.
 #include "ojk_common.h"
+#include "ojk_gq.h"
 
-typedef int gq_i4 __attribute__((ext_vector_type(4)));
 #define GQ_LDS 77824u
-
-__device__ __forceinline__ long gq_pack(uint lo, uint hi) { return (long)(((unsigned long)hi << 32) | lo); }
-
-struct GqW {            // lane (n, kg): its bytes of one super-block of row n
-    uint4 hdr;          // d, dmin, the 12 scale bytes
-    uint2 q[4];         // codes of positions 8 kg .. 8 kg + 7 of each 64-weight chunk (low | high nibbles)
-};
-__device__ __forceinline__ GqW gq_load(const uchar* blk, uint kg) {
-    GqW r;
-    r.hdr = *(const uint4*)blk;
-#pragma unroll
-    for (int c = 0; c < 4; c++) r.q[c] = *(const uint2*)(blk + 16u + 32u * c + 8u * kg);
-    return r;
-}
 
 template <int P, int RT>
 __device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
@@ -243,45 +229,6 @@ gemm_q8k_q4k_mf(const signed char* xq, const float* xs, const uchar* w, float* y
     if (left <= 16u) gemm_q8k_q4k_mf_body<1, 1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
     else if (left <= 32u) gemm_q8k_q4k_mf_body<2, 1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
     else gemm_q8k_q4k_mf_body<4, 1>(xq, xs, w, y, K, N, M, ACC, RW, lds_gq);
-}
-
-// One super-block of a 16-row tile against one pass of 16 tokens:
-//   acc[v] += sx * (d * sum_j sc_j idot_j - dmin * sum_j m_j bsum_j)   for token 4 kg + v, row n.
-// xp: the lane's 8 bytes of token n at this super-block (byte 8 kg); pq: token n's split sums
-// (eight lo parts, eight hi parts); sx16: the super-block's 16 token scales.
-__device__ __forceinline__ void gq_superblock(const GqW& cur, const uchar* xp, const uchar* pq, const float* sx16, uint kg,
-                                              float (&acc)[4]) {
-    const gq_i4 zero = {0, 0, 0, 0};
-    const float d = f16_bits_to_f32(cur.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
-    int sc[8];
-    long B[8], Bm = 0;
-#pragma unroll
-    for (int c = 0; c < 4; c++) {
-        uint a, b;
-        q4k_scale_min_pair(cur.hdr.y, cur.hdr.z, cur.hdr.w, (uint)c, a, b);
-        sc[2 * c] = (int)(a & 0xFFu); sc[2 * c + 1] = (int)(a >> 8);
-        Bm |= (long)(unsigned long)(b & 0xFFFFu) << (16 * c);    // mins 2c, 2c + 1 -> bytes 2c, 2c + 1
-        B[2 * c] = gq_pack(cur.q[c].x & 0x0F0F0F0Fu, cur.q[c].y & 0x0F0F0F0Fu);
-        B[2 * c + 1] = gq_pack((cur.q[c].x >> 4) & 0x0F0F0F0Fu, (cur.q[c].y >> 4) & 0x0F0F0F0Fu);
-    }
-    if (kg != 0u) Bm = 0;                                        // only positions 0..7 carry mins
-    int isum[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (int jj = 0; jj < 8; jj++) {
-        const long A = *(const long*)(xp + 32 * jj);
-        const gq_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B[jj], zero, 0, 0, 0);
-#pragma unroll
-        for (int v = 0; v < 4; v++) isum[v] += __mul24(sc[jj], D[v]);
-    }
-    long Alo = 0, Ahi = 0;
-    if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
-    const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
-    const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
-    const float4 sx = *(const float4*)(sx16 + 4u * kg);
-    acc[0] += sx.x * (d * (float)isum[0] - dmin * (float)(64 * Dhi[0] + Dlo[0]));
-    acc[1] += sx.y * (d * (float)isum[1] - dmin * (float)(64 * Dhi[1] + Dlo[1]));
-    acc[2] += sx.z * (d * (float)isum[2] - dmin * (float)(64 * Dhi[2] + Dlo[2]));
-    acc[3] += sx.w * (d * (float)isum[3] - dmin * (float)(64 * Dhi[3] + Dlo[3]));
 }
 
 // What the two entries below stage once per workgroup: token rows 0 .. M - 1 (S bytes apart, eight

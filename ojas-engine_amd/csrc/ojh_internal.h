@@ -69,7 +69,7 @@ struct ojh_device {
     uint32_t q4k_ml_min_m = 2;   // OJAS_HIP_Q4K_ML_MIN_M: tokens from which long Q4_K matrices (32768 rows or more) take the LDS-copy form (0: never)
     uint32_t q4k_mf_min_m = 5;   // OJAS_HIP_Q4K_MF_MIN_M: tokens from which Q4_K rows go to the int8 matrix cores
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
-                                 // 3 = per-assignment decode form always
+                                 // 3 = per-assignment decode form always, 4 = matrix cores in the workgroup-per-tile form always
     uint32_t moe_dec_tokens = 8; // OJAS_HIP_MOE_DEC_TOKENS: the decode form serves up to this many tokens
     bool gemm_exact = false;     // OJAS_HIP_GEMM_EXACT: Q4_K prefill through the tile that holds dequant_to_f16 bits
     bool fused_quant = false;    // OJAS_HIP_FUSED_QUANT=1: ojh_mm (m = 1, Q4_K) quantizes x inside the matvec launch
@@ -120,6 +120,8 @@ int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **o
 int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptrs,
                const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);
 void ojh_gemm_q8k_tiles(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M, uint32_t *rw, uint32_t *rt);   // row tiles per workgroup / per wave of gemm_q8k_q4k_mf
+uint32_t ojh_moe_mt_groups(const ojh_device *dev, uint32_t N, uint32_t E, uint32_t per_cu);   // workgroups per expert of those entries
+uint64_t ojh_moe_mt_lds(uint32_t K);                // LDS bytes of moe_{gu,down}_q4k_mt (ojh_manifest.cpp)
 uint64_t ojh_gemm_q8k_mk_lds(uint32_t K, uint32_t M);   // LDS bytes of gemm_q8k_q4k_mk (ojh_manifest.cpp)
 uint64_t ojh_gemm_q8k_ml_lds(uint32_t K);           // LDS bytes of gemm_q8k_q4k_ml (ojh_manifest.cpp)
 uint64_t ojh_q6k_mk_lds(uint32_t K, uint32_t M);   // LDS bytes of gemv_q8k_q6k_mk (ojh_manifest.cpp)

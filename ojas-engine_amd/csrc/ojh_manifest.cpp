@@ -635,6 +635,9 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
     return OJH_OK;
 }
 
+// LDS of the moe_*_mt entries: 16 token rows, their scales and split sums, a block of zeros, the pass's assignments
+uint64_t ojh_moe_mt_lds(uint32_t K) { return 16 * ((uint64_t)K + 32) + K / 4 + K + 256 + 64; }
+
 // The MoE family; the number of tokens of the batched entries is read off the grid.
 //   0 moe_topk(lg, idx, wgt, E, KSEL)            1 moe_topk_m(same)              grid [T,1,1] x 64
 //   2 moe_group(idx, counts, offsets, list, NA, E)                                grid [1,1,1] x 256
@@ -642,6 +645,7 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
 //   4 moe_down_q4k_m(aq, as, wd, dv, offsets, list, K, N, NA)                     grid [ceil(N/16), E, 1]; ceil(N/32) for K <= 1024
 //   5 moe_combine(dv, wgt, y, T, KSEL, D, ACC)                                    grid [ceil(T*D/256),1,1]
 //   6 moe_gu_q4k_mm, 7 moe_down_q4k_mm: the arguments of 3 and 4, grid [ceil(N/16), E, 1]
+//  12 moe_gu_q4k_mt, 13 moe_down_q4k_mt: the arguments of 3 and 4, grid [1 .. ceil(N/16), E, 1] x 512
 //   8 moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)                      grid [ceil(N/8), NA, 1]
 //   9 moe_down_q4k_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)                  grid [ceil(N/8), T, 1]
 //  10 moe_gu_q4k_slots, 11 moe_down_q4k_slots: 8 and 9 with a u64 byte offset per assignment into an arena
@@ -671,12 +675,17 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         need[2] = (size_t)(E + 1) * 4;
         return OJH_OK;
     }
-    case 3: case 6: {
+    case 3: case 6: case 12: {
         uint32_t K = c[0], N = c[1], KS = c[2], NA = c[3], E = grid[1];
         const uint32_t per = s->rows_per_wave == 3 ? 8 : 16;   // rows per workgroup
-        if ((rc = check_block(block, 256))) return rc;
+        const bool mt = s->rows_per_wave == 12;
+        if ((rc = check_block(block, mt ? 512 : 256))) return rc;
         if (!K || K % 256 || !N || !KS || !NA || NA % KS) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u KSEL=%u NA=%u", s->name, K, N, KS, NA);
-        if (grid[0] != (N + per - 1) / per || grid[2] != 1)
+        if (mt) {
+            if (ojh_moe_mt_lds(K) > 81920) return ojh_fail(OJH_ERR_ARG, "%s: 16 tokens of K=%u do not fit its 80 KB of LDS", s->name, K);
+            if (!grid[0] || grid[0] > (N + 15) / 16 || grid[2] != 1)
+                return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N/16), E, 1]", s->name);
+        } else if (grid[0] != (N + per - 1) / per || grid[2] != 1)
             return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/%u), E, 1]", s->name, per);
         size_t rb = (size_t)(K / 256) * 144;
         need[0] = (size_t)(NA / KS) * K;
@@ -688,12 +697,17 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         align[0] = align[2] = align[3] = 16;
         return OJH_OK;
     }
-    case 4: case 7: {
+    case 4: case 7: case 13: {
         uint32_t K = c[0], N = c[1], NA = c[2], E = grid[1];
         const uint32_t per = s->rows_per_wave == 4 && K <= 1024 ? 32 : 16;   // short rows: two row sets per wave
-        if ((rc = check_block(block, 256))) return rc;
+        const bool mt = s->rows_per_wave == 13;
+        if ((rc = check_block(block, mt ? 512 : 256))) return rc;
         if (!K || K % 256 || !N || !NA) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u NA=%u", s->name, K, N, NA);
-        if (grid[0] != (N + per - 1) / per || grid[2] != 1)
+        if (mt) {
+            if (ojh_moe_mt_lds(K) > 81920) return ojh_fail(OJH_ERR_ARG, "%s: 16 tokens of K=%u do not fit its 80 KB of LDS", s->name, K);
+            if (!grid[0] || grid[0] > (N + 15) / 16 || grid[2] != 1)
+                return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N/16), E, 1]", s->name);
+        } else if (grid[0] != (N + per - 1) / per || grid[2] != 1)
             return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/%u), E, 1]", s->name, per);
         need[0] = (size_t)NA * K;
         need[1] = (size_t)NA * (K / 256) * 4;
@@ -780,7 +794,19 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
 }
 
 // K, N as named by the kernel; M = tokens (topk, combine) or assignments (group)
-static int shape_moe(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, uint32_t N, uint32_t M,
+// Workgroups per expert for the moe_*_mt entries: about `per_cu` workgroups per CU over all experts (what
+// is resident at once: one for the gate/up entry, which holds two tensors' blocks of four steps in
+// registers, two for the down entry), fewer until the expert's tiles divide evenly over the workgroups'
+// eight waves (or one workgroup is left).
+uint32_t ojh_moe_mt_groups(const ojh_device *dev, uint32_t N, uint32_t E, uint32_t per_cu) {
+    const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, tiles = (N + 15) / 16;
+    uint32_t rg = per_cu * cus / (E ? E : 1), cap = (tiles + 7) / 8;
+    if (rg > cap) rg = cap;
+    if (rg < 1) rg = 1;
+    while (rg > 1 && tiles % (8 * rg)) rg--;
+    return rg;
+}
+static int shape_moe(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
                      uint32_t grid[3], uint32_t block[3]) {
     grid[0] = grid[1] = grid[2] = 1;
     block[0] = 256;
@@ -792,6 +818,7 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, u
     case 3: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = experts
     case 4: grid[0] = K <= 1024 ? (N + 31) / 32 : (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
     case 6: case 7: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;
+    case 12: case 13: grid[0] = ojh_moe_mt_groups(dev, N, M ? M : 1, s->rows_per_wave == 12 ? 1 : 2); grid[1] = M ? M : 1; block[0] = 512; break;  // M = experts
     case 8: case 10: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = assignments
     case 9: case 11: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = tokens
     default: grid[0] = (uint32_t)(((uint64_t)M * N + 255) / 256); break;  // N = D, M = tokens
@@ -993,6 +1020,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("moe_combine", "moe", 3, 4, 0, 5, check_moe, shape_moe);
     add("moe_gu_q4k_mm", "moe", 7, 4, OJH_Q4_K, 6, check_moe, shape_moe);
     add("moe_down_q4k_mm", "moe", 6, 3, OJH_Q4_K, 7, check_moe, shape_moe);
+    add("moe_gu_q4k_mt", "moe", 7, 4, OJH_Q4_K, 12, check_moe, shape_moe);
+    add("moe_down_q4k_mt", "moe", 6, 3, OJH_Q4_K, 13, check_moe, shape_moe);
     add("moe_gu_q4k_dec", "moe", 5, 5, OJH_Q4_K, 8, check_moe, shape_moe);
     add("moe_down_q4k_dec", "moe", 5, 5, OJH_Q4_K, 9, check_moe, shape_moe);
     add("moe_gu_q4k_slots", "moe", 6, 6, OJH_Q4_K, 10, check_moe, shape_moe);

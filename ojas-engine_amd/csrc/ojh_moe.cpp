@@ -88,7 +88,11 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     // Expert products: on the matrix cores once experts see a few tokens each (measured crossover on
     // MI355X: ~4 assignments per expert), on integer dots below that, where the launch is a pure
     // stream of weight rows.  The two forms round their f32 sums in different orders (last ulp).
-    const bool mm = dev->moe_mode == 1 || (dev->moe_mode == 0 && NA >= 4 * E);
+    const bool mm = dev->moe_mode == 1 || dev->moe_mode == 4 || (dev->moe_mode == 0 && NA >= 4 * E);
+    // ... a wave per row tile where 16 tokens of K fit the workgroup's LDS (OJAS_HIP_MOE=4 keeps the workgroup-per-tile form)
+    const bool mt_gu = mm && dev->moe_mode != 4 && ojh_moe_mt_lds(d) <= 81920;
+    const bool mt_down = mm && dev->moe_mode != 4 && !down5 && ojh_moe_mt_lds(n_ff) <= 81920;
+    const uint32_t b512[3] = {512, 1, 1};
     // 1. quantize the tokens once
     {
         uint32_t g[3] = {nsb_d, T, 1};
@@ -101,11 +105,11 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     }
     // 3. gate/up + SiLU*mul, one launch over all experts
     {
-        uint32_t g[3] = {mm ? (n_ff + 15) / 16 : (n_ff + 7) / 8, E, 1};
-        if ((rc = ojh_launch(dev, mm ? "moe_gu_q4k_mm" : "moe_gu_q4k_m",
+        uint32_t g[3] = {mt_gu ? ojh_moe_mt_groups(dev, n_ff, E, 1) : mm ? (n_ff + 15) / 16 : (n_ff + 7) / 8, E, 1};
+        if ((rc = ojh_launch(dev, mt_gu ? "moe_gu_q4k_mt" : mm ? "moe_gu_q4k_mm" : "moe_gu_q4k_m",
                              {xq->ptr, xs->ptr, (char *)gate->raw->ptr + gate->off, (char *)up->raw->ptr + up->off, act->ptr,
                               offsets, list},
-                             {d, n_ff, ksel, NA}, g, b256)))
+                             {d, n_ff, ksel, NA}, g, mt_gu ? b512 : b256)))
             return rc;
     }
     // 4. quantize every assignment's activation (the CPU path quantizes `act` inside matvec_kq)
@@ -116,11 +120,11 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     // 5. down, one launch over all experts
     {
         const bool dots = down5 || !mm;
-        uint32_t g[3] = {dots && n_ff <= 1024 ? (d + 31) / 32 : (d + 15) / 16, E, 1};
+        uint32_t g[3] = {mt_down ? ojh_moe_mt_groups(dev, d, E, 2) : dots && n_ff <= 1024 ? (d + 31) / 32 : (d + 15) / 16, E, 1};
         // (Q5_K rows have no matrix-core form: they stay on integer dots at every batch size)
-        if ((rc = ojh_launch(dev, down5 ? "moe_down_q5k_m" : mm ? "moe_down_q4k_mm" : "moe_down_q4k_m",
+        if ((rc = ojh_launch(dev, down5 ? "moe_down_q5k_m" : mt_down ? "moe_down_q4k_mt" : mm ? "moe_down_q4k_mm" : "moe_down_q4k_m",
                              {aq->ptr, as_->ptr, (char *)down->raw->ptr + down->off, dv->ptr, offsets, list},
-                             {n_ff, d, NA}, g, b256)))
+                             {n_ff, d, NA}, g, mt_down ? b512 : b256)))
             return rc;
     }
     // 6. router-weighted sum over slots, in slot order

@@ -146,6 +146,41 @@ def test_decode_form_is_bit_identical_to_the_grouped_integer_dots(gpu, pkg, monk
     assert np.all(np.isfinite(outs[0])) and np.any(outs[0] != (y0.ravel() if accum else 0.0))
 
 
+@pytest.mark.parametrize("T,E,ksel,d,nff,accum", [(40, 4, 2, 512, 768, False), (9, 16, 3, 2304, 256, True),
+                                                   (130, 6, 5, 1024, 1280, False), (64, 128, 8, 2048, 768, False)])
+def test_matrix_core_forms_agree(gpu, orc, pkg, monkeypatch, T, E, ksel, d, nff, accum):
+    """The two matrix-core forms of the grouped products (a wave per row tile with the expert's tokens
+    staged in LDS; a workgroup per tile with K split over its waves) and the grouped integer dots:
+    integer sums are exact in all three and the f32 sums over super-blocks associate differently, so
+    an int8 code of the intermediate activation may flip between forms.  Experts with no, few, 16 and
+    more than 16 assignments (several passes), sampled tokens against the CPU path."""
+    gate, up, down = _experts(pkg, E, d, nff, ("mt", E, d, nff))
+    x = pkg.synth.normal_f32(T * d, "moe", "mtx", T, d).reshape(T, d)
+    lg = pkg.synth.normal_f32(T * E, "moe", "mtlg", T, E).reshape(T, E)
+    lg[:, 1] -= 50.0                                    # expert 1 is never chosen
+    lg[: T // 2, 0] += 50.0                             # expert 0 takes half the tokens
+    gi, gw, _, _ = _route(gpu, lg, ksel)
+    y0 = pkg.synth.normal_f32(T * d, "moe", "mty0").reshape(T, d) if accum else np.zeros((T, d), np.float32)
+    outs = {}
+    for mode in ("1", "4", "2"):
+        monkeypatch.setenv("OJAS_HIP_MOE", mode)
+        g = pkg.HipGpu(0)
+        try:
+            lg_, lu_, ld_ = g.lin(Q4_K, E * nff, d, gate), g.lin(Q4_K, E * nff, d, up), g.lin(Q4_K, E * d, nff, down)
+            yd = g.upload(np.concatenate([y0.ravel(), np.full(d, 12345.5, np.float32)]))
+            g.moe_ffn(g.upload(x), T, d, nff, E, ksel, g.upload_bytes(gi), g.upload(gw), lg_, lu_, ld_, yd, accum=accum)
+            got = g.read(yd, T * d + d)
+            assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
+            outs[mode] = got[:T * d].reshape(T, d) - y0
+        finally:
+            g.close()
+    for t in (0, T // 2, T - 1):
+        want = orc.moe_ffn(x[t:t + 1], gi[t:t + 1], gw[t:t + 1], gate, up, Q4_K, down, Q4_K, E, nff, mode=0)
+        assert peak_err(outs["1"][t], want[0]) <= TOL_SEEN, t
+    assert peak_err(outs["1"], outs["4"]) <= TOL
+    assert peak_err(outs["1"], outs["2"]) <= TOL
+
+
 @pytest.mark.parametrize("T,E,ksel,d,nff", [(1, 16, 4, 512, 768), (3, 8, 8, 2304, 256), (20, 8, 3, 512, 768),
                                              (70, 4, 2, 256, 2304)])
 def test_expert_ffn_with_q5k_down_tensors(gpu, orc, pkg, T, E, ksel, d, nff):
