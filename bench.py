@@ -228,7 +228,7 @@ def main() -> int:
     if not args.no_extra:
         # free the decode sets first: the secondary shapes bring their own tensors
         graphs.clear()
-        lin_q = sets[0]["gate"], sets[0]["down"]
+        lin_q = sets[0]["gate"], sets[0]["down"], sets[0]["head"]
         result["extra"] = extras(gpu, pkg, lin_q)
     print(json.dumps(result))
     gpu.close()
@@ -274,8 +274,22 @@ def extras(gpu, pkg, lin_q) -> dict:
             i8[f"{name}_M{m}"] = {"us": round(us, 1), "tops": round(2.0 * m * n * k / us / 1e6, 1),
                                   "weight_gbs": round(n * (k // 256) * 144 / us / 1e3, 1)}
     out["verify_prefill_q4k_int8"] = {"arithmetic": "quant_q8k activations, int8 x u4 dots on v_mfma_i32_16x16x32_i8, "
-                                                    "the CPU reference's scale algebra (gemm_q8k_q4k_mf)",
-                                      "timed": "quantize_q8k + gemm_q8k_q4k_mf", **i8}
+                                                    "the CPU reference's scale algebra",
+                                      "timed": "quantize_q8k + gemm_q8k_q4k_mf (down at M = 8: gemm_q8k_q4k_mk, "
+                                               "a workgroup per row tile with K split over its waves)", **i8}
+    # ---- speculative verify on the Q4_K output head of the decode step, bf16 activations
+    head4 = lin_q[2]
+    v4 = {}
+    for m in (2, 4, 8, 16):
+        xb = gpu.upload_bytes(synth.to_bf16_bits(synth.normal_f32(m * head4.k, "bench", "ver4_x", m)))
+        y = gpu.alloc(m * head4.n)
+        us = _time(gpu, lambda i: gpu.mm(xb, head4, y, m, x_dtype=pkg.X_BF16), 10, 2)
+        b = head4.n * (head4.k // 256) * 144 + m * (2 * head4.k + 4 * head4.n)
+        v4[f"M{m}"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
+        del y
+    out["verify_q4k_head_128256x4096"] = {"activations": "bf16, quantized per 256 (quant_q8k)",
+                                          "kernels": "gemm_q8k_q4k_ml (int8 MFMA, rows copied through LDS)",
+                                          "timed": "quantize_q8k_bf16 + the kernel", **v4}
     # ---- config 0: Q8_0 matvec 4096x4096, f32 activations (dot_q80 contract)
     n = k = 4096
     wq8 = [gpu.lin(pkg.Q8_0, n, k, synth.q80_weights(n, k, "bench", "q80")) for _ in range(16)]
@@ -338,7 +352,7 @@ def extras(gpu, pkg, lin_q) -> dict:
         fl = 2.0 * T * ksel * 3 * nff * d
         moe[f"T{T}"] = {"us": round(us, 1), "distinct_experts": distinct, "gbs": round(b / us / 1e3, 1),
                         "tflops": round(fl / us / 1e6, 2)}
-    out["moe_ffn_q4k_128x_top8"] = {"timed": "router + expert FFN (T <= 8: gate/up and down launches addressed by assignment; above: quantize, group, gate/up, quantize, down, combine)", **moe}
+    out["moe_ffn_q4k_128x_top8"] = {"timed": "router + expert FFN (T <= 8: gate/up and down launches addressed by assignment; above: quantize, group, gate/up, quantize, down, combine; T = 256 on int8 MFMA, moe_{gu,down}_q4k_mt)", **moe}
     del gate, up, down
     # ---- speculative verify on a Q6_K output head 151936 x 4096, bf16 activations
     n, k = 151936, 4096
@@ -352,7 +366,8 @@ def extras(gpu, pkg, lin_q) -> dict:
         ver[f"M{m}"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4),
                         "tflops": round(2.0 * m * n * k / us / 1e6, 2)}
     out["verify_q6k_head_151936x4096"] = {"activations": "bf16, quantized per 256 (quant_q8k)",
-                                          "kernels": "M1 gemv_q8k_q6k_px, M2 gemv_q8k_q6k_mx, M4-16 gemv_q8k_q6k_mf (int8 MFMA)", **ver}
+                                          "kernels": "M1 gemv_q8k_q6k_px, M2-16 gemv_q8k_q6k_ml (int8 MFMA, rows copied through LDS)",
+                                          "timed": "quantize_q8k_bf16 + the kernel", **ver}
     return out
 
 
