@@ -46,7 +46,7 @@ enum {
 };
 
 /* GGUF tensor types handled by this path (crates/ojas-formats/src/gguf.rs:563-591). */
-enum { OJH_Q8_0 = 8, OJH_Q4_K = 12, OJH_Q5_K = 13, OJH_Q6_K = 14 };
+enum { OJH_Q8_0 = 8, OJH_Q4_K = 12, OJH_Q5_K = 13, OJH_Q6_K = 14, OJH_IQ4_NL = 20, OJH_IQ4_XS = 23 };
 
 /* Element type of an activation buffer handed to ojh_mm. */
 enum { OJH_X_F32 = 0, OJH_X_BF16 = 1, OJH_X_F16 = 2 };

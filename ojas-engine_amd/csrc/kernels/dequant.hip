@@ -1,6 +1,6 @@
 // Family "dequant": GGUF blocks -> IEEE binary16, bit-exact with the reference decoder
 // (crates/ojas-formats/src/gguf.rs:612-1116; arms :704-709 Q8_0, :1042-1059 Q4_K,
-// :1060-1085 Q5_K, :1086-1108 Q6_K).
+// :1060-1085 Q5_K, :1086-1108 Q6_K, :796-813 IQ4_NL, :814-840 IQ4_XS).
 //
 // Bit-exactness rules: every product and difference is a separately rounded f32 operation
 // (__fmul_rn / __fsub_rn, never an FMA), in the reference's association order, followed by one
@@ -144,4 +144,44 @@ relayout_q4k_q4l(const uchar* __restrict__ w, uchar* __restrict__ nib, ushort* _
         out[i] = p0 | (p1 << 8) | (p2 << 16) | (p3 << 24);
     }
     *(uint4*)(nib + tid * 16u) = make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+dequant_iq4nl_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
+    // one thread per weight: weights 0..15 are the low nibbles of qs[0..15], 16..31 the high nibbles
+    size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+    size_t b = i >> 5;
+    if (b >= nblocks) return;
+    const uchar* blk = w + b * IQ4NL_BYTES;
+    const uint j = (uint)i & 31u, byte = blk[2u + (j & 15u)];
+    const uint idx = j < 16u ? byte & 0xFu : byte >> 4;
+    const float d = f16_bits_to_f32(*(const ushort*)blk);
+    const float lv = (float)(signed char)(iq4_levels4(idx) & 0xFFu);
+    out[i] = f32_to_f16_bits(__fmul_rn(d, lv));
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+dequant_iq4xs_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
+    // 32 threads per super-block; thread t owns dword t of qs: sub-block ib = t / 4, four low-nibble
+    // weights at 32 ib + 4 (t % 4) and the four high-nibble weights 16 further on.
+    size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x;
+    size_t b = tid >> 5;
+    if (b >= nblocks) return;
+    const uint t = (uint)tid & 31u, ib = t >> 2, o = (t & 3u) * 4u;
+    const uchar* blk = w + b * IQ4XS_BYTES;
+    const uint* hdr = (const uint*)blk;
+    const uint h0 = hdr[0], sl = hdr[1];
+    const float d = f16_bits_to_f32(h0 & 0xFFFFu);
+    const uint sh = h0 >> 16;
+    const uint ls = ((sl >> (4u * ib)) & 0xFu) | (((sh >> (2u * ib)) & 3u) << 4);
+    const float dl = __fmul_rn(d, (float)((int)ls - 32));
+    const uint q = hdr[2 + t];
+    const uint lo = iq4_levels4(q & 0x0F0F0F0Fu), hi = iq4_levels4((q >> 4) & 0x0F0F0F0Fu);
+    ushort* o1 = out + b * 256u + ib * 32u + o;
+    ushort* o2 = o1 + 16;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        o1[i] = f32_to_f16_bits(__fmul_rn(dl, (float)(signed char)(lo >> (8 * i))));
+        o2[i] = f32_to_f16_bits(__fmul_rn(dl, (float)(signed char)(hi >> (8 * i))));
+    }
 }

@@ -1,7 +1,9 @@
 // Family "gemv": fused-dequant matvecs on raw GGUF blocks with f32 activations — the contract
 // of the reference's GPU kernels gemv_nat_<fmt>{,_accum,_bias,_m}
 // (crates/ojas-cuda/src/kernels/nat.rs:69-89; bodies crates/ojas-core/src/quant_src.rs:779-824
-// Q4_K, :833-867 Q6_K, :1028-1057 Q8_0, :1154-1180 batched).
+// Q4_K, :833-867 Q6_K, :1028-1057 Q8_0, :1154-1180 batched).  IQ4_NL and IQ4_XS rows ride the same
+// entries; their arithmetic is the CPU path's dot_iq4nl / dot_iq4xs, which also reads f32 activations
+// (crates/ojas-cpu/src/cpu_math.rs:993-1010, :943-967).
 //
 //   gemv_nat_<fmt>{,_accum}(x, w, y, K, N)        y[n] (=,+=) sum_k W[n,k] x[k]
 //   gemv_nat_<fmt>_bias(x, w, y, bs, K, N)        y[n] = ... + bs[n]
@@ -339,6 +341,198 @@ __device__ __forceinline__ void gemv_nat_q80_m_body(const float* __restrict__ x,
     }
 }
 
+// ------------------------------------------------------------------ IQ4_NL, IQ4_XS
+// Both store 4-bit indices into the sixteen-level codebook; within a 32-weight group the low
+// nibbles of its 16 bytes are weights 0..15 and the high nibbles weights 16..31.  A lane takes one
+// dword of indices: four low-nibble weights and the four 16 further on, against two float4 of x.
+// IQ4_NL: 18-byte blocks {f16 d; qs[16]}, four lanes per block, a wave walks 16 blocks per step.
+// IQ4_XS: 136-byte super-blocks {f16 d; u16 scales_h; u8 scales_l[4]; qs[128]}, 32 lanes per
+// super-block (lane / 4 = sub-block, its 6-bit scale minus 32 times d applied per lane).
+typedef uint u32_a2 __attribute__((aligned(2)));
+
+__device__ __forceinline__ float iq4_lane_dot(uint q, float4 x0, float4 x1) {
+    const uint lo = iq4_levels4(q & 0x0F0F0F0Fu), hi = iq4_levels4((q >> 4) & 0x0F0F0F0Fu);
+    float a = sb0(lo) * x0.x;
+    a = fmaf(sb0(hi), x1.x, a);
+    a = fmaf(sb1(lo), x0.y, a);
+    a = fmaf(sb1(hi), x1.y, a);
+    a = fmaf(sb2(lo), x0.z, a);
+    a = fmaf(sb2(hi), x1.z, a);
+    a = fmaf(sb3(lo), x0.w, a);
+    return fmaf(sb3(hi), x1.w, a);
+}
+
+struct Iq4nlW {
+    static constexpr uint STEP = 16u;            // blocks a wave walks per step
+    static __device__ __forceinline__ uint units(uint K) { return K >> 5; }
+    // lane -> (block of the step, float offset of its first x fragment inside the block)
+    static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 2; }
+    static __device__ __forceinline__ uint x_off(uint lane) { return (lane & 3u) * 4u; }
+    static __device__ __forceinline__ uint x_unit(uint) { return 32u; }
+    struct Frag { uint d16, q; };
+    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
+        const uchar* blk = row + (size_t)u * IQ4NL_BYTES;
+        Frag f;
+        f.d16 = *(const ushort*)blk;
+        f.q = *(const u32_a2*)(blk + 2u + (lane & 3u) * 4u);
+        return f;
+    }
+    static __device__ __forceinline__ float dot(const Frag& f, uint, float4 x0, float4 x1) {
+        return f16_bits_to_f32(f.d16) * iq4_lane_dot(f.q, x0, x1);
+    }
+};
+
+struct Iq4xsW {
+    static constexpr uint STEP = 2u;             // super-blocks per step
+    static __device__ __forceinline__ uint units(uint K) { return K >> 8; }
+    static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 5; }
+    static __device__ __forceinline__ uint x_off(uint lane) { return ((lane & 31u) >> 2) * 32u + (lane & 3u) * 4u; }
+    static __device__ __forceinline__ uint x_unit(uint) { return 256u; }
+    struct Frag { uint h0, sl, q; };
+    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
+        const uint* blk = (const uint*)(row + (size_t)u * IQ4XS_BYTES);
+        Frag f;
+        f.h0 = blk[0];
+        f.sl = blk[1];
+        f.q = blk[2u + (lane & 31u)];
+        return f;
+    }
+    static __device__ __forceinline__ float dot(const Frag& f, uint lane, float4 x0, float4 x1) {
+        const uint ib = (lane & 31u) >> 2;
+        const uint ls = ((f.sl >> (4u * ib)) & 0xFu) | ((((f.h0 >> 16) >> (2u * ib)) & 3u) << 4);
+        return f16_bits_to_f32(f.h0 & 0xFFFFu) * (float)((int)ls - 32) * iq4_lane_dot(f.q, x0, x1);
+    }
+};
+
+template <class W, int R, int MODE>
+__device__ __forceinline__ void gemv_nat_iq4_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                  float* __restrict__ y, const float* __restrict__ bs,
+                                                  uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 >= N) return;
+    const uint nu = W::units(K);
+    const size_t rb = (size_t)nu * (W::STEP == 16u ? IQ4NL_BYTES : IQ4XS_BYTES);
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (uint u = W::unit_of(lane); u < nu; u += W::STEP) {
+        typename W::Frag f[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) f[r] = W::load(w + (size_t)min(row0 + r, N - 1u) * rb, u, lane);
+        const float* xp = x + (size_t)u * W::x_unit(0) + W::x_off(lane);
+        const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + 16);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += W::dot(f[r], lane, x0, x1);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float s = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, s);
+    }
+}
+
+template <class W, int MT>
+__device__ __forceinline__ void gemv_nat_iq4_m_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                    float* __restrict__ y, uint K, uint N, uint M, uint ACC) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const uint nu = W::units(K);
+    const uchar* wr = w + (size_t)row * nu * (W::STEP == 16u ? IQ4NL_BYTES : IQ4XS_BYTES);
+    for (uint m0 = 0; m0 < M; m0 += MT) {
+        float acc[MT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) acc[i] = 0.0f;
+        for (uint u = W::unit_of(lane); u < nu; u += W::STEP) {
+            const typename W::Frag f = W::load(wr, u, lane);
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                const uint m = min(m0 + i, M - 1u);
+                const float* xp = x + (size_t)m * K + (size_t)u * W::x_unit(0) + W::x_off(lane);
+                acc[i] += W::dot(f, lane, *(const float4*)xp, *(const float4*)(xp + 16));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float s = wave_sum(acc[i]);
+            if (lane == 0 && m0 + i < M) {
+                float* o = y + (size_t)(m0 + i) * N + row;
+                *o = ACC ? *o + s : s;
+            }
+        }
+    }
+}
+
+// Many rows (an output head): a 4-bit row is an eighth of the bytes of the f32 activations it meets, so
+// a wave that fetches its activation fragments again for every few rows is bound by those loads, not
+// by HBM (2.7 TB/s at 128256 x 4096).  Here rows are grid-stride and the wave keeps its share of x —
+// 8 floats per lane and step, NS steps — in registers for the whole launch; out-of-range steps hold
+// zeros and repeat the last block.   gemv_nat_iq4{nl,xs}_px(x, w, y, K, N), K <= 4096 (64 floats of x per
+// lane; twice that would halve the resident waves).
+template <class W, int NS>
+__device__ __forceinline__ void gemv_nat_iq4_px_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                     float* __restrict__ y, uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint nu = W::units(K);
+    const size_t rb = (size_t)nu * (W::STEP == 16u ? IQ4NL_BYTES : IQ4XS_BYTES);
+    float4 xr[NS][2];
+    uint uc[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const uint u = W::unit_of(lane) + (uint)s * W::STEP;
+        uc[s] = min(u, nu - 1u);
+        xr[s][0] = xr[s][1] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (u < nu) {
+            const float* xp = x + (size_t)u * W::x_unit(0) + W::x_off(lane);
+            xr[s][0] = *(const float4*)xp;
+            xr[s][1] = *(const float4*)(xp + 16);
+        }
+    }
+    const uint nwaves = gridDim.x * (blockDim.x >> 6);
+    for (uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2u; row0 < N; row0 += nwaves * 2u) {
+        const uchar* r0 = w + (size_t)row0 * rb;
+        const uchar* r1 = w + (size_t)min(row0 + 1u, N - 1u) * rb;
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const typename W::Frag f0 = W::load(r0, uc[s], lane), f1 = W::load(r1, uc[s], lane);
+            a0 += W::dot(f0, lane, xr[s][0], xr[s][1]);
+            a1 += W::dot(f1, lane, xr[s][0], xr[s][1]);
+        }
+        a0 = wave_sum(a0);
+        a1 = wave_sum(a1);
+        if (lane == 0) {
+            y[row0] = a0;
+            if (row0 + 1u < N) y[row0 + 1u] = a1;
+        }
+    }
+}
+
+#define GEMV_NAT_IQ4_PX(FMT, W)                                                                            \
+    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_px(                                 \
+        const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
+        gemv_nat_iq4_px_body<W, 8>(x, w, y, K, N); }
+GEMV_NAT_IQ4_PX(iq4nl, Iq4nlW)
+GEMV_NAT_IQ4_PX(iq4xs, Iq4xsW)
+
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_iq4nl_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
+    gemv_nat_iq4_body<Iq4nlW, R, MODE>(x, w, y, bs, K, N);
+}
+template <int MT>
+__device__ __forceinline__ void gemv_nat_iq4nl_m_body(const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    gemv_nat_iq4_m_body<Iq4nlW, MT>(x, w, y, K, N, M, ACC);
+}
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_iq4xs_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
+    gemv_nat_iq4_body<Iq4xsW, R, MODE>(x, w, y, bs, K, N);
+}
+template <int MT>
+__device__ __forceinline__ void gemv_nat_iq4xs_m_body(const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    gemv_nat_iq4_m_body<Iq4xsW, MT>(x, w, y, K, N, M, ACC);
+}
+
 // ------------------------------------------------------------------ Q8_0, rows staged through LDS
 //   gemv_nat_q80_lds{,_accum}(x, w, y, K, N, KC)   gemv_nat_q80_lds_bias(x, w, y, bs, K, N, KC)
 // 34-byte blocks defeat wide per-lane loads, and f32 activations are four bytes per weight byte
@@ -476,3 +670,5 @@ gemv_nat_q80_lds_bias(const float* x, const uchar* w, float* y, const float* bs,
 GEMV_NAT_ENTRIES(q80)
 GEMV_NAT_ENTRIES(q4k)
 GEMV_NAT_ENTRIES(q6k)
+GEMV_NAT_ENTRIES(iq4nl)
+GEMV_NAT_ENTRIES(iq4xs)

@@ -16,6 +16,8 @@ typedef unsigned short ushort;
 #define Q4K_BYTES 144u
 #define Q5K_BYTES 176u
 #define Q6K_BYTES 210u
+#define IQ4NL_BYTES 18u
+#define IQ4XS_BYTES 136u
 
 // Vector types that may sit on a 2-byte boundary: Q8_0 (34 B) and Q6_K (210 B) blocks are only
 // 2-byte aligned inside a row.  gfx950 runs in unaligned-access mode, so these compile to one
@@ -125,6 +127,20 @@ __device__ __forceinline__ void q4k_scale_min_pair(uint s0, uint s1, uint s2, ui
     uint mn_hi = ((w >> 4) & 0x0F0Fu) | ((z >> 2) & 0x3030u);
     sc = c < 2u ? sc_lo : sc_hi;
     mn = c < 2u ? mn_lo : mn_hi;
+}
+
+// ---- the IQ4 codebook ---------------------------------------------------------------------------
+// IQ4_NL and IQ4_XS store 4-bit indices into sixteen fixed int8 levels
+// (-127 -104 -83 -65 -49 -35 -22 -10 1 13 25 38 53 69 89 113; crates/ojas-core/src/iq_tables.rs:881-884).
+// Four indices (one per byte, 0..15) -> their four levels as bytes: two byte-permutes over the halves
+// of the table, merged by bit 3 of each index.
+__device__ __forceinline__ uint iq4_levels4(uint idx4) {
+    const uint sel = idx4 & 0x07070707u;
+    const uint lo = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, sel);   // levels 0..7
+    const uint hi = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, sel);   // levels 8..15
+    const uint m1 = (idx4 >> 3) & 0x01010101u;
+    const uint mask = (m1 << 8) - m1;                                       // 0xFF in every byte whose index is >= 8
+    return (hi & mask) | (lo & ~mask);
 }
 
 // ---- global -> LDS copies by the memory system ------------------------------------------------

@@ -95,6 +95,7 @@ struct ojh_block_format {
     const char *tag;
 };
 const ojh_block_format *ojh_format(uint32_t ggml_type);
+bool ojh_float_rows(uint32_t ggml_type);   // the CPU path reads f32 activations for this format
 
 // What a kernel touches at given constants. Returns OJH_OK or fails with a message.
 typedef int (*ojh_check_fn)(const struct ojh_kernel_spec *spec, const uint32_t *consts,

@@ -14,7 +14,13 @@ static const ojh_block_format kFormats[] = {
     {OJH_Q4_K, 144, 256, "q4k"},
     {OJH_Q5_K, 176, 256, "q5k"},
     {OJH_Q6_K, 210, 256, "q6k"},
+    {OJH_IQ4_NL, 18, 32, "iq4nl"},
+    {OJH_IQ4_XS, 136, 256, "iq4xs"},
 };
+
+// Formats whose CPU path multiplies the raw row with f32 activations (dot_q80, dot_iq4nl, dot_iq4xs:
+// crates/ojas-cpu/src/cpu_math.rs:1131-1141, :1179) instead of quantizing them per 256.
+bool ojh_float_rows(uint32_t t) { return t == OJH_Q8_0 || t == OJH_IQ4_NL || t == OJH_IQ4_XS; }
 
 const ojh_block_format *ojh_format(uint32_t t) {
     for (const auto &f : kFormats)
@@ -68,7 +74,7 @@ static int check_gemv_nat(const ojh_kernel_spec *s, const uint32_t *c, const uin
     need[1] = (size_t)N * (K / f->weights) * f->bytes;
     need[2] = (size_t)N * 4;
     if (s->n_bufs == 4) need[3] = (size_t)N * 4;
-    align[1] = f->bytes % 16 ? 2 : 16;
+    align[1] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
     align[2] = align[3] = 4;
     return OJH_OK;
 }
@@ -256,8 +262,25 @@ static int check_gemv_q8k_px(const ojh_kernel_spec *s, const uint32_t *c, const 
     need[2] = (size_t)N * (K / f->weights) * f->bytes;
     need[3] = (size_t)N * 4;
     align[1] = 4;
-    align[2] = f->bytes % 16 ? 2 : 16;
+    align[2] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
     align[3] = 4;
+    return OJH_OK;
+}
+// gemv_nat_iq4{nl,xs}_px(x, w, y, K, N): rows grid-stride, two per wave and step, f32 activations in registers
+static int check_gemv_nat_px(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                             const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], N = c[1];
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if ((rc = check_block(block, 256))) return rc;
+    if (K > 4096) return ojh_fail(OJH_ERR_UNSUPPORTED, "%s: K=%u exceeds the 4096 activations a wave keeps in registers", s->name, K);
+    if (!grid[0] || grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1], x > 0", s->name);
+    need[0] = (size_t)K * 4;
+    need[1] = (size_t)N * (K / f->weights) * f->bytes;
+    need[2] = (size_t)N * 4;
+    align[1] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
+    align[2] = 4;
     return OJH_OK;
 }
 static int shape_px(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t N, uint32_t,
@@ -289,7 +312,7 @@ static int check_gemv_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uin
     need[3] = (size_t)N * 4;
     if (s->n_bufs == 5) need[4] = (size_t)N * 4;
     align[1] = 4;
-    align[2] = f->bytes % 16 ? 2 : 16;
+    align[2] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
     align[3] = align[4] = 4;
     return OJH_OK;
 }
@@ -316,7 +339,7 @@ static int check_gemv_q8k_x4(const ojh_kernel_spec *s, const uint32_t *c, const 
         size_t rows = E[i] - (i ? E[i - 1] : 0);
         need[2 + i] = rows * (K / f->weights) * f->bytes;
         need[6 + i] = rows * 4;
-        align[2 + i] = f->bytes % 16 ? 2 : 16;
+        align[2 + i] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
         align[6 + i] = 4;
     }
     return OJH_OK;
@@ -403,7 +426,7 @@ static int check_gemv_nat_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     need[0] = (size_t)M * K * 4;
     need[1] = (size_t)N * (K / f->weights) * f->bytes;
     need[2] = (size_t)M * N * 4;
-    align[1] = f->bytes % 16 ? 2 : 16;
+    align[1] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
     align[2] = 4;
     return OJH_OK;
 }
@@ -465,7 +488,7 @@ static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     need[2] = (size_t)N * (K / f->weights) * f->bytes;
     need[3] = (size_t)M * N * 4;
     align[1] = 4;
-    align[2] = f->bytes % 16 ? 2 : 16;
+    align[2] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
     align[3] = 4;
     if (mf || mk) {           // whole aligned dwords around every piece: the last one may end 2 bytes on
         need[2] = (need[2] + 3) & ~(size_t)3;
@@ -572,7 +595,7 @@ static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint
         return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover %u blocks", s->name, nb);
     need[0] = (size_t)nb * f->bytes;
     need[1] = (size_t)nb * f->weights * 2;
-    align[0] = f->bytes % 16 ? 2 : 16;
+    align[0] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
     align[1] = 8;
     return OJH_OK;
 }
@@ -609,7 +632,7 @@ static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_
     need[0] = (size_t)M * K * 2;
     need[1] = (size_t)N * (K / f->weights) * f->bytes;
     need[2] = (size_t)M * N * 4;
-    align[1] = f->bytes % 16 ? 2 : 16;
+    align[1] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
     align[2] = 4;
     return OJH_OK;
 }
@@ -959,6 +982,10 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g + "_accum", "gemv", 3, 2, f.type, 4, check_gemv_nat, shape_rows);
         add(g + "_bias", "gemv", 4, 2, f.type, 4, check_gemv_nat, shape_rows);
         add(g + "_m", "gemv", 3, 4, f.type, 1, check_gemv_nat_m, shape_rows);
+        if (f.type == OJH_IQ4_NL || f.type == OJH_IQ4_XS) {   // f32 activations only, no MFMA tile
+            add(g + "_px", "gemv", 3, 2, f.type, 2, check_gemv_nat_px, shape_px);
+            continue;
+        }
         if (f.type == OJH_Q8_0) {
             add(g + "_lds", "gemv", 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
             add(g + "_lds_accum", "gemv", 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
@@ -1001,7 +1028,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     // prefill / verify MFMA tiles: "q8_0" is the reference's spelling for this family
     for (const auto &f : kFormats) {
-        if (f.type == OJH_Q5_K) continue;
+        if (f.type == OJH_Q5_K || f.type == OJH_IQ4_NL || f.type == OJH_IQ4_XS) continue;
         std::string g = std::string("gemm_mm_") + (f.type == OJH_Q8_0 ? "q8_0" : f.tag);
         add(g, "gemm", 3, 4, f.type, 0, check_gemm, shape_gemm);
         add(g + "_sk", "gemm", 3, 4, f.type, 1, check_gemm, shape_gemm);

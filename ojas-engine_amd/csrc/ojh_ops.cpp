@@ -60,7 +60,7 @@ extern "C" int ojh_lin_wrap(ojh_device *dev, uint32_t type, uint32_t n, uint32_t
     int rc = lin_check(type, n, k, &rb);
     if (rc) return rc;
     const ojh_block_format *f = ojh_format(type);
-    if ((rc = span_ok("ojh_lin_wrap: raw", raw, off, rb * n, f->bytes % 16 ? 2 : 16))) return rc;
+    if ((rc = span_ok("ojh_lin_wrap: raw", raw, off, rb * n, f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16))) return rc;
     ojh_lin *l = new ojh_lin();
     l->type = type; l->n = n; l->k = k; l->row_bytes = rb; l->raw = raw; l->off = off; l->owns_raw = false;
     *out = l;
@@ -86,7 +86,7 @@ extern "C" int ojh_dequant_f16(ojh_device *dev, uint32_t type, const ojh_buf *ra
     size_t nb = n_weights / f->weights;
     if (nb > 0x7FFFFFFFu / 64) return ojh_fail(OJH_ERR_ARG, "dequant: too many blocks in one call (%zu)", nb);
     int rc;
-    if ((rc = span_ok("dequant: raw", raw, raw_off, nb * f->bytes, f->bytes % 16 ? 2 : 16))) return rc;
+    if ((rc = span_ok("dequant: raw", raw, raw_off, nb * f->bytes, f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16))) return rc;
     if ((rc = span_ok("dequant: out", out, out_off, n_weights * 2, 2))) return rc;
     if ((rc = ensure(dev, "dequant"))) return rc;
     std::string name = std::string("dequant_") + f->tag + "_f16";
@@ -273,7 +273,7 @@ static int mm_common_checks(const char *who, const ojh_lin *w, ojh_buf *y, size_
     int rc;
     if ((rc = span_ok("y", y, y_off, (size_t)m * w->n * 4, 4))) return rc;
     if (bias && (rc = span_ok("bias", bias, 0, (size_t)w->n * 4, 4))) return rc;
-    if ((rc = span_ok("w", w->raw, w->off, w->row_bytes * w->n, f->bytes % 16 ? 2 : 16))) return rc;
+    if ((rc = span_ok("w", w->raw, w->off, w->row_bytes * w->n, f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16))) return rc;
     *fmt = f;
     return OJH_OK;
 }
@@ -284,8 +284,8 @@ extern "C" int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xsc
     const ojh_block_format *f;
     int rc = mm_common_checks("ojh_mm_q8k", w, y, y_off, bias, m, accum, &f);
     if (rc) return rc;
-    if (w->type == OJH_Q8_0)
-        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm_q8k: Q8_0 rows take f32 activations, as dot_q80 does");
+    if (ojh_float_rows(w->type))
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm_q8k: %s rows take f32 activations, as their CPU dot does", f->tag);
     size_t nsb = w->k / 256;
     if ((rc = span_ok("xq", xq, 0, (size_t)m * nsb * 256, 16))) return rc;
     if ((rc = span_ok("xscales", xscales, 0, (size_t)m * nsb * 4, 4))) return rc;
@@ -303,8 +303,8 @@ extern "C" int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_bu
     for (int i = 0; i < count; i++) {
         const ojh_block_format *fi;
         if ((rc = mm_common_checks("ojh_mm_q8k_multi", ws[i], ys[i], y_offs ? y_offs[i] : 0, nullptr, 1, 0, &fi))) return rc;
-        if (ws[i]->type == OJH_Q8_0)
-            return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm_q8k_multi: Q8_0 rows take f32 activations, as dot_q80 does");
+        if (ojh_float_rows(ws[i]->type))
+            return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm_q8k_multi: %s rows take f32 activations, as their CPU dot does", fi->tag);
         if (ws[i]->k != ws[0]->k)
             return ojh_fail(OJH_ERR_ARG, "ojh_mm_q8k_multi: projection %d has K=%u, the first has K=%u", i, ws[i]->k, ws[0]->k);
         if (ws[i]->type != OJH_Q4_K) grouped = false;
@@ -365,9 +365,15 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         act_mode = OJH_ACT_Q8K;
     }
 
+    // IQ4_NL / IQ4_XS: f32 activations against the raw rows at every token count (dot_iq4nl / dot_iq4xs);
+    // no int8-activation form and no MFMA tile read them.
+    const bool iq4 = w->type == OJH_IQ4_NL || w->type == OJH_IQ4_XS;
+    if (iq4 && act_mode == OJH_ACT_Q8K)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: %s rows take f32 activations only (OJH_ACT_FLOAT or OJH_ACT_AUTO)", f->tag);
+
     // Above the crossover the MFMA tile wins over streaming the weights once per few tokens
     // (the reference switches at 8 rows, crates/ojas-models/src/decoder/dispatch.rs:70-75).
-    if (m >= dev->gemm_min_m && act_mode != OJH_ACT_Q8K && K % 64 == 0 && (uint64_t)m * K < 0x7FFFFFFFull &&
+    if (m >= dev->gemm_min_m && act_mode != OJH_ACT_Q8K && !iq4 && K % 64 == 0 && (uint64_t)m * K < 0x7FFFFFFFull &&
         (uint64_t)m * N < 0x7FFFFFFFull) {
         // Q4_K takes the 256-wide tile with the reference GPU kernel's arithmetic (f16 qa*q + qb)
         // unless the tile that reproduces dequant_to_f16 bit for bit is asked for.
@@ -404,7 +410,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         return ojh_launch(dev, base.c_str(), {xh->ptr, wp, yp}, {K, N, (uint32_t)(accum != 0), m}, sg, sb);
     }
 
-    bool q8k = w->type != OJH_Q8_0 && act_mode != OJH_ACT_FLOAT && act_mode != OJH_ACT_FLOAT_EXACT;
+    bool q8k = !ojh_float_rows(w->type) && act_mode != OJH_ACT_FLOAT && act_mode != OJH_ACT_FLOAT_EXACT;
     // Opt-in: one token, f32 in, plain store through the launch that quantizes x itself
     // (bit-identical results).  Measured slower than quantize + matvec at every decode shape on
     // MI355X — each block repeats the quantization and reads x through LDS — so it is off by default.
@@ -455,6 +461,12 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         if (bias) p.push_back(bias->ptr);
         return ojh_launch(dev, accum ? "gemv_nat_q80_lds_accum" : bias ? "gemv_nat_q80_lds_bias" : "gemv_nat_q80_lds", p,
                           {K, N, ojh_q80_lds_kc(K)}, sg, sb);
+    }
+    // IQ4 rows of an output head: rows grid-stride, the wave's f32 activations in registers
+    if (m == 1 && iq4 && dev->px && !accum && !bias && N >= 32768u && K <= 4096u) {
+        uint32_t sg[3], sb[3];
+        if ((rc = ojh_launch_shape(dev, (base + "_px").c_str(), K, N, 1, sg, sb))) return rc;
+        return ojh_launch(dev, (base + "_px").c_str(), {xp, wp, yp}, {K, N}, sg, sb);
     }
     if (m == 1) {
         int r = (accum || bias) ? 4 : pick_rows(dev, N);

@@ -12,8 +12,8 @@ from __future__ import annotations
 
 import numpy as np
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
-BLOCK_SHAPE = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
+Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
+BLOCK_SHAPE = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256), IQ4_NL: (18, 32), IQ4_XS: (136, 256)}
 
 
 def seed_of(*names) -> int:
@@ -116,8 +116,33 @@ def q6k_weights(n: int, k: int, *names) -> np.ndarray:
     return out.reshape(-1)
 
 
+def iq4nl_weights(n: int, k: int, *names) -> np.ndarray:
+    """IQ4_NL rows: per 32-weight block d = f16(|N(0,0.02)| / 127), 16 bytes of uniform codebook indices."""
+    g = rng(*names)
+    nb = n * (k // 32)
+    out = np.empty((nb, 18), np.uint8)
+    d = (np.abs(g.standard_normal(nb) * 0.02) / 127.0).astype(np.float16).view(np.uint16)
+    out[:, 0] = d & 0xFF
+    out[:, 1] = d >> 8
+    out[:, 2:] = g.integers(0, 256, size=(nb, 16), dtype=np.uint8)
+    return out.reshape(-1)
+
+
+def iq4xs_weights(n: int, k: int, *names) -> np.ndarray:
+    """IQ4_XS rows: d = f16(|N(0,0.01)| / 127), the eight 6-bit sub-scales and the 128 index bytes uniform."""
+    g = rng(*names)
+    nb = n * (k // 256)
+    out = np.empty((nb, 136), np.uint8)
+    d = (np.abs(g.standard_normal(nb) * 0.01) / 127.0).astype(np.float16).view(np.uint16)
+    out[:, 0] = d & 0xFF
+    out[:, 1] = d >> 8
+    out[:, 2:] = g.integers(0, 256, size=(nb, 134), dtype=np.uint8)
+    return out.reshape(-1)
+
+
 def weights(ty: int, n: int, k: int, *names) -> np.ndarray:
-    return {Q8_0: q80_weights, Q4_K: q4k_weights, Q5_K: q5k_weights, Q6_K: q6k_weights}[ty](n, k, *names)
+    return {Q8_0: q80_weights, Q4_K: q4k_weights, Q5_K: q5k_weights, Q6_K: q6k_weights,
+            IQ4_NL: iq4nl_weights, IQ4_XS: iq4xs_weights}[ty](n, k, *names)
 
 
 # ------------------------------------------------------------------ the reference tests' procedures

@@ -100,6 +100,8 @@ int ojo_block_shape(uint32_t ty, uint32_t *bytes, uint32_t *weights) { /* synth.
     case OJO_Q4_K: b = 144; w = 256; break;
     case OJO_Q5_K: b = 176; w = 256; break;
     case OJO_Q6_K: b = 210; w = 256; break;
+    case OJO_IQ4_NL: b = 18; w = 32; break;
+    case OJO_IQ4_XS: b = 136; w = 256; break;
     default: return 0;
     }
     if (bytes) *bytes = b;
@@ -136,6 +138,9 @@ int ojo_synth_blocks(uint32_t ty, size_t nb, uint8_t *out) { /* synth.rs:29-64 *
 
 /* ---------------------------------------------------------------- dequant */
 
+/* The 16 levels of the IQ4 codebook (crates/ojas-core/src/iq_tables.rs:881-884). */
+static const int8_t kvalues_iq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
 /* get_scale_min_k4 (gguf.rs:1132-1140; twin cpu_math.rs:566-574). */
 static inline void scale_min_k4(int j, const uint8_t *q, uint8_t *sc, uint8_t *m) {
     if (j < 4) {
@@ -158,6 +163,28 @@ int ojo_dequant_to_f16(const uint8_t *b, uint32_t ty, size_t n, uint16_t *out) {
         case OJO_Q8_0: { /* gguf.rs:704-709 */
             float d = rdh(blk, 0);
             for (int j = 0; j < 32; j++) o[j] = ojo_f32_to_f16(d * (float)(int8_t)blk[2 + j]);
+        } break;
+        case OJO_IQ4_NL: { /* gguf.rs:796-813: low nibbles fill the first half, high nibbles the second */
+            float d = rdh(blk, 0);
+            const uint8_t *qs = blk + 2;
+            for (int j = 0; j < 16; j++) {
+                o[j] = ojo_f32_to_f16(d * (float)kvalues_iq4nl[qs[j] & 0xF]);
+                o[j + 16] = ojo_f32_to_f16(d * (float)kvalues_iq4nl[qs[j] >> 4]);
+            }
+        } break;
+        case OJO_IQ4_XS: { /* gguf.rs:814-840 */
+            float d = rdh(blk, 0);
+            uint16_t sh = (uint16_t)(blk[2] | (blk[3] << 8));
+            const uint8_t *sl = blk + 4, *qs = blk + 8;
+            for (int ib = 0; ib < 8; ib++) {
+                uint32_t ls = (uint32_t)((sl[ib / 2] >> (4 * (ib % 2))) & 0xF) | ((uint32_t)((sh >> (2 * ib)) & 3) << 4);
+                float dl = d * (float)((int32_t)ls - 32);
+                const uint8_t *q = qs + ib * 16;
+                for (int j = 0; j < 16; j++) {
+                    o[ib * 32 + j] = ojo_f32_to_f16(dl * (float)kvalues_iq4nl[q[j] & 0xF]);
+                    o[ib * 32 + j + 16] = ojo_f32_to_f16(dl * (float)kvalues_iq4nl[q[j] >> 4]);
+                }
+            }
         } break;
         case OJO_Q4_K: { /* gguf.rs:1042-1059 */
             float d = rdh(blk, 0), dmin = rdh(blk, 2);
@@ -234,6 +261,25 @@ int ojo_dequant_to_f64(const uint8_t *b, uint32_t ty, size_t n, double *out) {
         case OJO_Q8_0: {
             double d = rdh(blk, 0);
             for (int j = 0; j < 32; j++) o[j] = d * (double)(int8_t)blk[2 + j];
+        } break;
+        case OJO_IQ4_NL: {
+            double d = rdh(blk, 0);
+            for (int j = 0; j < 16; j++) {
+                o[j] = d * (double)kvalues_iq4nl[blk[2 + j] & 0xF];
+                o[j + 16] = d * (double)kvalues_iq4nl[blk[2 + j] >> 4];
+            }
+        } break;
+        case OJO_IQ4_XS: {
+            double d = rdh(blk, 0);
+            uint16_t sh = (uint16_t)(blk[2] | (blk[3] << 8));
+            for (int ib = 0; ib < 8; ib++) {
+                int ls = ((blk[4 + ib / 2] >> (4 * (ib % 2))) & 0xF) | (((sh >> (2 * ib)) & 3) << 4);
+                double dl = d * (double)(ls - 32);
+                for (int j = 0; j < 16; j++) {
+                    o[ib * 32 + j] = dl * (double)kvalues_iq4nl[blk[8 + ib * 16 + j] & 0xF];
+                    o[ib * 32 + j + 16] = dl * (double)kvalues_iq4nl[blk[8 + ib * 16 + j] >> 4];
+                }
+            }
         } break;
         case OJO_Q4_K: case OJO_Q5_K: {
             double d = rdh(blk, 0), dmin = rdh(blk, 2);
@@ -336,6 +382,48 @@ float ojo_dot_q80(const uint8_t *row, const float *x, size_t k) { /* cpu_math.rs
         float acc = 0.0f;
         for (int j = 0; j < 32; j++) acc += (float)(int8_t)blk[2 + j] * xb[j];
         sum += d * acc;
+    }
+    return sum;
+}
+
+float ojo_dot_iq4nl(const uint8_t *row, const float *x, size_t k) { /* cpu_math.rs:993-1010 */
+    float sum = 0.0f;
+    for (size_t b = 0; b < k / 32; b++) {
+        const uint8_t *blk = row + b * 18;
+        const float *xb = x + b * 32;
+        float d = rdh(blk, 0);
+        float bsum = 0.0f;
+        for (int j = 0; j < 16; j++) {
+            uint8_t q = blk[2 + j];
+            bsum += (float)kvalues_iq4nl[q & 0xF] * xb[j];
+            bsum += (float)kvalues_iq4nl[q >> 4] * xb[j + 16];
+        }
+        sum += d * bsum;
+    }
+    return sum;
+}
+
+float ojo_dot_iq4xs(const uint8_t *row, const float *x, size_t k) { /* cpu_math.rs:943-967 */
+    float sum = 0.0f;
+    for (size_t b = 0; b < k / 256; b++) {
+        const uint8_t *blk = row + b * 136;
+        const float *xb = x + b * 256;
+        float d = rdh(blk, 0);
+        uint16_t sh = (uint16_t)(blk[2] | (blk[3] << 8));
+        const uint8_t *sl = blk + 4, *qs = blk + 8;
+        float bsum = 0.0f;
+        for (int g = 0; g < 8; g++) {
+            int32_t ls = (int32_t)((sl[g / 2] >> (4 * (g % 2))) & 0xF) | ((int32_t)((sh >> (2 * g)) & 3) << 4);
+            const float *xg = xb + g * 32;
+            float gsum = 0.0f;
+            for (int j = 0; j < 16; j++) {
+                uint8_t q = qs[16 * g + j];
+                gsum += (float)kvalues_iq4nl[q & 0xF] * xg[j];
+                gsum += (float)kvalues_iq4nl[q >> 4] * xg[j + 16];
+            }
+            bsum += (float)(ls - 32) * gsum;
+        }
+        sum += d * bsum;
     }
     return sum;
 }
@@ -501,6 +589,8 @@ static void kq_row(void *p, size_t row) {
     case OJO_Q4_K: v = ojo_dot_q4k(rb, c->k, c->scales, c->q, c->bsums); break;
     case OJO_Q5_K: v = ojo_dot_q5k(rb, c->k, c->scales, c->q, c->bsums); break;
     case OJO_Q8_0: v = ojo_dot_q80(rb, c->x, c->k); break;
+    case OJO_IQ4_NL: v = ojo_dot_iq4nl(rb, c->x, c->k); break;   /* dot_iq, cpu_math.rs:1131-1141: f32 activations */
+    case OJO_IQ4_XS: v = ojo_dot_iq4xs(rb, c->x, c->k); break;
     default:       v = ojo_dot_q6k(rb, c->k, c->scales, c->q, c->bsums);
     }
     c->y[row] = v;
@@ -514,6 +604,8 @@ int ojo_matvec_kq(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const flo
     case OJO_Q5_K: per256 = 176; break;
     case OJO_Q6_K: per256 = 210; break;
     case OJO_Q8_0: per256 = 272; break;
+    case OJO_IQ4_NL: per256 = 144; break;
+    case OJO_IQ4_XS: per256 = 136; break;
     default: return -1;
     }
     size_t nsb = (k + 255) / 256;

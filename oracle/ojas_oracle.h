@@ -11,10 +11,12 @@
  *
  * How each function is pinned (a function without such a check would say "parity unpinned"):
  *   dequant Q4_K/Q5_K/Q6_K  FNV-1a digests held by crates/ojas-formats/tests/quant_formats.rs:38-40
+ *   dequant IQ4_NL/IQ4_XS   the digests of the same table (quant_formats.rs:45,48), one-hot codes vs the codebook
  *   dequant Q8_0            closed form of crates/ojas-formats/tests/rows.rs:13-18
  *   f16 <-> f32             the digests above + exhaustive comparison with IEEE binary16 (numpy)
  *   quant_q8k               invariants (max|q|=127, bsums, half-away rounding, |x-s*q|<=s/2)
  *   dot_q80                 f64 dot over the dequantized row, brute force at K=32
+ *   dot_iq4nl / dot_iq4xs   f64 dot over the dequantized row (the check of cpu_math.rs:1206-1285), one-hot activations
  *   dot_q4k/q5k/q6k         identity dot(row, quant(x)) == sum dequant(row)*(scale*q) in f64,
  *                           one-hot activations (pins nibble / sub-block order)
  *   relayout_q4k_q4l        qa*nib+qb == dequant up to the two f16 roundings, one-hot blocks
@@ -33,7 +35,7 @@ extern "C" {
 #endif
 
 /* GGUF type ids (crates/ojas-formats/src/gguf.rs:563-591). */
-enum { OJO_Q8_0 = 8, OJO_Q4_K = 12, OJO_Q5_K = 13, OJO_Q6_K = 14 };
+enum { OJO_Q8_0 = 8, OJO_Q4_K = 12, OJO_Q5_K = 13, OJO_Q6_K = 14, OJO_IQ4_NL = 20, OJO_IQ4_XS = 23 };
 
 /* IEEE binary16 <-> binary32, round-to-nearest-even, subnormals kept
  * (crate half 2.7.1; call sites gguf.rs:602-608). */
@@ -66,6 +68,8 @@ void ojo_quant_q8k(const float *x, size_t k, float *scales, int8_t *q, int32_t *
 
 /* Row dots (cpu_math.rs:971-981, :609-635, :638-670, :674-722). */
 float ojo_dot_q80(const uint8_t *row, const float *x, size_t k);
+float ojo_dot_iq4nl(const uint8_t *row, const float *x, size_t k);
+float ojo_dot_iq4xs(const uint8_t *row, const float *x, size_t k);
 float ojo_dot_q4k(const uint8_t *row, size_t k, const float *scales, const int8_t *q, const int32_t *bsums);
 float ojo_dot_q5k(const uint8_t *row, size_t k, const float *scales, const int8_t *q, const int32_t *bsums);
 float ojo_dot_q6k(const uint8_t *row, size_t k, const float *scales, const int8_t *q, const int32_t *bsums);

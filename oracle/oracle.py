@@ -15,7 +15,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libojas_oracle.so")
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 
 
 def build(force: bool = False) -> str:
@@ -50,8 +50,10 @@ def lib() -> C.CDLL:
         L.ojo_digest_f16.argtypes = [vp, sz]
         L.ojo_quant_q8k.restype = None
         L.ojo_quant_q8k.argtypes = [vp, sz, vp, vp, vp]
-        L.ojo_dot_q80.restype = C.c_float
-        L.ojo_dot_q80.argtypes = [vp, vp, sz]
+        for name in ("ojo_dot_q80", "ojo_dot_iq4nl", "ojo_dot_iq4xs"):
+            f = getattr(L, name)
+            f.restype = C.c_float
+            f.argtypes = [vp, vp, sz]
         for name in ("ojo_dot_q4k", "ojo_dot_q5k", "ojo_dot_q6k"):
             f = getattr(L, name)
             f.restype = C.c_float
@@ -138,6 +140,14 @@ def dot_q80(row: np.ndarray, x: np.ndarray) -> float:
     row = np.ascontiguousarray(row, np.uint8)
     x = np.ascontiguousarray(x, np.float32)
     return float(lib().ojo_dot_q80(_p(row), _p(x), x.size))
+
+
+def dot_iq(ty: int, row: np.ndarray, x: np.ndarray) -> float:
+    """dot_iq4nl / dot_iq4xs: raw row against f32 activations."""
+    fn = {IQ4_NL: lib().ojo_dot_iq4nl, IQ4_XS: lib().ojo_dot_iq4xs}[ty]
+    row = np.ascontiguousarray(row, np.uint8)
+    x = np.ascontiguousarray(x, np.float32)
+    return float(fn(_p(row), _p(x), x.size))
 
 
 def dot_kq(ty: int, row: np.ndarray, k: int, act) -> float:

@@ -3,8 +3,9 @@ import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
-DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6}
+Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
+DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6,
+           IQ4_NL: 0xA5D4CF4E5DB3A1BF, IQ4_XS: 0x1429CAFB4DF9AF64}
 
 
 def _dequant(gpu, ty, raw, n):
@@ -14,16 +15,17 @@ def _dequant(gpu, ty, raw, n):
     return gpu.read(out, n, np.uint16)
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
-def test_reference_digests_on_device(gpu, orc, ty):
-    """The reference's own regression digests (crates/ojas-formats/tests/quant_formats.rs:38-40),
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
+def test_reference_digests_on_device(gpu, orc, pkg, ty):
+    """The reference's own regression digests (crates/ojas-formats/tests/quant_formats.rs:38-48),
     computed over what the GPU decoded."""
     raw = orc.synth_blocks(ty, 40)
-    bits = _dequant(gpu, ty, raw, 10240)
+    bits = _dequant(gpu, ty, raw, 40 * pkg.synth.BLOCK_SHAPE[ty][1])
     assert orc.digest_f16(bits) == DIGESTS[ty]
 
 
-@pytest.mark.parametrize("ty,n,k", [(Q8_0, 37, 4096), (Q4_K, 129, 4096), (Q6_K, 65, 4096), (Q5_K, 16, 1024)])
+@pytest.mark.parametrize("ty,n,k", [(Q8_0, 37, 4096), (Q4_K, 129, 4096), (Q6_K, 65, 4096), (Q5_K, 16, 1024),
+                                    (IQ4_NL, 33, 2080), (IQ4_XS, 21, 4096)])
 def test_bit_exact_on_benchmark_distributions(gpu, orc, pkg, ty, n, k):
     raw = orc.synth_blocks(ty, n * k // pkg.synth.BLOCK_SHAPE[ty][1]) if ty == Q5_K else \
         pkg.synth.weights(ty, n, k, "dq", ty)
@@ -31,7 +33,7 @@ def test_bit_exact_on_benchmark_distributions(gpu, orc, pkg, ty, n, k):
     assert np.array_equal(got, orc.dequant_to_f16(raw, ty, n * k))
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
 def test_bit_exact_with_extreme_scales(gpu, orc, pkg, ty):
     """Subnormal, tiny, huge and negative f16 scales: every rounding path of the decoder."""
     bb, wpb = pkg.synth.BLOCK_SHAPE[ty]

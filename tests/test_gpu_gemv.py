@@ -12,7 +12,7 @@ import pytest
 from conftest import peak_err
 
 pytestmark = pytest.mark.gpu
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 TAG = {Q8_0: "q80", Q4_K: "q4k", Q5_K: "q5k", Q6_K: "q6k"}
 TOL_Q8K = 1e-3     # the parity bar against the CPU reference
 TOL_Q8K_SEEN = 2e-5
@@ -68,7 +68,7 @@ def test_q8k_matvec_matches_cpu_reference(gpu, orc, pkg, ty, n, k):
     assert err <= TOL_Q8K_SEEN <= TOL_Q8K, err
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q6_K, IQ4_NL, IQ4_XS])
 @pytest.mark.parametrize("n,k", [(13, 2560), (1024, 4096), (96, 14336), (4099, 4096)])
 def test_float_matvec_matches_dequant_dot(gpu, orc, pkg, ty, n, k):
     w, x = _inputs(pkg, ty, n, k, "b")
@@ -95,6 +95,25 @@ def test_q80_matvec_matches_dot_q80(gpu, orc, pkg):
     assert peak_err(gpu.read(yd, n), want) <= 1e-5
 
 
+@pytest.mark.parametrize("ty", [IQ4_NL, IQ4_XS])
+@pytest.mark.parametrize("n,k,m", [(4096, 4096, 1), (37, 256, 1), (130, 2816, 5), (1000, 1024, 2), (33001, 2816, 1),
+                                   (40000, 4096, 1), (32768, 256, 1)])
+def test_iq4_rows_match_the_cpu_dots(gpu, orc, pkg, ty, n, k, m):
+    """IQ4_NL / IQ4_XS rows against `matvec_kq`, which sends these types to dot_iq4nl / dot_iq4xs on
+    f32 activations (crates/ojas-cpu/src/cpu_math.rs:1179); the int8-activation contract is refused."""
+    w = pkg.synth.weights(ty, n, k, "iq4", ty, n, k)
+    x = pkg.synth.normal_f32(m * k, "iq4", "x", ty, m, k).reshape(m, k)
+    lin = gpu.lin(ty, n, k, w)
+    yd = gpu.upload(np.full(m * n + 2, 12345.0, np.float32))
+    gpu.mm(gpu.upload(x), lin, yd, m, y_off=4)
+    got = gpu.read(yd, m * n + 2)
+    assert got[0] == 12345.0 and got[-1] == 12345.0, "wrote outside y"
+    for t in range(m):
+        assert peak_err(got[1 + t * n:1 + (t + 1) * n], orc.matvec_kq(w, ty, n, k, x[t])) <= 1e-5, t
+    with pytest.raises(pkg.OjasHipError, match="f32 activations"):
+        gpu.mm(gpu.upload(x), lin, yd, m, act_mode=pkg.ACT_Q8K)
+
+
 def test_q80_closed_form_rows_with_guards(gpu, pkg):
     """crates/ojas-metal/tests/dispatch.rs:357-429: K=2560, N=13, output between sentinels,
     absolute tolerance 2e-4 against an f64 loop over the same bytes."""
@@ -112,13 +131,13 @@ def test_q80_closed_form_rows_with_guards(gpu, pkg):
     assert np.max(np.abs(got[2:-2] - want)) < 2e-4
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
 @pytest.mark.parametrize("mode", ["float", "q8k"])
 def test_bias_accum_and_batched_variants(gpu, orc, pkg, ty, mode):
     """The five checks of crates/ojas-models/examples/nat_gemv_gate.rs:36-163: plain, bias
     (1000 + i), accumulate onto a seeded y, batched M=3 with different rows, batched accumulate."""
-    if ty == Q8_0 and mode == "q8k":
-        pytest.skip("Q8_0 keeps f32 activations in the CPU reference")
+    if ty in (Q8_0, IQ4_NL, IQ4_XS) and mode == "q8k":
+        pytest.skip("this format keeps f32 activations in the CPU reference")
     if ty == Q5_K and mode == "float":
         pytest.skip("Q5_K has the int8-activation matvec only")
     n, k, m = 200, 1024, 3

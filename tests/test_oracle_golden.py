@@ -3,21 +3,25 @@ brute force — each chosen so that a dropped term, a wrong index or a transpose
 import numpy as np
 import pytest
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 
-# crates/ojas-formats/tests/quant_formats.rs:38-40
-DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6}
+# crates/ojas-formats/tests/quant_formats.rs:38-40, 45, 48
+DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6,
+           IQ4_NL: 0xA5D4CF4E5DB3A1BF, IQ4_XS: 0x1429CAFB4DF9AF64}
+# crates/ojas-core/src/iq_tables.rs:881-884
+KVALUES_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float64)
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
-def test_dequant_digest_matches_reference(orc, ty):
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
+def test_dequant_digest_matches_reference(orc, pkg, ty):
+    wpb = pkg.synth.BLOCK_SHAPE[ty][1]
     raw = orc.synth_blocks(ty, 40)
-    bits = orc.dequant_to_f16(raw, ty, 40 * 256)
-    assert bits.size == 10240
+    bits = orc.dequant_to_f16(raw, ty, 40 * wpb)
+    assert bits.size == 40 * wpb                      # 10240 values; 1280 for the 32-weight IQ4_NL block
     assert orc.digest_f16(bits) == DIGESTS[ty]
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
 def test_synth_blocks_two_implementations_agree(orc, pkg, ty):
     assert np.array_equal(orc.synth_blocks(ty, 9), pkg.synth.synth_blocks(ty, 9))
 
@@ -166,6 +170,49 @@ def test_dot_q80_matches_f64_dot(orc, pkg):
         acc = np.float32(acc + np.float32(np.int8(blk[2 + j])) * x[j])
     d = blk[0:2].view(np.float16).astype(np.float32)[0]
     assert orc.dot_q80(blk, x[:32]) == np.float32(d * acc)
+
+
+def test_iq4_closed_forms(orc):
+    """A block whose every index is c decodes to d * codebook[c] (IQ4_NL) and d * (ls - 32) * codebook[c]
+    (IQ4_XS); low nibbles fill the first 16 weights of a 32-group, high nibbles the next 16; the 6-bit
+    sub-scale is 4 low bits from scales_l (nibble per sub-block) and 2 high bits from scales_h."""
+    d = np.array([0.5], np.float16).view(np.uint8)
+    for c in range(16):
+        blk = np.concatenate([d, np.full(16, c | ((15 - c) << 4), np.uint8)])
+        w = orc.dequant_to_f64(blk, IQ4_NL, 32)
+        assert np.all(w[:16] == 0.5 * KVALUES_IQ4NL[c]) and np.all(w[16:] == 0.5 * KVALUES_IQ4NL[15 - c])
+    for ib in range(8):
+        for ls in (0, 31, 32, 47, 63):
+            blk = np.zeros(136, np.uint8)
+            blk[0:2] = d
+            sh = (ls >> 4) << (2 * ib)
+            blk[2], blk[3] = sh & 0xFF, sh >> 8
+            blk[4 + ib // 2] = (ls & 0xF) << (4 * (ib % 2))
+            blk[8:] = 0x9C                     # low nibble 12 -> 53, high nibble 9 -> 13
+            w = orc.dequant_to_f64(blk, IQ4_XS, 256).reshape(8, 32)
+            for jb in range(8):
+                scale = 0.5 * ((ls if jb == ib else 0) - 32)
+                assert np.all(w[jb, :16] == scale * 53) and np.all(w[jb, 16:] == scale * 13), (ib, ls, jb)
+
+
+@pytest.mark.parametrize("ty", [IQ4_NL, IQ4_XS])
+def test_iq4_dot_matches_f64_dot(orc, pkg, ty):
+    """dot_iq4nl / dot_iq4xs against the dequantized row in double (the reference's own check,
+    crates/ojas-cpu/src/cpu_math.rs:1206-1285), one-hot activations (element order), matvec_kq routing."""
+    n, k = 5, 1024
+    bb, wpb = pkg.synth.BLOCK_SHAPE[ty]
+    rb = k // wpb * bb
+    raw = orc.synth_blocks(ty, n * k // wpb)
+    x = pkg.synth.normal_f32(k, "t", "xiq", ty)
+    w = orc.dequant_to_f64(raw, ty, n * k).reshape(n, k)
+    want = w @ x.astype(np.float64)
+    got = np.array([orc.dot_iq(ty, raw[r * rb:(r + 1) * rb], x) for r in range(n)])
+    assert np.max(np.abs(got - want)) <= 2e-6 * np.max(np.abs(want))
+    assert np.array_equal(orc.matvec_kq(raw, ty, n, k, x, threads=3), got.astype(np.float32))
+    for i in [0, 1, 15, 16, 17, 31, 32, 47, 48, 255, 256, 272, 1023]:
+        e = np.zeros(k, np.float32)
+        e[i] = 1.0
+        assert orc.dot_iq(ty, raw[:rb], e) == np.float32(w[0, i]), (ty, i)
 
 
 @pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
