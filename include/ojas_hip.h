@@ -54,7 +54,10 @@ enum { OJH_X_F32 = 0, OJH_X_BF16 = 1, OJH_X_F16 = 2 };
 /* Arithmetic contract of a matmul.
  *   OJH_ACT_Q8K — activations quantized to int8 per 256 (quant_q8k), integer dots: the arithmetic
  *                 of the CPU reference `matvec_kq` (crates/ojas-cpu/src/cpu_math.rs:1145-1189).
- *                 Q8_0 weights always take f32 activations, as `dot_q80` does (:971-981).
+ *                 Q8_0, IQ4_NL and IQ4_XS weights always take f32 activations, as `dot_q80`,
+ *                 `dot_iq4nl` and `dot_iq4xs` do (:971-981, :993-1010, :943-967): asking for
+ *                 OJH_ACT_Q8K on IQ4 rows is refused, and no MFMA tile reads them (every token
+ *                 count runs on the matvec entries).
  *   OJH_ACT_FLOAT — activations kept in floating point (f32 for the GEMV, rounded to f16 into the
  *                 MFMA tile for the GEMM): the contract of the reference's GPU kernels
  *                 (crates/ojas-core/src/quant_src.rs:779-867, crates/ojas-cuda/src/kernels/gemm_q.rs:1-56).
