@@ -81,12 +81,10 @@ __device__ __forceinline__ float q4k_lane_dot_f(uint4 hdr, uint4 qs, uint c, con
 }
 
 template <int R, int MODE>
-__device__ __forceinline__ void gemv_nat_q4k_body(const float* __restrict__ x, const uchar* __restrict__ w,
+__device__ __forceinline__ void gemv_nat_q4k_rows(const float* __restrict__ x, const uchar* __restrict__ w,
                                                   float* __restrict__ y, const float* __restrict__ bs,
-                                                  uint K, uint N) {
+                                                  uint K, uint N, uint row0) {
     const uint lane = threadIdx.x & 63u;
-    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
-    if (row0 >= N) return;
     const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
     float acc[R];
 #pragma unroll
@@ -109,6 +107,14 @@ __device__ __forceinline__ void gemv_nat_q4k_body(const float* __restrict__ x, c
         float t = wave_sum(acc[r]);
         if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, t);
     }
+}
+
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_q4k_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                  float* __restrict__ y, const float* __restrict__ bs,
+                                                  uint K, uint N) {
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 < N) gemv_nat_q4k_rows<R, MODE>(x, w, y, bs, K, N, row0);
 }
 
 template <int MT>
@@ -143,6 +149,53 @@ __device__ __forceinline__ void gemv_nat_q4k_m_body(const float* __restrict__ x,
         }
     }
 }
+
+// Many rows (an output head, K <= 4096): rows grid-stride, two per wave and step, and the wave's share of
+// the f32 activations — two fragments of 32 floats and their sums per lane — stays in registers for the
+// whole launch.  With a fragment fetched per row group the launch is bound by those fetches (eight
+// 16-byte loads per lane against two for the weights), not by HBM.  Same lane arithmetic and order
+// as the entries above: the same bits.   gemv_nat_q4k_px(x, w, y, K, N)
+__device__ __forceinline__ void gemv_nat_q4k_px_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                     float* __restrict__ y, uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    Q4kFragF f[2];
+    uint sbc[2];
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+        const uint sb = g + 8u * (uint)s;
+        sbc[s] = min(sb, nsb - 1u);
+        f[s] = q4k_load_frag_f(x, sbc[s], l);
+        if (sb >= nsb) {                              // a step past K: zeros, so that its repeated block adds nothing
+#pragma unroll
+            for (int i = 0; i < 4; i++) f[s].xl[i] = f[s].xh[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            f[s].sl = f[s].sh = 0.0f;
+        }
+    }
+    const uint nwaves = gridDim.x * (blockDim.x >> 6);
+    for (uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2u; row0 < N; row0 += nwaves * 2u) {
+        const uchar* r0 = w + (size_t)row0 * nsb * Q4K_BYTES;
+        const uchar* r1 = w + (size_t)min(row0 + 1u, N - 1u) * nsb * Q4K_BYTES;
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const uchar* b0 = r0 + (size_t)sbc[s] * Q4K_BYTES;
+            const uchar* b1 = r1 + (size_t)sbc[s] * Q4K_BYTES;
+            const uint4 h0 = *(const uint4*)b0, q0 = *(const uint4*)(b0 + 16u + l * 16u);
+            const uint4 h1 = *(const uint4*)b1, q1 = *(const uint4*)(b1 + 16u + l * 16u);
+            a0 += q4k_lane_dot_f(h0, q0, c, f[s]);
+            a1 += q4k_lane_dot_f(h1, q1, c, f[s]);
+        }
+        a0 = wave_sum(a0);
+        a1 = wave_sum(a1);
+        if (lane == 0) {
+            y[row0] = a0;
+            if (row0 + 1u < N) y[row0 + 1u] = a1;
+        }
+    }
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemv_nat_q4k_px(const float* x, const uchar* w, float* y, uint K, uint N) { gemv_nat_q4k_px_body(x, w, y, K, N); }
 
 // ------------------------------------------------------------------ Q6_K
 // Lane (g, t) = (lane/16, lane%16): half hf = t/8, weights l0..l0+3 (l0 = 4*(t%8)) of each of the
@@ -197,12 +250,10 @@ __device__ __forceinline__ float q6k_lane_dot_f(const Q6kRaw& r, const Q6kFragF&
 }
 
 template <int R, int MODE>
-__device__ __forceinline__ void gemv_nat_q6k_body(const float* __restrict__ x, const uchar* __restrict__ w,
+__device__ __forceinline__ void gemv_nat_q6k_rows(const float* __restrict__ x, const uchar* __restrict__ w,
                                                   float* __restrict__ y, const float* __restrict__ bs,
-                                                  uint K, uint N) {
+                                                  uint K, uint N, uint row0) {
     const uint lane = threadIdx.x & 63u;
-    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
-    if (row0 >= N) return;
     const uint nsb = K >> 8, g = lane >> 4, t = lane & 15u, hf = t >> 3, l0 = (t & 7u) * 4u;
     float acc[R];
 #pragma unroll
@@ -223,6 +274,14 @@ __device__ __forceinline__ void gemv_nat_q6k_body(const float* __restrict__ x, c
         float s = wave_sum(acc[r]);
         if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, s);
     }
+}
+
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_q6k_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                  float* __restrict__ y, const float* __restrict__ bs,
+                                                  uint K, uint N) {
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 < N) gemv_nat_q6k_rows<R, MODE>(x, w, y, bs, K, N, row0);
 }
 
 template <int MT>
@@ -255,6 +314,50 @@ __device__ __forceinline__ void gemv_nat_q6k_m_body(const float* __restrict__ x,
         }
     }
 }
+
+// The same for Q6_K rows: four fragments of 16 floats and their sums per lane (K <= 4096).
+//   gemv_nat_q6k_px(x, w, y, K, N)
+__device__ __forceinline__ void gemv_nat_q6k_px_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                     float* __restrict__ y, uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint nsb = K >> 8, g = lane >> 4, t = lane & 15u, hf = t >> 3, l0 = (t & 7u) * 4u;
+    Q6kFragF f[4];
+    uint sbc[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const uint sb = g + 4u * (uint)s;
+        sbc[s] = min(sb, nsb - 1u);
+        f[s] = q6k_load_frag_f(x, sbc[s], hf, l0);
+        if (sb >= nsb) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                f[s].x[q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                f[s].s[q] = 0.0f;
+            }
+        }
+    }
+    const uint nwaves = gridDim.x * (blockDim.x >> 6);
+    for (uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2u; row0 < N; row0 += nwaves * 2u) {
+        const uchar* r0 = w + (size_t)row0 * nsb * Q6K_BYTES;
+        const uchar* r1 = w + (size_t)min(row0 + 1u, N - 1u) * nsb * Q6K_BYTES;
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const Q6kRaw w0 = q6k_load_raw(r0 + (size_t)sbc[s] * Q6K_BYTES, hf, l0);
+            const Q6kRaw w1 = q6k_load_raw(r1 + (size_t)sbc[s] * Q6K_BYTES, hf, l0);
+            a0 += q6k_lane_dot_f(w0, f[s]);
+            a1 += q6k_lane_dot_f(w1, f[s]);
+        }
+        a0 = wave_sum(a0);
+        a1 = wave_sum(a1);
+        if (lane == 0) {
+            y[row0] = a0;
+            if (row0 + 1u < N) y[row0 + 1u] = a1;
+        }
+    }
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemv_nat_q6k_px(const float* x, const uchar* w, float* y, uint K, uint N) { gemv_nat_q6k_px_body(x, w, y, K, N); }
 
 // ------------------------------------------------------------------ Q8_0
 // Four lanes share a 34-byte block (8 int8 each); a wave walks 16 blocks (512 weights) per step.
@@ -348,8 +451,6 @@ __device__ __forceinline__ void gemv_nat_q80_m_body(const float* __restrict__ x,
 // IQ4_NL: 18-byte blocks {f16 d; qs[16]}, four lanes per block, a wave walks 16 blocks per step.
 // IQ4_XS: 136-byte super-blocks {f16 d; u16 scales_h; u8 scales_l[4]; qs[128]}, 32 lanes per
 // super-block (lane / 4 = sub-block, its 6-bit scale minus 32 times d applied per lane).
-typedef uint u32_a2 __attribute__((aligned(2)));
-
 __device__ __forceinline__ float iq4_lane_dot(uint q, float4 x0, float4 x1) {
     const uint lo = iq4_levels4(q & 0x0F0F0F0Fu), hi = iq4_levels4((q >> 4) & 0x0F0F0F0Fu);
     float a = sb0(lo) * x0.x;

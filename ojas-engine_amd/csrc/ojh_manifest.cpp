@@ -266,7 +266,7 @@ static int check_gemv_q8k_px(const ojh_kernel_spec *s, const uint32_t *c, const 
     align[3] = 4;
     return OJH_OK;
 }
-// gemv_nat_iq4{nl,xs}_px(x, w, y, K, N): rows grid-stride, two per wave and step, f32 activations in registers
+// gemv_nat_{q4k,q6k,iq4nl,iq4xs}_px(x, w, y, K, N): rows grid-stride, two per wave and step, f32 activations in registers
 static int check_gemv_nat_px(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                              const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f;
@@ -982,10 +982,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g + "_accum", "gemv", 3, 2, f.type, 4, check_gemv_nat, shape_rows);
         add(g + "_bias", "gemv", 4, 2, f.type, 4, check_gemv_nat, shape_rows);
         add(g + "_m", "gemv", 3, 4, f.type, 1, check_gemv_nat_m, shape_rows);
-        if (f.type == OJH_IQ4_NL || f.type == OJH_IQ4_XS) {   // f32 activations only, no MFMA tile
-            add(g + "_px", "gemv", 3, 2, f.type, 2, check_gemv_nat_px, shape_px);
-            continue;
-        }
+        if (f.type != OJH_Q8_0) add(g + "_px", "gemv", 3, 2, f.type, 2, check_gemv_nat_px, shape_px);
+        if (f.type == OJH_IQ4_NL || f.type == OJH_IQ4_XS) continue;   // f32 activations only, no MFMA tile
         if (f.type == OJH_Q8_0) {
             add(g + "_lds", "gemv", 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
             add(g + "_lds_accum", "gemv", 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);

@@ -462,14 +462,17 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         return ojh_launch(dev, accum ? "gemv_nat_q80_lds_accum" : bias ? "gemv_nat_q80_lds_bias" : "gemv_nat_q80_lds", p,
                           {K, N, ojh_q80_lds_kc(K)}, sg, sb);
     }
-    // IQ4 rows of an output head: rows grid-stride, the wave's f32 activations in registers
-    if (m == 1 && iq4 && dev->px && !accum && !bias && N >= 32768u && K <= 4096u) {
+    // an output head (K-quant or IQ4 rows): rows grid-stride, the wave's f32 activations in registers
+    if (m == 1 && w->type != OJH_Q8_0 && dev->px && !accum && !bias && N >= 32768u && K <= 4096u) {
         uint32_t sg[3], sb[3];
         if ((rc = ojh_launch_shape(dev, (base + "_px").c_str(), K, N, 1, sg, sb))) return rc;
         return ojh_launch(dev, (base + "_px").c_str(), {xp, wp, yp}, {K, N}, sg, sb);
     }
     if (m == 1) {
-        int r = (accum || bias) ? 4 : pick_rows(dev, N);
+        // rows per wave for the f32-activation kernels (measured on Q4_K and Q6_K, K = 4096 and 14336): the
+        // activation fragment is 4 bytes per weight, so sharing it pays earlier than for int8 activations —
+        // two rows everywhere, four from 8192 Q4_K rows; one row only when told to
+        int r = (accum || bias) ? 4 : dev->gemv_rows_override ? pick_rows(dev, N) : (w->type == OJH_Q4_K && N >= 8192u) ? 4 : 2;
         std::string name = base + (accum ? "_accum" : bias ? "_bias" : r == 4 ? "" : r == 2 ? "_r2" : "_r1");
         grid[0] = (N + 4 * r - 1) / (4 * r);
         std::vector<void *> p = {xp, wp, yp};

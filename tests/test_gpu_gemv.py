@@ -95,6 +95,34 @@ def test_q80_matvec_matches_dot_q80(gpu, orc, pkg):
     assert peak_err(gpu.read(yd, n), want) <= 1e-5
 
 
+@pytest.mark.parametrize("ty,tag", [(Q4_K, "q4k"), (Q6_K, "q6k")])
+@pytest.mark.parametrize("n,k", [(33000, 256), (40001, 2560), (32768, 4096)])
+def test_float_head_form_keeps_activations_in_registers(gpu, orc, pkg, ty, tag, n, k):
+    """From 32768 rows a float-activation matvec runs grid-stride with the wave's f32 activations in
+    registers: the lane arithmetic and order of the row-per-wave kernels, so the same bits (checked by
+    name against `_r2`), and the dequantized dot in f64; partly filled steps (K = 256, 2560), odd rows."""
+    w, x = _inputs(pkg, ty, n, k, "fpx")
+    gpu.ensure_family("gemv")
+    wd, xd = gpu.upload_bytes(w), gpu.upload(x)
+    outs = []
+    for name in (f"gemv_nat_{tag}_px", f"gemv_nat_{tag}_r2"):
+        grid, block = gpu.launch_shape(name, k, n, 1)
+        yd = gpu.upload(np.full(n + 2, 12345.0, np.float32))
+        gpu.dispatch(gpu.begin(), name, [(xd, 0), (wd, 0), (yd, 4)], [k, n], grid, block)
+        got = gpu.read(yd, n + 2)
+        assert got[0] == 12345.0 and got[-1] == 12345.0, "wrote outside y"
+        outs.append(got[1:-1].copy())
+    assert np.array_equal(outs[0], outs[1])
+    assert peak_err(outs[0], orc.matmul_ref(w, ty, n, k, x)[0]) <= TOL_FLOAT
+    # the router takes it for a plain store
+    lin = gpu.lin(ty, n, k, w)
+    yr = gpu.alloc(n)
+    gpu.mm(xd, lin, yr, 1, act_mode=pkg.ACT_FLOAT)
+    assert np.array_equal(gpu.read(yr, n), outs[0])
+    with pytest.raises(pkg.OjasHipError, match="registers"):
+        gpu.dispatch(gpu.begin(), f"gemv_nat_{tag}_px", [(xd, 0), (wd, 0), (yr, 0)], [4352, n, ], [8, 1, 1], [256, 1, 1])
+
+
 @pytest.mark.parametrize("ty", [IQ4_NL, IQ4_XS])
 @pytest.mark.parametrize("n,k,m", [(4096, 4096, 1), (37, 256, 1), (130, 2816, 5), (1000, 1024, 2), (33001, 2816, 1),
                                    (40000, 4096, 1), (32768, 256, 1)])
