@@ -614,7 +614,9 @@ int ojo_matvec_kq(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const flo
     int32_t *bsums = (int32_t *)malloc(nsb * 8 * sizeof(int32_t));
     ojo_quant_q8k(x, k, scales, q, bsums); /* done for every type, used by the K-quants */
     struct kq_ctx c = { raw, ty, k, k / 256 * per256, x, scales, q, bsums, y };
+    /* (the reference's k / 256 form covers whole multiples of 256 only; rows of 32-weight blocks are sized per block here) */
     if (ty == OJO_Q8_0) c.row_bytes = k / 32 * 34;
+    if (ty == OJO_IQ4_NL) c.row_bytes = k / 32 * 18;
     steal_rows(n, 8, threads, kq_row, &c);
     free(scales); free(q); free(bsums);
     return 0;

@@ -8,7 +8,7 @@ import pytest
 import gguf_writer as gw
 from conftest import peak_err
 
-Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q8_0, Q4_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 14, 20, 23
 
 
 def _model(pkg, tmp_path, alignment=None, version=3):
@@ -19,6 +19,9 @@ def _model(pkg, tmp_path, alignment=None, version=3):
         "blk.0.attn_v.weight": (pkg.synth.q4k_weights(16, k, "gguf", "v"), [k, 16], Q4_K),
         "output.weight": (pkg.synth.q6k_weights(40, k, "gguf", "o"), [k, 40], Q6_K),
         "tok.weight": (pkg.synth.q80_weights(24, 64, "gguf", "e"), [64, 24], Q8_0),
+        "blk.0.ffn_up.weight": (pkg.synth.iq4xs_weights(48, k, "gguf", "u"), [k, 48], IQ4_XS),
+        "blk.0.ffn_gate.weight": (pkg.synth.iq4xs_weights(48, k, "gguf", "g"), [k, 48], IQ4_XS),
+        "blk.0.ffn_down.weight": (pkg.synth.iq4nl_weights(40, 96, "gguf", "d"), [96, 40], IQ4_NL),
         "norm.weight": (pkg.synth.normal_f32(k, "gguf", "n"), [k], 0),
     }
     meta = [("general.architecture", gw.STR, "llama"), ("llama.block_count", gw.U32, 1),
@@ -112,6 +115,18 @@ def test_lin_load_stacks_tensors_and_keeps_the_files_bytes(gpu, orc, pkg, tmp_pa
     y3 = gpu.alloc(24)
     gpu.mm(gpu.upload(x64), emb, y3, 1)
     assert peak_err(gpu.read(y3, 24), orc.matvec_kq(t["tok.weight"][0], Q8_0, 24, 64, x64)) <= 1e-5
+    # IQ4 tensors stay in their block bytes too and stack like the others (f32 activations)
+    gu = gpu.lin_load(g, ["blk.0.ffn_gate.weight", "blk.0.ffn_up.weight"])
+    assert (gu.n, gu.k, gu.ty) == (96, k, IQ4_XS)
+    y4 = gpu.alloc(96)
+    gpu.mm(gpu.upload(x), gu, y4, 1)
+    both = np.concatenate([t["blk.0.ffn_gate.weight"][0], t["blk.0.ffn_up.weight"][0]])
+    assert peak_err(gpu.read(y4, 96), orc.matvec_kq(both, IQ4_XS, 96, k, x)) <= 1e-5
+    dn = gpu.lin_load(g, ["blk.0.ffn_down.weight"])
+    x96 = pkg.synth.normal_f32(96, "gguf", "x96")
+    y5 = gpu.alloc(40)
+    gpu.mm(gpu.upload(x96), dn, y5, 1)
+    assert peak_err(gpu.read(y5, 40), orc.matvec_kq(t["blk.0.ffn_down.weight"][0], IQ4_NL, 40, 96, x96)) <= 1e-5
     with pytest.raises(pkg.OjasHipError, match="type differs"):
         gpu.lin_load(g, ["blk.0.attn_q.weight", "output.weight"])
     with pytest.raises(pkg.OjasHipError, match="K 64 differs"):
