@@ -204,7 +204,7 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
     }
     const size_t w_bytes = w->row_bytes * N;
     const bool dwords_ok = (uintptr_t)wp % 4 == 0 && (w_bytes % 4 == 0 || w->off + w_bytes + 2 <= w->raw->bytes);
-    // Q6_K rows against 2 .. 64 tokens on the int8 matrix cores (beyond 16 tokens as launches of 16 or 8:
+    // Q6_K rows against 2 or more tokens on the int8 matrix cores (beyond 16 tokens as launches of 16 or 8:
     // each streams the rows once, which the per-token loop of the general entry does sixteen times
     // over).  Three shapes of the same tile arithmetic, picked by what was measured on K = 4096 and 14336:
     //   many rows (eight tiles per CU and wave, 32768 rows on this GPU): a wave per tile, rows copied
@@ -213,7 +213,7 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
     //     the integer-dot entry from 5 tokens (from 3 when K is long) and the only one that holds 8 tokens
     //     of K = 14336;
     //   between: a wave per tile with direct loads, ahead of the integer-dot entry from 5 tokens.
-    if (w->type == OJH_Q6_K && m >= 2 && m <= 64) {
+    if (w->type == OJH_Q6_K && m >= 2) {
         const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount, tiles = (N + 15) / 16;
         const uint32_t mc16 = m <= 8 ? m : 16;
         const bool ml_fits = dev->q6k_ml && (uint64_t)w_bytes <= 0xFFFFFFFFull && ojh_q6k_ml_lds(K, mc16) <= 163840;

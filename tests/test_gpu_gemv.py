@@ -413,7 +413,8 @@ def test_q80_rows_staged_through_lds(pkg, orc, monkeypatch, n, k):
 
 @pytest.mark.parametrize("m,n,k,accum", [(4, 50, 256, False), (8, 130, 4096, True), (9, 301, 4096, False),
                                          (16, 1000, 4096, False), (16, 17, 512, True), (12, 4099, 2560, False),
-                                         (6, 64, 7168, False), (40, 300, 4096, True), (64, 33, 1024, False)])
+                                         (6, 64, 7168, False), (40, 300, 4096, True), (64, 33, 1024, False),
+                                         (150, 40, 512, False)])
 def test_q6k_tokens_on_the_int8_matrix_cores(gpu, orc, pkg, m, n, k, accum):
     """5 to 16 tokens against Q6_K rows: `gemv_q8k_q6k_mf` by name and through the router, against
     matvec_kq per token and against the LDS-staged integer-dot entry on the same quantized
