@@ -27,18 +27,22 @@ __device__ __forceinline__ void gq_superblock(const GqW& cur, const uchar* xp, c
                                               float (&acc)[4]) {
     const gq_i4 zero = {0, 0, 0, 0};
     const float d = f16_bits_to_f32(cur.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
+    // all eight 6-bit scales and mins at once, a byte each (get_scale_min_k4, crates/ojas-formats/src/gguf.rs:1132-1140):
+    // sub-blocks 0-3 are the low six bits of bytes 0-3 / 4-7, sub-blocks 4-7 a nibble of bytes 8-11 under
+    // the top two bits of bytes 0-3 / 4-7
+    const uint sc_lo = cur.hdr.y & 0x3F3F3F3Fu, mn_lo = cur.hdr.z & 0x3F3F3F3Fu;
+    const uint sc_hi = (cur.hdr.w & 0x0F0F0F0Fu) | ((cur.hdr.y >> 2) & 0x30303030u);
+    const uint mn_hi = ((cur.hdr.w >> 4) & 0x0F0F0F0Fu) | ((cur.hdr.z >> 2) & 0x30303030u);
     int sc[8];
-    long B[8], Bm = 0;
+    long B[8];
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-        uint a, b;
-        q4k_scale_min_pair(cur.hdr.y, cur.hdr.z, cur.hdr.w, (uint)c, a, b);
-        sc[2 * c] = (int)(a & 0xFFu); sc[2 * c + 1] = (int)(a >> 8);
-        Bm |= (long)(unsigned long)(b & 0xFFFFu) << (16 * c);    // mins 2c, 2c + 1 -> bytes 2c, 2c + 1
+        sc[c] = (int)((sc_lo >> (8 * c)) & 0xFFu);
+        sc[4 + c] = (int)((sc_hi >> (8 * c)) & 0xFFu);
         B[2 * c] = gq_pack(cur.q[c].x & 0x0F0F0F0Fu, cur.q[c].y & 0x0F0F0F0Fu);
         B[2 * c + 1] = gq_pack((cur.q[c].x >> 4) & 0x0F0F0F0Fu, (cur.q[c].y >> 4) & 0x0F0F0F0Fu);
     }
-    if (kg != 0u) Bm = 0;                                        // only positions 0..7 carry mins
+    const long Bm = kg == 0u ? gq_pack(mn_lo, mn_hi) : 0;       // mins 0..7 in bytes 0..7; only positions 0..7 carry them
     int isum[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int jj = 0; jj < 8; jj++) {
