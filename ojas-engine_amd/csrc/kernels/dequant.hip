@@ -1,6 +1,6 @@
 // Family "dequant": GGUF blocks -> IEEE binary16, bit-exact with the reference decoder
 // (crates/ojas-formats/src/gguf.rs:612-1116; arms :704-709 Q8_0, :1042-1059 Q4_K,
-// :1060-1085 Q5_K, :1086-1108 Q6_K, :796-813 IQ4_NL, :814-840 IQ4_XS).
+// :1060-1085 Q5_K, :1086-1108 Q6_K, :796-813 IQ4_NL, :814-840 IQ4_XS, :653-703 Q4_0 / Q5_0 / Q4_1 / Q5_1).
 //
 // Bit-exactness rules: every product and difference is a separately rounded f32 operation
 // (__fmul_rn / __fsub_rn, never an FMA), in the reference's association order, followed by one
@@ -185,3 +185,33 @@ dequant_iq4xs_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nb
         o2[i] = f32_to_f16_bits(__fmul_rn(dl, (float)(signed char)(hi >> (8 * i))));
     }
 }
+
+// The legacy 32-weight blocks: one thread per weight.  AFFINE: {d, m} header and w = d * q + m (a product and
+// a sum, each rounded), else w = d * (q - 8 | 16); FIVE: a 4-byte field of fifth bits ahead of the nibbles.
+template <bool FIVE, bool AFFINE>
+__device__ __forceinline__ void dequant_legacy(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
+    const uint BYTES = 18u + (AFFINE ? 2u : 0u) + (FIVE ? 4u : 0u), HDR = AFFINE ? 4u : 2u;
+    size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+    size_t b = i >> 5;
+    if (b >= nblocks) return;
+    const uchar* blk = w + b * BYTES;
+    const uint j = (uint)i & 31u, byte = blk[HDR + (FIVE ? 4u : 0u) + (j & 15u)];
+    uint q = j < 16u ? byte & 0xFu : byte >> 4;
+    if (FIVE) {
+        const uint qh = (uint)blk[HDR] | ((uint)blk[HDR + 1] << 8) | ((uint)blk[HDR + 2] << 16) | ((uint)blk[HDR + 3] << 24);
+        q |= ((qh >> j) & 1u) << 4;
+    }
+    const float d = f16_bits_to_f32(*(const ushort*)blk);
+    float v;
+    if (AFFINE) v = __fadd_rn(__fmul_rn(d, (float)q), f16_bits_to_f32(*(const ushort*)(blk + 2)));
+    else v = __fmul_rn(d, __fsub_rn((float)q, FIVE ? 16.0f : 8.0f));
+    out[i] = f32_to_f16_bits(v);
+}
+extern "C" __global__ void __launch_bounds__(256)
+dequant_q40_f16(const uchar* w, ushort* out, uint nblocks) { dequant_legacy<false, false>(w, out, nblocks); }
+extern "C" __global__ void __launch_bounds__(256)
+dequant_q41_f16(const uchar* w, ushort* out, uint nblocks) { dequant_legacy<false, true>(w, out, nblocks); }
+extern "C" __global__ void __launch_bounds__(256)
+dequant_q50_f16(const uchar* w, ushort* out, uint nblocks) { dequant_legacy<true, false>(w, out, nblocks); }
+extern "C" __global__ void __launch_bounds__(256)
+dequant_q51_f16(const uchar* w, ushort* out, uint nblocks) { dequant_legacy<true, true>(w, out, nblocks); }

@@ -465,6 +465,7 @@ __device__ __forceinline__ float iq4_lane_dot(uint q, float4 x0, float4 x1) {
 
 struct Iq4nlW {
     static constexpr uint STEP = 16u;            // blocks a wave walks per step
+    static constexpr uint BYTES = IQ4NL_BYTES;
     static __device__ __forceinline__ uint units(uint K) { return K >> 5; }
     // lane -> (block of the step, float offset of its first x fragment inside the block)
     static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 2; }
@@ -478,13 +479,14 @@ struct Iq4nlW {
         f.q = *(const u32_a2*)(blk + 2u + (lane & 3u) * 4u);
         return f;
     }
-    static __device__ __forceinline__ float dot(const Frag& f, uint, float4 x0, float4 x1) {
+    static __device__ __forceinline__ float dot(const Frag& f, uint, float4 x0, float4 x1, float) {
         return f16_bits_to_f32(f.d16) * iq4_lane_dot(f.q, x0, x1);
     }
 };
 
 struct Iq4xsW {
     static constexpr uint STEP = 2u;             // super-blocks per step
+    static constexpr uint BYTES = IQ4XS_BYTES;
     static __device__ __forceinline__ uint units(uint K) { return K >> 8; }
     static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 5; }
     static __device__ __forceinline__ uint x_off(uint lane) { return ((lane & 31u) >> 2) * 32u + (lane & 3u) * 4u; }
@@ -498,12 +500,58 @@ struct Iq4xsW {
         f.q = blk[2u + (lane & 31u)];
         return f;
     }
-    static __device__ __forceinline__ float dot(const Frag& f, uint lane, float4 x0, float4 x1) {
+    static __device__ __forceinline__ float dot(const Frag& f, uint lane, float4 x0, float4 x1, float) {
         const uint ib = (lane & 31u) >> 2;
         const uint ls = ((f.sl >> (4u * ib)) & 0xFu) | ((((f.h0 >> 16) >> (2u * ib)) & 3u) << 4);
         return f16_bits_to_f32(f.h0 & 0xFFFFu) * (float)((int)ls - 32) * iq4_lane_dot(f.q, x0, x1);
     }
 };
+
+// The legacy 32-weight blocks Q4_0 / Q4_1 / Q5_0 / Q5_1 share IQ4_NL's layout — a header, then 16 bytes whose
+// low nibbles are weights 0..15 and high nibbles 16..31 — with a linear code instead of the table:
+// w = d (q - 8), d q + m, d (q5 - 16), d q5 + m, the fifth bit of weight j being bit j of a 4-byte field.
+// Four lanes per block; codes stay unsigned (v_cvt_f32_ubyteN) and the offset or minimum meets the sum of the
+// lane's eight activations once per block:  d * (sum q x - off * sum x)  or  d * sum q x + m * sum x.
+template <bool FIVE, bool AFFINE>
+struct LegacyW {
+    static constexpr uint STEP = 16u;
+    static constexpr uint BYTES = 18u + (AFFINE ? 2u : 0u) + (FIVE ? 4u : 0u);
+    static constexpr uint HDR = AFFINE ? 4u : 2u;
+    static __device__ __forceinline__ uint units(uint K) { return K >> 5; }
+    static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 2; }
+    static __device__ __forceinline__ uint x_off(uint lane) { return (lane & 3u) * 4u; }
+    static __device__ __forceinline__ uint x_unit(uint) { return 32u; }
+    struct Frag { uint hdr, q, qh; };
+    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
+        const uchar* blk = row + (size_t)u * BYTES;
+        Frag f;
+        f.hdr = AFFINE ? *(const u32_a2*)blk : (uint)*(const ushort*)blk;
+        f.qh = FIVE ? *(const u32_a2*)(blk + HDR) : 0u;
+        f.q = *(const u32_a2*)(blk + HDR + (FIVE ? 4u : 0u) + (lane & 3u) * 4u);
+        return f;
+    }
+    // bits b .. b + 3 of `v` -> bit 4 of bytes 0 .. 3
+    static __device__ __forceinline__ uint spread4(uint v, uint b) {
+        const uint n = (v >> b) & 0xFu;
+        return ((n & 1u) << 4) | ((n & 2u) << 11) | ((n & 4u) << 18) | ((n & 8u) << 25);
+    }
+    static __device__ __forceinline__ float dot(const Frag& f, uint lane, float4 x0, float4 x1, float xsum) {
+        uint lo = f.q & 0x0F0F0F0Fu, hi = (f.q >> 4) & 0x0F0F0F0Fu;
+        if (FIVE) {
+            const uint p4 = (lane & 3u) * 4u;
+            lo |= spread4(f.qh, p4);
+            hi |= spread4(f.qh, p4 + 16u);
+        }
+        const float a = dot4_ub(hi, x1, dot4_ub(lo, x0, 0.0f));
+        const float d = f16_bits_to_f32(f.hdr & 0xFFFFu);
+        if (AFFINE) return d * a + f16_bits_to_f32(f.hdr >> 16) * xsum;
+        return d * (a - (FIVE ? 16.0f : 8.0f) * xsum);
+    }
+};
+typedef LegacyW<false, false> Q40W;
+typedef LegacyW<false, true> Q41W;
+typedef LegacyW<true, false> Q50W;
+typedef LegacyW<true, true> Q51W;
 
 template <class W, int R, int MODE>
 __device__ __forceinline__ void gemv_nat_iq4_body(const float* __restrict__ x, const uchar* __restrict__ w,
@@ -513,7 +561,7 @@ __device__ __forceinline__ void gemv_nat_iq4_body(const float* __restrict__ x, c
     const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
     if (row0 >= N) return;
     const uint nu = W::units(K);
-    const size_t rb = (size_t)nu * (W::STEP == 16u ? IQ4NL_BYTES : IQ4XS_BYTES);
+    const size_t rb = (size_t)nu * W::BYTES;
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.0f;
@@ -523,8 +571,9 @@ __device__ __forceinline__ void gemv_nat_iq4_body(const float* __restrict__ x, c
         for (int r = 0; r < R; r++) f[r] = W::load(w + (size_t)min(row0 + r, N - 1u) * rb, u, lane);
         const float* xp = x + (size_t)u * W::x_unit(0) + W::x_off(lane);
         const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + 16);
+        const float xsum = sum4(x0) + sum4(x1);      // for the formats with an offset or a minimum
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r] += W::dot(f[r], lane, x0, x1);
+        for (int r = 0; r < R; r++) acc[r] += W::dot(f[r], lane, x0, x1, xsum);
     }
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -540,7 +589,7 @@ __device__ __forceinline__ void gemv_nat_iq4_m_body(const float* __restrict__ x,
     const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= N) return;
     const uint nu = W::units(K);
-    const uchar* wr = w + (size_t)row * nu * (W::STEP == 16u ? IQ4NL_BYTES : IQ4XS_BYTES);
+    const uchar* wr = w + (size_t)row * nu * W::BYTES;
     for (uint m0 = 0; m0 < M; m0 += MT) {
         float acc[MT];
 #pragma unroll
@@ -551,7 +600,8 @@ __device__ __forceinline__ void gemv_nat_iq4_m_body(const float* __restrict__ x,
             for (int i = 0; i < MT; i++) {
                 const uint m = min(m0 + i, M - 1u);
                 const float* xp = x + (size_t)m * K + (size_t)u * W::x_unit(0) + W::x_off(lane);
-                acc[i] += W::dot(f, lane, *(const float4*)xp, *(const float4*)(xp + 16));
+                const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + 16);
+                acc[i] += W::dot(f, lane, x0, x1, sum4(x0) + sum4(x1));
             }
         }
 #pragma unroll
@@ -576,8 +626,9 @@ __device__ __forceinline__ void gemv_nat_iq4_px_body(const float* __restrict__ x
                                                      float* __restrict__ y, uint K, uint N) {
     const uint lane = threadIdx.x & 63u;
     const uint nu = W::units(K);
-    const size_t rb = (size_t)nu * (W::STEP == 16u ? IQ4NL_BYTES : IQ4XS_BYTES);
+    const size_t rb = (size_t)nu * W::BYTES;
     float4 xr[NS][2];
+    float xsum[NS];
     uint uc[NS];
 #pragma unroll
     for (int s = 0; s < NS; s++) {
@@ -589,6 +640,7 @@ __device__ __forceinline__ void gemv_nat_iq4_px_body(const float* __restrict__ x
             xr[s][0] = *(const float4*)xp;
             xr[s][1] = *(const float4*)(xp + 16);
         }
+        xsum[s] = sum4(xr[s][0]) + sum4(xr[s][1]);
     }
     const uint nwaves = gridDim.x * (blockDim.x >> 6);
     for (uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2u; row0 < N; row0 += nwaves * 2u) {
@@ -598,8 +650,8 @@ __device__ __forceinline__ void gemv_nat_iq4_px_body(const float* __restrict__ x
 #pragma unroll
         for (int s = 0; s < NS; s++) {
             const typename W::Frag f0 = W::load(r0, uc[s], lane), f1 = W::load(r1, uc[s], lane);
-            a0 += W::dot(f0, lane, xr[s][0], xr[s][1]);
-            a1 += W::dot(f1, lane, xr[s][0], xr[s][1]);
+            a0 += W::dot(f0, lane, xr[s][0], xr[s][1], xsum[s]);
+            a1 += W::dot(f1, lane, xr[s][0], xr[s][1], xsum[s]);
         }
         a0 = wave_sum(a0);
         a1 = wave_sum(a1);
@@ -616,7 +668,43 @@ __device__ __forceinline__ void gemv_nat_iq4_px_body(const float* __restrict__ x
         gemv_nat_iq4_px_body<W, 8>(x, w, y, K, N); }
 GEMV_NAT_IQ4_PX(iq4nl, Iq4nlW)
 GEMV_NAT_IQ4_PX(iq4xs, Iq4xsW)
+GEMV_NAT_IQ4_PX(q40, Q40W)
+GEMV_NAT_IQ4_PX(q41, Q41W)
+GEMV_NAT_IQ4_PX(q50, Q50W)
+GEMV_NAT_IQ4_PX(q51, Q51W)
 
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_q40_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
+    gemv_nat_iq4_body<Q40W, R, MODE>(x, w, y, bs, K, N);
+}
+template <int MT>
+__device__ __forceinline__ void gemv_nat_q40_m_body(const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    gemv_nat_iq4_m_body<Q40W, MT>(x, w, y, K, N, M, ACC);
+}
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_q41_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
+    gemv_nat_iq4_body<Q41W, R, MODE>(x, w, y, bs, K, N);
+}
+template <int MT>
+__device__ __forceinline__ void gemv_nat_q41_m_body(const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    gemv_nat_iq4_m_body<Q41W, MT>(x, w, y, K, N, M, ACC);
+}
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_q50_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
+    gemv_nat_iq4_body<Q50W, R, MODE>(x, w, y, bs, K, N);
+}
+template <int MT>
+__device__ __forceinline__ void gemv_nat_q50_m_body(const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    gemv_nat_iq4_m_body<Q50W, MT>(x, w, y, K, N, M, ACC);
+}
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_q51_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
+    gemv_nat_iq4_body<Q51W, R, MODE>(x, w, y, bs, K, N);
+}
+template <int MT>
+__device__ __forceinline__ void gemv_nat_q51_m_body(const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    gemv_nat_iq4_m_body<Q51W, MT>(x, w, y, K, N, M, ACC);
+}
 template <int R, int MODE>
 __device__ __forceinline__ void gemv_nat_iq4nl_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
     gemv_nat_iq4_body<Iq4nlW, R, MODE>(x, w, y, bs, K, N);
@@ -773,3 +861,7 @@ GEMV_NAT_ENTRIES(q4k)
 GEMV_NAT_ENTRIES(q6k)
 GEMV_NAT_ENTRIES(iq4nl)
 GEMV_NAT_ENTRIES(iq4xs)
+GEMV_NAT_ENTRIES(q40)
+GEMV_NAT_ENTRIES(q41)
+GEMV_NAT_ENTRIES(q50)
+GEMV_NAT_ENTRIES(q51)

@@ -16,11 +16,20 @@ static const ojh_block_format kFormats[] = {
     {OJH_Q6_K, 210, 256, "q6k"},
     {OJH_IQ4_NL, 18, 32, "iq4nl"},
     {OJH_IQ4_XS, 136, 256, "iq4xs"},
+    {OJH_Q4_0, 18, 32, "q40"},
+    {OJH_Q4_1, 20, 32, "q41"},
+    {OJH_Q5_0, 22, 32, "q50"},
+    {OJH_Q5_1, 24, 32, "q51"},
 };
 
 // Formats whose CPU path multiplies the raw row with f32 activations (dot_q80, dot_iq4nl, dot_iq4xs:
 // crates/ojas-cpu/src/cpu_math.rs:1131-1141, :1179) instead of quantizing them per 256.
-bool ojh_float_rows(uint32_t t) { return t == OJH_Q8_0 || t == OJH_IQ4_NL || t == OJH_IQ4_XS; }
+bool ojh_float_rows(uint32_t t) { return t == OJH_Q8_0 || ojh_float_only(t); }
+// ... and for which this library has the f32-activation matvecs only: no int8-activation form, no MFMA tile
+// (the IQ4 types, and the legacy 32-weight blocks the reference runs on its GPU path alone)
+bool ojh_float_only(uint32_t t) {
+    return t == OJH_IQ4_NL || t == OJH_IQ4_XS || t == OJH_Q4_0 || t == OJH_Q4_1 || t == OJH_Q5_0 || t == OJH_Q5_1;
+}
 
 const ojh_block_format *ojh_format(uint32_t t) {
     for (const auto &f : kFormats)
@@ -983,7 +992,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g + "_bias", "gemv", 4, 2, f.type, 4, check_gemv_nat, shape_rows);
         add(g + "_m", "gemv", 3, 4, f.type, 1, check_gemv_nat_m, shape_rows);
         if (f.type != OJH_Q8_0) add(g + "_px", "gemv", 3, 2, f.type, 2, check_gemv_nat_px, shape_px);
-        if (f.type == OJH_IQ4_NL || f.type == OJH_IQ4_XS) continue;   // f32 activations only, no MFMA tile
+        if (ojh_float_only(f.type)) continue;   // f32 activations only, no MFMA tile
         if (f.type == OJH_Q8_0) {
             add(g + "_lds", "gemv", 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
             add(g + "_lds_accum", "gemv", 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
@@ -1026,7 +1035,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     // prefill / verify MFMA tiles: "q8_0" is the reference's spelling for this family
     for (const auto &f : kFormats) {
-        if (f.type == OJH_Q5_K || f.type == OJH_IQ4_NL || f.type == OJH_IQ4_XS) continue;
+        if (f.type == OJH_Q5_K || ojh_float_only(f.type)) continue;
         std::string g = std::string("gemm_mm_") + (f.type == OJH_Q8_0 ? "q8_0" : f.tag);
         add(g, "gemm", 3, 4, f.type, 0, check_gemm, shape_gemm);
         add(g + "_sk", "gemm", 3, 4, f.type, 1, check_gemm, shape_gemm);

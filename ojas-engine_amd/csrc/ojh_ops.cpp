@@ -365,9 +365,9 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         act_mode = OJH_ACT_Q8K;
     }
 
-    // IQ4_NL / IQ4_XS: f32 activations against the raw rows at every token count (dot_iq4nl / dot_iq4xs);
-    // no int8-activation form and no MFMA tile read them.
-    const bool iq4 = w->type == OJH_IQ4_NL || w->type == OJH_IQ4_XS;
+    // IQ4_NL / IQ4_XS (dot_iq4nl / dot_iq4xs) and Q4_0 / Q4_1 / Q5_0 / Q5_1: f32 activations against the raw
+    // rows at every token count; no int8-activation form and no MFMA tile read them.
+    const bool iq4 = ojh_float_only(w->type);   // (the IQ4 types and the legacy 32-weight blocks)
     if (iq4 && act_mode == OJH_ACT_Q8K)
         return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: %s rows take f32 activations only (OJH_ACT_FLOAT or OJH_ACT_AUTO)", f->tag);
 

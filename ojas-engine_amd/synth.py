@@ -13,7 +13,9 @@ from __future__ import annotations
 import numpy as np
 
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
-BLOCK_SHAPE = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256), IQ4_NL: (18, 32), IQ4_XS: (136, 256)}
+Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+BLOCK_SHAPE = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256), IQ4_NL: (18, 32), IQ4_XS: (136, 256),
+               Q4_0: (18, 32), Q4_1: (20, 32), Q5_0: (22, 32), Q5_1: (24, 32)}
 
 
 def seed_of(*names) -> int:
@@ -140,7 +142,26 @@ def iq4xs_weights(n: int, k: int, *names) -> np.ndarray:
     return out.reshape(-1)
 
 
+def legacy_weights(ty: int, n: int, k: int, *names) -> np.ndarray:
+    """Q4_0 / Q4_1 / Q5_0 / Q5_1 rows: d = f16(|N(0,0.02)| / 8), m = f16(N(0,0.01)) where the format has one,
+    every other byte (fifth-bit field, nibbles) uniform."""
+    g = rng(*names)
+    bb = BLOCK_SHAPE[ty][0]
+    nb = n * (k // 32)
+    out = g.integers(0, 256, size=(nb, bb), dtype=np.uint8)
+    d = (np.abs(g.standard_normal(nb) * 0.02) / 8.0).astype(np.float16).view(np.uint16)
+    out[:, 0] = d & 0xFF
+    out[:, 1] = d >> 8
+    if ty in (Q4_1, Q5_1):
+        m = (g.standard_normal(nb) * 0.01).astype(np.float16).view(np.uint16)
+        out[:, 2] = m & 0xFF
+        out[:, 3] = m >> 8
+    return out.reshape(-1)
+
+
 def weights(ty: int, n: int, k: int, *names) -> np.ndarray:
+    if ty in (Q4_0, Q4_1, Q5_0, Q5_1):
+        return legacy_weights(ty, n, k, *names)
     return {Q8_0: q80_weights, Q4_K: q4k_weights, Q5_K: q5k_weights, Q6_K: q6k_weights,
             IQ4_NL: iq4nl_weights, IQ4_XS: iq4xs_weights}[ty](n, k, *names)
 

@@ -101,6 +101,10 @@ int ojo_block_shape(uint32_t ty, uint32_t *bytes, uint32_t *weights) { /* synth.
     case OJO_Q5_K: b = 176; w = 256; break;
     case OJO_Q6_K: b = 210; w = 256; break;
     case OJO_IQ4_NL: b = 18; w = 32; break;
+    case OJO_Q4_0: b = 18; w = 32; break;
+    case OJO_Q4_1: b = 20; w = 32; break;
+    case OJO_Q5_0: b = 22; w = 32; break;
+    case OJO_Q5_1: b = 24; w = 32; break;
     case OJO_IQ4_XS: b = 136; w = 256; break;
     default: return 0;
     }
@@ -163,6 +167,40 @@ int ojo_dequant_to_f16(const uint8_t *b, uint32_t ty, size_t n, uint16_t *out) {
         case OJO_Q8_0: { /* gguf.rs:704-709 */
             float d = rdh(blk, 0);
             for (int j = 0; j < 32; j++) o[j] = ojo_f32_to_f16(d * (float)(int8_t)blk[2 + j]);
+        } break;
+        case OJO_Q4_0: { /* gguf.rs:653-661: w = d * (nib - 8); low nibbles first, then high nibbles */
+            float d = rdh(blk, 0);
+            for (int j = 0; j < 16; j++) {
+                o[j] = ojo_f32_to_f16(d * ((float)(blk[2 + j] & 0xF) - 8.0f));
+                o[j + 16] = ojo_f32_to_f16(d * ((float)(blk[2 + j] >> 4) - 8.0f));
+            }
+        } break;
+        case OJO_Q5_0: { /* gguf.rs:662-678: fifth bit of weight j is bit j of qh; w = d * (q - 16) */
+            float d = rdh(blk, 0);
+            uint32_t qh = (uint32_t)blk[2] | ((uint32_t)blk[3] << 8) | ((uint32_t)blk[4] << 16) | ((uint32_t)blk[5] << 24);
+            for (int j = 0; j < 16; j++) {
+                uint32_t lo = (uint32_t)(blk[6 + j] & 0xF) | (((qh >> j) & 1u) << 4);
+                uint32_t hi = (uint32_t)(blk[6 + j] >> 4) | (((qh >> (j + 16)) & 1u) << 4);
+                o[j] = ojo_f32_to_f16(d * ((float)lo - 16.0f));
+                o[j + 16] = ojo_f32_to_f16(d * ((float)hi - 16.0f));
+            }
+        } break;
+        case OJO_Q4_1: { /* gguf.rs:679-686: w = d * nib + m, a product and a sum, each rounded */
+            float d = rdh(blk, 0), m = rdh(blk, 2);
+            for (int j = 0; j < 16; j++) {
+                o[j] = ojo_f32_to_f16(d * (float)(blk[4 + j] & 0xF) + m);
+                o[j + 16] = ojo_f32_to_f16(d * (float)(blk[4 + j] >> 4) + m);
+            }
+        } break;
+        case OJO_Q5_1: { /* gguf.rs:687-703 (and the threaded copy :616-649): w = d * q + m */
+            float d = rdh(blk, 0), m = rdh(blk, 2);
+            uint32_t qh = (uint32_t)blk[4] | ((uint32_t)blk[5] << 8) | ((uint32_t)blk[6] << 16) | ((uint32_t)blk[7] << 24);
+            for (int j = 0; j < 16; j++) {
+                uint32_t lo = (uint32_t)(blk[8 + j] & 0xF) | (((qh >> j) & 1u) << 4);
+                uint32_t hi = (uint32_t)(blk[8 + j] >> 4) | (((qh >> (j + 16)) & 1u) << 4);
+                o[j] = ojo_f32_to_f16(d * (float)lo + m);
+                o[j + 16] = ojo_f32_to_f16(d * (float)hi + m);
+            }
         } break;
         case OJO_IQ4_NL: { /* gguf.rs:796-813: low nibbles fill the first half, high nibbles the second */
             float d = rdh(blk, 0);
@@ -261,6 +299,19 @@ int ojo_dequant_to_f64(const uint8_t *b, uint32_t ty, size_t n, double *out) {
         case OJO_Q8_0: {
             double d = rdh(blk, 0);
             for (int j = 0; j < 32; j++) o[j] = d * (double)(int8_t)blk[2 + j];
+        } break;
+        case OJO_Q4_0: case OJO_Q4_1: case OJO_Q5_0: case OJO_Q5_1: {
+            const int five = ty == OJO_Q5_0 || ty == OJO_Q5_1, affine = ty == OJO_Q4_1 || ty == OJO_Q5_1;
+            double d = rdh(blk, 0), m = affine ? (double)rdh(blk, 2) : 0.0;
+            const uint8_t *hb = blk + (affine ? 4 : 2), *qs = hb + (five ? 4 : 0);
+            uint32_t qh = five ? (uint32_t)hb[0] | ((uint32_t)hb[1] << 8) | ((uint32_t)hb[2] << 16) | ((uint32_t)hb[3] << 24) : 0;
+            double off = affine ? 0.0 : (five ? 16.0 : 8.0);
+            for (int j = 0; j < 16; j++) {
+                uint32_t lo = (uint32_t)(qs[j] & 0xF) | (((qh >> j) & 1u) << 4);
+                uint32_t hi = (uint32_t)(qs[j] >> 4) | (((qh >> (j + 16)) & 1u) << 4);
+                o[j] = d * ((double)lo - off) + m;
+                o[j + 16] = d * ((double)hi - off) + m;
+            }
         } break;
         case OJO_IQ4_NL: {
             double d = rdh(blk, 0);

@@ -13,6 +13,8 @@
  *   dequant Q4_K/Q5_K/Q6_K  FNV-1a digests held by crates/ojas-formats/tests/quant_formats.rs:38-40
  *   dequant IQ4_NL/IQ4_XS   the digests of the same table (quant_formats.rs:45,48), one-hot codes vs the codebook
  *   dequant Q8_0            closed form of crates/ojas-formats/tests/rows.rs:13-18
+ *   dequant Q4_0/Q4_1/Q5_0/Q5_1  closed forms only (d * (q - 8 | 16), d * q + m, nibble halves, the fifth-bit field):
+ *                           the reference's tests hold no digest for the legacy 32-weight blocks
  *   f16 <-> f32             the digests above + exhaustive comparison with IEEE binary16 (numpy)
  *   quant_q8k               invariants (max|q|=127, bsums, half-away rounding, |x-s*q|<=s/2)
  *   dot_q80                 f64 dot over the dequantized row, brute force at K=32
@@ -35,7 +37,8 @@ extern "C" {
 #endif
 
 /* GGUF type ids (crates/ojas-formats/src/gguf.rs:563-591). */
-enum { OJO_Q8_0 = 8, OJO_Q4_K = 12, OJO_Q5_K = 13, OJO_Q6_K = 14, OJO_IQ4_NL = 20, OJO_IQ4_XS = 23 };
+enum { OJO_Q4_0 = 2, OJO_Q4_1 = 3, OJO_Q5_0 = 6, OJO_Q5_1 = 7, OJO_Q8_0 = 8, OJO_Q4_K = 12, OJO_Q5_K = 13, OJO_Q6_K = 14,
+       OJO_IQ4_NL = 20, OJO_IQ4_XS = 23 };
 
 /* IEEE binary16 <-> binary32, round-to-nearest-even, subnormals kept
  * (crate half 2.7.1; call sites gguf.rs:602-608). */

@@ -4,6 +4,7 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
+Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6,
            IQ4_NL: 0xA5D4CF4E5DB3A1BF, IQ4_XS: 0x1429CAFB4DF9AF64}
 
@@ -25,7 +26,8 @@ def test_reference_digests_on_device(gpu, orc, pkg, ty):
 
 
 @pytest.mark.parametrize("ty,n,k", [(Q8_0, 37, 4096), (Q4_K, 129, 4096), (Q6_K, 65, 4096), (Q5_K, 16, 1024),
-                                    (IQ4_NL, 33, 2080), (IQ4_XS, 21, 4096)])
+                                    (IQ4_NL, 33, 2080), (IQ4_XS, 21, 4096), (Q4_0, 33, 2080), (Q4_1, 9, 4096),
+                                    (Q5_0, 33, 2080), (Q5_1, 9, 4096)])
 def test_bit_exact_on_benchmark_distributions(gpu, orc, pkg, ty, n, k):
     raw = orc.synth_blocks(ty, n * k // pkg.synth.BLOCK_SHAPE[ty][1]) if ty == Q5_K else \
         pkg.synth.weights(ty, n, k, "dq", ty)
@@ -33,7 +35,7 @@ def test_bit_exact_on_benchmark_distributions(gpu, orc, pkg, ty, n, k):
     assert np.array_equal(got, orc.dequant_to_f16(raw, ty, n * k))
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1])
 def test_bit_exact_with_extreme_scales(gpu, orc, pkg, ty):
     """Subnormal, tiny, huge and negative f16 scales: every rounding path of the decoder."""
     bb, wpb = pkg.synth.BLOCK_SHAPE[ty]
@@ -43,7 +45,7 @@ def test_bit_exact_with_extreme_scales(gpu, orc, pkg, ty):
     off = 208 if ty == Q6_K else 0
     for i in range(nb):
         raw[i, off:off + 2] = np.array([scales[i % scales.size]], np.uint16).view(np.uint8)
-        if ty in (Q4_K, Q5_K):
+        if ty in (Q4_K, Q5_K, Q4_1, Q5_1):
             raw[i, 2:4] = np.array([scales[(i * 7 + 3) % scales.size]], np.uint16).view(np.uint8)
     raw = raw.reshape(-1)
     got = _dequant(gpu, ty, raw, nb * wpb)

@@ -1,7 +1,7 @@
 """A seeded sweep over what `ojh_mm` can be asked: formats, row counts on both sides of every routing
 threshold (tiles per CU, output heads), K from one super-block to 14336, 1 to 40 tokens, plain and
 accumulating stores.  Whatever entry the router picks, every token must match the CPU reference's
-`matvec_kq` (int8-activation contract; f32 activations for Q8_0 and the IQ4 types), nothing may be
+`matvec_kq` (int8-activation contract; f32 activations for Q8_0, the IQ4 types and the legacy blocks), nothing may be
 written past the last token, and a token's result must not depend on the batch it came in."""
 import numpy as np
 import pytest
@@ -10,6 +10,9 @@ from conftest import peak_err
 
 pytestmark = pytest.mark.gpu
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
+Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+FLOAT_ROWS = (Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1)
+LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1)
 
 
 def _cases():
@@ -17,8 +20,8 @@ def _cases():
     rows = [17, 130, 1000, 4099, 6144, 8200, 14336, 24576, 33000, 40001]
     ks = [256, 512, 1024, 2560, 4096, 5120, 7168, 14336]
     out = []
-    for ty in (Q4_K, Q6_K, Q5_K, Q8_0, IQ4_NL, IQ4_XS):
-        for _ in range(7):
+    for ty in (Q4_K, Q6_K, Q5_K, Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1):
+        for _ in range(7 if ty not in LEGACY else 3):
             n, k = int(g.choice(rows)), int(g.choice(ks))
             m = int(g.choice([1, 2, 3, 4, 5, 7, 8, 9, 16, 17, 33, 40]))
             while n * k * m > 6.0e9 or n * k > 2.4e8:      # keep the oracle side to a second or so
@@ -35,17 +38,19 @@ def test_router_sweep(gpu, orc, pkg, ty, n, k, m, accum):
     lin = gpu.lin(ty, n, k, w)
     yd = gpu.upload(np.concatenate([y0.ravel(), np.full(16, 4242.5, np.float32)]))
     gpu.mm(gpu.upload(x), lin, yd, m, accum, act_mode=pkg.ACT_AUTO if m < 32 else
-           (pkg.ACT_FLOAT if ty in (Q8_0, IQ4_NL, IQ4_XS) else pkg.ACT_Q8K))
+           (pkg.ACT_FLOAT if ty in FLOAT_ROWS else pkg.ACT_Q8K))
     got = gpu.read(yd, m * n + 16)
     assert np.all(got[m * n:] == 4242.5), "wrote past the last token"
     got = got[:m * n].reshape(m, n) - y0
-    tol = 1e-5 if ty in (Q8_0, IQ4_NL, IQ4_XS) else 2e-5
+    tol = 1e-5 if ty in FLOAT_ROWS else 2e-5
     tile = ty == Q8_0 and m >= 32          # Q8_0 from 32 tokens: the f16 MFMA tile, activations rounded to f16 (its own contract)
     if tile:
         tol = 2e-3
     scale = 1.0 + (float(np.max(np.abs(y0))) if accum else 0.0)   # accumulating onto y0 rounds at y0's magnitude
     for t in sorted({0, m // 2, m - 1}):
-        want = orc.matvec_kq(w, ty, n, k, x[t])
+        # (the CPU path has no dot for the legacy blocks: the reference runs them on its GPU path, f32
+        # activations against the dequantized weights, which is what the f64 reference evaluates)
+        want = orc.matmul_ref(w, ty, n, k, x[t])[0] if ty in LEGACY else orc.matvec_kq(w, ty, n, k, x[t])
         assert peak_err(got[t], want) <= tol * max(1.0, scale * 4.0 / max(1e-30, float(np.max(np.abs(want))))), (t,)
     if m > 1 and not accum and not tile:
         # the middle token alone: the one-token kernels associate their f32 sums differently (last ulps)

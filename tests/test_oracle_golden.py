@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
+Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 
 # crates/ojas-formats/tests/quant_formats.rs:38-40, 45, 48
 DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6,
@@ -21,7 +22,7 @@ def test_dequant_digest_matches_reference(orc, pkg, ty):
     assert orc.digest_f16(bits) == DIGESTS[ty]
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1])
 def test_synth_blocks_two_implementations_agree(orc, pkg, ty):
     assert np.array_equal(orc.synth_blocks(ty, 9), pkg.synth.synth_blocks(ty, 9))
 
@@ -170,6 +171,39 @@ def test_dot_q80_matches_f64_dot(orc, pkg):
         acc = np.float32(acc + np.float32(np.int8(blk[2 + j])) * x[j])
     d = blk[0:2].view(np.float16).astype(np.float32)[0]
     assert orc.dot_q80(blk, x[:32]) == np.float32(d * acc)
+
+
+@pytest.mark.parametrize("ty", [Q4_0, Q4_1, Q5_0, Q5_1])
+def test_legacy_block_closed_forms(orc, pkg, ty):
+    """The 32-weight blocks against their definitions in numpy (the reference's tests hold no digest for
+    them): w = d (q - 8), d q + m, d (q5 - 16), d q5 + m; low nibbles are weights 0..15, high nibbles
+    16..31; the fifth bit of weight j is bit j of the little-endian qh field; and the f16 decoder equals
+    the f32 expression of the reference (a product, then where the format has one a sum, each rounded)."""
+    bb = pkg.synth.BLOCK_SHAPE[ty][0]
+    raw = orc.synth_blocks(ty, 50).reshape(50, bb).copy()
+    g = np.random.default_rng(ty)
+    raw[:, 2:4] = (g.standard_normal(50) * 0.3).astype(np.float16).view(np.uint8).reshape(50, 2)   # m (or qh / qs bytes)
+    five, affine = ty in (Q5_0, Q5_1), ty in (Q4_1, Q5_1)
+    hdr = 4 if affine else 2
+    d = raw[:, 0:2].copy().view(np.float16).astype(np.float32)[:, 0]
+    m = raw[:, 2:4].copy().view(np.float16).astype(np.float32)[:, 0] if affine else np.zeros(50, np.float32)
+    qh = raw[:, hdr:hdr + 4].copy().view(np.uint32)[:, 0] if five else np.zeros(50, np.uint32)
+    qs = raw[:, hdr + (4 if five else 0):]
+    j = np.arange(16)
+    lo = (qs & 0xF).astype(np.uint32) | (((qh[:, None] >> j) & 1) << 4)
+    hi = (qs >> 4).astype(np.uint32) | (((qh[:, None] >> (j + 16)) & 1) << 4)
+    q = np.concatenate([lo, hi], axis=1).astype(np.float32)
+    if affine:
+        want32 = (d[:, None] * q).astype(np.float32) + m[:, None]
+    else:
+        want32 = d[:, None] * (q - np.float32(16.0 if five else 8.0))
+    with np.errstate(over="ignore"):
+        want16 = want32.astype(np.float32).astype(np.float16).view(np.uint16)
+    got16 = orc.dequant_to_f16(raw.reshape(-1), ty, 50 * 32).reshape(50, 32)
+    assert np.array_equal(got16, want16)
+    got64 = orc.dequant_to_f64(raw.reshape(-1), ty, 50 * 32).reshape(50, 32)
+    exact = d.astype(np.float64)[:, None] * (q.astype(np.float64) - (0.0 if affine else (16.0 if five else 8.0))) + m.astype(np.float64)[:, None]
+    assert np.array_equal(got64, exact)
 
 
 def test_iq4_closed_forms(orc):
