@@ -251,7 +251,7 @@ int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uin
  * (crates/ojas-cpu/src/cpu_glm.rs:551-582; per-assignment GPU form
  * crates/ojas-metal/src/kernels/moe.rs:199-272):
  *   y[t] (+)= sum_j wgt[t][j] * Wd_e( silu(Wg_e x[t]) * (Wu_e x[t]) ),  e = idx[t][j].
- * gate/up: n_expert stacked Q4_K matrices [n_ff][d]; down: n_expert stacked [d][n_ff], Q4_K or Q5_K.
+ * gate/up: n_expert stacked Q4_K matrices [n_ff][d]; down: n_expert stacked [d][n_ff], Q4_K, Q5_K or Q6_K.
  * Expert indices must be below n_expert (one that is not never reads outside the tensors; what
  * it contributes is unspecified). Up to 8 tokens run as two launches addressed
  * by assignment (bit-identical to the grouped integer-dot pipeline); larger batches are grouped

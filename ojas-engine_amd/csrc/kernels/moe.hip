@@ -292,6 +292,12 @@ moe_down_q5k_m(const signed char* aq, const float* as_, const uchar* wd, float* 
                const uint* list, uint K, uint N, uint NA) {
     moe_down_m_body<W5k>(aq, as_, wd, dv, offsets, list, K, N, NA);
 }
+// ... and over Q6_K rows (two steps finer)
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q6k_m(const signed char* aq, const float* as_, const uchar* wd, float* dv, const uint* offsets,
+               const uint* list, uint K, uint N, uint NA) {
+    moe_down_m_body<W6k>(aq, as_, wd, dv, offsets, list, K, N, NA);
+}
 
 // ------------------------------------------------------------------ decode: a few tokens, two launches
 // With one or a few tokens almost every assignment has its expert to itself, so grouping buys
@@ -481,6 +487,11 @@ extern "C" __global__ void __launch_bounds__(256)
 moe_down_q5k_dec(const float* act, const uchar* wd, const uint* idx, const float* wgt, float* y, uint K, uint N,
                  uint KSEL, uint E, uint ACC) {
     moe_down_dec_body<W5k, false>(act, wd, idx, wgt, y, K, N, KSEL, E, ACC);
+}
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q6k_dec(const float* act, const uchar* wd, const uint* idx, const float* wgt, float* y, uint K, uint N,
+                 uint KSEL, uint E, uint ACC) {
+    moe_down_dec_body<W6k, false>(act, wd, idx, wgt, y, K, N, KSEL, E, ACC);
 }
 
 // ------------------------------------------------------------------ grouped products on the matrix cores

@@ -138,3 +138,43 @@ struct W5k {
     }
     __device__ __forceinline__ float dot(uint c, const Q4kFrag& f) const { return q5k_lane_dot(h, q, qh, c, f); }
 };
+
+// Q6_K on the same lane map (eight lanes per super-block; lane l: 64-weight chunk c = l / 2, run h = l % 2).
+// The lane's two runs of 16 activations — positions 64 c + 16 h + i and 32 further on — are quarters
+// q = 2 (c % 2) and q + 1 of half c / 2 at in-quarter offset 16 h: ql bytes 64 hf + 16 h + i and 32 further
+// on (low nibbles when c is even, high when odd), qh bytes 32 hf + 16 h + i (bit pairs 2 q and 2 q + 2), scales
+// 8 hf + 2 q + h and two further on, d at byte 208 (crates/ojas-formats/src/gguf.rs:1086-1108).  The
+// arithmetic is dot_q6k's per 16-weight group: sx * d * sum_g scale_g * (sum code x - 32 sum x)
+// (crates/ojas-cpu/src/cpu_math.rs:674-722), integer sums exact.
+struct W6k {
+    static constexpr uint BYTES = Q6K_BYTES;
+    u32x4_a2 qa, qb, qh;
+    uint sc2, d16;      // the two scales in bytes 0 and 1
+    __device__ __forceinline__ void load(const uchar* blk, uint l) {
+        const uint c = l >> 1, h = l & 1u, hf = c >> 1, q = 2u * (c & 1u);
+        qa = *(const u32x4_a2*)(blk + 64u * hf + 16u * h);
+        qb = *(const u32x4_a2*)(blk + 64u * hf + 32u + 16u * h);
+        qh = *(const u32x4_a2*)(blk + 128u + 32u * hf + 16u * h);
+        const uchar* ps = blk + 192u + 8u * hf + 2u * q + h;
+        sc2 = (uint)ps[0] | ((uint)ps[2] << 8);
+        d16 = *(const ushort*)(blk + 208u);
+    }
+    __device__ __forceinline__ float dot(uint c, const Q4kFrag& f) const {
+        const uint M4 = 0x0F0F0F0Fu, H2 = 0x30303030u;
+        const uint nsh = 4u * (c & 1u);            // nibble of ql; also the bit pair of qh for the first run
+        // codes 0..63 as bytes: ql nibble | two bits of qh moved to bits 4-5
+        #define OJK_Q6_CODE(QL, QH, SH) ((((QL) >> nsh) & M4) | ((((QH) >> (SH)) << 4) & H2))
+        int ia = dot4_i8(OJK_Q6_CODE(qa.x, qh.x, nsh), f.xl.x, 0);
+        ia = dot4_i8(OJK_Q6_CODE(qa.y, qh.y, nsh), f.xl.y, ia);
+        ia = dot4_i8(OJK_Q6_CODE(qa.z, qh.z, nsh), f.xl.z, ia);
+        ia = dot4_i8(OJK_Q6_CODE(qa.w, qh.w, nsh), f.xl.w, ia);
+        int ib = dot4_i8(OJK_Q6_CODE(qb.x, qh.x, nsh + 2u), f.xh.x, 0);
+        ib = dot4_i8(OJK_Q6_CODE(qb.y, qh.y, nsh + 2u), f.xh.y, ib);
+        ib = dot4_i8(OJK_Q6_CODE(qb.z, qh.z, nsh + 2u), f.xh.z, ib);
+        ib = dot4_i8(OJK_Q6_CODE(qb.w, qh.w, nsh + 2u), f.xh.w, ib);
+        #undef OJK_Q6_CODE
+        const int sa = (int)(signed char)(sc2 & 0xFFu), sb = (int)(signed char)(sc2 >> 8);
+        const int isum = sa * (ia - 32 * f.bl) + sb * (ib - 32 * f.bh);
+        return f.sx * f16_bits_to_f32(d16) * (float)isum;
+    }
+};

@@ -1062,6 +1062,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("moe_down_q4k_slots", "moe", 5, 5, OJH_Q4_K, 11, check_moe, shape_moe);
     add("moe_down_q5k_m", "moe", 6, 3, OJH_Q5_K, 4, check_moe, shape_moe);
     add("moe_down_q5k_dec", "moe", 5, 5, OJH_Q5_K, 9, check_moe, shape_moe);
+    add("moe_down_q6k_m", "moe", 6, 3, OJH_Q6_K, 4, check_moe, shape_moe);
+    add("moe_down_q6k_dec", "moe", 5, 5, OJH_Q6_K, 9, check_moe, shape_moe);
     add("copy_bf16_half", "glue", 2, 1, (2u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     // glue: `type` carries (input element bytes << 8 | output element bytes)
     add("copy_f32_half", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);

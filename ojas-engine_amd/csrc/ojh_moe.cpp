@@ -3,6 +3,7 @@
 // graph_decode.rs:441-499, prefill graph_chunk.rs:564-628; CPU crates/ojas-cpu/src/cpu_glm.rs:519-597):
 // router -> group assignments by expert -> gate/up (+SiLU*mul) -> quantize -> down -> weighted sum.
 #include "ojh_internal.h"
+#include <string>
 
 static int ensure(ojh_device *dev, const char *family) {
     return dev->modules.count(family) ? OJH_OK : ojh_ensure_family(dev, family);
@@ -38,10 +39,12 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_moe_ffn: only the quantized-activation contract (OJH_ACT_Q8K) is built");
     if (!T || !E || E > 1024 || !ksel || ksel > E || T > 65535u / ksel)
         return ojh_fail(OJH_ERR_ARG, "moe_ffn: tokens=%u experts=%u ksel=%u out of range", T, E, ksel);
-    if (gate->type != OJH_Q4_K || up->type != OJH_Q4_K || (down->type != OJH_Q4_K && down->type != OJH_Q5_K))
-        return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: gate and up must be Q4_K, down Q4_K or Q5_K (gate %u, up %u, down %u)",
+    if (gate->type != OJH_Q4_K || up->type != OJH_Q4_K || (down->type != OJH_Q4_K && down->type != OJH_Q5_K && down->type != OJH_Q6_K))
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: gate and up must be Q4_K, down Q4_K, Q5_K or Q6_K (gate %u, up %u, down %u)",
                         gate->type, up->type, down->type);
-    const bool down5 = down->type == OJH_Q5_K;
+    const bool down5 = down->type != OJH_Q4_K;   // Q5_K or Q6_K down tensors: integer dots at every batch size
+    const std::string down_dec = std::string("moe_down_") + ojh_format(down->type)->tag + "_dec";
+    const std::string down_m = std::string("moe_down_") + ojh_format(down->type)->tag + "_m";
     if (d % 256 || n_ff % 256) return ojh_fail(OJH_ERR_ARG, "moe_ffn: d=%u and n_ff=%u must be multiples of 256", d, n_ff);
     if (gate->k != d || up->k != d || gate->n != (uint64_t)E * n_ff || up->n != gate->n || down->k != n_ff ||
         down->n != (uint64_t)E * d)
@@ -71,7 +74,7 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
                              {d, n_ff, ksel, NA, E}, g1, b256)))
             return rc;
         uint32_t g2[3] = {(d + 7) / 8, T, 1};
-        return ojh_launch(dev, down5 ? "moe_down_q5k_dec" : "moe_down_q4k_dec", {act->ptr, (char *)down->raw->ptr + down->off, idx->ptr, wgt->ptr, y->ptr},
+        return ojh_launch(dev, down_dec.c_str(), {act->ptr, (char *)down->raw->ptr + down->off, idx->ptr, wgt->ptr, y->ptr},
                           {n_ff, d, ksel, E, (uint32_t)(accum != 0)}, g2, b256);
     }
     ojh_buf *xq, *xs, *act, *aq, *as_, *dv, *grp;
@@ -122,7 +125,7 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         const bool dots = down5 || !mm;
         uint32_t g[3] = {mt_down ? ojh_moe_mt_groups(dev, d, E, 2) : dots && n_ff <= 1024 ? (d + 31) / 32 : (d + 15) / 16, E, 1};
         // (Q5_K rows have no matrix-core form: they stay on integer dots at every batch size)
-        if ((rc = ojh_launch(dev, down5 ? "moe_down_q5k_m" : mt_down ? "moe_down_q4k_mt" : mm ? "moe_down_q4k_mm" : "moe_down_q4k_m",
+        if ((rc = ojh_launch(dev, down5 ? down_m.c_str() : mt_down ? "moe_down_q4k_mt" : mm ? "moe_down_q4k_mm" : "moe_down_q4k_m",
                              {aq->ptr, as_->ptr, (char *)down->raw->ptr + down->off, dv->ptr, offsets, list},
                              {n_ff, d, NA}, g, mt_down ? b512 : b256)))
             return rc;

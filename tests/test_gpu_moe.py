@@ -182,23 +182,25 @@ def test_matrix_core_forms_agree(gpu, orc, pkg, monkeypatch, T, E, ksel, d, nff,
 
 
 @pytest.mark.parametrize("T,E,ksel,d,nff", [(1, 16, 4, 512, 768), (3, 8, 8, 2304, 256), (20, 8, 3, 512, 768),
-                                             (70, 4, 2, 256, 2304)])
-def test_expert_ffn_with_q5k_down_tensors(gpu, orc, pkg, T, E, ksel, d, nff):
-    """Expert `down` tensors in Q5_K (dot_q5k, crates/ojas-cpu/src/cpu_math.rs:638-670) beside Q4_K
-    gate / up: the decode form, the grouped integer dots, and a batch large enough that gate / up
-    run on the matrix cores while down stays on integer dots."""
+                                             (70, 4, 2, 256, 2304), (5, 8, 2, 300 * 256 // 100, 1280)])
+@pytest.mark.parametrize("dty", [13, 14])
+def test_expert_ffn_with_q5k_down_tensors(gpu, orc, pkg, T, E, ksel, d, nff, dty):
+    """Expert `down` tensors in Q5_K or Q6_K (dot_q5k / dot_q6k, crates/ojas-cpu/src/cpu_math.rs:638-722)
+    beside Q4_K gate / up: the decode form, the grouped integer dots (short rows of 1 to 3 super-blocks,
+    up to 8, and longer), and a batch large enough that gate / up run on the matrix cores while down stays
+    on integer dots."""
     gate = pkg.synth.q4k_weights(E * nff, d, "moe5", "gate", E, d, nff)
     up = pkg.synth.q4k_weights(E * nff, d, "moe5", "up", E, d, nff)
-    down = pkg.synth.q5k_weights(E * d, nff, "moe5", "down", E, d, nff)
+    down = pkg.synth.weights(dty, E * d, nff, "moe5", "down", E, d, nff, dty)
     x = pkg.synth.normal_f32(T * d, "moe5", "x", T, d).reshape(T, d)
     lg = pkg.synth.normal_f32(T * E, "moe5", "lg", T, E).reshape(T, E)
     gi, gw, idx_d, wgt_d = _route(gpu, lg, ksel)
-    lg_, lu_, ld_ = gpu.lin(Q4_K, E * nff, d, gate), gpu.lin(Q4_K, E * nff, d, up), gpu.lin(13, E * d, nff, down)
+    lg_, lu_, ld_ = gpu.lin(Q4_K, E * nff, d, gate), gpu.lin(Q4_K, E * nff, d, up), gpu.lin(dty, E * d, nff, down)
     yd = gpu.upload(np.full(T * d + d, 12345.5, np.float32))
     gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd)
     got = gpu.read(yd, T * d + d)
     assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
-    want = orc.moe_ffn(x, gi, gw, gate, up, Q4_K, down, 13, E, nff, mode=0)
+    want = orc.moe_ffn(x, gi, gw, gate, up, Q4_K, down, dty, E, nff, mode=0)
     assert peak_err(got[:T * d].reshape(T, d), want) <= TOL
 
 
