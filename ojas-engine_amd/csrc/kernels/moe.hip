@@ -494,6 +494,93 @@ moe_down_q6k_dec(const float* act, const uchar* wd, const uint* idx, const float
     moe_down_dec_body<W6k, false>(act, wd, idx, wgt, y, K, N, KSEL, E, ACC);
 }
 
+// ------------------------------------------------------------------ Q8_0 experts, f32 activations
+//   moe_gu_q80(x, wg, wu, act, idx, K, N)              grid [ceil(N/8), KSEL, tokens], block 256
+//   moe_down_q80(act, wd, y, idx, wgt, K, N, KSEL)     grid [1 .. ceil(N/16), tokens, 1], block 256 (rows grid-stride,
+//                                                      so the reference's ceil(N/32) workgroups are a valid grid)
+// The reference's expert kernels by their own names and arguments
+// (crates/ojas-cuda/src/kernels/moe.rs:75-125): act[j][n] = silu(gate_e . x) * (up_e . x) for the expert
+// e = idx[j] of slot j, and y[n] += sum_j wgt[j] * (down_e . act[j]) — the down launch accumulates onto
+// y, slots in order.  Q8_0 rows meet f32 activations, as dot_q80 does
+// (crates/ojas-cpu/src/cpu_math.rs:971-981).  The third (second) grid dimension walks tokens: token t
+// reads x + t K, idx + t KSEL, wgt + t KSEL and writes act + t KSEL N, y + t N; a one-token caller
+// leaves it at 1.  Four lanes share a 34-byte block, a wave walks 16 blocks per step.  The trailing E is
+// not part of the reference's argument list: the dispatcher derives it from the extent of the expert
+// tensors, and a slot whose index is E or more contributes zeros rather than reading past them.
+__device__ __forceinline__ float q80f_block_part(const uchar* blk, uint p, float4 x0, float4 x1) {
+    const u32x2_a2 q = *(const u32x2_a2*)(blk + 2u + p * 8u);
+    float a = (float)(signed char)(q.x) * x0.x;
+    a = fmaf((float)(signed char)(q.x >> 8), x0.y, a);
+    a = fmaf((float)(signed char)(q.x >> 16), x0.z, a);
+    a = fmaf((float)((int)q.x >> 24), x0.w, a);
+    a = fmaf((float)(signed char)(q.y), x1.x, a);
+    a = fmaf((float)(signed char)(q.y >> 8), x1.y, a);
+    a = fmaf((float)(signed char)(q.y >> 16), x1.z, a);
+    a = fmaf((float)((int)q.y >> 24), x1.w, a);
+    return f16_bits_to_f32(*(const ushort*)blk) * a;
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+moe_gu_q80(const float* __restrict__ x, const uchar* __restrict__ wg, const uchar* __restrict__ wu,
+           float* __restrict__ act, const uint* __restrict__ idx, uint K, uint N, uint E) {
+    const uint lane = threadIdx.x & 63u, g = lane >> 2, p = lane & 3u;
+    const uint j = blockIdx.y, t = blockIdx.z, ksel = gridDim.y;
+    const uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 2u;
+    if (row0 >= N) return;
+    const uint e = idx[t * ksel + j], nb = e < E ? K >> 5 : 0u;
+    const size_t rb = (size_t)(K >> 5) * Q80_BYTES;
+    const float* xt = x + (size_t)t * K;
+    float ag[2] = {0.0f, 0.0f}, au[2] = {0.0f, 0.0f};
+    for (uint b = g; b < nb; b += 16u) {
+        const float4* xp = (const float4*)(xt + (size_t)b * 32u + p * 8u);
+        const float4 x0 = xp[0], x1 = xp[1];
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const size_t off = ((size_t)e * N + min(row0 + (uint)r, N - 1u)) * rb + (size_t)b * Q80_BYTES;
+            ag[r] += q80f_block_part(wg + off, p, x0, x1);
+            au[r] += q80f_block_part(wu + off, p, x0, x1);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        const float gs = wave_sum(ag[r]), us = wave_sum(au[r]);
+        if (lane == 0 && row0 + r < N) act[((size_t)t * ksel + j) * N + row0 + r] = (gs / (1.0f + expf(-gs))) * us;
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q80(const float* __restrict__ act, const uchar* __restrict__ wd, float* __restrict__ y,
+             const uint* __restrict__ idx, const float* __restrict__ wgt, uint K, uint N, uint KSEL, uint E) {
+    const uint lane = threadIdx.x & 63u, g = lane >> 2, p = lane & 3u;
+    const uint t = blockIdx.y;
+    const uint nb = K >> 5;
+    const size_t rb = (size_t)nb * Q80_BYTES;
+    for (uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 4u; row0 < N; row0 += gridDim.x * 16u) {
+        float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (uint j = 0; j < KSEL; j++) {
+            const uint e = idx[t * KSEL + j];
+            if (e >= E) continue;
+            const float wj = wgt[t * KSEL + j];
+            const float* xr = act + ((size_t)t * KSEL + j) * K;
+            float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (uint b = g; b < nb; b += 16u) {
+                const float4* xp = (const float4*)(xr + (size_t)b * 32u + p * 8u);
+                const float4 x0 = xp[0], x1 = xp[1];
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    a[r] += q80f_block_part(wd + ((size_t)e * N + min(row0 + (uint)r, N - 1u)) * rb + (size_t)b * Q80_BYTES, p, x0, x1);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) res[r] += wj * wave_sum(a[r]);
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (row0 + r < N) y[(size_t)t * N + row0 + r] += res[r];
+        }
+    }
+}
+
 // ------------------------------------------------------------------ grouped products on the matrix cores
 // A workgroup owns 16 rows of expert e and walks the expert's assignments 16 at a time.  Per 32-weight
 // sub-block one v_mfma_i32_16x16x32_i8 multiplies the tile of quantized activations (A: lane

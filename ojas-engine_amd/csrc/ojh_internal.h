@@ -113,6 +113,10 @@ struct ojh_kernel_spec {
     int rows_per_wave;   // for the row-parallel matvecs
     ojh_check_fn check;
     ojh_shape_fn shape;
+    // Expert kernels whose reference argument list carries no expert count: buffers 1 .. expert_bufs are
+    // expert tensors, need[] is one expert's bytes, and the dispatcher appends min(extent / need) as a
+    // trailing constant so that an index past the tensors multiplies nothing instead of reading past them.
+    int expert_bufs = 0;
 };
 const std::vector<ojh_kernel_spec> &ojh_manifest_table();
 const ojh_kernel_spec *ojh_find_kernel(const char *name);

@@ -5,6 +5,7 @@
 // that says "ensure_family first", read synchronises), none of its code.
 #include <dlfcn.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -335,7 +336,16 @@ extern "C" int ojh_dispatch(ojh_device *dev, const char *name, int n_bufs, ojh_b
             return ojh_fail(OJH_ERR_ARG, "%s: buffer %d (+%zu) must be %zu-byte aligned", name, i, off, align[i]);
         ptrs.push_back((void *)addr);
     }
-    return ojh_launch(dev, name, ptrs, std::vector<uint32_t>(consts, consts + n_consts), grid, block);
+    std::vector<uint32_t> cv(consts, consts + n_consts);
+    if (s->expert_bufs) {   // how many experts the tensors hold: the kernel's bound on the routed indices
+        size_t experts = 1024;
+        for (int i = 1; i <= s->expert_bufs; i++) {
+            size_t off = offsets ? (size_t)offsets[i] : 0;
+            experts = std::min(experts, (bufs[i]->bytes - off) / need[i]);
+        }
+        cv.push_back((uint32_t)experts);
+    }
+    return ojh_launch(dev, name, ptrs, cv, grid, block);
 }
 
 extern "C" int ojh_submit(ojh_device *dev) {

@@ -205,6 +205,32 @@ def tvec(n: int, seed: int) -> np.ndarray:
     return ((s >> np.uint32(9)).astype(np.float32) / np.float32(1 << 23)) - np.float32(1.0)
 
 
+def tvec_first(seeds: np.ndarray) -> np.ndarray:
+    """tvec(1, seed)[0] for an array of seeds."""
+    s = np.asarray(seeds, np.uint64) & np.uint64(0xFFFFFFFF)
+    s = (s * np.uint64(2654435761) + np.uint64(1)) & np.uint64(0xFFFFFFFF)
+    s = (s * np.uint64(1664525) + np.uint64(1013904223)) & np.uint64(0xFFFFFFFF)
+    return ((s >> np.uint64(9)).astype(np.float32) / np.float32(1 << 23)) - np.float32(1.0)
+
+
+def q80_rows_lcg(rows: int, k: int, seed: int) -> tuple[np.ndarray, np.ndarray]:
+    """Q8_0 rows of the reference's GPU conformance tests and the values they decode to
+    (crates/ojas-cuda/tests/conformance.rs:358-376): block (r, b) has d = f16(0.002 + 0.001 |tvec(1, seed ^ (r nb + b))|),
+    code i = round(127 tvec(1, seed + r k + 32 b + i)), halves away from zero."""
+    nb = k // 32
+    blk = np.arange(rows * nb, dtype=np.uint64)
+    d = (np.float32(0.002) + np.float32(0.001) * np.abs(tvec_first(np.uint64(seed) ^ blk))).astype(np.float16)
+    t = tvec_first(np.uint64(seed) + np.arange(rows * k, dtype=np.uint64)) * np.float32(127.0)
+    q = np.clip(np.sign(t) * np.floor(np.abs(t) + np.float32(0.5)), -127, 127).astype(np.int8).reshape(rows * nb, 32)
+    out = np.empty((rows * nb, 34), np.uint8)
+    dv = d.view(np.uint16)
+    out[:, 0] = dv & 0xFF
+    out[:, 1] = dv >> 8
+    out[:, 2:] = q.view(np.uint8)
+    plain = (q.astype(np.float32) * d.astype(np.float32)[:, None]).reshape(rows, k)
+    return out.reshape(-1), plain
+
+
 def q80_rows_closed_form(n: int, k: int):
     """Q8_0 rows and activations of the reference's `native_q8_matvec_ksplit_matches_cpu`:
     d = f16(0.003 + ((r+b) mod 7) * 0.001), q = ((17r + 11b + 5j) mod 31) - 15,

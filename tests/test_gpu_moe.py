@@ -14,6 +14,7 @@ from conftest import peak_err
 
 pytestmark = pytest.mark.gpu
 Q4_K = 12
+Q8_0 = 8
 TOL = 1e-3
 TOL_SEEN = 3e-4
 
@@ -256,6 +257,87 @@ def test_streamed_experts_by_slot_offsets(gpu, pkg, T, E, ksel, d, nff, accum):
     with pytest.raises(pkg.OjasHipError, match="needs"):
         gpu.moe_ffn_slots(gpu.upload(x), T, d, nff, ksel, ag, gpu.upload_bytes(og[:-1]), au, gpu.upload_bytes(og), ad,
                           gpu.upload_bytes(od), wgt_d, yd)
+
+
+def _rel_err(got, want):
+    """The reference's per-element measure (crates/ojas-cuda/tests/conformance.rs:215-220)."""
+    return float(np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-6)))
+
+
+def test_q80_experts_reference_procedure(gpu, pkg):
+    """Q8_0 experts through `moe_gu_q80` and `moe_down_q80` with the reference's own arguments and
+    launch geometry (crates/ojas-cuda/tests/conformance.rs:412-457): E=8, K=256, N=64, experts {3, 6}
+    weighted {0.7, 0.3}, against the plain products of the decoded values, bound 2e-3 per element."""
+    k, n, experts, ksel = 256, 64, 8, 2
+    x = pkg.synth.tvec(k, 61)
+    gbytes, gplain = pkg.synth.q80_rows_lcg(experts * n, k, 62)
+    ubytes, uplain = pkg.synth.q80_rows_lcg(experts * n, k, 63)
+    dbytes, dplain = pkg.synth.q80_rows_lcg(experts * k, n, 64)
+    idx, wgt = np.array([3, 6], np.uint32), np.array([0.7, 0.3], np.float32)
+    want = np.zeros(k, np.float64)
+    x64 = x.astype(np.float64)
+    for j, e in enumerate(idx):
+        gv = gplain[e * n:(e + 1) * n].astype(np.float64) @ x64
+        uv = uplain[e * n:(e + 1) * n].astype(np.float64) @ x64
+        act = gv / (1.0 + np.exp(-gv)) * uv
+        want += float(wgt[j]) * (dplain[e * k:(e + 1) * k].astype(np.float64) @ act)
+    gpu.ensure_family("moe")
+    xd, gd, ud, dd = gpu.upload(x), gpu.upload_bytes(gbytes), gpu.upload_bytes(ubytes), gpu.upload_bytes(dbytes)
+    idxd, wgtd = gpu.upload_bytes(idx), gpu.upload(wgt)
+    actd, outd = gpu.alloc(ksel * n), gpu.upload(np.zeros(k, np.float32))
+    enc = gpu.begin()
+    gpu.dispatch(enc, "moe_gu_q80", [(xd, 0), (gd, 0), (ud, 0), (actd, 0), (idxd, 0)], [k, n], [-(-n // 8), ksel, 1], [256, 1, 1])
+    gpu.dispatch(enc, "moe_down_q80", [(actd, 0), (dd, 0), (outd, 0), (idxd, 0), (wgtd, 0)], [n, k, ksel],
+                 [-(-k // 32), 1, 1], [256, 1, 1])
+    gpu.submit(enc)
+    got = gpu.read(outd, k)
+    assert _rel_err(got, want.astype(np.float32)) < 2e-3
+    assert peak_err(got, want) <= 2e-6
+    # the geometry the library itself names gives the same bits, and the down launch accumulates
+    g2, b2 = gpu.launch_shape("moe_down_q80", n, k, 1)
+    assert g2 == [-(-k // 16), 1, 1] and b2 == [256, 1, 1]
+    out2 = gpu.upload(np.ones(k, np.float32))
+    gpu.dispatch(gpu.begin(), "moe_down_q80", [(actd, 0), (dd, 0), (out2, 0), (idxd, 0), (wgtd, 0)], [n, k, ksel], g2, b2)
+    assert np.array_equal(gpu.read(out2, k), np.float32(1.0) + got)
+    # an index past the tensors multiplies nothing: the same as that slot with weight zero
+    bad = gpu.upload_bytes(np.array([3, experts], np.uint32))
+    act3, out3, out4 = gpu.alloc(ksel * n), gpu.upload(np.zeros(k, np.float32)), gpu.upload(np.zeros(k, np.float32))
+    gpu.dispatch(gpu.begin(), "moe_gu_q80", [(xd, 0), (gd, 0), (ud, 0), (act3, 0), (bad, 0)], [k, n], [-(-n // 8), ksel, 1], [256, 1, 1])
+    gpu.dispatch(gpu.begin(), "moe_down_q80", [(act3, 0), (dd, 0), (out3, 0), (bad, 0), (wgtd, 0)], [n, k, ksel], g2, b2)
+    assert np.all(gpu.read(act3, ksel * n)[n:] == 0.0)
+    w0 = gpu.upload(np.array([0.7, 0.0], np.float32))
+    gpu.dispatch(gpu.begin(), "moe_down_q80", [(actd, 0), (dd, 0), (out4, 0), (idxd, 0), (w0, 0)], [n, k, ksel], g2, b2)
+    assert np.array_equal(gpu.read(out3, k), gpu.read(out4, k))
+    with pytest.raises(pkg.OjasHipError, match="needs"):
+        gpu.dispatch(gpu.begin(), "moe_down_q80", [(actd, 0), (dd, len(dbytes) - 34), (out3, 0), (idxd, 0), (wgtd, 0)],
+                     [n, k, ksel], g2, b2)
+
+
+@pytest.mark.parametrize("T,E,ksel,d,nff,accum", [(1, 8, 2, 256, 64, False), (5, 16, 4, 512, 352, True),
+                                                   (40, 8, 8, 1024, 768, False), (3, 4, 1, 2080, 96, True)])
+def test_q80_experts_through_the_ffn_entry(gpu, orc, pkg, T, E, ksel, d, nff, accum):
+    """The same kernels under `ojh_moe_ffn`, many tokens in one launch, against the CPU path's f32
+    products over Q8_0 rows (crates/ojas-cpu/src/cpu_math.rs:971-981 under cpu_glm.rs:551-582)."""
+    gate = pkg.synth.q80_weights(E * nff, d, "moe8", "gate", E, d, nff)
+    up = pkg.synth.q80_weights(E * nff, d, "moe8", "up", E, d, nff)
+    down = pkg.synth.q80_weights(E * d, nff, "moe8", "down", E, d, nff)
+    x = pkg.synth.normal_f32(T * d, "moe8", "x", T, d).reshape(T, d)
+    lg = pkg.synth.normal_f32(T * E, "moe8", "lg", T, E).reshape(T, E)
+    gi, gw, idx_d, wgt_d = _route(gpu, lg, ksel)
+    # the running output is given the products' own magnitude, so its f32 rounding does not mask theirs
+    y0 = np.float32(0.01) * pkg.synth.normal_f32(T * d, "moe8", "y0").reshape(T, d) if accum else np.zeros((T, d), np.float32)
+    init = np.concatenate([y0.ravel() if accum else np.full(T * d, 777.0, np.float32), np.full(d, 12345.5, np.float32)])
+    yd = gpu.alloc(T * d + d)
+    lg_, lu_, ld_ = gpu.lin(Q8_0, E * nff, d, gate), gpu.lin(Q8_0, E * nff, d, up), gpu.lin(Q8_0, E * d, nff, down)
+    want = orc.moe_ffn(x, gi, gw, gate, up, Q8_0, down, Q8_0, E, nff, mode=0, y0=y0)
+    for mode in (pkg.ACT_AUTO, pkg.ACT_FLOAT):
+        gpu.write_bytes(yd, 0, init)
+        gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, accum=accum, act_mode=mode)
+        got = gpu.read(yd, T * d + d)
+        assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
+        assert peak_err(got[:T * d].reshape(T, d) - y0, want - y0) <= 2e-5
+    with pytest.raises(pkg.OjasHipError, match="f32 activations"):
+        gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, act_mode=pkg.ACT_Q8K)
 
 
 def test_expert_ffn_rejects_what_it_cannot_run(gpu, pkg):
