@@ -46,7 +46,7 @@ enum {
 };
 
 /* GGUF tensor types handled by this path (crates/ojas-formats/src/gguf.rs:563-591). */
-enum { OJH_Q4_0 = 2, OJH_Q4_1 = 3, OJH_Q5_0 = 6, OJH_Q5_1 = 7, OJH_Q8_0 = 8, OJH_Q4_K = 12, OJH_Q5_K = 13, OJH_Q6_K = 14,
+enum { OJH_Q4_0 = 2, OJH_Q4_1 = 3, OJH_Q5_0 = 6, OJH_Q5_1 = 7, OJH_Q8_0 = 8, OJH_Q2_K = 10, OJH_Q3_K = 11, OJH_Q4_K = 12, OJH_Q5_K = 13, OJH_Q6_K = 14,
        OJH_IQ4_NL = 20, OJH_IQ4_XS = 23 };
 
 /* Element type of an activation buffer handed to ojh_mm. */
@@ -59,8 +59,9 @@ enum { OJH_X_F32 = 0, OJH_X_BF16 = 1, OJH_X_F16 = 2 };
  *                 `dot_iq4nl` and `dot_iq4xs` do (:971-981, :993-1010, :943-967): asking for
  *                 OJH_ACT_Q8K on IQ4 rows is refused, and no MFMA tile reads them (every token
  *                 count runs on the matvec entries).  The same holds for the legacy 32-weight
- *                 blocks Q4_0, Q4_1, Q5_0, Q5_1, which the reference runs on its GPU path only
- *                 (f32 activations against the weights of `dequant_to_f16`'s arms :653-703).
+ *                 blocks Q4_0, Q4_1, Q5_0, Q5_1 and for Q2_K and Q3_K, which the reference runs on
+ *                 its GPU path only (f32 activations against the weights of `dequant_to_f16`'s
+ *                 arms :653-703 and :730-795).
  *   OJH_ACT_FLOAT — activations kept in floating point (f32 for the GEMV, rounded to f16 into the
  *                 MFMA tile for the GEMM): the contract of the reference's GPU kernels
  *                 (crates/ojas-core/src/quant_src.rs:779-867, crates/ojas-cuda/src/kernels/gemm_q.rs:1-56).

@@ -186,6 +186,61 @@ dequant_iq4xs_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nb
     }
 }
 
+// Q2_K and Q3_K keep four 2-bit planes per byte: within a half of 128 weights, byte l of the half's 32 code
+// bytes holds weights l, l + 32, l + 64, l + 96 at bits 0, 2, 4, 6, and scale 8 half + 2 j + l / 16 covers the
+// 16 weights (plane j, l / 16).  32 threads per super-block; thread t decodes the eight consecutive weights
+// 128 half + 32 j + 8 (t % 4) .. + 7 with half = t / 16, j = (t / 4) % 4.
+extern "C" __global__ void __launch_bounds__(256)
+dequant_q2k_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
+    // block { u8 scales[16]; u8 qs[64]; half d; half dmin; }: w = (d * sc) * q - dmin * m, every step rounded
+    // (crates/ojas-formats/src/gguf.rs:730-754)
+    size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x;
+    size_t b = tid >> 5;
+    if (b >= nblocks) return;
+    const uint t = (uint)tid & 31u, half = t >> 4, j = (t >> 2) & 3u, l0 = (t & 3u) * 8u;
+    const uchar* blk = w + b * Q2K_BYTES;
+    const uint sc = blk[half * 8u + j * 2u + (l0 >> 4)];
+    const uint dd = *(const uint*)(blk + 80);
+    const float dl = __fmul_rn(f16_bits_to_f32(dd & 0xFFFFu), (float)(sc & 0xFu));
+    const float ml = __fmul_rn(f16_bits_to_f32(dd >> 16), (float)(sc >> 4));
+    const uint* qp = (const uint*)(blk + 16u + half * 32u + l0);
+    const uint q0 = (qp[0] >> (2u * j)) & 0x03030303u, q1 = (qp[1] >> (2u * j)) & 0x03030303u;
+    ushort* o = out + b * 256u + half * 128u + j * 32u + l0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        o[i] = f32_to_f16_bits(__fsub_rn(__fmul_rn(dl, (float)((q0 >> (8 * i)) & 0xFFu)), ml));
+        o[4 + i] = f32_to_f16_bits(__fsub_rn(__fmul_rn(dl, (float)((q1 >> (8 * i)) & 0xFFu)), ml));
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+dequant_q3k_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
+    // block { u8 hmask[32]; u8 qs[64]; u8 scales[12]; half d; }: w = (d * (sc - 32)) * (q - (mask bit ? 0 : 4)),
+    // bit 4 half + j of hmask[l] belonging to weight (half, j, l) (crates/ojas-formats/src/gguf.rs:755-795).
+    // Blocks are 110 bytes: two-byte alignment is all a block has.
+    size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x;
+    size_t b = tid >> 5;
+    if (b >= nblocks) return;
+    const uint t = (uint)tid & 31u, half = t >> 4, j = (t >> 2) & 3u, l0 = (t & 3u) * 8u;
+    const uchar* blk = w + b * Q3K_BYTES;
+    const u32_a2* raw = (const u32_a2*)(blk + 96);
+    const int sc = q3k_scale6(raw[0], raw[1], raw[2], half * 8u + j * 2u + (l0 >> 4));
+    const float dl = __fmul_rn(f16_bits_to_f32(*(const ushort*)(blk + 108)), (float)sc);
+    const u32_a2* qp = (const u32_a2*)(blk + 32u + half * 32u + l0);
+    const u32_a2* hp = (const u32_a2*)(blk + l0);
+    const uint sh = half * 4u + j;
+    ushort* o = out + b * 256u + half * 128u + j * 32u + l0;
+#pragma unroll
+    for (int v = 0; v < 2; v++) {
+        const uint q = (qp[v] >> (2u * j)) & 0x03030303u, h = (hp[v] >> sh) & 0x01010101u;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int code = (int)((q >> (8 * i)) & 0xFFu) - (((h >> (8 * i)) & 1u) ? 0 : 4);
+            o[4 * v + i] = f32_to_f16_bits(__fmul_rn(dl, (float)code));
+        }
+    }
+}
+
 // The legacy 32-weight blocks: one thread per weight.  AFFINE: {d, m} header and w = d * q + m (a product and
 // a sum, each rounded), else w = d * (q - 8 | 16); FIVE: a 4-byte field of fifth bits ahead of the nibbles.
 template <bool FIVE, bool AFFINE>

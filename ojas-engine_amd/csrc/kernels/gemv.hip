@@ -835,6 +835,204 @@ gemv_nat_q80_lds_bias(const float* x, const uchar* w, float* y, const float* bs,
 }
 
 // ------------------------------------------------------------------ entries
+// ------------------------------------------------------------------ Q2_K and Q3_K rows, f32 activations
+// Both keep four 2-bit planes per byte: within a half of 128 weights, byte l of the half's 32 code bytes
+// holds weights l, l + 32, l + 64, l + 96 at bits 0, 2, 4, 6, and scale 8 half + 2 j + l / 16 covers
+// (plane j, l / 16).  Sixteen lanes share a super-block: lane c takes dword c of the 64 code bytes — half
+// c / 8, bytes 4 (c % 8) .. + 3 — so its 16 weights meet four float4 of x 32 floats apart, and a wave walks
+// four super-blocks per step.  Codes stay unsigned bytes (v_cvt_f32_ubyteN); what is subtracted meets the
+// sum of each plane's four activations:
+//   Q2_K  d * sum_j sc_j (q_j . x_j)  -  dmin * sum_j m_j sum(x_j)
+//   Q3_K  d * sum_j (sc_j - 32) ((q_j | bit << 2) . x_j  -  4 sum(x_j))      (mask bit set = no subtraction)
+// The reference has these two on its GPU path and in dequant_to_f16 only
+// (crates/ojas-core/src/quant_src.rs:97-98, :357-420; crates/ojas-formats/src/gguf.rs:730-795).
+struct Q2kW {
+    static constexpr uint BYTES = Q2K_BYTES;
+    struct Frag { uint q, s0, s1, dd; };
+    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
+        const uint* blk = (const uint*)(row + (size_t)u * Q2K_BYTES);
+        const uint c = lane & 15u;
+        Frag f;
+        f.s0 = blk[(c >> 3) * 2u];
+        f.s1 = blk[(c >> 3) * 2u + 1u];
+        f.q = blk[4u + c];
+        f.dd = blk[20];
+        return f;
+    }
+    static __device__ __forceinline__ float dot(const Frag& f, uint lane, const float4 (&xv)[4], const float (&xs)[4]) {
+        const uint sh = (lane & 4u) << 1;     // bytes 4 (c % 8) .. from 16 on: the second scale of each plane
+        float ad = 0.0f, am = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint sc = ((j < 2 ? f.s0 : f.s1) >> (16u * (j & 1) + sh)) & 0xFFu;
+            ad = fmaf((float)(sc & 0xFu), dot4_ub((f.q >> (2 * j)) & 0x03030303u, xv[j], 0.0f), ad);
+            am = fmaf((float)(sc >> 4), xs[j], am);
+        }
+        return f16_bits_to_f32(f.dd & 0xFFFFu) * ad - f16_bits_to_f32(f.dd >> 16) * am;
+    }
+};
+
+struct Q3kW {
+    static constexpr uint BYTES = Q3K_BYTES;
+    struct Frag { uint q, h, r0, r1, r2, d16; };
+    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
+        const uchar* blk = row + (size_t)u * Q3K_BYTES;     // 110 bytes: two-byte alignment only
+        const uint c = lane & 15u;
+        Frag f;
+        f.h = *(const u32_a2*)(blk + (c & 7u) * 4u);
+        f.q = *(const u32_a2*)(blk + 32u + c * 4u);
+        f.r0 = *(const u32_a2*)(blk + 96);
+        f.r1 = *(const u32_a2*)(blk + 100);
+        f.r2 = *(const u32_a2*)(blk + 104);
+        f.d16 = *(const ushort*)(blk + 108);
+        return f;
+    }
+    static __device__ __forceinline__ float dot(const Frag& f, uint lane, const float4 (&xv)[4], const float (&xs)[4]) {
+        const uint c = lane & 15u, half = c >> 3, part = (c >> 2) & 1u;
+        float a = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint code = ((f.q >> (2 * j)) & 0x03030303u) | (((f.h >> (half * 4u + j)) & 0x01010101u) << 2);
+            const int sc = q3k_scale6(f.r0, f.r1, f.r2, half * 8u + 2u * j + part);
+            a = fmaf((float)sc, dot4_ub(code, xv[j], 0.0f) - 4.0f * xs[j], a);
+        }
+        return f16_bits_to_f32(f.d16) * a;
+    }
+};
+
+// the lane's four activation fragments of super-block u
+__device__ __forceinline__ void kq2_x(const float* __restrict__ x, uint u, uint lane, float4 (&xv)[4], float (&xs)[4]) {
+    const uint c = lane & 15u;
+    const float* xp = x + (size_t)u * 256u + (c >> 3) * 128u + (c & 7u) * 4u;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        xv[j] = *(const float4*)(xp + 32 * j);
+        xs[j] = sum4(xv[j]);
+    }
+}
+
+template <class W, int R, int MODE>
+__device__ __forceinline__ void gemv_nat_kq2_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                  float* __restrict__ y, const float* __restrict__ bs,
+                                                  uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    if (row0 >= N) return;
+    const uint nu = K >> 8;
+    const size_t rb = (size_t)nu * W::BYTES;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (uint u = lane >> 4; u < nu; u += 4u) {
+        typename W::Frag f[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) f[r] = W::load(w + (size_t)min(row0 + r, N - 1u) * rb, u, lane);
+        float4 xv[4];
+        float xs[4];
+        kq2_x(x, u, lane, xv, xs);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += W::dot(f[r], lane, xv, xs);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float s = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, s);
+    }
+}
+
+template <class W, int MT>
+__device__ __forceinline__ void gemv_nat_kq2_m_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                    float* __restrict__ y, uint K, uint N, uint M, uint ACC) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const uint nu = K >> 8;
+    const uchar* wr = w + (size_t)row * nu * W::BYTES;
+    for (uint m0 = 0; m0 < M; m0 += MT) {
+        float acc[MT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) acc[i] = 0.0f;
+        for (uint u = lane >> 4; u < nu; u += 4u) {
+            const typename W::Frag f = W::load(wr, u, lane);
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                float4 xv[4];
+                float xs[4];
+                kq2_x(x + (size_t)min(m0 + i, M - 1u) * K, u, lane, xv, xs);
+                acc[i] += W::dot(f, lane, xv, xs);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float s = wave_sum(acc[i]);
+            if (lane == 0 && m0 + i < M) {
+                float* o = y + (size_t)(m0 + i) * N + row;
+                *o = ACC ? *o + s : s;
+            }
+        }
+    }
+}
+
+// Many rows, K <= 4096: rows grid-stride, the lane's share of x (four steps of 16 floats) in registers;
+// steps past the row hold zeros and repeat its last super-block.
+template <class W>
+__device__ __forceinline__ void gemv_nat_kq2_px_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                     float* __restrict__ y, uint K, uint N) {
+    const uint lane = threadIdx.x & 63u;
+    const uint nu = K >> 8;
+    const size_t rb = (size_t)nu * W::BYTES;
+    float4 xr[4][4];
+    float xs[4][4];
+    uint uc[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const uint u = (lane >> 4) + 4u * (uint)s;
+        uc[s] = min(u, nu - 1u);
+        if (u < nu) {
+            kq2_x(x, u, lane, xr[s], xs[s]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                xr[s][j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                xs[s][j] = 0.0f;
+            }
+        }
+    }
+    const uint nwaves = gridDim.x * (blockDim.x >> 6);
+    for (uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2u; row0 < N; row0 += nwaves * 2u) {
+        const uchar* r0 = w + (size_t)row0 * rb;
+        const uchar* r1 = w + (size_t)min(row0 + 1u, N - 1u) * rb;
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const typename W::Frag f0 = W::load(r0, uc[s], lane), f1 = W::load(r1, uc[s], lane);
+            a0 += W::dot(f0, lane, xr[s], xs[s]);
+            a1 += W::dot(f1, lane, xr[s], xs[s]);
+        }
+        a0 = wave_sum(a0);
+        a1 = wave_sum(a1);
+        if (lane == 0) {
+            y[row0] = a0;
+            if (row0 + 1u < N) y[row0 + 1u] = a1;
+        }
+    }
+}
+
+#define GEMV_NAT_KQ2(FMT, W)                                                                                \
+    template <int R, int MODE>                                                                              \
+    __device__ __forceinline__ void gemv_nat_##FMT##_body(const float* x, const uchar* w, float* y,         \
+                                                          const float* bs, uint K, uint N) {                \
+        gemv_nat_kq2_body<W, R, MODE>(x, w, y, bs, K, N); }                                                 \
+    template <int MT>                                                                                       \
+    __device__ __forceinline__ void gemv_nat_##FMT##_m_body(const float* x, const uchar* w, float* y,       \
+                                                            uint K, uint N, uint M, uint ACC) {             \
+        gemv_nat_kq2_m_body<W, MT>(x, w, y, K, N, M, ACC); }                                                \
+    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_px(                                  \
+        const float* x, const uchar* w, float* y, uint K, uint N) {                                         \
+        gemv_nat_kq2_px_body<W>(x, w, y, K, N); }
+GEMV_NAT_KQ2(q2k, Q2kW)
+GEMV_NAT_KQ2(q3k, Q3kW)
+
 #define GEMV_NAT_ENTRIES(FMT)                                                                              \
     extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_r1(                                 \
         const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
@@ -865,3 +1063,5 @@ GEMV_NAT_ENTRIES(q40)
 GEMV_NAT_ENTRIES(q41)
 GEMV_NAT_ENTRIES(q50)
 GEMV_NAT_ENTRIES(q51)
+GEMV_NAT_ENTRIES(q2k)
+GEMV_NAT_ENTRIES(q3k)

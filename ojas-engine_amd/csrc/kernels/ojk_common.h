@@ -18,6 +18,8 @@ typedef unsigned short ushort;
 #define Q6K_BYTES 210u
 #define IQ4NL_BYTES 18u
 #define IQ4XS_BYTES 136u
+#define Q2K_BYTES 84u
+#define Q3K_BYTES 110u
 
 // Vector types that may sit on a 2-byte boundary: Q8_0 (34 B) and Q6_K (210 B) blocks are only
 // 2-byte aligned inside a row.  gfx950 runs in unaligned-access mode, so these compile to one
@@ -25,6 +27,16 @@ typedef unsigned short ushort;
 struct __attribute__((packed, aligned(2))) u32x4_a2 { uint x, y, z, w; };
 struct __attribute__((packed, aligned(2))) u32x2_a2 { uint x, y; };
 typedef uint __attribute__((aligned(2))) u32_a2;
+
+// Scale i (0 .. 15) of a Q3_K block from its three packed words (crates/ojas-formats/src/gguf.rs:764-774):
+// the low nibble sits in byte i (i < 8) or in the high nibble of byte i - 8, the two high bits in byte
+// 8 + i % 4 at bit 2 (i / 4); stored biased by 32.
+__device__ __forceinline__ int q3k_scale6(uint r0, uint r1, uint r2, uint i) {
+    const uint src = (i & 4u) ? r1 : r0;
+    const uint lo = (src >> (8u * (i & 3u) + ((i & 8u) >> 1))) & 0xFu;
+    const uint hi = (r2 >> (8u * (i & 3u) + 2u * (i >> 2))) & 3u;
+    return (int)(lo | (hi << 4)) - 32;
+}
 
 __device__ __forceinline__ float f16_bits_to_f32(uint bits16) {
     return __half2float(__ushort_as_half((ushort)bits16));

@@ -20,15 +20,24 @@ static const ojh_block_format kFormats[] = {
     {OJH_Q4_1, 20, 32, "q41"},
     {OJH_Q5_0, 22, 32, "q50"},
     {OJH_Q5_1, 24, 32, "q51"},
+    {OJH_Q2_K, 84, 256, "q2k"},
+    {OJH_Q3_K, 110, 256, "q3k"},
 };
 
 // Formats whose CPU path multiplies the raw row with f32 activations (dot_q80, dot_iq4nl, dot_iq4xs:
 // crates/ojas-cpu/src/cpu_math.rs:1131-1141, :1179) instead of quantizing them per 256.
 bool ojh_float_rows(uint32_t t) { return t == OJH_Q8_0 || ojh_float_only(t); }
 // ... and for which this library has the f32-activation matvecs only: no int8-activation form, no MFMA tile
-// (the IQ4 types, and the legacy 32-weight blocks the reference runs on its GPU path alone)
+// (the IQ4 types, and the legacy 32-weight blocks and Q2_K / Q3_K, which the reference runs on its GPU path alone)
 bool ojh_float_only(uint32_t t) {
-    return t == OJH_IQ4_NL || t == OJH_IQ4_XS || t == OJH_Q4_0 || t == OJH_Q4_1 || t == OJH_Q5_0 || t == OJH_Q5_1;
+    return t == OJH_IQ4_NL || t == OJH_IQ4_XS || t == OJH_Q4_0 || t == OJH_Q4_1 || t == OJH_Q5_0 || t == OJH_Q5_1 ||
+           t == OJH_Q2_K || t == OJH_Q3_K;
+}
+
+// What the kernels' loads need of a block tensor's address: the widest power of two (up to 16) dividing the
+// block size, except that only Q2_K's kernels use the 4 of a block size that is 4 mod 8.
+size_t ojh_block_align(const ojh_block_format *f) {
+    return f->bytes % 16 == 0 ? 16 : f->bytes % 8 == 0 ? 8 : f->type == OJH_Q2_K ? 4 : 2;
 }
 
 const ojh_block_format *ojh_format(uint32_t t) {
@@ -83,7 +92,7 @@ static int check_gemv_nat(const ojh_kernel_spec *s, const uint32_t *c, const uin
     need[1] = (size_t)N * (K / f->weights) * f->bytes;
     need[2] = (size_t)N * 4;
     if (s->n_bufs == 4) need[3] = (size_t)N * 4;
-    align[1] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
+    align[1] = ojh_block_align(f);
     align[2] = align[3] = 4;
     return OJH_OK;
 }
@@ -271,7 +280,7 @@ static int check_gemv_q8k_px(const ojh_kernel_spec *s, const uint32_t *c, const 
     need[2] = (size_t)N * (K / f->weights) * f->bytes;
     need[3] = (size_t)N * 4;
     align[1] = 4;
-    align[2] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
+    align[2] = ojh_block_align(f);
     align[3] = 4;
     return OJH_OK;
 }
@@ -288,7 +297,7 @@ static int check_gemv_nat_px(const ojh_kernel_spec *s, const uint32_t *c, const 
     need[0] = (size_t)K * 4;
     need[1] = (size_t)N * (K / f->weights) * f->bytes;
     need[2] = (size_t)N * 4;
-    align[1] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
+    align[1] = ojh_block_align(f);
     align[2] = 4;
     return OJH_OK;
 }
@@ -321,7 +330,7 @@ static int check_gemv_q8k(const ojh_kernel_spec *s, const uint32_t *c, const uin
     need[3] = (size_t)N * 4;
     if (s->n_bufs == 5) need[4] = (size_t)N * 4;
     align[1] = 4;
-    align[2] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
+    align[2] = ojh_block_align(f);
     align[3] = align[4] = 4;
     return OJH_OK;
 }
@@ -348,7 +357,7 @@ static int check_gemv_q8k_x4(const ojh_kernel_spec *s, const uint32_t *c, const 
         size_t rows = E[i] - (i ? E[i - 1] : 0);
         need[2 + i] = rows * (K / f->weights) * f->bytes;
         need[6 + i] = rows * 4;
-        align[2 + i] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
+        align[2 + i] = ojh_block_align(f);
         align[6 + i] = 4;
     }
     return OJH_OK;
@@ -435,7 +444,7 @@ static int check_gemv_nat_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     need[0] = (size_t)M * K * 4;
     need[1] = (size_t)N * (K / f->weights) * f->bytes;
     need[2] = (size_t)M * N * 4;
-    align[1] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
+    align[1] = ojh_block_align(f);
     align[2] = 4;
     return OJH_OK;
 }
@@ -497,7 +506,7 @@ static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     need[2] = (size_t)N * (K / f->weights) * f->bytes;
     need[3] = (size_t)M * N * 4;
     align[1] = 4;
-    align[2] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
+    align[2] = ojh_block_align(f);
     align[3] = 4;
     if (mf || mk) {           // whole aligned dwords around every piece: the last one may end 2 bytes on
         need[2] = (need[2] + 3) & ~(size_t)3;
@@ -604,7 +613,7 @@ static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint
         return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover %u blocks", s->name, nb);
     need[0] = (size_t)nb * f->bytes;
     need[1] = (size_t)nb * f->weights * 2;
-    align[0] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
+    align[0] = ojh_block_align(f);
     align[1] = 8;
     return OJH_OK;
 }
@@ -641,7 +650,7 @@ static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_
     need[0] = (size_t)M * K * 2;
     need[1] = (size_t)N * (K / f->weights) * f->bytes;
     need[2] = (size_t)M * N * 4;
-    align[1] = f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16;
+    align[1] = ojh_block_align(f);
     align[2] = 4;
     return OJH_OK;
 }

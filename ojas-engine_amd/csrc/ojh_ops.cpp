@@ -60,7 +60,7 @@ extern "C" int ojh_lin_wrap(ojh_device *dev, uint32_t type, uint32_t n, uint32_t
     int rc = lin_check(type, n, k, &rb);
     if (rc) return rc;
     const ojh_block_format *f = ojh_format(type);
-    if ((rc = span_ok("ojh_lin_wrap: raw", raw, off, rb * n, f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16))) return rc;
+    if ((rc = span_ok("ojh_lin_wrap: raw", raw, off, rb * n, ojh_block_align(f)))) return rc;
     ojh_lin *l = new ojh_lin();
     l->type = type; l->n = n; l->k = k; l->row_bytes = rb; l->raw = raw; l->off = off; l->owns_raw = false;
     *out = l;
@@ -86,7 +86,7 @@ extern "C" int ojh_dequant_f16(ojh_device *dev, uint32_t type, const ojh_buf *ra
     size_t nb = n_weights / f->weights;
     if (nb > 0x7FFFFFFFu / 64) return ojh_fail(OJH_ERR_ARG, "dequant: too many blocks in one call (%zu)", nb);
     int rc;
-    if ((rc = span_ok("dequant: raw", raw, raw_off, nb * f->bytes, f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16))) return rc;
+    if ((rc = span_ok("dequant: raw", raw, raw_off, nb * f->bytes, ojh_block_align(f)))) return rc;
     if ((rc = span_ok("dequant: out", out, out_off, n_weights * 2, 2))) return rc;
     if ((rc = ensure(dev, "dequant"))) return rc;
     std::string name = std::string("dequant_") + f->tag + "_f16";
@@ -273,7 +273,7 @@ static int mm_common_checks(const char *who, const ojh_lin *w, ojh_buf *y, size_
     int rc;
     if ((rc = span_ok("y", y, y_off, (size_t)m * w->n * 4, 4))) return rc;
     if (bias && (rc = span_ok("bias", bias, 0, (size_t)w->n * 4, 4))) return rc;
-    if ((rc = span_ok("w", w->raw, w->off, w->row_bytes * w->n, f->bytes % 16 ? (f->bytes % 8 ? 2 : 8) : 16))) return rc;
+    if ((rc = span_ok("w", w->raw, w->off, w->row_bytes * w->n, ojh_block_align(f)))) return rc;
     *fmt = f;
     return OJH_OK;
 }
@@ -365,9 +365,9 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         act_mode = OJH_ACT_Q8K;
     }
 
-    // IQ4_NL / IQ4_XS (dot_iq4nl / dot_iq4xs) and Q4_0 / Q4_1 / Q5_0 / Q5_1: f32 activations against the raw
+    // IQ4_NL / IQ4_XS (dot_iq4nl / dot_iq4xs), Q4_0 / Q4_1 / Q5_0 / Q5_1 and Q2_K / Q3_K: f32 activations against the raw
     // rows at every token count; no int8-activation form and no MFMA tile read them.
-    const bool iq4 = ojh_float_only(w->type);   // (the IQ4 types and the legacy 32-weight blocks)
+    const bool iq4 = ojh_float_only(w->type);   // (the IQ4 types, the legacy 32-weight blocks, Q2_K, Q3_K)
     if (iq4 && act_mode == OJH_ACT_Q8K)
         return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: %s rows take f32 activations only (OJH_ACT_FLOAT or OJH_ACT_AUTO)", f->tag);
 

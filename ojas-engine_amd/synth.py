@@ -14,8 +14,9 @@ import numpy as np
 
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+Q2_K, Q3_K = 10, 11
 BLOCK_SHAPE = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256), IQ4_NL: (18, 32), IQ4_XS: (136, 256),
-               Q4_0: (18, 32), Q4_1: (20, 32), Q5_0: (22, 32), Q5_1: (24, 32)}
+               Q4_0: (18, 32), Q4_1: (20, 32), Q5_0: (22, 32), Q5_1: (24, 32), Q2_K: (84, 256), Q3_K: (110, 256)}
 
 
 def seed_of(*names) -> int:
@@ -159,9 +160,33 @@ def legacy_weights(ty: int, n: int, k: int, *names) -> np.ndarray:
     return out.reshape(-1)
 
 
+def q2k_weights(n: int, k: int, *names) -> np.ndarray:
+    """Q2_K rows: scales/mins nibbles and 2-bit codes uniform, d = f16(|N(0,0.02)| / 24), dmin = f16(|N(0,0.02)| / 60)
+    in the block's last four bytes."""
+    g = rng(*names)
+    nb = n * (k // 256)
+    out = g.integers(0, 256, size=(nb, 84), dtype=np.uint8)
+    d = (np.abs(g.standard_normal(nb) * 0.02) / 24.0).astype(np.float16).view(np.uint16)
+    m = (np.abs(g.standard_normal(nb) * 0.02) / 60.0).astype(np.float16).view(np.uint16)
+    out[:, 80], out[:, 81], out[:, 82], out[:, 83] = d & 0xFF, d >> 8, m & 0xFF, m >> 8
+    return out.reshape(-1)
+
+
+def q3k_weights(n: int, k: int, *names) -> np.ndarray:
+    """Q3_K rows: mask bits, 2-bit codes and packed 6-bit scales uniform, d = f16(|N(0,0.02)| / 64) in the last two bytes."""
+    g = rng(*names)
+    nb = n * (k // 256)
+    out = g.integers(0, 256, size=(nb, 110), dtype=np.uint8)
+    d = (np.abs(g.standard_normal(nb) * 0.02) / 64.0).astype(np.float16).view(np.uint16)
+    out[:, 108], out[:, 109] = d & 0xFF, d >> 8
+    return out.reshape(-1)
+
+
 def weights(ty: int, n: int, k: int, *names) -> np.ndarray:
     if ty in (Q4_0, Q4_1, Q5_0, Q5_1):
         return legacy_weights(ty, n, k, *names)
+    if ty in (Q2_K, Q3_K):
+        return {Q2_K: q2k_weights, Q3_K: q3k_weights}[ty](n, k, *names)
     return {Q8_0: q80_weights, Q4_K: q4k_weights, Q5_K: q5k_weights, Q6_K: q6k_weights,
             IQ4_NL: iq4nl_weights, IQ4_XS: iq4xs_weights}[ty](n, k, *names)
 
@@ -188,6 +213,11 @@ def synth_blocks(ty: int, nb: int) -> np.ndarray:
             blocks[i, 2], blocks[i, 3] = int(dmin) & 0xFF, int(dmin) >> 8
         elif ty == Q6_K:
             blocks[i, 208], blocks[i, 209] = d & 0xFF, d >> 8
+        elif ty == Q2_K:
+            blocks[i, 80], blocks[i, 81] = d & 0xFF, d >> 8
+            blocks[i, 82], blocks[i, 83] = int(dmin) & 0xFF, int(dmin) >> 8
+        elif ty == Q3_K:
+            blocks[i, 108], blocks[i, 109] = d & 0xFF, d >> 8
         else:
             blocks[i, 0], blocks[i, 1] = d & 0xFF, d >> 8
     return out

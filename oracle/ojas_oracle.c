@@ -97,6 +97,8 @@ int ojo_block_shape(uint32_t ty, uint32_t *bytes, uint32_t *weights) { /* synth.
     uint32_t b, w;
     switch (ty) {
     case OJO_Q8_0: b = 34; w = 32; break;
+    case OJO_Q2_K: b = 84; w = 256; break;
+    case OJO_Q3_K: b = 110; w = 256; break;
     case OJO_Q4_K: b = 144; w = 256; break;
     case OJO_Q5_K: b = 176; w = 256; break;
     case OJO_Q6_K: b = 210; w = 256; break;
@@ -133,6 +135,13 @@ int ojo_synth_blocks(uint32_t ty, size_t nb, uint8_t *out) { /* synth.rs:29-64 *
         case OJO_Q6_K:
             blk[208] = (uint8_t)d; blk[209] = (uint8_t)(d >> 8);
             break;
+        case OJO_Q2_K: /* d and dmin close the block */
+            blk[80] = (uint8_t)d; blk[81] = (uint8_t)(d >> 8);
+            blk[82] = (uint8_t)dmin; blk[83] = (uint8_t)(dmin >> 8);
+            break;
+        case OJO_Q3_K:
+            blk[108] = (uint8_t)d; blk[109] = (uint8_t)(d >> 8);
+            break;
         default:
             blk[0] = (uint8_t)d; blk[1] = (uint8_t)(d >> 8);
         }
@@ -156,6 +165,15 @@ static inline void scale_min_k4(int j, const uint8_t *q, uint8_t *sc, uint8_t *m
     }
 }
 
+/* Sixteen 6-bit scales of a Q3_K block from its 12 packed bytes (gguf.rs:764-774): scale i has its low
+ * nibble in byte i (i < 8) or in the high nibble of byte i - 8, and its two high bits in byte 8 + i % 4
+ * at bit 2 (i / 4).  Stored biased by 32. */
+static inline int q3k_scale(const uint8_t *raw, int i) {
+    int lo = i < 8 ? raw[i] & 0xF : raw[i - 8] >> 4;
+    int hi = (raw[8 + (i & 3)] >> (2 * (i >> 2))) & 3;
+    return (int)(int8_t)(lo | (hi << 4)) - 32;
+}
+
 int ojo_dequant_to_f16(const uint8_t *b, uint32_t ty, size_t n, uint16_t *out) {
     uint32_t bb, wpb;
     if (!ojo_block_shape(ty, &bb, &wpb) || n % wpb) return -1;
@@ -167,6 +185,35 @@ int ojo_dequant_to_f16(const uint8_t *b, uint32_t ty, size_t n, uint16_t *out) {
         case OJO_Q8_0: { /* gguf.rs:704-709 */
             float d = rdh(blk, 0);
             for (int j = 0; j < 32; j++) o[j] = ojo_f32_to_f16(d * (float)(int8_t)blk[2 + j]);
+        } break;
+        case OJO_Q2_K: { /* gguf.rs:730-754: scales[16], qs[64], d, dmin; w = (d * sc) * q - dmin * m */
+            const uint8_t *sc = blk, *qs = blk + 16;
+            float d = rdh(blk, 80), dmin = rdh(blk, 82);
+            int is = 0;
+            for (int half = 0; half < 2; half++)
+                for (int j = 0; j < 4; j++)
+                    for (int part = 0; part < 2; part++, is++) {
+                        float dl = d * (float)(sc[is] & 0xF), ml = dmin * (float)(sc[is] >> 4);
+                        for (int l = 0; l < 16; l++) {
+                            int q = (qs[half * 32 + part * 16 + l] >> (2 * j)) & 3;
+                            o[half * 128 + j * 32 + part * 16 + l] = ojo_f32_to_f16(dl * (float)q - ml);
+                        }
+                    }
+        } break;
+        case OJO_Q3_K: { /* gguf.rs:755-795: hmask[32], qs[64], scales[12], d; a clear mask bit subtracts 4 */
+            const uint8_t *hm = blk, *qs = blk + 32, *raw = blk + 96;
+            float d = rdh(blk, 108);
+            int is = 0;
+            for (int half = 0; half < 2; half++)
+                for (int j = 0; j < 4; j++)
+                    for (int part = 0; part < 2; part++, is++) {
+                        float dl = d * (float)q3k_scale(raw, is);
+                        for (int l = 0; l < 16; l++) {
+                            int q = (qs[half * 32 + part * 16 + l] >> (2 * j)) & 3;
+                            int hi = (hm[part * 16 + l] >> (half * 4 + j)) & 1 ? 0 : 4;
+                            o[half * 128 + j * 32 + part * 16 + l] = ojo_f32_to_f16(dl * (float)(q - hi));
+                        }
+                    }
         } break;
         case OJO_Q4_0: { /* gguf.rs:653-661: w = d * (nib - 8); low nibbles first, then high nibbles */
             float d = rdh(blk, 0);
@@ -299,6 +346,23 @@ int ojo_dequant_to_f64(const uint8_t *b, uint32_t ty, size_t n, double *out) {
         case OJO_Q8_0: {
             double d = rdh(blk, 0);
             for (int j = 0; j < 32; j++) o[j] = d * (double)(int8_t)blk[2 + j];
+        } break;
+        case OJO_Q2_K: {
+            double d = rdh(blk, 80), dmin = rdh(blk, 82);
+            for (int i = 0; i < 256; i++) {
+                int half = i >> 7, j = (i >> 5) & 3, l = i & 31, is = half * 8 + j * 2 + (l >> 4);
+                int q = (blk[16 + half * 32 + l] >> (2 * j)) & 3;
+                o[i] = d * (double)(blk[is] & 0xF) * (double)q - dmin * (double)(blk[is] >> 4);
+            }
+        } break;
+        case OJO_Q3_K: {
+            double d = rdh(blk, 108);
+            for (int i = 0; i < 256; i++) {
+                int half = i >> 7, j = (i >> 5) & 3, l = i & 31, is = half * 8 + j * 2 + (l >> 4);
+                int q = (blk[32 + half * 32 + l] >> (2 * j)) & 3;
+                int hi = (blk[l] >> (half * 4 + j)) & 1 ? 0 : 4;
+                o[i] = d * (double)q3k_scale(blk + 96, is) * (double)(q - hi);
+            }
         } break;
         case OJO_Q4_0: case OJO_Q4_1: case OJO_Q5_0: case OJO_Q5_1: {
             const int five = ty == OJO_Q5_0 || ty == OJO_Q5_1, affine = ty == OJO_Q4_1 || ty == OJO_Q5_1;

@@ -37,7 +37,7 @@ extern "C" {
 #endif
 
 /* GGUF type ids (crates/ojas-formats/src/gguf.rs:563-591). */
-enum { OJO_Q4_0 = 2, OJO_Q4_1 = 3, OJO_Q5_0 = 6, OJO_Q5_1 = 7, OJO_Q8_0 = 8, OJO_Q4_K = 12, OJO_Q5_K = 13, OJO_Q6_K = 14,
+enum { OJO_Q4_0 = 2, OJO_Q4_1 = 3, OJO_Q5_0 = 6, OJO_Q5_1 = 7, OJO_Q8_0 = 8, OJO_Q2_K = 10, OJO_Q3_K = 11, OJO_Q4_K = 12, OJO_Q5_K = 13, OJO_Q6_K = 14,
        OJO_IQ4_NL = 20, OJO_IQ4_XS = 23 };
 
 /* IEEE binary16 <-> binary32, round-to-nearest-even, subnormals kept

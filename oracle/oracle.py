@@ -17,6 +17,7 @@ _LIB_PATH = os.path.join(_HERE, "libojas_oracle.so")
 
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+Q2_K, Q3_K = 10, 11
 
 
 def build(force: bool = False) -> str:

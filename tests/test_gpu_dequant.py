@@ -5,8 +5,9 @@ import pytest
 pytestmark = pytest.mark.gpu
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+Q2_K, Q3_K = 10, 11
 DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6,
-           IQ4_NL: 0xA5D4CF4E5DB3A1BF, IQ4_XS: 0x1429CAFB4DF9AF64}
+           IQ4_NL: 0xA5D4CF4E5DB3A1BF, IQ4_XS: 0x1429CAFB4DF9AF64, Q2_K: 0xBDA788876D584945, Q3_K: 0xA3FCFCD97CE8A0A9}
 
 
 def _dequant(gpu, ty, raw, n):
@@ -16,7 +17,7 @@ def _dequant(gpu, ty, raw, n):
     return gpu.read(out, n, np.uint16)
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
+@pytest.mark.parametrize("ty", [Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
 def test_reference_digests_on_device(gpu, orc, pkg, ty):
     """The reference's own regression digests (crates/ojas-formats/tests/quant_formats.rs:38-48),
     computed over what the GPU decoded."""
@@ -27,7 +28,7 @@ def test_reference_digests_on_device(gpu, orc, pkg, ty):
 
 @pytest.mark.parametrize("ty,n,k", [(Q8_0, 37, 4096), (Q4_K, 129, 4096), (Q6_K, 65, 4096), (Q5_K, 16, 1024),
                                     (IQ4_NL, 33, 2080), (IQ4_XS, 21, 4096), (Q4_0, 33, 2080), (Q4_1, 9, 4096),
-                                    (Q5_0, 33, 2080), (Q5_1, 9, 4096)])
+                                    (Q5_0, 33, 2080), (Q5_1, 9, 4096), (Q2_K, 21, 2304), (Q3_K, 33, 4096)])
 def test_bit_exact_on_benchmark_distributions(gpu, orc, pkg, ty, n, k):
     raw = orc.synth_blocks(ty, n * k // pkg.synth.BLOCK_SHAPE[ty][1]) if ty == Q5_K else \
         pkg.synth.weights(ty, n, k, "dq", ty)
@@ -35,18 +36,19 @@ def test_bit_exact_on_benchmark_distributions(gpu, orc, pkg, ty, n, k):
     assert np.array_equal(got, orc.dequant_to_f16(raw, ty, n * k))
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K])
 def test_bit_exact_with_extreme_scales(gpu, orc, pkg, ty):
     """Subnormal, tiny, huge and negative f16 scales: every rounding path of the decoder."""
     bb, wpb = pkg.synth.BLOCK_SHAPE[ty]
     scales = np.array([0x0001, 0x0200, 0x03FF, 0x0400, 0x7BFF, 0x8001, 0xBC00, 0x3555, 0x0000, 0x1234], np.uint16)
     nb = scales.size * 3
     raw = orc.synth_blocks(ty, nb).reshape(nb, bb).copy()
-    off = 208 if ty == Q6_K else 0
+    off = {Q6_K: 208, Q2_K: 80, Q3_K: 108}.get(ty, 0)
     for i in range(nb):
         raw[i, off:off + 2] = np.array([scales[i % scales.size]], np.uint16).view(np.uint8)
-        if ty in (Q4_K, Q5_K, Q4_1, Q5_1):
-            raw[i, 2:4] = np.array([scales[(i * 7 + 3) % scales.size]], np.uint16).view(np.uint8)
+        if ty in (Q4_K, Q5_K, Q4_1, Q5_1, Q2_K):
+            at = 82 if ty == Q2_K else 2
+            raw[i, at:at + 2] = np.array([scales[(i * 7 + 3) % scales.size]], np.uint16).view(np.uint8)
     raw = raw.reshape(-1)
     got = _dequant(gpu, ty, raw, nb * wpb)
     want = orc.dequant_to_f16(raw, ty, nb * wpb)

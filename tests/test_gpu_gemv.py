@@ -14,6 +14,7 @@ from conftest import peak_err
 pytestmark = pytest.mark.gpu
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+Q2_K, Q3_K = 10, 11
 TAG = {Q8_0: "q80", Q4_K: "q4k", Q5_K: "q5k", Q6_K: "q6k"}
 TOL_Q8K = 1e-3     # the parity bar against the CPU reference
 TOL_Q8K_SEEN = 2e-5
@@ -69,7 +70,7 @@ def test_q8k_matvec_matches_cpu_reference(gpu, orc, pkg, ty, n, k):
     assert err <= TOL_Q8K_SEEN <= TOL_Q8K, err
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K])
 @pytest.mark.parametrize("n,k", [(13, 2560), (1024, 4096), (96, 14336), (4099, 4096), (33001, 2816)])
 def test_float_matvec_matches_dequant_dot(gpu, orc, pkg, ty, n, k):
     w, x = _inputs(pkg, ty, n, k, "b")
@@ -96,7 +97,7 @@ def test_q80_matvec_matches_dot_q80(gpu, orc, pkg):
     assert peak_err(gpu.read(yd, n), want) <= 1e-5
 
 
-@pytest.mark.parametrize("ty,tag", [(Q4_K, "q4k"), (Q6_K, "q6k")])
+@pytest.mark.parametrize("ty,tag", [(Q4_K, "q4k"), (Q6_K, "q6k"), (Q2_K, "q2k"), (Q3_K, "q3k")])
 @pytest.mark.parametrize("n,k", [(33000, 256), (40001, 2560), (32768, 4096)])
 def test_float_head_form_keeps_activations_in_registers(gpu, orc, pkg, ty, tag, n, k):
     """From 32768 rows a float-activation matvec runs grid-stride with the wave's f32 activations in
@@ -160,12 +161,12 @@ def test_q80_closed_form_rows_with_guards(gpu, pkg):
     assert np.max(np.abs(got[2:-2] - want)) < 2e-4
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K])
 @pytest.mark.parametrize("mode", ["float", "q8k"])
 def test_bias_accum_and_batched_variants(gpu, orc, pkg, ty, mode):
     """The five checks of crates/ojas-models/examples/nat_gemv_gate.rs:36-163: plain, bias
     (1000 + i), accumulate onto a seeded y, batched M=3 with different rows, batched accumulate."""
-    if ty in (Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1) and mode == "q8k":
+    if ty in (Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K) and mode == "q8k":
         pytest.skip("this format keeps f32 activations in the CPU reference")
     if ty == Q5_K and mode == "float":
         pytest.skip("Q5_K has the int8-activation matvec only")

@@ -11,8 +11,9 @@ from conftest import peak_err
 pytestmark = pytest.mark.gpu
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
-FLOAT_ROWS = (Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1)
-LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1)
+Q2_K, Q3_K = 10, 11
+FLOAT_ROWS = (Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K)
+LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K)   # no dot in the CPU path: GPU-path formats
 
 
 def _cases():
@@ -20,7 +21,7 @@ def _cases():
     rows = [17, 130, 1000, 4099, 6144, 8200, 14336, 24576, 33000, 40001]
     ks = [256, 512, 1024, 2560, 4096, 5120, 7168, 14336]
     out = []
-    for ty in (Q4_K, Q6_K, Q5_K, Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1):
+    for ty in (Q4_K, Q6_K, Q5_K, Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K):
         for _ in range(7 if ty not in LEGACY else 3):
             n, k = int(g.choice(rows)), int(g.choice(ks))
             m = int(g.choice([1, 2, 3, 4, 5, 7, 8, 9, 16, 17, 33, 40]))

@@ -5,15 +5,16 @@ import pytest
 
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+Q2_K, Q3_K = 10, 11
 
 # crates/ojas-formats/tests/quant_formats.rs:38-40, 45, 48
 DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6,
-           IQ4_NL: 0xA5D4CF4E5DB3A1BF, IQ4_XS: 0x1429CAFB4DF9AF64}
+           IQ4_NL: 0xA5D4CF4E5DB3A1BF, IQ4_XS: 0x1429CAFB4DF9AF64, Q2_K: 0xBDA788876D584945, Q3_K: 0xA3FCFCD97CE8A0A9}
 # crates/ojas-core/src/iq_tables.rs:881-884
 KVALUES_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float64)
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
+@pytest.mark.parametrize("ty", [Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
 def test_dequant_digest_matches_reference(orc, pkg, ty):
     wpb = pkg.synth.BLOCK_SHAPE[ty][1]
     raw = orc.synth_blocks(ty, 40)
@@ -22,7 +23,7 @@ def test_dequant_digest_matches_reference(orc, pkg, ty):
     assert orc.digest_f16(bits) == DIGESTS[ty]
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K])
 def test_synth_blocks_two_implementations_agree(orc, pkg, ty):
     assert np.array_equal(orc.synth_blocks(ty, 9), pkg.synth.synth_blocks(ty, 9))
 
@@ -204,6 +205,54 @@ def test_legacy_block_closed_forms(orc, pkg, ty):
     got64 = orc.dequant_to_f64(raw.reshape(-1), ty, 50 * 32).reshape(50, 32)
     exact = d.astype(np.float64)[:, None] * (q.astype(np.float64) - (0.0 if affine else (16.0 if five else 8.0))) + m.astype(np.float64)[:, None]
     assert np.array_equal(got64, exact)
+
+
+@pytest.mark.parametrize("ty", [Q2_K, Q3_K])
+def test_two_bit_plane_blocks_against_numpy(orc, pkg, ty):
+    """Q2_K and Q3_K decoded weight by weight in numpy from the block definitions: weight i of a super-block
+    sits in code byte 32 (i // 128) + i % 32 at bits 2 ((i // 32) % 4), its scale is number i // 16; Q2_K:
+    (d sc) q - dmin m with sc, m the nibbles of a scale byte; Q3_K: a third bit in hmask[i % 32] at bit i // 32
+    (clear = subtract 4), 6-bit scales biased by 32 whose low nibbles fill bytes 0..7 (low, then high nibble)
+    and whose high bit pairs fill bytes 8..11.  The f64 decoder must be exact, the f16 one the f32 expression
+    of the reference rounded once more; special blocks: all mask bits set / clear, every scale value."""
+    nb = 64
+    raw = orc.synth_blocks(ty, nb).reshape(nb, -1).copy()
+    if ty == Q3_K:
+        raw[0, :32], raw[1, :32] = 0xFF, 0x00
+        sc = (np.arange(16) * 4 + 1) % 64     # block 2: scale i = (4 i + 1) % 64, written with the packing rule
+        packed = np.zeros(12, np.uint8)
+        for i, v in enumerate(sc):
+            packed[i % 8] |= (v & 0xF) << (4 * (i // 8))
+            packed[8 + i % 4] |= (v >> 4) << (2 * (i // 4))
+        raw[2, 96:108] = packed
+    i = np.arange(256)
+    half, plane, l, grp = i // 128, (i // 32) % 4, i % 32, i // 16
+    if ty == Q2_K:
+        d = raw[:, 80:82].copy().view(np.float16).astype(np.float64)
+        dmin = raw[:, 82:84].copy().view(np.float16).astype(np.float64)
+        q = (raw[:, 16 + 32 * half + l] >> (2 * plane)) & 3
+        scb = raw[:, grp]
+        exact = d * (scb & 0xF) * q - dmin * (scb >> 4)
+        dl = (d.astype(np.float32) * (scb & 0xF).astype(np.float32)).astype(np.float32)
+        ml = (dmin.astype(np.float32) * (scb >> 4).astype(np.float32)).astype(np.float32)
+        f32 = (dl * q.astype(np.float32)).astype(np.float32) - ml
+    else:
+        d = raw[:, 108:110].copy().view(np.float16).astype(np.float64)
+        q = ((raw[:, 32 + 32 * half + l] >> (2 * plane)) & 3).astype(np.int64)
+        hbit = (raw[:, l] >> (i // 32)) & 1
+        code = q - 4 * (1 - hbit.astype(np.int64))
+        sraw = raw[:, 96:108]
+        lo = np.where(grp < 8, sraw[:, grp % 8] & 0xF, sraw[:, grp % 8] >> 4)
+        hi = (sraw[:, 8 + grp % 4] >> (2 * (grp // 4))) & 3
+        s6 = (lo | (hi << 4)).astype(np.int64) - 32
+        assert np.array_equal(s6[2, ::16] + 32, (np.arange(16) * 4 + 1) % 64)
+        exact = d * s6 * code
+        f32 = (d.astype(np.float32) * s6.astype(np.float32)).astype(np.float32) * code.astype(np.float32)
+    got64 = orc.dequant_to_f64(raw.reshape(-1), ty, nb * 256).reshape(nb, 256)
+    assert np.array_equal(got64, exact)
+    with np.errstate(over="ignore"):
+        want16 = f32.astype(np.float32).astype(np.float16).view(np.uint16)
+    assert np.array_equal(orc.dequant_to_f16(raw.reshape(-1), ty, nb * 256).reshape(nb, 256), want16)
 
 
 def test_iq4_closed_forms(orc):
