@@ -11,6 +11,7 @@
  *
  * How each function is pinned (a function without such a check would say "parity unpinned"):
  *   dequant Q4_K/Q5_K/Q6_K  FNV-1a digests held by crates/ojas-formats/tests/quant_formats.rs:38-40
+ *   dequant Q2_K/Q3_K       the digests of the same table (quant_formats.rs:36-37), weight-by-weight numpy restatement
  *   dequant IQ4_NL/IQ4_XS   the digests of the same table (quant_formats.rs:45,48), one-hot codes vs the codebook
  *   dequant Q8_0            closed form of crates/ojas-formats/tests/rows.rs:13-18
  *   dequant Q4_0/Q4_1/Q5_0/Q5_1  closed forms only (d * (q - 8 | 16), d * q + m, nibble halves, the fifth-bit field):
