@@ -253,10 +253,11 @@ int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uin
  * crates/ojas-metal/src/kernels/moe.rs:199-272):
  *   y[t] (+)= sum_j wgt[t][j] * Wd_e( silu(Wg_e x[t]) * (Wu_e x[t]) ),  e = idx[t][j].
  * gate/up: n_expert stacked Q4_K matrices [n_ff][d]; down: n_expert stacked [d][n_ff], Q4_K, Q5_K or Q6_K.
- * Or all three Q8_0: f32 activations meet the raw rows as dot_q80 does
- * (crates/ojas-cpu/src/cpu_math.rs:971-981) through the reference's own expert kernels moe_gu_q80 /
- * moe_down_q80 (crates/ojas-cuda/src/kernels/moe.rs:75-125), one launch each over all tokens; there
- * act_mode is OJH_ACT_AUTO or OJH_ACT_FLOAT, d and n_ff multiples of 32.
+ * Or gate+up and down each one of Q8_0, IQ4_XS, IQ4_NL: f32 activations meet the raw rows as dot_q80 /
+ * dot_iq4xs / dot_iq4nl do (crates/ojas-cpu/src/cpu_math.rs:943-1010) through the reference's own expert
+ * kernels moe_gu_<fmt> / moe_down_<fmt> (crates/ojas-cuda/src/kernels/moe.rs:75-125, moe_iq.rs:64-112),
+ * one launch each over all tokens; there act_mode is OJH_ACT_AUTO or OJH_ACT_FLOAT and d, n_ff are
+ * whole blocks of the formats.
  * Expert indices must be below n_expert (one that is not never reads outside the tensors; what
  * it contributes is unspecified). Up to 8 tokens run as two launches addressed
  * by assignment (bit-identical to the grouped integer-dot pipeline); larger batches are grouped

@@ -35,6 +35,7 @@ FAMILIES = {
     "gemm_xl": ("gemm_xl.hip", ["-ffp-contract=off"]),
     "gemm_q8k": ("gemm_q8k.hip", []),
     "moe": ("moe.hip", []),
+    "moe_iq": ("moe_iq.hip", []),
     "rowq8": ("rowq8.hip", ["-ffp-contract=off"]),
 }
 

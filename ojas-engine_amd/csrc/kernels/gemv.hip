@@ -14,6 +14,7 @@
 // the R rows of the wave.  Scales stay factored: the lane accumulates sum(code * x) per sub-block
 // and applies d*sc (and -dmin*m*sum(x) for Q4_K) once per sub-block.
 #include "ojk_common.h"
+#include "ojk_rows.h"
 
 enum { ST_SET = 0, ST_ACCUM = 1, ST_BIAS = 2 };
 
@@ -23,20 +24,6 @@ __device__ __forceinline__ void store_row(float* y, const float* bs, uint n, flo
     else if (MODE == ST_ACCUM) y[n] += v;
     else y[n] = v + bs[n];
 }
-
-__device__ __forceinline__ float ub0(uint v) { return (float)(v & 0xFFu); }
-__device__ __forceinline__ float ub1(uint v) { return (float)((v >> 8) & 0xFFu); }
-__device__ __forceinline__ float ub2(uint v) { return (float)((v >> 16) & 0xFFu); }
-__device__ __forceinline__ float ub3(uint v) { return (float)(v >> 24); }
-
-// sum of 4 unsigned bytes of `w` times 4 floats
-__device__ __forceinline__ float dot4_ub(uint w, float4 x, float acc) {
-    acc = fmaf(ub0(w), x.x, acc);
-    acc = fmaf(ub1(w), x.y, acc);
-    acc = fmaf(ub2(w), x.z, acc);
-    return fmaf(ub3(w), x.w, acc);
-}
-__device__ __forceinline__ float sum4(float4 v) { return (v.x + v.y) + (v.z + v.w); }
 
 // ------------------------------------------------------------------ Q4_K
 // Lane (g, l) = (lane/8, lane%8): 16 quant bytes l*16.. of super-block g -> 16 weights of
@@ -361,11 +348,6 @@ gemv_nat_q6k_px(const float* x, const uchar* w, float* y, uint K, uint N) { gemv
 
 // ------------------------------------------------------------------ Q8_0
 // Four lanes share a 34-byte block (8 int8 each); a wave walks 16 blocks (512 weights) per step.
-__device__ __forceinline__ float sb0(uint v) { return (float)(signed char)(v); }
-__device__ __forceinline__ float sb1(uint v) { return (float)(signed char)(v >> 8); }
-__device__ __forceinline__ float sb2(uint v) { return (float)(signed char)(v >> 16); }
-__device__ __forceinline__ float sb3(uint v) { return (float)((int)v >> 24); }
-
 __device__ __forceinline__ float q80_lane_dot(uint d16, u32x2_a2 q, float4 x0, float4 x1) {
     float a = sb0(q.x) * x0.x;
     a = fmaf(sb1(q.x), x0.y, a);
@@ -444,115 +426,8 @@ __device__ __forceinline__ void gemv_nat_q80_m_body(const float* __restrict__ x,
     }
 }
 
-// ------------------------------------------------------------------ IQ4_NL, IQ4_XS
-// Both store 4-bit indices into the sixteen-level codebook; within a 32-weight group the low
-// nibbles of its 16 bytes are weights 0..15 and the high nibbles weights 16..31.  A lane takes one
-// dword of indices: four low-nibble weights and the four 16 further on, against two float4 of x.
-// IQ4_NL: 18-byte blocks {f16 d; qs[16]}, four lanes per block, a wave walks 16 blocks per step.
-// IQ4_XS: 136-byte super-blocks {f16 d; u16 scales_h; u8 scales_l[4]; qs[128]}, 32 lanes per
-// super-block (lane / 4 = sub-block, its 6-bit scale minus 32 times d applied per lane).
-__device__ __forceinline__ float iq4_lane_dot(uint q, float4 x0, float4 x1) {
-    const uint lo = iq4_levels4(q & 0x0F0F0F0Fu), hi = iq4_levels4((q >> 4) & 0x0F0F0F0Fu);
-    float a = sb0(lo) * x0.x;
-    a = fmaf(sb0(hi), x1.x, a);
-    a = fmaf(sb1(lo), x0.y, a);
-    a = fmaf(sb1(hi), x1.y, a);
-    a = fmaf(sb2(lo), x0.z, a);
-    a = fmaf(sb2(hi), x1.z, a);
-    a = fmaf(sb3(lo), x0.w, a);
-    return fmaf(sb3(hi), x1.w, a);
-}
-
-struct Iq4nlW {
-    static constexpr uint STEP = 16u;            // blocks a wave walks per step
-    static constexpr uint BYTES = IQ4NL_BYTES;
-    static __device__ __forceinline__ uint units(uint K) { return K >> 5; }
-    // lane -> (block of the step, float offset of its first x fragment inside the block)
-    static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 2; }
-    static __device__ __forceinline__ uint x_off(uint lane) { return (lane & 3u) * 4u; }
-    static __device__ __forceinline__ uint x_unit(uint) { return 32u; }
-    struct Frag { uint d16, q; };
-    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
-        const uchar* blk = row + (size_t)u * IQ4NL_BYTES;
-        Frag f;
-        f.d16 = *(const ushort*)blk;
-        f.q = *(const u32_a2*)(blk + 2u + (lane & 3u) * 4u);
-        return f;
-    }
-    static __device__ __forceinline__ float dot(const Frag& f, uint, float4 x0, float4 x1, float) {
-        return f16_bits_to_f32(f.d16) * iq4_lane_dot(f.q, x0, x1);
-    }
-};
-
-struct Iq4xsW {
-    static constexpr uint STEP = 2u;             // super-blocks per step
-    static constexpr uint BYTES = IQ4XS_BYTES;
-    static __device__ __forceinline__ uint units(uint K) { return K >> 8; }
-    static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 5; }
-    static __device__ __forceinline__ uint x_off(uint lane) { return ((lane & 31u) >> 2) * 32u + (lane & 3u) * 4u; }
-    static __device__ __forceinline__ uint x_unit(uint) { return 256u; }
-    struct Frag { uint h0, sl, q; };
-    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
-        const uint* blk = (const uint*)(row + (size_t)u * IQ4XS_BYTES);
-        Frag f;
-        f.h0 = blk[0];
-        f.sl = blk[1];
-        f.q = blk[2u + (lane & 31u)];
-        return f;
-    }
-    static __device__ __forceinline__ float dot(const Frag& f, uint lane, float4 x0, float4 x1, float) {
-        const uint ib = (lane & 31u) >> 2;
-        const uint ls = ((f.sl >> (4u * ib)) & 0xFu) | ((((f.h0 >> 16) >> (2u * ib)) & 3u) << 4);
-        return f16_bits_to_f32(f.h0 & 0xFFFFu) * (float)((int)ls - 32) * iq4_lane_dot(f.q, x0, x1);
-    }
-};
-
-// The legacy 32-weight blocks Q4_0 / Q4_1 / Q5_0 / Q5_1 share IQ4_NL's layout — a header, then 16 bytes whose
-// low nibbles are weights 0..15 and high nibbles 16..31 — with a linear code instead of the table:
-// w = d (q - 8), d q + m, d (q5 - 16), d q5 + m, the fifth bit of weight j being bit j of a 4-byte field.
-// Four lanes per block; codes stay unsigned (v_cvt_f32_ubyteN) and the offset or minimum meets the sum of the
-// lane's eight activations once per block:  d * (sum q x - off * sum x)  or  d * sum q x + m * sum x.
-template <bool FIVE, bool AFFINE>
-struct LegacyW {
-    static constexpr uint STEP = 16u;
-    static constexpr uint BYTES = 18u + (AFFINE ? 2u : 0u) + (FIVE ? 4u : 0u);
-    static constexpr uint HDR = AFFINE ? 4u : 2u;
-    static __device__ __forceinline__ uint units(uint K) { return K >> 5; }
-    static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 2; }
-    static __device__ __forceinline__ uint x_off(uint lane) { return (lane & 3u) * 4u; }
-    static __device__ __forceinline__ uint x_unit(uint) { return 32u; }
-    struct Frag { uint hdr, q, qh; };
-    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
-        const uchar* blk = row + (size_t)u * BYTES;
-        Frag f;
-        f.hdr = AFFINE ? *(const u32_a2*)blk : (uint)*(const ushort*)blk;
-        f.qh = FIVE ? *(const u32_a2*)(blk + HDR) : 0u;
-        f.q = *(const u32_a2*)(blk + HDR + (FIVE ? 4u : 0u) + (lane & 3u) * 4u);
-        return f;
-    }
-    // bits b .. b + 3 of `v` -> bit 4 of bytes 0 .. 3
-    static __device__ __forceinline__ uint spread4(uint v, uint b) {
-        const uint n = (v >> b) & 0xFu;
-        return ((n & 1u) << 4) | ((n & 2u) << 11) | ((n & 4u) << 18) | ((n & 8u) << 25);
-    }
-    static __device__ __forceinline__ float dot(const Frag& f, uint lane, float4 x0, float4 x1, float xsum) {
-        uint lo = f.q & 0x0F0F0F0Fu, hi = (f.q >> 4) & 0x0F0F0F0Fu;
-        if (FIVE) {
-            const uint p4 = (lane & 3u) * 4u;
-            lo |= spread4(f.qh, p4);
-            hi |= spread4(f.qh, p4 + 16u);
-        }
-        const float a = dot4_ub(hi, x1, dot4_ub(lo, x0, 0.0f));
-        const float d = f16_bits_to_f32(f.hdr & 0xFFFFu);
-        if (AFFINE) return d * a + f16_bits_to_f32(f.hdr >> 16) * xsum;
-        return d * (a - (FIVE ? 16.0f : 8.0f) * xsum);
-    }
-};
-typedef LegacyW<false, false> Q40W;
-typedef LegacyW<false, true> Q41W;
-typedef LegacyW<true, false> Q50W;
-typedef LegacyW<true, true> Q51W;
-
+// ------------------------------------------------------------------ IQ4_NL, IQ4_XS and the legacy 32-weight blocks
+// (row traits Iq4nlW, Iq4xsW, Q40W, Q41W, Q50W, Q51W: ojk_rows.h)
 template <class W, int R, int MODE>
 __device__ __forceinline__ void gemv_nat_iq4_body(const float* __restrict__ x, const uchar* __restrict__ w,
                                                   float* __restrict__ y, const float* __restrict__ bs,

@@ -690,7 +690,8 @@ uint64_t ojh_moe_mt_lds(uint32_t K) { return 16 * ((uint64_t)K + 32) + K / 4 + K
 //   8 moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)                      grid [ceil(N/8), NA, 1]
 //   9 moe_down_q4k_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)                  grid [ceil(N/8), T, 1]
 //  14 moe_gu_q80(x, wg, wu, act, idx, K, N)                                     grid [ceil(N/8), KSEL, tokens]
-//  15 moe_down_q80(act, wd, y, idx, wgt, K, N, KSEL)                            grid [1 .. ceil(N/16), tokens, 1]
+//  15 moe_down_q80(act, wd, y, idx, wgt, K, N, KSEL)                            grid [1 .. ceil(N/8), tokens, 1]
+//  14 / 15 also moe_{gu,down}_{iq4xs,iq4nl} of family "moe_iq", the same arguments
 //     (the reference's Q8_0 expert kernels; the expert count is not an argument, so the weight buffers are
 //     checked for one expert only)
 //  10 moe_gu_q4k_slots, 11 moe_down_q4k_slots: 8 and 9 with a u64 byte offset per assignment into an arena
@@ -792,30 +793,32 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         align[0] = align[1] = 16;
         return OJH_OK;
     }
-    case 14: {  // moe_gu_q80(x, wg, wu, act, idx, K, N)
+    case 14: {  // moe_gu_{q80,iq4xs,iq4nl}(x, wg, wu, act, idx, K, N)
         uint32_t K = c[0], N = c[1], KS = grid[1], T = grid[2];
+        const ojh_block_format *f = ojh_format(s->type);
         if ((rc = check_block(block, 256))) return rc;
-        if (!K || K % 32 || !N || !KS || !T) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u slots=%u tokens=%u", s->name, K, N, KS, T);
+        if (!K || K % f->weights || !N || !KS || !T) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u slots=%u tokens=%u", s->name, K, N, KS, T);
         if (grid[0] != (N + 7) / 8) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/8), slots, tokens]", s->name);
         need[0] = (size_t)T * K * 4;
-        need[1] = need[2] = (size_t)N * (K / 32) * 34;
+        need[1] = need[2] = (size_t)N * (K / f->weights) * f->bytes;
         need[3] = (size_t)T * KS * N * 4;
         need[4] = (size_t)T * KS * 4;
         align[0] = 16;
-        align[1] = align[2] = 2;
+        align[1] = align[2] = ojh_block_align(f);
         return OJH_OK;
     }
-    case 15: {  // moe_down_q80(act, wd, y, idx, wgt, K, N, KSEL)
+    case 15: {  // moe_down_{q80,iq4xs,iq4nl}(act, wd, y, idx, wgt, K, N, KSEL): rows grid-stride, 16 per workgroup
         uint32_t K = c[0], N = c[1], KS = c[2], T = grid[1];
+        const ojh_block_format *f = ojh_format(s->type);
         if ((rc = check_block(block, 256))) return rc;
-        if (!K || K % 32 || !N || !KS || !T) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u KSEL=%u tokens=%u", s->name, K, N, KS, T);
-        if (!grid[0] || grid[0] > (N + 15) / 16 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N/16), tokens, 1]", s->name);
+        if (!K || K % f->weights || !N || !KS || !T) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u KSEL=%u tokens=%u", s->name, K, N, KS, T);
+        if (!grid[0] || grid[0] > (N + 7) / 8 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N/8), tokens, 1]", s->name);
         need[0] = (size_t)T * KS * K * 4;
-        need[1] = (size_t)N * (K / 32) * 34;
+        need[1] = (size_t)N * (K / f->weights) * f->bytes;
         need[2] = (size_t)T * N * 4;
         need[3] = need[4] = (size_t)T * KS * 4;
         align[0] = 16;
-        align[1] = 2;
+        align[1] = ojh_block_align(f);
         return OJH_OK;
     }
     case 10: {  // moe_gu_q4k_slots(x, arena_g, arena_u, act, off_g, off_u, K, N, KSEL, NA, LIM_G, LIM_U)
@@ -1107,6 +1110,14 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     m.back().expert_bufs = 2;
     add("moe_down_q80", "moe", 5, 3, OJH_Q8_0, 15, check_moe, shape_moe);
     m.back().expert_bufs = 1;
+    // the reference keeps the IQ expert kernels in a family of their own (crates/ojas-cuda/src/kernels/mod.rs:111-145)
+    for (uint32_t ty : {(uint32_t)OJH_IQ4_XS, (uint32_t)OJH_IQ4_NL}) {
+        std::string tag = ojh_format(ty)->tag;
+        add("moe_gu_" + tag, "moe_iq", 5, 2, ty, 14, check_moe, shape_moe);
+        m.back().expert_bufs = 2;
+        add("moe_down_" + tag, "moe_iq", 5, 3, ty, 15, check_moe, shape_moe);
+        m.back().expert_bufs = 1;
+    }
     add("moe_down_q6k_m", "moe", 6, 3, OJH_Q6_K, 4, check_moe, shape_moe);
     add("moe_down_q6k_dec", "moe", 5, 5, OJH_Q6_K, 9, check_moe, shape_moe);
     add("copy_bf16_half", "glue", 2, 1, (2u << 8) | 2u, 0, check_elementwise, shape_elementwise);

@@ -37,13 +37,19 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     if (!dev || !gate || !up || !down) return ojh_fail(OJH_ERR_ARG, "ojh_moe_ffn: NULL argument");
     if (!T || !E || E > 1024 || !ksel || ksel > E || T > 65535u / ksel)
         return ojh_fail(OJH_ERR_ARG, "moe_ffn: tokens=%u experts=%u ksel=%u out of range", T, E, ksel);
-    // Q8_0 experts: the reference's own expert kernels, f32 activations (dot_q80), one launch for gate/up and one
-    // for down over all tokens; the down launch accumulates onto y, so a plain store starts from zeros
-    if (gate->type == OJH_Q8_0 && up->type == OJH_Q8_0 && down->type == OJH_Q8_0) {
+    // Experts in a format whose rows meet f32 activations (Q8_0, IQ4_XS, IQ4_NL; gate and up alike, down
+    // any of the three): the reference's own expert kernels moe_gu_<fmt> / moe_down_<fmt>, one launch for
+    // gate/up and one for down over all tokens; the down launch accumulates onto y, so a plain store
+    // starts from zeros
+    auto float_expert = [](uint32_t t) { return t == OJH_Q8_0 || t == OJH_IQ4_XS || t == OJH_IQ4_NL; };
+    if (gate->type == up->type && float_expert(gate->type) && float_expert(down->type)) {
         if (act_mode == OJH_ACT_Q8K)
-            return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: Q8_0 experts take f32 activations, as dot_q80 does");
+            return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: %s / %s experts take f32 activations, as their CPU dots do",
+                            ojh_format(gate->type)->tag, ojh_format(down->type)->tag);
         int rc;
-        if (d % 32 || n_ff % 32) return ojh_fail(OJH_ERR_ARG, "moe_ffn: d=%u and n_ff=%u must be multiples of 32", d, n_ff);
+        const ojh_block_format *fg = ojh_format(gate->type), *fd = ojh_format(down->type);
+        if (d % fg->weights || n_ff % fd->weights || d % 32 || n_ff % 32)
+            return ojh_fail(OJH_ERR_ARG, "moe_ffn: d=%u and n_ff=%u must be whole blocks of the expert formats", d, n_ff);
         if (gate->k != d || up->k != d || down->k != n_ff || (uint64_t)gate->n != (uint64_t)E * n_ff ||
             (uint64_t)up->n != (uint64_t)E * n_ff || (uint64_t)down->n != (uint64_t)E * d)
             return ojh_fail(OJH_ERR_ARG, "moe_ffn: expert tensor shapes do not match E=%u d=%u n_ff=%u", E, d, n_ff);
@@ -52,7 +58,9 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         if ((rc = span("moe_ffn: idx", idx, (size_t)NA8 * 4, 4))) return rc;
         if ((rc = span("moe_ffn: wgt", wgt, (size_t)NA8 * 4, 4))) return rc;
         if ((rc = span("moe_ffn: y", y, (size_t)T * d * 4, 4))) return rc;
-        if ((rc = ensure(dev, "moe"))) return rc;
+        const std::string gu_name = std::string("moe_gu_") + fg->tag, down_name = std::string("moe_down_") + fd->tag;
+        if ((rc = ensure(dev, gate->type == OJH_Q8_0 ? "moe" : "moe_iq"))) return rc;
+        if ((rc = ensure(dev, down->type == OJH_Q8_0 ? "moe" : "moe_iq"))) return rc;
         ojh_buf *act8;
         if ((rc = ojh_scratch_get(dev, "moe_act", (size_t)NA8 * n_ff * 4, &act8))) return rc;
         uint32_t b256[3] = {256, 1, 1};
@@ -62,15 +70,15 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
             if ((rc = ojh_launch(dev, "fill_zero_u32", {y->ptr}, {n_y}, zg, b256))) return rc;
         }
         uint32_t g1[3] = {(n_ff + 7) / 8, ksel, T};
-        if ((rc = ojh_launch(dev, "moe_gu_q80", {x->ptr, (char *)gate->raw->ptr + gate->off, (char *)up->raw->ptr + up->off, act8->ptr, idx->ptr},
+        if ((rc = ojh_launch(dev, gu_name.c_str(), {x->ptr, (char *)gate->raw->ptr + gate->off, (char *)up->raw->ptr + up->off, act8->ptr, idx->ptr},
                              {d, n_ff, E}, g1, b256)))
             return rc;
         uint32_t g2[3] = {(d + 15) / 16, T, 1};
-        return ojh_launch(dev, "moe_down_q80", {act8->ptr, (char *)down->raw->ptr + down->off, y->ptr, idx->ptr, wgt->ptr},
+        return ojh_launch(dev, down_name.c_str(), {act8->ptr, (char *)down->raw->ptr + down->off, y->ptr, idx->ptr, wgt->ptr},
                           {n_ff, d, ksel, E}, g2, b256);
     }
     if (gate->type != OJH_Q4_K || up->type != OJH_Q4_K || (down->type != OJH_Q4_K && down->type != OJH_Q5_K && down->type != OJH_Q6_K))
-        return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: gate and up must be Q4_K with down Q4_K, Q5_K or Q6_K, or all three Q8_0 (gate %u, up %u, down %u)",
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: gate and up must be Q4_K with down Q4_K, Q5_K or Q6_K, or all three among Q8_0, IQ4_XS, IQ4_NL (gate %u, up %u, down %u)",
                         gate->type, up->type, down->type);
     if (act_mode == OJH_ACT_FLOAT)
         return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_moe_ffn: K-quant experts have the quantized-activation contract only (OJH_ACT_Q8K)");

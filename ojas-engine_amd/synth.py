@@ -261,6 +261,21 @@ def q80_rows_lcg(rows: int, k: int, seed: int) -> tuple[np.ndarray, np.ndarray]:
     return out.reshape(-1), plain
 
 
+def iq4_rows_lcg(ty: int, rows: int, k: int, seed: int) -> np.ndarray:
+    """IQ4_XS / IQ4_NL rows of the reference's GPU conformance test (crates/ojas-cuda/tests/conformance.rs:461-503):
+    byte i = trunc(255 |tvec(1, seed + i)|), then d of block (r, b) = f16(0.01 + 0.002 ((r + b) mod 7 | 5))."""
+    bb, wpb = BLOCK_SHAPE[ty]
+    nb = k // wpb
+    out = (np.abs(tvec_first(np.uint64(seed) + np.arange(rows * nb * bb, dtype=np.uint64))) * np.float32(255.0)).astype(np.uint8)
+    out = out.reshape(rows, nb, bb)
+    r, b = np.arange(rows)[:, None], np.arange(nb)[None, :]
+    d = (np.float32(0.01) + np.float32(0.002) * ((r + b) % (7 if ty == IQ4_XS else 5)).astype(np.float32)).astype(np.float16)
+    dv = d.view(np.uint16)
+    out[:, :, 0] = dv & 0xFF
+    out[:, :, 1] = dv >> 8
+    return out.reshape(-1)
+
+
 def q80_rows_closed_form(n: int, k: int):
     """Q8_0 rows and activations of the reference's `native_q8_matvec_ksplit_matches_cpu`:
     d = f16(0.003 + ((r+b) mod 7) * 0.001), q = ((17r + 11b + 5j) mod 31) - 15,

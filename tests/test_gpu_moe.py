@@ -15,6 +15,7 @@ from conftest import peak_err
 pytestmark = pytest.mark.gpu
 Q4_K = 12
 Q8_0 = 8
+IQ4_NL, IQ4_XS = 20, 23
 TOL = 1e-3
 TOL_SEEN = 3e-4
 
@@ -336,6 +337,68 @@ def test_q80_experts_through_the_ffn_entry(gpu, orc, pkg, T, E, ksel, d, nff, ac
         got = gpu.read(yd, T * d + d)
         assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
         assert peak_err(got[:T * d].reshape(T, d) - y0, want - y0) <= 2e-5
+    with pytest.raises(pkg.OjasHipError, match="f32 activations"):
+        gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, act_mode=pkg.ACT_Q8K)
+
+
+def test_iq4_experts_reference_procedure(gpu, orc, pkg):
+    """IQ4_XS gate/up and IQ4_NL down through `moe_gu_iq4xs` / `moe_down_iq4nl` of family "moe_iq" with the
+    reference's arguments and launch geometry (crates/ojas-cuda/tests/conformance.rs:505-560): E=8, K=512,
+    N=256, experts {1, 5} weighted {0.6, 0.4}, against the products of the values `dequant_to_f16` decodes,
+    largest deviation over the peak below 5e-3 as there (the f16 rounding of the decoded weights is most of it)."""
+    k, n, experts, ksel = 512, 256, 8, 2
+    x = pkg.synth.tvec(k, 71)
+    gbytes = pkg.synth.iq4_rows_lcg(IQ4_XS, experts * n, k, 72)
+    ubytes = pkg.synth.iq4_rows_lcg(IQ4_XS, experts * n, k, 73)
+    dbytes = pkg.synth.iq4_rows_lcg(IQ4_NL, experts * k, n, 74)
+    plain = lambda b, ty, rows, cols: orc.dequant_to_f16(b, ty, rows * cols).view(np.float16).astype(np.float64).reshape(rows, cols)
+    gplain, uplain, dplain = plain(gbytes, IQ4_XS, experts * n, k), plain(ubytes, IQ4_XS, experts * n, k), plain(dbytes, IQ4_NL, experts * k, n)
+    idx, wgt = np.array([1, 5], np.uint32), np.array([0.6, 0.4], np.float32)
+    want = np.zeros(k, np.float64)
+    silu = lambda v: v / (1.0 + np.exp(np.minimum(-v, 700.0)))      # random sub-scales make some gates very negative
+    for j, e in enumerate(idx):
+        gv, uv = gplain[e * n:(e + 1) * n] @ x.astype(np.float64), uplain[e * n:(e + 1) * n] @ x.astype(np.float64)
+        want += float(wgt[j]) * (dplain[e * k:(e + 1) * k] @ (silu(gv) * uv))
+    gpu.ensure_family("moe_iq")
+    xd, gd, ud, dd = gpu.upload(x), gpu.upload_bytes(gbytes), gpu.upload_bytes(ubytes), gpu.upload_bytes(dbytes)
+    idxd, wgtd = gpu.upload_bytes(idx), gpu.upload(wgt)
+    actd, outd = gpu.alloc(ksel * n), gpu.upload(np.zeros(k, np.float32))
+    enc = gpu.begin()
+    gpu.dispatch(enc, "moe_gu_iq4xs", [(xd, 0), (gd, 0), (ud, 0), (actd, 0), (idxd, 0)], [k, n], [-(-n // 8), ksel, 1], [256, 1, 1])
+    gpu.dispatch(enc, "moe_down_iq4nl", [(actd, 0), (dd, 0), (outd, 0), (idxd, 0), (wgtd, 0)], [n, k, ksel], [-(-k // 8), 1, 1], [256, 1, 1])
+    gpu.submit(enc)
+    got = gpu.read(outd, k)
+    assert peak_err(got, want) < 5e-3
+    # against the exact values of the same blocks the kernels are much closer
+    exact = lambda b, ty, rows, cols: orc.dequant_to_f64(b, ty, rows * cols).reshape(rows, cols)
+    ge, ue, de = exact(gbytes, IQ4_XS, experts * n, k), exact(ubytes, IQ4_XS, experts * n, k), exact(dbytes, IQ4_NL, experts * k, n)
+    want2 = np.zeros(k, np.float64)
+    for j, e in enumerate(idx):
+        gv, uv = ge[e * n:(e + 1) * n] @ x.astype(np.float64), ue[e * n:(e + 1) * n] @ x.astype(np.float64)
+        want2 += float(wgt[j]) * (de[e * k:(e + 1) * k] @ (silu(gv) * uv))
+    assert peak_err(got, want2) <= 1e-5
+
+
+@pytest.mark.parametrize("tg,td", [(IQ4_XS, IQ4_NL), (IQ4_NL, IQ4_XS), (IQ4_XS, Q8_0), (Q8_0, IQ4_NL)])
+@pytest.mark.parametrize("T,E,ksel,d,nff,accum", [(1, 8, 2, 256, 256, False), (6, 16, 4, 512, 768, True), (33, 4, 3, 1024, 256, False)])
+def test_iq4_experts_through_the_ffn_entry(gpu, orc, pkg, tg, td, T, E, ksel, d, nff, accum):
+    """Any mix of the f32-activation expert formats under `ojh_moe_ffn`, against the CPU path's dots
+    (dot_iq4xs / dot_iq4nl / dot_q80 under crates/ojas-cpu/src/cpu_glm.rs:551-582)."""
+    gate = pkg.synth.weights(tg, E * nff, d, "moeiq", "gate", tg, E, d, nff)
+    up = pkg.synth.weights(tg, E * nff, d, "moeiq", "up", tg, E, d, nff)
+    down = pkg.synth.weights(td, E * d, nff, "moeiq", "down", td, E, d, nff)
+    x = pkg.synth.normal_f32(T * d, "moeiq", "x", T, d).reshape(T, d)
+    lg = pkg.synth.normal_f32(T * E, "moeiq", "lg", T, E).reshape(T, E)
+    gi, gw, idx_d, wgt_d = _route(gpu, lg, ksel)
+    want0 = orc.moe_ffn(x, gi, gw, gate, up, tg, down, td, E, nff, mode=0)
+    peak = float(np.max(np.abs(want0)))
+    y0 = np.float32(peak) * pkg.synth.normal_f32(T * d, "moeiq", "y0").reshape(T, d) if accum else np.zeros((T, d), np.float32)
+    yd = gpu.upload(np.concatenate([y0.ravel() if accum else np.full(T * d, 777.0, np.float32), np.full(d, 12345.5, np.float32)]))
+    lg_, lu_, ld_ = gpu.lin(tg, E * nff, d, gate), gpu.lin(tg, E * nff, d, up), gpu.lin(td, E * d, nff, down)
+    gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, accum=accum)
+    got = gpu.read(yd, T * d + d)
+    assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
+    assert peak_err(got[:T * d].reshape(T, d) - y0, want0) <= 2e-5
     with pytest.raises(pkg.OjasHipError, match="f32 activations"):
         gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, act_mode=pkg.ACT_Q8K)
 
