@@ -496,8 +496,8 @@ moe_down_q6k_dec(const float* act, const uchar* wd, const uint* idx, const float
 
 // ------------------------------------------------------------------ Q8_0 experts, f32 activations
 //   moe_gu_q80(x, wg, wu, act, idx, K, N)              grid [ceil(N/8), KSEL, tokens], block 256
-//   moe_down_q80(act, wd, y, idx, wgt, K, N, KSEL)     grid [1 .. ceil(N/16), tokens, 1], block 256 (rows grid-stride,
-//                                                      so the reference's ceil(N/32) workgroups are a valid grid)
+//   moe_down_q80(act, wd, y, idx, wgt, K, N, KSEL)     grid [1 .. ceil(N/8), tokens, 1], block 256 (rows grid-stride,
+//                                                      16 per workgroup and step: the reference's ceil(N/32) is a valid grid)
 // The reference's expert kernels by their own names and arguments
 // (crates/ojas-cuda/src/kernels/moe.rs:75-125): act[j][n] = silu(gate_e . x) * (up_e . x) for the expert
 // e = idx[j] of slot j, and y[n] += sum_j wgt[j] * (down_e . act[j]) — the down launch accumulates onto
@@ -520,60 +520,105 @@ __device__ __forceinline__ float q80f_block_part(const uchar* blk, uint p, float
     return f16_bits_to_f32(*(const ushort*)blk) * a;
 }
 
-extern "C" __global__ void __launch_bounds__(256)
-moe_gu_q80(const float* __restrict__ x, const uchar* __restrict__ wg, const uchar* __restrict__ wu,
-           float* __restrict__ act, const uint* __restrict__ idx, uint K, uint N, uint E) {
+// gate/up rows of one expert (eg, eu: its first rows) against token row xt; nb = 0 skips the products
+__device__ __forceinline__ void moe_gu_q80_body(const float* __restrict__ xt, const uchar* __restrict__ eg,
+                                                const uchar* __restrict__ eu, float* __restrict__ act_row,
+                                                uint K, uint N, uint nb) {
     const uint lane = threadIdx.x & 63u, g = lane >> 2, p = lane & 3u;
-    const uint j = blockIdx.y, t = blockIdx.z, ksel = gridDim.y;
     const uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 2u;
     if (row0 >= N) return;
-    const uint e = idx[t * ksel + j], nb = e < E ? K >> 5 : 0u;
     const size_t rb = (size_t)(K >> 5) * Q80_BYTES;
-    const float* xt = x + (size_t)t * K;
     float ag[2] = {0.0f, 0.0f}, au[2] = {0.0f, 0.0f};
     for (uint b = g; b < nb; b += 16u) {
         const float4* xp = (const float4*)(xt + (size_t)b * 32u + p * 8u);
         const float4 x0 = xp[0], x1 = xp[1];
 #pragma unroll
         for (int r = 0; r < 2; r++) {
-            const size_t off = ((size_t)e * N + min(row0 + (uint)r, N - 1u)) * rb + (size_t)b * Q80_BYTES;
-            ag[r] += q80f_block_part(wg + off, p, x0, x1);
-            au[r] += q80f_block_part(wu + off, p, x0, x1);
+            const size_t off = (size_t)min(row0 + (uint)r, N - 1u) * rb + (size_t)b * Q80_BYTES;
+            ag[r] += q80f_block_part(eg + off, p, x0, x1);
+            au[r] += q80f_block_part(eu + off, p, x0, x1);
         }
     }
 #pragma unroll
     for (int r = 0; r < 2; r++) {
         const float gs = wave_sum(ag[r]), us = wave_sum(au[r]);
-        if (lane == 0 && row0 + r < N) act[((size_t)t * ksel + j) * N + row0 + r] = (gs / (1.0f + expf(-gs))) * us;
+        if (lane == 0 && row0 + r < N) act_row[row0 + r] = (gs / (1.0f + expf(-gs))) * us;
     }
+}
+
+// four down rows of one expert (ed: its first row) against one activation row
+__device__ __forceinline__ void moe_down_q80_part(const float* __restrict__ xr, const uchar* __restrict__ ed,
+                                                  uint K, uint N, uint row0, float wj, float (&res)[4]) {
+    const uint lane = threadIdx.x & 63u, g = lane >> 2, p = lane & 3u;
+    const uint nb = K >> 5;
+    const size_t rb = (size_t)nb * Q80_BYTES;
+    float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint b = g; b < nb; b += 16u) {
+        const float4* xp = (const float4*)(xr + (size_t)b * 32u + p * 8u);
+        const float4 x0 = xp[0], x1 = xp[1];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            a[r] += q80f_block_part(ed + (size_t)min(row0 + (uint)r, N - 1u) * rb + (size_t)b * Q80_BYTES, p, x0, x1);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++) res[r] += wj * wave_sum(a[r]);
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+moe_gu_q80(const float* __restrict__ x, const uchar* __restrict__ wg, const uchar* __restrict__ wu,
+           float* __restrict__ act, const uint* __restrict__ idx, uint K, uint N, uint E) {
+    const uint j = blockIdx.y, t = blockIdx.z, ksel = gridDim.y;
+    const uint e = idx[t * ksel + j];
+    const size_t eb = (size_t)(e < E ? e : 0u) * N * ((size_t)(K >> 5) * Q80_BYTES);
+    moe_gu_q80_body(x + (size_t)t * K, wg + eb, wu + eb, act + ((size_t)t * ksel + j) * N, K, N, e < E ? K >> 5 : 0u);
 }
 
 extern "C" __global__ void __launch_bounds__(256)
 moe_down_q80(const float* __restrict__ act, const uchar* __restrict__ wd, float* __restrict__ y,
              const uint* __restrict__ idx, const float* __restrict__ wgt, uint K, uint N, uint KSEL, uint E) {
-    const uint lane = threadIdx.x & 63u, g = lane >> 2, p = lane & 3u;
     const uint t = blockIdx.y;
-    const uint nb = K >> 5;
-    const size_t rb = (size_t)nb * Q80_BYTES;
+    const size_t eb = (size_t)N * ((size_t)(K >> 5) * Q80_BYTES);
     for (uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 4u; row0 < N; row0 += gridDim.x * 16u) {
         float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         for (uint j = 0; j < KSEL; j++) {
             const uint e = idx[t * KSEL + j];
             if (e >= E) continue;
-            const float wj = wgt[t * KSEL + j];
-            const float* xr = act + ((size_t)t * KSEL + j) * K;
-            float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            for (uint b = g; b < nb; b += 16u) {
-                const float4* xp = (const float4*)(xr + (size_t)b * 32u + p * 8u);
-                const float4 x0 = xp[0], x1 = xp[1];
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    a[r] += q80f_block_part(wd + ((size_t)e * N + min(row0 + (uint)r, N - 1u)) * rb + (size_t)b * Q80_BYTES, p, x0, x1);
-            }
-#pragma unroll
-            for (int r = 0; r < 4; r++) res[r] += wj * wave_sum(a[r]);
+            moe_down_q80_part(act + ((size_t)t * KSEL + j) * K, wd + (size_t)e * eb, K, N, row0, wgt[t * KSEL + j], res);
         }
-        if (lane == 0) {
+        if ((threadIdx.x & 63u) == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (row0 + r < N) y[(size_t)t * N + row0 + r] += res[r];
+        }
+    }
+}
+
+// Streamed Q8_0 experts (crates/ojas-cuda/src/kernels/moe.rs:133-174): the experts of a layer sit at whatever
+// slots of a cache arena were free, and the host passes one u32 byte offset per selected expert in place of
+// the index.   moe_gu_q80_slots(x, arena_g, arena_u, act, off_g, off_u, K, N)   grid [ceil(N/8), KSEL, tokens]
+//              moe_down_q80_slots(act, arena, y, off_d, wgt, K, N, KSEL)          grid [1 .. ceil(N/8), tokens, 1]
+// The trailing LIM constants are appended by the dispatcher — the last offset at which a whole expert still
+// fits its arena — and an offset is rounded down to the blocks' two-byte alignment and clamped to LIM, so a bad
+// table reads a wrong expert, never past the arena.
+extern "C" __global__ void __launch_bounds__(256)
+moe_gu_q80_slots(const float* __restrict__ x, const uchar* __restrict__ arena_g, const uchar* __restrict__ arena_u,
+                 float* __restrict__ act, const uint* __restrict__ off_g, const uint* __restrict__ off_u,
+                 uint K, uint N, uint LIM_G, uint LIM_U) {
+    const uint j = blockIdx.y, t = blockIdx.z, ksel = gridDim.y;
+    const uint og = min(off_g[t * ksel + j] & ~1u, LIM_G), ou = min(off_u[t * ksel + j] & ~1u, LIM_U);
+    moe_gu_q80_body(x + (size_t)t * K, arena_g + og, arena_u + ou, act + ((size_t)t * ksel + j) * N, K, N, K >> 5);
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+moe_down_q80_slots(const float* __restrict__ act, const uchar* __restrict__ arena, float* __restrict__ y,
+                   const uint* __restrict__ off_d, const float* __restrict__ wgt, uint K, uint N, uint KSEL, uint LIM) {
+    const uint t = blockIdx.y;
+    for (uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 4u; row0 < N; row0 += gridDim.x * 16u) {
+        float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (uint j = 0; j < KSEL; j++)
+            moe_down_q80_part(act + ((size_t)t * KSEL + j) * K, arena + min(off_d[t * KSEL + j] & ~1u, LIM), K, N, row0,
+                              wgt[t * KSEL + j], res);
+        if ((threadIdx.x & 63u) == 0) {
 #pragma unroll
             for (int r = 0; r < 4; r++)
                 if (row0 + r < N) y[(size_t)t * N + row0 + r] += res[r];

@@ -345,6 +345,10 @@ extern "C" int ojh_dispatch(ojh_device *dev, const char *name, int n_bufs, ojh_b
         }
         cv.push_back((uint32_t)experts);
     }
+    for (int i = 1; i <= s->arena_bufs; i++) {   // the kernels clamp their u32 offsets to this
+        size_t off = offsets ? (size_t)offsets[i] : 0;
+        cv.push_back((uint32_t)std::min<size_t>(bufs[i]->bytes - off - need[i], 0xFFFFFFFEu));
+    }
     return ojh_launch(dev, name, ptrs, cv, grid, block);
 }
 

@@ -341,6 +341,50 @@ def test_q80_experts_through_the_ffn_entry(gpu, orc, pkg, T, E, ksel, d, nff, ac
         gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, act_mode=pkg.ACT_Q8K)
 
 
+@pytest.mark.parametrize("T,E,ksel,k,n", [(1, 8, 2, 256, 64), (3, 6, 4, 512, 224)])
+def test_q80_streamed_experts_by_byte_offsets(gpu, pkg, T, E, ksel, k, n):
+    """`moe_gu_q80_slots` / `moe_down_q80_slots` (crates/ojas-cuda/src/kernels/moe.rs:133-174): experts at shuffled
+    slots of an arena, one u32 byte offset per selected expert — the same bits as the index-addressed kernels
+    on the same experts; an offset past the arena is clamped, never read."""
+    gate = pkg.synth.q80_weights(E * n, k, "slots8", "gate", E, k, n)
+    up = pkg.synth.q80_weights(E * n, k, "slots8", "up", E, k, n)
+    down = pkg.synth.q80_weights(E * k, n, "slots8", "down", E, k, n)
+    x = pkg.synth.normal_f32(T * k, "slots8", "x", T, k)
+    g = pkg.synth.rng("slots8", T, E)
+    idx = np.stack([g.permutation(E)[:ksel] for _ in range(T)]).astype(np.uint32)
+    wgt = g.random((T, ksel)).astype(np.float32)
+    gpu.ensure_family("moe")
+    xd, idxd, wgtd = gpu.upload(x), gpu.upload_bytes(idx), gpu.upload(wgt)
+    act1, y1 = gpu.alloc(T * ksel * n), gpu.upload(np.ones(T * k, np.float32))
+    gd, ud, dd = gpu.upload_bytes(gate), gpu.upload_bytes(up), gpu.upload_bytes(down)
+    gpu.dispatch(gpu.begin(), "moe_gu_q80", [(xd, 0), (gd, 0), (ud, 0), (act1, 0), (idxd, 0)], [k, n], [-(-n // 8), ksel, T], [256, 1, 1])
+    gpu.dispatch(gpu.begin(), "moe_down_q80", [(act1, 0), (dd, 0), (y1, 0), (idxd, 0), (wgtd, 0)], [n, k, ksel], [-(-k // 16), T, 1], [256, 1, 1])
+    # arenas: the experts in a shuffled order behind 70 bytes of padding (block alignment is two bytes)
+    eb_gu, eb_d, pad = n * (k // 32) * 34, k * (n // 32) * 34, 70
+    perm = g.permutation(E)
+    slot_of = np.empty(E, np.int64)
+    slot_of[perm] = np.arange(E)
+    arena = lambda w, eb: np.concatenate([np.full(pad, 0xEE, np.uint8), w.reshape(E, eb)[perm].reshape(-1)])
+    ag, au, ad = gpu.upload_bytes(arena(gate, eb_gu)), gpu.upload_bytes(arena(up, eb_gu)), gpu.upload_bytes(arena(down, eb_d))
+    og = (pad + slot_of[idx] * eb_gu).astype(np.uint32)
+    od = (pad + slot_of[idx] * eb_d).astype(np.uint32)
+    act2, y2 = gpu.alloc(T * ksel * n), gpu.upload(np.ones(T * k, np.float32))
+    ogd, odd = gpu.upload_bytes(og), gpu.upload_bytes(od)
+    gpu.dispatch(gpu.begin(), "moe_gu_q80_slots", [(xd, 0), (ag, 0), (au, 0), (act2, 0), (ogd, 0), (ogd, 0)], [k, n], [-(-n // 8), ksel, T], [256, 1, 1])
+    gpu.dispatch(gpu.begin(), "moe_down_q80_slots", [(act2, 0), (ad, 0), (y2, 0), (odd, 0), (wgtd, 0)], [n, k, ksel], [-(-k // 8), T, 1], [256, 1, 1])
+    assert np.array_equal(gpu.read(act1, T * ksel * n), gpu.read(act2, T * ksel * n))
+    assert np.array_equal(gpu.read(y1, T * k), gpu.read(y2, T * k))
+    # offsets far past the arena: clamped to the last whole expert, finite output, no fault
+    wild = gpu.upload_bytes(np.full((T, ksel), 0xFFFFFFF0, np.uint32))
+    y3 = gpu.upload(np.zeros(T * k, np.float32))
+    gpu.dispatch(gpu.begin(), "moe_gu_q80_slots", [(xd, 0), (ag, 0), (au, 0), (act2, 0), (wild, 0), (wild, 0)], [k, n], [-(-n // 8), ksel, T], [256, 1, 1])
+    gpu.dispatch(gpu.begin(), "moe_down_q80_slots", [(act2, 0), (ad, 0), (y3, 0), (wild, 0), (wgtd, 0)], [n, k, ksel], [-(-k // 8), T, 1], [256, 1, 1])
+    assert np.all(np.isfinite(gpu.read(y3, T * k)))
+    with pytest.raises(pkg.OjasHipError, match="needs"):
+        gpu.dispatch(gpu.begin(), "moe_down_q80_slots", [(act2, 0), (ad, pad + (E - 1) * eb_d + 2), (y3, 0), (odd, 0), (wgtd, 0)],
+                     [n, k, ksel], [-(-k // 8), T, 1], [256, 1, 1])
+
+
 def test_iq4_experts_reference_procedure(gpu, orc, pkg):
     """IQ4_XS gate/up and IQ4_NL down through `moe_gu_iq4xs` / `moe_down_iq4nl` of family "moe_iq" with the
     reference's arguments and launch geometry (crates/ojas-cuda/tests/conformance.rs:505-560): E=8, K=512,
