@@ -79,6 +79,7 @@ typedef struct ojh_device ojh_device; /* one GPU + one stream + loaded families 
 typedef struct ojh_buf ojh_buf;       /* device allocation with a known size */
 typedef struct ojh_lin ojh_lin;       /* a weight matrix W[N,K] in its GGUF block bytes */
 typedef struct ojh_graph ojh_graph;   /* a recorded chain of dispatches, replayable */
+typedef struct ojh_expert_cache ojh_expert_cache; /* device arena of expert slots, LRU */
 
 /* Mirrors `Caps` (crates/ojas-core/src/kernel.rs:26-41). */
 typedef struct ojh_caps {
@@ -279,6 +280,32 @@ int ojh_moe_ffn_slots(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint
                       uint32_t ksel, const ojh_buf *arena_gate, const ojh_buf *off_gate,
                       const ojh_buf *arena_up, const ojh_buf *off_up, const ojh_buf *arena_down,
                       const ojh_buf *off_down, const ojh_buf *wgt, ojh_buf *y, int accum);
+
+/* ---- resident expert cache ----------------------------------------------------------------------
+ * `ExpertCache` (crates/ojas-cuda/src/expert_cache.rs:34-152): a device arena of budget / expert_bytes
+ * (at least one) fixed-size slots.  `gather` makes every requested expert resident — hits are re-ticked,
+ * misses take a free slot or evict the least recently used one and are filled through `load`, which
+ * writes one expert's bytes into page-locked staging (where a caller does its pread from the model
+ * file) — and returns one byte offset into the arena per request, in the order asked: what
+ * ojh_moe_ffn_slots and the `_slots` kernels take.  More distinct experts in one call than the arena
+ * has slots is refused (OJH_ERR_BOUNDS), not absorbed.  Copies are queued on the device's stream: work
+ * queued afterwards sees them, work queued before has finished with the slot.  Two staging buffers
+ * alternate, so `load` of one miss overlaps the copy of the previous one.  Not while a chain is being
+ * recorded.  With dev = NULL the cache keeps the books only (no arena, `load` unused): hit rates of a
+ * routing trace under a budget, without a GPU. */
+typedef struct ojh_gather_stats {
+    uint64_t hits, misses, bytes_streamed, evictions;
+} ojh_gather_stats;
+/* Fill dst[0 .. bytes) with expert `id`; return 0, or non-zero to abort the gather. */
+typedef int (*ojh_expert_load_fn)(void *user, uint32_t id, void *dst, size_t bytes);
+int ojh_expert_cache_create(ojh_device *dev, size_t budget_bytes, size_t expert_bytes, ojh_expert_cache **out);
+int ojh_expert_cache_destroy(ojh_expert_cache *cache);
+uint32_t ojh_expert_cache_slots(const ojh_expert_cache *cache);
+size_t ojh_expert_cache_resident_bytes(const ojh_expert_cache *cache);   /* slots * expert_bytes */
+ojh_buf *ojh_expert_cache_arena(ojh_expert_cache *cache);                /* owned by the cache */
+int ojh_expert_cache_gather(ojh_expert_cache *cache, const uint32_t *ids, size_t n, ojh_expert_load_fn load,
+                            void *user, uint64_t *offsets);
+int ojh_expert_cache_stats(const ojh_expert_cache *cache, ojh_gather_stats *out);
 
 /* ---- GGUF files -> device (no GPU needed for the reader itself) --------------------------------
  * `Gguf::open` / `tensor_meta` / `read_tensor_raw` (crates/ojas-formats/src/gguf.rs:100-206, 297-339,

@@ -62,6 +62,12 @@ class Caps:
 
 
 _lib = None
+# int load(void *user, uint32_t id, void *dst, size_t bytes)
+EXPERT_LOAD_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_uint32, C.c_void_p, C.c_size_t)
+
+
+class _GatherStats(C.Structure):
+    _fields_ = [("hits", C.c_uint64), ("misses", C.c_uint64), ("bytes_streamed", C.c_uint64), ("evictions", C.c_uint64)]
 
 
 def load_library(path: str | None = None) -> C.CDLL:
@@ -132,6 +138,13 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_moe_route": (i32, [vp, vp, u32, u32, u32, vp, vp]),
         "ojh_moe_ffn": (i32, [vp, vp, u32, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp, i32, i32]),
         "ojh_moe_ffn_slots": (i32, [vp, vp, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp, vp, vp, i32]),
+        "ojh_expert_cache_create": (i32, [vp, sz, sz, C.POINTER(vp)]),
+        "ojh_expert_cache_destroy": (i32, [vp]),
+        "ojh_expert_cache_slots": (u32, [vp]),
+        "ojh_expert_cache_resident_bytes": (sz, [vp]),
+        "ojh_expert_cache_arena": (vp, [vp]),
+        "ojh_expert_cache_gather": (i32, [vp, vp, sz, EXPERT_LOAD_FN, vp, vp]),
+        "ojh_expert_cache_stats": (i32, [vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -141,6 +154,83 @@ def load_library(path: str | None = None) -> C.CDLL:
     if path is None:
         _lib = L
     return L
+
+
+class ExpertCache:
+    """Device arena of expert slots with LRU eviction (`ExpertCache`, crates/ojas-cuda/src/expert_cache.rs:34-152).
+    `gather(ids, load)` returns one u64 byte offset into `arena` per id; `load(id) -> bytes-like of expert_bytes`
+    supplies a missing expert.  With `gpu=None` only the bookkeeping runs (hit rates of a routing trace)."""
+
+    def __init__(self, gpu: "HipGpu | None", budget_bytes: int, expert_bytes: int):
+        self._L = gpu._L if gpu is not None else load_library()
+        self.gpu, self.expert_bytes = gpu, expert_bytes
+        h = C.c_void_p()
+        rc = self._L.ojh_expert_cache_create(gpu._dev if gpu is not None else None, budget_bytes, expert_bytes, C.byref(h))
+        if rc:
+            raise OjasHipError(rc, (self._L.ojh_last_error() or b"").decode())
+        self._h = h
+        self.arena = None
+        if gpu is not None:
+            self.arena = Buf(gpu, self._L.ojh_expert_cache_arena(h), self.resident_bytes)
+            self.arena.free = lambda: None      # the cache owns it
+
+    @property
+    def slots(self) -> int:
+        return self._L.ojh_expert_cache_slots(self._h)
+
+    @property
+    def resident_bytes(self) -> int:
+        return self._L.ojh_expert_cache_resident_bytes(self._h)
+
+    @property
+    def stats(self) -> dict:
+        st = _GatherStats()
+        rc = self._L.ojh_expert_cache_stats(self._h, C.byref(st))
+        if rc:
+            raise OjasHipError(rc, (self._L.ojh_last_error() or b"").decode())
+        return {k: int(getattr(st, k)) for k, _ in _GatherStats._fields_}
+
+    @property
+    def hit_rate(self) -> float:
+        st = self.stats
+        total = st["hits"] + st["misses"]
+        return st["hits"] / total if total else 0.0
+
+    def gather(self, ids, load=None) -> np.ndarray:
+        ids = np.ascontiguousarray(ids, np.uint32).ravel()
+        offs = np.empty(ids.size, np.uint64)
+        failure = []
+
+        def _cb(_user, eid, dst, nbytes):
+            try:
+                src = np.frombuffer(load(int(eid)), np.uint8)
+                if src.size != nbytes:
+                    raise ValueError(f"expert {eid}: load returned {src.size} bytes, the slot holds {nbytes}")
+                C.memmove(dst, src.ctypes.data, nbytes)
+                return 0
+            except Exception as e:      # an exception must not unwind through the C frame
+                failure.append(e)
+                return 1
+
+        cb = EXPERT_LOAD_FN(_cb) if load is not None else C.cast(None, EXPERT_LOAD_FN)
+        rc = self._L.ojh_expert_cache_gather(self._h, C.c_void_p(ids.ctypes.data), ids.size, cb, None,
+                                             C.c_void_p(offs.ctypes.data))
+        if failure:
+            raise failure[0]
+        if rc:
+            raise OjasHipError(rc, (self._L.ojh_last_error() or b"").decode())
+        return offs
+
+    def close(self) -> None:
+        if self._h:
+            self._L.ojh_expert_cache_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class Gguf:
