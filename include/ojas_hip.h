@@ -262,7 +262,7 @@ int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uin
  * Expert indices must be below n_expert (one that is not never reads outside the tensors; what
  * it contributes is unspecified). Up to 8 tokens run as two launches addressed
  * by assignment (bit-identical to the grouped integer-dot pipeline); larger batches are grouped
- * by expert, on int8 MFMA from four assignments per expert (sums associate differently there:
+ * by expert, on int8 MFMA from three to four assignments per expert (sums associate differently there:
  * last ulps). Environment: OJAS_HIP_MOE = 1 / 2 / 3 forces MFMA / grouped dots / the decode
  * form, OJAS_HIP_MOE_DEC_TOKENS moves the 8. */
 int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint32_t d, uint32_t n_ff,
