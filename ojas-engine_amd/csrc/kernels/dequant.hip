@@ -31,6 +31,33 @@ dequant_q80_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblo
     out[i] = f32_to_f16_bits(__fmul_rn(d, q));
 }
 
+// Embedding gather straight out of Q8_0 storage (crates/ojas-cuda/src/kernels/gemv_q8.rs:262-293): row `token`
+// of the table as f32, each value the exact f32 product d * q (the decoder above rounds it once more to
+// f16).  embed_q80(table, out, token, d) takes the id as a launch constant, embed_q80_g(table, out, ctl, d)
+// reads it from ctl[0] on the device, so a recorded decode step replays without re-recording per token.
+// Any grid of up to 256-thread blocks (a thread per weight, grid-stride).  ROWS, appended by the dispatcher
+// from the table's extent, is not in the reference's argument list: an id past the table yields zeros.
+__device__ __forceinline__ void embed_q80_row(const uchar* __restrict__ table, float* __restrict__ out,
+                                              uint token, uint d, uint ROWS) {
+    const uchar* row = table + (size_t)token * (d >> 5) * Q80_BYTES;
+    for (uint i = blockIdx.x * blockDim.x + threadIdx.x; i < d; i += gridDim.x * blockDim.x) {
+        float v = 0.0f;
+        if (token < ROWS) {
+            const uchar* blk = row + (size_t)(i >> 5) * Q80_BYTES;
+            v = __fmul_rn(f16_bits_to_f32(*(const ushort*)blk), (float)(signed char)blk[2u + (i & 31u)]);
+        }
+        out[i] = v;
+    }
+}
+extern "C" __global__ void __launch_bounds__(256)
+embed_q80(const uchar* __restrict__ table, float* __restrict__ out, uint token, uint d, uint ROWS) {
+    embed_q80_row(table, out, token, d, ROWS);
+}
+extern "C" __global__ void __launch_bounds__(256)
+embed_q80_g(const uchar* __restrict__ table, float* __restrict__ out, const uint* __restrict__ ctl, uint d, uint ROWS) {
+    embed_q80_row(table, out, ctl[0], d, ROWS);
+}
+
 extern "C" __global__ void __launch_bounds__(256)
 dequant_q4k_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
     // 32 threads per super-block; thread t owns dword t of qs: 4 low-nibble weights of

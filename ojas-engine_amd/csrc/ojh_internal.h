@@ -118,6 +118,7 @@ struct ojh_kernel_spec {
     // expert tensors, need[] is one expert's bytes, and the dispatcher appends min(extent / need) as a
     // trailing constant so that an index past the tensors multiplies nothing instead of reading past them.
     int expert_bufs = 0;
+    int bound_first = 1;   // index of the first such buffer (0 for a table that is the first argument)
     // Streamed-expert kernels: buffers 1 .. arena_bufs are cache arenas addressed by byte offsets, need[] is one
     // expert's bytes, and the dispatcher appends, per arena, the last offset at which an expert still fits.
     int arena_bufs = 0;

@@ -618,6 +618,30 @@ static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint
     return OJH_OK;
 }
 
+// embed_q80(table, out, token, d) / embed_q80_g(table, out, ctl, d): a thread per weight, grid-stride
+static int check_embed(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                       const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const uint32_t d = c[s->n_consts - 1];
+    if (!d || d % 32) return ojh_fail(OJH_ERR_ARG, "%s: d=%u must be a positive multiple of 32", s->name, d);
+    int rc = check_block(block, 0);
+    if (rc) return rc;
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    need[0] = (size_t)(d / 32) * 34;      // one row; the dispatcher turns the extent into the row bound
+    need[1] = (size_t)d * 4;
+    need[2] = 4;
+    align[0] = 2;
+    align[1] = align[2] = 4;
+    return OJH_OK;
+}
+static int shape_embed(const ojh_kernel_spec *, const ojh_device *, uint32_t K, uint32_t, uint32_t,
+                       uint32_t grid[3], uint32_t block[3]) {   // K = d
+    grid[0] = (K + 255) / 256;
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // gemm_mm_<fmt>(xh, w, y, K, N, accum, M) and gemm_mm_<fmt>_sk(xh, w, y, K, N, M, nsplit);
 // `rows_per_wave` = 1 marks the split-K form.
 // `rows_per_wave` carries the variant: bit 0 = split-K entry; 0/1 the 256 x 128 tile of family
@@ -1097,6 +1121,12 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("gemm_q8k_q4k_ml", "gemm_q8k", 4, 4, OJH_Q4_K, 1, check_gemm_q8k_ml, shape_ml);
     add("gemm_q8k_q4k_mk", "gemm_q8k", 4, 4, OJH_Q4_K, 2, check_gemm_q8k_ml, shape_mk);
     add("relayout_q4k_q4l", "dequant", 4, 1, OJH_Q4_K, 0, check_relayout, shape_relayout);
+    add("embed_q80", "dequant", 2, 2, OJH_Q8_0, 0, check_embed, shape_embed);
+    m.back().expert_bufs = 1;
+    m.back().bound_first = 0;
+    add("embed_q80_g", "dequant", 3, 1, OJH_Q8_0, 0, check_embed, shape_embed);
+    m.back().expert_bufs = 1;
+    m.back().bound_first = 0;
     add("rows_q8_from_f16", "rowq8", 3, 2, 0, 0, check_rowq8, shape_rowq8);
     add("quant_rows_i8", "rowq8", 3, 2, 0, 1, check_rowq8, shape_rowq8);
     add("matmul_q8row", "rowq8", 5, 3, 0, 2, check_rowq8, shape_rowq8);

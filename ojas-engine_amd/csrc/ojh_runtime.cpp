@@ -338,8 +338,8 @@ extern "C" int ojh_dispatch(ojh_device *dev, const char *name, int n_bufs, ojh_b
     }
     std::vector<uint32_t> cv(consts, consts + n_consts);
     if (s->expert_bufs) {   // how many experts the tensors hold: the kernel's bound on the routed indices
-        size_t experts = 1024;
-        for (int i = 1; i <= s->expert_bufs; i++) {
+        size_t experts = 0xFFFFFFFFu;
+        for (int i = s->bound_first; i < s->bound_first + s->expert_bufs; i++) {
             size_t off = offsets ? (size_t)offsets[i] : 0;
             experts = std::min(experts, (bufs[i]->bytes - off) / need[i]);
         }

@@ -261,6 +261,19 @@ def q80_rows_lcg(rows: int, k: int, seed: int) -> tuple[np.ndarray, np.ndarray]:
     return out.reshape(-1), plain
 
 
+def q80_weights_lcg(n: int, k: int, seed: int) -> np.ndarray:
+    """Q8_0 rows of crates/ojas-cuda/tests/conformance.rs:611-630: d = f16(0.004 + 0.001 ((r + b) mod 5)), codes as in
+    `q80_rows_lcg`."""
+    nb = k // 32
+    raw, _ = q80_rows_lcg(n, k, seed)
+    raw = raw.reshape(n, nb, 34).copy()
+    r, b = np.arange(n)[:, None], np.arange(nb)[None, :]
+    d = (np.float32(0.004) + np.float32(0.001) * ((r + b) % 5).astype(np.float32)).astype(np.float16).view(np.uint16)
+    raw[:, :, 0] = d & 0xFF
+    raw[:, :, 1] = d >> 8
+    return raw.reshape(-1)
+
+
 def iq4_rows_lcg(ty: int, rows: int, k: int, seed: int) -> np.ndarray:
     """IQ4_XS / IQ4_NL rows of the reference's GPU conformance test (crates/ojas-cuda/tests/conformance.rs:461-503):
     byte i = trunc(255 |tvec(1, seed + i)|), then d of block (r, b) = f16(0.01 + 0.002 ((r + b) mod 7 | 5))."""

@@ -88,3 +88,39 @@ def test_relayout_q4k_q4l_is_bit_exact(gpu, orc, pkg):
     assert np.array_equal(gpu.read(nib, n * k // 2, np.uint8), wn)
     assert np.array_equal(gpu.read(qa, n * k // 32, np.uint16), wa)
     assert np.array_equal(gpu.read(qb, n * k // 32, np.uint16), wb)
+
+
+def test_embed_q80_matches_reader(gpu, orc, pkg):
+    """`embed_q80` / `embed_q80_g` gather a row out of Q8_0 storage (crates/ojas-cuda/tests/conformance.rs:738-764:
+    vocab 64, d 512, tokens 0, 7, 63, the reference's grid [8] x 128 threads): rounding the output to f16
+    reproduces `dequant_to_f16` exactly, and the f32 values are the exact products d * q."""
+    vocab, d = 64, 512
+    raw = pkg.synth.q80_weights_lcg(vocab, d, 90)
+    vals16 = orc.dequant_to_f16(raw, Q8_0, vocab * d).reshape(vocab, d)
+    blocks = raw.reshape(vocab, d // 32, 34)
+    exact = (blocks[:, :, :2].copy().view(np.float16).astype(np.float32) * blocks[:, :, 2:].view(np.int8).astype(np.float32)).reshape(vocab, d)
+    gpu.ensure_family("dequant")
+    pad = 34 * 3
+    td = gpu.upload_bytes(np.concatenate([np.full(pad, 0xEE, np.uint8), raw]))
+    od = gpu.alloc(d + 2)
+    ctl = gpu.alloc_bytes(4)
+    for token in (0, 7, 63):
+        for name in ("embed_q80", "embed_q80_g"):
+            gpu.write_bytes(od, 0, np.full(d + 2, 777.0, np.float32))
+            if name == "embed_q80":
+                gpu.dispatch(gpu.begin(), name, [(td, pad), (od, 4)], [token, d], [8, 1, 1], [128, 1, 1])
+            else:
+                gpu.write_bytes(ctl, 0, np.array([token], np.uint32))
+                gpu.dispatch(gpu.begin(), name, [(td, pad), (od, 4), (ctl, 0)], [d], [8, 1, 1], [128, 1, 1])
+            got = gpu.read(od, d + 2)
+            assert got[0] == 777.0 and got[-1] == 777.0, "wrote outside the row"
+            assert np.array_equal(got[1:-1], exact[token]), (name, token)
+            assert np.array_equal(got[1:-1].astype(np.float16).view(np.uint16), vals16[token]), (name, token)
+    # the library's own geometry, and an id past the table: zeros, nothing read
+    grid, block = gpu.launch_shape("embed_q80", d, 0)
+    gpu.dispatch(gpu.begin(), "embed_q80", [(td, pad), (od, 4)], [63, d], grid, block)
+    assert np.array_equal(gpu.read(od, d + 2)[1:-1], exact[63])
+    gpu.dispatch(gpu.begin(), "embed_q80", [(td, pad), (od, 4)], [64, d], grid, block)
+    assert np.all(gpu.read(od, d + 2)[1:-1] == 0.0)
+    with pytest.raises(pkg.OjasHipError, match="multiple of 32"):
+        gpu.dispatch(gpu.begin(), "embed_q80", [(td, pad), (od, 4)], [0, 48], grid, block)
