@@ -169,17 +169,22 @@ def main() -> int:
         cal[kname] = {"bytes_moved": moved, "us": round(us, 1), "gbs": round(moved / us / 1e3, 1)}
     del cal_src, cal_dst
 
-    # ---- per-shape latency (each shape alone, back to back, rotating sets), for the record
+    # ---- per-shape latency (each shape alone, back to back, rotating sets), for the record.  The launches are
+    # recorded once and replayed from the library, like the step: issued one by one from Python the short
+    # ones would show the interpreter's call rate, not the kernel
     per_shape = {}
     reps = 50
     for name, n, k in SHAPES:
         st = next(s for s, _, names in STAGES if name in names)
-        for i in range(3):
-            one(st, sets[i % args.copies][name], ys[name])
-        gpu.timer_start()
+        gpu.capture_begin()
         for i in range(reps):
             one(st, sets[i % args.copies][name], ys[name])
+        chain = gpu.capture_end()
+        chain.launch()
+        gpu.timer_start()
+        chain.launch()
         us = gpu.timer_stop() / reps * 1e3
+        del chain
         b = algorithmic_bytes(n, k)
         per_shape[name] = {"n": n, "k": k, "us": round(us, 2), "gbs": round(b / us / 1e3, 1),
                            "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
