@@ -445,7 +445,7 @@ __device__ __forceinline__ void gemv_nat_iq4_body(const float* __restrict__ x, c
 #pragma unroll
         for (int r = 0; r < R; r++) f[r] = W::load(w + (size_t)min(row0 + r, N - 1u) * rb, u, lane);
         const float* xp = x + (size_t)u * W::x_unit(0) + W::x_off(lane);
-        const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + 16);
+        const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + W::XGAP);
         const float xsum = sum4(x0) + sum4(x1);      // for the formats with an offset or a minimum
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] += W::dot(f[r], lane, x0, x1, xsum);
@@ -475,7 +475,7 @@ __device__ __forceinline__ void gemv_nat_iq4_m_body(const float* __restrict__ x,
             for (int i = 0; i < MT; i++) {
                 const uint m = min(m0 + i, M - 1u);
                 const float* xp = x + (size_t)m * K + (size_t)u * W::x_unit(0) + W::x_off(lane);
-                const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + 16);
+                const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + W::XGAP);
                 acc[i] += W::dot(f, lane, x0, x1, sum4(x0) + sum4(x1));
             }
         }
@@ -513,7 +513,7 @@ __device__ __forceinline__ void gemv_nat_iq4_px_body(const float* __restrict__ x
         if (u < nu) {
             const float* xp = x + (size_t)u * W::x_unit(0) + W::x_off(lane);
             xr[s][0] = *(const float4*)xp;
-            xr[s][1] = *(const float4*)(xp + 16);
+            xr[s][1] = *(const float4*)(xp + W::XGAP);
         }
         xsum[s] = sum4(xr[s][0]) + sum4(xr[s][1]);
     }
@@ -547,7 +547,16 @@ GEMV_NAT_IQ4_PX(q40, Q40W)
 GEMV_NAT_IQ4_PX(q41, Q41W)
 GEMV_NAT_IQ4_PX(q50, Q50W)
 GEMV_NAT_IQ4_PX(q51, Q51W)
+GEMV_NAT_IQ4_PX(q5k, Q5kW)
 
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_q5k_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
+    gemv_nat_iq4_body<Q5kW, R, MODE>(x, w, y, bs, K, N);
+}
+template <int MT>
+__device__ __forceinline__ void gemv_nat_q5k_m_body(const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    gemv_nat_iq4_m_body<Q5kW, MT>(x, w, y, K, N, M, ACC);
+}
 template <int R, int MODE>
 __device__ __forceinline__ void gemv_nat_q40_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
     gemv_nat_iq4_body<Q40W, R, MODE>(x, w, y, bs, K, N);
@@ -940,3 +949,4 @@ GEMV_NAT_ENTRIES(q50)
 GEMV_NAT_ENTRIES(q51)
 GEMV_NAT_ENTRIES(q2k)
 GEMV_NAT_ENTRIES(q3k)
+GEMV_NAT_ENTRIES(q5k)

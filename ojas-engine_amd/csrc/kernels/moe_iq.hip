@@ -38,7 +38,7 @@ __device__ __forceinline__ void moe_gu_rows(const float* __restrict__ x, const u
         const typename W::Frag fg0 = W::load(g0, u, lane), fg1 = W::load(g0 + r1, u, lane);
         const typename W::Frag fu0 = W::load(u0, u, lane), fu1 = W::load(u0 + r1, u, lane);
         const float* xp = xt + (size_t)u * W::x_unit(0) + W::x_off(lane);
-        const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + 16);
+        const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + W::XGAP);
         const float xsum = sum4(x0) + sum4(x1);
         ag[0] += W::dot(fg0, lane, x0, x1, xsum);
         ag[1] += W::dot(fg1, lane, x0, x1, xsum);
@@ -73,7 +73,7 @@ __device__ __forceinline__ void moe_down_rows(const float* __restrict__ act, con
 #pragma unroll
                 for (int r = 0; r < 4; r++) f[r] = W::load(wd + ((size_t)e * N + min(row0 + (uint)r, N - 1u)) * rb, u, lane);
                 const float* xp = xr + (size_t)u * W::x_unit(0) + W::x_off(lane);
-                const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + 16);
+                const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + W::XGAP);
                 const float xsum = sum4(x0) + sum4(x1);
 #pragma unroll
                 for (int r = 0; r < 4; r++) a[r] += W::dot(f[r], lane, x0, x1, xsum);

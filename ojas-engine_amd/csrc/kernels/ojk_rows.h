@@ -2,7 +2,7 @@
 // weights 16..31 in the high nibbles (IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1), for kernels that multiply raw
 // rows with f32 activations: the dense matvecs and the expert products share them.
 // A trait W gives the lane map of one wave step — units(K) blocks in a row, STEP of them per step, lane ->
-// unit_of(lane), the lane's two float4 of x at x_unit * u + x_off(lane) and 16 floats further on — and
+// unit_of(lane), the lane's two float4 of x at x_unit * u + x_off(lane) and XGAP floats further on — and
 // load / dot for the lane's fragment of a block.
 #pragma once
 #include "ojk_common.h"
@@ -46,6 +46,7 @@ __device__ __forceinline__ float iq4_lane_dot(uint q, float4 x0, float4 x1) {
 }
 
 struct Iq4nlW {
+    static constexpr uint XGAP = 16u;            // floats between the lane's two x fragments
     static constexpr uint STEP = 16u;            // blocks a wave walks per step
     static constexpr uint BYTES = IQ4NL_BYTES;
     static __device__ __forceinline__ uint units(uint K) { return K >> 5; }
@@ -67,6 +68,7 @@ struct Iq4nlW {
 };
 
 struct Iq4xsW {
+    static constexpr uint XGAP = 16u;
     static constexpr uint STEP = 2u;             // super-blocks per step
     static constexpr uint BYTES = IQ4XS_BYTES;
     static __device__ __forceinline__ uint units(uint K) { return K >> 8; }
@@ -96,6 +98,7 @@ struct Iq4xsW {
 // lane's eight activations once per block:  d * (sum q x - off * sum x)  or  d * sum q x + m * sum x.
 template <bool FIVE, bool AFFINE>
 struct LegacyW {
+    static constexpr uint XGAP = 16u;
     static constexpr uint STEP = 16u;
     static constexpr uint BYTES = 18u + (AFFINE ? 2u : 0u) + (FIVE ? 4u : 0u);
     static constexpr uint HDR = AFFINE ? 4u : 2u;
@@ -135,3 +138,40 @@ typedef LegacyW<false, true> Q41W;
 typedef LegacyW<true, false> Q50W;
 typedef LegacyW<true, true> Q51W;
 
+
+// Q5_K on f32 activations (the reference's native matvec for the format, crates/ojas-core/src/quant_src.rs:100):
+// a 176-byte super-block {f16 d, dmin; 12 scale bytes; qh[32]; qs[128]}.  Within chunk c of 64 weights the low
+// nibbles of qs[32c .. 32c+31] are sub-block 2c and the high nibbles sub-block 2c+1, so a dword of qs meets two
+// float4 of x 32 floats apart; the fifth bit of weight l of sub-block s is bit s of qh[l].  32 lanes per
+// super-block, w = d sc q - dmin m (crates/ojas-formats/src/gguf.rs:1060-1085).
+struct Q5kW {
+    static constexpr uint XGAP = 32u;
+    static constexpr uint STEP = 2u;
+    static constexpr uint BYTES = Q5K_BYTES;
+    static __device__ __forceinline__ uint units(uint K) { return K >> 8; }
+    static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 5; }
+    static __device__ __forceinline__ uint x_off(uint lane) { return ((lane & 31u) >> 3) * 64u + (lane & 7u) * 4u; }
+    static __device__ __forceinline__ uint x_unit(uint) { return 256u; }
+    struct Frag { uint hdr, s0, s1, s2, h, q; };
+    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
+        const uint* blk = (const uint*)(row + (size_t)u * Q5K_BYTES);
+        Frag f;
+        f.hdr = blk[0];
+        f.s0 = blk[1];
+        f.s1 = blk[2];
+        f.s2 = blk[3];
+        f.h = blk[4u + (lane & 7u)];
+        f.q = blk[12u + (lane & 31u)];
+        return f;
+    }
+    static __device__ __forceinline__ float dot(const Frag& f, uint lane, float4 x0, float4 x1, float) {
+        const uint c = (lane & 31u) >> 3;
+        uint sc, mn;
+        q4k_scale_min_pair(f.s0, f.s1, f.s2, c, sc, mn);
+        const uint lo = (f.q & 0x0F0F0F0Fu) | (((f.h >> (2u * c)) & 0x01010101u) << 4);
+        const uint hi = ((f.q >> 4) & 0x0F0F0F0Fu) | (((f.h >> (2u * c + 1u)) & 0x01010101u) << 4);
+        const float a = (float)(sc & 0xFFu) * dot4_ub(lo, x0, 0.0f) + (float)(sc >> 8) * dot4_ub(hi, x1, 0.0f);
+        const float b = (float)(mn & 0xFFu) * sum4(x0) + (float)(mn >> 8) * sum4(x1);
+        return f16_bits_to_f32(f.hdr & 0xFFFFu) * a - f16_bits_to_f32(f.hdr >> 16) * b;
+    }
+};

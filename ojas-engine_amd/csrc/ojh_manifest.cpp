@@ -1069,7 +1069,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     for (const auto &f : kFormats) {
         std::string t = f.tag;
         add("dequant_" + t + "_f16", "dequant", 2, 1, f.type, 0, check_dequant, shape_dequant);
-        if (f.type == OJH_Q5_K) {   // Q5_K: the decoder and the CPU path's int8-activation matvec
+        if (f.type == OJH_Q5_K) {   // Q5_K: the decoder, the CPU path's int8-activation matvec
             std::string q5 = "gemv_q8k_" + t;
             add(q5, "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
             add(q5 + "_r1", "gemv_q8k", 4, 2, f.type, 1, check_gemv_q8k, shape_rows);
@@ -1078,6 +1078,15 @@ static std::vector<ojh_kernel_spec> build_manifest() {
             add(q5 + "_accum", "gemv_q8k", 4, 2, f.type, 1, check_gemv_q8k, shape_rows);
             add(q5 + "_bias", "gemv_q8k", 5, 2, f.type, 1, check_gemv_q8k, shape_rows);
             add(q5 + "_m", "gemv_q8k", 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
+            // ... and the f32-activation matvecs of the reference's GPU path (no MFMA tile)
+            std::string n5 = "gemv_nat_" + t;
+            add(n5, "gemv", 3, 2, f.type, 4, check_gemv_nat, shape_rows);
+            add(n5 + "_r1", "gemv", 3, 2, f.type, 1, check_gemv_nat, shape_rows);
+            add(n5 + "_r2", "gemv", 3, 2, f.type, 2, check_gemv_nat, shape_rows);
+            add(n5 + "_accum", "gemv", 3, 2, f.type, 4, check_gemv_nat, shape_rows);
+            add(n5 + "_bias", "gemv", 4, 2, f.type, 4, check_gemv_nat, shape_rows);
+            add(n5 + "_m", "gemv", 3, 4, f.type, 1, check_gemv_nat_m, shape_rows);
+            add(n5 + "_px", "gemv", 3, 2, f.type, 2, check_gemv_nat_px, shape_px);
             continue;
         }
         std::string g = "gemv_nat_" + t;

@@ -357,17 +357,14 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     void *wp = at(w->raw, w->off), *yp = at(y, y_off);
     uint32_t grid[3] = {1, 1, 1}, block[3] = {256, 1, 1};
 
-    // Q5_K has the CPU path's arithmetic only (dot_q5k over int8 activations); no floating-point
-    // matvec and no MFMA tile read it, at any token count.
-    if (w->type == OJH_Q5_K) {
-        if (act_mode == OJH_ACT_FLOAT || act_mode == OJH_ACT_FLOAT_EXACT)
-            return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: Q5_K rows take int8 activations only (OJH_ACT_Q8K or OJH_ACT_AUTO)");
-        act_mode = OJH_ACT_Q8K;
-    }
+    // Q5_K: the CPU path's arithmetic (dot_q5k over int8 activations) unless floating-point activations are
+    // asked for, which run on the f32-activation matvecs at any token count; no MFMA tile reads the format.
+    const bool q5_float = w->type == OJH_Q5_K && (act_mode == OJH_ACT_FLOAT || act_mode == OJH_ACT_FLOAT_EXACT);
+    if (w->type == OJH_Q5_K && !q5_float) act_mode = OJH_ACT_Q8K;
 
     // IQ4_NL / IQ4_XS (dot_iq4nl / dot_iq4xs), Q4_0 / Q4_1 / Q5_0 / Q5_1 and Q2_K / Q3_K: f32 activations against the raw
     // rows at every token count; no int8-activation form and no MFMA tile read them.
-    const bool iq4 = ojh_float_only(w->type);   // (the IQ4 types, the legacy 32-weight blocks, Q2_K, Q3_K)
+    const bool iq4 = ojh_float_only(w->type) || q5_float;   // (the IQ4 types, the legacy 32-weight blocks, Q2_K, Q3_K)
     if (iq4 && act_mode == OJH_ACT_Q8K)
         return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: %s rows take f32 activations only (OJH_ACT_FLOAT or OJH_ACT_AUTO)", f->tag);
 

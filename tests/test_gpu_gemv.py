@@ -70,7 +70,7 @@ def test_q8k_matvec_matches_cpu_reference(gpu, orc, pkg, ty, n, k):
     assert err <= TOL_Q8K_SEEN <= TOL_Q8K, err
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K])
 @pytest.mark.parametrize("n,k", [(13, 2560), (1024, 4096), (96, 14336), (4099, 4096), (33001, 2816)])
 def test_float_matvec_matches_dequant_dot(gpu, orc, pkg, ty, n, k):
     w, x = _inputs(pkg, ty, n, k, "b")
@@ -97,7 +97,7 @@ def test_q80_matvec_matches_dot_q80(gpu, orc, pkg):
     assert peak_err(gpu.read(yd, n), want) <= 1e-5
 
 
-@pytest.mark.parametrize("ty,tag", [(Q4_K, "q4k"), (Q6_K, "q6k"), (Q2_K, "q2k"), (Q3_K, "q3k")])
+@pytest.mark.parametrize("ty,tag", [(Q4_K, "q4k"), (Q6_K, "q6k"), (Q2_K, "q2k"), (Q3_K, "q3k"), (Q5_K, "q5k")])
 @pytest.mark.parametrize("n,k", [(33000, 256), (40001, 2560), (32768, 4096)])
 def test_float_head_form_keeps_activations_in_registers(gpu, orc, pkg, ty, tag, n, k):
     """From 32768 rows a float-activation matvec runs grid-stride with the wave's f32 activations in
@@ -168,8 +168,6 @@ def test_bias_accum_and_batched_variants(gpu, orc, pkg, ty, mode):
     (1000 + i), accumulate onto a seeded y, batched M=3 with different rows, batched accumulate."""
     if ty in (Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K) and mode == "q8k":
         pytest.skip("this format keeps f32 activations in the CPU reference")
-    if ty == Q5_K and mode == "float":
-        pytest.skip("Q5_K has the int8-activation matvec only")
     n, k, m = 200, 1024, 3
     w = pkg.synth.weights(ty, n, k, "var", ty)
     xs = pkg.synth.normal_f32(m * k, "var", "x").reshape(m, k)
@@ -355,9 +353,10 @@ def test_q6k_few_tokens_staged_and_streamed_forms_agree(gpu, orc, pkg, m, n, k, 
 
 
 def test_q5k_takes_the_int8_path_at_every_token_count(gpu, orc, pkg):
-    """Q5_K has dot_q5k's arithmetic (crates/ojas-cpu/src/cpu_math.rs:638-670) and nothing else:
-    AUTO resolves to it for one token and for a prefill-sized batch alike, a floating-point
-    contract is refused, and the wide-row form (N >= 32768) agrees with the oracle too."""
+    """Q5_K defaults to dot_q5k's arithmetic (crates/ojas-cpu/src/cpu_math.rs:638-670): AUTO resolves to it
+    for one token and for a prefill-sized batch alike (no MFMA tile reads the format); a floating-point
+    contract runs the f32-activation matvecs at any token count (the dequantized dot in f64 is the
+    judge); the wide-row form (N >= 32768) agrees with the oracle too."""
     n, k = 300, 1024
     w = pkg.synth.weights(Q5_K, n, k, "q5k", "any-m")
     lin = gpu.lin(Q5_K, n, k, w)
@@ -368,8 +367,8 @@ def test_q5k_takes_the_int8_path_at_every_token_count(gpu, orc, pkg):
         want = np.stack([orc.matvec_kq(w, Q5_K, n, k, xs[t]) for t in range(m)])
         assert peak_err(gpu.read(yd, m * n).reshape(m, n), want) <= TOL_Q8K_SEEN
     for act in (pkg.ACT_FLOAT, pkg.ACT_FLOAT_EXACT):
-        with pytest.raises(pkg.OjasHipError):
-            gpu.mm(gpu.upload(xs), lin, yd, 1, act_mode=act)
+        gpu.mm(gpu.upload(xs), lin, yd, m, act_mode=act)
+        assert peak_err(gpu.read(yd, m * n).reshape(m, n), orc.matmul_ref(w, Q5_K, n, k, xs)) <= TOL_FLOAT
     n, k = 33000, 256
     w, x = _inputs(pkg, Q5_K, n, k, "wide")
     yd = gpu.alloc(n)
