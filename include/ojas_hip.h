@@ -292,7 +292,7 @@ int ojh_moe_ffn_slots(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint
  * queued afterwards sees them, work queued before has finished with the slot.  Two staging buffers
  * alternate, so `load` of one miss overlaps the copy of the previous one.  Not while a chain is being
  * recorded.  With dev = NULL the cache keeps the books only (no arena, `load` unused): hit rates of a
- * routing trace under a budget, without a GPU. */
+ * routing trace under a budget, without a GPU.  Destroy a cache before closing its device. */
 typedef struct ojh_gather_stats {
     uint64_t hits, misses, bytes_streamed, evictions;
 } ojh_gather_stats;

@@ -222,9 +222,11 @@ class ExpertCache:
         return offs
 
     def close(self) -> None:
-        if self._h:
+        # a cache belongs to its device and is destroyed before it; one that outlived a closed device is dropped
+        # unreleased rather than handed a freed device (the arena then lives until the process ends)
+        if self._h and (self.gpu is None or self.gpu._dev):
             self._L.ojh_expert_cache_destroy(self._h)
-            self._h = None
+        self._h = None
 
     def __del__(self):
         try:
