@@ -496,12 +496,11 @@ moe_down_q6k_dec(const float* act, const uchar* wd, const uint* idx, const float
 
 // ------------------------------------------------------------------ Q8_0 experts, f32 activations
 //   moe_gu_q80(x, wg, wu, act, idx, K, N)              grid [ceil(N/8), KSEL, tokens], block 256
-//   moe_down_q80(act, wd, y, idx, wgt, K, N, KSEL)     grid [1 .. ceil(N/8), tokens, 1], block 256 (rows grid-stride,
-//                                                      16 per workgroup and step: the reference's ceil(N/32) is a valid grid)
+//   moe_down_q80(act, wd, y, idx, wgt, K, N, KSEL)     grid [1 .. ceil(N/4), tokens, 1], block 256 (rows grid-stride,
+//                                                      4 per workgroup and step: the reference's ceil(N/32) is a valid grid)
 // The reference's expert kernels by their own names and arguments
 // (crates/ojas-cuda/src/kernels/moe.rs:75-125): act[j][n] = silu(gate_e . x) * (up_e . x) for the expert
-// e = idx[j] of slot j, and y[n] += sum_j wgt[j] * (down_e . act[j]) — the down launch accumulates onto
-// y, slots in order.  Q8_0 rows meet f32 activations, as dot_q80 does
+// e = idx[j] of slot j, and y[n] += sum_j wgt[j] * (down_e . act[j]) — the down launch accumulates onto y.  Q8_0 rows meet f32 activations, as dot_q80 does
 // (crates/ojas-cpu/src/cpu_math.rs:971-981).  The third (second) grid dimension walks tokens: token t
 // reads x + t K, idx + t KSEL, wgt + t KSEL and writes act + t KSEL N, y + t N; a one-token caller
 // leaves it at 1.  Four lanes share a 34-byte block, a wave walks 16 blocks per step.  The trailing E is
@@ -573,30 +572,43 @@ moe_gu_q80(const float* __restrict__ x, const uchar* __restrict__ wg, const ucha
     moe_gu_q80_body(x + (size_t)t * K, wg + eb, wu + eb, act + ((size_t)t * ksel + j) * N, K, N, e < E ? K >> 5 : 0u);
 }
 
+// The down launches: a workgroup owns four rows at a time (rows grid-stride over the workgroups), its four
+// waves take the slots j = wave, wave + 4, ... and meet in LDS, where the partial sums are added in wave order
+// onto y — an expert row is short (a few hundred to a few thousand weights), so the slots are the parallelism
+// that fills the chip at one token.
+__device__ __forceinline__ void moe_down_finish(float (&res)[4], float* __restrict__ yt, uint N, uint row0) {
+    __shared__ float part[4][4];
+    const uint lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) part[wave][r] = res[r];
+    }
+    __syncthreads();
+    if (threadIdx.x < 4u && row0 + threadIdx.x < N)
+        yt[row0 + threadIdx.x] += ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) + part[3][threadIdx.x];
+    __syncthreads();
+}
+
 extern "C" __global__ void __launch_bounds__(256)
 moe_down_q80(const float* __restrict__ act, const uchar* __restrict__ wd, float* __restrict__ y,
              const uint* __restrict__ idx, const float* __restrict__ wgt, uint K, uint N, uint KSEL, uint E) {
-    const uint t = blockIdx.y;
+    const uint t = blockIdx.y, wave = threadIdx.x >> 6;
     const size_t eb = (size_t)N * ((size_t)(K >> 5) * Q80_BYTES);
-    for (uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 4u; row0 < N; row0 += gridDim.x * 16u) {
+    for (uint row0 = blockIdx.x * 4u; row0 < N; row0 += gridDim.x * 4u) {
         float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (uint j = 0; j < KSEL; j++) {
+        for (uint j = wave; j < KSEL; j += 4u) {
             const uint e = idx[t * KSEL + j];
             if (e >= E) continue;
             moe_down_q80_part(act + ((size_t)t * KSEL + j) * K, wd + (size_t)e * eb, K, N, row0, wgt[t * KSEL + j], res);
         }
-        if ((threadIdx.x & 63u) == 0) {
-#pragma unroll
-            for (int r = 0; r < 4; r++)
-                if (row0 + r < N) y[(size_t)t * N + row0 + r] += res[r];
-        }
+        moe_down_finish(res, y + (size_t)t * N, N, row0);
     }
 }
 
 // Streamed Q8_0 experts (crates/ojas-cuda/src/kernels/moe.rs:133-174): the experts of a layer sit at whatever
 // slots of a cache arena were free, and the host passes one u32 byte offset per selected expert in place of
 // the index.   moe_gu_q80_slots(x, arena_g, arena_u, act, off_g, off_u, K, N)   grid [ceil(N/8), KSEL, tokens]
-//              moe_down_q80_slots(act, arena, y, off_d, wgt, K, N, KSEL)          grid [1 .. ceil(N/8), tokens, 1]
+//              moe_down_q80_slots(act, arena, y, off_d, wgt, K, N, KSEL)          grid [1 .. ceil(N/4), tokens, 1]
 // The trailing LIM constants are appended by the dispatcher — the last offset at which a whole expert still
 // fits its arena — and an offset is rounded down to the blocks' two-byte alignment and clamped to LIM, so a bad
 // table reads a wrong expert, never past the arena.
@@ -612,17 +624,13 @@ moe_gu_q80_slots(const float* __restrict__ x, const uchar* __restrict__ arena_g,
 extern "C" __global__ void __launch_bounds__(256)
 moe_down_q80_slots(const float* __restrict__ act, const uchar* __restrict__ arena, float* __restrict__ y,
                    const uint* __restrict__ off_d, const float* __restrict__ wgt, uint K, uint N, uint KSEL, uint LIM) {
-    const uint t = blockIdx.y;
-    for (uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 4u; row0 < N; row0 += gridDim.x * 16u) {
+    const uint t = blockIdx.y, wave = threadIdx.x >> 6;
+    for (uint row0 = blockIdx.x * 4u; row0 < N; row0 += gridDim.x * 4u) {
         float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (uint j = 0; j < KSEL; j++)
+        for (uint j = wave; j < KSEL; j += 4u)
             moe_down_q80_part(act + ((size_t)t * KSEL + j) * K, arena + min(off_d[t * KSEL + j] & ~1u, LIM), K, N, row0,
                               wgt[t * KSEL + j], res);
-        if ((threadIdx.x & 63u) == 0) {
-#pragma unroll
-            for (int r = 0; r < 4; r++)
-                if (row0 + r < N) y[(size_t)t * N + row0 + r] += res[r];
-        }
+        moe_down_finish(res, y + (size_t)t * N, N, row0);
     }
 }
 

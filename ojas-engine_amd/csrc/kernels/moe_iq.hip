@@ -4,8 +4,8 @@
 // (crates/ojas-cuda/src/kernels/moe_iq.rs:64-112; the expert table crates/ojas-core/src/quant_src.rs:168-193):
 //   moe_gu_<fmt>(x, wg, wu, act, idx, K, N)             grid [ceil(N/8), KSEL, tokens], block 256
 //       act[j][n] = silu(gate_e . x) * (up_e . x),  e = idx[j]
-//   moe_down_<fmt>(act, wd, y, idx, wgt, K, N, KSEL)    grid [1 .. ceil(N/8), tokens, 1], block 256
-//       y[n] += sum_j wgt[j] * (down_e . act[j])        (accumulates onto y, slots in order)
+//   moe_down_<fmt>(act, wd, y, idx, wgt, K, N, KSEL)    grid [1 .. ceil(N/4), tokens, 1], block 256
+//       y[n] += sum_j wgt[j] * (down_e . act[j])        (accumulates onto y)
 // for <fmt> = iq4xs and iq4nl — the streamed models keep IQ4_XS gate/up and IQ4_NL down tensors; the table
 // also lists moe_down_iq4xs, and both roles of both formats cost nothing more here.  The raw rows meet f32
 // activations as dot_iq4xs / dot_iq4nl do (crates/ojas-cpu/src/cpu_math.rs:943-967, :993-1010).
@@ -14,7 +14,7 @@
 // tokens (token t reads x + t K, idx + t KSEL, wgt + t KSEL and writes act + t KSEL N, y + t N), and a
 // trailing constant E, appended by the dispatcher from the extent of the expert tensors, bounds the routed
 // indices: a slot whose index is E or more contributes zeros instead of reading past the tensors.
-// Rows of the down launch are grid-stride (16 per workgroup and step), so the reference's ceil(N/8)
+// Rows of the down launch are grid-stride (4 per workgroup and step), so the reference's ceil(N/8)
 // workgroups are a valid grid.
 #include "ojk_common.h"
 #include "ojk_rows.h"
@@ -52,17 +52,21 @@ __device__ __forceinline__ void moe_gu_rows(const float* __restrict__ x, const u
     }
 }
 
+// A workgroup owns four rows at a time (rows grid-stride over the workgroups); its four waves take the slots
+// j = wave, wave + 4, ... and meet in LDS, where the partial sums are added in wave order onto y: an expert
+// row is short, so the slots are the parallelism that fills the chip at one token.
 template <class W>
 __device__ __forceinline__ void moe_down_rows(const float* __restrict__ act, const uchar* __restrict__ wd,
                                               float* __restrict__ y, const uint* __restrict__ idx,
                                               const float* __restrict__ wgt, uint K, uint N, uint KSEL, uint E) {
-    const uint lane = threadIdx.x & 63u;
+    __shared__ float part[4][4];
+    const uint lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint t = blockIdx.y;
     const uint nu = W::units(K);
     const size_t rb = (size_t)nu * W::BYTES;
-    for (uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 4u; row0 < N; row0 += gridDim.x * 16u) {
+    for (uint row0 = blockIdx.x * 4u; row0 < N; row0 += gridDim.x * 4u) {
         float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (uint j = 0; j < KSEL; j++) {
+        for (uint j = wave; j < KSEL; j += 4u) {
             const uint e = idx[t * KSEL + j];
             if (e >= E) continue;
             const float wj = wgt[t * KSEL + j];
@@ -83,9 +87,12 @@ __device__ __forceinline__ void moe_down_rows(const float* __restrict__ act, con
         }
         if (lane == 0) {
 #pragma unroll
-            for (int r = 0; r < 4; r++)
-                if (row0 + r < N) y[(size_t)t * N + row0 + r] += res[r];
+            for (int r = 0; r < 4; r++) part[wave][r] = res[r];
         }
+        __syncthreads();
+        if (threadIdx.x < 4u && row0 + threadIdx.x < N)
+            y[(size_t)t * N + row0 + threadIdx.x] += ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) + part[3][threadIdx.x];
+        __syncthreads();
     }
 }
 

@@ -714,10 +714,10 @@ uint64_t ojh_moe_mt_lds(uint32_t K) { return 16 * ((uint64_t)K + 32) + K / 4 + K
 //   8 moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)                      grid [ceil(N/8), NA, 1]
 //   9 moe_down_q4k_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)                  grid [ceil(N/8), T, 1]
 //  14 moe_gu_q80(x, wg, wu, act, idx, K, N)                                     grid [ceil(N/8), KSEL, tokens]
-//  15 moe_down_q80(act, wd, y, idx, wgt, K, N, KSEL)                            grid [1 .. ceil(N/8), tokens, 1]
+//  15 moe_down_q80(act, wd, y, idx, wgt, K, N, KSEL)                            grid [1 .. ceil(N/4), tokens, 1]
 //  14 / 15 also moe_{gu,down}_{iq4xs,iq4nl} of family "moe_iq", the same arguments
 //  16 moe_gu_q80_slots(x, arena_g, arena_u, act, off_g, off_u, K, N)             grid [ceil(N/8), KSEL, tokens]
-//  17 moe_down_q80_slots(act, arena, y, off_d, wgt, K, N, KSEL)                  grid [1 .. ceil(N/8), tokens, 1]
+//  17 moe_down_q80_slots(act, arena, y, off_d, wgt, K, N, KSEL)                  grid [1 .. ceil(N/4), tokens, 1]
 //     (the reference's Q8_0 expert kernels; the expert count is not an argument, so the weight buffers are
 //     checked for one expert only)
 //  10 moe_gu_q4k_slots, 11 moe_down_q4k_slots: 8 and 9 with a u64 byte offset per assignment into an arena
@@ -833,12 +833,12 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         align[1] = align[2] = ojh_block_align(f);
         return OJH_OK;
     }
-    case 15: {  // moe_down_{q80,iq4xs,iq4nl}(act, wd, y, idx, wgt, K, N, KSEL): rows grid-stride, 16 per workgroup
+    case 15: {  // moe_down_{q80,iq4xs,iq4nl}(act, wd, y, idx, wgt, K, N, KSEL): rows grid-stride, 4 per workgroup
         uint32_t K = c[0], N = c[1], KS = c[2], T = grid[1];
         const ojh_block_format *f = ojh_format(s->type);
         if ((rc = check_block(block, 256))) return rc;
         if (!K || K % f->weights || !N || !KS || !T) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u KSEL=%u tokens=%u", s->name, K, N, KS, T);
-        if (!grid[0] || grid[0] > (N + 7) / 8 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N/8), tokens, 1]", s->name);
+        if (!grid[0] || grid[0] > (N + 3) / 4 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N/4), tokens, 1]", s->name);
         need[0] = (size_t)T * KS * K * 4;
         need[1] = (size_t)N * (K / f->weights) * f->bytes;
         need[2] = (size_t)T * N * 4;
@@ -864,7 +864,7 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         uint32_t K = c[0], N = c[1], KS = c[2], T = grid[1];
         if ((rc = check_block(block, 256))) return rc;
         if (!K || K % 32 || !N || !KS || !T) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u KSEL=%u tokens=%u", s->name, K, N, KS, T);
-        if (!grid[0] || grid[0] > (N + 7) / 8 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N/8), tokens, 1]", s->name);
+        if (!grid[0] || grid[0] > (N + 3) / 4 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [1 .. ceil(N/4), tokens, 1]", s->name);
         need[0] = (size_t)T * KS * K * 4;
         need[1] = (size_t)N * (K / 32) * 34;
         need[2] = (size_t)T * N * 4;
@@ -945,7 +945,7 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K
     case 4: grid[0] = K <= 1024 ? (N + 31) / 32 : (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
     case 6: case 7: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;
     case 14: case 16: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = slots, one token
-    case 15: case 17: grid[0] = (N + 15) / 16; break;                         // one token
+    case 15: case 17: grid[0] = (N + 3) / 4; break;                           // one token
     case 12: case 13: grid[0] = ojh_moe_mt_groups(dev, N, M ? M : 1, s->rows_per_wave == 12 ? 1 : 2); grid[1] = M ? M : 1; block[0] = 512; break;  // M = experts
     case 8: case 10: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = assignments
     case 9: case 11: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = tokens

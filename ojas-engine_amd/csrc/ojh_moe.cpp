@@ -73,7 +73,7 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         if ((rc = ojh_launch(dev, gu_name.c_str(), {x->ptr, (char *)gate->raw->ptr + gate->off, (char *)up->raw->ptr + up->off, act8->ptr, idx->ptr},
                              {d, n_ff, E}, g1, b256)))
             return rc;
-        uint32_t g2[3] = {(d + 15) / 16, T, 1};
+        uint32_t g2[3] = {(d + 3) / 4, T, 1};
         return ojh_launch(dev, down_name.c_str(), {act8->ptr, (char *)down->raw->ptr + down->off, y->ptr, idx->ptr, wgt->ptr},
                           {n_ff, d, ksel, E}, g2, b256);
     }

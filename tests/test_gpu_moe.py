@@ -296,7 +296,7 @@ def test_q80_experts_reference_procedure(gpu, pkg):
     assert peak_err(got, want) <= 2e-6
     # the geometry the library itself names gives the same bits, and the down launch accumulates
     g2, b2 = gpu.launch_shape("moe_down_q80", n, k, 1)
-    assert g2 == [-(-k // 16), 1, 1] and b2 == [256, 1, 1]
+    assert g2 == [-(-k // 4), 1, 1] and b2 == [256, 1, 1]
     out2 = gpu.upload(np.ones(k, np.float32))
     gpu.dispatch(gpu.begin(), "moe_down_q80", [(actd, 0), (dd, 0), (out2, 0), (idxd, 0), (wgtd, 0)], [n, k, ksel], g2, b2)
     assert np.array_equal(gpu.read(out2, k), np.float32(1.0) + got)
