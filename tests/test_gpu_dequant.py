@@ -1,4 +1,7 @@
 """Device decoders against the CPU oracle: dequantized weights must be bit-exact."""
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -6,8 +9,11 @@ pytestmark = pytest.mark.gpu
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 Q2_K, Q3_K = 10, 11
-DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6,
-           IQ4_NL: 0xA5D4CF4E5DB3A1BF, IQ4_XS: 0x1429CAFB4DF9AF64, Q2_K: 0xBDA788876D584945, Q3_K: 0xA3FCFCD97CE8A0A9}
+# the reference's own regression digests, kept as a fixture (tests/golden/quant_format_digests.json)
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "quant_format_digests.json")) as _f:
+    _GOLDEN = json.load(_f)["digests"]
+DIGESTS = {int(ty): int(row["digest"], 16) for ty, row in _GOLDEN.items()}
+COUNTS = {int(ty): row["values"] for ty, row in _GOLDEN.items()}
 
 
 def _dequant(gpu, ty, raw, n):

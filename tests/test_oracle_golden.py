@@ -1,5 +1,8 @@
 """Pins the CPU oracle: golden vectors the reference's own tests hold, closed forms, invariants and
 brute force — each chosen so that a dropped term, a wrong index or a transposed nibble fails."""
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -7,9 +10,11 @@ Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 Q2_K, Q3_K = 10, 11
 
-# crates/ojas-formats/tests/quant_formats.rs:38-40, 45, 48
-DIGESTS = {Q4_K: 0x6536B83E8B2292B4, Q5_K: 0x361CBD8F84E79ADE, Q6_K: 0x38ECABE858257DB6,
-           IQ4_NL: 0xA5D4CF4E5DB3A1BF, IQ4_XS: 0x1429CAFB4DF9AF64, Q2_K: 0xBDA788876D584945, Q3_K: 0xA3FCFCD97CE8A0A9}
+# the reference's own regression digests (crates/ojas-formats/tests/quant_formats.rs:36-48), kept as a fixture
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "quant_format_digests.json")) as _f:
+    _GOLDEN = json.load(_f)["digests"]
+DIGESTS = {int(ty): int(row["digest"], 16) for ty, row in _GOLDEN.items()}
+COUNTS = {int(ty): row["values"] for ty, row in _GOLDEN.items()}
 # crates/ojas-core/src/iq_tables.rs:881-884
 KVALUES_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float64)
 
@@ -19,7 +24,7 @@ def test_dequant_digest_matches_reference(orc, pkg, ty):
     wpb = pkg.synth.BLOCK_SHAPE[ty][1]
     raw = orc.synth_blocks(ty, 40)
     bits = orc.dequant_to_f16(raw, ty, 40 * wpb)
-    assert bits.size == 40 * wpb                      # 10240 values; 1280 for the 32-weight IQ4_NL block
+    assert bits.size == 40 * wpb == COUNTS[ty]        # 10240 values; 1280 for the 32-weight IQ4_NL block
     assert orc.digest_f16(bits) == DIGESTS[ty]
 
 
