@@ -186,6 +186,20 @@ size_t ojh_row_bytes(uint32_t ggml_type, uint32_t k); /* 0 for an unknown type /
 int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, const ojh_lin *w,
            ojh_buf *y, size_t y_off, const ojh_buf *bias, uint32_t m, int accum, int act_mode);
 
+/* `ojh_mm` with OJH_ACT_Q8K for callers that cannot allocate device memory — code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
+ * The int8 activations and their per-256 scales are staged in a static device array of
+ * `ojh_noalloc_scratch_bytes()` bytes (1 MiB of activations + their scales) that each GPU holds
+ * until the process ends, so the call allocates and frees nothing; the launches and results are
+ * those of `ojh_mm(..., OJH_ACT_Q8K)` bit for bit.  K-quant weights (Q4_K, Q5_K, Q6_K), f32 or bf16
+ * activations, m * K <= OJH_NOALLOC_MAX_ACT (OJH_ERR_BOUNDS beyond); the families "gemv_q8k" and
+ * "gemm_q8k" must already be loaded (OJH_ERR_NOT_LOADED otherwise: loading allocates).  Every
+ * handle on one GPU shares that GPU's array: calls that overlap on one GPU race. */
+#define OJH_NOALLOC_MAX_ACT (1u << 20)
+int ojh_mm_noalloc(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, const ojh_lin *w,
+                   ojh_buf *y, size_t y_off, const ojh_buf *bias, uint32_t m, int accum);
+size_t ojh_noalloc_scratch_bytes(void);
+
 /* The same product from activations that are already quantized (`ojh_quant_q8k`): one
  * quantization feeds every projection that reads the same vector (q/k/v, gate/up), the split the
  * reference's CUDA path makes between `quantize_q8_1` and `gemv_q80_dp4a`

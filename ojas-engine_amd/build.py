@@ -39,7 +39,7 @@ FAMILIES = {
     "rowq8": ("rowq8.hip", ["-ffp-contract=off"]),
 }
 
-HOST_SOURCES = ["ojh_runtime.cpp", "ojh_manifest.cpp", "ojh_ops.cpp", "ojh_moe.cpp", "ojh_gguf.cpp", "ojh_expert_cache.cpp"]
+HOST_SOURCES = ["ojh_runtime.cpp", "ojh_manifest.cpp", "ojh_ops.cpp", "ojh_moe.cpp", "ojh_gguf.cpp", "ojh_expert_cache.cpp", "ojh_noalloc.cpp"]
 
 
 def _newer(target: str, deps: list[str]) -> bool:

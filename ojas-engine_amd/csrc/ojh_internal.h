@@ -77,6 +77,7 @@ struct ojh_device {
     bool capturing = false;      // between ojh_capture_begin and ojh_capture_end
     bool capture_hip_graph = false;
     std::vector<ojh_command> recorded;
+    void *noalloc_scratch = nullptr;   // this GPU's copy of the static scratch array of ojh_mm_noalloc (ojh_noalloc.cpp)
 };
 
 // ---- errors ------------------------------------------------------------------------------------
@@ -130,6 +131,13 @@ const ojh_kernel_spec *ojh_find_kernel(const char *name);
 int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out);
 int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptrs,
                const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);
+// shared by ojh_mm / ojh_mm_q8k / ojh_mm_noalloc (ojh_ops.cpp)
+int ojh_mm_checks(const char *who, const ojh_lin *w, ojh_buf *y, size_t y_off, const ojh_buf *bias, uint32_t m, int accum,
+                  const ojh_block_format **fmt);
+int ojh_quant_q8k_launch(ojh_device *dev, const void *x, int x_dtype, uint32_t m, uint32_t k, void *q, void *scales);
+int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, const ojh_block_format *f, void *yp,
+                      const ojh_buf *bias, uint32_t m, int accum);
+int ojh_noalloc_setup(ojh_device *dev);   // resolves the static scratch array on the current GPU (ojh_noalloc.cpp)
 void ojh_gemm_q8k_tiles(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M, uint32_t *rw, uint32_t *rt);   // row tiles per workgroup / per wave of gemm_q8k_q4k_mf
 uint32_t ojh_moe_mt_groups(const ojh_device *dev, uint32_t N, uint32_t E, uint32_t per_cu);   // workgroups per expert of those entries
 uint64_t ojh_moe_mt_lds(uint32_t K);                // LDS bytes of moe_{gu,down}_q4k_mt (ojh_manifest.cpp)

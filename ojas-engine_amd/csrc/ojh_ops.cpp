@@ -112,7 +112,7 @@ extern "C" int ojh_relayout_q4k_q4l(ojh_device *dev, const ojh_buf *raw, size_t 
 }
 
 // ---- activation quantizer ----------------------------------------------------------------------
-static int quant_q8k_launch(ojh_device *dev, const void *x, int x_dtype, uint32_t m, uint32_t k, void *q,
+int ojh_quant_q8k_launch(ojh_device *dev, const void *x, int x_dtype, uint32_t m, uint32_t k, void *q,
                             void *scales) {
     const char *name = x_dtype == OJH_X_BF16 ? "quantize_q8k_bf16" : "quantize_q8k";
     uint32_t grid[3] = {(k + 255) / 256, m, 1}, block[3] = {256, 1, 1};
@@ -131,7 +131,7 @@ extern "C" int ojh_quant_q8k(ojh_device *dev, const ojh_buf *x, size_t x_off, in
     if ((rc = span_ok("quant_q8k: q", q, 0, (size_t)m * nsb * 256, 16))) return rc;
     if ((rc = span_ok("quant_q8k: scales", scales, 0, (size_t)m * nsb * 4, 4))) return rc;
     if ((rc = ensure(dev, "gemv_q8k"))) return rc;
-    return quant_q8k_launch(dev, at(x, x_off), x_dtype, m, k, q->ptr, scales->ptr);
+    return ojh_quant_q8k_launch(dev, at(x, x_off), x_dtype, m, k, q->ptr, scales->ptr);
 }
 
 // ---- mm ----------------------------------------------------------------------------------------
@@ -147,7 +147,7 @@ static int pick_rows(const ojh_device *dev, uint32_t n) {
 }
 
 // y (=,+=,+bias) quantized-x . W^T for K-quant weights: the matvec (m = 1) and its batched form.
-static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, const ojh_block_format *f, void *yp,
+int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, const ojh_block_format *f, void *yp,
                          const ojh_buf *bias, uint32_t m, int accum) {
     const uint32_t K = w->k, N = w->n;
     void *wp = at(w->raw, w->off);
@@ -262,7 +262,7 @@ static int mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, 
     return ojh_launch(dev, (base + "_m").c_str(), {xq, xs, wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, grid, block);
 }
 
-static int mm_common_checks(const char *who, const ojh_lin *w, ojh_buf *y, size_t y_off, const ojh_buf *bias,
+int ojh_mm_checks(const char *who, const ojh_lin *w, ojh_buf *y, size_t y_off, const ojh_buf *bias,
                             uint32_t m, int accum, const ojh_block_format **fmt) {
     if (!w) return ojh_fail(OJH_ERR_ARG, "%s: NULL weights", who);
     if (!m || m > 65535) return ojh_fail(OJH_ERR_ARG, "%s: m=%u out of range", who, m);
@@ -282,7 +282,7 @@ extern "C" int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xsc
                           size_t y_off, const ojh_buf *bias, uint32_t m, int accum) {
     if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_mm_q8k: NULL device");
     const ojh_block_format *f;
-    int rc = mm_common_checks("ojh_mm_q8k", w, y, y_off, bias, m, accum, &f);
+    int rc = ojh_mm_checks("ojh_mm_q8k", w, y, y_off, bias, m, accum, &f);
     if (rc) return rc;
     if (ojh_float_rows(w->type))
         return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm_q8k: %s rows take f32 activations, as their CPU dot does", f->tag);
@@ -290,7 +290,7 @@ extern "C" int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xsc
     if ((rc = span_ok("xq", xq, 0, (size_t)m * nsb * 256, 16))) return rc;
     if ((rc = span_ok("xscales", xscales, 0, (size_t)m * nsb * 4, 4))) return rc;
     if ((rc = ensure(dev, "gemv_q8k"))) return rc;
-    return mm_q8k_launch(dev, xq->ptr, xscales->ptr, w, f, at(y, y_off), bias, m, accum);
+    return ojh_mm_q8k_launch(dev, xq->ptr, xscales->ptr, w, f, at(y, y_off), bias, m, accum);
 }
 
 extern "C" int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, int count,
@@ -302,7 +302,7 @@ extern "C" int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_bu
     uint64_t total = 0;
     for (int i = 0; i < count; i++) {
         const ojh_block_format *fi;
-        if ((rc = mm_common_checks("ojh_mm_q8k_multi", ws[i], ys[i], y_offs ? y_offs[i] : 0, nullptr, 1, 0, &fi))) return rc;
+        if ((rc = ojh_mm_checks("ojh_mm_q8k_multi", ws[i], ys[i], y_offs ? y_offs[i] : 0, nullptr, 1, 0, &fi))) return rc;
         if (ojh_float_rows(ws[i]->type))
             return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm_q8k_multi: %s rows take f32 activations, as their CPU dot does", fi->tag);
         if (ws[i]->k != ws[0]->k)
@@ -318,7 +318,7 @@ extern "C" int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_bu
     if (!grouped || count == 1) {   // formats without a grouped entry: one launch per projection
         for (int i = 0; i < count; i++) {
             const ojh_block_format *fi = ojh_format(ws[i]->type);
-            if ((rc = mm_q8k_launch(dev, xq->ptr, xscales->ptr, ws[i], fi, at(ys[i], y_offs ? y_offs[i] : 0), nullptr, 1, 0)))
+            if ((rc = ojh_mm_q8k_launch(dev, xq->ptr, xscales->ptr, ws[i], fi, at(ys[i], y_offs ? y_offs[i] : 0), nullptr, 1, 0)))
                 return rc;
         }
         return OJH_OK;
@@ -346,7 +346,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
                       size_t y_off, const ojh_buf *bias, uint32_t m, int accum, int act_mode) {
     if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_mm: NULL device");
     const ojh_block_format *f;
-    int rc = mm_common_checks("ojh_mm", w, y, y_off, bias, m, accum, &f);
+    int rc = ojh_mm_checks("ojh_mm", w, y, y_off, bias, m, accum, &f);
     if (rc) return rc;
     if (x_dtype != OJH_X_F32 && x_dtype != OJH_X_BF16)
         return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: activations must be f32 or bf16");
@@ -432,8 +432,8 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         ojh_buf *xq, *xs;
         if ((rc = ojh_scratch_get(dev, "xq", (size_t)m * nsb * 256, &xq))) return rc;
         if ((rc = ojh_scratch_get(dev, "xs", (size_t)m * nsb * 4, &xs))) return rc;
-        if ((rc = quant_q8k_launch(dev, at(x, x_off), x_dtype, m, K, xq->ptr, xs->ptr))) return rc;
-        return mm_q8k_launch(dev, xq->ptr, xs->ptr, w, f, yp, bias, m, accum);
+        if ((rc = ojh_quant_q8k_launch(dev, at(x, x_off), x_dtype, m, K, xq->ptr, xs->ptr))) return rc;
+        return ojh_mm_q8k_launch(dev, xq->ptr, xs->ptr, w, f, yp, bias, m, accum);
     }
 
     // floating-point activations: the matvec kernels read f32

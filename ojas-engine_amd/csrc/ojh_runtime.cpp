@@ -89,6 +89,11 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_MOE_DEC_TOKENS")) d->moe_dec_tokens = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_FUSED_QUANT")) d->fused_quant = atoi(r) != 0;
     if (const char *r = getenv("OJAS_HIP_FQ_BLOCKS")) d->fq_blocks_per_cu = atoi(r) > 0 ? (uint32_t)atoi(r) : 8u;
+    int rc = ojh_noalloc_setup(d);
+    if (rc) {
+        ojh_close(d);
+        return rc;
+    }
     *out = d;
     return OJH_OK;
 }

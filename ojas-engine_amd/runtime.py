@@ -111,6 +111,8 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_lin_free": (i32, [vp, vp]),
         "ojh_row_bytes": (sz, [u32, u32]),
         "ojh_mm": (i32, [vp, vp, sz, i32, vp, vp, sz, vp, u32, i32, i32]),
+        "ojh_mm_noalloc": (i32, [vp, vp, sz, i32, vp, vp, sz, vp, u32, i32]),
+        "ojh_noalloc_scratch_bytes": (sz, []),
         "ojh_mm_q8k": (i32, [vp, vp, vp, vp, vp, sz, vp, u32, i32]),
         "ojh_mm_q8k_multi": (i32, [vp, vp, vp, i32, vp, vp, vp]),
         "ojh_gguf_open": (i32, [C.c_char_p, vp]),
@@ -525,6 +527,12 @@ class HipGpu:
            act_mode: int = ACT_AUTO, bias: Buf | None = None, x_off: int = 0, y_off: int = 0) -> None:
         self._check(self._L.ojh_mm(self._dev, x.handle, x_off, x_dtype, w.handle, y.handle, y_off,
                                    bias.handle if bias else None, m, int(accum), act_mode))
+
+    def mm_noalloc(self, x: Buf, w: Lin, y: Buf, m: int = 1, accum: bool = False, *, x_dtype: int = X_F32,
+                   bias: Buf | None = None, x_off: int = 0, y_off: int = 0) -> None:
+        """`mm` with ACT_Q8K through the entry that allocates nothing (activations staged in a static device array)."""
+        self._check(self._L.ojh_mm_noalloc(self._dev, x.handle, x_off, x_dtype, w.handle, y.handle, y_off,
+                                           bias.handle if bias else None, m, int(accum)))
 
     def mm_q8k(self, xq: Buf, xscales: Buf, w: Lin, y: Buf, m: int = 1, accum: bool = False, *,
                bias: Buf | None = None, y_off: int = 0) -> None:
