@@ -168,6 +168,26 @@ def main() -> int:
         us = _time(gpu, lambda i: gpu.dispatch(gpu.begin(), kname, [(cal_src, 0), (cal_dst, 0)], [cal_n16], cgrid, cblock), 5, 2)
         cal[kname] = {"bytes_moved": moved, "us": round(us, 1), "gbs": round(moved / us / 1e3, 1)}
     del cal_src, cal_dst
+    # ... and what the matrix pipe sustains on this part (it is power-limited: the figure depends on the operands):
+    # one workgroup of four waves per CU, 16 independent 32x32x16 f16 MFMAs per trip, operands constant / N(0,1),
+    # held in registers / read back from LDS per group of 16 as the prefill tile does / with the copies, LDS writes and
+    # vector-ALU work a dequantizing 256x256x64 tile step adds (the ceiling any such tile can reach on this part)
+    mf_iters = 1024
+    mgrid, mblock = gpu.launch_shape("calib_mfma_f16", 0, 0, 0)
+    mf_flops = mgrid[0] * 4 * mf_iters * 64 * 2 * 32 * 32 * 16
+    mf_out = gpu.alloc(mgrid[0] * 256)
+    n_ops = 8 * 256 * 8 + (4 << 20) // 2      # a workgroup's fragments, then the 4 MB window mode 2 copies from
+    ops_const = np.full(n_ops, 1.0, np.float16)
+    ops_rand = synth.normal_f32(n_ops, "bench", "mfma_calibration").astype(np.float16)
+    for tag, ops in (("constant", ops_const), ("normal", ops_rand)):
+        src = gpu.upload_bytes(ops)
+        for mode, where in ((0, "registers"), (1, "lds"), (2, "lds_tile_step_mix")):
+            us = _time(gpu, lambda i: gpu.dispatch(gpu.begin(), "calib_mfma_f16", [(src, 0), (mf_out, 0)], [mf_iters, mode],
+                                                    mgrid, mblock), 5, 2)
+            cal[f"mfma_f16_{tag}_{where}"] = {"flops": mf_flops, "us": round(us, 1), "tflops": round(mf_flops / us / 1e6, 1),
+                                              "mfma_frac": round(mf_flops / us / 1e6 / 2500.0, 4)}
+        del src
+    del mf_out
 
     # ---- per-shape latency (each shape alone, back to back, rotating sets), for the record.  The launches are
     # recorded once and replayed from the library, like the step: issued one by one from Python the short

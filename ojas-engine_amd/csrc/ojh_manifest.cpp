@@ -988,11 +988,33 @@ static int check_stream(const ojh_kernel_spec *s, const uint32_t *c, const uint3
     return OJH_OK;
 }
 
+// calib_mfma_f16(x, y, iters, mode): 32 KB of operands, one dword out per thread
+static int check_calib_mfma(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                            const uint32_t block[3], size_t need[16], size_t align[16]) {
+    (void)align;
+    if (!c[0] || c[0] > (1u << 20)) return ojh_fail(OJH_ERR_ARG, "%s: iters=%u out of range (1 .. 2^20)", s->name, c[0]);
+    if (c[1] > 2) return ojh_fail(OJH_ERR_ARG, "%s: mode=%u (0 = operands in registers, 1 = read from LDS, 2 = with a tile step's copies, LDS writes and vector ALU work)", s->name, c[1]);
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    need[0] = 8 * 256 * 16 + (c[1] == 2 ? (4u << 20) : 0u);
+    need[1] = (size_t)grid[0] * 256 * 4;
+    return OJH_OK;
+}
+
 // ---- launch shapes ---------------------------------------------------------------------------
 static int shape_elementwise(const ojh_kernel_spec *, const ojh_device *, uint32_t, uint32_t N, uint32_t,
                              uint32_t grid[3], uint32_t block[3]) {
     grid[0] = (N / 8 + 255) / 256;  // N = element count; a thread takes 8 elements per trip
     if (!grid[0]) grid[0] = 1;
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+static int shape_calib_mfma(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t, uint32_t,
+                            uint32_t grid[3], uint32_t block[3]) {
+    grid[0] = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;   // one workgroup of four waves per CU
     grid[1] = grid[2] = 1;
     block[0] = 256;
     block[1] = block[2] = 1;
@@ -1199,6 +1221,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("fill_zero_u32", "glue", 1, 1, 4u, 0, check_elementwise, shape_elementwise);
     add("stream_copy_u32x4", "glue", 2, 1, 0, 0, check_stream, shape_stream);
     add("stream_read_u32x4", "glue", 2, 1, 1, 0, check_stream, shape_stream);
+    add("calib_mfma_f16", "glue", 2, 2, 0, 0, check_calib_mfma, shape_calib_mfma);
     return m;
 }
 
