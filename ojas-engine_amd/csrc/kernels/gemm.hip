@@ -19,8 +19,8 @@
 // owns 128 x 64 of the tile as 4 x 2 blocks of v_mfma_f32_32x32x16_f16 (A = activations, B =
 // weights, so a D register holds 32 consecutive outputs of one token: coalesced stores).
 // With one wave per SIMD nothing else hides latency, so the step is a hand-built pipeline:
-//   * global loads run three steps ahead in registers, issued as opaque instructions so the
-//     compiler cannot sink them to their use, and awaited with an explicit s_waitcnt;
+//   * global loads run three steps ahead in registers: ordinary loads the compiler tracks itself, held in
+//     place by a scheduling fence so that they are not sunk to their use;
 //   * the dequantization of step t+1 (vector ALU) is interleaved with the MFMAs of step t
 //     (sched_group_barrier), its LDS writes go to the other stage, one barrier per step.
 #include "ojk_common.h"
@@ -46,35 +46,18 @@ __device__ __forceinline__ uint pack2(float a, float b) {
     return __builtin_bit_cast(uint, __builtin_convertvector(f, half2v));
 }
 
-// ---- global loads whose issue point the compiler may not move -----------------------------------
-// The compiler sinks ordinary loads down to their first use to save registers, which turns a
-// three-steps-ahead prefetch into load-then-wait.  These loads are opaque to it: they are issued
-// where they are written, and the consumer waits with an explicit s_waitcnt (gm_wait) that also
-// re-defines the destination registers, so nothing that reads them can be scheduled above it.
-// Vector memory operations retire in order, so "at most n outstanding" means every load issued
-// before the last n has landed.
+// ---- global loads --------------------------------------------------------------------------------
+// Ordinary loads: the compiler sees every one of them, counts them in its own s_waitcnt and never reads a
+// destination register before its load has landed.  What keeps a prefetch three steps ahead of its use is the
+// scheduling fence behind each group of loads (gm_fence): the scheduler may not sink them past it.
 __device__ __forceinline__ u32x4 gm_load16(const void* p) {
-    u32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-    return v;
+    // (blocks of 34 and 210 bytes are only 2-byte aligned; the target runs in unaligned-access mode)
+    typedef u32x4 __attribute__((aligned(2))) u32x4_u;
+    return *(const u32x4_u*)p;
 }
-__device__ __forceinline__ uint gm_load_u16(const void* p) {
-    uint v;
-    asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-    return v;
-}
-__device__ __forceinline__ uint gm_load_u8(const void* p) {
-    uint v;
-    asm volatile("global_load_ubyte %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-    return v;
-}
-template <int N>
-__device__ __forceinline__ void gm_wait(u32x4 (&x)[8]) {
-    asm volatile("s_waitcnt vmcnt(%8)"
-                 : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])
-                 : "n"(N)
-                 : "memory");
-}
+__device__ __forceinline__ uint gm_load_u16(const void* p) { return *(const ushort*)p; }
+__device__ __forceinline__ uint gm_load_u8(const void* p) { return *(const uchar*)p; }
+__device__ __forceinline__ void gm_fence() { __builtin_amdgcn_sched_barrier(0); }
 
 // ------------------------------------------------------------------ per-format slab loaders
 // A loader owns, for one thread, 32 weights of one row of the 128 x 64 slab: thread t -> row
@@ -88,7 +71,6 @@ struct LoaderQ4K {
     float dl1, ml1, dl2, ml2;
     uint lo[8], hi[8];
     static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * Q4K_BYTES; }
-    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(hdr), "+v"(qs)::"memory"); }
     __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
         const uchar* blk = row + (size_t)(k0 >> 8) * Q4K_BYTES;
         c = (k0 >> 6) & 3u;  // 32-byte chunk of the super-block = sub-blocks 2c, 2c+1
@@ -135,9 +117,6 @@ struct LoaderQ6K {
     float s0, s1;
     uint o0[8], o1[8];
     static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * Q6K_BYTES; }
-    __device__ __forceinline__ void pin() {
-        asm volatile("" : "+v"(qa), "+v"(qb), "+v"(qh), "+v"(sca), "+v"(scb), "+v"(d16)::"memory");
-    }
     __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
         const uchar* blk = row + (size_t)(k0 >> 8) * Q6K_BYTES;
         uint j = (k0 >> 6) & 3u, hf = j >> 1;
@@ -190,7 +169,6 @@ struct LoaderQ80 {
     float d;
     uint o[16];
     static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 5) * Q80_BYTES; }
-    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(qa), "+v"(qb), "+v"(d16)::"memory"); }
     __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
         const uchar* blk = row + (size_t)((k0 >> 5) + h) * Q80_BYTES;
         d16 = gm_load_u16(blk);
@@ -257,21 +235,13 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
     u32x4 xs0[8], xs1[8], xs2[8];
     Loader ld0, ld1, ld2;
     const uint nt = (k_end - k_begin) / GM_BK;
-    constexpr int LPS = 8 + Loader::NL;  // loads per slab
 
 #define GM_LOAD(XS, LD, T)                                                                       \
     do {                                                                                         \
         const uint kk_ = k_begin + (T) * GM_BK;                                                  \
         _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++) XS[i_] = gm_load16(xrow[i_] + kk_);      \
         LD.load(wrow, kk_, wh);                                                                  \
-    } while (0)
-// wait for the slab of step T: the slabs of steps T+1 and T+2, where they exist, were issued later
-#define GM_WAIT_FOR(XS, LD, T)                                                                   \
-    do {                                                                                         \
-        if ((T) + 2u < nt) gm_wait<2 * LPS>(XS);                                                 \
-        else if ((T) + 1u < nt) gm_wait<LPS>(XS);                                                \
-        else gm_wait<0>(XS);                                                                     \
-        LD.pin();                                                                                \
+        gm_fence();                                                                              \
     } while (0)
 #define GM_STORE_X(XS, STG)                                                                      \
     do {                                                                                         \
@@ -317,8 +287,6 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
         half8 afA[4], bfA[2], afB[4], bfB[2];                                                    \
         GM_READ(cur_, 0, afA, bfA);                                                              \
         GM_LOAD(XS_FREE, LD_FREE, (T) + 3u);                                                     \
-        gm_wait<2 * LPS>(XS_NEXT);                                                               \
-        LD_NEXT.pin();                                                                           \
         LD_NEXT.prep();                                                                          \
         GM_READ(cur_, 1, afB, bfB); GM_MMA(afA, bfA); LD_NEXT.template part<0>(); GM_MIX();      \
         GM_READ(cur_, 2, afA, bfA); GM_MMA(afB, bfB); LD_NEXT.template part<1>(); GM_MIX();      \
@@ -335,7 +303,6 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
         const uint cur_ = (T) & 1u, nxt_ = cur_ ^ 1u;                                            \
         GM_MFMA(cur_, 0); GM_MFMA(cur_, 1); GM_MFMA(cur_, 2); GM_MFMA(cur_, 3);                  \
         if ((T) + 1u < nt) {                                                                     \
-            GM_WAIT_FOR(XS_NEXT, LD_NEXT, (T) + 1u);                                             \
             LD_NEXT.prep();                                                                      \
             LD_NEXT.template part<0>(); LD_NEXT.template part<1>();                              \
             LD_NEXT.template part<2>(); LD_NEXT.template part<3>();                              \
@@ -348,7 +315,6 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
     GM_LOAD(xs0, ld0, 0u);
     if (nt > 1u) GM_LOAD(xs1, ld1, 1u);
     if (nt > 2u) GM_LOAD(xs2, ld2, 2u);
-    GM_WAIT_FOR(xs0, ld0, 0u);
     ld0.prep();
     ld0.template part<0>(); ld0.template part<1>(); ld0.template part<2>(); ld0.template part<3>();
     GM_STORE_X(xs0, 0u);
@@ -367,7 +333,6 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
         if (t + 2u < nt) GM_STEP_ANY(t + 2u, xs2, ld2, xs0, ld0);
     }
 #undef GM_LOAD
-#undef GM_WAIT_FOR
 #undef GM_STORE_X
 #undef GM_MFMA
 #undef GM_READ
