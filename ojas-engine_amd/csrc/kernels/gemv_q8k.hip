@@ -42,7 +42,7 @@ __device__ __forceinline__ void quantize_q8k_body(const void* __restrict__ xv, s
     float scale = mx > 0.0f ? __fdiv_rn(mx, 127.0f) : 1.0f;
     float inv = __fdiv_rn(1.0f, scale);
     float r = roundf(__fmul_rn(v, inv));
-    r = fminf(fmaxf(r, -127.0f), 127.0f);
+    r = sat127(r);
     // the padded tail of a ragged last segment is written as zero
     q[((size_t)m * nsb + sb) * 256u + tid] = (signed char)(int)r;
     if (tid == 0) scales[(size_t)m * nsb + sb] = scale;
@@ -411,7 +411,7 @@ rmsnorm_q8k(const float* __restrict__ x, const float* __restrict__ gamma, signed
         uint packed = 0;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const int qi = (int)fminf(fmaxf(roundf(__fmul_rn(t[e], is)), -127.0f), 127.0f);
+            const int qi = (int)sat127(roundf(__fmul_rn(t[e], is)));
             packed |= (uint)(qi & 0xFF) << (8 * e);
             if (WRITE_XN && i0 + e < K) xn[(size_t)m * K + i0 + e] = t[e];
         }
@@ -459,10 +459,10 @@ __device__ __forceinline__ void gemv_fq8k_q4k_body(const float* __restrict__ x, 
         float a = wave_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
         float scale = a > 0.0f ? __fdiv_rn(a, 127.0f) : 1.0f;
         float inv = __fdiv_rn(1.0f, scale);
-        int q0 = (int)fminf(fmaxf(roundf(__fmul_rn(v.x, inv)), -127.0f), 127.0f);
-        int q1 = (int)fminf(fmaxf(roundf(__fmul_rn(v.y, inv)), -127.0f), 127.0f);
-        int q2 = (int)fminf(fmaxf(roundf(__fmul_rn(v.z, inv)), -127.0f), 127.0f);
-        int q3 = (int)fminf(fmaxf(roundf(__fmul_rn(v.w, inv)), -127.0f), 127.0f);
+        int q0 = (int)sat127(roundf(__fmul_rn(v.x, inv)));
+        int q1 = (int)sat127(roundf(__fmul_rn(v.y, inv)));
+        int q2 = (int)sat127(roundf(__fmul_rn(v.z, inv)));
+        int q3 = (int)sat127(roundf(__fmul_rn(v.w, inv)));
         *(uint*)(sx + seg * FQ_SEG + lane * 4u) =
             (uint)(q0 & 0xFF) | ((uint)(q1 & 0xFF) << 8) | ((uint)(q2 & 0xFF) << 16) | ((uint)(q3 & 0xFF) << 24);
         if (lane == 0) ss[seg] = scale;

@@ -101,6 +101,13 @@ __device__ __forceinline__ float wave_sum(float v) {
     float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
     return (a + b) + (c + d);
 }
+// Saturation of a rounded activation to the int8 range as the reference's quantizers do it,
+// `.round().clamp(-127.0, 127.0) as i8` (crates/ojas-cpu/src/cpu_math.rs:174-179, :545-563): a NaN passes through
+// clamp and becomes 0 in the cast (fmaxf alone would turn it into -127).
+__device__ __forceinline__ float sat127(float r) {
+    const float c = fminf(fmaxf(r, -127.0f), 127.0f);
+    return r == r ? c : 0.0f;
+}
 __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, dpp_f32<OJK_DPP_QUAD_XOR1>(v));
     v = fmaxf(v, dpp_f32<OJK_DPP_QUAD_XOR2>(v));

@@ -39,10 +39,10 @@ __device__ __forceinline__ Q4kFrag q4k_load_frag(const signed char* xq, const fl
 // maximum over the group and nothing outside registers.  Same operations as the quantize_q8k
 // kernel, hence the same bytes.
 __device__ __forceinline__ uint q8k_pack4(float4 v, float inv) {
-    float a = fminf(fmaxf(roundf(__fmul_rn(v.x, inv)), -127.0f), 127.0f);
-    float b = fminf(fmaxf(roundf(__fmul_rn(v.y, inv)), -127.0f), 127.0f);
-    float c = fminf(fmaxf(roundf(__fmul_rn(v.z, inv)), -127.0f), 127.0f);
-    float d = fminf(fmaxf(roundf(__fmul_rn(v.w, inv)), -127.0f), 127.0f);
+    float a = sat127(roundf(__fmul_rn(v.x, inv)));
+    float b = sat127(roundf(__fmul_rn(v.y, inv)));
+    float c = sat127(roundf(__fmul_rn(v.z, inv)));
+    float d = sat127(roundf(__fmul_rn(v.w, inv)));
     return ((uint)(int)a & 0xFFu) | (((uint)(int)b & 0xFFu) << 8) | (((uint)(int)c & 0xFFu) << 16) | ((uint)(int)d << 24);
 }
 

@@ -34,7 +34,7 @@ rows_q8_from_f16(const ushort* __restrict__ w16, signed char* __restrict__ q, fl
     if (tid == 0) scale[r] = sv;
     for (uint c = tid; c < K; c += 256u) {
         float v = roundf(__fdiv_rn(f16_bits_to_f32(row[c]), sv));
-        q[(size_t)r * K + c] = (signed char)(int)fminf(fmaxf(v, -127.0f), 127.0f);
+        q[(size_t)r * K + c] = (signed char)(int)sat127(v);
     }
 }
 
@@ -51,7 +51,7 @@ quant_rows_i8(const float* __restrict__ x, signed char* __restrict__ q, float* _
     if (tid == 0) scale[r] = s;
     for (uint c = tid; c < K; c += 256u) {
         float v = roundf(__fmul_rn(row[c], inv));
-        q[(size_t)r * K + c] = (signed char)(int)fminf(fmaxf(v, -127.0f), 127.0f);
+        q[(size_t)r * K + c] = (signed char)(int)sat127(v);
     }
 }
 

@@ -456,6 +456,9 @@ uint64_t ojo_digest_f16(const uint16_t *v, size_t n) { /* quant_formats.rs:20-31
 /* ---------------------------------------------------------------- activations */
 
 static inline float clampf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
+/* `x.round().clamp(-127.0, 127.0) as i8`: clamp passes a NaN through and Rust's float-to-int cast maps NaN to 0
+ * (in C that cast is undefined, so the case is spelled out). */
+static inline int8_t sat_i8(float r) { return r != r ? (int8_t)0 : (int8_t)clampf(r, -127.0f, 127.0f); }
 
 void ojo_quant_q8k(const float *x, size_t k, float *scales, int8_t *q, int32_t *bsums) {
     /* cpu_math.rs:545-563. f32::round is round-half-away-from-zero == roundf. */
@@ -470,7 +473,7 @@ void ojo_quant_q8k(const float *x, size_t k, float *scales, int8_t *q, int32_t *
         float inv = 1.0f / scale;
         scales[sb] = scale;
         for (size_t i = lo; i < hi; i++) {
-            int8_t qi = (int8_t)clampf(roundf(x[i] * inv), -127.0f, 127.0f);
+            int8_t qi = sat_i8(roundf(x[i] * inv));
             q[i] = qi;
             bsums[sb * 8 + (i - lo) / 32] += qi;
         }
@@ -482,7 +485,7 @@ float ojo_quant_row_i8(const float *row, size_t k, int8_t *q) { /* cpu_math.rs:1
     for (size_t i = 0; i < k; i++) { float a = fabsf(row[i]); if (a > m) m = a; }
     float scale = m > 0.0f ? m / 127.0f : 1.0f;
     float inv = 1.0f / scale;
-    for (size_t i = 0; i < k; i++) q[i] = (int8_t)clampf(roundf(row[i] * inv), -127.0f, 127.0f);
+    for (size_t i = 0; i < k; i++) q[i] = sat_i8(roundf(row[i] * inv));
     return scale;
 }
 
@@ -750,7 +753,7 @@ void ojo_q8_rows_from_f16(const uint16_t *w16, size_t n, size_t k, int8_t *q, fl
         float sv = amax > 0.0f ? amax / 127.0f : 1.0f;
         scale[r] = sv;
         for (size_t c = 0; c < k; c++)
-            q[r * k + c] = (int8_t)clampf(roundf(ojo_f16_to_f32(w16[r * k + c]) / sv), -127.0f, 127.0f);
+            q[r * k + c] = sat_i8(roundf(ojo_f16_to_f32(w16[r * k + c]) / sv));
     }
 }
 

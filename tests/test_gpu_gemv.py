@@ -31,6 +31,8 @@ def test_quantize_q8k_is_bit_exact(gpu, orc, pkg):
         x[0, :7] = [0.5, -0.5, 1.5, -2.5, 0.0, 1e-30, -1e-30]
         if k >= 512:
             x[-1, 256:512] = 0.0
+        if k >= 4096:     # non-finite inputs: NaN -> code 0 and outside the maximum; an infinity zeroes its segment's codes
+            x[0, 1000], x[0, 2000], x[0, 2001] = np.nan, np.inf, -np.inf
         nsb = (k + 255) // 256
         xd = gpu.upload(x)
         q, s = gpu.alloc_bytes(m * nsb * 256), gpu.alloc(m * nsb)

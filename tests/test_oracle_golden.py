@@ -160,6 +160,16 @@ def test_quant_q8k_invariants(orc):
     s, q, b = orc.quant_q8k(x)
     assert s.size == 2 and q.size == 512 and not q[300:].any()
     assert s[1] == np.float32(np.max(np.abs(x[256:]))) / np.float32(127.0)
+    # non-finite inputs, as Rust's `fold(max)`, `clamp` and `as i8` treat them (cpu_math.rs:552-557): a NaN does not
+    # enter the maximum and quantizes to 0; an infinity makes the scale infinite, 1/scale zero, and every code of its
+    # segment 0 (finite * 0 = 0, inf * 0 = NaN -> 0)
+    x = rng.standard_normal(512).astype(np.float32)
+    x[5], x[300], x[301] = np.nan, np.inf, -np.inf
+    s, q, b = orc.quant_q8k(x)
+    finite = np.delete(x[:256], 5)
+    assert s[0] == np.float32(np.max(np.abs(finite))) / np.float32(127.0) and q[5] == 0
+    assert np.max(np.abs(q[:256])) == 127
+    assert np.isinf(s[1]) and not q[256:].any() and not b[8:].any()
 
 
 def test_dot_q80_matches_f64_dot(orc, pkg):
