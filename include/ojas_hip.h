@@ -152,7 +152,15 @@ int ojh_submit(ojh_device *dev);
  * submit, a scratch buffer that has to grow) fail with OJH_ERR_ARG — run the chain once eagerly
  * first.  `ojh_graph_launch` replays the chain on the device's stream with one host call: by
  * default from a native loop over the recorded launches, or as an instantiated hipGraph when
- * OJAS_HIP_REPLAY=graph is set in the environment at `ojh_capture_begin`. */
+ * OJAS_HIP_REPLAY=graph is set in the environment at `ojh_capture_begin`.
+ * A chain keeps the device addresses it was recorded with, including those of the library's own
+ * scratch buffers (ojh_mm, ojh_matmul_q8, ojh_moe_ffn stage activations there).  While any chain of
+ * a device is alive, a scratch buffer that a later eager call outgrows is kept (parked) rather than
+ * freed, so replays stay valid; the parked memory is released when the last chain is freed.  Buffers
+ * the caller passed in must outlive the chain, as with any recorded pointer.
+ * If a call fails between begin and end, call `ojh_capture_end` all the same: it ends the recording
+ * (its own result may be an error in hipGraph mode, where a failed HIP call invalidates the capture)
+ * and the device runs eagerly again. */
 int ojh_capture_begin(ojh_device *dev);
 int ojh_capture_end(ojh_device *dev, ojh_graph **out);
 int ojh_graph_launch(ojh_device *dev, ojh_graph *graph);
@@ -275,7 +283,9 @@ int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uin
  * whole blocks of the formats.
  * Expert indices must be below n_expert (one that is not never reads outside the tensors; what
  * it contributes is unspecified). Up to 8 tokens run as two launches addressed
- * by assignment (bit-identical to the grouped integer-dot pipeline); larger batches are grouped
+ * by assignment (bit-identical to the grouped integer-dot pipeline) when d <= 8192, n_ff <= 2048,
+ * ksel <= 64 and ksel * n_ff <= 32768 (beyond that the grouped pipeline serves them; forcing the
+ * two-launch form with OJAS_HIP_MOE=3 then returns OJH_ERR_UNSUPPORTED); larger batches are grouped
  * by expert, on int8 MFMA from three to four assignments per expert (sums associate differently there:
  * last ulps). Environment: OJAS_HIP_MOE = 1 / 2 / 3 forces MFMA / grouped dots / the decode
  * form, OJAS_HIP_MOE_DEC_TOKENS moves the 8. */

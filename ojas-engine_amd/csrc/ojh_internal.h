@@ -77,6 +77,10 @@ struct ojh_device {
     bool capturing = false;      // between ojh_capture_begin and ojh_capture_end
     bool capture_hip_graph = false;
     std::vector<ojh_command> recorded;
+    // Recorded chains hold raw pointers into the scratch buffers.  While any chain of this device is alive, a scratch
+    // buffer that has to grow is parked here instead of freed, and released when the last chain is.
+    int live_graphs = 0;
+    std::vector<ojh_buf *> parked;
     void *noalloc_scratch = nullptr;   // this GPU's copy of the static scratch array of ojh_mm_noalloc (ojh_noalloc.cpp)
 };
 

@@ -66,6 +66,7 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         uint32_t b256[3] = {256, 1, 1};
         if (!accum) {
             if ((rc = ensure(dev, "glue"))) return rc;
+            if ((uint64_t)T * d > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "moe_ffn: %u tokens of %u outputs exceed 2^32 elements", T, d);
             uint32_t n_y = T * d, zg[3] = {(n_y / 4 + 255) / 256 + 1, 1, 1};
             if ((rc = ojh_launch(dev, "fill_zero_u32", {y->ptr}, {n_y}, zg, b256))) return rc;
         }
@@ -102,10 +103,11 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     // A few tokens: two launches addressed by assignment, activations quantized in registers,
     // weighted sum inside the down launch (bit-identical to the grouped integer-dot pipeline).
     // Measured on MI355X the grouped pipeline takes over once tokens start sharing experts.
-    const bool dec_fits = d <= 8192 && n_ff <= 2048 && (uint64_t)ksel * n_ff <= 32768;   // what the two launches stage in LDS
+    // what the two launches stage in LDS; the down launch keeps one partial sum per slot and lane group for up to 64 slots
+    const bool dec_fits = d <= 8192 && n_ff <= 2048 && ksel <= 64 && (uint64_t)ksel * n_ff <= 32768;
     if (dev->moe_mode == 3 || (dev->moe_mode == 0 && T <= dev->moe_dec_tokens && dec_fits)) {
         if (!dec_fits)
-            return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: the decode form serves d <= 8192, n_ff <= 2048 and ksel * n_ff <= 32768");
+            return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: the decode form serves d <= 8192, n_ff <= 2048, ksel <= 64 and ksel * n_ff <= 32768");
         ojh_buf *act;
         if ((rc = ojh_scratch_get(dev, "moe_act", (size_t)NA * n_ff * 4, &act))) return rc;
         uint32_t g1[3] = {(n_ff + 7) / 8, NA, 1};

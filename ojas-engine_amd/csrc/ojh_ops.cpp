@@ -441,6 +441,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     if (x_dtype == OJH_X_BF16) {
         if ((rc = ensure(dev, "glue"))) return rc;
         ojh_buf *xf;
+        if ((uint64_t)m * K > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "ojh_mm: %u x %u bf16 activations exceed 2^32 elements", m, K);
         if ((rc = ojh_scratch_get(dev, "xf", (size_t)m * K * 4, &xf))) return rc;
         uint32_t n_el = m * K, eg[3] = {(n_el / 8 + 255) / 256 + 1, 1, 1};
         if ((rc = ojh_launch(dev, "copy_bf16_f32", {xp, xf->ptr}, {n_el}, eg, block))) return rc;

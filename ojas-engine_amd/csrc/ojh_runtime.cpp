@@ -108,6 +108,10 @@ extern "C" int ojh_close(ojh_device *dev) {
             delete kv.second;
         }
     }
+    for (ojh_buf *b : dev->parked) {
+        if (b->owned) hipFree(b->ptr);
+        delete b;
+    }
     for (auto &kv : dev->modules) hipModuleUnload(kv.second);
     for (auto e : dev->marks)
         if (e) hipEventDestroy(e);
@@ -225,7 +229,10 @@ int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **o
         if (dev->capturing)
             return ojh_fail(OJH_ERR_ARG, "scratch '%s' would have to grow while recording a graph: run the call once "
                                           "eagerly first", name);
-        if (slot) {
+        if (slot && dev->live_graphs > 0) {   // a recorded chain may still replay into it
+            dev->parked.push_back(slot);
+            slot = nullptr;
+        } else if (slot) {
             int rc = ojh_free(dev, slot);
             slot = nullptr;
             if (rc) return rc;
@@ -426,14 +433,17 @@ extern "C" int ojh_capture_end(ojh_device *dev, ojh_graph **out) {
         hipError_t e = hipStreamEndCapture(dev->stream, &g);
         if (e == hipSuccess) e = hipGraphInstantiate(&gr->exec, g, nullptr, nullptr, 0);
         if (e != hipSuccess) {
+            // the capture has ended either way (an invalidated one too): the stream runs eagerly again
             if (g) hipGraphDestroy(g);
             delete gr;
+            (void)hipGetLastError();
             return ojh_fail(OJH_ERR_HIP, "graph capture/instantiate: %s", hipGetErrorString(e));
         }
         gr->graph = g;
     } else {
         gr->list.swap(dev->recorded);
     }
+    dev->live_graphs++;
     *out = gr;
     return OJH_OK;
 }
@@ -462,5 +472,12 @@ extern "C" int ojh_graph_free(ojh_device *dev, ojh_graph *graph) {
     if (graph->exec) hipGraphExecDestroy(graph->exec);
     if (graph->graph) hipGraphDestroy(graph->graph);
     delete graph;
+    if (dev && dev->live_graphs > 0 && --dev->live_graphs == 0) {   // nothing can replay into the outgrown buffers any more
+        for (ojh_buf *b : dev->parked) {
+            if (b->owned) hipFree(b->ptr);
+            delete b;
+        }
+        dev->parked.clear();
+    }
     return OJH_OK;
 }
