@@ -280,7 +280,10 @@ int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uin
  * dot_iq4xs / dot_iq4nl do (crates/ojas-cpu/src/cpu_math.rs:943-1010) through the reference's own expert
  * kernels moe_gu_<fmt> / moe_down_<fmt> (crates/ojas-cuda/src/kernels/moe.rs:75-125, moe_iq.rs:64-112),
  * one launch each over all tokens; there act_mode is OJH_ACT_AUTO or OJH_ACT_FLOAT and d, n_ff are
- * whole blocks of the formats.
+ * whole blocks of the formats.  K-quant experts take the same two launches under OJH_ACT_FLOAT
+ * (`moe_gu_q4k`, `moe_down_{q4k,q5k,q6k}`: f32 activations against the dequantized weights, the
+ * reference's GPU expert kernels for those formats, crates/ojas-core/src/quant_src.rs:174-179);
+ * OJH_ACT_AUTO and OJH_ACT_Q8K keep the CPU path's int8-activation arithmetic for them.
  * Expert indices must be below n_expert (one that is not never reads outside the tensors; what
  * it contributes is unspecified). Up to 8 tokens run as two launches addressed
  * by assignment (bit-identical to the grouped integer-dot pipeline) when d <= 8192, n_ff <= 2048,

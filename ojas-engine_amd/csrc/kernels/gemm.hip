@@ -58,14 +58,30 @@ __device__ __forceinline__ u32x4 gm_load16(const void* p) {
 __device__ __forceinline__ uint gm_load_u16(const void* p) { return *(const ushort*)p; }
 __device__ __forceinline__ uint gm_load_u8(const void* p) { return *(const uchar*)p; }
 __device__ __forceinline__ void gm_fence() { __builtin_amdgcn_sched_barrier(0); }
+// 8 activations at element offset `at` as f16: loaded as such, or converted from f32 (round to nearest even)
+template <bool XF32>
+__device__ __forceinline__ u32x4 gm_load_x(const ushort* xh, const float* xf, size_t at) {
+    if (!XF32) return *(const u32x4*)(xh + at);
+    const float4 a = *(const float4*)(xf + at), b = *(const float4*)(xf + at + 4);
+    return (u32x4){pack2(a.x, a.y), pack2(a.z, a.w), pack2(b.x, b.y), pack2(b.z, b.w)};
+}
 
 // ------------------------------------------------------------------ per-format slab loaders
 // A loader owns, for one thread, 32 weights of one row of the 128 x 64 slab: thread t -> row
 // t/2, half h = t%2.  `load` issues the global loads (NL of them); after the wait, `prep` unpacks
 // the scales, `part<I>` dequantizes a quarter of the weights (so the work can be spread between
 // MFMAs), `flush` writes the 32 f16 to the LDS row.
+// What a kernel passes for its weights: the block bytes, plus the side arrays of the formats that have them.
+struct GmSrc {
+    const uchar* w;
+    const ushort* qa;
+    const ushort* qb;
+};
+
 struct LoaderQ4K {
     static constexpr int NL = 2;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
     u32x4 hdr, qs;
     uint c;
     float dl1, ml1, dl2, ml2;
@@ -112,6 +128,8 @@ struct LoaderQ4K {
 // per quarter: sc[2q + h].
 struct LoaderQ6K {
     static constexpr int NL = 6;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
     u32x4 qa, qb, qh;
     uint sca, scb, d16, p;  // p = j%2: which nibble of ql and which bit pairs of qh
     float s0, s1;
@@ -164,6 +182,8 @@ struct LoaderQ6K {
 // The slab's two Q8_0 blocks: thread half h owns block h = slab columns 32h..32h+31.
 struct LoaderQ80 {
     static constexpr int NL = 3;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
     u32x4 qa, qb;
     uint d16;
     float d;
@@ -194,10 +214,59 @@ struct LoaderQ80 {
     }
 };
 
+// Q4L: Q4_K relaid by `relayout_q4k_q4l` (crates/ojas-formats/src/quant.rs:192-222) — nibbles w4[N][K/2], byte i of a
+// 32-weight block = weights 2i (low nibble) and 2i+1 (high), and per block the f16 pair qa = d*sc, qb = -dmin*m.  Every
+// weight enters the tile as the binary16 fma qa*q + qb, the arithmetic of the reference's `gemm_mm_q4l`
+// (crates/ojas-cuda/src/kernels/gemm_q.rs:104-142).  Thread half h owns block h of the slab = columns 32h..32h+31.
+struct LoaderQ4L {
+    static constexpr int NL = 3;
+    struct Row { const uchar* w; const ushort* qa; const ushort* qb; };
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) {
+        return {s.w + (size_t)n * (K >> 1), s.qa + (size_t)n * (K >> 5), s.qb + (size_t)n * (K >> 5)};
+    }
+    u32x4 nib;
+    uint a16, c16;
+    half2v a2, c2;
+    uint o[16];
+    __device__ __forceinline__ void load(const Row& r, uint k0, uint h) {
+        nib = gm_load16(r.w + (k0 >> 1) + h * 16u);
+        a16 = gm_load_u16(r.qa + (k0 >> 5) + h);
+        c16 = gm_load_u16(r.qb + (k0 >> 5) + h);
+    }
+    __device__ __forceinline__ void prep() {
+        const _Float16 a = __builtin_bit_cast(_Float16, (ushort)a16), c = __builtin_bit_cast(_Float16, (ushort)c16);
+        a2 = (half2v){a, a};
+        c2 = (half2v){c, c};
+    }
+    template <int I>
+    __device__ __forceinline__ void part() {
+        const half2v k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+        const uint u = nib[I];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint by = (u >> (8 * j)) & 0xFFu;
+            // the nibbles as the halves 1024 + q, then q exactly, then one rounding in the fma
+            const uint hbits = 0x64006400u | (by & 0x0Fu) | ((by & 0xF0u) << 12);
+            const half2v q = __builtin_bit_cast(half2v, hbits) - k1024;
+            o[4 * I + j] = __builtin_bit_cast(uint, __builtin_elementwise_fma(q, a2, c2));
+        }
+    }
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* q = (u32x4*)(lds_row + h * 64u);
+#pragma unroll
+        for (int i = 0; i < 4; i++) q[i] = (u32x4){o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+    }
+};
+
 // ------------------------------------------------------------------ the tile
-template <class Loader, bool SPLITK>
-__device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, const uchar* __restrict__ w,
+// XF32: the activations arrive as f32 [M][K] and are rounded to f16 on their way into the tile (the reference's plain
+// entries); each slab's loads are then consumed where they are issued, which is correct but not pipelined — callers
+// that care convert once (copy_f32_half) and take the f16 entries, as the reference's own `mm` does for split-K.
+template <class Loader, bool SPLITK, bool XF32 = false>
+__device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const GmSrc src,
                                              float* __restrict__ y, uint K, uint N, uint accum, uint M, uint nsplit) {
+    const ushort* xh = (const ushort*)xv;
+    const float* xf = (const float*)xv;
     __shared__ __attribute__((aligned(16))) uchar lds[2 * GM_STAGE];
     const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint n0 = blockIdx.x * GM_BN, m0 = blockIdx.y * GM_BM;
@@ -212,10 +281,10 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
     // staging roles
     const uint xr = tid >> 3, xc = (tid & 7u) * 8u;  // activation slab: rows xr + 32 i, 8 f16 at column xc
     const uint wr = tid >> 1, wh = tid & 1u;         // weight slab: row wr, half wh
-    const uchar* wrow = w + (size_t)min(n0 + wr, N - 1u) * Loader::row_bytes(K);
-    const ushort* xrow[8];
+    const typename Loader::Row wrow = Loader::row(src, min(n0 + wr, N - 1u), K);
+    size_t xrow[8];   // element offset of the thread's 8 activations in each of its rows
 #pragma unroll
-    for (int i = 0; i < 8; i++) xrow[i] = xh + (size_t)min(m0 + xr + 32u * i, M - 1u) * K + xc;
+    for (int i = 0; i < 8; i++) xrow[i] = (size_t)min(m0 + xr + 32u * i, M - 1u) * K + xc;
     const uint x_lds = xr * GM_STRIDE + xc * 2u;                   // + i * 32 rows
     const uint w_lds = GM_BM * GM_STRIDE + wr * GM_STRIDE;
 
@@ -239,7 +308,7 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
 #define GM_LOAD(XS, LD, T)                                                                       \
     do {                                                                                         \
         const uint kk_ = k_begin + (T) * GM_BK;                                                  \
-        _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++) XS[i_] = gm_load16(xrow[i_] + kk_);      \
+        _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++) XS[i_] = gm_load_x<XF32>(xh, xf, xrow[i_] + kk_); \
         LD.load(wrow, kk_, wh);                                                                  \
         gm_fence();                                                                              \
     } while (0)
@@ -363,11 +432,28 @@ __device__ __forceinline__ void gemm_mm_body(const ushort* __restrict__ xh, cons
 #define GEMM_ENTRIES(FMT, LOADER)                                                                                 \
     extern "C" __global__ void __launch_bounds__(256) gemm_mm_##FMT(                                              \
         const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {                         \
-        gemm_mm_body<LOADER, false>(xh, w, y, K, N, accum, M, 1u); }                                              \
+        gemm_mm_body<LOADER, false>(xh, GmSrc{w, nullptr, nullptr}, y, K, N, accum, M, 1u); }                     \
     extern "C" __global__ void __launch_bounds__(256) gemm_mm_##FMT##_sk(                                         \
         const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {                        \
-        gemm_mm_body<LOADER, true>(xh, w, y, K, N, 1u, M, nsplit); }
+        gemm_mm_body<LOADER, true>(xh, GmSrc{w, nullptr, nullptr}, y, K, N, 1u, M, nsplit); }
 
 GEMM_ENTRIES(q4k, LoaderQ4K)
 GEMM_ENTRIES(q6k, LoaderQ6K)
 GEMM_ENTRIES(q8_0, LoaderQ80)
+
+// The reference's entries for Q4L weights, under their names and argument lists
+// (crates/ojas-cuda/src/kernels/gemm_q.rs:26-38, :505-542; dispatched by `CudaSsm::mm`, crates/ojas-cuda/src/qwen35.rs:683,690):
+//   gemm_mm_q4l(x f32, w4, y, qa, qb, K, N, accum, M)      gemm_mm_q4l_hb(xh f16, ...)      gemm_mm_q4l_sk(xh f16, w4, y, qa, qb, K, N, M, nsplit)
+// on this library's tile: grid [ceil(N/128), ceil(M/256), nsplit].
+extern "C" __global__ void __launch_bounds__(256) gemm_mm_q4l(
+    const float* x, const uchar* w4, float* y, const ushort* qa, const ushort* qb, uint K, uint N, uint accum, uint M) {
+    gemm_mm_body<LoaderQ4L, false, true>(x, GmSrc{w4, qa, qb}, y, K, N, accum, M, 1u);
+}
+extern "C" __global__ void __launch_bounds__(256) gemm_mm_q4l_hb(
+    const ushort* xh, const uchar* w4, float* y, const ushort* qa, const ushort* qb, uint K, uint N, uint accum, uint M) {
+    gemm_mm_body<LoaderQ4L, false>(xh, GmSrc{w4, qa, qb}, y, K, N, accum, M, 1u);
+}
+extern "C" __global__ void __launch_bounds__(256) gemm_mm_q4l_sk(
+    const ushort* xh, const uchar* w4, float* y, const ushort* qa, const ushort* qb, uint K, uint N, uint M, uint nsplit) {
+    gemm_mm_body<LoaderQ4L, true>(xh, GmSrc{w4, qa, qb}, y, K, N, 1u, M, nsplit);
+}

@@ -31,6 +31,7 @@
 #include "ojk_common.h"
 #include "ojk_q4k_dot.h"
 #include "ojk_gq.h"
+#include "ojk_moe_rows.h"
 
 // ------------------------------------------------------------------ router
 template <int NI>
@@ -1009,3 +1010,16 @@ moe_combine(const float* __restrict__ dv, const float* __restrict__ wgt, float* 
     for (uint j = 0; j < KSEL; j++) acc += wgt[(size_t)t * KSEL + j] * dv[((size_t)t * KSEL + j) * D + col];
     y[i] = acc;
 }
+
+// ------------------------------------------------------------------ K-quant experts on f32 activations
+// The reference's expert kernels for raw K-quant rows under their own names (the expert table,
+// crates/ojas-core/src/quant_src.rs:168-193; bodies crates/ojas-metal/src/kernels/moe.rs:497-527, :722-815), with
+// the argument lists of the Q8_0 pair above:
+//   moe_gu_q4k(x, wg, wu, act, idx, K, N)              moe_down_{q5k,q6k}(act, wd, y, idx, wgt, K, N, KSEL)
+// f32 activations meet the dequantized weights (the float contract; the CPU path's int8-activation arithmetic is
+// what the _dec / _m / _mm / _mt entries above compute).  moe_down_q4k is this library's addition, so that an
+// all-Q4_K layer runs under the same contract.
+MOE_ROWS_GU_ENTRY(q4k, Q4kW)
+MOE_ROWS_DOWN_ENTRY(q4k, Q4kW)
+MOE_ROWS_DOWN_ENTRY(q5k, Q5kW)
+MOE_ROWS_DOWN_ENTRY(q6k, Q6kW)

@@ -175,3 +175,71 @@ struct Q5kW {
         return f16_bits_to_f32(f.hdr & 0xFFFFu) * a - f16_bits_to_f32(f.hdr >> 16) * b;
     }
 };
+
+// Q4_K on f32 activations with the same lane map (the reference's `moe_gu_q4k` multiplies the raw rows with f32
+// activations, crates/ojas-metal/src/kernels/moe.rs:497-527): 144-byte super-blocks {f16 d, dmin; 12 scale bytes;
+// qs[128]}, 32 lanes per super-block, a dword of qs against two float4 of x 32 floats apart.
+struct Q4kW {
+    static constexpr uint XGAP = 32u;
+    static constexpr uint STEP = 2u;
+    static constexpr uint BYTES = Q4K_BYTES;
+    static __device__ __forceinline__ uint units(uint K) { return K >> 8; }
+    static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 5; }
+    static __device__ __forceinline__ uint x_off(uint lane) { return ((lane & 31u) >> 3) * 64u + (lane & 7u) * 4u; }
+    static __device__ __forceinline__ uint x_unit(uint) { return 256u; }
+    struct Frag { uint hdr, s0, s1, s2, q; };
+    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
+        const uint* blk = (const uint*)(row + (size_t)u * Q4K_BYTES);
+        Frag f;
+        f.hdr = blk[0];
+        f.s0 = blk[1];
+        f.s1 = blk[2];
+        f.s2 = blk[3];
+        f.q = blk[4u + (lane & 31u)];
+        return f;
+    }
+    static __device__ __forceinline__ float dot(const Frag& f, uint lane, float4 x0, float4 x1, float) {
+        const uint c = (lane & 31u) >> 3;
+        uint sc, mn;
+        q4k_scale_min_pair(f.s0, f.s1, f.s2, c, sc, mn);
+        const float a = (float)(sc & 0xFFu) * dot4_ub(f.q & 0x0F0F0F0Fu, x0, 0.0f) + (float)(sc >> 8) * dot4_ub((f.q >> 4) & 0x0F0F0F0Fu, x1, 0.0f);
+        const float b = (float)(mn & 0xFFu) * sum4(x0) + (float)(mn >> 8) * sum4(x1);
+        return f16_bits_to_f32(f.hdr & 0xFFFFu) * a - f16_bits_to_f32(f.hdr >> 16) * b;
+    }
+};
+
+// Q6_K on f32 activations (the reference's `moe_down_q6k`, crates/ojas-metal/src/kernels/moe.rs:768-815): 210-byte
+// super-blocks {ql[128]; qh[64]; i8 scales[16]; f16 d}, only 2-byte aligned.  Per half of 128 weights the low nibbles
+// of its 64 ql bytes are weights 0..63 and the high nibbles weights 64..127, so a dword of ql meets two float4 of x
+// 64 floats apart; qh byte l % 32 of the half carries the upper two bits of weights l, l+32, l+64, l+96 (bit pairs
+// 0..3); one int8 scale per 16 weights; w = d * sc * (code - 32) (crates/ojas-formats/src/gguf.rs:1086-1108).
+struct Q6kW {
+    static constexpr uint XGAP = 64u;
+    static constexpr uint STEP = 2u;
+    static constexpr uint BYTES = Q6K_BYTES;
+    static __device__ __forceinline__ uint units(uint K) { return K >> 8; }
+    static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 5; }
+    static __device__ __forceinline__ uint x_off(uint lane) { return ((lane & 31u) >> 4) * 128u + (lane & 15u) * 4u; }
+    static __device__ __forceinline__ uint x_unit(uint) { return 256u; }
+    struct Frag { uint ql, qh, sa, sb, d; };
+    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
+        typedef uint __attribute__((aligned(2))) uint_u;
+        const uchar* blk = row + (size_t)u * Q6K_BYTES;
+        const uint hf = (lane & 31u) >> 4, i = lane & 15u;
+        const uint quarter = i >> 3, grp = (i & 7u) >> 2;   // low-nibble weights: quarter 0 or 1; 16-weight group within it
+        Frag f;
+        f.ql = *(const uint_u*)(blk + hf * 64u + i * 4u);
+        f.qh = *(const uint_u*)(blk + 128u + hf * 32u + (i & 7u) * 4u) >> (2u * quarter);
+        f.sa = blk[192u + hf * 8u + 2u * quarter + grp];
+        f.sb = blk[192u + hf * 8u + 2u * (quarter + 2u) + grp];
+        f.d = *(const ushort*)(blk + 208u);
+        return f;
+    }
+    static __device__ __forceinline__ float dot(const Frag& f, uint, float4 x0, float4 x1, float) {
+        const uint lo = (f.ql & 0x0F0F0F0Fu) | ((f.qh << 4) & 0x30303030u);        // bit pair `quarter`
+        const uint hi = ((f.ql >> 4) & 0x0F0F0F0Fu) | (f.qh & 0x30303030u);        // bit pair `quarter + 2`
+        const float a = (float)(signed char)f.sa * (dot4_ub(lo, x0, 0.0f) - 32.0f * sum4(x0));
+        const float b = (float)(signed char)f.sb * (dot4_ub(hi, x1, 0.0f) - 32.0f * sum4(x1));
+        return f16_bits_to_f32(f.d) * (a + b);
+    }
+};

@@ -648,8 +648,8 @@ static int shape_embed(const ojh_kernel_spec *, const ojh_device *, uint32_t K, 
 // "gemm", 2/3 the 256 x 256 tile and 4/5 the 128 x 256 tile of family "gemm_xl".
 static void gemm_tile(const ojh_kernel_spec *s, uint32_t *bm, uint32_t *bn, bool *sk) {
     *sk = s->rows_per_wave & 1;
-    *bn = s->rows_per_wave >= 2 ? 256 : 128;
-    *bm = s->rows_per_wave >= 4 ? 128 : 256;
+    *bn = (s->rows_per_wave >= 2 && s->rows_per_wave < 8) ? 256 : 128;
+    *bm = (s->rows_per_wave >= 4 && s->rows_per_wave < 8) ? 128 : 256;
 }
 
 static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
@@ -676,6 +676,28 @@ static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_
     need[2] = (size_t)M * N * 4;
     align[1] = ojh_block_align(f);
     align[2] = 4;
+    return OJH_OK;
+}
+
+// gemm_mm_q4l(x f32, w4, y, qa, qb, K, N, accum, M), gemm_mm_q4l_hb(xh f16, ...), gemm_mm_q4l_sk(xh, w4, y, qa, qb, K, N, M, nsplit):
+// the reference's argument lists (crates/ojas-cuda/src/kernels/gemm_q.rs:26-38).  `rows_per_wave`: 8 plain with f32
+// activations, 9 split-K, 10 plain with f16 activations; all on the 256 x 128 tile.
+static int check_gemm_q4l(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                          const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const bool sk = s->rows_per_wave == 9, xf32 = s->rows_per_wave == 8;
+    uint32_t K = c[0], N = c[1], M = sk ? c[2] : c[3], nsplit = sk ? c[3] : 1;
+    if (!K || !N || K % 256) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u (Q4L is relaid Q4_K: K a positive multiple of 256)", s->name, K, N);
+    if (M == 0 || nsplit == 0) return ojh_fail(OJH_ERR_ARG, "%s: M and nsplit must be positive", s->name);
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (grid[0] != (N + 127) / 128 || grid[1] != (M + 255) / 256 || grid[2] != nsplit)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, (N + 127) / 128, (M + 255) / 256, nsplit);
+    need[0] = (size_t)M * K * (xf32 ? 4 : 2);
+    need[1] = (size_t)N * (K / 2);
+    need[2] = (size_t)M * N * 4;
+    need[3] = need[4] = (size_t)N * (K / 32) * 2;
+    align[2] = 4;
+    align[3] = align[4] = 2;
     return OJH_OK;
 }
 
@@ -1173,6 +1195,10 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g, "gemm", 3, 4, f.type, 0, check_gemm, shape_gemm);
         add(g + "_sk", "gemm", 3, 4, f.type, 1, check_gemm, shape_gemm);
     }
+    // Q4L (relaid Q4_K + side arrays) under the reference's names and argument lists
+    add("gemm_mm_q4l", "gemm", 5, 4, 0, 8, check_gemm_q4l, shape_gemm);
+    add("gemm_mm_q4l_sk", "gemm", 5, 4, 0, 9, check_gemm_q4l, shape_gemm);
+    add("gemm_mm_q4l_hb", "gemm", 5, 4, 0, 10, check_gemm_q4l, shape_gemm);
     // Q4_K with the arithmetic of the reference's `gemm_mm_q4l` (f16 qa*q + qb), 256-wide tiles
     add("gemm_mm_q4kl", "gemm_xl", 3, 4, OJH_Q4_K, 2, check_gemm, shape_gemm);
     add("gemm_mm_q4kl_sk", "gemm_xl", 3, 4, OJH_Q4_K, 3, check_gemm, shape_gemm);
@@ -1209,6 +1235,13 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add("moe_gu_" + tag, "moe_iq", 5, 2, ty, 14, check_moe, shape_moe);
         m.back().expert_bufs = 2;
         add("moe_down_" + tag, "moe_iq", 5, 3, ty, 15, check_moe, shape_moe);
+        m.back().expert_bufs = 1;
+    }
+    // K-quant experts on f32 activations, the reference's names (crates/ojas-core/src/quant_src.rs:174-179)
+    add("moe_gu_q4k", "moe", 5, 2, OJH_Q4_K, 14, check_moe, shape_moe);
+    m.back().expert_bufs = 2;
+    for (uint32_t ty : {(uint32_t)OJH_Q4_K, (uint32_t)OJH_Q5_K, (uint32_t)OJH_Q6_K}) {
+        add(std::string("moe_down_") + ojh_format(ty)->tag, "moe", 5, 3, ty, 15, check_moe, shape_moe);
         m.back().expert_bufs = 1;
     }
     add("moe_down_q6k_m", "moe", 6, 3, OJH_Q6_K, 4, check_moe, shape_moe);

@@ -41,8 +41,12 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     // any of the three): the reference's own expert kernels moe_gu_<fmt> / moe_down_<fmt>, one launch for
     // gate/up and one for down over all tokens; the down launch accumulates onto y, so a plain store
     // starts from zeros
+    // K-quant experts take the same two launches when floating-point activations are asked for (OJH_ACT_FLOAT):
+    // moe_gu_q4k / moe_down_{q4k,q5k,q6k}, the reference's GPU expert kernels for those formats.
     auto float_expert = [](uint32_t t) { return t == OJH_Q8_0 || t == OJH_IQ4_XS || t == OJH_IQ4_NL; };
-    if (gate->type == up->type && float_expert(gate->type) && float_expert(down->type)) {
+    const bool kq_float = act_mode == OJH_ACT_FLOAT && gate->type == OJH_Q4_K && up->type == OJH_Q4_K &&
+                          (down->type == OJH_Q4_K || down->type == OJH_Q5_K || down->type == OJH_Q6_K);
+    if (kq_float || (gate->type == up->type && float_expert(gate->type) && float_expert(down->type))) {
         if (act_mode == OJH_ACT_Q8K)
             return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: %s / %s experts take f32 activations, as their CPU dots do",
                             ojh_format(gate->type)->tag, ojh_format(down->type)->tag);
@@ -59,8 +63,9 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         if ((rc = span("moe_ffn: wgt", wgt, (size_t)NA8 * 4, 4))) return rc;
         if ((rc = span("moe_ffn: y", y, (size_t)T * d * 4, 4))) return rc;
         const std::string gu_name = std::string("moe_gu_") + fg->tag, down_name = std::string("moe_down_") + fd->tag;
-        if ((rc = ensure(dev, gate->type == OJH_Q8_0 ? "moe" : "moe_iq"))) return rc;
-        if ((rc = ensure(dev, down->type == OJH_Q8_0 ? "moe" : "moe_iq"))) return rc;
+        auto family_of = [](uint32_t t) { return t == OJH_IQ4_XS || t == OJH_IQ4_NL ? "moe_iq" : "moe"; };
+        if ((rc = ensure(dev, family_of(gate->type)))) return rc;
+        if ((rc = ensure(dev, family_of(down->type)))) return rc;
         ojh_buf *act8;
         if ((rc = ojh_scratch_get(dev, "moe_act", (size_t)NA8 * n_ff * 4, &act8))) return rc;
         uint32_t b256[3] = {256, 1, 1};
@@ -81,8 +86,6 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     if (gate->type != OJH_Q4_K || up->type != OJH_Q4_K || (down->type != OJH_Q4_K && down->type != OJH_Q5_K && down->type != OJH_Q6_K))
         return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: gate and up must be Q4_K with down Q4_K, Q5_K or Q6_K, or all three among Q8_0, IQ4_XS, IQ4_NL (gate %u, up %u, down %u)",
                         gate->type, up->type, down->type);
-    if (act_mode == OJH_ACT_FLOAT)
-        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_moe_ffn: K-quant experts have the quantized-activation contract only (OJH_ACT_Q8K)");
     const bool down5 = down->type != OJH_Q4_K;   // Q5_K or Q6_K down tensors: integer dots at every batch size
     const std::string down_dec = std::string("moe_down_") + ojh_format(down->type)->tag + "_dec";
     const std::string down_m = std::string("moe_down_") + ojh_format(down->type)->tag + "_m";

@@ -128,6 +128,56 @@ def test_split_k_entry_through_the_kernel_seam(gpu, orc, pkg, kernel, family, bm
         gpu.dispatch(enc, kernel, [(xh, 0), (wd, 0), (yd, 0)], [k, n, m, 2], [3, 1, 1], [256, 1, 1])
 
 
+def test_q4l_entries_by_their_reference_names(gpu, orc, pkg):
+    """`gemm_mm_q4l` (f32 x), `gemm_mm_q4l_hb` (f16 x) and `gemm_mm_q4l_sk` with the reference's argument lists
+    (crates/ojas-cuda/src/kernels/gemm_q.rs:26-38: x, w4, y, qa, qb; K, N, accum, M | K, N, M, nsplit) on weights relaid
+    by `relayout_q4k_q4l` — on the device here, checked bit for bit elsewhere.  Ragged M and N, accumulate, sentinels
+    behind row M, and a one-hot read-back of the tile's bits."""
+    gpu.ensure_family("gemm")
+    gpu.ensure_family("dequant")
+    for m, k, n in ((140, 2048, 300), (64, 256, 128), (300, 512, 72)):
+        w = pkg.synth.q4k_weights(n, k, "q4l", "w", n, k)
+        x = pkg.synth.normal_f32(m * k, "q4l", "x", m, k).reshape(m, k)
+        raw = gpu.upload_bytes(w)
+        nib, qa, qb = gpu.alloc_bytes(n * k // 2), gpu.alloc_bytes(n * k // 32 * 2), gpu.alloc_bytes(n * k // 32 * 2)
+        gpu.relayout_q4k_q4l(raw, n, k, nib, qa, qb)
+        xf, xh = gpu.upload(x), gpu.upload_bytes(x.astype(np.float16))
+        want = orc.matmul_ref(w, Q4_K, n, k, x, wmode=2, xmode=1)
+        grid = [(n + 127) // 128, (m + 255) // 256, 1]
+        sent = np.full(n, 12345.5, np.float32)
+        for kernel, xbuf in (("gemm_mm_q4l", xf), ("gemm_mm_q4l_hb", xh)):
+            for accum in (0, 1):
+                y0 = pkg.synth.normal_f32(m * n, "q4l", "y0", accum).reshape(m, n)
+                yd = gpu.upload(np.concatenate([y0.ravel(), sent]))
+                gpu.dispatch(gpu.begin(), kernel, [(xbuf, 0), (nib, 0), (yd, 0), (qa, 0), (qb, 0)], [k, n, accum, m], grid, [256, 1, 1])
+                got = gpu.read(yd, m * n + n)
+                assert np.all(got[m * n:] == 12345.5), "wrote past row M"
+                e = rms_errs(got[:m * n].reshape(m, n), want + (y0 if accum else 0))
+                assert e[0] < TIGHT[0] and e[1] < TIGHT[1], (kernel, accum, m, k, n, e)
+        for nsplit in (1, 3):
+            if k // 64 < nsplit:
+                continue
+            y0 = pkg.synth.normal_f32(m * n, "q4l", "y0sk", nsplit).reshape(m, n)
+            yd = gpu.upload(y0)
+            gpu.dispatch(gpu.begin(), "gemm_mm_q4l_sk", [(xh, 0), (nib, 0), (yd, 0), (qa, 0), (qb, 0)], [k, n, m, nsplit],
+                         [grid[0], grid[1], nsplit], [256, 1, 1])
+            e = rms_errs(gpu.read(yd, m * n).reshape(m, n), want + y0)
+            assert e[0] < 1e-4 and e[1] < 2e-5, (nsplit, e)
+    # the tile's bits: one-hot activations read every weight back
+    k, n = 512, 160
+    w = orc.synth_blocks(Q4_K, n * k // 256)
+    raw = gpu.upload_bytes(w)
+    nib, qa, qb = gpu.alloc_bytes(n * k // 2), gpu.alloc_bytes(n * k // 32 * 2), gpu.alloc_bytes(n * k // 32 * 2)
+    gpu.relayout_q4k_q4l(raw, n, k, nib, qa, qb)
+    yd = gpu.alloc(k * n)
+    gpu.dispatch(gpu.begin(), "gemm_mm_q4l", [(gpu.upload(np.eye(k, dtype=np.float32)), 0), (nib, 0), (yd, 0), (qa, 0), (qb, 0)],
+                 [k, n, 0, k], [(n + 127) // 128, (k + 255) // 256, 1], [256, 1, 1])
+    want = orc.q4l_weights_f16(w, k, n).view(np.float16).astype(np.float32).reshape(n, k)
+    assert np.array_equal(gpu.read(yd, k * n).reshape(k, n), want.T)
+    with pytest.raises(pkg.OjasHipError, match="takes 5 buffers"):
+        gpu.dispatch(gpu.begin(), "gemm_mm_q4l", [(xh, 0), (nib, 0), (yd, 0)], [k, n, 0, k], [2, 2, 1], [256, 1, 1])
+
+
 def test_router_prefers_the_tile_only_above_the_crossover(gpu, orc, pkg):
     """ACT_AUTO: small M keeps the CPU-reference arithmetic (int8 activations); large M takes the
     f16 tile.  Both must sit within their own oracle's bound."""

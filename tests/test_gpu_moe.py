@@ -447,6 +447,47 @@ def test_iq4_experts_through_the_ffn_entry(gpu, orc, pkg, tg, td, T, E, ksel, d,
         gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, act_mode=pkg.ACT_Q8K)
 
 
+@pytest.mark.parametrize("td", [12, 13, 14])
+def test_kquant_experts_on_f32_activations_by_their_reference_names(gpu, orc, pkg, td):
+    """`moe_gu_q4k` and `moe_down_{q5k,q6k}` (and this library's `moe_down_q4k`) — the reference's expert table
+    (crates/ojas-core/src/quant_src.rs:174-179) — dispatched by name with the Q8_0 pair's argument lists and the
+    reference's grids, against products of the exact block values in double (the float contract: f32 activations meet
+    the dequantized weights, crates/ojas-metal/src/kernels/moe.rs:497-527, :722-815); then through `ojh_moe_ffn` with
+    OJH_ACT_FLOAT."""
+    tag = {12: "q4k", 13: "q5k", 14: "q6k"}[td]
+    k, n, E, ksel, T = 512, 256, 8, 3, 2
+    x = pkg.synth.normal_f32(T * k, "moekq", "x").reshape(T, k)
+    gbytes, ubytes = pkg.synth.q4k_weights(E * n, k, "moekq", "g"), pkg.synth.q4k_weights(E * n, k, "moekq", "u")
+    dbytes = pkg.synth.weights(td, E * k, n, "moekq", "d", td)
+    idx = np.array([[1, 5, 2], [7, 0, 5]], np.uint32)
+    wgt = np.array([[0.5, 0.3, 0.2], [0.6, 0.25, 0.15]], np.float32)
+    want = orc.moe_ffn(x, idx, wgt, gbytes, ubytes, Q4_K, dbytes, td, E, n, mode=1)
+    gpu.ensure_family("moe")
+    xd, gd, ud, dd = gpu.upload(x), gpu.upload_bytes(gbytes), gpu.upload_bytes(ubytes), gpu.upload_bytes(dbytes)
+    idxd, wgtd = gpu.upload_bytes(idx), gpu.upload(wgt)
+    actd, outd = gpu.alloc(T * ksel * n), gpu.upload(np.zeros(T * k, np.float32))
+    enc = gpu.begin()
+    gpu.dispatch(enc, "moe_gu_q4k", [(xd, 0), (gd, 0), (ud, 0), (actd, 0), (idxd, 0)], [k, n], [-(-n // 8), ksel, T], [256, 1, 1])
+    gpu.dispatch(enc, "moe_down_" + tag, [(actd, 0), (dd, 0), (outd, 0), (idxd, 0), (wgtd, 0)], [n, k, ksel], [-(-k // 8), T, 1], [256, 1, 1])
+    gpu.submit(enc)
+    got = gpu.read(outd, T * k).reshape(T, k)
+    assert peak_err(got, want) <= 1e-5
+    # the op seam under the float contract, accumulating onto y
+    lg_, lu_, ld_ = gpu.lin(Q4_K, E * n, k, gbytes), gpu.lin(Q4_K, E * n, k, ubytes), gpu.lin(td, E * k, n, dbytes)
+    y0 = pkg.synth.normal_f32(T * k, "moekq", "y0").reshape(T, k)
+    yd = gpu.upload(y0)
+    gpu.moe_ffn(xd, T, k, n, E, ksel, idxd, wgtd, lg_, lu_, ld_, yd, accum=True, act_mode=pkg.ACT_FLOAT)
+    assert peak_err(gpu.read(yd, T * k).reshape(T, k) - y0, want) <= 1e-5
+    # an index past the tensors multiplies nothing
+    bad = gpu.upload_bytes(np.array([[1, 99, 2], [7, 0, 5]], np.uint32))
+    gpu.memset0(outd)
+    gpu.dispatch(enc, "moe_gu_q4k", [(xd, 0), (gd, 0), (ud, 0), (actd, 0), (bad, 0)], [k, n], [-(-n // 8), ksel, T], [256, 1, 1])
+    gpu.dispatch(enc, "moe_down_" + tag, [(actd, 0), (dd, 0), (outd, 0), (bad, 0), (wgtd, 0)], [n, k, ksel], [-(-k // 8), T, 1], [256, 1, 1])
+    idx2, wgt2 = np.array([[1, 2], [7, 0]], np.uint32), np.array([[0.5, 0.2], [0.6, 0.25]], np.float32)
+    want2 = orc.moe_ffn(x[:1], idx2[:1], wgt2[:1], gbytes, ubytes, Q4_K, dbytes, td, E, n, mode=1)
+    assert peak_err(gpu.read(outd, k), want2[0]) <= 1e-5
+
+
 def test_expert_ffn_rejects_what_it_cannot_run(gpu, pkg):
     E, d, nff = 4, 256, 256
     gate, up, down = _experts(pkg, E, d, nff, "err")
@@ -455,7 +496,5 @@ def test_expert_ffn_rejects_what_it_cannot_run(gpu, pkg):
     idx, wgt = gpu.upload_bytes(np.array([1, 2], np.uint32)), gpu.upload(np.array([0.5, 0.5], np.float32))
     with pytest.raises(pkg.OjasHipError, match="shapes do not match"):
         gpu.moe_ffn(x, 1, d, nff, E + 1, 2, idx, wgt, lg_, lu_, ld_, y)
-    with pytest.raises(pkg.OjasHipError, match="quantized-activation"):
-        gpu.moe_ffn(x, 1, d, nff, E, 2, idx, wgt, lg_, lu_, ld_, y, act_mode=pkg.ACT_FLOAT)
     with pytest.raises(pkg.OjasHipError, match="needs"):
         gpu.moe_ffn(x, 2, d, nff, E, 2, idx, wgt, lg_, lu_, ld_, y)
