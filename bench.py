@@ -59,6 +59,8 @@ def main() -> int:
     ap.add_argument("--fused-quant", action="store_true",
                     help="quantize x inside every matvec launch (8 launches per step) instead of once per "
                          "stage in a launch of its own (5 + 8 launches); measured slower")
+    ap.add_argument("--split-quant", action="store_true",
+                    help="always quantize in a launch of its own (5 + 5 launches) instead of one ojh_mm_multi call per stage")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
     args = ap.parse_args()
@@ -87,18 +89,24 @@ def main() -> int:
     dom = "head"  # the launch that dominates the step: 295.5 MB of its 418 MB
 
     def one(st: str, lin, y) -> None:
-        """One projection from the f32 stage input: by default a single launch that quantizes x
-        in-kernel; with --split-quant, from the stage's separately quantized copy."""
+        """One projection alone: from the stage's separately quantized vector, or (--fused-quant) from the f32 vector
+        through the single-tensor launch that quantizes it itself."""
         if (not args.fused_quant):
             gpu.mm_q8k(xq[st], xsc[st], lin, y)
         else:
             gpu.mm(xs[st], lin, y, 1, act_mode=pkg.ACT_Q8K)
 
     grouped = not args.fused_quant and not args.per_projection
+    staged = grouped and not args.split_quant
 
     def step(i: int) -> None:
         w = sets[i % args.copies]
         for st, k, names in STAGES:
+            if staged:
+                # one call per stage from the f32 vector: the library folds the quantizer into the launch where that is
+                # faster (the small q/k/v stage) and otherwise issues a quantizer launch and one grouped launch
+                gpu.mm_multi(xs[st], [w[n] for n in names], [ys[n] for n in names])
+                continue
             if (not args.fused_quant):
                 gpu.quant_q8k(xs[st], 1, k, xq[st], xsc[st])
             if grouped and len(names) > 1:
@@ -189,25 +197,40 @@ def main() -> int:
         del src
     del mf_out
 
-    # ---- per-shape latency (each shape alone, back to back, rotating sets), for the record.  The launches are
-    # recorded once and replayed from the library, like the step: issued one by one from Python the short
-    # ones would show the interpreter's call rate, not the kernel
+    # ---- per-shape latency (each shape alone, back to back), for the record, twice: streaming from HBM — as many
+    # copies of the shape as it takes to exceed the 256 MB Infinity Cache, visited in turn — and cache-resident (two
+    # copies).  The launches are recorded once and replayed from the library, like the step: issued one by one from
+    # Python the short ones would show the interpreter's call rate, not the kernel.  The stage's quantized vector is
+    # prepared beforehand: these are the matvec launches alone.
     per_shape = {}
-    reps = 50
+    reps = 60
+    mall = 256 << 20
     for name, n, k in SHAPES:
         st = next(s for s, _, names in STAGES if name in names)
-        gpu.capture_begin()
-        for i in range(reps):
-            one(st, sets[i % args.copies][name], ys[name])
-        chain = gpu.capture_end()
-        chain.launch()
-        gpu.timer_start()
-        chain.launch()
-        us = gpu.timer_stop() / reps * 1e3
-        del chain
         b = algorithmic_bytes(n, k)
-        per_shape[name] = {"n": n, "k": k, "us": round(us, 2), "gbs": round(b / us / 1e3, 1),
-                           "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+        wbytes = n * (k // 256) * 144
+        ncold = max(2, mall // wbytes + 2)
+        extra_lins = [gpu.lin(Q4_K, n, k, host[name]) for _ in range(max(0, ncold - args.copies))]
+        pool = [sets[i][name] for i in range(args.copies)] + extra_lins
+        entry_ = {"n": n, "k": k}
+        for tag, lins in (("hbm", pool[:ncold]), ("cache", pool[:2])):
+            gpu.capture_begin()
+            for i in range(reps):
+                one(st, lins[i % len(lins)], ys[name])
+            chain = gpu.capture_end()
+            chain.launch()
+            gpu.timer_start()
+            chain.launch()
+            us = gpu.timer_stop() / reps * 1e3
+            del chain
+            if tag == "hbm":
+                entry_.update({"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4),
+                               "copies": len(lins)})
+            else:
+                entry_.update({"cache_resident_us": round(us, 2), "cache_resident_gbs": round(b / us / 1e3, 1)})
+        per_shape[name] = entry_
+        for l in extra_lins:
+            l.free()
 
     result = {
         "metric": "Q4_K decode GEMV GB/s (% HBM peak); prefill dequant-GEMM TFLOPS, 1 GPU",
@@ -226,7 +249,10 @@ def main() -> int:
                                "(q,k,v,o 4096; gate,up 14336x4096; down 4096x14336; head 128256x4096), "
                                "f32 activations N(0,1) quantized once per stage, weights in HBM",
                    "bytes_per_step": step_bytes, "weight_sets": args.copies,
-                   "launches_per_step": "5 quantize_q8k + 5 gemv_q8k_q4k* (q/k/v and gate/up each one grouped "
+                   "launches_per_step": "one ojh_mm_multi call per stage: q/k/v in 1 launch with the quantizer folded in "
+                                        "(gemv_fq8k_q4k_x4_r2), the other four stages quantize_q8k + one gemv_q8k_q4k* launch "
+                                        "(gate/up grouped over separate tensors): 9 launches" if staged else
+                                        "5 quantize_q8k + 5 gemv_q8k_q4k* (q/k/v and gate/up each one grouped "
                                         "launch over separate tensors)" if grouped else
                                         "5 quantize_q8k + 8 gemv_q8k_q4k*" if (not args.fused_quant) else
                                         "8 gemv_fq8k_q4k* (activation quantizer folded into each launch)",

@@ -224,6 +224,16 @@ int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const
 int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, int count,
                      const ojh_lin *const *ws, ojh_buf *const *ys, const size_t *y_offs);
 
+/* One stage of a decode layer in ONE launch: ys[i] (=, +=) x . ws[i]^T for one to four projections of the same
+ * f32 vector x[K] (q/k/v, gate/up, or a single o / down / head), the vector quantized as `quant_q8k` does inside the
+ * launch — the reference's CUDA decode path fuses the same steps (`qkv_q80_dp4a`, `ffn_gu_q80_dp4a` after
+ * `quantize_q8_1`, crates/ojas-cuda/src/kernels/gemv_q8.rs:178-260).  Bit-identical to `ojh_quant_q8k` followed by
+ * `ojh_mm_q8k` per projection (OJH_ACT_Q8K arithmetic); `accum` adds onto every y.  Q4_K tensors with K <= 16384 take
+ * the single launch; other K-quant formats or longer rows run as a quantizer launch plus the per-format launches.
+ * `y_offs` (bytes) may be NULL. */
+int ojh_mm_multi(ojh_device *dev, const ojh_buf *x, size_t x_off, int count, const ojh_lin *const *ws,
+                 ojh_buf *const *ys, const size_t *y_offs, int accum);
+
 /* Decode-layer epilogues around the matvec (the reference fuses the same steps on its GPU path:
  * `rmsnorm_q8` / `quantize_q8_1` and `ffn_gu_q80_dp4a`, crates/ojas-cuda/src/kernels/gemv.rs:37-53,
  * gemv_q8.rs:246-260).

@@ -515,6 +515,149 @@ gemv_fq8k_q4k_wide(const float* x, const uchar* w, float* y, uint K, uint N, uin
     gemv_fq8k_q4k_body<2>(x, w, y, K, N, NRB);
 }
 
+// ---- the folded quantizer over up to four tensors ----------------------------------------------
+//   gemv_fq8k_q4k_x4_{r1,r2}(x, w0, w1, w2, w3, y0, y1, y2, y3, K, E0, E1, E2, E3, NRB, ACC)     x: f32[K], K <= 16384
+// One launch per stage of a decode layer: the stage's f32 activations are quantized by every workgroup into LDS (the
+// arithmetic of quantize_q8k: results are bit-identical to quantizer + matvec launches) and multiplied with up to four
+// weight tensors that share them (q/k/v, gate/up; a single tensor passes E0 = E1 = E2 = E3).  ACC adds onto y (the
+// residual).  Vector memory operations return in order, so the activations are requested FIRST and the workgroup's
+// first weights second: the quantization then runs while those weights are still on their way instead of queueing
+// behind them.  A workgroup (256, 512 or 1024 threads) walks NRB rows, its waves R at a time.  The quantization is
+// about 110 vector instructions per segment and wave — as much as the dot products of twenty rows for K = 4096 — and
+// every workgroup repeats it, so the launch wants few, large workgroups: one or two per CU.
+template <int R>
+__device__ __forceinline__ void gemv_fq8k_q4k_x4_body(const float* __restrict__ x, const uchar* w0, const uchar* w1,
+                                                      const uchar* w2, const uchar* w3, float* y0, float* y1, float* y2,
+                                                      float* y3, uint K, uint E0, uint E1, uint E2, uint E3, uint NRB,
+                                                      uint ACC) {
+    __shared__ __attribute__((aligned(16))) signed char sx[(FQ_MAX_K / 256u) * FQ_SEG];
+    __shared__ float ss[FQ_MAX_K / 256u];
+    const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, nw = blockDim.x >> 6;
+    const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
+    const uint row_end = min((blockIdx.x + 1u) * NRB, E3);
+    uint row0 = blockIdx.x * NRB + wave * R;
+    // row r0 + r of the stacked tensors -> its block bytes and its output
+    auto locate = [&](uint r0, X4Row (&rw)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint gr = min(r0 + r, E3 - 1u);
+            const uchar* w;
+            float* y;
+            uint lr;
+            if (gr < E0) { w = w0; y = y0; lr = gr; }
+            else if (gr < E1) { w = w1; y = y1; lr = gr - E0; }
+            else if (gr < E2) { w = w2; y = y2; lr = gr - E1; }
+            else { w = w3; y = y3; lr = gr - E2; }
+            rw[r].w = w + (size_t)lr * nsb * Q4K_BYTES;
+            rw[r].y = y + lr;
+        }
+    };
+    auto fetch = [&](const X4Row (&rw)[R], uint sb, uint4 (&hdr)[R], uint4 (&qs)[R]) {
+        const uint sbc = min(sb, nsb - 1u);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uchar* blk = rw[r].w + (size_t)sbc * Q4K_BYTES;
+            hdr[r] = *(const uint4*)blk;
+            qs[r] = *(const uint4*)(blk + 16u + l * 16u);
+        }
+    };
+    // 1. the activations, four segments per wave at a time (wave `wave` owns segments wave, wave + nw, ...; a lane
+    //    holds 4 consecutive values), the first batch requested before anything else
+    constexpr int NB = 4;
+    float4 v[NB];
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+        const uint seg = wave + nw * (uint)i;
+        v[i] = *(const float4*)(x + (size_t)min(seg, nsb - 1u) * 256u + lane * 4u);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // 2. the first step's weights
+    X4Row rwc[R], rwn[R];
+    uint4 hc[R], qc[R], hn[R], qn[R];
+    locate(row0, rwc);
+    fetch(rwc, g, hc, qc);
+    __builtin_amdgcn_sched_barrier(0);
+    // 3. quantize into LDS
+    for (uint s0 = 0; s0 < nsb; s0 += nw * NB) {
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const uint seg = s0 + wave + nw * (uint)i;
+            const float4 t = v[i];
+            // the next batch's request goes out as soon as the register is free
+            const uint nseg = seg + nw * NB;
+            if (s0 + nw * NB < nsb) v[i] = *(const float4*)(x + (size_t)min(nseg, nsb - 1u) * 256u + lane * 4u);
+            if (seg < nsb) {
+                float a = wave_max(fmaxf(fmaxf(fabsf(t.x), fabsf(t.y)), fmaxf(fabsf(t.z), fabsf(t.w))));
+                float scale = a > 0.0f ? __fdiv_rn(a, 127.0f) : 1.0f;
+                float inv = __fdiv_rn(1.0f, scale);
+                int q0 = (int)sat127(roundf(__fmul_rn(t.x, inv)));
+                int q1 = (int)sat127(roundf(__fmul_rn(t.y, inv)));
+                int q2 = (int)sat127(roundf(__fmul_rn(t.z, inv)));
+                int q3 = (int)sat127(roundf(__fmul_rn(t.w, inv)));
+                *(uint*)(sx + seg * FQ_SEG + lane * 4u) =
+                    (uint)(q0 & 0xFF) | ((uint)(q1 & 0xFF) << 8) | ((uint)(q2 & 0xFF) << 16) | ((uint)(q3 & 0xFF) << 24);
+                if (lane == 0) ss[seg] = scale;
+            }
+        }
+    }
+    __syncthreads();
+    // 4. the rows: one stream of (row group, super-block step) units, the next unit's weights requested before the
+    //    current one is multiplied
+    float acc[R], add[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.0f;
+        add[r] = (ACC && row0 < row_end) ? *rwc[r].y : 0.0f;
+    }
+    uint sb = g;
+    while (row0 < row_end) {
+        uint nsb_next = sb + 8u, nrow = row0;
+        const bool last = nsb_next >= nsb + g;    // (sb - g) + 8 >= nsb: this was the group's last step
+        if (last) { nsb_next = g; nrow = row0 + nw * R; }
+        if (last) locate(nrow, rwn);
+        else {
+#pragma unroll
+            for (int r = 0; r < R; r++) rwn[r] = rwc[r];
+        }
+        if (nrow < row_end) fetch(rwn, nsb_next, hn, qn);
+        if (sb < nsb) {
+            Q4kFrag f;
+            const signed char* p = sx + sb * FQ_SEG + c * 64u + (l & 1u) * 16u;
+            f.xl = *(const uint4*)p;
+            f.xh = *(const uint4*)(p + 32);
+            f.bl = bytesum4(f.xl);
+            f.bh = bytesum4(f.xh);
+            f.sx = ss[sb];
+#pragma unroll
+            for (int r = 0; r < R; r++) acc[r] += q4k_lane_dot(hc[r], qc[r], c, f);
+        }
+        if (last) {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                float t = wave_sum(acc[r]);
+                if (lane == 0 && row0 + r < row_end) *rwc[r].y = ACC ? add[r] + t : t;
+                acc[r] = 0.0f;
+                add[r] = (ACC && nrow < row_end) ? *rwn[r].y : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) { rwc[r] = rwn[r]; hc[r] = hn[r]; qc[r] = qn[r]; }
+        sb = nsb_next;
+        row0 = nrow;
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(1024)
+gemv_fq8k_q4k_x4_r1(const float* x, const uchar* w0, const uchar* w1, const uchar* w2, const uchar* w3, float* y0, float* y1,
+                    float* y2, float* y3, uint K, uint E0, uint E1, uint E2, uint E3, uint NRB, uint ACC) {
+    gemv_fq8k_q4k_x4_body<1>(x, w0, w1, w2, w3, y0, y1, y2, y3, K, E0, E1, E2, E3, NRB, ACC);
+}
+extern "C" __global__ void __launch_bounds__(1024)
+gemv_fq8k_q4k_x4_r2(const float* x, const uchar* w0, const uchar* w1, const uchar* w2, const uchar* w3, float* y0, float* y1,
+                    float* y2, float* y3, uint K, uint E0, uint E1, uint E2, uint E3, uint NRB, uint ACC) {
+    gemv_fq8k_q4k_x4_body<2>(x, w0, w1, w2, w3, y0, y1, y2, y3, K, E0, E1, E2, E3, NRB, ACC);
+}
+
 // Batched form: y[M][N] (+)= quantized x[M][K] . W^T.  One wave per row; the row's weights are
 // read and unpacked once per tile of MT tokens.
 template <int MT>

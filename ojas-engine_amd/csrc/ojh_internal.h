@@ -74,6 +74,10 @@ struct ojh_device {
     bool gemm_exact = false;     // OJAS_HIP_GEMM_EXACT: Q4_K prefill through the tile that holds dequant_to_f16 bits
     bool fused_quant = false;    // OJAS_HIP_FUSED_QUANT=1: ojh_mm (m = 1, Q4_K) quantizes x inside the matvec launch
     uint32_t fq_blocks_per_cu = 8; // OJAS_HIP_FQ_BLOCKS: blocks per CU the fused-quantizer matvec aims for
+    uint32_t fq_threads = 1024;    // OJAS_HIP_FQ_THREADS: threads per workgroup of ojh_mm_multi's launch (256, 512, 1024)
+    int fq_rows = 0;               // OJAS_HIP_FQ_ROWS: rows per wave of ojh_mm_multi's launch (0: by row count)
+    int fq_multi = 1;              // OJAS_HIP_FQ_MULTI: 0 = ojh_mm_multi always quantizes in a launch of its own, 2 = never
+    uint32_t fq_multi_blocks = 1;  // OJAS_HIP_FQ_MULTI_BLOCKS: workgroups per CU of its single launch
     bool capturing = false;      // between ojh_capture_begin and ojh_capture_end
     bool capture_hip_graph = false;
     std::vector<ojh_command> recorded;

@@ -429,6 +429,33 @@ static int check_gemv_fq8k(const ojh_kernel_spec *s, const uint32_t *c, const ui
     return OJH_OK;
 }
 
+// gemv_fq8k_<fmt>_x4_{r1,r2}(x, w0..w3, y0..y3, K, E0..E3, NRB, ACC): the folded quantizer over up to four tensors
+static int check_gemv_fq8k_x4(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                              const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const ojh_block_format *f;
+    uint32_t K = c[0], E[4] = {c[1], c[2], c[3], c[4]}, NRB = c[5], ACC = c[6];
+    int rc = check_kn(s, K, E[3], &f);
+    if (rc) return rc;
+    if ((rc = check_block(block, 0))) return rc;
+    if (block[0] > 1024) return ojh_fail(OJH_ERR_ARG, "%s: at most 1024 threads per workgroup", s->name);
+    if (K > 16384) return ojh_fail(OJH_ERR_ARG, "%s: K=%u exceeds 16384", s->name, K);
+    if (ACC > 1) return ojh_fail(OJH_ERR_ARG, "%s: ACC=%u", s->name, ACC);
+    if (E[0] > E[1] || E[1] > E[2] || E[2] > E[3])
+        return ojh_fail(OJH_ERR_ARG, "%s: row totals %u,%u,%u,%u must not decrease", s->name, E[0], E[1], E[2], E[3]);
+    if (!NRB) return ojh_fail(OJH_ERR_ARG, "%s: NRB must be positive", s->name);
+    if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * NRB < E[3])
+        return ojh_fail(OJH_ERR_ARG, "%s: grid x NRB does not cover N=%u rows", s->name, E[3]);
+    need[0] = (size_t)K * 4;
+    for (int i = 0; i < 4; i++) {
+        size_t rows = E[i] - (i ? E[i - 1] : 0);
+        need[1 + i] = rows * (K / f->weights) * f->bytes;
+        need[5 + i] = rows * 4;
+        align[1 + i] = ojh_block_align(f);
+        align[5 + i] = 4;
+    }
+    return OJH_OK;
+}
+
 // gemv_nat_<fmt>_m(x, w, y, K, N, M, ACC)
 static int check_gemv_nat_m(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                             const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -1168,6 +1195,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
             add(fq + "_r1", "gemv_q8k", 3, 3, f.type, 1, check_gemv_fq8k, shape_rows);
             add(fq + "_r2", "gemv_q8k", 3, 3, f.type, 2, check_gemv_fq8k, shape_rows);
             add(fq + "_wide", "gemv_q8k", 3, 3, f.type, 2, check_gemv_fq8k, shape_rows);
+            add(fq + "_x4_r1", "gemv_q8k", 9, 7, f.type, 1, check_gemv_fq8k_x4, shape_rows);
+            add(fq + "_x4_r2", "gemv_q8k", 9, 7, f.type, 2, check_gemv_fq8k_x4, shape_rows);
         }
     }
     add("gemm_q8k_q4k_mf", "gemm_q8k", 4, 6, OJH_Q4_K, 1, check_gemm_q8k, shape_gemm_q8k);

@@ -342,6 +342,71 @@ extern "C" int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_bu
                       {ws[0]->k, ends[0], ends[1], ends[2], ends[3]}, grid, block);
 }
 
+// One stage of a decode layer in ONE launch: 1 to 4 projections of one f32 vector, the vector quantized inside the launch.
+extern "C" int ojh_mm_multi(ojh_device *dev, const ojh_buf *x, size_t x_off, int count, const ojh_lin *const *ws,
+                            ojh_buf *const *ys, const size_t *y_offs, int accum) {
+    if (!dev || !ws || !ys) return ojh_fail(OJH_ERR_ARG, "ojh_mm_multi: NULL argument");
+    if (count < 1 || count > 4) return ojh_fail(OJH_ERR_ARG, "ojh_mm_multi: count=%d, takes 1 to 4 projections", count);
+    int rc;
+    bool fused = true;
+    uint64_t total = 0;
+    for (int i = 0; i < count; i++) {
+        const ojh_block_format *fi;
+        if ((rc = ojh_mm_checks("ojh_mm_multi", ws[i], ys[i], y_offs ? y_offs[i] : 0, nullptr, 1, accum, &fi))) return rc;
+        if (ojh_float_rows(ws[i]->type))
+            return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm_multi: %s rows take f32 activations and need no quantizer: call ojh_mm", fi->tag);
+        if (ws[i]->k != ws[0]->k)
+            return ojh_fail(OJH_ERR_ARG, "ojh_mm_multi: projection %d has K=%u, the first has K=%u", i, ws[i]->k, ws[0]->k);
+        if (ws[i]->type != OJH_Q4_K) fused = false;
+        total += ws[i]->n;
+    }
+    if (total > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "ojh_mm_multi: too many rows");
+    const uint32_t K = ws[0]->k;
+    if ((rc = span_ok("ojh_mm_multi: x", x, x_off, (size_t)K * 4, 16))) return rc;
+    if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+    // Measured on MI355X (weights streamed from HBM): the single launch wins on a small stage (q/k/v of an 8B model:
+    // 6.6 against 7.7 us), ties on 4096 x 4096 and loses from there on — few large workgroups cannot keep as many bytes
+    // in flight as the plain matvec's thousands of small ones, and many small ones repeat the quantization too often.
+    // OJAS_HIP_FQ_MULTI = 0 never takes it, 2 takes it at every size.
+    const bool small_stage = total * K <= 32u * 1024u * 1024u && K <= 4096u;
+    if (!fused || K > 16384 || dev->fq_multi == 0 || (dev->fq_multi == 1 && !small_stage)) {   // quantize once, then the per-format launches
+        size_t nsb = K / 256;
+        ojh_buf *xq, *xs;
+        if ((rc = ojh_scratch_get(dev, "xq", nsb * 256, &xq))) return rc;
+        if ((rc = ojh_scratch_get(dev, "xs", nsb * 4, &xs))) return rc;
+        if ((rc = ojh_quant_q8k_launch(dev, at(x, x_off), OJH_X_F32, 1, K, xq->ptr, xs->ptr))) return rc;
+        if (!accum) return ojh_mm_q8k_multi(dev, xq, xs, count, ws, ys, y_offs);
+        for (int i = 0; i < count; i++)
+            if ((rc = ojh_mm_q8k_launch(dev, xq->ptr, xs->ptr, ws[i], ojh_format(ws[i]->type), at(ys[i], y_offs ? y_offs[i] : 0),
+                                        nullptr, 1, 1)))
+                return rc;
+        return OJH_OK;
+    }
+    std::vector<void *> p = {at(x, x_off)};
+    uint32_t ends[4], run = 0;
+    for (int i = 0; i < 4; i++) {
+        int j = i < count ? i : count - 1;
+        p.push_back(at(ws[j]->raw, ws[j]->off));
+        if (i < count) run += ws[i]->n;
+        ends[i] = run;
+    }
+    for (int i = 0; i < 4; i++) {
+        int j = i < count ? i : count - 1;
+        p.push_back(at(ys[j], y_offs ? y_offs[j] : 0));
+    }
+    // Every workgroup repeats the quantization (as many vector instructions as the dots of some twenty rows), so the
+    // launch takes few, large workgroups — `fq_blocks_per_cu` per CU, `fq_threads` threads each — and deals the rows
+    // evenly between them.
+    const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;
+    int r = dev->fq_rows ? dev->fq_rows : 2;
+    uint32_t want = cus * dev->fq_multi_blocks;
+    uint32_t nrb = (run + want - 1) / want;
+    nrb = (nrb + (uint32_t)r - 1) / (uint32_t)r * (uint32_t)r;
+    uint32_t grid[3] = {(run + nrb - 1) / nrb, 1, 1}, block[3] = {dev->fq_threads, 1, 1};
+    return ojh_launch(dev, r == 2 ? "gemv_fq8k_q4k_x4_r2" : "gemv_fq8k_q4k_x4_r1", p,
+                      {K, ends[0], ends[1], ends[2], ends[3], nrb, (uint32_t)(accum != 0)}, grid, block);
+}
+
 extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, const ojh_lin *w, ojh_buf *y,
                       size_t y_off, const ojh_buf *bias, uint32_t m, int accum, int act_mode) {
     if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_mm: NULL device");

@@ -88,6 +88,10 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_MOE")) d->moe_mode = atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE_DEC_TOKENS")) d->moe_dec_tokens = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_FUSED_QUANT")) d->fused_quant = atoi(r) != 0;
+    if (const char *r = getenv("OJAS_HIP_FQ_ROWS")) d->fq_rows = atoi(r) == 1 || atoi(r) == 2 ? atoi(r) : 0;
+    if (const char *r = getenv("OJAS_HIP_FQ_THREADS")) d->fq_threads = atoi(r) == 512 ? 512u : atoi(r) == 256 ? 256u : 1024u;
+    if (const char *r = getenv("OJAS_HIP_FQ_MULTI_BLOCKS")) d->fq_multi_blocks = atoi(r) > 0 ? (uint32_t)atoi(r) : 1u;
+    if (const char *r = getenv("OJAS_HIP_FQ_MULTI")) d->fq_multi = atoi(r);
     if (const char *r = getenv("OJAS_HIP_FQ_BLOCKS")) d->fq_blocks_per_cu = atoi(r) > 0 ? (uint32_t)atoi(r) : 8u;
     int rc = ojh_noalloc_setup(d);
     if (rc) {

@@ -115,6 +115,7 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_noalloc_scratch_bytes": (sz, []),
         "ojh_mm_q8k": (i32, [vp, vp, vp, vp, vp, sz, vp, u32, i32]),
         "ojh_mm_q8k_multi": (i32, [vp, vp, vp, i32, vp, vp, vp]),
+        "ojh_mm_multi": (i32, [vp, vp, sz, i32, vp, vp, vp, i32]),
         "ojh_gguf_open": (i32, [C.c_char_p, vp]),
         "ojh_gguf_close": (i32, [vp]),
         "ojh_gguf_tensor_count": (i32, [vp]),
@@ -549,6 +550,16 @@ class HipGpu:
         ya = (C.c_void_p * n)(*[y.handle for y in ys])
         oa = (C.c_size_t * n)(*y_offs) if y_offs is not None else None
         self._check(self._L.ojh_mm_q8k_multi(self._dev, xq.handle, xscales.handle, n, wa, ya, oa))
+
+    def mm_multi(self, x: Buf, ws: list, ys: list, y_offs: list | None = None, accum: bool = False, x_off: int = 0) -> None:
+        """One decode stage in one launch: up to four projections of one f32 vector, quantized inside the launch."""
+        n = len(ws)
+        if n != len(ys) or (y_offs is not None and len(y_offs) != n):
+            raise ValueError("mm_multi: ws, ys and y_offs must have the same length")
+        wa = (C.c_void_p * n)(*[w.handle for w in ws])
+        ya = (C.c_void_p * n)(*[y.handle for y in ys])
+        oa = (C.c_size_t * n)(*y_offs) if y_offs is not None else None
+        self._check(self._L.ojh_mm_multi(self._dev, x.handle, x_off, n, wa, ya, oa, int(accum)))
 
     def rmsnorm_quant_q8k(self, x: Buf, gamma: Buf, eps: float, m: int, k: int, q: Buf, scales: Buf,
                           xn: Buf | None = None, x_off: int = 0) -> None:

@@ -302,6 +302,52 @@ def test_grouped_projections_equal_separate_launches(gpu, orc, pkg, ns, k):
         assert peak_err(got[:n], orc.matvec_kq(w, Q4_K, n, k, x)) <= TOL_Q8K_SEEN
 
 
+@pytest.mark.parametrize("ns,k", [((4096, 1024, 1024), 4096), ((14336, 14336), 4096), ((13, 1, 7, 2), 512),
+                                  ((5, 300), 2560), ((33,), 256), ((40,), 14336), ((4096,), 8192)])
+@pytest.mark.parametrize("accum", [False, True])
+def test_stage_launch_with_the_quantizer_inside(gpu, orc, pkg, ns, k, accum):
+    """ojh_mm_multi: f32 activations in, one launch per stage (quantizer folded in for small Q4_K stages, a quantizer
+    launch plus the grouped launch otherwise) — every output bit-equal to quantizer + single-tensor launches, within
+    the parity bar of matvec_kq, nothing written past a tensor's rows; also with the single launch forced at every
+    size and workgroup shape."""
+    import os
+    x = pkg.synth.normal_f32(k, "stage", "x", k)
+    ws = [pkg.synth.q4k_weights(n, k, "stage", i, n, k) for i, n in enumerate(ns)]
+    y0s = [pkg.synth.normal_f32(n, "stage", "y0", i) for i, n in enumerate(ns)]
+    guard = np.float32(-7.25)
+    xd = gpu.upload(x)
+    xq, xs = gpu.alloc_bytes(k), gpu.alloc(k // 256)
+    gpu.quant_q8k(xd, 1, k, xq, xs)
+    lins = [gpu.lin(Q4_K, n, k, w) for n, w in zip(ns, ws)]
+    want = []
+    for n, lin, y0 in zip(ns, lins, y0s):
+        y1 = gpu.upload(y0)
+        gpu.mm_q8k(xq, xs, lin, y1, accum=accum)
+        want.append(gpu.read(y1, n))
+    for env in ({}, {"OJAS_HIP_FQ_MULTI": "2"}, {"OJAS_HIP_FQ_MULTI": "2", "OJAS_HIP_FQ_THREADS": "256", "OJAS_HIP_FQ_MULTI_BLOCKS": "8", "OJAS_HIP_FQ_ROWS": "1"},
+                {"OJAS_HIP_FQ_MULTI": "2", "OJAS_HIP_FQ_THREADS": "512", "OJAS_HIP_FQ_MULTI_BLOCKS": "3"}):
+        old = {k_: os.environ.get(k_) for k_ in env}
+        os.environ.update(env)
+        g2 = pkg.HipGpu(0) if env else gpu            # the settings are read when a device is opened
+        try:
+            l2 = lins if not env else [g2.lin(Q4_K, n, k, w) for n, w in zip(ns, ws)]
+            ys = [g2.upload(np.concatenate([y0, np.full(4, guard, np.float32)])) for y0 in y0s]
+            g2.mm_multi(g2.upload(x), l2, ys, accum=accum)
+            for n, w, y, wnt, y0 in zip(ns, ws, ys, want, y0s):
+                got = g2.read(y, n + 4)
+                assert np.all(got[n:] == guard), env
+                assert np.array_equal(got[:n].view(np.uint32), wnt.view(np.uint32)), env
+                assert peak_err(got[:n] - (y0 if accum else 0), orc.matvec_kq(w, Q4_K, n, k, x)) <= TOL_Q8K_SEEN
+        finally:
+            for k_, v_ in old.items():
+                if v_ is None:
+                    os.environ.pop(k_, None)
+                else:
+                    os.environ[k_] = v_
+            if env:
+                g2.close()
+
+
 def test_grouped_projections_other_formats_and_errors(gpu, orc, pkg):
     k = 512
     x = pkg.synth.normal_f32(k, "multi", "x6", k)
@@ -320,6 +366,16 @@ def test_grouped_projections_other_formats_and_errors(gpu, orc, pkg):
         gpu.mm_q8k_multi(xq, xs, [l4] * 5, [y4] * 5)
     with pytest.raises(pkg.OjasHipError, match="needs"):
         gpu.mm_q8k_multi(xq, xs, [l4, l4], [y4, y6])
+    # the stage entry over mixed formats: a quantizer launch, then one launch per format
+    xd = gpu.upload(x)
+    gpu.memset0(y4)
+    gpu.memset0(y6)
+    gpu.mm_multi(xd, [l4, l6], [y4, y6])
+    assert peak_err(gpu.read(y4, 40), orc.matvec_kq(w4, Q4_K, 40, k, x)) <= TOL_Q8K_SEEN
+    assert peak_err(gpu.read(y6, 24), orc.matvec_kq(w6, Q6_K, 24, k, x)) <= TOL_Q8K_SEEN
+    q80 = gpu.lin(8, 8, k, pkg.synth.q80_weights(8, k, "multi", "q80"))
+    with pytest.raises(pkg.OjasHipError, match="need no quantizer"):
+        gpu.mm_multi(xd, [q80], [y4])
 
 
 @pytest.mark.parametrize("m,n,k,accum", [(3, 50, 256, False), (4, 130, 14336, True), (16, 301, 4096, False),
