@@ -131,6 +131,61 @@ __device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restri
                     const uint sc_lo = cur.hdr.y & 0x3F3F3F3Fu, mn_lo = cur.hdr.z & 0x3F3F3F3Fu;
                     const uint sc_hi = (cur.hdr.w & 0x0F0F0F0Fu) | ((cur.hdr.y >> 2) & 0x30303030u);
                     const uint mn_hi = ((cur.hdr.w >> 4) & 0x0F0F0F0Fu) | ((cur.hdr.z >> 2) & 0x30303030u);
+                    const long Bm = kg == 0u ? gq_pack(mn_lo, mn_hi) : 0;    // only positions 0..7 carry mins
+                    if (P >= 2) {
+                        // Several passes share the row tile: fold the 6-bit scales into the codes once instead of
+                        // into every result.  sc = 8 sh + sl with sl, sh <= 7, so sl * q and sh * q (<= 105) are
+                        // int8 again and a packed 16-bit multiply scales four codes at once without a carry between
+                        // bytes; two accumulating MFMAs per sub-block then give  sum_j sl_j idot_j  and
+                        // sum_j sh_j idot_j, and  sum_j sc_j idot_j = 8 * (the second) + (the first)  exactly.
+                        // One v_mfma_i32_16x16x64_i8 then covers a whole 64-weight chunk — its low-nibble
+                        // sub-block in positions 0..7 of the lane's sixteen, its high-nibble sub-block in positions
+                        // 8..15, each under its own folded scale — against the lane's 8 + 8 activations of the two
+                        // sub-blocks (what matters is that A and B put the same weight position in the same slot).
+                        gq_i4 BA[4], BB[4];
+#pragma unroll
+                        for (int c = 0; c < 4; c++) {
+                            // chunk c = sub-blocks 2c (low nibbles) and 2c + 1 (high nibbles)
+                            const uint se = 2 * c < 4 ? (sc_lo >> (16 * c)) & 0xFFu : (sc_hi >> (16 * (c - 2))) & 0xFFu;
+                            const uint so = 2 * c < 4 ? (sc_lo >> (16 * c + 8)) & 0xFFu : (sc_hi >> (16 * (c - 2) + 8)) & 0xFFu;
+                            const gq_u16x2 el = {(ushort)(se & 7u), (ushort)(se & 7u)}, eh = {(ushort)(se >> 3), (ushort)(se >> 3)};
+                            const gq_u16x2 ol = {(ushort)(so & 7u), (ushort)(so & 7u)}, oh = {(ushort)(so >> 3), (ushort)(so >> 3)};
+                            const uint2 qq = cur.q[c];
+                            const uint lx = qq.x & 0x0F0F0F0Fu, ly = qq.y & 0x0F0F0F0Fu;
+                            const uint hx = (qq.x >> 4) & 0x0F0F0F0Fu, hy = (qq.y >> 4) & 0x0F0F0F0Fu;
+                            BA[c] = (gq_i4){(int)gq_mul4(lx, el), (int)gq_mul4(ly, el), (int)gq_mul4(hx, ol), (int)gq_mul4(hy, ol)};
+                            BB[c] = (gq_i4){(int)gq_mul4(lx, eh), (int)gq_mul4(ly, eh), (int)gq_mul4(hx, oh), (int)gq_mul4(hy, oh)};
+                        }
+#pragma unroll
+                        for (int p = 0; p < P; p++) {
+                            const uchar* xp = xa + (size_t)(16 * p) * S + s * 256u;
+                            gq_i4 DA0 = zero, DA1 = zero, DB0 = zero, DB1 = zero;
+#pragma unroll
+                            for (int c = 0; c < 4; c += 2) {
+                                const uint2 a00 = *(const uint2*)(xp + 64 * c), a01 = *(const uint2*)(xp + 64 * c + 32);
+                                const uint2 a10 = *(const uint2*)(xp + 64 * c + 64), a11 = *(const uint2*)(xp + 64 * c + 96);
+                                const gq_i4 A0 = {(int)a00.x, (int)a00.y, (int)a01.x, (int)a01.y};
+                                const gq_i4 A1 = {(int)a10.x, (int)a10.y, (int)a11.x, (int)a11.y};
+                                DA0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A0, BA[c], DA0, 0, 0, 0);
+                                DB0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A0, BB[c], DB0, 0, 0, 0);
+                                DA1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, BA[c + 1], DA1, 0, 0, 0);
+                                DB1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, BB[c + 1], DB1, 0, 0, 0);
+                            }
+                            const uchar* pq = lbq + ((size_t)s * BM + 16u * p + n) * 16u;
+                            long Alo = 0, Ahi = 0;
+                            if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
+                            const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
+                            const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
+                            const float4 sx = *(const float4*)(lsx + s * BM + 16u * p + 4u * kg);
+                            const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
+#pragma unroll
+                            for (int v = 0; v < 4; v++) {
+                                const int isum = 8 * (DB0[v] + DB1[v]) + (DA0[v] + DA1[v]);
+                                acc[q][p][v] += sxv[v] * (d * (float)isum - dmin * (float)(64 * Dhi[v] + Dlo[v]));
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    } else {
                     int sc[8];
                     long B[8];
 #pragma unroll
@@ -140,7 +195,6 @@ __device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restri
                         B[2 * c] = gq_pack(cur.q[c].x & 0x0F0F0F0Fu, cur.q[c].y & 0x0F0F0F0Fu);
                         B[2 * c + 1] = gq_pack((cur.q[c].x >> 4) & 0x0F0F0F0Fu, (cur.q[c].y >> 4) & 0x0F0F0F0Fu);
                     }
-                    const long Bm = kg == 0u ? gq_pack(mn_lo, mn_hi) : 0;    // only positions 0..7 carry mins
 #pragma unroll
                     for (int p = 0; p < P; p++) {
                         int isum[4] = {0, 0, 0, 0};
@@ -166,6 +220,7 @@ __device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restri
                         // (keeps the passes apart: let loose, the scheduler hoists every pass's reads and
                         // products to the front and the kernel spills)
                         __builtin_amdgcn_sched_barrier(0);
+                    }
                     }
                     cur = nx;
                     // the tokens are read from LDS again for the next row tile: kept in registers across

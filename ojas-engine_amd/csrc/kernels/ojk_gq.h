@@ -7,6 +7,13 @@ typedef int gq_i4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ long gq_pack(uint lo, uint hi) { return (long)(((unsigned long)hi << 32) | lo); }
 
+// Four codes (a byte each, <= 15) times a factor <= 7 given as a pair of equal 16-bit halves: no byte's product
+// (<= 105) carries into its neighbour, so one packed 16-bit multiply scales all four.
+typedef ushort gq_u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint gq_mul4(uint codes, gq_u16x2 f) {
+    return __builtin_bit_cast(uint, __builtin_bit_cast(gq_u16x2, codes) * f);
+}
+
 struct GqW {            // lane (n, kg): its bytes of one super-block of row n
     uint4 hdr;          // d, dmin, the 12 scale bytes
     uint2 q[4];         // codes of positions 8 kg .. 8 kg + 7 of each 64-weight chunk (low | high nibbles)

@@ -83,6 +83,34 @@ def test_q6k_verify_head_at_full_size(gpu, orc, pkg, m):
 
 
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("m", [128, 512])
+def test_prefill_in_the_cpu_arithmetic_at_full_size(gpu, orc, pkg, n, k, m):
+    """The same shapes under OJH_ACT_Q8K — activations quantized per 256, integer dots on the int8 matrix cores —
+    against `matvec_kq`, the CPU reference itself, token by token on sampled weight rows (tile borders included):
+    the prefill path that meets the parity bar of the CPU reference.  A token's outputs do not depend on its
+    position in the batch (bit for bit)."""
+    w = pkg.synth.q4k_weights(n, k, "full", "gemm", n, k)
+    xb = pkg.synth.to_bf16_bits(pkg.synth.normal_f32(m * k, "full", "q8k-x", m, k))
+    xf = pkg.synth.bf16_bits_to_f32(xb).reshape(m, k)
+    lin = gpu.lin(Q4_K, n, k, w)
+    yd = gpu.upload(np.full(m * n + 64, 12345.5, np.float32))
+    gpu.mm(gpu.upload_bytes(xb), lin, yd, m, x_dtype=pkg.X_BF16, act_mode=pkg.ACT_Q8K)
+    got = gpu.read(yd, m * n + 64)
+    assert np.all(got[m * n:] == 12345.5), "wrote past row M"
+    got = got[:m * n].reshape(m, n)
+    g = pkg.synth.rng("full", "q8k-rows", n, k, m)
+    rows = np.unique(np.concatenate([[0, 15, 16, 63, 64, n - 17, n - 1], g.integers(0, n, 25)]))
+    wsub = _rows(w, Q4_K, pkg, k, rows)
+    for t in range(m):
+        want = orc.matvec_kq(wsub, Q4_K, len(rows), k, xf[t], threads=1 if len(rows) < 64 else 8)
+        assert peak_err(got[t, rows], want) <= 2e-5, t
+    perm = np.roll(np.arange(m), 37)
+    y2 = gpu.alloc(m * n)
+    gpu.mm(gpu.upload_bytes(xb.reshape(m, k)[perm].copy()), lin, y2, m, x_dtype=pkg.X_BF16, act_mode=pkg.ACT_Q8K)
+    assert np.array_equal(gpu.read(y2, m * n).reshape(m, n), got[perm])
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
 @pytest.mark.parametrize("m", [512, 2048])
 def test_prefill_gemm_at_full_size(gpu, orc, pkg, n, k, m):
     """Q4_K gate/up and down shapes, bf16 activations: 48 sampled weight rows against every token
