@@ -172,8 +172,9 @@ __device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restri
                                 DB1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, BB[c + 1], DB1, 0, 0, 0);
                             }
                             const uchar* pq = lbq + ((size_t)s * BM + 16u * p + n) * 16u;
-                            long Alo = 0, Ahi = 0;
-                            if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
+                            // (masked, not branched over: a branch here splits the unrolled code into basic blocks and costs registers)
+                            const long km_ = kg == 0u ? -1l : 0l;
+                            const long Alo = *(const long*)pq & km_, Ahi = *(const long*)(pq + 8) & km_;
                             const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
                             const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
                             const float4 sx = *(const float4*)(lsx + s * BM + 16u * p + 4u * kg);
@@ -208,8 +209,9 @@ __device__ __forceinline__ void gemm_q8k_q4k_mf_body(const signed char* __restri
                         }
                         // token n of this pass: its eight lo parts, then its eight hi parts (lanes kg = 0 only)
                         const uchar* pq = lbq + ((size_t)s * BM + 16u * p + n) * 16u;
-                        long Alo = 0, Ahi = 0;
-                        if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
+                        // (masked, not branched over: a branch here splits the unrolled code into basic blocks and costs registers)
+                        const long km_ = kg == 0u ? -1l : 0l;
+                        const long Alo = *(const long*)pq & km_, Ahi = *(const long*)(pq + 8) & km_;
                         const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
                         const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
                         const float4 sx = *(const float4*)(lsx + s * BM + 16u * p + 4u * kg);
@@ -471,4 +473,211 @@ gemm_q8k_q4k_mk(const signed char* xq, const float* xs, const uchar* w, float* y
         }
         __syncthreads();                           // before the next tile's partial sums
     }
+}
+
+// ---- prefill-sized batches: 128 tokens x 128 rows per workgroup, tokens copied into LDS by the memory system ----
+//   q8k_token_sides(xq, xs, xst, sums, K, M, MP)      grid [K / 256, ceil(MP / 256), 1], block 256
+//       xst [K/256][MP] f32: the token scales, super-block major;  sums [K/256][MP][16] int8: every 32-position sum of a
+//       token's activations split as 64 hi + lo (eight lo parts, then eight hi parts); rows M .. MP - 1 are zeros.
+//   gemm_q8k_q4k_xt(xq, xst, sums, w, y, K, N, M, ACC, MP)    grid [ceil(N / 128), MP / 128, 1], block 512;  MP = M rounded up to 128
+//   gemm_q8k_q4k_xt64(the same)                                grid [ceil(N / 64), MP / 128, 1]
+//
+// gemm_q8k_q4k_mf stages its tokens through registers, one chunk of K at a time, with nothing else going on: from
+// a hundred tokens up that staging, not the arithmetic, is what the launch waits for.  Here a workgroup owns
+// 128 tokens x 128 rows and walks K one super-block per step; the step's tokens (32 KB), their scales and split
+// sums travel global -> LDS by global_load_lds_dwordx4 into the stage the previous step is not reading, and are
+// awaited with one s_waitcnt + barrier per step.  A token row is 256 bytes; its 16-byte piece j sits in slot
+// j ^ (token % 16), applied on the global side of the copy, so that the sixteen tokens of a pass read a given piece
+// from sixteen different bank groups.  A wave owns one 16-row tile and the eight passes of 16 tokens (the _xt64 entry:
+// 64 rows per workgroup, two waves per tile with four passes each, for matrices with few rows): the tile's
+// weights, scales folded into two int8 planes (see gemm_q8k_q4k_mf), are built once per step, and every 16 bytes of
+// activations read from LDS feed four v_mfma_i32_16x16x64_i8 (two tiles x two planes).  The weights of the next step
+// are ordinary loads into registers, issued a step ahead.  Same arithmetic per (token, row, super-block) as
+// gemm_q8k_q4k_mf, super-blocks added in order: the same bits.
+#define GXT_TOK 128u
+#define GXT_ROWS 128u
+#define GXT_STAGE (GXT_TOK * 256u + GXT_TOK * 16u + GXT_TOK * 4u)     // tokens | split sums | scales = 35328 bytes
+
+extern "C" __global__ void __launch_bounds__(256)
+q8k_token_sides(const signed char* __restrict__ xq, const float* __restrict__ xs, float* __restrict__ xst,
+                uchar* __restrict__ sums, uint K, uint M, uint MP) {
+    const uint nsb = K >> 8, sb = blockIdx.x, t = blockIdx.y * 256u + threadIdx.x;
+    if (t >= MP) return;
+    uint lo[2] = {0u, 0u}, hi[2] = {0u, 0u};
+    float sc = 0.0f;
+    if (t < M) {
+        sc = xs[(size_t)t * nsb + sb];
+        const uint4* px = (const uint4*)(xq + (size_t)t * K + (size_t)sb * 256u);
+#pragma unroll
+        for (int jj = 0; jj < 8; jj++) {
+            const uint4 a = px[2 * jj], b = px[2 * jj + 1];
+            int bs = dot4_i8(a.x, 0x01010101u, 0);
+            bs = dot4_i8(a.y, 0x01010101u, bs); bs = dot4_i8(a.z, 0x01010101u, bs); bs = dot4_i8(a.w, 0x01010101u, bs);
+            bs = dot4_i8(b.x, 0x01010101u, bs); bs = dot4_i8(b.y, 0x01010101u, bs);
+            bs = dot4_i8(b.z, 0x01010101u, bs); bs = dot4_i8(b.w, 0x01010101u, bs);
+            lo[jj >> 2] |= (uint)(bs & 63) << (8 * (jj & 3));
+            hi[jj >> 2] |= ((uint)(bs >> 6) & 0xFFu) << (8 * (jj & 3));
+        }
+    }
+    xst[(size_t)sb * MP + t] = sc;
+    *(uint4*)(sums + ((size_t)sb * MP + t) * 16u) = make_uint4(lo[0], lo[1], hi[0], hi[1]);
+}
+
+__device__ __forceinline__ void gxt_copy16(const void* base, uint voff, uint lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr) : "memory");
+}
+
+// the two planes of one 16-row tile's super-block: BA = (sc & 7) * code, BB = (sc >> 3) * code, a chunk per register quad
+__device__ __forceinline__ void gxt_planes(const GqW& w, gq_i4 (&BA)[4], gq_i4 (&BB)[4], long& Bm, float& d, float& dmin, uint kg) {
+    d = f16_bits_to_f32(w.hdr.x & 0xFFFFu);
+    dmin = f16_bits_to_f32(w.hdr.x >> 16);
+    const uint sc_lo = w.hdr.y & 0x3F3F3F3Fu, mn_lo = w.hdr.z & 0x3F3F3F3Fu;
+    const uint sc_hi = (w.hdr.w & 0x0F0F0F0Fu) | ((w.hdr.y >> 2) & 0x30303030u);
+    const uint mn_hi = ((w.hdr.w >> 4) & 0x0F0F0F0Fu) | ((w.hdr.z >> 2) & 0x30303030u);
+    Bm = kg == 0u ? gq_pack(mn_lo, mn_hi) : 0;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const uint se = 2 * c < 4 ? (sc_lo >> (16 * c)) & 0xFFu : (sc_hi >> (16 * (c - 2))) & 0xFFu;
+        const uint so = 2 * c < 4 ? (sc_lo >> (16 * c + 8)) & 0xFFu : (sc_hi >> (16 * (c - 2) + 8)) & 0xFFu;
+        const gq_u16x2 el = {(ushort)(se & 7u), (ushort)(se & 7u)}, eh = {(ushort)(se >> 3), (ushort)(se >> 3)};
+        const gq_u16x2 ol = {(ushort)(so & 7u), (ushort)(so & 7u)}, oh = {(ushort)(so >> 3), (ushort)(so >> 3)};
+        const uint2 qq = w.q[c];
+        const uint lx = qq.x & 0x0F0F0F0Fu, ly = qq.y & 0x0F0F0F0Fu;
+        const uint hx = (qq.x >> 4) & 0x0F0F0F0Fu, hy = (qq.y >> 4) & 0x0F0F0F0Fu;
+        BA[c] = (gq_i4){(int)gq_mul4(lx, el), (int)gq_mul4(ly, el), (int)gq_mul4(hx, ol), (int)gq_mul4(hy, ol)};
+        BB[c] = (gq_i4){(int)gq_mul4(lx, eh), (int)gq_mul4(ly, eh), (int)gq_mul4(hx, oh), (int)gq_mul4(hy, oh)};
+    }
+}
+
+// TH = 1: eight row tiles (128 rows) per workgroup, a wave takes one of them against all eight passes of 16 tokens;
+// TH = 2: four row tiles (64 rows), two waves per tile with four passes each — for matrices with too few rows to give
+// every CU a 128-row tile.
+template <int TH>
+__device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restrict__ xq, const float* __restrict__ xst,
+                                                     const uchar* __restrict__ sums, const uchar* __restrict__ w,
+                                                     float* __restrict__ y, uint K, uint N, uint M, uint ACC, uint MP, uchar* lds) {
+    constexpr int P = 8 / TH;
+    constexpr uint RT = 8u / TH;                                    // row tiles per workgroup
+    const uint tid = threadIdx.x, lane = tid & 63u;
+    const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint rt = wave % RT, th = wave / RT;                     // the wave's 16 rows and its 16 P tokens
+    const uint nsb = K >> 8, n = lane & 15u, kg = lane >> 4;
+    const uint t0 = blockIdx.y * GXT_TOK, r0 = blockIdx.x * (16u * RT) + rt * 16u;
+    const uint lds0 = (uint)(size_t)(__attribute__((address_space(3))) uchar*)lds;
+    const gq_i4 zero = {0, 0, 0, 0};
+
+    // copies of one step: 32 of 1 KB for the tokens (wave w takes tokens 16 w .. 16 w + 15, four per copy: lane ->
+    // token lane / 16 of the four, slot lane % 16, which holds the token's piece slot ^ (token % 16)), two for the
+    // split sums (128 tokens x 16 bytes, contiguous in `sums`), one of 512 bytes for the scales.
+    const uint lane16 = lane * 16u;
+    const uint x_lds = lds0 + wave * 4096u;                        // + stage * GXT_STAGE + i * 1024
+    auto copies = [&](uint sb, uint stage) {
+        const uchar* xb = (const uchar*)xq + (size_t)sb * 256u;
+        // (the four source offsets are formed again at every step — a dozen instructions — rather than kept in
+        // registers across the loop, which this kernel does not have: the lane id is made opaque to stop the hoisting)
+        uint lo = lane;
+        asm volatile("" : "+v"(lo));
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint tk = wave * 16u + (uint)i * 4u + (lo >> 4);
+            const uint tg = min(t0 + tk, M - 1u);                  // tokens past M: any row (their sides are zeros)
+            gxt_copy16(xb, tg * K + (((lo & 15u) ^ (tk & 15u)) << 4), x_lds + stage * GXT_STAGE + (uint)i * 1024u);
+        }
+        if (wave < 2u) gxt_copy16(sums + ((size_t)sb * MP + t0) * 16u + wave * 1024u, lane16,
+                                  lds0 + stage * GXT_STAGE + GXT_TOK * 256u + wave * 1024u);
+        else if (wave == 2u) {
+            if (lane < 32u) gxt_copy16(xst + (size_t)sb * MP + t0, lane16, lds0 + stage * GXT_STAGE + GXT_TOK * 272u);
+        }
+    };
+    // this lane's row (clamped past N; a 32-bit byte offset from a uniform base: the tensor stays below 4 GiB)
+    const uint wrow = min(r0 + n, N - 1u) * nsb * Q4K_BYTES;
+
+    float acc[P][4];
+#pragma unroll
+    for (int p = 0; p < P; p++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[p][v] = 0.0f;
+
+    // byte offsets of the lane's pieces within a token row, per chunk: pieces 4 c + kg / 2 (first sub-block) and
+    // 4 c + 2 + kg / 2 (second), slot = piece ^ (token % 16), half kg % 2
+    const uint tok_lds = (th * (16u * P) + n) * 256u + 8u * (kg & 1u);
+    // (the second piece's slot differs from the first's in bit 1 only: its byte offset is the first's ^ 32)
+    uint o0[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) o0[c] = tok_lds + (((4u * (uint)c + (kg >> 1)) ^ n) << 4);
+    const uint side_lds = GXT_TOK * 256u + (th * (16u * P) + n) * 16u, sc_lds = GXT_TOK * 272u + (th * (16u * P) + 4u * kg) * 4u;
+    // (only positions 0..7 carry split sums; masked rather than branched over: a branch inside the unrolled passes cuts
+    // the step into many basic blocks, which the register allocator answers with spills)
+    const long kmask = kg == 0u ? -1l : 0l;
+
+    GqW cur = gq_load(w + wrow, kg);
+    copies(0u, 0u);
+    for (uint sb = 0; sb < nsb; sb++) {
+        const uint stage = sb & 1u;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();                                            // stage `stage` complete; the other one is free
+        if (sb + 1u < nsb) copies(sb + 1u, stage ^ 1u);
+        const uint sbn = min(sb + 1u, nsb - 1u);
+        const uchar* st = lds + stage * GXT_STAGE;
+        gq_i4 BA[4], BB[4];
+        long Bm;
+        float d, dmin;
+        gxt_planes(cur, BA, BB, Bm, d, dmin, kg);
+        __builtin_amdgcn_sched_barrier(0);
+        // the next step's weights take over the registers of this step's raw bytes, which the planes have replaced
+        cur = gq_load((w + (size_t)sbn * Q4K_BYTES) + wrow, kg);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            // (one accumulation chain per plane: the two chains alternate, which is distance enough between dependent
+            // MFMAs here, and saves the registers and the additions of split chains)
+            gq_i4 DA = zero, DB = zero;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const uint2 a0 = *(const uint2*)(st + o0[c] + 4096u * (uint)p), a1 = *(const uint2*)(st + (o0[c] ^ 32u) + 4096u * (uint)p);
+                const gq_i4 A = {(int)a0.x, (int)a0.y, (int)a1.x, (int)a1.y};
+                DA = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, BA[c], DA, 0, 0, 0);
+                DB = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, BB[c], DB, 0, 0, 0);
+            }
+            const uchar* pq = st + side_lds + 256u * (uint)p;
+            const long Alo = *(const long*)pq & kmask, Ahi = *(const long*)(pq + 8) & kmask;
+            const float4 sx = *(const float4*)(st + sc_lds + 64u * (uint)p);
+            const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
+            const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
+            const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int isum = 8 * DB[v] + DA[v];
+                acc[p][v] += sxv[v] * (d * (float)isum - dmin * (float)(64 * Dhi[v] + Dlo[v]));
+            }
+            // (keeps the passes apart: let loose, the scheduler hoists every pass's reads to the front)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // (the lane id asked of the hardware again, so that nothing of it has to live through the loop)
+    const uint le = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const uint r = blockIdx.x * (16u * RT) + rt * 16u + (le & 15u);
+#pragma unroll
+    for (int p = 0; p < P; p++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const uint t = t0 + th * (16u * P) + 16u * (uint)p + 4u * (le >> 4) + (uint)v;
+            if (t < M && r < N) {
+                float* o = y + (size_t)t * N + r;
+                *o = ACC ? *o + acc[p][v] : acc[p][v];
+            }
+        }
+}
+
+extern "C" __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
+gemm_q8k_q4k_xt(const signed char* xq, const float* xst, const uchar* sums, const uchar* w, float* y, uint K, uint N, uint M,
+                uint ACC, uint MP) {
+    __shared__ __attribute__((aligned(1024))) uchar lds_xt[2 * GXT_STAGE];
+    gemm_q8k_q4k_xt_body<1>(xq, xst, sums, w, y, K, N, M, ACC, MP, lds_xt);
+}
+extern "C" __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
+gemm_q8k_q4k_xt64(const signed char* xq, const float* xst, const uchar* sums, const uchar* w, float* y, uint K, uint N, uint M,
+                  uint ACC, uint MP) {
+    __shared__ __attribute__((aligned(1024))) uchar lds_xt[2 * GXT_STAGE];
+    gemm_q8k_q4k_xt_body<2>(xq, xst, sums, w, y, K, N, M, ACC, MP, lds_xt);
 }

@@ -58,8 +58,9 @@ __device__ __forceinline__ void gq_superblock(const GqW& cur, const uchar* xp, c
 #pragma unroll
         for (int v = 0; v < 4; v++) isum[v] += __mul24(sc[jj], D[v]);
     }
-    long Alo = 0, Ahi = 0;
-    if (kg == 0u) { Alo = *(const long*)pq; Ahi = *(const long*)(pq + 8); }
+    // (masked, not branched over: a branch here splits the unrolled code into basic blocks and costs registers)
+    const long km_ = kg == 0u ? -1l : 0l;
+    const long Alo = *(const long*)pq & km_, Ahi = *(const long*)(pq + 8) & km_;
     const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
     const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
     const float4 sx = *(const float4*)(sx16 + 4u * kg);

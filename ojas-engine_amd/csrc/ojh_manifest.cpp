@@ -194,6 +194,53 @@ void ojh_gemm_q8k_tiles(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t 
     *rw_out = rw;
     *rt_out = 1;
 }
+// q8k_token_sides(xq, xs, xst, sums, K, M, MP): grid [K / 256, ceil(MP / 256), 1] x 256
+// gemm_q8k_q4k_xt(xq, xst, sums, w, y, K, N, M, ACC, MP): grid [ceil(N / 128), MP / 128, 1] x 512; MP = M rounded up to 128
+static int check_gemm_q8k_xt(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                             const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const bool sides = s->rows_per_wave == 0;
+    const uint32_t K = c[0], N = sides ? 1 : c[1], M = sides ? c[1] : c[2], MP = sides ? c[2] : c[4];
+    if (!K || K % 256 || !N || !M) return ojh_fail(OJH_ERR_ARG, "%s: K=%u (a multiple of 256) N=%u M=%u", s->name, K, N, M);
+    if (MP != (M + 127) / 128 * 128) return ojh_fail(OJH_ERR_ARG, "%s: MP=%u must be M=%u rounded up to 128", s->name, MP, M);
+    if ((uint64_t)M * K > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "%s: M*K exceeds 2^32 activations", s->name);
+    const size_t nsb = K / 256;
+    int rc;
+    if (sides) {
+        if ((rc = check_block(block, 256))) return rc;
+        if (grid[0] != nsb || grid[1] != (MP + 255) / 256 || grid[2] != 1)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%zu,%u,1]", s->name, nsb, (MP + 255) / 256);
+        need[0] = (size_t)M * K;
+        need[1] = (size_t)M * nsb * 4;
+        need[2] = nsb * MP * 4;
+        need[3] = nsb * MP * 16;
+        align[1] = align[2] = 4;
+        return OJH_OK;
+    }
+    if (c[3] > 1) return ojh_fail(OJH_ERR_ARG, "%s: ACC=%u", s->name, c[3]);
+    if ((rc = check_block(block, 512))) return rc;
+    const uint32_t br = s->rows_per_wave == 2 ? 64 : 128;
+    if (grid[0] != (N + br - 1) / br || grid[1] != MP / 128 || grid[2] != 1)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,1]", s->name, (N + br - 1) / br, MP / 128);
+    if ((uint64_t)N * nsb * 144 > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "%s: the weight tensor exceeds 4 GiB", s->name);
+    need[0] = (size_t)M * K;
+    need[1] = nsb * MP * 4;
+    need[2] = nsb * MP * 16;
+    need[3] = (size_t)N * nsb * 144;
+    need[4] = (size_t)M * N * 4;
+    align[1] = align[4] = 4;
+    return OJH_OK;
+}
+static int shape_gemm_q8k_xt(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, uint32_t N, uint32_t M,
+                             uint32_t grid[3], uint32_t block[3]) {
+    if (!M) M = 1;
+    const uint32_t MP = (M + 127) / 128 * 128;
+    if (s->rows_per_wave == 0) { grid[0] = K / 256; grid[1] = (MP + 255) / 256; block[0] = 256; }
+    else { const uint32_t br = s->rows_per_wave == 2 ? 64 : 128; grid[0] = (N + br - 1) / br; grid[1] = MP / 128; block[0] = 512; }
+    if (!grid[0]) grid[0] = 1;
+    grid[2] = 1;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
 static int shape_gemm_q8k(const ojh_kernel_spec *, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
                           uint32_t grid[3], uint32_t block[3]) {
     if (!M) M = 1;
@@ -1201,6 +1248,9 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     }
     add("gemm_q8k_q4k_mf", "gemm_q8k", 4, 6, OJH_Q4_K, 1, check_gemm_q8k, shape_gemm_q8k);
     add("gemm_q8k_q4k_ml", "gemm_q8k", 4, 4, OJH_Q4_K, 1, check_gemm_q8k_ml, shape_ml);
+    add("q8k_token_sides", "gemm_q8k", 4, 3, 0, 0, check_gemm_q8k_xt, shape_gemm_q8k_xt);
+    add("gemm_q8k_q4k_xt", "gemm_q8k", 5, 5, OJH_Q4_K, 1, check_gemm_q8k_xt, shape_gemm_q8k_xt);
+    add("gemm_q8k_q4k_xt64", "gemm_q8k", 5, 5, OJH_Q4_K, 2, check_gemm_q8k_xt, shape_gemm_q8k_xt);
     add("gemm_q8k_q4k_mk", "gemm_q8k", 4, 4, OJH_Q4_K, 2, check_gemm_q8k_ml, shape_mk);
     add("relayout_q4k_q4l", "dequant", 4, 1, OJH_Q4_K, 0, check_relayout, shape_relayout);
     add("embed_q80", "dequant", 2, 2, OJH_Q8_0, 0, check_embed, shape_embed);

@@ -66,5 +66,8 @@ extern "C" int ojh_mm_noalloc(ojh_device *dev, const ojh_buf *x, size_t x_off, i
         return ojh_fail(OJH_ERR_NOT_LOADED, "ojh_mm_noalloc: ensure_family(\"gemv_q8k\") and (\"gemm_q8k\") first");
     void *xq = dev->noalloc_scratch, *xs = (char *)dev->noalloc_scratch + OJH_NOALLOC_MAX_ACT;
     if ((rc = ojh_quant_q8k_launch(dev, (const char *)x->ptr + x_off, x_dtype, m, K, xq, xs))) return rc;
-    return ojh_mm_q8k_launch(dev, xq, xs, w, f, (char *)y->ptr + y_off, bias, m, accum);
+    dev->no_scratch = true;    // kernels that need further library scratch (which would be allocated) are not taken
+    rc = ojh_mm_q8k_launch(dev, xq, xs, w, f, (char *)y->ptr + y_off, bias, m, accum);
+    dev->no_scratch = false;
+    return rc;
 }

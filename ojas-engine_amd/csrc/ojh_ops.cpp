@@ -2,6 +2,7 @@
 // router that picks a kernel per call — the role `Lin::load` and `CudaSsm::mm` play in the
 // reference (crates/ojas-cuda/src/qwen35.rs:174-201, :644-702; Metal twin
 // crates/ojas-models/src/decoder/dispatch.rs:288-626).
+#include <cstdlib>
 #include <cstring>
 
 #include "ojh_internal.h"
@@ -169,6 +170,29 @@ int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, con
         std::vector<void *> p = {xq, xs, wp, yp};
         if (bias) p.push_back(bias->ptr);
         return ojh_launch(dev, name.c_str(), p, {K, N}, grid, block);
+    }
+    // Q4_K rows against a prefill-sized batch: 128 x 128 tiles, the tokens copied into LDS by the memory system
+    // (needs two side arrays, built by one small launch into the library's scratch)
+    // (taken when its tiles cover at least half of the CUs: a 4096-row matrix against 128 tokens stays below)
+    const uint32_t xt_mp = (m + 127) / 128 * 128;
+    if (w->type == OJH_Q4_K && dev->q4k_xt_min_m && m >= dev->q4k_xt_min_m && !dev->no_scratch &&
+        (uint64_t)((N + 63) / 64) * (xt_mp / 128) * 2 >= (uint32_t)dev->prop.multiProcessorCount &&
+        (uint64_t)m * K <= 0xFFFFFFFFull && (uint64_t)w->row_bytes * N <= 0xFFFFFFFFull && (uintptr_t)wp % 16 == 0) {
+        int rc = ensure(dev, "gemm_q8k");
+        if (rc) return rc;
+        const uint32_t mp = (m + 127) / 128 * 128;
+        const size_t nsb = K / 256;
+        ojh_buf *xst, *sums;
+        if ((rc = ojh_scratch_get(dev, "xt_xst", nsb * mp * 4, &xst))) return rc;
+        if ((rc = ojh_scratch_get(dev, "xt_sums", nsb * mp * 16, &sums))) return rc;
+        uint32_t sg[3], sb[3];
+        if ((rc = ojh_launch_shape(dev, "q8k_token_sides", K, N, m, sg, sb))) return rc;
+        if ((rc = ojh_launch(dev, "q8k_token_sides", {xq, xs, xst->ptr, sums->ptr}, {K, m, mp}, sg, sb))) return rc;
+        // 128-row tiles when they give every CU one, 64-row tiles otherwise
+        const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;
+        const char *xt = (uint64_t)((N + 127) / 128) * (mp / 128) >= cus && !getenv("OJAS_HIP_Q4K_XT64") ? "gemm_q8k_q4k_xt" : "gemm_q8k_q4k_xt64";
+        if ((rc = ojh_launch_shape(dev, xt, K, N, m, sg, sb))) return rc;
+        return ojh_launch(dev, xt, {xq, xst->ptr, sums->ptr, wp, yp}, {K, N, m, (uint32_t)(accum != 0), mp}, sg, sb);
     }
     // Q4_K rows against several tokens: the int8 matrix cores, in the shape measured fastest on K = 4096 and 14336.
     // A long matrix (six 16-row tiles per CU and wave: 24576 rows on this GPU) against 2 .. 16 tokens: a wave

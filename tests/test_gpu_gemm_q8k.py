@@ -148,3 +148,48 @@ def test_a_token_does_not_depend_on_its_batch(gpu, pkg):
     perm = np.roll(np.arange(m), 37)
     gpu.mm(gpu.upload(x[perm].copy()), lin, y2, m, act_mode=pkg.ACT_Q8K)
     assert np.array_equal(gpu.read(y2, m * n).reshape(m, n), gpu.read(y1, m * n).reshape(m, n)[perm])
+
+
+@pytest.mark.parametrize("m,n,k", [(130, 200, 512), (128, 128, 256), (300, 77, 2048), (97, 1000, 4096)])
+def test_prefill_tiles_by_name(gpu, orc, pkg, m, n, k):
+    """`q8k_token_sides` + `gemm_q8k_q4k_xt` / `_xt64` by name: ragged tokens and rows, plain store and accumulate,
+    nothing written past row M — against matvec_kq and, bit for bit, against `gemm_q8k_q4k_mf` with one wave per row
+    tile over all of K (RW = 4: super-blocks added in order there too)."""
+    w, x = _case(pkg, m, n, k, "xt")
+    gpu.ensure_family("gemm_q8k")
+    gpu.ensure_family("gemv_q8k")
+    nsb, mp = k // 256, (m + 127) // 128 * 128
+    xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
+    gpu.quant_q8k(gpu.upload(x), m, k, xq, xs)
+    wd = gpu.upload_bytes(w)
+    xst, sums = gpu.alloc(nsb * mp), gpu.alloc_bytes(nsb * mp * 16)
+    gpu.dispatch(gpu.begin(), "q8k_token_sides", [(xq, 0), (xs, 0), (xst, 0), (sums, 0)], [k, m, mp], [nsb, (mp + 255) // 256, 1], [256, 1, 1])
+    # the side arrays: scales transposed, sums split as 64 hi + lo, zeros past row M
+    q = gpu.read(xq, m * k, np.int8).reshape(m, nsb, 8, 32).astype(np.int32).sum(3)
+    sd = gpu.read(sums, nsb * mp * 16, np.int8).reshape(nsb, mp, 2, 8).astype(np.int32)
+    assert np.array_equal(64 * sd[:, :m, 1] + sd[:, :m, 0], q.transpose(1, 0, 2)) and not sd[:, m:].any()
+    assert np.all((sd[:, :, 0] >= 0) & (sd[:, :, 0] < 64))
+    st = gpu.read(xst, nsb * mp).reshape(nsb, mp)
+    assert np.array_equal(st[:, :m], gpu.read(xs, m * nsb).reshape(m, nsb).T) and not st[:, m:].any()
+    want = np.stack([orc.matvec_kq(w, Q4_K, n, k, x[t]) for t in range(m)])
+    ymf = gpu.alloc(m * n)
+    gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (ymf, 0)], [k, n, m, 0, 4, 1],
+                 [(n + 63) // 64, (m + 63) // 64, 1], [256, 1, 1])
+    ref = gpu.read(ymf, m * n).reshape(m, n)
+    for name, br in (("gemm_q8k_q4k_xt", 128), ("gemm_q8k_q4k_xt64", 64)):
+        for acc in (0, 1):
+            y0 = pkg.synth.normal_f32(m * n, "gq", "xt-y0", acc).reshape(m, n)
+            yd = gpu.upload(np.concatenate([y0.ravel(), np.full(n, 4242.5, np.float32)]))
+            gpu.dispatch(gpu.begin(), name, [(xq, 0), (xst, 0), (sums, 0), (wd, 0), (yd, 0)], [k, n, m, acc, mp],
+                         [(n + br - 1) // br, mp // 128, 1], [512, 1, 1])
+            got = gpu.read(yd, m * n + n)
+            assert np.all(got[m * n:] == 4242.5), "wrote past the last token"
+            got = got[:m * n].reshape(m, n)
+            if acc:
+                assert peak_err(got - y0, want) <= TOL_SEEN
+            else:
+                assert peak_err(got, want) <= TOL_SEEN
+                assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), name
+    with pytest.raises(pkg.OjasHipError, match="rounded up to 128"):
+        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_xt", [(xq, 0), (xst, 0), (sums, 0), (wd, 0), (ymf, 0)], [k, n, m, 0, mp + 128],
+                     [(n + 127) // 128, mp // 128, 1], [512, 1, 1])
