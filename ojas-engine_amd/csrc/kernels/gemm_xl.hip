@@ -108,13 +108,14 @@ struct GxQ4K {
 };
 
 // MI = 32-row blocks per wave along M: the tile is (64 MI) x 256.
-template <int MI, bool SPLITK>
+// ACCUM is a template parameter, not the kernel's run-time flag: with the choice made per stored element the
+// 256 x 256 instance, which has no register to spare, spills in its epilogue.
+template <int MI, bool SPLITK, bool ACCUM>
 __device__ __forceinline__ void gemm_xl_body(const ushort* __restrict__ xh, const uchar* __restrict__ w,
-                                             float* __restrict__ y, uint K, uint N, uint accum, uint M, uint nsplit) {
+                                             float* __restrict__ y, uint K, uint N, uint M, uint nsplit, uchar* lds) {
     constexpr uint BM = 64u * MI;
     constexpr uint XSTAGE = BM * GX_ROW;
     constexpr int XL = MI * 2;  // LDS-direct loads per wave and slab
-    __shared__ __attribute__((aligned(1024))) uchar lds[2 * XSTAGE + 2 * GX_WSTAGE + 2 * GX_RAW];
     const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint n0 = blockIdx.x * GX_BN, m0 = blockIdx.y * BM;
     uint k_begin = 0, k_end = K;
@@ -299,37 +300,52 @@ __device__ __forceinline__ void gemm_xl_body(const ushort* __restrict__ xh, cons
 #undef GX_STEP
 
     // epilogue: D register v of block (i, j) holds token row 8*(v/4) + 4*kg + v%4, output fr
+    // (lane and wave ids are asked of the hardware again here, so that nothing derived from them has to stay in a
+    // register through the loop — the 256 x 256 instance has none to spare)
+    const uint le = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const uint we = (uint)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint efr = le & 31u, ekg = le >> 5, ewy = we >> 1, ewx = we & 1u;
 #pragma unroll
     for (int i = 0; i < MI; i++) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint n = n0 + wx * 128u + 32u * j + fr;
+            const uint n = blockIdx.x * GX_BN + ewx * 128u + 32u * j + efr;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const uint m = m0 + wy * 32u * MI + 32u * i + 8u * (v >> 2) + 4u * kg + (v & 3u);
+                const uint m = blockIdx.y * BM + ewy * 32u * MI + 32u * i + 8u * (v >> 2) + 4u * ekg + (v & 3u);
                 if (m < M && n < N) {
                     float* o = y + (size_t)m * N + n;
                     if (SPLITK) atomicAdd(o, acc[i][j][v]);
-                    else *o = accum ? *o + acc[i][j][v] : acc[i][j][v];
+                    else if (ACCUM) *o += acc[i][j][v];
+                    else *o = acc[i][j][v];
                 }
             }
         }
     }
 }
 
+// LDS of a tile: two activation stages, two dequantized-weight stages, two raw-weight slots
+#define GX_LDS(MI) __shared__ __attribute__((aligned(1024))) uchar lds[2 * 64 * (MI) * GX_ROW + 2 * GX_WSTAGE + 2 * GX_RAW]
+
 extern "C" __global__ void __launch_bounds__(256)
 gemm_mm_q4kl(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
-    gemm_xl_body<4, false>(xh, w, y, K, N, accum, M, 1u);
+    GX_LDS(4);
+    if (accum) gemm_xl_body<4, false, true>(xh, w, y, K, N, M, 1u, lds);
+    else gemm_xl_body<4, false, false>(xh, w, y, K, N, M, 1u, lds);
 }
 extern "C" __global__ void __launch_bounds__(256)
 gemm_mm_q4kl_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
-    gemm_xl_body<4, true>(xh, w, y, K, N, 1u, M, nsplit);
+    GX_LDS(4);
+    gemm_xl_body<4, true, true>(xh, w, y, K, N, M, nsplit, lds);
 }
 extern "C" __global__ void __launch_bounds__(256)
 gemm_mm_q4kl_m128(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
-    gemm_xl_body<2, false>(xh, w, y, K, N, accum, M, 1u);
+    GX_LDS(2);
+    if (accum) gemm_xl_body<2, false, true>(xh, w, y, K, N, M, 1u, lds);
+    else gemm_xl_body<2, false, false>(xh, w, y, K, N, M, 1u, lds);
 }
 extern "C" __global__ void __launch_bounds__(256)
 gemm_mm_q4kl_m128_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
-    gemm_xl_body<2, true>(xh, w, y, K, N, 1u, M, nsplit);
+    GX_LDS(2);
+    gemm_xl_body<2, true, true>(xh, w, y, K, N, M, nsplit, lds);
 }
