@@ -318,16 +318,19 @@ def extras(gpu, pkg, lin_q) -> dict:
     i8 = {}
     for name, lin in zip(("gate_up_14336x4096", "down_4096x14336"), lin_q):
         n, k = lin.n, lin.k
-        for m in (8, 16, 128, 512):
+        for m in (8, 16, 128, 512, 2048):
             xf = gpu.upload(synth.normal_f32(m * k, "bench", "i8_x", m, k))
             y = gpu.alloc(m * n)
             us = _time(gpu, lambda i: gpu.mm(xf, lin, y, m, act_mode=pkg.ACT_Q8K), 20, 5)
             i8[f"{name}_M{m}"] = {"us": round(us, 1), "tops": round(2.0 * m * n * k / us / 1e6, 1),
+                                  "int8_mfma_frac": round(2.0 * m * n * k / us / 1e6 / 5000.0, 4),
                                   "weight_gbs": round(n * (k // 256) * 144 / us / 1e3, 1)}
-    out["verify_prefill_q4k_int8"] = {"arithmetic": "quant_q8k activations, int8 x u4 dots on v_mfma_i32_16x16x32_i8, "
-                                                    "the CPU reference's scale algebra",
-                                      "timed": "quantize_q8k + gemm_q8k_q4k_mf (down at M = 8: gemm_q8k_q4k_mk, "
-                                               "a workgroup per row tile with K split over its waves)", **i8}
+    out["verify_prefill_q4k_int8"] = {"arithmetic": "quant_q8k activations, int8 x u4 dots on the int8 matrix cores, the CPU "
+                                                    "reference's scale algebra (results within 2e-5 of matvec_kq)",
+                                      "peak_tops": 5000.0,
+                                      "timed": "quantize_q8k + the tile: from 96 tokens q8k_token_sides + gemm_q8k_q4k_xt{,64} "
+                                               "(128-token tiles, scales folded into int8 planes, v_mfma_i32_16x16x64_i8); below, "
+                                               "gemm_q8k_q4k_mf (down at M = 8: gemm_q8k_q4k_mk)", **i8}
     # ---- speculative verify on the Q4_K output head of the decode step, bf16 activations
     head4 = lin_q[2]
     v4 = {}

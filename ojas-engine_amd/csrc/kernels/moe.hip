@@ -107,6 +107,104 @@ moe_topk_m(const float* lg, uint* idx, float* wgt, uint E, uint KSEL) {
     moe_topk_body(lg + t * E, idx + t * KSEL, wgt + t * KSEL, E, KSEL);
 }
 
+// ---- the reference's other routers (Metal twins crates/ojas-metal/src/kernels/moe.rs:130-150, :531-551) ----
+//   moe_topk_nonorm(lg, idx, wgt, E, KSEL)                     DeepSeek-V2: softmax, top-KSEL, the raw probabilities
+//   moe_topk_v3(lg, bias, idx, wgt, E, KSEL, RSCALE, NORM)     DeepSeek-V3 / GLM: s = sigmoid(logit); experts chosen by
+//       s + bias (strict '>', lowest index wins ties); weight = s of the chosen, times 1 / (their sum) when NORM and the
+//       sum is positive, times the routed scaling factor (RSCALE: its f32 bits) — crates/ojas-cpu/src/cpu_glm.rs:526-548
+// grid [tokens,1,1] x 64: token t reads lg + t E and writes idx / wgt + t KSEL (one token: grid [1,1,1]).
+template <int NI, bool V3>
+__device__ __forceinline__ void moe_topk_alt_lanes(const float* __restrict__ lg, const float* __restrict__ bias,
+                                                   uint* __restrict__ idx, float* __restrict__ wgt, uint E, uint KSEL,
+                                                   float rscale, uint norm) {
+    const uint lane = threadIdx.x & 63u;
+    float ch[NI], val[NI];      // what the experts are chosen by; what a chosen expert's weight is made of
+    float sum = 1.0f;
+    if (V3) {
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const uint e = lane + 64u * i;
+            const float sg = e < E ? 1.0f / (1.0f + expf(-lg[e])) : 0.0f;
+            val[i] = sg;
+            ch[i] = e < E ? sg + bias[e] : -3.4028235e38f;
+        }
+    } else {
+        float mx = -1e30f;
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const uint e = lane + 64u * i;
+            ch[i] = e < E ? lg[e] : -3.4028235e38f;
+            if (e < E) mx = fmaxf(mx, ch[i]);
+        }
+        mx = wave_max(mx);
+        sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const uint e = lane + 64u * i;
+            ch[i] = e < E ? expf(ch[i] - mx) : -3.4028235e38f;
+            val[i] = ch[i];
+            if (e < E) sum += ch[i];
+        }
+        sum = wave_sum(sum);
+    }
+    float wsum = 0.0f, mine = 0.0f;
+    uint mine_idx = 0;
+    for (uint j = 0; j < KSEL; j++) {
+        float bv = V3 ? -1e30f : -1.0f, bval = 0.0f;
+        uint bi = 0xFFFFFFFFu;
+#pragma unroll
+        for (int i = 0; i < NI; i++)
+            if (ch[i] > bv) { bv = ch[i]; bval = val[i]; bi = lane + 64u * i; }
+        const float m2 = wave_max(bv);
+        uint cand = (bv == m2 && bi != 0xFFFFFFFFu) ? bi : 0xFFFFFFFFu;
+        cand = min(cand, (uint)dpp_i32<OJK_DPP_QUAD_XOR1>((int)cand));
+        cand = min(cand, (uint)dpp_i32<OJK_DPP_QUAD_XOR2>((int)cand));
+        cand = min(cand, (uint)dpp_i32<OJK_DPP_ROW_HALF_MIRROR>((int)cand));
+        cand = min(cand, (uint)dpp_i32<OJK_DPP_ROW_MIRROR>((int)cand));
+        const uint c0 = (uint)__builtin_amdgcn_readlane((int)cand, 0), c1 = (uint)__builtin_amdgcn_readlane((int)cand, 16);
+        const uint c2 = (uint)__builtin_amdgcn_readlane((int)cand, 32), c3 = (uint)__builtin_amdgcn_readlane((int)cand, 48);
+        const uint win = min(min(c0, c1), min(c2, c3));
+        // the winner's value (its lane holds it): all lanes learn it
+        const uint wl = win & 63u;
+        float wv = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NI; i++)
+            if (lane + 64u * i == win) wv = val[i];
+        wv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv), (int)__builtin_amdgcn_readfirstlane((int)wl)));
+        (void)bval;
+        wsum += wv;
+        if (lane == j) { mine = wv; mine_idx = win; }
+#pragma unroll
+        for (int i = 0; i < NI; i++)
+            if (lane + 64u * i == win) ch[i] = V3 ? -1e30f : -1.0f;
+    }
+    if (lane < KSEL) {
+        idx[lane] = mine_idx;
+        if (V3) {
+            const float inv = (norm != 0u && wsum > 0.0f) ? 1.0f / wsum : 1.0f;
+            wgt[lane] = mine * inv * rscale;
+        } else {
+            wgt[lane] = mine / sum;
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(64)
+moe_topk_nonorm(const float* lg, uint* idx, float* wgt, uint E, uint KSEL) {
+    const size_t t = blockIdx.x;
+    if (E <= 128u) moe_topk_alt_lanes<2, false>(lg + t * E, nullptr, idx + t * KSEL, wgt + t * KSEL, E, KSEL, 1.0f, 0u);
+    else if (E <= 256u) moe_topk_alt_lanes<4, false>(lg + t * E, nullptr, idx + t * KSEL, wgt + t * KSEL, E, KSEL, 1.0f, 0u);
+    else moe_topk_alt_lanes<16, false>(lg + t * E, nullptr, idx + t * KSEL, wgt + t * KSEL, E, KSEL, 1.0f, 0u);
+}
+extern "C" __global__ void __launch_bounds__(64)
+moe_topk_v3(const float* lg, const float* bias, uint* idx, float* wgt, uint E, uint KSEL, uint RSCALE, uint NORM) {
+    const size_t t = blockIdx.x;
+    const float rs = __uint_as_float(RSCALE);
+    if (E <= 128u) moe_topk_alt_lanes<2, true>(lg + t * E, bias, idx + t * KSEL, wgt + t * KSEL, E, KSEL, rs, NORM);
+    else if (E <= 256u) moe_topk_alt_lanes<4, true>(lg + t * E, bias, idx + t * KSEL, wgt + t * KSEL, E, KSEL, rs, NORM);
+    else moe_topk_alt_lanes<16, true>(lg + t * E, bias, idx + t * KSEL, wgt + t * KSEL, E, KSEL, rs, NORM);
+}
+
 // ------------------------------------------------------------------ grouping
 // Counting sort of the NA assignments by expert: counts[E], offsets[E+1], list[NA] (assignment
 // ids, expert-major; the order inside an expert's group is arbitrary and has no effect on the

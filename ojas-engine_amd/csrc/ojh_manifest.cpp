@@ -833,6 +833,17 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         need[1] = need[2] = (size_t)T * KS * 4;
         return OJH_OK;
     }
+    case 18: case 19: {  // moe_topk_nonorm(lg, idx, wgt, E, KSEL); moe_topk_v3(lg, bias, idx, wgt, E, KSEL, RSCALE, NORM)
+        const bool v3 = s->rows_per_wave == 19;
+        uint32_t E = c[0], KS = c[1], T = grid[0];
+        if ((rc = check_block(block, 64))) return rc;
+        if (!E || E > 1024 || !KS || KS > E || KS > 64) return ojh_fail(OJH_ERR_ARG, "%s: E=%u KSEL=%u out of range", s->name, E, KS);
+        if (!T || grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [tokens,1,1]", s->name);
+        need[0] = (size_t)T * E * 4;
+        if (v3) need[1] = (size_t)E * 4;
+        need[v3 ? 2 : 1] = need[v3 ? 3 : 2] = (size_t)T * KS * 4;
+        return OJH_OK;
+    }
     case 2: {
         uint32_t NA = c[0], E = c[1];
         if ((rc = check_block(block, 256))) return rc;
@@ -1035,7 +1046,7 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K
     block[1] = block[2] = 1;
     switch (s->rows_per_wave) {
     case 0: block[0] = 64; break;
-    case 1: block[0] = 64; grid[0] = M ? M : 1; break;
+    case 1: case 18: case 19: block[0] = 64; grid[0] = M ? M : 1; break;
     case 2: break;
     case 3: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = experts
     case 4: grid[0] = K <= 1024 ? (N + 31) / 32 : (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
@@ -1285,6 +1296,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("gemm_mm_q4kl_m128_sk", "gemm_xl", 3, 4, OJH_Q4_K, 5, check_gemm, shape_gemm);
     // MoE: `rows_per_wave` selects the kernel inside check_moe / shape_moe
     add("moe_topk", "moe", 3, 2, 0, 0, check_moe, shape_moe);
+    add("moe_topk_nonorm", "moe", 3, 2, 0, 18, check_moe, shape_moe);
+    add("moe_topk_v3", "moe", 4, 4, 0, 19, check_moe, shape_moe);
     add("moe_topk_m", "moe", 3, 2, 0, 1, check_moe, shape_moe);
     add("moe_group", "moe", 4, 2, 0, 2, check_moe, shape_moe);
     add("moe_gu_q4k_m", "moe", 7, 4, OJH_Q4_K, 3, check_moe, shape_moe);

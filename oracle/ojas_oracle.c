@@ -939,6 +939,43 @@ void ojo_moe_topk(const float *lg, int E, int ksel, uint32_t *idx, float *wgt) {
     free(pr);
 }
 
+/* The reference's other routers.  nonorm (DeepSeek-V2): softmax, top-k by strict '>' (lowest index wins ties), the raw
+ * probability exp(l - max) / sum of the chosen — crates/ojas-metal/src/kernels/moe.rs:130-150,
+ * crates/ojas-cpu/src/cpu_deepseek.rs:286-305.  v3 (DeepSeek-V3 / GLM): s = sigmoid(l); chosen by s + bias; weight = s of
+ * the chosen times 1/sum(chosen s) when `norm` and the sum is positive, times the routed scaling factor —
+ * crates/ojas-metal/src/kernels/moe.rs:531-551, crates/ojas-cpu/src/cpu_glm.rs:526-548. */
+void ojo_moe_topk_nonorm(const float *lg, int E, int ksel, uint32_t *idx, float *wgt) {
+    float *pr = (float *)malloc((size_t)E * sizeof(float));
+    float mx = -1e30f;
+    for (int e = 0; e < E; e++) if (lg[e] > mx) mx = lg[e];
+    float sum = 0.0f;
+    for (int e = 0; e < E; e++) { pr[e] = expf(lg[e] - mx); sum += pr[e]; }
+    for (int j = 0; j < ksel; j++) {
+        float bv = -1.0f; int bi = 0;
+        for (int e = 0; e < E; e++) if (pr[e] > bv) { bv = pr[e]; bi = e; }
+        idx[j] = (uint32_t)bi;
+        wgt[j] = bv / sum;
+        pr[bi] = -1.0f;
+    }
+    free(pr);
+}
+void ojo_moe_topk_v3(const float *lg, const float *bias, int E, int ksel, float rscale, int norm, uint32_t *idx, float *wgt) {
+    float *sg = (float *)malloc((size_t)E * sizeof(float)), *ch = (float *)malloc((size_t)E * sizeof(float));
+    for (int e = 0; e < E; e++) { sg[e] = 1.0f / (1.0f + expf(-lg[e])); ch[e] = sg[e] + bias[e]; }
+    float sum = 0.0f;
+    for (int j = 0; j < ksel; j++) {
+        float bv = -1e30f; int bi = 0;
+        for (int e = 0; e < E; e++) if (ch[e] > bv) { bv = ch[e]; bi = e; }
+        idx[j] = (uint32_t)bi;
+        wgt[j] = sg[bi];
+        sum += sg[bi];
+        ch[bi] = -1e30f;
+    }
+    float inv = (norm && sum > 0.0f) ? 1.0f / sum : 1.0f;
+    for (int j = 0; j < ksel; j++) wgt[j] = wgt[j] * inv * rscale;
+    free(sg); free(ch);
+}
+
 static inline float silu(float x) { return x / (1.0f + expf(-x)); } /* cpu_math.rs:486 */
 
 static int matvec_mode(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const float *x,

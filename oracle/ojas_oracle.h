@@ -114,6 +114,8 @@ float ojo_ffn_act(float g, int act);
 /* Router: softmax, ksel argmax passes with strict '>', lowest index wins, renormalise
  * (crates/ojas-cuda/src/kernels/moe.rs:45-70; oracle crates/ojas-cuda/tests/conformance.rs:385-392). */
 void ojo_moe_topk(const float *logits, int n_expert, int ksel, uint32_t *idx, float *wgt);
+void ojo_moe_topk_nonorm(const float *lg, int E, int ksel, uint32_t *idx, float *wgt);
+void ojo_moe_topk_v3(const float *lg, const float *bias, int E, int ksel, float rscale, int norm, uint32_t *idx, float *wgt);
 
 /* Expert FFN for T tokens (crates/ojas-cpu/src/cpu_glm.rs:551-582; silu cpu_math.rs:486):
  * for each token t and slot j (in slot order): act = silu(Wg_e x) * (Wu_e x);

@@ -78,6 +78,10 @@ def lib() -> C.CDLL:
         L.ojo_ffn_act.argtypes = [C.c_float, i32]
         L.ojo_moe_topk.restype = None
         L.ojo_moe_topk.argtypes = [vp, i32, i32, vp, vp]
+        L.ojo_moe_topk_nonorm.restype = None
+        L.ojo_moe_topk_nonorm.argtypes = [vp, i32, i32, vp, vp]
+        L.ojo_moe_topk_v3.restype = None
+        L.ojo_moe_topk_v3.argtypes = [vp, vp, i32, i32, C.c_float, i32, vp, vp]
         L.ojo_moe_ffn.argtypes = [vp, sz, sz, sz, i32, i32, vp, vp, vp, vp, u32, vp, u32, i32, i32, vp]
         _lib = L
     return _lib
@@ -248,6 +252,26 @@ def moe_topk(logits: np.ndarray, ksel: int):
     for t in range(T):
         lib().ojo_moe_topk(C.c_void_p(lg[t].ctypes.data), E, ksel,
                            C.c_void_p(idx[t].ctypes.data), C.c_void_p(wgt[t].ctypes.data))
+    return idx, wgt
+
+
+def moe_topk_nonorm(logits: np.ndarray, ksel: int):
+    lg = np.ascontiguousarray(logits, np.float32).reshape(-1, logits.shape[-1])
+    T, E = lg.shape
+    idx, wgt = np.empty((T, ksel), np.uint32), np.empty((T, ksel), np.float32)
+    for t in range(T):
+        lib().ojo_moe_topk_nonorm(C.c_void_p(lg[t].ctypes.data), E, ksel, C.c_void_p(idx[t].ctypes.data), C.c_void_p(wgt[t].ctypes.data))
+    return idx, wgt
+
+
+def moe_topk_v3(logits: np.ndarray, bias: np.ndarray, ksel: int, rscale: float = 1.0, norm: bool = True):
+    lg = np.ascontiguousarray(logits, np.float32).reshape(-1, logits.shape[-1])
+    b = np.ascontiguousarray(bias, np.float32)
+    T, E = lg.shape
+    idx, wgt = np.empty((T, ksel), np.uint32), np.empty((T, ksel), np.float32)
+    for t in range(T):
+        lib().ojo_moe_topk_v3(C.c_void_p(lg[t].ctypes.data), C.c_void_p(b.ctypes.data), E, ksel, C.c_float(rscale), int(norm),
+                              C.c_void_p(idx[t].ctypes.data), C.c_void_p(wgt[t].ctypes.data))
     return idx, wgt
 
 

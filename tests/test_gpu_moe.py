@@ -61,6 +61,37 @@ def test_router_ties_take_the_lowest_index(gpu):
     assert list(gi[1]) == [3, 70, 127, 0]
 
 
+@pytest.mark.parametrize("T,E,ksel", [(1, 64, 6), (9, 160, 6), (4, 256, 8), (3, 1000, 5), (2, 7, 7)])
+def test_other_routers_by_their_reference_names(gpu, orc, pkg, T, E, ksel):
+    """moe_topk_nonorm (raw softmax probabilities) and moe_topk_v3 (sigmoid scores, bias-corrected choice, renormalised
+    and scaled weights): crates/ojas-metal/src/kernels/moe.rs:130-150, :531-551."""
+    gpu.ensure_family("moe")
+    lg = pkg.synth.normal_f32(T * E, "moe", "logits2", T, E).reshape(T, E)
+    bias = (0.3 * pkg.synth.normal_f32(E, "moe", "bias", E)).astype(np.float32)
+    ld, bd = gpu.upload(lg), gpu.upload(bias)
+    idx, wgt = gpu.alloc_bytes(T * ksel * 4), gpu.alloc(T * ksel)
+    grid, block = gpu.launch_shape("moe_topk_nonorm", 0, 0, T)
+    assert grid == [T, 1, 1] and block == [64, 1, 1]
+    gpu.dispatch(gpu.begin(), "moe_topk_nonorm", [(ld, 0), (idx, 0), (wgt, 0)], [E, ksel], grid, block)
+    wi, ww = orc.moe_topk_nonorm(lg, ksel)
+    assert np.array_equal(gpu.read(idx, T * ksel, np.uint32).reshape(T, ksel), wi)
+    assert np.max(np.abs(gpu.read(wgt, T * ksel).reshape(T, ksel) - ww)) < 1e-6
+    for norm, rs in ((1, 1.0), (1, 2.5), (0, 1.0)):
+        rbits = int(np.float32(rs).view(np.uint32))
+        gpu.dispatch(gpu.begin(), "moe_topk_v3", [(ld, 0), (bd, 0), (idx, 0), (wgt, 0)], [E, ksel, rbits, norm], grid, block)
+        wi, ww = orc.moe_topk_v3(lg, bias, ksel, rs, bool(norm))
+        assert np.array_equal(gpu.read(idx, T * ksel, np.uint32).reshape(T, ksel), wi)
+        assert np.max(np.abs(gpu.read(wgt, T * ksel).reshape(T, ksel) - ww)) < 2e-6 * rs
+    # ties take the lowest index; an out-of-range request is refused before any launch
+    z = gpu.upload(np.zeros((1, E), np.float32))
+    gpu.dispatch(gpu.begin(), "moe_topk_v3", [(z, 0), (z, 0), (idx, 0), (wgt, 0)], [E, ksel, int(np.float32(1).view(np.uint32)), 0],
+                 [1, 1, 1], block)
+    assert list(gpu.read(idx, ksel, np.uint32)) == list(range(ksel))
+    assert np.all(gpu.read(wgt, ksel) == 0.5)
+    with pytest.raises(Exception):
+        gpu.dispatch(gpu.begin(), "moe_topk_nonorm", [(ld, 0), (idx, 0), (wgt, 0)], [E, E + 1], grid, block)
+
+
 def _experts(pkg, E, d, nff, tag):
     gate = pkg.synth.q4k_weights(E * nff, d, "moe", tag, "gate")
     up = pkg.synth.q4k_weights(E * nff, d, "moe", tag, "up")

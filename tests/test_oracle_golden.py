@@ -429,6 +429,38 @@ def test_moe_topk_matches_closed_form(orc, pkg):
     assert list(idx[0]) == [0, 1, 2, 3]
 
 
+def test_other_routers_match_closed_forms(orc, pkg):
+    """nonorm: the raw softmax probabilities of the top-k (crates/ojas-metal/src/kernels/moe.rs:130-150); v3: sigmoid
+    scores, chosen by score + bias, weights from the unbiased scores, renormalised and scaled
+    (crates/ojas-metal/src/kernels/moe.rs:531-551, crates/ojas-cpu/src/cpu_glm.rs:526-548)."""
+    lg = pkg.synth.tvec(64, 51)
+    ex = np.exp(lg.astype(np.float64) - lg.max())
+    p = ex / ex.sum()
+    order = sorted(range(64), key=lambda i: (-p[i], i))[:6]
+    idx, wgt = orc.moe_topk_nonorm(lg[None, :], 6)
+    assert list(idx[0]) == order
+    assert np.max(np.abs(wgt[0] - p[order])) < 1e-6
+    assert float(wgt[0].sum()) < 1.0           # not renormalised
+    # v3: a bias that reverses the order changes who is chosen and leaves the weights unbiased
+    sg = 1.0 / (1.0 + np.exp(-lg.astype(np.float64)))
+    bias = (-2.0 * sg).astype(np.float32)      # choice = sg - 2 sg (as f32) : smallest sigmoid wins
+    ch = sg.astype(np.float32).astype(np.float64) + bias
+    order = sorted(range(64), key=lambda i: (-ch[i], i))[:8]
+    for norm, rs in ((True, 1.0), (True, 2.5), (False, 1.0), (False, 0.5)):
+        idx, wgt = orc.moe_topk_v3(lg[None, :], bias, 8, rs, norm)
+        assert list(idx[0]) == order
+        want = sg[order] / (sg[order].sum() if norm else 1.0) * rs
+        assert np.max(np.abs(wgt[0] - want)) < 1e-6 * max(1.0, rs)
+    # zero bias: plain top-k of the sigmoid = top-k of the logits; ties take the lowest index
+    idx, wgt = orc.moe_topk_v3(lg[None, :], np.zeros(64, np.float32), 8, 1.0, True)
+    assert list(idx[0]) == sorted(range(64), key=lambda i: (-lg[i], i))[:8]
+    assert abs(float(wgt[0].sum()) - 1.0) < 1e-6
+    idx, wgt = orc.moe_topk_v3(np.zeros((1, 16), np.float32), np.zeros(16, np.float32), 4, 1.0, False)
+    assert list(idx[0]) == [0, 1, 2, 3] and np.all(wgt[0] == 0.5)
+    idx, _ = orc.moe_topk_nonorm(np.zeros((1, 16), np.float32), 4)
+    assert list(idx[0]) == [0, 1, 2, 3]
+
+
 def test_matmul_q8_row_int8_path(orc):
     rng = np.random.default_rng(7)
     n, k, m = 9, 64, 3
