@@ -1272,20 +1272,28 @@ gemv_q8k_q6k_mk(const signed char* xq, const float* xs, const uchar* w, float* y
 }
 
 // ---- the same tile with the weights copied through LDS ----------------------------------------
-//   gemv_q8k_q6k_ml(xq, xs, w, y, K, N, M, ACC)    M <= 16, 512 threads, rows within 4 GiB,
-//       8 (K + 32) + K / 4 + 101632 <= 163840 (M <= 8)   16 (K + 32) + K / 4 + 67840 <= 163840 (M > 8)
+//   gemv_q8k_q6k_ml(xq, xs, w, y, K, N, M, ACC)    M <= 16, 512 threads, w 16-byte aligned and readable up to the next
+//       multiple of 16 past its last row, rows within 4 GiB,
+//       8 (K + 32) + K / 4 + 87040 <= 163840 (M <= 8)   16 (K + 32) + K / 4 + 58112 <= 163840 (M > 8)
 // gemv_q8k_q6k_mf is bound by its loads: 8-byte pieces of sixteen rows a row apart, three aligned
 // dwords fetched and shifted for each.  Here the memory system copies them: one
 // global_load_lds_dwordx4 moves four super-blocks (rows 4 i .. 4 i + 3 of the tile at one k),
-// fourteen lanes each, into 224-byte LDS slots, so every piece a lane then reads is 8-byte aligned
-// in LDS whatever its alignment in memory.  A super-block is 210 bytes: the fourteenth lane copies
-// its last 16 bytes (194 .. 209) rather than 208 .. 223, so nothing is read past the row and the
-// f16 scale sits at slot byte 222.  Each wave owns a ring of D units (one unit = the wave's 16 rows
-// at one super-block, four copies) and walks its tiles as one stream of units, D - 1 copies ahead
-// across tile borders; waves never wait for each other after the tokens are staged.
-// Slots of copy i start at 1024 i + 128 (i & 1): the sixteen rows then spread over all 64 banks.
+// fourteen lanes each, into 224-byte LDS slots.  A super-block is 210 bytes and starts at any even
+// address; the copy starts at the 16-byte boundary below it (copies from 2-byte-aligned addresses
+// run a tenth slower: 102 -> 92 us for the bare copy stream of a 151936 x 4096 head), and 224
+// bytes from there always hold the block, m = 0, 2 .. 14 bytes into the slot.  The readers fetch
+// the aligned dwords around each 8-byte piece and shift (m & 2), as gemv_q8k_q6k_mf does from
+// memory.  Each wave owns a ring of D units (one unit = the wave's 16 rows at one super-block,
+// four copies) and walks its tiles as one stream of units, D copies ahead across tile borders (a
+// unit's slot is given to the copy D units on as soon as its bytes are in registers);
+// waves never wait for each other after the tokens are staged.
+// The sixteen slots of a unit are packed (row n at 224 n, 16 bytes further for n >= 8): 224 bytes are 56 banks, so rows
+// 0 .. 7 start at banks 0, 56, .. 8 and rows 8 .. 15 between them, and the pieces that half a wave reads (sixteen rows,
+// two k groups) fall on all 64 banks once.  A unit is 3616 bytes (the last slot's readers may fetch a dword past it):
+// rings are 4 units deep up to 8 tokens and 3 beyond where that fits beside the tokens (one less where not), so 4 (3)
+// units of 3360 weight bytes are on their way per wave while it works.
 #define Q6K_ML_SLOT 224u
-#define Q6K_ML_UNIT 4224u
+#define Q6K_ML_UNIT 3616u
 #define Q6K_ML_LDS 163840u
 
 template <int P, int D>
@@ -1312,17 +1320,16 @@ __device__ __forceinline__ void gemv_q8k_q6k_ml_body(const signed char* __restri
     // the copy stream: lane -> slot cq of a copy, piece cpc of the slot
     const uint cq = lane / 14u, cpc = lane - cq * 14u;
     const bool con = lane < 56u;
-    const uint pc_off = cpc < 13u ? cpc * 16u : Q6K_BYTES - 16u;
     uint i_off[4], iu = 0u, i_sb = 0u, i_tile = first, i_slot = 0u;
     auto issue_next = [&]() {
         if (i_sb == 0u) {
 #pragma unroll
-            for (uint i = 0; i < 4u; i++) i_off[i] = min(i_tile * 16u + 4u * i + cq, N - 1u) * row_bytes + pc_off;
+            for (uint i = 0; i < 4u; i++) i_off[i] = min(i_tile * 16u + 4u * i + cq, N - 1u) * row_bytes;
         }
-        const uint dst = lds_addr + o_ring + i_slot * Q6K_ML_UNIT;
+        const uint dst = lds_addr + o_ring + i_slot * Q6K_ML_UNIT, sbo = i_sb * Q6K_BYTES;
         if (con) {
 #pragma unroll
-            for (uint i = 0; i < 4u; i++) lds_dma16(w, i_off[i] + i_sb * Q6K_BYTES, dst + i * 1024u + (i & 1u) * 128u);
+            for (uint i = 0; i < 4u; i++) lds_dma16(w, ((i_off[i] + sbo) & ~15u) + cpc * 16u, dst + i * 896u + (i >> 1) * 16u);
         }
         iu++;
         i_slot = i_slot + 1u == (uint)D ? 0u : i_slot + 1u;
@@ -1331,13 +1338,15 @@ __device__ __forceinline__ void gemv_q8k_q6k_ml_body(const signed char* __restri
             i_tile += stride;
         }
     };
-    for (uint k = 0; k + 1u < (uint)D; k++)
+    for (uint k = 0; k < (uint)D; k++)
         if (iu < total) issue_next();
     const uint n = lane & 15u, kg = lane >> 4;
     const bool live = (n < 8u) == (kg < 2u);
     const uchar* xa = live ? lds + (size_t)(n & 7u) * S + 8u * kg : lds + o_zero + 8u * kg;
     const uint xstep = live ? 256u : 0u, xpass = live ? 8u * S : 0u;
-    const uchar* rd = lds + o_ring + (n >> 2) * 1024u + ((n >> 2) & 1u) * 128u + (n & 3u) * Q6K_ML_SLOT;
+    const uchar* rd = lds + o_ring + n * Q6K_ML_SLOT + (n >> 3) * 16u;
+    // the lane's row starts (row nsb) & 7 super-blocks past a 16-byte boundary, each 2 bytes further
+    uint c_r8 = min(first * 16u + n, N - 1u) * nsb;
     float acc[P][4];
 #pragma unroll
     for (int p = 0; p < P; p++)
@@ -1345,24 +1354,13 @@ __device__ __forceinline__ void gemv_q8k_q6k_ml_body(const signed char* __restri
         for (int v = 0; v < 4; v++) acc[p][v] = 0.0f;
     uint c_sb = 0u, c_tile = first, c_slot = 0u;
     for (uint u = 0; u < total; u++) {
-        if (iu < total) issue_next();              // unit u + D - 1, into the slot read during unit u - 1
         vm_wait(min(total - 1u - u, (uint)D - 1u) * 4u);
-        const uchar* blk = rd + c_slot * Q6K_ML_UNIT;
+        const uchar* blk = rd + c_slot * Q6K_ML_UNIT + (((c_r8 + c_sb) & 7u) << 1);
         c_slot = c_slot + 1u == (uint)D ? 0u : c_slot + 1u;
-        Q6kMfW cur;
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-            const uint2 a = *(const uint2*)(blk + 64u * hf + 8u * kg), b = *(const uint2*)(blk + 64u * hf + 32u + 8u * kg),
-                        h = *(const uint2*)(blk + 128u + 32u * hf + 8u * kg);
-            cur.la[hf].x = a.x; cur.la[hf].y = a.y;
-            cur.lb[hf].x = b.x; cur.lb[hf].y = b.y;
-            cur.qh[hf].x = h.x; cur.qh[hf].y = h.y;
-        }
-        {
-            const uint4 sc = *(const uint4*)(blk + 192u);
-            cur.sc.x = sc.x; cur.sc.y = sc.y; cur.sc.z = sc.z; cur.sc.w = sc.w;
-            cur.d16 = *(const ushort*)(blk + Q6K_ML_SLOT - 2u);
-        }
+        const Q6kMfW cur = q6k_mf_load(blk, kg);
+        // the unit is in registers: its slot takes unit u + D while this one is worked on
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (iu < total) issue_next();
         const uchar* xp[P];
 #pragma unroll
         for (int p = 0; p < P; p++) xp[p] = xa + c_sb * xstep + p * xpass;
@@ -1383,6 +1381,7 @@ __device__ __forceinline__ void gemv_q8k_q6k_ml_body(const signed char* __restri
                 }
             c_sb = 0u;
             c_tile += stride;
+            c_r8 = min(c_tile * 16u + n, N - 1u) * nsb;
         }
     }
 }
@@ -1391,6 +1390,13 @@ extern "C" __global__ void __launch_bounds__(512)
 gemv_q8k_q6k_ml(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
     __shared__ __attribute__((aligned(16))) uchar lds_ml[Q6K_ML_LDS];
     const uint lds_addr = (uint)(size_t)(__attribute__((address_space(3))) uchar*)lds_ml;
-    if (M <= 8) gemv_q8k_q6k_ml_body<1, 3>(xq, xs, w, y, K, N, M, ACC, lds_ml, lds_addr);
-    else gemv_q8k_q6k_ml_body<2, 2>(xq, xs, w, y, K, N, M, ACC, lds_ml, lds_addr);
+    // the deepest ring that fits beside the tokens
+    const uint fixed = (M <= 8 ? 8u : 16u) * (K + 32u) + (K >> 2) + 256u;
+    if (M <= 8) {
+        if (fixed + 8u * 4u * Q6K_ML_UNIT <= Q6K_ML_LDS) gemv_q8k_q6k_ml_body<1, 4>(xq, xs, w, y, K, N, M, ACC, lds_ml, lds_addr);
+        else gemv_q8k_q6k_ml_body<1, 3>(xq, xs, w, y, K, N, M, ACC, lds_ml, lds_addr);
+    } else {
+        if (fixed + 8u * 3u * Q6K_ML_UNIT <= Q6K_ML_LDS) gemv_q8k_q6k_ml_body<2, 3>(xq, xs, w, y, K, N, M, ACC, lds_ml, lds_addr);
+        else gemv_q8k_q6k_ml_body<2, 2>(xq, xs, w, y, K, N, M, ACC, lds_ml, lds_addr);
+    }
 }

@@ -528,10 +528,11 @@ uint64_t ojh_q6k_mk_lds(uint32_t K, uint32_t M) {
     const uint64_t p = M <= 8 ? 1 : 2;
     return 8 * p * ((uint64_t)K + 32) + K / 4 + 256 + 4096 * p;
 }
-// LDS of gemv_q8k_q6k_ml: token rows, their scales, eight waves' copy rings (3 units deep up to 8 tokens, 2 beyond)
+// least LDS of gemv_q8k_q6k_ml: token rows, their scales, eight waves' copy rings (3 units deep up to 8 tokens, 2
+// beyond; the kernel takes one more where it fits)
 uint64_t ojh_q6k_ml_lds(uint32_t K, uint32_t M) {
     const uint64_t p = M <= 8 ? 1 : 2;
-    return 8 * p * ((uint64_t)K + 32) + K / 4 + 256 + 8 * (p == 1 ? 3 : 2) * 4224;
+    return 8 * p * ((uint64_t)K + 32) + K / 4 + 256 + 8 * (p == 1 ? 3 : 2) * 3616;
 }
 
 // gemv_q8k_<fmt>_m(xq, xs, w, y, K, N, M, ACC)
@@ -585,6 +586,10 @@ static int check_gemv_q8k_m(const ojh_kernel_spec *s, const uint32_t *c, const u
     if (mf || mk) {           // whole aligned dwords around every piece: the last one may end 2 bytes on
         need[2] = (need[2] + 3) & ~(size_t)3;
         align[2] = 4;
+    }
+    if (ml) {                 // whole aligned 16-byte pieces around every super-block
+        need[2] = (need[2] + 15) & ~(size_t)15;
+        align[2] = 16;
     }
     return OJH_OK;
 }

@@ -42,7 +42,8 @@ extern "C" int ojh_lin_create(ojh_device *dev, uint32_t type, uint32_t n, uint32
     int rc = lin_check(type, n, k, &rb);
     if (rc) return rc;
     ojh_buf *buf = nullptr;
-    if ((rc = ojh_alloc(dev, rb * n, &buf))) return rc;
+    // up to the next multiple of 16: kernels that copy whole aligned 16-byte pieces may read that far
+    if ((rc = ojh_alloc(dev, (rb * n + 15) & ~(size_t)15, &buf))) return rc;
     if ((rc = ojh_upload(dev, buf, 0, raw, rb * n))) {
         ojh_free(dev, buf);
         return rc;
@@ -240,7 +241,8 @@ int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, con
     if (w->type == OJH_Q6_K && m >= 2) {
         const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount, tiles = (N + 15) / 16;
         const uint32_t mc16 = m <= 8 ? m : 16;
-        const bool ml_fits = dev->q6k_ml && (uint64_t)w_bytes <= 0xFFFFFFFFull && ojh_q6k_ml_lds(K, mc16) <= 163840;
+        const bool ml_fits = dev->q6k_ml && (uint64_t)w_bytes <= 0xFFFFFFFFull && ojh_q6k_ml_lds(K, mc16) <= 163840 &&
+                             (uintptr_t)wp % 16 == 0 && w->off + ((w_bytes + 15) & ~(size_t)15) <= w->raw->bytes;
         const bool mf_fits = dwords_ok && (uint64_t)(m <= 8 ? 8 : 16) * (K + 32) + K / 4 + 256 <= 69632;
         const bool mk16 = dwords_ok && ojh_q6k_mk_lds(K, mc16) <= 163840, mk8 = dwords_ok && ojh_q6k_mk_lds(K, 8) <= 163840;
         const bool mx_fits = m <= 16 && (uint64_t)m * ((K + 4095) / 4096) <= 19;

@@ -515,8 +515,9 @@ def test_q6k_tokens_with_rows_copied_through_lds(gpu, orc, pkg, m, n, k, accum, 
     """`gemv_q8k_q6k_ml`: the matrix-core tile with each wave's rows copied global -> LDS a
     super-block at a time.  Against matvec_kq per token and, bit for bit, the direct-load entry on
     the same quantized activations (the same arithmetic on the same bytes).  Small grids make a
-    wave walk many tiles, so its copy ring wraps and runs ahead across tile borders; the last rows
-    of the weights end exactly at the end of their buffer."""
+    wave walk many tiles, so its copy ring wraps and runs ahead across tile borders.  The copies
+    move whole aligned 16-byte pieces: the buffer must reach the next multiple of 16 past the last
+    row (poisoned here), and a shorter one is refused."""
     w = pkg.synth.q6k_weights(n, k, "ml", n, k)
     x = pkg.synth.normal_f32(m * k, "ml", "x", m, k).reshape(m, k)
     y0 = pkg.synth.normal_f32(m * n, "ml", "y0").reshape(m, n) if accum else np.zeros((m, n), np.float32)
@@ -525,9 +526,13 @@ def test_q6k_tokens_with_rows_copied_through_lds(gpu, orc, pkg, m, n, k, accum, 
     nsb = k // 256
     xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
     gpu.quant_q8k(gpu.upload(x), m, k, xq, xs)
-    wd = gpu.upload_bytes(w)
+    wd = gpu.upload_bytes(np.concatenate([w, np.full(-w.size % 16, 0xA5, np.uint8)]))
     outs = {}
     mf_fits = (8 if m <= 8 else 16) * (k + 32) + k // 4 + 256 <= 69632
+    if w.size % 16:
+        with pytest.raises(pkg.OjasHipError):
+            gpu.dispatch(gpu.begin(), "gemv_q8k_q6k_ml", [(xq, 0), (xs, 0), (gpu.upload_bytes(w), 0), (gpu.alloc(m * n), 0)],
+                         [k, n, m, 0], [8, 1, 1], [512, 1, 1])
     for name in ("gemv_q8k_q6k_ml", "gemv_q8k_q6k_mf") if mf_fits else ("gemv_q8k_q6k_ml",):
         grid, block = gpu.launch_shape(name, k, n, m)
         if grid_x and name.endswith("ml"):
