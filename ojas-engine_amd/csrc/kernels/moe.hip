@@ -945,29 +945,34 @@ moe_down_q4k_mm(const signed char* __restrict__ aq, const float* __restrict__ as
 // pair) and writes its own outputs; no partial sums meet.  Tile i of the expert belongs to
 // workgroup i % RG, wave (i / RG) % 8.  Super-blocks are added in order.
 #define MT_LDS 81920u
-template <bool GU>
+// A pass stages 16 P assignments; P = 2 where 32 token rows fit (32 (K + 32) + 5 K / 2 + 384 <= 81920): an expert with
+// 17 .. 32 assignments then has its rows read and unpacked once instead of twice (at 256 tokens over 128 experts with
+// 8 slots each, 16 per expert on average, that is every other expert).
+template <bool GU, int P>
 __device__ __forceinline__ void moe_mt_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
                                             const uchar* __restrict__ w0, const uchar* __restrict__ w1, float* __restrict__ out,
                                             const uint* __restrict__ offsets, const uint* __restrict__ list,
                                             uint K, uint N, uint KSEL, uint NA, uchar* lds) {
+    constexpr uint TP = 16u * P;
+    constexpr int NT = GU ? 2 : 1;
     const uint e = blockIdx.y;
     const uint a0 = min(offsets[e], NA), a1 = min(offsets[e + 1], NA);
     if (a0 >= a1) return;
     const uint tid = threadIdx.x, lane = tid & 63u, nt = blockDim.x;
     const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6)), nw = nt >> 6;
     const uint nsb = K >> 8, S = K + 32u, per_row = K >> 4;
-    const uint o_lsx = 16u * S, o_lbq = o_lsx + nsb * 64u, o_zero = o_lbq + nsb * 256u, o_av = o_zero + 256u;
-    float* lsx = (float*)(lds + o_lsx);            // [sb][16] token scales
-    uchar* lbq = lds + o_lbq;                      // [sb][16][16]: lo_0..7, hi_0..7 of the bsums
-    uint* lav = (uint*)(lds + o_av);               // [16] the pass's assignments
+    const uint o_lsx = TP * S, o_lbq = o_lsx + nsb * TP * 4u, o_zero = o_lbq + nsb * TP * 16u, o_av = o_zero + 256u;
+    float* lsx = (float*)(lds + o_lsx);            // [sb][TP] token scales
+    uchar* lbq = lds + o_lbq;                      // [sb][TP][16]: lo_0..7, hi_0..7 of the bsums
+    uint* lav = (uint*)(lds + o_av);               // [TP] the pass's assignments
     if (tid < 64u) ((uint*)(lds + o_zero))[tid] = 0u;
     const uint n = lane & 15u, kg = lane >> 4;
     const size_t rb = (size_t)nsb * Q4K_BYTES;
     const uint tiles = (N + 15u) >> 4;
-    for (uint tt = a0; tt < a1; tt += 16u) {
-        const uint cnt = min(16u, a1 - tt);
+    for (uint tt = a0; tt < a1; tt += TP) {
+        const uint cnt = min(TP, a1 - tt);
         __syncthreads();                           // the previous pass is done with the staged tokens
-        if (tid < 16u) lav[tid] = min(list[min(tt + tid, a1 - 1u)], NA - 1u);
+        if (tid < TP) lav[tid] = min(list[min(tt + tid, a1 - 1u)], NA - 1u);
         __syncthreads();
         // token rows 0 .. cnt - 1, eight loads in flight per thread
         const uint total = cnt * per_row;
@@ -976,7 +981,7 @@ __device__ __forceinline__ void moe_mt_body(const signed char* __restrict__ xq, 
             uint dst[8];
 #pragma unroll
             for (int u = 0; u < 8; u++) {
-                const uint i = i0 + (uint)u * nt, t = min(i / per_row, 15u), o = (i - (i / per_row) * per_row) << 4;
+                const uint i = i0 + (uint)u * nt, t = min(i / per_row, TP - 1u), o = (i - (i / per_row) * per_row) << 4;
                 const uint src = GU ? lav[t] / KSEL : lav[t];
                 v[u] = make_uint4(0u, 0u, 0u, 0u);
                 dst[u] = t * S + o;
@@ -986,14 +991,14 @@ __device__ __forceinline__ void moe_mt_body(const signed char* __restrict__ xq, 
             for (int u = 0; u < 8; u++)
                 if (i0 + (uint)u * nt < total) *(uint4*)(lds + dst[u]) = v[u];
         }
-        for (uint i = tid; i < nsb * 16u; i += nt) {
-            const uint sb = i >> 4, t = i & 15u;
+        for (uint i = tid; i < nsb * TP; i += nt) {
+            const uint sb = i / TP, t = i - sb * TP;
             const uint src = GU ? lav[t] / KSEL : lav[t];
             lsx[i] = t < cnt ? xs[(size_t)src * nsb + sb] : 0.0f;
         }
         __syncthreads();
-        for (uint i = tid; i < nsb * 128u; i += nt) {
-            const uint jj = i & 7u, t = (i >> 3) & 15u, sb = i >> 7;
+        for (uint i = tid; i < nsb * TP * 8u; i += nt) {
+            const uint jj = i & 7u, t = (i >> 3) % TP, sb = (i >> 3) / TP;
             int bs = 0;
             if (t < cnt) {
                 const uint4* px = (const uint4*)(lds + (size_t)t * S + sb * 256u + jj * 32u);
@@ -1003,13 +1008,20 @@ __device__ __forceinline__ void moe_mt_body(const signed char* __restrict__ xq, 
                 bs = dot4_i8(b.x, 0x01010101u, bs); bs = dot4_i8(b.y, 0x01010101u, bs);
                 bs = dot4_i8(b.z, 0x01010101u, bs); bs = dot4_i8(b.w, 0x01010101u, bs);
             }
-            uchar* o = lbq + ((size_t)sb * 16u + t) * 16u;
+            uchar* o = lbq + ((size_t)sb * TP + t) * 16u;
             o[jj] = (uchar)(bs & 63);
             o[8u + jj] = (uchar)(bs >> 6);
         }
         __syncthreads();
-        const uchar* xa = n < cnt ? lds + (size_t)n * S + 8u * kg : lds + o_zero + 8u * kg;
-        const uint xstep = n < cnt ? 256u : 0u;
+        const uint np = (cnt + 15u) >> 4;          // token tiles of 16 this pass holds
+        const uchar* xa[P];
+        uint xstep[P];
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            const bool on = n + 16u * p < cnt;
+            xa[p] = on ? lds + (size_t)(n + 16u * p) * S + 8u * kg : lds + o_zero + 8u * kg;
+            xstep[p] = on ? 256u : 0u;
+        }
         // This wave's tiles as one stream of (tile, super-block) steps, the blocks of three steps on their
         // way: a wave that loads a step only when it starts the one before it walks a chain of memory
         // latencies (32 of them per pass at 768 x 2048) and the launch is bound by that chain.
@@ -1017,10 +1029,10 @@ __device__ __forceinline__ void moe_mt_body(const signed char* __restrict__ xq, 
         const uint my_tiles = first < tiles ? (tiles - first + stride - 1u) / stride : 0u;
         const uint steps = my_tiles * nsb;
         uint i_u = 0u, i_sb = 0u, i_tile = first;
-        auto next_step = [&](GqW (&blk)[GU ? 2 : 1]) {   // loads past the last step repeat it
+        auto next_step = [&](GqW (&blk)[NT]) {   // loads past the last step repeat it
             const size_t off = ((size_t)e * N + min(i_tile * 16u + n, N - 1u)) * rb + (size_t)i_sb * Q4K_BYTES;
             blk[0] = gq_load(w0 + off, kg);
-            if (GU) blk[GU ? 1 : 0] = gq_load(w1 + off, kg);
+            if (GU) blk[NT - 1] = gq_load(w1 + off, kg);
             if (i_u + 1u < steps) {
                 i_u++;
                 if (++i_sb == nsb) {
@@ -1030,49 +1042,59 @@ __device__ __forceinline__ void moe_mt_body(const signed char* __restrict__ xq, 
             }
         };
         if (steps == 0u) continue;
-        GqW c0[GU ? 2 : 1], c1[GU ? 2 : 1], c2[GU ? 2 : 1];
+        GqW c0[NT], c1[NT], c2[NT];
         next_step(c0);
         next_step(c1);
         next_step(c2);
-        float acc[GU ? 2 : 1][4];
+        float acc[NT][P][4];
 #pragma unroll
-        for (int w = 0; w < (GU ? 2 : 1); w++)
+        for (int w = 0; w < NT; w++)
 #pragma unroll
-            for (int v = 0; v < 4; v++) acc[w][v] = 0.0f;
+            for (int p = 0; p < P; p++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) acc[w][p][v] = 0.0f;
         uint c_sb = 0u, c_tile = first;
         for (uint u = 0; u < steps; u++) {
-            GqW c3[GU ? 2 : 1];
+            GqW c3[NT];
             next_step(c3);
 #pragma unroll
-            for (int w = 0; w < (GU ? 2 : 1); w++)
-                gq_superblock(c0[w], xa + c_sb * xstep, lbq + ((size_t)c_sb * 16u + n) * 16u, lsx + c_sb * 16u, kg, acc[w]);
+            for (int w = 0; w < NT; w++)
 #pragma unroll
-            for (int w = 0; w < (GU ? 2 : 1); w++) {
+                for (int p = 0; p < P; p++)
+                    if ((uint)p < np)
+                        gq_superblock(c0[w], xa[p] + c_sb * xstep[p], lbq + ((size_t)c_sb * TP + 16u * p + n) * 16u,
+                                      lsx + c_sb * TP + 16u * p, kg, acc[w][p]);
+#pragma unroll
+            for (int w = 0; w < NT; w++) {
                 c0[w] = c1[w];
                 c1[w] = c2[w];
                 c2[w] = c3[w];
             }
             if (++c_sb == nsb) {
-                // D register v of lane (n, kg): assignment 4 kg + v of the pass, row n of the tile
+                // D register v of lane (n, kg): assignment 16 p + 4 kg + v of the pass, row n of the tile
                 if (c_tile * 16u + n < N) {
 #pragma unroll
-                    for (int v = 0; v < 4; v++) {
-                        const uint t = 4u * kg + (uint)v;
-                        if (t < cnt) {
-                            float* o = out + (size_t)lav[t] * N + c_tile * 16u + n;
-                            if (GU) {
-                                const float g = acc[0][v];
-                                *o = (g / (1.0f + expf(-g))) * acc[GU ? 1 : 0][v];
-                            } else {
-                                *o = acc[0][v];
+                    for (int p = 0; p < P; p++)
+#pragma unroll
+                        for (int v = 0; v < 4; v++) {
+                            const uint t = 16u * p + 4u * kg + (uint)v;
+                            if (t < cnt) {
+                                float* o = out + (size_t)lav[t] * N + c_tile * 16u + n;
+                                if (GU) {
+                                    const float g = acc[0][p][v];
+                                    *o = (g / (1.0f + expf(-g))) * acc[NT - 1][p][v];
+                                } else {
+                                    *o = acc[0][p][v];
+                                }
                             }
                         }
-                    }
                 }
 #pragma unroll
-                for (int w = 0; w < (GU ? 2 : 1); w++)
+                for (int w = 0; w < NT; w++)
 #pragma unroll
-                    for (int v = 0; v < 4; v++) acc[w][v] = 0.0f;
+                    for (int p = 0; p < P; p++)
+#pragma unroll
+                        for (int v = 0; v < 4; v++) acc[w][p][v] = 0.0f;
                 c_sb = 0u;
                 c_tile += stride;
             }
@@ -1085,7 +1107,8 @@ moe_gu_q4k_mt(const signed char* __restrict__ xq, const float* __restrict__ xs, 
               const uchar* __restrict__ wu, float* __restrict__ act, const uint* __restrict__ offsets,
               const uint* __restrict__ list, uint K, uint N, uint KSEL, uint NA) {
     __shared__ __attribute__((aligned(16))) uchar lds_mt[MT_LDS];
-    moe_mt_body<true>(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA, lds_mt);
+    if (32u * (K + 32u) + 5u * (K >> 1) + 384u <= MT_LDS) moe_mt_body<true, 2>(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA, lds_mt);
+    else moe_mt_body<true, 1>(xq, xs, wg, wu, act, offsets, list, K, N, KSEL, NA, lds_mt);
 }
 
 extern "C" __global__ void __launch_bounds__(512)
@@ -1093,7 +1116,8 @@ moe_down_q4k_mt(const signed char* __restrict__ aq, const float* __restrict__ as
                 float* __restrict__ dv, const uint* __restrict__ offsets, const uint* __restrict__ list,
                 uint K, uint N, uint NA) {
     __shared__ __attribute__((aligned(16))) uchar lds_mt[MT_LDS];
-    moe_mt_body<false>(aq, as_, wd, wd, dv, offsets, list, K, N, 1u, NA, lds_mt);
+    if (32u * (K + 32u) + 5u * (K >> 1) + 384u <= MT_LDS) moe_mt_body<false, 2>(aq, as_, wd, wd, dv, offsets, list, K, N, 1u, NA, lds_mt);
+    else moe_mt_body<false, 1>(aq, as_, wd, wd, dv, offsets, list, K, N, 1u, NA, lds_mt);
 }
 
 // ------------------------------------------------------------------ combine
