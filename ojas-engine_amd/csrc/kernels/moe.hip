@@ -209,11 +209,8 @@ moe_topk_v3(const float* lg, const float* bias, uint* idx, float* wgt, uint E, u
 // Counting sort of the NA assignments by expert: counts[E], offsets[E+1], list[NA] (assignment
 // ids, expert-major; the order inside an expert's group is arbitrary and has no effect on the
 // results, which are stored per assignment).  One workgroup; E <= 1024.
-extern "C" __global__ void __launch_bounds__(256)
-moe_group(const uint* __restrict__ idx, uint* __restrict__ counts, uint* __restrict__ offsets,
-          uint* __restrict__ list, uint NA, uint E) {
-    __shared__ uint cnt[1024];
-    __shared__ uint off[1025];
+__device__ __forceinline__ void moe_group_body(const uint* __restrict__ idx, uint* __restrict__ counts, uint* __restrict__ offsets,
+                                               uint* __restrict__ list, uint NA, uint E, uint* cnt, uint* off) {
     const uint tid = threadIdx.x;
     for (uint e = tid; e < E; e += 256u) cnt[e] = 0u;
     __syncthreads();
@@ -238,6 +235,13 @@ moe_group(const uint* __restrict__ idx, uint* __restrict__ counts, uint* __restr
         uint e = idx[a];
         if (e < E) list[off[e] + atomicAdd(&cnt[e], 1u)] = a;
     }
+}
+extern "C" __global__ void __launch_bounds__(256)
+moe_group(const uint* __restrict__ idx, uint* __restrict__ counts, uint* __restrict__ offsets,
+          uint* __restrict__ list, uint NA, uint E) {
+    __shared__ uint cnt[1024];
+    __shared__ uint off[1025];
+    moe_group_body(idx, counts, offsets, list, NA, E, cnt, off);
 }
 
 // ------------------------------------------------------------------ grouped gate / up
@@ -591,6 +595,23 @@ extern "C" __global__ void __launch_bounds__(256)
 moe_down_q6k_dec(const float* act, const uchar* wd, const uint* idx, const float* wgt, float* y, uint K, uint N,
                  uint KSEL, uint E, uint ACC) {
     moe_down_dec_body<W6k, false>(act, wd, idx, wgt, y, K, N, KSEL, E, ACC);
+}
+
+// ------------------------------------------------------------------ the quantizer and the grouping in one launch
+//   moe_quant_group(x, xq, xs, idx, counts, offsets, list, K, T, NA, E)   grid [T + 1,1,1]: block t quantizes token t
+//       (quant_q8k's rule, the operations of quantize_q8k), the last block sorts the assignments by expert (moe_group).
+// Neither depends on the other; both are a few microseconds of launch and little else.
+extern "C" __global__ void __launch_bounds__(256)
+moe_quant_group(const float* __restrict__ x, signed char* __restrict__ xq, float* __restrict__ xs, const uint* __restrict__ idx,
+                uint* __restrict__ counts, uint* __restrict__ offsets, uint* __restrict__ list, uint K, uint T, uint NA, uint E) {
+    __shared__ uint cnt[1024];
+    __shared__ uint off[1025];
+    if (blockIdx.x >= T) {
+        moe_group_body(idx, counts, offsets, list, NA, E, cnt, off);
+        return;
+    }
+    const size_t t = blockIdx.x;
+    block_quant_q8k(x + t * K, K, xq + t * K, xs + t * (K >> 8));
 }
 
 // ------------------------------------------------------------------ Q8_0 experts, f32 activations

@@ -73,6 +73,7 @@ struct ojh_device {
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
                                  // 3 = per-assignment decode form always, 4 = matrix cores in the workgroup-per-tile form always
     uint32_t moe_dec_tokens = 8; // OJAS_HIP_MOE_DEC_TOKENS: the decode form serves up to this many tokens
+    bool moe_fuse = true;        // OJAS_HIP_MOE_FUSE=0: the grouped pipeline keeps its quantizer and grouping launches apart
     bool gemm_exact = false;     // OJAS_HIP_GEMM_EXACT: Q4_K prefill through the tile that holds dequant_to_f16 bits
     bool fused_quant = false;    // OJAS_HIP_FUSED_QUANT=1: ojh_mm (m = 1, Q4_K) quantizes x inside the matvec launch
     uint32_t fq_blocks_per_cu = 8; // OJAS_HIP_FQ_BLOCKS: blocks per CU the fused-quantizer matvec aims for

@@ -849,6 +849,20 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         need[v3 ? 2 : 1] = need[v3 ? 3 : 2] = (size_t)T * KS * 4;
         return OJH_OK;
     }
+    case 20: {   // moe_quant_group(x, xq, xs, idx, counts, offsets, list, K, T, NA, E)   grid [T + 1,1,1]
+        uint32_t K = c[0], T = c[1], NA = c[2], E = c[3];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!K || K % 256 || !T || !NA || !E || E > 1024) return ojh_fail(OJH_ERR_ARG, "%s: K=%u T=%u NA=%u E=%u out of range", s->name, K, T, NA, E);
+        if (grid[0] != T + 1 || grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [T + 1,1,1]", s->name);
+        need[0] = (size_t)T * K * 4;
+        need[1] = (size_t)T * K;
+        need[2] = (size_t)T * (K / 256) * 4;
+        need[3] = need[6] = (size_t)NA * 4;
+        need[4] = (size_t)E * 4;
+        need[5] = (size_t)(E + 1) * 4;
+        align[0] = align[1] = 16;
+        return OJH_OK;
+    }
     case 2: {
         uint32_t NA = c[0], E = c[1];
         if ((rc = check_block(block, 256))) return rc;
@@ -1055,6 +1069,7 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K
     case 2: break;
     case 3: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = experts
     case 4: grid[0] = K <= 1024 ? (N + 31) / 32 : (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
+    case 20: grid[0] = M + 1; break;  // M = tokens
     case 6: case 7: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;
     case 14: case 16: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = slots, one token
     case 15: case 17: grid[0] = (N + 3) / 4; break;                           // one token
@@ -1305,6 +1320,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("moe_topk_v3", "moe", 4, 4, 0, 19, check_moe, shape_moe);
     add("moe_topk_m", "moe", 3, 2, 0, 1, check_moe, shape_moe);
     add("moe_group", "moe", 4, 2, 0, 2, check_moe, shape_moe);
+    add("moe_quant_group", "moe", 7, 4, 0, 20, check_moe, shape_moe);
     add("moe_gu_q4k_m", "moe", 7, 4, OJH_Q4_K, 3, check_moe, shape_moe);
     add("moe_down_q4k_m", "moe", 6, 3, OJH_Q4_K, 4, check_moe, shape_moe);
     add("moe_combine", "moe", 3, 4, 0, 5, check_moe, shape_moe);

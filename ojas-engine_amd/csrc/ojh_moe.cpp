@@ -144,15 +144,17 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     const bool mt_gu = mm && dev->moe_mode != 4 && ojh_moe_mt_lds(d) <= 81920;
     const bool mt_down = mm && dev->moe_mode != 4 && !down5 && ojh_moe_mt_lds(n_ff) <= 81920;
     const uint32_t b512[3] = {512, 1, 1};
-    // 1. quantize the tokens once
-    {
+    // 1. quantize the tokens once, 2. group the (token, slot) assignments by expert: one launch where a token is one
+    //    workgroup's work (the grouping rides along as an extra workgroup), two otherwise
+    if (dev->moe_fuse && d <= 8192) {
+        uint32_t g[3] = {T + 1, 1, 1};
+        if ((rc = ojh_launch(dev, "moe_quant_group", {x->ptr, xq->ptr, xs->ptr, idx->ptr, counts, offsets, list}, {d, T, NA, E}, g, b256)))
+            return rc;
+    } else {
         uint32_t g[3] = {nsb_d, T, 1};
         if ((rc = ojh_launch(dev, "quantize_q8k", {x->ptr, xq->ptr, xs->ptr}, {d, T}, g, b256))) return rc;
-    }
-    // 2. group the (token, slot) assignments by expert
-    {
-        uint32_t g[3] = {1, 1, 1};
-        if ((rc = ojh_launch(dev, "moe_group", {idx->ptr, counts, offsets, list}, {NA, E}, g, b256))) return rc;
+        uint32_t g1[3] = {1, 1, 1};
+        if ((rc = ojh_launch(dev, "moe_group", {idx->ptr, counts, offsets, list}, {NA, E}, g1, b256))) return rc;
     }
     // 3. gate/up + SiLU*mul, one launch over all experts
     {

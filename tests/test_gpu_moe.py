@@ -92,6 +92,36 @@ def test_other_routers_by_their_reference_names(gpu, orc, pkg, T, E, ksel):
         gpu.dispatch(gpu.begin(), "moe_topk_nonorm", [(ld, 0), (idx, 0), (wgt, 0)], [E, E + 1], grid, block)
 
 
+@pytest.mark.parametrize("T,E,ksel,d", [(16, 128, 8, 2048), (3, 7, 2, 768), (40, 1000, 5, 256)])
+def test_quantizer_and_grouping_in_one_launch(gpu, orc, pkg, T, E, ksel, d):
+    """`moe_quant_group` against the two launches it stands for: the quantizer's bytes bit for bit (and the CPU
+    oracle's), and a grouping that holds every assignment once under its expert."""
+    gpu.ensure_family("moe")
+    gpu.ensure_family("gemv_q8k")
+    x = pkg.synth.normal_f32(T * d, "moe", "qg-x", T, d).reshape(T, d)
+    idx_h = pkg.synth.rng("moe", "qg-idx", T, E).integers(0, E, T * ksel).astype(np.uint32)
+    NA, nsb = T * ksel, d // 256
+    xd, idx = gpu.upload(x), gpu.upload_bytes(idx_h.view(np.uint8))
+    xq, xs = gpu.alloc_bytes(T * d), gpu.alloc(T * nsb)
+    counts, offsets, lst = gpu.alloc_bytes(E * 4), gpu.alloc_bytes((E + 1) * 4), gpu.alloc_bytes(NA * 4)
+    grid, block = gpu.launch_shape("moe_quant_group", d, 0, T)
+    assert grid == [T + 1, 1, 1]
+    gpu.dispatch(gpu.begin(), "moe_quant_group", [(xd, 0), (xq, 0), (xs, 0), (idx, 0), (counts, 0), (offsets, 0), (lst, 0)],
+                 [d, T, NA, E], grid, block)
+    q2, s2 = gpu.alloc_bytes(T * d), gpu.alloc(T * nsb)
+    gpu.quant_q8k(xd, T, d, q2, s2)
+    assert np.array_equal(gpu.read(xq, T * d, np.int8), gpu.read(q2, T * d, np.int8))
+    assert np.array_equal(gpu.read(xs, T * nsb), gpu.read(s2, T * nsb))
+    ws, wq, _ = orc.quant_q8k(x[T - 1])
+    assert np.array_equal(gpu.read(xq, T * d, np.int8).reshape(T, d)[T - 1], wq)
+    cnt, off, ls = gpu.read(counts, E, np.uint32), gpu.read(offsets, E + 1, np.uint32), gpu.read(lst, NA, np.uint32)
+    assert np.array_equal(cnt, np.bincount(idx_h, minlength=E))
+    assert np.array_equal(off, np.concatenate([[0], np.cumsum(cnt)]))
+    assert sorted(ls) == list(range(NA))
+    for e in range(E):
+        assert np.all(idx_h[ls[off[e]:off[e + 1]]] == e)
+
+
 def _experts(pkg, E, d, nff, tag):
     gate = pkg.synth.q4k_weights(E * nff, d, "moe", tag, "gate")
     up = pkg.synth.q4k_weights(E * nff, d, "moe", tag, "up")
