@@ -71,8 +71,12 @@ enum { OJH_X_F32 = 0, OJH_X_BF16 = 1, OJH_X_F16 = 2 };
  *                 weights are the bits of `dequant_to_f16`.
  *   OJH_ACT_FLOAT_EXACT — as OJH_ACT_FLOAT, but a Q4_K weight too enters the tile as the bits of
  *                 `dequant_to_f16` (crates/ojas-formats/src/gguf.rs:612-1116); a slower tile.
+ *   OJH_ACT_Q8_1 — Q8_0 rows only, f32 activations: quantized to int8 per 32 values (`quantize_q8_1`), integer dots
+ *                 against the blocks as the file stores them, token by token: the arithmetic of the reference's GPU
+ *                 decode path for Q8_0 models (crates/ojas-cuda/src/kernels/gemv_q8.rs:152-215, gemv.rs:33-52; its
+ *                 own bar 1e-2 of the output peak against the dequantized dot).  Never chosen by OJH_ACT_AUTO.
  *   OJH_ACT_AUTO  — OJH_ACT_Q8K for K-quant GEMV-shaped calls, OJH_ACT_FLOAT above the crossover. */
-enum { OJH_ACT_AUTO = 0, OJH_ACT_Q8K = 1, OJH_ACT_FLOAT = 2, OJH_ACT_FLOAT_EXACT = 3 };
+enum { OJH_ACT_AUTO = 0, OJH_ACT_Q8K = 1, OJH_ACT_FLOAT = 2, OJH_ACT_FLOAT_EXACT = 3, OJH_ACT_Q8_1 = 4 };
 
 typedef struct ojh_gguf ojh_gguf;     /* an open GGUF file: metadata + tensor index */
 typedef struct ojh_device ojh_device; /* one GPU + one stream + loaded families */

@@ -655,6 +655,68 @@ static int shape_rowq8(const ojh_kernel_spec *s, const ojh_device *, uint32_t, u
     return OJH_OK;
 }
 
+// Family "q80_dp4a" (block_q8_0 rows against activations quantized per 32): `rows_per_wave` selects the entry
+//   0 quantize_q8_1(x, q8, d8, d8sum, K)                           grid [ceil(K/256),1,1]
+//   1 gemv_q80_dp4a(w, q8, d8, y, K, N)   2 .._bias(+ bias)   3 .._accum    grid [ceil(N/8),1,1]
+//   4 qkv_q80_dp4a(wq, wk, wv, q8, d8, q, k, v, bias, K, Nq, Nkv)    grid [ceil((Nq + 2 Nkv)/8),1,1]
+//   5 ffn_gu_q80_dp4a(wg, wu, q8, d8, out, K, N, act)               grid [ceil(N/4),1,1]
+static int check_q80_dp4a(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                          const uint32_t block[3], size_t need[16], size_t align[16]) {
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    const uint32_t K = c[0];
+    if (!K || K % 32) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a positive multiple of 32", s->name, K);
+    const size_t nblk = K / 32, rb = nblk * 34;
+    uint32_t rows = 0, per = 8;
+    switch (s->rows_per_wave) {
+    case 0:
+        rows = K; per = 256;
+        need[0] = (size_t)K * 4; need[1] = K; need[2] = need[3] = nblk * 4;
+        align[0] = align[2] = align[3] = 4;
+        break;
+    case 1: case 2: case 3: {
+        const uint32_t N = c[1];
+        if (!N) return ojh_fail(OJH_ERR_ARG, "%s: N must be positive", s->name);
+        rows = N;
+        need[0] = (size_t)N * rb; need[1] = K; need[2] = nblk * 4; need[3] = (size_t)N * 4;
+        if (s->rows_per_wave == 2) need[4] = (size_t)N * 4;
+        align[0] = 2; align[1] = 8; align[2] = align[3] = align[4] = 4;
+        break;
+    }
+    case 4: {
+        const uint32_t Nq = c[1], Nkv = c[2];
+        if (!Nq || !Nkv || (uint64_t)Nq + 2ull * Nkv > 0x7FFFFFFFull) return ojh_fail(OJH_ERR_ARG, "%s: Nq=%u Nkv=%u", s->name, Nq, Nkv);
+        rows = Nq + 2 * Nkv;
+        need[0] = (size_t)Nq * rb; need[1] = need[2] = (size_t)Nkv * rb; need[3] = K; need[4] = nblk * 4;
+        need[5] = (size_t)Nq * 4; need[6] = need[7] = (size_t)Nkv * 4; need[8] = (size_t)rows * 4;
+        align[0] = align[1] = align[2] = 2; align[3] = 8;
+        for (int i = 4; i < 9; i++) align[i] = 4;
+        break;
+    }
+    default: {
+        const uint32_t N = c[1], act = c[2];
+        if (!N || act > 1) return ojh_fail(OJH_ERR_ARG, "%s: N=%u act=%u", s->name, N, act);
+        rows = N; per = 4;
+        need[0] = need[1] = (size_t)N * rb; need[2] = K; need[3] = nblk * 4; need[4] = (size_t)N * 4;
+        align[0] = align[1] = 2; align[2] = 8; align[3] = align[4] = 4;
+        break;
+    }
+    }
+    if ((uint64_t)grid[0] * per < rows || !grid[0])
+        return ojh_fail(OJH_ERR_ARG, "%s: grid [%u] x %u does not cover %u", s->name, grid[0], per, rows);
+    return OJH_OK;
+}
+// (K, N, M) = (K, rows — for qkv: Nq + 2 Nkv, -)
+static int shape_q80_dp4a(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, uint32_t N, uint32_t,
+                          uint32_t grid[3], uint32_t block[3]) {
+    grid[0] = s->rows_per_wave == 0 ? (K + 255) / 256 : s->rows_per_wave == 5 ? (N + 3) / 4 : (N + 7) / 8;
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // relayout_q4k_q4l(w, nib, qa, qb, nblocks): 8 threads per super-block
 static int check_relayout(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                           const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -1290,6 +1352,12 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("embed_q80_g", "dequant", 3, 1, OJH_Q8_0, 0, check_embed, shape_embed);
     m.back().expert_bufs = 1;
     m.back().bound_first = 0;
+    add("quantize_q8_1", "q80_dp4a", 4, 1, OJH_Q8_0, 0, check_q80_dp4a, shape_q80_dp4a);
+    add("gemv_q80_dp4a", "q80_dp4a", 4, 2, OJH_Q8_0, 1, check_q80_dp4a, shape_q80_dp4a);
+    add("gemv_q80_dp4a_bias", "q80_dp4a", 5, 2, OJH_Q8_0, 2, check_q80_dp4a, shape_q80_dp4a);
+    add("gemv_q80_dp4a_accum", "q80_dp4a", 4, 2, OJH_Q8_0, 3, check_q80_dp4a, shape_q80_dp4a);
+    add("qkv_q80_dp4a", "q80_dp4a", 9, 3, OJH_Q8_0, 4, check_q80_dp4a, shape_q80_dp4a);
+    add("ffn_gu_q80_dp4a", "q80_dp4a", 5, 3, OJH_Q8_0, 5, check_q80_dp4a, shape_q80_dp4a);
     add("rows_q8_from_f16", "rowq8", 3, 2, 0, 0, check_rowq8, shape_rowq8);
     add("quant_rows_i8", "rowq8", 3, 2, 0, 1, check_rowq8, shape_rowq8);
     add("matmul_q8row", "rowq8", 5, 3, 0, 2, check_rowq8, shape_rowq8);

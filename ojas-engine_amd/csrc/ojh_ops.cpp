@@ -448,6 +448,32 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     void *wp = at(w->raw, w->off), *yp = at(y, y_off);
     uint32_t grid[3] = {1, 1, 1}, block[3] = {256, 1, 1};
 
+    // Q8_0 rows on the reference GPU decode path's arithmetic: activations quantized per 32 (quantize_q8_1), integer
+    // dots against the blocks as the file stores them (crates/ojas-cuda/src/kernels/gemv_q8.rs:152-215), token by token.
+    if (act_mode == OJH_ACT_Q8_1) {
+        if (w->type != OJH_Q8_0) return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: OJH_ACT_Q8_1 serves Q8_0 rows, not %s", f->tag);
+        if (x_dtype != OJH_X_F32) return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: OJH_ACT_Q8_1 takes f32 activations");
+        if ((rc = ensure(dev, "q80_dp4a"))) return rc;
+        const size_t nblk = K / 32;
+        ojh_buf *q8, *d8, *d8s;
+        if ((rc = ojh_scratch_get(dev, "q81_q", (size_t)m * K, &q8))) return rc;
+        if ((rc = ojh_scratch_get(dev, "q81_d", (size_t)m * nblk * 4, &d8))) return rc;
+        if ((rc = ojh_scratch_get(dev, "q81_s", (size_t)m * nblk * 4, &d8s))) return rc;
+        const char *name = accum ? "gemv_q80_dp4a_accum" : bias ? "gemv_q80_dp4a_bias" : "gemv_q80_dp4a";
+        if (accum && bias) return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: OJH_ACT_Q8_1 adds a bias or accumulates, not both");
+        uint32_t qg[3] = {(K + 255) / 256, 1, 1}, gg[3] = {(N + 7) / 8, 1, 1};
+        for (uint32_t t = 0; t < m; t++) {
+            void *tq = (char *)q8->ptr + (size_t)t * K, *td = (char *)d8->ptr + (size_t)t * nblk * 4;
+            if ((rc = ojh_launch(dev, "quantize_q8_1", {(char *)at(x, x_off) + (size_t)t * K * 4, tq, td, (char *)d8s->ptr + (size_t)t * nblk * 4},
+                                 {K}, qg, block)))
+                return rc;
+            std::vector<void *> p = {wp, tq, td, (char *)yp + (size_t)t * N * 4};
+            if (bias && !accum) p.push_back(bias->ptr);
+            if ((rc = ojh_launch(dev, name, p, {K, N}, gg, block))) return rc;
+        }
+        return OJH_OK;
+    }
+
     // Q5_K: the CPU path's arithmetic (dot_q5k over int8 activations) unless floating-point activations are
     // asked for, which run on the f32-activation matvecs at any token count; no MFMA tile reads the format.
     const bool q5_float = w->type == OJH_Q5_K && (act_mode == OJH_ACT_FLOAT || act_mode == OJH_ACT_FLOAT_EXACT);

@@ -243,6 +243,24 @@ def tvec_first(seeds: np.ndarray) -> np.ndarray:
     return ((s >> np.uint64(9)).astype(np.float32) / np.float32(1 << 23)) - np.float32(1.0)
 
 
+def q80_rows_mod5(rows: int, k: int, seed: int) -> tuple[np.ndarray, np.ndarray]:
+    """Q8_0 rows of the reference's integer-dot conformance tests and the values a reader decodes them to
+    (crates/ojas-cuda/tests/conformance.rs:607-628): block (r, b) has d = f16(0.004 + 0.001 ((r + b) % 5)),
+    code i = round(127 tvec(1, seed + r k + 32 b + i)), halves away from zero."""
+    nb = k // 32
+    r, b = np.divmod(np.arange(rows * nb), nb)
+    d = (np.float32(0.004) + np.float32(0.001) * ((r + b) % 5).astype(np.float32)).astype(np.float16)
+    t = tvec_first(np.uint64(seed) + np.arange(rows * k, dtype=np.uint64)) * np.float32(127.0)
+    q = np.clip(np.sign(t) * np.floor(np.abs(t) + np.float32(0.5)), -127, 127).astype(np.int8).reshape(rows * nb, 32)
+    out = np.empty((rows * nb, 34), np.uint8)
+    dv = d.view(np.uint16)
+    out[:, 0] = dv & 0xFF
+    out[:, 1] = dv >> 8
+    out[:, 2:] = q.view(np.uint8)
+    plain = (q.astype(np.float32) * d.astype(np.float32)[:, None]).reshape(rows, k)
+    return out.reshape(-1), plain
+
+
 def q80_rows_lcg(rows: int, k: int, seed: int) -> tuple[np.ndarray, np.ndarray]:
     """Q8_0 rows of the reference's GPU conformance tests and the values they decode to
     (crates/ojas-cuda/tests/conformance.rs:358-376): block (r, b) has d = f16(0.002 + 0.001 |tvec(1, seed ^ (r nb + b))|),

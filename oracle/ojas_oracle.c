@@ -489,6 +489,44 @@ float ojo_quant_row_i8(const float *row, size_t k, int8_t *q) { /* cpu_math.rs:1
     return scale;
 }
 
+/* The reference GPU decode path's activation quantizer (crates/ojas-cuda/src/kernels/gemv.rs:33-52): per block of 32,
+ * d8 = amax / 127, id = d8 > 0 ? 1 / d8 : 0, q = clamp(round-to-nearest-even(x * id), -127, 127), d8sum = d8 * sum q. */
+void ojo_quantize_q8_1(const float *x, size_t k, int8_t *q8, float *d8, float *d8sum) {
+    for (size_t b = 0; b < k / 32; b++) {
+        const float *xb = x + b * 32;
+        float a = 0.0f;
+        for (int i = 0; i < 32; i++) a = fmaxf(a, fabsf(xb[i]));
+        float d = a / 127.0f, id = d > 0.0f ? 1.0f / d : 0.0f, s = 0.0f;
+        for (int i = 0; i < 32; i++) {
+            float r = rintf(xb[i] * id);
+            int qi = r != r ? 0 : r > 127.0f ? 127 : r < -127.0f ? -127 : (int)r;
+            q8[b * 32 + i] = (int8_t)qi;
+            s += (float)qi;
+        }
+        d8[b] = d;
+        d8sum[b] = d * s;
+    }
+}
+/* One block_q8_0 row against q8_1 activations (crates/ojas-cuda/src/kernels/gemv_q8.rs:178-193): a lane's term is
+ * dw * d8[b] * (float) idot over its 8 weights; the GPU adds the terms in a lane and then across lanes in an order of its
+ * own, here they meet in a double (the kernels are compared to a tolerance of a few f32 roundings). */
+double ojo_row_q80_dp4a(const uint8_t *row, const int8_t *q8, const float *d8, size_t k) {
+    double sum = 0.0;
+    for (size_t b = 0; b < k / 32; b++) {
+        const uint8_t *blk = row + b * 34;
+        float dw = rdh(blk, 0);
+        for (int sub = 0; sub < 4; sub++) {
+            int32_t si = 0;
+            for (int i = 0; i < 8; i++) si += (int32_t)(int8_t)blk[2 + sub * 8 + i] * (int32_t)q8[b * 32 + sub * 8 + i];
+            sum += (double)(dw * d8[b] * (float)si);
+        }
+    }
+    return sum;
+}
+void ojo_gemv_q80_dp4a(const uint8_t *w, const int8_t *q8, const float *d8, size_t k, size_t n, float *y) {
+    for (size_t r = 0; r < n; r++) y[r] = (float)ojo_row_q80_dp4a(w + r * (k / 32) * 34, q8, d8, k);
+}
+
 /* ---------------------------------------------------------------- row dots */
 
 float ojo_dot_q80(const uint8_t *row, const float *x, size_t k) { /* cpu_math.rs:971-981 */

@@ -84,6 +84,9 @@ int ojo_matvec_kq(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const flo
 
 /* Row-int8 path every dense CPU model runs (cpu_math.rs:174-179, :187-274, :404-415)
  * and its load-time requantizer (crates/ojas-formats/src/quant.rs:16-39). */
+void ojo_quantize_q8_1(const float *x, size_t k, int8_t *q8, float *d8, float *d8sum);
+double ojo_row_q80_dp4a(const uint8_t *row, const int8_t *q8, const float *d8, size_t k);
+void ojo_gemv_q80_dp4a(const uint8_t *w, const int8_t *q8, const float *d8, size_t k, size_t n, float *y);
 float ojo_quant_row_i8(const float *row, size_t k, int8_t *q);
 void  ojo_q8_rows_from_f16(const uint16_t *w16, size_t n, size_t k, int8_t *q, float *scale);
 void  ojo_matmul_q8(const int8_t *wq, const float *wscale, size_t n, size_t k,

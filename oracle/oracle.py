@@ -63,6 +63,10 @@ def lib() -> C.CDLL:
         L.ojo_matvec_kq.argtypes = [vp, u32, sz, sz, vp, i32, vp]
         L.ojo_quant_row_i8.restype = C.c_float
         L.ojo_quant_row_i8.argtypes = [vp, sz, vp]
+        L.ojo_quantize_q8_1.restype = None
+        L.ojo_quantize_q8_1.argtypes = [vp, sz, vp, vp, vp]
+        L.ojo_gemv_q80_dp4a.restype = None
+        L.ojo_gemv_q80_dp4a.argtypes = [vp, vp, vp, sz, sz, vp]
         L.ojo_q8_rows_from_f16.restype = None
         L.ojo_q8_rows_from_f16.argtypes = [vp, sz, sz, vp, vp]
         L.ojo_matmul_q8.restype = None
@@ -177,6 +181,21 @@ def quant_row_i8(row: np.ndarray):
     q = np.empty(row.size, np.int8)
     s = lib().ojo_quant_row_i8(_p(row), row.size, _p(q))
     return q, float(s)
+
+
+def quantize_q8_1(x: np.ndarray):
+    x = np.ascontiguousarray(x, np.float32)
+    q8, d8, d8sum = np.empty(x.size, np.int8), np.empty(x.size // 32, np.float32), np.empty(x.size // 32, np.float32)
+    lib().ojo_quantize_q8_1(_p(x), x.size, _p(q8), _p(d8), _p(d8sum))
+    return q8, d8, d8sum
+
+
+def gemv_q80_dp4a(raw: np.ndarray, q8: np.ndarray, d8: np.ndarray, n: int, k: int) -> np.ndarray:
+    raw, q8, d8 = np.ascontiguousarray(raw, np.uint8), np.ascontiguousarray(q8, np.int8), np.ascontiguousarray(d8, np.float32)
+    assert raw.size == n * (k // 32) * 34 and q8.size == k and d8.size == k // 32
+    y = np.empty(n, np.float32)
+    lib().ojo_gemv_q80_dp4a(_p(raw), _p(q8), _p(d8), k, n, _p(y))
+    return y
 
 
 def q8_rows_from_f16(w16: np.ndarray, n: int, k: int):

@@ -461,6 +461,43 @@ def test_other_routers_match_closed_forms(orc, pkg):
     assert list(idx[0]) == [0, 1, 2, 3]
 
 
+def test_q8_1_quantizer_and_integer_dot_restatements(orc, pkg):
+    """`quantize_q8_1` (crates/ojas-cuda/src/kernels/gemv.rs:33-52) against its closed form, and the block_q8_0 integer
+    dot (crates/ojas-cuda/src/kernels/gemv_q8.rs:178-193) against exact integer arithmetic in f64 and, by the reference's
+    own test (crates/ojas-cuda/tests/conformance.rs:563-605: K = 1024, N = 128, x = tvec(K, 81), its block generator),
+    within 1e-2 of the output peak of the dequantized dot."""
+    k, n = 1024, 128
+    x = pkg.synth.tvec(k, 81)
+    q8, d8, d8sum = orc.quantize_q8_1(x)
+    xb = x.reshape(-1, 32)
+    d = (np.abs(xb).max(1) / np.float32(127.0)).astype(np.float32)
+    assert np.array_equal(d8, d)
+    inv = (np.float32(1.0) / d).astype(np.float32)
+    want_q = np.clip(np.rint(xb * inv[:, None]), -127, 127).astype(np.int8)
+    assert np.array_equal(q8.reshape(-1, 32), want_q)
+    assert np.array_equal(d8sum, d * want_q.sum(1).astype(np.float32))
+    assert np.abs(q8.reshape(-1, 32)).max(1).min() == 127          # every block reaches the end of the range
+    # an all-zero block: scale 0, codes 0 (id = 0, not 1 / 0)
+    z = x.copy(); z[64:96] = 0.0
+    qz, dz, sz = orc.quantize_q8_1(z)
+    assert dz[2] == 0.0 and sz[2] == 0.0 and not qz[64:96].any()
+    w, plain = pkg.synth.q80_rows_mod5(n, k, 82)
+    got = orc.gemv_q80_dp4a(w, q8, d8, n, k)
+    blocks = w.reshape(n, k // 32, 34)
+    dw = blocks[:, :, :2].copy().view(np.float16).astype(np.float64)[:, :, 0]
+    wq = blocks[:, :, 2:].view(np.int8).astype(np.int64)
+    idot = (wq * q8.reshape(1, -1, 32).astype(np.int64)).sum(2)
+    exact = (dw * d8.astype(np.float64)[None, :] * idot).sum(1)
+    assert np.max(np.abs(got - exact)) <= 1e-6 * np.max(np.abs(exact))
+    reader = (plain.astype(np.float64) * x.astype(np.float64)).sum(1)
+    assert np.max(np.abs(got - reader)) / np.max(np.abs(reader)) < 1e-2
+    # a transposed operand or a dropped block would not survive this: one nonzero block, one nonzero code
+    w1 = np.zeros((1, k // 32, 34), np.uint8)
+    w1[0, 5, :2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    w1[0, 5, 2 + 9] = np.uint8(np.int8(-3))
+    assert orc.gemv_q80_dp4a(w1.reshape(-1), q8, d8, 1, k)[0] == np.float32(0.5) * d8[5] * np.float32(-3 * int(q8[5 * 32 + 9]))
+
+
 def test_matmul_q8_row_int8_path(orc):
     rng = np.random.default_rng(7)
     n, k, m = 9, 64, 3
