@@ -4,8 +4,9 @@
 // `ojh_mm` under OJH_ACT_Q8K stages the int8 form of the activations and their per-256 scales in a
 // per-device scratch buffer that it allocates and grows on demand.  Here that staging lives in a
 // file-scope device array of fixed size instead, so nothing in the call allocates or frees: the
-// quantizer writes into the array, the matvec / MFMA entries read it back, exactly the launches
-// `ojh_mm` issues (results are bit-identical).
+// quantizer writes into the array, the matvec / MFMA entries read it back: the launches `ojh_mm`
+// issues for up to 95 tokens (bit-identical results); beyond, `ojh_mm` may take a prefill tile that
+// stages more in library scratch, which this entry never does.
 //
 // The array's name is a host-side stand-in, not a device address.  Its address on each GPU is
 // asked of the runtime once, when a device handle is opened with that GPU current, and only that
