@@ -39,7 +39,7 @@ STAGES = [("x_attn", 4096, ["q", "k", "v"]), ("x_o", 4096, ["o"]), ("x_ffn", 409
 # HBM bytes per launch of the head matvec (128256 x 4096 Q4_K) from hardware counters: FETCH_SIZE
 # 144 324.7 KiB x 2.000 (the factor the same counter needs to read a 512 MiB copy correctly) +
 # WRITE_SIZE 501.4 KiB.  Algorithmic bytes of the launch: 296 031 232.
-HEAD_TRAFFIC_BYTES = 296_090_000
+HEAD_TRAFFIC_BYTES = 296_101_824
 
 
 def algorithmic_bytes(n: int, k: int) -> int:
@@ -351,6 +351,10 @@ def extras(gpu, pkg, lin_q) -> dict:
     us = _time(gpu, lambda i: gpu.mm(x, wq8[i % 16], y), 64, 16)
     b = n * (k // 32) * 34 + 4 * k + 4 * n
     out["q80_gemv_4096x4096"] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
+    # the same matrix on the reference GPU decode path's arithmetic: activations quantized per 32, integer dots
+    us = _time(gpu, lambda i: gpu.mm(x, wq8[i % 16], y, act_mode=pkg.ACT_Q8_1), 64, 16)
+    out["q80_dp4a_gemv_4096x4096"] = {"timed": "quantize_q8_1 + gemv_q80_dp4a", "us": round(us, 2), "gbs": round(b / us / 1e3, 1),
+                                      "hbm_frac": round(b / us / 8e6, 4)}
     del wq8
     # the same contract on a tall matrix (rows staged through LDS, activations in registers)
     n = 128256
@@ -415,7 +419,7 @@ def extras(gpu, pkg, lin_q) -> dict:
         fl = 2.0 * T * ksel * 3 * nff * d
         moe[f"T{T}"] = {"us": round(us, 1), "distinct_experts": distinct, "gbs": round(b / us / 1e3, 1),
                         "tflops": round(fl / us / 1e6, 2)}
-    out["moe_ffn_q4k_128x_top8"] = {"timed": "router + expert FFN (T <= 8: gate/up and down launches addressed by assignment; above: quantize, group, gate/up, quantize, down, combine; T = 256 on int8 MFMA, moe_{gu,down}_q4k_mt)", **moe}
+    out["moe_ffn_q4k_128x_top8"] = {"timed": "router + expert FFN (T <= 8: gate/up and down launches addressed by assignment; above: quantize + group in one launch, gate/up, quantize, down, combine; T = 256 on int8 MFMA, moe_{gu,down}_q4k_mt, 32 assignments per staged pass)", **moe}
     del gate, up, down
     # ---- speculative verify on a Q6_K output head 151936 x 4096, bf16 activations
     n, k = 151936, 4096

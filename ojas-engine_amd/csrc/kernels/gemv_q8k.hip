@@ -1287,9 +1287,10 @@ gemv_q8k_q6k_mk(const signed char* xq, const float* xs, const uchar* w, float* y
 // four copies) and walks its tiles as one stream of units, D copies ahead across tile borders (a
 // unit's slot is given to the copy D units on as soon as its bytes are in registers);
 // waves never wait for each other after the tokens are staged.
-// The sixteen slots of a unit are packed (row n at 224 n, 16 bytes further for n >= 8): 224 bytes are 56 banks, so rows
-// 0 .. 7 start at banks 0, 56, .. 8 and rows 8 .. 15 between them, and the pieces that half a wave reads (sixteen rows,
-// two k groups) fall on all 64 banks once.  A unit is 3616 bytes (the last slot's readers may fetch a dword past it):
+// The sixteen slots of a unit are packed (row n at 224 n, 16 bytes further for n >= 8: 224 bytes are 56 banks, so rows
+// 0 .. 7 start at banks 0, 56, .. 8 and rows 8 .. 15 between them).  The readers' dword fetches still meet two to a bank
+// (the conflict counter reads 57 % of LDS-active cycles with this layout as with slots 1024 bytes apart); LDS time is
+// not what bounds the kernel.  A unit is 3616 bytes (the last slot's readers may fetch a dword past it):
 // rings are 4 units deep up to 8 tokens and 3 beyond where that fits beside the tokens (one less where not), so 4 (3)
 // units of 3360 weight bytes are on their way per wave while it works.
 #define Q6K_ML_SLOT 224u
