@@ -324,6 +324,239 @@ __device__ __forceinline__ void gemm_xl_body(const ushort* __restrict__ xh, cons
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same product with the weights dequantized straight into the matrix cores' B registers:
+//   gemm_mm_q4kl_bd(xh, w, y, K, N, accum, M)         grid [ceil(N/256), ceil(M/128), 1]
+//   gemm_mm_q4kl_bd_sk(xh, w, y, K, N, M, nsplit)     grid.z = nsplit (slices of whole super-blocks); f32 atomic adds
+// In the tiles above a thread dequantizes one weight row into LDS and every wave reads the f16 tile back as B
+// fragments: per K step 32 KB of LDS writes, a barrier's worth of waiting for them, and 64 KB of fragment reads that
+// carry nothing the wave could not have made itself.  Here a wave owns 64 weight rows against all 128 tokens of the
+// tile (4 x 2 blocks of v_mfma_f32_32x32x16_f16, 128 accumulators): lane (n, g) of the B operand holds 8 consecutive
+// k of row n, and 8 consecutive weights of a Q4_K chunk are the low (or high) nibbles of 8 consecutive bytes, so the
+// lane fetches 16 bytes of its two rows per K step and turns them into the four sub-steps' B registers itself — the
+// same two vector instructions per weight, no LDS round trip, and only the activations are shared through LDS
+// (one 16 KB stage per K step, all four waves read all of it).  The K order inside a step is the lane's:
+// sub-steps cover weights {0, 8, 32, 40} + 16 g + 0..7 (low nibbles of its bytes 0-7 and 8-15, then the high ones),
+// and the activation fragments are read from the same positions.  Raw bytes travel global -> LDS -> the same lane
+// (three K steps ahead for the nibbles, a header slot per super-block), so nothing asynchronous targets a register
+// and no barrier guards them; the one barrier per step is for the activation stage.  80 KB of LDS and at most 128
+// vector registers beside the accumulators: two workgroups per CU, one's dequantization under the other's MFMAs.
+#define GB_BM 128u
+#define GB_XSTAGE (GB_BM * GX_ROW)        // 16 KB
+#define GB_NIB(XS) ((XS) * GB_XSTAGE)      // 4 slots x 4 waves x 2 rows x 1 KB
+#define GB_HDR(XS) (GB_NIB(XS) + 32768u)   // 2 slots x 4 waves x 2 rows x 1 KB
+#define GB_LDS(XS) (GB_HDR(XS) + 16384u)
+
+struct GbRow {
+    u32x4 hdr, q;
+    half2v a_lo, c_lo, a_hi, c_hi;
+    __device__ __forceinline__ void prep(uint c) {
+        uint sc, mn;
+        q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
+        const float d = f16_bits_to_f32(hdr.x & 0xFFFFu), ndm = -f16_bits_to_f32(hdr.x >> 16);
+        float p1 = d * (float)(sc & 0xFFu), r1 = ndm * (float)(mn & 0xFFu);
+        float p2 = d * (float)(sc >> 8), r2 = ndm * (float)(mn >> 8);
+        asm volatile("" : "+v"(p1), "+v"(r1), "+v"(p2), "+v"(r2));
+        const _Float16 a1 = (_Float16)p1, b1 = (_Float16)r1, a2 = (_Float16)p2, b2 = (_Float16)r2;
+        a_lo = (half2v){a1, a1};
+        c_lo = (half2v){b1, b1};
+        a_hi = (half2v){a2, a2};
+        c_hi = (half2v){b2, b2};
+    }
+    // sub-step S (0, 1: low nibbles of bytes 0-7, 8-15; 2, 3: the high ones) as a B fragment of 8 weights
+    template <int S>
+    __device__ __forceinline__ half8 frag(uint magic) const {
+        const uint v0 = q[2 * (S & 1)], v1 = q[2 * (S & 1) + 1];
+        constexpr uint sh = S >= 2 ? 4u : 0u;
+        const half2v a = S >= 2 ? a_hi : a_lo, c = S >= 2 ? c_hi : c_lo;
+        const uint p0 = __builtin_amdgcn_perm(0u, v0, 0x0C010C00u) >> sh, p1 = __builtin_amdgcn_perm(0u, v0, 0x0C030C02u) >> sh;
+        const uint p2 = __builtin_amdgcn_perm(0u, v1, 0x0C010C00u) >> sh, p3 = __builtin_amdgcn_perm(0u, v1, 0x0C030C02u) >> sh;
+        const u32x4 r = {GxQ4K::fma2(GxQ4K::nib2h(p0, magic), a, c), GxQ4K::fma2(GxQ4K::nib2h(p1, magic), a, c),
+                         GxQ4K::fma2(GxQ4K::nib2h(p2, magic), a, c), GxQ4K::fma2(GxQ4K::nib2h(p3, magic), a, c)};
+        return __builtin_bit_cast(half8, r);
+    }
+};
+
+template <bool SPLITK, bool ACCUM, int XS>   // XS activation stages: 2 (80 KB of LDS, two workgroups per CU) or 3 (96 KB)
+__device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, const uchar* __restrict__ w,
+                                             float* __restrict__ y, uint K, uint N, uint M, uint nsplit, uchar* lds) {
+    const uint tid = threadIdx.x, lane = tid & 63u;
+    const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint n0 = blockIdx.x * GX_BN, m0 = blockIdx.y * GB_BM;
+    const uint nsb = K >> 8;
+    uint sb_begin = 0, sb_end = nsb;
+    if (SPLITK) {
+        const uint per = (nsb + nsplit - 1) / nsplit;
+        sb_begin = min(blockIdx.z * per, nsb);
+        sb_end = min((blockIdx.z + 1) * per, nsb);
+        if (sb_begin >= sb_end) return;
+    }
+    const uint nt = (sb_end - sb_begin) * 4u, last = nt - 1u;
+    const uint k_begin = sb_begin << 8;
+    const uint lds0 = (uint)(size_t)(__attribute__((address_space(3))) uchar*)lds;
+
+    // activation stage: wave `wave`, copy i moves rows (wave*4 + i)*8 .. +7; lane -> row lane/8, slot lane%8, which
+    // holds source chunk (lane%8) ^ ((row/2)%8)
+    uint xoff[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint r = (wave * 4u + i) * 8u + (lane >> 3);
+        const uint m = min(m0 + r, M - 1u);
+        xoff[i] = m * K * 2u + (((lane & 7u) ^ ((r >> 1) & 7u)) << 4);
+    }
+    const uint x_lds = lds0 + wave * 4096u;                      // + stage * GB_XSTAGE + i * 1024
+    // the lane's two weight rows: B column fr of blocks j = 0, 1; its 16 nibble bytes are bytes 16 g .. of a chunk
+    const uint fr = lane & 31u, kg = lane >> 5, sw = (fr >> 1) & 7u;
+    const uint row_bytes = nsb * Q4K_BYTES;
+    const uint ro0 = min(n0 + wave * 64u + fr, N - 1u) * row_bytes, ro1 = min(n0 + wave * 64u + 32u + fr, N - 1u) * row_bytes;
+    const uint nib_lds = lds0 + GB_NIB(XS) + wave * 2048u;           // + slot * 8192 + j * 1024
+    const uint hdr_lds = lds0 + GB_HDR(XS) + wave * 2048u;           // + slot * 8192 + j * 1024
+    const uchar* const nib_rd = lds + GB_NIB(XS) + wave * 2048u + lane * 16u;
+    const uchar* const hdr_rd = lds + GB_HDR(XS) + wave * 2048u + lane * 16u;
+    const uchar* const a_rd = lds + fr * GX_ROW;                 // + stage * GB_XSTAGE + i * 32 rows + chunk slot
+
+    float16v acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+    uint magic = 0x64006400u;
+    asm volatile("" : "+v"(magic));
+    const uchar* xbase = (const uchar*)xh;
+
+    // requests past the last step are clamped onto it, so that every step issues the same eight copies
+    auto copy_x = [&](uint t) {
+        const uchar* b = xbase + (size_t)(k_begin + min(t, last) * GX_BK) * 2u;
+#pragma unroll
+        for (int i = 0; i < 4; i++) gx_load_lds16(b, xoff[i], x_lds + (XS == 2 ? (t & 1u) : t % 3u) * GB_XSTAGE + i * 1024u);
+    };
+    auto copy_w = [&](uint t) {
+        const uint tc = min(t, last), sb = sb_begin + (tc >> 2);
+        const uchar* bh = w + (size_t)sb * Q4K_BYTES;
+        const uchar* bn = bh + 16u + (tc & 3u) * 32u;
+        gx_load_lds16(bn, ro0 + 16u * kg, nib_lds + (t & 3u) * 8192u);
+        gx_load_lds16(bn, ro1 + 16u * kg, nib_lds + (t & 3u) * 8192u + 1024u);
+        gx_load_lds16(bh, ro0, hdr_lds + ((tc >> 2) & 1u) * 8192u);
+        gx_load_lds16(bh, ro1, hdr_lds + ((tc >> 2) & 1u) * 8192u + 1024u);
+    };
+    GbRow r0, r1;
+    half8 afA[4], afB[4], b0, b1, c0, c1;
+#define GB_READ_A(T, CH, AF)                                                                           \
+    do {                                                                                               \
+        const uchar* xa_ = a_rd + (XS == 2 ? ((T) & 1u) : (T) % 3u) * GB_XSTAGE + ((((CH) + 2u * kg) ^ sw) << 4);             \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) AF[i] = *(const half8*)(xa_ + i * 32u * GX_ROW); \
+    } while (0)
+#define GB_READ_W(T)                                                                                   \
+    do {                                                                                               \
+        const uint tc_ = min((T), last), slot_ = ((T) & 3u) * 8192u, hs_ = ((tc_ >> 2) & 1u) * 8192u;  \
+        r0.q = *(const u32x4*)(nib_rd + slot_);                                                        \
+        r1.q = *(const u32x4*)(nib_rd + slot_ + 1024u);                                                \
+        r0.hdr = *(const u32x4*)(hdr_rd + hs_);                                                        \
+        r1.hdr = *(const u32x4*)(hdr_rd + hs_ + 1024u);                                                \
+        r0.prep(tc_ & 3u);                                                                             \
+        r1.prep(tc_ & 3u);                                                                             \
+    } while (0)
+#define GB_MMA(AF, B0, B1)                                                                             \
+    do {                                                                                               \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                \
+            acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(AF[i], B0, acc[i][0], 0, 0, 0);         \
+            acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(AF[i], B1, acc[i][1], 0, 0, 0);         \
+        }                                                                                              \
+    } while (0)
+// eight MFMAs with the next fragments' LDS reads behind the first two and NV vector instructions behind each
+#define GB_MIX(NV)                                                                                     \
+    do {                                                                                               \
+        _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {                                             \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                         \
+            if (g_ < 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                             \
+            __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);                                        \
+        }                                                                                              \
+    } while (0)
+    // prologue: the state a step expects on entry — the first sub-step's activation and weight fragments in
+    // registers, the step's raw rows unpacked, the copies for the next step and the weights two steps on under way
+    copy_w(0u);
+    copy_w(1u);
+    copy_x(0u);
+    if (XS == 3) copy_x(1u);
+    gx_wait<0>();
+    __syncthreads();
+    GB_READ_A(0u, 0u, afA);
+    GB_READ_W(0u);
+    b0 = r0.frag<0>(magic);
+    b1 = r1.frag<0>(magic);
+    copy_x(XS == 2 ? 1u : 2u);
+    copy_w(2u);
+    for (uint t = 0; t < nt; t++) {
+        __builtin_amdgcn_sched_barrier(0);
+        GB_READ_A(t, 1u, afB); GB_MMA(afA, b0, b1);
+        c0 = r0.frag<1>(magic); c1 = r1.frag<1>(magic);
+        GB_MIX(4);
+        GB_READ_A(t, 4u, afA); GB_MMA(afB, c0, c1);
+        b0 = r0.frag<2>(magic); b1 = r1.frag<2>(magic);
+        GB_MIX(5);
+        GB_READ_A(t, 5u, afB); GB_MMA(afA, b0, b1);
+        c0 = r0.frag<3>(magic); c1 = r1.frag<3>(magic);
+        GB_MIX(5);
+        __builtin_amdgcn_sched_barrier(0);
+        // x(t + 1) has landed, and with it everything older (the weights of t + 1 among them); only what was issued
+        // behind it (four weight copies; with three stages the whole batch of the step before) may still be on its
+        // way.  Past the barrier nobody reads the stage of step t any more.
+        gx_wait<XS == 2 ? 4 : 8>();
+        __syncthreads();
+        copy_x(t + (uint)XS);
+        copy_w(t + 3u);
+        __builtin_amdgcn_sched_barrier(0);
+        GB_READ_A(t + 1u, 0u, afA);
+        GB_READ_W(t + 1u);
+        GB_MMA(afB, c0, c1);
+        b0 = r0.frag<0>(magic); b1 = r1.frag<0>(magic);
+        _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (g_ < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 11, 0);
+        }
+    }
+    gx_wait<0>();
+#undef GB_READ_A
+#undef GB_READ_W
+#undef GB_MMA
+#undef GB_MIX
+
+    // epilogue: D register v of block (i, j) holds token row 32 i + 8 (v / 4) + 4 kg + v % 4, output 64 wave + 32 j + fr
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const uint n = n0 + wave * 64u + 32u * j + fr;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const uint m = m0 + 32u * i + 8u * (v >> 2) + 4u * kg + (v & 3u);
+                if (m < M && n < N) {
+                    float* o = y + (size_t)m * N + n;
+                    if (SPLITK) atomicAdd(o, acc[i][j][v]);
+                    else if (ACCUM) *o += acc[i][j][v];
+                    else *o = acc[i][j][v];
+                }
+            }
+        }
+    }
+}
+
+// (A variant with three activation stages, copies two steps ahead, 96 KB and one workgroup per CU, measured the same at
+// 224 workgroups and is not built: the activation copies are not what a step waits for.)
+extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+gemm_mm_q4kl_bd(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
+    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(2)];
+    if (accum) gemm_bd_body<false, true, 2>(xh, w, y, K, N, M, 1u, lds);
+    else gemm_bd_body<false, false, 2>(xh, w, y, K, N, M, 1u, lds);
+}
+extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+gemm_mm_q4kl_bd_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
+    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(2)];
+    gemm_bd_body<true, true, 2>(xh, w, y, K, N, M, nsplit, lds);
+}
 // LDS of a tile: two activation stages, two dequantized-weight stages, two raw-weight slots
 #define GX_LDS(MI) __shared__ __attribute__((aligned(1024))) uchar lds[2 * 64 * (MI) * GX_ROW + 2 * GX_WSTAGE + 2 * GX_RAW]
 

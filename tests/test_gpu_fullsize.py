@@ -142,7 +142,7 @@ def test_prefill_gemm_at_full_size(gpu, orc, pkg, n, k, m):
     assert e[0] < 2e-6, e          # three or more K slices meet in f32 atomics, in no fixed order
     gpu.ensure_family("gemm_xl")
     tall = gpu.launch_shape("gemm_mm_q4kl_sk", k, n, m)[0][2]
-    half = gpu.launch_shape("gemm_mm_q4kl_m128_sk", k, n, m)[0][2]
+    half = gpu.launch_shape("gemm_mm_q4kl_bd_sk", k, n, m)[0][2]
     if max(tall, half) <= 2:       # one or two slices: a + b = b + a, so bit for bit
         assert np.array_equal(got2, got[perm])
     # the first 128 tokens alone: another tile height and K split, so sums associate differently

@@ -14,7 +14,7 @@ below); for Q4_K under ACT_FLOAT the binary16 fma qa*q + qb of the reference's `
 import numpy as np
 import pytest
 
-from conftest import rms_errs
+from conftest import peak_err, rms_errs
 
 pytestmark = pytest.mark.gpu
 Q8_0, Q4_K, Q6_K = 8, 12, 14
@@ -104,7 +104,8 @@ def test_tile_holds_the_reference_decoders_bits(gpu, orc, pkg, ty):
 
 @pytest.mark.parametrize("kernel,family,bm,bn,wmode", [("gemm_mm_q4k_sk", "gemm", 256, 128, 1),
                                                        ("gemm_mm_q4kl_sk", "gemm_xl", 256, 256, 2),
-                                                       ("gemm_mm_q4kl_m128_sk", "gemm_xl", 128, 256, 2)])
+                                                       ("gemm_mm_q4kl_m128_sk", "gemm_xl", 128, 256, 2),
+                                                       ("gemm_mm_q4kl_bd_sk", "gemm_xl", 128, 256, 2)])
 def test_split_k_entry_through_the_kernel_seam(gpu, orc, pkg, kernel, family, bm, bn, wmode):
     """Split-K entries dispatched by name with several K slices; y holds what is accumulated into."""
     gpu.ensure_family(family)
@@ -126,6 +127,33 @@ def test_split_k_entry_through_the_kernel_seam(gpu, orc, pkg, kernel, family, bm
         assert e[0] < 1e-4 and e[1] < 2e-5, (nsplit, e)
     with pytest.raises(pkg.OjasHipError, match="grid must be"):
         gpu.dispatch(enc, kernel, [(xh, 0), (wd, 0), (yd, 0)], [k, n, m, 2], [3, 1, 1], [256, 1, 1])
+
+
+@pytest.mark.parametrize("m,k,n", [(140, 2048, 300), (128, 256, 256), (77, 512, 64), (260, 1024, 513)])
+def test_tile_with_weights_dequantized_into_registers(gpu, orc, pkg, m, k, n):
+    """`gemm_mm_q4kl_bd` by name: the 128 x 256 tile whose waves dequantize their own 64 rows into the B operand.  Ragged
+    M and N, store and accumulate, sentinels behind row M; the oracle holds the tile's specified f16 weights, and the
+    tile that shares the dequantized weights through LDS agrees to the order of the f32 sums inside a K step."""
+    gpu.ensure_family("gemm_xl")
+    w = pkg.synth.q4k_weights(n, k, "bd", "w", n, k)
+    x = pkg.synth.normal_f32(m * k, "bd", "x", m, k).reshape(m, k)
+    xh, wd = gpu.upload_bytes(x.astype(np.float16)), gpu.upload_bytes(w)
+    want = orc.matmul_ref(w, Q4_K, n, k, x, wmode=2, xmode=1)
+    grid = [(n + 255) // 256, (m + 127) // 128, 1]
+    sent = np.full(n, 12345.5, np.float32)
+    outs = {}
+    for kernel in ("gemm_mm_q4kl_bd", "gemm_mm_q4kl_m128"):
+        for accum in (0, 1):
+            y0 = pkg.synth.normal_f32(m * n, "bd", "y0", accum).reshape(m, n)
+            yd = gpu.upload(np.concatenate([y0.ravel(), sent]))
+            gpu.dispatch(gpu.begin(), kernel, [(xh, 0), (wd, 0), (yd, 0)], [k, n, accum, m], grid, [256, 1, 1])
+            got = gpu.read(yd, m * n + n)
+            assert np.array_equal(got[m * n:], sent), "wrote past row M"
+            got = got[:m * n].reshape(m, n)
+            e = rms_errs(got, want + (y0 if accum else 0.0))
+            assert e[0] < 1e-4 and e[1] < 2e-5, (kernel, accum, e)
+            outs[kernel, accum] = got
+    assert peak_err(outs["gemm_mm_q4kl_bd", 0], outs["gemm_mm_q4kl_m128", 0]) <= 2e-6
 
 
 def test_q4l_entries_by_their_reference_names(gpu, orc, pkg):
