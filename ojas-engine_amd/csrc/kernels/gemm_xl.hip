@@ -343,9 +343,9 @@ __device__ __forceinline__ void gemm_xl_body(const ushort* __restrict__ xh, cons
 // vector registers beside the accumulators: two workgroups per CU, one's dequantization under the other's MFMAs.
 #define GB_BM 128u
 #define GB_XSTAGE (GB_BM * GX_ROW)        // 16 KB
-#define GB_NIB(XS) ((XS) * GB_XSTAGE)      // 4 slots x 4 waves x 2 rows x 1 KB
-#define GB_HDR(XS) (GB_NIB(XS) + 32768u)   // 2 slots x 4 waves x 2 rows x 1 KB
-#define GB_LDS(XS) (GB_HDR(XS) + 16384u)
+#define GB_NIB (2u * GB_XSTAGE)            // 4 slots x 4 waves x 2 rows x 1 KB
+#define GB_HDR (GB_NIB + 32768u)           // 2 slots x 4 waves x 2 rows x 1 KB
+#define GB_LDS (GB_HDR + 16384u)
 
 struct GbRow {
     u32x4 hdr, q;
@@ -377,7 +377,7 @@ struct GbRow {
     }
 };
 
-template <bool SPLITK, bool ACCUM, int XS>   // XS activation stages: 2 (80 KB of LDS, two workgroups per CU) or 3 (96 KB)
+template <bool SPLITK, bool ACCUM>
 __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, const uchar* __restrict__ w,
                                              float* __restrict__ y, uint K, uint N, uint M, uint nsplit, uchar* lds) {
     const uint tid = threadIdx.x, lane = tid & 63u;
@@ -409,10 +409,10 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
     const uint fr = lane & 31u, kg = lane >> 5, sw = (fr >> 1) & 7u;
     const uint row_bytes = nsb * Q4K_BYTES;
     const uint ro0 = min(n0 + wave * 64u + fr, N - 1u) * row_bytes, ro1 = min(n0 + wave * 64u + 32u + fr, N - 1u) * row_bytes;
-    const uint nib_lds = lds0 + GB_NIB(XS) + wave * 2048u;           // + slot * 8192 + j * 1024
-    const uint hdr_lds = lds0 + GB_HDR(XS) + wave * 2048u;           // + slot * 8192 + j * 1024
-    const uchar* const nib_rd = lds + GB_NIB(XS) + wave * 2048u + lane * 16u;
-    const uchar* const hdr_rd = lds + GB_HDR(XS) + wave * 2048u + lane * 16u;
+    const uint nib_lds = lds0 + GB_NIB + wave * 2048u;           // + slot * 8192 + j * 1024
+    const uint hdr_lds = lds0 + GB_HDR + wave * 2048u;           // + slot * 8192 + j * 1024
+    const uchar* const nib_rd = lds + GB_NIB + wave * 2048u + lane * 16u;
+    const uchar* const hdr_rd = lds + GB_HDR + wave * 2048u + lane * 16u;
     const uchar* const a_rd = lds + fr * GX_ROW;                 // + stage * GB_XSTAGE + i * 32 rows + chunk slot
 
     float16v acc[4][2];
@@ -430,14 +430,17 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
     auto copy_x = [&](uint t) {
         const uchar* b = xbase + (size_t)(k_begin + min(t, last) * GX_BK) * 2u;
 #pragma unroll
-        for (int i = 0; i < 4; i++) gx_load_lds16(b, xoff[i], x_lds + (XS == 2 ? (t & 1u) : t % 3u) * GB_XSTAGE + i * 1024u);
+        for (int i = 0; i < 4; i++) gx_load_lds16(b, xoff[i], x_lds + (t & 1u) * GB_XSTAGE + i * 1024u);
     };
-    auto copy_w = [&](uint t) {
-        const uint tc = min(t, last), sb = sb_begin + (tc >> 2);
-        const uchar* bh = w + (size_t)sb * Q4K_BYTES;
-        const uchar* bn = bh + 16u + (tc & 3u) * 32u;
+    auto copy_nib = [&](uint t) {
+        const uint tc = min(t, last);
+        const uchar* bn = w + (size_t)(sb_begin + (tc >> 2)) * Q4K_BYTES + 16u + (tc & 3u) * 32u;
         gx_load_lds16(bn, ro0 + 16u * kg, nib_lds + (t & 3u) * 8192u);
         gx_load_lds16(bn, ro1 + 16u * kg, nib_lds + (t & 3u) * 8192u + 1024u);
+    };
+    auto copy_hdr = [&](uint t) {               // the header of step t's super-block (a slot per super-block parity)
+        const uint tc = min(t, last);
+        const uchar* bh = w + (size_t)(sb_begin + (tc >> 2)) * Q4K_BYTES;
         gx_load_lds16(bh, ro0, hdr_lds + ((tc >> 2) & 1u) * 8192u);
         gx_load_lds16(bh, ro1, hdr_lds + ((tc >> 2) & 1u) * 8192u + 1024u);
     };
@@ -445,18 +448,22 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
     half8 afA[4], afB[4], b0, b1, c0, c1;
 #define GB_READ_A(T, CH, AF)                                                                           \
     do {                                                                                               \
-        const uchar* xa_ = a_rd + (XS == 2 ? ((T) & 1u) : (T) % 3u) * GB_XSTAGE + ((((CH) + 2u * kg) ^ sw) << 4);             \
+        const uchar* xa_ = a_rd + ((T) & 1u) * GB_XSTAGE + ((((CH) + 2u * kg) ^ sw) << 4);             \
         _Pragma("unroll") for (int i = 0; i < 4; i++) AF[i] = *(const half8*)(xa_ + i * 32u * GX_ROW); \
     } while (0)
-#define GB_READ_W(T)                                                                                   \
+// the raw rows of step T out of their slots (the header only where T starts a super-block), scales of chunk C1
+#define GB_READ_W(T, C1, HDR)                                                                          \
     do {                                                                                               \
-        const uint tc_ = min((T), last), slot_ = ((T) & 3u) * 8192u, hs_ = ((tc_ >> 2) & 1u) * 8192u;  \
+        const uint slot_ = ((T) & 3u) * 8192u;                                                         \
         r0.q = *(const u32x4*)(nib_rd + slot_);                                                        \
         r1.q = *(const u32x4*)(nib_rd + slot_ + 1024u);                                                \
-        r0.hdr = *(const u32x4*)(hdr_rd + hs_);                                                        \
-        r1.hdr = *(const u32x4*)(hdr_rd + hs_ + 1024u);                                                \
-        r0.prep(tc_ & 3u);                                                                             \
-        r1.prep(tc_ & 3u);                                                                             \
+        if (HDR) {                                                                                     \
+            const uint hs_ = ((min((T), last) >> 2) & 1u) * 8192u;                                     \
+            r0.hdr = *(const u32x4*)(hdr_rd + hs_);                                                    \
+            r1.hdr = *(const u32x4*)(hdr_rd + hs_ + 1024u);                                            \
+        }                                                                                              \
+        r0.prep(C1);                                                                                   \
+        r1.prep(C1);                                                                                   \
     } while (0)
 #define GB_MMA(AF, B0, B1)                                                                             \
     do {                                                                                               \
@@ -474,55 +481,68 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
             __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);                                        \
         }                                                                                              \
     } while (0)
-    // prologue: the state a step expects on entry — the first sub-step's activation and weight fragments in
-    // registers, the step's raw rows unpacked, the copies for the next step and the weights two steps on under way
-    copy_w(0u);
-    copy_w(1u);
+// Step T = 4 s + C of super-block s, entered with the fragments of its first sub-step in afA / b0 / b1 and its raw rows
+// unpacked in r0 / r1.  Sub-steps 0..2 build the next sub-step's B fragments under their MFMAs.  Then the copies are
+// awaited (stage (T + 1) & 1 must be whole, and everyone done with stage T & 1 before it is overwritten) and the next
+// requests go out: activations two steps ahead, nibbles three, the next super-block's header from its second step
+// (one header copy per super-block, not per step: a copy instruction walks 32 rows' cache lines whatever it moves).
+// Copies complete in order, so the wait names how many younger ones may still be on their way.  Sub-step 3, its
+// fragments already in registers, covers the next step's first activation fragments and raw rows.  The chunk index
+// C is a compile-time constant of each of the four unrolled steps, which is what makes the scale unpacking cheap.
+#define GB_STEP(C, T)                                                                                  \
+    do {                                                                                               \
+        __builtin_amdgcn_sched_barrier(0);                                                             \
+        GB_READ_A(T, 1u, afB); GB_MMA(afA, b0, b1);                                                    \
+        c0 = r0.frag<1>(magic); c1 = r1.frag<1>(magic);                                                \
+        GB_MIX(4);                                                                                     \
+        GB_READ_A(T, 4u, afA); GB_MMA(afB, c0, c1);                                                    \
+        b0 = r0.frag<2>(magic); b1 = r1.frag<2>(magic);                                                \
+        GB_MIX(5);                                                                                     \
+        GB_READ_A(T, 5u, afB); GB_MMA(afA, b0, b1);                                                    \
+        c0 = r0.frag<3>(magic); c1 = r1.frag<3>(magic);                                                \
+        GB_MIX(5);                                                                                     \
+        __builtin_amdgcn_sched_barrier(0);                                                             \
+        gx_wait<(C) == 2 ? 4 : 2>();                                                                   \
+        __syncthreads();                                                                               \
+        copy_x((T) + 2u);                                                                              \
+        copy_nib((T) + 3u);                                                                            \
+        if ((C) == 1) copy_hdr((T) + 3u);                                                              \
+        __builtin_amdgcn_sched_barrier(0);                                                             \
+        GB_READ_A((T) + 1u, 0u, afA);                                                                  \
+        GB_READ_W((T) + 1u, ((C) + 1) & 3, (C) == 3);                                                  \
+        GB_MMA(afB, c0, c1);                                                                           \
+        b0 = r0.frag<0>(magic); b1 = r1.frag<0>(magic);                                                \
+        _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {                                             \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                         \
+            if (g_ < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                             \
+            __builtin_amdgcn_sched_group_barrier(0x002, 11, 0);                                        \
+        }                                                                                              \
+    } while (0)
+    // prologue: the state a step expects on entry
+    copy_nib(0u);
+    copy_hdr(0u);
+    copy_nib(1u);
     copy_x(0u);
-    if (XS == 3) copy_x(1u);
     gx_wait<0>();
     __syncthreads();
     GB_READ_A(0u, 0u, afA);
-    GB_READ_W(0u);
+    GB_READ_W(0u, 0, true);
     b0 = r0.frag<0>(magic);
     b1 = r1.frag<0>(magic);
-    copy_x(XS == 2 ? 1u : 2u);
-    copy_w(2u);
-    for (uint t = 0; t < nt; t++) {
-        __builtin_amdgcn_sched_barrier(0);
-        GB_READ_A(t, 1u, afB); GB_MMA(afA, b0, b1);
-        c0 = r0.frag<1>(magic); c1 = r1.frag<1>(magic);
-        GB_MIX(4);
-        GB_READ_A(t, 4u, afA); GB_MMA(afB, c0, c1);
-        b0 = r0.frag<2>(magic); b1 = r1.frag<2>(magic);
-        GB_MIX(5);
-        GB_READ_A(t, 5u, afB); GB_MMA(afA, b0, b1);
-        c0 = r0.frag<3>(magic); c1 = r1.frag<3>(magic);
-        GB_MIX(5);
-        __builtin_amdgcn_sched_barrier(0);
-        // x(t + 1) has landed, and with it everything older (the weights of t + 1 among them); only what was issued
-        // behind it (four weight copies; with three stages the whole batch of the step before) may still be on its
-        // way.  Past the barrier nobody reads the stage of step t any more.
-        gx_wait<XS == 2 ? 4 : 8>();
-        __syncthreads();
-        copy_x(t + (uint)XS);
-        copy_w(t + 3u);
-        __builtin_amdgcn_sched_barrier(0);
-        GB_READ_A(t + 1u, 0u, afA);
-        GB_READ_W(t + 1u);
-        GB_MMA(afB, c0, c1);
-        b0 = r0.frag<0>(magic); b1 = r1.frag<0>(magic);
-        _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (g_ < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 11, 0);
-        }
+    copy_x(1u);
+    copy_nib(2u);
+    for (uint t = 0; t < nt; t += 4u) {
+        GB_STEP(0, t);
+        GB_STEP(1, t + 1u);
+        GB_STEP(2, t + 2u);
+        GB_STEP(3, t + 3u);
     }
     gx_wait<0>();
 #undef GB_READ_A
 #undef GB_READ_W
 #undef GB_MMA
 #undef GB_MIX
+#undef GB_STEP
 
     // epilogue: D register v of block (i, j) holds token row 32 i + 8 (v / 4) + 4 kg + v % 4, output 64 wave + 32 j + fr
 #pragma unroll
@@ -544,19 +564,20 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
     }
 }
 
-// (A variant with three activation stages, copies two steps ahead, 96 KB and one workgroup per CU, measured the same at
-// 224 workgroups and is not built: the activation copies are not what a step waits for.)
+// (Variants with three activation stages, or four and a barrier every other step, were built and measured: 96 / 112 KB,
+// one workgroup per CU, slower at 224 workgroups — the activation copies are not what a step waits for.)
 extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemm_mm_q4kl_bd(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
-    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(2)];
-    if (accum) gemm_bd_body<false, true, 2>(xh, w, y, K, N, M, 1u, lds);
-    else gemm_bd_body<false, false, 2>(xh, w, y, K, N, M, 1u, lds);
+    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS];
+    if (accum) gemm_bd_body<false, true>(xh, w, y, K, N, M, 1u, lds);
+    else gemm_bd_body<false, false>(xh, w, y, K, N, M, 1u, lds);
 }
 extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemm_mm_q4kl_bd_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
-    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(2)];
-    gemm_bd_body<true, true, 2>(xh, w, y, K, N, M, nsplit, lds);
+    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS];
+    gemm_bd_body<true, true>(xh, w, y, K, N, M, nsplit, lds);
 }
+
 // LDS of a tile: two activation stages, two dequantized-weight stages, two raw-weight slots
 #define GX_LDS(MI) __shared__ __attribute__((aligned(1024))) uchar lds[2 * 64 * (MI) * GX_ROW + 2 * GX_WSTAGE + 2 * GX_RAW]
 
