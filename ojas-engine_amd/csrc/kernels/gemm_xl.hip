@@ -341,11 +341,11 @@ __device__ __forceinline__ void gemm_xl_body(const ushort* __restrict__ xh, cons
 // (three K steps ahead for the nibbles, a header slot per super-block), so nothing asynchronous targets a register
 // and no barrier guards them; the one barrier per step is for the activation stage.  80 KB of LDS and at most 128
 // vector registers beside the accumulators: two workgroups per CU, one's dequantization under the other's MFMAs.
-#define GB_BM 128u
-#define GB_XSTAGE (GB_BM * GX_ROW)        // 16 KB
-#define GB_NIB (2u * GB_XSTAGE)            // 4 slots x 4 waves x 2 rows x 1 KB
-#define GB_HDR (GB_NIB + 32768u)           // 2 slots x 4 waves x 2 rows x 1 KB
-#define GB_LDS (GB_HDR + 16384u)
+// MI = 32-token blocks per tile: 4 (128 tokens) or 8 (256 tokens: all 256 accumulators, one workgroup per CU).
+#define GB_XSTAGE(MI) (32u * (MI) * GX_ROW)        // 16 / 32 KB
+#define GB_NIB(MI) (2u * GB_XSTAGE(MI))            // 4 slots x 4 waves x 2 rows x 1 KB
+#define GB_HDR(MI) (GB_NIB(MI) + 32768u)           // 2 slots x 4 waves x 2 rows x 1 KB
+#define GB_LDS(MI) (GB_HDR(MI) + 16384u)
 
 struct GbRow {
     u32x4 hdr, q;
@@ -377,12 +377,12 @@ struct GbRow {
     }
 };
 
-template <bool SPLITK, bool ACCUM>
+template <bool SPLITK, bool ACCUM, int MI>
 __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, const uchar* __restrict__ w,
                                              float* __restrict__ y, uint K, uint N, uint M, uint nsplit, uchar* lds) {
     const uint tid = threadIdx.x, lane = tid & 63u;
     const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint n0 = blockIdx.x * GX_BN, m0 = blockIdx.y * GB_BM;
+    const uint n0 = blockIdx.x * GX_BN, m0 = blockIdx.y * (32u * MI);
     const uint nsb = K >> 8;
     uint sb_begin = 0, sb_end = nsb;
     if (SPLITK) {
@@ -395,29 +395,29 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
     const uint k_begin = sb_begin << 8;
     const uint lds0 = (uint)(size_t)(__attribute__((address_space(3))) uchar*)lds;
 
-    // activation stage: wave `wave`, copy i moves rows (wave*4 + i)*8 .. +7; lane -> row lane/8, slot lane%8, which
+    // activation stage: wave `wave`, copy i moves rows (wave*MI + i)*8 .. +7; lane -> row lane/8, slot lane%8, which
     // holds source chunk (lane%8) ^ ((row/2)%8)
-    uint xoff[4];
+    uint xoff[MI];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint r = (wave * 4u + i) * 8u + (lane >> 3);
+    for (int i = 0; i < MI; i++) {
+        const uint r = (wave * (uint)MI + i) * 8u + (lane >> 3);
         const uint m = min(m0 + r, M - 1u);
         xoff[i] = m * K * 2u + (((lane & 7u) ^ ((r >> 1) & 7u)) << 4);
     }
-    const uint x_lds = lds0 + wave * 4096u;                      // + stage * GB_XSTAGE + i * 1024
+    const uint x_lds = lds0 + wave * ((uint)MI * 1024u);         // + stage * GB_XSTAGE + i * 1024
     // the lane's two weight rows: B column fr of blocks j = 0, 1; its 16 nibble bytes are bytes 16 g .. of a chunk
     const uint fr = lane & 31u, kg = lane >> 5, sw = (fr >> 1) & 7u;
     const uint row_bytes = nsb * Q4K_BYTES;
     const uint ro0 = min(n0 + wave * 64u + fr, N - 1u) * row_bytes, ro1 = min(n0 + wave * 64u + 32u + fr, N - 1u) * row_bytes;
-    const uint nib_lds = lds0 + GB_NIB + wave * 2048u;           // + slot * 8192 + j * 1024
-    const uint hdr_lds = lds0 + GB_HDR + wave * 2048u;           // + slot * 8192 + j * 1024
-    const uchar* const nib_rd = lds + GB_NIB + wave * 2048u + lane * 16u;
-    const uchar* const hdr_rd = lds + GB_HDR + wave * 2048u + lane * 16u;
+    const uint nib_lds = lds0 + GB_NIB(MI) + wave * 2048u;           // + slot * 8192 + j * 1024
+    const uint hdr_lds = lds0 + GB_HDR(MI) + wave * 2048u;           // + slot * 8192 + j * 1024
+    const uchar* const nib_rd = lds + GB_NIB(MI) + wave * 2048u + lane * 16u;
+    const uchar* const hdr_rd = lds + GB_HDR(MI) + wave * 2048u + lane * 16u;
     const uchar* const a_rd = lds + fr * GX_ROW;                 // + stage * GB_XSTAGE + i * 32 rows + chunk slot
 
-    float16v acc[4][2];
+    float16v acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -430,7 +430,7 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
     auto copy_x = [&](uint t) {
         const uchar* b = xbase + (size_t)(k_begin + min(t, last) * GX_BK) * 2u;
 #pragma unroll
-        for (int i = 0; i < 4; i++) gx_load_lds16(b, xoff[i], x_lds + (t & 1u) * GB_XSTAGE + i * 1024u);
+        for (int i = 0; i < MI; i++) gx_load_lds16(b, xoff[i], x_lds + (t & 1u) * GB_XSTAGE(MI) + i * 1024u);
     };
     auto copy_nib = [&](uint t) {
         const uint tc = min(t, last);
@@ -445,11 +445,11 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
         gx_load_lds16(bh, ro1, hdr_lds + ((tc >> 2) & 1u) * 8192u + 1024u);
     };
     GbRow r0, r1;
-    half8 afA[4], afB[4], b0, b1, c0, c1;
+    half8 afA[MI], afB[MI], b0, b1, c0, c1;
 #define GB_READ_A(T, CH, AF)                                                                           \
     do {                                                                                               \
-        const uchar* xa_ = a_rd + ((T) & 1u) * GB_XSTAGE + ((((CH) + 2u * kg) ^ sw) << 4);             \
-        _Pragma("unroll") for (int i = 0; i < 4; i++) AF[i] = *(const half8*)(xa_ + i * 32u * GX_ROW); \
+        const uchar* xa_ = a_rd + ((T) & 1u) * GB_XSTAGE(MI) + ((((CH) + 2u * kg) ^ sw) << 4);         \
+        _Pragma("unroll") for (int i = 0; i < MI; i++) AF[i] = *(const half8*)(xa_ + i * 32u * GX_ROW); \
     } while (0)
 // the raw rows of step T out of their slots (the header only where T starts a super-block), scales of chunk C1
 #define GB_READ_W(T, C1, HDR)                                                                          \
@@ -467,18 +467,19 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
     } while (0)
 #define GB_MMA(AF, B0, B1)                                                                             \
     do {                                                                                               \
-        _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                \
+        _Pragma("unroll") for (int i = 0; i < MI; i++) {                                               \
             acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(AF[i], B0, acc[i][0], 0, 0, 0);         \
             acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(AF[i], B1, acc[i][1], 0, 0, 0);         \
         }                                                                                              \
     } while (0)
-// eight MFMAs with the next fragments' LDS reads behind the first two and NV vector instructions behind each
+// a sub-step's 2 MI MFMAs with the next fragments' LDS reads behind the first ones and NV vector instructions
+// (NV / 2 when the sub-step has sixteen MFMAs to spread them over) behind each
 #define GB_MIX(NV)                                                                                     \
     do {                                                                                               \
-        _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {                                             \
+        _Pragma("unroll") for (int g_ = 0; g_ < 2 * MI; g_++) {                                        \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                         \
-            if (g_ < 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                             \
-            __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);                                        \
+            if (g_ < MI / 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                        \
+            __builtin_amdgcn_sched_group_barrier(0x002, MI == 4 ? (NV) : ((NV) + 1) / 2, 0);           \
         }                                                                                              \
     } while (0)
 // Step T = 4 s + C of super-block s, entered with the fragments of its first sub-step in afA / b0 / b1 and its raw rows
@@ -512,10 +513,10 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
         GB_READ_W((T) + 1u, ((C) + 1) & 3, (C) == 3);                                                  \
         GB_MMA(afB, c0, c1);                                                                           \
         b0 = r0.frag<0>(magic); b1 = r1.frag<0>(magic);                                                \
-        _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {                                             \
+        _Pragma("unroll") for (int g_ = 0; g_ < 2 * MI; g_++) {                                        \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                         \
-            if (g_ < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                             \
-            __builtin_amdgcn_sched_group_barrier(0x002, 11, 0);                                        \
+            if (g_ < MI / 2 + 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                    \
+            __builtin_amdgcn_sched_group_barrier(0x002, MI == 4 ? 11 : 6, 0);                          \
         }                                                                                              \
     } while (0)
     // prologue: the state a step expects on entry
@@ -546,7 +547,7 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
 
     // epilogue: D register v of block (i, j) holds token row 32 i + 8 (v / 4) + 4 kg + v % 4, output 64 wave + 32 j + fr
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < MI; i++) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const uint n = n0 + wave * 64u + 32u * j + fr;
@@ -568,14 +569,26 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
 // one workgroup per CU, slower at 224 workgroups — the activation copies are not what a step waits for.)
 extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemm_mm_q4kl_bd(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
-    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS];
-    if (accum) gemm_bd_body<false, true>(xh, w, y, K, N, M, 1u, lds);
-    else gemm_bd_body<false, false>(xh, w, y, K, N, M, 1u, lds);
+    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(4)];
+    if (accum) gemm_bd_body<false, true, 4>(xh, w, y, K, N, M, 1u, lds);
+    else gemm_bd_body<false, false, 4>(xh, w, y, K, N, M, 1u, lds);
 }
 extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemm_mm_q4kl_bd_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
-    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS];
-    gemm_bd_body<true, true>(xh, w, y, K, N, M, nsplit, lds);
+    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(4)];
+    gemm_bd_body<true, true, 4>(xh, w, y, K, N, M, nsplit, lds);
+}
+// 256 tokens per tile: the wave's 64 rows are dequantized once for twice the MFMAs
+extern "C" __global__ void __launch_bounds__(256)
+gemm_mm_q4kl_bd256(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
+    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(8)];
+    if (accum) gemm_bd_body<false, true, 8>(xh, w, y, K, N, M, 1u, lds);
+    else gemm_bd_body<false, false, 8>(xh, w, y, K, N, M, 1u, lds);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemm_mm_q4kl_bd256_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
+    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(8)];
+    gemm_bd_body<true, true, 8>(xh, w, y, K, N, M, nsplit, lds);
 }
 
 // LDS of a tile: two activation stages, two dequantized-weight stages, two raw-weight slots

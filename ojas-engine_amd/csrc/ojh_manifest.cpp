@@ -1384,6 +1384,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("gemm_mm_q4kl_m128_sk", "gemm_xl", 3, 4, OJH_Q4_K, 5, check_gemm, shape_gemm);
     add("gemm_mm_q4kl_bd", "gemm_xl", 3, 4, OJH_Q4_K, 6, check_gemm, shape_gemm);      // 128 x 256, weights dequantized into B registers
     add("gemm_mm_q4kl_bd_sk", "gemm_xl", 3, 4, OJH_Q4_K, 7, check_gemm, shape_gemm);
+    add("gemm_mm_q4kl_bd256", "gemm_xl", 3, 4, OJH_Q4_K, 2, check_gemm, shape_gemm);   // ... 256 x 256
+    add("gemm_mm_q4kl_bd256_sk", "gemm_xl", 3, 4, OJH_Q4_K, 3, check_gemm, shape_gemm);
     // MoE: `rows_per_wave` selects the kernel inside check_moe / shape_moe
     add("moe_topk", "moe", 3, 2, 0, 0, check_moe, shape_moe);
     add("moe_topk_nonorm", "moe", 3, 2, 0, 18, check_moe, shape_moe);

@@ -514,6 +514,11 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         uint32_t sg[3], sb[3];
         if ((rc = ojh_launch_shape(dev, (base + "_sk").c_str(), K, N, m, sg, sb))) return rc;
         if (dev->gemm_split_override > 0) sg[2] = (uint32_t)dev->gemm_split_override;
+        // 256-token tiles that fill the chip: the form that dequantizes into the B registers (same grid).  Its step
+        // time does not grow with the number of busy CUs as the LDS-shared tile's does (measured: 2.2 us per K step
+        // at 224 and at 448 workgroups against 2.0 and 2.4).
+        if (xl && base == "gemm_mm_q4kl" && (uint64_t)sg[0] * sg[1] * sg[2] >= (uint32_t)dev->prop.multiProcessorCount)
+            base = "gemm_mm_q4kl_bd256";
         if (sg[2] > 1) {
             if (!accum) {
                 uint32_t n_y = m * N, zg[3] = {(n_y / 4 + 255) / 256 + 1, 1, 1};

@@ -105,7 +105,8 @@ def test_tile_holds_the_reference_decoders_bits(gpu, orc, pkg, ty):
 @pytest.mark.parametrize("kernel,family,bm,bn,wmode", [("gemm_mm_q4k_sk", "gemm", 256, 128, 1),
                                                        ("gemm_mm_q4kl_sk", "gemm_xl", 256, 256, 2),
                                                        ("gemm_mm_q4kl_m128_sk", "gemm_xl", 128, 256, 2),
-                                                       ("gemm_mm_q4kl_bd_sk", "gemm_xl", 128, 256, 2)])
+                                                       ("gemm_mm_q4kl_bd_sk", "gemm_xl", 128, 256, 2),
+                                                       ("gemm_mm_q4kl_bd256_sk", "gemm_xl", 256, 256, 2)])
 def test_split_k_entry_through_the_kernel_seam(gpu, orc, pkg, kernel, family, bm, bn, wmode):
     """Split-K entries dispatched by name with several K slices; y holds what is accumulated into."""
     gpu.ensure_family(family)
@@ -131,7 +132,8 @@ def test_split_k_entry_through_the_kernel_seam(gpu, orc, pkg, kernel, family, bm
 
 @pytest.mark.parametrize("m,k,n", [(140, 2048, 300), (128, 256, 256), (77, 512, 64), (260, 1024, 513)])
 def test_tile_with_weights_dequantized_into_registers(gpu, orc, pkg, m, k, n):
-    """`gemm_mm_q4kl_bd` by name: the 128 x 256 tile whose waves dequantize their own 64 rows into the B operand.  Ragged
+    """`gemm_mm_q4kl_bd` and `gemm_mm_q4kl_bd256` by name: the 128 x 256 and 256 x 256 tiles whose waves dequantize their own
+    64 rows into the B operand.  Ragged
     M and N, store and accumulate, sentinels behind row M; the oracle holds the tile's specified f16 weights, and the
     tile that shares the dequantized weights through LDS agrees to the order of the f32 sums inside a K step."""
     gpu.ensure_family("gemm_xl")
@@ -139,10 +141,10 @@ def test_tile_with_weights_dequantized_into_registers(gpu, orc, pkg, m, k, n):
     x = pkg.synth.normal_f32(m * k, "bd", "x", m, k).reshape(m, k)
     xh, wd = gpu.upload_bytes(x.astype(np.float16)), gpu.upload_bytes(w)
     want = orc.matmul_ref(w, Q4_K, n, k, x, wmode=2, xmode=1)
-    grid = [(n + 255) // 256, (m + 127) // 128, 1]
     sent = np.full(n, 12345.5, np.float32)
     outs = {}
-    for kernel in ("gemm_mm_q4kl_bd", "gemm_mm_q4kl_m128"):
+    for kernel, bm in (("gemm_mm_q4kl_bd", 128), ("gemm_mm_q4kl_bd256", 256), ("gemm_mm_q4kl_m128", 128)):
+        grid = [(n + 255) // 256, (m + bm - 1) // bm, 1]
         for accum in (0, 1):
             y0 = pkg.synth.normal_f32(m * n, "bd", "y0", accum).reshape(m, n)
             yd = gpu.upload(np.concatenate([y0.ravel(), sent]))
@@ -154,6 +156,7 @@ def test_tile_with_weights_dequantized_into_registers(gpu, orc, pkg, m, k, n):
             assert e[0] < 1e-4 and e[1] < 2e-5, (kernel, accum, e)
             outs[kernel, accum] = got
     assert peak_err(outs["gemm_mm_q4kl_bd", 0], outs["gemm_mm_q4kl_m128", 0]) <= 2e-6
+    assert np.array_equal(outs["gemm_mm_q4kl_bd256", 0], outs["gemm_mm_q4kl_bd", 0])      # the same sums in the same order
 
 
 def test_q4l_entries_by_their_reference_names(gpu, orc, pkg):
