@@ -15,8 +15,12 @@ import numpy as np
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 Q2_K, Q3_K = 10, 11
+IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M = 16, 17, 18, 19, 21, 22, 29
+GRID_TYPES = (IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M)
 BLOCK_SHAPE = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256), IQ4_NL: (18, 32), IQ4_XS: (136, 256),
-               Q4_0: (18, 32), Q4_1: (20, 32), Q5_0: (22, 32), Q5_1: (24, 32), Q2_K: (84, 256), Q3_K: (110, 256)}
+               Q4_0: (18, 32), Q4_1: (20, 32), Q5_0: (22, 32), Q5_1: (24, 32), Q2_K: (84, 256), Q3_K: (110, 256),
+               IQ2_XXS: (66, 256), IQ2_XS: (74, 256), IQ3_XXS: (98, 256), IQ1_S: (50, 256), IQ3_S: (110, 256), IQ2_S: (82, 256),
+               IQ1_M: (56, 256)}
 
 
 def seed_of(*names) -> int:
@@ -187,8 +191,28 @@ def weights(ty: int, n: int, k: int, *names) -> np.ndarray:
         return legacy_weights(ty, n, k, *names)
     if ty in (Q2_K, Q3_K):
         return {Q2_K: q2k_weights, Q3_K: q3k_weights}[ty](n, k, *names)
+    if ty in GRID_TYPES:
+        return grid_weights(ty, n, k, *names)
     return {Q8_0: q80_weights, Q4_K: q4k_weights, Q5_K: q5k_weights, Q6_K: q6k_weights,
             IQ4_NL: iq4nl_weights, IQ4_XS: iq4xs_weights}[ty](n, k, *names)
+
+
+def grid_weights(ty: int, n: int, k: int, *names) -> np.ndarray:
+    """Rows of a grid-codebook format: every byte uniform (each bit pattern is a legal block: indices are masked into
+    their tables), the block scale d = f16(|N(0, 0.01)| / 16 + 1e-4); IQ1_M spreads its d over the top nibbles of its
+    four scale words."""
+    bb, _ = BLOCK_SHAPE[ty]
+    nb = n * k // 256
+    g = rng("grid", ty, n, k, *names)
+    blocks = g.integers(0, 256, (nb, bb), dtype=np.uint8)
+    d = (np.abs(g.normal(0.0, 0.01, nb)) / 16.0 + 1e-4).astype(np.float32).astype(np.float16).view(np.uint16)
+    if ty == IQ1_M:
+        for w in range(4):
+            blocks[:, 49 + 2 * w] = (blocks[:, 49 + 2 * w] & 0x0F) | ((((d >> (4 * w)) & 0xF) << 4).astype(np.uint8))
+    else:
+        blocks[:, 0] = (d & 0xFF).astype(np.uint8)
+        blocks[:, 1] = (d >> 8).astype(np.uint8)
+    return blocks.reshape(-1)
 
 
 # ------------------------------------------------------------------ the reference tests' procedures
@@ -218,6 +242,10 @@ def synth_blocks(ty: int, nb: int) -> np.ndarray:
             blocks[i, 82], blocks[i, 83] = int(dmin) & 0xFF, int(dmin) >> 8
         elif ty == Q3_K:
             blocks[i, 108], blocks[i, 109] = d & 0xFF, d >> 8
+        elif ty == IQ1_M:      # no d field: f16(0.05) in the top nibbles of the four scale words, low nibble first
+            db = int(np.array([0.05], np.float32).astype(np.float16).view(np.uint16)[0])
+            for w in range(4):
+                blocks[i, 49 + 2 * w] = (int(blocks[i, 49 + 2 * w]) & 0x0F) | (((db >> (4 * w)) & 0xF) << 4)
         else:
             blocks[i, 0], blocks[i, 1] = d & 0xFF, d >> 8
     return out

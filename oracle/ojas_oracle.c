@@ -108,6 +108,13 @@ int ojo_block_shape(uint32_t ty, uint32_t *bytes, uint32_t *weights) { /* synth.
     case OJO_Q5_0: b = 22; w = 32; break;
     case OJO_Q5_1: b = 24; w = 32; break;
     case OJO_IQ4_XS: b = 136; w = 256; break;
+    case OJO_IQ2_XXS: b = 66; w = 256; break;
+    case OJO_IQ2_XS: b = 74; w = 256; break;
+    case OJO_IQ3_XXS: b = 98; w = 256; break;
+    case OJO_IQ1_S: b = 50; w = 256; break;
+    case OJO_IQ3_S: b = 110; w = 256; break;
+    case OJO_IQ2_S: b = 82; w = 256; break;
+    case OJO_IQ1_M: b = 56; w = 256; break;
     default: return 0;
     }
     if (bytes) *bytes = b;
@@ -142,6 +149,14 @@ int ojo_synth_blocks(uint32_t ty, size_t nb, uint8_t *out) { /* synth.rs:29-64 *
         case OJO_Q3_K:
             blk[108] = (uint8_t)d; blk[109] = (uint8_t)(d >> 8);
             break;
+        case OJO_IQ1_M: { /* no d field: f16(0.05) spread over the top nibbles of the four scale words, low nibble first */
+            uint16_t db = ojo_f32_to_f16(0.05f);
+            for (int w = 0; w < 4; w++) {
+                uint16_t cur = (uint16_t)(blk[48 + 2 * w] | (blk[49 + 2 * w] << 8));
+                uint16_t v = (uint16_t)((cur & 0x0FFF) | (((db >> (4 * w)) & 0xF) << 12));
+                blk[48 + 2 * w] = (uint8_t)v; blk[49 + 2 * w] = (uint8_t)(v >> 8);
+            }
+        } break;
         default:
             blk[0] = (uint8_t)d; blk[1] = (uint8_t)(d >> 8);
         }
@@ -178,6 +193,14 @@ int ojo_dequant_to_f16(const uint8_t *b, uint32_t ty, size_t n, uint16_t *out) {
     uint32_t bb, wpb;
     if (!ojo_block_shape(ty, &bb, &wpb) || n % wpb) return -1;
     size_t nblk = n / wpb;
+    if (ojo_iq_is_grid_type(ty)) { /* gguf.rs:840-1041 */
+        float w32[256];
+        for (size_t ib = 0; ib < nblk; ib++) {
+            ojo_iq_block(ty, b + ib * bb, w32, NULL);
+            for (int j = 0; j < 256; j++) out[ib * 256 + j] = ojo_f32_to_f16(w32[j]);
+        }
+        return 0;
+    }
     for (size_t ib = 0; ib < nblk; ib++) {
         const uint8_t *blk = b + ib * bb;
         uint16_t *o = out + ib * wpb;
@@ -339,6 +362,10 @@ int ojo_dequant_to_f64(const uint8_t *b, uint32_t ty, size_t n, double *out) {
     uint32_t bb, wpb;
     if (!ojo_block_shape(ty, &bb, &wpb) || n % wpb) return -1;
     size_t nblk = n / wpb;
+    if (ojo_iq_is_grid_type(ty)) {
+        for (size_t ib = 0; ib < nblk; ib++) ojo_iq_block(ty, b + ib * bb, NULL, out + ib * 256);
+        return 0;
+    }
     for (size_t ib = 0; ib < nblk; ib++) {
         const uint8_t *blk = b + ib * bb;
         double *o = out + ib * wpb;
@@ -747,6 +774,9 @@ static void kq_row(void *p, size_t row) {
     case OJO_Q8_0: v = ojo_dot_q80(rb, c->x, c->k); break;
     case OJO_IQ4_NL: v = ojo_dot_iq4nl(rb, c->x, c->k); break;   /* dot_iq, cpu_math.rs:1131-1141: f32 activations */
     case OJO_IQ4_XS: v = ojo_dot_iq4xs(rb, c->x, c->k); break;
+    case OJO_IQ2_XXS: v = ojo_dot_iq2xxs_q8k(rb, c->k, c->scales, c->q); break;
+    case OJO_IQ3_XXS: v = ojo_dot_iq3xxs_q8k(rb, c->k, c->scales, c->q); break;
+    case OJO_IQ3_S: case OJO_IQ2_S: v = ojo_dot_iq_grid(c->ty, rb, c->x, c->k); break;
     default:       v = ojo_dot_q6k(rb, c->k, c->scales, c->q, c->bsums);
     }
     c->y[row] = v;
@@ -762,6 +792,10 @@ int ojo_matvec_kq(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const flo
     case OJO_Q8_0: per256 = 272; break;
     case OJO_IQ4_NL: per256 = 144; break;
     case OJO_IQ4_XS: per256 = 136; break;
+    case OJO_IQ2_XXS: per256 = 66; break;
+    case OJO_IQ3_XXS: per256 = 98; break;
+    case OJO_IQ3_S: per256 = 110; break;
+    case OJO_IQ2_S: per256 = 82; break;
     default: return -1;
     }
     size_t nsb = (k + 255) / 256;

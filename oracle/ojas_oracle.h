@@ -18,7 +18,12 @@
  *                           the reference's tests hold no digest for the legacy 32-weight blocks
  *   f16 <-> f32             the digests above + exhaustive comparison with IEEE binary16 (numpy)
  *   quant_q8k               invariants (max|q|=127, bsums, half-away rounding, |x-s*q|<=s/2)
+ *   dequant IQ2_XXS/IQ2_XS/IQ2_S/IQ3_XXS/IQ3_S/IQ1_S/IQ1_M   (ojas_oracle_iq.c) the digests of the same table
+ *                           (quant_formats.rs:41-44,46-47,49), closed forms on hand-built blocks; the packed codebooks
+ *                           by a digest of every published table (tests/golden/iq_grid_digests.json)
  *   dot_q80                 f64 dot over the dequantized row, brute force at K=32
+ *   dot_iq2xxs/iq3xxs/iq2s/iq3s   f64 dot over the exactly decoded row, one-hot activations
+ *   dot_iq2xxs_q8k/iq3xxs_q8k     identity dot(row, quant(x)) == sum xs * sum w * q in f64
  *   dot_iq4nl / dot_iq4xs   f64 dot over the dequantized row (the check of cpu_math.rs:1206-1285), one-hot activations
  *   dot_q4k/q5k/q6k         identity dot(row, quant(x)) == sum dequant(row)*(scale*q) in f64,
  *                           one-hot activations (pins nibble / sub-block order)
@@ -39,7 +44,8 @@ extern "C" {
 
 /* GGUF type ids (crates/ojas-formats/src/gguf.rs:563-591). */
 enum { OJO_Q4_0 = 2, OJO_Q4_1 = 3, OJO_Q5_0 = 6, OJO_Q5_1 = 7, OJO_Q8_0 = 8, OJO_Q2_K = 10, OJO_Q3_K = 11, OJO_Q4_K = 12, OJO_Q5_K = 13, OJO_Q6_K = 14,
-       OJO_IQ4_NL = 20, OJO_IQ4_XS = 23 };
+       OJO_IQ4_NL = 20, OJO_IQ4_XS = 23,
+       OJO_IQ2_XXS = 16, OJO_IQ2_XS = 17, OJO_IQ3_XXS = 18, OJO_IQ1_S = 19, OJO_IQ3_S = 21, OJO_IQ2_S = 22, OJO_IQ1_M = 29 };
 
 /* IEEE binary16 <-> binary32, round-to-nearest-even, subnormals kept
  * (crate half 2.7.1; call sites gguf.rs:602-608). */
@@ -77,6 +83,20 @@ float ojo_dot_iq4xs(const uint8_t *row, const float *x, size_t k);
 float ojo_dot_q4k(const uint8_t *row, size_t k, const float *scales, const int8_t *q, const int32_t *bsums);
 float ojo_dot_q5k(const uint8_t *row, size_t k, const float *scales, const int8_t *q, const int32_t *bsums);
 float ojo_dot_q6k(const uint8_t *row, size_t k, const float *scales, const int8_t *q, const int32_t *bsums);
+
+/* Grid-codebook formats (ojas_oracle_iq.c): one 256-weight block as the f32 values the reference rounds to f16 and
+ * exactly in double; the f32-activation dots (cpu_math.rs:728-757, :884-913, :915-941, :1023-1052) and the
+ * int8-activation dots (:1057-1128); a published codebook expanded from its packed form. */
+int    ojo_iq_is_grid_type(uint32_t ty);
+void   ojo_iq_block(uint32_t ty, const uint8_t *blk, float *of, double *od);
+size_t ojo_iq_grid_bytes(int which, uint8_t *out);
+float  ojo_dot_iq2xxs(const uint8_t *row, const float *x, size_t k);
+float  ojo_dot_iq3xxs(const uint8_t *row, const float *x, size_t k);
+float  ojo_dot_iq2s(const uint8_t *row, const float *x, size_t k);
+float  ojo_dot_iq3s(const uint8_t *row, const float *x, size_t k);
+float  ojo_dot_iq_grid(uint32_t ty, const uint8_t *row, const float *x, size_t k);
+float  ojo_dot_iq2xxs_q8k(const uint8_t *row, size_t k, const float *scales, const int8_t *q);
+float  ojo_dot_iq3xxs_q8k(const uint8_t *row, size_t k, const float *scales, const int8_t *q);
 
 /* matvec_kq (cpu_math.rs:1145-1189): 8-row work stealing over `threads` workers. */
 int ojo_matvec_kq(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const float *x,

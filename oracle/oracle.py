@@ -16,6 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libojas_oracle.so")
 
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
+IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M = 16, 17, 18, 19, 21, 22, 29
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 Q2_K, Q3_K = 10, 11
 
@@ -56,6 +57,14 @@ def lib() -> C.CDLL:
             f = getattr(L, name)
             f.restype = C.c_float
             f.argtypes = [vp, vp, sz]
+        L.ojo_dot_iq_grid.restype = C.c_float
+        L.ojo_dot_iq_grid.argtypes = [u32, vp, vp, sz]
+        for name in ("ojo_dot_iq2xxs_q8k", "ojo_dot_iq3xxs_q8k"):
+            f = getattr(L, name)
+            f.restype = C.c_float
+            f.argtypes = [vp, sz, vp, vp]
+        L.ojo_iq_grid_bytes.restype = sz
+        L.ojo_iq_grid_bytes.argtypes = [i32, vp]
         for name in ("ojo_dot_q4k", "ojo_dot_q5k", "ojo_dot_q6k"):
             f = getattr(L, name)
             f.restype = C.c_float
@@ -153,11 +162,35 @@ def dot_q80(row: np.ndarray, x: np.ndarray) -> float:
 
 
 def dot_iq(ty: int, row: np.ndarray, x: np.ndarray) -> float:
-    """dot_iq4nl / dot_iq4xs: raw row against f32 activations."""
-    fn = {IQ4_NL: lib().ojo_dot_iq4nl, IQ4_XS: lib().ojo_dot_iq4xs}[ty]
+    """dot_iq4nl / dot_iq4xs / dot_iq2xxs / dot_iq3xxs / dot_iq2s / dot_iq3s: raw row against f32 activations."""
     row = np.ascontiguousarray(row, np.uint8)
     x = np.ascontiguousarray(x, np.float32)
+    if ty in (IQ2_XXS, IQ3_XXS, IQ3_S, IQ2_S):
+        return float(lib().ojo_dot_iq_grid(ty, _p(row), _p(x), x.size))
+    fn = {IQ4_NL: lib().ojo_dot_iq4nl, IQ4_XS: lib().ojo_dot_iq4xs}[ty]
     return float(fn(_p(row), _p(x), x.size))
+
+
+def dot_iq_q8k(ty: int, row: np.ndarray, k: int, act) -> float:
+    """dot_iq2xxs_q8k / dot_iq3xxs_q8k: raw row against quant_q8k activations."""
+    fn = {IQ2_XXS: lib().ojo_dot_iq2xxs_q8k, IQ3_XXS: lib().ojo_dot_iq3xxs_q8k}[ty]
+    row = np.ascontiguousarray(row, np.uint8)
+    s, q, _ = act
+    return float(fn(_p(row), k, _p(s), _p(q)))
+
+
+def matvec_iq_f32(raw: np.ndarray, ty: int, n: int, k: int, x: np.ndarray) -> np.ndarray:
+    """Rows of an IQ format against f32 activations (dot_iq, cpu_math.rs:1131-1141), row by row."""
+    rb = row_bytes(ty, k)
+    raw = np.ascontiguousarray(raw, np.uint8)
+    return np.array([dot_iq(ty, raw[r * rb:(r + 1) * rb], x) for r in range(n)], np.float32)
+
+
+def iq_grid_bytes(which: int) -> np.ndarray:
+    """A published codebook (0 iq2xxs, 1 iq2xs, 2 iq2s, 3 iq3xxs, 4 iq3s, 5 iq1s) expanded from its packed form."""
+    out = np.empty(lib().ojo_iq_grid_bytes(which, None), np.uint8)
+    lib().ojo_iq_grid_bytes(which, _p(out))
+    return out
 
 
 def dot_kq(ty: int, row: np.ndarray, k: int, act) -> float:

@@ -19,7 +19,11 @@ COUNTS = {int(ty): row["values"] for ty, row in _GOLDEN.items()}
 KVALUES_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float64)
 
 
-@pytest.mark.parametrize("ty", [Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS])
+IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M = 16, 17, 18, 19, 21, 22, 29
+GRID_TYPES = [IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M]
+
+
+@pytest.mark.parametrize("ty", [Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS] + GRID_TYPES)
 def test_dequant_digest_matches_reference(orc, pkg, ty):
     wpb = pkg.synth.BLOCK_SHAPE[ty][1]
     raw = orc.synth_blocks(ty, 40)
@@ -28,7 +32,7 @@ def test_dequant_digest_matches_reference(orc, pkg, ty):
     assert orc.digest_f16(bits) == DIGESTS[ty]
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K] + GRID_TYPES)
 def test_synth_blocks_two_implementations_agree(orc, pkg, ty):
     assert np.array_equal(orc.synth_blocks(ty, 9), pkg.synth.synth_blocks(ty, 9))
 
@@ -553,3 +557,157 @@ def test_rmsnorm_and_activations_closed_forms(orc):
     assert np.allclose(orc.ffn_act(g, 0), g64 / (1.0 + np.exp(-g64)), rtol=1e-6, atol=1e-12)
     gelu = 0.5 * g64 * (1.0 + np.tanh(0.7978845608028654 * g64 * (1.0 + 0.044715 * g64 * g64)))
     assert np.allclose(orc.ffn_act(g, 1), gelu, rtol=2e-6, atol=1e-7)
+
+
+# ------------------------------------------------------------------ grid-codebook formats
+def _fnv(data: bytes) -> int:
+    h = 0xCBF29CE484222325
+    for b in data:
+        h = ((h ^ b) * 0x100000001B3) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+def test_iq_codebooks_expand_to_the_published_tables(orc):
+    """The packed codebooks, expanded, hash to the digests taken from the published tables when the header was written
+    (tests/golden/iq_grid_digests.json), and hold the entries quoted here from crates/ojas-core/src/iq_tables.rs."""
+    with open(os.path.join(os.path.dirname(__file__), "golden", "iq_grid_digests.json")) as f:
+        want = json.load(f)["tables"]
+    known = {  # (table, entry) -> value, little-endian
+        (0, 1): 0x080808080808082B, (0, 2): 0x0808080808081919, (0, 131): 0x082B2B2B19081908, (0, 255): 0x2B2B2B1908081908,
+        (1, 259): 0x190808080819082B, (1, 511): 0x2B2B2B2B2B2B2B2B, (2, 515): 0x190808191908192B, (2, 1023): 0x2B2B2B2B2B2B2B2B,
+        (3, 0): 0x04040404, (3, 1): 0x04040414, (3, 131): 0x14242C1C, (3, 255): 0x3E341C04,
+        (4, 0): 0x01010101, (4, 2): 0x01010105, (4, 259): 0x05090903, (4, 511): 0x0F0F0101,
+        (5, 0): 0xFFFFFFFFFFFFFFFF, (5, 1): 0xFFFFFFFFFFFFFF01, (5, 2): 0xFFFFFFFFFFFF0000, (5, 1027): 0xFF01, (5, 2047): 0x0101010101010101,
+    }
+    for which, name in enumerate(["iq2xxs", "iq2xs", "iq2s", "iq3xxs", "iq3s", "iq1s"]):
+        raw = orc.iq_grid_bytes(which)
+        row = want[name]
+        assert raw.size == row["entries"] * row["entry_bytes"]
+        assert _fnv(raw.tobytes()) == int(row["fnv1a64"], 16), name
+        table = raw.reshape(row["entries"], row["entry_bytes"])
+        for (w, i), v in known.items():
+            if w == which:
+                assert int.from_bytes(table[i].tobytes(), "little") == v, (name, i)
+
+
+def _f16(v):
+    return np.array([v], np.float16).view(np.uint8)
+
+
+def test_grid_format_closed_forms(orc):
+    """Hand-built blocks: which bits are the grid index, the signs, the sub-block scale, the delta; all products exact."""
+    d = 0.5
+    # IQ2_XXS: group 3 of sub-block 5 -> entry 1 (43, 8 x 7); sign index 1 = 0b10000001 (even parity): weights 0 and 7 negative
+    blk = np.zeros(66, np.uint8)
+    blk[0:2] = _f16(d)
+    a1 = (9 << 28) | (1 << 21)
+    blk[2 + 8 * 5 + 3] = 1
+    blk[2 + 8 * 5 + 4:2 + 8 * 5 + 8] = np.frombuffer(int(a1).to_bytes(4, "little"), np.uint8)
+    w = orc.dequant_to_f64(blk, IQ2_XXS, 256).reshape(8, 4, 8)
+    db = d * 9.5 * 0.25
+    assert np.array_equal(w[5, 3], db * np.array([-43, 8, 8, 8, 8, 8, 8, -8.0]))
+    assert np.all(w[5, :3] == db * 8) and np.all(w[4] == d * 0.5 * 0.25 * 8)
+    # IQ2_XS: 9-bit index 259 (low byte 0x2b ... ) with sign index 2 -> bits 1 and 7; scale nibbles: low for groups 0-1, high for 2-3
+    blk = np.zeros(74, np.uint8)
+    blk[0:2] = _f16(d)
+    q = 259 | (2 << 9)
+    blk[2 + 2 * (4 * 6 + 2):2 + 2 * (4 * 6 + 2) + 2] = [q & 0xFF, q >> 8]
+    blk[66 + 6] = 0xA3
+    w = orc.dequant_to_f64(blk, IQ2_XS, 256).reshape(8, 4, 8)
+    e259 = np.array([0x2B, 0x08, 0x19, 0x08, 0x08, 0x08, 0x08, 0x19], np.float64)
+    sg = np.array([1, -1, 1, 1, 1, 1, 1, -1.0])
+    assert np.array_equal(w[6, 2], d * 10.5 * 0.25 * e259 * sg)
+    assert np.all(w[6, 0] == d * 3.5 * 0.25 * 8) and np.all(w[6, 3] == d * 10.5 * 0.25 * 8)
+    # IQ2_S: index = qs | (two bits of qh per group) << 8; raw sign byte
+    blk = np.zeros(82, np.uint8)
+    blk[0:2] = _f16(d)
+    blk[2 + 4 * 2 + 1] = 515 & 0xFF
+    blk[66 + 2] = (515 >> 8) << 2                     # group l = 1 reads qh bits 2..3
+    blk[2 + 32 + 4 * 2 + 1] = 0x05                    # weights 0 and 2 negative
+    blk[74 + 2] = 0x07                                # groups 0-1: (0.5 + 7) / 4
+    w = orc.dequant_to_f64(blk, IQ2_S, 256).reshape(8, 4, 8)
+    e515 = np.array([0x2B, 0x19, 0x08, 0x19, 0x19, 0x08, 0x08, 0x19], np.float64)
+    assert np.array_equal(w[2, 1], d * 7.5 * 0.25 * e515 * np.array([-1, 1, -1, 1, 1, 1, 1, 1.0]))
+    assert np.all(w[2, 2] == d * 0.5 * 0.25 * 8)
+    # IQ3_XXS: two 4-entry indices per group of 8, scale and signs in the trailing 32 bytes
+    blk = np.zeros(98, np.uint8)
+    blk[0:2] = _f16(d)
+    blk[2 + 8 * 1 + 2 * 2] = 131
+    blk[2 + 8 * 1 + 2 * 2 + 1] = 255
+    a = (4 << 28) | (1 << 14)                           # group 2: sign index 1 -> weights 0 and 7
+    blk[66 + 4:66 + 8] = np.frombuffer(int(a).to_bytes(4, "little"), np.uint8)
+    w = orc.dequant_to_f64(blk, IQ3_XXS, 256).reshape(8, 4, 8)
+    assert np.array_equal(w[1, 2], d * 4.5 * 0.5 * np.array([-0x1C, 0x2C, 0x24, 0x14, 0x04, 0x1C, 0x34, -0x3E], np.float64))
+    assert np.all(w[1, 0] == d * 4.5 * 0.5 * 4)
+    # IQ3_S: ninth index bit from qh, raw sign bytes, scale 1 + 2 s per 64 weights half by half
+    blk = np.zeros(110, np.uint8)
+    blk[0:2] = _f16(d)
+    blk[2 + 8 * 3 + 2 * 1] = 259 & 0xFF                # sub-block 3, group 1, first index = 259
+    blk[66 + 3] = 1 << 2                               # its ninth bit: (h << (8 - 2 l)) & 256 with l = 1
+    blk[2 + 8 * 3 + 2 * 1 + 1] = 2                     # second index = 2
+    blk[74 + 4 * 3 + 1] = 0x90                         # weights 4 and 7 negative
+    blk[106 + 1] = 0x60                                # sub-block 3 = high nibble of scales[1]
+    w = orc.dequant_to_f64(blk, IQ3_S, 256).reshape(8, 4, 8)
+    assert np.array_equal(w[3, 1], d * 13 * np.array([0x03, 0x09, 0x09, 0x05, -0x05, 0x01, 0x01, -0x01], np.float64))
+    assert np.all(w[2] == d * 1)
+    # IQ1_S: index = qs | 3 bits of qh << 8, scale 2 s + 1 from bits 12..14, bit 15 flips the delta
+    blk = np.zeros(50, np.uint8)
+    blk[0:2] = _f16(d)
+    blk[2 + 4 * 4 + 2] = 1027 & 0xFF
+    qh = (5 << 12) | 0x8000 | ((1027 >> 8) << 6)
+    blk[34 + 2 * 4:34 + 2 * 4 + 2] = [qh & 0xFF, qh >> 8]
+    w = orc.dequant_to_f64(blk, IQ1_S, 256).reshape(8, 4, 8)
+    assert np.array_equal(w[4, 2], d * 11 * (np.array([1, -1, 0, 0, 0, 0, 0, 0.0]) - 0.125))
+    assert np.all(w[4, 0] == d * 11 * (-1 - 0.125)) and np.all(w[3] == d * (-1 + 0.125))
+    # IQ1_M: d from the top nibbles of the four scale words; two 3-bit scales per sub-block; delta bits 3 and 7 of qh
+    blk = np.zeros(56, np.uint8)
+    dbits = int(np.array([d], np.float16).view(np.uint16)[0])
+    sc = [((dbits >> (4 * i)) & 0xF) << 12 for i in range(4)]
+    sc[1] |= (3 << 6) | (6 << 9)                        # sub-block 3 = second half of word 1: scales 3 and 6
+    for i in range(4):
+        blk[48 + 2 * i:50 + 2 * i] = [sc[i] & 0xFF, sc[i] >> 8]
+    blk[4 * 3 + 3] = 1027 & 0xFF                        # group 3: index 1027, high bits from qh[2 * 3 + 1] bits 4..6
+    blk[32 + 2 * 3 + 1] = ((1027 >> 8) << 4) | 0x80     # and its delta negative
+    w = orc.dequant_to_f64(blk, IQ1_M, 256).reshape(8, 4, 8)
+    assert np.array_equal(w[3, 3], d * 13 * (np.array([1, -1, 0, 0, 0, 0, 0, 0.0]) - 0.125))
+    assert np.all(w[3, 0] == d * 7 * (-1 + 0.125)) and np.all(w[3, 2] == d * 13 * (-1 + 0.125))
+    assert np.all(w[0] == d * 1 * (-1 + 0.125))
+
+
+@pytest.mark.parametrize("ty", GRID_TYPES)
+def test_grid_format_f16_is_the_rounded_exact_value(orc, ty):
+    """dequant_to_f16 of random blocks == the exact products (double) rounded once: every factor chain of these formats
+    (an f16 d, small odd or half-integer scales, magnitudes below 64) is exact in f32."""
+    raw = orc.synth_blocks(ty, 12)
+    exact = orc.dequant_to_f64(raw, ty, 12 * 256)
+    assert np.array_equal(orc.dequant_to_f16(raw, ty, 12 * 256), exact.astype(np.float16).view(np.uint16))
+
+
+@pytest.mark.parametrize("ty", [IQ2_XXS, IQ3_XXS, IQ3_S, IQ2_S])
+def test_grid_format_f32_dots(orc, pkg, ty):
+    """dot_iq2xxs / dot_iq3xxs / dot_iq2s / dot_iq3s against the exactly decoded row in double, one-hot activations
+    (element order), and matvec_kq's routing: f32 activations for IQ3_S / IQ2_S, quant_q8k for the two XXS types."""
+    n, k = 5, 1024
+    rb = k // 256 * pkg.synth.BLOCK_SHAPE[ty][0]
+    raw = orc.synth_blocks(ty, n * k // 256)
+    x = pkg.synth.normal_f32(k, "t", "xgrid", ty)
+    w = orc.dequant_to_f64(raw, ty, n * k).reshape(n, k)
+    want = w @ x.astype(np.float64)
+    got = np.array([orc.dot_iq(ty, raw[r * rb:(r + 1) * rb], x) for r in range(n)])
+    assert np.max(np.abs(got - want)) <= 2e-6 * np.max(np.abs(want))
+    for i in [0, 1, 7, 8, 31, 32, 100, 255, 256, 1023]:
+        e = np.zeros(k, np.float32)
+        e[i] = 1.0
+        assert orc.dot_iq(ty, raw[:rb], e) == np.float32(w[0, i]), (ty, i)
+    mv = orc.matvec_kq(raw, ty, n, k, x, threads=3)
+    if ty in (IQ3_S, IQ2_S):
+        assert np.array_equal(mv, got.astype(np.float32))
+    else:
+        act = orc.quant_q8k(x)
+        s, q, _ = act
+        ident = np.array([sum(float(s[b]) * (w[r, b * 256:(b + 1) * 256] @ q[b * 256:(b + 1) * 256].astype(np.float64))
+                              for b in range(k // 256)) for r in range(n)])
+        q8 = np.array([orc.dot_iq_q8k(ty, raw[r * rb:(r + 1) * rb], k, act) for r in range(n)])
+        assert np.max(np.abs(q8 - ident)) <= 2e-6 * np.max(np.abs(ident))
+        assert np.array_equal(mv, q8.astype(np.float32))
+        assert np.max(np.abs(q8 - want)) <= 2e-2 * np.max(np.abs(want))      # activation quantization only
