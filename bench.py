@@ -366,13 +366,21 @@ def extras(gpu, pkg, lin_q) -> dict:
     del wq8
     # ---- the other block formats on f32 activations (the reference GPU path's contract): a tall head, one token
     fr = {}
-    for ty, tag in ((pkg.IQ4_XS, "iq4xs"), (pkg.IQ4_NL, "iq4nl"), (pkg.Q3_K, "q3k"), (pkg.Q2_K, "q2k"), (pkg.Q5_0, "q50")):
+    for ty, tag in ((pkg.IQ4_XS, "iq4xs"), (pkg.IQ4_NL, "iq4nl"), (pkg.Q3_K, "q3k"), (pkg.Q2_K, "q2k"), (pkg.Q5_0, "q50"),
+                    (pkg.IQ3_S, "iq3s"), (pkg.IQ2_XXS, "iq2xxs")):
         wf = [gpu.lin(ty, n, k, synth.weights(ty, n, k, "bench", tag, "head")) for _ in range(2)]
-        us = _time(gpu, lambda i: gpu.mm(x, wf[i % 2], y), 20, 3)
+        us = _time(gpu, lambda i: gpu.mm(x, wf[i % 2], y, act_mode=pkg.ACT_FLOAT), 20, 3)
         b = pkg.row_bytes(ty, k) * n + 4 * k + 4 * n
         fr[tag] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
         del wf
     out["float_rows_gemv_128256x4096"] = {"activations": "f32", "kernels": "gemv_nat_<fmt>_px", **fr}
+    # IQ2_XXS as the CPU path multiplies it: int8 activations per 256, integer dots (dot_iq2xxs_q8k)
+    wf = [gpu.lin(pkg.IQ2_XXS, n, k, synth.weights(pkg.IQ2_XXS, n, k, "bench", "iq2xxs", "head")) for _ in range(2)]
+    us = _time(gpu, lambda i: gpu.mm(x, wf[i % 2], y), 20, 3)
+    b = pkg.row_bytes(pkg.IQ2_XXS, k) * n + 4 * k + 4 * n
+    out["iq2xxs_q8k_gemv_128256x4096"] = {"timed": "quantize_q8k + gemv_q8k_iq2xxs_wide", "us": round(us, 2),
+                                          "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
+    del wf
     # ---- one FFN block of a decode layer with the fused epilogues: rmsnorm+quantize, gate/up+SiLU,
     # quantize, down accumulated onto the residual (4 launches, recorded and replayed)
     d, nff = 4096, 14336

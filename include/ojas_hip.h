@@ -47,7 +47,10 @@ enum {
 
 /* GGUF tensor types handled by this path (crates/ojas-formats/src/gguf.rs:563-591). */
 enum { OJH_Q4_0 = 2, OJH_Q4_1 = 3, OJH_Q5_0 = 6, OJH_Q5_1 = 7, OJH_Q8_0 = 8, OJH_Q2_K = 10, OJH_Q3_K = 11, OJH_Q4_K = 12, OJH_Q5_K = 13, OJH_Q6_K = 14,
-       OJH_IQ4_NL = 20, OJH_IQ4_XS = 23 };
+       OJH_IQ4_NL = 20, OJH_IQ4_XS = 23,
+       /* the grid-codebook formats (gguf.rs:840-1041): decoders and f32-activation matvecs for all seven; IQ2_XXS and
+        * IQ3_XXS also on int8 activations, which is what matvec_kq runs for them (cpu_math.rs:1177-1178) */
+       OJH_IQ2_XXS = 16, OJH_IQ2_XS = 17, OJH_IQ3_XXS = 18, OJH_IQ1_S = 19, OJH_IQ3_S = 21, OJH_IQ2_S = 22, OJH_IQ1_M = 29 };
 
 /* Element type of an activation buffer handed to ojh_mm. */
 enum { OJH_X_F32 = 0, OJH_X_BF16 = 1, OJH_X_F16 = 2 };
@@ -61,7 +64,12 @@ enum { OJH_X_F32 = 0, OJH_X_BF16 = 1, OJH_X_F16 = 2 };
  *                 count runs on the matvec entries).  The same holds for the legacy 32-weight
  *                 blocks Q4_0, Q4_1, Q5_0, Q5_1 and for Q2_K and Q3_K, which the reference runs on
  *                 its GPU path only (f32 activations against the weights of `dequant_to_f16`'s
- *                 arms :653-703 and :730-795).
+ *                 arms :653-703 and :730-795).  Of the grid-codebook formats IQ2_XXS and IQ3_XXS
+ *                 take this contract (dot_iq2xxs_q8k / dot_iq3xxs_q8k, :1057-1128: what matvec_kq
+ *                 runs for them, and what OJH_ACT_AUTO picks at every token count); IQ3_S and
+ *                 IQ2_S are f32-activation rows on the CPU path (dot_iq3s, dot_iq2s) and IQ2_XS,
+ *                 IQ1_S, IQ1_M exist on the reference's GPU path only: those five refuse it.  No
+ *                 MFMA tile reads a grid-codebook format.
  *   OJH_ACT_FLOAT — activations kept in floating point (f32 for the GEMV, rounded to f16 into the
  *                 MFMA tile for the GEMM): the contract of the reference's GPU kernels
  *                 (crates/ojas-core/src/quant_src.rs:779-867, crates/ojas-cuda/src/kernels/gemm_q.rs:1-56).

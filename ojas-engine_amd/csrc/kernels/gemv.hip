@@ -15,15 +15,7 @@
 // and applies d*sc (and -dmin*m*sum(x) for Q4_K) once per sub-block.
 #include "ojk_common.h"
 #include "ojk_rows.h"
-
-enum { ST_SET = 0, ST_ACCUM = 1, ST_BIAS = 2 };
-
-template <int MODE>
-__device__ __forceinline__ void store_row(float* y, const float* bs, uint n, float v) {
-    if (MODE == ST_SET) y[n] = v;
-    else if (MODE == ST_ACCUM) y[n] += v;
-    else y[n] = v + bs[n];
-}
+#include "ojk_rowdot.h"
 
 // ------------------------------------------------------------------ Q4_K
 // Lane (g, l) = (lane/8, lane%8): 16 quant bytes l*16.. of super-block g -> 16 weights of
@@ -428,119 +420,6 @@ __device__ __forceinline__ void gemv_nat_q80_m_body(const float* __restrict__ x,
 
 // ------------------------------------------------------------------ IQ4_NL, IQ4_XS and the legacy 32-weight blocks
 // (row traits Iq4nlW, Iq4xsW, Q40W, Q41W, Q50W, Q51W: ojk_rows.h)
-template <class W, int R, int MODE>
-__device__ __forceinline__ void gemv_nat_iq4_body(const float* __restrict__ x, const uchar* __restrict__ w,
-                                                  float* __restrict__ y, const float* __restrict__ bs,
-                                                  uint K, uint N) {
-    const uint lane = threadIdx.x & 63u;
-    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
-    if (row0 >= N) return;
-    const uint nu = W::units(K);
-    const size_t rb = (size_t)nu * W::BYTES;
-    float acc[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.0f;
-    for (uint u = W::unit_of(lane); u < nu; u += W::STEP) {
-        typename W::Frag f[R];
-#pragma unroll
-        for (int r = 0; r < R; r++) f[r] = W::load(w + (size_t)min(row0 + r, N - 1u) * rb, u, lane);
-        const float* xp = x + (size_t)u * W::x_unit(0) + W::x_off(lane);
-        const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + W::XGAP);
-        const float xsum = sum4(x0) + sum4(x1);      // for the formats with an offset or a minimum
-#pragma unroll
-        for (int r = 0; r < R; r++) acc[r] += W::dot(f[r], lane, x0, x1, xsum);
-    }
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        float s = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < N) store_row<MODE>(y, bs, row0 + r, s);
-    }
-}
-
-template <class W, int MT>
-__device__ __forceinline__ void gemv_nat_iq4_m_body(const float* __restrict__ x, const uchar* __restrict__ w,
-                                                    float* __restrict__ y, uint K, uint N, uint M, uint ACC) {
-    const uint lane = threadIdx.x & 63u;
-    const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (row >= N) return;
-    const uint nu = W::units(K);
-    const uchar* wr = w + (size_t)row * nu * W::BYTES;
-    for (uint m0 = 0; m0 < M; m0 += MT) {
-        float acc[MT];
-#pragma unroll
-        for (int i = 0; i < MT; i++) acc[i] = 0.0f;
-        for (uint u = W::unit_of(lane); u < nu; u += W::STEP) {
-            const typename W::Frag f = W::load(wr, u, lane);
-#pragma unroll
-            for (int i = 0; i < MT; i++) {
-                const uint m = min(m0 + i, M - 1u);
-                const float* xp = x + (size_t)m * K + (size_t)u * W::x_unit(0) + W::x_off(lane);
-                const float4 x0 = *(const float4*)xp, x1 = *(const float4*)(xp + W::XGAP);
-                acc[i] += W::dot(f, lane, x0, x1, sum4(x0) + sum4(x1));
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < MT; i++) {
-            float s = wave_sum(acc[i]);
-            if (lane == 0 && m0 + i < M) {
-                float* o = y + (size_t)(m0 + i) * N + row;
-                *o = ACC ? *o + s : s;
-            }
-        }
-    }
-}
-
-// Many rows (an output head): a 4-bit row is an eighth of the bytes of the f32 activations it meets, so
-// a wave that fetches its activation fragments again for every few rows is bound by those loads, not
-// by HBM (2.7 TB/s at 128256 x 4096).  Here rows are grid-stride and the wave keeps its share of x —
-// 8 floats per lane and step, NS steps — in registers for the whole launch; out-of-range steps hold
-// zeros and repeat the last block.   gemv_nat_iq4{nl,xs}_px(x, w, y, K, N), K <= 4096 (64 floats of x per
-// lane; twice that would halve the resident waves).
-template <class W, int NS>
-__device__ __forceinline__ void gemv_nat_iq4_px_body(const float* __restrict__ x, const uchar* __restrict__ w,
-                                                     float* __restrict__ y, uint K, uint N) {
-    const uint lane = threadIdx.x & 63u;
-    const uint nu = W::units(K);
-    const size_t rb = (size_t)nu * W::BYTES;
-    float4 xr[NS][2];
-    float xsum[NS];
-    uint uc[NS];
-#pragma unroll
-    for (int s = 0; s < NS; s++) {
-        const uint u = W::unit_of(lane) + (uint)s * W::STEP;
-        uc[s] = min(u, nu - 1u);
-        xr[s][0] = xr[s][1] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if (u < nu) {
-            const float* xp = x + (size_t)u * W::x_unit(0) + W::x_off(lane);
-            xr[s][0] = *(const float4*)xp;
-            xr[s][1] = *(const float4*)(xp + W::XGAP);
-        }
-        xsum[s] = sum4(xr[s][0]) + sum4(xr[s][1]);
-    }
-    const uint nwaves = gridDim.x * (blockDim.x >> 6);
-    for (uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2u; row0 < N; row0 += nwaves * 2u) {
-        const uchar* r0 = w + (size_t)row0 * rb;
-        const uchar* r1 = w + (size_t)min(row0 + 1u, N - 1u) * rb;
-        float a0 = 0.0f, a1 = 0.0f;
-#pragma unroll
-        for (int s = 0; s < NS; s++) {
-            const typename W::Frag f0 = W::load(r0, uc[s], lane), f1 = W::load(r1, uc[s], lane);
-            a0 += W::dot(f0, lane, xr[s][0], xr[s][1], xsum[s]);
-            a1 += W::dot(f1, lane, xr[s][0], xr[s][1], xsum[s]);
-        }
-        a0 = wave_sum(a0);
-        a1 = wave_sum(a1);
-        if (lane == 0) {
-            y[row0] = a0;
-            if (row0 + 1u < N) y[row0 + 1u] = a1;
-        }
-    }
-}
-
-#define GEMV_NAT_IQ4_PX(FMT, W)                                                                            \
-    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_px(                                 \
-        const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
-        gemv_nat_iq4_px_body<W, 8>(x, w, y, K, N); }
 GEMV_NAT_IQ4_PX(iq4nl, Iq4nlW)
 GEMV_NAT_IQ4_PX(iq4xs, Iq4xsW)
 GEMV_NAT_IQ4_PX(q40, Q40W)
@@ -916,27 +795,6 @@ __device__ __forceinline__ void gemv_nat_kq2_px_body(const float* __restrict__ x
         gemv_nat_kq2_px_body<W>(x, w, y, K, N); }
 GEMV_NAT_KQ2(q2k, Q2kW)
 GEMV_NAT_KQ2(q3k, Q3kW)
-
-#define GEMV_NAT_ENTRIES(FMT)                                                                              \
-    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_r1(                                 \
-        const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
-        gemv_nat_##FMT##_body<1, ST_SET>(x, w, y, nullptr, K, N); }                                        \
-    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_r2(                                 \
-        const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
-        gemv_nat_##FMT##_body<2, ST_SET>(x, w, y, nullptr, K, N); }                                        \
-    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT(                                      \
-        const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
-        gemv_nat_##FMT##_body<4, ST_SET>(x, w, y, nullptr, K, N); }                                        \
-    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_accum(                              \
-        const float* x, const uchar* w, float* y, uint K, uint N) {                                        \
-        gemv_nat_##FMT##_body<4, ST_ACCUM>(x, w, y, nullptr, K, N); }                                      \
-    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_bias(                               \
-        const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {                       \
-        gemv_nat_##FMT##_body<4, ST_BIAS>(x, w, y, bs, K, N); }                                            \
-    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_m(                                  \
-        const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {                      \
-        if (M <= 2) gemv_nat_##FMT##_m_body<2>(x, w, y, K, N, M, ACC);                                     \
-        else gemv_nat_##FMT##_m_body<4>(x, w, y, K, N, M, ACC); }
 
 GEMV_NAT_ENTRIES(q80)
 GEMV_NAT_ENTRIES(q4k)

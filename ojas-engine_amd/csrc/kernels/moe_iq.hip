@@ -16,8 +16,19 @@
 // indices: a slot whose index is E or more contributes zeros instead of reading past the tensors.
 // Rows of the down launch are grid-stride (4 per workgroup and step), so the reference's ceil(N/8)
 // workgroups are a valid grid.
+//
+// The grid-codebook experts of the same table ride the same bodies over the traits of ojk_iq_grid_rows.h:
+//   moe_gu_iq3s, moe_gu_iq3s_slots(x, arena_g, arena_u, act, off_g, off_u, K, N)    (moe_iq.rs:173-191; IQ3_S gate/up with
+//   IQ4_NL down is the combination the streamed models ship in), moe_gu_iq2xxs, moe_down_iq2xxs, moe_down_iq3xxs,
+//   moe_gu_iq2s (the table's remaining IQ rows).
 #include "ojk_moe_rows.h"
+#include "ojk_iq_grid_rows.h"
 
 #define MOE_IQ_ENTRIES(FMT, W) MOE_ROWS_GU_ENTRY(FMT, W) MOE_ROWS_DOWN_ENTRY(FMT, W)
 MOE_IQ_ENTRIES(iq4xs, Iq4xsW)
 MOE_IQ_ENTRIES(iq4nl, Iq4nlW)
+MOE_ROWS_GU_ENTRY(iq3s, Iq3sW)
+MOE_ROWS_GU_SLOTS_ENTRY(iq3s, Iq3sW)
+MOE_IQ_ENTRIES(iq2xxs, Iq2xxsW)
+MOE_ROWS_DOWN_ENTRY(iq3xxs, Iq3xxsW)
+MOE_ROWS_GU_ENTRY(iq2s, Iq2sW)

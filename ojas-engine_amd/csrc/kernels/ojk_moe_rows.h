@@ -1,5 +1,5 @@
 // Expert products over raw rows with f32 activations, shared by the families "moe" and "moe_iq": templates over the
-// row traits of ojk_rows.h.
+// row traits of ojk_rows.h and ojk_iq_grid_rows.h.
 //   moe_gu_rows:    act[j][n] = silu(gate_e . x) * (up_e . x),  e = idx[j]      grid [ceil(N/8), KSEL, tokens] x 256
 //   moe_down_rows:  y[n] += sum_j wgt[j] * (down_e . act[j])                     grid [1 .. ceil(N/4), tokens, 1] x 256
 // A slot whose expert index is E or more contributes zeros instead of reading past the tensors.
@@ -7,19 +7,18 @@
 #include "ojk_common.h"
 #include "ojk_rows.h"
 
+// The rows of one (token, slot): ge / ue point at the slot's gate and up expert (N rows each), nu = the row's units,
+// or 0 for a slot that contributes zeros.
 template <class W>
-__device__ __forceinline__ void moe_gu_rows(const float* __restrict__ x, const uchar* __restrict__ wg,
-                                            const uchar* __restrict__ wu, float* __restrict__ act,
-                                            const uint* __restrict__ idx, uint K, uint N, uint E) {
+__device__ __forceinline__ void moe_gu_rows_at(const float* __restrict__ xt, const uchar* __restrict__ ge,
+                                               const uchar* __restrict__ ue, float* __restrict__ out, uint K, uint N,
+                                               uint nu) {
     const uint lane = threadIdx.x & 63u;
-    const uint j = blockIdx.y, t = blockIdx.z, ksel = gridDim.y;
     const uint row0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 2u;
     if (row0 >= N) return;
-    const uint e = idx[t * ksel + j], nu = e < E ? W::units(K) : 0u;
     const size_t rb = (size_t)W::units(K) * W::BYTES;
-    const float* xt = x + (size_t)t * K;
-    const uchar* g0 = wg + ((size_t)e * N + row0) * rb;
-    const uchar* u0 = wu + ((size_t)e * N + row0) * rb;
+    const uchar* g0 = ge + (size_t)row0 * rb;
+    const uchar* u0 = ue + (size_t)row0 * rb;
     const size_t r1 = row0 + 1u < N ? rb : 0;        // the last odd row is computed twice, stored once
     float ag[2] = {0.0f, 0.0f}, au[2] = {0.0f, 0.0f};
     for (uint u = W::unit_of(lane); u < nu; u += W::STEP) {
@@ -36,8 +35,32 @@ __device__ __forceinline__ void moe_gu_rows(const float* __restrict__ x, const u
 #pragma unroll
     for (int r = 0; r < 2; r++) {
         const float gs = wave_sum(ag[r]), us = wave_sum(au[r]);
-        if (lane == 0 && row0 + r < N) act[((size_t)t * ksel + j) * N + row0 + r] = (gs / (1.0f + expf(-gs))) * us;
+        if (lane == 0 && row0 + r < N) out[row0 + r] = (gs / (1.0f + expf(-gs))) * us;
     }
+}
+
+template <class W>
+__device__ __forceinline__ void moe_gu_rows(const float* __restrict__ x, const uchar* __restrict__ wg,
+                                            const uchar* __restrict__ wu, float* __restrict__ act,
+                                            const uint* __restrict__ idx, uint K, uint N, uint E) {
+    const uint j = blockIdx.y, t = blockIdx.z, ksel = gridDim.y;
+    const uint e = idx[t * ksel + j];
+    const size_t eb = (size_t)N * W::units(K) * W::BYTES;
+    moe_gu_rows_at<W>(x + (size_t)t * K, wg + (size_t)e * eb, wu + (size_t)e * eb, act + ((size_t)t * ksel + j) * N, K, N,
+                      e < E ? W::units(K) : 0u);
+}
+
+// Streamed experts: one u32 byte offset per (token, slot) into a cache arena instead of an expert index
+// (crates/ojas-cuda/src/kernels/moe_iq.rs:181-191); offsets are rounded down to the blocks' two-byte alignment and
+// clamped to LIM, the last offset at which a whole expert still fits its arena.
+template <class W>
+__device__ __forceinline__ void moe_gu_rows_slots(const float* __restrict__ x, const uchar* __restrict__ arena_g,
+                                                  const uchar* __restrict__ arena_u, float* __restrict__ act,
+                                                  const uint* __restrict__ off_g, const uint* __restrict__ off_u, uint K,
+                                                  uint N, uint LIM_G, uint LIM_U) {
+    const uint j = blockIdx.y, t = blockIdx.z, ksel = gridDim.y;
+    const uint og = min(off_g[t * ksel + j] & ~1u, LIM_G), ou = min(off_u[t * ksel + j] & ~1u, LIM_U);
+    moe_gu_rows_at<W>(x + (size_t)t * K, arena_g + og, arena_u + ou, act + ((size_t)t * ksel + j) * N, K, N, W::units(K));
 }
 
 // A workgroup owns four rows at a time (rows grid-stride over the workgroups); its four waves take the slots
@@ -88,6 +111,11 @@ __device__ __forceinline__ void moe_down_rows(const float* __restrict__ act, con
     extern "C" __global__ void __launch_bounds__(256) moe_gu_##FMT(                                         \
         const float* x, const uchar* wg, const uchar* wu, float* act, const uint* idx, uint K, uint N,      \
         uint E) { moe_gu_rows<W>(x, wg, wu, act, idx, K, N, E); }
+#define MOE_ROWS_GU_SLOTS_ENTRY(FMT, W)                                                                     \
+    extern "C" __global__ void __launch_bounds__(256) moe_gu_##FMT##_slots(                                 \
+        const float* x, const uchar* arena_g, const uchar* arena_u, float* act, const uint* off_g,          \
+        const uint* off_u, uint K, uint N, uint LIM_G, uint LIM_U) {                                        \
+        moe_gu_rows_slots<W>(x, arena_g, arena_u, act, off_g, off_u, K, N, LIM_G, LIM_U); }
 #define MOE_ROWS_DOWN_ENTRY(FMT, W)                                                                         \
     extern "C" __global__ void __launch_bounds__(256) moe_down_##FMT(                                       \
         const float* act, const uchar* wd, float* y, const uint* idx, const float* wgt, uint K, uint N,     \

@@ -300,7 +300,7 @@ extern "C" int ojh_lin_load(ojh_device *dev, ojh_gguf *g, const char *const *nam
     }
     const ojh_block_format *f = ojh_format(ty0);
     if (!f || k0 % f->weights)
-        return ojh_fail(OJH_ERR_UNSUPPORTED, "GGUF type %u with K=%llu is not kept in place by this backend (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K .. Q6_K, IQ4_NL, IQ4_XS with whole blocks)",
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "GGUF type %u with K=%llu is not kept in place by this backend (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K .. Q6_K, IQ4_NL, IQ4_XS, the grid-codebook IQ types, with whole blocks)",
                         ty0, (unsigned long long)k0);
     if (n > 0xFFFFFFFFull || k0 > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "ojh_lin_load: tensor too large");
     ojh_buf *buf = nullptr;

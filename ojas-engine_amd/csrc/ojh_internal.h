@@ -109,6 +109,7 @@ struct ojh_block_format {
 const ojh_block_format *ojh_format(uint32_t ggml_type);
 bool ojh_float_rows(uint32_t ggml_type);   // the CPU path reads f32 activations for this format
 size_t ojh_block_align(const ojh_block_format *f);
+bool ojh_grid_type(uint32_t ggml_type);    // a grid-codebook format: its kernels live in the family "iq_grid"
 bool ojh_float_only(uint32_t ggml_type);   // ... and only the f32-activation matvecs exist for it
 
 // What a kernel touches at given constants. Returns OJH_OK or fails with a message.

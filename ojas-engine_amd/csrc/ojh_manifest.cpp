@@ -22,6 +22,13 @@ static const ojh_block_format kFormats[] = {
     {OJH_Q5_1, 24, 32, "q51"},
     {OJH_Q2_K, 84, 256, "q2k"},
     {OJH_Q3_K, 110, 256, "q3k"},
+    {OJH_IQ2_XXS, 66, 256, "iq2xxs"},
+    {OJH_IQ2_XS, 74, 256, "iq2xs"},
+    {OJH_IQ2_S, 82, 256, "iq2s"},
+    {OJH_IQ3_XXS, 98, 256, "iq3xxs"},
+    {OJH_IQ3_S, 110, 256, "iq3s"},
+    {OJH_IQ1_S, 50, 256, "iq1s"},
+    {OJH_IQ1_M, 56, 256, "iq1m"},
 };
 
 // Formats whose CPU path multiplies the raw row with f32 activations (dot_q80, dot_iq4nl, dot_iq4xs:
@@ -29,9 +36,17 @@ static const ojh_block_format kFormats[] = {
 bool ojh_float_rows(uint32_t t) { return t == OJH_Q8_0 || ojh_float_only(t); }
 // ... and for which this library has the f32-activation matvecs only: no int8-activation form, no MFMA tile
 // (the IQ4 types, and the legacy 32-weight blocks and Q2_K / Q3_K, which the reference runs on its GPU path alone)
+// (of the grid-codebook formats the CPU path multiplies IQ3_S and IQ2_S with f32 activations, dot_iq3s / dot_iq2s, and
+// IQ2_XXS and IQ3_XXS with int8 activations, dot_iq2xxs_q8k / dot_iq3xxs_q8k: cpu_math.rs:1177-1179; IQ2_XS, IQ1_S and
+// IQ1_M run on the reference's GPU path alone)
 bool ojh_float_only(uint32_t t) {
     return t == OJH_IQ4_NL || t == OJH_IQ4_XS || t == OJH_Q4_0 || t == OJH_Q4_1 || t == OJH_Q5_0 || t == OJH_Q5_1 ||
-           t == OJH_Q2_K || t == OJH_Q3_K;
+           t == OJH_Q2_K || t == OJH_Q3_K || t == OJH_IQ3_S || t == OJH_IQ2_S || t == OJH_IQ2_XS || t == OJH_IQ1_S ||
+           t == OJH_IQ1_M;
+}
+bool ojh_grid_type(uint32_t t) {
+    return t == OJH_IQ2_XXS || t == OJH_IQ2_XS || t == OJH_IQ2_S || t == OJH_IQ3_XXS || t == OJH_IQ3_S || t == OJH_IQ1_S ||
+           t == OJH_IQ1_M;
 }
 
 // What the kernels' loads need of a block tensor's address: the widest power of two (up to 16) dividing the
@@ -1035,13 +1050,14 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         align[1] = ojh_block_align(f);
         return OJH_OK;
     }
-    case 16: {  // moe_gu_q80_slots(x, arena_g, arena_u, act, off_g, off_u, K, N)
+    case 16: {  // moe_gu_{q80,iq3s}_slots(x, arena_g, arena_u, act, off_g, off_u, K, N)
         uint32_t K = c[0], N = c[1], KS = grid[1], T = grid[2];
+        const ojh_block_format *f = ojh_format(s->type);
         if ((rc = check_block(block, 256))) return rc;
-        if (!K || K % 32 || !N || !KS || !T) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u slots=%u tokens=%u", s->name, K, N, KS, T);
+        if (!K || K % f->weights || !N || !KS || !T) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u slots=%u tokens=%u", s->name, K, N, KS, T);
         if (grid[0] != (N + 7) / 8) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/8), slots, tokens]", s->name);
         need[0] = (size_t)T * K * 4;
-        need[1] = need[2] = (size_t)N * (K / 32) * 34;
+        need[1] = need[2] = (size_t)N * (K / f->weights) * f->bytes;
         need[3] = (size_t)T * KS * N * 4;
         need[4] = need[5] = (size_t)T * KS * 4;
         align[0] = 16;
@@ -1279,7 +1295,10 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     };
     for (const auto &f : kFormats) {
         std::string t = f.tag;
-        add("dequant_" + t + "_f16", "dequant", 2, 1, f.type, 0, check_dequant, shape_dequant);
+        // the grid-codebook formats keep decoder and matvecs in one code object of their own
+        const bool grid_fmt = ojh_grid_type(f.type);
+        const char *fam_nat = grid_fmt ? "iq_grid" : "gemv", *fam_q8k = grid_fmt ? "iq_grid" : "gemv_q8k";
+        add("dequant_" + t + "_f16", grid_fmt ? "iq_grid" : "dequant", 2, 1, f.type, 0, check_dequant, shape_dequant);
         if (f.type == OJH_Q5_K) {   // Q5_K: the decoder, the CPU path's int8-activation matvec
             std::string q5 = "gemv_q8k_" + t;
             add(q5, "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
@@ -1301,28 +1320,28 @@ static std::vector<ojh_kernel_spec> build_manifest() {
             continue;
         }
         std::string g = "gemv_nat_" + t;
-        add(g, "gemv", 3, 2, f.type, 4, check_gemv_nat, shape_rows);
-        add(g + "_r1", "gemv", 3, 2, f.type, 1, check_gemv_nat, shape_rows);
-        add(g + "_r2", "gemv", 3, 2, f.type, 2, check_gemv_nat, shape_rows);
-        add(g + "_accum", "gemv", 3, 2, f.type, 4, check_gemv_nat, shape_rows);
-        add(g + "_bias", "gemv", 4, 2, f.type, 4, check_gemv_nat, shape_rows);
-        add(g + "_m", "gemv", 3, 4, f.type, 1, check_gemv_nat_m, shape_rows);
-        if (f.type != OJH_Q8_0) add(g + "_px", "gemv", 3, 2, f.type, 2, check_gemv_nat_px, shape_px);
+        add(g, fam_nat, 3, 2, f.type, 4, check_gemv_nat, shape_rows);
+        add(g + "_r1", fam_nat, 3, 2, f.type, 1, check_gemv_nat, shape_rows);
+        add(g + "_r2", fam_nat, 3, 2, f.type, 2, check_gemv_nat, shape_rows);
+        add(g + "_accum", fam_nat, 3, 2, f.type, 4, check_gemv_nat, shape_rows);
+        add(g + "_bias", fam_nat, 4, 2, f.type, 4, check_gemv_nat, shape_rows);
+        add(g + "_m", fam_nat, 3, 4, f.type, 1, check_gemv_nat_m, shape_rows);
+        if (f.type != OJH_Q8_0) add(g + "_px", fam_nat, 3, 2, f.type, 2, check_gemv_nat_px, shape_px);
         if (ojh_float_only(f.type)) continue;   // f32 activations only, no MFMA tile
         if (f.type == OJH_Q8_0) {
-            add(g + "_lds", "gemv", 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
-            add(g + "_lds_accum", "gemv", 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
-            add(g + "_lds_bias", "gemv", 4, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
+            add(g + "_lds", fam_nat, 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
+            add(g + "_lds_accum", fam_nat, 3, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
+            add(g + "_lds_bias", fam_nat, 4, 3, f.type, 1, check_gemv_q80_lds, shape_q80_lds);
             continue;  // the CPU path keeps f32 activations for Q8_0
         }
         std::string q = "gemv_q8k_" + t;
-        add(q, "gemv_q8k", 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
-        add(q + "_r1", "gemv_q8k", 4, 2, f.type, 1, check_gemv_q8k, shape_rows);
-        add(q + "_r2", "gemv_q8k", 4, 2, f.type, 2, check_gemv_q8k, shape_rows);
-        add(q + "_wide", "gemv_q8k", 4, 2, f.type, 2, check_gemv_q8k, shape_rows);
-        add(q + "_accum", "gemv_q8k", 4, 2, f.type, 1, check_gemv_q8k, shape_rows);
-        add(q + "_bias", "gemv_q8k", 5, 2, f.type, 1, check_gemv_q8k, shape_rows);
-        add(q + "_m", "gemv_q8k", 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
+        add(q, fam_q8k, 4, 2, f.type, 4, check_gemv_q8k, shape_rows);
+        add(q + "_r1", fam_q8k, 4, 2, f.type, 1, check_gemv_q8k, shape_rows);
+        add(q + "_r2", fam_q8k, 4, 2, f.type, 2, check_gemv_q8k, shape_rows);
+        add(q + "_wide", fam_q8k, 4, 2, f.type, 2, check_gemv_q8k, shape_rows);
+        add(q + "_accum", fam_q8k, 4, 2, f.type, 1, check_gemv_q8k, shape_rows);
+        add(q + "_bias", fam_q8k, 5, 2, f.type, 1, check_gemv_q8k, shape_rows);
+        add(q + "_m", fam_q8k, 4, 4, f.type, 1, check_gemv_q8k_m, shape_rows);
         if (f.type == OJH_Q6_K) add(q + "_mx", "gemv_q8k", 4, 4, f.type, 0, check_gemv_q8k_m, shape_mx);
         if (f.type == OJH_Q6_K) add(q + "_mf", "gemv_q8k", 4, 4, f.type, -1, check_gemv_q8k_m, shape_mf);
         if (f.type == OJH_Q6_K) add(q + "_ml", "gemv_q8k", 4, 4, f.type, -2, check_gemv_q8k_m, shape_ml);
@@ -1368,7 +1387,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     // prefill / verify MFMA tiles: "q8_0" is the reference's spelling for this family
     for (const auto &f : kFormats) {
-        if (f.type == OJH_Q5_K || ojh_float_only(f.type)) continue;
+        if (f.type == OJH_Q5_K || ojh_float_only(f.type) || ojh_grid_type(f.type)) continue;
         std::string g = std::string("gemm_mm_") + (f.type == OJH_Q8_0 ? "q8_0" : f.tag);
         add(g, "gemm", 3, 4, f.type, 0, check_gemm, shape_gemm);
         add(g + "_sk", "gemm", 3, 4, f.type, 1, check_gemm, shape_gemm);
@@ -1422,6 +1441,17 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add("moe_down_" + tag, "moe_iq", 5, 3, ty, 15, check_moe, shape_moe);
         m.back().expert_bufs = 1;
     }
+    // ... and the grid-codebook rows of the expert table (crates/ojas-core/src/quant_src.rs:180-190)
+    for (uint32_t ty : {(uint32_t)OJH_IQ3_S, (uint32_t)OJH_IQ2_XXS, (uint32_t)OJH_IQ2_S}) {
+        add(std::string("moe_gu_") + ojh_format(ty)->tag, "moe_iq", 5, 2, ty, 14, check_moe, shape_moe);
+        m.back().expert_bufs = 2;
+    }
+    for (uint32_t ty : {(uint32_t)OJH_IQ2_XXS, (uint32_t)OJH_IQ3_XXS}) {
+        add(std::string("moe_down_") + ojh_format(ty)->tag, "moe_iq", 5, 3, ty, 15, check_moe, shape_moe);
+        m.back().expert_bufs = 1;
+    }
+    add("moe_gu_iq3s_slots", "moe_iq", 6, 2, OJH_IQ3_S, 16, check_moe, shape_moe);
+    m.back().arena_bufs = 2;
     // K-quant experts on f32 activations, the reference's names (crates/ojas-core/src/quant_src.rs:174-179)
     add("moe_gu_q4k", "moe", 5, 2, OJH_Q4_K, 14, check_moe, shape_moe);
     m.back().expert_bufs = 2;

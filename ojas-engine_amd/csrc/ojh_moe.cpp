@@ -43,10 +43,17 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     // starts from zeros
     // K-quant experts take the same two launches when floating-point activations are asked for (OJH_ACT_FLOAT):
     // moe_gu_q4k / moe_down_{q4k,q5k,q6k}, the reference's GPU expert kernels for those formats.
-    auto float_expert = [](uint32_t t) { return t == OJH_Q8_0 || t == OJH_IQ4_XS || t == OJH_IQ4_NL; };
+    // The grid-codebook rows of the reference's expert table (crates/ojas-core/src/quant_src.rs:180-190) join them:
+    // IQ3_S, IQ2_XXS, IQ2_S gate/up and IQ2_XXS, IQ3_XXS down, on f32 activations like the reference's GPU kernels.
+    auto float_gu = [](uint32_t t) {
+        return t == OJH_Q8_0 || t == OJH_IQ4_XS || t == OJH_IQ4_NL || t == OJH_IQ3_S || t == OJH_IQ2_XXS || t == OJH_IQ2_S;
+    };
+    auto float_down = [](uint32_t t) {
+        return t == OJH_Q8_0 || t == OJH_IQ4_XS || t == OJH_IQ4_NL || t == OJH_IQ2_XXS || t == OJH_IQ3_XXS;
+    };
     const bool kq_float = act_mode == OJH_ACT_FLOAT && gate->type == OJH_Q4_K && up->type == OJH_Q4_K &&
                           (down->type == OJH_Q4_K || down->type == OJH_Q5_K || down->type == OJH_Q6_K);
-    if (kq_float || (gate->type == up->type && float_expert(gate->type) && float_expert(down->type))) {
+    if (kq_float || (gate->type == up->type && float_gu(gate->type) && float_down(down->type))) {
         if (act_mode == OJH_ACT_Q8K)
             return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: %s / %s experts take f32 activations, as their CPU dots do",
                             ojh_format(gate->type)->tag, ojh_format(down->type)->tag);
@@ -63,7 +70,7 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         if ((rc = span("moe_ffn: wgt", wgt, (size_t)NA8 * 4, 4))) return rc;
         if ((rc = span("moe_ffn: y", y, (size_t)T * d * 4, 4))) return rc;
         const std::string gu_name = std::string("moe_gu_") + fg->tag, down_name = std::string("moe_down_") + fd->tag;
-        auto family_of = [](uint32_t t) { return t == OJH_IQ4_XS || t == OJH_IQ4_NL ? "moe_iq" : "moe"; };
+        auto family_of = [](uint32_t t) { return t == OJH_IQ4_XS || t == OJH_IQ4_NL || ojh_grid_type(t) ? "moe_iq" : "moe"; };
         if ((rc = ensure(dev, family_of(gate->type)))) return rc;
         if ((rc = ensure(dev, family_of(down->type)))) return rc;
         ojh_buf *act8;
@@ -84,7 +91,7 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
                           {n_ff, d, ksel, E}, g2, b256);
     }
     if (gate->type != OJH_Q4_K || up->type != OJH_Q4_K || (down->type != OJH_Q4_K && down->type != OJH_Q5_K && down->type != OJH_Q6_K))
-        return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: gate and up must be Q4_K with down Q4_K, Q5_K or Q6_K, or all three among Q8_0, IQ4_XS, IQ4_NL (gate %u, up %u, down %u)",
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "moe_ffn: gate and up must be Q4_K with down Q4_K, Q5_K or Q6_K, or gate/up among Q8_0, IQ4_XS, IQ4_NL, IQ3_S, IQ2_XXS, IQ2_S with down among Q8_0, IQ4_XS, IQ4_NL, IQ2_XXS, IQ3_XXS (gate %u, up %u, down %u)",
                         gate->type, up->type, down->type);
     const bool down5 = down->type != OJH_Q4_K;   // Q5_K or Q6_K down tensors: integer dots at every batch size
     const std::string down_dec = std::string("moe_down_") + ojh_format(down->type)->tag + "_dec";

@@ -90,7 +90,7 @@ extern "C" int ojh_dequant_f16(ojh_device *dev, uint32_t type, const ojh_buf *ra
     int rc;
     if ((rc = span_ok("dequant: raw", raw, raw_off, nb * f->bytes, ojh_block_align(f)))) return rc;
     if ((rc = span_ok("dequant: out", out, out_off, n_weights * 2, 2))) return rc;
-    if ((rc = ensure(dev, "dequant"))) return rc;
+    if ((rc = ensure(dev, ojh_grid_type(type) ? "iq_grid" : "dequant"))) return rc;
     std::string name = std::string("dequant_") + f->tag + "_f16";
     uint32_t grid[3], block[3];
     if ((rc = ojh_launch_shape(dev, name.c_str(), 0, (uint32_t)nb, 0, grid, block))) return rc;
@@ -315,7 +315,7 @@ extern "C" int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xsc
     size_t nsb = w->k / 256;
     if ((rc = span_ok("xq", xq, 0, (size_t)m * nsb * 256, 16))) return rc;
     if ((rc = span_ok("xscales", xscales, 0, (size_t)m * nsb * 4, 4))) return rc;
-    if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+    if ((rc = ensure(dev, "gemv_q8k")) || (ojh_grid_type(w->type) && (rc = ensure(dev, "iq_grid")))) return rc;
     return ojh_mm_q8k_launch(dev, xq->ptr, xscales->ptr, w, f, at(y, y_off), bias, m, accum);
 }
 
@@ -341,6 +341,8 @@ extern "C" int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_bu
     if ((rc = span_ok("xq", xq, 0, nsb * 256, 16))) return rc;
     if ((rc = span_ok("xscales", xscales, 0, nsb * 4, 4))) return rc;
     if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+    for (int i = 0; i < count; i++)
+        if (ojh_grid_type(ws[i]->type) && (rc = ensure(dev, "iq_grid"))) return rc;
     if (!grouped || count == 1) {   // formats without a grouped entry: one launch per projection
         for (int i = 0; i < count; i++) {
             const ojh_block_format *fi = ojh_format(ws[i]->type);
@@ -390,6 +392,8 @@ extern "C" int ojh_mm_multi(ojh_device *dev, const ojh_buf *x, size_t x_off, int
     const uint32_t K = ws[0]->k;
     if ((rc = span_ok("ojh_mm_multi: x", x, x_off, (size_t)K * 4, 16))) return rc;
     if ((rc = ensure(dev, "gemv_q8k"))) return rc;
+    for (int i = 0; i < count; i++)
+        if (ojh_grid_type(ws[i]->type) && (rc = ensure(dev, "iq_grid"))) return rc;
     // Measured on MI355X (weights streamed from HBM): the single launch wins on a small stage (q/k/v of an 8B model:
     // 6.6 against 7.7 us), ties on 4096 x 4096 and loses from there on — few large workgroups cannot keep as many bytes
     // in flight as the plain matvec's thousands of small ones, and many small ones repeat the quantization too often.
@@ -481,13 +485,18 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
 
     // IQ4_NL / IQ4_XS (dot_iq4nl / dot_iq4xs), Q4_0 / Q4_1 / Q5_0 / Q5_1 and Q2_K / Q3_K: f32 activations against the raw
     // rows at every token count; no int8-activation form and no MFMA tile read them.
-    const bool iq4 = ojh_float_only(w->type) || q5_float;   // (the IQ4 types, the legacy 32-weight blocks, Q2_K, Q3_K)
+    // The grid-codebook formats likewise have no MFMA tile; IQ2_XXS and IQ3_XXS take int8 activations unless f32
+    // ones are asked for (dot_iq2xxs_q8k / dot_iq3xxs_q8k under matvec_kq, dot_iq2xxs / dot_iq3xxs under dot_iq).
+    const bool grid_fmt = ojh_grid_type(w->type);
+    const bool iq4 = ojh_float_only(w->type) || q5_float;   // (the IQ4 types, the legacy 32-weight blocks, Q2_K, Q3_K, ...)
     if (iq4 && act_mode == OJH_ACT_Q8K)
         return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: %s rows take f32 activations only (OJH_ACT_FLOAT or OJH_ACT_AUTO)", f->tag);
 
     // Above the crossover the MFMA tile wins over streaming the weights once per few tokens
     // (the reference switches at 8 rows, crates/ojas-models/src/decoder/dispatch.rs:70-75).
-    if (m >= dev->gemm_min_m && act_mode != OJH_ACT_Q8K && !iq4 && K % 64 == 0 && (uint64_t)m * K < 0x7FFFFFFFull &&
+    if (grid_fmt && !iq4 && act_mode == OJH_ACT_AUTO) act_mode = OJH_ACT_Q8K;
+    if (grid_fmt && (rc = ensure(dev, "iq_grid"))) return rc;
+    if (m >= dev->gemm_min_m && act_mode != OJH_ACT_Q8K && !iq4 && !grid_fmt && K % 64 == 0 && (uint64_t)m * K < 0x7FFFFFFFull &&
         (uint64_t)m * N < 0x7FFFFFFFull) {
         // Q4_K takes the 256-wide tile with the reference GPU kernel's arithmetic (f16 qa*q + qb)
         // unless the tile that reproduces dequant_to_f16 bit for bit is asked for.
@@ -531,6 +540,8 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     }
 
     bool q8k = !ojh_float_rows(w->type) && act_mode != OJH_ACT_FLOAT && act_mode != OJH_ACT_FLOAT_EXACT;
+    if (grid_fmt && act_mode == OJH_ACT_FLOAT_EXACT)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_mm: %s rows have no MFMA tile; OJH_ACT_FLOAT runs their f32-activation matvec", f->tag);
     // Opt-in: one token, f32 in, plain store through the launch that quantizes x itself
     // (bit-identical results).  Measured slower than quantize + matvec at every decode shape on
     // MI355X — each block repeats the quantization and reads x through LDS — so it is off by default.
@@ -570,7 +581,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         if ((rc = ojh_launch(dev, "copy_bf16_f32", {xp, xf->ptr}, {n_el}, eg, block))) return rc;
         xp = xf->ptr;
     }
-    if ((rc = ensure(dev, "gemv"))) return rc;
+    if (!grid_fmt && (rc = ensure(dev, "gemv"))) return rc;
     std::string base = std::string("gemv_nat_") + f->tag;
     // Q8_0 rows from a few thousand up: activations in registers, rows copied into LDS by the
     // memory system (needs 16-byte aligned rows and a K that chunks)
