@@ -22,6 +22,9 @@ def _model(pkg, tmp_path, alignment=None, version=3):
         "blk.0.ffn_up.weight": (pkg.synth.iq4xs_weights(48, k, "gguf", "u"), [k, 48], IQ4_XS),
         "blk.0.ffn_gate.weight": (pkg.synth.iq4xs_weights(48, k, "gguf", "g"), [k, 48], IQ4_XS),
         "blk.0.ffn_down.weight": (pkg.synth.iq4nl_weights(40, 96, "gguf", "d"), [96, 40], IQ4_NL),
+        "blk.0.exp_gate.weight": (pkg.synth.grid_weights(21, 24, k, "gguf", "eg"), [k, 24], 21),     # IQ3_S
+        "blk.0.exp_up.weight": (pkg.synth.grid_weights(21, 24, k, "gguf", "eu"), [k, 24], 21),
+        "blk.0.exp_down.weight": (pkg.synth.grid_weights(16, 8, k, "gguf", "ed"), [k, 8], 16),       # IQ2_XXS
         "norm.weight": (pkg.synth.normal_f32(k, "gguf", "n"), [k], 0),
     }
     meta = [("general.architecture", gw.STR, "llama"), ("llama.block_count", gw.U32, 1),
@@ -127,6 +130,17 @@ def test_lin_load_stacks_tensors_and_keeps_the_files_bytes(gpu, orc, pkg, tmp_pa
     y5 = gpu.alloc(40)
     gpu.mm(gpu.upload(x96), dn, y5, 1)
     assert peak_err(gpu.read(y5, 40), orc.matvec_kq(t["blk.0.ffn_down.weight"][0], IQ4_NL, 40, 96, x96)) <= 1e-5
+    # grid-codebook tensors: IQ3_S stacked (f32 activations, dot_iq3s), IQ2_XXS on int8 activations (dot_iq2xxs_q8k)
+    eg = gpu.lin_load(g, ["blk.0.exp_gate.weight", "blk.0.exp_up.weight"])
+    assert (eg.n, eg.k, eg.ty) == (48, k, 21)
+    y6 = gpu.alloc(48)
+    gpu.mm(gpu.upload(x), eg, y6, 1)
+    both = np.concatenate([t["blk.0.exp_gate.weight"][0], t["blk.0.exp_up.weight"][0]])
+    assert peak_err(gpu.read(y6, 48), orc.matvec_kq(both, 21, 48, k, x)) <= 1e-5
+    ed = gpu.lin_load(g, ["blk.0.exp_down.weight"])
+    y7 = gpu.alloc(8)
+    gpu.mm(gpu.upload(x), ed, y7, 1)
+    assert peak_err(gpu.read(y7, 8), orc.matvec_kq(t["blk.0.exp_down.weight"][0], 16, 8, k, x)) <= 2e-5
     with pytest.raises(pkg.OjasHipError, match="type differs"):
         gpu.lin_load(g, ["blk.0.attn_q.weight", "output.weight"])
     with pytest.raises(pkg.OjasHipError, match="K 64 differs"):
