@@ -377,15 +377,20 @@ struct GbRow {
     }
 };
 
-template <bool SPLITK, bool ACCUM, int MI>
+// SPLITK: 0 the whole K; 1 K slices that add into y with f32 atomics (y zeroed or holding the sum to extend: the
+// reference's `_sk` contract, crates/ojas-cuda/src/kernels/gemm_q.rs:26-38); 2 K slices that leave their partial tiles
+// in `part` and count themselves in `cnt`, the last one to arrive adding the slices in order and storing y (`_sr`).
+template <int SPLITK, bool ACCUM, int MI>
 __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, const uchar* __restrict__ w,
-                                             float* __restrict__ y, uint K, uint N, uint M, uint nsplit, uchar* lds) {
+                                             float* __restrict__ y, uint K, uint N, uint M, uint nsplit, uchar* lds,
+                                             float* __restrict__ part = nullptr, uint* __restrict__ cnt = nullptr,
+                                             uint acc_y = 0u) {
     const uint tid = threadIdx.x, lane = tid & 63u;
     const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint n0 = blockIdx.x * GX_BN, m0 = blockIdx.y * (32u * MI);
     const uint nsb = K >> 8;
     uint sb_begin = 0, sb_end = nsb;
-    if (SPLITK) {
+    if (SPLITK != 0) {
         const uint per = (nsb + nsplit - 1) / nsplit;
         sb_begin = min(blockIdx.z * per, nsb);
         sb_end = min((blockIdx.z + 1) * per, nsb);
@@ -545,6 +550,59 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
 #undef GB_MIX
 #undef GB_STEP
 
+    if (SPLITK == 2) {
+        // The slice's tile goes to `part` as the registers hold it (the halves of thread t's q-th float4 at [q][half][t]:
+        // 512 contiguous bytes per wave and store), then the slice counts itself; the workgroup that finds every other slice counted reads them all back —
+        // its own too, so that the sum ((s0 + s1) + s2) + ... does not depend on who came last — and owns y.  Nobody
+        // waits: a slice that is not last is done.
+        const uint per = (nsb + nsplit - 1) / nsplit, ns_eff = (nsb + per - 1) / per;
+        const uint tile = blockIdx.y * gridDim.x + blockIdx.x;
+        constexpr uint TILE_F4 = (uint)MI * 8u * 256u;
+        // The partial tiles bypass the L2 both ways (system-scope accesses: written through, read from behind the
+        // cache): the slices of a tile run on different XCDs, whose L2s do not see each other's lines, and a fence
+        // of device scope would write back and invalidate a whole L2 per workgroup (measured: twice the kernel time).
+        // Reading the slices back is what this form costs: one workgroup per tile, every load a trip to memory.
+        typedef unsigned long long u64;
+        u64* const mine = (u64*)part + ((size_t)tile * ns_eff + blockIdx.z) * TILE_F4 * 2u + tid;      // [q][half][thread]
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    u64* const o = mine + (size_t)((i * 2 + j) * 4 + q) * 512u;
+                    const u64 lo = (u64)__float_as_uint(acc[i][j][4 * q]) | ((u64)__float_as_uint(acc[i][j][4 * q + 1]) << 32);
+                    const u64 hi = (u64)__float_as_uint(acc[i][j][4 * q + 2]) | ((u64)__float_as_uint(acc[i][j][4 * q + 3]) << 32);
+                    __hip_atomic_store(o, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    __hip_atomic_store(o + 256, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");      // the stores have left before the slice is counted
+        __syncthreads();
+        if (tid == 0u) *(volatile uint*)lds = atomicAdd(cnt + tile, 1u);
+        __syncthreads();
+        if ((uint)__builtin_amdgcn_readfirstlane((int)*(volatile uint*)lds) != ns_eff - 1u) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        const u64* const all = (const u64*)part + (size_t)tile * ns_eff * TILE_F4 * 2u + tid;
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const u64* const at = all + (size_t)((i * 2 + j) * 4 + q) * 512u;
+                    float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    for (uint sl = 0; sl < ns_eff; sl++) {
+                        const u64 lo = __hip_atomic_load(at + (size_t)sl * TILE_F4 * 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                        const u64 hi = __hip_atomic_load(at + (size_t)sl * TILE_F4 * 2u + 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                        const float4 v = make_float4(__uint_as_float((uint)lo), __uint_as_float((uint)(lo >> 32)),
+                                                     __uint_as_float((uint)hi), __uint_as_float((uint)(hi >> 32)));
+                        if (sl == 0u) sum = v;
+                        else { sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w; }
+                    }
+                    acc[i][j][4 * q] = sum.x; acc[i][j][4 * q + 1] = sum.y; acc[i][j][4 * q + 2] = sum.z; acc[i][j][4 * q + 3] = sum.w;
+                }
+        if (tid == 0u) cnt[tile] = 0u;        // ready for the next launch
+    }
     // epilogue: D register v of block (i, j) holds token row 32 i + 8 (v / 4) + 4 kg + v % 4, output 64 wave + 32 j + fr
 #pragma unroll
     for (int i = 0; i < MI; i++) {
@@ -556,7 +614,8 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
                 const uint m = m0 + 32u * i + 8u * (v >> 2) + 4u * kg + (v & 3u);
                 if (m < M && n < N) {
                     float* o = y + (size_t)m * N + n;
-                    if (SPLITK) atomicAdd(o, acc[i][j][v]);
+                    if (SPLITK == 1) atomicAdd(o, acc[i][j][v]);
+                    else if (SPLITK == 2) *o = acc_y ? *o + acc[i][j][v] : acc[i][j][v];
                     else if (ACCUM) *o += acc[i][j][v];
                     else *o = acc[i][j][v];
                 }
@@ -570,25 +629,41 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
 extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemm_mm_q4kl_bd(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
     __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(4)];
-    if (accum) gemm_bd_body<false, true, 4>(xh, w, y, K, N, M, 1u, lds);
-    else gemm_bd_body<false, false, 4>(xh, w, y, K, N, M, 1u, lds);
+    if (accum) gemm_bd_body<0, true, 4>(xh, w, y, K, N, M, 1u, lds);
+    else gemm_bd_body<0, false, 4>(xh, w, y, K, N, M, 1u, lds);
 }
 extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemm_mm_q4kl_bd_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
     __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(4)];
-    gemm_bd_body<true, true, 4>(xh, w, y, K, N, M, nsplit, lds);
+    gemm_bd_body<1, true, 4>(xh, w, y, K, N, M, nsplit, lds);
 }
 // 256 tokens per tile: the wave's 64 rows are dequantized once for twice the MFMAs
 extern "C" __global__ void __launch_bounds__(256)
 gemm_mm_q4kl_bd256(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
     __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(8)];
-    if (accum) gemm_bd_body<false, true, 8>(xh, w, y, K, N, M, 1u, lds);
-    else gemm_bd_body<false, false, 8>(xh, w, y, K, N, M, 1u, lds);
+    if (accum) gemm_bd_body<0, true, 8>(xh, w, y, K, N, M, 1u, lds);
+    else gemm_bd_body<0, false, 8>(xh, w, y, K, N, M, 1u, lds);
 }
 extern "C" __global__ void __launch_bounds__(256)
 gemm_mm_q4kl_bd256_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
     __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(8)];
-    gemm_bd_body<true, true, 8>(xh, w, y, K, N, M, nsplit, lds);
+    gemm_bd_body<1, true, 8>(xh, w, y, K, N, M, nsplit, lds);
+}
+// K slices without atomics and without a zero fill: partial tiles through `part` (tiles x slices x 128 KB, 256 KB for
+// the 256-token tile), one counter per tile in `cnt` (zero before the first launch; every launch leaves zeros), the
+// slices added in their order: results do not depend on arrival.
+//   gemm_mm_q4kl_bd{,256}_sr(xh, w, y, part, cnt, K, N, M, nsplit, ACC)     grid [ceil(N/256), ceil(M/128 | 256), nsplit]
+extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+gemm_mm_q4kl_bd_sr(const ushort* xh, const uchar* w, float* y, float* part, uint* cnt, uint K, uint N, uint M, uint nsplit,
+                   uint ACC) {
+    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(4)];
+    gemm_bd_body<2, true, 4>(xh, w, y, K, N, M, nsplit, lds, part, cnt, ACC);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemm_mm_q4kl_bd256_sr(const ushort* xh, const uchar* w, float* y, float* part, uint* cnt, uint K, uint N, uint M,
+                      uint nsplit, uint ACC) {
+    __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(8)];
+    gemm_bd_body<2, true, 8>(xh, w, y, K, N, M, nsplit, lds, part, cnt, ACC);
 }
 
 // LDS of a tile: two activation stages, two dequantized-weight stages, two raw-weight slots

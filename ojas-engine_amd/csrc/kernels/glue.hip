@@ -8,6 +8,7 @@
 //   copy_bf16_f32(x, y, n)   bf16 -> f32 (exact)
 //   copy_bf16_half(x, y, n)  bf16 -> f16, round to nearest even
 //   fill_zero_u32(y, n)      y[i] = 0 for n dwords (a fill kernel, safe inside a captured graph)
+//   copy_{bf16,f32}_half_zero(x, y, z, n, nz, CB)  the conversion and a zero fill of nz dwords at z in one launch
 //   stream_copy_u32x4(x, y, n16)  y = x for n16 16-byte units: a copy of known size
 //   stream_read_u32x4(x, y, n16)  reads n16 16-byte units, writes one dword per wave (y: grid*4 dwords)
 //   calib_mfma_f16(x, y, iters, mode)  matrix-pipe calibration: what v_mfma_f32_32x32x16_f16 sustains on the
@@ -21,8 +22,7 @@
 // The element-wise kernels are grid-stride loops over groups of 8 elements (128-bit accesses when
 // both pointers are 16-byte aligned), plus a scalar tail: any grid of 256-thread blocks is valid.
 template <class In, class Out, class F>
-__device__ __forceinline__ void map8(const In* __restrict__ x, Out* __restrict__ y, uint n, F f) {
-    const uint stride = gridDim.x * 256u, t = blockIdx.x * 256u + threadIdx.x;
+__device__ __forceinline__ void map8_at(const In* __restrict__ x, Out* __restrict__ y, uint n, F f, uint t, uint stride) {
     uint done = 0;
     if ((((size_t)x | (size_t)y) & 15u) == 0) {
         const uint n8 = n >> 3;
@@ -39,6 +39,10 @@ __device__ __forceinline__ void map8(const In* __restrict__ x, Out* __restrict__
         done = n8 << 3;
     }
     for (uint i = done + t; i < n; i += stride) y[i] = f(x[i]);
+}
+template <class In, class Out, class F>
+__device__ __forceinline__ void map8(const In* __restrict__ x, Out* __restrict__ y, uint n, F f) {
+    map8_at(x, y, n, f, blockIdx.x * 256u + threadIdx.x, gridDim.x * 256u);
 }
 
 extern "C" __global__ void __launch_bounds__(256)
@@ -62,9 +66,7 @@ copy_bf16_half(const ushort* __restrict__ x, ushort* __restrict__ y, uint n) {
     map8(x, y, n, [](ushort v) { return __half_as_ushort(__float2half_rn(bf16_bits_to_f32(v))); });
 }
 
-extern "C" __global__ void __launch_bounds__(256)
-fill_zero_u32(uint* __restrict__ y, uint n) {
-    const uint stride = gridDim.x * 256u, t = blockIdx.x * 256u + threadIdx.x;
+__device__ __forceinline__ void fill_zero_at(uint* __restrict__ y, uint n, uint t, uint stride) {
     uint done = 0;
     if (((size_t)y & 15u) == 0) {
         const uint n4 = n >> 2;
@@ -72,6 +74,27 @@ fill_zero_u32(uint* __restrict__ y, uint n) {
         done = n4 << 2;
     }
     for (uint i = done + t; i < n; i += stride) y[i] = 0u;
+}
+extern "C" __global__ void __launch_bounds__(256)
+fill_zero_u32(uint* __restrict__ y, uint n) {
+    fill_zero_at(y, n, blockIdx.x * 256u + threadIdx.x, gridDim.x * 256u);
+}
+
+// The two launches ahead of a split-K tile in one: the first CB workgroups convert n activations to f16, the others
+// clear nz dwords of the output the K slices will add into.   copy_{bf16,f32}_half_zero(x, y, z, n, nz, CB), any
+// grid with more than CB workgroups.
+extern "C" __global__ void __launch_bounds__(256)
+copy_bf16_half_zero(const ushort* __restrict__ x, ushort* __restrict__ y, uint* __restrict__ z, uint n, uint nz, uint CB) {
+    if (blockIdx.x < CB)
+        map8_at(x, y, n, [](ushort v) { return __half_as_ushort(__float2half_rn(bf16_bits_to_f32(v))); },
+                blockIdx.x * 256u + threadIdx.x, CB * 256u);
+    else fill_zero_at(z, nz, (blockIdx.x - CB) * 256u + threadIdx.x, (gridDim.x - CB) * 256u);
+}
+extern "C" __global__ void __launch_bounds__(256)
+copy_f32_half_zero(const float* __restrict__ x, ushort* __restrict__ y, uint* __restrict__ z, uint n, uint nz, uint CB) {
+    if (blockIdx.x < CB)
+        map8_at(x, y, n, [](float v) { return __half_as_ushort(__float2half_rn(v)); }, blockIdx.x * 256u + threadIdx.x, CB * 256u);
+    else fill_zero_at(z, nz, (blockIdx.x - CB) * 256u + threadIdx.x, (gridDim.x - CB) * 256u);
 }
 
 extern "C" __global__ void __launch_bounds__(256)

@@ -73,6 +73,7 @@ struct ojh_device {
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
                                  // 3 = per-assignment decode form always, 4 = matrix cores in the workgroup-per-tile form always
     uint32_t moe_dec_tokens = 8; // OJAS_HIP_MOE_DEC_TOKENS: the decode form serves up to this many tokens
+    bool gemm_sr = false;        // OJAS_HIP_GEMM_SR=1: K slices of the prefill tile meet in scratch, added in slice order (reproducible bits), instead of in f32 atomics
     bool moe_fuse = true;        // OJAS_HIP_MOE_FUSE=0: the grouped pipeline keeps its quantizer and grouping launches apart
     bool gemm_exact = false;     // OJAS_HIP_GEMM_EXACT: Q4_K prefill through the tile that holds dequant_to_f16 bits
     bool fused_quant = false;    // OJAS_HIP_FUSED_QUANT=1: ojh_mm (m = 1, Q4_K) quantizes x inside the matvec launch
@@ -109,6 +110,7 @@ struct ojh_block_format {
 const ojh_block_format *ojh_format(uint32_t ggml_type);
 bool ojh_float_rows(uint32_t ggml_type);   // the CPU path reads f32 activations for this format
 size_t ojh_block_align(const ojh_block_format *f);
+uint32_t ojh_gemm_sr_slices(uint32_t K, uint32_t nsplit);   // K slices of the `_sr` tiles that hold a super-block
 bool ojh_grid_type(uint32_t ggml_type);    // a grid-codebook format: its kernels live in the family "iq_grid"
 bool ojh_float_only(uint32_t ggml_type);   // ... and only the f32-activation matvecs exist for it
 
@@ -141,6 +143,8 @@ const ojh_kernel_spec *ojh_find_kernel(const char *name);
 
 // ---- helpers -----------------------------------------------------------------------------------
 int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out);
+// ... a slot whose kernels leave zeros behind: cleared whenever it is (re)allocated
+int ojh_scratch_get_zeroed(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out);
 int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptrs,
                const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);
 // shared by ojh_mm / ojh_mm_q8k / ojh_mm_noalloc (ojh_ops.cpp)

@@ -835,6 +835,53 @@ static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_
     return OJH_OK;
 }
 
+// gemm_mm_q4kl_bd{,256}_sr(xh, w, y, part, cnt, K, N, M, nsplit, ACC): K slices that meet in `part` (one tile per
+// slice, 4 bytes x tile outputs) under one counter per tile; `rows_per_wave` = tokens per tile.
+uint32_t ojh_gemm_sr_slices(uint32_t K, uint32_t nsplit) {   // slices that hold at least one super-block
+    const uint32_t nsb = K / 256, per = (nsb + nsplit - 1) / nsplit;
+    return per ? (nsb + per - 1) / per : 0;
+}
+static int check_gemm_sr(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                         const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const ojh_block_format *f;
+    const uint32_t bm = (uint32_t)s->rows_per_wave, bn = 256;
+    uint32_t K = c[0], N = c[1], M = c[2], nsplit = c[3];
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if (M == 0 || nsplit == 0 || nsplit > K / 256) return ojh_fail(OJH_ERR_ARG, "%s: M=%u and nsplit=%u (1 .. K/256) out of range", s->name, M, nsplit);
+    if ((rc = check_block(block, 256))) return rc;
+    if (grid[0] != (N + bn - 1) / bn || grid[1] != (M + bm - 1) / bm || grid[2] != nsplit)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, (N + bn - 1) / bn, (M + bm - 1) / bm, nsplit);
+    if ((uint64_t)M * K * 2 > 0xFFFFFFFFull)
+        return ojh_fail(OJH_ERR_ARG, "%s: M*K=%llu exceeds 2^31 activations", s->name, (unsigned long long)M * K);
+    if ((uint64_t)N * (K / f->weights) * f->bytes > 0xFFFFFFFFull)
+        return ojh_fail(OJH_ERR_ARG, "%s: the weight tensor exceeds 4 GiB", s->name);
+    const size_t tiles = (size_t)grid[0] * grid[1];
+    need[0] = (size_t)M * K * 2;
+    need[1] = (size_t)N * (K / f->weights) * f->bytes;
+    need[2] = (size_t)M * N * 4;
+    need[3] = tiles * ojh_gemm_sr_slices(K, nsplit) * bm * bn * 4;
+    need[4] = tiles * 4;
+    align[1] = ojh_block_align(f);
+    align[2] = align[4] = 4;
+    return OJH_OK;
+}
+static int shape_gemm_sr(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
+                         uint32_t grid[3], uint32_t block[3]) {
+    const uint32_t bm = (uint32_t)s->rows_per_wave;
+    grid[0] = (N + 255) / 256;
+    grid[1] = (M + bm - 1) / bm;
+    uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
+    uint32_t tiles = grid[0] * grid[1], nsb = K / 256;
+    uint32_t z = tiles ? cus / tiles : 1;
+    if (z > nsb) z = nsb;
+    if (z > 16) z = 16;
+    grid[2] = z ? z : 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // gemm_mm_q4l(x f32, w4, y, qa, qb, K, N, accum, M), gemm_mm_q4l_hb(xh f16, ...), gemm_mm_q4l_sk(xh, w4, y, qa, qb, K, N, M, nsplit):
 // the reference's argument lists (crates/ojas-cuda/src/kernels/gemm_q.rs:26-38).  `rows_per_wave`: 8 plain with f32
 // activations, 9 split-K, 10 plain with f16 activations; all on the 256 x 128 tile.
@@ -1179,6 +1226,24 @@ static int check_elementwise(const ojh_kernel_spec *s, const uint32_t *c, const 
     return OJH_OK;
 }
 
+// copy_{bf16,f32}_half_zero(x, y, z, n, nz, CB): CB converting workgroups, the rest of the grid clears z
+static int check_convert_zero(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                              const uint32_t block[3], size_t need[16], size_t align[16]) {
+    uint32_t n = c[0], nz = c[1], cb = c[2];
+    if (!n || !nz) return ojh_fail(OJH_ERR_ARG, "%s: n=%u and nz=%u must be positive", s->name, n, nz);
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (grid[1] != 1 || grid[2] != 1 || !cb || grid[0] <= cb)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1] with x > CB=%u > 0 (CB workgroups convert, the others clear)", s->name, cb);
+    need[0] = (size_t)n * (s->type >> 8);
+    need[1] = (size_t)n * 2;
+    need[2] = (size_t)nz * 4;
+    align[0] = s->type >> 8;
+    align[1] = 2;
+    align[2] = 4;
+    return OJH_OK;
+}
+
 // stream_copy_u32x4(x, y, n16) / stream_read_u32x4(x, y, n16): grid-stride over 16-byte units
 static int check_stream(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                         const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -1212,6 +1277,15 @@ static int shape_elementwise(const ojh_kernel_spec *, const ojh_device *, uint32
                              uint32_t grid[3], uint32_t block[3]) {
     grid[0] = (N / 8 + 255) / 256;  // N = element count; a thread takes 8 elements per trip
     if (!grid[0]) grid[0] = 1;
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+// N = activations to convert, M = dwords to clear, a thread takes 8 elements or 4 dwords; CB = ceil(N / 2048)
+static int shape_convert_zero(const ojh_kernel_spec *, const ojh_device *, uint32_t, uint32_t N, uint32_t M,
+                              uint32_t grid[3], uint32_t block[3]) {
+    grid[0] = (N / 8 + 255) / 256 + 1 + (M / 4 + 255) / 256 + 1;
     grid[1] = grid[2] = 1;
     block[0] = 256;
     block[1] = block[2] = 1;
@@ -1397,6 +1471,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("gemm_mm_q4l_sk", "gemm", 5, 4, 0, 9, check_gemm_q4l, shape_gemm);
     add("gemm_mm_q4l_hb", "gemm", 5, 4, 0, 10, check_gemm_q4l, shape_gemm);
     // Q4_K with the arithmetic of the reference's `gemm_mm_q4l` (f16 qa*q + qb), 256-wide tiles
+    add("gemm_mm_q4kl_bd_sr", "gemm_xl", 5, 5, OJH_Q4_K, 128, check_gemm_sr, shape_gemm_sr);
+    add("gemm_mm_q4kl_bd256_sr", "gemm_xl", 5, 5, OJH_Q4_K, 256, check_gemm_sr, shape_gemm_sr);
     add("gemm_mm_q4kl", "gemm_xl", 3, 4, OJH_Q4_K, 2, check_gemm, shape_gemm);
     add("gemm_mm_q4kl_sk", "gemm_xl", 3, 4, OJH_Q4_K, 3, check_gemm, shape_gemm);
     add("gemm_mm_q4kl_m128", "gemm_xl", 3, 4, OJH_Q4_K, 4, check_gemm, shape_gemm);
@@ -1467,6 +1543,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("copy_f32_bf16", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     add("copy_bf16_f32", "glue", 2, 1, (2u << 8) | 4u, 0, check_elementwise, shape_elementwise);
     add("fill_zero_u32", "glue", 1, 1, 4u, 0, check_elementwise, shape_elementwise);
+    add("copy_bf16_half_zero", "glue", 3, 3, (2u << 8) | 2u, 0, check_convert_zero, shape_convert_zero);
+    add("copy_f32_half_zero", "glue", 3, 3, (4u << 8) | 2u, 0, check_convert_zero, shape_convert_zero);
     add("stream_copy_u32x4", "glue", 2, 1, 0, 0, check_stream, shape_stream);
     add("stream_read_u32x4", "glue", 2, 1, 1, 0, check_stream, shape_stream);
     add("calib_mfma_f16", "glue", 2, 2, 0, 0, check_calib_mfma, shape_calib_mfma);

@@ -505,10 +505,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         if ((rc = ensure(dev, "glue")) || (rc = ensure(dev, xl ? "gemm_xl" : "gemm"))) return rc;
         ojh_buf *xh;
         if ((rc = ojh_scratch_get(dev, "xh", (size_t)m * K * 2, &xh))) return rc;
-        uint32_t n_el = m * K, eg[3] = {(n_el / 8 + 255) / 256 + 1, 1, 1};
-        if ((rc = ojh_launch(dev, x_dtype == OJH_X_BF16 ? "copy_bf16_half" : "copy_f32_half", {at(x, x_off), xh->ptr},
-                             {n_el}, eg, block)))
-            return rc;
+        const uint32_t n_el = m * K, conv_blocks = (n_el / 8 + 255) / 256 + 1;
         std::string base = std::string("gemm_mm_") + (w->type == OJH_Q8_0 ? "q8_0" : f->tag);
         if (xl) {
             // 256-token tiles when they give every CU a tile, or half of them with a K long enough
@@ -528,13 +525,35 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         // at 224 and at 448 workgroups against 2.0 and 2.4).
         if (xl && base == "gemm_mm_q4kl" && (uint64_t)sg[0] * sg[1] * sg[2] >= (uint32_t)dev->prop.multiProcessorCount)
             base = "gemm_mm_q4kl_bd256";
-        if (sg[2] > 1) {
-            if (!accum) {
-                uint32_t n_y = m * N, zg[3] = {(n_y / 4 + 255) / 256 + 1, 1, 1};
-                if ((rc = ojh_launch(dev, "fill_zero_u32", {yp}, {n_y}, zg, block))) return rc;
-            }
-            return ojh_launch(dev, (base + "_sk").c_str(), {xh->ptr, wp, yp}, {K, N, m, sg[2]}, sg, sb);
+        // On request (OJAS_HIP_GEMM_SR=1) the K slices of the tiles that dequantize into the B registers meet in
+        // scratch, the last slice of a tile to finish adding them in slice order: bits that do not depend on arrival, no
+        // zero fill.  Measured slower than the atomics (one workgroup per tile reads every slice back from behind the
+        // L2: gate/up at 128 tokens 60 against 45 us, down 142 against 46), so it is not the default.
+        if (sg[2] > 1 && xl && base != "gemm_mm_q4kl" && dev->gemm_sr && !dev->no_scratch) {
+            uint32_t eg[3] = {conv_blocks, 1, 1};
+            if ((rc = ojh_launch(dev, x_dtype == OJH_X_BF16 ? "copy_bf16_half" : "copy_f32_half", {at(x, x_off), xh->ptr},
+                                 {n_el}, eg, block)))
+                return rc;
+            const size_t tiles = (size_t)sg[0] * sg[1], bm = base == "gemm_mm_q4kl_bd256" ? 256 : 128;
+            ojh_buf *part, *cnt;
+            if ((rc = ojh_scratch_get(dev, "gemm_part", tiles * ojh_gemm_sr_slices(K, sg[2]) * bm * 256 * 4, &part))) return rc;
+            if ((rc = ojh_scratch_get_zeroed(dev, "gemm_cnt", tiles * 4, &cnt))) return rc;
+            return ojh_launch(dev, (base + "_sr").c_str(), {xh->ptr, wp, yp, part->ptr, cnt->ptr},
+                              {K, N, m, sg[2], (uint32_t)(accum != 0)}, sg, sb);
         }
+        // activations to f16 — and, ahead of K slices that add into y, the zero fill of y in the same launch
+        if (sg[2] > 1 && !accum) {
+            uint32_t n_y = m * N, cg[3] = {conv_blocks + (n_y / 4 + 255) / 256 + 1, 1, 1};
+            if ((rc = ojh_launch(dev, x_dtype == OJH_X_BF16 ? "copy_bf16_half_zero" : "copy_f32_half_zero",
+                                 {at(x, x_off), xh->ptr, yp}, {n_el, n_y, conv_blocks}, cg, block)))
+                return rc;
+        } else {
+            uint32_t eg[3] = {conv_blocks, 1, 1};
+            if ((rc = ojh_launch(dev, x_dtype == OJH_X_BF16 ? "copy_bf16_half" : "copy_f32_half", {at(x, x_off), xh->ptr},
+                                 {n_el}, eg, block)))
+                return rc;
+        }
+        if (sg[2] > 1) return ojh_launch(dev, (base + "_sk").c_str(), {xh->ptr, wp, yp}, {K, N, m, sg[2]}, sg, sb);
         sg[2] = 1;
         return ojh_launch(dev, base.c_str(), {xh->ptr, wp, yp}, {K, N, (uint32_t)(accum != 0), m}, sg, sb);
     }

@@ -89,6 +89,7 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_MOE")) d->moe_mode = atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE_DEC_TOKENS")) d->moe_dec_tokens = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE_FUSE")) d->moe_fuse = atoi(r) != 0;
+    if (const char *r = getenv("OJAS_HIP_GEMM_SR")) d->gemm_sr = atoi(r) != 0;
     if (const char *r = getenv("OJAS_HIP_FUSED_QUANT")) d->fused_quant = atoi(r) != 0;
     if (const char *r = getenv("OJAS_HIP_FQ_ROWS")) d->fq_rows = atoi(r) == 1 || atoi(r) == 2 ? atoi(r) : 0;
     if (const char *r = getenv("OJAS_HIP_FQ_THREADS")) d->fq_threads = atoi(r) == 512 ? 512u : atoi(r) == 256 ? 256u : 1024u;
@@ -248,6 +249,15 @@ int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **o
         if (rc) return rc;
     }
     *out = slot;
+    return OJH_OK;
+}
+
+int ojh_scratch_get_zeroed(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out) {
+    auto it = dev->scratch.find(name);
+    const void *before = it != dev->scratch.end() && it->second ? it->second->ptr : nullptr;
+    int rc = ojh_scratch_get(dev, name, bytes, out);
+    if (rc) return rc;
+    if ((*out)->ptr != before) OJH_HIP(hipMemsetAsync((*out)->ptr, 0, (*out)->bytes, dev->stream));   // (never while capturing: growth is refused there)
     return OJH_OK;
 }
 

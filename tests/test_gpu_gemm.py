@@ -130,6 +130,48 @@ def test_split_k_entry_through_the_kernel_seam(gpu, orc, pkg, kernel, family, bm
         gpu.dispatch(enc, kernel, [(xh, 0), (wd, 0), (yd, 0)], [k, n, m, 2], [3, 1, 1], [256, 1, 1])
 
 
+@pytest.mark.parametrize("kernel,bm", [("gemm_mm_q4kl_bd_sr", 128), ("gemm_mm_q4kl_bd256_sr", 256)])
+def test_split_k_slices_meeting_in_scratch(gpu, orc, pkg, kernel, bm):
+    """`_sr`: K slices leave partial tiles in a scratch buffer and the last to arrive adds them in slice order — store
+    or accumulate, no zero fill, the counters back at zero for the next launch, the same bits on every run and the bits
+    of the unsplit tile when there is one slice; more slices than super-blocks leave the surplus empty."""
+    gpu.ensure_family("gemm_xl")
+    m, k, n = 300, 2048, 520
+    w = pkg.synth.q4k_weights(n, k, "gemmsr", "w")
+    x = pkg.synth.normal_f32(m * k, "gemmsr", "x").reshape(m, k)
+    xh, wd = gpu.upload_bytes(x.astype(np.float16)), gpu.upload_bytes(w)
+    want = orc.matmul_ref(w, Q4_K, n, k, x, wmode=2, xmode=1)
+    tiles = ((n + 255) // 256) * ((m + bm - 1) // bm)
+    cnt = gpu.upload_bytes(np.zeros(tiles, np.uint32))
+    sent = np.full(n, 12345.5, np.float32)
+    plain = kernel[:-3]
+    yp = gpu.alloc(m * n)
+    gpu.dispatch(gpu.begin(), plain, [(xh, 0), (wd, 0), (yp, 0)], [k, n, 0, m], [(n + 255) // 256, (m + bm - 1) // bm, 1], [256, 1, 1])
+    unsplit = gpu.read(yp, m * n)
+    for nsplit in (1, 2, 3, 8):
+        slices = -(-(k // 256) // -(-(k // 256) // nsplit))
+        part = gpu.upload(np.full(tiles * slices * bm * 256, np.nan, np.float32))
+        grid = [(n + 255) // 256, (m + bm - 1) // bm, nsplit]
+        runs = []
+        for accum in (0, 1, 0):
+            y0 = pkg.synth.normal_f32(m * n, "gemmsr", "y0", nsplit, accum).reshape(m, n)
+            yd = gpu.upload(np.concatenate([y0.ravel(), sent]))
+            gpu.dispatch(gpu.begin(), kernel, [(xh, 0), (wd, 0), (yd, 0), (part, 0), (cnt, 0)], [k, n, m, nsplit, accum], grid, [256, 1, 1])
+            got = gpu.read(yd, m * n + n)
+            assert np.array_equal(got[m * n:], sent), "wrote past row M"
+            e = rms_errs(got[:m * n].reshape(m, n), want + (y0 if accum else 0.0))
+            assert e[0] < 1e-4 and e[1] < 2e-5, (nsplit, accum, e)
+            assert not np.any(gpu.read(cnt, tiles, np.uint32)), "a tile counter was left non-zero"
+            if not accum:
+                runs.append(got[:m * n].copy())
+        assert np.array_equal(runs[0], runs[1]), "slices added in an order that depends on arrival"
+        if nsplit == 1:
+            assert np.array_equal(runs[0], unsplit)
+    with pytest.raises(pkg.OjasHipError, match="needs"):
+        gpu.dispatch(gpu.begin(), kernel, [(xh, 0), (wd, 0), (yp, 0), (cnt, 0), (cnt, 0)], [k, n, m, 2, 0],
+                     [(n + 255) // 256, (m + bm - 1) // bm, 2], [256, 1, 1])
+
+
 @pytest.mark.parametrize("m,k,n", [(140, 2048, 300), (128, 256, 256), (77, 512, 64), (260, 1024, 513)])
 def test_tile_with_weights_dequantized_into_registers(gpu, orc, pkg, m, k, n):
     """`gemm_mm_q4kl_bd` and `gemm_mm_q4kl_bd256` by name: the 128 x 256 and 256 x 256 tiles whose waves dequantize their own
