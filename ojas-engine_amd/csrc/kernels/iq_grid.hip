@@ -12,8 +12,8 @@
 //                                                                  (cpu_math.rs:1057-1128), what matvec_kq runs for these two
 //
 // One lane decodes one group of eight weights (ojk_iq_grid_rows.h); the matvec bodies are the trait-driven ones the
-// other raw-row formats use (ojk_rowdot.h).  A first version: the codebook entry is fetched by the lane that needs
-// it (a dependent load behind the row's bytes) and the group's signs and digits are unpacked per lane.
+// other raw-row formats use (ojk_rowdot.h).  The matvec workgroups expand their codebook into LDS first (1 to 16 KB);
+// the decoders, eight blocks per workgroup, read the packed table in place.
 #include "ojk_iq_grid_rows.h"
 #include "ojk_rowdot.h"
 
@@ -26,7 +26,7 @@ __device__ __forceinline__ void dequant_grid_body(const uchar* __restrict__ w, u
     const size_t b = tid >> 5;
     if (b >= nblocks) return;
     const uint t = (uint)tid & 31u;
-    const IqgFrag f = G::decode(w + b * G::BYTES, t);
+    const IqgFrag f = G::template decode<false>(w + b * G::BYTES, t);
     const float v[8] = {sb0(f.w0), sb1(f.w0), sb2(f.w0), sb3(f.w0), sb0(f.w1), sb1(f.w1), sb2(f.w1), sb3(f.w1)};
     uint o[4];
 #pragma unroll
@@ -54,13 +54,21 @@ IQ_GRID_DEQUANT(iq1m, Iq1mG)
     template <int R, int MODE>                                                                              \
     __device__ __forceinline__ void gemv_nat_##FMT##_body(const float* x, const uchar* w, float* y,         \
                                                           const float* bs, uint K, uint N) {                \
+        W::init();                                                                                          \
+        __syncthreads();                                                                                    \
         gemv_nat_iq4_body<W, R, MODE>(x, w, y, bs, K, N); }                                                 \
     template <int MT>                                                                                       \
     __device__ __forceinline__ void gemv_nat_##FMT##_m_body(const float* x, const uchar* w, float* y,       \
                                                             uint K, uint N, uint M, uint ACC) {             \
+        W::init();                                                                                          \
+        __syncthreads();                                                                                    \
         gemv_nat_iq4_m_body<W, MT>(x, w, y, K, N, M, ACC); }                                                \
     GEMV_NAT_ENTRIES(FMT)                                                                                   \
-    GEMV_NAT_IQ4_PX(FMT, W)
+    extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_px(                                  \
+        const float* x, const uchar* w, float* y, uint K, uint N) {                                         \
+        W::init();                                                                                          \
+        __syncthreads();                                                                                    \
+        gemv_nat_iq4_px_body<W, 8>(x, w, y, K, N); }
 IQ_GRID_NAT(iq2xxs, Iq2xxsW)
 IQ_GRID_NAT(iq2xs, Iq2xsW)
 IQ_GRID_NAT(iq2s, Iq2sW)
@@ -77,6 +85,8 @@ template <class G, int R, int MODE>
 __device__ __forceinline__ void gemv_q8k_grid_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
                                                    const uchar* __restrict__ w, float* __restrict__ y,
                                                    const float* __restrict__ bs, uint K, uint N) {
+    G::init();
+    __syncthreads();
     const uint lane = threadIdx.x & 63u, t = lane & 31u;
     const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
     if (row0 >= N) return;
@@ -88,7 +98,7 @@ __device__ __forceinline__ void gemv_q8k_grid_body(const signed char* __restrict
     for (uint u = lane >> 5; u < nu; u += 2u) {
         IqgFrag f[R];
 #pragma unroll
-        for (int r = 0; r < R; r++) f[r] = G::decode(w + (size_t)min(row0 + r, N - 1u) * rb + (size_t)u * G::BYTES, t);
+        for (int r = 0; r < R; r++) f[r] = G::template decode<true>(w + (size_t)min(row0 + r, N - 1u) * rb + (size_t)u * G::BYTES, t);
         const uint2 q = *(const uint2*)(xq + (size_t)u * 256u + t * 8u);
         const float s = xs[u];
 #pragma unroll
@@ -106,6 +116,8 @@ template <class G, int MT>
 __device__ __forceinline__ void gemv_q8k_grid_m_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
                                                      const uchar* __restrict__ w, float* __restrict__ y, uint K, uint N,
                                                      uint M, uint ACC) {
+    G::init();
+    __syncthreads();
     const uint lane = threadIdx.x & 63u, t = lane & 31u;
     const uint row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= N) return;
@@ -116,7 +128,7 @@ __device__ __forceinline__ void gemv_q8k_grid_m_body(const signed char* __restri
 #pragma unroll
         for (int i = 0; i < MT; i++) acc[i] = 0.0f;
         for (uint u = lane >> 5; u < nu; u += 2u) {
-            const IqgFrag f = G::decode(wr + (size_t)u * G::BYTES, t);
+            const IqgFrag f = G::template decode<true>(wr + (size_t)u * G::BYTES, t);
 #pragma unroll
             for (int i = 0; i < MT; i++) {
                 const uint m = min(m0 + i, M - 1u);

@@ -27,8 +27,24 @@
 #define MOE_IQ_ENTRIES(FMT, W) MOE_ROWS_GU_ENTRY(FMT, W) MOE_ROWS_DOWN_ENTRY(FMT, W)
 MOE_IQ_ENTRIES(iq4xs, Iq4xsW)
 MOE_IQ_ENTRIES(iq4nl, Iq4nlW)
-MOE_ROWS_GU_ENTRY(iq3s, Iq3sW)
-MOE_ROWS_GU_SLOTS_ENTRY(iq3s, Iq3sW)
-MOE_IQ_ENTRIES(iq2xxs, Iq2xxsW)
-MOE_ROWS_DOWN_ENTRY(iq3xxs, Iq3xxsW)
-MOE_ROWS_GU_ENTRY(iq2s, Iq2sW)
+// (their workgroups expand the codebook into LDS before the rows)
+#define MOE_GRID_GU_ENTRY(FMT, W)                                                                           \
+    extern "C" __global__ void __launch_bounds__(256) moe_gu_##FMT(                                         \
+        const float* x, const uchar* wg, const uchar* wu, float* act, const uint* idx, uint K, uint N,      \
+        uint E) { W::init(); __syncthreads(); moe_gu_rows<W>(x, wg, wu, act, idx, K, N, E); }
+#define MOE_GRID_GU_SLOTS_ENTRY(FMT, W)                                                                     \
+    extern "C" __global__ void __launch_bounds__(256) moe_gu_##FMT##_slots(                                 \
+        const float* x, const uchar* arena_g, const uchar* arena_u, float* act, const uint* off_g,          \
+        const uint* off_u, uint K, uint N, uint LIM_G, uint LIM_U) {                                        \
+        W::init(); __syncthreads();                                                                         \
+        moe_gu_rows_slots<W>(x, arena_g, arena_u, act, off_g, off_u, K, N, LIM_G, LIM_U); }
+#define MOE_GRID_DOWN_ENTRY(FMT, W)                                                                         \
+    extern "C" __global__ void __launch_bounds__(256) moe_down_##FMT(                                       \
+        const float* act, const uchar* wd, float* y, const uint* idx, const float* wgt, uint K, uint N,     \
+        uint KSEL, uint E) { W::init(); __syncthreads(); moe_down_rows<W>(act, wd, y, idx, wgt, K, N, KSEL, E); }
+MOE_GRID_GU_ENTRY(iq3s, Iq3sW)
+MOE_GRID_GU_SLOTS_ENTRY(iq3s, Iq3sW)
+MOE_GRID_GU_ENTRY(iq2xxs, Iq2xxsW)
+MOE_GRID_DOWN_ENTRY(iq2xxs, Iq2xxsW)
+MOE_GRID_DOWN_ENTRY(iq3xxs, Iq3xxsW)
+MOE_GRID_GU_ENTRY(iq2s, Iq2sW)

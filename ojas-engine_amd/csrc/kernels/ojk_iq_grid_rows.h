@@ -42,68 +42,97 @@ __device__ __forceinline__ uint iqg_apply_signs(uint m, uint sg) {
     const uint s4 = (sg & 1u) | ((sg & 2u) << 7) | ((sg & 4u) << 14) | ((sg & 8u) << 21);
     return (m ^ (s4 * 0xFFu)) + s4;      // -m = ~m + 1 byte by byte; m > 0, so no byte carries into the next
 }
-__device__ __forceinline__ void iqg_iq2_entry(uint e, uint sg, IqgFrag& f) {      // magnitudes {8, 25, 43}
-    f.w0 = iqg_apply_signs(__builtin_amdgcn_perm(0u, 0x002B1908u, iqg_spread2(e & 0xFFu)), sg & 15u);
-    f.w1 = iqg_apply_signs(__builtin_amdgcn_perm(0u, 0x002B1908u, iqg_spread2(e >> 8)), sg >> 4);
+// A workgroup may expand the codebook it needs into LDS once (G::init(), then a barrier) and decode with
+// decode<true>: one ds_read per entry instead of a dependent global load and the digit unpacking.  decode<false>
+// reads the packed table in global memory — for the decoders, whose workgroups each see eight blocks only.
+template <uint N2>
+__device__ __forceinline__ uint2* iqg_lds64() { __shared__ uint2 tab[N2]; return tab; }
+template <uint N1>
+__device__ __forceinline__ uint* iqg_lds32() { __shared__ uint tab[N1]; return tab; }
+__device__ __forceinline__ uint2 iqg_iq2_mags(uint e) {
+    return make_uint2(__builtin_amdgcn_perm(0u, 0x002B1908u, iqg_spread2(e & 0xFFu)), __builtin_amdgcn_perm(0u, 0x002B1908u, iqg_spread2(e >> 8)));
 }
-__device__ __forceinline__ void iqg_iq1_entry(uint e, IqgFrag& f) {               // values {-1, 0, +1}
-    f.w0 = __builtin_amdgcn_perm(0u, 0x000100FFu, iqg_spread2(e & 0xFFu));
-    f.w1 = __builtin_amdgcn_perm(0u, 0x000100FFu, iqg_spread2(e >> 8));
+#define IQG_TABLE64(NAME, N, PK, EXPAND)                                                                    \
+    static __device__ __forceinline__ uint2* table() { return iqg_lds64<N>(); }                             \
+    static __device__ __forceinline__ void init() {                                                         \
+        uint2* t = table();                                                                                 \
+        for (uint i = threadIdx.x; i < N; i += blockDim.x) t[i] = EXPAND((uint)PK[i]);                      \
+    }                                                                                                       \
+    template <bool LDS> static __device__ __forceinline__ uint2 entry(uint i) { return LDS ? table()[i] : EXPAND((uint)PK[i]); }
+#define IQG_TABLE32(NAME, N, PK, EXPAND)                                                                    \
+    static __device__ __forceinline__ uint* table() { return iqg_lds32<N>(); }                              \
+    static __device__ __forceinline__ void init() {                                                         \
+        uint* t = table();                                                                                  \
+        for (uint i = threadIdx.x; i < N; i += blockDim.x) t[i] = EXPAND((uint)PK[i]);                      \
+    }                                                                                                       \
+    template <bool LDS> static __device__ __forceinline__ uint entry(uint i) { return LDS ? table()[i] : EXPAND((uint)PK[i]); }
+__device__ __forceinline__ uint2 iqg_iq1_vals(uint e) {
+    return make_uint2(__builtin_amdgcn_perm(0u, 0x000100FFu, iqg_spread2(e & 0xFFu)), __builtin_amdgcn_perm(0u, 0x000100FFu, iqg_spread2(e >> 8)));
+}
+__device__ __forceinline__ uint iqg_iq3xxs_mags(uint e) { return __builtin_amdgcn_perm(0x3E342C24u, 0x1C140C04u, iqg_spread3(e)); }
+__device__ __forceinline__ uint iqg_iq3s_mags(uint e) { return __builtin_amdgcn_perm(0x0F0D0B09u, 0x07050301u, iqg_spread3(e)); }
+__device__ __forceinline__ void iqg_signed(uint2 m, uint sg, IqgFrag& f) {
+    f.w0 = iqg_apply_signs(m.x, sg & 15u);
+    f.w1 = iqg_apply_signs(m.y, sg >> 4);
 }
 
 struct Iq2xxsG {   // { f16 d; u16 qs[32] }: per sub-block 4 index bytes, then 4 x 7 sign-table bits + a 4-bit scale
     static constexpr uint BYTES = IQ2XXS_BYTES;
-    static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
+    IQG_TABLE64(iq2xxs, 256u, ojk_iq2xxs_grid_pk, iqg_iq2_mags)
+    template <bool LDS = false> static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
         const uint ib = t >> 2, l = t & 3u;
         const uint a0 = *(const u32_a2*)(blk + 2u + 8u * ib), a1 = *(const u32_a2*)(blk + 6u + 8u * ib);
         IqgFrag f;
         f.dl = f16_bits_to_f32(*(const ushort*)blk) * (0.5f + (float)(a1 >> 28)) * 0.25f;
         f.delta = 0.0f;
-        iqg_iq2_entry(ojk_iq2xxs_grid_pk[(a0 >> (8u * l)) & 255u], iqg_ksigns(a1 >> (7u * l)), f);
+        iqg_signed(entry<LDS>((a0 >> (8u * l)) & 255u), iqg_ksigns(a1 >> (7u * l)), f);
         return f;
     }
 };
 struct Iq2xsG {    // { f16 d; u16 qs[32]; u8 scales[8] }: 9 index bits + 7 sign-table bits per group, a scale nibble per 16
     static constexpr uint BYTES = IQ2XS_BYTES;
-    static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
+    IQG_TABLE64(iq2xs, 512u, ojk_iq2xs_grid_pk, iqg_iq2_mags)
+    template <bool LDS = false> static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
         const uint ib = t >> 2, l = t & 3u;
         const uint q = *(const ushort*)(blk + 2u + 2u * t), sc = blk[66u + ib];
         IqgFrag f;
         f.dl = f16_bits_to_f32(*(const ushort*)blk) * (0.5f + (float)(l < 2u ? sc & 15u : sc >> 4)) * 0.25f;
         f.delta = 0.0f;
-        iqg_iq2_entry(ojk_iq2xs_grid_pk[q & 511u], iqg_ksigns(q >> 9), f);
+        iqg_signed(entry<LDS>(q & 511u), iqg_ksigns(q >> 9), f);
         return f;
     }
 };
 struct Iq2sG {     // { f16 d; u8 qs[32]; u8 signs[32]; u8 qh[8]; u8 scales[8] }: 10 index bits, a raw sign byte
     static constexpr uint BYTES = IQ2S_BYTES;
-    static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
+    IQG_TABLE64(iq2s, 1024u, ojk_iq2s_grid_pk, iqg_iq2_mags)
+    template <bool LDS = false> static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
         const uint ib = t >> 2, l = t & 3u;
         const uint idx = (uint)blk[2u + t] | ((((uint)blk[66u + ib]) << (8u - 2u * l)) & 0x300u), sc = blk[74u + ib];
         IqgFrag f;
         f.dl = f16_bits_to_f32(*(const ushort*)blk) * (0.5f + (float)(l < 2u ? sc & 15u : sc >> 4)) * 0.25f;
         f.delta = 0.0f;
-        iqg_iq2_entry(ojk_iq2s_grid_pk[idx], blk[34u + t], f);
+        iqg_signed(entry<LDS>(idx), blk[34u + t], f);
         return f;
     }
 };
 struct Iq3xxsG {   // { f16 d; u8 qs[64]; u32 ss[8] }: two 4-weight entries per group; ss as IQ2_XXS's second word
     static constexpr uint BYTES = IQ3XXS_BYTES;
-    static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
+    IQG_TABLE32(iq3xxs, 256u, ojk_iq3xxs_grid_pk, iqg_iq3xxs_mags)
+    template <bool LDS = false> static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
         const uint ib = t >> 2, l = t & 3u;
         const uint q = *(const ushort*)(blk + 2u + 2u * t), a = *(const u32_a2*)(blk + 66u + 4u * ib);
         const uint sg = iqg_ksigns(a >> (7u * l));
         IqgFrag f;
         f.dl = f16_bits_to_f32(*(const ushort*)blk) * (0.5f + (float)(a >> 28)) * 0.5f;
         f.delta = 0.0f;
-        f.w0 = iqg_apply_signs(__builtin_amdgcn_perm(0x3E342C24u, 0x1C140C04u, iqg_spread3(ojk_iq3xxs_grid_pk[q & 255u])), sg & 15u);
-        f.w1 = iqg_apply_signs(__builtin_amdgcn_perm(0x3E342C24u, 0x1C140C04u, iqg_spread3(ojk_iq3xxs_grid_pk[q >> 8])), sg >> 4);
+        iqg_signed(make_uint2(entry<LDS>(q & 255u), entry<LDS>(q >> 8)), sg, f);
         return f;
     }
 };
 struct Iq3sG {     // { f16 d; u8 qs[64]; u8 qh[8]; u8 signs[32]; u8 scales[4] }: 9 index bits, raw signs, scale 1 + 2 s
     static constexpr uint BYTES = IQ3S_BYTES;
-    static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
+    IQG_TABLE32(iq3s, 512u, ojk_iq3s_grid_pk, iqg_iq3s_mags)
+    template <bool LDS = false> static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
         const uint g = t >> 2, l = t & 3u;
         const uint q = *(const ushort*)(blk + 2u + 2u * t), h = blk[66u + g], sg = blk[74u + t];
         const uint s = ((uint)blk[106u + (g >> 1)] >> (4u * (g & 1u))) & 15u;
@@ -111,26 +140,29 @@ struct Iq3sG {     // { f16 d; u8 qs[64]; u8 qh[8]; u8 signs[32]; u8 scales[4] }
         IqgFrag f;
         f.dl = f16_bits_to_f32(*(const ushort*)blk) * (1.0f + 2.0f * (float)s);
         f.delta = 0.0f;
-        f.w0 = iqg_apply_signs(__builtin_amdgcn_perm(0x0F0D0B09u, 0x07050301u, iqg_spread3(ojk_iq3s_grid_pk[i1])), sg & 15u);
-        f.w1 = iqg_apply_signs(__builtin_amdgcn_perm(0x0F0D0B09u, 0x07050301u, iqg_spread3(ojk_iq3s_grid_pk[i2])), sg >> 4);
+        iqg_signed(make_uint2(entry<LDS>(i1), entry<LDS>(i2)), sg, f);
         return f;
     }
 };
 struct Iq1sG {     // { f16 d; u8 qs[32]; u16 qh[8] }: qh = 4 x 3 high index bits, a 3-bit scale, the sign of delta
     static constexpr uint BYTES = IQ1S_BYTES;
-    static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
+    IQG_TABLE64(iq1s, 2048u, ojk_iq1s_grid_pk, iqg_iq1_vals)
+    template <bool LDS = false> static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
         const uint ib = t >> 2, l = t & 3u;
         const uint qh = *(const ushort*)(blk + 34u + 2u * ib);
         IqgFrag f;
         f.dl = f16_bits_to_f32(*(const ushort*)blk) * (float)(2u * ((qh >> 12) & 7u) + 1u);
         f.delta = qh & 0x8000u ? -0.125f : 0.125f;
-        iqg_iq1_entry(ojk_iq1s_grid_pk[(uint)blk[2u + t] | (((qh >> (3u * l)) & 7u) << 8)], f);
+        const uint2 v = entry<LDS>((uint)blk[2u + t] | (((qh >> (3u * l)) & 7u) << 8));
+        f.w0 = v.x;
+        f.w1 = v.y;
         return f;
     }
 };
 struct Iq1mG {     // { u8 qs[32]; u8 qh[16]; u16 scales[4] }: d in the top nibbles of the scale words, two 3-bit scales per 32
     static constexpr uint BYTES = IQ1M_BYTES;
-    static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
+    IQG_TABLE64(iq1m, 2048u, ojk_iq1s_grid_pk, iqg_iq1_vals)
+    template <bool LDS = false> static __device__ __forceinline__ IqgFrag decode(const uchar* blk, uint t) {
         const uint ib = t >> 2, l = t & 3u;
         const u32x2_a2 sc = *(const u32x2_a2*)(blk + 48u);      // scale words 0, 1 | 2, 3
         const uint dbits = ((sc.x >> 12) & 0xFu) | ((sc.x >> 24) & 0xF0u) | ((sc.y >> 4) & 0xF00u) | ((sc.y >> 16) & 0xF000u);
@@ -141,12 +173,14 @@ struct Iq1mG {     // { u8 qs[32]; u8 qh[16]; u16 scales[4] }: d in the top nibb
         IqgFrag f;
         f.dl = f16_bits_to_f32(dbits) * (float)(2u * s + 1u);
         f.delta = h & (l & 1u ? 0x80u : 0x08u) ? -0.125f : 0.125f;
-        iqg_iq1_entry(ojk_iq1s_grid_pk[(uint)blk[t] | hi], f);
+        const uint2 v = entry<LDS>((uint)blk[t] | hi);
+        f.w0 = v.x;
+        f.w1 = v.y;
         return f;
     }
 };
 
-// The trait the matvec and expert bodies take: lane -> (block of the step, group of the block); the lane's eight
+// The trait the matvec and expert bodies take (their kernels call W::init() and a barrier first): lane -> (block of the step, group of the block); the lane's eight
 // activations are two consecutive float4.
 template <class G>
 struct IqGridW {
@@ -158,8 +192,9 @@ struct IqGridW {
     static __device__ __forceinline__ uint x_off(uint lane) { return (lane & 31u) * 8u; }
     static __device__ __forceinline__ uint x_unit(uint) { return 256u; }
     typedef IqgFrag Frag;
+    static __device__ __forceinline__ void init() { G::init(); }
     static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
-        return G::decode(row + (size_t)u * G::BYTES, lane & 31u);
+        return G::template decode<true>(row + (size_t)u * G::BYTES, lane & 31u);     // after G::init() and a barrier
     }
     static __device__ __forceinline__ float dot(const Frag& f, uint, float4 x0, float4 x1, float xsum) {
         float a = sb0(f.w0) * x0.x;
