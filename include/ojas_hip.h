@@ -50,7 +50,12 @@ enum { OJH_Q4_0 = 2, OJH_Q4_1 = 3, OJH_Q5_0 = 6, OJH_Q5_1 = 7, OJH_Q8_0 = 8, OJH
        OJH_IQ4_NL = 20, OJH_IQ4_XS = 23,
        /* the grid-codebook formats (gguf.rs:840-1041): decoders and f32-activation matvecs for all seven; IQ2_XXS and
         * IQ3_XXS also on int8 activations, which is what matvec_kq runs for them (cpu_math.rs:1177-1178) */
-       OJH_IQ2_XXS = 16, OJH_IQ2_XS = 17, OJH_IQ3_XXS = 18, OJH_IQ1_S = 19, OJH_IQ3_S = 21, OJH_IQ2_S = 22, OJH_IQ1_M = 29 };
+       OJH_IQ2_XXS = 16, OJH_IQ2_XS = 17, OJH_IQ3_XXS = 18, OJH_IQ1_S = 19, OJH_IQ3_S = 21, OJH_IQ2_S = 22, OJH_IQ1_M = 29,
+       /* MXFP4 as the reference packs it for its native matvec: { u8 e8m0 scale; u8 qs[16] } = 17 bytes per 32 weights,
+        * weight 2j the low and 2j+1 the high nibble of qs[j]; 139 is the reference's synthetic id (this is a safetensors
+        * format, not a GGUF type: crates/ojas-core/src/quant_src.rs:91-95, crates/ojas-formats/src/mxfp4.rs).  f32
+        * activations only, no MFMA tile. */
+       OJH_MXFP4 = 139 };
 
 /* Element type of an activation buffer handed to ojh_mm. */
 enum { OJH_X_F32 = 0, OJH_X_BF16 = 1, OJH_X_F16 = 2 };

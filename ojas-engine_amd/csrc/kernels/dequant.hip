@@ -1,6 +1,6 @@
 // Family "dequant": GGUF blocks -> IEEE binary16, bit-exact with the reference decoder
 // (crates/ojas-formats/src/gguf.rs:612-1116; arms :704-709 Q8_0, :1042-1059 Q4_K,
-// :1060-1085 Q5_K, :1086-1108 Q6_K, :796-813 IQ4_NL, :814-840 IQ4_XS, :653-703 Q4_0 / Q5_0 / Q4_1 / Q5_1).
+// :1060-1085 Q5_K, :1086-1108 Q6_K, :796-813 IQ4_NL, :814-840 IQ4_XS, :653-703 Q4_0 / Q5_0 / Q4_1 / Q5_1; MXFP4: crates/ojas-formats/src/mxfp4.rs).
 //
 // Bit-exactness rules: every product and difference is a separately rounded f32 operation
 // (__fmul_rn / __fsub_rn, never an FMA), in the reference's association order, followed by one
@@ -297,3 +297,25 @@ extern "C" __global__ void __launch_bounds__(256)
 dequant_q50_f16(const uchar* w, ushort* out, uint nblocks) { dequant_legacy<true, false>(w, out, nblocks); }
 extern "C" __global__ void __launch_bounds__(256)
 dequant_q51_f16(const uchar* w, ushort* out, uint nblocks) { dequant_legacy<true, true>(w, out, nblocks); }
+
+// MXFP4 (crates/ojas-formats/src/mxfp4.rs:40-58): { u8 e; u8 qs[16] }, w = 2^(e - 127) * E2M1[code], weight 2j the low
+// and 2j + 1 the high nibble of qs[j]; one thread per byte of codes (32 threads per pair of blocks would leave half a
+// wave idle: 16 threads per block).  The product of a power of two and a 2-bit significand is exact; one rounding to f16.
+extern "C" __global__ void __launch_bounds__(256)
+dequant_mxfp4_f16(const uchar* __restrict__ w, ushort* __restrict__ out, uint nblocks) {
+    const size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x;
+    const size_t b = tid >> 4;
+    if (b >= nblocks) return;
+    const uint j = (uint)tid & 15u;
+    const uchar* blk = w + b * 17u;
+    const float d = __uint_as_float((uint)blk[0] << 23);
+    const uint q = blk[1u + j];
+    float v[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const uint c = h ? q >> 4 : q & 15u, m = c & 7u;
+        const float a = 0.5f * (float)(m < 5u ? m : m == 5u ? 6u : m == 6u ? 8u : 12u);
+        v[h] = __fmul_rn(d, __uint_as_float(__float_as_uint(a) | ((c >> 3) << 31)));
+    }
+    *(uint*)(out + b * 32u + 2u * j) = (uint)f32_to_f16_bits(v[0]) | ((uint)f32_to_f16_bits(v[1]) << 16);
+}

@@ -419,13 +419,14 @@ __device__ __forceinline__ void gemv_nat_q80_m_body(const float* __restrict__ x,
 }
 
 // ------------------------------------------------------------------ IQ4_NL, IQ4_XS and the legacy 32-weight blocks
-// (row traits Iq4nlW, Iq4xsW, Q40W, Q41W, Q50W, Q51W: ojk_rows.h)
+// (row traits Iq4nlW, Iq4xsW, Q40W, Q41W, Q50W, Q51W, Mxfp4W: ojk_rows.h)
 GEMV_NAT_IQ4_PX(iq4nl, Iq4nlW)
 GEMV_NAT_IQ4_PX(iq4xs, Iq4xsW)
 GEMV_NAT_IQ4_PX(q40, Q40W)
 GEMV_NAT_IQ4_PX(q41, Q41W)
 GEMV_NAT_IQ4_PX(q50, Q50W)
 GEMV_NAT_IQ4_PX(q51, Q51W)
+GEMV_NAT_IQ4_PX(mxfp4, Mxfp4W)
 GEMV_NAT_IQ4_PX(q5k, Q5kW)
 
 template <int R, int MODE>
@@ -459,6 +460,14 @@ __device__ __forceinline__ void gemv_nat_q50_body(const float* x, const uchar* w
 template <int MT>
 __device__ __forceinline__ void gemv_nat_q50_m_body(const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
     gemv_nat_iq4_m_body<Q50W, MT>(x, w, y, K, N, M, ACC);
+}
+template <int R, int MODE>
+__device__ __forceinline__ void gemv_nat_mxfp4_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
+    gemv_nat_iq4_body<Mxfp4W, R, MODE>(x, w, y, bs, K, N);
+}
+template <int MT>
+__device__ __forceinline__ void gemv_nat_mxfp4_m_body(const float* x, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) {
+    gemv_nat_iq4_m_body<Mxfp4W, MT>(x, w, y, K, N, M, ACC);
 }
 template <int R, int MODE>
 __device__ __forceinline__ void gemv_nat_q51_body(const float* x, const uchar* w, float* y, const float* bs, uint K, uint N) {
@@ -805,6 +814,7 @@ GEMV_NAT_ENTRIES(q40)
 GEMV_NAT_ENTRIES(q41)
 GEMV_NAT_ENTRIES(q50)
 GEMV_NAT_ENTRIES(q51)
+GEMV_NAT_ENTRIES(mxfp4)
 GEMV_NAT_ENTRIES(q2k)
 GEMV_NAT_ENTRIES(q3k)
 GEMV_NAT_ENTRIES(q5k)

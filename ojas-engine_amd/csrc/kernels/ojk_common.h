@@ -27,6 +27,8 @@ typedef unsigned short ushort;
 struct __attribute__((packed, aligned(2))) u32x4_a2 { uint x, y, z, w; };
 struct __attribute__((packed, aligned(2))) u32x2_a2 { uint x, y; };
 typedef uint __attribute__((aligned(2))) u32_a2;
+typedef uint __attribute__((aligned(1))) u32_a1;
+#define MXFP4_BYTES 17u
 
 // Scale i (0 .. 15) of a Q3_K block from its three packed words (crates/ojas-formats/src/gguf.rs:764-774):
 // the low nibble sits in byte i (i < 8) or in the high nibble of byte i - 8, the two high bits in byte

@@ -243,3 +243,46 @@ struct Q6kW {
         return f16_bits_to_f32(f.d) * (a + b);
     }
 };
+
+// ------------------------------------------------------------------ MXFP4
+// The reference's native MXFP4 block (crates/ojas-core/src/quant_src.rs:333-353): { u8 e; u8 qs[16] }, 17 bytes per 32
+// weights, w = 2^(e - 127) * E2M1[code], weight 2j the low and 2j + 1 the high nibble of qs[j].  Four lanes per
+// block: a lane's dword of codes is eight consecutive weights.  The E2M1 magnitudes are halves of {0, 1, 2, 3, 4, 6,
+// 8, 12} — one byte permute — and a code's bit 3 is the sign; the scale, a power of two, meets the lane's sum once.
+// Blocks sit at odd addresses: every load is byte-aligned.
+struct Mxfp4W {
+    static constexpr uint XGAP = 4u;
+    static constexpr uint STEP = 16u;
+    static constexpr uint BYTES = MXFP4_BYTES;
+    static __device__ __forceinline__ uint units(uint K) { return K >> 5; }
+    static __device__ __forceinline__ uint unit_of(uint lane) { return lane >> 2; }
+    static __device__ __forceinline__ uint x_off(uint lane) { return (lane & 3u) * 8u; }
+    static __device__ __forceinline__ uint x_unit(uint) { return 32u; }
+    struct Frag { uint e, q; };
+    static __device__ __forceinline__ Frag load(const uchar* row, uint u, uint lane) {
+        const uchar* blk = row + (size_t)u * MXFP4_BYTES;
+        Frag f;
+        f.e = blk[0];
+        f.q = *(const u32_a1*)(blk + 1u + (lane & 3u) * 4u);
+        return f;
+    }
+    // twice the magnitudes of four codes (one per byte, bits 0 .. 2), and the codes' sign bits moved to bit 31
+    static __device__ __forceinline__ uint mags4(uint n) { return __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, n & 0x07070707u); }
+    static __device__ __forceinline__ float val(uint m, uint n, uint byte) {
+        const float a = (float)((m >> (8u * byte)) & 0xFFu);
+        return __uint_as_float(__float_as_uint(a) | (((n >> (8u * byte + 3u)) & 1u) << 31));
+    }
+    static __device__ __forceinline__ float dot(const Frag& f, uint, float4 x0, float4 x1, float) {
+        const uint lo = f.q & 0x0F0F0F0Fu, hi = (f.q >> 4) & 0x0F0F0F0Fu;      // weights 0, 2, 4, 6 and 1, 3, 5, 7 of the eight
+        const uint ml = mags4(lo), mh = mags4(hi);
+        float a = val(ml, lo, 0) * x0.x;
+        a = fmaf(val(mh, hi, 0), x0.y, a);
+        a = fmaf(val(ml, lo, 1), x0.z, a);
+        a = fmaf(val(mh, hi, 1), x0.w, a);
+        a = fmaf(val(ml, lo, 2), x1.x, a);
+        a = fmaf(val(mh, hi, 2), x1.y, a);
+        a = fmaf(val(ml, lo, 3), x1.z, a);
+        a = fmaf(val(mh, hi, 3), x1.w, a);
+        return __uint_as_float(f.e << 23) * (0.5f * a);
+    }
+};

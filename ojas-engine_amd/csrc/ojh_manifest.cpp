@@ -29,6 +29,7 @@ static const ojh_block_format kFormats[] = {
     {OJH_IQ3_S, 110, 256, "iq3s"},
     {OJH_IQ1_S, 50, 256, "iq1s"},
     {OJH_IQ1_M, 56, 256, "iq1m"},
+    {OJH_MXFP4, 17, 32, "mxfp4"},
 };
 
 // Formats whose CPU path multiplies the raw row with f32 activations (dot_q80, dot_iq4nl, dot_iq4xs:
@@ -42,7 +43,7 @@ bool ojh_float_rows(uint32_t t) { return t == OJH_Q8_0 || ojh_float_only(t); }
 bool ojh_float_only(uint32_t t) {
     return t == OJH_IQ4_NL || t == OJH_IQ4_XS || t == OJH_Q4_0 || t == OJH_Q4_1 || t == OJH_Q5_0 || t == OJH_Q5_1 ||
            t == OJH_Q2_K || t == OJH_Q3_K || t == OJH_IQ3_S || t == OJH_IQ2_S || t == OJH_IQ2_XS || t == OJH_IQ1_S ||
-           t == OJH_IQ1_M;
+           t == OJH_IQ1_M || t == OJH_MXFP4;
 }
 bool ojh_grid_type(uint32_t t) {
     return t == OJH_IQ2_XXS || t == OJH_IQ2_XS || t == OJH_IQ2_S || t == OJH_IQ3_XXS || t == OJH_IQ3_S || t == OJH_IQ1_S ||
@@ -52,7 +53,7 @@ bool ojh_grid_type(uint32_t t) {
 // What the kernels' loads need of a block tensor's address: the widest power of two (up to 16) dividing the
 // block size, except that only Q2_K's kernels use the 4 of a block size that is 4 mod 8.
 size_t ojh_block_align(const ojh_block_format *f) {
-    return f->bytes % 16 == 0 ? 16 : f->bytes % 8 == 0 ? 8 : f->type == OJH_Q2_K ? 4 : 2;
+    return f->bytes % 16 == 0 ? 16 : f->bytes % 8 == 0 ? 8 : f->type == OJH_Q2_K ? 4 : f->bytes % 2 == 0 ? 2 : 1;
 }
 
 const ojh_block_format *ojh_format(uint32_t t) {
@@ -764,7 +765,7 @@ static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint
     if (!f || nb == 0) return ojh_fail(OJH_ERR_ARG, "%s: nblocks must be positive", s->name);
     int rc = check_block(block, 256);
     if (rc) return rc;
-    uint32_t tpb = s->type == OJH_Q6_K ? 64 : 32;  // threads per block of the format
+    uint32_t tpb = s->type == OJH_Q6_K ? 64 : s->type == OJH_MXFP4 ? 16 : 32;  // threads per block of the format
     if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * 256 < (uint64_t)nb * tpb)
         return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover %u blocks", s->name, nb);
     need[0] = (size_t)nb * f->bytes;
@@ -1350,7 +1351,7 @@ static int shape_quantize(const ojh_kernel_spec *, const ojh_device *, uint32_t 
 // dequant: N is the number of blocks
 static int shape_dequant(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t,
                          uint32_t grid[3], uint32_t block[3]) {
-    uint32_t tpb = s->type == OJH_Q6_K ? 64 : 32;
+    uint32_t tpb = s->type == OJH_Q6_K ? 64 : s->type == OJH_MXFP4 ? 16 : 32;
     grid[0] = (uint32_t)(((uint64_t)N * tpb + 255) / 256);
     grid[1] = grid[2] = 1;
     block[0] = 256;

@@ -26,13 +26,14 @@ Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 Q2_K, Q3_K = 10, 11
 IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M = 16, 17, 18, 19, 21, 22, 29
 GRID_TYPES = (IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M)
+MXFP4 = 139     # the reference's synthetic id for its 17-byte MXFP4 blocks (a safetensors format, not a GGUF type)
 X_F32, X_BF16, X_F16 = 0, 1, 2
 ACT_AUTO, ACT_Q8K, ACT_FLOAT, ACT_FLOAT_EXACT, ACT_Q8_1 = 0, 1, 2, 3, 4
 
 BLOCK_SHAPE = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256), IQ4_NL: (18, 32), IQ4_XS: (136, 256),
                Q4_0: (18, 32), Q4_1: (20, 32), Q5_0: (22, 32), Q5_1: (24, 32), Q2_K: (84, 256), Q3_K: (110, 256),
                IQ2_XXS: (66, 256), IQ2_XS: (74, 256), IQ3_XXS: (98, 256), IQ1_S: (50, 256), IQ3_S: (110, 256), IQ2_S: (82, 256),
-               IQ1_M: (56, 256)}
+               IQ1_M: (56, 256), MXFP4: (17, 32)}
 
 
 class OjasHipError(RuntimeError):

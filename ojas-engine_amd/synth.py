@@ -17,10 +17,11 @@ Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 Q2_K, Q3_K = 10, 11
 IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M = 16, 17, 18, 19, 21, 22, 29
 GRID_TYPES = (IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M)
+MXFP4 = 139     # the reference's synthetic id for its 17-byte MXFP4 blocks (a safetensors format, not a GGUF type)
 BLOCK_SHAPE = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256), IQ4_NL: (18, 32), IQ4_XS: (136, 256),
                Q4_0: (18, 32), Q4_1: (20, 32), Q5_0: (22, 32), Q5_1: (24, 32), Q2_K: (84, 256), Q3_K: (110, 256),
                IQ2_XXS: (66, 256), IQ2_XS: (74, 256), IQ3_XXS: (98, 256), IQ1_S: (50, 256), IQ3_S: (110, 256), IQ2_S: (82, 256),
-               IQ1_M: (56, 256)}
+               IQ1_M: (56, 256), MXFP4: (17, 32)}
 
 
 def seed_of(*names) -> int:
@@ -193,8 +194,19 @@ def weights(ty: int, n: int, k: int, *names) -> np.ndarray:
         return {Q2_K: q2k_weights, Q3_K: q3k_weights}[ty](n, k, *names)
     if ty in GRID_TYPES:
         return grid_weights(ty, n, k, *names)
+    if ty == MXFP4:
+        return mxfp4_weights(n, k, *names)
     return {Q8_0: q80_weights, Q4_K: q4k_weights, Q5_K: q5k_weights, Q6_K: q6k_weights,
             IQ4_NL: iq4nl_weights, IQ4_XS: iq4xs_weights}[ty](n, k, *names)
+
+
+def mxfp4_weights(n: int, k: int, *names) -> np.ndarray:
+    """MXFP4 rows: 17-byte blocks, an e8m0 scale exponent uniform in 112..124 (2^-15 .. 2^-3), 16 bytes of E2M1 codes uniform."""
+    g = rng("mxfp4", n, k, *names)
+    nb = n * (k // 32)
+    out = g.integers(0, 256, size=(nb, 17), dtype=np.uint8)
+    out[:, 0] = g.integers(112, 125, nb, dtype=np.uint8)
+    return out.reshape(-1)
 
 
 def grid_weights(ty: int, n: int, k: int, *names) -> np.ndarray:
@@ -242,6 +254,8 @@ def synth_blocks(ty: int, nb: int) -> np.ndarray:
             blocks[i, 82], blocks[i, 83] = int(dmin) & 0xFF, int(dmin) >> 8
         elif ty == Q3_K:
             blocks[i, 108], blocks[i, 109] = d & 0xFF, d >> 8
+        elif ty == MXFP4:      # (not a synth.rs type) an e8m0 exponent near 1.0 in byte 0
+            blocks[i, 0] = 120 + i % 7
         elif ty == IQ1_M:      # no d field: f16(0.05) in the top nibbles of the four scale words, low nibble first
             db = int(np.array([0.05], np.float32).astype(np.float16).view(np.uint16)[0])
             for w in range(4):

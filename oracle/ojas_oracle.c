@@ -108,6 +108,7 @@ int ojo_block_shape(uint32_t ty, uint32_t *bytes, uint32_t *weights) { /* synth.
     case OJO_Q5_0: b = 22; w = 32; break;
     case OJO_Q5_1: b = 24; w = 32; break;
     case OJO_IQ4_XS: b = 136; w = 256; break;
+    case OJO_MXFP4: b = 17; w = 32; break;
     case OJO_IQ2_XXS: b = 66; w = 256; break;
     case OJO_IQ2_XS: b = 74; w = 256; break;
     case OJO_IQ3_XXS: b = 98; w = 256; break;
@@ -148,6 +149,9 @@ int ojo_synth_blocks(uint32_t ty, size_t nb, uint8_t *out) { /* synth.rs:29-64 *
             break;
         case OJO_Q3_K:
             blk[108] = (uint8_t)d; blk[109] = (uint8_t)(d >> 8);
+            break;
+        case OJO_MXFP4: /* not a synth.rs type: an e8m0 exponent near 1.0 in byte 0 keeps the values finite */
+            blk[0] = (uint8_t)(120 + i % 7);
             break;
         case OJO_IQ1_M: { /* no d field: f16(0.05) spread over the top nibbles of the four scale words, low nibble first */
             uint16_t db = ojo_f32_to_f16(0.05f);
@@ -205,6 +209,14 @@ int ojo_dequant_to_f16(const uint8_t *b, uint32_t ty, size_t n, uint16_t *out) {
         const uint8_t *blk = b + ib * bb;
         uint16_t *o = out + ib * wpb;
         switch (ty) {
+        case OJO_MXFP4: { /* crates/ojas-formats/src/mxfp4.rs:40-58: weight 2j = low nibble of qs[j], 2j+1 = high; d = 2^(e-127) */
+            static const float lut[16] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f, -0.0f, -0.5f, -1.0f, -1.5f, -2.0f, -3.0f, -4.0f, -6.0f};
+            union { uint32_t u; float f; } d = { (uint32_t)blk[0] << 23 };
+            for (int j = 0; j < 16; j++) {
+                o[2 * j] = ojo_f32_to_f16(d.f * lut[blk[1 + j] & 0xF]);
+                o[2 * j + 1] = ojo_f32_to_f16(d.f * lut[blk[1 + j] >> 4]);
+            }
+        } break;
         case OJO_Q8_0: { /* gguf.rs:704-709 */
             float d = rdh(blk, 0);
             for (int j = 0; j < 32; j++) o[j] = ojo_f32_to_f16(d * (float)(int8_t)blk[2 + j]);
@@ -370,6 +382,14 @@ int ojo_dequant_to_f64(const uint8_t *b, uint32_t ty, size_t n, double *out) {
         const uint8_t *blk = b + ib * bb;
         double *o = out + ib * wpb;
         switch (ty) {
+        case OJO_MXFP4: {
+            static const double lut[16] = {0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0};
+            union { uint32_t u; float f; } d = { (uint32_t)blk[0] << 23 };
+            for (int j = 0; j < 16; j++) {
+                o[2 * j] = (double)d.f * lut[blk[1 + j] & 0xF];
+                o[2 * j + 1] = (double)d.f * lut[blk[1 + j] >> 4];
+            }
+        } break;
         case OJO_Q8_0: {
             double d = rdh(blk, 0);
             for (int j = 0; j < 32; j++) o[j] = d * (double)(int8_t)blk[2 + j];

@@ -21,6 +21,8 @@
  *   dequant IQ2_XXS/IQ2_XS/IQ2_S/IQ3_XXS/IQ3_S/IQ1_S/IQ1_M   (ojas_oracle_iq.c) the digests of the same table
  *                           (quant_formats.rs:41-44,46-47,49), closed forms on hand-built blocks; the packed codebooks
  *                           by a digest of every published table (tests/golden/iq_grid_digests.json)
+ *   dequant MXFP4           the hand-computed blocks of crates/ojas-core/src/quant_src.rs:1376-1420 and
+ *                           crates/ojas-formats/src/mxfp4.rs:127-160 (codebook sweep, scales 2^2 and 2^-1, e8m0 table)
  *   dot_q80                 f64 dot over the dequantized row, brute force at K=32
  *   dot_iq2xxs/iq3xxs/iq2s/iq3s   f64 dot over the exactly decoded row, one-hot activations
  *   dot_iq2xxs_q8k/iq3xxs_q8k     identity dot(row, quant(x)) == sum xs * sum w * q in f64
@@ -45,6 +47,7 @@ extern "C" {
 /* GGUF type ids (crates/ojas-formats/src/gguf.rs:563-591). */
 enum { OJO_Q4_0 = 2, OJO_Q4_1 = 3, OJO_Q5_0 = 6, OJO_Q5_1 = 7, OJO_Q8_0 = 8, OJO_Q2_K = 10, OJO_Q3_K = 11, OJO_Q4_K = 12, OJO_Q5_K = 13, OJO_Q6_K = 14,
        OJO_IQ4_NL = 20, OJO_IQ4_XS = 23,
+       OJO_MXFP4 = 139, /* the reference's synthetic id for 17-byte MXFP4 blocks (crates/ojas-core/src/quant_src.rs:91-95) */
        OJO_IQ2_XXS = 16, OJO_IQ2_XS = 17, OJO_IQ3_XXS = 18, OJO_IQ1_S = 19, OJO_IQ3_S = 21, OJO_IQ2_S = 22, OJO_IQ1_M = 29 };
 
 /* IEEE binary16 <-> binary32, round-to-nearest-even, subnormals kept

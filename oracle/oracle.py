@@ -17,6 +17,7 @@ _LIB_PATH = os.path.join(_HERE, "libojas_oracle.so")
 
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M = 16, 17, 18, 19, 21, 22, 29
+MXFP4 = 139
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 Q2_K, Q3_K = 10, 11
 

@@ -167,12 +167,12 @@ IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M = 16, 17, 18, 19, 21, 22, 2
 
 
 @pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K,
-                                IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M])
+                                IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M, 139])
 @pytest.mark.parametrize("mode", ["float", "q8k"])
 def test_bias_accum_and_batched_variants(gpu, orc, pkg, ty, mode):
     """The five checks of crates/ojas-models/examples/nat_gemv_gate.rs:36-163: plain, bias
     (1000 + i), accumulate onto a seeded y, batched M=3 with different rows, batched accumulate."""
-    if ty in (Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, IQ2_XS, IQ1_S, IQ3_S, IQ2_S, IQ1_M) and mode == "q8k":
+    if ty in (Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, IQ2_XS, IQ1_S, IQ3_S, IQ2_S, IQ1_M, 139) and mode == "q8k":
         pytest.skip("this format keeps f32 activations in the CPU reference")
     n, k, m = 200, 1024, 3
     w = pkg.synth.weights(ty, n, k, "var", ty)

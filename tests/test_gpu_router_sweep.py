@@ -13,8 +13,9 @@ Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 8, 12, 13, 14, 20, 23
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 Q2_K, Q3_K = 10, 11
 IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M = 16, 17, 18, 19, 21, 22, 29
-FLOAT_ROWS = (Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, IQ3_S, IQ2_S, IQ2_XS, IQ1_S, IQ1_M)
-LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, IQ2_XS, IQ1_S, IQ1_M)   # no dot in the CPU path: GPU-path formats
+MXFP4 = 139
+FLOAT_ROWS = (Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, IQ3_S, IQ2_S, IQ2_XS, IQ1_S, IQ1_M, MXFP4)
+LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, IQ2_XS, IQ1_S, IQ1_M, MXFP4)   # no dot in the CPU path: GPU-path formats
 
 
 def _cases():
@@ -23,7 +24,7 @@ def _cases():
     ks = [256, 512, 1024, 2560, 4096, 5120, 7168, 14336]
     out = []
     for ty in (Q4_K, Q6_K, Q5_K, Q8_0, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K,
-               IQ2_XXS, IQ3_XXS, IQ3_S, IQ2_S, IQ2_XS, IQ1_S, IQ1_M):     # (new formats go last: the draws before them stay)
+               IQ2_XXS, IQ3_XXS, IQ3_S, IQ2_S, IQ2_XS, IQ1_S, IQ1_M, MXFP4):     # (new formats go last: the draws before them stay)
         for _ in range(7 if ty not in LEGACY and ty not in (IQ3_S, IQ2_S) else 3):
             n, k = int(g.choice(rows)), int(g.choice(ks))
             m = int(g.choice([1, 2, 3, 4, 5, 7, 8, 9, 16, 17, 33, 40]))

@@ -32,7 +32,7 @@ def test_dequant_digest_matches_reference(orc, pkg, ty):
     assert orc.digest_f16(bits) == DIGESTS[ty]
 
 
-@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K] + GRID_TYPES)
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, 139] + GRID_TYPES)
 def test_synth_blocks_two_implementations_agree(orc, pkg, ty):
     assert np.array_equal(orc.synth_blocks(ty, 9), pkg.synth.synth_blocks(ty, 9))
 
@@ -711,3 +711,31 @@ def test_grid_format_f32_dots(orc, pkg, ty):
         assert np.max(np.abs(q8 - ident)) <= 2e-6 * np.max(np.abs(ident))
         assert np.array_equal(mv, q8.astype(np.float32))
         assert np.max(np.abs(q8 - want)) <= 2e-2 * np.max(np.abs(want))      # activation quantization only
+
+
+def test_mxfp4_hand_computed_blocks(orc):
+    """The reference's own known answers for its 17-byte MXFP4 block (crates/ojas-core/src/quant_src.rs:1376-1420,
+    crates/ojas-formats/src/mxfp4.rs:127-160): a codebook sweep at scale 1, code 5 / 13 at scale 2^2, code 2 at 2^-1, and
+    the e8m0 table (127 -> 1, 128 -> 2, 126 -> 0.5, 120 -> 2^-7, 0 -> 0); weight 2j is the low nibble of qs[j]."""
+    MXFP4 = 139
+    a = np.zeros(17, np.uint8)
+    a[0] = 127
+    a[1:9] = [0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]
+    wa = orc.dequant_to_f64(a, MXFP4, 32)
+    want = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0])
+    assert np.array_equal(wa[:16], want) and np.array_equal(np.signbit(wa[:16]), np.signbit(want)) and np.all(wa[16:] == 0.0)
+    b = np.full(17, 0xD5, np.uint8)
+    b[0] = 129
+    wb = orc.dequant_to_f64(b, MXFP4, 32)
+    assert np.all(wb[0::2] == 12.0) and np.all(wb[1::2] == -12.0)
+    c = np.zeros(17, np.uint8)
+    c[0], c[1] = 126, 0x22
+    wc = orc.dequant_to_f64(c, MXFP4, 32)
+    assert wc[0] == 0.5 and wc[1] == 0.5 and np.all(wc[2:] == 0.0)
+    for e, v in [(127, 1.0), (128, 2.0), (129, 4.0), (126, 0.5), (120, 2.0 ** -7), (0, 0.0)]:
+        blk = np.full(17, 0x22, np.uint8)
+        blk[0] = e
+        assert np.all(orc.dequant_to_f64(blk, MXFP4, 32) == v), e
+    # the f16 decoder is the same value rounded once
+    raw = orc.synth_blocks(MXFP4, 64)
+    assert np.array_equal(orc.dequant_to_f16(raw, MXFP4, 64 * 32), orc.dequant_to_f64(raw, MXFP4, 64 * 32).astype(np.float16).view(np.uint16))
