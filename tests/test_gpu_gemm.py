@@ -172,6 +172,33 @@ def test_split_k_slices_meeting_in_scratch(gpu, orc, pkg, kernel, bm):
                      [(n + 255) // 256, (m + bm - 1) // bm, 2], [256, 1, 1])
 
 
+def test_mm_with_reproducible_split_k(gpu, orc, pkg, monkeypatch):
+    """A device handle opened under OJAS_HIP_GEMM_SR=1 routes the split-K launches of `mm` to the `_sr` entries: the
+    same result to the order of the f32 sums as the default handle's atomics, and the same bits on every run."""
+    m, k, n = 128, 4096, 1536          # 6 tiles of 256 rows: split into K slices on any GPU with more than 6 CUs
+    w = pkg.synth.q4k_weights(n, k, "gemmsr", "mm")
+    xb = pkg.synth.to_bf16_bits(pkg.synth.normal_f32(m * k, "gemmsr", "mmx"))
+    gpu.ensure_family("gemm_xl")
+    assert gpu.launch_shape("gemm_mm_q4kl_bd_sk", k, n, m)[0][2] > 1
+    yd = gpu.alloc(m * n)
+    gpu.mm(gpu.upload_bytes(xb), gpu.lin(12, n, k, w), yd, m, x_dtype=pkg.X_BF16, act_mode=pkg.ACT_FLOAT)
+    base = gpu.read(yd, m * n)
+    monkeypatch.setenv("OJAS_HIP_GEMM_SR", "1")
+    g2 = pkg.HipGpu(0)
+    try:
+        lin, xd = g2.lin(12, n, k, w), g2.upload_bytes(xb)
+        runs = []
+        for accum in (False, False, True):
+            y2 = g2.upload(np.full(m * n, 3.0, np.float32))
+            g2.mm(xd, lin, y2, m, accum, x_dtype=pkg.X_BF16, act_mode=pkg.ACT_FLOAT)
+            runs.append(g2.read(y2, m * n))
+        assert np.array_equal(runs[0], runs[1])
+        assert peak_err(runs[0], base) <= 2e-6
+        assert peak_err(runs[2] - 3.0, base) <= 1e-5
+    finally:
+        g2.close()
+
+
 @pytest.mark.parametrize("m,k,n", [(140, 2048, 300), (128, 256, 256), (77, 512, 64), (260, 1024, 513)])
 def test_tile_with_weights_dequantized_into_registers(gpu, orc, pkg, m, k, n):
     """`gemm_mm_q4kl_bd` and `gemm_mm_q4kl_bd256` by name: the 128 x 256 and 256 x 256 tiles whose waves dequantize their own
