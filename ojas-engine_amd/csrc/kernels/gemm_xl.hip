@@ -380,14 +380,22 @@ struct GbRow {
 // SPLITK: 0 the whole K; 1 K slices that add into y with f32 atomics (y zeroed or holding the sum to extend: the
 // reference's `_sk` contract, crates/ojas-cuda/src/kernels/gemm_q.rs:26-38); 2 K slices that leave their partial tiles
 // in `part` and count themselves in `cnt`, the last one to arrive adding the slices in order and storing y (`_sr`).
-template <int SPLITK, bool ACCUM, int MI>
+// KW: the workgroup's four waves share 64 weight rows and split K between them instead (a quarter of the slice's
+// super-blocks each, met in LDS at the end, in wave order): 64-row tiles for shapes whose 256-row tiles are too few to
+// fill the chip.  Every wave then runs a pipeline of its own — its own activation stages, no barrier inside the loop.
+template <int SPLITK, bool ACCUM, int MI, bool KW = false>
 __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, const uchar* __restrict__ w,
                                              float* __restrict__ y, uint K, uint N, uint M, uint nsplit, uchar* lds,
                                              float* __restrict__ part = nullptr, uint* __restrict__ cnt = nullptr,
                                              uint acc_y = 0u) {
+    static_assert(!KW || (MI == 4 && SPLITK != 2), "the K-over-waves form: 128 tokens, plain or atomic stores");
+    constexpr uint XS = GB_XSTAGE(MI);
+    constexpr uint NX = KW ? 4u * MI : (uint)MI;                 // activation copies a wave issues per step
+    constexpr uint NSLOT = KW ? 3u : 4u, HSLOT = KW ? 1u : 2u;   // nibble / header slots (KW: 160 KB of LDS in all)
+    constexpr uint NIB0 = KW ? 8u * XS : GB_NIB(MI), HDR0 = NIB0 + NSLOT * 8192u;
     const uint tid = threadIdx.x, lane = tid & 63u;
     const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint n0 = blockIdx.x * GX_BN, m0 = blockIdx.y * (32u * MI);
+    const uint n0 = blockIdx.x * (KW ? 64u : GX_BN), m0 = blockIdx.y * (32u * MI);
     const uint nsb = K >> 8;
     uint sb_begin = 0, sb_end = nsb;
     if (SPLITK != 0) {
@@ -396,29 +404,38 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
         sb_end = min((blockIdx.z + 1) * per, nsb);
         if (sb_begin >= sb_end) return;
     }
-    const uint nt = (sb_end - sb_begin) * 4u, last = nt - 1u;
+    if (KW) {
+        const uint per4 = (sb_end - sb_begin + 3u) / 4u;
+        sb_begin = min(sb_begin + wave * per4, sb_end);
+        sb_end = min(sb_begin + per4, sb_end);
+    }
+    const uint nt = (sb_end - sb_begin) * 4u, last = nt - 1u;       // (KW: a wave may be left without a share, nt = 0)
     const uint k_begin = sb_begin << 8;
     const uint lds0 = (uint)(size_t)(__attribute__((address_space(3))) uchar*)lds;
 
     // activation stage: wave `wave`, copy i moves rows (wave*MI + i)*8 .. +7; lane -> row lane/8, slot lane%8, which
     // holds source chunk (lane%8) ^ ((row/2)%8)
-    uint xoff[MI];
+    // (KW: every wave copies all 32 MI rows into stages of its own)
+    uint xoff[NX];
 #pragma unroll
-    for (int i = 0; i < MI; i++) {
-        const uint r = (wave * (uint)MI + i) * 8u + (lane >> 3);
+    for (uint i = 0; i < NX; i++) {
+        const uint r = ((KW ? 0u : wave * (uint)MI) + i) * 8u + (lane >> 3);
         const uint m = min(m0 + r, M - 1u);
         xoff[i] = m * K * 2u + (((lane & 7u) ^ ((r >> 1) & 7u)) << 4);
     }
-    const uint x_lds = lds0 + wave * ((uint)MI * 1024u);         // + stage * GB_XSTAGE + i * 1024
+    const uint x_lds = KW ? lds0 + wave * 2u * XS : lds0 + wave * ((uint)MI * 1024u);   // + stage * XS + i * 1024
     // the lane's two weight rows: B column fr of blocks j = 0, 1; its 16 nibble bytes are bytes 16 g .. of a chunk
     const uint fr = lane & 31u, kg = lane >> 5, sw = (fr >> 1) & 7u;
     const uint row_bytes = nsb * Q4K_BYTES;
-    const uint ro0 = min(n0 + wave * 64u + fr, N - 1u) * row_bytes, ro1 = min(n0 + wave * 64u + 32u + fr, N - 1u) * row_bytes;
-    const uint nib_lds = lds0 + GB_NIB(MI) + wave * 2048u;           // + slot * 8192 + j * 1024
-    const uint hdr_lds = lds0 + GB_HDR(MI) + wave * 2048u;           // + slot * 8192 + j * 1024
-    const uchar* const nib_rd = lds + GB_NIB(MI) + wave * 2048u + lane * 16u;
-    const uchar* const hdr_rd = lds + GB_HDR(MI) + wave * 2048u + lane * 16u;
-    const uchar* const a_rd = lds + fr * GX_ROW;                 // + stage * GB_XSTAGE + i * 32 rows + chunk slot
+    const uint nw = n0 + (KW ? 0u : wave * 64u);
+    const uint ro0 = min(nw + fr, N - 1u) * row_bytes, ro1 = min(nw + 32u + fr, N - 1u) * row_bytes;
+    const uint nib_lds = lds0 + NIB0 + wave * 2048u;           // + slot * 8192 + j * 1024
+    const uint hdr_lds = lds0 + HDR0 + wave * 2048u;           // + slot * 8192 + j * 1024
+    const uchar* const nib_rd = lds + NIB0 + wave * 2048u + lane * 16u;
+    const uchar* const hdr_rd = lds + HDR0 + wave * 2048u + lane * 16u;
+    const uchar* const a_rd = lds + (KW ? wave * 2u * XS : 0u) + fr * GX_ROW;   // + stage * XS + i * 32 rows + chunk slot
+    // nibble slot of step t: t mod 4, or t mod 3 (t < 2^16: K < 2^22)
+    auto nslot = [](uint t) -> uint { return NSLOT == 4u ? t & 3u : t - 3u * ((t * 0xAAABu) >> 17); };
 
     float16v acc[MI][2];
 #pragma unroll
@@ -435,35 +452,35 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
     auto copy_x = [&](uint t) {
         const uchar* b = xbase + (size_t)(k_begin + min(t, last) * GX_BK) * 2u;
 #pragma unroll
-        for (int i = 0; i < MI; i++) gx_load_lds16(b, xoff[i], x_lds + (t & 1u) * GB_XSTAGE(MI) + i * 1024u);
+        for (uint i = 0; i < NX; i++) gx_load_lds16(b, xoff[i], x_lds + (t & 1u) * XS + i * 1024u);
     };
     auto copy_nib = [&](uint t) {
         const uint tc = min(t, last);
         const uchar* bn = w + (size_t)(sb_begin + (tc >> 2)) * Q4K_BYTES + 16u + (tc & 3u) * 32u;
-        gx_load_lds16(bn, ro0 + 16u * kg, nib_lds + (t & 3u) * 8192u);
-        gx_load_lds16(bn, ro1 + 16u * kg, nib_lds + (t & 3u) * 8192u + 1024u);
+        gx_load_lds16(bn, ro0 + 16u * kg, nib_lds + nslot(t) * 8192u);
+        gx_load_lds16(bn, ro1 + 16u * kg, nib_lds + nslot(t) * 8192u + 1024u);
     };
     auto copy_hdr = [&](uint t) {               // the header of step t's super-block (a slot per super-block parity)
         const uint tc = min(t, last);
         const uchar* bh = w + (size_t)(sb_begin + (tc >> 2)) * Q4K_BYTES;
-        gx_load_lds16(bh, ro0, hdr_lds + ((tc >> 2) & 1u) * 8192u);
-        gx_load_lds16(bh, ro1, hdr_lds + ((tc >> 2) & 1u) * 8192u + 1024u);
+        gx_load_lds16(bh, ro0, hdr_lds + (HSLOT == 2u ? (tc >> 2) & 1u : 0u) * 8192u);
+        gx_load_lds16(bh, ro1, hdr_lds + (HSLOT == 2u ? (tc >> 2) & 1u : 0u) * 8192u + 1024u);
     };
     GbRow r0, r1;
     half8 afA[MI], afB[MI], b0, b1, c0, c1;
 #define GB_READ_A(T, CH, AF)                                                                           \
     do {                                                                                               \
-        const uchar* xa_ = a_rd + ((T) & 1u) * GB_XSTAGE(MI) + ((((CH) + 2u * kg) ^ sw) << 4);         \
+        const uchar* xa_ = a_rd + ((T) & 1u) * XS + ((((CH) + 2u * kg) ^ sw) << 4);                    \
         _Pragma("unroll") for (int i = 0; i < MI; i++) AF[i] = *(const half8*)(xa_ + i * 32u * GX_ROW); \
     } while (0)
 // the raw rows of step T out of their slots (the header only where T starts a super-block), scales of chunk C1
 #define GB_READ_W(T, C1, HDR)                                                                          \
     do {                                                                                               \
-        const uint slot_ = ((T) & 3u) * 8192u;                                                         \
+        const uint slot_ = nslot(T) * 8192u;                                                           \
         r0.q = *(const u32x4*)(nib_rd + slot_);                                                        \
         r1.q = *(const u32x4*)(nib_rd + slot_ + 1024u);                                                \
         if (HDR) {                                                                                     \
-            const uint hs_ = ((min((T), last) >> 2) & 1u) * 8192u;                                     \
+            const uint hs_ = (HSLOT == 2u ? (min((T), last) >> 2) & 1u : 0u) * 8192u;                  \
             r0.hdr = *(const u32x4*)(hdr_rd + hs_);                                                    \
             r1.hdr = *(const u32x4*)(hdr_rd + hs_ + 1024u);                                            \
         }                                                                                              \
@@ -509,7 +526,7 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
         GB_MIX(5);                                                                                     \
         __builtin_amdgcn_sched_barrier(0);                                                             \
         gx_wait<(C) == 2 ? 4 : 2>();                                                                   \
-        __syncthreads();                                                                               \
+        if (!KW) __syncthreads();                                                                      \
         copy_x((T) + 2u);                                                                              \
         copy_nib((T) + 3u);                                                                            \
         if ((C) == 1) copy_hdr((T) + 3u);                                                              \
@@ -525,25 +542,27 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
         }                                                                                              \
     } while (0)
     // prologue: the state a step expects on entry
-    copy_nib(0u);
-    copy_hdr(0u);
-    copy_nib(1u);
-    copy_x(0u);
-    gx_wait<0>();
-    __syncthreads();
-    GB_READ_A(0u, 0u, afA);
-    GB_READ_W(0u, 0, true);
-    b0 = r0.frag<0>(magic);
-    b1 = r1.frag<0>(magic);
-    copy_x(1u);
-    copy_nib(2u);
-    for (uint t = 0; t < nt; t += 4u) {
-        GB_STEP(0, t);
-        GB_STEP(1, t + 1u);
-        GB_STEP(2, t + 2u);
-        GB_STEP(3, t + 3u);
+    if (!KW || nt != 0u) {
+        copy_nib(0u);
+        copy_hdr(0u);
+        copy_nib(1u);
+        copy_x(0u);
+        gx_wait<0>();
+        if (!KW) __syncthreads();
+        GB_READ_A(0u, 0u, afA);
+        GB_READ_W(0u, 0, true);
+        b0 = r0.frag<0>(magic);
+        b1 = r1.frag<0>(magic);
+        copy_x(1u);
+        copy_nib(2u);
+        for (uint t = 0; t < nt; t += 4u) {
+            GB_STEP(0, t);
+            GB_STEP(1, t + 1u);
+            GB_STEP(2, t + 2u);
+            GB_STEP(3, t + 3u);
+        }
+        gx_wait<0>();
     }
-    gx_wait<0>();
 #undef GB_READ_A
 #undef GB_READ_W
 #undef GB_MMA
@@ -603,15 +622,43 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
                 }
         if (tid == 0u) cnt[tile] = 0u;        // ready for the next launch
     }
-    // epilogue: D register v of block (i, j) holds token row 32 i + 8 (v / 4) + 4 kg + v % 4, output 64 wave + 32 j + fr
+    if (KW) {
+        // The waves' partial tiles meet in LDS: each wave leaves its 128 accumulators in its own activation stages (32 KB,
+        // a float4 of every lane per row: 1 KB), then wave w adds token block w of all four, in wave order, and stores it.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        float4* const dump = (float4*)(lds + wave * 2u * XS) + lane;
 #pragma unroll
-    for (int i = 0; i < MI; i++) {
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    dump[((i * 2 + j) * 4 + q) * 64] = make_float4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4* const src = (const float4*)lds + ((wave * 2u + j) * 4u + q) * 64u + lane;
+                float4 sum = src[0];
+#pragma unroll
+                for (uint o = 1; o < 4u; o++) {
+                    const float4 v = src[o * (2u * XS / 16u)];
+                    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+                }
+                acc[0][j][4 * q] = sum.x; acc[0][j][4 * q + 1] = sum.y; acc[0][j][4 * q + 2] = sum.z; acc[0][j][4 * q + 3] = sum.w;
+            }
+    }
+    // epilogue: D register v of block (i, j) holds token row 32 i + 8 (v / 4) + 4 kg + v % 4, output 64 wave + 32 j + fr
+    // (KW: the wave stores token block `wave` alone, summed into acc[0])
+#pragma unroll
+    for (int i = 0; i < (KW ? 1 : MI); i++) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            const uint n = n0 + wave * 64u + 32u * j + fr;
+            const uint n = nw + 32u * j + fr;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const uint m = m0 + 32u * i + 8u * (v >> 2) + 4u * kg + (v & 3u);
+                const uint m = m0 + 32u * (KW ? wave : (uint)i) + 8u * (v >> 2) + 4u * kg + (v & 3u);
                 if (m < M && n < N) {
                     float* o = y + (size_t)m * N + n;
                     if (SPLITK == 1) atomicAdd(o, acc[i][j][v]);
@@ -648,6 +695,18 @@ extern "C" __global__ void __launch_bounds__(256)
 gemm_mm_q4kl_bd256_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
     __shared__ __attribute__((aligned(1024))) uchar lds[GB_LDS(8)];
     gemm_bd_body<1, true, 8>(xh, w, y, K, N, M, nsplit, lds);
+}
+// 64-row tiles, K over the workgroup's waves: grid [ceil(N/64), ceil(M/128), 1 | nsplit]
+extern "C" __global__ void __launch_bounds__(256)
+gemm_mm_q4kl_bdk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
+    __shared__ __attribute__((aligned(1024))) uchar lds[8u * GB_XSTAGE(4) + 4u * 8192u];
+    if (accum) gemm_bd_body<0, true, 4, true>(xh, w, y, K, N, M, 1u, lds);
+    else gemm_bd_body<0, false, 4, true>(xh, w, y, K, N, M, 1u, lds);
+}
+extern "C" __global__ void __launch_bounds__(256)
+gemm_mm_q4kl_bdk_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
+    __shared__ __attribute__((aligned(1024))) uchar lds[8u * GB_XSTAGE(4) + 4u * 8192u];
+    gemm_bd_body<1, true, 4, true>(xh, w, y, K, N, M, nsplit, lds);
 }
 // K slices without atomics and without a zero fill: partial tiles through `part` (tiles x slices x 128 KB, 256 KB for
 // the 256-token tile), one counter per tile in `cnt` (zero before the first launch; every launch leaves zeros), the

@@ -807,6 +807,10 @@ static void gemm_tile(const ojh_kernel_spec *s, uint32_t *bm, uint32_t *bn, bool
     *sk = s->rows_per_wave & 1;
     *bn = (s->rows_per_wave >= 2 && s->rows_per_wave < 8) ? 256 : 128;
     *bm = (s->rows_per_wave >= 4 && s->rows_per_wave < 8) ? 128 : 256;
+    if (s->rows_per_wave == 12 || s->rows_per_wave == 13) {   // 64 rows x 128 tokens, K over the workgroup's waves
+        *bn = 64;
+        *bm = 128;
+    }
 }
 
 static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
@@ -824,9 +828,9 @@ static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_
     if (grid[0] != (N + bn - 1) / bn || grid[1] != (M + bm - 1) / bm || grid[2] != nsplit)
         return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, (N + bn - 1) / bn, (M + bm - 1) / bm, nsplit);
     // the 256-wide tiles address activations with 32-bit byte offsets
-    if (bn == 256 && (uint64_t)M * K * 2 > 0xFFFFFFFFull)
+    if (bn != 128 && (uint64_t)M * K * 2 > 0xFFFFFFFFull)
         return ojh_fail(OJH_ERR_ARG, "%s: M*K=%llu exceeds 2^31 activations", s->name, (unsigned long long)M * K);
-    if (bn == 256 && (uint64_t)N * (K / f->weights) * f->bytes > 0xFFFFFFFFull)
+    if (bn != 128 && (uint64_t)N * (K / f->weights) * f->bytes > 0xFFFFFFFFull)
         return ojh_fail(OJH_ERR_ARG, "%s: the weight tensor exceeds 4 GiB", s->name);
     need[0] = (size_t)M * K * 2;
     need[1] = (size_t)N * (K / f->weights) * f->bytes;
@@ -918,6 +922,7 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
         uint32_t tiles = grid[0] * grid[1], steps = K / 64;
         uint32_t z = tiles ? cus / tiles : 1;  // floor: 224 tiles on 256 CUs are better left whole
         if (z > steps / 4) z = steps / 4;
+        if (s->rows_per_wave == 13 && z > steps / 16) z = steps / 16;   // K over the waves: a super-block per wave and slice at least
         if (z > 16) z = 16;
         grid[2] = z ? z : 1;
     }
@@ -1472,6 +1477,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("gemm_mm_q4l_sk", "gemm", 5, 4, 0, 9, check_gemm_q4l, shape_gemm);
     add("gemm_mm_q4l_hb", "gemm", 5, 4, 0, 10, check_gemm_q4l, shape_gemm);
     // Q4_K with the arithmetic of the reference's `gemm_mm_q4l` (f16 qa*q + qb), 256-wide tiles
+    add("gemm_mm_q4kl_bdk", "gemm_xl", 3, 4, OJH_Q4_K, 12, check_gemm, shape_gemm);
+    add("gemm_mm_q4kl_bdk_sk", "gemm_xl", 3, 4, OJH_Q4_K, 13, check_gemm, shape_gemm);
     add("gemm_mm_q4kl_bd_sr", "gemm_xl", 5, 5, OJH_Q4_K, 128, check_gemm_sr, shape_gemm_sr);
     add("gemm_mm_q4kl_bd256_sr", "gemm_xl", 5, 5, OJH_Q4_K, 256, check_gemm_sr, shape_gemm_sr);
     add("gemm_mm_q4kl", "gemm_xl", 3, 4, OJH_Q4_K, 2, check_gemm, shape_gemm);

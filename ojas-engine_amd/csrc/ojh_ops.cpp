@@ -516,9 +516,22 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
             uint32_t t256 = ((N + 255) / 256) * ((m + 255) / 256);
             bool tall = m > 128 && (t256 >= cus || (2 * t256 >= cus && K >= 8192));
             base = tall ? "gemm_mm_q4kl" : "gemm_mm_q4kl_bd";
+            // 128-token tiles of 256 rows too few to fill the chip: 64-row tiles whose four waves split K between them
+            // and meet in LDS — four times the tiles before any K slice has to meet another through atomics
+            // (measured: gate/up at 128 tokens 26 against 42 us, down at 512 tokens 74 against 88, 4096 x 4096 at 512
+            // tokens 33 against 51 with the conversion)
+            // — wherever the 256-row tiles would have to split K in two or more (from four slices when K is long: there
+            // the longer loop pays more for the waves' separate activation copies than two slices' atomics cost)
+            const uint32_t t_bd = ((N + 255) / 256) * ((m + 127) / 128), z_bd = t_bd ? cus / t_bd : 0;
+            if (!tall && K >= 1024 && (dev->gemm_bdk == 2 || (dev->gemm_bdk == 1 && z_bd >= 2 && (K <= 8192 || z_bd >= 4))))
+                base = "gemm_mm_q4kl_bdk";
         }
         uint32_t sg[3], sb[3];
         if ((rc = ojh_launch_shape(dev, (base + "_sk").c_str(), K, N, m, sg, sb))) return rc;
+        if (dev->gemm_sr && base == "gemm_mm_q4kl_bdk" && sg[2] > 1) {   // reproducible bits asked for: its K slices meet in atomics
+            base = "gemm_mm_q4kl_bd";
+            if ((rc = ojh_launch_shape(dev, (base + "_sk").c_str(), K, N, m, sg, sb))) return rc;
+        }
         if (dev->gemm_split_override > 0) sg[2] = (uint32_t)dev->gemm_split_override;
         // 256-token tiles that fill the chip: the form that dequantizes into the B registers (same grid).  Its step
         // time does not grow with the number of busy CUs as the LDS-shared tile's does (measured: 2.2 us per K step
@@ -529,7 +542,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         // scratch, the last slice of a tile to finish adding them in slice order: bits that do not depend on arrival, no
         // zero fill.  Measured slower than the atomics (one workgroup per tile reads every slice back from behind the
         // L2: gate/up at 128 tokens 60 against 45 us, down 142 against 46), so it is not the default.
-        if (sg[2] > 1 && xl && base != "gemm_mm_q4kl" && dev->gemm_sr && !dev->no_scratch) {
+        if (sg[2] > 1 && xl && (base == "gemm_mm_q4kl_bd" || base == "gemm_mm_q4kl_bd256") && dev->gemm_sr && !dev->no_scratch) {
             uint32_t eg[3] = {conv_blocks, 1, 1};
             if ((rc = ojh_launch(dev, x_dtype == OJH_X_BF16 ? "copy_bf16_half" : "copy_f32_half", {at(x, x_off), xh->ptr},
                                  {n_el}, eg, block)))
