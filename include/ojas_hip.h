@@ -326,6 +326,17 @@ int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint32_t d
                 const ojh_lin *gate, const ojh_lin *up, const ojh_lin *down, ojh_buf *y,
                 int accum, int act_mode);
 
+/* Router and expert FFN in one call: logits [n_tokens][n_expert] f32 -> idx, wgt [n_tokens][ksel] (written: softmax,
+ * top ksel, renormalised — ojh_moe_route's arithmetic, the same bits) -> y as ojh_moe_ffn.  For up to 8 tokens over
+ * Q4_K gate / up experts (the decode form of ojh_moe_ffn and its limits) the router runs inside the gate/up launch:
+ * two launches per layer and token instead of three; every other case is ojh_moe_route followed by ojh_moe_ffn.
+ * The op-level seam of the reference takes router logits or (idx, wgt) alike (ojas-cuda moe.rs:45-125 run back to
+ * back by its decoders); OJAS_HIP_MOE_ROUTE_FUSE=0 keeps the router a launch of its own. */
+int ojh_moe_ffn_routed(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint32_t d, uint32_t n_ff,
+                       uint32_t n_expert, uint32_t ksel, const ojh_buf *logits, ojh_buf *idx, ojh_buf *wgt,
+                       const ojh_lin *gate, const ojh_lin *up, const ojh_lin *down, ojh_buf *y, int accum,
+                       int act_mode);
+
 /* The same over streamed experts: the matrices of assignment a = (token, slot) start at byte
  * offset off_*[a] (u64, 16-byte aligned) of their arena, wherever the caller's expert cache put
  * them (crates/ojas-cuda/src/kernels/moe.rs:133-174 `moe_{gu,down}_*_slots`,

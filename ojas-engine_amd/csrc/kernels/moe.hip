@@ -23,6 +23,7 @@
 //   moe_down_{q4k,q5k}_m(aq, as, wd, dv, offsets, list, K, N, NA)      grid (ceil(N/16), E); ceil(N/32) for K <= 1024
 //   moe_combine(dv, wgt, y, T, KSEL, D, ACC)                 grid ceil(T*D/256)
 //   moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)   grid (ceil(N/8), NA): few tokens, f32 in
+//   moe_gu_q4k_decr(x, wg, wu, act, lg, idx, wgt, K, N, KSEL, NA, E)  the same with the router inside (writes idx, wgt)
 //   moe_down_{q4k,q5k}_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)  grid (ceil(N/8), T): down + weighted sum
 //   moe_gu_q4k_slots(x, arena_g, arena_u, act, off_g, off_u, K, N, KSEL, NA, LIM_G, LIM_U)   the decode form over
 //   moe_down_q4k_slots(act, arena, off_d, wgt, y, K, N, KSEL, LIM, ACC)                     streamed experts (u64 byte offsets)
@@ -445,14 +446,31 @@ __device__ __forceinline__ size_t expert_base(const void* sel, uint a, bool slot
 }
 
 // Block (rb, a): 4 waves x 2 rows of gate and up of assignment a's expert against token a / KSEL.
-template <bool SLOTS>
+// ROUTE: the workgroup routes its token itself first — wave 0 runs the router over lg[t], the slot's expert is read
+// from LDS, and one workgroup per token writes idx / wgt out for the down launch (sel_g / sel_u are not read).
+template <bool SLOTS, bool ROUTE = false>
 __device__ __forceinline__ void moe_gu_dec_body(const float* __restrict__ x, const uchar* __restrict__ wg,
                                                 const uchar* __restrict__ wu, float* __restrict__ act,
                                                 const void* __restrict__ sel_g, const void* __restrict__ sel_u,
-                                                uint K, uint N, uint KSEL, uint EG, uint EU) {
+                                                uint K, uint N, uint KSEL, uint EG, uint EU,
+                                                const float* __restrict__ lg = nullptr, uint* __restrict__ idx_out = nullptr,
+                                                float* __restrict__ wgt_out = nullptr) {
     __shared__ __align__(16) signed char xq[MOE_DEC_GU_K];
     __shared__ float xs[MOE_DEC_GU_K / 256u];
-    const uint a = blockIdx.y, t = a / KSEL;
+    __shared__ uint r_idx[64];
+    __shared__ float r_wgt[64];
+    uint a = blockIdx.y;
+    const uint t = a / KSEL;
+    if (ROUTE) {
+        if (threadIdx.x < 64u) moe_topk_body(lg + (size_t)t * EG, r_idx, r_wgt, EG, KSEL);
+        __syncthreads();
+        if (blockIdx.x == 0u && a == t * KSEL && threadIdx.x < KSEL) {
+            idx_out[a + threadIdx.x] = r_idx[threadIdx.x];
+            wgt_out[a + threadIdx.x] = r_wgt[threadIdx.x];
+        }
+        sel_g = sel_u = r_idx;
+        a -= t * KSEL;              // the slot: index into the token's own table
+    }
     const uint lane = threadIdx.x & 63u;
     const uint row0 = min((blockIdx.x * 4u + (threadIdx.x >> 6)) * 2u, N - 1u);   // surplus waves repeat the last row
     const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
@@ -486,7 +504,7 @@ __device__ __forceinline__ void moe_gu_dec_body(const float* __restrict__ x, con
     }
     vg0 = wave_sum(vg0); vg1 = wave_sum(vg1); vu0 = wave_sum(vu0); vu1 = wave_sum(vu1);
     if (lane == 0) {
-        float* o_ = act + (size_t)a * N + row0;
+        float* o_ = act + (size_t)blockIdx.y * N + row0;
         o_[0] = (vg0 / (1.0f + expf(-vg0))) * vu0;
         if (two) o_[1] = (vg1 / (1.0f + expf(-vg1))) * vu1;
     }
@@ -495,6 +513,14 @@ extern "C" __global__ void __launch_bounds__(256)
 moe_gu_q4k_dec(const float* x, const uchar* wg, const uchar* wu, float* act, const uint* idx, uint K, uint N, uint KSEL,
                uint NA, uint E) {
     moe_gu_dec_body<false>(x, wg, wu, act, idx, idx, K, N, KSEL, E, E);
+}
+// The decode form with the router inside: moe_gu_q4k_decr(x, wg, wu, act, lg, idx, wgt, K, N, KSEL, NA, E) — lg: the
+// router logits [tokens][E]; idx / wgt [tokens][KSEL] are written (softmax, top KSEL, renormalised: moe_topk's
+// arithmetic, the same bits) for the down launch that follows.  One launch less per layer and token.
+extern "C" __global__ void __launch_bounds__(256)
+moe_gu_q4k_decr(const float* x, const uchar* wg, const uchar* wu, float* act, const float* lg, uint* idx, float* wgt,
+                uint K, uint N, uint KSEL, uint NA, uint E) {
+    moe_gu_dec_body<false, true>(x, wg, wu, act, nullptr, nullptr, K, N, KSEL, E, E, lg, idx, wgt);
 }
 extern "C" __global__ void __launch_bounds__(256)
 moe_gu_q4k_slots(const float* x, const uchar* arena_g, const uchar* arena_u, float* act, const unsigned long* off_g,

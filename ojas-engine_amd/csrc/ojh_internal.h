@@ -75,6 +75,7 @@ struct ojh_device {
     uint32_t moe_dec_tokens = 8; // OJAS_HIP_MOE_DEC_TOKENS: the decode form serves up to this many tokens
     int gemm_bdk = 1;            // OJAS_HIP_GEMM_BDK: 0 never takes the 64-row tile whose waves split K, 2 takes it wherever the 128-token tile would run
     bool gemm_sr = false;        // OJAS_HIP_GEMM_SR=1: K slices of the prefill tile meet in scratch, added in slice order (reproducible bits), instead of in f32 atomics
+    bool moe_route_fuse = true;  // OJAS_HIP_MOE_ROUTE_FUSE=0: ojh_moe_ffn_routed keeps the router a launch of its own
     bool moe_fuse = true;        // OJAS_HIP_MOE_FUSE=0: the grouped pipeline keeps its quantizer and grouping launches apart
     bool gemm_exact = false;     // OJAS_HIP_GEMM_EXACT: Q4_K prefill through the tile that holds dequant_to_f16 bits
     bool fused_quant = false;    // OJAS_HIP_FUSED_QUANT=1: ojh_mm (m = 1, Q4_K) quantizes x inside the matvec launch

@@ -1060,6 +1060,23 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         align[0] = align[1] = align[2] = 16;
         return OJH_OK;
     }
+    case 21: {  // moe_gu_q4k_decr(x, wg, wu, act, lg, idx, wgt, K, N, KSEL, NA, E): the decode form, router inside
+        uint32_t K = c[0], N = c[1], KS = c[2], NA = c[3], E = c[4];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!K || K % 256 || !N || !KS || KS > 64 || !NA || NA % KS || !E || E > 1024 || KS > E)
+            return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u KSEL=%u (<= 64, <= E) NA=%u E=%u (<= 1024)", s->name, K, N, KS, NA, E);
+        if (K > 8192) return ojh_fail(OJH_ERR_UNSUPPORTED, "%s: K=%u exceeds the 8192 activations staged in LDS", s->name, K);
+        if (grid[0] != (N + 7) / 8 || grid[1] != NA || grid[2] != 1)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/8), NA, 1]", s->name);
+        need[0] = (size_t)(NA / KS) * K * 4;
+        need[1] = need[2] = (size_t)E * N * (K / 256) * 144;
+        need[3] = (size_t)NA * N * 4;
+        need[4] = (size_t)(NA / KS) * E * 4;
+        need[5] = need[6] = (size_t)NA * 4;
+        align[0] = align[1] = align[2] = 16;
+        align[4] = align[5] = align[6] = 4;
+        return OJH_OK;
+    }
     case 9: {   // moe_down_q4k_dec(act, wd, idx, wgt, y, K, N, KSEL, E, ACC)
         uint32_t K = c[0], N = c[1], KS = c[2], E = c[3], T = grid[1];
         if ((rc = check_block(block, 256))) return rc;
@@ -1201,6 +1218,7 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K
     case 3: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = experts
     case 4: grid[0] = K <= 1024 ? (N + 31) / 32 : (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
     case 20: grid[0] = M + 1; break;  // M = tokens
+    case 21: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;   // M = assignments
     case 6: case 7: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;
     case 14: case 16: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = slots, one token
     case 15: case 17: grid[0] = (N + 3) / 4; break;                           // one token
@@ -1504,6 +1522,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("moe_gu_q4k_mt", "moe", 7, 4, OJH_Q4_K, 12, check_moe, shape_moe);
     add("moe_down_q4k_mt", "moe", 6, 3, OJH_Q4_K, 13, check_moe, shape_moe);
     add("moe_gu_q4k_dec", "moe", 5, 5, OJH_Q4_K, 8, check_moe, shape_moe);
+    add("moe_gu_q4k_decr", "moe", 7, 5, OJH_Q4_K, 21, check_moe, shape_moe);
     add("moe_down_q4k_dec", "moe", 5, 5, OJH_Q4_K, 9, check_moe, shape_moe);
     add("moe_gu_q4k_slots", "moe", 6, 6, OJH_Q4_K, 10, check_moe, shape_moe);
     add("moe_down_q4k_slots", "moe", 5, 5, OJH_Q4_K, 11, check_moe, shape_moe);

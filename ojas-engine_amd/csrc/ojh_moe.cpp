@@ -31,6 +31,48 @@ extern "C" int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_
     return ojh_launch(dev, "moe_topk_m", {logits->ptr, idx->ptr, wgt->ptr}, {n_expert, ksel}, grid, block);
 }
 
+// Router + expert FFN.  A few tokens over Q4_K gate / up experts: the router runs inside the gate/up launch of the
+// decode form (every workgroup routes its token itself; idx / wgt are written for the down launch and for the
+// caller) — two launches per layer instead of three; otherwise ojh_moe_route, then ojh_moe_ffn.
+extern "C" int ojh_moe_ffn_routed(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32_t d, uint32_t n_ff, uint32_t E,
+                                  uint32_t ksel, const ojh_buf *logits, ojh_buf *idx, ojh_buf *wgt, const ojh_lin *gate,
+                                  const ojh_lin *up, const ojh_lin *down, ojh_buf *y, int accum, int act_mode) {
+    if (!dev || !gate || !up || !down) return ojh_fail(OJH_ERR_ARG, "ojh_moe_ffn_routed: NULL argument");
+    if (!T || !E || E > 1024 || !ksel || ksel > E || ksel > 64 || T > 65535u / ksel)
+        return ojh_fail(OJH_ERR_ARG, "moe_ffn_routed: tokens=%u experts=%u (<= 1024) ksel=%u (<= 64, <= experts) out of range", T, E, ksel);
+    const bool kq = gate->type == OJH_Q4_K && up->type == OJH_Q4_K &&
+                    (down->type == OJH_Q4_K || down->type == OJH_Q5_K || down->type == OJH_Q6_K);
+    const bool dec_fits = d && n_ff && d % 256 == 0 && n_ff % 256 == 0 && d <= 8192 && n_ff <= 2048 && (uint64_t)ksel * n_ff <= 32768;
+    const bool fused = kq && act_mode != OJH_ACT_FLOAT && act_mode != OJH_ACT_FLOAT_EXACT && dec_fits &&
+                       (dev->moe_mode == 3 || (dev->moe_mode == 0 && T <= dev->moe_dec_tokens)) && dev->moe_route_fuse;
+    int rc;
+    if (!fused) {
+        if ((rc = ojh_moe_route(dev, logits, T, E, ksel, idx, wgt))) return rc;
+        return ojh_moe_ffn(dev, x, T, d, n_ff, E, ksel, idx, wgt, gate, up, down, y, accum, act_mode);
+    }
+    if (gate->k != d || up->k != d || gate->n != (uint64_t)E * n_ff || up->n != gate->n || down->k != n_ff ||
+        down->n != (uint64_t)E * d)
+        return ojh_fail(OJH_ERR_ARG, "moe_ffn_routed: expert tensor shapes do not match E=%u d=%u n_ff=%u", E, d, n_ff);
+    const uint32_t NA = T * ksel;
+    if ((rc = span("moe_ffn_routed: x", x, (size_t)T * d * 4, 16))) return rc;
+    if ((rc = span("moe_ffn_routed: logits", logits, (size_t)T * E * 4, 4))) return rc;
+    if ((rc = span("moe_ffn_routed: idx", idx, (size_t)NA * 4, 4))) return rc;
+    if ((rc = span("moe_ffn_routed: wgt", wgt, (size_t)NA * 4, 4))) return rc;
+    if ((rc = span("moe_ffn_routed: y", y, (size_t)T * d * 4, 4))) return rc;
+    if ((rc = ensure(dev, "moe"))) return rc;
+    ojh_buf *act;
+    if ((rc = ojh_scratch_get(dev, "moe_act", (size_t)NA * n_ff * 4, &act))) return rc;
+    uint32_t b256[3] = {256, 1, 1}, g1[3] = {(n_ff + 7) / 8, NA, 1}, g2[3] = {(d + 7) / 8, T, 1};
+    if ((rc = ojh_launch(dev, "moe_gu_q4k_decr",
+                         {x->ptr, (char *)gate->raw->ptr + gate->off, (char *)up->raw->ptr + up->off, act->ptr, logits->ptr,
+                          idx->ptr, wgt->ptr},
+                         {d, n_ff, ksel, NA, E}, g1, b256)))
+        return rc;
+    const std::string down_dec = std::string("moe_down_") + ojh_format(down->type)->tag + "_dec";
+    return ojh_launch(dev, down_dec.c_str(), {act->ptr, (char *)down->raw->ptr + down->off, idx->ptr, wgt->ptr, y->ptr},
+                      {n_ff, d, ksel, E, (uint32_t)(accum != 0)}, g2, b256);
+}
+
 extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32_t d, uint32_t n_ff, uint32_t E,
                            uint32_t ksel, const ojh_buf *idx, const ojh_buf *wgt, const ojh_lin *gate,
                            const ojh_lin *up, const ojh_lin *down, ojh_buf *y, int accum, int act_mode) {

@@ -89,6 +89,7 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_MOE")) d->moe_mode = atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE_DEC_TOKENS")) d->moe_dec_tokens = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE_FUSE")) d->moe_fuse = atoi(r) != 0;
+    if (const char *r = getenv("OJAS_HIP_MOE_ROUTE_FUSE")) d->moe_route_fuse = atoi(r) != 0;
     if (const char *r = getenv("OJAS_HIP_GEMM_SR")) d->gemm_sr = atoi(r) != 0;
     if (const char *r = getenv("OJAS_HIP_GEMM_BDK")) d->gemm_bdk = atoi(r);
     if (const char *r = getenv("OJAS_HIP_FUSED_QUANT")) d->fused_quant = atoi(r) != 0;

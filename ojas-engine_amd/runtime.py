@@ -145,6 +145,7 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_quant_q8k": (i32, [vp, vp, sz, i32, u32, u32, vp, vp]),
         "ojh_moe_route": (i32, [vp, vp, u32, u32, u32, vp, vp]),
         "ojh_moe_ffn": (i32, [vp, vp, u32, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp, i32, i32]),
+        "ojh_moe_ffn_routed": (i32, [vp, vp, u32, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp, vp, i32, i32]),
         "ojh_moe_ffn_slots": (i32, [vp, vp, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp, vp, vp, i32]),
         "ojh_expert_cache_create": (i32, [vp, sz, sz, C.POINTER(vp)]),
         "ojh_expert_cache_destroy": (i32, [vp]),
@@ -624,6 +625,13 @@ class HipGpu:
         self._check(self._L.ojh_moe_ffn_slots(self._dev, x.handle, n_tokens, d, n_ff, ksel, arena_gate.handle,
                                               off_gate.handle, arena_up.handle, off_up.handle, arena_down.handle,
                                               off_down.handle, wgt.handle, y.handle, int(accum)))
+
+    def moe_ffn_routed(self, x: Buf, n_tokens: int, d: int, n_ff: int, n_expert: int, ksel: int, logits: Buf, idx: Buf,
+                       wgt: Buf, gate: Lin, up: Lin, down: Lin, y: Buf, accum: bool = False, act_mode: int = ACT_AUTO) -> None:
+        """Router + expert FFN; idx and wgt are written.  A few tokens: the router runs inside the gate/up launch."""
+        self._check(self._L.ojh_moe_ffn_routed(self._dev, x.handle, n_tokens, d, n_ff, n_expert, ksel, logits.handle,
+                                               idx.handle, wgt.handle, gate.handle, up.handle, down.handle, y.handle,
+                                               int(accum), act_mode))
 
     def moe_ffn(self, x: Buf, n_tokens: int, d: int, n_ff: int, n_expert: int, ksel: int, idx: Buf, wgt: Buf,
                 gate: Lin, up: Lin, down: Lin, y: Buf, accum: bool = False, act_mode: int = ACT_AUTO) -> None:

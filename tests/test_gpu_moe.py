@@ -209,6 +209,34 @@ def test_decode_form_is_bit_identical_to_the_grouped_integer_dots(gpu, pkg, monk
     assert np.all(np.isfinite(outs[0])) and np.any(outs[0] != (y0.ravel() if accum else 0.0))
 
 
+@pytest.mark.parametrize("T,E,ksel,d,nff,accum,dty", [(1, 128, 8, 2048, 768, False, Q4_K), (3, 16, 5, 2304, 512, True, Q4_K),
+                                                       (8, 8, 8, 768, 256, False, 13), (2, 70, 64, 256, 256, False, 14),
+                                                       (5, 300, 6, 512, 256, True, Q4_K), (33, 16, 4, 512, 512, False, Q4_K)])
+def test_router_inside_the_decode_form(gpu, orc, pkg, T, E, ksel, d, nff, accum, dty):
+    """`ojh_moe_ffn_routed`: for a few tokens the router runs inside the gate/up launch (`moe_gu_q4k_decr`) — the idx and
+    wgt it writes are the bits of `moe_route`, the output the bits of route + `moe_ffn`; more tokens (33) take the two
+    calls as they are."""
+    gate = pkg.synth.q4k_weights(E * nff, d, "moer", "g", E, d, nff)
+    up = pkg.synth.q4k_weights(E * nff, d, "moer", "u", E, d, nff)
+    down = pkg.synth.weights(dty, E * d, nff, "moer", "d", dty, E, d, nff)
+    x = pkg.synth.normal_f32(T * d, "moer", "x", T, d).reshape(T, d)
+    lg = pkg.synth.normal_f32(T * E, "moer", "lg", T, E).reshape(T, E)
+    lg[0, :4] = lg[0, 4]                                  # ties: the lowest index wins
+    gi, gw, idx_d, wgt_d = _route(gpu, lg, ksel)
+    lg_, lu_, ld_ = gpu.lin(Q4_K, E * nff, d, gate), gpu.lin(Q4_K, E * nff, d, up), gpu.lin(dty, E * d, nff, down)
+    y0 = pkg.synth.normal_f32(T * d, "moer", "y0").reshape(T, d)
+    ya = gpu.upload(np.concatenate([y0.ravel(), np.full(d, 12345.5, np.float32)]))
+    gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, ya, accum=accum)
+    want = gpu.read(ya, T * d + d)
+    yb = gpu.upload(np.concatenate([y0.ravel(), np.full(d, 12345.5, np.float32)]))
+    idx2, wgt2 = gpu.upload_bytes(np.full(T * ksel + 2, 0xFFFFFFFF, np.uint32)), gpu.upload(np.full(T * ksel + 2, 777.0, np.float32))
+    gpu.moe_ffn_routed(gpu.upload(x), T, d, nff, E, ksel, gpu.upload(lg), idx2, wgt2, lg_, lu_, ld_, yb, accum=accum)
+    assert np.array_equal(gpu.read(idx2, T * ksel + 2, np.uint32), np.concatenate([gi.ravel(), [0xFFFFFFFF, 0xFFFFFFFF]]))
+    assert np.array_equal(gpu.read(wgt2, T * ksel + 2), np.concatenate([gw.ravel(), [777.0, 777.0]]))
+    assert np.array_equal(gpu.read(yb, T * d + d), want)
+    assert peak_err(want[:T * d].reshape(T, d) - (y0 if accum else 0.0), orc.moe_ffn(x, gi, gw, gate, up, Q4_K, down, dty, E, nff)) <= 2e-5
+
+
 @pytest.mark.parametrize("T,E,ksel,d,nff,accum", [(40, 4, 2, 512, 768, False), (9, 16, 3, 2304, 256, True),
                                                    (130, 6, 5, 1024, 1280, False), (64, 128, 8, 2048, 768, False)])
 def test_matrix_core_forms_agree(gpu, orc, pkg, monkeypatch, T, E, ksel, d, nff, accum):
