@@ -311,7 +311,7 @@ def extras(gpu, pkg, lin_q) -> dict:
             tf = 2.0 * m * n * k / us / 1e6
             gemm[f"{name}_M{m}"] = {"us": round(us, 1), "tflops": round(tf, 1), "mfma_frac": round(tf / 2500.0, 4)}
     out["prefill_gemm_q4k"] = {"activations": "bf16 N(0,1), converted to f16 into the tile", "accumulate": "f32",
-                               "tile": "v_mfma_f32_32x32x16_f16, 256x256 outputs per workgroup (128x256, its weights dequantized straight into the B registers, when that fills more CUs); "
+                               "tile": "v_mfma_f32_32x32x16_f16, weights dequantized straight into the B registers: 256 tokens x 256 rows per workgroup where that fills the chip (M = 2048), 128 x 256 below (gate/up M = 512), 128 x 64 with K split over the workgroup's waves where 256-row tiles are too few (M = 128, down M = 512); "
                                        "weights = binary16 fma(qa, q, qb), the bits of the reference's gemm_mm_q4l",
                                "peak_tflops": 2500.0, "timed": "conversion + zero fill (split-K) + tile", **gemm}
     # ---- the same two matrices in the CPU path's arithmetic (quant_q8k activations, int8 MFMA), f32 in
