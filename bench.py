@@ -328,7 +328,7 @@ def extras(gpu, pkg, lin_q) -> dict:
     out["verify_prefill_q4k_int8"] = {"arithmetic": "quant_q8k activations, int8 x u4 dots on the int8 matrix cores, the CPU "
                                                     "reference's scale algebra (results within 2e-5 of matvec_kq)",
                                       "peak_tops": 5000.0,
-                                      "timed": "quantize_q8k + the tile: from 96 tokens q8k_token_sides + gemm_q8k_q4k_xt{,64} "
+                                      "timed": "quantizer + the tile: from 96 tokens quantize_q8k_sides + gemm_q8k_q4k_xt{,64} "
                                                "(128-token tiles, scales folded into int8 planes, v_mfma_i32_16x16x64_i8); below, "
                                                "gemm_q8k_q4k_mf (down at M = 8: gemm_q8k_q4k_mk)", **i8}
     # ---- speculative verify on the Q4_K output head of the decode step, bf16 activations

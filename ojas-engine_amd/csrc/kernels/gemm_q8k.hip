@@ -523,6 +523,77 @@ q8k_token_sides(const signed char* __restrict__ xq, const float* __restrict__ xs
     *(uint4*)(sums + ((size_t)sb * MP + t) * 16u) = make_uint4(lo[0], lo[1], hi[0], hi[1]);
 }
 
+// The activation quantizer and q8k_token_sides in one launch, for callers that hand over f32 or bf16 tokens:
+//   quantize_q8k{,_bf16}_sides(x, q, scales, xst, sums, K, M, MP)    grid [K / 256 * MP / 4, 1, 1], block 256
+// One wave per 256-segment, segments numbered token-major (segment s = token s / (K / 256), super-block s % (K / 256)),
+// four values per lane: the segment is quantized exactly as quantize_q8k does (amax / 127, 1 for a zero segment, round
+// half away, clamp), and its scale and split 32-position sums go to the transposed side arrays as well; the segments of
+// rows M .. MP - 1 write zeros there and nothing else.  No barrier and no LDS: the maximum and the sums travel by DPP.
+template <bool BF16>
+__device__ __forceinline__ void quantize_q8k_sides_body(const void* __restrict__ xv, signed char* __restrict__ q,
+                                                        float* __restrict__ scales, float* __restrict__ xst,
+                                                        uchar* __restrict__ sums, uint K, uint M, uint MP) {
+    const uint nsb = K >> 8, lane = threadIdx.x & 63u;
+    const uint seg = blockIdx.x * 4u + (threadIdx.x >> 6);
+    const uint m = seg / nsb, sb = seg - m * nsb;
+    if (m >= MP) return;
+    if (m >= M) {
+        if (lane == 0) {
+            xst[(size_t)sb * MP + m] = 0.0f;
+            *(uint4*)(sums + ((size_t)sb * MP + m) * 16u) = make_uint4(0u, 0u, 0u, 0u);
+        }
+        return;
+    }
+    const size_t i = (size_t)seg * 256u + lane * 4u;
+    float v[4];
+    if (BF16) {
+        const uint2 b = *(const uint2*)((const ushort*)xv + i);
+        v[0] = __uint_as_float(b.x << 16);
+        v[1] = __uint_as_float(b.x & 0xFFFF0000u);
+        v[2] = __uint_as_float(b.y << 16);
+        v[3] = __uint_as_float(b.y & 0xFFFF0000u);
+    } else {
+        const float4 f = *(const float4*)((const float*)xv + i);
+        v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
+    }
+    const float mx = wave_max(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
+    const float scale = mx > 0.0f ? __fdiv_rn(mx, 127.0f) : 1.0f;
+    const float inv = __fdiv_rn(1.0f, scale);
+    int s32 = 0;
+    uint pk = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int r = (int)sat127(roundf(__fmul_rn(v[e], inv)));
+        s32 += r;
+        pk |= ((uint)r & 0xFFu) << (8 * e);
+    }
+    *(uint*)(q + i) = pk;
+    // eight lanes hold one run of 32 positions
+    s32 += dpp_i32<OJK_DPP_QUAD_XOR1>(s32);
+    s32 += dpp_i32<OJK_DPP_QUAD_XOR2>(s32);
+    s32 += dpp_i32<OJK_DPP_ROW_HALF_MIRROR>(s32);
+    uint lo[2] = {0u, 0u}, hi[2] = {0u, 0u};
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++) {
+        const int bs = __builtin_amdgcn_readlane(s32, 8 * jj);
+        lo[jj >> 2] |= (uint)(bs & 63) << (8 * (jj & 3));
+        hi[jj >> 2] |= ((uint)(bs >> 6) & 0xFFu) << (8 * (jj & 3));
+    }
+    if (lane == 0) {
+        scales[seg] = scale;
+        xst[(size_t)sb * MP + m] = scale;
+        *(uint4*)(sums + ((size_t)sb * MP + m) * 16u) = make_uint4(lo[0], lo[1], hi[0], hi[1]);
+    }
+}
+extern "C" __global__ void __launch_bounds__(256)
+quantize_q8k_sides(const float* x, signed char* q, float* scales, float* xst, uchar* sums, uint K, uint M, uint MP) {
+    quantize_q8k_sides_body<false>(x, q, scales, xst, sums, K, M, MP);
+}
+extern "C" __global__ void __launch_bounds__(256)
+quantize_q8k_bf16_sides(const ushort* x, signed char* q, float* scales, float* xst, uchar* sums, uint K, uint M, uint MP) {
+    quantize_q8k_sides_body<true>(x, q, scales, xst, sums, K, M, MP);
+}
+
 __device__ __forceinline__ void gxt_copy16(const void* base, uint voff, uint lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr) : "memory");
 }

@@ -154,7 +154,8 @@ int ojh_mm_checks(const char *who, const ojh_lin *w, ojh_buf *y, size_t y_off, c
                   const ojh_block_format **fmt);
 int ojh_quant_q8k_launch(ojh_device *dev, const void *x, int x_dtype, uint32_t m, uint32_t k, void *q, void *scales);
 int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, const ojh_block_format *f, void *yp,
-                      const ojh_buf *bias, uint32_t m, int accum);
+                      const ojh_buf *bias, uint32_t m, int accum, bool sides_ready = false);
+bool ojh_q4k_xt_taken(const ojh_device *dev, const ojh_lin *w, uint32_t m, const void *wp);
 int ojh_noalloc_setup(ojh_device *dev);   // resolves the static scratch array on the current GPU (ojh_noalloc.cpp)
 void ojh_gemm_q8k_tiles(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M, uint32_t *rw, uint32_t *rt);   // row tiles per workgroup / per wave of gemm_q8k_q4k_mf
 uint32_t ojh_moe_mt_groups(const ojh_device *dev, uint32_t N, uint32_t E, uint32_t per_cu);   // workgroups per expert of those entries

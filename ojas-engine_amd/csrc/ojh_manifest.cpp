@@ -246,6 +246,37 @@ static int check_gemm_q8k_xt(const ojh_kernel_spec *s, const uint32_t *c, const 
     align[1] = align[4] = 4;
     return OJH_OK;
 }
+// quantize_q8k{,_bf16}_sides(x, q, scales, xst, sums, K, M, MP): grid [K / 256 * MP / 4, 1, 1]
+static int check_quantize_sides(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                                const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const uint32_t K = c[0], M = c[1], MP = c[2];
+    if (!K || K % 256 || !M) return ojh_fail(OJH_ERR_ARG, "%s: K=%u (a multiple of 256) M=%u", s->name, K, M);
+    if (MP != (M + 127) / 128 * 128) return ojh_fail(OJH_ERR_ARG, "%s: MP=%u must be M=%u rounded up to 128", s->name, MP, M);
+    if ((uint64_t)M * K > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "%s: M*K exceeds 2^32 activations", s->name);
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    const size_t nsb = K / 256, esz = strstr(s->name, "bf16") ? 2 : 4;
+    if ((uint64_t)nsb * MP / 4 > 0x7FFFFFFFull) return ojh_fail(OJH_ERR_ARG, "%s: too many segments for one launch", s->name);
+    if (grid[0] != nsb * MP / 4 || grid[1] != 1 || grid[2] != 1)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%zu,1,1]", s->name, nsb * MP / 4);
+    need[0] = (size_t)M * K * esz;
+    need[1] = (size_t)M * K;
+    need[2] = (size_t)M * nsb * 4;
+    need[3] = nsb * MP * 4;
+    need[4] = nsb * MP * 16;
+    align[0] = 4 * esz;
+    align[1] = align[2] = align[3] = 4;
+    return OJH_OK;
+}
+static int shape_quantize_sides(const ojh_kernel_spec *, const ojh_device *, uint32_t K, uint32_t, uint32_t M,
+                                uint32_t grid[3], uint32_t block[3]) {
+    if (!M) M = 1;
+    grid[0] = (K / 256 ? K / 256 : 1) * ((M + 127) / 128 * 32);
+    grid[1] = grid[2] = 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
 static int shape_gemm_q8k_xt(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, uint32_t N, uint32_t M,
                              uint32_t grid[3], uint32_t block[3]) {
     if (!M) M = 1;
@@ -1459,6 +1490,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("gemm_q8k_q4k_mf", "gemm_q8k", 4, 6, OJH_Q4_K, 1, check_gemm_q8k, shape_gemm_q8k);
     add("gemm_q8k_q4k_ml", "gemm_q8k", 4, 4, OJH_Q4_K, 1, check_gemm_q8k_ml, shape_ml);
     add("q8k_token_sides", "gemm_q8k", 4, 3, 0, 0, check_gemm_q8k_xt, shape_gemm_q8k_xt);
+    add("quantize_q8k_sides", "gemm_q8k", 5, 3, 0, 0, check_quantize_sides, shape_quantize_sides);
+    add("quantize_q8k_bf16_sides", "gemm_q8k", 5, 3, 0, 0, check_quantize_sides, shape_quantize_sides);
     add("gemm_q8k_q4k_xt", "gemm_q8k", 5, 5, OJH_Q4_K, 1, check_gemm_q8k_xt, shape_gemm_q8k_xt);
     add("gemm_q8k_q4k_xt64", "gemm_q8k", 5, 5, OJH_Q4_K, 2, check_gemm_q8k_xt, shape_gemm_q8k_xt);
     add("gemm_q8k_q4k_mk", "gemm_q8k", 4, 4, OJH_Q4_K, 2, check_gemm_q8k_ml, shape_mk);

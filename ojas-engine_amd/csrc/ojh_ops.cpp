@@ -149,8 +149,17 @@ static int pick_rows(const ojh_device *dev, uint32_t n) {
 }
 
 // y (=,+=,+bias) quantized-x . W^T for K-quant weights: the matvec (m = 1) and its batched form.
+// Whether a Q4_K product of m tokens takes the 128-token int8 tile (when its tiles cover at least half of the CUs: a
+// 4096-row matrix against 128 tokens stays below).
+bool ojh_q4k_xt_taken(const ojh_device *dev, const ojh_lin *w, uint32_t m, const void *wp) {
+    const uint32_t K = w->k, N = w->n, xt_mp = (m + 127) / 128 * 128;
+    return w->type == OJH_Q4_K && dev->q4k_xt_min_m && m >= dev->q4k_xt_min_m && !dev->no_scratch &&
+           (uint64_t)((N + 63) / 64) * (xt_mp / 128) * 2 >= (uint32_t)dev->prop.multiProcessorCount &&
+           (uint64_t)m * K <= 0xFFFFFFFFull && (uint64_t)w->row_bytes * N <= 0xFFFFFFFFull && (uintptr_t)wp % 16 == 0;
+}
+
 int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, const ojh_block_format *f, void *yp,
-                         const ojh_buf *bias, uint32_t m, int accum) {
+                         const ojh_buf *bias, uint32_t m, int accum, bool sides_ready) {
     const uint32_t K = w->k, N = w->n;
     void *wp = at(w->raw, w->off);
     uint32_t grid[3] = {1, 1, 1}, block[3] = {256, 1, 1};
@@ -173,12 +182,9 @@ int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, con
         return ojh_launch(dev, name.c_str(), p, {K, N}, grid, block);
     }
     // Q4_K rows against a prefill-sized batch: 128 x 128 tiles, the tokens copied into LDS by the memory system
-    // (needs two side arrays, built by one small launch into the library's scratch)
-    // (taken when its tiles cover at least half of the CUs: a 4096-row matrix against 128 tokens stays below)
-    const uint32_t xt_mp = (m + 127) / 128 * 128;
-    if (w->type == OJH_Q4_K && dev->q4k_xt_min_m && m >= dev->q4k_xt_min_m && !dev->no_scratch &&
-        (uint64_t)((N + 63) / 64) * (xt_mp / 128) * 2 >= (uint32_t)dev->prop.multiProcessorCount &&
-        (uint64_t)m * K <= 0xFFFFFFFFull && (uint64_t)w->row_bytes * N <= 0xFFFFFFFFull && (uintptr_t)wp % 16 == 0) {
+    // (needs two side arrays, built by one small launch into the library's scratch — or by the quantizer itself when
+    // ojh_mm quantizes: it then comes here with the side arrays ready)
+    if (ojh_q4k_xt_taken(dev, w, m, wp)) {
         int rc = ensure(dev, "gemm_q8k");
         if (rc) return rc;
         const uint32_t mp = (m + 127) / 128 * 128;
@@ -187,8 +193,10 @@ int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, con
         if ((rc = ojh_scratch_get(dev, "xt_xst", nsb * mp * 4, &xst))) return rc;
         if ((rc = ojh_scratch_get(dev, "xt_sums", nsb * mp * 16, &sums))) return rc;
         uint32_t sg[3], sb[3];
-        if ((rc = ojh_launch_shape(dev, "q8k_token_sides", K, N, m, sg, sb))) return rc;
-        if ((rc = ojh_launch(dev, "q8k_token_sides", {xq, xs, xst->ptr, sums->ptr}, {K, m, mp}, sg, sb))) return rc;
+        if (!sides_ready) {
+            if ((rc = ojh_launch_shape(dev, "q8k_token_sides", K, N, m, sg, sb))) return rc;
+            if ((rc = ojh_launch(dev, "q8k_token_sides", {xq, xs, xst->ptr, sums->ptr}, {K, m, mp}, sg, sb))) return rc;
+        }
         // 128-row tiles when they give every CU one, 64-row tiles otherwise
         const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;
         const char *xt = (uint64_t)((N + 127) / 128) * (mp / 128) >= cus && !getenv("OJAS_HIP_Q4K_XT64") ? "gemm_q8k_q4k_xt" : "gemm_q8k_q4k_xt64";
@@ -598,6 +606,19 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         ojh_buf *xq, *xs;
         if ((rc = ojh_scratch_get(dev, "xq", (size_t)m * nsb * 256, &xq))) return rc;
         if ((rc = ojh_scratch_get(dev, "xs", (size_t)m * nsb * 4, &xs))) return rc;
+        // ahead of the 128-token int8 tile the quantizer writes that tile's side arrays too (one launch less)
+        if (ojh_q4k_xt_taken(dev, w, m, wp) && K % 256 == 0 && (uintptr_t)at(x, x_off) % (x_dtype == OJH_X_BF16 ? 8 : 16) == 0) {
+            if ((rc = ensure(dev, "gemm_q8k"))) return rc;
+            const uint32_t mp = (m + 127) / 128 * 128;
+            ojh_buf *xst, *sums;
+            if ((rc = ojh_scratch_get(dev, "xt_xst", nsb * mp * 4, &xst))) return rc;
+            if ((rc = ojh_scratch_get(dev, "xt_sums", nsb * mp * 16, &sums))) return rc;
+            uint32_t qg[3] = {K / 256 * (mp / 4), 1, 1};
+            if ((rc = ojh_launch(dev, x_dtype == OJH_X_BF16 ? "quantize_q8k_bf16_sides" : "quantize_q8k_sides",
+                                 {at(x, x_off), xq->ptr, xs->ptr, xst->ptr, sums->ptr}, {K, m, mp}, qg, block)))
+                return rc;
+            return ojh_mm_q8k_launch(dev, xq->ptr, xs->ptr, w, f, yp, bias, m, accum, true);
+        }
         if ((rc = ojh_quant_q8k_launch(dev, at(x, x_off), x_dtype, m, K, xq->ptr, xs->ptr))) return rc;
         return ojh_mm_q8k_launch(dev, xq->ptr, xs->ptr, w, f, yp, bias, m, accum);
     }

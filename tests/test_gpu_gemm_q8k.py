@@ -171,6 +171,27 @@ def test_prefill_tiles_by_name(gpu, orc, pkg, m, n, k):
     assert np.all((sd[:, :, 0] >= 0) & (sd[:, :, 0] < 64))
     st = gpu.read(xst, nsb * mp).reshape(nsb, mp)
     assert np.array_equal(st[:, :m], gpu.read(xs, m * nsb).reshape(m, nsb).T) and not st[:, m:].any()
+    # the quantizer that leaves the side arrays as well: the same bytes in all four outputs, from f32 and from bf16 tokens
+    xb = (x.view(np.uint32) >> 16).astype(np.uint16)
+    for name, src in (("quantize_q8k_sides", gpu.upload(x)), ("quantize_q8k_bf16_sides", gpu.upload_bytes(xb))):
+        q2, s2 = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
+        xst2 = gpu.upload(np.full(nsb * mp, 7.5, np.float32))
+        sums2 = gpu.upload_bytes(np.full(nsb * mp * 16, 0x55, np.uint8))
+        gpu.dispatch(gpu.begin(), name, [(src, 0), (q2, 0), (s2, 0), (xst2, 0), (sums2, 0)], [k, m, mp], [nsb * mp // 4, 1, 1], [256, 1, 1])
+        if "bf16" in name:
+            q1, s1 = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
+            gpu.quant_q8k(gpu.upload((xb.astype(np.uint32) << 16).view(np.float32)), m, k, q1, s1)
+            xst1, sums1 = gpu.alloc(nsb * mp), gpu.alloc_bytes(nsb * mp * 16)
+            gpu.dispatch(gpu.begin(), "q8k_token_sides", [(q1, 0), (s1, 0), (xst1, 0), (sums1, 0)], [k, m, mp], [nsb, (mp + 255) // 256, 1], [256, 1, 1])
+        else:
+            q1, s1, xst1, sums1 = xq, xs, xst, sums
+        assert np.array_equal(gpu.read(q2, m * k, np.int8), gpu.read(q1, m * k, np.int8)), name
+        assert np.array_equal(gpu.read(s2, m * nsb).view(np.uint32), gpu.read(s1, m * nsb).view(np.uint32)), name
+        assert np.array_equal(gpu.read(xst2, nsb * mp).view(np.uint32), gpu.read(xst1, nsb * mp).view(np.uint32)), name
+        assert np.array_equal(gpu.read(sums2, nsb * mp * 16, np.uint8), gpu.read(sums1, nsb * mp * 16, np.uint8)), name
+    with pytest.raises(pkg.OjasHipError, match="rounded up to 128"):
+        gpu.dispatch(gpu.begin(), "quantize_q8k_sides", [(gpu.upload(x), 0), (xq, 0), (xs, 0), (xst, 0), (sums, 0)], [k, m, mp + 128],
+                     [nsb * (mp + 128) // 4, 1, 1], [256, 1, 1])
     want = np.stack([orc.matvec_kq(w, Q4_K, n, k, x[t]) for t in range(m)])
     ymf = gpu.alloc(m * n)
     gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (ymf, 0)], [k, n, m, 0, 4, 1],
