@@ -195,6 +195,17 @@ def main() -> int:
             cal[f"mfma_f16_{tag}_{where}"] = {"flops": mf_flops, "us": round(us, 1), "tflops": round(mf_flops / us / 1e6, 1),
                                               "mfma_frac": round(mf_flops / us / 1e6 / 2500.0, 4)}
         del src
+    # ... and the int8 matrix instruction of the CPU-arithmetic prefill tile, v_mfma_i32_16x16x64_i8, the same way
+    i8_ops = mgrid[0] * 4 * mf_iters * 64 * 2 * 16 * 16 * 64
+    for tag, ops in (("constant", np.full(8 * 256 * 16, 1, np.int8)),
+                     ("normal", (synth.normal_f32(8 * 256 * 16, "bench", "mfma_i8_calibration") * 60).clip(-127, 127).astype(np.int8))):
+        src = gpu.upload_bytes(ops)
+        for mode, where in ((0, "registers"), (1, "lds")):
+            us = _time(gpu, lambda i: gpu.dispatch(gpu.begin(), "calib_mfma_i8", [(src, 0), (mf_out, 0)], [mf_iters, mode],
+                                                    mgrid, mblock), 5, 2)
+            cal[f"mfma_i8_{tag}_{where}"] = {"ops": i8_ops, "us": round(us, 1), "tops": round(i8_ops / us / 1e6, 1),
+                                             "int8_mfma_frac": round(i8_ops / us / 1e6 / 5000.0, 4)}
+        del src
     del mf_out
 
     # ---- per-shape latency (each shape alone, back to back), for the record, twice: streaming from HBM — as many

@@ -477,8 +477,8 @@ gemm_q8k_q4k_mk(const signed char* xq, const float* xs, const uchar* w, float* y
 
 // ---- prefill-sized batches: 128 tokens x 128 rows per workgroup, tokens copied into LDS by the memory system ----
 //   q8k_token_sides(xq, xs, xst, sums, K, M, MP)      grid [K / 256, ceil(MP / 256), 1], block 256
-//       xst [K/256][MP] f32: the token scales, super-block major;  sums [K/256][MP][16] int8: every 32-position sum of a
-//       token's activations split as 64 hi + lo (eight lo parts, then eight hi parts); rows M .. MP - 1 are zeros.
+//       xst [K/256][MP] f32: the token scales, super-block major;  sums [K/256][MP][8] f32: scale x every 32-position
+//       sum of a token's activations, in the order 0 4 1 5 2 6 3 7; rows M .. MP - 1 are zeros.
 //   gemm_q8k_q4k_xt(xq, xst, sums, w, y, K, N, M, ACC, MP)    grid [ceil(N / 128), MP / 128, 1], block 512;  MP = M rounded up to 128
 //   gemm_q8k_q4k_xt64(the same)                                grid [ceil(N / 64), MP / 128, 1]
 //
@@ -491,19 +491,22 @@ gemm_q8k_q4k_mk(const signed char* xq, const float* xs, const uchar* w, float* y
 // from sixteen different bank groups.  A wave owns one 16-row tile and the eight passes of 16 tokens (the _xt64 entry:
 // 64 rows per workgroup, two waves per tile with four passes each, for matrices with few rows): the tile's
 // weights, scales folded into two int8 planes (see gemm_q8k_q4k_mf), are built once per step, and every 16 bytes of
-// activations read from LDS feed four v_mfma_i32_16x16x64_i8 (two tiles x two planes).  The weights of the next step
-// are ordinary loads into registers, issued a step ahead.  Same arithmetic per (token, row, super-block) as
-// gemm_q8k_q4k_mf, super-blocks added in order: the same bits.
+// activations read from LDS feed two v_mfma_i32_16x16x64_i8 (the two planes).  The weights of the next step
+// are ordinary loads into registers, issued a step ahead.  Per (token, row, super-block) the sum takes
+//     - sum_j (xs bsum_j) (dmin m_j)     two v_mfma_f32_16x16x4_f32 onto the running sums, factors rounded to f32 once
+//     + xs (d isum)                      isum exact in int32
+// super-blocks in order: gemm_q8k_q4k_mf's terms with the min part associated per run instead of per super-block
+// (a few ulp of the result apart; four vector instructions per result and super-block instead of seven).
 #define GXT_TOK 128u
 #define GXT_ROWS 128u
-#define GXT_STAGE (GXT_TOK * 256u + GXT_TOK * 16u + GXT_TOK * 4u)     // tokens | split sums | scales = 35328 bytes
+#define GXT_STAGE (GXT_TOK * 256u + GXT_TOK * 32u + GXT_TOK * 4u)     // tokens | scaled sums | scales = 37376 bytes
 
 extern "C" __global__ void __launch_bounds__(256)
 q8k_token_sides(const signed char* __restrict__ xq, const float* __restrict__ xs, float* __restrict__ xst,
-                uchar* __restrict__ sums, uint K, uint M, uint MP) {
+                float* __restrict__ sums, uint K, uint M, uint MP) {
     const uint nsb = K >> 8, sb = blockIdx.x, t = blockIdx.y * 256u + threadIdx.x;
     if (t >= MP) return;
-    uint lo[2] = {0u, 0u}, hi[2] = {0u, 0u};
+    float f[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     float sc = 0.0f;
     if (t < M) {
         sc = xs[(size_t)t * nsb + sb];
@@ -515,33 +518,32 @@ q8k_token_sides(const signed char* __restrict__ xq, const float* __restrict__ xs
             bs = dot4_i8(a.y, 0x01010101u, bs); bs = dot4_i8(a.z, 0x01010101u, bs); bs = dot4_i8(a.w, 0x01010101u, bs);
             bs = dot4_i8(b.x, 0x01010101u, bs); bs = dot4_i8(b.y, 0x01010101u, bs);
             bs = dot4_i8(b.z, 0x01010101u, bs); bs = dot4_i8(b.w, 0x01010101u, bs);
-            lo[jj >> 2] |= (uint)(bs & 63) << (8 * (jj & 3));
-            hi[jj >> 2] |= ((uint)(bs >> 6) & 0xFFu) << (8 * (jj & 3));
+            f[2 * (jj & 3) + (jj >> 2)] = __fmul_rn(sc, (float)bs);
         }
     }
     xst[(size_t)sb * MP + t] = sc;
-    *(uint4*)(sums + ((size_t)sb * MP + t) * 16u) = make_uint4(lo[0], lo[1], hi[0], hi[1]);
+    float4* o = (float4*)(sums + ((size_t)sb * MP + t) * 8u);
+    o[0] = make_float4(f[0], f[1], f[2], f[3]);
+    o[1] = make_float4(f[4], f[5], f[6], f[7]);
 }
 
 // The activation quantizer and q8k_token_sides in one launch, for callers that hand over f32 or bf16 tokens:
 //   quantize_q8k{,_bf16}_sides(x, q, scales, xst, sums, K, M, MP)    grid [K / 256 * MP / 4, 1, 1], block 256
 // One wave per 256-segment, segments numbered token-major (segment s = token s / (K / 256), super-block s % (K / 256)),
 // four values per lane: the segment is quantized exactly as quantize_q8k does (amax / 127, 1 for a zero segment, round
-// half away, clamp), and its scale and split 32-position sums go to the transposed side arrays as well; the segments of
+// half away, clamp), and its scale and scaled 32-position sums go to the transposed side arrays as well; the segments of
 // rows M .. MP - 1 write zeros there and nothing else.  No barrier and no LDS: the maximum and the sums travel by DPP.
 template <bool BF16>
 __device__ __forceinline__ void quantize_q8k_sides_body(const void* __restrict__ xv, signed char* __restrict__ q,
                                                         float* __restrict__ scales, float* __restrict__ xst,
-                                                        uchar* __restrict__ sums, uint K, uint M, uint MP) {
+                                                        float* __restrict__ sums, uint K, uint M, uint MP) {
     const uint nsb = K >> 8, lane = threadIdx.x & 63u;
     const uint seg = blockIdx.x * 4u + (threadIdx.x >> 6);
     const uint m = seg / nsb, sb = seg - m * nsb;
     if (m >= MP) return;
     if (m >= M) {
-        if (lane == 0) {
-            xst[(size_t)sb * MP + m] = 0.0f;
-            *(uint4*)(sums + ((size_t)sb * MP + m) * 16u) = make_uint4(0u, 0u, 0u, 0u);
-        }
+        if (lane == 0) xst[(size_t)sb * MP + m] = 0.0f;
+        if (lane < 8u) sums[((size_t)sb * MP + m) * 8u + lane] = 0.0f;
         return;
     }
     const size_t i = (size_t)seg * 256u + lane * 4u;
@@ -572,25 +574,19 @@ __device__ __forceinline__ void quantize_q8k_sides_body(const void* __restrict__
     s32 += dpp_i32<OJK_DPP_QUAD_XOR1>(s32);
     s32 += dpp_i32<OJK_DPP_QUAD_XOR2>(s32);
     s32 += dpp_i32<OJK_DPP_ROW_HALF_MIRROR>(s32);
-    uint lo[2] = {0u, 0u}, hi[2] = {0u, 0u};
-#pragma unroll
-    for (int jj = 0; jj < 8; jj++) {
-        const int bs = __builtin_amdgcn_readlane(s32, 8 * jj);
-        lo[jj >> 2] |= (uint)(bs & 63) << (8 * (jj & 3));
-        hi[jj >> 2] |= ((uint)(bs >> 6) & 0xFFu) << (8 * (jj & 3));
-    }
+    // lane 8 j holds the sum of run j, which goes to position 2 (j % 4) + j / 4
+    if ((lane & 7u) == 0) sums[((size_t)sb * MP + m) * 8u + ((lane >> 2) & 6u) + (lane >> 5)] = __fmul_rn(scale, (float)s32);
     if (lane == 0) {
         scales[seg] = scale;
         xst[(size_t)sb * MP + m] = scale;
-        *(uint4*)(sums + ((size_t)sb * MP + m) * 16u) = make_uint4(lo[0], lo[1], hi[0], hi[1]);
     }
 }
 extern "C" __global__ void __launch_bounds__(256)
-quantize_q8k_sides(const float* x, signed char* q, float* scales, float* xst, uchar* sums, uint K, uint M, uint MP) {
+quantize_q8k_sides(const float* x, signed char* q, float* scales, float* xst, float* sums, uint K, uint M, uint MP) {
     quantize_q8k_sides_body<false>(x, q, scales, xst, sums, K, M, MP);
 }
 extern "C" __global__ void __launch_bounds__(256)
-quantize_q8k_bf16_sides(const ushort* x, signed char* q, float* scales, float* xst, uchar* sums, uint K, uint M, uint MP) {
+quantize_q8k_bf16_sides(const ushort* x, signed char* q, float* scales, float* xst, float* sums, uint K, uint M, uint MP) {
     quantize_q8k_sides_body<true>(x, q, scales, xst, sums, K, M, MP);
 }
 
@@ -598,14 +594,16 @@ __device__ __forceinline__ void gxt_copy16(const void* base, uint voff, uint lds
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr) : "memory");
 }
 
-// the two planes of one 16-row tile's super-block: BA = (sc & 7) * code, BB = (sc >> 3) * code, a chunk per register quad
-__device__ __forceinline__ void gxt_planes(const GqW& w, gq_i4 (&BA)[4], gq_i4 (&BB)[4], long& Bm, float& d, float& dmin, uint kg) {
+// the two planes of one 16-row tile's super-block: BA = (sc & 7) * code, BB = (sc >> 3) * code, a chunk per register quad;
+// and the row's side of the min term for the f32 matrix unit: n0 = -dmin * m[kg], n1 = -dmin * m[kg + 4] (sh = 8 kg)
+__device__ __forceinline__ void gxt_planes(const GqW& w, gq_i4 (&BA)[4], gq_i4 (&BB)[4], float& n0, float& n1, float& d, uint sh) {
     d = f16_bits_to_f32(w.hdr.x & 0xFFFFu);
-    dmin = f16_bits_to_f32(w.hdr.x >> 16);
+    const float ndmin = -f16_bits_to_f32(w.hdr.x >> 16);
     const uint sc_lo = w.hdr.y & 0x3F3F3F3Fu, mn_lo = w.hdr.z & 0x3F3F3F3Fu;
     const uint sc_hi = (w.hdr.w & 0x0F0F0F0Fu) | ((w.hdr.y >> 2) & 0x30303030u);
     const uint mn_hi = ((w.hdr.w >> 4) & 0x0F0F0F0Fu) | ((w.hdr.z >> 2) & 0x30303030u);
-    Bm = kg == 0u ? gq_pack(mn_lo, mn_hi) : 0;
+    n0 = __fmul_rn(ndmin, (float)((mn_lo >> sh) & 0xFFu));
+    n1 = __fmul_rn(ndmin, (float)((mn_hi >> sh) & 0xFFu));
 #pragma unroll
     for (int c = 0; c < 4; c++) {
         const uint se = 2 * c < 4 ? (sc_lo >> (16 * c)) & 0xFFu : (sc_hi >> (16 * (c - 2))) & 0xFFu;
@@ -625,7 +623,7 @@ __device__ __forceinline__ void gxt_planes(const GqW& w, gq_i4 (&BA)[4], gq_i4 (
 // every CU a 128-row tile.
 template <int TH>
 __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restrict__ xq, const float* __restrict__ xst,
-                                                     const uchar* __restrict__ sums, const uchar* __restrict__ w,
+                                                     const float* __restrict__ sums, const uchar* __restrict__ w,
                                                      float* __restrict__ y, uint K, uint N, uint M, uint ACC, uint MP, uchar* lds) {
     constexpr int P = 8 / TH;
     constexpr uint RT = 8u / TH;                                    // row tiles per workgroup
@@ -638,8 +636,8 @@ __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restri
     const gq_i4 zero = {0, 0, 0, 0};
 
     // copies of one step: 32 of 1 KB for the tokens (wave w takes tokens 16 w .. 16 w + 15, four per copy: lane ->
-    // token lane / 16 of the four, slot lane % 16, which holds the token's piece slot ^ (token % 16)), two for the
-    // split sums (128 tokens x 16 bytes, contiguous in `sums`), one of 512 bytes for the scales.
+    // token lane / 16 of the four, slot lane % 16, which holds the token's piece slot ^ (token % 16)), four for the
+    // scaled sums (128 tokens x 32 bytes, contiguous in `sums`), one of 512 bytes for the scales.
     const uint lane16 = lane * 16u;
     const uint x_lds = lds0 + wave * 4096u;                        // + stage * GXT_STAGE + i * 1024
     auto copies = [&](uint sb, uint stage) {
@@ -654,20 +652,18 @@ __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restri
             const uint tg = min(t0 + tk, M - 1u);                  // tokens past M: any row (their sides are zeros)
             gxt_copy16(xb, tg * K + (((lo & 15u) ^ (tk & 15u)) << 4), x_lds + stage * GXT_STAGE + (uint)i * 1024u);
         }
-        if (wave < 2u) gxt_copy16(sums + ((size_t)sb * MP + t0) * 16u + wave * 1024u, lane16,
+        if (wave < 4u) gxt_copy16((const uchar*)sums + ((size_t)sb * MP + t0) * 32u + wave * 1024u, lane16,
                                   lds0 + stage * GXT_STAGE + GXT_TOK * 256u + wave * 1024u);
-        else if (wave == 2u) {
-            if (lane < 32u) gxt_copy16(xst + (size_t)sb * MP + t0, lane16, lds0 + stage * GXT_STAGE + GXT_TOK * 272u);
+        else if (wave == 4u) {
+            if (lane < 32u) gxt_copy16(xst + (size_t)sb * MP + t0, lane16, lds0 + stage * GXT_STAGE + GXT_TOK * 288u);
         }
     };
     // this lane's row (clamped past N; a 32-bit byte offset from a uniform base: the tensor stays below 4 GiB)
     const uint wrow = min(r0 + n, N - 1u) * nsb * Q4K_BYTES;
 
-    float acc[P][4];
+    gq_f4 acc[P];
 #pragma unroll
-    for (int p = 0; p < P; p++)
-#pragma unroll
-        for (int v = 0; v < 4; v++) acc[p][v] = 0.0f;
+    for (int p = 0; p < P; p++) acc[p] = (gq_f4){0.0f, 0.0f, 0.0f, 0.0f};
 
     // byte offsets of the lane's pieces within a token row, per chunk: pieces 4 c + kg / 2 (first sub-block) and
     // 4 c + 2 + kg / 2 (second), slot = piece ^ (token % 16), half kg % 2
@@ -676,10 +672,10 @@ __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restri
     uint o0[4];
 #pragma unroll
     for (int c = 0; c < 4; c++) o0[c] = tok_lds + (((4u * (uint)c + (kg >> 1)) ^ n) << 4);
-    const uint side_lds = GXT_TOK * 256u + (th * (16u * P) + n) * 16u, sc_lds = GXT_TOK * 272u + (th * (16u * P) + 4u * kg) * 4u;
-    // (only positions 0..7 carry split sums; masked rather than branched over: a branch inside the unrolled passes cuts
-    // the step into many basic blocks, which the register allocator answers with spills)
-    const long kmask = kg == 0u ? -1l : 0l;
+    // the lane's two scaled sums of its token (runs kg and kg + 4 sit side by side), and the scales of the four tokens
+    // whose results it holds
+    const uint side_lds = GXT_TOK * 256u + (th * (16u * P) + n) * 32u + 8u * kg, sc_lds = GXT_TOK * 288u + (th * (16u * P) + 4u * kg) * 4u;
+    const uint sh = 8u * kg;
 
     GqW cur = gq_load(w + wrow, kg);
     copies(0u, 0u);
@@ -691,9 +687,8 @@ __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restri
         const uint sbn = min(sb + 1u, nsb - 1u);
         const uchar* st = lds + stage * GXT_STAGE;
         gq_i4 BA[4], BB[4];
-        long Bm;
-        float d, dmin;
-        gxt_planes(cur, BA, BB, Bm, d, dmin, kg);
+        float n0, n1, d;
+        gxt_planes(cur, BA, BB, n0, n1, d, sh);
         __builtin_amdgcn_sched_barrier(0);
         // the next step's weights take over the registers of this step's raw bytes, which the planes have replaced
         cur = gq_load((w + (size_t)sbn * Q4K_BYTES) + wrow, kg);
@@ -702,6 +697,10 @@ __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restri
         for (int p = 0; p < P; p++) {
             // (one accumulation chain per plane: the two chains alternate, which is distance enough between dependent
             // MFMAs here, and saves the registers and the additions of split chains)
+            // the min term goes straight onto the sums through the f32 matrix unit: - sum_j (xs bsum_j) (dmin m_j)
+            const float2 am = *(const float2*)(st + side_lds + 512u * (uint)p);
+            acc[p] = __builtin_amdgcn_mfma_f32_16x16x4f32(am.x, n0, acc[p], 0, 0, 0);
+            acc[p] = __builtin_amdgcn_mfma_f32_16x16x4f32(am.y, n1, acc[p], 0, 0, 0);
             gq_i4 DA = zero, DB = zero;
 #pragma unroll
             for (int c = 0; c < 4; c++) {
@@ -710,17 +709,10 @@ __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restri
                 DA = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, BA[c], DA, 0, 0, 0);
                 DB = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, BB[c], DB, 0, 0, 0);
             }
-            const uchar* pq = st + side_lds + 256u * (uint)p;
-            const long Alo = *(const long*)pq & kmask, Ahi = *(const long*)(pq + 8) & kmask;
             const float4 sx = *(const float4*)(st + sc_lds + 64u * (uint)p);
             const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
-            const gq_i4 Dlo = __builtin_amdgcn_mfma_i32_16x16x32_i8(Alo, Bm, zero, 0, 0, 0);
-            const gq_i4 Dhi = __builtin_amdgcn_mfma_i32_16x16x32_i8(Ahi, Bm, zero, 0, 0, 0);
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int isum = 8 * DB[v] + DA[v];
-                acc[p][v] += sxv[v] * (d * (float)isum - dmin * (float)(64 * Dhi[v] + Dlo[v]));
-            }
+            for (int v = 0; v < 4; v++) acc[p][v] += sxv[v] * (d * (float)(8 * DB[v] + DA[v]));
             // (keeps the passes apart: let loose, the scheduler hoists every pass's reads to the front)
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -741,13 +733,13 @@ __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restri
 }
 
 extern "C" __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
-gemm_q8k_q4k_xt(const signed char* xq, const float* xst, const uchar* sums, const uchar* w, float* y, uint K, uint N, uint M,
+gemm_q8k_q4k_xt(const signed char* xq, const float* xst, const float* sums, const uchar* w, float* y, uint K, uint N, uint M,
                 uint ACC, uint MP) {
     __shared__ __attribute__((aligned(1024))) uchar lds_xt[2 * GXT_STAGE];
     gemm_q8k_q4k_xt_body<1>(xq, xst, sums, w, y, K, N, M, ACC, MP, lds_xt);
 }
 extern "C" __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
-gemm_q8k_q4k_xt64(const signed char* xq, const float* xst, const uchar* sums, const uchar* w, float* y, uint K, uint N, uint M,
+gemm_q8k_q4k_xt64(const signed char* xq, const float* xst, const float* sums, const uchar* w, float* y, uint K, uint N, uint M,
                   uint ACC, uint MP) {
     __shared__ __attribute__((aligned(1024))) uchar lds_xt[2 * GXT_STAGE];
     gemm_q8k_q4k_xt_body<2>(xq, xst, sums, w, y, K, N, M, ACC, MP, lds_xt);

@@ -11,6 +11,7 @@
 //   copy_{bf16,f32}_half_zero(x, y, z, n, nz, CB)  the conversion and a zero fill of nz dwords at z in one launch
 //   stream_copy_u32x4(x, y, n16)  y = x for n16 16-byte units: a copy of known size
 //   stream_read_u32x4(x, y, n16)  reads n16 16-byte units, writes one dword per wave (y: grid*4 dwords)
+//   calib_mfma_i8(x, y, iters, mode)   the same for v_mfma_i32_16x16x64_i8 (modes 0 and 1)
 //   calib_mfma_f16(x, y, iters, mode)  matrix-pipe calibration: what v_mfma_f32_32x32x16_f16 sustains on the
 //                            operands found in x (32 KB: a workgroup's 8 fragments per thread), one wave per SIMD,
 //                            16 independent accumulator blocks per wave as in the prefill tile; mode 0 keeps the
@@ -199,6 +200,60 @@ __device__ __forceinline__ void calib_mfma_body(uint4* tile, const uint4* __rest
 #pragma unroll
     for (int i = 0; i < 5; i++) sum += (float)va[i][0] + (float)va[i][1];
     y[blockIdx.x * 256u + tid] = __float_as_uint(sum);
+}
+
+// The same for the int8 matrix instruction of the prefill tiles in the CPU path's arithmetic: v_mfma_i32_16x16x64_i8,
+// 2 * 16 * 16 * 64 operations each, 64 per trip over 16 independent sums; mode 0 operands in registers, mode 1 read
+// back from LDS per group of 16.  ops = grid * 4 * iters * 64 * 32768.
+typedef int cal_i32x4 __attribute__((ext_vector_type(4)));
+template <int mode>
+__device__ __forceinline__ void calib_mfma_i8_body(uint4* tile, const uint4* __restrict__ x, uint* __restrict__ y, uint iters) {
+    const uint tid = threadIdx.x;
+    cal_i32x4 a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 8; i++) tile[i * 256 + tid] = x[i * 256 + tid];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        a[i] = __builtin_bit_cast(cal_i32x4, tile[i * 256 + tid]);
+        b[i] = __builtin_bit_cast(cal_i32x4, tile[(4 + i) * 256 + tid]);
+    }
+    cal_i32x4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = (cal_i32x4){0, 0, 0, 0};
+    for (uint t = 0; t < iters; t++) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            if (mode) {
+                const uint s = (tid + 64u * ((t + ks) & 3u)) & 255u;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    a[i] = __builtin_bit_cast(cal_i32x4, tile[i * 256 + s]);
+                    b[i] = __builtin_bit_cast(cal_i32x4, tile[(4 + i) * 256 + s]);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) sum += acc[i][j][v];
+    y[blockIdx.x * 256u + tid] = (uint)sum;
+}
+extern "C" __global__ void __launch_bounds__(256)
+calib_mfma_i8(const uint4* __restrict__ x, uint* __restrict__ y, uint iters, uint mode) {
+    __shared__ __attribute__((aligned(1024))) uint4 tile[8 * 256];
+    if (mode == 0) calib_mfma_i8_body<0>(tile, x, y, iters);
+    else calib_mfma_i8_body<1>(tile, x, y, iters);
 }
 
 extern "C" __global__ void __launch_bounds__(256)

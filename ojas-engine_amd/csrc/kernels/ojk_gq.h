@@ -4,6 +4,7 @@
 #include "ojk_common.h"
 
 typedef int gq_i4 __attribute__((ext_vector_type(4)));
+typedef float gq_f4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ long gq_pack(uint lo, uint hi) { return (long)(((unsigned long)hi << 32) | lo); }
 

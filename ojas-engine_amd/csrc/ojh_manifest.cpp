@@ -228,7 +228,7 @@ static int check_gemm_q8k_xt(const ojh_kernel_spec *s, const uint32_t *c, const 
         need[0] = (size_t)M * K;
         need[1] = (size_t)M * nsb * 4;
         need[2] = nsb * MP * 4;
-        need[3] = nsb * MP * 16;
+        need[3] = nsb * MP * 32;
         align[1] = align[2] = 4;
         return OJH_OK;
     }
@@ -240,7 +240,7 @@ static int check_gemm_q8k_xt(const ojh_kernel_spec *s, const uint32_t *c, const 
     if ((uint64_t)N * nsb * 144 > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "%s: the weight tensor exceeds 4 GiB", s->name);
     need[0] = (size_t)M * K;
     need[1] = nsb * MP * 4;
-    need[2] = nsb * MP * 16;
+    need[2] = nsb * MP * 32;
     need[3] = (size_t)N * nsb * 144;
     need[4] = (size_t)M * N * 4;
     align[1] = align[4] = 4;
@@ -263,7 +263,7 @@ static int check_quantize_sides(const ojh_kernel_spec *s, const uint32_t *c, con
     need[1] = (size_t)M * K;
     need[2] = (size_t)M * nsb * 4;
     need[3] = nsb * MP * 4;
-    need[4] = nsb * MP * 16;
+    need[4] = nsb * MP * 32;
     align[0] = 4 * esz;
     align[1] = align[2] = align[3] = 4;
     return OJH_OK;
@@ -1318,7 +1318,7 @@ static int check_calib_mfma(const ojh_kernel_spec *s, const uint32_t *c, const u
                             const uint32_t block[3], size_t need[16], size_t align[16]) {
     (void)align;
     if (!c[0] || c[0] > (1u << 20)) return ojh_fail(OJH_ERR_ARG, "%s: iters=%u out of range (1 .. 2^20)", s->name, c[0]);
-    if (c[1] > 2) return ojh_fail(OJH_ERR_ARG, "%s: mode=%u (0 = operands in registers, 1 = read from LDS, 2 = with a tile step's copies, LDS writes and vector ALU work)", s->name, c[1]);
+    if (c[1] > (strstr(s->name, "_i8") ? 1u : 2u)) return ojh_fail(OJH_ERR_ARG, "%s: mode=%u (0 = operands in registers, 1 = read from LDS, 2 = with a tile step's copies, LDS writes and vector ALU work)", s->name, c[1]);
     int rc = check_block(block, 256);
     if (rc) return rc;
     if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
@@ -1608,6 +1608,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("stream_copy_u32x4", "glue", 2, 1, 0, 0, check_stream, shape_stream);
     add("stream_read_u32x4", "glue", 2, 1, 1, 0, check_stream, shape_stream);
     add("calib_mfma_f16", "glue", 2, 2, 0, 0, check_calib_mfma, shape_calib_mfma);
+    add("calib_mfma_i8", "glue", 2, 2, 0, 0, check_calib_mfma, shape_calib_mfma);
     return m;
 }
 

@@ -191,7 +191,7 @@ int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, con
         const size_t nsb = K / 256;
         ojh_buf *xst, *sums;
         if ((rc = ojh_scratch_get(dev, "xt_xst", nsb * mp * 4, &xst))) return rc;
-        if ((rc = ojh_scratch_get(dev, "xt_sums", nsb * mp * 16, &sums))) return rc;
+        if ((rc = ojh_scratch_get(dev, "xt_sums", nsb * mp * 32, &sums))) return rc;
         uint32_t sg[3], sb[3];
         if (!sides_ready) {
             if ((rc = ojh_launch_shape(dev, "q8k_token_sides", K, N, m, sg, sb))) return rc;
@@ -612,7 +612,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
             const uint32_t mp = (m + 127) / 128 * 128;
             ojh_buf *xst, *sums;
             if ((rc = ojh_scratch_get(dev, "xt_xst", nsb * mp * 4, &xst))) return rc;
-            if ((rc = ojh_scratch_get(dev, "xt_sums", nsb * mp * 16, &sums))) return rc;
+            if ((rc = ojh_scratch_get(dev, "xt_sums", nsb * mp * 32, &sums))) return rc;
             uint32_t qg[3] = {K / 256 * (mp / 4), 1, 1};
             if ((rc = ojh_launch(dev, x_dtype == OJH_X_BF16 ? "quantize_q8k_bf16_sides" : "quantize_q8k_sides",
                                  {at(x, x_off), xq->ptr, xs->ptr, xst->ptr, sums->ptr}, {K, m, mp}, qg, block)))

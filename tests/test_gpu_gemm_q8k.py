@@ -153,8 +153,8 @@ def test_a_token_does_not_depend_on_its_batch(gpu, pkg):
 @pytest.mark.parametrize("m,n,k", [(130, 200, 512), (128, 128, 256), (300, 77, 2048), (97, 1000, 4096)])
 def test_prefill_tiles_by_name(gpu, orc, pkg, m, n, k):
     """`q8k_token_sides` + `gemm_q8k_q4k_xt` / `_xt64` by name: ragged tokens and rows, plain store and accumulate,
-    nothing written past row M — against matvec_kq and, bit for bit, against `gemm_q8k_q4k_mf` with one wave per row
-    tile over all of K (RW = 4: super-blocks added in order there too)."""
+    nothing written past row M — against matvec_kq and (a few ulp: the min term is associated per 32-position run
+    there, per super-block here) against `gemm_q8k_q4k_mf`; the two tile heights give the same bits."""
     w, x = _case(pkg, m, n, k, "xt")
     gpu.ensure_family("gemm_q8k")
     gpu.ensure_family("gemv_q8k")
@@ -162,33 +162,34 @@ def test_prefill_tiles_by_name(gpu, orc, pkg, m, n, k):
     xq, xs = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
     gpu.quant_q8k(gpu.upload(x), m, k, xq, xs)
     wd = gpu.upload_bytes(w)
-    xst, sums = gpu.alloc(nsb * mp), gpu.alloc_bytes(nsb * mp * 16)
+    xst, sums = gpu.alloc(nsb * mp), gpu.alloc(nsb * mp * 8)
     gpu.dispatch(gpu.begin(), "q8k_token_sides", [(xq, 0), (xs, 0), (xst, 0), (sums, 0)], [k, m, mp], [nsb, (mp + 255) // 256, 1], [256, 1, 1])
-    # the side arrays: scales transposed, sums split as 64 hi + lo, zeros past row M
+    # the side arrays: scales transposed; scale x the sum of every 32-position run, runs in the order 0 4 1 5 2 6 3 7;
+    # zeros past row M
     q = gpu.read(xq, m * k, np.int8).reshape(m, nsb, 8, 32).astype(np.int32).sum(3)
-    sd = gpu.read(sums, nsb * mp * 16, np.int8).reshape(nsb, mp, 2, 8).astype(np.int32)
-    assert np.array_equal(64 * sd[:, :m, 1] + sd[:, :m, 0], q.transpose(1, 0, 2)) and not sd[:, m:].any()
-    assert np.all((sd[:, :, 0] >= 0) & (sd[:, :, 0] < 64))
     st = gpu.read(xst, nsb * mp).reshape(nsb, mp)
     assert np.array_equal(st[:, :m], gpu.read(xs, m * nsb).reshape(m, nsb).T) and not st[:, m:].any()
+    sd = gpu.read(sums, nsb * mp * 8).reshape(nsb, mp, 8)
+    scaled = st[:, :m, None] * q.transpose(1, 0, 2)[:, :, [0, 4, 1, 5, 2, 6, 3, 7]].astype(np.float32)
+    assert np.array_equal(sd[:, :m].view(np.uint32), scaled.astype(np.float32).view(np.uint32)) and not sd[:, m:].any()
     # the quantizer that leaves the side arrays as well: the same bytes in all four outputs, from f32 and from bf16 tokens
     xb = (x.view(np.uint32) >> 16).astype(np.uint16)
     for name, src in (("quantize_q8k_sides", gpu.upload(x)), ("quantize_q8k_bf16_sides", gpu.upload_bytes(xb))):
         q2, s2 = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
         xst2 = gpu.upload(np.full(nsb * mp, 7.5, np.float32))
-        sums2 = gpu.upload_bytes(np.full(nsb * mp * 16, 0x55, np.uint8))
+        sums2 = gpu.upload(np.full(nsb * mp * 8, 7.5, np.float32))
         gpu.dispatch(gpu.begin(), name, [(src, 0), (q2, 0), (s2, 0), (xst2, 0), (sums2, 0)], [k, m, mp], [nsb * mp // 4, 1, 1], [256, 1, 1])
         if "bf16" in name:
             q1, s1 = gpu.alloc_bytes(m * k), gpu.alloc(m * nsb)
             gpu.quant_q8k(gpu.upload((xb.astype(np.uint32) << 16).view(np.float32)), m, k, q1, s1)
-            xst1, sums1 = gpu.alloc(nsb * mp), gpu.alloc_bytes(nsb * mp * 16)
+            xst1, sums1 = gpu.alloc(nsb * mp), gpu.alloc(nsb * mp * 8)
             gpu.dispatch(gpu.begin(), "q8k_token_sides", [(q1, 0), (s1, 0), (xst1, 0), (sums1, 0)], [k, m, mp], [nsb, (mp + 255) // 256, 1], [256, 1, 1])
         else:
             q1, s1, xst1, sums1 = xq, xs, xst, sums
         assert np.array_equal(gpu.read(q2, m * k, np.int8), gpu.read(q1, m * k, np.int8)), name
         assert np.array_equal(gpu.read(s2, m * nsb).view(np.uint32), gpu.read(s1, m * nsb).view(np.uint32)), name
         assert np.array_equal(gpu.read(xst2, nsb * mp).view(np.uint32), gpu.read(xst1, nsb * mp).view(np.uint32)), name
-        assert np.array_equal(gpu.read(sums2, nsb * mp * 16, np.uint8), gpu.read(sums1, nsb * mp * 16, np.uint8)), name
+        assert np.array_equal(gpu.read(sums2, nsb * mp * 8).view(np.uint32), gpu.read(sums1, nsb * mp * 8).view(np.uint32)), name
     with pytest.raises(pkg.OjasHipError, match="rounded up to 128"):
         gpu.dispatch(gpu.begin(), "quantize_q8k_sides", [(gpu.upload(x), 0), (xq, 0), (xs, 0), (xst, 0), (sums, 0)], [k, m, mp + 128],
                      [nsb * (mp + 128) // 4, 1, 1], [256, 1, 1])
@@ -196,7 +197,7 @@ def test_prefill_tiles_by_name(gpu, orc, pkg, m, n, k):
     ymf = gpu.alloc(m * n)
     gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_mf", [(xq, 0), (xs, 0), (wd, 0), (ymf, 0)], [k, n, m, 0, 4, 1],
                  [(n + 63) // 64, (m + 63) // 64, 1], [256, 1, 1])
-    ref = gpu.read(ymf, m * n).reshape(m, n)
+    ref, bits = gpu.read(ymf, m * n).reshape(m, n), {}
     for name, br in (("gemm_q8k_q4k_xt", 128), ("gemm_q8k_q4k_xt64", 64)):
         for acc in (0, 1):
             y0 = pkg.synth.normal_f32(m * n, "gq", "xt-y0", acc).reshape(m, n)
@@ -209,8 +210,9 @@ def test_prefill_tiles_by_name(gpu, orc, pkg, m, n, k):
             if acc:
                 assert peak_err(got - y0, want) <= TOL_SEEN
             else:
-                assert peak_err(got, want) <= TOL_SEEN
-                assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), name
+                assert peak_err(got, want) <= TOL_SEEN and peak_err(got, ref) <= 2e-6
+                bits[name] = got.view(np.uint32).copy()
+    assert np.array_equal(bits["gemm_q8k_q4k_xt"], bits["gemm_q8k_q4k_xt64"])
     with pytest.raises(pkg.OjasHipError, match="rounded up to 128"):
         gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_xt", [(xq, 0), (xst, 0), (sums, 0), (wd, 0), (ymf, 0)], [k, n, m, 0, mp + 128],
                      [(n + 127) // 128, mp // 128, 1], [512, 1, 1])
