@@ -75,6 +75,32 @@ __device__ __forceinline__ void iqg_signed(uint2 m, uint sg, IqgFrag& f) {
     f.w0 = iqg_apply_signs(m.x, sg & 15u);
     f.w1 = iqg_apply_signs(m.y, sg >> 4);
 }
+// The 128-entry sign table expanded in LDS: entry i = eight byte masks, 0xFF where weight j of the group is negative
+// (bit j of i, and for j = 7 the bit that makes the parity even).  iqg_signs_init(), then a barrier, then
+// iqg_masked(m, iqg_sign_masks()[i]) = the magnitudes m with those signs: (m ^ s) - s byte by byte, and since m > 0 no
+// byte borrows from the next.
+__device__ __forceinline__ uint2* iqg_sign_masks() { __shared__ uint2 tab[128]; return tab; }
+__device__ __forceinline__ void iqg_signs_init() {
+    uint2* t = iqg_sign_masks();
+    for (uint i = threadIdx.x; i < 128u; i += blockDim.x) {
+        const uint sg = iqg_ksigns(i), lo = sg & 15u, hi = sg >> 4;
+        const uint l4 = (lo & 1u) | ((lo & 2u) << 7) | ((lo & 4u) << 14) | ((lo & 8u) << 21);
+        const uint h4 = (hi & 1u) | ((hi & 2u) << 7) | ((hi & 4u) << 14) | ((hi & 8u) << 21);
+        t[i] = make_uint2(l4 * 0xFFu, h4 * 0xFFu);
+    }
+}
+__device__ __forceinline__ uint iqg_masked(uint m, uint s) { return (m ^ s) + (s & 0x01010101u); }
+// ... and the same for the formats that store a raw sign byte per group (IQ2_S, IQ3_S): 256 entries
+__device__ __forceinline__ uint2* iqg_sign_masks256() { __shared__ uint2 tab[256]; return tab; }
+__device__ __forceinline__ void iqg_signs256_init() {
+    uint2* t = iqg_sign_masks256();
+    for (uint i = threadIdx.x; i < 256u; i += blockDim.x) {
+        const uint lo = i & 15u, hi = i >> 4;
+        const uint l4 = (lo & 1u) | ((lo & 2u) << 7) | ((lo & 4u) << 14) | ((lo & 8u) << 21);
+        const uint h4 = (hi & 1u) | ((hi & 2u) << 7) | ((hi & 4u) << 14) | ((hi & 8u) << 21);
+        t[i] = make_uint2(l4 * 0xFFu, h4 * 0xFFu);
+    }
+}
 
 struct Iq2xxsG {   // { f16 d; u16 qs[32] }: per sub-block 4 index bytes, then 4 x 7 sign-table bits + a 4-bit scale
     static constexpr uint BYTES = IQ2XXS_BYTES;
@@ -87,6 +113,22 @@ struct Iq2xxsG {   // { f16 d; u16 qs[32] }: per sub-block 4 index bytes, then 4
         f.delta = 0.0f;
         iqg_signed(entry<LDS>((a0 >> (8u * l)) & 255u), iqg_ksigns(a1 >> (7u * l)), f);
         return f;
+    }
+    // One lane, one 32-weight sub-block against its 32 int8 activations: d * scale * idot32, the integer dot exact
+    // (after init(), iqg_signs_init() and a barrier).
+    // One lane, one 32-weight sub-block (after init(), signs_init() and a barrier): its weights as signed bytes, four to
+    // a word, and the scale of its first and second sixteen.
+    static __device__ __forceinline__ void signs_init() { iqg_signs_init(); }
+    static __device__ __forceinline__ void vals32(const uchar* blk, uint ib, uint (&w)[8], float& dl0, float& dl1) {
+        const u32x2_a2 a = *(const u32x2_a2*)(blk + 2u + 8u * ib);
+        const uint2* sm = iqg_sign_masks();
+#pragma unroll
+        for (uint l = 0; l < 4u; l++) {
+            const uint2 m = table()[(a.x >> (8u * l)) & 255u], s = sm[(a.y >> (7u * l)) & 127u];
+            w[2 * l] = iqg_masked(m.x, s.x);
+            w[2 * l + 1] = iqg_masked(m.y, s.y);
+        }
+        dl0 = dl1 = f16_bits_to_f32(*(const ushort*)blk) * ((0.5f + (float)(a.y >> 28)) * 0.25f);
     }
 };
 struct Iq2xsG {    // { f16 d; u16 qs[32]; u8 scales[8] }: 9 index bits + 7 sign-table bits per group, a scale nibble per 16
@@ -114,6 +156,21 @@ struct Iq2sG {     // { f16 d; u8 qs[32]; u8 signs[32]; u8 qh[8]; u8 scales[8] }
         iqg_signed(entry<LDS>(idx), blk[34u + t], f);
         return f;
     }
+    static __device__ __forceinline__ void signs_init() { iqg_signs256_init(); }
+    static __device__ __forceinline__ void vals32(const uchar* blk, uint ib, uint (&w)[8], float& dl0, float& dl1) {
+        const uint lo = *(const u32_a2*)(blk + 2u + 4u * ib), sg = *(const u32_a2*)(blk + 34u + 4u * ib);
+        const uint h = blk[66u + ib], sc = blk[74u + ib];
+        const uint2* sm = iqg_sign_masks256();
+#pragma unroll
+        for (uint l = 0; l < 4u; l++) {
+            const uint2 m = table()[((lo >> (8u * l)) & 255u) | ((h << (8u - 2u * l)) & 0x300u)], s = sm[(sg >> (8u * l)) & 255u];
+            w[2 * l] = iqg_masked(m.x, s.x);
+            w[2 * l + 1] = iqg_masked(m.y, s.y);
+        }
+        const float d = f16_bits_to_f32(*(const ushort*)blk);
+        dl0 = d * ((0.5f + (float)(sc & 15u)) * 0.25f);
+        dl1 = d * ((0.5f + (float)(sc >> 4)) * 0.25f);
+    }
 };
 struct Iq3xxsG {   // { f16 d; u8 qs[64]; u32 ss[8] }: two 4-weight entries per group; ss as IQ2_XXS's second word
     static constexpr uint BYTES = IQ3XXS_BYTES;
@@ -127,6 +184,21 @@ struct Iq3xxsG {   // { f16 d; u8 qs[64]; u32 ss[8] }: two 4-weight entries per 
         f.delta = 0.0f;
         iqg_signed(make_uint2(entry<LDS>(q & 255u), entry<LDS>(q >> 8)), sg, f);
         return f;
+    }
+    static __device__ __forceinline__ void signs_init() { iqg_signs_init(); }
+    static __device__ __forceinline__ void vals32(const uchar* blk, uint ib, uint (&w)[8], float& dl0, float& dl1) {
+        const u32x2_a2 ix = *(const u32x2_a2*)(blk + 2u + 8u * ib);
+        const uint a = *(const u32_a2*)(blk + 66u + 4u * ib);
+        const uint2* sm = iqg_sign_masks();
+        const uint* tb = table();
+#pragma unroll
+        for (uint l = 0; l < 4u; l++) {
+            const uint q = l < 2u ? ix.x >> (16u * l) : ix.y >> (16u * (l - 2u));
+            const uint2 s = sm[(a >> (7u * l)) & 127u];
+            w[2 * l] = iqg_masked(tb[q & 255u], s.x);
+            w[2 * l + 1] = iqg_masked(tb[(q >> 8) & 255u], s.y);
+        }
+        dl0 = dl1 = f16_bits_to_f32(*(const ushort*)blk) * ((0.5f + (float)(a >> 28)) * 0.5f);
     }
 };
 struct Iq3sG {     // { f16 d; u8 qs[64]; u8 qh[8]; u8 signs[32]; u8 scales[4] }: 9 index bits, raw signs, scale 1 + 2 s
@@ -142,6 +214,22 @@ struct Iq3sG {     // { f16 d; u8 qs[64]; u8 qh[8]; u8 signs[32]; u8 scales[4] }
         f.delta = 0.0f;
         iqg_signed(make_uint2(entry<LDS>(i1), entry<LDS>(i2)), sg, f);
         return f;
+    }
+    static __device__ __forceinline__ void signs_init() { iqg_signs256_init(); }
+    static __device__ __forceinline__ void vals32(const uchar* blk, uint ib, uint (&w)[8], float& dl0, float& dl1) {
+        const u32x2_a2 ix = *(const u32x2_a2*)(blk + 2u + 8u * ib);
+        const uint sg = *(const u32_a2*)(blk + 74u + 4u * ib), h = blk[66u + ib];
+        const uint sc = ((uint)blk[106u + (ib >> 1)] >> (4u * (ib & 1u))) & 15u;
+        const uint2* sm = iqg_sign_masks256();
+        const uint* tb = table();
+#pragma unroll
+        for (uint l = 0; l < 4u; l++) {
+            const uint q = l < 2u ? ix.x >> (16u * l) : ix.y >> (16u * (l - 2u));
+            const uint2 s = sm[(sg >> (8u * l)) & 255u];
+            w[2 * l] = iqg_masked(tb[(q & 255u) | ((h << (8u - 2u * l)) & 256u)], s.x);
+            w[2 * l + 1] = iqg_masked(tb[((q >> 8) & 255u) | ((h << (7u - 2u * l)) & 256u)], s.y);
+        }
+        dl0 = dl1 = f16_bits_to_f32(*(const ushort*)blk) * (1.0f + 2.0f * (float)sc);
     }
 };
 struct Iq1sG {     // { f16 d; u8 qs[32]; u16 qh[8] }: qh = 4 x 3 high index bits, a 3-bit scale, the sign of delta
