@@ -117,7 +117,7 @@ def test_entries_by_name(gpu, orc, pkg, ty):
 
 
 @pytest.mark.parametrize("ty", [IQ3_S, IQ2_S])
-@pytest.mark.parametrize("n,k,m", [(4096, 4096, 1), (37, 256, 1), (130, 2816, 5), (33001, 2816, 1)])
+@pytest.mark.parametrize("n,k,m", [(4096, 4096, 1), (37, 256, 1), (130, 2816, 5), (33001, 2816, 1), (8201, 768, 1)])
 def test_f32_rows_match_the_cpu_dots(gpu, orc, pkg, ty, n, k, m):
     """IQ3_S / IQ2_S: `matvec_kq` sends them to dot_iq3s / dot_iq2s on f32 activations; int8 activations are refused."""
     w = pkg.synth.weights(ty, n, k, "grids", n, k)
