@@ -420,12 +420,16 @@ __device__ __forceinline__ void gemv_nat_q80_m_body(const float* __restrict__ x,
 
 // ------------------------------------------------------------------ IQ4_NL, IQ4_XS and the legacy 32-weight blocks
 // (row traits Iq4nlW, Iq4xsW, Q40W, Q41W, Q50W, Q51W, Mxfp4W: ojk_rows.h)
-GEMV_NAT_IQ4_PX(iq4nl, Iq4nlW)
-GEMV_NAT_IQ4_PX(iq4xs, Iq4xsW)
-GEMV_NAT_IQ4_PX(q40, Q40W)
-GEMV_NAT_IQ4_PX(q41, Q41W)
-GEMV_NAT_IQ4_PX(q50, Q50W)
-GEMV_NAT_IQ4_PX(q51, Q51W)
+GEMV_NAT_SUB32_PX(iq4nl, Iq4nlS32)
+GEMV_NAT_SUB32_PX(iq4xs, Iq4xsS32)
+typedef LegacyS32<false, false> Q40S32;
+typedef LegacyS32<false, true> Q41S32;
+typedef LegacyS32<true, false> Q50S32;
+typedef LegacyS32<true, true> Q51S32;
+GEMV_NAT_SUB32_PX(q40, Q40S32)
+GEMV_NAT_SUB32_PX(q41, Q41S32)
+GEMV_NAT_SUB32_PX(q50, Q50S32)
+GEMV_NAT_SUB32_PX(q51, Q51S32)
 GEMV_NAT_IQ4_PX(mxfp4, Mxfp4W)
 GEMV_NAT_IQ4_PX(q5k, Q5kW)
 

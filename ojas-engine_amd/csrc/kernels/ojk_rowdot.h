@@ -122,6 +122,55 @@ __device__ __forceinline__ void gemv_nat_iq4_px_body(const float* __restrict__ x
     }
 }
 
+// The head form with a lane per 32-weight group: lane l of step s owns group l + 64 s of the row (its 16 code bytes in
+// one load where the group-per-four-lanes map above issues four narrow ones — the address unit of the vector memory
+// path takes a wave-wide load about as long whatever its width, and bounds those launches) and keeps the group's 32
+// activations, and their sum, in registers.  A trait T gives row_bytes(K) and dot32(row, group, x[8], xsum): the
+// group's term with its scale.  K <= 4096 (two steps).
+template <class T>
+__device__ __forceinline__ void gemv_nat_sub32_px_body(const float* __restrict__ x, const uchar* __restrict__ w,
+                                                       float* __restrict__ y, uint K, uint N) {
+    constexpr int NS = 2;
+    const uint lane = threadIdx.x & 63u, nsub = K >> 5;
+    const size_t rb = T::row_bytes(K);
+    float4 xr[NS][8];
+    float xsum[NS];
+    uint sc[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const uint sub = lane + 64u * (uint)s;
+        sc[s] = min(sub, nsub - 1u);
+        float t = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            xr[s][j] = sub < nsub ? *(const float4*)(x + (size_t)sub * 32u + 4u * (uint)j) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            t += (xr[s][j].x + xr[s][j].y) + (xr[s][j].z + xr[s][j].w);
+        }
+        xsum[s] = t;
+    }
+    const uint nwaves = gridDim.x * (blockDim.x >> 6);
+    for (uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2u; row0 < N; row0 += nwaves * 2u) {
+        const uchar* r0 = w + (size_t)row0 * rb;
+        const uchar* r1 = w + (size_t)min(row0 + 1u, N - 1u) * rb;
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            a0 += T::dot32(r0, sc[s], xr[s], xsum[s]);
+            a1 += T::dot32(r1, sc[s], xr[s], xsum[s]);
+        }
+        a0 = wave_sum(a0);
+        a1 = wave_sum(a1);
+        if (lane == 0) {
+            y[row0] = a0;
+            if (row0 + 1u < N) y[row0 + 1u] = a1;
+        }
+    }
+}
+#define GEMV_NAT_SUB32_PX(FMT, T)                                                                          \
+    extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))           \
+    gemv_nat_##FMT##_px(const float* x, const uchar* w, float* y, uint K, uint N) {                        \
+        gemv_nat_sub32_px_body<T>(x, w, y, K, N); }
+
 #define GEMV_NAT_IQ4_PX(FMT, W)                                                                            \
     extern "C" __global__ void __launch_bounds__(256) gemv_nat_##FMT##_px(                                 \
         const float* x, const uchar* w, float* y, uint K, uint N) {                                        \

@@ -67,6 +67,45 @@ struct Iq4nlW {
     }
 };
 
+// ... and a lane per 32-weight group, for the head form (gemv_nat_sub32_px_body): the group's 16 code bytes in one load.
+struct __attribute__((packed, aligned(4))) u32x4_a4 { uint x, y, z, w; };
+__device__ __forceinline__ float iq4_dot32(uint q0, uint q1, uint q2, uint q3, const float4 (&x)[8]) {
+    const uint q[4] = {q0, q1, q2, q3};
+    float a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint lo = iq4_levels4(q[i] & 0x0F0F0F0Fu), hi = iq4_levels4((q[i] >> 4) & 0x0F0F0F0Fu);
+        a = fmaf(sb0(lo), x[i].x, a);
+        a = fmaf(sb1(lo), x[i].y, a);
+        a = fmaf(sb2(lo), x[i].z, a);
+        a = fmaf(sb3(lo), x[i].w, a);
+        a = fmaf(sb0(hi), x[4 + i].x, a);
+        a = fmaf(sb1(hi), x[4 + i].y, a);
+        a = fmaf(sb2(hi), x[4 + i].z, a);
+        a = fmaf(sb3(hi), x[4 + i].w, a);
+    }
+    return a;
+}
+struct Iq4nlS32 {
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 5) * IQ4NL_BYTES; }
+    static __device__ __forceinline__ float dot32(const uchar* row, uint sub, const float4 (&x)[8], float) {
+        const uchar* blk = row + (size_t)sub * IQ4NL_BYTES;
+        const u32x4_a2 q = *(const u32x4_a2*)(blk + 2u);
+        return f16_bits_to_f32(*(const ushort*)blk) * iq4_dot32(q.x, q.y, q.z, q.w, x);
+    }
+};
+struct Iq4xsS32 {
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * IQ4XS_BYTES; }
+    static __device__ __forceinline__ float dot32(const uchar* row, uint sub, const float4 (&x)[8], float) {
+        const uchar* blk = row + (size_t)(sub >> 3) * IQ4XS_BYTES;
+        const uint ib = sub & 7u;
+        const uint2 h = *(const uint2*)blk;
+        const u32x4_a4 q = *(const u32x4_a4*)(blk + 8u + 16u * ib);
+        const uint ls = ((h.y >> (4u * ib)) & 0xFu) | ((((h.x >> 16) >> (2u * ib)) & 3u) << 4);
+        return f16_bits_to_f32(h.x & 0xFFFFu) * (float)((int)ls - 32) * iq4_dot32(q.x, q.y, q.z, q.w, x);
+    }
+};
+
 struct Iq4xsW {
     static constexpr uint XGAP = 16u;
     static constexpr uint STEP = 2u;             // super-blocks per step
@@ -130,6 +169,32 @@ struct LegacyW {
         const float a = dot4_ub(hi, x1, dot4_ub(lo, x0, 0.0f));
         const float d = f16_bits_to_f32(f.hdr & 0xFFFFu);
         if (AFFINE) return d * a + f16_bits_to_f32(f.hdr >> 16) * xsum;
+        return d * (a - (FIVE ? 16.0f : 8.0f) * xsum);
+    }
+};
+// ... a lane per block, for the head form
+template <bool FIVE, bool AFFINE>
+struct LegacyS32 {
+    typedef LegacyW<FIVE, AFFINE> W;
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 5) * W::BYTES; }
+    static __device__ __forceinline__ float dot32(const uchar* row, uint sub, const float4 (&x)[8], float xsum) {
+        const uchar* blk = row + (size_t)sub * W::BYTES;
+        const uint hdr = AFFINE ? *(const u32_a2*)blk : (uint)*(const ushort*)blk;
+        const uint qh = FIVE ? *(const u32_a2*)(blk + W::HDR) : 0u;
+        const u32x4_a2 qq = *(const u32x4_a2*)(blk + W::HDR + (FIVE ? 4u : 0u));
+        const uint q[4] = {qq.x, qq.y, qq.z, qq.w};
+        float a = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint lo = q[i] & 0x0F0F0F0Fu, hi = (q[i] >> 4) & 0x0F0F0F0Fu;
+            if (FIVE) {
+                lo |= W::spread4(qh, 4u * (uint)i);
+                hi |= W::spread4(qh, 4u * (uint)i + 16u);
+            }
+            a = dot4_ub(hi, x[4 + i], dot4_ub(lo, x[i], a));
+        }
+        const float d = f16_bits_to_f32(hdr & 0xFFFFu);
+        if (AFFINE) return d * a + f16_bits_to_f32(hdr >> 16) * xsum;
         return d * (a - (FIVE ? 16.0f : 8.0f) * xsum);
     }
 };
