@@ -39,9 +39,10 @@ FAMILIES = {
     "rowq8": ("rowq8.hip", ["-ffp-contract=off"]),
     "q80_dp4a": ("q80_dp4a.hip", []),
     "iq_grid": ("iq_grid.hip", ["-ffp-contract=off"]),
+    "chain": ("chain.hip", []),
 }
 
-HOST_SOURCES = ["ojh_runtime.cpp", "ojh_manifest.cpp", "ojh_ops.cpp", "ojh_moe.cpp", "ojh_gguf.cpp", "ojh_expert_cache.cpp", "ojh_noalloc.cpp"]
+HOST_SOURCES = ["ojh_runtime.cpp", "ojh_manifest.cpp", "ojh_ops.cpp", "ojh_moe.cpp", "ojh_gguf.cpp", "ojh_expert_cache.cpp", "ojh_noalloc.cpp", "ojh_chain.cpp"]
 
 
 def _newer(target: str, deps: list[str]) -> bool:
@@ -75,7 +76,8 @@ def build_kernels(force: bool = False) -> list[str]:
 
 def build_library(force: bool = False) -> str:
     srcs = [os.path.join(CSRC, s) for s in HOST_SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    deps = srcs + [os.path.join(CSRC, "ojh_internal.h"), os.path.join(HERE, "..", "include", "ojas_hip.h")]
+    deps = srcs + [os.path.join(CSRC, "ojh_internal.h"), os.path.join(HERE, "..", "include", "ojas_hip.h"),
+                   os.path.join(KERNELS, "ojk_chain.h")]
     if force or _newer(LIB, deps):
         _run([HIPCC, f"--offload-arch={ARCH}", *DEVICE_FLAGS, "-fPIC", "-shared", "-Wall", "-o", LIB, *srcs, "-ldl"])
     return LIB

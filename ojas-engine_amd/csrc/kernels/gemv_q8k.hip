@@ -20,6 +20,7 @@
 // reference's (lanes own different super-blocks), which moves the last ulp only.
 #include "ojk_common.h"
 #include "ojk_q4k_dot.h"
+#include "ojk_act.h"
 
 // ------------------------------------------------------------------ activation quantizer
 template <bool BF16>
@@ -292,13 +293,6 @@ gemv_q8k_q4k_x4_r2(const signed char* xq, const float* xs, const uchar* w0, cons
 // (:497-501).  The reference's decode path fuses the same three steps
 // (`ffn_gu_q80_dp4a`, crates/ojas-cuda/src/kernels/gemv_q8.rs:246-260); each dot is the
 // single-tensor arithmetic of gemv_q8k_q4k.
-__device__ __forceinline__ float ffn_act(float g, uint act) {
-    if (act == 1u) {
-        const float c = 0.7978845608028654f, a = 0.044715f;
-        return 0.5f * g * (1.0f + tanhf(c * g * (1.0f + a * g * g)));
-    }
-    return g / (1.0f + expf(-g));
-}
 
 extern "C" __global__ void __launch_bounds__(256)
 ffn_gu_q8k_q4k(const signed char* __restrict__ xq, const float* __restrict__ xs, const uchar* __restrict__ wg,

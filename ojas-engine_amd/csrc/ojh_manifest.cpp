@@ -1346,6 +1346,19 @@ static int shape_convert_zero(const ojh_kernel_spec *, const ojh_device *, uint3
     block[1] = block[2] = 1;
     return OJH_OK;
 }
+// decode_chain_q4k takes one argument block (kernels/ojk_chain.h), not buffers and constants: it is launched by
+// ojh_decode_chain, which validates every stage, and cannot be dispatched by name.
+static int check_chain(const ojh_kernel_spec *s, const uint32_t *, const uint32_t[3], const uint32_t[3], size_t[16], size_t[16]) {
+    return ojh_fail(OJH_ERR_UNSUPPORTED, "%s takes an argument block, not a buffer list: call ojh_decode_chain", s->name);
+}
+static int shape_chain(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t, uint32_t, uint32_t grid[3],
+                       uint32_t block[3]) {
+    grid[0] = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
+    grid[1] = grid[2] = 1;
+    block[0] = 1024; block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 static int shape_calib_mfma(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t, uint32_t,
                             uint32_t grid[3], uint32_t block[3]) {
     grid[0] = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;   // one workgroup of four waves per CU
@@ -1609,6 +1622,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("stream_read_u32x4", "glue", 2, 1, 1, 0, check_stream, shape_stream);
     add("calib_mfma_f16", "glue", 2, 2, 0, 0, check_calib_mfma, shape_calib_mfma);
     add("calib_mfma_i8", "glue", 2, 2, 0, 0, check_calib_mfma, shape_calib_mfma);
+    add("decode_chain_q4k", "chain", 0, 0, OJH_Q4_K, 2, check_chain, shape_chain);
     return m;
 }
 

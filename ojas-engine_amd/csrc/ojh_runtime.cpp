@@ -97,6 +97,7 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_FQ_THREADS")) d->fq_threads = atoi(r) == 512 ? 512u : atoi(r) == 256 ? 256u : 1024u;
     if (const char *r = getenv("OJAS_HIP_FQ_MULTI_BLOCKS")) d->fq_multi_blocks = atoi(r) > 0 ? (uint32_t)atoi(r) : 1u;
     if (const char *r = getenv("OJAS_HIP_FQ_MULTI")) d->fq_multi = atoi(r);
+    if (const char *r = getenv("OJAS_HIP_CHAIN_SPIN")) d->chain_spin = (uint32_t)strtoul(r, nullptr, 10);
     if (const char *r = getenv("OJAS_HIP_FQ_BLOCKS")) d->fq_blocks_per_cu = atoi(r) > 0 ? (uint32_t)atoi(r) : 8u;
     int rc = ojh_noalloc_setup(d);
     if (rc) {
@@ -121,6 +122,7 @@ extern "C" int ojh_close(ojh_device *dev) {
         if (b->owned) hipFree(b->ptr);
         delete b;
     }
+    if (dev->chain_status) hipHostFree(dev->chain_status);
     for (auto &kv : dev->modules) hipModuleUnload(kv.second);
     for (auto e : dev->marks)
         if (e) hipEventDestroy(e);
@@ -219,7 +221,7 @@ extern "C" int ojh_download(ojh_device *dev, const ojh_buf *src, size_t off, voi
     if (!bytes) return OJH_OK;
     OJH_HIP(hipMemcpyAsync(host, (const char *)src->ptr + off, bytes, hipMemcpyDeviceToHost, dev->stream));
     OJH_HIP(hipStreamSynchronize(dev->stream));
-    return OJH_OK;
+    return ojh_chain_check_status(dev);
 }
 
 extern "C" int ojh_memset0(ojh_device *dev, ojh_buf *dst, size_t off, size_t bytes) {
@@ -232,8 +234,10 @@ extern "C" int ojh_memset0(ojh_device *dev, ojh_buf *dst, size_t off, size_t byt
     return OJH_OK;
 }
 
-int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out) {
+// `fresh` (optional) tells whether the slot was (re)allocated by this call: its contents are then undefined.
+static int scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out, bool *fresh) {
     ojh_buf *&slot = dev->scratch[name];
+    if (fresh) *fresh = false;
     if (!slot || slot->bytes < bytes) {
         if (dev->capturing)
             return ojh_fail(OJH_ERR_ARG, "scratch '%s' would have to grow while recording a graph: run the call once "
@@ -249,17 +253,23 @@ int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **o
         size_t cap = bytes < 4096 ? 4096 : bytes + bytes / 4;
         int rc = ojh_alloc(dev, cap, &slot);
         if (rc) return rc;
+        if (fresh) *fresh = true;
     }
     *out = slot;
     return OJH_OK;
 }
 
+int ojh_scratch_get(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out) {
+    return scratch_get(dev, name, bytes, out, nullptr);
+}
+
+// Cleared whenever the slot is (re)allocated — decided by the allocation itself, not by comparing addresses: the
+// allocator may hand a grown slot the address the freed one had.
 int ojh_scratch_get_zeroed(ojh_device *dev, const char *name, size_t bytes, ojh_buf **out) {
-    auto it = dev->scratch.find(name);
-    const void *before = it != dev->scratch.end() && it->second ? it->second->ptr : nullptr;
-    int rc = ojh_scratch_get(dev, name, bytes, out);
+    bool fresh = false;
+    int rc = scratch_get(dev, name, bytes, out, &fresh);
     if (rc) return rc;
-    if ((*out)->ptr != before) OJH_HIP(hipMemsetAsync((*out)->ptr, 0, (*out)->bytes, dev->stream));   // (never while capturing: growth is refused there)
+    if (fresh) OJH_HIP(hipMemsetAsync((*out)->ptr, 0, (*out)->bytes, dev->stream));   // (never while capturing: growth is refused there)
     return OJH_OK;
 }
 
@@ -337,6 +347,40 @@ int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptr
     return OJH_OK;
 }
 
+static hipError_t launch_command(ojh_device *dev, ojh_command &c) {
+    if (!c.blob.empty()) {
+        size_t bytes = c.blob.size();
+        void *extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, c.blob.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END};
+        return hipModuleLaunchKernel(c.fn, c.grid[0], c.grid[1], c.grid[2], c.block[0], c.block[1], c.block[2], 0, dev->stream,
+                                     nullptr, extra);
+    }
+    void *args[16];
+    int n = 0;
+    for (auto &p : c.ptrs) args[n++] = &p;
+    for (auto &v : c.consts) args[n++] = &v;
+    return hipModuleLaunchKernel(c.fn, c.grid[0], c.grid[1], c.grid[2], c.block[0], c.block[1], c.block[2], 0, dev->stream, args,
+                                 nullptr);
+}
+
+int ojh_launch_blob(ojh_device *dev, const char *name, const void *args, size_t bytes, const uint32_t grid[3],
+                    const uint32_t block[3]) {
+    auto it = dev->functions.find(name);
+    if (it == dev->functions.end())
+        return ojh_fail(OJH_ERR_NOT_LOADED, "kernel '%s' not loaded — ensure_family first", name);
+    if (!grid[0] || !grid[1] || !grid[2] || !block[0] || !block[1] || !block[2])
+        return ojh_fail(OJH_ERR_ARG, "%s: empty grid or block", name);
+    ojh_command cmd;
+    cmd.fn = it->second;
+    cmd.blob.assign((const uint8_t *)args, (const uint8_t *)args + bytes);
+    for (int i = 0; i < 3; i++) { cmd.grid[i] = grid[i]; cmd.block[i] = block[i]; }
+    if (dev->capturing && !dev->capture_hip_graph) {
+        dev->recorded.push_back(std::move(cmd));
+        return OJH_OK;
+    }
+    OJH_HIP(launch_command(dev, cmd));
+    return OJH_OK;
+}
+
 extern "C" int ojh_dispatch(ojh_device *dev, const char *name, int n_bufs, ojh_buf *const *bufs,
                             const uint64_t *offsets, int n_consts, const uint32_t *consts,
                             const uint32_t grid[3], const uint32_t block[3]) {
@@ -386,7 +430,7 @@ extern "C" int ojh_submit(ojh_device *dev) {
     if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_submit: NULL device");
     if (dev->capturing) return ojh_fail(OJH_ERR_ARG, "ojh_submit while recording a graph");
     OJH_HIP(hipStreamSynchronize(dev->stream));
-    return OJH_OK;
+    return ojh_chain_check_status(dev);
 }
 
 extern "C" int ojh_timer_start(ojh_device *dev) {
@@ -473,14 +517,7 @@ extern "C" int ojh_graph_launch(ojh_device *dev, ojh_graph *graph) {
         OJH_HIP(hipGraphLaunch(graph->exec, dev->stream));
         return OJH_OK;
     }
-    for (auto &c : graph->list) {
-        void *args[16];
-        int n = 0;
-        for (auto &p : c.ptrs) args[n++] = &p;
-        for (auto &v : c.consts) args[n++] = &v;
-        OJH_HIP(hipModuleLaunchKernel(c.fn, c.grid[0], c.grid[1], c.grid[2], c.block[0], c.block[1], c.block[2], 0,
-                                      dev->stream, args, nullptr));
-    }
+    for (auto &c : graph->list) OJH_HIP(launch_command(dev, c));
     return OJH_OK;
 }
 

@@ -71,6 +71,17 @@ _lib = None
 EXPERT_LOAD_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_uint32, C.c_void_p, C.c_size_t)
 
 
+class _ChainStage(C.Structure):
+    """`ojh_chain_stage` of include/ojas_hip.h."""
+    _fields_ = [("x", C.c_void_p), ("x_off", C.c_size_t), ("x2", C.c_void_p), ("x2_off", C.c_size_t),
+                ("prologue", C.c_int), ("eps", C.c_float), ("count", C.c_int), ("ws", C.c_void_p * 4),
+                ("ys", C.c_void_p * 4), ("y_offs", C.c_size_t * 4), ("accum", C.c_int)]
+
+
+CHAIN_X_PLAIN, CHAIN_X_SILU_MUL, CHAIN_X_GELU_MUL, CHAIN_X_RMSNORM = 0, 1, 2, 3
+CHAIN_MAX_STAGES = 8
+
+
 class _GatherStats(C.Structure):
     _fields_ = [("hits", C.c_uint64), ("misses", C.c_uint64), ("bytes_streamed", C.c_uint64), ("evictions", C.c_uint64)]
 
@@ -121,6 +132,9 @@ def load_library(path: str | None = None) -> C.CDLL:
         "ojh_mm_q8k": (i32, [vp, vp, vp, vp, vp, sz, vp, u32, i32]),
         "ojh_mm_q8k_multi": (i32, [vp, vp, vp, i32, vp, vp, vp]),
         "ojh_mm_multi": (i32, [vp, vp, sz, i32, vp, vp, vp, i32]),
+        "ojh_decode_chain": (i32, [vp, C.POINTER(_ChainStage), i32]),
+        "ojh_chain_spin_limit": (i32, [vp, u32]),
+        "ojh_chain_trace": (i32, [vp, vp]),
         "ojh_gguf_open": (i32, [C.c_char_p, vp]),
         "ojh_gguf_close": (i32, [vp]),
         "ojh_gguf_tensor_count": (i32, [vp]),
@@ -566,6 +580,33 @@ class HipGpu:
         ya = (C.c_void_p * n)(*[y.handle for y in ys])
         oa = (C.c_size_t * n)(*y_offs) if y_offs is not None else None
         self._check(self._L.ojh_mm_multi(self._dev, x.handle, x_off, n, wa, ya, oa, int(accum)))
+
+    def decode_chain(self, stages: list) -> None:
+        """Dependent decode stages in ONE launch.  Each stage is a dict: x (Buf), ws (list of Lin), ys (list of Buf)
+        and optionally x_off, x2, x2_off, prologue (CHAIN_X_*), eps, y_offs, accum."""
+        n = len(stages)
+        arr = (_ChainStage * max(n, 1))()
+        for st, d in zip(arr, stages):
+            ws, ys = d["ws"], d["ys"]
+            if len(ws) != len(ys) or not 1 <= len(ws) <= 4:
+                raise ValueError("decode_chain: a stage takes 1 to 4 projections and as many outputs")
+            st.x, st.x_off = d["x"].handle, d.get("x_off", 0)
+            x2 = d.get("x2")
+            st.x2, st.x2_off = (x2.handle if x2 is not None else None), d.get("x2_off", 0)
+            st.prologue, st.eps, st.count = d.get("prologue", CHAIN_X_PLAIN), d.get("eps", 0.0), len(ws)
+            offs = d.get("y_offs") or [0] * len(ws)
+            for i, (w, y) in enumerate(zip(ws, ys)):
+                st.ws[i], st.ys[i], st.y_offs[i] = w.handle, y.handle, offs[i]
+            st.accum = int(bool(d.get("accum", False)))
+        self._check(self._L.ojh_decode_chain(self._dev, arr, n))
+
+    def chain_trace(self, buf: "Buf | None") -> None:
+        """Timestamps of the following chain launches go to `buf` (u64 [compute units][8 stages][6 events]); None: off."""
+        self._check(self._L.ojh_chain_trace(self._dev, buf.handle if buf is not None else None))
+
+    def chain_spin_limit(self, polls: int) -> None:
+        """Polls a chain's device-wide waits may take (0: every wait gives up at once)."""
+        self._check(self._L.ojh_chain_spin_limit(self._dev, polls))
 
     def rmsnorm_quant_q8k(self, x: Buf, gamma: Buf, eps: float, m: int, k: int, q: Buf, scales: Buf,
                           xn: Buf | None = None, x_off: int = 0) -> None:
