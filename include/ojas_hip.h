@@ -258,26 +258,31 @@ int ojh_mm_multi(ojh_device *dev, const ojh_buf *x, size_t x_off, int count, con
  * of the same call wrote (x of stage s = a y of stage s-1, or the residual an earlier stage accumulated onto):
  * q/k/v -> o -> gate/up -> down -> output head, or a feed-forward block norm -> gate/up -> SiLU*up -> down.  The
  * reference fuses neighbouring projections per launch (`qkv_q80_dp4a`, `ffn_gu_q80_dp4a`,
- * crates/ojas-cuda/src/kernels/gemv_q8.rs:229-260) and still pays a dispatch per dependent stage; here one
- * workgroup per compute unit stays resident for the whole chain, the stages meet at a device-wide barrier, and
- * because weights never depend on activations the loads of stage s+1's first rows are already in flight while
- * stage s finishes and the barrier is crossed.  The arithmetic of a stage starts only after the barrier.
- * Results are bit-identical to the same stages run as separate `ojh_mm_multi` (and, for the prologues,
- * `ojh_ffn_gu_q8k`-style) launches.
+ * crates/ojas-cuda/src/kernels/gemv_q8.rs:229-260) and still pays dispatches per dependent stage; here the grid
+ * is the concatenation of all stages' workgroups (per stage a few quantizer workgroups, then the row workgroups
+ * of the separate launch), the hardware hands them out in index order, and what one workgroup hands to another
+ * travels as {value, launch tag} pairs that the reader polls a bounded number of times.  The arithmetic of a
+ * stage starts only after every element of its input has arrived.  Results are bit-identical to the same stages
+ * run as separate `ojh_mm_multi` (and, for the prologues, `ojh_ffn_gu_q8k` / `ojh_rmsnorm_quant_q8k`) launches.
+ * Measured on MI355X the single launch is SLOWER than the separate launches for the 8B decode step (the waits'
+ * round trips run through a memory system the other workgroups keep saturated); the separate launches stay the
+ * library's default path and this entry point is for callers that need one launch.
  *
  * `prologue` says how the stage's input is formed from `x` (and `x2`) before it is quantized:
  *   OJH_CHAIN_X_PLAIN     x
  *   OJH_CHAIN_X_SILU_MUL  silu(x) * x2        (x = gate projection, x2 = up projection; cpu_math.rs:486)
  *   OJH_CHAIN_X_GELU_MUL  gelu_tanh(x) * x2   (cpu_math.rs:497-501)
  *   OJH_CHAIN_X_RMSNORM   x * (1 / sqrt(mean(x^2) + eps)) * x2, x2 = the norm's weights (cpu_math.rs:456-460;
- *                         the mean of squares is summed in f64 and rounded once)
+ *                         the mean of squares is summed in f64 and rounded once, as ojh_rmsnorm_quant_q8k does)
  * Limits: 1..OJH_CHAIN_MAX_STAGES stages; Q4_K tensors; all tensors of a stage share K, K % 256 == 0,
- * K <= 16384; at most 512 Ki rows per stage (32 Ki for a stage with `accum`); a stage's x / x2 must not overlap
- * its own outputs.  Workgroups wait for each other with a bounded number of polls (OJAS_HIP_CHAIN_SPIN, default
- * 2^22, or `ojh_chain_spin_limit`): if the grid is not resident as a whole (another process holds compute
- * units) a wait gives up, every kernel still exits, and the next `ojh_submit` / `ojh_download` on the device
- * returns OJH_ERR_HIP; outputs of chain calls since the last successful one are then undefined.  The call is
- * asynchronous like every other launch and can be recorded (`ojh_capture_begin`) after one eager call. */
+ * K <= 16384; a stage's x / x2 must not overlap its own outputs; an input that lies inside an output of an
+ * earlier stage is followed inside the launch, one that only straddles such an output is refused; a stage that
+ * accumulates onto an output of an earlier stage must take that whole vector and depend on that stage through
+ * its inputs.  Waits are bounded (OJAS_HIP_CHAIN_SPIN looks, default 2^22, or `ojh_chain_spin_limit`): if one
+ * gives up, every kernel still exits and the next `ojh_submit` / `ojh_download` on the device returns
+ * OJH_ERR_HIP; outputs of chain calls since the last successful one are then undefined.  The call is
+ * asynchronous like every other launch and can be recorded (`ojh_capture_begin`, the library's own replay; a
+ * captured hipGraph would freeze the launch tag and is refused) after one eager call. */
 #define OJH_CHAIN_MAX_STAGES 8
 enum { OJH_CHAIN_X_PLAIN = 0, OJH_CHAIN_X_SILU_MUL = 1, OJH_CHAIN_X_GELU_MUL = 2, OJH_CHAIN_X_RMSNORM = 3 };
 typedef struct ojh_chain_stage {
@@ -294,9 +299,9 @@ typedef struct ojh_chain_stage {
     int accum;             /* ys[i] += instead of = */
 } ojh_chain_stage;
 int ojh_decode_chain(ojh_device *dev, const ojh_chain_stage *stages, int n_stages);
-/* Timestamps of the chain launches that follow, for profiling: `buf` receives, per workgroup, stage and event
- * (stage entered, input quantized, rows done, results stored, arrival counted, wait over), the 100 MHz counter's
- * value as u64 [compute_units][OJH_CHAIN_MAX_STAGES][6]; NULL switches it off.  The buffer must outlive the
+/* Timestamps of the chain launches that follow, for profiling: `buf` receives, per stage, when the stage's first
+ * quantizer workgroup started, had its input (i.e. the rows it waited for were done) and had published it, as
+ * the 100 MHz counter's value, u64 [OJH_CHAIN_MAX_STAGES][3]; NULL switches it off.  The buffer must outlive the
  * launches (also recorded ones). */
 int ojh_chain_trace(ojh_device *dev, ojh_buf *buf);
 /* Polls a chain's waits may take from now on (0: every wait gives up at once — the failure path, for tests). */

@@ -1,13 +1,14 @@
 // Argument block of the single-launch decode chain (kernel `decode_chain_q4k`, family "chain"), shared by the host
-// side that fills it and the kernel that reads it from its kernarg segment.  Plain C layout, no padding surprises:
-// pointers first, then 32-bit words.
+// side that fills it and the kernel that reads it from its kernarg segment.  Plain C layout: pointers first, then
+// 32-bit words.
 #pragma once
 #include <stdint.h>
 
 #define OJK_CHAIN_MAX_STAGES 8
-#define OJK_CHAIN_THREADS 1024u     // one workgroup of sixteen waves per compute unit
-#define OJK_CHAIN_WAVES 16u
+#define OJK_CHAIN_THREADS 256u      // four waves per workgroup
 #define OJK_CHAIN_MAX_K 16384u
+#define OJK_CHAIN_QSEGS 4u          // 256-element segments of a stage's input one quantizer workgroup converts
+#define OJK_CHAIN_REPLICAS 64u      // copies of a stage's {scale, tag} table: the row workgroups poll different lines
 
 // How a stage's f32 input vector is formed before it is quantized per 256 (quant_q8k).
 enum {
@@ -17,14 +18,8 @@ enum {
     OJK_CHAIN_X_RMSNORM = 3,    // x * (1 / sqrt(mean(x^2) + eps)) * x2    (x2 = the norm's weights)
 };
 
-// Words of the device-side state block (uint32 each), zero when allocated and never reset: eight 64-bit launch
-// counters on separate 128-byte lines (workgroup b adds one to counter b % 8 when it starts), and the abort word.
-#define OJK_CHAIN_SYNC_TICKET(g) ((g) * 32u)
-#define OJK_CHAIN_SYNC_ABORT 256u   // set by a workgroup whose wait gave up: the others stop waiting too; the host clears it
-#define OJK_CHAIN_SYNC_WORDS 288u
-
-// A result that a later stage of the same launch reads travels as a pair {value, tag}, written and read as one
-// 8-byte access: the tag says which launch wrote the value, so a reader knows whether it has arrived.
+// A value one workgroup hands to another inside the launch travels as a pair {value, tag}, written and read as
+// one 8-byte access: the tag names the launch that wrote the value, so a reader knows whether it has arrived.
 struct ojk_chain_pair {
     float value;
     uint32_t tag;
@@ -35,30 +30,36 @@ struct ojk_chain_stage {
     const void *x2;         // second operand of the prologue, likewise (bit 1)
     const void *w[4];       // Q4_K rows of up to four tensors sharing x (unused slots repeat the last)
     void *y[4];             // f32 outputs, one per tensor
-    struct ojk_chain_pair *xchg[4];   // where tensor i's results go as pairs for later stages, NULL if none reads them
+    struct ojk_chain_pair *xchg[4];         // where tensor i's results also go as pairs (a later stage reads them), or NULL
+    const struct ojk_chain_pair *addsrc[4]; // accumulating stage: the old values as pairs of an earlier stage, or NULL (read y)
+    signed char *xq;                        // K bytes: this stage's quantized input
+    struct ojk_chain_pair *xs;              // [OJK_CHAIN_REPLICAS][64]: {scale of segment i, tag}
     uint32_t ends[4];       // cumulative row counts: tensor i owns stacked rows ends[i-1] .. ends[i]-1
     uint32_t K;
     uint32_t prologue;
     uint32_t accum;         // y += W x instead of y = W x
     uint32_t eps_bits;      // RMS norm epsilon, as float bits
     uint32_t tagged;
-    uint32_t pad_;
+    uint32_t rows_per_wave; // 1 or 2
+    uint32_t wg_first;      // the stage's first workgroup: n_quant quantizer workgroups, then its row workgroups
+    uint32_t n_quant;
 };
 
 struct ojk_chain_args {
     struct ojk_chain_stage st[OJK_CHAIN_MAX_STAGES];
-    uint32_t *sync;         // OJK_CHAIN_SYNC_WORDS words
+    uint32_t *abort_word;   // device word: set by a wait that gave up, the other waits stop at their next look at it
     uint32_t *status;       // host-visible word: set to 1 + stage index when a bounded wait gives up
-    uint64_t *trace;        // optional: OJK_CHAIN_TRACE_EVENTS timestamps (100 MHz counter) per workgroup and stage
+    uint64_t *trace;        // optional: OJK_CHAIN_TRACE_EVENTS timestamps (100 MHz counter) per stage
     uint32_t nstages;
-    uint32_t spin_cap;      // polls a wait may take before it gives up (0: gives up at once)
+    uint32_t spin_cap;      // looks a wait may take before it gives up (0: gives up at once)
+    uint32_t tag;           // this launch's tag: never 0, never the tag of an earlier launch of the device
+    uint32_t pad_;
 };
 
-// trace[(workgroup * OJK_CHAIN_MAX_STAGES + stage) * OJK_CHAIN_TRACE_EVENTS + event], written by the workgroup's first wave
-#define OJK_CHAIN_TRACE_EVENTS 4u
+// trace[stage * OJK_CHAIN_TRACE_EVENTS + event], written by the stage's first quantizer workgroup
+#define OJK_CHAIN_TRACE_EVENTS 3u
 enum {
-    OJK_CHAIN_T_ENTER = 0,     // the wave turns to the stage's input
-    OJK_CHAIN_T_ARRIVED = 1,   // its part of the input has arrived
-    OJK_CHAIN_T_INPUT = 2,     // the whole input is quantized in LDS
-    OJK_CHAIN_T_ROWS = 3,      // the wave's rows are done and stored
+    OJK_CHAIN_T_QUANT_ENTER = 0,    // it starts
+    OJK_CHAIN_T_QUANT_ARRIVED = 1,  // it has the stage's whole input (the norm) or its own part of it: the rows it waited for are done
+    OJK_CHAIN_T_QUANT_DONE = 2,     // it has published its segments
 };

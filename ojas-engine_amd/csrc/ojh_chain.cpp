@@ -3,6 +3,7 @@
 // with one workgroup per compute unit.  The op-level counterpart in the reference is a sequence of `CudaSsm::mm`
 // calls (crates/ojas-cuda/src/qwen35.rs:644-702), one or more launches each; see the kernel for what the single
 // launch changes.
+#include <cstddef>
 #include <cstring>
 
 #include "kernels/ojk_chain.h"
@@ -23,16 +24,16 @@ static bool within(const void *a, size_t na, const void *b, size_t nb) {   // [a
     return x >= y && x + na <= y + nb;
 }
 
-// Device state: the launch counters and the abort word (zeroed once, never reallocated: the counters only grow),
-// and the pinned status word.
-static int chain_state(ojh_device *dev, uint32_t **sync) {
+// Device state: the abort word (zeroed when allocated, cleared by the host after a failure) and the pinned status
+// word the kernels write to.
+static int chain_state(ojh_device *dev, uint32_t **abort_word) {
     ojh_buf *b;
-    int rc = ojh_scratch_get_zeroed(dev, "chain_sync", OJK_CHAIN_SYNC_WORDS * 4, &b);
+    int rc = ojh_scratch_get_zeroed(dev, "chain_abort", 256, &b);
     if (rc) return rc;
-    *sync = (uint32_t *)b->ptr;
+    *abort_word = (uint32_t *)b->ptr;
     if (!dev->chain_status) {
         if (dev->capturing)
-            return ojh_fail(OJH_ERR_ARG, "ojh_decode_chain: first call while recording a graph: run it once eagerly first");
+            return ojh_fail(OJH_ERR_ARG, "ojh_decode_chain: first call while recording: run it once eagerly first");
         void *p = nullptr;
         OJH_HIP(hipHostMalloc(&p, 64, hipHostMallocDefault));
         memset(p, 0, 64);
@@ -47,9 +48,9 @@ int ojh_chain_check_status(ojh_device *dev) {
     if (!st) return OJH_OK;
     __atomic_store_n(dev->chain_status, 0u, __ATOMIC_RELEASE);
     // every kernel has exited (the stream was just synchronised): let the next launch wait again
-    auto it = dev->scratch.find("chain_sync");
+    auto it = dev->scratch.find("chain_abort");
     if (it != dev->scratch.end() && it->second) {
-        OJH_HIP(hipMemsetAsync((char *)it->second->ptr + OJK_CHAIN_SYNC_ABORT * 4, 0, 4, dev->stream));
+        OJH_HIP(hipMemsetAsync(it->second->ptr, 0, 4, dev->stream));
         OJH_HIP(hipStreamSynchronize(dev->stream));
     }
     return ojh_fail(OJH_ERR_HIP, "ojh_decode_chain: a wait for the input of stage %u gave up after its bounded number of polls — "
@@ -59,7 +60,7 @@ int ojh_chain_check_status(ojh_device *dev) {
 
 extern "C" int ojh_chain_trace(ojh_device *dev, ojh_buf *buf) {
     if (!dev) return ojh_fail(OJH_ERR_ARG, "ojh_chain_trace: NULL device");
-    const size_t need = (size_t)dev->prop.multiProcessorCount * OJK_CHAIN_MAX_STAGES * OJK_CHAIN_TRACE_EVENTS * 8;
+    const size_t need = (size_t)OJK_CHAIN_MAX_STAGES * OJK_CHAIN_TRACE_EVENTS * 8;
     if (buf && buf->bytes < need)
         return ojh_fail(OJH_ERR_BOUNDS, "ojh_chain_trace: the buffer has %zu bytes, %zu are needed", buf->bytes, need);
     if (buf && (uintptr_t)buf->ptr % 8) return ojh_fail(OJH_ERR_ARG, "ojh_chain_trace: the buffer must be 8-byte aligned");
@@ -73,15 +74,15 @@ extern "C" int ojh_chain_spin_limit(ojh_device *dev, uint32_t polls) {
     return OJH_OK;
 }
 
-// rows a wave multiplies per unit in a stage of `rows` rows: the kernel's rule (ch_view)
-static uint32_t rows_per_unit(uint64_t rows, uint32_t nw) { return (rows + 1) / 2 < nw ? 1u : 2u; }
+// rows per wave of a stage of `rows` rows: two once every compute unit gets several workgroups (the separate
+// launches' rule, measured on Q4_K with K = 4096)
+static uint32_t rows_per_wave(uint64_t rows, uint32_t cus) { return rows >= (uint64_t)cus * 32u ? 2u : 1u; }
 
 extern "C" int ojh_decode_chain(ojh_device *dev, const ojh_chain_stage *stages, int n_stages) {
     if (!dev || !stages) return ojh_fail(OJH_ERR_ARG, "ojh_decode_chain: NULL argument");
     if (n_stages < 1 || n_stages > OJK_CHAIN_MAX_STAGES)
         return ojh_fail(OJH_ERR_ARG, "ojh_decode_chain: %d stages, takes 1 to %d", n_stages, OJK_CHAIN_MAX_STAGES);
     const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;
-    const uint32_t nw = cus * OJK_CHAIN_WAVES;
     ojk_chain_args args;
     memset(&args, 0, sizeof args);
     uint64_t rows_of[OJK_CHAIN_MAX_STAGES] = {0};
@@ -109,7 +110,7 @@ extern "C" int ojh_decode_chain(ojh_device *dev, const ojh_chain_stage *stages, 
         if (K % 256 || K > OJK_CHAIN_MAX_K)
             return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_decode_chain: stage %d has K=%u; needs a multiple of 256 up to %u", s, K,
                             OJK_CHAIN_MAX_K);
-        if (total > 0x7FFFFFFFull) return ojh_fail(OJH_ERR_ARG, "ojh_decode_chain: stage %d has too many rows", s);
+        if (total > 0x3FFFFFFFull) return ojh_fail(OJH_ERR_ARG, "ojh_decode_chain: stage %d has too many rows", s);
         rows_of[s] = total;
         if (!in.x) return ojh_fail(OJH_ERR_ARG, "ojh_decode_chain: stage %d: x is NULL", s);
         if (in.x_off > in.x->bytes || (size_t)K * 4 > in.x->bytes - in.x_off)
@@ -194,50 +195,85 @@ extern "C" int ojh_decode_chain(ojh_device *dev, const ojh_chain_stage *stages, 
             // every workgroup has read its stage-s input, so only the same stage could (refused above)
         }
     }
-    // An accumulating stage reads the old values of its outputs row by row, each by the wave that will store the
-    // row.  If an earlier stage of this launch wrote those bytes, the same wave must have written them: same
-    // buffer, same row count and the same place in the stacked rows.
+    // An accumulating stage reads the old values of its outputs.  If an earlier stage of this launch wrote them, they
+    // are read from that stage's pairs (whose tags say that they have arrived): the two must then be the same vector,
+    // and the stage must depend on the earlier one through its inputs, or nothing orders the two.
+    uint32_t dep[OJK_CHAIN_MAX_STAGES] = {0};      // bit e: stage s reads (directly or not) what stage e wrote
+    for (int s = 0; s < n_stages; s++)
+        for (int which = 0; which < 2; which++)
+            if (from[s][which].stage >= 0) dep[s] |= (1u << from[s][which].stage) | dep[from[s][which].stage];
+    struct { int stage, tensor; } addfrom[OJK_CHAIN_MAX_STAGES][4];
+    for (int s = 0; s < n_stages; s++)
+        for (int i = 0; i < 4; i++) addfrom[s][i] = {-1, -1};
     for (int s = 0; s < n_stages; s++) {
         if (!stages[s].accum) continue;
         for (int i = 0; i < stages[s].count; i++)
-            for (int e = 0; e < s; e++)
+            for (int e = s - 1; e >= 0 && addfrom[s][i].stage < 0; e--)
                 for (int j = 0; j < stages[e].count; j++) {
                     const size_t yb = (size_t)stages[s].ws[i]->n * 4, eb = (size_t)stages[e].ws[j]->n * 4;
                     if (!overlaps(args.st[s].y[i], yb, args.st[e].y[j], eb)) continue;
-                    const uint32_t start_s = i ? args.st[s].ends[i - 1] : 0, start_e = j ? args.st[e].ends[j - 1] : 0;
-                    if (args.st[s].y[i] != args.st[e].y[j] || yb != eb || start_s != start_e ||
-                        rows_per_unit(rows_of[s], nw) != rows_per_unit(rows_of[e], nw))
-                        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_decode_chain: stage %d accumulates onto output %d of stage %d, which "
-                                                             "other waves wrote (different rows per wave or place among the stage's tensors)", s, j, e);
+                    if (args.st[s].y[i] != args.st[e].y[j] || yb != eb)
+                        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_decode_chain: stage %d accumulates onto a part of output %d of stage %d; "
+                                                             "it must be that whole vector", s, j, e);
+                    if (!(dep[s] & (1u << e)))
+                        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_decode_chain: stage %d accumulates onto output %d of stage %d without "
+                                                             "reading anything that depends on that stage", s, j, e);
+                    addfrom[s][i] = {e, j};
+                    xchg_used[e][j] = true;
+                    break;
                 }
     }
     if ((rc = ojh_ensure_family(dev, "chain"))) return rc;
-    uint32_t *sync = nullptr;
-    if ((rc = chain_state(dev, &sync))) return rc;
+    if (dev->capturing && dev->capture_hip_graph)
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_decode_chain: every launch takes a fresh tag, which a captured hipGraph would "
+                                             "freeze: record it with the library's own replay (unset OJAS_HIP_REPLAY)");
+    uint32_t *abort_word = nullptr;
+    if ((rc = chain_state(dev, &abort_word))) return rc;
+    // scratch: the handed-on pairs, and per stage the int8 input and the copies of its {scale, tag} table
+    size_t xq_bytes = 0;
+    for (int s = 0; s < n_stages; s++) xq_bytes += ((size_t)args.st[s].K + 255) & ~(size_t)255;
+    const size_t xs_pairs = (size_t)OJK_CHAIN_REPLICAS * 64;
+    ojh_buf *xqb, *xsb;
+    if ((rc = ojh_scratch_get(dev, "chain_xq", xq_bytes, &xqb))) return rc;
+    if ((rc = ojh_scratch_get_zeroed(dev, "chain_xs", (size_t)n_stages * xs_pairs * sizeof(ojk_chain_pair), &xsb))) return rc;
     ojk_chain_pair *xchg = nullptr;
     if (xchg_pairs) {   // zero tags never match: a launch's tag is at least 1
         ojh_buf *xb;
         if ((rc = ojh_scratch_get_zeroed(dev, "chain_xchg", xchg_pairs * sizeof(ojk_chain_pair), &xb))) return rc;
         xchg = (ojk_chain_pair *)xb->ptr;
     }
+    uint32_t wg = 0;
+    size_t xq_off = 0;
     for (int s = 0; s < n_stages; s++) {
+        ojk_chain_stage &st = args.st[s];
         for (int i = 0; i < 4; i++) {
             const int j = i < stages[s].count ? i : stages[s].count - 1;
-            args.st[s].xchg[i] = xchg_used[s][j] ? xchg + xchg_off[s][j] : nullptr;
+            st.xchg[i] = xchg_used[s][j] ? xchg + xchg_off[s][j] : nullptr;
+            st.addsrc[i] = addfrom[s][j].stage >= 0 ? xchg + xchg_off[addfrom[s][j].stage][addfrom[s][j].tensor] : nullptr;
         }
         for (int which = 0; which < 2; which++) {
             const src &f = from[s][which];
             if (f.stage < 0) continue;
             const void *p = xchg + xchg_off[f.stage][f.tensor] + f.first;
-            if (which) args.st[s].x2 = p; else args.st[s].x = p;
-            args.st[s].tagged |= 1u << which;
+            if (which) st.x2 = p; else st.x = p;
+            st.tagged |= 1u << which;
         }
+        st.xq = (signed char *)xqb->ptr + xq_off;
+        xq_off += ((size_t)st.K + 255) & ~(size_t)255;
+        st.xs = (ojk_chain_pair *)xsb->ptr + (size_t)s * xs_pairs;
+        st.rows_per_wave = rows_per_wave(rows_of[s], cus);
+        st.wg_first = wg;
+        st.n_quant = (st.K / 256 + OJK_CHAIN_QSEGS - 1) / OJK_CHAIN_QSEGS;
+        const uint64_t row_wgs = (rows_of[s] + 4 * st.rows_per_wave - 1) / (4 * st.rows_per_wave);
+        if ((uint64_t)wg + st.n_quant + row_wgs > 0x7FFFFFFFull) return ojh_fail(OJH_ERR_ARG, "ojh_decode_chain: too many workgroups");
+        wg += st.n_quant + (uint32_t)row_wgs;
     }
-    args.sync = sync;
+    args.abort_word = abort_word;
     args.status = dev->chain_status;
     args.trace = (uint64_t *)dev->chain_trace;
     args.nstages = (uint32_t)n_stages;
     args.spin_cap = dev->chain_spin;
-    const uint32_t grid[3] = {cus, 1, 1}, block[3] = {OJK_CHAIN_THREADS, 1, 1};
-    return ojh_launch_blob(dev, "decode_chain_q4k", &args, sizeof args, grid, block);
+    args.tag = 0;   // filled in at every launch (also of a recorded one)
+    const uint32_t grid[3] = {wg, 1, 1}, block[3] = {OJK_CHAIN_THREADS, 1, 1};
+    return ojh_launch_blob(dev, "decode_chain_q4k", &args, sizeof args, grid, block, (int)offsetof(ojk_chain_args, tag));
 }

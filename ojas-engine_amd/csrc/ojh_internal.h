@@ -30,6 +30,7 @@ struct ojh_command {
     std::vector<void *> ptrs;
     std::vector<uint32_t> consts;
     std::vector<uint8_t> blob;   // a kernel whose arguments are one struct: its bytes, passed as the argument buffer
+    int tag_offset = -1;         // ... and where in it every launch writes a fresh 32-bit tag (-1: nowhere)
     uint32_t grid[3] = {1, 1, 1}, block[3] = {1, 1, 1};
 };
 
@@ -96,6 +97,7 @@ struct ojh_device {
     // (pinned host memory the kernels write to), the number of polls a wait may take
     uint32_t *chain_status = nullptr;
     uint32_t chain_spin = 1u << 22;    // OJAS_HIP_CHAIN_SPIN
+    uint32_t chain_tag = 0;            // the last launch's tag (never 0)
     void *chain_trace = nullptr;       // ojh_chain_trace: timestamps of the next chain launches go here
     void *noalloc_scratch = nullptr;   // this GPU's copy of the static scratch array of ojh_mm_noalloc (ojh_noalloc.cpp)
 };
@@ -157,7 +159,7 @@ int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptr
                const std::vector<uint32_t> &consts, const uint32_t grid[3], const uint32_t block[3]);
 // a kernel that takes one struct as its argument list
 int ojh_launch_blob(ojh_device *dev, const char *name, const void *args, size_t bytes, const uint32_t grid[3],
-                    const uint32_t block[3]);
+                    const uint32_t block[3], int tag_offset = -1);
 int ojh_chain_check_status(ojh_device *dev);   // after a synchronisation: did a chain's bounded wait give up? (ojh_chain.cpp)
 // shared by ojh_mm / ojh_mm_q8k / ojh_mm_noalloc (ojh_ops.cpp)
 int ojh_mm_checks(const char *who, const ojh_lin *w, ojh_buf *y, size_t y_off, const ojh_buf *bias, uint32_t m, int accum,

@@ -1353,9 +1353,9 @@ static int check_chain(const ojh_kernel_spec *s, const uint32_t *, const uint32_
 }
 static int shape_chain(const ojh_kernel_spec *, const ojh_device *dev, uint32_t, uint32_t, uint32_t, uint32_t grid[3],
                        uint32_t block[3]) {
-    grid[0] = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
-    grid[1] = grid[2] = 1;
-    block[0] = 1024; block[1] = block[2] = 1;
+    (void)dev;
+    grid[0] = grid[1] = grid[2] = 1;   // the grid is the sum of the stages' workgroups: ojh_decode_chain computes it
+    block[0] = 256; block[1] = block[2] = 1;
     return OJH_OK;
 }
 

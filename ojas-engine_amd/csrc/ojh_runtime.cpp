@@ -349,6 +349,10 @@ int ojh_launch(ojh_device *dev, const char *name, const std::vector<void *> &ptr
 
 static hipError_t launch_command(ojh_device *dev, ojh_command &c) {
     if (!c.blob.empty()) {
+        if (c.tag_offset >= 0) {   // a tag no earlier launch of this device had (0 is never one)
+            if (++dev->chain_tag == 0) ++dev->chain_tag;
+            memcpy(c.blob.data() + c.tag_offset, &dev->chain_tag, 4);
+        }
         size_t bytes = c.blob.size();
         void *extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, c.blob.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END};
         return hipModuleLaunchKernel(c.fn, c.grid[0], c.grid[1], c.grid[2], c.block[0], c.block[1], c.block[2], 0, dev->stream,
@@ -363,7 +367,7 @@ static hipError_t launch_command(ojh_device *dev, ojh_command &c) {
 }
 
 int ojh_launch_blob(ojh_device *dev, const char *name, const void *args, size_t bytes, const uint32_t grid[3],
-                    const uint32_t block[3]) {
+                    const uint32_t block[3], int tag_offset) {
     auto it = dev->functions.find(name);
     if (it == dev->functions.end())
         return ojh_fail(OJH_ERR_NOT_LOADED, "kernel '%s' not loaded — ensure_family first", name);
@@ -372,6 +376,7 @@ int ojh_launch_blob(ojh_device *dev, const char *name, const void *args, size_t 
     ojh_command cmd;
     cmd.fn = it->second;
     cmd.blob.assign((const uint8_t *)args, (const uint8_t *)args + bytes);
+    cmd.tag_offset = tag_offset;
     for (int i = 0; i < 3; i++) { cmd.grid[i] = grid[i]; cmd.block[i] = block[i]; }
     if (dev->capturing && !dev->capture_hip_graph) {
         dev->recorded.push_back(std::move(cmd));
