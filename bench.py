@@ -137,6 +137,15 @@ def main() -> int:
     for i in range(args.warmup):
         run_step(i)
     gpu.submit()
+    # ... and about 10 ms more of untimed steps, whatever --warmup says: after the uploads above the part needs
+    # milliseconds to bring its clocks back up, and steady-state decode is what the metric means
+    gpu.timer_start()
+    run_step(0)
+    one_ms = max(gpu.timer_stop(), 1e-3)
+    preroll_steps = min(2000, int(10.0 / one_ms))
+    for i in range(preroll_steps):
+        run_step(i)
+    preroll_ms = preroll_steps * one_ms     # (no synchronisation here: the timed steps follow on the stream at once)
 
     # ---- timed region: exactly `steps` steps, events on the launching stream + host clock
     t_host = time.perf_counter()
@@ -254,6 +263,8 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "preroll_ms": round(preroll_ms, 2),
+        "preroll_steps": preroll_steps,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -292,10 +303,11 @@ def main() -> int:
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(host, dims)
     if not args.no_extra:
-        # free the decode sets first: the secondary shapes bring their own tensors
         graphs.clear()
+        chain = chain_leg(gpu, pkg, sets, dims, step_bytes)
         lin_q = sets[0]["gate"], sets[0]["down"], sets[0]["head"]
         result["extra"] = extras(gpu, pkg, lin_q)
+        result["extra"]["decode_chain_dependent"] = chain
     print(json.dumps(result))
     gpu.close()
     return 0
@@ -318,6 +330,62 @@ def _time(gpu, fn, reps: int, warm: int = 3) -> float:
     return gpu.timer_stop() / reps * 1e3
 
 
+def chain_leg(gpu, pkg, sets, dims, step_bytes) -> dict:
+    """The same eight projections as a chain in which every stage reads what the one before it wrote (x -> q,k,v;
+    q -> o; rmsnorm(o) -> gate,up; silu(gate) * up -> down; rmsnorm(down) -> head), once as ONE launch
+    (ojh_decode_chain) and once as the separate launches that compute the same bits."""
+    R, synth = pkg.runtime, pkg.synth
+    d, nff = dims["q"][1], dims["gate"][0]
+    x0 = gpu.upload(synth.normal_f32(d, "bench", "chain_x0"))
+    gamma = gpu.upload(np.ones(d, np.float32))
+    y = {n: gpu.alloc(dims[n][0]) for n in dims}
+    xq, xs, act = gpu.alloc_bytes(d), gpu.alloc(d // 256), gpu.alloc(nff)
+    eps = 1e-5
+
+    def stages(w):
+        return [dict(x=x0, ws=[w["q"], w["k"], w["v"]], ys=[y["q"], y["k"], y["v"]]),
+                dict(x=y["q"], ws=[w["o"]], ys=[y["o"]]),
+                dict(x=y["o"], x2=gamma, prologue=R.CHAIN_X_RMSNORM, eps=eps, ws=[w["gate"], w["up"]], ys=[y["gate"], y["up"]]),
+                dict(x=y["gate"], x2=y["up"], prologue=R.CHAIN_X_SILU_MUL, ws=[w["down"]], ys=[y["down"]]),
+                dict(x=y["down"], x2=gamma, prologue=R.CHAIN_X_RMSNORM, eps=eps, ws=[w["head"]], ys=[y["head"]])]
+
+    def separate(w):
+        gpu.mm_multi(x0, [w["q"], w["k"], w["v"]], [y["q"], y["k"], y["v"]])
+        gpu.mm_multi(y["q"], [w["o"]], [y["o"]])
+        gpu.rmsnorm_quant_q8k(y["o"], gamma, eps, 1, d, xq, xs)
+        gpu.ffn_gu_q8k(xq, xs, w["gate"], w["up"], act)
+        gpu.mm_multi(act, [w["down"]], [y["down"]])
+        gpu.rmsnorm_quant_q8k(y["down"], gamma, eps, 1, d, xq, xs)
+        gpu.mm_q8k_multi(xq, xs, [w["head"]], [y["head"]])
+
+    out = {}
+    for tag, fn in (("one_launch", lambda w: gpu.decode_chain(stages(w))), ("separate_launches", separate)):
+        fn(sets[0])
+        gpu.submit()
+        recorded = []
+        for w in sets:
+            gpu.capture_begin()
+            fn(w)
+            recorded.append(gpu.capture_end())
+        us = _time(gpu, lambda i: recorded[i % len(recorded)].launch(), 200, 10)
+        out[tag] = {"us": round(us, 2), "gbs": round(step_bytes / us / 1e3, 1), "hbm_frac": round(step_bytes / us / 8e6, 4)}
+        del recorded
+    # where the single launch spends its time: per stage, when its first quantizer workgroup had its input (= the rows
+    # it depends on were done) and when it had published it, microseconds after the first stage's quantizer started
+    tb = gpu.alloc_bytes(8 * 3 * 8)
+    gpu.chain_trace(tb)
+    gpu.decode_chain(stages(sets[0]))
+    gpu.submit()
+    gpu.chain_trace(None)
+    t = gpu.read(tb, 24, np.uint64).reshape(8, 3).astype(np.float64) / 100.0
+    out["one_launch"]["stage_input_arrived_published_us"] = [[round(float(t[s, 1] - t[0, 0]), 2), round(float(t[s, 2] - t[0, 0]), 2)]
+                                                             for s in range(5)]
+    out["what"] = ("every stage reads the previous stage's output; separate = ojh_mm_multi / ojh_rmsnorm_quant_q8k / "
+                   "ojh_ffn_gu_q8k (gate, up and SiLU in one launch) / ojh_mm_q8k_multi, 8 launches; one_launch = "
+                   "ojh_decode_chain, bit-identical to them (gate and up stored as well)")
+    return out
+
+
 def extras(gpu, pkg, lin_q) -> dict:
     """Secondary configurations: prefill GEMM, Q8_0 matvec, MoE grouped FFN, Q6_K head verify."""
     synth = pkg.synth
@@ -336,6 +404,21 @@ def extras(gpu, pkg, lin_q) -> dict:
                                "tile": "v_mfma_f32_32x32x16_f16, weights dequantized straight into the B registers: 256 tokens x 256 rows per workgroup where that fills the chip (M = 2048), 128 x 256 below (gate/up M = 512), 128 x 64 with K split over the workgroup's waves where 256-row tiles are too few (M = 128, down M = 512); "
                                        "weights = binary16 fma(qa, q, qb), the bits of the reference's gemm_mm_q4l",
                                "peak_tflops": 2500.0, "timed": "conversion + zero fill (split-K) + tile", **gemm}
+    # ---- the same contraction over Q6_K and Q8_0 weights (the other two formats the path names), bf16 in
+    for ty, tag, gen in ((pkg.Q6_K, "q6k", synth.q6k_weights), (pkg.Q8_0, "q8_0", synth.q80_weights)):
+        fam = {}
+        for name, (n, k) in (("gate_up_14336x4096", (14336, 4096)), ("down_4096x14336", (4096, 14336))):
+            lin = gpu.lin(ty, n, k, gen(n, k, "bench", tag, name))
+            for m in (128, 512, 2048):
+                xb = gpu.upload_bytes(synth.to_bf16_bits(synth.normal_f32(m * k, "bench", "gemm_x", m, k)))
+                y = gpu.alloc(m * n)
+                us = _time(gpu, lambda i: gpu.mm(xb, lin, y, m, x_dtype=pkg.X_BF16, act_mode=pkg.ACT_FLOAT), 20, 5)
+                tf = 2.0 * m * n * k / us / 1e6
+                fam[f"{name}_M{m}"] = {"us": round(us, 1), "tflops": round(tf, 1), "mfma_frac": round(tf / 2500.0, 4)}
+                del xb, y
+            lin.free()
+        out[f"prefill_gemm_{tag}"] = {"activations": "bf16 N(0,1), converted to f16 into the tile", "accumulate": "f32",
+                                      "peak_tflops": 2500.0, "timed": "conversion + zero fill (split-K) + tile", **fam}
     # ---- the same two matrices in the CPU path's arithmetic (quant_q8k activations, int8 MFMA), f32 in
     i8 = {}
     for name, lin in zip(("gate_up_14336x4096", "down_4096x14336"), lin_q):

@@ -84,23 +84,26 @@ __device__ __forceinline__ void gemv_q8k_q4k_body(const signed char* __restrict_
                                                   const uchar* __restrict__ w, float* __restrict__ y,
                                                   const float* __restrict__ bs, uint K, uint N) {
     const uint lane = threadIdx.x & 63u;
-    const uint row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+    // (the wave's rows are the same in every lane: said so, the row addresses are scalar arithmetic and the loads take
+    // a scalar base plus a 32-bit lane offset instead of 64-bit multiplies per lane)
+    const uint row0 = (uint)__builtin_amdgcn_readfirstlane((int)((blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R));
     if (row0 >= N) return;
     const uint nsb = K >> 8, g = lane >> 3, l = lane & 7u, c = l >> 1;
     float acc[R], add[R];
+    const uchar* wrow[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
         acc[r] = 0.0f;
         add[r] = store_addend<MODE>(y, bs, min(row0 + r, N - 1u));
+        wrow[r] = w + (size_t)min(row0 + r, N - 1u) * nsb * Q4K_BYTES;
     }
     for (uint sb = g; sb < nsb; sb += 8u) {
         uint4 hdr[R], qs[R];
+        const uint off = __umul24(sb, Q4K_BYTES);
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            uint row = min(row0 + r, N - 1u);
-            const uchar* blk = w + ((size_t)row * nsb + sb) * Q4K_BYTES;
-            hdr[r] = *(const uint4*)blk;
-            qs[r] = *(const uint4*)(blk + 16u + l * 16u);
+            hdr[r] = *(const uint4*)(wrow[r] + off);
+            qs[r] = *(const uint4*)(wrow[r] + (off + 16u + l * 16u));
         }
         Q4kFrag f = q4k_load_frag(xq, xs, sb, l);
 #pragma unroll

@@ -82,8 +82,10 @@ __device__ __forceinline__ float q4k_lane_dot(uint4 hdr, uint4 qs, uint c, const
     ih = dot4_i8((qs.w >> 4) & M4, f.xh.w, ih);
     uint sc, mn;
     q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
-    int isum = (int)(sc & 0xFFu) * il + (int)(sc >> 8) * ih;
-    int msum = (int)(mn & 0xFFu) * f.bl + (int)(mn >> 8) * f.bh;
+    // 24-bit multiplies (full rate; a 32-bit integer multiply is a quarter-rate instruction): the scales are 6 bits,
+    // a sum of sixteen nibble x int8 products stays below 2^15, a sum of sixteen int8 below 2^11
+    int isum = __mul24((int)(sc & 0xFFu), il) + __mul24((int)(sc >> 8), ih);
+    int msum = __mul24((int)(mn & 0xFFu), f.bl) + __mul24((int)(mn >> 8), f.bh);
     float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
     return f.sx * (d * (float)isum - dmin * (float)msum);
 }
