@@ -83,7 +83,7 @@ def test_q6k_verify_head_at_full_size(gpu, orc, pkg, m):
 
 
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
-@pytest.mark.parametrize("m", [128, 512])
+@pytest.mark.parametrize("m", [128, 512, 2048])
 def test_prefill_in_the_cpu_arithmetic_at_full_size(gpu, orc, pkg, n, k, m):
     """The same shapes under OJH_ACT_Q8K — activations quantized per 256, integer dots on the int8 matrix cores —
     against `matvec_kq`, the CPU reference itself, token by token on sampled weight rows (tile borders included):
@@ -101,7 +101,9 @@ def test_prefill_in_the_cpu_arithmetic_at_full_size(gpu, orc, pkg, n, k, m):
     g = pkg.synth.rng("full", "q8k-rows", n, k, m)
     rows = np.unique(np.concatenate([[0, 15, 16, 63, 64, n - 17, n - 1], g.integers(0, n, 25)]))
     wsub = _rows(w, Q4_K, pkg, k, rows)
-    for t in range(m):
+    # every token up to 512; of 2048 (sixteen token tiles in grid.y) the borders of every 128-token tile and every 11th
+    tokens = range(m) if m <= 512 else np.unique(np.concatenate([np.arange(0, m, 128), np.arange(127, m, 128), np.arange(0, m, 11)]))
+    for t in tokens:
         want = orc.matvec_kq(wsub, Q4_K, len(rows), k, xf[t], threads=1 if len(rows) < 64 else 8)
         assert peak_err(got[t, rows], want) <= 2e-5, t
     perm = np.roll(np.arange(m), 37)
@@ -148,5 +150,9 @@ def test_prefill_gemm_at_full_size(gpu, orc, pkg, n, k, m):
     # the first 128 tokens alone: another tile height and K split, so sums associate differently
     y3 = gpu.alloc(128 * n)
     gpu.mm(gpu.upload_bytes(xb[:128 * k].copy()), lin, y3, 128, x_dtype=pkg.X_BF16, act_mode=pkg.ACT_FLOAT)
-    e = rms_errs(gpu.read(y3, 128 * n).reshape(128, n), got[:128])
+    got3 = gpu.read(y3, 128 * n).reshape(128, n)
+    e = rms_errs(got3, got[:128])
     assert e[0] < 5e-5 and e[1] < 5e-6, e
+    # ... and against the oracle itself, like the big launch
+    e = rms_errs(got3[:, rows], want[:128])
+    assert e[0] < 5e-4 and e[1] < 5e-5, e
