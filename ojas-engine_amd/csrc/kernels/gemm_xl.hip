@@ -599,7 +599,11 @@ __device__ __forceinline__ void gemm_bd_body(const ushort* __restrict__ xh, cons
                     __hip_atomic_store(o, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                     __hip_atomic_store(o + 256, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                 }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");      // the stores have left before the slice is counted
+        // Every wave's partial-tile stores (written through, system scope) must have been acknowledged before the
+        // slice is counted: said with the instruction itself — a workgroup-scope release fence need not wait for
+        // vector memory on this target, and nothing wider is affordable here (see above).
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (tid == 0u) *(volatile uint*)lds = atomicAdd(cnt + tile, 1u);
         __syncthreads();

@@ -70,6 +70,7 @@ struct ojh_device {
     int px = 1;                  // OJAS_HIP_PX: 0 = never take it
     uint32_t q4k_ml_min_m = 2;   // OJAS_HIP_Q4K_ML_MIN_M: tokens from which long Q4_K matrices (32768 rows or more) take the LDS-copy form (0: never)
     uint32_t q4k_xt_min_m = 96;  // OJAS_HIP_Q4K_XT_MIN_M: tokens from which Q4_K rows take the 128 x 128 int8 tile (0: never)
+    bool q4k_xt64 = false;       // OJAS_HIP_Q4K_XT64=1: that tile always in its 64-row form
     bool no_scratch = false;     // set around calls that may not allocate (ojh_mm_noalloc): paths that need library scratch are skipped
     uint32_t q4k_mf_min_m = 5;   // OJAS_HIP_Q4K_MF_MIN_M: tokens from which Q4_K rows go to the int8 matrix cores
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,

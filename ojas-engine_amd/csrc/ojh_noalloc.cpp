@@ -65,6 +65,8 @@ extern "C" int ojh_mm_noalloc(ojh_device *dev, const ojh_buf *x, size_t x_off, i
     // loading a code object allocates: both families must be resident before the call
     if (!dev->modules.count("gemv_q8k") || !dev->modules.count("gemm_q8k"))
         return ojh_fail(OJH_ERR_NOT_LOADED, "ojh_mm_noalloc: ensure_family(\"gemv_q8k\") and (\"gemm_q8k\") first");
+    if (ojh_grid_type(w->type) && !dev->modules.count("iq_grid"))   // (before anything is queued into the static scratch)
+        return ojh_fail(OJH_ERR_NOT_LOADED, "ojh_mm_noalloc: ensure_family(\"iq_grid\") first");
     void *xq = dev->noalloc_scratch, *xs = (char *)dev->noalloc_scratch + OJH_NOALLOC_MAX_ACT;
     if ((rc = ojh_quant_q8k_launch(dev, (const char *)x->ptr + x_off, x_dtype, m, K, xq, xs))) return rc;
     dev->no_scratch = true;    // kernels that need further library scratch (which would be allocated) are not taken

@@ -199,7 +199,7 @@ int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, con
         }
         // 128-row tiles when they give every CU one, 64-row tiles otherwise
         const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;
-        const char *xt = (uint64_t)((N + 127) / 128) * (mp / 128) >= cus && !getenv("OJAS_HIP_Q4K_XT64") ? "gemm_q8k_q4k_xt" : "gemm_q8k_q4k_xt64";
+        const char *xt = (uint64_t)((N + 127) / 128) * (mp / 128) >= cus && !dev->q4k_xt64 ? "gemm_q8k_q4k_xt" : "gemm_q8k_q4k_xt64";
         if ((rc = ojh_launch_shape(dev, xt, K, N, m, sg, sb))) return rc;
         return ojh_launch(dev, xt, {xq, xst->ptr, sums->ptr, wp, yp}, {K, N, m, (uint32_t)(accum != 0), mp}, sg, sb);
     }
@@ -536,11 +536,18 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         }
         uint32_t sg[3], sb[3];
         if ((rc = ojh_launch_shape(dev, (base + "_sk").c_str(), K, N, m, sg, sb))) return rc;
+        // (a forced split counts before the tile is chosen, so that what follows sees the split that will run)
+        if (dev->gemm_split_override > 0) sg[2] = (uint32_t)dev->gemm_split_override;
         if (dev->gemm_sr && base == "gemm_mm_q4kl_bdk" && sg[2] > 1) {   // reproducible bits asked for: its K slices meet in atomics
             base = "gemm_mm_q4kl_bd";
             if ((rc = ojh_launch_shape(dev, (base + "_sk").c_str(), K, N, m, sg, sb))) return rc;
+            if (dev->gemm_split_override > 0) sg[2] = (uint32_t)dev->gemm_split_override;
         }
-        if (dev->gemm_split_override > 0) sg[2] = (uint32_t)dev->gemm_split_override;
+        // ... and tiles without a slice-ordered form (the LDS-shared Q4_K tile, Q6_K, Q8_0) keep K whole under that request:
+        // their slices could only meet in f32 atomics, in arrival order
+        if (dev->gemm_sr && sg[2] > 1 && !(xl && (base == "gemm_mm_q4kl_bd" || (base == "gemm_mm_q4kl" &&
+                (uint64_t)sg[0] * sg[1] * sg[2] >= (uint32_t)dev->prop.multiProcessorCount))))
+            sg[2] = 1;
         // 256-token tiles that fill the chip: the form that dequantizes into the B registers (same grid).  Its step
         // time does not grow with the number of busy CUs as the LDS-shared tile's does (measured: 2.2 us per K step
         // at 224 and at 448 workgroups against 2.0 and 2.4).
