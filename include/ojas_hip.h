@@ -238,7 +238,9 @@ int ojh_mm_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const
  * Lin its own allocation, all with the same K.  The reference's fused q/k/v and gate/up launches
  * (`qkv_q80_dp4a`, `ffn_gu_q80_dp4a`: crates/ojas-core/src/kernels/gemv_q8.rs:229-260) take one
  * pointer per projection in the same way.  Results are bit-identical to `count` calls of
- * `ojh_mm_q8k`; formats without a grouped kernel (Q5_K, Q6_K) run as that many launches.
+ * `ojh_mm_q8k`.  Q4_K, Q5_K and Q6_K tensors may be mixed in one call (a Q4_K_M file keeps attention v and
+ * the feed-forward down in Q6_K): still one launch, every row in its own format's arithmetic; other formats
+ * run as that many launches.
  * `y_offs` (bytes) may be NULL. */
 int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, int count,
                      const ojh_lin *const *ws, ojh_buf *const *ys, const size_t *y_offs);
@@ -314,7 +316,8 @@ int ojh_chain_spin_limit(ojh_device *dev, uint32_t polls);
  *     (`rmsnorm`, crates/ojas-cpu/src/cpu_math.rs:456-460) quantized as `quant_q8k` does, in one
  *     launch; `xn` (f32 [m][k]) may be NULL when only the quantized form is needed.
  *   ojh_ffn_gu_q8k: out[n] = act(gate[n] . x) * (up[n] . x) from one quantized vector; act 0 = SiLU
- *     (cpu_math.rs:486), 1 = GELU tanh form (:497-501).  Q4_K tensors of equal shape. */
+ *     (cpu_math.rs:486), 1 = GELU tanh form (:497-501).  Q4_K, Q5_K or Q6_K tensors of equal shape (the two
+ *     may differ in format); each dot has the bits of that format's matvec. */
 int ojh_rmsnorm_quant_q8k(ojh_device *dev, const ojh_buf *x, size_t x_off, const ojh_buf *gamma, float eps,
                           uint32_t m, uint32_t k, ojh_buf *q, ojh_buf *scales, ojh_buf *xn);
 int ojh_ffn_gu_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const ojh_lin *gate,

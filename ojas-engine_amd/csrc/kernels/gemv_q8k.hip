@@ -811,6 +811,77 @@ __device__ __forceinline__ void gemv_q8k_q6k_body(const signed char* __restrict_
 
 GEMV_Q8K_ENTRIES(q6k, gemv_q8k_q6k_body)
 
+// ---- the fused launches for the other K-quants ---------------------------------------------------
+// A Q4_K_M file keeps some tensors of a stage in Q6_K or Q5_K (attention v, the feed-forward down) beside Q4_K ones;
+// the reference fuses q/k/v and gate/up+activation for every format it decodes with
+// (crates/ojas-cuda/src/kernels/gemv_q8.rs:105-143, :229-260).  These entries take a GGUF type per tensor (12 = Q4_K,
+// 13 = Q5_K, 14 = Q6_K, one per byte of TYPES) and give every row the lane map and the order of operations of that
+// type's single-tensor matvec — gemv_q8k_<fmt> — so each output has the bits of a launch of its own.  One row per wave.
+//   gemv_q8k_kq_x4(xq, xs, w0, w1, w2, w3, y0, y1, y2, y3, K, E0, E1, E2, E3, TYPES)
+//   ffn_gu_q8k_kq(xq, xs, wg, wu, out, K, N, ACT, TYPES)        TYPES: byte 0 gate, byte 1 up
+__device__ __forceinline__ float kq_row_dot(uint type, const uchar* __restrict__ wrow, const signed char* __restrict__ xq,
+                                            const float* __restrict__ xs, uint nsb, uint lane) {
+    float acc = 0.0f;
+    if (type == 14u) {            // gemv_q8k_q6k_body: four lanes per super-block
+        const uint g = lane >> 2, hf = (lane >> 1) & 1u, l0 = (lane & 1u) * 16u;
+        for (uint sb = g; sb < nsb; sb += 16u) {
+            const Q6kW raw = q6k_load_w(wrow + (size_t)sb * Q6K_BYTES, hf, l0);
+            const Q6kX f = q6k_load_x(xq, xs, sb, hf, l0);
+            acc += q6k_lane_dot(raw, f);
+        }
+    } else {
+        const uint g = lane >> 3, l = lane & 7u, c = l >> 1;
+        if (type == 13u) {        // gemv_q8k_q5k_body
+            for (uint sb = g; sb < nsb; sb += 8u) {
+                const uchar* blk = wrow + (size_t)sb * Q5K_BYTES;
+                const uint4 hdr = *(const uint4*)blk, qh = *(const uint4*)(blk + 16u + (l & 1u) * 16u);
+                const uint4 qs = *(const uint4*)(blk + 48u + l * 16u);
+                const Q4kFrag f = q4k_load_frag(xq, xs, sb, l);
+                acc += q5k_lane_dot(hdr, qs, qh, c, f);
+            }
+        } else {                  // gemv_q8k_q4k_body
+            for (uint sb = g; sb < nsb; sb += 8u) {
+                const uchar* blk = wrow + (size_t)sb * Q4K_BYTES;
+                const uint4 hdr = *(const uint4*)blk, qs = *(const uint4*)(blk + 16u + l * 16u);
+                const Q4kFrag f = q4k_load_frag(xq, xs, sb, l);
+                acc += q4k_lane_dot(hdr, qs, c, f);
+            }
+        }
+    }
+    return wave_sum(acc);
+}
+__device__ __forceinline__ uint kq_block_bytes(uint type) { return type == 14u ? Q6K_BYTES : type == 13u ? Q5K_BYTES : Q4K_BYTES; }
+
+extern "C" __global__ void __launch_bounds__(256)
+gemv_q8k_kq_x4(const signed char* xq, const float* xs, const uchar* w0, const uchar* w1, const uchar* w2, const uchar* w3,
+               float* y0, float* y1, float* y2, float* y3, uint K, uint E0, uint E1, uint E2, uint E3, uint TYPES) {
+    const uint lane = threadIdx.x & 63u;
+    const uint gr = (uint)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)));
+    if (gr >= E3) return;
+    const uint nsb = K >> 8;
+    const uchar* w;
+    float* y;
+    uint lr, type;
+    if (gr < E0) { w = w0; y = y0; lr = gr; type = TYPES & 0xFFu; }
+    else if (gr < E1) { w = w1; y = y1; lr = gr - E0; type = (TYPES >> 8) & 0xFFu; }
+    else if (gr < E2) { w = w2; y = y2; lr = gr - E1; type = (TYPES >> 16) & 0xFFu; }
+    else { w = w3; y = y3; lr = gr - E2; type = TYPES >> 24; }
+    const float t = kq_row_dot(type, w + (size_t)lr * nsb * kq_block_bytes(type), xq, xs, nsb, lane);
+    if (lane == 0) y[lr] = t;
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+ffn_gu_q8k_kq(const signed char* __restrict__ xq, const float* __restrict__ xs, const uchar* __restrict__ wg,
+              const uchar* __restrict__ wu, float* __restrict__ out, uint K, uint N, uint ACT, uint TYPES) {
+    const uint lane = threadIdx.x & 63u;
+    const uint row = (uint)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)));
+    if (row >= N) return;
+    const uint nsb = K >> 8, tg = TYPES & 0xFFu, tu = (TYPES >> 8) & 0xFFu;
+    const float sg = kq_row_dot(tg, wg + (size_t)row * nsb * kq_block_bytes(tg), xq, xs, nsb, lane);
+    const float su = kq_row_dot(tu, wu + (size_t)row * nsb * kq_block_bytes(tu), xq, xs, nsb, lane);
+    if (lane == 0) out[row] = ffn_act(sg, ACT) * su;
+}
+
 // Tall matrices (an output head): rows grid-stride, the wave's share of the quantized activations
 // loaded once and kept in registers (21 per 4096 of K), so the per-row traffic through the vector
 // memory path is the row's own bytes only (head 151936 x 4096: 104 -> 93 us; the same form of the

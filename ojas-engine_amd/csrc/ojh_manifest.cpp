@@ -457,6 +457,61 @@ static int check_gemv_q8k_x4(const ojh_kernel_spec *s, const uint32_t *c, const 
     return OJH_OK;
 }
 
+// The same launches with a GGUF type per tensor (a byte each of the last constant): Q4_K, Q5_K or Q6_K.
+static const ojh_block_format *kq_type(const ojh_kernel_spec *s, uint32_t t, int which) {
+    if (t != OJH_Q4_K && t != OJH_Q5_K && t != OJH_Q6_K) {
+        ojh_fail(OJH_ERR_UNSUPPORTED, "%s: tensor %d has GGUF type %u; takes Q4_K (12), Q5_K (13) or Q6_K (14)", s->name, which, t);
+        return nullptr;
+    }
+    return ojh_format(t);
+}
+static int check_gemv_q8k_kq_x4(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                                const uint32_t block[3], size_t need[16], size_t align[16]) {
+    uint32_t K = c[0], E[4] = {c[1], c[2], c[3], c[4]}, T = c[5];
+    if (K == 0 || K % 256) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a positive multiple of 256", s->name, K);
+    int rc;
+    if ((rc = check_block(block, 0))) return rc;
+    if (E[0] > E[1] || E[1] > E[2] || E[2] > E[3] || E[3] == 0)
+        return ojh_fail(OJH_ERR_ARG, "%s: row totals %u,%u,%u,%u must not decrease", s->name, E[0], E[1], E[2], E[3]);
+    if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * (block[0] / 64) < E[3])
+        return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover N=%u rows", s->name, E[3]);
+    need[0] = (size_t)K;
+    need[1] = (size_t)(K / 256) * 4;
+    align[1] = 4;
+    for (int i = 0; i < 4; i++) {
+        const ojh_block_format *f = kq_type(s, (T >> (8 * i)) & 0xFFu, i);
+        if (!f) return OJH_ERR_UNSUPPORTED;
+        size_t rows = E[i] - (i ? E[i - 1] : 0);
+        need[2 + i] = rows * (K / 256) * f->bytes;
+        need[6 + i] = rows * 4;
+        align[2 + i] = ojh_block_align(f);
+        align[6 + i] = 4;
+    }
+    return OJH_OK;
+}
+static int check_ffn_gu_kq(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                           const uint32_t block[3], size_t need[16], size_t align[16]) {
+    uint32_t K = c[0], N = c[1], ACT = c[2], T = c[3];
+    if (K == 0 || K % 256 || N == 0) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a positive multiple of 256, N=%u positive", s->name, K, N);
+    if (ACT > 1) return ojh_fail(OJH_ERR_ARG, "%s: ACT=%u (0 = SiLU, 1 = GELU)", s->name, ACT);
+    if (T >> 16) return ojh_fail(OJH_ERR_ARG, "%s: TYPES=%#x carries two type bytes", s->name, T);
+    int rc;
+    if ((rc = check_block(block, 0))) return rc;
+    if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * (block[0] / 64) < N)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover N=%u rows", s->name, N);
+    const ojh_block_format *fg = kq_type(s, T & 0xFFu, 0), *fu = kq_type(s, (T >> 8) & 0xFFu, 1);
+    if (!fg || !fu) return OJH_ERR_UNSUPPORTED;
+    need[0] = (size_t)K;
+    need[1] = (size_t)(K / 256) * 4;
+    need[2] = (size_t)N * (K / 256) * fg->bytes;
+    need[3] = (size_t)N * (K / 256) * fu->bytes;
+    need[4] = (size_t)N * 4;
+    align[1] = align[4] = 4;
+    align[2] = ojh_block_align(fg);
+    align[3] = ojh_block_align(fu);
+    return OJH_OK;
+}
+
 // ffn_gu_q8k_<fmt>(xq, xs, wg, wu, out, K, N, ACT): one wave per row
 static int check_ffn_gu(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                         const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -1526,6 +1581,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("matmul_q8row", "rowq8", 5, 3, 0, 2, check_rowq8, shape_rowq8);
     add("matmul_q8row_bias", "rowq8", 6, 3, 0, 3, check_rowq8, shape_rowq8);
     add("ffn_gu_q8k_q4k", "gemv_q8k", 5, 3, OJH_Q4_K, 1, check_ffn_gu, shape_rows);
+    add("ffn_gu_q8k_kq", "gemv_q8k", 5, 4, 0, 1, check_ffn_gu_kq, shape_rows);
+    add("gemv_q8k_kq_x4", "gemv_q8k", 10, 6, 0, 1, check_gemv_q8k_kq_x4, shape_rows);
     add("rmsnorm_q8k", "gemv_q8k", 5, 4, 0, 0, check_rmsnorm_q8k, shape_rmsnorm);
     add("quantize_q8k", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);

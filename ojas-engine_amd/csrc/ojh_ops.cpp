@@ -351,6 +351,28 @@ extern "C" int ojh_mm_q8k_multi(ojh_device *dev, const ojh_buf *xq, const ojh_bu
     if ((rc = ensure(dev, "gemv_q8k"))) return rc;
     for (int i = 0; i < count; i++)
         if (ojh_grid_type(ws[i]->type) && (rc = ensure(dev, "iq_grid"))) return rc;
+    // a stage that mixes Q4_K, Q5_K and Q6_K tensors (a Q4_K_M file does): still one launch, every row in its own
+    // format's arithmetic
+    bool kquants = count > 1;
+    for (int i = 0; i < count; i++)
+        if (ws[i]->type != OJH_Q4_K && ws[i]->type != OJH_Q5_K && ws[i]->type != OJH_Q6_K) kquants = false;
+    if (!grouped && kquants) {
+        std::vector<void *> p = {xq->ptr, xscales->ptr};
+        uint32_t ends[4], run = 0, types = 0;
+        for (int i = 0; i < 4; i++) {
+            int j = i < count ? i : count - 1;
+            p.push_back(at(ws[j]->raw, ws[j]->off));
+            if (i < count) run += ws[i]->n;
+            ends[i] = run;
+            types |= ws[j]->type << (8 * i);
+        }
+        for (int i = 0; i < 4; i++) {
+            int j = i < count ? i : count - 1;
+            p.push_back(at(ys[j], y_offs ? y_offs[j] : 0));
+        }
+        uint32_t grid[3] = {(run + 3) / 4, 1, 1}, block[3] = {256, 1, 1};
+        return ojh_launch(dev, "gemv_q8k_kq_x4", p, {ws[0]->k, ends[0], ends[1], ends[2], ends[3], types}, grid, block);
+    }
     if (!grouped || count == 1) {   // formats without a grouped entry: one launch per projection
         for (int i = 0; i < count; i++) {
             const ojh_block_format *fi = ojh_format(ws[i]->type);
@@ -743,8 +765,9 @@ extern "C" int ojh_rmsnorm_quant_q8k(ojh_device *dev, const ojh_buf *x, size_t x
 extern "C" int ojh_ffn_gu_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf *xscales, const ojh_lin *gate,
                               const ojh_lin *up, ojh_buf *out, size_t out_off, int act) {
     if (!dev || !gate || !up) return ojh_fail(OJH_ERR_ARG, "ojh_ffn_gu_q8k: NULL argument");
-    if (gate->type != OJH_Q4_K || up->type != OJH_Q4_K)
-        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_ffn_gu_q8k: gate and up must be Q4_K (got %u, %u)", gate->type, up->type);
+    auto kq = [](uint32_t t) { return t == OJH_Q4_K || t == OJH_Q5_K || t == OJH_Q6_K; };
+    if (!kq(gate->type) || !kq(up->type))
+        return ojh_fail(OJH_ERR_UNSUPPORTED, "ojh_ffn_gu_q8k: gate and up must be Q4_K, Q5_K or Q6_K (got %u, %u)", gate->type, up->type);
     if (gate->n != up->n || gate->k != up->k)
         return ojh_fail(OJH_ERR_ARG, "ojh_ffn_gu_q8k: gate is %ux%u, up is %ux%u", gate->n, gate->k, up->n, up->k);
     if (act != 0 && act != 1) return ojh_fail(OJH_ERR_ARG, "ojh_ffn_gu_q8k: act=%d (0 = SiLU, 1 = GELU)", act);
@@ -754,10 +777,13 @@ extern "C" int ojh_ffn_gu_q8k(ojh_device *dev, const ojh_buf *xq, const ojh_buf 
     if ((rc = span_ok("ffn_gu: xq", xq, 0, nsb * 256, 16))) return rc;
     if ((rc = span_ok("ffn_gu: xscales", xscales, 0, nsb * 4, 4))) return rc;
     if ((rc = span_ok("ffn_gu: out", out, out_off, (size_t)N * 4, 4))) return rc;
-    if ((rc = span_ok("ffn_gu: gate", gate->raw, gate->off, gate->row_bytes * N, 16))) return rc;
-    if ((rc = span_ok("ffn_gu: up", up->raw, up->off, up->row_bytes * N, 16))) return rc;
+    if ((rc = span_ok("ffn_gu: gate", gate->raw, gate->off, gate->row_bytes * N, ojh_block_align(ojh_format(gate->type))))) return rc;
+    if ((rc = span_ok("ffn_gu: up", up->raw, up->off, up->row_bytes * N, ojh_block_align(ojh_format(up->type))))) return rc;
     if ((rc = ensure(dev, "gemv_q8k"))) return rc;
     uint32_t grid[3] = {(N + 3) / 4, 1, 1}, block[3] = {256, 1, 1};
+    if (gate->type != OJH_Q4_K || up->type != OJH_Q4_K)   // every row in its own format's arithmetic
+        return ojh_launch(dev, "ffn_gu_q8k_kq", {xq->ptr, xscales->ptr, at(gate->raw, gate->off), at(up->raw, up->off), at(out, out_off)},
+                          {K, N, (uint32_t)act, gate->type | (up->type << 8)}, grid, block);
     return ojh_launch(dev, "ffn_gu_q8k_q4k", {xq->ptr, xscales->ptr, at(gate->raw, gate->off), at(up->raw, up->off), at(out, out_off)},
                       {K, N, (uint32_t)act}, grid, block);
 }

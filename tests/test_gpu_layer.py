@@ -93,3 +93,63 @@ def test_errors(gpu, pkg):
         gpu.ffn_gu_q8k(q, s, a, b, gpu.alloc(8))
     with pytest.raises(pkg.OjasHipError, match="act="):
         gpu.ffn_gu_q8k(q, s, a, a, gpu.alloc(8), act=3)
+
+
+Q5_K, Q6_K = 13, 14
+
+
+def _kq_weights(pkg, ty, n, k, *tag):
+    gen = {Q4_K: pkg.synth.q4k_weights, Q5_K: pkg.synth.q5k_weights, Q6_K: pkg.synth.q6k_weights}[ty]
+    return gen(n, k, "layer-kq", *tag)
+
+
+@pytest.mark.parametrize("act", [0, 1])
+@pytest.mark.parametrize("tg,tu", [(Q6_K, Q6_K), (Q5_K, Q5_K), (Q4_K, Q6_K), (Q5_K, Q4_K)])
+@pytest.mark.parametrize("n,k", [(50, 256), (1001, 4096), (333, 2560)])
+def test_gate_up_with_activation_in_the_other_k_quants(gpu, orc, pkg, n, k, tg, tu, act):
+    """`ojh_ffn_gu_q8k` over Q5_K / Q6_K / mixed tensors (the reference fuses gate/up for every format it decodes
+    with, crates/ojas-cuda/src/kernels/gemv_q8.rs:105-143): the CPU path's dots, and bit for bit the product of the
+    two single-tensor matvecs."""
+    wg, wu = _kq_weights(pkg, tg, n, k, "wg", n, k, tg), _kq_weights(pkg, tu, n, k, "wu", n, k, tu)
+    x = pkg.synth.normal_f32(k, "layer-kq", "gx", k)
+    xq, xs = gpu.alloc_bytes(k), gpu.alloc(k // 256)
+    gpu.quant_q8k(gpu.upload(x), 1, k, xq, xs)
+    lg, lu = gpu.lin(tg, n, k, wg), gpu.lin(tu, n, k, wu)
+    out = gpu.upload(np.full(n + 4, 55.5, np.float32))
+    gpu.ffn_gu_q8k(xq, xs, lg, lu, out, act)
+    got = gpu.read(out, n + 4)
+    assert np.all(got[n:] == 55.5)
+    want = orc.ffn_act(orc.matvec_kq(wg, tg, n, k, x), act) * orc.matvec_kq(wu, tu, n, k, x)
+    assert peak_err(got[:n], want) <= TOL_SEEN
+    yg, yu = gpu.alloc(n), gpu.alloc(n)
+    gpu.mm_q8k(xq, xs, lg, yg)
+    gpu.mm_q8k(xq, xs, lu, yu)
+    sep = (orc.ffn_act(gpu.read(yg, n), act) * gpu.read(yu, n)).astype(np.float32)
+    assert peak_err(got[:n], sep) <= 1e-6          # the activation function itself runs on the GPU in one, on the host in the other
+
+
+@pytest.mark.parametrize("types", [(Q4_K, Q4_K, Q6_K), (Q6_K, Q5_K), (Q5_K, Q6_K, Q4_K, Q6_K), (Q6_K, Q6_K)])
+@pytest.mark.parametrize("k", [256, 4096, 2304])
+def test_mixed_k_quant_stage_is_one_launch_with_each_formats_bits(gpu, orc, pkg, types, k):
+    """q/k/v (or any group) of one quantized vector with Q4_K, Q5_K and Q6_K tensors side by side —
+    `ojh_mm_q8k_multi` / `ojh_mm_multi`: every output bit for bit what `ojh_mm_q8k` gives for that tensor alone, and
+    the CPU path's `matvec_kq` within 2e-5."""
+    ns = [300, 129, 64, 1000][:len(types)]
+    hs = [_kq_weights(pkg, t, n, k, "mix", i, n, k) for i, (t, n) in enumerate(zip(types, ns))]
+    lins = [gpu.lin(t, n, k, h) for t, n, h in zip(types, ns, hs)]
+    x = pkg.synth.normal_f32(k, "layer-kq", "mixx", k)
+    xd = gpu.upload(x)
+    xq, xs = gpu.alloc_bytes(k), gpu.alloc(k // 256)
+    gpu.quant_q8k(xd, 1, k, xq, xs)
+    ys = [gpu.upload(np.full(n + 2, 9.25, np.float32)) for n in ns]
+    gpu.mm_q8k_multi(xq, xs, lins, ys)
+    ym = [gpu.upload(np.full(n + 2, 9.25, np.float32)) for n in ns]
+    gpu.mm_multi(xd, lins, ym)
+    for t, n, h, l, y, y2 in zip(types, ns, hs, lins, ys, ym):
+        got = gpu.read(y, n + 2)
+        assert np.all(got[n:] == 9.25)
+        one = gpu.alloc(n)
+        gpu.mm_q8k(xq, xs, l, one)
+        assert np.array_equal(got[:n].view(np.uint32), gpu.read(one, n).view(np.uint32)), (t, n)
+        assert np.array_equal(gpu.read(y2, n + 2).view(np.uint32), got.view(np.uint32))
+        assert peak_err(got[:n], orc.matvec_kq(h, t, n, k, x)) <= 2e-5
