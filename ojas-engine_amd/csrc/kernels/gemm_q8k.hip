@@ -621,10 +621,15 @@ __device__ __forceinline__ void gxt_planes(const GqW& w, gq_i4 (&BA)[4], gq_i4 (
 // TH = 1: eight row tiles (128 rows) per workgroup, a wave takes one of them against all eight passes of 16 tokens;
 // TH = 2: four row tiles (64 rows), two waves per tile with four passes each — for matrices with too few rows to give
 // every CU a 128-row tile.
-template <int TH>
+// SPLIT: the workgroup takes slice blockIdx.z of the super-blocks; the slices' partial tiles meet in `part`, one counter
+// per tile in `cnt` (zero before the first launch, every launch leaves zeros): the slice that finds all the others
+// counted adds them in slice order — its own read back too, so the sum does not depend on who came last — and owns y.
+template <int TH, bool SPLIT = false>
 __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restrict__ xq, const float* __restrict__ xst,
                                                      const float* __restrict__ sums, const uchar* __restrict__ w,
-                                                     float* __restrict__ y, uint K, uint N, uint M, uint ACC, uint MP, uchar* lds) {
+                                                     float* __restrict__ y, uint K, uint N, uint M, uint ACC, uint MP, uchar* lds,
+                                                     float* __restrict__ part = nullptr, uint* __restrict__ cnt = nullptr,
+                                                     uint nsplit = 1u) {
     constexpr int P = 8 / TH;
     constexpr uint RT = 8u / TH;                                    // row tiles per workgroup
     const uint tid = threadIdx.x, lane = tid & 63u;
@@ -677,14 +682,18 @@ __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restri
     const uint side_lds = GXT_TOK * 256u + (th * (16u * P) + n) * 32u + 8u * kg, sc_lds = GXT_TOK * 288u + (th * (16u * P) + 4u * kg) * 4u;
     const uint sh = 8u * kg;
 
-    GqW cur = gq_load(w + wrow, kg);
-    copies(0u, 0u);
-    for (uint sb = 0; sb < nsb; sb++) {
-        const uint stage = sb & 1u;
+    // the super-blocks of this workgroup: all of them, or slice blockIdx.z of ceil(nsb / nsplit) each
+    const uint per = SPLIT ? (nsb + nsplit - 1u) / nsplit : nsb;
+    const uint sb0 = SPLIT ? blockIdx.z * per : 0u, sb1 = SPLIT ? min(nsb, sb0 + per) : nsb;
+
+    GqW cur = gq_load((w + (size_t)sb0 * Q4K_BYTES) + wrow, kg);
+    copies(sb0, 0u);
+    for (uint sb = sb0; sb < sb1; sb++) {
+        const uint stage = (sb - sb0) & 1u;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();                                            // stage `stage` complete; the other one is free
-        if (sb + 1u < nsb) copies(sb + 1u, stage ^ 1u);
-        const uint sbn = min(sb + 1u, nsb - 1u);
+        if (sb + 1u < sb1) copies(sb + 1u, stage ^ 1u);
+        const uint sbn = min(sb + 1u, sb1 - 1u);
         const uchar* st = lds + stage * GXT_STAGE;
         gq_i4 BA[4], BB[4];
         float n0, n1, d;
@@ -717,6 +726,45 @@ __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restri
             __builtin_amdgcn_sched_barrier(0);
         }
     }
+    if (SPLIT) {
+        // The partial tile goes out as the registers hold it ([pair][thread]: 512 contiguous bytes per wave and store),
+        // written through and read from behind the L2 (system-scope accesses): a tile's slices run on different XCDs,
+        // whose L2s do not see each other's lines.  The stores are awaited by instruction before the slice is counted.
+        typedef unsigned long long u64;
+        const uint ns_eff = (nsb + per - 1u) / per;
+        const uint tile = blockIdx.y * gridDim.x + blockIdx.x;
+        const uint te = threadIdx.x;
+        u64* const mine = (u64*)part + ((size_t)tile * ns_eff + blockIdx.z) * (uint)(P * 2) * 512u + te;
+#pragma unroll
+        for (int p = 0; p < P; p++)
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                __hip_atomic_store(mine + (size_t)(p * 2 + h) * 512u,
+                                   (u64)__float_as_uint(acc[p][2 * h]) | ((u64)__float_as_uint(acc[p][2 * h + 1]) << 32),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (te == 0u) *(volatile uint*)lds = atomicAdd(cnt + tile, 1u);
+        __syncthreads();
+        if ((uint)__builtin_amdgcn_readfirstlane((int)*(volatile uint*)lds) != ns_eff - 1u) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        // (a slice's loads all in flight before the first is added: one trip to memory per slice, not one per load)
+        const u64* const all = (const u64*)part + (size_t)tile * ns_eff * (uint)(P * 2) * 512u + te;
+        for (uint sl = 0; sl < ns_eff; sl++) {
+            u64 v[P * 2];
+#pragma unroll
+            for (int i = 0; i < P * 2; i++)
+                v[i] = __hip_atomic_load(all + ((size_t)sl * (uint)(P * 2) + (uint)i) * 512u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+#pragma unroll
+            for (int i = 0; i < P * 2; i++) {
+                const float a = __uint_as_float((uint)v[i]), b = __uint_as_float((uint)(v[i] >> 32));
+                acc[i / 2][2 * (i % 2)] = sl == 0u ? a : acc[i / 2][2 * (i % 2)] + a;
+                acc[i / 2][2 * (i % 2) + 1] = sl == 0u ? b : acc[i / 2][2 * (i % 2) + 1] + b;
+            }
+        }
+        if (te == 0u) cnt[tile] = 0u;                               // ready for the next launch
+    }
     // (the lane id asked of the hardware again, so that nothing of it has to live through the loop)
     const uint le = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     const uint r = blockIdx.x * (16u * RT) + rt * 16u + (le & 15u);
@@ -743,4 +791,13 @@ gemm_q8k_q4k_xt64(const signed char* xq, const float* xst, const float* sums, co
                   uint ACC, uint MP) {
     __shared__ __attribute__((aligned(1024))) uchar lds_xt[2 * GXT_STAGE];
     gemm_q8k_q4k_xt_body<2>(xq, xst, sums, w, y, K, N, M, ACC, MP, lds_xt);
+}
+// the 64-row tile over K slices, for matrices whose 64-row tiles alone leave most CUs idle:
+//   gemm_q8k_q4k_xt64_sr(xq, xst, sums, w, y, part, cnt, K, N, M, ACC, MP, NSPLIT)
+//   grid [ceil(N / 64), MP / 128, slices]; slices = ceil(nsb / ceil(nsb / NSPLIT)); part: tiles x slices x 32 KB
+extern "C" __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
+gemm_q8k_q4k_xt64_sr(const signed char* xq, const float* xst, const float* sums, const uchar* w, float* y, float* part, uint* cnt,
+                     uint K, uint N, uint M, uint ACC, uint MP, uint NSPLIT) {
+    __shared__ __attribute__((aligned(1024))) uchar lds_xt[2 * GXT_STAGE];
+    gemm_q8k_q4k_xt_body<2, true>(xq, xst, sums, w, y, K, N, M, ACC, MP, lds_xt, part, cnt, NSPLIT);
 }

@@ -246,6 +246,51 @@ static int check_gemm_q8k_xt(const ojh_kernel_spec *s, const uint32_t *c, const 
     align[1] = align[4] = 4;
     return OJH_OK;
 }
+// gemm_q8k_q4k_xt64_sr(xq, xst, sums, w, y, part, cnt, K, N, M, ACC, MP, NSPLIT): grid [ceil(N / 64), MP / 128, slices],
+// slices = those of NSPLIT that hold a super-block; part: 32 KB per tile and slice; cnt: a zeroed word per tile
+static int check_gemm_q8k_xt_sr(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                                const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const uint32_t K = c[0], N = c[1], M = c[2], MP = c[4], nsplit = c[5];
+    if (!K || K % 256 || !N || !M) return ojh_fail(OJH_ERR_ARG, "%s: K=%u (a multiple of 256) N=%u M=%u", s->name, K, N, M);
+    if (MP != (M + 127) / 128 * 128) return ojh_fail(OJH_ERR_ARG, "%s: MP=%u must be M=%u rounded up to 128", s->name, MP, M);
+    if ((uint64_t)M * K > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "%s: M*K exceeds 2^32 activations", s->name);
+    if (c[3] > 1) return ojh_fail(OJH_ERR_ARG, "%s: ACC=%u", s->name, c[3]);
+    const size_t nsb = K / 256;
+    if (!nsplit || nsplit > nsb) return ojh_fail(OJH_ERR_ARG, "%s: NSPLIT=%u (1 .. K/256)", s->name, nsplit);
+    int rc;
+    if ((rc = check_block(block, 512))) return rc;
+    const uint32_t slices = ojh_gemm_sr_slices(K, nsplit);
+    if (grid[0] != (N + 63) / 64 || grid[1] != MP / 128 || grid[2] != slices)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, (N + 63) / 64, MP / 128, slices);
+    if ((uint64_t)N * nsb * 144 > 0xFFFFFFFFull) return ojh_fail(OJH_ERR_ARG, "%s: the weight tensor exceeds 4 GiB", s->name);
+    const size_t tiles = (size_t)grid[0] * grid[1];
+    need[0] = (size_t)M * K;
+    need[1] = nsb * MP * 4;
+    need[2] = nsb * MP * 32;
+    need[3] = (size_t)N * nsb * 144;
+    need[4] = (size_t)M * N * 4;
+    need[5] = tiles * slices * 32768;
+    need[6] = tiles * 4;
+    align[1] = align[4] = align[6] = 4;
+    align[5] = 8;
+    return OJH_OK;
+}
+static int shape_gemm_q8k_xt_sr(const ojh_kernel_spec *, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
+                                uint32_t grid[3], uint32_t block[3]) {
+    if (!M) M = 1;
+    grid[0] = (N + 63) / 64;
+    grid[1] = (M + 127) / 128;
+    if (!grid[0]) grid[0] = 1;
+    const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, nsb = K / 256;
+    uint32_t z = (cus + grid[0] * grid[1] - 1) / (grid[0] * grid[1]);
+    if (z > nsb / 2) z = nsb / 2;
+    if (z > 8) z = 8;
+    if (z < 1) z = 1;
+    grid[2] = ojh_gemm_sr_slices(K, z);
+    block[0] = 512;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
 // quantize_q8k{,_bf16}_sides(x, q, scales, xst, sums, K, M, MP): grid [K / 256 * MP / 4, 1, 1]
 static int check_quantize_sides(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                                 const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -1562,6 +1607,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("quantize_q8k_bf16_sides", "gemm_q8k", 5, 3, 0, 0, check_quantize_sides, shape_quantize_sides);
     add("gemm_q8k_q4k_xt", "gemm_q8k", 5, 5, OJH_Q4_K, 1, check_gemm_q8k_xt, shape_gemm_q8k_xt);
     add("gemm_q8k_q4k_xt64", "gemm_q8k", 5, 5, OJH_Q4_K, 2, check_gemm_q8k_xt, shape_gemm_q8k_xt);
+    add("gemm_q8k_q4k_xt64_sr", "gemm_q8k", 7, 6, OJH_Q4_K, 2, check_gemm_q8k_xt_sr, shape_gemm_q8k_xt_sr);
     add("gemm_q8k_q4k_mk", "gemm_q8k", 4, 4, OJH_Q4_K, 2, check_gemm_q8k_ml, shape_mk);
     add("relayout_q4k_q4l", "dequant", 4, 1, OJH_Q4_K, 0, check_relayout, shape_relayout);
     add("embed_q80", "dequant", 2, 2, OJH_Q8_0, 0, check_embed, shape_embed);

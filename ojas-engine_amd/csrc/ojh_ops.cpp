@@ -151,10 +151,24 @@ static int pick_rows(const ojh_device *dev, uint32_t n) {
 // y (=,+=,+bias) quantized-x . W^T for K-quant weights: the matvec (m = 1) and its batched form.
 // Whether a Q4_K product of m tokens takes the 128-token int8 tile (when its tiles cover at least half of the CUs: a
 // 4096-row matrix against 128 tokens stays below).
+// K slices the 64-row int8 tile is launched over: 1 when the tiles alone give every CU one, otherwise as many as fill
+// the chip with at least two super-blocks each (at most eight); 0 when even those leave more than half the CUs idle.
+static uint32_t q4k_xt_slices(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t m) {
+    const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount, nsb = K / 256;
+    const uint64_t tiles = (uint64_t)((N + 63) / 64) * ((m + 127) / 128);
+    const uint32_t whole = tiles * 2 >= cus ? 1u : 0u;
+    if (tiles >= cus || dev->q4k_xt_split == 0) return whole;
+    uint32_t z = (uint32_t)((cus + tiles - 1) / tiles);
+    if (z > nsb / 2) z = nsb / 2;
+    if (z > 8) z = 8;
+    if (dev->q4k_xt_split > 1) z = dev->q4k_xt_split <= nsb ? dev->q4k_xt_split : nsb;
+    if (z < 2 || tiles * z * 2 < cus) return whole;
+    return ojh_gemm_sr_slices(K, z);
+}
 bool ojh_q4k_xt_taken(const ojh_device *dev, const ojh_lin *w, uint32_t m, const void *wp) {
-    const uint32_t K = w->k, N = w->n, xt_mp = (m + 127) / 128 * 128;
+    const uint32_t K = w->k, N = w->n;
     return w->type == OJH_Q4_K && dev->q4k_xt_min_m && m >= dev->q4k_xt_min_m && !dev->no_scratch &&
-           (uint64_t)((N + 63) / 64) * (xt_mp / 128) * 2 >= (uint32_t)dev->prop.multiProcessorCount &&
+           q4k_xt_slices(dev, K, N, m) >= 1 &&
            (uint64_t)m * K <= 0xFFFFFFFFull && (uint64_t)w->row_bytes * N <= 0xFFFFFFFFull && (uintptr_t)wp % 16 == 0;
 }
 
@@ -196,6 +210,17 @@ int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, con
         if (!sides_ready) {
             if ((rc = ojh_launch_shape(dev, "q8k_token_sides", K, N, m, sg, sb))) return rc;
             if ((rc = ojh_launch(dev, "q8k_token_sides", {xq, xs, xst->ptr, sums->ptr}, {K, m, mp}, sg, sb))) return rc;
+        }
+        // too few 64-row tiles for the chip: K slices of them, summed in slice order by the last to finish
+        if (const uint32_t z = q4k_xt_slices(dev, K, N, m); z > 1) {
+            const size_t tiles = (size_t)((N + 63) / 64) * (mp / 128);
+            ojh_buf *part, *cnt;
+            if ((rc = ojh_scratch_get(dev, "xt_part", tiles * z * 32768, &part))) return rc;
+            if ((rc = ojh_scratch_get_zeroed(dev, "xt_cnt", tiles * 4, &cnt))) return rc;
+            sg[0] = (N + 63) / 64; sg[1] = mp / 128; sg[2] = z;
+            sb[0] = 512; sb[1] = sb[2] = 1;
+            return ojh_launch(dev, "gemm_q8k_q4k_xt64_sr", {xq, xst->ptr, sums->ptr, wp, yp, part->ptr, cnt->ptr},
+                              {K, N, m, (uint32_t)(accum != 0), mp, z}, sg, sb);
         }
         // 128-row tiles when they give every CU one, 64-row tiles otherwise
         const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;

@@ -213,6 +213,36 @@ def test_prefill_tiles_by_name(gpu, orc, pkg, m, n, k):
                 assert peak_err(got, want) <= TOL_SEEN and peak_err(got, ref) <= 2e-6
                 bits[name] = got.view(np.uint32).copy()
     assert np.array_equal(bits["gemm_q8k_q4k_xt"], bits["gemm_q8k_q4k_xt64"])
+    # the 64-row tile over K slices: one slice gives the unsliced bits; more give the slice sums added in slice order
+    # (the same bits on every launch, whoever finishes last), and every launch leaves the tile counters at zero
+    tiles = (n + 63) // 64 * (mp // 128)
+    cnt = gpu.alloc_bytes(tiles * 4)
+    gpu.memset0(cnt)
+    for nsplit in sorted({min(s, nsb) for s in (1, 2, 3, nsb)}):
+        per = (nsb + nsplit - 1) // nsplit
+        slices = (nsb + per - 1) // per
+        part = gpu.alloc(tiles * slices * 8192)
+        seen = []
+        for acc in (0, 1, 0):
+            y0 = pkg.synth.normal_f32(m * n, "gq", "xt-y0", acc).reshape(m, n)
+            yd = gpu.upload(np.concatenate([y0.ravel(), np.full(n, 4242.5, np.float32)]))
+            gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_xt64_sr", [(xq, 0), (xst, 0), (sums, 0), (wd, 0), (yd, 0), (part, 0), (cnt, 0)],
+                         [k, n, m, acc, mp, nsplit], [(n + 63) // 64, mp // 128, slices], [512, 1, 1])
+            got = gpu.read(yd, m * n + n)
+            assert np.all(got[m * n:] == 4242.5), "wrote past the last token"
+            assert not gpu.read(cnt, tiles, np.uint32).any()
+            got = got[:m * n].reshape(m, n)
+            if acc:
+                assert peak_err(got - y0, want) <= TOL_SEEN
+            else:
+                assert peak_err(got, want) <= TOL_SEEN and peak_err(got, ref) <= 2e-6
+                seen.append(got.view(np.uint32).copy())
+        assert np.array_equal(seen[0], seen[1]), nsplit
+        if slices == 1:
+            assert np.array_equal(seen[0], bits["gemm_q8k_q4k_xt64"])
+    with pytest.raises(pkg.OjasHipError, match="grid must be"):
+        gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_xt64_sr", [(xq, 0), (xst, 0), (sums, 0), (wd, 0), (ymf, 0), (part, 0), (cnt, 0)],
+                     [k, n, m, 0, mp, 1], [(n + 63) // 64, mp // 128, 2], [512, 1, 1])
     with pytest.raises(pkg.OjasHipError, match="rounded up to 128"):
         gpu.dispatch(gpu.begin(), "gemm_q8k_q4k_xt", [(xq, 0), (xst, 0), (sums, 0), (wd, 0), (ymf, 0)], [k, n, m, 0, mp + 128],
                      [(n + 127) // 128, mp // 128, 1], [512, 1, 1])

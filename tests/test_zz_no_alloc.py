@@ -84,25 +84,29 @@ def test_no_alloc_limits_and_errors(gpu, pkg):
         other.close()
 
 
-def test_no_alloc_records_where_every_allocation_is_refused(gpu, pkg):
+def test_no_alloc_records_where_every_allocation_is_refused(pkg):
     """While a chain of launches is being recorded the library refuses to allocate (scratch that would have to grow,
-    code objects that would have to load: OJH_ERR_ARG).  `ojh_mm_noalloc` must go through there with shapes no earlier
-    call has sized any scratch for, `ojh_mm` on the same shapes must be refused, and the replay must give the bits of
-    an eager `ojh_mm`."""
-    gpu.ensure_family("gemv_q8k")
-    gpu.ensure_family("gemm_q8k")
-    n, k, m = 768, 8192, 96        # 786 432 activations: more than any test before this one quantized at once
-    lin = gpu.lin(Q4_K, n, k, _weights(pkg, Q4_K, n, k, "rec"))
-    xd = gpu.upload(pkg.synth.normal_f32(m * k, "noalloc", "xrec"))
-    ya, yb = gpu.alloc(m * n), gpu.alloc(m * n)
-    gpu.capture_begin()
+    code objects that would have to load: OJH_ERR_ARG).  `ojh_mm_noalloc` must go through there on a handle whose
+    scratch no earlier call has sized (a handle of its own: the other tests' calls cannot have grown it), `ojh_mm` on
+    the same shapes must be refused, and the replay must give the bits of an eager `ojh_mm`."""
+    gpu = pkg.HipGpu(0)
     try:
-        with pytest.raises(pkg.OjasHipError):
-            gpu.mm(xd, lin, ya, m, act_mode=pkg.ACT_Q8K)       # would grow the library's scratch
-        gpu.mm_noalloc(xd, lin, yb, m)
+        gpu.ensure_family("gemv_q8k")
+        gpu.ensure_family("gemm_q8k")
+        n, k, m = 768, 8192, 96
+        lin = gpu.lin(Q4_K, n, k, _weights(pkg, Q4_K, n, k, "rec"))
+        xd = gpu.upload(pkg.synth.normal_f32(m * k, "noalloc", "xrec"))
+        ya, yb = gpu.alloc(m * n), gpu.alloc(m * n)
+        gpu.capture_begin()
+        try:
+            with pytest.raises(pkg.OjasHipError):
+                gpu.mm(xd, lin, ya, m, act_mode=pkg.ACT_Q8K)       # would have to allocate the library's scratch
+            gpu.mm_noalloc(xd, lin, yb, m)
+        finally:
+            graph = gpu.capture_end()
+        graph.launch()
+        gpu.submit()
+        gpu.mm(xd, lin, ya, m, act_mode=pkg.ACT_Q8K)
+        assert np.array_equal(gpu.read(yb, m * n).view(np.uint32), gpu.read(ya, m * n).view(np.uint32))
     finally:
-        graph = gpu.capture_end()
-    graph.launch()
-    gpu.submit()
-    gpu.mm(xd, lin, ya, m, act_mode=pkg.ACT_Q8K)
-    assert np.array_equal(gpu.read(yb, m * n).view(np.uint32), gpu.read(ya, m * n).view(np.uint32))
+        gpu.close()
