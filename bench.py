@@ -435,7 +435,7 @@ def extras(gpu, pkg, lin_q) -> dict:
                                       "peak_tops": 5000.0,
                                       "timed": "quantizer + the tile: from 96 tokens quantize_q8k_sides + gemm_q8k_q4k_xt{,64} "
                                                "(128-token tiles, scales folded into int8 planes, v_mfma_i32_16x16x64_i8; where the "
-                                               "64-row tiles number fewer than the CUs — down at M = 128 — gemm_q8k_q4k_xt64_sr: K slices "
+                                               "64-row tiles alone leave CUs idle or singly occupied — down up to M = 512 — gemm_q8k_q4k_xt64_sr: K slices "
                                                "summed in slice order by the last to finish); below, "
                                                "gemm_q8k_q4k_mf (down at M = 8: gemm_q8k_q4k_mk)", **i8}
     # ---- speculative verify on the Q4_K output head of the decode step, bf16 activations

@@ -151,16 +151,21 @@ static int pick_rows(const ojh_device *dev, uint32_t n) {
 // y (=,+=,+bias) quantized-x . W^T for K-quant weights: the matvec (m = 1) and its batched form.
 // Whether a Q4_K product of m tokens takes the 128-token int8 tile (when its tiles cover at least half of the CUs: a
 // 4096-row matrix against 128 tokens stays below).
-// K slices the 64-row int8 tile is launched over: 1 when the tiles alone give every CU one, otherwise as many as fill
-// the chip with at least two super-blocks each (at most eight); 0 when even those leave more than half the CUs idle.
+// K slices the 64-row int8 tile is launched over (measured on 4096 / 14336-wide matrices at 128 .. 2048 tokens): two
+// workgroups per CU is the aim, with at most eight slices of at least four super-blocks each (two, where four would
+// leave more than half the CUs idle); a grid that already covers more than half the CUs is sliced only when a slice
+// keeps sixteen super-blocks.  1 = unsliced; 0 = even sliced, most CUs would idle: another kernel takes the product.
 static uint32_t q4k_xt_slices(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t m) {
     const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount, nsb = K / 256;
     const uint64_t tiles = (uint64_t)((N + 63) / 64) * ((m + 127) / 128);
     const uint32_t whole = tiles * 2 >= cus ? 1u : 0u;
-    if (tiles >= cus || dev->q4k_xt_split == 0) return whole;
-    uint32_t z = (uint32_t)((cus + tiles - 1) / tiles);
-    if (z > nsb / 2) z = nsb / 2;
+    if (dev->q4k_xt_split == 0 || (tiles > cus && dev->q4k_xt_split == 1)) return whole;
+    uint32_t z = (uint32_t)(2 * (uint64_t)cus / tiles);
     if (z > 8) z = 8;
+    uint32_t cap = nsb / 4;
+    if (tiles * (z < cap ? z : cap) * 2 < cus) cap = nsb / 2;
+    if (z > cap) z = cap;
+    if (tiles * 2 > cus && z > 1 && nsb / z < 16) z = 1;
     if (dev->q4k_xt_split > 1) z = dev->q4k_xt_split <= nsb ? dev->q4k_xt_split : nsb;
     if (z < 2 || tiles * z * 2 < cus) return whole;
     return ojh_gemm_sr_slices(K, z);
