@@ -749,18 +749,29 @@ __device__ __forceinline__ void gemm_q8k_q4k_xt_body(const signed char* __restri
         __syncthreads();
         if ((uint)__builtin_amdgcn_readfirstlane((int)*(volatile uint*)lds) != ns_eff - 1u) return;
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        // (a slice's loads all in flight before the first is added: one trip to memory per slice, not one per load)
+        // (four slices' loads in flight before the first is added: a trip to memory per four slices, not one per load;
+        // past the last slice the loads repeat it and are dropped)
         const u64* const all = (const u64*)part + (size_t)tile * ns_eff * (uint)(P * 2) * 512u + te;
-        for (uint sl = 0; sl < ns_eff; sl++) {
-            u64 v[P * 2];
+        for (uint s0 = 0; s0 < ns_eff; s0 += 4u) {
+            u64 v[4][P * 2];
 #pragma unroll
-            for (int i = 0; i < P * 2; i++)
-                v[i] = __hip_atomic_load(all + ((size_t)sl * (uint)(P * 2) + (uint)i) * 512u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            for (int q = 0; q < 4; q++) {
+                const uint sl = min(s0 + (uint)q, ns_eff - 1u);
 #pragma unroll
-            for (int i = 0; i < P * 2; i++) {
-                const float a = __uint_as_float((uint)v[i]), b = __uint_as_float((uint)(v[i] >> 32));
-                acc[i / 2][2 * (i % 2)] = sl == 0u ? a : acc[i / 2][2 * (i % 2)] + a;
-                acc[i / 2][2 * (i % 2) + 1] = sl == 0u ? b : acc[i / 2][2 * (i % 2) + 1] + b;
+                for (int i = 0; i < P * 2; i++)
+                    v[q][i] = __hip_atomic_load(all + ((size_t)sl * (uint)(P * 2) + (uint)i) * 512u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                if (s0 + (uint)q < ns_eff) {
+#pragma unroll
+                    for (int i = 0; i < P * 2; i++) {
+                        const float a = __uint_as_float((uint)v[q][i]), b = __uint_as_float((uint)(v[q][i] >> 32));
+                        const bool first = s0 + (uint)q == 0u;
+                        acc[i / 2][2 * (i % 2)] = first ? a : acc[i / 2][2 * (i % 2)] + a;
+                        acc[i / 2][2 * (i % 2) + 1] = first ? b : acc[i / 2][2 * (i % 2) + 1] + b;
+                    }
+                }
             }
         }
         if (te == 0u) cnt[tile] = 0u;                               // ready for the next launch
