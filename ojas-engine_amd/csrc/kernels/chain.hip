@@ -148,9 +148,10 @@ __device__ __forceinline__ void ch_quantizer(ChArgs a, uint s, uint q, double* p
     }
     if (pro == OJK_CHAIN_X_RMSNORM) {
         // x * (1 / sqrt(mean(x^2) + eps)) * gamma (crates/ojas-cpu/src/cpu_math.rs:456-460).  Every quantizer
-        // workgroup of the stage sums the whole vector, in the order rmsnorm_q8k does: wave w the segments w, w + 4,
-        // ..., a lane its four values of each, in f64, rounded once.
-        double sq = 0.0;
+        // workgroup of the stage sums the whole vector, in the order rmsnorm_q8k does: a lane the squares of its four
+        // values of a segment, the segment's lanes by wave_sum_f64, the segment sums likewise (tree_sum_f64); in f64, rounded once.
+        if (tid == 0) part[64] = 0.0;
+        __syncthreads();
         for (uint sg = wave; sg < nsb && !gave_up; sg += 8u) {   // two segments of this wave per look
             for (;;) {
                 ChSeg t[2];
@@ -166,23 +167,24 @@ __device__ __forceinline__ void ch_quantizer(ChArgs a, uint s, uint q, double* p
                 }
                 if (!(tg & 1u) || __all(ok)) {
 #pragma unroll
-                    for (int i = 0; i < 2; i++)
-#pragma unroll
-                        for (int e = 0; e < 4; e++) sq += (double)f[i][e] * (double)f[i][e];
+                    for (int i = 0; i < 2; i++) {
+                        double sq = (double)f[i][0] * (double)f[i][0];
+                        sq += (double)f[i][1] * (double)f[i][1];
+                        sq += (double)f[i][2] * (double)f[i][2];
+                        sq += (double)f[i][3] * (double)f[i][3];
+                        sq = wave_sum_f64(sq);
+                        if (lane == 0 && sg + 4u * (uint)i < nsb) part[sg + 4u * (uint)i] = sq;
+                    }
                     break;
                 }
                 if (!ch_again(a, it, cap)) { gave_up = true; break; }
             }
         }
-        for (int off = 32; off > 0; off >>= 1) {
-            const long bits = __double_as_longlong(sq);
-            const int lo = __shfl_xor((int)bits, off), hi = __shfl_xor((int)(bits >> 32), off);
-            sq += __longlong_as_double(((long)hi << 32) | (unsigned int)lo);
-        }
-        if (lane == 0) part[wave] = gave_up ? -1.0 : sq;   // (a sum of squares is never negative)
+        if (gave_up && lane == 0) part[64] = -1.0;          // (a sum of squares is never negative)
         __syncthreads();   // all four waves get here, also one whose wait gave up
-        if (part[0] < 0.0 || part[1] < 0.0 || part[2] < 0.0 || part[3] < 0.0) gave_up = true;
-        const float mean = (float)(((part[0] + part[1]) + (part[2] + part[3])) / (double)a->st[s].K);
+        if (part[64] < 0.0) gave_up = true;
+        const double total = tree_sum_f64(part, nsb, lane);
+        const float mean = (float)(total / (double)a->st[s].K);
         const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(mean, __uint_as_float(a->st[s].eps_bits))));
         const float* gamma = (const float*)x2;
         if (has0) {
@@ -311,7 +313,7 @@ extern "C" __global__ void __launch_bounds__(OJK_CHAIN_THREADS)
 decode_chain_q4k(ojk_chain_args in_kernarg) {
     (void)in_kernarg;   // read through the kernarg segment: stages are indexed at run time
     ChArgs a = (ChArgs)__builtin_amdgcn_kernarg_segment_ptr();
-    __shared__ double part[4];
+    __shared__ double part[65];     // the norm's segment sums; [64]: negative once a wave's wait gave up
     const uint b = blockIdx.x, nst = a->nstages;
     uint s = 0;
     for (uint t = 1; t < nst; t++)

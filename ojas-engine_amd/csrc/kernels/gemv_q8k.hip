@@ -331,20 +331,23 @@ ffn_gu_q8k_q4k(const signed char* __restrict__ xq, const float* __restrict__ xs,
 }
 
 // ---- RMS norm and activation quantizer in one launch --------------------------------------------
-//   rmsnorm_q8k(x, gamma, q, scales, xn, K, M, EPS_BITS, WRITE_XN)    grid M, block 256, K <= 16384
+//   rmsnorm_q8k(x, gamma, q, scales, xn, K, M, EPS_BITS, WRITE_XN)    grid M, block 256 or 1024, K <= 16384
 // xn = x * (1 / sqrt(mean(x^2) + eps)) * gamma  (crates/ojas-cpu/src/cpu_math.rs:456-460), then
 // quant_q8k(xn) (:539-563) without a trip through memory: a decode layer's projections read the
 // normalized vector only through its quantized form.  The mean of squares is summed in f64 and
 // rounded once; the reference sums in f32 in index order, so `inv` may differ in its last bit.
-extern "C" __global__ void __launch_bounds__(256)
+// The order of the f64 sum does not depend on the block size: a lane adds the squares of its four values of a
+// 256-value segment (in index order), the segment's 64 lane sums meet as wave_sum_f64 adds them, and so do the segment
+// sums (segment i in lane i).  A wave owns segments w, w + waves, ...: with sixteen waves, one each up to K = 4096.
+extern "C" __global__ void __launch_bounds__(1024)
 rmsnorm_q8k(const float* __restrict__ x, const float* __restrict__ gamma, signed char* __restrict__ q,
             float* __restrict__ scales, float* __restrict__ xn, uint K, uint M, uint EPS_BITS, uint WRITE_XN) {
-    __shared__ double part[4];
-    const uint m = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    __shared__ double part[64];
+    const uint m = blockIdx.x, tid = threadIdx.x, lane = tid & 63u;
+    const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6)), nw = blockDim.x >> 6;
     const uint nsb = (K + 255u) >> 8;
     const float* row = x + (size_t)m * K;
     const bool vec = (K & 3u) == 0 && (((size_t)row | (size_t)gamma) & 15u) == 0;   // 128-bit loads
-    // wave w owns segments w, w + 4, ...; a lane holds 4 consecutive values of each
     auto load4 = [&](const float* p, uint i0, float (&o)[4]) {
         if (vec && i0 + 3u < K) {
             const float4 t = *(const float4*)(p + i0);
@@ -354,43 +357,39 @@ rmsnorm_q8k(const float* __restrict__ x, const float* __restrict__ gamma, signed
             for (int e = 0; e < 4; e++) o[e] = i0 + e < K ? p[i0 + e] : 0.0f;
         }
     };
-    // up to 4096 values the row and gamma stay in registers between the two passes
-    const bool keep = nsb <= 16u;
+    // the wave's first four segments stay in registers between the two passes (all of them up to 4 x waves x 256 values)
     float kv[4][4], kg[4][4];
-    double ss = 0.0;
-    if (keep) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint i0 = (wave + 4u * j) * 256u + lane * 4u;
-            load4(row, i0, kv[j]);        // past the row: zeros
-            load4(gamma, i0, kg[j]);
+    for (int j = 0; j < 4; j++) {
+        const uint seg = wave + nw * (uint)j;
+        if (seg < nsb) {
+            load4(row, seg * 256u + lane * 4u, kv[j]);      // past the row: zeros
+            load4(gamma, seg * 256u + lane * 4u, kg[j]);
         }
+    }
+    for (uint seg = wave, j = 0; seg < nsb; seg += nw, j++) {
+        float v[4];
+        if (j < 4u) {
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) ss += (double)kv[j][e] * (double)kv[j][e];
-    } else {
-        for (uint seg = wave; seg < nsb; seg += 4u) {
-            float v[4];
+            for (int e = 0; e < 4; e++) v[e] = j == 0 ? kv[0][e] : j == 1 ? kv[1][e] : j == 2 ? kv[2][e] : kv[3][e];
+        } else {
             load4(row, seg * 256u + lane * 4u, v);
-#pragma unroll
-            for (int e = 0; e < 4; e++) ss += (double)v[e] * (double)v[e];
         }
+        double ss = (double)v[0] * (double)v[0];
+        ss += (double)v[1] * (double)v[1];
+        ss += (double)v[2] * (double)v[2];
+        ss += (double)v[3] * (double)v[3];
+        ss = wave_sum_f64(ss);      // the segment's 64 lane sums
+        if (lane == 0) part[seg] = ss;
     }
-    // wave reduction in f64 through two 32-bit halves
-    for (int off = 32; off > 0; off >>= 1) {
-        const long b = __double_as_longlong(ss);
-        const int lo = __shfl_xor((int)b, off), hi = __shfl_xor((int)(b >> 32), off);
-        ss += __longlong_as_double(((long)hi << 32) | (unsigned int)lo);
-    }
-    if (lane == 0) part[wave] = ss;
     __syncthreads();
-    const float mean = (float)(((part[0] + part[1]) + (part[2] + part[3])) / (double)K);
+    const double total = tree_sum_f64(part, nsb, lane);
+    const float mean = (float)(total / (double)K);
     const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(mean, __uint_as_float(EPS_BITS))));
-    for (uint seg = wave, j = 0; seg < nsb; seg += 4u, j++) {
+    for (uint seg = wave, j = 0; seg < nsb; seg += nw, j++) {
         const uint i0 = seg * 256u + lane * 4u;
         float v[4], gm[4], t[4];
-        if (keep) {
+        if (j < 4u) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 v[e] = j == 0 ? kv[0][e] : j == 1 ? kv[1][e] : j == 2 ? kv[2][e] : kv[3][e];

@@ -103,6 +103,33 @@ __device__ __forceinline__ float wave_sum(float v) {
     float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
     return (a + b) + (c + d);
 }
+// The same in f64 (the two halves of a double travel as two 32-bit DPP moves): lanes 1, 2 apart, mirrored in eights and
+// sixteens, then the four rows as (r0 + r1) + (r2 + r3).  One fixed order: whoever sums a segment's 64 lane values with
+// this gets the same bits.
+template <int CTRL>
+__device__ __forceinline__ double dpp_f64(double v) {
+    const long b = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_update_dpp(0, (int)b, CTRL, 0xF, 0xF, true);
+    const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, 0xF, 0xF, true);
+    return __longlong_as_double(((long)hi << 32) | (unsigned int)lo);
+}
+__device__ __forceinline__ double readlane_f64(double v, int lane) {
+    const long b = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_readlane((int)b, lane), hi = __builtin_amdgcn_readlane((int)(b >> 32), lane);
+    return __longlong_as_double(((long)hi << 32) | (unsigned int)lo);
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+    v += dpp_f64<OJK_DPP_QUAD_XOR1>(v);
+    v += dpp_f64<OJK_DPP_QUAD_XOR2>(v);
+    v += dpp_f64<OJK_DPP_ROW_HALF_MIRROR>(v);
+    v += dpp_f64<OJK_DPP_ROW_MIRROR>(v);
+    return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
+}
+// The sum of part[0 .. n - 1] (n <= 64, in LDS) in one fixed order: term i in lane i, zeros above (adding 0.0 changes
+// nothing), then wave_sum_f64's tree — one LDS trip and a dozen steps instead of n dependent ones.
+__device__ __forceinline__ double tree_sum_f64(const double* part, uint n, uint lane) {
+    return wave_sum_f64(lane < n ? part[lane] : 0.0);
+}
 // Saturation of a rounded activation to the int8 range as the reference's quantizers do it,
 // `.round().clamp(-127.0, 127.0) as i8` (crates/ojas-cpu/src/cpu_math.rs:174-179, :545-563): a NaN passes through
 // clamp and becomes 0 in the cast (fmaxf alone would turn it into -127).

@@ -581,7 +581,7 @@ static int check_rmsnorm_q8k(const ojh_kernel_spec *s, const uint32_t *c, const 
                              const uint32_t block[3], size_t need[16], size_t align[16]) {
     uint32_t K = c[0], M = c[1], WR = c[3];
     if (!K || !M || K > 16384) return ojh_fail(OJH_ERR_ARG, "%s: K=%u (1..16384) M=%u", s->name, K, M);
-    int rc = check_block(block, 256);
+    int rc = check_block(block, block[0] == 1024 ? 1024 : 256);     // four or sixteen waves: the same bits
     if (rc) return rc;
     if (grid[0] != M || grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,1,1]", s->name, M);
     uint32_t nsb = (K + 255) / 256;

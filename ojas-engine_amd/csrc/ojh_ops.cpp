@@ -787,7 +787,9 @@ extern "C" int ojh_rmsnorm_quant_q8k(ojh_device *dev, const ojh_buf *x, size_t x
     if ((rc = ensure(dev, "gemv_q8k"))) return rc;
     uint32_t eps_bits;
     memcpy(&eps_bits, &eps, 4);
-    uint32_t grid[3] = {m, 1, 1}, block[3] = {256, 1, 1};
+    // a few rows: sixteen waves, a segment each up to 4096 values (the launch is one dependent chain of latencies);
+    // many rows: four, so that several rows share a CU
+    uint32_t grid[3] = {m, 1, 1}, block[3] = {dev->rms_threads ? dev->rms_threads : (m <= 64 ? 1024u : 256u), 1, 1};
     return ojh_launch(dev, "rmsnorm_q8k", {at(x, x_off), gamma->ptr, q->ptr, scales->ptr, xn ? xn->ptr : q->ptr},
                       {k, m, eps_bits, (uint32_t)(xn != nullptr)}, grid, block);
 }

@@ -85,6 +85,7 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_PX_BPC")) d->px_bpc = (uint32_t)std::max(0, atoi(r));
     if (const char *r = getenv("OJAS_HIP_PX")) d->px = atoi(r);
     if (const char *r = getenv("OJAS_HIP_Q4K_XT_MIN_M")) d->q4k_xt_min_m = (uint32_t)atoi(r);
+    if (const char *r = getenv("OJAS_HIP_RMS_THREADS")) d->rms_threads = atoi(r) == 1024 ? 1024u : atoi(r) == 256 ? 256u : 0u;
     if (const char *r = getenv("OJAS_HIP_Q4K_XT_SPLIT")) d->q4k_xt_split = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_Q4K_XT64")) d->q4k_xt64 = atoi(r) != 0;
     if (const char *r = getenv("OJAS_HIP_Q4K_MF_MIN_M")) d->q4k_mf_min_m = (uint32_t)atoi(r);
