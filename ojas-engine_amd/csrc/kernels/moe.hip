@@ -220,10 +220,34 @@ __device__ __forceinline__ void moe_group_body(const uint* __restrict__ idx, uin
         if (e < E) atomicAdd(&cnt[e], 1u);
     }
     __syncthreads();
-    if (tid == 0) {
-        uint run = 0;
-        for (uint e = 0; e < E; e++) { off[e] = run; run += cnt[e]; }
-        off[E] = run;
+    {
+        // exclusive prefix sums of the counts: a thread takes four consecutive experts (E <= 1024), the threads' totals
+        // are scanned across the wave by shuffles and across the four waves through off[1024] .. (free until the end)
+        const uint lane = tid & 63u, wv = tid >> 6;
+        uint c[4], local = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            c[i] = 4u * tid + (uint)i < E ? cnt[4u * tid + (uint)i] : 0u;
+            local += c[i];
+        }
+        uint incl = local;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint up = (uint)__shfl_up((int)incl, d);
+            if (lane >= (uint)d) incl += up;
+        }
+        __shared__ uint wtot[4];
+        if (lane == 63u) wtot[wv] = incl;
+        __syncthreads();
+        uint base = 0;
+        for (uint w = 0; w < wv; w++) base += wtot[w];
+        uint run = base + incl - local;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (4u * tid + (uint)i < E) off[4u * tid + (uint)i] = run;
+            run += c[i];
+        }
+        if (tid == 255u) off[E] = run;      // thread 255 ends at the grand total
     }
     __syncthreads();
     for (uint e = tid; e <= E; e += 256u) {
@@ -1176,7 +1200,19 @@ moe_combine(const float* __restrict__ dv, const float* __restrict__ wgt, float* 
     if (i >= (size_t)T * D) return;
     const uint t = (uint)(i / D), col = (uint)(i % D);
     float acc = ACC ? y[i] : 0.0f;
-    for (uint j = 0; j < KSEL; j++) acc += wgt[(size_t)t * KSEL + j] * dv[((size_t)t * KSEL + j) * D + col];
+    // (eight slots' loads in flight before the first is added — slot order kept; past the last slot they repeat it)
+    for (uint j0 = 0; j0 < KSEL; j0 += 8u) {
+        float w[8], d[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const size_t a = (size_t)t * KSEL + min(j0 + (uint)u, KSEL - 1u);
+            w[u] = wgt[a];
+            d[u] = dv[a * D + col];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (j0 + (uint)u < KSEL) acc += w[u] * d[u];
+    }
     y[i] = acc;
 }
 
