@@ -301,12 +301,10 @@ moe_gu_q4k_m(const signed char* __restrict__ xq, const float* __restrict__ xs, c
             Q4kFrag f = q4k_load_frag(xq + (size_t)t * nsb * 256u, xs + (size_t)t * nsb, on ? g : 0u, l);
             float vg0 = on ? q4k_lane_dot(hg0, qg0, c, f) : 0.0f, vg1 = on ? q4k_lane_dot(hg1, qg1, c, f) : 0.0f;
             float vu0 = on ? q4k_lane_dot(hu0, qu0, c, f) : 0.0f, vu1 = on ? q4k_lane_dot(hu1, qu1, c, f) : 0.0f;
-            vg0 = wave_sum(vg0); vg1 = wave_sum(vg1); vu0 = wave_sum(vu0); vu1 = wave_sum(vu1);
-            if (lane == 0) {
-                float* o_ = act + (size_t)a * N + row0;
-                o_[0] = (vg0 / (1.0f + expf(-vg0))) * vu0;
-                if (two) o_[1] = (vg1 / (1.0f + expf(-vg1))) * vu1;
-            }
+            // the four sums in one pass: lanes 0 / 1 end with the gate sums of the two rows, lanes 2 / 3 with the up sums
+            const float tot = wave_sum4(vg0, vg1, vu0, vu1, lane);
+            const float upv = dpp_f32<OJK_DPP_QUAD_XOR2>(tot);
+            if (lane < (two ? 2u : 1u)) act[(size_t)a * N + row0 + lane] = (tot / (1.0f + expf(-tot))) * upv;
         }
     } else {
         for (uint i = a0; i < a1; i++) {
@@ -320,12 +318,9 @@ moe_gu_q4k_m(const signed char* __restrict__ xq, const float* __restrict__ xs, c
                 vu0 += q4k_lane_dot(*(const uint4*)(u0 + o), *(const uint4*)(u0 + o + 16u + l * 16u), c, f);
                 vu1 += q4k_lane_dot(*(const uint4*)(u0 + r1 + o), *(const uint4*)(u0 + r1 + o + 16u + l * 16u), c, f);
             }
-            vg0 = wave_sum(vg0); vg1 = wave_sum(vg1); vu0 = wave_sum(vu0); vu1 = wave_sum(vu1);
-            if (lane == 0) {
-                float* o_ = act + (size_t)a * N + row0;
-                o_[0] = (vg0 / (1.0f + expf(-vg0))) * vu0;
-                if (two) o_[1] = (vg1 / (1.0f + expf(-vg1))) * vu1;
-            }
+            const float tot = wave_sum4(vg0, vg1, vu0, vu1, lane);
+            const float upv = dpp_f32<OJK_DPP_QUAD_XOR2>(tot);
+            if (lane < (two ? 2u : 1u)) act[(size_t)a * N + row0 + lane] = (tot / (1.0f + expf(-tot))) * upv;
         }
     }
 }
@@ -358,15 +353,12 @@ __device__ __forceinline__ void moe_down_m_body(const signed char* __restrict__ 
         for (uint i = a0; i < a1; i++) {
             const uint a = min(list[i], NA - 1u);
             Q4kFrag f = q4k_load_frag(aq + (size_t)a * nsb * 256u, as_ + (size_t)a * nsb, on ? G : 0u, l);
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const float v = row16_sum(on ? wr[r].dot(c, f) : 0.0f);
-                const float s0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)) +
-                                 __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
-                const float s1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32)) +
-                                 __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
-                if ((lane & 31u) == 0 && rowh + r < N) dv[(size_t)a * N + rowh + r] = hf ? s1 : s0;
-            }
+            // the half's four rows in one pass: lane j of each row of 16 gets row j's 16-lane sum, the half's two
+            // such sums are added as wave_sum adds them
+            float v = row16_sum4(on ? wr[0].dot(c, f) : 0.0f, on ? wr[1].dot(c, f) : 0.0f, on ? wr[2].dot(c, f) : 0.0f,
+                                 on ? wr[3].dot(c, f) : 0.0f, lane);
+            v += __shfl_xor(v, 16);
+            if ((lane & 31u) < 4u && rowh + (lane & 3u) < N) dv[(size_t)a * N + rowh + (lane & 3u)] = v;
         }
         return;
     }
@@ -382,11 +374,9 @@ __device__ __forceinline__ void moe_down_m_body(const signed char* __restrict__ 
         for (uint i = a0; i < a1; i++) {
             const uint a = min(list[i], NA - 1u);
             Q4kFrag f = q4k_load_frag(aq + (size_t)a * nsb * 256u, as_ + (size_t)a * nsb, on ? g : 0u, l);
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                float v = wave_sum(on ? wr[r].dot(c, f) : 0.0f);
-                if (lane == 0 && row0 + r < N) dv[(size_t)a * N + row0 + r] = v;
-            }
+            const float v = wave_sum4(on ? wr[0].dot(c, f) : 0.0f, on ? wr[1].dot(c, f) : 0.0f, on ? wr[2].dot(c, f) : 0.0f,
+                                      on ? wr[3].dot(c, f) : 0.0f, lane);
+            if (lane < 4u && row0 + lane < N) dv[(size_t)a * N + row0 + lane] = v;
         }
     } else {
         for (uint i = a0; i < a1; i++) {

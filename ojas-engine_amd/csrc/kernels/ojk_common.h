@@ -59,6 +59,8 @@ __device__ __forceinline__ ushort f32_to_bf16_bits(float f) {
 #define OJK_DPP_QUAD_XOR2 0x4E   // quad_perm:[2,3,0,1]
 #define OJK_DPP_ROW_HALF_MIRROR 0x141
 #define OJK_DPP_ROW_MIRROR 0x140
+#define OJK_DPP_ROW_SHL4 0x104          // lane i reads lane i + 4 of its row of 16 (zero past the row)
+#define OJK_DPP_ROW_SHL8 0x108
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
@@ -102,6 +104,27 @@ __device__ __forceinline__ float wave_sum(float v) {
     float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
     float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
     return (a + b) + (c + d);
+}
+// Four sums at once, with the additions of row16_sum / wave_sum in their order (so: their bits) but a third of the
+// instructions: after each of the first two steps a lane keeps only the value its position names — value (lane & 3) —
+// and hands the other to the neighbour that keeps it; the steps across quads read the same position of the next quad.
+// row16_sum4: lane j (j < 4) of every row of 16 ends with that row's total of value j; the other lanes hold partial sums.
+// wave_sum4: lanes 0 .. 3 end with the wave's totals of values 0 .. 3.
+__device__ __forceinline__ float row16_sum4(float v0, float v1, float v2, float v3, uint lane) {
+    v0 = rounded(v0); v1 = rounded(v1); v2 = rounded(v2); v3 = rounded(v3);
+    const bool odd = (lane & 1u) != 0u, up = (lane & 2u) != 0u;
+    const float a = (odd ? v1 : v0) + dpp_f32<OJK_DPP_QUAD_XOR1>(odd ? v0 : v1);
+    const float b = (odd ? v3 : v2) + dpp_f32<OJK_DPP_QUAD_XOR1>(odd ? v2 : v3);
+    float c = (up ? b : a) + dpp_f32<OJK_DPP_QUAD_XOR2>(up ? a : b);
+    c += dpp_f32<OJK_DPP_ROW_SHL4>(c);
+    c += dpp_f32<OJK_DPP_ROW_SHL8>(c);
+    return c;
+}
+__device__ __forceinline__ float wave_sum4(float v0, float v1, float v2, float v3, uint lane) {
+    float c = row16_sum4(v0, v1, v2, v3, lane);
+    c += __shfl_xor(c, 16);
+    c += __shfl_xor(c, 32);
+    return c;
 }
 // The same in f64 (the two halves of a double travel as two 32-bit DPP moves): lanes 1, 2 apart, mirrored in eights and
 // sixteens, then the four rows as (r0 + r1) + (r2 + r3).  One fixed order: whoever sums a segment's 64 lane values with
