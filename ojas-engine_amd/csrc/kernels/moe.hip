@@ -299,8 +299,11 @@ moe_gu_q4k_m(const signed char* __restrict__ xq, const float* __restrict__ xs, c
         for (uint i = a0; i < a1; i++) {
             const uint a = min(list[i], NA - 1u), t = a / KSEL;
             Q4kFrag f = q4k_load_frag(xq + (size_t)t * nsb * 256u, xs + (size_t)t * nsb, on ? g : 0u, l);
-            float vg0 = on ? q4k_lane_dot(hg0, qg0, c, f) : 0.0f, vg1 = on ? q4k_lane_dot(hg1, qg1, c, f) : 0.0f;
-            float vu0 = on ? q4k_lane_dot(hu0, qu0, c, f) : 0.0f, vu1 = on ? q4k_lane_dot(hu1, qu1, c, f) : 0.0f;
+            // (lanes past the row's last super-block multiply by a zero scale: a product of zero, and no branch around
+            // each of the four dots)
+            f.sx = on ? f.sx : 0.0f;
+            float vg0 = q4k_lane_dot(hg0, qg0, c, f), vg1 = q4k_lane_dot(hg1, qg1, c, f);
+            float vu0 = q4k_lane_dot(hu0, qu0, c, f), vu1 = q4k_lane_dot(hu1, qu1, c, f);
             // the four sums in one pass: lanes 0 / 1 end with the gate sums of the two rows, lanes 2 / 3 with the up sums
             const float tot = wave_sum4(vg0, vg1, vu0, vu1, lane);
             const float upv = dpp_f32<OJK_DPP_QUAD_XOR2>(tot);
@@ -353,10 +356,10 @@ __device__ __forceinline__ void moe_down_m_body(const signed char* __restrict__ 
         for (uint i = a0; i < a1; i++) {
             const uint a = min(list[i], NA - 1u);
             Q4kFrag f = q4k_load_frag(aq + (size_t)a * nsb * 256u, as_ + (size_t)a * nsb, on ? G : 0u, l);
+            f.sx = on ? f.sx : 0.0f;        // lanes without a super-block of the row: products of zero, no branches
             // the half's four rows in one pass: lane j of each row of 16 gets row j's 16-lane sum, the half's two
             // such sums are added as wave_sum adds them
-            float v = row16_sum4(on ? wr[0].dot(c, f) : 0.0f, on ? wr[1].dot(c, f) : 0.0f, on ? wr[2].dot(c, f) : 0.0f,
-                                 on ? wr[3].dot(c, f) : 0.0f, lane);
+            float v = row16_sum4(wr[0].dot(c, f), wr[1].dot(c, f), wr[2].dot(c, f), wr[3].dot(c, f), lane);
             v += __shfl_xor(v, 16);
             if ((lane & 31u) < 4u && rowh + (lane & 3u) < N) dv[(size_t)a * N + rowh + (lane & 3u)] = v;
         }
@@ -374,8 +377,8 @@ __device__ __forceinline__ void moe_down_m_body(const signed char* __restrict__ 
         for (uint i = a0; i < a1; i++) {
             const uint a = min(list[i], NA - 1u);
             Q4kFrag f = q4k_load_frag(aq + (size_t)a * nsb * 256u, as_ + (size_t)a * nsb, on ? g : 0u, l);
-            const float v = wave_sum4(on ? wr[0].dot(c, f) : 0.0f, on ? wr[1].dot(c, f) : 0.0f, on ? wr[2].dot(c, f) : 0.0f,
-                                      on ? wr[3].dot(c, f) : 0.0f, lane);
+            f.sx = on ? f.sx : 0.0f;
+            const float v = wave_sum4(wr[0].dot(c, f), wr[1].dot(c, f), wr[2].dot(c, f), wr[3].dot(c, f), lane);
             if (lane < 4u && row0 + lane < N) dv[(size_t)a * N + row0 + lane] = v;
         }
     } else {
