@@ -185,6 +185,15 @@ __device__ __forceinline__ int dot4_i8(uint a, uint b, int acc) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, acc, false);
 }
 
+// The first product of a chain: the three-operand encoding with a literal zero as the addend.  (Left to itself the
+// compiler picks the two-operand form, which accumulates in place and so needs a register cleared first: one more
+// vector instruction per chain.)
+__device__ __forceinline__ int dot4_i8_first(uint a, uint b) {
+    int r;
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
 // ---- Q4_K scale / min unpack ---------------------------------------------------------------
 // The 12 scale bytes of a Q4_K / Q5_K super-block as three dwords (s0 = bytes 0..3, s1 = 4..7,
 // s2 = 8..11).  Returns, for the sub-block pair (2c, 2c+1), the two 6-bit scales in bytes 0/1 of

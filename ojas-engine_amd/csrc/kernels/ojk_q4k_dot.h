@@ -5,7 +5,7 @@
 #include "ojk_common.h"
 
 __device__ __forceinline__ int bytesum4(uint4 v) {
-    int s = dot4_i8(v.x, 0x01010101u, 0);
+    int s = dot4_i8_first(v.x, 0x01010101u);
     s = dot4_i8(v.y, 0x01010101u, s);
     s = dot4_i8(v.z, 0x01010101u, s);
     return dot4_i8(v.w, 0x01010101u, s);
@@ -72,11 +72,11 @@ __device__ __forceinline__ Q4kFrag q4k_quant_frag(const float* x, uint sb, uint 
 // One lane's 32 weights of one super-block against one activation fragment.
 __device__ __forceinline__ float q4k_lane_dot(uint4 hdr, uint4 qs, uint c, const Q4kFrag& f) {
     const uint M4 = 0x0F0F0F0Fu;
-    int il = dot4_i8(qs.x & M4, f.xl.x, 0);
+    int il = dot4_i8_first(qs.x & M4, f.xl.x);
     il = dot4_i8(qs.y & M4, f.xl.y, il);
     il = dot4_i8(qs.z & M4, f.xl.z, il);
     il = dot4_i8(qs.w & M4, f.xl.w, il);
-    int ih = dot4_i8((qs.x >> 4) & M4, f.xh.x, 0);
+    int ih = dot4_i8_first((qs.x >> 4) & M4, f.xh.x);
     ih = dot4_i8((qs.y >> 4) & M4, f.xh.y, ih);
     ih = dot4_i8((qs.z >> 4) & M4, f.xh.z, ih);
     ih = dot4_i8((qs.w >> 4) & M4, f.xh.w, ih);
