@@ -109,6 +109,16 @@ __device__ __forceinline__ void gemv_q8k_q4k_body(const signed char* __restrict_
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] += q4k_lane_dot(hdr[r], qs[r], c, f);
     }
+    if (R == 2 && MODE == ST_SET) {         // the wave's two sums in one pass (wave_sum's additions, in its order)
+        const float t = wave_sum2(acc[0], acc[R - 1], lane);
+        if (lane < 2u && row0 + lane < N) y[row0 + lane] = t;
+        return;
+    }
+    if (R == 4 && MODE == ST_SET) {
+        const float t = wave_sum4(acc[0], acc[1 % R], acc[2 % R], acc[3 % R], lane);
+        if (lane < 4u && row0 + lane < N) y[row0 + lane] = t;
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < R; r++) {
         float t = wave_sum(acc[r]);

@@ -120,6 +120,18 @@ __device__ __forceinline__ float row16_sum4(float v0, float v1, float v2, float 
     c += dpp_f32<OJK_DPP_ROW_SHL8>(c);
     return c;
 }
+// ... and two: lanes 0 / 1 end with the wave's totals of v0 / v1
+__device__ __forceinline__ float wave_sum2(float v0, float v1, uint lane) {
+    v0 = rounded(v0); v1 = rounded(v1);
+    const bool odd = (lane & 1u) != 0u;
+    float c = (odd ? v1 : v0) + dpp_f32<OJK_DPP_QUAD_XOR1>(odd ? v0 : v1);
+    c += dpp_f32<OJK_DPP_QUAD_XOR2>(c);
+    c += dpp_f32<OJK_DPP_ROW_SHL4>(c);
+    c += dpp_f32<OJK_DPP_ROW_SHL8>(c);
+    c += __shfl_xor(c, 16);
+    c += __shfl_xor(c, 32);
+    return c;
+}
 __device__ __forceinline__ float wave_sum4(float v0, float v1, float v2, float v3, uint lane) {
     float c = row16_sum4(v0, v1, v2, v3, lane);
     c += __shfl_xor(c, 16);
