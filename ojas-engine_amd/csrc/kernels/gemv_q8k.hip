@@ -280,6 +280,11 @@ __device__ __forceinline__ void gemv_q8k_q4k_x4_body(const signed char* __restri
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] += q4k_lane_dot(hdr[r], qs[r], c, f);
     }
+    if (R == 2) {       // both sums in one pass
+        const float t = wave_sum2(acc[0], acc[R - 1], lane);
+        if (lane < 2u && row0 + lane < E3) *(lane ? rw[R - 1].y : rw[0].y) = t;
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < R; r++) {
         float t = wave_sum(acc[r]);
@@ -333,10 +338,10 @@ ffn_gu_q8k_q4k(const signed char* __restrict__ xq, const float* __restrict__ xs,
             au[r] += q4k_lane_dot(hu[r], qu[r], c, f);
         }
     }
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        const float sg = wave_sum(ag[r]), su = wave_sum(au[r]);
-        if (lane == 0 && row0 + r < N) out[row0 + r] = ffn_act(sg, ACT) * su;
+    {   // the gate and the up sum in one pass: lane 0 ends with the gate sum, lane 1 with the up sum
+        const float t = wave_sum2(ag[0], au[0], lane);
+        const float su = dpp_f32<OJK_DPP_QUAD_XOR1>(t);
+        if (lane == 0 && row0 < N) out[row0] = ffn_act(t, ACT) * su;
     }
 }
 
@@ -640,8 +645,12 @@ __device__ __forceinline__ void gemv_fq8k_q4k_x4_body(const float* __restrict__ 
         if (last) {
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                float t = wave_sum(acc[r]);
-                if (lane == 0 && row0 + r < row_end) *rwc[r].y = ACC ? add[r] + t : t;
+                float t = R == 2 ? 0.0f : wave_sum(acc[r]);
+                if (R == 2 && r == 0) {     // both sums in one pass; lane r holds row r's
+                    const float t2 = wave_sum2(acc[0], acc[R - 1], lane);
+                    if (lane < 2u && row0 + lane < row_end) *(lane ? rwc[R - 1].y : rwc[0].y) = ACC ? (lane ? add[R - 1] : add[0]) + t2 : t2;
+                }
+                if (R != 2 && lane == 0 && row0 + r < row_end) *rwc[r].y = ACC ? add[r] + t : t;
                 acc[r] = 0.0f;
                 add[r] = (ACC && nrow < row_end) ? *rwn[r].y : 0.0f;
             }
