@@ -70,15 +70,15 @@ __device__ __forceinline__ void moe_topk_lanes(const float* __restrict__ lg, uin
             if (p[i] > bv) { bv = p[i]; bi = lane + 64u * i; }
         }
         float m2 = wave_max(bv);
-        // lowest index among the lanes holding the maximum
-        uint cand = (bv == m2) ? bi : 0xFFFFFFFFu;
-        cand = min(cand, (uint)dpp_i32<OJK_DPP_QUAD_XOR1>((int)cand));
-        cand = min(cand, (uint)dpp_i32<OJK_DPP_QUAD_XOR2>((int)cand));
-        cand = min(cand, (uint)dpp_i32<OJK_DPP_ROW_HALF_MIRROR>((int)cand));
-        cand = min(cand, (uint)dpp_i32<OJK_DPP_ROW_MIRROR>((int)cand));
-        uint c0 = (uint)__builtin_amdgcn_readlane((int)cand, 0), c1 = (uint)__builtin_amdgcn_readlane((int)cand, 16);
-        uint c2 = (uint)__builtin_amdgcn_readlane((int)cand, 32), c3 = (uint)__builtin_amdgcn_readlane((int)cand, 48);
-        uint win = min(min(c0, c1), min(c2, c3));
+        // lowest index among the lanes holding the maximum: an expert's index is lane + 64 i, so the lowest i with any
+        // such lane decides, and within it the lowest lane — one vote per i and scalar bit scans instead of a second
+        // reduction across the wave
+        uint win = 0xFFFFFFFFu;
+#pragma unroll
+        for (int i = NI - 1; i >= 0; i--) {
+            const unsigned long long vote = __ballot(bv == m2 && bi == lane + 64u * (uint)i);
+            if (vote) win = (uint)__builtin_ctzll(vote) + 64u * (uint)i;
+        }
         wsum += m2;
         if (lane == j) { mine = m2; mine_idx = win; }
 #pragma unroll
