@@ -96,19 +96,19 @@ __device__ __forceinline__ float q4k_lane_dot(uint4 hdr, uint4 qs, uint c, const
 __device__ __forceinline__ float q5k_lane_dot(uint4 hdr, uint4 qs, uint4 qh, uint c, const Q4kFrag& f) {
     const uint M4 = 0x0F0F0F0Fu, B1 = 0x01010101u;
     const uint sl = 2u * c, sh = 2u * c + 1u;
-    int il = dot4_i8(qs.x & M4, f.xl.x, 0);
+    int il = dot4_i8_first(qs.x & M4, f.xl.x);
     il = dot4_i8(qs.y & M4, f.xl.y, il);
     il = dot4_i8(qs.z & M4, f.xl.z, il);
     il = dot4_i8(qs.w & M4, f.xl.w, il);
-    int bl = dot4_i8((qh.x >> sl) & B1, f.xl.x, 0);
+    int bl = dot4_i8_first((qh.x >> sl) & B1, f.xl.x);
     bl = dot4_i8((qh.y >> sl) & B1, f.xl.y, bl);
     bl = dot4_i8((qh.z >> sl) & B1, f.xl.z, bl);
     bl = dot4_i8((qh.w >> sl) & B1, f.xl.w, bl);
-    int ih = dot4_i8((qs.x >> 4) & M4, f.xh.x, 0);
+    int ih = dot4_i8_first((qs.x >> 4) & M4, f.xh.x);
     ih = dot4_i8((qs.y >> 4) & M4, f.xh.y, ih);
     ih = dot4_i8((qs.z >> 4) & M4, f.xh.z, ih);
     ih = dot4_i8((qs.w >> 4) & M4, f.xh.w, ih);
-    int bh = dot4_i8((qh.x >> sh) & B1, f.xh.x, 0);
+    int bh = dot4_i8_first((qh.x >> sh) & B1, f.xh.x);
     bh = dot4_i8((qh.y >> sh) & B1, f.xh.y, bh);
     bh = dot4_i8((qh.z >> sh) & B1, f.xh.z, bh);
     bh = dot4_i8((qh.w >> sh) & B1, f.xh.w, bh);
@@ -166,11 +166,11 @@ struct W6k {
         const uint nsh = 4u * (c & 1u);            // nibble of ql; also the bit pair of qh for the first run
         // codes 0..63 as bytes: ql nibble | two bits of qh moved to bits 4-5
         #define OJK_Q6_CODE(QL, QH, SH) ((((QL) >> nsh) & M4) | ((((QH) >> (SH)) << 4) & H2))
-        int ia = dot4_i8(OJK_Q6_CODE(qa.x, qh.x, nsh), f.xl.x, 0);
+        int ia = dot4_i8_first(OJK_Q6_CODE(qa.x, qh.x, nsh), f.xl.x);
         ia = dot4_i8(OJK_Q6_CODE(qa.y, qh.y, nsh), f.xl.y, ia);
         ia = dot4_i8(OJK_Q6_CODE(qa.z, qh.z, nsh), f.xl.z, ia);
         ia = dot4_i8(OJK_Q6_CODE(qa.w, qh.w, nsh), f.xl.w, ia);
-        int ib = dot4_i8(OJK_Q6_CODE(qb.x, qh.x, nsh + 2u), f.xh.x, 0);
+        int ib = dot4_i8_first(OJK_Q6_CODE(qb.x, qh.x, nsh + 2u), f.xh.x);
         ib = dot4_i8(OJK_Q6_CODE(qb.y, qh.y, nsh + 2u), f.xh.y, ib);
         ib = dot4_i8(OJK_Q6_CODE(qb.z, qh.z, nsh + 2u), f.xh.z, ib);
         ib = dot4_i8(OJK_Q6_CODE(qb.w, qh.w, nsh + 2u), f.xh.w, ib);
