@@ -61,7 +61,7 @@ struct ojh_device {
     uint32_t gemm_min_m = 32;    // OJAS_HIP_GEMM_MIN_M: rows from which ojh_mm takes the MFMA tile
     int gemm_split_override = 0; // OJAS_HIP_GEMM_SPLIT
     int q80_lds = 1;             // OJAS_HIP_Q80_LDS: 0 = never take the LDS-staged Q8_0 matvec
-    uint32_t q80_lds_min_n = 16384; // OJAS_HIP_Q80_LDS_MIN_N: rows from which it is taken (measured crossover)
+    uint32_t q80_lds_min_n = 8192;  // OJAS_HIP_Q80_LDS_MIN_N: rows from which it is taken (weights from HBM, K = 4096: 14336 rows 15.3 against 17.8 us, 4096 rows 7.9 against 7.0)
     uint32_t q80_lds_bpc = 0;       // OJAS_HIP_Q80_LDS_BPC: workgroups per CU its grid is sized for (0: 2 or 3 by K chunking)
     uint32_t q6k_mf_min_m = 5;   // OJAS_HIP_Q6K_MF_MIN_M: tokens from which Q6_K rows (fewer than 32768) go to the int8 matrix cores
     uint32_t q6k_ml_min_m = 2;   // OJAS_HIP_Q6K_ML_MIN_M: ... with the rows copied through LDS (32768 rows or more)
