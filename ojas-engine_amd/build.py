@@ -25,16 +25,17 @@ DEVICE_FLAGS = ["-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-
                 "-Wno-unused-command-line-argument"]
 
 # family -> (source, extra flags).  The decoder family and the GEMM's in-tile decoder must round
-# every operation separately (no fused multiply-add).
+# every operation separately (no fused multiply-add).  OJK_ASM_FIRST_DOT: the three-operand first dot of a chain
+# (ojk_common.h), where it was measured to pay.
 FAMILIES = {
     "dequant": ("dequant.hip", ["-ffp-contract=off"]),
     "gemv": ("gemv.hip", []),
-    "gemv_q8k": ("gemv_q8k.hip", []),
+    "gemv_q8k": ("gemv_q8k.hip", ["-DOJK_ASM_FIRST_DOT"]),
     "glue": ("glue.hip", []),
     "gemm": ("gemm.hip", ["-ffp-contract=off"]),
     "gemm_xl": ("gemm_xl.hip", ["-ffp-contract=off"]),
     "gemm_q8k": ("gemm_q8k.hip", []),
-    "moe": ("moe.hip", []),
+    "moe": ("moe.hip", ["-DOJK_ASM_FIRST_DOT"]),
     "moe_iq": ("moe_iq.hip", []),
     "rowq8": ("rowq8.hip", ["-ffp-contract=off"]),
     "q80_dp4a": ("q80_dp4a.hip", []),

@@ -197,13 +197,19 @@ __device__ __forceinline__ int dot4_i8(uint a, uint b, int acc) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, acc, false);
 }
 
-// The first product of a chain: the three-operand encoding with a literal zero as the addend.  (Left to itself the
-// compiler picks the two-operand form, which accumulates in place and so needs a register cleared first: one more
-// vector instruction per chain.)
+// The first product of a chain.  Built with OJK_ASM_FIRST_DOT it is the three-operand encoding with a literal zero as
+// the addend: left to itself the compiler picks the two-operand form, which accumulates in place and so needs a register
+// cleared first — one more vector instruction per chain.  A family asks for it where that was measured to pay (the
+// matvecs and the grouped expert dots, which issue instructions most of their time); in the single-launch chain the
+// same change made the row workgroups a fifth slower, so the default is the builtin.
 __device__ __forceinline__ int dot4_i8_first(uint a, uint b) {
+#ifdef OJK_ASM_FIRST_DOT
     int r;
     asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(b));
     return r;
+#else
+    return __builtin_amdgcn_sdot4((int)a, (int)b, 0, false);
+#endif
 }
 
 // ---- Q4_K scale / min unpack ---------------------------------------------------------------
