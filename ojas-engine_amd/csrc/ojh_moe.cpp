@@ -183,12 +183,11 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     uint32_t *counts = (uint32_t *)grp->ptr, *offsets = counts + E, *list = offsets + E + 1;
 
     // Expert products: on the matrix cores once experts see a few tokens each (measured crossover on
-    // MI355X: ~4 assignments per expert for the workgroup-per-tile form, ~3 where the wave-per-tile form
-    // fits), on integer dots below that, where the launch is a pure stream of weight rows.  The two
+    // MI355X, 128 experts of 2048 x 768: 4 assignments per expert — 48 tokens of top-8 take 105 us on dots and 115 on
+    // the matrix cores, 64 tokens 120 and 116), on integer dots below that.  The two
     // forms round their f32 sums in different orders (last ulp).
-    const bool mt_fits = dev->moe_mode != 4 && ojh_moe_mt_lds(d) <= 81920;
     const bool mm = dev->moe_mode == 1 || dev->moe_mode == 4 ||
-                    (dev->moe_mode == 0 && (uint64_t)NA >= (uint64_t)(mt_fits ? 3 : 4) * E);
+                    (dev->moe_mode == 0 && (uint64_t)NA >= (uint64_t)4 * E);
     // ... a wave per row tile where 16 tokens of K fit the workgroup's LDS (OJAS_HIP_MOE=4 keeps the workgroup-per-tile form)
     const bool mt_gu = mm && dev->moe_mode != 4 && ojh_moe_mt_lds(d) <= 81920;
     const bool mt_down = mm && dev->moe_mode != 4 && !down5 && ojh_moe_mt_lds(n_ff) <= 81920;
