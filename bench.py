@@ -533,7 +533,7 @@ def extras(gpu, pkg, lin_q) -> dict:
         fl = 2.0 * T * ksel * 3 * nff * d
         moe[f"T{T}"] = {"us": round(us, 1), "distinct_experts": distinct, "gbs": round(b / us / 1e3, 1),
                         "tflops": round(fl / us / 1e6, 2)}
-    out["moe_ffn_q4k_128x_top8"] = {"timed": "router + expert FFN, ojh_moe_ffn_routed (T <= 8: gate/up, the router inside it, and down launches addressed by assignment; above: router, quantize + group in one launch, gate/up, quantize, down, combine; T = 256 on int8 MFMA, moe_{gu,down}_q4k_mt, 32 assignments per staged pass)", **moe}
+    out["moe_ffn_q4k_128x_top8"] = {"timed": "router + expert FFN, ojh_moe_ffn_routed (T <= 2: gate/up, the router inside it, and down launches addressed by assignment; above: router, quantize + group in one launch, gate/up, quantize, down, combine; T = 256 on int8 MFMA, moe_{gu,down}_q4k_mt, 32 assignments per staged pass)", **moe}
     del gate, up, down
     # ---- speculative verify on a Q6_K output head 151936 x 4096, bf16 activations
     n, k = 151936, 4096

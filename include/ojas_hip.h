@@ -371,7 +371,7 @@ int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uin
  * reference's GPU expert kernels for those formats, crates/ojas-core/src/quant_src.rs:174-179);
  * OJH_ACT_AUTO and OJH_ACT_Q8K keep the CPU path's int8-activation arithmetic for them.
  * Expert indices must be below n_expert (one that is not never reads outside the tensors; what
- * it contributes is unspecified). Up to 8 tokens run as two launches addressed
+ * it contributes is unspecified). Up to 2 tokens run as two launches addressed
  * by assignment (bit-identical to the grouped integer-dot pipeline) when d <= 8192, n_ff <= 2048,
  * ksel <= 64 and ksel * n_ff <= 32768 (beyond that the grouped pipeline serves them; forcing the
  * two-launch form with OJAS_HIP_MOE=3 then returns OJH_ERR_UNSUPPORTED); larger batches are grouped
@@ -384,7 +384,7 @@ int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t n_tokens, uint32_t d
                 int accum, int act_mode);
 
 /* Router and expert FFN in one call: logits [n_tokens][n_expert] f32 -> idx, wgt [n_tokens][ksel] (written: softmax,
- * top ksel, renormalised — ojh_moe_route's arithmetic, the same bits) -> y as ojh_moe_ffn.  For up to 8 tokens over
+ * top ksel, renormalised — ojh_moe_route's arithmetic, the same bits) -> y as ojh_moe_ffn.  For up to 2 tokens over
  * Q4_K gate / up experts (the decode form of ojh_moe_ffn and its limits) the router runs inside the gate/up launch:
  * two launches per layer and token instead of three; every other case is ojh_moe_route followed by ojh_moe_ffn.
  * The op-level seam of the reference takes router logits or (idx, wgt) alike (ojas-cuda moe.rs:45-125 run back to

@@ -77,7 +77,7 @@ struct ojh_device {
     uint32_t q4k_mf_min_m = 5;   // OJAS_HIP_Q4K_MF_MIN_M: tokens from which Q4_K rows go to the int8 matrix cores
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
                                  // 3 = per-assignment decode form always, 4 = matrix cores in the workgroup-per-tile form always
-    uint32_t moe_dec_tokens = 8; // OJAS_HIP_MOE_DEC_TOKENS: the decode form serves up to this many tokens
+    uint32_t moe_dec_tokens = 2; // OJAS_HIP_MOE_DEC_TOKENS: the decode form serves up to this many tokens (128 experts, top 8, weights from HBM: 2 tokens 21.0 against 23.3 us grouped, 3 tokens 27.4 against 25.9, 8 tokens 59 against 38)
     int gemm_bdk = 1;            // OJAS_HIP_GEMM_BDK: 0 never takes the 64-row tile whose waves split K, 2 takes it wherever the 128-token tile would run
     bool gemm_sr = false;        // OJAS_HIP_GEMM_SR=1: K slices of the prefill tile meet in scratch, added in slice order (reproducible bits), instead of in f32 atomics
     bool moe_route_fuse = true;  // OJAS_HIP_MOE_ROUTE_FUSE=0: ojh_moe_ffn_routed keeps the router a launch of its own
