@@ -423,7 +423,7 @@ def extras(gpu, pkg, lin_q) -> dict:
     i8 = {}
     for name, lin in zip(("gate_up_14336x4096", "down_4096x14336"), lin_q):
         n, k = lin.n, lin.k
-        for m in (8, 16, 128, 512, 2048):
+        for m in (8, 16, 64, 128, 512, 2048):
             xf = gpu.upload(synth.normal_f32(m * k, "bench", "i8_x", m, k))
             y = gpu.alloc(m * n)
             us = _time(gpu, lambda i: gpu.mm(xf, lin, y, m, act_mode=pkg.ACT_Q8K), 20, 5)
@@ -433,7 +433,7 @@ def extras(gpu, pkg, lin_q) -> dict:
     out["verify_prefill_q4k_int8"] = {"arithmetic": "quant_q8k activations, int8 x u4 dots on the int8 matrix cores, the CPU "
                                                     "reference's scale algebra (results within 2e-5 of matvec_kq)",
                                       "peak_tops": 5000.0,
-                                      "timed": "quantizer + the tile: from 96 tokens quantize_q8k_sides + gemm_q8k_q4k_xt{,64} "
+                                      "timed": "quantizer + the tile: from 33 tokens (17 where K >= 2 N: down) quantize_q8k_sides + gemm_q8k_q4k_xt{,64} "
                                                "(128-token tiles, scales folded into int8 planes, v_mfma_i32_16x16x64_i8; where the "
                                                "64-row tiles alone leave CUs idle or singly occupied — down up to M = 512 — gemm_q8k_q4k_xt64_sr: K slices "
                                                "summed in slice order by the last to finish); below, "

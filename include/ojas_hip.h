@@ -216,7 +216,7 @@ int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, const o
  * The int8 activations and their per-256 scales are staged in a static device array of
  * `ojh_noalloc_scratch_bytes()` bytes (1 MiB of activations + their scales) that each GPU holds
  * until the process ends, so the call allocates and frees nothing; the launches and results are
- * those of `ojh_mm(..., OJH_ACT_Q8K)` bit for bit below 96 tokens; from there `ojh_mm` may take a
+ * those of `ojh_mm(..., OJH_ACT_Q8K)` bit for bit below 17 tokens; from there `ojh_mm` may take a
  * prefill tile that stages more in library scratch, which this entry never does (it stays on the
  * few-token kernels: the same integer sums, f32 terms in the same order).  K-quant weights (Q4_K, Q5_K, Q6_K), f32 or bf16
  * activations, m * K <= OJH_NOALLOC_MAX_ACT (OJH_ERR_BOUNDS beyond); the families "gemv_q8k" and

@@ -71,7 +71,7 @@ struct ojh_device {
     uint32_t q4k_ml_min_m = 2;   // OJAS_HIP_Q4K_ML_MIN_M: tokens from which long Q4_K matrices (32768 rows or more) take the LDS-copy form (0: never)
     uint32_t rms_threads = 0;    // OJAS_HIP_RMS_THREADS: block size of rmsnorm_q8k (256 or 1024; 0: by the number of rows)
     uint32_t q4k_xt_split = 1;   // OJAS_HIP_Q4K_XT_SPLIT: K slices of the 64-row int8 tile when its tiles leave CUs idle (0: never, 1: chosen, n: n)
-    uint32_t q4k_xt_min_m = 96;  // OJAS_HIP_Q4K_XT_MIN_M: tokens from which Q4_K rows take the 128 x 128 int8 tile (0: never)
+    uint32_t q4k_xt_min_m = 1;   // OJAS_HIP_Q4K_XT_MIN_M: tokens from which Q4_K rows take the 128-token int8 tile (0: never, 1: by shape)
     bool q4k_xt64 = false;       // OJAS_HIP_Q4K_XT64=1: that tile always in its 64-row form
     bool no_scratch = false;     // set around calls that may not allocate (ojh_mm_noalloc): paths that need library scratch are skipped
     uint32_t q4k_mf_min_m = 5;   // OJAS_HIP_Q4K_MF_MIN_M: tokens from which Q4_K rows go to the int8 matrix cores

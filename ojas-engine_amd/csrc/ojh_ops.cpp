@@ -170,9 +170,20 @@ static uint32_t q4k_xt_slices(const ojh_device *dev, uint32_t K, uint32_t N, uin
     if (z < 2 || tiles * z * 2 < cus) return whole;
     return ojh_gemm_sr_slices(K, z);
 }
+// Tokens from which that tile is taken (measured with the rows streamed from HBM, K = 2048 .. 14336): the tile costs
+// the same from 1 to 128 tokens, the matrix-core kernel below it doubles past 32 tokens.  So from 33 tokens; from 17
+// where K is at least twice the row count (few tiles, each a long walk: 4096 x 14336 takes 38 us here against 45);
+// and only from 65 for a matrix of more than one and a half 64-row tiles per CU, where two 32-token passes of the
+// other kernel are still ahead (32000 x 4096 at 64 tokens: 56 us against 62).
+static uint32_t q4k_xt_min_tokens(const ojh_device *dev, uint32_t K, uint32_t N) {
+    if (dev->q4k_xt_min_m != 1) return dev->q4k_xt_min_m;
+    const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;
+    if (2 * (uint64_t)((N + 63) / 64) > 3ull * cus) return 65;
+    return K >= 2ull * N ? 17 : 33;
+}
 bool ojh_q4k_xt_taken(const ojh_device *dev, const ojh_lin *w, uint32_t m, const void *wp) {
     const uint32_t K = w->k, N = w->n;
-    return w->type == OJH_Q4_K && dev->q4k_xt_min_m && m >= dev->q4k_xt_min_m && !dev->no_scratch &&
+    return w->type == OJH_Q4_K && dev->q4k_xt_min_m && m >= q4k_xt_min_tokens(dev, K, N) && !dev->no_scratch &&
            q4k_xt_slices(dev, K, N, m) >= 1 &&
            (uint64_t)m * K <= 0xFFFFFFFFull && (uint64_t)w->row_bytes * N <= 0xFFFFFFFFull && (uintptr_t)wp % 16 == 0;
 }

@@ -21,7 +21,9 @@ def _case(pkg, m, n, k, tag):
 @pytest.mark.parametrize("m,n,k,accum", [(2, 50, 256, False), (16, 130, 4096, True), (17, 333, 2560, False),
                                          (40, 64, 14336, True), (128, 100, 1024, False), (129, 300, 512, False),
                                          (300, 40, 4096, True), (8, 4099, 4096, False), (64, 17, 8192, False),
-                                         (130, 6200, 512, True)])
+                                         (130, 6200, 512, True),
+                                         # the 128-token tile in K slices below 128 tokens: from 17 tokens where K >= 2 N, from 33 otherwise
+                                         (20, 1030, 4096, True), (33, 2100, 2048, False), (64, 4096, 4096, False)])
 def test_router_path_matches_the_cpu_reference(gpu, orc, pkg, m, n, k, accum):
     w, x = _case(pkg, m, n, k, "a")
     lin = gpu.lin(Q4_K, n, k, w)
