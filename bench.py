@@ -438,6 +438,23 @@ def extras(gpu, pkg, lin_q) -> dict:
                                                "64-row tiles alone leave CUs idle or singly occupied — down up to M = 512 — gemm_q8k_q4k_xt64_sr: K slices "
                                                "summed in slice order by the last to finish); below, "
                                                "gemm_q8k_q4k_mf (down at M = 8: gemm_q8k_q4k_mk)", **i8}
+    # ---- the same arithmetic over Q6_K and Q5_K rows (a Q4_K_M / Q5_K_M file mixes them in), f32 in
+    for ty, tag, gen in ((pkg.Q6_K, "q6k", synth.q6k_weights), (pkg.Q5_K, "q5k", synth.q5k_weights)):
+        fam = {}
+        for name, (n, k) in (("gate_up_14336x4096", (14336, 4096)), ("down_4096x14336", (4096, 14336))):
+            lin = gpu.lin(ty, n, k, gen(n, k, "bench", tag, name))
+            for m in (64, 128, 512):
+                xf = gpu.upload(synth.normal_f32(m * k, "bench", "i8_x", m, k))
+                y = gpu.alloc(m * n)
+                us = _time(gpu, lambda i: gpu.mm(xf, lin, y, m, act_mode=pkg.ACT_Q8K), 20, 5)
+                fam[f"{name}_M{m}"] = {"us": round(us, 1), "tops": round(2.0 * m * n * k / us / 1e6, 1),
+                                       "int8_mfma_frac": round(2.0 * m * n * k / us / 1e6 / 5000.0, 4)}
+                del xf, y
+            lin.free()
+        out[f"verify_prefill_{tag}_int8"] = {"arithmetic": "quant_q8k activations, integer dots per scale group on the int8 matrix cores "
+                                                           f"(v_mfma_i32_32x32x16_i8 per 16 weights of Q6_K, 32x32x32 per 32 of Q5_K), the scale "
+                                                           "a 24-bit multiply-add per result: dot_q6k / dot_q5k within 2e-5 of peak",
+                                             "peak_tops": 5000.0, "timed": f"quantize_q8k + gemm_q8k_{tag}_gs{{,_sr}}", **fam}
     # ---- speculative verify on the Q4_K output head of the decode step, bf16 activations
     head4 = lin_q[2]
     v4 = {}

@@ -812,3 +812,364 @@ gemm_q8k_q4k_xt64_sr(const signed char* xq, const float* xst, const float* sums,
     __shared__ __attribute__((aligned(1024))) uchar lds_xt[2 * GXT_STAGE];
     gemm_q8k_q4k_xt_body<2, true>(xq, xst, sums, w, y, K, N, M, ACC, MP, lds_xt, part, cnt, NSPLIT);
 }
+
+// ---- Q6_K and Q5_K rows against 128 tokens: one matrix instruction per scale group ---------------------------------
+//   gemm_q8k_{q6k,q5k}_gs(xq, xs, w, y, K, N, M, ACC)                      block 256, grid [ceil(N / 64), ceil(M / 128), 1]
+//   gemm_q8k_{q6k,q5k}_gs_sr(xq, xs, w, y, part, cnt, K, N, M, ACC, NSPLIT)       grid [.., .., slices]
+// The CPU path's arithmetic (dot_q6k / dot_q5k over quant_q8k activations, crates/ojas-cpu/src/cpu_math.rs:638-722) for
+// prefill-sized batches.  A Q6_K scale covers 16 weights and is a full int8, so it cannot be folded into int8 codes the
+// way the Q4_K tile above folds its 6-bit scales; instead v_mfma_i32_32x32x16_i8, whose 16 positions are exactly one
+// scale group, gives the group's integer dots for 32 tokens x 32 rows, and the scale enters with one v_mad_i32_i24 per
+// D register (the row is lane-constant in D).  Q5_K: two instructions per 32-weight sub-block (codes 0..31 are one
+// int8 plane), the 6-bit scale likewise, and sum_j m_j bsum_j from two more instructions per super-block over the
+// sub-block sums split as 64 hi + lo (the workgroup splits them while it stages the tokens).
+// A workgroup owns 64 rows x 128 tokens: wave (r, t) = (wave % 2, wave / 2) takes rows 32 r .. and tokens 64 t ..
+// as two blocks of 32.  B (weights): lane (n, kg) = (lane % 32, lane / 32) builds the codes of positions 8 kg .. 8 kg + 7
+// of every group of row n from the raw bytes it loads itself, one super-block ahead.  A (tokens): a super-block's 128 x 256
+// int8 wait in LDS, rows 264 bytes apart (32 tokens' 8-byte reads then cover all banks), two stages, one barrier per
+// super-block.  Integer sums are exact; per super-block acc += sx * d * (float) isum, super-blocks in order.
+// `_sr`: K slices whose partial tiles meet in `part` (tiles x slices x 32 KB), added in slice order by the last to arrive.
+#include "ojk_q6k_mfma.h"
+
+typedef int gs_i16 __attribute__((ext_vector_type(16)));
+#define GS_STRIDE 264u
+#define GS_SX (128u * GS_STRIDE)        // the stage's 128 token scales
+#define GS_BS (GS_SX + 512u)            // Q5_K: the split sub-block sums, 16 bytes per token (lo_0..7, hi_0..7)
+#define GS_STAGE (GS_BS + 2048u)
+
+// A running integer sum, pinned after every group: integer additions may be reassociated, and left to itself the
+// compiler turns sixteen groups' multiply-adds into one tree at the end of the super-block, every group's sixteen result
+// registers alive until then (hundreds of spills).
+__device__ __forceinline__ int gs_pin(int v) {
+    asm("" : "+v"(v));
+    return v;
+}
+
+struct GsQ6K {
+    static constexpr uint BYTES = Q6K_BYTES;
+    static constexpr bool BSUMS = false;
+    struct Raw {
+        u32x2_a2 la[2][2], lb[2][2], qh[2][2];   // [half][group of the quarter]: ql[16 h + 8 kg ..], ql[32 + ..], qh[..]
+        u32x4_a2 sc;
+        uint d16;
+    };
+    static __device__ __forceinline__ Raw load(const uchar* blk, uint kg) {
+        Raw r;
+        const uint sh = ((uint)(size_t)blk & 2u) << 3;
+        const uchar* b4 = blk - ((size_t)blk & 2u);
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                r.la[hf][h] = q6k_ld8(b4 + 64u * hf + 16u * h + 8u * kg, sh);
+                r.lb[hf][h] = q6k_ld8(b4 + 64u * hf + 32u + 16u * h + 8u * kg, sh);
+                r.qh[hf][h] = q6k_ld8(b4 + 128u + 32u * hf + 16u * h + 8u * kg, sh);
+            }
+        const uint* ps = (const uint*)(b4 + 192u);
+        const uint s0 = ps[0], s1 = ps[1], s2 = ps[2], s3 = ps[3], s4 = ps[4];
+        r.sc.x = __builtin_amdgcn_alignbit(s1, s0, sh);
+        r.sc.y = __builtin_amdgcn_alignbit(s2, s1, sh);
+        r.sc.z = __builtin_amdgcn_alignbit(s3, s2, sh);
+        r.sc.w = __builtin_amdgcn_alignbit(s4, s3, sh);
+        r.d16 = (s4 >> sh) & 0xFFFFu;
+        return r;
+    }
+    // st: the stage; tok0: the wave's first token in it
+    static __device__ __forceinline__ void superblock(const Raw& r, const uchar* st, uint tok0, uint fr, uint kg,
+                                                      float (&acc)[2][16]) {
+        const uchar* xa = st + (tok0 + fr) * GS_STRIDE + 8u * kg;            // the lane's token row of block 0, its 8 positions
+        const float* sx = (const float*)(st + GS_SX) + tok0 + 4u * kg;       // scales of its D registers' tokens: + 32 i + 8 (v / 4) + v % 4
+        int isum[2][16];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) isum[i][v] = 0;
+        const gs_i16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        // group g = 8 hf + 2 q + h: quarter q of half hf, its positions 16 h .. 16 h + 15; scale byte g
+        auto codes = [&](int g) -> long {
+            const int hf = g >> 3, q = (g >> 1) & 3, h = g & 1;
+            const u32x2_a2 ql = (q & 1) ? r.lb[hf][h] : r.la[hf][h];
+            return q6k_signed8(ql.x, ql.y, r.qh[hf][h].x, r.qh[hf][h].y, q);
+        };
+        auto tokens = [&](int g, int i) -> long {
+            return *(const long*)(xa + (uint)i * 32u * GS_STRIDE + 16u * (uint)g);
+        };
+        // the next group's operands are fetched and built under this group's matrix instructions, ahead of its multiply-adds
+        long B = codes(0), A0 = tokens(0, 0), A1 = tokens(0, 1);
+#pragma unroll
+        for (int g = 0; g < 16; g++) {
+            const uint sw = g < 4 ? r.sc.x : g < 8 ? r.sc.y : g < 12 ? r.sc.z : r.sc.w;
+            const int s = (int)(signed char)(sw >> (8 * (g & 3)));
+            const gs_i16 D0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(A0, B, zero, 0, 0, 0);
+            const gs_i16 D1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(A1, B, zero, 0, 0, 0);
+            if (g < 15) {
+                A0 = tokens(g + 1, 0);
+                A1 = tokens(g + 1, 1);
+                B = codes(g + 1);
+            }
+#pragma unroll
+            for (int v = 0; v < 16; v++) isum[0][v] = gs_pin(isum[0][v] + __mul24(s, D0[v]));
+#pragma unroll
+            for (int v = 0; v < 16; v++) isum[1][v] = gs_pin(isum[1][v] + __mul24(s, D1[v]));
+            // (keeps the groups apart: let loose, the scheduler issues every group's matrix instructions first and
+            // spills their results)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const float d = f16_bits_to_f32(r.d16);
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const float4 x4 = *(const float4*)(sx + 32 * i + 8 * g);
+                acc[i][4 * g] += x4.x * d * (float)isum[i][4 * g];
+                acc[i][4 * g + 1] += x4.y * d * (float)isum[i][4 * g + 1];
+                acc[i][4 * g + 2] += x4.z * d * (float)isum[i][4 * g + 2];
+                acc[i][4 * g + 3] += x4.w * d * (float)isum[i][4 * g + 3];
+            }
+    }
+};
+
+struct GsQ5K {
+    static constexpr uint BYTES = Q5K_BYTES;
+    static constexpr bool BSUMS = true;
+    struct Raw {
+        uint4 hdr;          // d, dmin, the 12 scale bytes
+        uint2 qh[2];        // fifth bits of positions 16 h + 8 kg .. + 7 (bit j: sub-block j)
+        uint2 qs[4][2];     // [chunk][h]: nibbles of the same positions (low: sub-block 2 c, high: 2 c + 1)
+    };
+    static __device__ __forceinline__ Raw load(const uchar* blk, uint kg) {
+        Raw r;
+        r.hdr = *(const uint4*)blk;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            r.qh[h] = *(const uint2*)(blk + 16u + 16u * h + 8u * kg);
+#pragma unroll
+            for (int c = 0; c < 4; c++) r.qs[c][h] = *(const uint2*)(blk + 48u + 32u * c + 16u * h + 8u * kg);
+        }
+        return r;
+    }
+    static __device__ __forceinline__ void superblock(const Raw& r, const uchar* st, uint tok0, uint fr, uint kg,
+                                                      float (&acc)[2][16]) {
+        const uchar* xa = st + (tok0 + fr) * GS_STRIDE + 8u * kg;            // the lane's token row of block 0, its 8 positions
+        const float* sx = (const float*)(st + GS_SX) + tok0 + 4u * kg;       // scales of its D registers' tokens: + 32 i + 8 (v / 4) + v % 4
+        int isum[2][16];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) isum[i][v] = 0;
+        const gs_i16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        // the eight 6-bit scales and mins, a byte each (get_scale_min_k4, crates/ojas-formats/src/gguf.rs:1132-1140)
+        const uint sc_lo = r.hdr.y & 0x3F3F3F3Fu, mn_lo = r.hdr.z & 0x3F3F3F3Fu;
+        const uint sc_hi = (r.hdr.w & 0x0F0F0F0Fu) | ((r.hdr.y >> 2) & 0x30303030u);
+        const uint mn_hi = ((r.hdr.w >> 4) & 0x0F0F0F0Fu) | ((r.hdr.z >> 2) & 0x30303030u);
+        // sub-block j, half h: the codes of positions 16 h + 8 kg .. of chunk j / 2 (low or high nibbles) under fifth bit j
+        auto codes = [&](int j, int h) -> long {
+            const uint2 p = r.qs[j >> 1][h];
+            const uint n0 = (j & 1) ? (p.x >> 4) & 0x0F0F0F0Fu : p.x & 0x0F0F0F0Fu;
+            const uint n1 = (j & 1) ? (p.y >> 4) & 0x0F0F0F0Fu : p.y & 0x0F0F0F0Fu;
+            const uint b0 = j < 4 ? (r.qh[h].x << (4 - j)) & 0x10101010u : (r.qh[h].x >> (j - 4)) & 0x10101010u;
+            const uint b1 = j < 4 ? (r.qh[h].y << (4 - j)) & 0x10101010u : (r.qh[h].y >> (j - 4)) & 0x10101010u;
+            return gq_pack(n0 | b0, n1 | b1);
+        };
+        auto tokens = [&](int j, int h, int i) -> long {
+            return *(const long*)(xa + (uint)i * 32u * GS_STRIDE + 32u * (uint)j + 16u * (uint)h);
+        };
+        // the next sub-block's operands are fetched and built under this one's matrix instructions
+        long B[2] = {codes(0, 0), codes(0, 1)};
+        long A[2][2] = {{tokens(0, 0, 0), tokens(0, 0, 1)}, {tokens(0, 1, 0), tokens(0, 1, 1)}};
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int s = (int)(((j < 4 ? sc_lo : sc_hi) >> (8 * (j & 3))) & 0xFFu);
+            // (one instruction over all 32 positions of the sub-block: a lane's sixteen are 8 kg .. and 16 + 8 kg ..)
+            gs_i16 D[2];
+            const gq_i4 Bj = {(int)B[0], (int)(B[0] >> 32), (int)B[1], (int)(B[1] >> 32)};
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const gq_i4 Aj = {(int)A[0][i], (int)(A[0][i] >> 32), (int)A[1][i], (int)(A[1][i] >> 32)};
+                D[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(Aj, Bj, zero, 0, 0, 0);
+            }
+            if (j < 7) {
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    B[h] = codes(j + 1, h);
+                    A[h][0] = tokens(j + 1, h, 0);
+                    A[h][1] = tokens(j + 1, h, 1);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) isum[i][v] = gs_pin(isum[i][v] + __mul24(s, D[i][v]));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // sum_j m_j bsum_j, bsum = 64 hi + lo: positions 0..7 of A carry the lo parts, 8..15 the hi parts, B the mins twice:
+        // D1 = sum m lo + sum m hi; with the lo half of A blanked D2 = sum m hi; the term is D1 + 63 D2
+        const long Bm = gq_pack(mn_lo, mn_hi);
+        const long km = kg ? -1l : 0l;
+        const float d = f16_bits_to_f32(r.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(r.hdr.x >> 16);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const long A1 = *(const long*)(st + GS_BS + (tok0 + 32u * (uint)i + fr) * 16u + 8u * kg);
+            const gs_i16 D1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(A1, Bm, zero, 0, 0, 0);
+            const gs_i16 D2 = __builtin_amdgcn_mfma_i32_32x32x16_i8(A1 & km, Bm, zero, 0, 0, 0);
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const float4 x4 = *(const float4*)(sx + 32 * i + 8 * g);
+                const float xv[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int v = 4 * g + e;
+                    acc[i][v] += xv[e] * (d * (float)isum[i][v] - dmin * (float)(D1[v] + 63 * D2[v]));
+                }
+            }
+        }
+    }
+};
+
+template <class F, bool SPLIT>
+__device__ __forceinline__ void gemm_q8k_gs_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
+                                                 const uchar* __restrict__ w, float* __restrict__ y, uint K, uint N, uint M,
+                                                 uint ACC, uchar* lds, float* part = nullptr, uint* cnt = nullptr,
+                                                 uint nsplit = 1u) {
+    const uint tid = threadIdx.x, lane = tid & 63u;
+    const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint nsb = K >> 8;
+    const uint per = SPLIT ? (nsb + nsplit - 1u) / nsplit : nsb;
+    const uint sb0 = SPLIT ? blockIdx.z * per : 0u, sb1 = SPLIT ? min(nsb, sb0 + per) : nsb;
+    if (SPLIT && sb0 >= sb1) return;                      // (the host launches only slices that hold a super-block)
+    const uint m0 = blockIdx.y * 128u, fr = lane & 31u, kg = lane >> 5;
+    const uint row = min(blockIdx.x * 64u + 32u * (wave & 1u) + fr, N - 1u);
+    const uint tok0 = 64u * (wave >> 1);
+    const uchar* wr = w + (size_t)row * nsb * F::BYTES;
+
+    // staging: thread -> chunk tid % 16 (16 bytes) of tokens tid / 16 + 16 p, p = 0..7
+    const uint s_tok = tid >> 4, s_ch = tid & 15u;
+    uint4 tv[8];
+    float tsx = 0.0f;
+    auto fetch = [&](uint sb) {
+#pragma unroll
+        for (int p = 0; p < 8; p++) {
+            const uint m = m0 + s_tok + 16u * (uint)p;
+            tv[p] = make_uint4(0u, 0u, 0u, 0u);
+            if (m < M) tv[p] = *(const uint4*)(xq + (size_t)m * K + (size_t)sb * 256u + s_ch * 16u);
+        }
+        if (tid < 128u) tsx = m0 + tid < M ? xs[(size_t)(m0 + tid) * nsb + sb] : 0.0f;
+    };
+    auto put = [&](uchar* st) {
+#pragma unroll
+        for (int p = 0; p < 8; p++) {
+            uchar* o = st + (s_tok + 16u * (uint)p) * GS_STRIDE + s_ch * 16u;
+            *(uint2*)o = make_uint2(tv[p].x, tv[p].y);
+            *(uint2*)(o + 8) = make_uint2(tv[p].z, tv[p].w);
+            if (F::BSUMS) {
+                // half a sub-block per thread; its neighbour holds the other half
+                int s = dot4_i8(tv[p].x, 0x01010101u, 0);
+                s = dot4_i8(tv[p].y, 0x01010101u, s);
+                s = dot4_i8(tv[p].z, 0x01010101u, s);
+                s = dot4_i8(tv[p].w, 0x01010101u, s);
+                s += dpp_i32<OJK_DPP_QUAD_XOR1>(s);
+                if (!(s_ch & 1u)) {
+                    uchar* b = st + GS_BS + (s_tok + 16u * (uint)p) * 16u + (s_ch >> 1);
+                    b[0] = (uchar)(s & 63);
+                    b[8] = (uchar)(s >> 6);
+                }
+            }
+        }
+        if (tid < 128u) ((float*)(st + GS_SX))[tid] = tsx;
+    };
+
+    float acc[2][16];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[i][v] = 0.0f;
+
+    fetch(sb0);
+    typename F::Raw nx = F::load(wr + (size_t)sb0 * F::BYTES, kg);
+    put(lds);
+    __syncthreads();
+    for (uint sb = sb0; sb < sb1; sb++) {
+        const typename F::Raw cur = nx;
+        const uint nb = min(sb + 1u, sb1 - 1u);
+        nx = F::load(wr + (size_t)nb * F::BYTES, kg);
+        fetch(nb);
+        const uchar* st = lds + ((sb - sb0) & 1u) * GS_STAGE;
+        F::superblock(cur, st, tok0, fr, kg, acc);
+        put(lds + (((sb - sb0) & 1u) ^ 1u) * GS_STAGE);
+        __syncthreads();
+    }
+
+    if (SPLIT) {
+        // partial tiles out as the registers hold them ([pair][thread]), written through and read from behind the L2
+        // (a tile's slices run on different XCDs); the stores are awaited by instruction before the slice is counted
+        typedef unsigned long long u64;
+        const uint ns_eff = (nsb + per - 1u) / per;
+        const uint tile = blockIdx.y * gridDim.x + blockIdx.x;
+        u64* const mine = (u64*)part + ((size_t)tile * ns_eff + blockIdx.z) * 16u * 256u + tid;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int h = 0; h < 8; h++)
+                __hip_atomic_store(mine + (size_t)(i * 8 + h) * 256u,
+                                   (u64)__float_as_uint(acc[i][2 * h]) | ((u64)__float_as_uint(acc[i][2 * h + 1]) << 32),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (tid == 0u) *(volatile uint*)lds = atomicAdd(cnt + tile, 1u);
+        __syncthreads();
+        if ((uint)__builtin_amdgcn_readfirstlane((int)*(volatile uint*)lds) != ns_eff - 1u) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        const u64* const all = (const u64*)part + (size_t)tile * ns_eff * 16u * 256u + tid;
+        for (uint s0 = 0; s0 < ns_eff; s0 += 2u) {
+            u64 v[2][16];
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const uint sl = min(s0 + (uint)q, ns_eff - 1u);
+#pragma unroll
+                for (int i = 0; i < 16; i++)
+                    v[q][i] = __hip_atomic_load(all + ((size_t)sl * 16u + (uint)i) * 256u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                if (s0 + (uint)q < ns_eff) {
+                    const bool first = s0 + (uint)q == 0u;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const float a = __uint_as_float((uint)v[q][i]), b = __uint_as_float((uint)(v[q][i] >> 32));
+                        acc[i / 8][2 * (i % 8)] = first ? a : acc[i / 8][2 * (i % 8)] + a;
+                        acc[i / 8][2 * (i % 8) + 1] = first ? b : acc[i / 8][2 * (i % 8) + 1] + b;
+                    }
+                }
+            }
+        }
+        if (tid == 0u) cnt[tile] = 0u;                               // ready for the next launch
+    }
+    // D register v of block i: token 32 i + 8 (v / 4) + 4 kg + v % 4, row fr
+    const uint n = blockIdx.x * 64u + 32u * (wave & 1u) + fr;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const uint t = m0 + tok0 + 32u * (uint)i + 8u * (uint)(v >> 2) + 4u * kg + (uint)(v & 3);
+            if (t < M && n < N) {
+                float* o = y + (size_t)t * N + n;
+                *o = ACC ? *o + acc[i][v] : acc[i][v];
+            }
+        }
+}
+
+#define GEMM_Q8K_GS(FMT, F)                                                                                              \
+    extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))                         \
+    gemm_q8k_##FMT##_gs(const signed char* xq, const float* xs, const uchar* w, float* y, uint K, uint N, uint M, uint ACC) { \
+        __shared__ __attribute__((aligned(16))) uchar lds_gs[2 * GS_STAGE];                                              \
+        gemm_q8k_gs_body<F, false>(xq, xs, w, y, K, N, M, ACC, lds_gs);                                                  \
+    }                                                                                                                    \
+    extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))                         \
+    gemm_q8k_##FMT##_gs_sr(const signed char* xq, const float* xs, const uchar* w, float* y, float* part, uint* cnt,     \
+                           uint K, uint N, uint M, uint ACC, uint NSPLIT) {                                              \
+        __shared__ __attribute__((aligned(16))) uchar lds_gs[2 * GS_STAGE];                                              \
+        gemm_q8k_gs_body<F, true>(xq, xs, w, y, K, N, M, ACC, lds_gs, part, cnt, NSPLIT);                                \
+    }
+GEMM_Q8K_GS(q6k, GsQ6K)
+GEMM_Q8K_GS(q5k, GsQ5K)

@@ -291,6 +291,67 @@ static int shape_gemm_q8k_xt_sr(const ojh_kernel_spec *, const ojh_device *dev, 
     block[1] = block[2] = 1;
     return OJH_OK;
 }
+// gemm_q8k_{q6k,q5k}_gs(xq, xs, w, y, K, N, M, ACC): grid [ceil(N / 64), ceil(M / 128), 1] x 256
+// gemm_q8k_{q6k,q5k}_gs_sr(xq, xs, w, y, part, cnt, K, N, M, ACC, NSPLIT): grid [.., .., slices]; part: 32 KB per tile
+// and slice; cnt: a zeroed word per tile (`rows_per_wave` = 1 marks the sliced entry)
+static int check_gemm_q8k_gs(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                             const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const bool sr = s->rows_per_wave == 1;
+    const ojh_block_format *f;
+    const uint32_t K = c[0], N = c[1], M = c[2], nsplit = sr ? c[4] : 1;
+    int rc = check_kn(s, K, N, &f);
+    if (rc) return rc;
+    if (K % 256) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a multiple of 256", s->name, K);
+    if (!M || M > 65535) return ojh_fail(OJH_ERR_ARG, "%s: M=%u out of range", s->name, M);
+    if (c[3] > 1) return ojh_fail(OJH_ERR_ARG, "%s: ACC=%u", s->name, c[3]);
+    if ((rc = check_block(block, 256))) return rc;
+    const size_t nsb = K / 256;
+    if (!nsplit || nsplit > nsb) return ojh_fail(OJH_ERR_ARG, "%s: NSPLIT=%u (1 .. K/256)", s->name, nsplit);
+    const uint32_t slices = sr ? ojh_gemm_sr_slices(K, nsplit) : 1;
+    if (grid[0] != (N + 63) / 64 || grid[1] != (M + 127) / 128 || grid[2] != slices)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, (N + 63) / 64, (M + 127) / 128, slices);
+    need[0] = (size_t)M * K;
+    need[1] = (size_t)M * nsb * 4;
+    need[2] = (size_t)N * nsb * f->bytes;
+    need[3] = (size_t)M * N * 4;
+    align[0] = 16;
+    align[1] = align[3] = 4;
+    align[2] = s->type == OJH_Q5_K ? 16 : 2;
+    if (sr) {
+        const size_t tiles = (size_t)grid[0] * grid[1];
+        need[4] = tiles * slices * 32768;
+        need[5] = tiles * 4;
+        align[4] = 8;
+        align[5] = 4;
+    }
+    return OJH_OK;
+}
+// K slices of that tile: two workgroups per CU is the aim (a wave alone on its SIMD waits for every matrix result and
+// LDS read itself), at most eight slices of at least two super-blocks — eight, where the tiles already cover more than
+// half the CUs.  OJAS_HIP_KQ_GS_SPLIT: 0 never, n > 1 that many.
+uint32_t ojh_gemm_q8k_gs_slices(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M) {
+    const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, nsb = K / 256;
+    const uint32_t mode = dev ? dev->kq_gs_split : 1u;
+    const uint64_t tiles = (uint64_t)((N + 63) / 64) * ((M + 127) / 128);
+    if (!tiles || mode == 0) return 1;
+    uint32_t z = (uint32_t)(2 * (uint64_t)cus / tiles);
+    if (z > 8) z = 8;
+    const uint32_t cap = tiles * 2 > cus ? nsb / 8 : nsb / 2;
+    if (z > cap) z = cap;
+    if (mode > 1) z = mode <= nsb ? mode : nsb;
+    return z < 2 ? 1 : ojh_gemm_sr_slices(K, z);
+}
+static int shape_gemm_q8k_gs(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
+                             uint32_t grid[3], uint32_t block[3]) {
+    if (!M) M = 1;
+    grid[0] = (N + 63) / 64;
+    if (!grid[0]) grid[0] = 1;
+    grid[1] = (M + 127) / 128;
+    grid[2] = s->rows_per_wave == 1 ? ojh_gemm_q8k_gs_slices(dev, K, N, M) : 1;
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
 // quantize_q8k{,_bf16}_sides(x, q, scales, xst, sums, K, M, MP): grid [K / 256 * MP / 4, 1, 1]
 static int check_quantize_sides(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                                 const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -1608,6 +1669,10 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("gemm_q8k_q4k_xt", "gemm_q8k", 5, 5, OJH_Q4_K, 1, check_gemm_q8k_xt, shape_gemm_q8k_xt);
     add("gemm_q8k_q4k_xt64", "gemm_q8k", 5, 5, OJH_Q4_K, 2, check_gemm_q8k_xt, shape_gemm_q8k_xt);
     add("gemm_q8k_q4k_xt64_sr", "gemm_q8k", 7, 6, OJH_Q4_K, 2, check_gemm_q8k_xt_sr, shape_gemm_q8k_xt_sr);
+    add("gemm_q8k_q6k_gs", "gemm_q8k", 4, 4, OJH_Q6_K, 0, check_gemm_q8k_gs, shape_gemm_q8k_gs);
+    add("gemm_q8k_q6k_gs_sr", "gemm_q8k", 6, 5, OJH_Q6_K, 1, check_gemm_q8k_gs, shape_gemm_q8k_gs);
+    add("gemm_q8k_q5k_gs", "gemm_q8k", 4, 4, OJH_Q5_K, 0, check_gemm_q8k_gs, shape_gemm_q8k_gs);
+    add("gemm_q8k_q5k_gs_sr", "gemm_q8k", 6, 5, OJH_Q5_K, 1, check_gemm_q8k_gs, shape_gemm_q8k_gs);
     add("gemm_q8k_q4k_mk", "gemm_q8k", 4, 4, OJH_Q4_K, 2, check_gemm_q8k_ml, shape_mk);
     add("relayout_q4k_q4l", "dequant", 4, 1, OJH_Q4_K, 0, check_relayout, shape_relayout);
     add("embed_q80", "dequant", 2, 2, OJH_Q8_0, 0, check_embed, shape_embed);

@@ -278,6 +278,32 @@ int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, con
     }
     const size_t w_bytes = w->row_bytes * N;
     const bool dwords_ok = (uintptr_t)wp % 4 == 0 && (w_bytes % 4 == 0 || w->off + w_bytes + 2 <= w->raw->bytes);
+    // Q6_K / Q5_K rows against a prefill-sized batch: 64-row x 128-token tiles, one matrix instruction per scale group;
+    // over K slices where the tiles alone would leave CUs idle (partial tiles in library scratch, added in slice order)
+    // (from where it was measured ahead of launches of 16 tokens, rows streamed from HBM: Q6_K from 33 tokens — 14336 x 4096
+    // at 48 tokens 51 against 60 us, at 128 54 against 152 — and from 17 where K is long, 4096 x 14336: 48 against 49 .. 67;
+    // Q5_K, whose few-token form is the integer-dot kernel, from 17 everywhere and from 9 on large matrices)
+    const uint32_t gs_min = dev->kq_gs_min_m != 1 ? dev->kq_gs_min_m
+                            : w->type == OJH_Q6_K ? (K > 8192 ? 17u : 33u)
+                                                  : (N >= 8192 || K > 8192 ? 9u : 17u);
+    if ((w->type == OJH_Q6_K || w->type == OJH_Q5_K) && gs_min && m >= gs_min && K % 256 == 0 &&
+        (uintptr_t)xq % 16 == 0 && (w->type == OJH_Q6_K ? dwords_ok : (uintptr_t)wp % 16 == 0)) {
+        int rc = ensure(dev, "gemm_q8k");
+        if (rc) return rc;
+        const std::string gs = std::string("gemm_q8k_") + f->tag + "_gs";
+        uint32_t sg[3] = {(N + 63) / 64, (m + 127) / 128, 1}, sb[3] = {256, 1, 1};
+        const uint32_t z = dev->no_scratch ? 1 : ojh_gemm_q8k_gs_slices(dev, K, N, m);
+        if (z > 1) {
+            const size_t tiles = (size_t)sg[0] * sg[1];
+            ojh_buf *part, *cnt;
+            if ((rc = ojh_scratch_get(dev, "gs_part", tiles * z * 32768, &part))) return rc;
+            if ((rc = ojh_scratch_get_zeroed(dev, "gs_cnt", tiles * 4, &cnt))) return rc;
+            sg[2] = z;
+            return ojh_launch(dev, (gs + "_sr").c_str(), {xq, xs, wp, yp, part->ptr, cnt->ptr},
+                              {K, N, m, (uint32_t)(accum != 0), z}, sg, sb);
+        }
+        return ojh_launch(dev, gs.c_str(), {xq, xs, wp, yp}, {K, N, m, (uint32_t)(accum != 0)}, sg, sb);
+    }
     // Q6_K rows against 2 or more tokens on the int8 matrix cores (beyond 16 tokens as launches of 16 or 8:
     // each streams the rows once, which the per-token loop of the general entry does sixteen times
     // over).  Three shapes of the same tile arithmetic, picked by what was measured on K = 4096 and 14336:
