@@ -488,6 +488,19 @@ def extras(gpu, pkg, lin_q) -> dict:
     b = n * (k // 32) * 34 + 4 * k + 4 * n
     out["q80_gemv_128256x4096"] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
     del wq8
+    # ---- row-int8 weights (K int8 + one f32 scale per row), f32 activations: the reference GPU decoder's `gemv_q8` by name
+    gpu.ensure_family("gemv_q8")
+    rq = {}
+    rng8 = np.random.default_rng(synth.seed_of("bench", "gemv_q8"))
+    for name, (n, copies, reps) in (("4096x4096", (4096, 20, 64)), ("128256x4096", (128256, 2, 20))):
+        ws = [gpu.upload_bytes(rng8.integers(-127, 128, n * k, dtype=np.int8).view(np.uint8)) for _ in range(copies)]
+        sc, y = gpu.upload(np.full(n, 0.01, np.float32)), gpu.alloc(n)
+        g, blk = gpu.launch_shape("gemv_q8", k, n)
+        us = _time(gpu, lambda i: gpu.dispatch(None, "gemv_q8", [(x, 0), (ws[i % copies], 0), (y, 0), (sc, 0)], [k, n], g, blk), reps, 5)
+        b = n * k + 4 * k + 8 * n
+        rq[name] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
+        del ws
+    out["rowq8_gemv_q8"] = {"what": "y[n] = scale[n] * sum_k w[n][k] x[k], w int8 rows streamed from HBM (rotating copies)", **rq}
     # ---- the other block formats on f32 activations (the reference GPU path's contract): a tall head, one token
     fr = {}
     for ty, tag in ((pkg.IQ4_XS, "iq4xs"), (pkg.IQ4_NL, "iq4nl"), (pkg.Q3_K, "q3k"), (pkg.Q2_K, "q2k"), (pkg.Q5_0, "q50"),

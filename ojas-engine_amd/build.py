@@ -41,6 +41,7 @@ FAMILIES = {
     "q80_dp4a": ("q80_dp4a.hip", []),
     "iq_grid": ("iq_grid.hip", ["-ffp-contract=off"]),
     "chain": ("chain.hip", []),
+    "gemv_q8": ("gemv_q8.hip", ["-ffp-contract=off"]),
 }
 
 HOST_SOURCES = ["ojh_runtime.cpp", "ojh_manifest.cpp", "ojh_ops.cpp", "ojh_moe.cpp", "ojh_gguf.cpp", "ojh_expert_cache.cpp", "ojh_noalloc.cpp", "ojh_chain.cpp"]

@@ -291,6 +291,97 @@ static int shape_gemm_q8k_xt_sr(const ojh_kernel_spec *, const ojh_device *dev, 
     block[1] = block[2] = 1;
     return OJH_OK;
 }
+// Family "gemv_q8": row-int8 weights (K int8 per row, one f32 scale per row) against f32 activations, the reference's
+// own names and argument order (crates/ojas-cuda/src/kernels/gemv_q8.rs:48-152).  `rows_per_wave` tells the entries apart:
+//   0 gemv_q8 / gemv_q8_accum(x, w, y, scale, K, N)       2 gemv_q8_bias(x, w, y, scale, bias, K, N)
+//   3 gemv_q8_ksplit(x, w, y, scale, K, N): grid [N]      4 ffn_gu_q8(x, wg, wu, out, sg, su, K, N, act)
+//   5 qkv_q8(x, wq, wk, wv, yq, yk, yv, sq, sk, sv, bq, bk, bv, K, Nq, Nkv): the three biases may be NULL
+//   6 embed_q8(table, scale, out, token, D)               7 quantize_q8_pertoken(x, q8, d8, K): grid [M]
+static int check_gemv_q8(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                         const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const int kind = s->rows_per_wave;
+    if (grid[1] != 1 || grid[2] != 1 || !grid[0]) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+    const uint32_t bmax = kind >= 6 ? 256u : 1024u;
+    if (block[1] != 1 || block[2] != 1 || !block[0] || block[0] % 64 || block[0] > bmax)
+        return ojh_fail(OJH_ERR_ARG, "%s: block must be [64 .. %u in whole waves,1,1]", s->name, bmax);
+    if (kind == 6) {
+        const size_t token = c[0], D = c[1];
+        if (!D) return ojh_fail(OJH_ERR_ARG, "%s: D=0", s->name);
+        need[0] = (token + 1) * D;
+        need[1] = (token + 1) * 4;
+        need[2] = D * 4;
+        align[0] = 1;
+        align[1] = align[2] = 4;
+        return OJH_OK;
+    }
+    const size_t K = c[0];
+    if (kind == 7) {
+        if (!K) return ojh_fail(OJH_ERR_ARG, "%s: K=0", s->name);
+        const size_t M = grid[0];
+        need[0] = M * K * 4;
+        need[1] = M * K;
+        need[2] = M * 4;
+        align[0] = align[2] = 4;
+        align[1] = 1;
+        return OJH_OK;
+    }
+    if (!K || K % 4) return ojh_fail(OJH_ERR_ARG, "%s: K=%zu must be a positive multiple of 4", s->name, K);
+    const size_t wa = K % 16 ? 4 : 16;
+    need[0] = K * 4;
+    if (kind == 5) {
+        const size_t Nq = c[1], Nkv = c[2];
+        if (!Nq || !Nkv) return ojh_fail(OJH_ERR_ARG, "%s: Nq=%zu Nkv=%zu", s->name, Nq, Nkv);
+        for (int i = 0; i < 3; i++) {
+            const size_t n = i ? Nkv : Nq;
+            need[1 + i] = n * K;
+            align[1 + i] = wa;
+            need[4 + i] = need[7 + i] = need[10 + i] = n * 4;
+            align[4 + i] = align[7 + i] = 4;
+            align[10 + i] = 0;                  // 0: the buffer may be NULL (4-byte aligned when given)
+        }
+        return OJH_OK;
+    }
+    const size_t N = c[1];
+    if (!N) return ojh_fail(OJH_ERR_ARG, "%s: N=0", s->name);
+    if (kind == 3 && grid[0] != N) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [N,1,1]", s->name);
+    if (kind == 4) {
+        if (c[2] > 1) return ojh_fail(OJH_ERR_ARG, "%s: act=%u (0 SiLU, 1 GELU)", s->name, c[2]);
+        need[1] = need[2] = N * K;
+        align[1] = align[2] = wa;
+        need[3] = need[4] = need[5] = N * 4;
+        align[3] = align[4] = align[5] = 4;
+        return OJH_OK;
+    }
+    need[1] = N * K;
+    align[1] = wa;
+    need[2] = need[3] = N * 4;
+    align[2] = align[3] = 4;
+    if (kind == 2) { need[4] = N * 4; align[4] = 4; }
+    return OJH_OK;
+}
+// rows grid-stride: four workgroups per CU at most (the activations are staged once per workgroup)
+static int shape_gemv_q8(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
+                         uint32_t grid[3], uint32_t block[3]) {
+    const int kind = s->rows_per_wave;
+    const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
+    block[0] = 256;
+    block[1] = block[2] = grid[1] = grid[2] = 1;
+    if (kind == 3) { grid[0] = N ? N : 1; block[0] = K >= 8192 ? 512 : 256; return OJH_OK; }
+    if (kind == 7) { grid[0] = M ? M : 1; return OJH_OK; }
+    if (kind == 6) { grid[0] = (N + 255) / 256 ? (N + 255) / 256 : 1; return OJH_OK; }   // N: the row length D
+    // Up to two workgroups per CU (each stages the activations in 64 KB of LDS), as many waves in each as the rows give
+    // work for: a wave takes two rows (one output of ffn_gu_q8) per pass.
+    const uint32_t per_wave = kind == 4 ? 1 : 2;
+    // (measured, K = 4096: 4096 rows 256 threads x 512 workgroups 6.2 us against 7.3 for 512 x 256; 14336 rows 1024 x 448
+    // 14.9 against 17.1 for 256 x 512; 128256 rows 1024 x 256 96.6 us = 5.4 TB/s against 125 for 256 x 512)
+    uint32_t waves = 4;
+    while (waves < 16 && (uint64_t)2 * cus * waves * per_wave < N) waves *= 2;
+    block[0] = 64 * waves;
+    uint32_t g = (N + waves * per_wave - 1) / (waves * per_wave);
+    if (g > 2 * cus) g = cus;                 // several passes: one large workgroup per CU
+    grid[0] = g ? g : 1;
+    return OJH_OK;
+}
 // gemm_q8k_{q6k,q5k}_gs(xq, xs, w, y, K, N, M, ACC): grid [ceil(N / 64), ceil(M / 128), 1] x 256
 // gemm_q8k_{q6k,q5k}_gs_sr(xq, xs, w, y, part, cnt, K, N, M, ACC, NSPLIT): grid [.., .., slices]; part: 32 KB per tile
 // and slice; cnt: a zeroed word per tile (`rows_per_wave` = 1 marks the sliced entry)
@@ -1669,6 +1760,14 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("gemm_q8k_q4k_xt", "gemm_q8k", 5, 5, OJH_Q4_K, 1, check_gemm_q8k_xt, shape_gemm_q8k_xt);
     add("gemm_q8k_q4k_xt64", "gemm_q8k", 5, 5, OJH_Q4_K, 2, check_gemm_q8k_xt, shape_gemm_q8k_xt);
     add("gemm_q8k_q4k_xt64_sr", "gemm_q8k", 7, 6, OJH_Q4_K, 2, check_gemm_q8k_xt_sr, shape_gemm_q8k_xt_sr);
+    add("gemv_q8", "gemv_q8", 4, 2, 0, 0, check_gemv_q8, shape_gemv_q8);
+    add("gemv_q8_accum", "gemv_q8", 4, 2, 0, 0, check_gemv_q8, shape_gemv_q8);
+    add("gemv_q8_bias", "gemv_q8", 5, 2, 0, 2, check_gemv_q8, shape_gemv_q8);
+    add("gemv_q8_ksplit", "gemv_q8", 4, 2, 0, 3, check_gemv_q8, shape_gemv_q8);
+    add("ffn_gu_q8", "gemv_q8", 6, 3, 0, 4, check_gemv_q8, shape_gemv_q8);
+    add("qkv_q8", "gemv_q8", 13, 3, 0, 5, check_gemv_q8, shape_gemv_q8);
+    add("embed_q8", "gemv_q8", 3, 2, 0, 6, check_gemv_q8, shape_gemv_q8);
+    add("quantize_q8_pertoken", "gemv_q8", 3, 1, 0, 7, check_gemv_q8, shape_gemv_q8);
     add("gemm_q8k_q6k_gs", "gemm_q8k", 4, 4, OJH_Q6_K, 0, check_gemm_q8k_gs, shape_gemm_q8k_gs);
     add("gemm_q8k_q6k_gs_sr", "gemm_q8k", 6, 5, OJH_Q6_K, 1, check_gemm_q8k_gs, shape_gemm_q8k_gs);
     add("gemm_q8k_q5k_gs", "gemm_q8k", 4, 4, OJH_Q5_K, 0, check_gemm_q8k_gs, shape_gemm_q8k_gs);

@@ -411,7 +411,12 @@ extern "C" int ojh_dispatch(ojh_device *dev, const char *name, int n_bufs, ojh_b
     std::vector<void *> ptrs;
     for (int i = 0; i < n_bufs; i++) {
         size_t off = offsets ? (size_t)offsets[i] : 0;
+        if (!bufs[i] && align[i] == 0) {     // a buffer the kernel takes as optional (a bias that may be absent)
+            ptrs.push_back(nullptr);
+            continue;
+        }
         if (!bufs[i]) return ojh_fail(OJH_ERR_ARG, "%s: buffer %d is NULL", name, i);
+        if (align[i] == 0) align[i] = 4;
         if (off > bufs[i]->bytes || need[i] > bufs[i]->bytes - off)
             return ojh_fail(OJH_ERR_BOUNDS, "%s: buffer %d needs %zu bytes at offset %zu, has %zu", name, i,
                             need[i], off, bufs[i]->bytes);

@@ -502,9 +502,10 @@ class HipGpu:
         return list(g), list(b)
 
     def dispatch(self, enc: Enc, name: str, bufs, consts, grid, block) -> None:
-        """`bufs` is a list of (Buf, byte_offset); buffers first, then u32 constants."""
+        """`bufs` is a list of (Buf, byte_offset); buffers first, then u32 constants.  A Buf of None is passed as NULL,
+        for the few kernels that take an optional buffer (the biases of `qkv_q8`)."""
         n = len(bufs)
-        hs = (C.c_void_p * max(n, 1))(*[b.handle for b, _ in bufs])
+        hs = (C.c_void_p * max(n, 1))(*[b.handle if b is not None else None for b, _ in bufs])
         offs = (C.c_uint64 * max(n, 1))(*[o for _, o in bufs])
         cs = (C.c_uint32 * max(len(consts), 1))(*consts)
         g, b = (C.c_uint32 * 3)(*grid), (C.c_uint32 * 3)(*block)

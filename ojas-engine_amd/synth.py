@@ -285,6 +285,17 @@ def tvec_first(seeds: np.ndarray) -> np.ndarray:
     return ((s >> np.uint64(9)).astype(np.float32) / np.float32(1 << 23)) - np.float32(1.0)
 
 
+def q8_rows(rows: int, k: int, seed: int) -> tuple[np.ndarray, np.ndarray]:
+    """Row-int8 weights and their per-row scales as the reference's conformance tests make them
+    (crates/ojas-cuda/tests/conformance.rs:248-258): w[i] = round(127 tvec(1, seed + i)) (halves away from zero),
+    scale[r] = 0.01 + 0.001 |tvec(1, seed ^ (r + 7))|."""
+    v = tvec_first((np.arange(rows * k, dtype=np.uint64) + np.uint64(seed)) & np.uint64(0xFFFFFFFF)) * np.float32(127.0)
+    w = np.clip(np.sign(v) * np.floor(np.abs(v) + np.float32(0.5)), -127, 127).astype(np.int8).reshape(rows, k)
+    t = tvec_first(np.uint64(seed) ^ (np.arange(rows, dtype=np.uint64) + np.uint64(7)))
+    scale = (np.float32(0.01) + np.float32(0.001) * np.abs(t)).astype(np.float32)
+    return w, scale
+
+
 def q80_rows_mod5(rows: int, k: int, seed: int) -> tuple[np.ndarray, np.ndarray]:
     """Q8_0 rows of the reference's integer-dot conformance tests and the values a reader decodes them to
     (crates/ojas-cuda/tests/conformance.rs:607-628): block (r, b) has d = f16(0.004 + 0.001 ((r + b) % 5)),

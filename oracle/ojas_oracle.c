@@ -554,6 +554,33 @@ void ojo_quantize_q8_1(const float *x, size_t k, int8_t *q8, float *d8, float *d
         d8sum[b] = d * s;
     }
 }
+/* The reference GPU decoder's row-int8 matvec (crates/ojas-cuda/src/kernels/gemv_q8.rs:31-55): K plain int8 per row and
+ * one f32 scale per row against f32 activations, y[n] = scale[n] * sum_k (float) w[n][k] * x[k].  The GPU adds a lane's
+ * terms and then the lanes in an order of its own; here the terms (exact in a double) meet in a double and the row scale
+ * is applied in f32, as the reference's test oracle does after its own f32 sum (crates/ojas-cuda/tests/conformance.rs:259-268). */
+void ojo_gemv_q8_rows(const int8_t *w, const float *scale, const float *x, size_t k, size_t n, float *y) {
+    for (size_t r = 0; r < n; r++) {
+        double acc = 0.0;
+        for (size_t i = 0; i < k; i++) acc += (double)w[r * k + i] * (double)x[i];
+        y[r] = (float)acc * scale[r];
+    }
+}
+/* Per-token activation quantizer of the reference's batched int8 GEMM (crates/ojas-cuda/src/kernels/gemv.rs:57-74):
+ * d = amax / 127, id = d > 0 ? 1 / d : 0, q = clamp(round-to-nearest-even(x * id), -127, 127); d8[token] = d. */
+void ojo_quantize_q8_pertoken(const float *x, size_t m, size_t k, int8_t *q8, float *d8) {
+    for (size_t t = 0; t < m; t++) {
+        const float *xr = x + t * k;
+        float a = 0.0f;
+        for (size_t i = 0; i < k; i++) a = fmaxf(a, fabsf(xr[i]));
+        float d = a / 127.0f, id = d > 0.0f ? 1.0f / d : 0.0f;
+        for (size_t i = 0; i < k; i++) {
+            float r = rintf(xr[i] * id);
+            int qi = r != r ? 0 : r > 127.0f ? 127 : r < -127.0f ? -127 : (int)r;
+            q8[t * k + i] = (int8_t)qi;
+        }
+        d8[t] = d;
+    }
+}
 /* One block_q8_0 row against q8_1 activations (crates/ojas-cuda/src/kernels/gemv_q8.rs:178-193): a lane's term is
  * dw * d8[b] * (float) idot over its 8 weights; the GPU adds the terms in a lane and then across lanes in an order of its
  * own, here they meet in a double (the kernels are compared to a tolerance of a few f32 roundings). */

@@ -30,6 +30,9 @@
  *   dot_q4k/q5k/q6k         identity dot(row, quant(x)) == sum dequant(row)*(scale*q) in f64,
  *                           one-hot activations (pins nibble / sub-block order)
  *   relayout_q4k_q4l        qa*nib+qb == dequant up to the two f16 roundings, one-hot blocks
+ *   gemv_q8_rows            numpy f64 product on the generators of crates/ojas-cuda/tests/conformance.rs:248-268 (q8_rows,
+ *                           tvec), all-ones rows (y = scale * sum x), one-hot activations
+ *   quantize_q8_pertoken    invariants (max|q| = 127, d = amax / 127, ties to even at x = 0.5 d and 1.5 d, zero tokens -> d = 0, q = 0)
  *   moe_topk                softmax + stable sort closed form (numpy)
  *   moe_ffn                 composition of the above
  * The f32 association order inside dot_q4k / dot_q6k is pinned by the source text only; it
@@ -108,6 +111,10 @@ int ojo_matvec_kq(const uint8_t *raw, uint32_t ty, size_t n, size_t k, const flo
 /* Row-int8 path every dense CPU model runs (cpu_math.rs:174-179, :187-274, :404-415)
  * and its load-time requantizer (crates/ojas-formats/src/quant.rs:16-39). */
 void ojo_quantize_q8_1(const float *x, size_t k, int8_t *q8, float *d8, float *d8sum);
+/* The reference GPU decoder's row-int8 matvec and its per-token quantizer (crates/ojas-cuda/src/kernels/gemv_q8.rs:31-55,
+ * gemv.rs:57-74). */
+void ojo_gemv_q8_rows(const int8_t *w, const float *scale, const float *x, size_t k, size_t n, float *y);
+void ojo_quantize_q8_pertoken(const float *x, size_t m, size_t k, int8_t *q8, float *d8);
 double ojo_row_q80_dp4a(const uint8_t *row, const int8_t *q8, const float *d8, size_t k);
 void ojo_gemv_q80_dp4a(const uint8_t *w, const int8_t *q8, const float *d8, size_t k, size_t n, float *y);
 float ojo_quant_row_i8(const float *row, size_t k, int8_t *q);

@@ -77,6 +77,10 @@ def lib() -> C.CDLL:
         L.ojo_quantize_q8_1.argtypes = [vp, sz, vp, vp, vp]
         L.ojo_gemv_q80_dp4a.restype = None
         L.ojo_gemv_q80_dp4a.argtypes = [vp, vp, vp, sz, sz, vp]
+        L.ojo_gemv_q8_rows.argtypes = [vp, vp, vp, sz, sz, vp]
+        L.ojo_gemv_q8_rows.restype = None
+        L.ojo_quantize_q8_pertoken.argtypes = [vp, sz, sz, vp, vp]
+        L.ojo_quantize_q8_pertoken.restype = None
         L.ojo_q8_rows_from_f16.restype = None
         L.ojo_q8_rows_from_f16.argtypes = [vp, sz, sz, vp, vp]
         L.ojo_matmul_q8.restype = None
@@ -230,6 +234,24 @@ def gemv_q80_dp4a(raw: np.ndarray, q8: np.ndarray, d8: np.ndarray, n: int, k: in
     y = np.empty(n, np.float32)
     lib().ojo_gemv_q80_dp4a(_p(raw), _p(q8), _p(d8), k, n, _p(y))
     return y
+
+
+def gemv_q8_rows(w: np.ndarray, scale: np.ndarray, x: np.ndarray) -> np.ndarray:
+    """y[n] = scale[n] * sum_k w[n][k] x[k] for row-int8 weights w [N][K] (the reference GPU decoder's `gemv_q8`)."""
+    w, scale, x = np.ascontiguousarray(w, np.int8), np.ascontiguousarray(scale, np.float32), np.ascontiguousarray(x, np.float32)
+    n, k = w.shape
+    assert scale.size == n and x.size == k
+    y = np.empty(n, np.float32)
+    lib().ojo_gemv_q8_rows(_p(w), _p(scale), _p(x), k, n, _p(y))
+    return y
+
+
+def quantize_q8_pertoken(x: np.ndarray):
+    x = np.ascontiguousarray(x, np.float32)
+    m, k = x.shape
+    q8, d8 = np.empty((m, k), np.int8), np.empty(m, np.float32)
+    lib().ojo_quantize_q8_pertoken(_p(x), m, k, _p(q8), _p(d8))
+    return q8, d8
 
 
 def q8_rows_from_f16(w16: np.ndarray, n: int, k: int):

@@ -739,3 +739,43 @@ def test_mxfp4_hand_computed_blocks(orc):
     # the f16 decoder is the same value rounded once
     raw = orc.synth_blocks(MXFP4, 64)
     assert np.array_equal(orc.dequant_to_f16(raw, MXFP4, 64 * 32), orc.dequant_to_f64(raw, MXFP4, 64 * 32).astype(np.float16).view(np.uint16))
+
+
+def test_row_int8_gemv_and_per_token_quantizer_restatements(orc, pkg):
+    """`gemv_q8` (crates/ojas-cuda/src/kernels/gemv_q8.rs:31-55) on the generators of the reference's own test
+    (crates/ojas-cuda/tests/conformance.rs:248-286: K = 512, N = 256, seeds 11 / 12) against a numpy f64 product, all-ones
+    rows and one-hot activations; `quantize_q8_pertoken` (gemv.rs:57-74) against its invariants."""
+    k, n = 512, 256
+    x = pkg.synth.tvec(k, 11)
+    w, scale = pkg.synth.q8_rows(n, k, 12)
+    assert w.dtype == np.int8 and np.abs(w.astype(np.int32)).max() <= 127 and 0.01 <= scale.min() and scale.max() <= 0.011
+    # the generator itself, value by value on a few entries (Rust: (tvec(1, seed + i)[0] * 127).round())
+    for i in (0, 1, 777, n * k - 1):
+        v = float(pkg.synth.tvec(1, 12 + i)[0]) * 127.0
+        assert int(w.ravel()[i]) == int(np.sign(v) * np.floor(abs(v) + 0.5))
+    y = orc.gemv_q8_rows(w, scale, x)
+    want = (w.astype(np.float64) @ x.astype(np.float64)).astype(np.float32) * scale
+    assert np.array_equal(y, want)
+    # the reference's oracle sums in f32, term by term: the two agree far inside its 1e-4 bound
+    acc = np.zeros(n, np.float32)
+    for i in range(k):
+        acc += w[:, i].astype(np.float32) * x[i]
+    assert np.max(np.abs(acc * scale - y) / np.maximum(np.abs(y), 1e-6)) < 1e-4
+    ones = np.ones((3, k), np.int8)
+    assert np.allclose(orc.gemv_q8_rows(ones, np.float32([1, 2, 0.5]), x), np.float32([1, 2, 0.5]) * x.astype(np.float64).sum(), rtol=1e-6)
+    e = np.zeros(k, np.float32)
+    e[37] = 2.0
+    assert np.array_equal(orc.gemv_q8_rows(w, scale, e), (2.0 * w[:, 37].astype(np.float32)) * scale)
+    # the per-token quantizer
+    xs = pkg.synth.normal_f32(5 * 640, "oracle", "pertoken").reshape(5, 640)
+    xs[3] = 0.0
+    xs[4, 0] = 127.0                      # d = 1: the codes are rint(x)
+    xs[4, 1:5] = [0.5, 1.5, -2.5, 126.5]  # ties go to the even neighbour
+    xs[4, 5:] = np.clip(xs[4, 5:], -100, 100)
+    q, d = orc.quantize_q8_pertoken(xs)
+    assert np.array_equal(d, (np.abs(xs).max(1) / np.float32(127.0)).astype(np.float32))
+    assert d[3] == 0.0 and not q[3].any()
+    assert list(q[4, :5]) == [127, 0, 2, -2, 126]
+    for t in (0, 1, 2):
+        assert np.abs(q[t].astype(np.int32)).max() == 127
+        assert np.all(np.abs(xs[t] - d[t] * q[t].astype(np.float32)) <= d[t] * 0.5 * (1 + 1e-5))
