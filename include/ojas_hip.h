@@ -217,8 +217,9 @@ int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dtype, const o
  * `ojh_noalloc_scratch_bytes()` bytes (1 MiB of activations + their scales) that each GPU holds
  * until the process ends, so the call allocates and frees nothing; the launches and results are
  * those of `ojh_mm(..., OJH_ACT_Q8K)` bit for bit below 17 tokens; from there `ojh_mm` may take a
- * prefill tile that stages more in library scratch, which this entry never does (it stays on the
- * few-token kernels: the same integer sums, f32 terms in the same order).  K-quant weights (Q4_K, Q5_K, Q6_K), f32 or bf16
+ * prefill tile or K slices that stage more in library scratch, which this entry never does (Q4_K stays
+ * on the few-token kernels, Q6_K / Q5_K take their 128-token tile unsliced: the same integer sums, the
+ * f32 terms equal to rounding).  K-quant weights (Q4_K, Q5_K, Q6_K), f32 or bf16
  * activations, m * K <= OJH_NOALLOC_MAX_ACT (OJH_ERR_BOUNDS beyond); the families "gemv_q8k" and
  * "gemm_q8k" must already be loaded (OJH_ERR_NOT_LOADED otherwise: loading allocates).  Every
  * handle on one GPU shares that GPU's array: calls that overlap on one GPU race. */

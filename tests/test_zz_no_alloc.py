@@ -53,6 +53,25 @@ def test_no_alloc_matches_mm_on_consecutive_calls(gpu, pkg, orc):
     _both(gpu, pkg, orc, Q6_K, 130, 256, 1, "e", accum=True)
 
 
+def test_no_alloc_takes_the_unsliced_prefill_tile(gpu, pkg, orc):
+    """Q6_K rows against 40 tokens: `ojh_mm` runs the 128-token tile over K slices that meet in library scratch, the entry
+    that allocates nothing runs the same tile whole — the same integer sums, the super-blocks' f32 terms added in one
+    pass instead of per slice: equal to rounding, and each within the bar of matvec_kq."""
+    gpu.ensure_family("gemv_q8k")
+    gpu.ensure_family("gemm_q8k")
+    n, k, m = 256, 2048, 40
+    w = _weights(pkg, Q6_K, n, k, "tile")
+    lin = gpu.lin(Q6_K, n, k, w)
+    x = pkg.synth.normal_f32(m * k, "noalloc", "xtile").reshape(m, k)
+    xd, ya, yb = gpu.upload(x), gpu.alloc(m * n), gpu.alloc(m * n)
+    gpu.mm(xd, lin, ya, m, act_mode=pkg.ACT_Q8K)
+    gpu.mm_noalloc(xd, lin, yb, m)
+    a, b = gpu.read(ya, m * n), gpu.read(yb, m * n)
+    ref = np.stack([orc.matvec_kq(w, Q6_K, n, k, x[t]) for t in range(m)]).ravel()
+    assert peak_err(a, ref) <= 2e-5 and peak_err(b, ref) <= 2e-5 and peak_err(a, b) <= 2e-6
+    lin.free()
+
+
 def test_no_alloc_limits_and_errors(gpu, pkg):
     n, k = 64, 4096
     lin = gpu.lin(Q4_K, n, k, _weights(pkg, Q4_K, n, k, "lim"))
