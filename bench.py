@@ -404,8 +404,8 @@ def extras(gpu, pkg, lin_q) -> dict:
                                "tile": "v_mfma_f32_32x32x16_f16, weights dequantized straight into the B registers: 256 tokens x 256 rows per workgroup where that fills the chip (M = 2048), 128 x 256 below (gate/up M = 512), 128 x 64 with K split over the workgroup's waves where 256-row tiles are too few (M = 128, down M = 512); "
                                        "weights = binary16 fma(qa, q, qb), the bits of the reference's gemm_mm_q4l",
                                "peak_tflops": 2500.0, "timed": "conversion + zero fill (split-K) + tile", **gemm}
-    # ---- the same contraction over Q6_K and Q8_0 weights (the other two formats the path names), bf16 in
-    for ty, tag, gen in ((pkg.Q6_K, "q6k", synth.q6k_weights), (pkg.Q8_0, "q8_0", synth.q80_weights)):
+    # ---- the same contraction over Q6_K, Q5_K and Q8_0 weights (the other formats the path names), bf16 in
+    for ty, tag, gen in ((pkg.Q6_K, "q6k", synth.q6k_weights), (pkg.Q5_K, "q5k", synth.q5k_weights), (pkg.Q8_0, "q8_0", synth.q80_weights)):
         fam = {}
         for name, (n, k) in (("gate_up_14336x4096", (14336, 4096)), ("down_4096x14336", (4096, 14336))):
             lin = gpu.lin(ty, n, k, gen(n, k, "bench", tag, name))

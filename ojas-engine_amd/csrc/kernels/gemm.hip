@@ -123,6 +123,55 @@ struct LoaderQ4K {
     }
 };
 
+// Q5_K: the Q4_K slab with a fifth bit per weight out of qh[32] (bit 2c for the low-nibble sub-block of chunk c,
+// bit 2c + 1 for the high-nibble one): w = f16(d*sc * (nibble + 16 bit) - dmin*m), every operation rounded on its own
+// (crates/ojas-formats/src/gguf.rs:1060-1085).  176-byte blocks: d, dmin, scales[12], qh[32], qs[128].
+struct LoaderQ5K {
+    static constexpr int NL = 3;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
+    u32x4 hdr, qs, qh;
+    uint c;
+    float dl1, ml1, dl2, ml2;
+    uint lo[8], hi[8];
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * Q5K_BYTES; }
+    __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
+        const uchar* blk = row + (size_t)(k0 >> 8) * Q5K_BYTES;
+        c = (k0 >> 6) & 3u;
+        hdr = gm_load16(blk);
+        qh = gm_load16(blk + 16u + h * 16u);
+        qs = gm_load16(blk + 48u + c * 32u + h * 16u);
+    }
+    __device__ __forceinline__ void prep() {
+        uint sc, mn;
+        q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, sc, mn);
+        float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
+        dl1 = __fmul_rn(d, (float)(sc & 0xFFu));
+        ml1 = __fmul_rn(dmin, (float)(mn & 0xFFu));
+        dl2 = __fmul_rn(d, (float)(sc >> 8));
+        ml2 = __fmul_rn(dmin, (float)(mn >> 8));
+    }
+    template <int I>
+    __device__ __forceinline__ void part() {
+        const uint v = qs[I], b = qh[I] >> (2u * c);
+        const uint l = (v & 0x0F0F0F0Fu) | ((b << 4) & 0x10101010u), u = ((v >> 4) & 0x0F0F0F0Fu) | ((b << 3) & 0x10101010u);
+        float a0 = (float)(l & 0xFFu), a1 = (float)((l >> 8) & 0xFFu), a2 = (float)((l >> 16) & 0xFFu), a3 = (float)(l >> 24);
+        float b0 = (float)(u & 0xFFu), b1 = (float)((u >> 8) & 0xFFu), b2 = (float)((u >> 16) & 0xFFu), b3 = (float)(u >> 24);
+        lo[2 * I] = pack2(__fsub_rn(__fmul_rn(dl1, a0), ml1), __fsub_rn(__fmul_rn(dl1, a1), ml1));
+        lo[2 * I + 1] = pack2(__fsub_rn(__fmul_rn(dl1, a2), ml1), __fsub_rn(__fmul_rn(dl1, a3), ml1));
+        hi[2 * I] = pack2(__fsub_rn(__fmul_rn(dl2, b0), ml2), __fsub_rn(__fmul_rn(dl2, b1), ml2));
+        hi[2 * I + 1] = pack2(__fsub_rn(__fmul_rn(dl2, b2), ml2), __fsub_rn(__fmul_rn(dl2, b3), ml2));
+    }
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* p = (u32x4*)(lds_row + h * 32u);
+        p[0] = (u32x4){lo[0], lo[1], lo[2], lo[3]};
+        p[1] = (u32x4){lo[4], lo[5], lo[6], lo[7]};
+        u32x4* ph = (u32x4*)(lds_row + 64u + h * 32u);
+        ph[0] = (u32x4){hi[0], hi[1], hi[2], hi[3]};
+        ph[1] = (u32x4){hi[4], hi[5], hi[6], hi[7]};
+    }
+};
+
 // 64-column slab j of a Q6_K super-block = half hf = j/2, quarters 2(j%2) and 2(j%2)+1: thread half
 // h owns columns 16h..16h+15 of each quarter (ql[16h..], ql[32+16h..], qh[16h..]), one sub-scale
 // per quarter: sc[2q + h].
@@ -438,6 +487,7 @@ __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const 
         gemm_mm_body<LOADER, true>(xh, GmSrc{w, nullptr, nullptr}, y, K, N, 1u, M, nsplit); }
 
 GEMM_ENTRIES(q4k, LoaderQ4K)
+GEMM_ENTRIES(q5k, LoaderQ5K)
 GEMM_ENTRIES(q6k, LoaderQ6K)
 GEMM_ENTRIES(q8_0, LoaderQ80)
 

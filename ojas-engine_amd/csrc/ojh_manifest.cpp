@@ -1798,7 +1798,7 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     // prefill / verify MFMA tiles: "q8_0" is the reference's spelling for this family
     for (const auto &f : kFormats) {
-        if (f.type == OJH_Q5_K || ojh_float_only(f.type) || ojh_grid_type(f.type)) continue;
+        if (ojh_float_only(f.type) || ojh_grid_type(f.type)) continue;
         std::string g = std::string("gemm_mm_") + (f.type == OJH_Q8_0 ? "q8_0" : f.tag);
         add(g, "gemm", 3, 4, f.type, 0, check_gemm, shape_gemm);
         add(g + "_sk", "gemm", 3, 4, f.type, 1, check_gemm, shape_gemm);

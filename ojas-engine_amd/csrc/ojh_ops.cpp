@@ -576,9 +576,12 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     }
 
     // Q5_K: the CPU path's arithmetic (dot_q5k over int8 activations) unless floating-point activations are
-    // asked for, which run on the f32-activation matvecs at any token count; no MFMA tile reads the format.
-    const bool q5_float = w->type == OJH_Q5_K && (act_mode == OJH_ACT_FLOAT || act_mode == OJH_ACT_FLOAT_EXACT);
-    if (w->type == OJH_Q5_K && !q5_float) act_mode = OJH_ACT_Q8K;
+    // asked for, which run on the f32-activation matvecs; from the tile crossover both that request and
+    // OJH_ACT_AUTO take the f16 tile (dequant_to_f16 bits), as Q6_K and Q8_0 do.
+    const bool q5_tile = w->type == OJH_Q5_K && act_mode != OJH_ACT_Q8K && m >= dev->gemm_min_m && K % 64 == 0 &&
+                         (uint64_t)m * K < 0x7FFFFFFFull && (uint64_t)m * N < 0x7FFFFFFFull;
+    const bool q5_float = w->type == OJH_Q5_K && !q5_tile && (act_mode == OJH_ACT_FLOAT || act_mode == OJH_ACT_FLOAT_EXACT);
+    if (w->type == OJH_Q5_K && !q5_float && !q5_tile) act_mode = OJH_ACT_Q8K;
 
     // IQ4_NL / IQ4_XS (dot_iq4nl / dot_iq4xs), Q4_0 / Q4_1 / Q5_0 / Q5_1 and Q2_K / Q3_K: f32 activations against the raw
     // rows at every token count; no int8-activation form and no MFMA tile read them.

@@ -7,7 +7,7 @@ error) and once with x and W unrounded.  Metrics and the reference's bounds:
 the unrounded one (prefill_gemm_q.rs:288-343).  Every tile here feeds the MFMA exactly the
 specified f16 bits, so the first pair is held to (2e-5, 5e-6).
 
-The specified bits: `dequant_to_f16` for Q6_K, Q8_0 and for Q4_K under ACT_FLOAT_EXACT ("x4"
+The specified bits: `dequant_to_f16` for Q5_K, Q6_K, Q8_0 and for Q4_K under ACT_FLOAT_EXACT ("x4"
 below); for Q4_K under ACT_FLOAT the binary16 fma qa*q + qb of the reference's `gemm_mm_q4l`
 (crates/ojas-cuda/src/kernels/gemm_q.rs:104-140), oracle weight mode 2.
 """
@@ -17,7 +17,7 @@ import pytest
 from conftest import peak_err, rms_errs
 
 pytestmark = pytest.mark.gpu
-Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
 X4 = "q4k-exact"   # Q4_K through the tile that holds dequant_to_f16 bits
 TIGHT = (2e-5, 5e-6)
 
@@ -58,7 +58,7 @@ SWEEP = [(64, 256, 128, False), (33, 512, 130, False), (100, 1024, 200, True), (
          (700, 768, 300, True)]
 
 
-@pytest.mark.parametrize("ty", [Q4_K, X4, Q6_K, Q8_0])
+@pytest.mark.parametrize("ty", [Q4_K, X4, Q5_K, Q6_K, Q8_0])
 @pytest.mark.parametrize("m,k,n,accum", SWEEP)
 def test_gemm_sweep(gpu, orc, pkg, ty, m, k, n, accum):
     e16, e32 = _run(gpu, pkg, orc, ty, m, k, n, accum)
@@ -66,7 +66,7 @@ def test_gemm_sweep(gpu, orc, pkg, ty, m, k, n, accum):
     assert e32[0] < 2e-2 and e32[1] < 3e-3, (e32, "vs the unrounded oracle")
 
 
-@pytest.mark.parametrize("ty", [Q4_K, X4, Q6_K])
+@pytest.mark.parametrize("ty", [Q4_K, X4, Q5_K, Q6_K])
 def test_gemm_bf16_activations(gpu, orc, pkg, ty):
     """bf16 activations (the prefill / verify input type) convert to f16 exactly in range."""
     e16, e32 = _run(gpu, pkg, orc, ty, 128, 2048, 256, x_dtype="bf16")
@@ -74,7 +74,7 @@ def test_gemm_bf16_activations(gpu, orc, pkg, ty):
     assert e32[0] < 2e-2 and e32[1] < 3e-3, e32
 
 
-@pytest.mark.parametrize("ty", [Q4_K, X4, Q6_K, Q8_0])
+@pytest.mark.parametrize("ty", [Q4_K, X4, Q5_K, Q6_K, Q8_0])
 def test_tile_holds_the_reference_decoders_bits(gpu, orc, pkg, ty):
     """One-hot activations read the tile back: y[m][n] must be the specified f16 weight [n][m]
     exactly, for every weight of two super-blocks per row and for extreme scales."""
@@ -86,7 +86,7 @@ def test_tile_holds_the_reference_decoders_bits(gpu, orc, pkg, ty):
     off = 208 if ty == Q6_K else 0
     for i in range(raw.shape[0]):
         raw[i, off:off + 2] = scales[i % 8:i % 8 + 1].view(np.uint8)
-        if ty == Q4_K:
+        if ty in (Q4_K, Q5_K):
             raw[i, 2:4] = scales[(i * 3 + 1) % 8:(i * 3 + 1) % 8 + 1].view(np.uint8)
     raw = raw.reshape(-1)
     bits = orc.q4l_weights_f16(raw, k, n) if wmode == 2 else orc.dequant_to_f16(raw, ty, n * k)
