@@ -311,14 +311,17 @@ struct LoaderQ4L {
 // XF32: the activations arrive as f32 [M][K] and are rounded to f16 on their way into the tile (the reference's plain
 // entries); each slab's loads are then consumed where they are issued, which is correct but not pipelined — callers
 // that care convert once (copy_f32_half) and take the f16 entries, as the reference's own `mm` does for split-K.
-template <class Loader, bool SPLITK, bool XF32 = false>
+// MI: 32-token blocks per wave along M — the tile is 64 MI tokens x 128 rows: 4 (256 tokens), or 2 for batches of up to 128
+// tokens, which would leave half of the taller tile's matrix instructions multiplying padding.
+template <class Loader, bool SPLITK, bool XF32 = false, int MI = 4>
 __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const GmSrc src,
                                              float* __restrict__ y, uint K, uint N, uint accum, uint M, uint nsplit) {
     const ushort* xh = (const ushort*)xv;
     const float* xf = (const float*)xv;
-    __shared__ __attribute__((aligned(16))) uchar lds[2 * GM_STAGE];
+    constexpr uint BM = 64u * MI, STAGE = (BM + GM_BN) * GM_STRIDE, NX = 2u * MI;   // NX: activation rows per thread and slab
+    __shared__ __attribute__((aligned(16))) uchar lds[2 * STAGE];
     const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint n0 = blockIdx.x * GM_BN, m0 = blockIdx.y * GM_BM;
+    const uint n0 = blockIdx.x * GM_BN, m0 = blockIdx.y * BM;
     // this block's K range (whole multiples of 64)
     uint k_begin = 0, k_end = K;
     if (SPLITK) {
@@ -331,70 +334,70 @@ __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const 
     const uint xr = tid >> 3, xc = (tid & 7u) * 8u;  // activation slab: rows xr + 32 i, 8 f16 at column xc
     const uint wr = tid >> 1, wh = tid & 1u;         // weight slab: row wr, half wh
     const typename Loader::Row wrow = Loader::row(src, min(n0 + wr, N - 1u), K);
-    size_t xrow[8];   // element offset of the thread's 8 activations in each of its rows
+    size_t xrow[NX];   // element offset of the thread's 8 activations in each of its rows
 #pragma unroll
-    for (int i = 0; i < 8; i++) xrow[i] = (size_t)min(m0 + xr + 32u * i, M - 1u) * K + xc;
+    for (int i = 0; i < (int)NX; i++) xrow[i] = (size_t)min(m0 + xr + 32u * i, M - 1u) * K + xc;
     const uint x_lds = xr * GM_STRIDE + xc * 2u;                   // + i * 32 rows
-    const uint w_lds = GM_BM * GM_STRIDE + wr * GM_STRIDE;
+    const uint w_lds = BM * GM_STRIDE + wr * GM_STRIDE;
 
-    // wave tile: 128 (m) x 64 (n)
-    const uint wm = (wave >> 1) * 128u, wn = (wave & 1u) * 64u;
+    // wave tile: 32 MI (m) x 64 (n)
+    const uint wm = (wave >> 1) * (32u * MI), wn = (wave & 1u) * 64u;
     const uint fr = lane & 31u, kg = lane >> 5;
     const uint a_lds = (wm + fr) * GM_STRIDE + kg * 16u;           // + i * 32 rows, + ks * 32 bytes
-    const uint b_lds = GM_BM * GM_STRIDE + (wn + fr) * GM_STRIDE + kg * 16u;
-    float16v acc[4][2];
+    const uint b_lds = BM * GM_STRIDE + (wn + fr) * GM_STRIDE + kg * 16u;
+    float16v acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    u32x4 xs0[8], xs1[8], xs2[8];
+    u32x4 xs0[NX], xs1[NX], xs2[NX];
     Loader ld0, ld1, ld2;
     const uint nt = (k_end - k_begin) / GM_BK;
 
 #define GM_LOAD(XS, LD, T)                                                                       \
     do {                                                                                         \
         const uint kk_ = k_begin + (T) * GM_BK;                                                  \
-        _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++) XS[i_] = gm_load_x<XF32>(xh, xf, xrow[i_] + kk_); \
+        _Pragma("unroll") for (int i_ = 0; i_ < (int)NX; i_++) XS[i_] = gm_load_x<XF32>(xh, xf, xrow[i_] + kk_); \
         LD.load(wrow, kk_, wh);                                                                  \
         gm_fence();                                                                              \
     } while (0)
 #define GM_STORE_X(XS, STG)                                                                      \
     do {                                                                                         \
-        uchar* a_ = lds + (STG) * GM_STAGE + x_lds;                                              \
-        _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++) *(u32x4*)(a_ + i_ * 32u * GM_STRIDE) = XS[i_]; \
+        uchar* a_ = lds + (STG) * STAGE + x_lds;                                                 \
+        _Pragma("unroll") for (int i_ = 0; i_ < (int)NX; i_++) *(u32x4*)(a_ + i_ * 32u * GM_STRIDE) = XS[i_]; \
     } while (0)
 // fragments of K sub-step KS of stage STG into registers AF/BF; the MFMAs that consume them
 #define GM_READ(STG, KS, AF, BF)                                                                 \
     do {                                                                                         \
-        const uchar* s_ = lds + (STG) * GM_STAGE;                                                \
-        _Pragma("unroll") for (int i = 0; i < 4; i++)                                            \
+        const uchar* s_ = lds + (STG) * STAGE;                                                   \
+        _Pragma("unroll") for (int i = 0; i < MI; i++)                                            \
             AF[i] = *(const half8*)(s_ + a_lds + i * 32u * GM_STRIDE + (KS) * 32u);              \
         _Pragma("unroll") for (int j = 0; j < 2; j++)                                            \
             BF[j] = *(const half8*)(s_ + b_lds + j * 32u * GM_STRIDE + (KS) * 32u);              \
     } while (0)
 #define GM_MMA(AF, BF)                                                                           \
     do {                                                                                         \
-        _Pragma("unroll") for (int i = 0; i < 4; i++)                                            \
+        _Pragma("unroll") for (int i = 0; i < MI; i++)                                           \
             _Pragma("unroll") for (int j = 0; j < 2; j++)                                        \
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(AF[i], BF[j], acc[i][j], 0, 0, 0); \
     } while (0)
 #define GM_MFMA(STG, KS)                                                                         \
     do {                                                                                         \
-        half8 af_[4], bf_[2];                                                                    \
+        half8 af_[MI], bf_[2];                                                                    \
         GM_READ(STG, KS, af_, bf_);                                                              \
         GM_MMA(af_, bf_);                                                                        \
     } while (0)
 // interleave: one MFMA, one LDS read (the next sub-step's fragments), a few vector-ALU
-// instructions (the next step's dequantization) — eight times
+// instructions (the next step's dequantization) — once per matrix instruction of the sub-step
 #define GM_MIX()                                                                                 \
     do {                                                                                         \
-        _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {                                       \
+        _Pragma("unroll") for (int g_ = 0; g_ < 2 * MI; g_++) {                                  \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                   \
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                   \
-            __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);                                   \
+            __builtin_amdgcn_sched_group_barrier(0x002, MI == 4 ? 5 : 10, 0);                                   \
         }                                                                                        \
     } while (0)
 // Interior step T (steps T+1 .. T+3 exist): no branches, so MFMAs and dequantization share one
@@ -402,7 +405,7 @@ __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const 
 #define GM_STEP_FULL(T, XS_FREE, LD_FREE, XS_NEXT, LD_NEXT)                                      \
     do {                                                                                         \
         const uint cur_ = (T) & 1u, nxt_ = cur_ ^ 1u;                                            \
-        half8 afA[4], bfA[2], afB[4], bfB[2];                                                    \
+        half8 afA[MI], bfA[2], afB[MI], bfB[2];                                                    \
         GM_READ(cur_, 0, afA, bfA);                                                              \
         GM_LOAD(XS_FREE, LD_FREE, (T) + 3u);                                                     \
         LD_NEXT.prep();                                                                          \
@@ -411,7 +414,7 @@ __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const 
         GM_READ(cur_, 3, afB, bfB); GM_MMA(afA, bfA); LD_NEXT.template part<2>(); GM_MIX();      \
         GM_MMA(afB, bfB); LD_NEXT.template part<3>(); GM_MIX();                                  \
         GM_STORE_X(XS_NEXT, nxt_);                                                               \
-        LD_NEXT.flush(lds + nxt_ * GM_STAGE + w_lds, wh);                                        \
+        LD_NEXT.flush(lds + nxt_ * STAGE + w_lds, wh);                                           \
         __syncthreads();                                                                         \
     } while (0)
 // Guarded step for the head and tail of the K range.
@@ -425,7 +428,7 @@ __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const 
             LD_NEXT.template part<0>(); LD_NEXT.template part<1>();                              \
             LD_NEXT.template part<2>(); LD_NEXT.template part<3>();                              \
             GM_STORE_X(XS_NEXT, nxt_);                                                           \
-            LD_NEXT.flush(lds + nxt_ * GM_STAGE + w_lds, wh);                                    \
+            LD_NEXT.flush(lds + nxt_ * STAGE + w_lds, wh);                                       \
         }                                                                                        \
         __syncthreads();                                                                         \
     } while (0)
@@ -461,7 +464,7 @@ __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const 
 
     // epilogue: D register v of block (i, j) holds row 8*(v/4) + 4*kg + v%4, column fr
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < MI; i++) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const uint n = n0 + wn + 32u * j + fr;
@@ -478,13 +481,20 @@ __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const 
     }
 }
 
+// `_m128`: the 128-token tile, grid [ceil(N/128), ceil(M/128), nsplit]
 #define GEMM_ENTRIES(FMT, LOADER)                                                                                 \
     extern "C" __global__ void __launch_bounds__(256) gemm_mm_##FMT(                                              \
         const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {                         \
         gemm_mm_body<LOADER, false>(xh, GmSrc{w, nullptr, nullptr}, y, K, N, accum, M, 1u); }                     \
     extern "C" __global__ void __launch_bounds__(256) gemm_mm_##FMT##_sk(                                         \
         const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {                        \
-        gemm_mm_body<LOADER, true>(xh, GmSrc{w, nullptr, nullptr}, y, K, N, 1u, M, nsplit); }
+        gemm_mm_body<LOADER, true>(xh, GmSrc{w, nullptr, nullptr}, y, K, N, 1u, M, nsplit); }                     \
+    extern "C" __global__ void __launch_bounds__(256) gemm_mm_##FMT##_m128(                                       \
+        const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {                         \
+        gemm_mm_body<LOADER, false, false, 2>(xh, GmSrc{w, nullptr, nullptr}, y, K, N, accum, M, 1u); }           \
+    extern "C" __global__ void __launch_bounds__(256) gemm_mm_##FMT##_m128_sk(                                    \
+        const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {                        \
+        gemm_mm_body<LOADER, true, false, 2>(xh, GmSrc{w, nullptr, nullptr}, y, K, N, 1u, M, nsplit); }
 
 GEMM_ENTRIES(q4k, LoaderQ4K)
 GEMM_ENTRIES(q5k, LoaderQ5K)

@@ -1094,6 +1094,10 @@ static void gemm_tile(const ojh_kernel_spec *s, uint32_t *bm, uint32_t *bn, bool
         *bn = 64;
         *bm = 128;
     }
+    if (s->rows_per_wave == 14 || s->rows_per_wave == 15) {   // 128 rows x 128 tokens (the `_m128` entries of family "gemm")
+        *bn = 128;
+        *bm = 128;
+    }
 }
 
 static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
@@ -1802,6 +1806,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         std::string g = std::string("gemm_mm_") + (f.type == OJH_Q8_0 ? "q8_0" : f.tag);
         add(g, "gemm", 3, 4, f.type, 0, check_gemm, shape_gemm);
         add(g + "_sk", "gemm", 3, 4, f.type, 1, check_gemm, shape_gemm);
+        add(g + "_m128", "gemm", 3, 4, f.type, 14, check_gemm, shape_gemm);
+        add(g + "_m128_sk", "gemm", 3, 4, f.type, 15, check_gemm, shape_gemm);
     }
     // Q4L (relaid Q4_K + side arrays) under the reference's names and argument lists
     add("gemm_mm_q4l", "gemm", 5, 4, 0, 8, check_gemm_q4l, shape_gemm);
