@@ -608,7 +608,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         const uint32_t n_el = m * K, conv_blocks = (n_el / 8 + 255) / 256 + 1;
         std::string base = std::string("gemm_mm_") + (w->type == OJH_Q8_0 ? "q8_0" : f->tag);
         // (the tile that shares the dequantized weights through LDS is 256 tokens tall; up to 128 tokens its 128-token form)
-        if (!xl && m <= 128 && dev->gemm_m128) base += "_m128";
+        if (!xl && m <= (uint32_t)dev->gemm_m128) base += "_m128";
         if (xl) {
             // 256-token tiles when they give every CU a tile, or half of them with a K long enough
             // to split in two without the slices' fixed costs showing (measured on MI355X);
