@@ -6,9 +6,8 @@
 // load-time relayout pass; here they are formed in the kernel from the raw super-block header, so
 // the weights stay in the file's layout.  Activations are f16 [M][K], accumulation is f32.
 //
-//   gemm_mm_q4kl{,_m128}(xh, w, y, K, N, accum, M)        grid [ceil(N/256), ceil(M/BM), 1]
-//   gemm_mm_q4kl{,_m128}_sk(xh, w, y, K, N, M, nsplit)    grid.z = nsplit; f32 atomic adds into y
-//   (BM = 256 tokens per tile, 128 for the _m128 entries)
+//   gemm_mm_q4kl(xh, w, y, K, N, accum, M)        grid [ceil(N/256), ceil(M/256), 1]
+//   gemm_mm_q4kl_sk(xh, w, y, K, N, M, nsplit)    grid.z = nsplit; f32 atomic adds into y
 //
 // CDNA4 plan.  One workgroup of 4 waves (one per SIMD) owns BM x 256 outputs and walks K in steps
 // of 64; a wave owns (BM/2) x 128 as (BM/64) x 4 blocks of v_mfma_f32_32x32x16_f16, 256
@@ -746,15 +745,4 @@ extern "C" __global__ void __launch_bounds__(256)
 gemm_mm_q4kl_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
     GX_LDS(4);
     gemm_xl_body<4, true, true>(xh, w, y, K, N, M, nsplit, lds);
-}
-extern "C" __global__ void __launch_bounds__(256)
-gemm_mm_q4kl_m128(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {
-    GX_LDS(2);
-    if (accum) gemm_xl_body<2, false, true>(xh, w, y, K, N, M, 1u, lds);
-    else gemm_xl_body<2, false, false>(xh, w, y, K, N, M, 1u, lds);
-}
-extern "C" __global__ void __launch_bounds__(256)
-gemm_mm_q4kl_m128_sk(const ushort* xh, const uchar* w, float* y, uint K, uint N, uint M, uint nsplit) {
-    GX_LDS(2);
-    gemm_xl_body<2, true, true>(xh, w, y, K, N, M, nsplit, lds);
 }

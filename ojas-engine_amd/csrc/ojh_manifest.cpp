@@ -1820,8 +1820,6 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("gemm_mm_q4kl_bd256_sr", "gemm_xl", 5, 5, OJH_Q4_K, 256, check_gemm_sr, shape_gemm_sr);
     add("gemm_mm_q4kl", "gemm_xl", 3, 4, OJH_Q4_K, 2, check_gemm, shape_gemm);
     add("gemm_mm_q4kl_sk", "gemm_xl", 3, 4, OJH_Q4_K, 3, check_gemm, shape_gemm);
-    add("gemm_mm_q4kl_m128", "gemm_xl", 3, 4, OJH_Q4_K, 4, check_gemm, shape_gemm);
-    add("gemm_mm_q4kl_m128_sk", "gemm_xl", 3, 4, OJH_Q4_K, 5, check_gemm, shape_gemm);
     add("gemm_mm_q4kl_bd", "gemm_xl", 3, 4, OJH_Q4_K, 6, check_gemm, shape_gemm);      // 128 x 256, weights dequantized into B registers
     add("gemm_mm_q4kl_bd_sk", "gemm_xl", 3, 4, OJH_Q4_K, 7, check_gemm, shape_gemm);
     add("gemm_mm_q4kl_bd256", "gemm_xl", 3, 4, OJH_Q4_K, 2, check_gemm, shape_gemm);   // ... 256 x 256

@@ -104,7 +104,6 @@ def test_tile_holds_the_reference_decoders_bits(gpu, orc, pkg, ty):
 
 @pytest.mark.parametrize("kernel,family,bm,bn,wmode", [("gemm_mm_q4k_sk", "gemm", 256, 128, 1),
                                                        ("gemm_mm_q4kl_sk", "gemm_xl", 256, 256, 2),
-                                                       ("gemm_mm_q4kl_m128_sk", "gemm_xl", 128, 256, 2),
                                                        ("gemm_mm_q4kl_bd_sk", "gemm_xl", 128, 256, 2),
                                                        ("gemm_mm_q4kl_bd256_sk", "gemm_xl", 256, 256, 2),
                                                        ("gemm_mm_q4kl_bdk_sk", "gemm_xl", 128, 64, 2)])
@@ -204,8 +203,7 @@ def test_mm_with_reproducible_split_k(gpu, orc, pkg, monkeypatch):
 def test_tile_with_weights_dequantized_into_registers(gpu, orc, pkg, m, k, n):
     """`gemm_mm_q4kl_bd`, `gemm_mm_q4kl_bd256` and `gemm_mm_q4kl_bdk` by name: the 128 x 256 and 256 x 256 tiles whose waves
     dequantize their own 64 rows into the B operand, and the 128 x 64 tile whose waves share 64 rows and split K.  Ragged
-    M and N, store and accumulate, sentinels behind row M; the oracle holds the tile's specified f16 weights, and the
-    tile that shares the dequantized weights through LDS agrees to the order of the f32 sums inside a K step."""
+    M and N, store and accumulate, sentinels behind row M; the oracle holds the tile's specified f16 weights."""
     gpu.ensure_family("gemm_xl")
     w = pkg.synth.q4k_weights(n, k, "bd", "w", n, k)
     x = pkg.synth.normal_f32(m * k, "bd", "x", m, k).reshape(m, k)
@@ -213,7 +211,7 @@ def test_tile_with_weights_dequantized_into_registers(gpu, orc, pkg, m, k, n):
     want = orc.matmul_ref(w, Q4_K, n, k, x, wmode=2, xmode=1)
     sent = np.full(n, 12345.5, np.float32)
     outs = {}
-    for kernel, bm in (("gemm_mm_q4kl_bd", 128), ("gemm_mm_q4kl_bd256", 256), ("gemm_mm_q4kl_m128", 128), ("gemm_mm_q4kl_bdk", 128)):
+    for kernel, bm in (("gemm_mm_q4kl_bd", 128), ("gemm_mm_q4kl_bd256", 256), ("gemm_mm_q4kl_bdk", 128)):
         grid = [(n + 63) // 64 if kernel.endswith("bdk") else (n + 255) // 256, (m + bm - 1) // bm, 1]
         for accum in (0, 1):
             y0 = pkg.synth.normal_f32(m * n, "bd", "y0", accum).reshape(m, n)
@@ -225,7 +223,6 @@ def test_tile_with_weights_dequantized_into_registers(gpu, orc, pkg, m, k, n):
             e = rms_errs(got, want + (y0 if accum else 0.0))
             assert e[0] < 1e-4 and e[1] < 2e-5, (kernel, accum, e)
             outs[kernel, accum] = got
-    assert peak_err(outs["gemm_mm_q4kl_bd", 0], outs["gemm_mm_q4kl_m128", 0]) <= 2e-6
     assert np.array_equal(outs["gemm_mm_q4kl_bd256", 0], outs["gemm_mm_q4kl_bd", 0])      # the same sums in the same order
     # 64-row tiles whose four waves split K: the same products, the K quarters added at the end
     assert peak_err(outs["gemm_mm_q4kl_bdk", 0], outs["gemm_mm_q4kl_bd", 0]) <= 2e-6
