@@ -13,7 +13,7 @@ import pytest
 from conftest import peak_err, rms_errs
 
 pytestmark = pytest.mark.gpu
-Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
 
 
 def _rows(raw, ty, pkg, k, rows):
@@ -110,6 +110,37 @@ def test_prefill_in_the_cpu_arithmetic_at_full_size(gpu, orc, pkg, n, k, m):
     y2 = gpu.alloc(m * n)
     gpu.mm(gpu.upload_bytes(xb.reshape(m, k)[perm].copy()), lin, y2, m, x_dtype=pkg.X_BF16, act_mode=pkg.ACT_Q8K)
     assert np.array_equal(gpu.read(y2, m * n).reshape(m, n), got[perm])
+
+
+@pytest.mark.parametrize("ty", [Q6_K, Q5_K])
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("m", [64, 512])
+def test_q6k_q5k_prefill_in_the_cpu_arithmetic_at_full_size(gpu, orc, pkg, ty, n, k, m):
+    """Q6_K and Q5_K rows under OJH_ACT_Q8K at the sizes the benchmark times (`gemm_q8k_{q6k,q5k}_gs`, whole and over K
+    slices as the library picks them): sampled weight rows (tile borders included) against `matvec_kq`, every token up
+    to 64, every seventh of 512 and the borders of the 128-token tiles; a token's outputs do not depend on its
+    position in the batch (bit for bit)."""
+    gen = {Q6_K: pkg.synth.q6k_weights, Q5_K: pkg.synth.q5k_weights}[ty]
+    w = gen(n, k, "full", "gs", n, k)
+    xf = pkg.synth.normal_f32(m * k, "full", "gs-x", m, k).reshape(m, k)
+    lin = gpu.lin(ty, n, k, w)
+    yd = gpu.upload(np.full(m * n + 64, 12345.5, np.float32))
+    gpu.mm(gpu.upload(xf), lin, yd, m, act_mode=pkg.ACT_Q8K)
+    got = gpu.read(yd, m * n + 64)
+    assert np.all(got[m * n:] == 12345.5), "wrote past row M"
+    got = got[:m * n].reshape(m, n)
+    g = pkg.synth.rng("full", "gs-rows", n, k, m)
+    rows = np.unique(np.concatenate([[0, 31, 32, 63, 64, n - 33, n - 1], g.integers(0, n, 25)]))
+    wsub = _rows(w, ty, pkg, k, rows)
+    tokens = range(m) if m <= 64 else np.unique(np.concatenate([np.arange(0, m, 128), np.arange(127, m, 128), np.arange(0, m, 7)]))
+    for t in tokens:
+        want = orc.matvec_kq(wsub, ty, len(rows), k, xf[t], threads=1)
+        assert peak_err(got[t, rows], want) <= 2e-5, t
+    perm = np.roll(np.arange(m), 37)
+    y2 = gpu.alloc(m * n)
+    gpu.mm(gpu.upload(xf[perm].copy()), lin, y2, m, act_mode=pkg.ACT_Q8K)
+    assert np.array_equal(gpu.read(y2, m * n).reshape(m, n), got[perm])
+    lin.free()
 
 
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
