@@ -813,29 +813,31 @@ gemm_q8k_q4k_xt64_sr(const signed char* xq, const float* xst, const float* sums,
     gemm_q8k_q4k_xt_body<2, true>(xq, xst, sums, w, y, K, N, M, ACC, MP, lds_xt, part, cnt, NSPLIT);
 }
 
-// ---- Q6_K and Q5_K rows against 128 tokens: one matrix instruction per scale group ---------------------------------
-//   gemm_q8k_{q6k,q5k}_gs(xq, xs, w, y, K, N, M, ACC)                      block 256, grid [ceil(N / 64), ceil(M / 128), 1]
+// ---- Q6_K and Q5_K rows against batches of tokens: one matrix instruction per scale group ---------------------------
+//   gemm_q8k_{q6k,q5k}_gs(xq, xs, w, y, K, N, M, ACC)                      block 256, grid [ceil(N / 128), ceil(M / 64), 1]
 //   gemm_q8k_{q6k,q5k}_gs_sr(xq, xs, w, y, part, cnt, K, N, M, ACC, NSPLIT)       grid [.., .., slices]
 // The CPU path's arithmetic (dot_q6k / dot_q5k over quant_q8k activations, crates/ojas-cpu/src/cpu_math.rs:638-722) for
-// prefill-sized batches.  A Q6_K scale covers 16 weights and is a full int8, so it cannot be folded into int8 codes the
-// way the Q4_K tile above folds its 6-bit scales; instead v_mfma_i32_32x32x16_i8, whose 16 positions are exactly one
-// scale group, gives the group's integer dots for 32 tokens x 32 rows, and the scale enters with one v_mad_i32_i24 per
-// D register (the row is lane-constant in D).  Q5_K: two instructions per 32-weight sub-block (codes 0..31 are one
-// int8 plane), the 6-bit scale likewise, and sum_j m_j bsum_j from two more instructions per super-block over the
-// sub-block sums split as 64 hi + lo (the workgroup splits them while it stages the tokens).
-// A workgroup owns 64 rows x 128 tokens: wave (r, t) = (wave % 2, wave / 2) takes rows 32 r .. and tokens 64 t ..
-// as two blocks of 32.  B (weights): lane (n, kg) = (lane % 32, lane / 32) builds the codes of positions 8 kg .. 8 kg + 7
-// of every group of row n from the raw bytes it loads itself, one super-block ahead.  A (tokens): a super-block's 128 x 256
-// int8 wait in LDS, rows 264 bytes apart (32 tokens' 8-byte reads then cover all banks), two stages, one barrier per
-// super-block.  Integer sums are exact; per super-block acc += sx * d * (float) isum, super-blocks in order.
+// batches from a handful of tokens to prefill sizes.  A Q6_K scale covers 16 weights and is a full int8, so it cannot be
+// folded into int8 codes the way the Q4_K tile above folds its 6-bit scales; instead v_mfma_i32_32x32x16_i8, whose 16
+// positions are exactly one scale group, gives the group's integer dots for 32 tokens x 32 rows, and the scale enters
+// with one v_mad_i32_i24 per D register (the row is lane-constant in D).  Q5_K: one v_mfma_i32_32x32x32_i8 per 32-weight
+// sub-block (codes 0..31 are one int8 plane), the 6-bit scale likewise, and sum_j m_j bsum_j from two more
+// instructions per super-block over the sub-block sums split as 64 hi + lo (the workgroup splits them while it stages
+// the tokens).
+// A workgroup owns 128 rows x 64 tokens: wave w takes rows 32 w .. against both blocks of 32 tokens (only the first where
+// the last token tile holds no more).  B (weights): lane (n, kg) = (lane % 32, lane / 32) builds the codes of
+// positions 8 kg .. 8 kg + 7 of every group of row n from the raw bytes it loads itself, one super-block ahead — no two
+// waves of a workgroup build the same codes.  A (tokens): a super-block's 64 x 256 int8 wait in LDS, rows 264 bytes
+// apart (32 tokens' 8-byte reads then cover all banks), two stages, one barrier per super-block.  Integer sums are
+// exact; per super-block acc += sx * d * (float) isum, super-blocks in order.
 // `_sr`: K slices whose partial tiles meet in `part` (tiles x slices x 32 KB), added in slice order by the last to arrive.
 #include "ojk_q6k_mfma.h"
 
 typedef int gs_i16 __attribute__((ext_vector_type(16)));
 #define GS_STRIDE 264u
-#define GS_SX (128u * GS_STRIDE)        // the stage's 128 token scales
-#define GS_BS (GS_SX + 512u)            // Q5_K: the split sub-block sums, 16 bytes per token (lo_0..7, hi_0..7)
-#define GS_STAGE (GS_BS + 2048u)
+#define GS_SX (64u * GS_STRIDE)         // the stage's 64 token scales
+#define GS_BS (GS_SX + 256u)            // Q5_K: the split sub-block sums, 16 bytes per token (lo_0..7, hi_0..7)
+#define GS_STAGE (GS_BS + 1024u)
 
 // A running integer sum, pinned after every group: integer additions may be reassociated, and left to itself the
 // compiler turns sixteen groups' multiply-adds into one tree at the end of the super-block, every group's sixteen result
@@ -875,13 +877,14 @@ struct GsQ6K {
         return r;
     }
     // st: the stage; tok0: the wave's first token in it
+    template <int NB>   // NB: how many of the wave's two 32-token blocks hold tokens
     static __device__ __forceinline__ void superblock(const Raw& r, const uchar* st, uint tok0, uint fr, uint kg,
                                                       float (&acc)[2][16]) {
         const uchar* xa = st + (tok0 + fr) * GS_STRIDE + 8u * kg;            // the lane's token row of block 0, its 8 positions
         const float* sx = (const float*)(st + GS_SX) + tok0 + 4u * kg;       // scales of its D registers' tokens: + 32 i + 8 (v / 4) + v % 4
-        int isum[2][16];
+        int isum[NB][16];
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < NB; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) isum[i][v] = 0;
         const gs_i16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -895,36 +898,41 @@ struct GsQ6K {
             return *(const long*)(xa + (uint)i * 32u * GS_STRIDE + 16u * (uint)g);
         };
         // the next group's operands are fetched and built under this group's matrix instructions, ahead of its multiply-adds
-        long B = codes(0), A0 = tokens(0, 0), A1 = tokens(0, 1);
+        long B = codes(0), A0 = tokens(0, 0), A1 = NB == 2 ? tokens(0, 1) : 0;
 #pragma unroll
         for (int g = 0; g < 16; g++) {
             const uint sw = g < 4 ? r.sc.x : g < 8 ? r.sc.y : g < 12 ? r.sc.z : r.sc.w;
             const int s = (int)(signed char)(sw >> (8 * (g & 3)));
             const gs_i16 D0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(A0, B, zero, 0, 0, 0);
-            const gs_i16 D1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(A1, B, zero, 0, 0, 0);
+            gs_i16 D1 = zero;
+            if (NB == 2) D1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(A1, B, zero, 0, 0, 0);
             if (g < 15) {
                 A0 = tokens(g + 1, 0);
-                A1 = tokens(g + 1, 1);
+                if (NB == 2) A1 = tokens(g + 1, 1);
                 B = codes(g + 1);
             }
 #pragma unroll
             for (int v = 0; v < 16; v++) isum[0][v] = gs_pin(isum[0][v] + __mul24(s, D0[v]));
+            if (NB == 2) {
 #pragma unroll
-            for (int v = 0; v < 16; v++) isum[1][v] = gs_pin(isum[1][v] + __mul24(s, D1[v]));
+                for (int v = 0; v < 16; v++) isum[NB - 1][v] = gs_pin(isum[NB - 1][v] + __mul24(s, D1[v]));
+            }
             // (keeps the groups apart: let loose, the scheduler issues every group's matrix instructions first and
             // spills their results)
             __builtin_amdgcn_sched_barrier(0);
         }
         const float d = f16_bits_to_f32(r.d16);
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < NB; i++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
+                // (spelled out: left to contract `acc += sx * d * isum` as it likes, the compiler fuses the last product
+                // into the addition for one token block and not for the other, and a token's bits depend on its block)
                 const float4 x4 = *(const float4*)(sx + 32 * i + 8 * g);
-                acc[i][4 * g] += x4.x * d * (float)isum[i][4 * g];
-                acc[i][4 * g + 1] += x4.y * d * (float)isum[i][4 * g + 1];
-                acc[i][4 * g + 2] += x4.z * d * (float)isum[i][4 * g + 2];
-                acc[i][4 * g + 3] += x4.w * d * (float)isum[i][4 * g + 3];
+                acc[i][4 * g] = __fmaf_rn(__fmul_rn(x4.x, d), (float)isum[i][4 * g], acc[i][4 * g]);
+                acc[i][4 * g + 1] = __fmaf_rn(__fmul_rn(x4.y, d), (float)isum[i][4 * g + 1], acc[i][4 * g + 1]);
+                acc[i][4 * g + 2] = __fmaf_rn(__fmul_rn(x4.z, d), (float)isum[i][4 * g + 2], acc[i][4 * g + 2]);
+                acc[i][4 * g + 3] = __fmaf_rn(__fmul_rn(x4.w, d), (float)isum[i][4 * g + 3], acc[i][4 * g + 3]);
             }
     }
 };
@@ -948,13 +956,14 @@ struct GsQ5K {
         }
         return r;
     }
+    template <int NB>   // NB: how many of the wave's two 32-token blocks hold tokens
     static __device__ __forceinline__ void superblock(const Raw& r, const uchar* st, uint tok0, uint fr, uint kg,
                                                       float (&acc)[2][16]) {
         const uchar* xa = st + (tok0 + fr) * GS_STRIDE + 8u * kg;            // the lane's token row of block 0, its 8 positions
         const float* sx = (const float*)(st + GS_SX) + tok0 + 4u * kg;       // scales of its D registers' tokens: + 32 i + 8 (v / 4) + v % 4
-        int isum[2][16];
+        int isum[NB][16];
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < NB; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) isum[i][v] = 0;
         const gs_i16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -976,15 +985,15 @@ struct GsQ5K {
         };
         // the next sub-block's operands are fetched and built under this one's matrix instructions
         long B[2] = {codes(0, 0), codes(0, 1)};
-        long A[2][2] = {{tokens(0, 0, 0), tokens(0, 0, 1)}, {tokens(0, 1, 0), tokens(0, 1, 1)}};
+        long A[2][2] = {{tokens(0, 0, 0), NB == 2 ? tokens(0, 0, 1) : 0}, {tokens(0, 1, 0), NB == 2 ? tokens(0, 1, 1) : 0}};
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const int s = (int)(((j < 4 ? sc_lo : sc_hi) >> (8 * (j & 3))) & 0xFFu);
             // (one instruction over all 32 positions of the sub-block: a lane's sixteen are 8 kg .. and 16 + 8 kg ..)
-            gs_i16 D[2];
+            gs_i16 D[NB];
             const gq_i4 Bj = {(int)B[0], (int)(B[0] >> 32), (int)B[1], (int)(B[1] >> 32)};
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
+            for (int i = 0; i < NB; i++) {
                 const gq_i4 Aj = {(int)A[0][i], (int)(A[0][i] >> 32), (int)A[1][i], (int)(A[1][i] >> 32)};
                 D[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(Aj, Bj, zero, 0, 0, 0);
             }
@@ -993,11 +1002,11 @@ struct GsQ5K {
                 for (int h = 0; h < 2; h++) {
                     B[h] = codes(j + 1, h);
                     A[h][0] = tokens(j + 1, h, 0);
-                    A[h][1] = tokens(j + 1, h, 1);
+                    if (NB == 2) A[h][1] = tokens(j + 1, h, 1);
                 }
             }
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < NB; i++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) isum[i][v] = gs_pin(isum[i][v] + __mul24(s, D[i][v]));
             __builtin_amdgcn_sched_barrier(0);
@@ -1008,7 +1017,7 @@ struct GsQ5K {
         const long km = kg ? -1l : 0l;
         const float d = f16_bits_to_f32(r.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(r.hdr.x >> 16);
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < NB; i++) {
             const long A1 = *(const long*)(st + GS_BS + (tok0 + 32u * (uint)i + fr) * 16u + 8u * kg);
             const gs_i16 D1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(A1, Bm, zero, 0, 0, 0);
             const gs_i16 D2 = __builtin_amdgcn_mfma_i32_32x32x16_i8(A1 & km, Bm, zero, 0, 0, 0);
@@ -1019,7 +1028,8 @@ struct GsQ5K {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const int v = 4 * g + e;
-                    acc[i][v] += xv[e] * (d * (float)isum[i][v] - dmin * (float)(D1[v] + 63 * D2[v]));
+                    const float inner = __fmaf_rn(-dmin, (float)(D1[v] + 63 * D2[v]), __fmul_rn(d, (float)isum[i][v]));
+                    acc[i][v] = __fmaf_rn(xv[e], inner, acc[i][v]);
                 }
             }
         }
@@ -1037,27 +1047,31 @@ __device__ __forceinline__ void gemm_q8k_gs_body(const signed char* __restrict__
     const uint per = SPLIT ? (nsb + nsplit - 1u) / nsplit : nsb;
     const uint sb0 = SPLIT ? blockIdx.z * per : 0u, sb1 = SPLIT ? min(nsb, sb0 + per) : nsb;
     if (SPLIT && sb0 >= sb1) return;                      // (the host launches only slices that hold a super-block)
-    const uint m0 = blockIdx.y * 128u, fr = lane & 31u, kg = lane >> 5;
-    const uint row = min(blockIdx.x * 64u + 32u * (wave & 1u) + fr, N - 1u);
-    const uint tok0 = 64u * (wave >> 1);
+    constexpr uint TPG = 64u, RPG = 128u;                     // tokens and rows per workgroup
+    const uint m0 = blockIdx.y * TPG, fr = lane & 31u, kg = lane >> 5;
+    const uint row = min(blockIdx.x * RPG + 32u * wave + fr, N - 1u);
+    const uint tok0 = 0u;
+    // 32-token blocks that hold tokens: the last token tile may need only the first
+    const uint nblk = M - m0 > 32u ? 2u : 1u;
     const uchar* wr = w + (size_t)row * nsb * F::BYTES;
 
-    // staging: thread -> chunk tid % 16 (16 bytes) of tokens tid / 16 + 16 p, p = 0..7
+    // staging: thread -> chunk tid % 16 (16 bytes) of tokens tid / 16 + 16 p, p = 0 .. 3
+    constexpr int NP = 4;
     const uint s_tok = tid >> 4, s_ch = tid & 15u;
-    uint4 tv[8];
+    uint4 tv[NP];
     float tsx = 0.0f;
     auto fetch = [&](uint sb) {
 #pragma unroll
-        for (int p = 0; p < 8; p++) {
+        for (int p = 0; p < NP; p++) {
             const uint m = m0 + s_tok + 16u * (uint)p;
             tv[p] = make_uint4(0u, 0u, 0u, 0u);
             if (m < M) tv[p] = *(const uint4*)(xq + (size_t)m * K + (size_t)sb * 256u + s_ch * 16u);
         }
-        if (tid < 128u) tsx = m0 + tid < M ? xs[(size_t)(m0 + tid) * nsb + sb] : 0.0f;
+        if (tid < TPG) tsx = m0 + tid < M ? xs[(size_t)(m0 + tid) * nsb + sb] : 0.0f;
     };
     auto put = [&](uchar* st) {
 #pragma unroll
-        for (int p = 0; p < 8; p++) {
+        for (int p = 0; p < NP; p++) {
             uchar* o = st + (s_tok + 16u * (uint)p) * GS_STRIDE + s_ch * 16u;
             *(uint2*)o = make_uint2(tv[p].x, tv[p].y);
             *(uint2*)(o + 8) = make_uint2(tv[p].z, tv[p].w);
@@ -1075,7 +1089,7 @@ __device__ __forceinline__ void gemm_q8k_gs_body(const signed char* __restrict__
                 }
             }
         }
-        if (tid < 128u) ((float*)(st + GS_SX))[tid] = tsx;
+        if (tid < TPG) ((float*)(st + GS_SX))[tid] = tsx;
     };
 
     float acc[2][16];
@@ -1094,7 +1108,8 @@ __device__ __forceinline__ void gemm_q8k_gs_body(const signed char* __restrict__
         nx = F::load(wr + (size_t)nb * F::BYTES, kg);
         fetch(nb);
         const uchar* st = lds + ((sb - sb0) & 1u) * GS_STAGE;
-        F::superblock(cur, st, tok0, fr, kg, acc);
+        if (nblk == 2u) F::template superblock<2>(cur, st, tok0, fr, kg, acc);
+        else F::template superblock<1>(cur, st, tok0, fr, kg, acc);
         put(lds + (((sb - sb0) & 1u) ^ 1u) * GS_STAGE);
         __syncthreads();
     }
@@ -1146,7 +1161,7 @@ __device__ __forceinline__ void gemm_q8k_gs_body(const signed char* __restrict__
         if (tid == 0u) cnt[tile] = 0u;                               // ready for the next launch
     }
     // D register v of block i: token 32 i + 8 (v / 4) + 4 kg + v % 4, row fr
-    const uint n = blockIdx.x * 64u + 32u * (wave & 1u) + fr;
+    const uint n = blockIdx.x * RPG + 32u * wave + fr;
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll

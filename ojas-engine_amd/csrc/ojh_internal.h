@@ -76,7 +76,7 @@ struct ojh_device {
     bool no_scratch = false;     // set around calls that may not allocate (ojh_mm_noalloc): paths that need library scratch are skipped
     int gemm_m128 = 128;         // OJAS_HIP_GEMM_M128: tokens up to which Q5_K / Q6_K / Q8_0 batches take the 128-token f16 tile (0: never)
     uint32_t kq_gs_split = 1;    // OJAS_HIP_KQ_GS_SPLIT: K slices of that tile (0: never, 1: chosen, n: n)
-    uint32_t kq_gs_min_m = 1;    // OJAS_HIP_KQ_GS_MIN_M: tokens from which Q6_K / Q5_K rows take the 128-token int8 tile (0: never, 1: by shape)
+    uint32_t kq_gs_min_m = 1;    // OJAS_HIP_KQ_GS_MIN_M: tokens from which Q6_K / Q5_K rows take the 128-row x 64-token int8 tile (0: never, 1: by shape)
     uint32_t q4k_mf_min_m = 5;   // OJAS_HIP_Q4K_MF_MIN_M: tokens from which Q4_K rows go to the int8 matrix cores
     int moe_mode = 0;            // OJAS_HIP_MOE: 0 = by batch size, 1 = matrix cores always, 2 = grouped integer dots always,
                                  // 3 = per-assignment decode form always, 4 = matrix cores in the workgroup-per-tile form always
@@ -126,7 +126,7 @@ struct ojh_block_format {
 const ojh_block_format *ojh_format(uint32_t ggml_type);
 bool ojh_float_rows(uint32_t ggml_type);   // the CPU path reads f32 activations for this format
 size_t ojh_block_align(const ojh_block_format *f);
-uint32_t ojh_gemm_q8k_gs_slices(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M);   // K slices of the Q6_K / Q5_K 128-token tile (1: whole)
+uint32_t ojh_gemm_q8k_gs_slices(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M);   // K slices of the Q6_K / Q5_K int8 tile (1: whole)
 uint32_t ojh_gemm_sr_slices(uint32_t K, uint32_t nsplit);   // K slices of the `_sr` tiles that hold a super-block
 bool ojh_grid_type(uint32_t ggml_type);    // a grid-codebook format: its kernels live in the family "iq_grid"
 bool ojh_float_only(uint32_t ggml_type);   // ... and only the f32-activation matvecs exist for it

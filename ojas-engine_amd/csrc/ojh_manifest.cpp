@@ -382,12 +382,13 @@ static int shape_gemv_q8(const ojh_kernel_spec *s, const ojh_device *dev, uint32
     grid[0] = g ? g : 1;
     return OJH_OK;
 }
-// gemm_q8k_{q6k,q5k}_gs(xq, xs, w, y, K, N, M, ACC): grid [ceil(N / 64), ceil(M / 128), 1] x 256
+// gemm_q8k_{q6k,q5k}_gs(xq, xs, w, y, K, N, M, ACC): grid [ceil(N / 128), ceil(M / 64), 1] x 256
 // gemm_q8k_{q6k,q5k}_gs_sr(xq, xs, w, y, part, cnt, K, N, M, ACC, NSPLIT): grid [.., .., slices]; part: 32 KB per tile
-// and slice; cnt: a zeroed word per tile (`rows_per_wave` = 1 marks the sliced entry)
+// and slice; cnt: a zeroed word per tile (`rows_per_wave` = 1 marks the sliced entries)
 static int check_gemm_q8k_gs(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                              const uint32_t block[3], size_t need[16], size_t align[16]) {
-    const bool sr = s->rows_per_wave == 1;
+    const bool sr = s->rows_per_wave & 1;
+    const uint32_t br = 128, bt = 64;
     const ojh_block_format *f;
     const uint32_t K = c[0], N = c[1], M = c[2], nsplit = sr ? c[4] : 1;
     int rc = check_kn(s, K, N, &f);
@@ -399,8 +400,8 @@ static int check_gemm_q8k_gs(const ojh_kernel_spec *s, const uint32_t *c, const 
     const size_t nsb = K / 256;
     if (!nsplit || nsplit > nsb) return ojh_fail(OJH_ERR_ARG, "%s: NSPLIT=%u (1 .. K/256)", s->name, nsplit);
     const uint32_t slices = sr ? ojh_gemm_sr_slices(K, nsplit) : 1;
-    if (grid[0] != (N + 63) / 64 || grid[1] != (M + 127) / 128 || grid[2] != slices)
-        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, (N + 63) / 64, (M + 127) / 128, slices);
+    if (grid[0] != (N + br - 1) / br || grid[1] != (M + bt - 1) / bt || grid[2] != slices)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, (N + br - 1) / br, (M + bt - 1) / bt, slices);
     need[0] = (size_t)M * K;
     need[1] = (size_t)M * nsb * 4;
     need[2] = (size_t)N * nsb * f->bytes;
@@ -423,7 +424,8 @@ static int check_gemm_q8k_gs(const ojh_kernel_spec *s, const uint32_t *c, const 
 uint32_t ojh_gemm_q8k_gs_slices(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M) {
     const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, nsb = K / 256;
     const uint32_t mode = dev ? dev->kq_gs_split : 1u;
-    const uint64_t tiles = (uint64_t)((N + 63) / 64) * ((M + 127) / 128);
+    const uint32_t br = 128, bt = 64;
+    const uint64_t tiles = (uint64_t)((N + br - 1) / br) * ((M + bt - 1) / bt);
     if (!tiles || mode == 0) return 1;
     uint32_t z = (uint32_t)(2 * (uint64_t)cus / tiles);
     if (z > 8) z = 8;
@@ -435,10 +437,10 @@ uint32_t ojh_gemm_q8k_gs_slices(const ojh_device *dev, uint32_t K, uint32_t N, u
 static int shape_gemm_q8k_gs(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
                              uint32_t grid[3], uint32_t block[3]) {
     if (!M) M = 1;
-    grid[0] = (N + 63) / 64;
+    grid[0] = (N + 127) / 128;
     if (!grid[0]) grid[0] = 1;
-    grid[1] = (M + 127) / 128;
-    grid[2] = s->rows_per_wave == 1 ? ojh_gemm_q8k_gs_slices(dev, K, N, M) : 1;
+    grid[1] = (M + 63) / 64;
+    grid[2] = s->rows_per_wave & 1 ? ojh_gemm_q8k_gs_slices(dev, K, N, M) : 1;
     block[0] = 256;
     block[1] = block[2] = 1;
     return OJH_OK;

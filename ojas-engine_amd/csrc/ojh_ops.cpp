@@ -278,20 +278,22 @@ int ojh_mm_q8k_launch(ojh_device *dev, void *xq, void *xs, const ojh_lin *w, con
     }
     const size_t w_bytes = w->row_bytes * N;
     const bool dwords_ok = (uintptr_t)wp % 4 == 0 && (w_bytes % 4 == 0 || w->off + w_bytes + 2 <= w->raw->bytes);
-    // Q6_K / Q5_K rows against a prefill-sized batch: 64-row x 128-token tiles, one matrix instruction per scale group;
+    // Q6_K / Q5_K rows against a batch: 128-row x 64-token tiles, one matrix instruction per scale group;
     // over K slices where the tiles alone would leave CUs idle (partial tiles in library scratch, added in slice order)
-    // (from where it was measured ahead of launches of 16 tokens, rows streamed from HBM: Q6_K from 33 tokens — 14336 x 4096
-    // at 48 tokens 51 against 60 us, at 128 54 against 152 — and from 17 where K is long, 4096 x 14336: 48 against 49 .. 67;
-    // Q5_K, whose few-token form is the integer-dot kernel, from 17 everywhere and from 9 on large matrices)
+    // (from where it was measured ahead of what it replaces, rows streamed from HBM.  Q6_K: from 17 tokens on large
+    // matrices — 14336 x 4096 at 24 tokens 28.6 against 39 us for two launches of 16, 4096 x 14336 32.6 against 50 — and
+    // from 33 on small ones, where two launches still win (4096 x 4096: 18 against 19.4).  Q5_K, whose few-token form is
+    // the integer-dot kernel: from 5 tokens on large matrices (14336 x 4096 at 8 tokens 25.5 against 31.8), from 9 on
+    // small ones (4096 x 4096 at 12 tokens 17.8 against 20.5).)
+    const bool gs_large = N >= 8192 || K > 8192;
     const uint32_t gs_min = dev->kq_gs_min_m != 1 ? dev->kq_gs_min_m
-                            : w->type == OJH_Q6_K ? (K > 8192 ? 17u : 33u)
-                                                  : (N >= 8192 || K > 8192 ? 9u : 17u);
+                            : w->type == OJH_Q6_K ? (gs_large ? 17u : 33u) : (gs_large ? 5u : 9u);
     if ((w->type == OJH_Q6_K || w->type == OJH_Q5_K) && gs_min && m >= gs_min && K % 256 == 0 &&
         (uintptr_t)xq % 16 == 0 && (w->type == OJH_Q6_K ? dwords_ok : (uintptr_t)wp % 16 == 0)) {
         int rc = ensure(dev, "gemm_q8k");
         if (rc) return rc;
         const std::string gs = std::string("gemm_q8k_") + f->tag + "_gs";
-        uint32_t sg[3] = {(N + 63) / 64, (m + 127) / 128, 1}, sb[3] = {256, 1, 1};
+        uint32_t sg[3] = {(N + 127) / 128, (m + 63) / 64, 1}, sb[3] = {256, 1, 1};
         const uint32_t z = dev->no_scratch ? 1 : ojh_gemm_q8k_gs_slices(dev, K, N, m);
         if (z > 1) {
             const size_t tiles = (size_t)sg[0] * sg[1];

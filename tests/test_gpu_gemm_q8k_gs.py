@@ -1,4 +1,4 @@
-"""Q6_K and Q5_K rows against prefill-sized batches in the CPU path's arithmetic (`gemm_q8k_{q6k,q5k}_gs{,_sr}`):
+"""Q6_K and Q5_K rows against batches of 5 to hundreds of tokens in the CPU path's arithmetic (`gemm_q8k_{q6k,q5k}_gs{,_sr}`):
 every token against matvec_kq (crates/ojas-cpu/src/cpu_math.rs:638-722, :1145-1189), the bar of the few-token kernels."""
 import numpy as np
 import pytest
@@ -21,7 +21,7 @@ def _case(pkg, ty, m, n, k, tag):
 
 
 @pytest.mark.parametrize("ty", [Q6_K, Q5_K])
-@pytest.mark.parametrize("m,n,k", [(17, 100, 512), (128, 64, 256), (130, 77, 2048), (300, 1000, 1024)])
+@pytest.mark.parametrize("m,n,k", [(17, 100, 512), (128, 64, 256), (130, 77, 2048), (300, 1000, 1024), (33, 130, 768)])
 def test_tiles_by_name(gpu, orc, pkg, ty, m, n, k):
     """Ragged tokens and rows, plain store and accumulate, nothing written past row M; K slices: one slice gives the
     unsliced bits, more give the same bits on every launch and leave the tile counters at zero."""
@@ -34,7 +34,7 @@ def test_tiles_by_name(gpu, orc, pkg, ty, m, n, k):
     wd = gpu.upload_bytes(w)
     want = np.stack([orc.matvec_kq(w, ty, n, k, x[t]) for t in range(m)])
     name = f"gemm_q8k_{FMT[ty]}_gs"
-    grid = [(n + 63) // 64, (m + 127) // 128, 1]
+    grid = [(n + 127) // 128, (m + 63) // 64, 1]
     plain = None
     for acc in (0, 1):
         y0 = pkg.synth.normal_f32(m * n, "gs", "y0", acc).reshape(m, n)
