@@ -580,7 +580,15 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     // Q5_K: the CPU path's arithmetic (dot_q5k over int8 activations) unless floating-point activations are
     // asked for, which run on the f32-activation matvecs; from the tile crossover both that request and
     // OJH_ACT_AUTO take the f16 tile (dequant_to_f16 bits), as Q6_K and Q8_0 do.
-    const bool q5_tile = w->type == OJH_Q5_K && act_mode != OJH_ACT_Q8K && m >= dev->gemm_min_m && K % 64 == 0 &&
+    // Where OJH_ACT_AUTO hands over from the int8 kernels to the f16 tile: 32 tokens (OJAS_HIP_GEMM_MIN_M); for Q6_K and
+    // Q5_K rows later — their int8 tile is ahead of their f16 tile up to 128 / 64 tokens (measured, 14336 x 4096 at 64
+    // tokens: Q6_K 34.5 against 45.9 us, Q5_K 31.9 against 38.7; a 151936-row head at 32 tokens 164 against 341).
+    uint32_t tile_min = dev->gemm_min_m;
+    if (act_mode == OJH_ACT_AUTO && dev->kq_gs_min_m && K % 256 == 0 && (w->type == OJH_Q6_K || w->type == OJH_Q5_K)) {
+        const uint32_t later = w->type == OJH_Q6_K ? 129u : 65u;
+        if (tile_min < later) tile_min = later;
+    }
+    const bool q5_tile = w->type == OJH_Q5_K && act_mode != OJH_ACT_Q8K && m >= tile_min && K % 64 == 0 &&
                          (uint64_t)m * K < 0x7FFFFFFFull && (uint64_t)m * N < 0x7FFFFFFFull;
     const bool q5_float = w->type == OJH_Q5_K && !q5_tile && (act_mode == OJH_ACT_FLOAT || act_mode == OJH_ACT_FLOAT_EXACT);
     if (w->type == OJH_Q5_K && !q5_float && !q5_tile) act_mode = OJH_ACT_Q8K;
@@ -598,7 +606,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     // (the reference switches at 8 rows, crates/ojas-models/src/decoder/dispatch.rs:70-75).
     if (grid_fmt && !iq4 && act_mode == OJH_ACT_AUTO) act_mode = OJH_ACT_Q8K;
     if (grid_fmt && (rc = ensure(dev, "iq_grid"))) return rc;
-    if (m >= dev->gemm_min_m && act_mode != OJH_ACT_Q8K && !iq4 && !grid_fmt && K % 64 == 0 && (uint64_t)m * K < 0x7FFFFFFFull &&
+    if (m >= tile_min && act_mode != OJH_ACT_Q8K && !iq4 && !grid_fmt && K % 64 == 0 && (uint64_t)m * K < 0x7FFFFFFFull &&
         (uint64_t)m * N < 0x7FFFFFFFull) {
         // Q4_K takes the 256-wide tile with the reference GPU kernel's arithmetic (f16 qa*q + qb)
         // unless the tile that reproduces dequant_to_f16 bit for bit is asked for.

@@ -416,22 +416,23 @@ def test_q6k_few_tokens_staged_and_streamed_forms_agree(gpu, orc, pkg, m, n, k, 
 
 def test_q5k_takes_the_int8_path_below_the_tile_crossover(gpu, orc, pkg):
     """Q5_K defaults to dot_q5k's arithmetic (crates/ojas-cpu/src/cpu_math.rs:638-670): AUTO resolves to it below the
-    crossover to the f16 tile (32 tokens), OJH_ACT_Q8K at every token count; a floating-point contract runs the
-    f32-activation matvecs below the crossover and the f16 tile from there, as AUTO does (the dequantized dot in f64
-    is the judge; the tile rounds the activations to f16); the wide-row form (N >= 32768) agrees with the oracle too."""
+    crossover to the f16 tile (for Q5_K 65 tokens: its int8 tile is the faster one up to 64), OJH_ACT_Q8K at every token
+    count; a floating-point contract runs the f32-activation matvecs below 32 tokens and the f16 tile from there (the
+    dequantized dot in f64 is the judge; the tile rounds the activations to f16); the wide-row form (N >= 32768) agrees
+    with the oracle too."""
     n, k = 300, 1024
     w = pkg.synth.weights(Q5_K, n, k, "q5k", "any-m")
     lin = gpu.lin(Q5_K, n, k, w)
-    for m, act in ((1, pkg.ACT_AUTO), (9, pkg.ACT_AUTO), (24, pkg.ACT_AUTO), (40, pkg.ACT_Q8K), (200, pkg.ACT_Q8K)):
+    for m, act in ((1, pkg.ACT_AUTO), (9, pkg.ACT_AUTO), (24, pkg.ACT_AUTO), (40, pkg.ACT_AUTO), (64, pkg.ACT_AUTO), (200, pkg.ACT_Q8K)):
         xs = pkg.synth.normal_f32(m * k, "q5k", "x", m).reshape(m, k)
         yd = gpu.alloc(m * n)
         gpu.mm(gpu.upload(xs), lin, yd, m, act_mode=act)
         want = np.stack([orc.matvec_kq(w, Q5_K, n, k, xs[t]) for t in range(m)])
         assert peak_err(gpu.read(yd, m * n).reshape(m, n), want) <= TOL_Q8K_SEEN
-    for m in (24, 40):
+    for m in (24, 40, 80):
         xs = pkg.synth.normal_f32(m * k, "q5k", "x", m).reshape(m, k)
         yd = gpu.alloc(m * n)
-        for act in (pkg.ACT_FLOAT, pkg.ACT_FLOAT_EXACT) + ((pkg.ACT_AUTO,) if m >= 32 else ()):
+        for act in (pkg.ACT_FLOAT, pkg.ACT_FLOAT_EXACT) + ((pkg.ACT_AUTO,) if m >= 65 else ()):
             gpu.mm(gpu.upload(xs), lin, yd, m, act_mode=act)
             got = gpu.read(yd, m * n).reshape(m, n)
             assert peak_err(got, orc.matmul_ref(w, Q5_K, n, k, xs)) <= (2e-3 if m >= 32 else TOL_FLOAT)
