@@ -588,6 +588,14 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         const uint32_t later = w->type == OJH_Q6_K ? 129u : 65u;
         if (tile_min < later) tile_min = later;
     }
+    // Q8_0 rows have no few-token kernel on the matrix cores: their f32-activation matvec walks the rows once per token
+    // (14336 x 4096 at 8 tokens 84 us, a 128256-row head 810), and the 128-token f16 tile — the contract the reference's
+    // own GPU path switches to from 8 rows (crates/ojas-models/src/decoder/dispatch.rs:70-75) — takes 38 and 251: under
+    // OJH_ACT_AUTO from 4 tokens on large matrices, 6 on small ones (4096 x 4096: 12.3 against 17.0 at 4, 21.4 at 8).
+    if (act_mode == OJH_ACT_AUTO && w->type == OJH_Q8_0 && dev->q80_tile_min_m) {
+        const uint32_t early = dev->q80_tile_min_m != 1 ? dev->q80_tile_min_m : (uint64_t)N * K >= (32ull << 20) ? 4u : 6u;
+        if (tile_min > early) tile_min = early;
+    }
     const bool q5_tile = w->type == OJH_Q5_K && act_mode != OJH_ACT_Q8K && m >= tile_min && K % 64 == 0 &&
                          (uint64_t)m * K < 0x7FFFFFFFull && (uint64_t)m * N < 0x7FFFFFFFull;
     const bool q5_float = w->type == OJH_Q5_K && !q5_tile && (act_mode == OJH_ACT_FLOAT || act_mode == OJH_ACT_FLOAT_EXACT);
