@@ -46,7 +46,7 @@ enum {
 };
 
 /* GGUF tensor types handled by this path (crates/ojas-formats/src/gguf.rs:563-591). */
-enum { OJH_Q4_0 = 2, OJH_Q4_1 = 3, OJH_Q5_0 = 6, OJH_Q5_1 = 7, OJH_Q8_0 = 8, OJH_Q2_K = 10, OJH_Q3_K = 11, OJH_Q4_K = 12, OJH_Q5_K = 13, OJH_Q6_K = 14,
+enum { OJH_F16 = 1 /* plain f16 rows: the `gemm_mm_f16*` entries only (ojh_lin_create does not take it) */, OJH_Q4_0 = 2, OJH_Q4_1 = 3, OJH_Q5_0 = 6, OJH_Q5_1 = 7, OJH_Q8_0 = 8, OJH_Q2_K = 10, OJH_Q3_K = 11, OJH_Q4_K = 12, OJH_Q5_K = 13, OJH_Q6_K = 14,
        OJH_IQ4_NL = 20, OJH_IQ4_XS = 23,
        /* the grid-codebook formats (gguf.rs:840-1041): decoders and f32-activation matvecs for all seven; IQ2_XXS and
         * IQ3_XXS also on int8 activations, which is what matvec_kq runs for them (cpu_math.rs:1177-1178) */

@@ -263,6 +263,29 @@ struct LoaderQ80 {
     }
 };
 
+// Plain f16 rows [N][K] (a tensor the caller keeps in f16, or any block format decoded into scratch by its
+// `dequant_<fmt>_f16` kernel ahead of the product): thread half h owns columns 32h..32h+31 of the slab, 64 bytes.
+struct LoaderF16 {
+    static constexpr int NL = 4;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
+    u32x4 q[4];
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)K * 2u; }
+    __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
+        const uchar* p = row + (size_t)(k0 + 32u * h) * 2u;
+#pragma unroll
+        for (int i = 0; i < 4; i++) q[i] = *(const u32x4*)(p + 16 * i);
+    }
+    __device__ __forceinline__ void prep() {}
+    template <int I>
+    __device__ __forceinline__ void part() {}
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* o = (u32x4*)(lds_row + h * 64u);
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = q[i];
+    }
+};
+
 // Q4L: Q4_K relaid by `relayout_q4k_q4l` (crates/ojas-formats/src/quant.rs:192-222) — nibbles w4[N][K/2], byte i of a
 // 32-weight block = weights 2i (low nibble) and 2i+1 (high), and per block the f16 pair qa = d*sc, qb = -dmin*m.  Every
 // weight enters the tile as the binary16 fma qa*q + qb, the arithmetic of the reference's `gemm_mm_q4l`
@@ -500,6 +523,7 @@ GEMM_ENTRIES(q4k, LoaderQ4K)
 GEMM_ENTRIES(q5k, LoaderQ5K)
 GEMM_ENTRIES(q6k, LoaderQ6K)
 GEMM_ENTRIES(q8_0, LoaderQ80)
+GEMM_ENTRIES(f16, LoaderF16)
 
 // The reference's entries for Q4L weights, under their names and argument lists
 // (crates/ojas-cuda/src/kernels/gemm_q.rs:26-38, :505-542; dispatched by `CudaSsm::mm`, crates/ojas-cuda/src/qwen35.rs:683,690):

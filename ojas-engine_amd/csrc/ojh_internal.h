@@ -74,6 +74,7 @@ struct ojh_device {
     uint32_t q4k_xt_min_m = 1;   // OJAS_HIP_Q4K_XT_MIN_M: tokens from which Q4_K rows take the 128-token int8 tile (0: never, 1: by shape)
     bool q4k_xt64 = false;       // OJAS_HIP_Q4K_XT64=1: that tile always in its 64-row form
     bool no_scratch = false;     // set around calls that may not allocate (ojh_mm_noalloc): paths that need library scratch are skipped
+    uint32_t deq_min_m = 1;      // OJAS_HIP_DEQ_MIN_M: tokens from which a format without a tile of its own is decoded into scratch and multiplied on the f16 tile (0: never, 1: by format, n: n)
     uint32_t q80_tile_min_m = 1; // OJAS_HIP_Q80_TILE_MIN_M: tokens from which OJH_ACT_AUTO sends Q8_0 rows to the f16 tile (0: GEMM_MIN_M, 1: by shape, n: n)
     int gemm_m128 = 128;         // OJAS_HIP_GEMM_M128: tokens up to which Q5_K / Q6_K / Q8_0 batches take the 128-token f16 tile (0: never)
     uint32_t kq_gs_split = 1;    // OJAS_HIP_KQ_GS_SPLIT: K slices of that tile (0: never, 1: chosen, n: n)

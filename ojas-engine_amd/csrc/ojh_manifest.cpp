@@ -1109,7 +1109,14 @@ static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_
     uint32_t bm, bn;
     gemm_tile(s, &bm, &bn, &sk);
     uint32_t K = c[0], N = c[1], M = sk ? c[2] : c[3], nsplit = sk ? c[3] : 1;
-    int rc = check_kn(s, K, N, &f);
+    static const ojh_block_format plain_f16 = {OJH_F16, 2, 1, "f16"};   // (rows of plain f16: the `gemm_mm_f16*` entries)
+    int rc = OJH_OK;
+    if (s->type == OJH_F16) {
+        f = &plain_f16;
+        if (!K || !N) rc = ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u", s->name, K, N);
+    } else {
+        rc = check_kn(s, K, N, &f);
+    }
     if (rc) return rc;
     if (K % 64) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a multiple of 64", s->name, K);
     if (M == 0 || nsplit == 0) return ojh_fail(OJH_ERR_ARG, "%s: M and nsplit must be positive", s->name);
@@ -1124,7 +1131,7 @@ static int check_gemm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_
     need[0] = (size_t)M * K * 2;
     need[1] = (size_t)N * (K / f->weights) * f->bytes;
     need[2] = (size_t)M * N * 4;
-    align[1] = ojh_block_align(f);
+    align[1] = s->type == OJH_F16 ? 16 : ojh_block_align(f);
     align[2] = 4;
     return OJH_OK;
 }
@@ -1811,6 +1818,11 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g + "_m128", "gemm", 3, 4, f.type, 14, check_gemm, shape_gemm);
         add(g + "_m128_sk", "gemm", 3, 4, f.type, 15, check_gemm, shape_gemm);
     }
+    // plain f16 rows on the same tile: what every format without a tile of its own is decoded into ahead of a batch
+    add("gemm_mm_f16", "gemm", 3, 4, OJH_F16, 0, check_gemm, shape_gemm);
+    add("gemm_mm_f16_sk", "gemm", 3, 4, OJH_F16, 1, check_gemm, shape_gemm);
+    add("gemm_mm_f16_m128", "gemm", 3, 4, OJH_F16, 14, check_gemm, shape_gemm);
+    add("gemm_mm_f16_m128_sk", "gemm", 3, 4, OJH_F16, 15, check_gemm, shape_gemm);
     // Q4L (relaid Q4_K + side arrays) under the reference's names and argument lists
     add("gemm_mm_q4l", "gemm", 5, 4, 0, 8, check_gemm_q4l, shape_gemm);
     add("gemm_mm_q4l_sk", "gemm", 5, 4, 0, 9, check_gemm_q4l, shape_gemm);

@@ -612,10 +612,33 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
 
     // Above the crossover the MFMA tile wins over streaming the weights once per few tokens
     // (the reference switches at 8 rows, crates/ojas-models/src/decoder/dispatch.rs:70-75).
+    const int act_asked = act_mode;
     if (grid_fmt && !iq4 && act_mode == OJH_ACT_AUTO) act_mode = OJH_ACT_Q8K;
     if (grid_fmt && (rc = ensure(dev, "iq_grid"))) return rc;
-    if (m >= tile_min && act_mode != OJH_ACT_Q8K && !iq4 && !grid_fmt && K % 64 == 0 && (uint64_t)m * K < 0x7FFFFFFFull &&
-        (uint64_t)m * N < 0x7FFFFFFFull) {
+    // Formats without a tile of their own (the IQ4 types, the legacy 32-weight blocks, Q2_K / Q3_K, MXFP4, the grid
+    // codebooks) against a batch: their matvec walks the rows once per token (14336 x 4096: 8 us a token, 1 ms at 128
+    // tokens).  From `deq_min_m` tokens the rows are decoded once into library scratch (`dequant_<fmt>_f16`:
+    // dequant_to_f16's bits) and the batch runs on the f16 tile — what the reference does at load time for every
+    // tensor it cannot keep in place (crates/ojas-cuda/src/qwen35.rs:174-201), without holding the f16 copy.
+    // (from where the decode pass plus the tile beat the per-token walk: 8 tokens for the grid codebooks, whose decoders
+    // are the quick ones — 52 us in all on 14336 x 4096 —, 14 for the others — 95 to 130 us)
+    const uint32_t deq_min = dev->deq_min_m != 1 ? dev->deq_min_m : grid_fmt ? 8u : 14u;
+    const bool deq_tile = (iq4 || grid_fmt) && !q5_float && act_asked != OJH_ACT_Q8K && deq_min && m >= deq_min &&
+                          !dev->no_scratch && K % 64 == 0 && (uint64_t)N * K / f->weights <= 0x7FFFFFFFu / 64;
+    void *tile_w = wp;
+    if (deq_tile) {
+        ojh_buf *wdeq;
+        if ((rc = ojh_scratch_get(dev, "wdeq", (size_t)N * K * 2, &wdeq))) return rc;
+        if ((rc = ensure(dev, grid_fmt ? "iq_grid" : "dequant"))) return rc;
+        const std::string dq = std::string("dequant_") + f->tag + "_f16";
+        const uint32_t nb = (uint32_t)((uint64_t)N * K / f->weights);
+        uint32_t dg[3], db[3];
+        if ((rc = ojh_launch_shape(dev, dq.c_str(), 0, nb, 0, dg, db))) return rc;
+        if ((rc = ojh_launch(dev, dq.c_str(), {wp, wdeq->ptr}, {nb}, dg, db))) return rc;
+        tile_w = wdeq->ptr;
+    }
+    if ((deq_tile || (m >= tile_min && act_mode != OJH_ACT_Q8K && !iq4 && !grid_fmt)) && K % 64 == 0 &&
+        (uint64_t)m * K < 0x7FFFFFFFull && (uint64_t)m * N < 0x7FFFFFFFull) {
         // Q4_K takes the 256-wide tile with the reference GPU kernel's arithmetic (f16 qa*q + qb)
         // unless the tile that reproduces dequant_to_f16 bit for bit is asked for.
         const bool xl = w->type == OJH_Q4_K && !dev->gemm_exact && act_mode != OJH_ACT_FLOAT_EXACT &&
@@ -624,7 +647,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         ojh_buf *xh;
         if ((rc = ojh_scratch_get(dev, "xh", (size_t)m * K * 2, &xh))) return rc;
         const uint32_t n_el = m * K, conv_blocks = (n_el / 8 + 255) / 256 + 1;
-        std::string base = std::string("gemm_mm_") + (w->type == OJH_Q8_0 ? "q8_0" : f->tag);
+        std::string base = std::string("gemm_mm_") + (deq_tile ? "f16" : w->type == OJH_Q8_0 ? "q8_0" : f->tag);
         // (the tile that shares the dequantized weights through LDS is 256 tokens tall; up to 128 tokens its 128-token form)
         if (!xl && m <= (uint32_t)dev->gemm_m128) base += "_m128";
         if (xl) {
@@ -693,9 +716,9 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
                                  {n_el}, eg, block)))
                 return rc;
         }
-        if (sg[2] > 1) return ojh_launch(dev, (base + "_sk").c_str(), {xh->ptr, wp, yp}, {K, N, m, sg[2]}, sg, sb);
+        if (sg[2] > 1) return ojh_launch(dev, (base + "_sk").c_str(), {xh->ptr, tile_w, yp}, {K, N, m, sg[2]}, sg, sb);
         sg[2] = 1;
-        return ojh_launch(dev, base.c_str(), {xh->ptr, wp, yp}, {K, N, (uint32_t)(accum != 0), m}, sg, sb);
+        return ojh_launch(dev, base.c_str(), {xh->ptr, tile_w, yp}, {K, N, (uint32_t)(accum != 0), m}, sg, sb);
     }
 
     bool q8k = !ojh_float_rows(w->type) && act_mode != OJH_ACT_FLOAT && act_mode != OJH_ACT_FLOAT_EXACT;

@@ -92,6 +92,7 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_KQ_GS_MIN_M")) d->kq_gs_min_m = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_GEMM_M128")) d->gemm_m128 = atoi(r);
     if (const char *r = getenv("OJAS_HIP_Q80_TILE_MIN_M")) d->q80_tile_min_m = (uint32_t)atoi(r);
+    if (const char *r = getenv("OJAS_HIP_DEQ_MIN_M")) d->deq_min_m = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_KQ_GS_SPLIT")) d->kq_gs_split = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE")) d->moe_mode = atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE_DEC_TOKENS")) d->moe_dec_tokens = (uint32_t)atoi(r);

@@ -295,3 +295,34 @@ def test_router_prefers_the_tile_only_above_the_crossover(gpu, orc, pkg):
         else:
             e = rms_errs(got, orc.matmul_ref(w, Q4_K, n, k, x, wmode=2, xmode=1))
             assert e[0] < TIGHT[0] and e[1] < TIGHT[1], e
+
+
+@pytest.mark.parametrize("ty", ["iq4xs", "iq4nl", "q40", "q51", "q2k", "q3k", "mxfp4", "iq2xxs", "iq2s", "iq3s", "iq1m"])
+@pytest.mark.parametrize("m,k,n,accum", [(40, 1024, 200, False), (300, 2048, 130, True)])
+def test_formats_without_a_tile_are_decoded_into_scratch_for_a_batch(gpu, orc, pkg, ty, m, k, n, accum):
+    """A batch on a format that has only matvecs: `ojh_mm` decodes the rows once (`dequant_<fmt>_f16`, dequant_to_f16's
+    bits) into library scratch and runs the f16 tile — the contract of the Q6_K / Q8_0 tiles: activations rounded to
+    f16, f32 accumulation, held to the tile's own bound against the rounded oracle and to the reference's bound against
+    the unrounded one.  Below the crossover the per-token matvec still answers (f32 activations, the dequantized dot)."""
+    S = pkg.synth
+    types = {"iq4xs": S.IQ4_XS, "iq4nl": S.IQ4_NL, "q40": S.Q4_0, "q51": S.Q5_1, "q2k": S.Q2_K, "q3k": S.Q3_K, "mxfp4": pkg.MXFP4,
+             "iq2xxs": S.IQ2_XXS, "iq2s": S.IQ2_S, "iq3s": S.IQ3_S, "iq1m": S.IQ1_M}
+    t = types[ty]
+    w = S.mxfp4_weights(n, k, "deq", ty) if ty == "mxfp4" else S.grid_weights(t, n, k, "deq", ty) if t in S.GRID_TYPES else S.weights(t, n, k, "deq", ty)
+    x = S.normal_f32(m * k, "deq", "x", m, k).reshape(m, k)
+    y0 = S.normal_f32(m * n, "deq", "y0").reshape(m, n) if accum else np.zeros((m, n), np.float32)
+    yd = gpu.upload(np.concatenate([y0.ravel(), np.full(n, 12345.5, np.float32)]))
+    lin = gpu.lin(t, n, k, w)
+    gpu.mm(gpu.upload(x), lin, yd, m, accum)
+    got = gpu.read(yd, m * n + n)
+    assert np.all(got[m * n:] == 12345.5), "wrote past row M"
+    got = got[:m * n].reshape(m, n)
+    e16 = rms_errs(got, orc.matmul_ref(w, t, n, k, x, wmode=1, xmode=1) + y0)
+    e32 = rms_errs(got, orc.matmul_ref(w, t, n, k, x) + y0)
+    assert e16[0] < TIGHT[0] and e16[1] < TIGHT[1], e16
+    assert e32[0] < 2e-2 and e32[1] < 3e-3, e32
+    # four tokens: the matvec path, within its own (tighter) bound of the same oracle
+    y4 = gpu.alloc(4 * n)
+    gpu.mm(gpu.upload(x[:4].copy()), lin, y4, 4, act_mode=pkg.ACT_FLOAT)
+    assert peak_err(gpu.read(y4, 4 * n).reshape(4, n), orc.matmul_ref(w, t, n, k, x[:4])) <= 1e-5
+    lin.free()

@@ -137,12 +137,13 @@ def test_f32_rows_match_the_cpu_dots(gpu, orc, pkg, ty, n, k, m):
 @pytest.mark.parametrize("n,k,m", [(4096, 4096, 1), (37, 256, 1), (130, 2816, 5), (33001, 2816, 1), (777, 14336, 2), (64, 1024, 40)])
 def test_int8_rows_match_the_cpu_dots(gpu, orc, pkg, ty, n, k, m):
     """IQ2_XXS / IQ3_XXS: `matvec_kq` quantizes the activations per 256 and runs dot_iq2xxs_q8k / dot_iq3xxs_q8k —
-    what `mm` does unless f32 activations are asked for, which give dot_iq2xxs / dot_iq3xxs (dot_iq)."""
+    what `mm` does for a few tokens unless f32 activations are asked for, which give dot_iq2xxs / dot_iq3xxs (dot_iq);
+    from 8 tokens OJH_ACT_AUTO decodes the rows for the f16 tile, and the int8 kernels answer to OJH_ACT_Q8K."""
     w = pkg.synth.weights(ty, n, k, "gridq", n, k)
     x = pkg.synth.normal_f32(m * k, "gridq", "x", ty, m, k).reshape(m, k)
     lin = gpu.lin(ty, n, k, w)
     yd = gpu.upload(np.full(m * n + 2, 12345.0, np.float32))
-    gpu.mm(gpu.upload(x), lin, yd, m, y_off=4)
+    gpu.mm(gpu.upload(x), lin, yd, m, y_off=4, act_mode=pkg.ACT_Q8K if m >= 8 else pkg.ACT_AUTO)
     got = gpu.read(yd, m * n + 2)
     assert got[0] == 12345.0 and got[-1] == 12345.0, "wrote outside y"
     for t in sorted({0, m // 2, m - 1}):

@@ -50,13 +50,18 @@ def test_router_sweep(gpu, orc, pkg, ty, n, k, m, accum):
     # Q8_0 under OJH_ACT_AUTO from 4 tokens (6 on matrices below 32 Mi weights): the f16 MFMA tile, activations rounded
     # to f16 (its own contract, the one the reference's GPU path switches to from 8 rows)
     tile = ty == Q8_0 and m >= (4 if n * k >= (32 << 20) else 6)
+    # formats with matvecs only: from 8 (grid codebooks) / 14 tokens decoded into scratch and run on the f16 tile
+    # (IQ2_XXS / IQ3_XXS keep the int8 kernels where OJH_ACT_Q8K is asked for: here from 32 tokens)
+    grid = ty in (IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M)
+    if ty not in (Q8_0, Q4_K, Q5_K, Q6_K) and k % 64 == 0 and m >= (8 if grid else 14) and (m < 32 or ty in FLOAT_ROWS):
+        tile = True
     if tile:
         tol = 2e-3
     scale = 1.0 + (float(np.max(np.abs(y0))) if accum else 0.0)   # accumulating onto y0 rounds at y0's magnitude
     for t in sorted({0, m // 2, m - 1}):
         # (the CPU path has no dot for the legacy blocks: the reference runs them on its GPU path, f32
         # activations against the dequantized weights, which is what the f64 reference evaluates)
-        want = orc.matmul_ref(w, ty, n, k, x[t])[0] if ty in LEGACY else orc.matvec_kq(w, ty, n, k, x[t])
+        want = orc.matmul_ref(w, ty, n, k, x[t])[0] if ty in LEGACY or (tile and ty != Q8_0) else orc.matvec_kq(w, ty, n, k, x[t])
         assert peak_err(got[t], want) <= tol * max(1.0, scale * 4.0 / max(1e-30, float(np.max(np.abs(want))))), (t,)
     if m > 1 and not accum and not tile:
         # the middle token alone: the one-token kernels associate their f32 sums differently (last ulps)
