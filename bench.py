@@ -501,6 +501,22 @@ def extras(gpu, pkg, lin_q) -> dict:
         rq[name] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
         del ws
     out["rowq8_gemv_q8"] = {"what": "y[n] = scale[n] * sum_k w[n][k] x[k], w int8 rows streamed from HBM (rotating copies)", **rq}
+    # ---- the CPU models' row-int8 matmul (per-token int8 activations, integer dots): 1 .. 8 tokens stream the rows
+    # against tokens staged in LDS, batches run on the int8 matrix instruction; the quantizer's launch is in the time
+    rm = {}
+    n, copies = 14336, 4
+    ws = [gpu.upload_bytes(rng8.integers(-127, 128, n * k, dtype=np.int8).view(np.uint8)) for _ in range(copies)]
+    sc = gpu.upload(np.full(n, 0.01, np.float32))
+    for m in (1, 8, 64, 512, 2048):
+        xm, ym = gpu.upload(synth.normal_f32(m * k, "bench", "rowq8x", m)), gpu.alloc(m * n)
+        us = _time(gpu, lambda i: gpu.matmul_q8(xm, ws[i % copies], sc, ym, n, k, m), 16, 3)
+        b = n * k + 4 * m * k + 4 * m * n + 8 * n
+        rm["M%d" % m] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "int8_tops": round(2.0 * m * n * k / us / 1e6, 1),
+                         "mfma_frac": round(2.0 * m * n * k / us / 1e6 / 5000.0, 4)}
+        del xm, ym
+    del ws
+    out["rowq8_matmul_14336x4096"] = {"what": "ojh_matmul_q8: quant_rows_i8 + matmul_q8row_{dec,mt_sr,mt,mt128}; int8 rows streamed from HBM (rotating copies)", **rm}
+    n = 128256
     # ---- the other block formats on f32 activations (the reference GPU path's contract): a tall head, one token
     fr = {}
     for ty, tag in ((pkg.IQ4_XS, "iq4xs"), (pkg.IQ4_NL, "iq4nl"), (pkg.Q3_K, "q3k"), (pkg.Q2_K, "q2k"), (pkg.Q5_0, "q50"),

@@ -74,6 +74,10 @@ struct ojh_device {
     uint32_t q4k_xt_min_m = 1;   // OJAS_HIP_Q4K_XT_MIN_M: tokens from which Q4_K rows take the 128-token int8 tile (0: never, 1: by shape)
     bool q4k_xt64 = false;       // OJAS_HIP_Q4K_XT64=1: that tile always in its 64-row form
     bool no_scratch = false;     // set around calls that may not allocate (ojh_mm_noalloc): paths that need library scratch are skipped
+    uint32_t q8row_mt_min_m = 1; // OJAS_HIP_Q8ROW_MT_MIN_M: tokens from which ojh_matmul_q8 takes the int8 matrix tile (0: never, 1: measured default, n: n)
+    bool q8row_dec = true;       // OJAS_HIP_Q8ROW_DEC=0: 1 to 8 tokens on the per-row kernel instead of the one that stages the tokens in LDS
+    uint32_t q8row_t128_min_m = 1; // OJAS_HIP_Q8ROW_T128_MIN_M: tokens from which that tile covers 128 tokens (0: never, 1: measured default, n: n)
+    uint32_t q8row_split = 1;    // OJAS_HIP_Q8ROW_SPLIT: K slices of that tile (0: never, 1: by shape, n: n)
     uint32_t deq_min_m = 1;      // OJAS_HIP_DEQ_MIN_M: tokens from which a format without a tile of its own is decoded into scratch and multiplied on the f16 tile (0: never, 1: by format, n: n)
     uint32_t q80_tile_min_m = 1; // OJAS_HIP_Q80_TILE_MIN_M: tokens from which OJH_ACT_AUTO sends Q8_0 rows to the f16 tile (0: GEMM_MIN_M, 1: by shape, n: n)
     int gemm_m128 = 128;         // OJAS_HIP_GEMM_M128: tokens up to which Q5_K / Q6_K / Q8_0 batches take the 128-token f16 tile (0: never)
@@ -128,6 +132,7 @@ struct ojh_block_format {
 const ojh_block_format *ojh_format(uint32_t ggml_type);
 bool ojh_float_rows(uint32_t ggml_type);   // the CPU path reads f32 activations for this format
 size_t ojh_block_align(const ojh_block_format *f);
+uint32_t ojh_matmul_q8row_slices(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M);  // K slices of the row-int8 tile (1: whole)
 uint32_t ojh_gemm_q8k_gs_slices(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M);   // K slices of the Q6_K / Q5_K int8 tile (1: whole)
 uint32_t ojh_gemm_sr_slices(uint32_t K, uint32_t nsplit);   // K slices of the `_sr` tiles that hold a super-block
 bool ojh_grid_type(uint32_t ggml_type);    // a grid-codebook format: its kernels live in the family "iq_grid"

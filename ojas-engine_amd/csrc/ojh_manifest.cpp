@@ -917,13 +917,72 @@ static int check_quantize(const ojh_kernel_spec *s, const uint32_t *c, const uin
 // The row-int8 family; `rows_per_wave` selects the entry:
 //   0 rows_q8_from_f16(w16, q, scale, K, N)   1 quant_rows_i8(x, q, scale, K, M)       grid [rows,1,1]
 //   2 matmul_q8row(xq, sx, wq, sw, y, K, N, M)   3 matmul_q8row_bias(.., y, bs, K, N, M)  grid [ceil(N/4),1,1]
+//   4 matmul_q8row_mt(xq, sx, wq, sw, y, bs, K, N, M)                                   grid [ceil(N/128),ceil(M/64),1]
+//   5 matmul_q8row_mt_sr(xq, sx, wq, sw, y, bs, part, cnt, K, N, M, NSPLIT)             grid [.., .., slices]
+//   6 matmul_q8row_mt128(xq, sx, wq, sw, y, bs, K, N, M)                                grid [ceil(N/128),ceil(M/128),1]
+//   7 matmul_q8row_dec(xq, sx, wq, sw, y, bs, K, N, M)     M <= 8, M K <= 64 KB          grid [x,1,1] (rows grid-stride),
+//   8 matmul_q8row_dec_l(..)                               M <= 8, M K <= 128 KB         block 64 .. 1024 in whole waves
+//     (bs may be NULL; part: tiles x slices x 32 KB; cnt: a zeroed uint per tile)
 static int check_rowq8(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                        const uint32_t block[3], size_t need[16], size_t align[16]) {
-    int rc = check_block(block, 256);
-    if (rc) return rc;
-    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
     uint32_t K = c[0], R = c[1];
     if (!K || !R) return ojh_fail(OJH_ERR_ARG, "%s: K and the row count must be positive", s->name);
+    if (s->rows_per_wave >= 7) {
+        const uint32_t N = R, M = c[2];
+        const size_t lds = s->rows_per_wave == 7 ? 65536 : 131072;
+        if (grid[1] != 1 || grid[2] != 1 || !grid[0]) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+        if (block[1] != 1 || block[2] != 1 || !block[0] || block[0] % 64 || block[0] > 1024)
+            return ojh_fail(OJH_ERR_ARG, "%s: block must be [64 .. 1024 in whole waves,1,1]", s->name);
+        if (!M || M > 8 || K % 16) return ojh_fail(OJH_ERR_ARG, "%s: M=%u (1 .. 8), K=%u a multiple of 16", s->name, M, K);
+        if ((size_t)M * K > lds) return ojh_fail(OJH_ERR_ARG, "%s: M K = %zu exceeds the %zu bytes staged", s->name, (size_t)M * K, lds);
+        need[0] = (size_t)M * K;
+        need[1] = (size_t)M * 4;
+        need[2] = (size_t)N * K;
+        need[3] = (size_t)N * 4;
+        need[4] = (size_t)M * N * 4;
+        need[5] = (size_t)N * 4;
+        align[0] = align[2] = 16;
+        align[1] = align[3] = align[4] = 4;
+        align[5] = 0;                               // 0: the buffer may be NULL (4-byte aligned when given)
+        return OJH_OK;
+    }
+    int rc = OJH_OK;
+    if (s->rows_per_wave == 1) {
+        if (block[1] != 1 || block[2] != 1 || !block[0] || block[0] % 64 || block[0] > 1024)
+            return ojh_fail(OJH_ERR_ARG, "%s: block must be [64 .. 1024 in whole waves,1,1]", s->name);
+    } else if ((rc = check_block(block, 256))) {
+        return rc;
+    }
+    if (s->rows_per_wave >= 4) {
+        const uint32_t N = R, M = c[2];
+        if (!M || K % 16) return ojh_fail(OJH_ERR_ARG, "%s: M must be positive and K=%u a multiple of 16", s->name, K);
+        const bool sr = s->rows_per_wave == 5;
+        const uint32_t nks = (K + 127) / 128, nsplit = sr ? c[3] : 1;
+        if (!nsplit || nsplit > nks) return ojh_fail(OJH_ERR_ARG, "%s: NSPLIT=%u of %u steps of 128", s->name, nsplit, nks);
+        const uint32_t per = (nks + nsplit - 1) / nsplit, slices = (nks + per - 1) / per;
+        const uint32_t bt = s->rows_per_wave == 6 ? 128 : 64;
+        const uint32_t gx = (N + 127) / 128, gy = (M + bt - 1) / bt;
+        if (gy > 65535) return ojh_fail(OJH_ERR_ARG, "%s: M=%u gives more than 65535 token tiles", s->name, M);
+        if (grid[0] != gx || grid[1] != gy || grid[2] != slices)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,%u]", s->name, gx, gy, slices);
+        need[0] = (size_t)M * K;
+        need[1] = (size_t)M * 4;
+        need[2] = (size_t)N * K;
+        need[3] = (size_t)N * 4;
+        need[4] = (size_t)M * N * 4;
+        need[5] = (size_t)N * 4;
+        align[0] = align[2] = 16;
+        align[1] = align[3] = align[4] = 4;
+        align[5] = 0;                               // 0: the buffer may be NULL (4-byte aligned when given)
+        if (sr) {
+            need[6] = (size_t)gx * gy * slices * 32768;
+            need[7] = (size_t)gx * gy * 4;
+            align[6] = 8;
+            align[7] = 4;
+        }
+        return OJH_OK;
+    }
+    if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
     if (s->rows_per_wave < 2) {
         if (grid[0] != R) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,1,1]", s->name, R);
         size_t esz = s->rows_per_wave == 0 ? 2 : 4;
@@ -947,10 +1006,50 @@ static int check_rowq8(const ojh_kernel_spec *s, const uint32_t *c, const uint32
     align[1] = align[3] = align[4] = align[5] = 4;
     return OJH_OK;
 }
-static int shape_rowq8(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t M,
+// K slices of the row-int8 tile: two workgroups per CU is the aim, at most sixteen slices of at least four steps of 128.
+// OJAS_HIP_Q8ROW_SPLIT: 0 never, n > 1 that many.
+uint32_t ojh_matmul_q8row_slices(const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M) {
+    const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u, nks = (K + 127) / 128;
+    const uint32_t mode = dev ? dev->q8row_split : 1u;
+    const uint64_t tiles = (uint64_t)((N + 127) / 128) * ((M + 63) / 64);
+    if (!tiles || mode == 0) return 1;
+    uint32_t z = (uint32_t)(2 * (uint64_t)cus / tiles);
+    if (z > 16) z = 16;
+    if (z > nks / 4) z = nks / 4;
+    if (mode > 1) z = mode <= nks ? mode : nks;
+    if (z < 2) return 1;
+    const uint32_t per = (nks + z - 1) / z;
+    return (nks + per - 1) / per;
+}
+static int shape_rowq8(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K, uint32_t N, uint32_t M,
                        uint32_t grid[3], uint32_t block[3]) {
     grid[0] = s->rows_per_wave == 0 ? N : s->rows_per_wave == 1 ? M : (N + 3) / 4;
     grid[1] = grid[2] = 1;
+    if (s->rows_per_wave == 1) {
+        // a float4 per thread where the row gives as many (every load in flight at once), sixteen waves at most
+        const uint32_t want = (K / 4 + 63) / 64 * 64;
+        block[0] = want < 256 ? 256 : want > 1024 ? 1024 : want;
+        block[1] = block[2] = 1;
+        return OJH_OK;
+    }
+    if (s->rows_per_wave >= 7) {
+        // a wave takes two rows per pass; two workgroups per CU where the staged tokens are small, else one
+        const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
+        const uint32_t lim = s->rows_per_wave == 7 && (uint64_t)(M ? M : 1) * K <= 16384 ? 2 : 1;
+        uint32_t waves = 4;
+        while (waves < 16 && (uint64_t)lim * cus * waves * 2 < N) waves *= 2;
+        block[0] = 64 * waves;
+        block[1] = block[2] = 1;
+        uint32_t g = (N + waves * 2 - 1) / (waves * 2);
+        if (g > lim * cus) g = cus;
+        grid[0] = g ? g : 1;
+        return OJH_OK;
+    }
+    if (s->rows_per_wave >= 4) {
+        grid[0] = (N + 127) / 128;
+        grid[1] = s->rows_per_wave == 6 ? ((M ? M : 1) + 127) / 128 : ((M ? M : 1) + 63) / 64;
+        if (s->rows_per_wave == 5) grid[2] = ojh_matmul_q8row_slices(dev, K, N, M ? M : 1);
+    }
     block[0] = 256;
     block[1] = block[2] = 1;
     return OJH_OK;
@@ -1803,6 +1902,11 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("quant_rows_i8", "rowq8", 3, 2, 0, 1, check_rowq8, shape_rowq8);
     add("matmul_q8row", "rowq8", 5, 3, 0, 2, check_rowq8, shape_rowq8);
     add("matmul_q8row_bias", "rowq8", 6, 3, 0, 3, check_rowq8, shape_rowq8);
+    add("matmul_q8row_mt", "rowq8", 6, 3, 0, 4, check_rowq8, shape_rowq8);
+    add("matmul_q8row_mt_sr", "rowq8", 8, 4, 0, 5, check_rowq8, shape_rowq8);
+    add("matmul_q8row_mt128", "rowq8", 6, 3, 0, 6, check_rowq8, shape_rowq8);
+    add("matmul_q8row_dec", "rowq8", 6, 3, 0, 7, check_rowq8, shape_rowq8);
+    add("matmul_q8row_dec_l", "rowq8", 6, 3, 0, 8, check_rowq8, shape_rowq8);
     add("ffn_gu_q8k_q4k", "gemv_q8k", 5, 3, OJH_Q4_K, 1, check_ffn_gu, shape_rows);
     add("ffn_gu_q8k_kq", "gemv_q8k", 5, 4, 0, 1, check_ffn_gu_kq, shape_rows);
     add("gemv_q8k_kq_x4", "gemv_q8k", 10, 6, 0, 1, check_gemv_q8k_kq_x4, shape_rows);

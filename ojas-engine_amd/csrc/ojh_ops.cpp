@@ -847,8 +847,40 @@ extern "C" int ojh_matmul_q8(ojh_device *dev, const ojh_buf *x, size_t x_off, co
     ojh_buf *xq, *sx;
     if ((rc = ojh_scratch_get(dev, "q8_xq", (size_t)m * k, &xq))) return rc;
     if ((rc = ojh_scratch_get(dev, "q8_sx", (size_t)m * 4, &sx))) return rc;
-    uint32_t block[3] = {256, 1, 1}, gq[3] = {m, 1, 1}, gm[3] = {(n + 3) / 4, 1, 1};
-    if ((rc = ojh_launch(dev, "quant_rows_i8", {at(x, x_off), xq->ptr, sx->ptr}, {k, m}, gq, block))) return rc;
+    uint32_t block[3] = {256, 1, 1}, gq[3], bq[3], gm[3] = {(n + 3) / 4, 1, 1};
+    if ((rc = ojh_launch_shape(dev, "quant_rows_i8", k, 0, m, gq, bq))) return rc;
+    if ((rc = ojh_launch(dev, "quant_rows_i8", {at(x, x_off), xq->ptr, sx->ptr}, {k, m}, gq, bq))) return rc;
+    // a batch: the integer sums on the int8 matrix instruction (the same bits; the per-row kernel reads a row once per
+    // 8 tokens, so its time grows with the tokens)
+    const uint32_t mt_min = dev->q8row_mt_min_m != 1 ? dev->q8row_mt_min_m : 9u;
+    if (mt_min && m >= mt_min) {
+        uint32_t gt[3] = {(n + 127) / 128, (m + 63) / 64, 1};
+        void *bp = bias ? bias->ptr : nullptr;
+        // 128 tokens a tile where that still leaves a tile and a half per CU
+        const bool many = (uint64_t)gt[0] * ((m + 127) / 128) * 2 >= (uint64_t)3 * dev->prop.multiProcessorCount;
+        const uint32_t t128 = dev->q8row_t128_min_m != 1 ? dev->q8row_t128_min_m : many ? 129u : 0u;
+        if (t128 && m >= t128) {
+            gt[1] = (m + 127) / 128;
+            return ojh_launch(dev, "matmul_q8row_mt128", {xq->ptr, sx->ptr, wq->ptr, wscale->ptr, at(y, y_off), bp}, {k, n, m}, gt, block);
+        }
+        const uint32_t z = dev->no_scratch ? 1 : ojh_matmul_q8row_slices(dev, k, n, m);
+        if (z > 1) {
+            const size_t tiles = (size_t)gt[0] * gt[1];
+            ojh_buf *part, *cnt;
+            if ((rc = ojh_scratch_get(dev, "q8r_part", tiles * z * 32768, &part))) return rc;
+            if ((rc = ojh_scratch_get_zeroed(dev, "q8r_cnt", tiles * 4, &cnt))) return rc;
+            gt[2] = z;
+            return ojh_launch(dev, "matmul_q8row_mt_sr", {xq->ptr, sx->ptr, wq->ptr, wscale->ptr, at(y, y_off), bp, part->ptr, cnt->ptr},
+                              {k, n, m, z}, gt, block);
+        }
+        return ojh_launch(dev, "matmul_q8row_mt", {xq->ptr, sx->ptr, wq->ptr, wscale->ptr, at(y, y_off), bp}, {k, n, m}, gt, block);
+    }
+    if (dev->q8row_dec && m <= 8 && (size_t)m * k <= 131072) {
+        const char *name = (size_t)m * k <= 65536 ? "matmul_q8row_dec" : "matmul_q8row_dec_l";
+        uint32_t gd[3], bd[3];
+        if ((rc = ojh_launch_shape(dev, name, k, n, m, gd, bd))) return rc;
+        return ojh_launch(dev, name, {xq->ptr, sx->ptr, wq->ptr, wscale->ptr, at(y, y_off), bias ? bias->ptr : nullptr}, {k, n, m}, gd, bd);
+    }
     if (bias)
         return ojh_launch(dev, "matmul_q8row_bias", {xq->ptr, sx->ptr, wq->ptr, wscale->ptr, at(y, y_off), bias->ptr},
                           {k, n, m}, gm, block);
