@@ -1036,11 +1036,20 @@ struct GsQ5K {
     }
 };
 
-template <class F, bool SPLIT>
+// which row of xq / xs / y token m of the launch is: itself, or (grouped expert products) an entry of a list
+struct GsDense {
+    __device__ __forceinline__ uint row(uint m) const { return m; }
+};
+struct GsList {
+    const uint* lst;
+    uint last;
+    __device__ __forceinline__ uint row(uint m) const { return min(lst[m], last); }
+};
+template <class F, bool SPLIT, class TM = GsDense>
 __device__ __forceinline__ void gemm_q8k_gs_body(const signed char* __restrict__ xq, const float* __restrict__ xs,
                                                  const uchar* __restrict__ w, float* __restrict__ y, uint K, uint N, uint M,
                                                  uint ACC, uchar* lds, float* part = nullptr, uint* cnt = nullptr,
-                                                 uint nsplit = 1u) {
+                                                 uint nsplit = 1u, const TM tm = TM(), uint ty = blockIdx.y) {
     const uint tid = threadIdx.x, lane = tid & 63u;
     const uint wave = (uint)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint nsb = K >> 8;
@@ -1048,7 +1057,7 @@ __device__ __forceinline__ void gemm_q8k_gs_body(const signed char* __restrict__
     const uint sb0 = SPLIT ? blockIdx.z * per : 0u, sb1 = SPLIT ? min(nsb, sb0 + per) : nsb;
     if (SPLIT && sb0 >= sb1) return;                      // (the host launches only slices that hold a super-block)
     constexpr uint TPG = 64u, RPG = 128u;                     // tokens and rows per workgroup
-    const uint m0 = blockIdx.y * TPG, fr = lane & 31u, kg = lane >> 5;
+    const uint m0 = ty * TPG, fr = lane & 31u, kg = lane >> 5;
     const uint row = min(blockIdx.x * RPG + 32u * wave + fr, N - 1u);
     const uint tok0 = 0u;
     // 32-token blocks that hold tokens: the last token tile may need only the first
@@ -1060,14 +1069,19 @@ __device__ __forceinline__ void gemm_q8k_gs_body(const signed char* __restrict__
     const uint s_tok = tid >> 4, s_ch = tid & 15u;
     uint4 tv[NP];
     float tsx = 0.0f;
+    // the rows of this thread's tokens (one lookup per tile, not per super-block)
+    uint trow[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) trow[p] = tm.row(min(m0 + s_tok + 16u * (uint)p, M - 1u));
+    const uint xrow = tm.row(min(m0 + tid, M - 1u));
     auto fetch = [&](uint sb) {
 #pragma unroll
         for (int p = 0; p < NP; p++) {
             const uint m = m0 + s_tok + 16u * (uint)p;
             tv[p] = make_uint4(0u, 0u, 0u, 0u);
-            if (m < M) tv[p] = *(const uint4*)(xq + (size_t)m * K + (size_t)sb * 256u + s_ch * 16u);
+            if (m < M) tv[p] = *(const uint4*)(xq + (size_t)trow[p] * K + (size_t)sb * 256u + s_ch * 16u);
         }
-        if (tid < TPG) tsx = m0 + tid < M ? xs[(size_t)(m0 + tid) * nsb + sb] : 0.0f;
+        if (tid < TPG) tsx = m0 + tid < M ? xs[(size_t)xrow * nsb + sb] : 0.0f;
     };
     auto put = [&](uchar* st) {
 #pragma unroll
@@ -1168,7 +1182,7 @@ __device__ __forceinline__ void gemm_q8k_gs_body(const signed char* __restrict__
         for (int v = 0; v < 16; v++) {
             const uint t = m0 + tok0 + 32u * (uint)i + 8u * (uint)(v >> 2) + 4u * kg + (uint)(v & 3);
             if (t < M && n < N) {
-                float* o = y + (size_t)t * N + n;
+                float* o = y + (size_t)tm.row(t) * N + n;
                 *o = ACC ? *o + acc[i][v] : acc[i][v];
             }
         }
@@ -1188,3 +1202,28 @@ __device__ __forceinline__ void gemm_q8k_gs_body(const signed char* __restrict__
     }
 GEMM_Q8K_GS(q6k, GsQ6K)
 GEMM_Q8K_GS(q5k, GsQ5K)
+
+// The same tile over grouped expert products (the down projection of a mixture-of-experts layer whose down tensors are
+// Q6_K / Q5_K): expert e = blockIdx.z owns rows e N .. of `wd` and the assignments list[offsets[e] .. offsets[e + 1]);
+// token tiles blockIdx.y, + gridDim.y, .. of them (workgroups past the expert's count leave at once), results unweighted
+// into dv[a][n].
+//   moe_down_{q6k,q5k}_gs(aq, as, wd, dv, offsets, list, K, N, NA)     grid [ceil(N / 128), 1 .. ceil(T / 64), E] x 256
+#define MOE_DOWN_GS(FMT, F)                                                                                              \
+    extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))                         \
+    moe_down_##FMT##_gs(const signed char* aq, const float* as_, const uchar* wd, float* dv, const uint* offsets,        \
+                        const uint* list, uint K, uint N, uint NA) {                                                     \
+        __shared__ __attribute__((aligned(16))) uchar lds_gs[2 * GS_STAGE];                                              \
+        const uint e = blockIdx.z;                                                                                       \
+        const uint a0 = min(offsets[e], NA), a1 = min(offsets[e + 1], NA);                                               \
+        if (a0 >= a1) return;                                                                                            \
+        GsList tm;                                                                                                       \
+        tm.lst = list + a0;                                                                                              \
+        tm.last = NA - 1u;                                                                                               \
+        for (uint ty = blockIdx.y; ty * 64u < a1 - a0; ty += gridDim.y) {                                                \
+            gemm_q8k_gs_body<F, false, GsList>(aq, as_, wd + (size_t)e * N * (K >> 8) * F::BYTES, dv, K, N, a1 - a0, 0u, \
+                                               lds_gs, nullptr, nullptr, 1u, tm, ty);                                    \
+            __syncthreads();                                                                                             \
+        }                                                                                                                \
+    }
+MOE_DOWN_GS(q6k, GsQ6K)
+MOE_DOWN_GS(q5k, GsQ5K)

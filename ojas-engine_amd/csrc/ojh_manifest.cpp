@@ -1441,6 +1441,21 @@ static int check_moe(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t
         align[0] = align[2] = 16;
         return OJH_OK;
     }
+    case 22: {  // moe_down_{q6k,q5k}_gs(aq, as, wd, dv, offsets, list, K, N, NA)   grid [ceil(N/128), 1 .. , E]
+        uint32_t K = c[0], N = c[1], NA = c[2], E = grid[2];
+        if ((rc = check_block(block, 256))) return rc;
+        if (!K || K % 256 || !N || !NA) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u NA=%u", s->name, K, N, NA);
+        if (grid[0] != (N + 127) / 128 || !grid[1] || grid[1] > 65535 || !E || E > 65535)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/128), token tiles (any, up to 65535), E]", s->name);
+        need[0] = (size_t)NA * K;
+        need[1] = (size_t)NA * (K / 256) * 4;
+        need[2] = (size_t)E * N * (K / 256) * ojh_format(s->type)->bytes;
+        need[3] = (size_t)NA * N * 4;
+        need[4] = (size_t)(E + 1) * 4;
+        need[5] = (size_t)NA * 4;
+        align[0] = align[2] = 16;
+        return OJH_OK;
+    }
     case 8: {   // moe_gu_q4k_dec(x, wg, wu, act, idx, K, N, KSEL, NA, E)
         uint32_t K = c[0], N = c[1], KS = c[2], NA = c[3], E = c[4];
         if ((rc = check_block(block, 256))) return rc;
@@ -1613,6 +1628,7 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K
     case 3: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = experts
     case 4: grid[0] = K <= 1024 ? (N + 31) / 32 : (N + 15) / 16; grid[1] = M ? M : 1; break;  // M = experts
     case 20: grid[0] = M + 1; break;  // M = tokens
+    case 22: grid[0] = (N + 127) / 128; grid[2] = M ? M : 1; break;   // M = experts; grid[1]: the caller's token tiles per expert
     case 21: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;   // M = assignments
     case 6: case 7: grid[0] = (N + 15) / 16; grid[1] = M ? M : 1; break;
     case 14: case 16: grid[0] = (N + 7) / 8; grid[1] = M ? M : 1; break;    // M = slots, one token
@@ -1962,6 +1978,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("moe_gu_q4k_slots", "moe", 6, 6, OJH_Q4_K, 10, check_moe, shape_moe);
     add("moe_down_q4k_slots", "moe", 5, 5, OJH_Q4_K, 11, check_moe, shape_moe);
     add("moe_down_q5k_m", "moe", 6, 3, OJH_Q5_K, 4, check_moe, shape_moe);
+    add("moe_down_q5k_gs", "gemm_q8k", 6, 3, OJH_Q5_K, 22, check_moe, shape_moe);
+    add("moe_down_q6k_gs", "gemm_q8k", 6, 3, OJH_Q6_K, 22, check_moe, shape_moe);
     add("moe_down_q5k_dec", "moe", 5, 5, OJH_Q5_K, 9, check_moe, shape_moe);
     add("moe_gu_q80", "moe", 5, 2, OJH_Q8_0, 14, check_moe, shape_moe);
     m.back().expert_bufs = 2;

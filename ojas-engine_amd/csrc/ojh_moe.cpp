@@ -218,8 +218,20 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         uint32_t g[3] = {nsb_f, NA, 1};
         if ((rc = ojh_launch(dev, "quantize_q8k", {act->ptr, aq->ptr, as_->ptr}, {n_ff, NA}, g, b256))) return rc;
     }
-    // 5. down, one launch over all experts
-    {
+    // 5. down, one launch over all experts.  Q5_K / Q6_K down tensors: once experts see a handful of tokens each, the
+    //    int8 matrix tile of the dense path (one scale group per instruction) over each expert's assignments; the
+    //    integer-dot form below keeps an expert's rows in registers and walks its assignments one by one
+    const uint32_t gs_from = dev->moe_down_gs != 1 ? dev->moe_down_gs : 10u;
+    if (down5 && gs_from && (uint64_t)NA >= (uint64_t)gs_from * E && dev->moe_mode != 2) {
+        if ((rc = ensure(dev, "gemm_q8k"))) return rc;
+        const std::string down_gs = std::string("moe_down_") + ojh_format(down->type)->tag + "_gs";
+        uint32_t tiles = (T + 63) / 64;
+        if (tiles > 65535) tiles = 65535;
+        uint32_t g[3] = {(d + 127) / 128, tiles, E};
+        if ((rc = ojh_launch(dev, down_gs.c_str(), {aq->ptr, as_->ptr, (char *)down->raw->ptr + down->off, dv->ptr, offsets, list},
+                             {n_ff, d, NA}, g, b256)))
+            return rc;
+    } else {
         const bool dots = down5 || !mm;
         uint32_t g[3] = {mt_down ? ojh_moe_mt_groups(dev, d, E, 2) : dots && n_ff <= 1024 ? (d + 31) / 32 : (d + 15) / 16, E, 1};
         // (Q5_K rows have no matrix-core form: they stay on integer dots at every batch size)

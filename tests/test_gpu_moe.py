@@ -180,6 +180,83 @@ def test_expert_ffn_at_the_benchmark_shape(gpu, orc, pkg):
             assert np.array_equal(gpu.read(y2, T * d).reshape(T, d), got[perm])
 
 
+@pytest.mark.parametrize("T,E,ksel,d,nff", [(200, 8, 2, 512, 768), (130, 4, 3, 256, 1280), (64, 2, 2, 384 * 2, 256)])
+@pytest.mark.parametrize("dty", [13, 14])
+def test_q5k_q6k_down_tensors_on_the_int8_matrix_tile(gpu, orc, pkg, T, E, ksel, d, nff, dty):
+    """From a handful of assignments per expert `ojh_moe_ffn` sends Q5_K / Q6_K down tensors to
+    `moe_down_{q5k,q6k}_gs` (experts with one, two and three token tiles, ragged last tiles): sampled tokens against the
+    CPU arithmetic, every token against the integer-dot form, and — by name — one token tile per expert in the grid
+    (the workgroup walks the others) against one workgroup per tile, bit for bit."""
+    gate = pkg.synth.q4k_weights(E * nff, d, "moe5g", "gate", E, d, nff)
+    up = pkg.synth.q4k_weights(E * nff, d, "moe5g", "up", E, d, nff)
+    down = pkg.synth.weights(dty, E * d, nff, "moe5g", "down", E, d, nff, dty)
+    x = pkg.synth.normal_f32(T * d, "moe5g", "x", T, d).reshape(T, d)
+    lg = pkg.synth.normal_f32(T * E, "moe5g", "lg", T, E).reshape(T, E)
+    lg[:, 0] += 1.0                                      # a popular expert: more than one tile of assignments
+    outs = {}
+    for gs in ("1", "0"):
+        monkey = pytest.MonkeyPatch()
+        monkey.setenv("OJAS_HIP_MOE_DOWN_GS", gs)
+        g = pkg.HipGpu(0)
+        try:
+            gi, gw, idx_d, wgt_d = _route(g, lg, ksel)
+            lg_, lu_, ld_ = g.lin(Q4_K, E * nff, d, gate), g.lin(Q4_K, E * nff, d, up), g.lin(dty, E * d, nff, down)
+            yd = g.upload(np.full(T * d + d, 12345.5, np.float32))
+            g.moe_ffn(g.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd)
+            got = g.read(yd, T * d + d)
+            assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
+            outs[gs] = got[:T * d].reshape(T, d)
+            if gs == "1":
+                assert g.has_kernel("moe_down_%s_gs" % {13: "q5k", 14: "q6k"}[dty]), "the tile was not taken"
+        finally:
+            g.close()
+            monkey.undo()
+    for t in (0, T // 2, T - 1):
+        want = orc.moe_ffn(x[t:t + 1], gi[t:t + 1], gw[t:t + 1], gate, up, Q4_K, down, dty, E, nff, mode=0)
+        assert peak_err(outs["1"][t], want[0]) <= TOL, t
+    assert peak_err(outs["1"], outs["0"]) <= TOL
+
+
+@pytest.mark.parametrize("dty", [13, 14])
+def test_grouped_int8_tile_by_name(gpu, orc, pkg, dty):
+    """`moe_down_{q5k,q6k}_gs(aq, as, wd, dv, offsets, list, K, N, NA)`: every assignment's row against matvec_kq of its
+    expert; an empty expert; any number of token tiles in the grid gives the same bits."""
+    tag = {13: "q5k", 14: "q6k"}[dty]
+    E, n, k = 3, 200, 512
+    counts = [150, 0, 37]
+    na = sum(counts)
+    w = pkg.synth.weights(dty, E * n, k, "moegs", "w", dty)
+    act = pkg.synth.normal_f32(na * k, "moegs", "act", dty).reshape(na, k)
+    perm = pkg.synth.rng("moegs", "perm").permutation(na).astype(np.uint32)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+    gpu.ensure_family("gemm_q8k")
+    gpu.ensure_family("gemv_q8k")
+    nsb = k // 256
+    aq, as_ = gpu.alloc_bytes(na * k), gpu.alloc(na * nsb)
+    gpu.quant_q8k(gpu.upload(act), na, k, aq, as_)
+    wd, od, ld = gpu.upload_bytes(w), gpu.upload_bytes(offsets), gpu.upload_bytes(perm)
+    rb = len(w) // (E * n)
+    seen = []
+    for tiles in (1, 2, 3, 7):
+        dv = gpu.upload(np.full(na * n + n, 777.25, np.float32))
+        gpu.dispatch(gpu.begin(), "moe_down_%s_gs" % tag, [(aq, 0), (as_, 0), (wd, 0), (dv, 0), (od, 0), (ld, 0)], [k, n, na],
+                     [(n + 127) // 128, tiles, E], [256, 1, 1])
+        got = gpu.read(dv, na * n + n)
+        assert np.all(got[na * n:] == np.float32(777.25))
+        seen.append(got[:na * n].reshape(na, n).view(np.uint32).copy())
+    for other in seen[1:]:
+        assert np.array_equal(seen[0], other)
+    got = seen[0].view(np.float32)
+    for e in range(E):
+        we = w[e * n * rb:(e + 1) * n * rb]
+        for i in list(range(offsets[e], offsets[e + 1]))[::9]:
+            a = int(perm[i])
+            assert peak_err(got[a], orc.matvec_kq(we, dty, n, k, act[a])) <= 2e-5, (e, a)
+    with pytest.raises(pkg.OjasHipError, match="grid must be"):
+        gpu.dispatch(gpu.begin(), "moe_down_%s_gs" % tag, [(aq, 0), (as_, 0), (wd, 0), (gpu.alloc(na * n), 0), (od, 0), (ld, 0)],
+                     [k, n, na], [(n + 127) // 128 + 1, 1, E], [256, 1, 1])
+
+
 @pytest.mark.parametrize("T,E,ksel,d,nff,accum", [(1, 128, 8, 2048, 768, False), (3, 16, 5, 2304, 512, True),
                                                    (4, 8, 8, 768, 256, False), (2, 70, 64, 256, 256, False)])
 def test_decode_form_is_bit_identical_to_the_grouped_integer_dots(gpu, pkg, monkeypatch, T, E, ksel, d, nff, accum):
