@@ -581,6 +581,25 @@ def extras(gpu, pkg, lin_q) -> dict:
                         "tflops": round(fl / us / 1e6, 2)}
     out["moe_ffn_q4k_128x_top8"] = {"timed": "router + expert FFN, ojh_moe_ffn_routed (T <= 2: gate/up, the router inside it, and down launches addressed by assignment; above: router, quantize + group in one launch, gate/up, quantize, down, combine; T = 256 on int8 MFMA, moe_{gu,down}_q4k_mt, 32 assignments per staged pass)", **moe}
     del gate, up, down
+    # the same layer with finer expert tensors in a prefill batch: Q6_K down (int8 matrix tile per expert from 10
+    # assignments per expert) and all-Q8_0 experts (grouped f16 matrix tile from 4 per expert)
+    mixed = {}
+    gate = gpu.lin(pkg.Q4_K, E * nff, d, synth.q4k_weights(E * nff, d, "bench", "moe_gate"))
+    up = gpu.lin(pkg.Q4_K, E * nff, d, synth.q4k_weights(E * nff, d, "bench", "moe_up"))
+    down6 = gpu.lin(pkg.Q6_K, E * d, nff, synth.q6k_weights(E * d, nff, "bench", "moe_down6"))
+    g8 = gpu.lin(pkg.Q8_0, E * nff, d, synth.q80_weights(E * nff, d, "bench", "moe_gate8"))
+    u8 = gpu.lin(pkg.Q8_0, E * nff, d, synth.q80_weights(E * nff, d, "bench", "moe_up8"))
+    d8 = gpu.lin(pkg.Q8_0, E * d, nff, synth.q80_weights(E * d, nff, "bench", "moe_down8"))
+    for T in (256, 1024):
+        lg = gpu.upload(synth.normal_f32(T * E, "bench", "moe_lg", T))
+        xt, yt = gpu.upload(synth.normal_f32(T * d, "bench", "moe_x", T)), gpu.alloc(T * d)
+        idx, wgt = gpu.alloc_bytes(T * ksel * 4), gpu.alloc(T * ksel)
+        fl = 2.0 * T * ksel * 3 * nff * d
+        for tag, (a, b_, c) in (("q4k_gate_up_q6k_down", (gate, up, down6)), ("q8_0", (g8, u8, d8))):
+            us = _time(gpu, lambda i: gpu.moe_ffn_routed(xt, T, d, nff, E, ksel, lg, idx, wgt, a, b_, c, yt), 10, 2)
+            mixed[f"{tag}_T{T}"] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 2)}
+    out["moe_ffn_other_formats_128x_top8"] = {"timed": "router + expert FFN, ojh_moe_ffn_routed", **mixed}
+    del gate, up, down6, g8, u8, d8
     # ---- speculative verify on a Q6_K output head 151936 x 4096, bf16 activations
     n, k = 151936, 4096
     head = gpu.lin(pkg.Q6_K, n, k, synth.q6k_weights(n, k, "bench", "q6k_head"))

@@ -367,7 +367,10 @@ int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uin
  * dot_iq4xs / dot_iq4nl do (crates/ojas-cpu/src/cpu_math.rs:943-1010) through the reference's own expert
  * kernels moe_gu_<fmt> / moe_down_<fmt> (crates/ojas-cuda/src/kernels/moe.rs:75-125, moe_iq.rs:64-112),
  * one launch each over all tokens; there act_mode is OJH_ACT_AUTO or OJH_ACT_FLOAT and d, n_ff are
- * whole blocks of the formats.  K-quant experts take the same two launches under OJH_ACT_FLOAT
+ * whole blocks of the formats.  Under OJH_ACT_AUTO a batch of such experts (4 assignments per expert on
+ * average for Q8_0, 16 otherwise; d and n_ff multiples of 64) is grouped by expert on the f16 matrix tile:
+ * activations and silu * up rounded to f16, f32 accumulate, within 1e-3 of the output peak of the f32
+ * products; OJH_ACT_FLOAT keeps the per-assignment kernels at every batch size.  K-quant experts take the same two launches under OJH_ACT_FLOAT
  * (`moe_gu_q4k`, `moe_down_{q4k,q5k,q6k}`: f32 activations against the dequantized weights, the
  * reference's GPU expert kernels for those formats, crates/ojas-core/src/quant_src.rs:174-179);
  * OJH_ACT_AUTO and OJH_ACT_Q8K keep the CPU path's int8-activation arithmetic for them.

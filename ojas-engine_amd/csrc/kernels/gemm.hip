@@ -336,15 +336,28 @@ struct LoaderQ4L {
 // that care convert once (copy_f32_half) and take the f16 entries, as the reference's own `mm` does for split-K.
 // MI: 32-token blocks per wave along M — the tile is 64 MI tokens x 128 rows: 4 (256 tokens), or 2 for batches of up to 128
 // tokens, which would leave half of the taller tile's matrix instructions multiplying padding.
-template <class Loader, bool SPLITK, bool XF32 = false, int MI = 4>
+// which row of x and of y token m of the launch is: itself, or (grouped expert products) an entry of a list — the
+// activation row that entry divided by DIV (an assignment's token), the output row the entry itself
+struct GmDense {
+    __device__ __forceinline__ uint in_row(uint m) const { return m; }
+    __device__ __forceinline__ uint out_row(uint m) const { return m; }
+};
+struct GmList {
+    const uint* lst;
+    uint last, div;
+    __device__ __forceinline__ uint out_row(uint m) const { return min(lst[m], last); }
+    __device__ __forceinline__ uint in_row(uint m) const { return out_row(m) / div; }
+};
+template <class Loader, bool SPLITK, bool XF32 = false, int MI = 4, class TM = GmDense>
 __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const GmSrc src,
-                                             float* __restrict__ y, uint K, uint N, uint accum, uint M, uint nsplit) {
+                                             float* __restrict__ y, uint K, uint N, uint accum, uint M, uint nsplit,
+                                             const TM tm = TM(), uint ty = blockIdx.y) {
     const ushort* xh = (const ushort*)xv;
     const float* xf = (const float*)xv;
     constexpr uint BM = 64u * MI, STAGE = (BM + GM_BN) * GM_STRIDE, NX = 2u * MI;   // NX: activation rows per thread and slab
     __shared__ __attribute__((aligned(16))) uchar lds[2 * STAGE];
     const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint n0 = blockIdx.x * GM_BN, m0 = blockIdx.y * BM;
+    const uint n0 = blockIdx.x * GM_BN, m0 = ty * BM;
     // this block's K range (whole multiples of 64)
     uint k_begin = 0, k_end = K;
     if (SPLITK) {
@@ -359,7 +372,7 @@ __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const 
     const typename Loader::Row wrow = Loader::row(src, min(n0 + wr, N - 1u), K);
     size_t xrow[NX];   // element offset of the thread's 8 activations in each of its rows
 #pragma unroll
-    for (int i = 0; i < (int)NX; i++) xrow[i] = (size_t)min(m0 + xr + 32u * i, M - 1u) * K + xc;
+    for (int i = 0; i < (int)NX; i++) xrow[i] = (size_t)tm.in_row(min(m0 + xr + 32u * i, M - 1u)) * K + xc;
     const uint x_lds = xr * GM_STRIDE + xc * 2u;                   // + i * 32 rows
     const uint w_lds = BM * GM_STRIDE + wr * GM_STRIDE;
 
@@ -495,7 +508,7 @@ __device__ __forceinline__ void gemm_mm_body(const void* __restrict__ xv, const 
             for (int v = 0; v < 16; v++) {
                 const uint m = m0 + wm + 32u * i + 8u * (v >> 2) + 4u * kg + (v & 3u);
                 if (m < M && n < N) {
-                    float* o = y + (size_t)m * N + n;
+                    float* o = y + (size_t)tm.out_row(m) * N + n;
                     if (SPLITK) atomicAdd(o, acc[i][j][v]);
                     else *o = accum ? *o + acc[i][j][v] : acc[i][j][v];
                 }
@@ -524,6 +537,44 @@ GEMM_ENTRIES(q5k, LoaderQ5K)
 GEMM_ENTRIES(q6k, LoaderQ6K)
 GEMM_ENTRIES(q8_0, LoaderQ80)
 GEMM_ENTRIES(f16, LoaderF16)
+
+// Grouped expert products on the same tile (128 tokens x 128 rows): expert e = blockIdx.z % E owns rows e N .. of its
+// tensor and the assignments list[offsets[e] .. offsets[e + 1]); blockIdx.z / E picks the tensor and output of a pair
+// (gate and up of a mixture-of-experts layer in one launch; w1 / y1 unused with a grid of E).  Assignment a reads
+// activation row a / DIV (its token: DIV = slots per token; 1 where the activations are per assignment, as for the
+// down projection) and writes row a.  Token tiles blockIdx.y, + gridDim.y, .. of the expert; workgroups past its count
+// leave at once.
+//   moe_mm_<fmt>(xh, w0, w1, y0, y1, offsets, list, K, N, NA, E, DIV)    grid [ceil(N / 128), 1 .., E or 2 E] x 256
+#define MOE_MM_ENTRY(FMT, LOADER, ROWBYTES)                                                                       \
+    extern "C" __global__ void __launch_bounds__(256) moe_mm_##FMT(                                               \
+        const ushort* xh, const uchar* w0, const uchar* w1, float* y0, float* y1, const uint* offsets,            \
+        const uint* list, uint K, uint N, uint NA, uint E, uint DIV) {                                            \
+        const uint e = blockIdx.z % E, second = blockIdx.z / E;                                                   \
+        const uint a0 = min(offsets[e], NA), a1 = min(offsets[e + 1], NA);                                        \
+        if (a0 >= a1) return;                                                                                     \
+        GmList tm;                                                                                                \
+        tm.lst = list + a0;                                                                                       \
+        tm.last = NA - 1u;                                                                                        \
+        tm.div = DIV;                                                                                             \
+        const uchar* w = (second ? w1 : w0) + (size_t)e * N * (ROWBYTES);                                         \
+        for (uint ty = blockIdx.y; ty * 128u < a1 - a0; ty += gridDim.y) {                                        \
+            gemm_mm_body<LOADER, false, false, 2, GmList>(xh, GmSrc{w, nullptr, nullptr}, second ? y1 : y0, K, N, \
+                                                          0u, a1 - a0, 1u, tm, ty);                               \
+            __syncthreads();                                                                                      \
+        }                                                                                                         \
+    }
+MOE_MM_ENTRY(q8_0, LoaderQ80, (size_t)(K / 32u) * 34u)
+MOE_MM_ENTRY(f16, LoaderF16, (size_t)K * 2u)          // (experts decoded into f16 beforehand: formats without a loader here)
+
+// act16[i] = f16(silu(g[i]) * u[i]): what the grouped gate / up launch hands to the grouped down launch
+// (crates/ojas-cuda/src/kernels/moe.rs:75-102 forms the same product in f32)
+extern "C" __global__ void __launch_bounds__(256)
+moe_act_half(const float* __restrict__ g, const float* __restrict__ u, ushort* __restrict__ act16, uint n) {
+    for (uint i = blockIdx.x * 256u + threadIdx.x; i < n; i += gridDim.x * 256u) {
+        const float gs = g[i];
+        act16[i] = __half_as_ushort(__float2half_rn((gs / (1.0f + expf(-gs))) * u[i]));
+    }
+}
 
 // The reference's entries for Q4L weights, under their names and argument lists
 // (crates/ojas-cuda/src/kernels/gemm_q.rs:26-38, :505-542; dispatched by `CudaSsm::mm`, crates/ojas-cuda/src/qwen35.rs:683,690):

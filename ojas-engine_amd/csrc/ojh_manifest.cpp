@@ -1641,6 +1641,60 @@ static int shape_moe(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t K
     return OJH_OK;
 }
 
+// moe_mm_<fmt>(xh, w0, w1, y0, y1, offsets, list, K, N, NA, E, DIV): grid [ceil(N/128), token tiles (any), E or 2 E];
+// w1 / y1 may be NULL with a grid of E.  moe_act_half(g, u, act16, n): grid [x,1,1], grid-stride.
+static int check_moe_mm(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                        const uint32_t block[3], size_t need[16], size_t align[16]) {
+    int rc = check_block(block, 256);
+    if (rc) return rc;
+    if (s->rows_per_wave == 1) {
+        const size_t n = c[0];
+        if (!n) return ojh_fail(OJH_ERR_ARG, "%s: n must be positive", s->name);
+        if (grid[1] != 1 || grid[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: grid must be [x,1,1]", s->name);
+        need[0] = need[1] = n * 4;
+        need[2] = n * 2;
+        align[0] = align[1] = 4;
+        align[2] = 2;
+        return OJH_OK;
+    }
+    const uint32_t K = c[0], N = c[1], NA = c[2], E = c[3], DIV = c[4];
+    static const ojh_block_format plain_f16 = {OJH_F16, 2, 1, "f16"};   // (rows of plain f16: `moe_mm_f16`)
+    const ojh_block_format *f = &plain_f16;
+    if (s->type == OJH_F16) {
+        if (!K || !N) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u", s->name, K, N);
+    } else if ((rc = check_kn(s, K, N, &f))) {
+        return rc;
+    }
+    if (K % 64) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a multiple of 64", s->name, K);
+    if (!NA || !E || !DIV) return ojh_fail(OJH_ERR_ARG, "%s: NA=%u E=%u DIV=%u", s->name, NA, E, DIV);
+    if (grid[0] != (N + 127) / 128 || !grid[1] || grid[1] > 65535 || (grid[2] != E && grid[2] != 2 * E) || grid[2] > 65535)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/128), token tiles (any, up to 65535), E or 2 E]", s->name);
+    const bool pair = grid[2] == 2 * E;
+    const size_t wbytes = (size_t)E * N * (K / f->weights) * f->bytes;
+    need[0] = ((size_t)(NA - 1) / DIV + 1) * K * 2;
+    need[1] = need[2] = wbytes;
+    need[3] = need[4] = (size_t)NA * N * 4;
+    need[5] = (size_t)(E + 1) * 4;
+    need[6] = (size_t)NA * 4;
+    align[0] = 16;
+    const size_t wal = s->type == OJH_F16 ? 16 : ojh_block_align(f);
+    align[1] = wal;
+    align[2] = pair ? wal : 0;                     // 0: the buffer may be NULL (unused with a grid of E)
+    align[3] = 4;
+    align[4] = pair ? 4 : 0;
+    align[5] = align[6] = 4;
+    return OJH_OK;
+}
+static int shape_moe_mm(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t M,
+                        uint32_t grid[3], uint32_t block[3]) {
+    grid[0] = s->rows_per_wave == 1 ? (uint32_t)(((uint64_t)(N ? N : 1) + 1023) / 1024) : (N + 127) / 128;   // (act: N = elements)
+    grid[1] = 1;
+    grid[2] = s->rows_per_wave == 1 ? 1 : (M ? M : 1);     // M = experts
+    block[0] = 256;
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // copy_*(x, y, n) / fill_zero_u32(y, n): grid-stride, any positive grid of 256-thread blocks
 static int check_elementwise(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                              const uint32_t block[3], size_t need[16], size_t align[16]) {
@@ -2019,6 +2073,9 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("moe_down_q6k_dec", "moe", 5, 5, OJH_Q6_K, 9, check_moe, shape_moe);
     add("copy_bf16_half", "glue", 2, 1, (2u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     // glue: `type` carries (input element bytes << 8 | output element bytes)
+    add("moe_mm_q8_0", "gemm", 7, 5, OJH_Q8_0, 0, check_moe_mm, shape_moe_mm);
+    add("moe_mm_f16", "gemm", 7, 5, OJH_F16, 0, check_moe_mm, shape_moe_mm);
+    add("moe_act_half", "gemm", 3, 1, 0, 1, check_moe_mm, shape_moe_mm);
     add("copy_f32_half", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     add("copy_f32_bf16", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     add("copy_bf16_f32", "glue", 2, 1, (2u << 8) | 4u, 0, check_elementwise, shape_elementwise);

@@ -111,6 +111,66 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         if ((rc = span("moe_ffn: idx", idx, (size_t)NA8 * 4, 4))) return rc;
         if ((rc = span("moe_ffn: wgt", wgt, (size_t)NA8 * 4, 4))) return rc;
         if ((rc = span("moe_ffn: y", y, (size_t)T * d * 4, 4))) return rc;
+        // A batch of such experts under OJH_ACT_AUTO: the per-assignment kernels below read an expert's matrices once
+        // per assignment, so their time grows with the tokens; from a few assignments per expert the products run
+        // grouped by expert on the f16 matrix tile (f16 activations, f32 accumulate: the contract of the dense f16
+        // tile): gate and up in one launch, silu * up rounded to f16, down, the router-weighted sum.  Q8_0 rows are
+        // read by the tile itself; the other formats are decoded into f16 scratch first (2 bytes per weight of all
+        // three tensors), which pays from more assignments per expert.
+        const bool q80_all = gate->type == OJH_Q8_0 && down->type == OJH_Q8_0;
+        const uint32_t mm_from = dev->moe_mm_tile != 1 ? dev->moe_mm_tile : q80_all ? 4u : 16u;
+        const uint64_t w_gu = (uint64_t)E * n_ff * d, w_dn = (uint64_t)E * d * n_ff;
+        if (act_mode == OJH_ACT_AUTO && !kq_float && mm_from && (uint64_t)NA8 >= (uint64_t)mm_from * E && d % 64 == 0 &&
+            n_ff % 64 == 0 && (uint64_t)NA8 * (d > n_ff ? d : n_ff) <= 0xFFFFFFFFull && w_gu / fg->weights <= 0x7FFFFFFFu / 64 &&
+            w_dn / fd->weights <= 0x7FFFFFFFu / 64) {
+            if ((rc = ensure(dev, "moe")) || (rc = ensure(dev, "gemm")) || (rc = ensure(dev, "glue"))) return rc;
+            ojh_buf *xh, *gv, *uv, *a16, *dv, *grp;
+            if ((rc = ojh_scratch_get(dev, "moe_xh", (size_t)T * d * 2, &xh))) return rc;
+            if ((rc = ojh_scratch_get(dev, "moe_g", (size_t)NA8 * n_ff * 4, &gv))) return rc;
+            if ((rc = ojh_scratch_get(dev, "moe_u", (size_t)NA8 * n_ff * 4, &uv))) return rc;
+            if ((rc = ojh_scratch_get(dev, "moe_a16", (size_t)NA8 * n_ff * 2, &a16))) return rc;
+            if ((rc = ojh_scratch_get(dev, "moe_dv", (size_t)NA8 * d * 4, &dv))) return rc;
+            if ((rc = ojh_scratch_get(dev, "moe_grp", ((size_t)2 * E + 1 + NA8) * 4, &grp))) return rc;
+            void *wg = (char *)gate->raw->ptr + gate->off, *wu = (char *)up->raw->ptr + up->off, *wd = (char *)down->raw->ptr + down->off;
+            const char *tile = "moe_mm_q8_0";
+            if (!q80_all) {
+                ojh_buf *dq[3];
+                const ojh_lin *ls[3] = {gate, up, down};
+                const char *names[3] = {"moe_wg16", "moe_wu16", "moe_wd16"};
+                void **outs[3] = {&wg, &wu, &wd};
+                for (int i = 0; i < 3; i++) {
+                    const ojh_block_format *fi = ojh_format(ls[i]->type);
+                    const uint64_t nw = i < 2 ? w_gu : w_dn;
+                    if ((rc = ojh_scratch_get(dev, names[i], (size_t)nw * 2, &dq[i]))) return rc;
+                    if ((rc = ensure(dev, ojh_grid_type(ls[i]->type) ? "iq_grid" : "dequant"))) return rc;
+                    const std::string k = std::string("dequant_") + fi->tag + "_f16";
+                    const uint32_t nb = (uint32_t)(nw / fi->weights);
+                    uint32_t dg[3], db[3];
+                    if ((rc = ojh_launch_shape(dev, k.c_str(), 0, nb, 0, dg, db))) return rc;
+                    if ((rc = ojh_launch(dev, k.c_str(), {*outs[i], dq[i]->ptr}, {nb}, dg, db))) return rc;
+                    *outs[i] = dq[i]->ptr;
+                }
+                tile = "moe_mm_f16";
+            }
+            uint32_t *counts = (uint32_t *)grp->ptr, *offsets = counts + E, *list = offsets + E + 1;
+            uint32_t b256[3] = {256, 1, 1}, g1[3] = {1, 1, 1};
+            if ((rc = ojh_launch(dev, "moe_group", {idx->ptr, counts, offsets, list}, {NA8, E}, g1, b256))) return rc;
+            const uint32_t n_x = T * d, n_a = NA8 * n_ff;
+            uint32_t gc[3] = {(n_x / 8 + 255) / 256 + 1, 1, 1};
+            if ((rc = ojh_launch(dev, "copy_f32_half", {x->ptr, xh->ptr}, {n_x}, gc, b256))) return rc;
+            uint32_t tiles = (T + 127) / 128;
+            uint32_t gg[3] = {(n_ff + 127) / 128, tiles, 2 * E};
+            if ((rc = ojh_launch(dev, tile, {xh->ptr, wg, wu, gv->ptr, uv->ptr, offsets, list}, {d, n_ff, NA8, E, ksel}, gg, b256)))
+                return rc;
+            uint32_t ga[3] = {(n_a + 1023) / 1024, 1, 1};
+            if ((rc = ojh_launch(dev, "moe_act_half", {gv->ptr, uv->ptr, a16->ptr}, {n_a}, ga, b256))) return rc;
+            uint32_t gd[3] = {(d + 127) / 128, tiles, E};
+            if ((rc = ojh_launch(dev, tile, {a16->ptr, wd, nullptr, dv->ptr, nullptr, offsets, list}, {n_ff, d, NA8, E, 1u}, gd, b256)))
+                return rc;
+            uint64_t n = (uint64_t)T * d;
+            uint32_t gs[3] = {(uint32_t)((n + 255) / 256), 1, 1};
+            return ojh_launch(dev, "moe_combine", {dv->ptr, wgt->ptr, y->ptr}, {T, ksel, d, (uint32_t)(accum != 0)}, gs, b256);
+        }
         const std::string gu_name = std::string("moe_gu_") + fg->tag, down_name = std::string("moe_down_") + fd->tag;
         auto family_of = [](uint32_t t) { return t == OJH_IQ4_XS || t == OJH_IQ4_NL || ojh_grid_type(t) ? "moe_iq" : "moe"; };
         if ((rc = ensure(dev, family_of(gate->type)))) return rc;

@@ -502,9 +502,93 @@ def test_q80_experts_through_the_ffn_entry(gpu, orc, pkg, T, E, ksel, d, nff, ac
         gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, accum=accum, act_mode=mode)
         got = gpu.read(yd, T * d + d)
         assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
-        assert peak_err(got[:T * d].reshape(T, d) - y0, want - y0) <= 2e-5
+        # a batch under ACT_AUTO runs grouped on the f16 matrix tile: activations rounded to f16 on the way in
+        tiled = mode == pkg.ACT_AUTO and T * ksel >= 4 * E and d % 64 == 0 and nff % 64 == 0
+        assert peak_err(got[:T * d].reshape(T, d) - y0, want - y0) <= (1e-3 if tiled else 2e-5)
     with pytest.raises(pkg.OjasHipError, match="f32 activations"):
         gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, act_mode=pkg.ACT_Q8K)
+
+
+@pytest.mark.parametrize("T,E,ksel,d,nff,accum", [(300, 4, 2, 512, 320, False), (130, 16, 3, 256, 768, True)])
+def test_q80_experts_in_batches_on_the_grouped_matrix_tile(gpu, orc, pkg, T, E, ksel, d, nff, accum):
+    """From 4 assignments per expert `ojh_moe_ffn(..., OJH_ACT_AUTO)` groups Q8_0 experts' products on the f16 matrix
+    tile (experts with one and several 128-token tiles, ragged last tiles, N no multiple of 128): sampled tokens
+    against the f32 products of the CPU path, every token against the per-assignment kernels (OJH_ACT_FLOAT)."""
+    gate = pkg.synth.q80_weights(E * nff, d, "moe8t", "gate", E, d, nff)
+    up = pkg.synth.q80_weights(E * nff, d, "moe8t", "up", E, d, nff)
+    down = pkg.synth.q80_weights(E * d, nff, "moe8t", "down", E, d, nff)
+    x = pkg.synth.normal_f32(T * d, "moe8t", "x", T, d).reshape(T, d)
+    lg = pkg.synth.normal_f32(T * E, "moe8t", "lg", T, E).reshape(T, E)
+    lg[:, 1] += 1.5                                     # a popular expert
+    gi, gw, idx_d, wgt_d = _route(gpu, lg, ksel)
+    y0 = np.float32(0.01) * pkg.synth.normal_f32(T * d, "moe8t", "y0").reshape(T, d) if accum else np.zeros((T, d), np.float32)
+    lg_, lu_, ld_ = gpu.lin(Q8_0, E * nff, d, gate), gpu.lin(Q8_0, E * nff, d, up), gpu.lin(Q8_0, E * d, nff, down)
+    outs = {}
+    for mode in (pkg.ACT_AUTO, pkg.ACT_FLOAT):
+        yd = gpu.upload(np.concatenate([y0.ravel() if accum else np.full(T * d, 777.0, np.float32), np.full(d, 12345.5, np.float32)]))
+        gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, accum=accum, act_mode=mode)
+        got = gpu.read(yd, T * d + d)
+        assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
+        outs[mode] = got[:T * d].reshape(T, d) - y0
+    assert gpu.has_kernel("moe_mm_q8_0"), "the tile was not taken"
+    assert peak_err(outs[pkg.ACT_AUTO], outs[pkg.ACT_FLOAT]) <= 1e-3
+    for t in (0, T // 2, T - 1):
+        want = orc.moe_ffn(x[t:t + 1], gi[t:t + 1], gw[t:t + 1], gate, up, Q8_0, down, Q8_0, E, nff, mode=0)
+        assert peak_err(outs[pkg.ACT_AUTO][t], want[0]) <= 1e-3, t
+        assert peak_err(outs[pkg.ACT_FLOAT][t], want[0]) <= 2e-5, t
+
+
+def test_grouped_f16_tile_by_name(gpu, orc, pkg):
+    """`moe_mm_q8_0(xh, w0, w1, y0, y1, offsets, list, K, N, NA, E, DIV)`: a pair of tensors in one launch (gate and up:
+    assignment a reads token a / DIV) and a single tensor (down: DIV = 1, NULL second tensor); an empty expert; any
+    number of token tiles in the grid gives the same bits; every row against the f64 product of the exact block values
+    with the f16-rounded activations."""
+    E, n, k, div = 3, 200, 256, 2
+    counts = [150, 0, 38]
+    na = sum(counts)
+    tokens = na // div
+    w0, w1 = pkg.synth.q80_weights(E * n, k, "moemm", "w0"), pkg.synth.q80_weights(E * n, k, "moemm", "w1")
+    x = pkg.synth.normal_f32(tokens * k, "moemm", "x").reshape(tokens, k)
+    xh = x.astype(np.float16)
+    perm = pkg.synth.rng("moemm", "perm").permutation(na).astype(np.uint32)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+    gpu.ensure_family("gemm")
+    xd, od, ld = gpu.upload_bytes(xh.view(np.uint8)), gpu.upload_bytes(offsets), gpu.upload_bytes(perm)
+    w0d, w1d = gpu.upload_bytes(w0), gpu.upload_bytes(w1)
+    rb = len(w0) // (E * n)
+    seen = []
+    for tiles in (1, 2, 5):
+        y0d, y1d = (gpu.upload(np.full(na * n + n, 777.25, np.float32)) for _ in range(2))
+        gpu.dispatch(gpu.begin(), "moe_mm_q8_0", [(xd, 0), (w0d, 0), (w1d, 0), (y0d, 0), (y1d, 0), (od, 0), (ld, 0)],
+                     [k, n, na, E, div], [(n + 127) // 128, tiles, 2 * E], [256, 1, 1])
+        g0, g1 = gpu.read(y0d, na * n + n), gpu.read(y1d, na * n + n)
+        assert np.all(g0[na * n:] == np.float32(777.25)) and np.all(g1[na * n:] == np.float32(777.25))
+        seen.append(np.stack([g0[:na * n], g1[:na * n]]).reshape(2, na, n).view(np.uint32).copy())
+    for other in seen[1:]:
+        assert np.array_equal(seen[0], other)
+    got = seen[0].view(np.float32)
+    for e in range(E):
+        for i in list(range(offsets[e], offsets[e + 1]))[::7]:
+            a = int(perm[i])
+            for which, w in enumerate((w0, w1)):
+                want = orc.matmul_ref(w[e * n * rb:(e + 1) * n * rb], Q8_0, n, k, xh[a // div].astype(np.float32)[None, :], wmode=1)[0]
+                assert peak_err(got[which, a], want) <= 1e-5, (e, a, which)
+    # a single tensor: per-assignment activation rows (DIV = 1), the second tensor and output NULL
+    xa = pkg.synth.normal_f32(na * k, "moemm", "xa").reshape(na, k).astype(np.float16)
+    yd = gpu.upload(np.full(na * n + n, 777.25, np.float32))
+    gpu.dispatch(gpu.begin(), "moe_mm_q8_0", [(gpu.upload_bytes(xa.view(np.uint8)), 0), (w0d, 0), (None, 0), (yd, 0), (None, 0), (od, 0), (ld, 0)],
+                 [k, n, na, E, 1], [(n + 127) // 128, 2, E], [256, 1, 1])
+    g = gpu.read(yd, na * n + n)
+    assert np.all(g[na * n:] == np.float32(777.25))
+    g = g[:na * n].reshape(na, n)
+    for e in (0, 2):
+        for i in list(range(offsets[e], offsets[e + 1]))[::11]:
+            a = int(perm[i])
+            want = orc.matmul_ref(w0[e * n * rb:(e + 1) * n * rb], Q8_0, n, k, xa[a].astype(np.float32)[None, :], wmode=1)[0]
+            assert peak_err(g[a], want) <= 1e-5, (e, a)
+    with pytest.raises(pkg.OjasHipError, match="grid must be"):
+        gpu.dispatch(gpu.begin(), "moe_mm_q8_0", [(xd, 0), (w0d, 0), (w1d, 0), (gpu.alloc(na * n), 0), (gpu.alloc(na * n), 0), (od, 0), (ld, 0)],
+                     [k, n, na, E, div], [(n + 127) // 128, 1, E + 1], [256, 1, 1])
 
 
 @pytest.mark.parametrize("T,E,ksel,k,n", [(1, 8, 2, 256, 64), (3, 6, 4, 512, 224)])
@@ -608,7 +692,14 @@ def test_iq4_experts_through_the_ffn_entry(gpu, orc, pkg, tg, td, T, E, ksel, d,
     gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, accum=accum)
     got = gpu.read(yd, T * d + d)
     assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
-    assert peak_err(got[:T * d].reshape(T, d) - y0, want0) <= 2e-5
+    # from 16 assignments per expert a batch is decoded into f16 and grouped on the f16 matrix tile (activations
+    # rounded to f16 on the way in); OJH_ACT_FLOAT keeps the per-assignment kernels at every size
+    tiled = T * ksel >= 16 * E and d % 64 == 0 and nff % 64 == 0
+    assert peak_err(got[:T * d].reshape(T, d) - y0, want0) <= (1e-3 if tiled else 2e-5)
+    if tiled:
+        gpu.write_bytes(yd, 0, np.concatenate([y0.ravel() if accum else np.full(T * d, 777.0, np.float32), np.full(d, 12345.5, np.float32)]))
+        gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, accum=accum, act_mode=pkg.ACT_FLOAT)
+        assert peak_err(gpu.read(yd, T * d).reshape(T, d) - y0, want0) <= 2e-5
     with pytest.raises(pkg.OjasHipError, match="f32 activations"):
         gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, act_mode=pkg.ACT_Q8K)
 
