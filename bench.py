@@ -37,9 +37,9 @@ STAGES = [("x_attn", 4096, ["q", "k", "v"]), ("x_o", 4096, ["o"]), ("x_ffn", 409
 
 
 # HBM bytes per launch of the head matvec (128256 x 4096 Q4_K) from hardware counters: FETCH_SIZE
-# 144 331 KiB x 2.000 (the factor the same counter needs to read a 512 MiB copy correctly) +
+# 144 328 KiB x 2.000 (the factor the same counter needs to read a 512 MiB copy correctly) +
 # WRITE_SIZE 502 KiB.  Algorithmic bytes of the launch: 296 031 232.
-HEAD_TRAFFIC_BYTES = 296_103_936
+HEAD_TRAFFIC_BYTES = 296_088_772
 
 
 def algorithmic_bytes(n: int, k: int) -> int:
