@@ -1142,6 +1142,11 @@ static int shape_relayout(const ojh_kernel_spec *, const ojh_device *, uint32_t,
 }
 
 // dequant_<fmt>_f16(w, out, nblocks)
+// threads a decoder spends on one block of its format: a thread per eight weights
+static uint32_t dequant_threads_per_block(uint32_t type) {
+    const ojh_block_format *f = ojh_format(type);
+    return f && f->weights == 32 ? 4 : 32;
+}
 static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
                          const uint32_t block[3], size_t need[16], size_t align[16]) {
     const ojh_block_format *f = ojh_format(s->type);
@@ -1149,7 +1154,7 @@ static int check_dequant(const ojh_kernel_spec *s, const uint32_t *c, const uint
     if (!f || nb == 0) return ojh_fail(OJH_ERR_ARG, "%s: nblocks must be positive", s->name);
     int rc = check_block(block, 256);
     if (rc) return rc;
-    uint32_t tpb = s->type == OJH_Q6_K ? 64 : s->type == OJH_MXFP4 ? 16 : 32;  // threads per block of the format
+    uint32_t tpb = dequant_threads_per_block(s->type);
     if (grid[1] != 1 || grid[2] != 1 || (uint64_t)grid[0] * 256 < (uint64_t)nb * tpb)
         return ojh_fail(OJH_ERR_ARG, "%s: grid does not cover %u blocks", s->name, nb);
     need[0] = (size_t)nb * f->bytes;
@@ -1852,7 +1857,7 @@ static int shape_quantize(const ojh_kernel_spec *, const ojh_device *, uint32_t 
 // dequant: N is the number of blocks
 static int shape_dequant(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t,
                          uint32_t grid[3], uint32_t block[3]) {
-    uint32_t tpb = s->type == OJH_Q6_K ? 64 : s->type == OJH_MXFP4 ? 16 : 32;
+    uint32_t tpb = dequant_threads_per_block(s->type);
     grid[0] = (uint32_t)(((uint64_t)N * tpb + 255) / 256);
     grid[1] = grid[2] = 1;
     block[0] = 256;

@@ -620,9 +620,10 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     // tokens).  From `deq_min_m` tokens the rows are decoded once into library scratch (`dequant_<fmt>_f16`:
     // dequant_to_f16's bits) and the batch runs on the f16 tile — what the reference does at load time for every
     // tensor it cannot keep in place (crates/ojas-cuda/src/qwen35.rs:174-201), without holding the f16 copy.
-    // (from where the decode pass plus the tile beat the per-token walk: 8 tokens for the grid codebooks, whose decoders
-    // are the quick ones — 52 us in all on 14336 x 4096 —, 14 for the others — 95 to 130 us)
-    const uint32_t deq_min = dev->deq_min_m != 1 ? dev->deq_min_m : grid_fmt ? 8u : 14u;
+    // (from where the decode pass plus the tile beat the matvec that walks the rows once per four tokens: measured with
+    // the decoders at 22 - 31 us for 14336 x 4096, pass + tile 50 - 56 us flat against 37 - 41 / 66 / 98 us at 4 / 8 / 12
+    // tokens; on 4096 x 4096 28 against 13 / 22 / 31 / 39 at 4 / 8 / 12 / 16)
+    const uint32_t deq_min = dev->deq_min_m != 1 ? dev->deq_min_m : (uint64_t)N * K >= (32ull << 20) ? 5u : 9u;
     const bool deq_tile = (iq4 || grid_fmt) && !q5_float && act_asked != OJH_ACT_Q8K && deq_min && m >= deq_min &&
                           !dev->no_scratch && K % 64 == 0 && (uint64_t)N * K / f->weights <= 0x7FFFFFFFu / 64;
     void *tile_w = wp;

@@ -130,3 +130,21 @@ def test_embed_q80_matches_reader(gpu, orc, pkg):
     assert np.all(gpu.read(od, d + 2)[1:-1] == 0.0)
     with pytest.raises(pkg.OjasHipError, match="multiple of 32"):
         gpu.dispatch(gpu.begin(), "embed_q80", [(td, pad), (od, 4)], [0, 48], grid, block)
+
+
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, Q4_0, Q5_1, Q2_K, Q3_K])
+@pytest.mark.parametrize("out_off", [2, 8, 14])
+def test_output_that_is_not_16_byte_aligned(gpu, orc, pkg, ty, out_off):
+    """A thread writes its eight values as one 16-byte store where the output is 16-byte aligned; an output that starts
+    2, 8 or 14 bytes past such a boundary gets the same bits, nothing before or after them."""
+    bb, wpb = pkg.synth.BLOCK_SHAPE[ty]
+    nb = 48
+    raw = orc.synth_blocks(ty, nb)
+    n = nb * wpb
+    want = _dequant(gpu, ty, raw, n)
+    assert np.array_equal(want, orc.dequant_to_f16(raw, ty, n))
+    out = gpu.upload_bytes(np.full(n * 2 + 64, 0xA5, np.uint8))
+    gpu.dequant_f16(ty, gpu.upload_bytes(raw), n, out, out_off=out_off)
+    got = gpu.read(out, n * 2 + 64, np.uint8)
+    assert np.all(got[:out_off] == 0xA5) and np.all(got[out_off + n * 2:] == 0xA5)
+    assert np.array_equal(got[out_off:out_off + n * 2].view(np.uint16), want)

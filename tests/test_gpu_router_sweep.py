@@ -50,10 +50,9 @@ def test_router_sweep(gpu, orc, pkg, ty, n, k, m, accum):
     # Q8_0 under OJH_ACT_AUTO from 4 tokens (6 on matrices below 32 Mi weights): the f16 MFMA tile, activations rounded
     # to f16 (its own contract, the one the reference's GPU path switches to from 8 rows)
     tile = ty == Q8_0 and m >= (4 if n * k >= (32 << 20) else 6)
-    # formats with matvecs only: from 8 (grid codebooks) / 14 tokens decoded into scratch and run on the f16 tile
-    # (IQ2_XXS / IQ3_XXS keep the int8 kernels where OJH_ACT_Q8K is asked for: here from 32 tokens)
-    grid = ty in (IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_S, IQ3_S, IQ2_S, IQ1_M)
-    if ty not in (Q8_0, Q4_K, Q5_K, Q6_K) and k % 64 == 0 and m >= (8 if grid else 14) and (m < 32 or ty in FLOAT_ROWS):
+    # formats with matvecs only: from 5 tokens (9 on matrices below 32 Mi weights) decoded into scratch and run on the
+    # f16 tile (IQ2_XXS / IQ3_XXS keep the int8 kernels where OJH_ACT_Q8K is asked for: here from 32 tokens)
+    if ty not in (Q8_0, Q4_K, Q5_K, Q6_K) and k % 64 == 0 and m >= (5 if n * k >= (32 << 20) else 9) and (m < 32 or ty in FLOAT_ROWS):
         tile = True
     if tile:
         tol = 2e-3
