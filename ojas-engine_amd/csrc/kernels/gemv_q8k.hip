@@ -24,30 +24,59 @@
 #include "ojk_q6k_mfma.h"
 
 // ------------------------------------------------------------------ activation quantizer
-template <bool BF16>
+// A workgroup per 256-value segment, as the grid has always been; its first wave does the work, four consecutive
+// values a lane (one 16- or 8-byte load, the maximum across the wave, one 4-byte store of codes), and the other waves
+// leave at once.  (A value per thread — four partial maxima through LDS, a barrier, 1-byte stores — ran at 2.3-2.6 TB/s
+// on prefill-sized batches.)
+// FLAT (`quantize_q8k{,_bf16}_w`, grid [ceil(segments / 4)]): a segment per wave, four per workgroup, segments numbered
+// token-major — for batches of many short rows, where a workgroup per segment is mostly launch overhead.
+template <bool BF16, bool FLAT = false>
 __device__ __forceinline__ void quantize_q8k_body(const void* __restrict__ xv, signed char* __restrict__ q,
                                                   float* __restrict__ scales, uint K, uint M) {
-    __shared__ float wmax[4];
-    const uint sb = blockIdx.x, m = blockIdx.y, tid = threadIdx.x;
-    const uint nsb = (K + 255u) >> 8;
-    const uint i = sb * 256u + tid;
-    float v = 0.0f;
-    if (i < K) {
-        if (BF16) v = bf16_bits_to_f32(((const ushort*)xv)[(size_t)m * K + i]);
-        else v = ((const float*)xv)[(size_t)m * K + i];
+    const uint nsb = (K + 255u) >> 8, lane = threadIdx.x & 63u;
+    uint sb, m;
+    if (FLAT) {
+        const uint seg = blockIdx.x * 4u + (threadIdx.x >> 6);
+        if (seg >= nsb * M) return;
+        m = seg / nsb;
+        sb = seg - m * nsb;
+    } else {
+        if (threadIdx.x >= 64u) return;
+        sb = blockIdx.x;
+        m = blockIdx.y;
     }
-    float a = wave_max(fabsf(v));
-    if ((tid & 63u) == 0) wmax[tid >> 6] = a;
-    __syncthreads();
-    float mx = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+    const uint i = sb * 256u + 4u * lane;
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (BF16) {
+        const ushort* p = (const ushort*)xv + (size_t)m * K + i;
+        if (i + 3u < K && ((size_t)p & 7u) == 0) {
+            const uint2 t = *(const uint2*)p;
+            v[0] = bf16_bits_to_f32(t.x & 0xFFFFu); v[1] = bf16_bits_to_f32(t.x >> 16);
+            v[2] = bf16_bits_to_f32(t.y & 0xFFFFu); v[3] = bf16_bits_to_f32(t.y >> 16);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) if (i + (uint)j < K) v[j] = bf16_bits_to_f32(p[j]);
+        }
+    } else {
+        const float* p = (const float*)xv + (size_t)m * K + i;
+        if (i + 3u < K && ((size_t)p & 15u) == 0) {
+            const float4 t = *(const float4*)p;
+            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) if (i + (uint)j < K) v[j] = p[j];
+        }
+    }
+    const float mx = wave_max(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
     // scale = amax/127 (1 when the segment is all zero); q = clamp(round_half_away(v * (1/scale)))
-    float scale = mx > 0.0f ? __fdiv_rn(mx, 127.0f) : 1.0f;
-    float inv = __fdiv_rn(1.0f, scale);
-    float r = roundf(__fmul_rn(v, inv));
-    r = sat127(r);
+    const float scale = mx > 0.0f ? __fdiv_rn(mx, 127.0f) : 1.0f;
+    const float inv = __fdiv_rn(1.0f, scale);
+    uint packed = 0u;
+#pragma unroll
+    for (int j = 0; j < 4; j++) packed |= ((uint)(int)sat127(roundf(__fmul_rn(v[j], inv))) & 0xFFu) << (8 * j);
     // the padded tail of a ragged last segment is written as zero
-    q[((size_t)m * nsb + sb) * 256u + tid] = (signed char)(int)r;
-    if (tid == 0) scales[(size_t)m * nsb + sb] = scale;
+    *(uint*)(q + ((size_t)m * nsb + sb) * 256u + 4u * lane) = packed;
+    if (lane == 0) scales[(size_t)m * nsb + sb] = scale;
 }
 
 extern "C" __global__ void __launch_bounds__(256)
@@ -57,6 +86,14 @@ quantize_q8k(const float* x, signed char* q, float* scales, uint K, uint M) {
 extern "C" __global__ void __launch_bounds__(256)
 quantize_q8k_bf16(const ushort* x, signed char* q, float* scales, uint K, uint M) {
     quantize_q8k_body<true>(x, q, scales, K, M);
+}
+extern "C" __global__ void __launch_bounds__(256)
+quantize_q8k_w(const float* x, signed char* q, float* scales, uint K, uint M) {
+    quantize_q8k_body<false, true>(x, q, scales, K, M);
+}
+extern "C" __global__ void __launch_bounds__(256)
+quantize_q8k_bf16_w(const ushort* x, signed char* q, float* scales, uint K, uint M) {
+    quantize_q8k_body<true, true>(x, q, scales, K, M);
 }
 
 // ------------------------------------------------------------------ store modes

@@ -903,7 +903,11 @@ static int check_quantize(const ojh_kernel_spec *s, const uint32_t *c, const uin
     int rc = check_block(block, 256);
     if (rc) return rc;
     uint32_t nsb = (K + 255) / 256;
-    if (grid[0] != nsb || grid[1] != M || grid[2] != 1)
+    if (s->rows_per_wave == 1) {   // the `_w` entries: a segment per wave, grid [ceil(nsb M / 4),1,1]
+        const uint64_t segs = (uint64_t)nsb * M;
+        if (segs > 0xFFFFFFFFull || grid[0] != (segs + 3) / 4 || grid[1] != 1 || grid[2] != 1)
+            return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%llu,1,1]", s->name, (unsigned long long)((segs + 3) / 4));
+    } else if (grid[0] != nsb || grid[1] != M || grid[2] != 1)
         return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,%u,1]", s->name, nsb, M);
     size_t esz = strstr(s->name, "bf16") ? 2 : 4;
     need[0] = (size_t)M * K * esz;
@@ -1845,11 +1849,15 @@ static int shape_rows(const ojh_kernel_spec *s, const ojh_device *, uint32_t, ui
     block[1] = block[2] = 1;
     return OJH_OK;
 }
-static int shape_quantize(const ojh_kernel_spec *, const ojh_device *, uint32_t K, uint32_t, uint32_t M,
+static int shape_quantize(const ojh_kernel_spec *s, const ojh_device *, uint32_t K, uint32_t, uint32_t M,
                           uint32_t grid[3], uint32_t block[3]) {
     grid[0] = (K + 255) / 256;
     grid[1] = M ? M : 1;
     grid[2] = 1;
+    if (s->rows_per_wave == 1) {
+        grid[0] = (uint32_t)(((uint64_t)grid[0] * grid[1] + 3) / 4);
+        grid[1] = 1;
+    }
     block[0] = 256;
     block[1] = block[2] = 1;
     return OJH_OK;
@@ -1988,6 +1996,8 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     add("rmsnorm_q8k", "gemv_q8k", 5, 4, 0, 0, check_rmsnorm_q8k, shape_rmsnorm);
     add("quantize_q8k", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
     add("quantize_q8k_bf16", "gemv_q8k", 3, 2, 0, 0, check_quantize, shape_quantize);
+    add("quantize_q8k_w", "gemv_q8k", 3, 2, 0, 1, check_quantize, shape_quantize);
+    add("quantize_q8k_bf16_w", "gemv_q8k", 3, 2, 0, 1, check_quantize, shape_quantize);
     // prefill / verify MFMA tiles: "q8_0" is the reference's spelling for this family
     for (const auto &f : kFormats) {
         if (ojh_float_only(f.type) || ojh_grid_type(f.type)) continue;

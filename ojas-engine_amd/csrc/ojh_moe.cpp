@@ -259,8 +259,7 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         if ((rc = ojh_launch(dev, "moe_quant_group", {x->ptr, xq->ptr, xs->ptr, idx->ptr, counts, offsets, list}, {d, T, NA, E}, g, b256)))
             return rc;
     } else {
-        uint32_t g[3] = {nsb_d, T, 1};
-        if ((rc = ojh_launch(dev, "quantize_q8k", {x->ptr, xq->ptr, xs->ptr}, {d, T}, g, b256))) return rc;
+        if ((rc = ojh_quant_q8k_launch(dev, x->ptr, OJH_X_F32, T, d, xq->ptr, xs->ptr))) return rc;
         uint32_t g1[3] = {1, 1, 1};
         if ((rc = ojh_launch(dev, "moe_group", {idx->ptr, counts, offsets, list}, {NA, E}, g1, b256))) return rc;
     }
@@ -275,8 +274,7 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
     }
     // 4. quantize every assignment's activation (the CPU path quantizes `act` inside matvec_kq)
     {
-        uint32_t g[3] = {nsb_f, NA, 1};
-        if ((rc = ojh_launch(dev, "quantize_q8k", {act->ptr, aq->ptr, as_->ptr}, {n_ff, NA}, g, b256))) return rc;
+        if ((rc = ojh_quant_q8k_launch(dev, act->ptr, OJH_X_F32, NA, n_ff, aq->ptr, as_->ptr))) return rc;
     }
     // 5. down, one launch over all experts.  Q5_K / Q6_K down tensors: once experts see a handful of tokens each, the
     //    int8 matrix tile of the dense path (one scale group per instruction) over each expert's assignments; the

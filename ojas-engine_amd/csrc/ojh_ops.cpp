@@ -118,6 +118,12 @@ int ojh_quant_q8k_launch(ojh_device *dev, const void *x, int x_dtype, uint32_t m
                             void *scales) {
     const char *name = x_dtype == OJH_X_BF16 ? "quantize_q8k_bf16" : "quantize_q8k";
     uint32_t grid[3] = {(k + 255) / 256, m, 1}, block[3] = {256, 1, 1};
+    // many segments (a batch): a segment per wave, four to a workgroup
+    const uint64_t segs = (uint64_t)grid[0] * m;
+    if (segs >= 1024) {
+        uint32_t gw[3] = {(uint32_t)((segs + 3) / 4), 1, 1};
+        return ojh_launch(dev, x_dtype == OJH_X_BF16 ? "quantize_q8k_bf16_w" : "quantize_q8k_w", {(void *)x, q, scales}, {k, m}, gw, block);
+    }
     return ojh_launch(dev, name, {(void *)x, q, scales}, {k, m}, grid, block);
 }
 

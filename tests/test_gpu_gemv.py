@@ -45,6 +45,40 @@ def test_quantize_q8k_is_bit_exact(gpu, orc, pkg):
             assert np.array_equal(gq[t], wq), (k, t)
 
 
+@pytest.mark.parametrize("k,m,off,dt", [(768, 400, 0, "f32"), (300, 700, 0, "f32"), (4096, 70, 1, "f32"), (1024, 300, 0, "bf16"),
+                                        (300, 600, 1, "bf16")])
+def test_quantize_q8k_batches_a_segment_per_wave(gpu, orc, pkg, k, m, off, dt):
+    """From 1024 segments `ojh_quant_q8k` launches `quantize_q8k{,_bf16}_w` (a segment per wave): sampled tokens bit for
+    bit, a ragged last segment zero-padded, an input that starts off the vector alignment, nothing past the outputs; and
+    by name the same bits as the workgroup-per-segment entry."""
+    nsb = (k + 255) // 256
+    assert nsb * m >= 1024
+    x = pkg.synth.normal_f32(m * k + off, "q8kw", k, m)
+    if dt == "bf16":
+        bits = pkg.synth.to_bf16_bits(x)
+        xd, esz, xf = gpu.upload_bytes(bits), 2, pkg.synth.bf16_bits_to_f32(bits)
+    else:
+        xd, esz, xf = gpu.upload(x), 4, x
+    xf = xf[off:].reshape(m, k)
+    q, s = gpu.alloc_bytes(m * nsb * 256 + 16), gpu.alloc(m * nsb + 1)
+    gpu.memset0(q)
+    gpu.quant_q8k(xd, m, k, q, s, x_dtype=pkg.X_BF16 if dt == "bf16" else pkg.X_F32, x_off=off * esz)
+    gq = gpu.read(q, m * nsb * 256 + 16, np.int8)
+    assert not gq[m * nsb * 256:].any()
+    gq, gs = gq[:m * nsb * 256].reshape(m, -1), gpu.read(s, m * nsb).reshape(m, -1)
+    for t in sorted({0, 1, m // 2, m - 1}):
+        ws, wq, _ = orc.quant_q8k(xf[t])
+        assert np.array_equal(gs[t], ws) and np.array_equal(gq[t], wq), t
+    gpu.ensure_family("gemv_q8k")
+    name = "quantize_q8k_bf16" if dt == "bf16" else "quantize_q8k"
+    q2, s2 = gpu.alloc_bytes(m * nsb * 256), gpu.alloc(m * nsb)
+    gpu.dispatch(gpu.begin(), name, [(xd, off * esz), (q2, 0), (s2, 0)], [k, m], [nsb, m, 1], [256, 1, 1])
+    assert np.array_equal(gpu.read(q2, m * nsb * 256, np.int8).reshape(m, -1), gq)
+    assert np.array_equal(gpu.read(s2, m * nsb).view(np.uint32).reshape(m, -1), gs.view(np.uint32))
+    with pytest.raises(pkg.OjasHipError, match="grid must be"):
+        gpu.dispatch(gpu.begin(), name + "_w", [(xd, off * esz), (q2, 0), (s2, 0)], [k, m], [nsb, m, 1], [256, 1, 1])
+
+
 def test_quantize_q8k_bf16_input(gpu, orc, pkg):
     k, m = 4096, 2
     xb = pkg.synth.to_bf16_bits(pkg.synth.normal_f32(m * k, "q8kb"))
