@@ -215,9 +215,15 @@ __device__ __forceinline__ void moe_group_body(const uint* __restrict__ idx, uin
     const uint tid = threadIdx.x;
     for (uint e = tid; e < E; e += 256u) cnt[e] = 0u;
     __syncthreads();
-    for (uint a = tid; a < NA; a += 256u) {
-        uint e = idx[a];
-        if (e < E) atomicAdd(&cnt[e], 1u);
+    // (eight loads in flight per thread: one at a time, each pass over the assignments cost a round trip to memory per
+    // 256 of them — 8 us per pass at 2048)
+    for (uint a0 = tid; a0 < NA; a0 += 8u * 256u) {
+        uint e[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) e[u] = a0 + (uint)u * 256u < NA ? idx[a0 + (uint)u * 256u] : 0xFFFFFFFFu;
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (e[u] < E) atomicAdd(&cnt[e[u]], 1u);
     }
     __syncthreads();
     {
@@ -256,9 +262,13 @@ __device__ __forceinline__ void moe_group_body(const uint* __restrict__ idx, uin
     }
     for (uint e = tid; e < E; e += 256u) cnt[e] = 0u;  // reused as the per-expert cursor
     __syncthreads();
-    for (uint a = tid; a < NA; a += 256u) {
-        uint e = idx[a];
-        if (e < E) list[off[e] + atomicAdd(&cnt[e], 1u)] = a;
+    for (uint a0 = tid; a0 < NA; a0 += 8u * 256u) {
+        uint e[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) e[u] = a0 + (uint)u * 256u < NA ? idx[a0 + (uint)u * 256u] : 0xFFFFFFFFu;
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (e[u] < E) list[off[e[u]] + atomicAdd(&cnt[e[u]], 1u)] = a0 + (uint)u * 256u;
     }
 }
 extern "C" __global__ void __launch_bounds__(256)
