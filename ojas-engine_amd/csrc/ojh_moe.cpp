@@ -162,7 +162,7 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
             uint32_t gg[3] = {(n_ff + 127) / 128, tiles, 2 * E};
             if ((rc = ojh_launch(dev, tile, {xh->ptr, wg, wu, gv->ptr, uv->ptr, offsets, list}, {d, n_ff, NA8, E, ksel}, gg, b256)))
                 return rc;
-            uint32_t ga[3] = {(n_a + 1023) / 1024, 1, 1};
+            uint32_t ga[3] = {(n_a / 8 + 255) / 256 + 1, 1, 1};
             if ((rc = ojh_launch(dev, "moe_act_half", {gv->ptr, uv->ptr, a16->ptr}, {n_a}, ga, b256))) return rc;
             uint32_t gd[3] = {(d + 127) / 128, tiles, E};
             if ((rc = ojh_launch(dev, tile, {a16->ptr, wd, nullptr, dv->ptr, nullptr, offsets, list}, {n_ff, d, NA8, E, 1u}, gd, b256)))
