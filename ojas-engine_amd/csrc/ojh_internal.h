@@ -80,6 +80,7 @@ struct ojh_device {
     bool q8row_dec = true;       // OJAS_HIP_Q8ROW_DEC=0: 1 to 8 tokens on the per-row kernel instead of the one that stages the tokens in LDS
     uint32_t q8row_t128_min_m = 1; // OJAS_HIP_Q8ROW_T128_MIN_M: tokens from which that tile covers 128 tokens (0: never, 1: measured default, n: n)
     uint32_t q8row_split = 1;    // OJAS_HIP_Q8ROW_SPLIT: K slices of that tile (0: never, 1: by shape, n: n)
+    uint32_t deq_big_m = 1024;   // OJAS_HIP_DEQ_BIG_M: tokens from which Q6_K rows of a large matrix are decoded into scratch ahead of the f16 tile (Q5_K / Q8_0 rows from twice as many; 0: never)
     uint32_t deq_min_m = 1;      // OJAS_HIP_DEQ_MIN_M: tokens from which a format without a tile of its own is decoded into scratch and multiplied on the f16 tile (0: never, 1: by matrix size, n: n)
     uint32_t q80_tile_min_m = 1; // OJAS_HIP_Q80_TILE_MIN_M: tokens from which OJH_ACT_AUTO sends Q8_0 rows to the f16 tile (0: GEMM_MIN_M, 1: by shape, n: n)
     int gemm_m128 = 128;         // OJAS_HIP_GEMM_M128: tokens up to which Q5_K / Q6_K / Q8_0 batches take the 128-token f16 tile (0: never)

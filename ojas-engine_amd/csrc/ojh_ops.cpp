@@ -630,7 +630,14 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     // the decoders at 22 - 31 us for 14336 x 4096, pass + tile 50 - 56 us flat against 37 - 41 / 66 / 98 us at 4 / 8 / 12
     // tokens; on 4096 x 4096 28 against 13 / 22 / 31 / 39 at 4 / 8 / 12 / 16)
     const uint32_t deq_min = dev->deq_min_m != 1 ? dev->deq_min_m : (uint64_t)N * K >= (32ull << 20) ? 5u : 9u;
-    const bool deq_tile = (iq4 || grid_fmt) && !q5_float && act_asked != OJH_ACT_Q8K && deq_min && m >= deq_min &&
+    // Q6_K rows against a long prefill batch likewise: the tile that dequantizes them on the way into LDS spends a fifth
+    // of its time on that (14336 x 4096 at 2048 tokens 399 us against 288 for plain f16 rows), and the decode pass costs
+    // 29 us — the same weights, dequant_to_f16's bits, either way (OJAS_HIP_DEQ_BIG_M: tokens from which, 0 = never).
+    // (Q5_K and Q8_0 rows, whose loaders are lighter, from twice as many tokens: 14336 x 4096 at 2048 tokens 368 / 352 us
+    // against 327)
+    const uint32_t big_from = w->type == OJH_Q6_K ? dev->deq_big_m : w->type == OJH_Q5_K || w->type == OJH_Q8_0 ? 2 * dev->deq_big_m : 0u;
+    const bool deq_big = big_from && m >= big_from && m >= tile_min && act_mode != OJH_ACT_Q8K && (uint64_t)N * K >= (32ull << 20);
+    const bool deq_tile = ((iq4 || grid_fmt) && !q5_float && act_asked != OJH_ACT_Q8K && deq_min && m >= deq_min || deq_big) &&
                           !dev->no_scratch && K % 64 == 0 && (uint64_t)N * K / f->weights <= 0x7FFFFFFFu / 64;
     void *tile_w = wp;
     if (deq_tile) {
@@ -655,8 +662,12 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         if ((rc = ojh_scratch_get(dev, "xh", (size_t)m * K * 2, &xh))) return rc;
         const uint32_t n_el = m * K, conv_blocks = (n_el / 8 + 255) / 256 + 1;
         std::string base = std::string("gemm_mm_") + (deq_tile ? "f16" : w->type == OJH_Q8_0 ? "q8_0" : f->tag);
-        // (the tile that shares the dequantized weights through LDS is 256 tokens tall; up to 128 tokens its 128-token form)
-        if (!xl && m <= (uint32_t)dev->gemm_m128) base += "_m128";
+        // (the tile that shares the dequantized weights through LDS is 256 tokens tall; its 128-token form up to 128 tokens
+        // and wherever the taller one would give at most half of the CUs a tile — 14336 x 4096 at 256 tokens: Q8_0 78 ->
+        // 55 us, Q6_K 100 -> 77; plain f16 rows take it at every size, 322 -> 288 us at 2048 tokens)
+        const uint64_t t256 = (uint64_t)((N + 127) / 128) * ((m + 255) / 256);
+        if (!xl && dev->gemm_m128 && (m <= (uint32_t)dev->gemm_m128 || 2 * t256 <= (uint32_t)dev->prop.multiProcessorCount || deq_tile))
+            base += "_m128";
         if (xl) {
             // 256-token tiles when they give every CU a tile, or half of them with a K long enough
             // to split in two without the slices' fixed costs showing (measured on MI355X);

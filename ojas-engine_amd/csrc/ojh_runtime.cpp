@@ -98,6 +98,7 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_MOE_DOWN_GS")) d->moe_down_gs = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_Q8ROW_DEC")) d->q8row_dec = atoi(r) != 0;
     if (const char *r = getenv("OJAS_HIP_Q8ROW_SPLIT")) d->q8row_split = (uint32_t)atoi(r);
+    if (const char *r = getenv("OJAS_HIP_DEQ_BIG_M")) d->deq_big_m = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_DEQ_MIN_M")) d->deq_min_m = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_KQ_GS_SPLIT")) d->kq_gs_split = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE")) d->moe_mode = atoi(r);

@@ -326,3 +326,38 @@ def test_formats_without_a_tile_are_decoded_into_scratch_for_a_batch(gpu, orc, p
     gpu.mm(gpu.upload(x[:4].copy()), lin, y4, 4, act_mode=pkg.ACT_FLOAT)
     assert peak_err(gpu.read(y4, 4 * n).reshape(4, n), orc.matmul_ref(w, t, n, k, x[:4])) <= 1e-5
     lin.free()
+
+
+@pytest.mark.parametrize("ty,m", [(Q6_K, 1024), (Q8_0, 2048)])
+def test_long_batches_decode_the_rows_ahead_of_the_tile(gpu, orc, pkg, ty, m):
+    """Q6_K rows from 1024 tokens (Q5_K / Q8_0 from 2048) of a matrix of 32 Mi weights: `ojh_mm` decodes them into
+    scratch and runs the plain-f16 tile — the same weights (dequant_to_f16's bits) as the tile that dequantizes on the
+    way into LDS, so the two agree to the last bits of an f32 sum; sampled rows against the oracle at the tile's bound."""
+    n, k = 8192, 4096
+    gen = {Q6_K: pkg.synth.q6k_weights, Q8_0: pkg.synth.q80_weights}[ty]
+    w = gen(n, k, "big", ty)
+    x = pkg.synth.normal_f32(m * k, "big", "x", m).reshape(m, k)
+    outs = {}
+    for big in ("1024", "0"):
+        monkey = pytest.MonkeyPatch()
+        monkey.setenv("OJAS_HIP_DEQ_BIG_M", big)
+        g = pkg.HipGpu(0)
+        try:
+            yd = g.upload(np.full(m * n + n, 12345.5, np.float32))
+            g.mm(g.upload(x), g.lin(ty, n, k, w), yd, m, act_mode=pkg.ACT_FLOAT)
+            got = g.read(yd, m * n + n)
+            assert np.all(got[m * n:] == 12345.5), "wrote past row M"
+            outs[big] = got[:m * n].reshape(m, n)
+            if big != "0":
+                assert g.has_kernel("dequant_%s_f16" % {Q6_K: "q6k", Q8_0: "q80"}[ty]), "the rows were not decoded first"
+        finally:
+            g.close()
+            monkey.undo()
+    assert peak_err(outs["1024"], outs["0"]) <= 2e-6
+    rows = np.r_[0:16, n // 2:n // 2 + 16, n - 16:n]
+    rb = len(w) // n
+    wr = np.concatenate([w[r * rb:(r + 1) * rb] for r in rows])
+    toks = np.r_[0:8, m // 2:m // 2 + 8, m - 8:m]
+    want = orc.matmul_ref(wr, ty, len(rows), k, x[toks], wmode=1, xmode=1)
+    e = rms_errs(outs["1024"][np.ix_(toks, rows)], want)
+    assert e[0] < TIGHT[0] and e[1] < TIGHT[1], e
