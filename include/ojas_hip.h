@@ -368,7 +368,7 @@ int ojh_moe_route(ojh_device *dev, const ojh_buf *logits, uint32_t n_tokens, uin
  * kernels moe_gu_<fmt> / moe_down_<fmt> (crates/ojas-cuda/src/kernels/moe.rs:75-125, moe_iq.rs:64-112),
  * one launch each over all tokens; there act_mode is OJH_ACT_AUTO or OJH_ACT_FLOAT and d, n_ff are
  * whole blocks of the formats.  Under OJH_ACT_AUTO a batch of such experts (4 assignments per expert on
- * average for Q8_0, 16 otherwise; d and n_ff multiples of 64) is grouped by expert on the f16 matrix tile:
+ * average for Q8_0, IQ4_NL and IQ4_XS, 8 where a tensor is in a grid codebook; d and n_ff multiples of 64) is grouped by expert on the f16 matrix tile:
  * activations and silu * up rounded to f16, f32 accumulate, within 1e-3 of the output peak of the f32
  * products; OJH_ACT_FLOAT keeps the per-assignment kernels at every batch size.  K-quant experts take the same two launches under OJH_ACT_FLOAT
  * (`moe_gu_q4k`, `moe_down_{q4k,q5k,q6k}`: f32 activations against the dequantized weights, the

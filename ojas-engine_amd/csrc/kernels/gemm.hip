@@ -263,6 +263,174 @@ struct LoaderQ80 {
     }
 };
 
+// IQ4_NL: an 18-byte block = f16 d + 16 bytes of 4-bit indices into the sixteen non-linear levels; weight j < 16 is
+// the low nibble of byte j, weight 16 + j its high nibble; value f16(d * level), the bits of `dequant_iq4nl_f16`
+// (crates/ojas-formats/src/gguf.rs:796-812).  Thread half h owns block h of the slab = columns 32h..32h+31.
+struct LoaderIQ4NL {
+    static constexpr int NL = 2;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
+    u32x4 q;
+    uint d16;
+    float d;
+    uint o[16];
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 5) * IQ4NL_BYTES; }
+    __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
+        const uchar* blk = row + (size_t)((k0 >> 5) + h) * IQ4NL_BYTES;
+        d16 = gm_load_u16(blk);
+        q = gm_load16(blk + 2u);
+    }
+    __device__ __forceinline__ void prep() { d = f16_bits_to_f32(d16); }
+    template <int I>
+    __device__ __forceinline__ void part() {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const uint lv = iq4_levels4((q[I] >> (4 * s)) & 0x0F0F0F0Fu);
+            float v0 = __fmul_rn(d, (float)(signed char)(lv)), v1 = __fmul_rn(d, (float)(signed char)(lv >> 8));
+            float v2 = __fmul_rn(d, (float)(signed char)(lv >> 16)), v3 = __fmul_rn(d, (float)((int)lv >> 24));
+            o[8 * s + 2 * I] = pack2(v0, v1);
+            o[8 * s + 2 * I + 1] = pack2(v2, v3);
+        }
+    }
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* p = (u32x4*)(lds_row + h * 64u);
+#pragma unroll
+        for (int i = 0; i < 4; i++) p[i] = (u32x4){o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+    }
+};
+
+// IQ4_XS: a 136-byte super-block of 256 = f16 d, 16 bits of scale high pairs, 4 bytes of scale low nibbles, 128 bytes
+// of indices (sub-block ib of 32: bytes 16 ib .., nibbles laid out as in IQ4_NL); value f16((d * (ls - 32)) * level),
+// the bits of `dequant_iq4xs_f16` (crates/ojas-formats/src/gguf.rs:814-838).  Thread half h owns sub-block
+// (k0 / 32 + h) % 8 of super-block k0 / 256; rows are whole super-blocks (K a multiple of 256).
+struct LoaderIQ4XS {
+    static constexpr int NL = 3;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
+    u32x4 q;
+    uint h0, sl, ib;
+    float d;
+    uint o[16];
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * IQ4XS_BYTES; }
+    __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
+        const uchar* blk = row + (size_t)(k0 >> 8) * IQ4XS_BYTES;      // 136-byte blocks: 8-byte aligned with the tensor
+        ib = ((k0 >> 5) & 7u) + h;
+        h0 = *(const uint*)blk;
+        sl = *(const uint*)(blk + 4u);
+        q = gm_load16(blk + 8u + 16u * ib);
+    }
+    __device__ __forceinline__ void prep() {
+        const uint ls = ((sl >> (4u * ib)) & 0xFu) | ((((h0 >> 16) >> (2u * ib)) & 3u) << 4);
+        d = __fmul_rn(f16_bits_to_f32(h0 & 0xFFFFu), (float)((int)ls - 32));
+    }
+    template <int I>
+    __device__ __forceinline__ void part() {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const uint lv = iq4_levels4((q[I] >> (4 * s)) & 0x0F0F0F0Fu);
+            float v0 = __fmul_rn(d, (float)(signed char)(lv)), v1 = __fmul_rn(d, (float)(signed char)(lv >> 8));
+            float v2 = __fmul_rn(d, (float)(signed char)(lv >> 16)), v3 = __fmul_rn(d, (float)((int)lv >> 24));
+            o[8 * s + 2 * I] = pack2(v0, v1);
+            o[8 * s + 2 * I + 1] = pack2(v2, v3);
+        }
+    }
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* p = (u32x4*)(lds_row + h * 64u);
+#pragma unroll
+        for (int i = 0; i < 4; i++) p[i] = (u32x4){o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+    }
+};
+
+// The legacy 32-weight blocks Q4_0 / Q4_1 / Q5_0 / Q5_1: {f16 d [, f16 m]} [4 bytes of fifth bits] 16 bytes of nibbles;
+// weight j < 16 is the low nibble of byte j, weight 16 + j its high nibble, fifth bit = bit (weight index) of the
+// 4-byte field.  AFFINE: w = d * q + m (a product and a sum, each rounded), else w = d * (q - 8 | 16) — the bits of
+// `dequant_q{40,41,50,51}_f16` (crates/ojas-formats/src/gguf.rs:653-700).  Thread half h owns block h of the slab.
+template <bool FIVE, bool AFFINE>
+struct LoaderLegacy {
+    static constexpr int NL = 2 + (FIVE ? 1 : 0);
+    static constexpr uint BYTES = 18u + (AFFINE ? 2u : 0u) + (FIVE ? 4u : 0u), HDR = AFFINE ? 4u : 2u;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
+    u32x4 q;
+    uint hdr, qh;
+    float d, m;
+    uint o[16];
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 5) * BYTES; }
+    __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
+        const uchar* blk = row + (size_t)((k0 >> 5) + h) * BYTES;
+        typedef uint __attribute__((aligned(2))) u32_u;
+        if (AFFINE) hdr = *(const u32_u*)blk;
+        else hdr = gm_load_u16(blk);
+        qh = 0u;
+        if (FIVE) qh = *(const u32_u*)(blk + HDR);
+        q = gm_load16(blk + HDR + (FIVE ? 4u : 0u));
+    }
+    __device__ __forceinline__ void prep() {
+        d = f16_bits_to_f32(hdr & 0xFFFFu);
+        m = AFFINE ? f16_bits_to_f32(hdr >> 16) : 0.0f;
+    }
+    __device__ __forceinline__ float value(uint code) const {
+        if (AFFINE) return __fadd_rn(__fmul_rn(d, (float)code), m);
+        return __fmul_rn(d, __fsub_rn((float)code, FIVE ? 16.0f : 8.0f));
+    }
+    template <int I>
+    __device__ __forceinline__ void part() {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            uint nib = (q[I] >> (4 * s)) & 0x0F0F0F0Fu;
+            if (FIVE) {
+                const uint f = qh >> (16 * s + 4 * I);      // bits 0..3: the four weights of this dword and nibble half
+                nib |= ((f & 1u) << 4) | ((f & 2u) << 11) | ((f & 4u) << 18) | ((f & 8u) << 25);
+            }
+            o[8 * s + 2 * I] = pack2(value(nib & 0xFFu), value((nib >> 8) & 0xFFu));
+            o[8 * s + 2 * I + 1] = pack2(value((nib >> 16) & 0xFFu), value(nib >> 24));
+        }
+    }
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* p = (u32x4*)(lds_row + h * 64u);
+#pragma unroll
+        for (int i = 0; i < 4; i++) p[i] = (u32x4){o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+    }
+};
+
+// MXFP4 (crates/ojas-formats/src/mxfp4.rs:40-58): a 17-byte block { u8 e; u8 qs[16] }, w = 2^(e - 127) * E2M1[code],
+// weight 2j the low and 2j + 1 the high nibble of qs[j]: consecutive weights sit in consecutive nibbles.  The bits of
+// `dequant_mxfp4_f16`.  Blocks start at any byte.
+struct LoaderMXFP4 {
+    static constexpr int NL = 2;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
+    u32x4 q;
+    uint e8;
+    float d;
+    uint o[16];
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 5) * 17u; }
+    __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
+        const uchar* blk = row + (size_t)((k0 >> 5) + h) * 17u;
+        typedef u32x4 __attribute__((aligned(1))) u32x4_b;
+        e8 = gm_load_u8(blk);
+        q = *(const u32x4_b*)(blk + 1u);
+    }
+    __device__ __forceinline__ void prep() { d = __uint_as_float(e8 << 23); }
+    __device__ __forceinline__ float value(uint c) const {
+        const uint m = c & 7u;
+        const float a = 0.5f * (float)(m < 5u ? m : m == 5u ? 6u : m == 6u ? 8u : 12u);
+        return __fmul_rn(d, __uint_as_float(__float_as_uint(a) | ((c >> 3) << 31)));
+    }
+    template <int I>
+    __device__ __forceinline__ void part() {      // dword I: weights 8 I .. 8 I + 7, nibble by nibble
+        const uint v = q[I];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            o[4 * I + j] = pack2(value((v >> (8 * j)) & 15u), value((v >> (8 * j + 4)) & 15u));
+    }
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* p = (u32x4*)(lds_row + h * 64u);
+#pragma unroll
+        for (int i = 0; i < 4; i++) p[i] = (u32x4){o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+    }
+};
+
 // Plain f16 rows [N][K] (a tensor the caller keeps in f16, or any block format decoded into scratch by its
 // `dequant_<fmt>_f16` kernel ahead of the product): thread half h owns columns 32h..32h+31 of the slab, 64 bytes.
 struct LoaderF16 {
@@ -537,6 +705,17 @@ GEMM_ENTRIES(q5k, LoaderQ5K)
 GEMM_ENTRIES(q6k, LoaderQ6K)
 GEMM_ENTRIES(q8_0, LoaderQ80)
 GEMM_ENTRIES(f16, LoaderF16)
+GEMM_ENTRIES(iq4nl, LoaderIQ4NL)
+GEMM_ENTRIES(iq4xs, LoaderIQ4XS)
+typedef LoaderLegacy<false, false> LoaderQ40;
+typedef LoaderLegacy<false, true> LoaderQ41;
+typedef LoaderLegacy<true, false> LoaderQ50;
+typedef LoaderLegacy<true, true> LoaderQ51;
+GEMM_ENTRIES(q40, LoaderQ40)
+GEMM_ENTRIES(q41, LoaderQ41)
+GEMM_ENTRIES(q50, LoaderQ50)
+GEMM_ENTRIES(q51, LoaderQ51)
+GEMM_ENTRIES(mxfp4, LoaderMXFP4)
 
 // Grouped expert products on the same tile (128 tokens x 128 rows): expert e = blockIdx.z % E owns rows e N .. of its
 // tensor and the assignments list[offsets[e] .. offsets[e + 1]); blockIdx.z / E picks the tensor and output of a pair
@@ -564,6 +743,8 @@ GEMM_ENTRIES(f16, LoaderF16)
         }                                                                                                         \
     }
 MOE_MM_ENTRY(q8_0, LoaderQ80, (size_t)(K / 32u) * 34u)
+MOE_MM_ENTRY(iq4nl, LoaderIQ4NL, (size_t)(K / 32u) * IQ4NL_BYTES)
+MOE_MM_ENTRY(iq4xs, LoaderIQ4XS, (size_t)(K / 256u) * IQ4XS_BYTES)
 MOE_MM_ENTRY(f16, LoaderF16, (size_t)K * 2u)          // (experts decoded into f16 beforehand: formats without a loader here)
 
 // act16[i] = f16(silu(g[i]) * u[i]): what the grouped gate / up launch hands to the grouped down launch

@@ -2007,6 +2007,18 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g + "_m128", "gemm", 3, 4, f.type, 14, check_gemm, shape_gemm);
         add(g + "_m128_sk", "gemm", 3, 4, f.type, 15, check_gemm, shape_gemm);
     }
+    // IQ4_NL / IQ4_XS, the legacy 32-weight blocks and MXFP4 (f32-activation formats on the decode path) have loaders
+    // in the same tile; the IQ4 pair also in its grouped form
+    for (uint32_t t : {(uint32_t)OJH_IQ4_NL, (uint32_t)OJH_IQ4_XS, (uint32_t)OJH_Q4_0, (uint32_t)OJH_Q4_1, (uint32_t)OJH_Q5_0,
+                       (uint32_t)OJH_Q5_1, (uint32_t)OJH_MXFP4}) {
+        std::string g = std::string("gemm_mm_") + ojh_format(t)->tag;
+        add(g, "gemm", 3, 4, t, 0, check_gemm, shape_gemm);
+        add(g + "_sk", "gemm", 3, 4, t, 1, check_gemm, shape_gemm);
+        add(g + "_m128", "gemm", 3, 4, t, 14, check_gemm, shape_gemm);
+        add(g + "_m128_sk", "gemm", 3, 4, t, 15, check_gemm, shape_gemm);
+        if (t == OJH_IQ4_NL || t == OJH_IQ4_XS)
+            add(std::string("moe_mm_") + ojh_format(t)->tag, "gemm", 7, 5, t, 0, check_moe_mm, shape_moe_mm);
+    }
     // plain f16 rows on the same tile: what every format without a tile of its own is decoded into ahead of a batch
     add("gemm_mm_f16", "gemm", 3, 4, OJH_F16, 0, check_gemm, shape_gemm);
     add("gemm_mm_f16_sk", "gemm", 3, 4, OJH_F16, 1, check_gemm, shape_gemm);

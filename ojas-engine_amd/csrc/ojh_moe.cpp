@@ -114,11 +114,14 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
         // A batch of such experts under OJH_ACT_AUTO: the per-assignment kernels below read an expert's matrices once
         // per assignment, so their time grows with the tokens; from a few assignments per expert the products run
         // grouped by expert on the f16 matrix tile (f16 activations, f32 accumulate: the contract of the dense f16
-        // tile): gate and up in one launch, silu * up rounded to f16, down, the router-weighted sum.  Q8_0 rows are
-        // read by the tile itself; the other formats are decoded into f16 scratch first (2 bytes per weight of all
-        // three tensors), which pays from more assignments per expert.
-        const bool q80_all = gate->type == OJH_Q8_0 && down->type == OJH_Q8_0;
-        const uint32_t mm_from = dev->moe_mm_tile != 1 ? dev->moe_mm_tile : q80_all ? 4u : 16u;
+        // tile): gate and up in one launch, silu * up rounded to f16, down, the router-weighted sum.  Q8_0, IQ4_NL and
+        // IQ4_XS rows are read by the tile's own loaders; the other formats are decoded into f16 scratch first (2 bytes
+        // per weight of the tensors concerned), which pays from more assignments per expert.
+        auto tile_of = [](uint32_t t) -> const char * {
+            return t == OJH_Q8_0 ? "moe_mm_q8_0" : t == OJH_IQ4_NL ? "moe_mm_iq4nl" : t == OJH_IQ4_XS ? "moe_mm_iq4xs" : nullptr;
+        };
+        const char *tile_gu = tile_of(gate->type), *tile_dn = tile_of(down->type);
+        const uint32_t mm_from = dev->moe_mm_tile != 1 ? dev->moe_mm_tile : tile_gu && tile_dn ? 4u : 8u;
         const uint64_t w_gu = (uint64_t)E * n_ff * d, w_dn = (uint64_t)E * d * n_ff;
         if (act_mode == OJH_ACT_AUTO && !kq_float && mm_from && (uint64_t)NA8 >= (uint64_t)mm_from * E && d % 64 == 0 &&
             n_ff % 64 == 0 && (uint64_t)NA8 * (d > n_ff ? d : n_ff) <= 0xFFFFFFFFull && w_gu / fg->weights <= 0x7FFFFFFFu / 64 &&
@@ -132,13 +135,13 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
             if ((rc = ojh_scratch_get(dev, "moe_dv", (size_t)NA8 * d * 4, &dv))) return rc;
             if ((rc = ojh_scratch_get(dev, "moe_grp", ((size_t)2 * E + 1 + NA8) * 4, &grp))) return rc;
             void *wg = (char *)gate->raw->ptr + gate->off, *wu = (char *)up->raw->ptr + up->off, *wd = (char *)down->raw->ptr + down->off;
-            const char *tile = "moe_mm_q8_0";
-            if (!q80_all) {
+            {
                 ojh_buf *dq[3];
                 const ojh_lin *ls[3] = {gate, up, down};
                 const char *names[3] = {"moe_wg16", "moe_wu16", "moe_wd16"};
                 void **outs[3] = {&wg, &wu, &wd};
                 for (int i = 0; i < 3; i++) {
+                    if (i < 2 ? tile_gu != nullptr : tile_dn != nullptr) continue;
                     const ojh_block_format *fi = ojh_format(ls[i]->type);
                     const uint64_t nw = i < 2 ? w_gu : w_dn;
                     if ((rc = ojh_scratch_get(dev, names[i], (size_t)nw * 2, &dq[i]))) return rc;
@@ -150,7 +153,8 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
                     if ((rc = ojh_launch(dev, k.c_str(), {*outs[i], dq[i]->ptr}, {nb}, dg, db))) return rc;
                     *outs[i] = dq[i]->ptr;
                 }
-                tile = "moe_mm_f16";
+                if (!tile_gu) tile_gu = "moe_mm_f16";
+                if (!tile_dn) tile_dn = "moe_mm_f16";
             }
             uint32_t *counts = (uint32_t *)grp->ptr, *offsets = counts + E, *list = offsets + E + 1;
             uint32_t b256[3] = {256, 1, 1}, g1[3] = {1, 1, 1};
@@ -160,12 +164,12 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
             if ((rc = ojh_launch(dev, "copy_f32_half", {x->ptr, xh->ptr}, {n_x}, gc, b256))) return rc;
             uint32_t tiles = (T + 127) / 128;
             uint32_t gg[3] = {(n_ff + 127) / 128, tiles, 2 * E};
-            if ((rc = ojh_launch(dev, tile, {xh->ptr, wg, wu, gv->ptr, uv->ptr, offsets, list}, {d, n_ff, NA8, E, ksel}, gg, b256)))
+            if ((rc = ojh_launch(dev, tile_gu, {xh->ptr, wg, wu, gv->ptr, uv->ptr, offsets, list}, {d, n_ff, NA8, E, ksel}, gg, b256)))
                 return rc;
             uint32_t ga[3] = {(n_a / 8 + 255) / 256 + 1, 1, 1};
             if ((rc = ojh_launch(dev, "moe_act_half", {gv->ptr, uv->ptr, a16->ptr}, {n_a}, ga, b256))) return rc;
             uint32_t gd[3] = {(d + 127) / 128, tiles, E};
-            if ((rc = ojh_launch(dev, tile, {a16->ptr, wd, nullptr, dv->ptr, nullptr, offsets, list}, {n_ff, d, NA8, E, 1u}, gd, b256)))
+            if ((rc = ojh_launch(dev, tile_dn, {a16->ptr, wd, nullptr, dv->ptr, nullptr, offsets, list}, {n_ff, d, NA8, E, 1u}, gd, b256)))
                 return rc;
             uint64_t n = (uint64_t)T * d;
             uint32_t gs[3] = {(uint32_t)((n + 255) / 256), 1, 1};

@@ -637,7 +637,18 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
     // against 327)
     const uint32_t big_from = w->type == OJH_Q6_K ? dev->deq_big_m : w->type == OJH_Q5_K || w->type == OJH_Q8_0 ? 2 * dev->deq_big_m : 0u;
     const bool deq_big = big_from && m >= big_from && m >= tile_min && act_mode != OJH_ACT_Q8K && (uint64_t)N * K >= (32ull << 20);
-    const bool deq_tile = ((iq4 || grid_fmt) && !q5_float && act_asked != OJH_ACT_Q8K && deq_min && m >= deq_min || deq_big) &&
+    // IQ4_NL / IQ4_XS rows have loaders in the tile: short of the long batches they skip the decode pass (14336 x 4096:
+    // 53 - 62 -> 32 - 42 us up to 128 tokens, 114 -> 93 at 512; 4096 x 4096 at 16 tokens 29 -> 14; from 1024 tokens
+    // the pass pays for itself as it does for Q6_K) and take the tile from 5 tokens on every shape (the matvec that
+    // walks the rows once per four tokens: 13 / 22 us at 4 / 8 tokens on 4096 x 4096)
+    // (the legacy 32-weight blocks and MXFP4 likewise)
+    const bool own_loader = w->type == OJH_IQ4_NL || (w->type == OJH_IQ4_XS && K % 256 == 0) || w->type == OJH_Q4_0 ||
+                            w->type == OJH_Q4_1 || w->type == OJH_Q5_0 || w->type == OJH_Q5_1 || w->type == OJH_MXFP4;
+    const bool iq4_own = dev->iq4_tile && own_loader &&
+                         act_asked != OJH_ACT_Q8K && m >= dev->iq4_tile && (!dev->deq_big_m || m < dev->deq_big_m) &&
+                         (w->type != OJH_MXFP4 || m <= 128) &&   // (17-byte blocks: its loads are byte-aligned and slow; 14336 x 4096 at 64 / 256 tokens 55 / 97 us against 61 / 80 through the pass)
+                         K % 64 == 0;
+    const bool deq_tile = ((iq4 || grid_fmt) && !iq4_own && !q5_float && act_asked != OJH_ACT_Q8K && deq_min && m >= deq_min || deq_big) &&
                           !dev->no_scratch && K % 64 == 0 && (uint64_t)N * K / f->weights <= 0x7FFFFFFFu / 64;
     void *tile_w = wp;
     if (deq_tile) {
@@ -651,7 +662,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
         if ((rc = ojh_launch(dev, dq.c_str(), {wp, wdeq->ptr}, {nb}, dg, db))) return rc;
         tile_w = wdeq->ptr;
     }
-    if ((deq_tile || (m >= tile_min && act_mode != OJH_ACT_Q8K && !iq4 && !grid_fmt)) && K % 64 == 0 &&
+    if ((deq_tile || iq4_own || (m >= tile_min && act_mode != OJH_ACT_Q8K && !iq4 && !grid_fmt)) && K % 64 == 0 &&
         (uint64_t)m * K < 0x7FFFFFFFull && (uint64_t)m * N < 0x7FFFFFFFull) {
         // Q4_K takes the 256-wide tile with the reference GPU kernel's arithmetic (f16 qa*q + qb)
         // unless the tile that reproduces dequant_to_f16 bit for bit is asked for.

@@ -361,3 +361,38 @@ def test_long_batches_decode_the_rows_ahead_of_the_tile(gpu, orc, pkg, ty, m):
     want = orc.matmul_ref(wr, ty, len(rows), k, x[toks], wmode=1, xmode=1)
     e = rms_errs(outs["1024"][np.ix_(toks, rows)], want)
     assert e[0] < TIGHT[0] and e[1] < TIGHT[1], e
+
+
+@pytest.mark.parametrize("ty,tag", [(20, "iq4nl"), (23, "iq4xs"), (2, "q40"), (3, "q41"), (6, "q50"), (7, "q51"), (139, "mxfp4")])
+def test_iq4_rows_on_the_tile_by_name(gpu, orc, pkg, ty, tag):
+    """`gemm_mm_<fmt>{,_m128}` read IQ4_NL / IQ4_XS, Q4_0 / Q4_1 / Q5_0 / Q5_1 and MXFP4 rows through loaders of their own: one-hot activations read back
+    `dequant_to_f16`'s bits of every weight, and a product equals, bit for bit, the plain-f16 tile on the decoded rows
+    (`dequant_<fmt>_f16` + `gemm_mm_f16`: the same weights meet the same sums in the same order)."""
+    k, n, m = 512, 200, 150
+    bb, wpb = pkg.synth.BLOCK_SHAPE[ty]
+    raw = pkg.synth.weights(ty, n, k, "iq4tile", tag)
+    want = orc.dequant_to_f16(raw, ty, n * k).view(np.float16).astype(np.float32).reshape(n, k)
+    gpu.ensure_family("gemm")
+    gpu.ensure_family("dequant")
+    wd = gpu.upload_bytes(raw)
+    eye = gpu.upload_bytes(np.eye(k, dtype=np.float16).view(np.uint8))
+    yd = gpu.upload(np.full(k * n + 64, 777.25, np.float32))
+    gpu.dispatch(gpu.begin(), "gemm_mm_" + tag, [(eye, 0), (wd, 0), (yd, 0)], [k, n, 0, k], [(n + 127) // 128, (k + 255) // 256, 1], [256, 1, 1])
+    got = gpu.read(yd, k * n + 64)
+    assert np.all(got[k * n:] == np.float32(777.25))
+    assert np.array_equal(got[:k * n].reshape(k, n), want.T)
+    x = pkg.synth.normal_f32(m * k, "iq4tile", "x").astype(np.float16)
+    xd = gpu.upload_bytes(x.view(np.uint8))
+    w16 = gpu.alloc_bytes(n * k * 2)
+    grid, block = gpu.launch_shape("dequant_%s_f16" % tag, 0, n * k // wpb, 0)
+    gpu.dispatch(gpu.begin(), "dequant_%s_f16" % tag, [(wd, 0), (w16, 0)], [n * k // wpb], grid, block)
+    outs = {}
+    for kernel, src, bm in (("gemm_mm_" + tag, wd, 256), ("gemm_mm_f16", w16, 256), ("gemm_mm_%s_m128" % tag, wd, 128),
+                            ("gemm_mm_f16_m128", w16, 128)):
+        yk = gpu.alloc(m * n)
+        gpu.dispatch(gpu.begin(), kernel, [(xd, 0), (src, 0), (yk, 0)], [k, n, 0, m], [(n + 127) // 128, (m + bm - 1) // bm, 1], [256, 1, 1])
+        outs[kernel] = gpu.read(yk, m * n).view(np.uint32)
+    assert np.array_equal(outs["gemm_mm_" + tag], outs["gemm_mm_f16"])
+    assert np.array_equal(outs["gemm_mm_%s_m128" % tag], outs["gemm_mm_f16_m128"])
+    ref = x.astype(np.float32).reshape(m, k).astype(np.float64) @ want.astype(np.float64).T
+    assert peak_err(outs["gemm_mm_" + tag].view(np.float32).reshape(m, n), ref) <= 1e-5

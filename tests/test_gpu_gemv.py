@@ -162,7 +162,7 @@ def test_float_head_form_keeps_activations_in_registers(gpu, orc, pkg, ty, tag, 
 
 
 @pytest.mark.parametrize("ty", [IQ4_NL, IQ4_XS])
-@pytest.mark.parametrize("n,k,m", [(4096, 4096, 1), (37, 256, 1), (130, 2816, 5), (1000, 1024, 2), (33001, 2816, 1),
+@pytest.mark.parametrize("n,k,m", [(4096, 4096, 1), (37, 256, 1), (130, 2816, 4), (1000, 1024, 2), (33001, 2816, 1),
                                    (40000, 4096, 1), (32768, 256, 1)])
 def test_iq4_rows_match_the_cpu_dots(gpu, orc, pkg, ty, n, k, m):
     """IQ4_NL / IQ4_XS rows against `matvec_kq`, which sends these types to dot_iq4nl / dot_iq4xs on

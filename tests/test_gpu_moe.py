@@ -538,8 +538,9 @@ def test_q80_experts_in_batches_on_the_grouped_matrix_tile(gpu, orc, pkg, T, E, 
         assert peak_err(outs[pkg.ACT_FLOAT][t], want[0]) <= 2e-5, t
 
 
-def test_grouped_f16_tile_by_name(gpu, orc, pkg):
-    """`moe_mm_q8_0(xh, w0, w1, y0, y1, offsets, list, K, N, NA, E, DIV)`: a pair of tensors in one launch (gate and up:
+@pytest.mark.parametrize("fmt,tile", [(Q8_0, "moe_mm_q8_0"), (IQ4_NL, "moe_mm_iq4nl"), (IQ4_XS, "moe_mm_iq4xs")])
+def test_grouped_f16_tile_by_name(gpu, orc, pkg, fmt, tile):
+    """`moe_mm_<fmt>(xh, w0, w1, y0, y1, offsets, list, K, N, NA, E, DIV)`: a pair of tensors in one launch (gate and up:
     assignment a reads token a / DIV) and a single tensor (down: DIV = 1, NULL second tensor); an empty expert; any
     number of token tiles in the grid gives the same bits; every row against the f64 product of the exact block values
     with the f16-rounded activations."""
@@ -547,7 +548,7 @@ def test_grouped_f16_tile_by_name(gpu, orc, pkg):
     counts = [150, 0, 38]
     na = sum(counts)
     tokens = na // div
-    w0, w1 = pkg.synth.q80_weights(E * n, k, "moemm", "w0"), pkg.synth.q80_weights(E * n, k, "moemm", "w1")
+    w0, w1 = pkg.synth.weights(fmt, E * n, k, "moemm", "w0"), pkg.synth.weights(fmt, E * n, k, "moemm", "w1")
     x = pkg.synth.normal_f32(tokens * k, "moemm", "x").reshape(tokens, k)
     xh = x.astype(np.float16)
     perm = pkg.synth.rng("moemm", "perm").permutation(na).astype(np.uint32)
@@ -559,7 +560,7 @@ def test_grouped_f16_tile_by_name(gpu, orc, pkg):
     seen = []
     for tiles in (1, 2, 5):
         y0d, y1d = (gpu.upload(np.full(na * n + n, 777.25, np.float32)) for _ in range(2))
-        gpu.dispatch(gpu.begin(), "moe_mm_q8_0", [(xd, 0), (w0d, 0), (w1d, 0), (y0d, 0), (y1d, 0), (od, 0), (ld, 0)],
+        gpu.dispatch(gpu.begin(), tile, [(xd, 0), (w0d, 0), (w1d, 0), (y0d, 0), (y1d, 0), (od, 0), (ld, 0)],
                      [k, n, na, E, div], [(n + 127) // 128, tiles, 2 * E], [256, 1, 1])
         g0, g1 = gpu.read(y0d, na * n + n), gpu.read(y1d, na * n + n)
         assert np.all(g0[na * n:] == np.float32(777.25)) and np.all(g1[na * n:] == np.float32(777.25))
@@ -571,12 +572,12 @@ def test_grouped_f16_tile_by_name(gpu, orc, pkg):
         for i in list(range(offsets[e], offsets[e + 1]))[::7]:
             a = int(perm[i])
             for which, w in enumerate((w0, w1)):
-                want = orc.matmul_ref(w[e * n * rb:(e + 1) * n * rb], Q8_0, n, k, xh[a // div].astype(np.float32)[None, :], wmode=1)[0]
+                want = orc.matmul_ref(w[e * n * rb:(e + 1) * n * rb], fmt, n, k, xh[a // div].astype(np.float32)[None, :], wmode=1)[0]
                 assert peak_err(got[which, a], want) <= 1e-5, (e, a, which)
     # a single tensor: per-assignment activation rows (DIV = 1), the second tensor and output NULL
     xa = pkg.synth.normal_f32(na * k, "moemm", "xa").reshape(na, k).astype(np.float16)
     yd = gpu.upload(np.full(na * n + n, 777.25, np.float32))
-    gpu.dispatch(gpu.begin(), "moe_mm_q8_0", [(gpu.upload_bytes(xa.view(np.uint8)), 0), (w0d, 0), (None, 0), (yd, 0), (None, 0), (od, 0), (ld, 0)],
+    gpu.dispatch(gpu.begin(), tile, [(gpu.upload_bytes(xa.view(np.uint8)), 0), (w0d, 0), (None, 0), (yd, 0), (None, 0), (od, 0), (ld, 0)],
                  [k, n, na, E, 1], [(n + 127) // 128, 2, E], [256, 1, 1])
     g = gpu.read(yd, na * n + n)
     assert np.all(g[na * n:] == np.float32(777.25))
@@ -584,10 +585,10 @@ def test_grouped_f16_tile_by_name(gpu, orc, pkg):
     for e in (0, 2):
         for i in list(range(offsets[e], offsets[e + 1]))[::11]:
             a = int(perm[i])
-            want = orc.matmul_ref(w0[e * n * rb:(e + 1) * n * rb], Q8_0, n, k, xa[a].astype(np.float32)[None, :], wmode=1)[0]
+            want = orc.matmul_ref(w0[e * n * rb:(e + 1) * n * rb], fmt, n, k, xa[a].astype(np.float32)[None, :], wmode=1)[0]
             assert peak_err(g[a], want) <= 1e-5, (e, a)
     with pytest.raises(pkg.OjasHipError, match="grid must be"):
-        gpu.dispatch(gpu.begin(), "moe_mm_q8_0", [(xd, 0), (w0d, 0), (w1d, 0), (gpu.alloc(na * n), 0), (gpu.alloc(na * n), 0), (od, 0), (ld, 0)],
+        gpu.dispatch(gpu.begin(), tile, [(xd, 0), (w0d, 0), (w1d, 0), (gpu.alloc(na * n), 0), (gpu.alloc(na * n), 0), (od, 0), (ld, 0)],
                      [k, n, na, E, div], [(n + 127) // 128, 1, E + 1], [256, 1, 1])
 
 
@@ -692,9 +693,9 @@ def test_iq4_experts_through_the_ffn_entry(gpu, orc, pkg, tg, td, T, E, ksel, d,
     gpu.moe_ffn(gpu.upload(x), T, d, nff, E, ksel, idx_d, wgt_d, lg_, lu_, ld_, yd, accum=accum)
     got = gpu.read(yd, T * d + d)
     assert np.all(got[T * d:] == 12345.5), "wrote past the last token"
-    # from 16 assignments per expert a batch is decoded into f16 and grouped on the f16 matrix tile (activations
-    # rounded to f16 on the way in); OJH_ACT_FLOAT keeps the per-assignment kernels at every size
-    tiled = T * ksel >= 16 * E and d % 64 == 0 and nff % 64 == 0
+    # from 4 assignments per expert a batch is grouped on the f16 matrix tile (activations rounded to f16 on the way
+    # in); OJH_ACT_FLOAT keeps the per-assignment kernels at every size
+    tiled = T * ksel >= 4 * E and d % 64 == 0 and nff % 64 == 0      # (Q8_0 and IQ4 rows: read by the tile's own loaders)
     assert peak_err(got[:T * d].reshape(T, d) - y0, want0) <= (1e-3 if tiled else 2e-5)
     if tiled:
         gpu.write_bytes(yd, 0, np.concatenate([y0.ravel() if accum else np.full(T * d, 777.0, np.float32), np.full(d, 12345.5, np.float32)]))
