@@ -527,6 +527,19 @@ def extras(gpu, pkg, lin_q) -> dict:
         fr[tag] = {"us": round(us, 2), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 8e6, 4)}
         del wf
     out["float_rows_gemv_128256x4096"] = {"activations": "f32", "kernels": "gemv_nat_<fmt>_px", **fr}
+    # ---- the same formats against a batch (f32 in, OJH_ACT_AUTO): the f16 tile through the formats' own loaders, or the
+    # decode pass into f16 scratch + the plain-f16 tile for those without one
+    fb = {}
+    nb, kb = 14336, 4096
+    for ty, tag in ((pkg.IQ4_XS, "iq4xs"), (pkg.Q4_0, "q40"), (pkg.Q5_1, "q51"), (pkg.MXFP4, "mxfp4"), (pkg.Q3_K, "q3k"),
+                    (pkg.IQ3_S, "iq3s")):
+        wf = [gpu.lin(ty, nb, kb, synth.weights(ty, nb, kb, "bench", tag, "batch")) for _ in range(2)]
+        for m in (16, 128, 512):
+            xb, yb = gpu.upload(synth.normal_f32(m * kb, "bench", "xb", m)), gpu.alloc(m * nb)
+            us = _time(gpu, lambda i: gpu.mm(xb, wf[i % 2], yb, m), 10, 2)
+            fb[f"{tag}_M{m}"] = {"us": round(us, 1), "mfma_frac": round(2.0 * m * nb * kb / us / 1e6 / 2500.0, 4)}
+        del wf
+    out["float_rows_batch_14336x4096"] = {"activations": "f32 -> f16", "kernels": "gemm_mm_<fmt>{,_m128}{,_sk} (IQ4_NL / IQ4_XS, Q4_0 .. Q5_1, MXFP4 up to 128 tokens) or dequant_<fmt>_f16 + gemm_mm_f16_m128{,_sk}", **fb}
     # IQ2_XXS as the CPU path multiplies it: int8 activations per 256, integer dots (dot_iq2xxs_q8k)
     wf = [gpu.lin(pkg.IQ2_XXS, n, k, synth.weights(pkg.IQ2_XXS, n, k, "bench", "iq2xxs", "head")) for _ in range(2)]
     us = _time(gpu, lambda i: gpu.mm(x, wf[i % 2], y), 20, 3)
@@ -590,12 +603,17 @@ def extras(gpu, pkg, lin_q) -> dict:
     g8 = gpu.lin(pkg.Q8_0, E * nff, d, synth.q80_weights(E * nff, d, "bench", "moe_gate8"))
     u8 = gpu.lin(pkg.Q8_0, E * nff, d, synth.q80_weights(E * nff, d, "bench", "moe_up8"))
     d8 = gpu.lin(pkg.Q8_0, E * d, nff, synth.q80_weights(E * d, nff, "bench", "moe_down8"))
+    # (IQ4_XS gate / up with IQ4_NL down, the mix the reference's streamed models ship in: the grouped tile's own loaders)
+    gx = gpu.lin(pkg.IQ4_XS, E * nff, d, synth.weights(pkg.IQ4_XS, E * nff, d, "bench", "moe_gatex"))
+    ux = gpu.lin(pkg.IQ4_XS, E * nff, d, synth.weights(pkg.IQ4_XS, E * nff, d, "bench", "moe_upx"))
+    dn = gpu.lin(pkg.IQ4_NL, E * d, nff, synth.weights(pkg.IQ4_NL, E * d, nff, "bench", "moe_downn"))
     for T in (256, 1024):
         lg = gpu.upload(synth.normal_f32(T * E, "bench", "moe_lg", T))
         xt, yt = gpu.upload(synth.normal_f32(T * d, "bench", "moe_x", T)), gpu.alloc(T * d)
         idx, wgt = gpu.alloc_bytes(T * ksel * 4), gpu.alloc(T * ksel)
         fl = 2.0 * T * ksel * 3 * nff * d
-        for tag, (a, b_, c) in (("q4k_gate_up_q6k_down", (gate, up, down6)), ("q8_0", (g8, u8, d8))):
+        for tag, (a, b_, c) in (("q4k_gate_up_q6k_down", (gate, up, down6)), ("q8_0", (g8, u8, d8)),
+                                ("iq4xs_gate_up_iq4nl_down", (gx, ux, dn))):
             us = _time(gpu, lambda i: gpu.moe_ffn_routed(xt, T, d, nff, E, ksel, lg, idx, wgt, a, b_, c, yt), 10, 2)
             mixed[f"{tag}_T{T}"] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 2)}
     out["moe_ffn_other_formats_128x_top8"] = {"timed": "router + expert FFN, ojh_moe_ffn_routed", **mixed}

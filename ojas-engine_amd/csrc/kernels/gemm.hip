@@ -431,6 +431,108 @@ struct LoaderMXFP4 {
     }
 };
 
+// Q2_K and Q3_K keep four 2-bit planes per byte: within a half of 128 weights, byte l of the half's 32 code bytes holds
+// weights l, l + 32, l + 64, l + 96 at bits 0, 2, 4, 6, and scale 8 half + 2 j + l / 16 covers (plane j, l / 16).  The
+// thread's 32 consecutive weights are one plane of one half: s = (k0 / 32 + h) % 8, half = s / 4, j = s % 4 — all 32 code
+// bytes of the half at bits 2 j.  Rows are whole super-blocks (K a multiple of 256).
+// Q2_K: w = (d * sc) * q - dmin * m, every step rounded — the bits of `dequant_q2k_f16`
+// (crates/ojas-formats/src/gguf.rs:730-754).
+struct LoaderQ2K {
+    static constexpr int NL = 4;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
+    u32x4 qa, qb;
+    uint sc2, dd, j;
+    float dl[2], ml[2];
+    uint o[16];
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * Q2K_BYTES; }
+    __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
+        const uchar* blk = row + (size_t)(k0 >> 8) * Q2K_BYTES;       // 84-byte blocks: 4-byte aligned with the tensor
+        const uint s = ((k0 >> 5) & 7u) + h, half = s >> 2;
+        j = s & 3u;
+        sc2 = gm_load_u16(blk + half * 8u + j * 2u);
+        dd = *(const uint*)(blk + 80u);
+        typedef u32x4 __attribute__((aligned(4))) u32x4_a4;
+        qa = *(const u32x4_a4*)(blk + 16u + half * 32u);
+        qb = *(const u32x4_a4*)(blk + 32u + half * 32u);
+    }
+    __device__ __forceinline__ void prep() {
+        const float d = f16_bits_to_f32(dd & 0xFFFFu), dmin = f16_bits_to_f32(dd >> 16);
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            const uint sc = (sc2 >> (8 * g)) & 0xFFu;
+            dl[g] = __fmul_rn(d, (float)(sc & 0xFu));
+            ml[g] = __fmul_rn(dmin, (float)(sc >> 4));
+        }
+    }
+    template <int I>
+    __device__ __forceinline__ void part() {      // weights 8 I .. 8 I + 7 of the 32: code bytes 8 I .. of the half
+        const float a = dl[I >> 1], b = ml[I >> 1];
+#pragma unroll
+        for (int v = 0; v < 2; v++) {
+            const uint q = ((I < 2 ? qa : qb)[2 * (I & 1) + v] >> (2u * j)) & 0x03030303u;
+            o[4 * I + 2 * v] = pack2(__fsub_rn(__fmul_rn(a, (float)(q & 0xFFu)), b), __fsub_rn(__fmul_rn(a, (float)((q >> 8) & 0xFFu)), b));
+            o[4 * I + 2 * v + 1] = pack2(__fsub_rn(__fmul_rn(a, (float)((q >> 16) & 0xFFu)), b), __fsub_rn(__fmul_rn(a, (float)(q >> 24)), b));
+        }
+    }
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* p = (u32x4*)(lds_row + h * 64u);
+#pragma unroll
+        for (int i = 0; i < 4; i++) p[i] = (u32x4){o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+    }
+};
+
+// Q3_K: block { u8 hmask[32]; u8 qs[64]; u8 scales[12]; half d; } of 110 bytes (two-byte alignment only);
+// w = (d * (sc - 32)) * (q - (mask bit ? 0 : 4)), bit 4 half + j of hmask[l] belonging to weight (half, j, l) — the bits
+// of `dequant_q3k_f16` (crates/ojas-formats/src/gguf.rs:755-795).
+struct LoaderQ3K {
+    static constexpr int NL = 8;
+    typedef const uchar* Row;
+    static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
+    u32x4 qa, qb, ha, hb;
+    uint r0, r1, r2, d16, s;
+    float dl[2];
+    uint o[16];
+    static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 8) * Q3K_BYTES; }
+    __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
+        const uchar* blk = row + (size_t)(k0 >> 8) * Q3K_BYTES;
+        s = ((k0 >> 5) & 7u) + h;
+        const uint half = s >> 2;
+        ha = gm_load16(blk);
+        hb = gm_load16(blk + 16u);
+        qa = gm_load16(blk + 32u + half * 32u);
+        qb = gm_load16(blk + 48u + half * 32u);
+        r0 = *(const u32_a2*)(blk + 96u);
+        r1 = *(const u32_a2*)(blk + 100u);
+        r2 = *(const u32_a2*)(blk + 104u);
+        d16 = gm_load_u16(blk + 108u);
+    }
+    __device__ __forceinline__ void prep() {
+        const float d = f16_bits_to_f32(d16);
+        const uint half = s >> 2, j = s & 3u;
+#pragma unroll
+        for (int g = 0; g < 2; g++) dl[g] = __fmul_rn(d, (float)q3k_scale6(r0, r1, r2, half * 8u + j * 2u + (uint)g));
+    }
+    __device__ __forceinline__ float value(float a, uint q, uint hbit) const { return __fmul_rn(a, (float)((int)q - (hbit ? 0 : 4))); }
+    template <int I>
+    __device__ __forceinline__ void part() {
+        const float a = dl[I >> 1];
+        const uint j = s & 3u, sh = (s >> 2) * 4u + j;
+#pragma unroll
+        for (int v = 0; v < 2; v++) {
+            const uint q = ((I < 2 ? qa : qb)[2 * (I & 1) + v] >> (2u * j)) & 0x03030303u;
+            const uint hm = ((I < 2 ? ha : hb)[2 * (I & 1) + v] >> sh) & 0x01010101u;
+            o[4 * I + 2 * v] = pack2(value(a, q & 0xFFu, hm & 1u), value(a, (q >> 8) & 0xFFu, (hm >> 8) & 1u));
+            o[4 * I + 2 * v + 1] = pack2(value(a, (q >> 16) & 0xFFu, (hm >> 16) & 1u), value(a, q >> 24, hm >> 24));
+        }
+    }
+    __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
+        u32x4* p = (u32x4*)(lds_row + h * 64u);
+#pragma unroll
+        for (int i = 0; i < 4; i++) p[i] = (u32x4){o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+    }
+};
+
 // Plain f16 rows [N][K] (a tensor the caller keeps in f16, or any block format decoded into scratch by its
 // `dequant_<fmt>_f16` kernel ahead of the product): thread half h owns columns 32h..32h+31 of the slab, 64 bytes.
 struct LoaderF16 {
@@ -716,6 +818,8 @@ GEMM_ENTRIES(q41, LoaderQ41)
 GEMM_ENTRIES(q50, LoaderQ50)
 GEMM_ENTRIES(q51, LoaderQ51)
 GEMM_ENTRIES(mxfp4, LoaderMXFP4)
+GEMM_ENTRIES(q2k, LoaderQ2K)
+GEMM_ENTRIES(q3k, LoaderQ3K)
 
 // Grouped expert products on the same tile (128 tokens x 128 rows): expert e = blockIdx.z % E owns rows e N .. of its
 // tensor and the assignments list[offsets[e] .. offsets[e + 1]); blockIdx.z / E picks the tensor and output of a pair

@@ -2007,10 +2007,10 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g + "_m128", "gemm", 3, 4, f.type, 14, check_gemm, shape_gemm);
         add(g + "_m128_sk", "gemm", 3, 4, f.type, 15, check_gemm, shape_gemm);
     }
-    // IQ4_NL / IQ4_XS, the legacy 32-weight blocks and MXFP4 (f32-activation formats on the decode path) have loaders
+    // IQ4_NL / IQ4_XS, the legacy 32-weight blocks, MXFP4 and Q2_K / Q3_K (f32-activation formats on the decode path) have loaders
     // in the same tile; the IQ4 pair also in its grouped form
     for (uint32_t t : {(uint32_t)OJH_IQ4_NL, (uint32_t)OJH_IQ4_XS, (uint32_t)OJH_Q4_0, (uint32_t)OJH_Q4_1, (uint32_t)OJH_Q5_0,
-                       (uint32_t)OJH_Q5_1, (uint32_t)OJH_MXFP4}) {
+                       (uint32_t)OJH_Q5_1, (uint32_t)OJH_MXFP4, (uint32_t)OJH_Q2_K, (uint32_t)OJH_Q3_K}) {
         std::string g = std::string("gemm_mm_") + ojh_format(t)->tag;
         add(g, "gemm", 3, 4, t, 0, check_gemm, shape_gemm);
         add(g + "_sk", "gemm", 3, 4, t, 1, check_gemm, shape_gemm);

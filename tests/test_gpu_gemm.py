@@ -363,9 +363,9 @@ def test_long_batches_decode_the_rows_ahead_of_the_tile(gpu, orc, pkg, ty, m):
     assert e[0] < TIGHT[0] and e[1] < TIGHT[1], e
 
 
-@pytest.mark.parametrize("ty,tag", [(20, "iq4nl"), (23, "iq4xs"), (2, "q40"), (3, "q41"), (6, "q50"), (7, "q51"), (139, "mxfp4")])
+@pytest.mark.parametrize("ty,tag", [(20, "iq4nl"), (23, "iq4xs"), (2, "q40"), (3, "q41"), (6, "q50"), (7, "q51"), (139, "mxfp4"), (10, "q2k"), (11, "q3k")])
 def test_iq4_rows_on_the_tile_by_name(gpu, orc, pkg, ty, tag):
-    """`gemm_mm_<fmt>{,_m128}` read IQ4_NL / IQ4_XS, Q4_0 / Q4_1 / Q5_0 / Q5_1 and MXFP4 rows through loaders of their own: one-hot activations read back
+    """`gemm_mm_<fmt>{,_m128}` read IQ4_NL / IQ4_XS, Q4_0 / Q4_1 / Q5_0 / Q5_1, MXFP4, Q2_K and Q3_K rows through loaders of their own: one-hot activations read back
     `dequant_to_f16`'s bits of every weight, and a product equals, bit for bit, the plain-f16 tile on the decoded rows
     (`dequant_<fmt>_f16` + `gemm_mm_f16`: the same weights meet the same sums in the same order)."""
     k, n, m = 512, 200, 150
