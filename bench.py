@@ -539,7 +539,7 @@ def extras(gpu, pkg, lin_q) -> dict:
             us = _time(gpu, lambda i: gpu.mm(xb, wf[i % 2], yb, m), 10, 2)
             fb[f"{tag}_M{m}"] = {"us": round(us, 1), "mfma_frac": round(2.0 * m * nb * kb / us / 1e6 / 2500.0, 4)}
         del wf
-    out["float_rows_batch_14336x4096"] = {"activations": "f32 -> f16", "kernels": "gemm_mm_<fmt>{,_m128}{,_sk} (IQ4_NL / IQ4_XS, Q4_0 .. Q5_1, MXFP4 up to 128 tokens) or dequant_<fmt>_f16 + gemm_mm_f16_m128{,_sk}", **fb}
+    out["float_rows_batch_14336x4096"] = {"activations": "f32 -> f16", "kernels": "gemm_mm_<fmt>{,_m128}{,_sk} (IQ4_NL / IQ4_XS, Q4_0 .. Q5_1, MXFP4, Q2_K; Q3_K up to 128 tokens) or dequant_<fmt>_f16 + gemm_mm_f16_m128{,_sk} (Q3_K beyond, the grid codebooks)", **fb}
     # IQ2_XXS as the CPU path multiplies it: int8 activations per 256, integer dots (dot_iq2xxs_q8k)
     wf = [gpu.lin(pkg.IQ2_XXS, n, k, synth.weights(pkg.IQ2_XXS, n, k, "bench", "iq2xxs", "head")) for _ in range(2)]
     us = _time(gpu, lambda i: gpu.mm(x, wf[i % 2], y), 20, 3)

@@ -395,34 +395,56 @@ struct LoaderLegacy {
 
 // MXFP4 (crates/ojas-formats/src/mxfp4.rs:40-58): a 17-byte block { u8 e; u8 qs[16] }, w = 2^(e - 127) * E2M1[code],
 // weight 2j the low and 2j + 1 the high nibble of qs[j]: consecutive weights sit in consecutive nibbles.  The bits of
-// `dequant_mxfp4_f16`.  Blocks start at any byte.
+// `dequant_mxfp4_f16`.  Blocks start at any byte (the tensor itself at a multiple of four: what `ojh_lin_create` and
+// every device allocation give).
 struct LoaderMXFP4 {
-    static constexpr int NL = 2;
+    static constexpr int NL = 3;
     typedef const uchar* Row;
     static __device__ __forceinline__ Row row(const GmSrc& s, uint n, uint K) { return s.w + (size_t)n * row_bytes(K); }
     u32x4 q;
-    uint e8;
+    uint e8, q4, sh;
     float d;
     uint o[16];
     static __device__ __forceinline__ size_t row_bytes(uint K) { return (size_t)(K >> 5) * 17u; }
     __device__ __forceinline__ void load(const uchar* row, uint k0, uint h) {
         const uchar* blk = row + (size_t)((k0 >> 5) + h) * 17u;
-        typedef u32x4 __attribute__((aligned(1))) u32x4_b;
+        // the 16 code bytes start at any byte: the aligned dwords around them, shifted into place after the wait (a
+        // byte-aligned 16-byte load is split into narrow ones).  The fifth dword holds code bytes whenever it is used.
+        typedef u32x4 __attribute__((aligned(4))) u32x4_a4;
+        const uchar* cb = blk + 1u;
+        sh = (uint)((size_t)cb & 3u);
+        const uchar* al = cb - sh;
         e8 = gm_load_u8(blk);
-        q = *(const u32x4_b*)(blk + 1u);
+        q = *(const u32x4_a4*)al;
+        q4 = *(const uint*)(al + (sh ? 16u : 12u));
     }
-    __device__ __forceinline__ void prep() { d = __uint_as_float(e8 << 23); }
-    __device__ __forceinline__ float value(uint c) const {
-        const uint m = c & 7u;
-        const float a = 0.5f * (float)(m < 5u ? m : m == 5u ? 6u : m == 6u ? 8u : 12u);
-        return __fmul_rn(d, __uint_as_float(__float_as_uint(a) | ((c >> 3) << 31)));
+    __device__ __forceinline__ void prep() {
+        d = __uint_as_float(e8 << 23);
+        const uint a0 = q[0], a1 = q[1], a2 = q[2], a3 = q[3];
+        q[0] = __builtin_amdgcn_alignbyte(a1, a0, sh);
+        q[1] = __builtin_amdgcn_alignbyte(a2, a1, sh);
+        q[2] = __builtin_amdgcn_alignbyte(a3, a2, sh);
+        q[3] = __builtin_amdgcn_alignbyte(q4, a3, sh);
+    }
+    // four codes (one per byte) -> twice their E2M1 values as signed bytes (0 1 2 3 4 6 8 12 and their negatives): two
+    // byte permutes over the halves of the table, merged by the sign bit.  (Code 8, -0, comes out as +0: the same
+    // product in every sum.)  d/2 * level is exact, so the one rounding to f16 is the decoder's.
+    static __device__ __forceinline__ uint levels4(uint idx4) {
+        const uint sel = idx4 & 0x07070707u;
+        const uint pos = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, sel);
+        const uint neg = __builtin_amdgcn_perm(0xF4F8FAFCu, 0xFDFEFF00u, sel);
+        const uint m1 = (idx4 >> 3) & 0x01010101u;
+        const uint mask = (m1 << 8) - m1;
+        return (neg & mask) | (pos & ~mask);
     }
     template <int I>
     __device__ __forceinline__ void part() {      // dword I: weights 8 I .. 8 I + 7, nibble by nibble
-        const uint v = q[I];
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-            o[4 * I + j] = pack2(value((v >> (8 * j)) & 15u), value((v >> (8 * j + 4)) & 15u));
+        const float dh = __fmul_rn(d, 0.5f);
+        const uint lo = levels4(q[I] & 0x0F0F0F0Fu), hi = levels4((q[I] >> 4) & 0x0F0F0F0Fu);
+        o[4 * I] = pack2(__fmul_rn(dh, (float)(signed char)lo), __fmul_rn(dh, (float)(signed char)hi));
+        o[4 * I + 1] = pack2(__fmul_rn(dh, (float)(signed char)(lo >> 8)), __fmul_rn(dh, (float)(signed char)(hi >> 8)));
+        o[4 * I + 2] = pack2(__fmul_rn(dh, (float)(signed char)(lo >> 16)), __fmul_rn(dh, (float)(signed char)(hi >> 16)));
+        o[4 * I + 3] = pack2(__fmul_rn(dh, (float)((int)lo >> 24)), __fmul_rn(dh, (float)((int)hi >> 24)));
     }
     __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {
         u32x4* p = (u32x4*)(lds_row + h * 64u);
@@ -513,7 +535,7 @@ struct LoaderQ3K {
 #pragma unroll
         for (int g = 0; g < 2; g++) dl[g] = __fmul_rn(d, (float)q3k_scale6(r0, r1, r2, half * 8u + j * 2u + (uint)g));
     }
-    __device__ __forceinline__ float value(float a, uint q, uint hbit) const { return __fmul_rn(a, (float)((int)q - (hbit ? 0 : 4))); }
+    __device__ __forceinline__ float value(float a, uint c) const { return __fmul_rn(a, __fsub_rn((float)c, 4.0f)); }
     template <int I>
     __device__ __forceinline__ void part() {
         const float a = dl[I >> 1];
@@ -522,8 +544,9 @@ struct LoaderQ3K {
         for (int v = 0; v < 2; v++) {
             const uint q = ((I < 2 ? qa : qb)[2 * (I & 1) + v] >> (2u * j)) & 0x03030303u;
             const uint hm = ((I < 2 ? ha : hb)[2 * (I & 1) + v] >> sh) & 0x01010101u;
-            o[4 * I + 2 * v] = pack2(value(a, q & 0xFFu, hm & 1u), value(a, (q >> 8) & 0xFFu, (hm >> 8) & 1u));
-            o[4 * I + 2 * v + 1] = pack2(value(a, (q >> 16) & 0xFFu, (hm >> 16) & 1u), value(a, q >> 24, hm >> 24));
+            const uint c = q | (hm << 2);       // 0..7 per byte: the weight is c - 4 (an exact difference, then the decoder's one product)
+            o[4 * I + 2 * v] = pack2(value(a, c & 0xFFu), value(a, (c >> 8) & 0xFFu));
+            o[4 * I + 2 * v + 1] = pack2(value(a, (c >> 16) & 0xFFu), value(a, c >> 24));
         }
     }
     __device__ __forceinline__ void flush(uchar* lds_row, uint h) const {

@@ -647,7 +647,7 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
                             ((w->type == OJH_Q2_K || w->type == OJH_Q3_K) && K % 256 == 0);
     const bool iq4_own = dev->iq4_tile && own_loader &&
                          act_asked != OJH_ACT_Q8K && m >= dev->iq4_tile && (!dev->deq_big_m || m < dev->deq_big_m) &&
-                         ((w->type != OJH_MXFP4 && w->type != OJH_Q3_K) || m <= 128) &&   // (Q3_K: eight loads at 2-byte alignment per thread and step, 58 against 67 us at 128 tokens, 96 against 83 at 256)   // (17-byte blocks: its loads are byte-aligned and slow; 14336 x 4096 at 64 / 256 tokens 55 / 97 us against 61 / 80 through the pass)
+                         (w->type != OJH_Q3_K || m <= dev->iq4_tile_cap) &&   // (Q3_K: eight loads at 2-byte alignment per thread and step, 55 against 68 us at 128 tokens, 86 against 82 at 256)
                          K % 64 == 0;
     const bool deq_tile = ((iq4 || grid_fmt) && !iq4_own && !q5_float && act_asked != OJH_ACT_Q8K && deq_min && m >= deq_min || deq_big) &&
                           !dev->no_scratch && K % 64 == 0 && (uint64_t)N * K / f->weights <= 0x7FFFFFFFu / 64;

@@ -54,7 +54,7 @@ def test_router_sweep(gpu, orc, pkg, ty, n, k, m, accum):
     # f16 tile (IQ2_XXS / IQ3_XXS keep the int8 kernels where OJH_ACT_Q8K is asked for: here from 32 tokens)
     # (IQ4_NL / IQ4_XS, Q4_0 .. Q5_1, MXFP4, Q2_K and Q3_K rows, which the tile reads through loaders of its own, from 5 tokens on
     # every shape)
-    own = ty in (20, 23, 2, 3, 6, 7, 139, 10, 11) and (ty not in (23, 10, 11) or k % 256 == 0) and (ty not in (139, 11) or m <= 128)
+    own = ty in (20, 23, 2, 3, 6, 7, 139, 10, 11) and (ty not in (23, 10, 11) or k % 256 == 0) and (ty != 11 or m <= 128)
     if ty not in (Q8_0, Q4_K, Q5_K, Q6_K) and k % 64 == 0 and m >= (5 if own or n * k >= (32 << 20) else 9) and (m < 32 or ty in FLOAT_ROWS):
         tile = True
     if tile:
