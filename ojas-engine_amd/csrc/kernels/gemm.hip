@@ -395,8 +395,7 @@ struct LoaderLegacy {
 
 // MXFP4 (crates/ojas-formats/src/mxfp4.rs:40-58): a 17-byte block { u8 e; u8 qs[16] }, w = 2^(e - 127) * E2M1[code],
 // weight 2j the low and 2j + 1 the high nibble of qs[j]: consecutive weights sit in consecutive nibbles.  The bits of
-// `dequant_mxfp4_f16`.  Blocks start at any byte (the tensor itself at a multiple of four: what `ojh_lin_create` and
-// every device allocation give).
+// `dequant_mxfp4_f16`.  Blocks start at any byte.
 struct LoaderMXFP4 {
     static constexpr int NL = 3;
     typedef const uchar* Row;
@@ -843,6 +842,132 @@ GEMM_ENTRIES(q51, LoaderQ51)
 GEMM_ENTRIES(mxfp4, LoaderMXFP4)
 GEMM_ENTRIES(q2k, LoaderQ2K)
 GEMM_ENTRIES(q3k, LoaderQ3K)
+
+// ------------------------------------------------------------------ few tokens: weights straight into the matrix operand
+// The tile above stages 128 rows x 64 weights through LDS for 128 token columns; with a handful of tokens seven eighths of
+// its matrix work multiply padding and every K step still pays the staging and a barrier (14336 x 4096 at 8 .. 64 tokens:
+// 32 - 36 us whatever the format).  Here a workgroup owns 16 rows, its waves take the 128-weight chunks of K in turn, and
+// nothing goes through LDS but the final sums: v_mfma_f32_16x16x32_f16 with A = 16 tokens, B = 16 rows; lane (i, g) of
+// either operand holds 8 consecutive positions of K group g.  The order of K inside an instruction is free as long as both
+// operands agree, so lane (n, g) decodes the whole 32-weight block g of the chunk for row n (the per-thread loaders of the
+// tile: one or two wide loads) and feeds it to four instructions, 8 weights each; lane (m, g) reads the matching 64 bytes
+// of token m.  Up to 16 TG tokens per launch (TG accumulators); partial sums of the waves meet in LDS in wave order.
+//   gemm_few_<fmt>{,_r4}_t{1,2,4}(xh, w, y, K, N, accum, M)     grid [ceil(N / 16 RG),1,1] x 256 (or 512 where RG TG <= 4),
+//   K a multiple of 128, M <= 16 TG; `_r4`: RG = 4 groups of 16 rows per workgroup
+typedef float float4v __attribute__((ext_vector_type(4)));
+template <int J, class L>
+__device__ __forceinline__ half8 gm_frag(const L& ld) {
+    return __builtin_bit_cast(half8, (u32x4){ld.o[4 * J], ld.o[4 * J + 1], ld.o[4 * J + 2], ld.o[4 * J + 3]});
+}
+template <int J>
+__device__ __forceinline__ half8 gm_frag(const LoaderF16& ld) { return __builtin_bit_cast(half8, ld.q[J]); }
+
+template <class Loader, int TG, int RG, class TM>
+__device__ __forceinline__ void gemm_few_body(const ushort* __restrict__ xh, const uchar* __restrict__ w, float* __restrict__ y,
+                                              uint K, uint N, uint accum, uint M, const TM tm) {
+    // RG groups of 16 rows per workgroup share every token fragment a lane reads (the tokens' bytes, re-read by every
+    // workgroup, are most of the traffic of the 16-row form: 14336 rows x 16 tokens of K = 4096 read them 896 times)
+    __shared__ float red[RG * TG > 4 ? 4 : 8][RG * TG][256];     // (eight waves only where that stays within 32 KB)
+    const uint tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, nw = blockDim.x >> 6;
+    const uint i16 = lane & 15u, g = lane >> 4;
+    const uint n0 = blockIdx.x * (16u * RG);
+    const size_t rb = Loader::row_bytes(K);
+    const uchar* wrow[RG];
+#pragma unroll
+    for (int r = 0; r < RG; r++) wrow[r] = w + (size_t)min(n0 + 16u * r + i16, N - 1u) * rb;
+    const ushort* xrow[TG];
+#pragma unroll
+    for (int tg = 0; tg < TG; tg++) xrow[tg] = xh + (size_t)tm.in_row(min(16u * tg + i16, M - 1u)) * K + g * 32u;
+    float4v acc[RG][TG];
+#pragma unroll
+    for (int r = 0; r < RG; r++)
+#pragma unroll
+        for (int tg = 0; tg < TG; tg++) acc[r][tg] = (float4v){0.0f, 0.0f, 0.0f, 0.0f};
+    const uint nchunk = K >> 7;
+    Loader ld0, ld1;
+    // one row group of one chunk: the next group's (or the next chunk's first group's) block is asked for first
+#define GF_GROUP(CUR, NXT, R, NEXT_ROW, NEXT_C)                                                                   \
+    do {                                                                                                          \
+        if ((NEXT_C) < nchunk) NXT.load(NEXT_ROW, (NEXT_C) * 128u + g * 32u, 0u);                                 \
+        gm_fence();                                                                                               \
+        CUR.prep();                                                                                               \
+        CUR.template part<0>(); CUR.template part<1>(); CUR.template part<2>(); CUR.template part<3>();           \
+        _Pragma("unroll") for (int tg = 0; tg < TG; tg++) {                                                      \
+            acc[R][tg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv[tg][0], gm_frag<0>(CUR), acc[R][tg], 0, 0, 0);  \
+            acc[R][tg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv[tg][1], gm_frag<1>(CUR), acc[R][tg], 0, 0, 0);  \
+            acc[R][tg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv[tg][2], gm_frag<2>(CUR), acc[R][tg], 0, 0, 0);  \
+            acc[R][tg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv[tg][3], gm_frag<3>(CUR), acc[R][tg], 0, 0, 0);  \
+        }                                                                                                         \
+    } while (0)
+    uint c = wave;
+    if (c < nchunk) ld0.load(wrow[0], c * 128u + g * 32u, 0u);
+    for (; c < nchunk; c += nw) {
+        half8 xv[TG][4];
+#pragma unroll
+        for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) xv[tg][j] = *(const half8*)(xrow[tg] + c * 128u + 8u * j);
+        if (RG == 1) {
+            // (two chunks per trip so that the loaders alternate by name)
+            GF_GROUP(ld0, ld1, 0, wrow[0], c + nw);
+            c += nw;
+            if (c < nchunk) {
+#pragma unroll
+                for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) xv[tg][j] = *(const half8*)(xrow[tg] + c * 128u + 8u * j);
+                GF_GROUP(ld1, ld0, 0, wrow[0], c + nw);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < RG; r += 2) {
+                GF_GROUP(ld0, ld1, r, wrow[r + 1 < RG ? r + 1 : 0], c);
+                GF_GROUP(ld1, ld0, r + 1 < RG ? r + 1 : 0, wrow[r + 2 < RG ? r + 2 : 0], r + 2 < RG ? c : c + nw);
+            }
+        }
+    }
+#undef GF_GROUP
+    // D: lane (n = lane % 16, g) holds tokens 4 g + v of its group against row n
+#pragma unroll
+    for (int r = 0; r < RG; r++)
+#pragma unroll
+        for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) red[wave][r * TG + tg][(g * 4u + v) * 16u + i16] = acc[r][tg][v];
+    __syncthreads();
+    for (uint e = tid; e < (uint)(RG * TG) * 256u; e += blockDim.x) {
+        const uint rt = e >> 8, r = rt / TG, tg = rt % TG, idx = e & 255u, tok = 16u * tg + (idx >> 4), row = n0 + 16u * r + (idx & 15u);
+        float sum = red[0][rt][idx];
+        for (uint k = 1; k < nw; k++) sum += red[k][rt][idx];
+        if (tok < M && row < N) {
+            float* o = y + (size_t)tm.out_row(tok) * N + row;
+            *o = accum ? *o + sum : sum;
+        }
+    }
+}
+
+#define GEMM_FEW_ENTRY(FMT, LOADER, SUF, TG, RG)                                                                  \
+    extern "C" __global__ void __launch_bounds__(512) gemm_few_##FMT##SUF(                                        \
+        const ushort* xh, const uchar* w, float* y, uint K, uint N, uint accum, uint M) {                         \
+        gemm_few_body<LOADER, TG, RG, GmDense>(xh, w, y, K, N, accum, M, GmDense()); }
+#define GEMM_FEW_ENTRIES(FMT, LOADER)                                                                             \
+    GEMM_FEW_ENTRY(FMT, LOADER, _t1, 1, 1)                                                                        \
+    GEMM_FEW_ENTRY(FMT, LOADER, _t2, 2, 1)                                                                        \
+    GEMM_FEW_ENTRY(FMT, LOADER, _t4, 4, 1)                                                                        \
+    GEMM_FEW_ENTRY(FMT, LOADER, _r4_t1, 1, 4)                                                                     \
+    GEMM_FEW_ENTRY(FMT, LOADER, _r4_t2, 2, 4)                                                                     \
+    GEMM_FEW_ENTRY(FMT, LOADER, _r4_t4, 4, 4)
+GEMM_FEW_ENTRIES(q8_0, LoaderQ80)
+GEMM_FEW_ENTRIES(f16, LoaderF16)
+GEMM_FEW_ENTRIES(iq4nl, LoaderIQ4NL)
+GEMM_FEW_ENTRIES(iq4xs, LoaderIQ4XS)
+GEMM_FEW_ENTRIES(q40, LoaderQ40)
+GEMM_FEW_ENTRIES(q41, LoaderQ41)
+GEMM_FEW_ENTRIES(q50, LoaderQ50)
+GEMM_FEW_ENTRIES(q51, LoaderQ51)
+GEMM_FEW_ENTRIES(mxfp4, LoaderMXFP4)
+GEMM_FEW_ENTRIES(q2k, LoaderQ2K)
+GEMM_FEW_ENTRIES(q3k, LoaderQ3K)
 
 // Grouped expert products on the same tile (128 tokens x 128 rows): expert e = blockIdx.z % E owns rows e N .. of its
 // tensor and the assignments list[offsets[e] .. offsets[e + 1]); blockIdx.z / E picks the tensor and output of a pair

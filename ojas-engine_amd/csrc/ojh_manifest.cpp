@@ -1335,6 +1335,45 @@ static int shape_gemm(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t 
     return OJH_OK;
 }
 
+// gemm_few_<fmt>{,_r4}_t{1,2,4}(xh, w, y, K, N, accum, M): grid [ceil(N / 16 RG),1,1] x 256 (or 512 where RG TG <= 4); K a
+// multiple of 128 (and whole blocks of the format); up to 16 TG tokens (`rows_per_wave` = 16 RG + TG)
+static int check_gemm_few(const ojh_kernel_spec *s, const uint32_t *c, const uint32_t grid[3],
+                          const uint32_t block[3], size_t need[16], size_t align[16]) {
+    const uint32_t K = c[0], N = c[1], M = c[3], TG = (uint32_t)s->rows_per_wave & 15u, RG = (uint32_t)s->rows_per_wave >> 4;
+    static const ojh_block_format plain_f16 = {OJH_F16, 2, 1, "f16"};
+    const ojh_block_format *f = &plain_f16;
+    int rc;
+    if (s->type == OJH_F16) {
+        if (!K || !N) return ojh_fail(OJH_ERR_ARG, "%s: K=%u N=%u", s->name, K, N);
+    } else if ((rc = check_kn(s, K, N, &f))) {
+        return rc;
+    }
+    if (K % 128) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a multiple of 128", s->name, K);
+    if (!M || M > 16 * TG) return ojh_fail(OJH_ERR_ARG, "%s: M=%u, takes 1 to %u tokens", s->name, M, 16 * TG);
+    if (block[0] != 256 && !(block[0] == 512 && RG * TG <= 4))
+        return ojh_fail(OJH_ERR_ARG, "%s: block must be 256%s threads", s->name, RG * TG <= 4 ? " or 512" : "");
+    if (block[1] != 1 || block[2] != 1) return ojh_fail(OJH_ERR_ARG, "%s: block must be [x,1,1]", s->name);
+    if (grid[0] != (N + 16 * RG - 1) / (16 * RG) || grid[1] != 1 || grid[2] != 1)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [%u,1,1]", s->name, (N + 16 * RG - 1) / (16 * RG));
+    need[0] = (size_t)M * K * 2;
+    need[1] = (size_t)N * (K / f->weights) * f->bytes;
+    need[2] = (size_t)M * N * 4;
+    align[0] = 16;
+    align[1] = s->type == OJH_F16 ? 16 : ojh_block_align(f);
+    align[2] = 4;
+    return OJH_OK;
+}
+static int shape_gemm_few(const ojh_kernel_spec *s, const ojh_device *dev, uint32_t, uint32_t N, uint32_t,
+                          uint32_t grid[3], uint32_t block[3]) {
+    const uint32_t cus = dev ? (uint32_t)dev->prop.multiProcessorCount : 256u;
+    const uint32_t TG = (uint32_t)s->rows_per_wave & 15u, RG = (uint32_t)s->rows_per_wave >> 4;
+    grid[0] = (N + 16 * RG - 1) / (16 * RG);
+    grid[1] = grid[2] = 1;
+    block[0] = grid[0] < 2 * cus && RG * TG <= 4 ? 512 : 256;     // few workgroups: eight waves share their K
+    block[1] = block[2] = 1;
+    return OJH_OK;
+}
+
 // LDS of the moe_*_mt entries: 16 token rows, their scales and split sums, a block of zeros, the pass's assignments
 uint64_t ojh_moe_mt_lds(uint32_t K) { return 16 * ((uint64_t)K + 32) + K / 4 + K + 256 + 64; }
 
@@ -2018,6 +2057,16 @@ static std::vector<ojh_kernel_spec> build_manifest() {
         add(g + "_m128_sk", "gemm", 3, 4, t, 15, check_gemm, shape_gemm);
         if (t == OJH_IQ4_NL || t == OJH_IQ4_XS)
             add(std::string("moe_mm_") + ojh_format(t)->tag, "gemm", 7, 5, t, 0, check_moe_mm, shape_moe_mm);
+    }
+    // a few tokens: 16 rows per workgroup, the weights decoded straight into the matrix operand
+    for (uint32_t t : {(uint32_t)OJH_Q8_0, (uint32_t)OJH_F16, (uint32_t)OJH_IQ4_NL, (uint32_t)OJH_IQ4_XS, (uint32_t)OJH_Q4_0,
+                       (uint32_t)OJH_Q4_1, (uint32_t)OJH_Q5_0, (uint32_t)OJH_Q5_1, (uint32_t)OJH_MXFP4, (uint32_t)OJH_Q2_K,
+                       (uint32_t)OJH_Q3_K}) {
+        const std::string g = std::string("gemm_few_") + (t == OJH_Q8_0 ? "q8_0" : t == OJH_F16 ? "f16" : ojh_format(t)->tag);
+        for (int tg : {1, 2, 4}) {
+            add(g + "_t" + std::to_string(tg), "gemm", 3, 4, t, 16 + tg, check_gemm_few, shape_gemm_few);
+            add(g + "_r4_t" + std::to_string(tg), "gemm", 3, 4, t, 64 + tg, check_gemm_few, shape_gemm_few);
+        }
     }
     // plain f16 rows on the same tile: what every format without a tile of its own is decoded into ahead of a batch
     add("gemm_mm_f16", "gemm", 3, 4, OJH_F16, 0, check_gemm, shape_gemm);

@@ -699,6 +699,26 @@ extern "C" int ojh_mm(ojh_device *dev, const ojh_buf *x, size_t x_off, int x_dty
             if (!tall && K >= 1024 && (dev->gemm_bdk == 2 || (dev->gemm_bdk == 1 && z_bd >= 2 && (K <= 8192 || z_bd >= 4))))
                 base = "gemm_mm_q4kl_bdk";
         }
+        // A few tokens on the formats whose 32 weights per thread come out of one or two wide loads: 16 (or 64) rows per
+        // workgroup with the weights decoded straight into the matrix operand, no LDS staging, no barrier per K step
+        // (`gemm_few_*`; 14336 x 4096 at 8 / 16 / 32 tokens, kernel alone: IQ4_XS 14 / 15 / 23 us against 30 of the tile,
+        // Q8_0 26 / 28 / 32 against 36; 4096 x 4096 IQ4_XS 7 / 9 / 11 against 12 .. 14).  Four row groups per workgroup where
+        // that still gives most CUs a workgroup: the tokens' bytes, re-read by every workgroup, are most of its traffic.
+        // (with 16 rows per workgroup a long K costs more: up to 16 tokens there; Q8_0, twice the bytes per weight, only
+        // where the tile is no better — 4096 x 14336 at 32 tokens: IQ4_XS 34 against 31 us, Q8_0 48 against 36)
+        const uint32_t cus = (uint32_t)dev->prop.multiProcessorCount;
+        const bool r4 = (uint64_t)(N + 63) / 64 * 4 >= 3ull * cus;
+        const uint32_t few_cap = r4 ? dev->gemm_few : K > 4096 ? (w->type == OJH_Q8_0 ? 0u : 16u) : w->type == OJH_Q8_0 ? 16u : dev->gemm_few;
+        if (dev->gemm_few && !xl && !deq_tile && (own_loader || w->type == OJH_Q8_0) && m <= few_cap && m <= 64 && K % 128 == 0) {
+            const std::string few = std::string("gemm_few_") + (w->type == OJH_Q8_0 ? "q8_0" : f->tag) + (r4 ? "_r4" : "") +
+                                    (m <= 16 ? "_t1" : m <= 32 ? "_t2" : "_t4");
+            uint32_t fg[3], fb[3], eg[3] = {conv_blocks, 1, 1};
+            if ((rc = ojh_launch_shape(dev, few.c_str(), K, N, m, fg, fb))) return rc;
+            if ((rc = ojh_launch(dev, x_dtype == OJH_X_BF16 ? "copy_bf16_half" : "copy_f32_half", {at(x, x_off), xh->ptr},
+                                 {n_el}, eg, block)))
+                return rc;
+            return ojh_launch(dev, few.c_str(), {xh->ptr, wp, yp}, {K, N, (uint32_t)(accum != 0), m}, fg, fb);
+        }
         uint32_t sg[3], sb[3];
         if ((rc = ojh_launch_shape(dev, (base + "_sk").c_str(), K, N, m, sg, sb))) return rc;
         // (a forced split counts before the tile is chosen, so that what follows sees the split that will run)

@@ -396,3 +396,35 @@ def test_iq4_rows_on_the_tile_by_name(gpu, orc, pkg, ty, tag):
     assert np.array_equal(outs["gemm_mm_%s_m128" % tag], outs["gemm_mm_f16_m128"])
     ref = x.astype(np.float32).reshape(m, k).astype(np.float64) @ want.astype(np.float64).T
     assert peak_err(outs["gemm_mm_" + tag].view(np.float32).reshape(m, n), ref) <= 1e-5
+
+
+@pytest.mark.parametrize("ty,tag", [(8, "q8_0"), (20, "iq4nl"), (23, "iq4xs"), (2, "q40"), (7, "q51"), (139, "mxfp4"), (10, "q2k"),
+                                    (11, "q3k")])
+@pytest.mark.parametrize("m,k,n,accum,threads", [(1, 256, 16, False, 256), (5, 384, 200, False, 256), (16, 512, 37, True, 512),
+                                                 (17, 1024, 130, False, 256), (33, 2048, 64, False, 512), (64, 768, 48, True, 256)])
+def test_few_token_kernel_by_name(gpu, orc, pkg, ty, tag, m, k, n, accum, threads):
+    """`gemm_few_<fmt>{,_r4}_t{1,2,4}(xh, w, y, K, N, accum, M)`: 16 or 64 rows per workgroup, the K chunks dealt to its 4 or 8 waves,
+    up to 16 / 32 / 64 tokens.  Every output against the f64 product of `dequant_to_f16`'s weights with the f16 activations;
+    nothing written past row N or token M; more tokens than the entry holds are refused."""
+    if ty in (23, 10, 11) and k % 256:
+        pytest.skip("rows of this format are whole super-blocks of 256")
+    raw = pkg.synth.weights(ty, n, k, "few", tag, n, k)
+    wf = orc.dequant_to_f16(raw, ty, n * k).view(np.float16).astype(np.float64).reshape(n, k)
+    x = pkg.synth.normal_f32(m * k, "few", "x", m, k).astype(np.float16)
+    want = x.astype(np.float64).reshape(m, k) @ wf.T
+    y0 = pkg.synth.normal_f32(m * n, "few", "y0", m, n) if accum else np.full(m * n, 777.25, np.float32)
+    gpu.ensure_family("gemm")
+    wd, xd = gpu.upload_bytes(raw), gpu.upload_bytes(x.view(np.uint8))
+    tg = 1 if m <= 16 else 2 if m <= 32 else 4
+    for t, rg in ((tg, 1), (4, 1), (tg, 4), (4, 4)):
+        yd = gpu.upload(np.concatenate([y0, np.full(n, 4242.5, np.float32)]))
+        gpu.dispatch(gpu.begin(), "gemm_few_%s%s_t%d" % (tag, "_r4" if rg == 4 else "", t), [(xd, 0), (wd, 0), (yd, 0)], [k, n, int(accum), m],
+                     [(n + 16 * rg - 1) // (16 * rg), 1, 1], [threads if rg * t <= 4 else 256, 1, 1])
+        got = gpu.read(yd, m * n + n)
+        assert np.all(got[m * n:] == np.float32(4242.5)), "wrote past the last token"
+        got = got[:m * n].reshape(m, n) - (y0.reshape(m, n) if accum else 0.0)
+        assert peak_err(got, want) <= (2e-5 if accum else 2e-6), (t, rg)
+    if tg < 4:
+        with pytest.raises(pkg.OjasHipError, match="tokens"):
+            gpu.dispatch(gpu.begin(), "gemm_few_%s_t%d" % (tag, tg), [(xd, 0), (wd, 0), (yd, 0)], [k, n, 0, 16 * tg + 1], [(n + 15) // 16, 1, 1],
+                         [256, 1, 1])
