@@ -999,6 +999,30 @@ MOE_MM_ENTRY(iq4nl, LoaderIQ4NL, (size_t)(K / 32u) * IQ4NL_BYTES)
 MOE_MM_ENTRY(iq4xs, LoaderIQ4XS, (size_t)(K / 256u) * IQ4XS_BYTES)
 MOE_MM_ENTRY(f16, LoaderF16, (size_t)K * 2u)          // (experts decoded into f16 beforehand: formats without a loader here)
 
+// The same grouped products for experts that received a few dozen tokens, on the few-token kernel (64 rows per workgroup,
+// 32 assignments per pass, weights decoded straight into the matrix operand): passes blockIdx.y, + gridDim.y, .. of the expert.
+//   moe_few_<fmt>(xh, w0, w1, y0, y1, offsets, list, K, N, NA, E, DIV)    grid [ceil(N / 64), 1 .., E or 2 E] x 256, K % 128 == 0
+#define MOE_FEW_ENTRY(FMT, LOADER, ROWBYTES)                                                                      \
+    extern "C" __global__ void __launch_bounds__(256) moe_few_##FMT(                                              \
+        const ushort* xh, const uchar* w0, const uchar* w1, float* y0, float* y1, const uint* offsets,            \
+        const uint* list, uint K, uint N, uint NA, uint E, uint DIV) {                                            \
+        const uint e = blockIdx.z % E, second = blockIdx.z / E;                                                   \
+        const uint a0 = min(offsets[e], NA), a1 = min(offsets[e + 1], NA);                                        \
+        if (a0 >= a1) return;                                                                                     \
+        const uchar* w = (second ? w1 : w0) + (size_t)e * N * (ROWBYTES);                                         \
+        for (uint ty = blockIdx.y; ty * 32u < a1 - a0; ty += gridDim.y) {                                         \
+            GmList tm;                                                                                            \
+            tm.lst = list + a0 + ty * 32u;                                                                        \
+            tm.last = NA - 1u;                                                                                    \
+            tm.div = DIV;                                                                                         \
+            gemm_few_body<LOADER, 2, 4, GmList>(xh, w, second ? y1 : y0, K, N, 0u, min(32u, a1 - a0 - ty * 32u), tm); \
+            __syncthreads();                                                                                      \
+        }                                                                                                         \
+    }
+MOE_FEW_ENTRY(q8_0, LoaderQ80, (size_t)(K / 32u) * 34u)
+MOE_FEW_ENTRY(iq4nl, LoaderIQ4NL, (size_t)(K / 32u) * IQ4NL_BYTES)
+MOE_FEW_ENTRY(iq4xs, LoaderIQ4XS, (size_t)(K / 256u) * IQ4XS_BYTES)
+
 // act16[i] = f16(silu(g[i]) * u[i]): what the grouped gate / up launch hands to the grouped down launch
 // (crates/ojas-cuda/src/kernels/moe.rs:75-102 forms the same product in f32)
 extern "C" __global__ void __launch_bounds__(256)

@@ -1713,10 +1713,11 @@ static int check_moe_mm(const ojh_kernel_spec *s, const uint32_t *c, const uint3
     } else if ((rc = check_kn(s, K, N, &f))) {
         return rc;
     }
-    if (K % 64) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a multiple of 64", s->name, K);
+    const uint32_t bn = s->rows_per_wave == 2 ? 64u : 128u, bk = s->rows_per_wave == 2 ? 128u : 64u;   // (2: the `moe_few_*` entries)
+    if (K % bk) return ojh_fail(OJH_ERR_ARG, "%s: K=%u must be a multiple of %u", s->name, K, bk);
     if (!NA || !E || !DIV) return ojh_fail(OJH_ERR_ARG, "%s: NA=%u E=%u DIV=%u", s->name, NA, E, DIV);
-    if (grid[0] != (N + 127) / 128 || !grid[1] || grid[1] > 65535 || (grid[2] != E && grid[2] != 2 * E) || grid[2] > 65535)
-        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/128), token tiles (any, up to 65535), E or 2 E]", s->name);
+    if (grid[0] != (N + bn - 1) / bn || !grid[1] || grid[1] > 65535 || (grid[2] != E && grid[2] != 2 * E) || grid[2] > 65535)
+        return ojh_fail(OJH_ERR_ARG, "%s: grid must be [ceil(N/%u), token tiles (any, up to 65535), E or 2 E]", s->name, bn);
     const bool pair = grid[2] == 2 * E;
     const size_t wbytes = (size_t)E * N * (K / f->weights) * f->bytes;
     need[0] = ((size_t)(NA - 1) / DIV + 1) * K * 2;
@@ -1735,7 +1736,7 @@ static int check_moe_mm(const ojh_kernel_spec *s, const uint32_t *c, const uint3
 }
 static int shape_moe_mm(const ojh_kernel_spec *s, const ojh_device *, uint32_t, uint32_t N, uint32_t M,
                         uint32_t grid[3], uint32_t block[3]) {
-    grid[0] = s->rows_per_wave == 1 ? (uint32_t)(((uint64_t)(N ? N : 1) + 1023) / 1024) : (N + 127) / 128;   // (act: N = elements)
+    grid[0] = s->rows_per_wave == 1 ? (uint32_t)(((uint64_t)(N ? N : 1) + 1023) / 1024) : s->rows_per_wave == 2 ? (N + 63) / 64 : (N + 127) / 128;   // (act: N = elements)
     grid[1] = 1;
     grid[2] = s->rows_per_wave == 1 ? 1 : (M ? M : 1);     // M = experts
     block[0] = 256;
@@ -2151,6 +2152,9 @@ static std::vector<ojh_kernel_spec> build_manifest() {
     // glue: `type` carries (input element bytes << 8 | output element bytes)
     add("moe_mm_q8_0", "gemm", 7, 5, OJH_Q8_0, 0, check_moe_mm, shape_moe_mm);
     add("moe_mm_f16", "gemm", 7, 5, OJH_F16, 0, check_moe_mm, shape_moe_mm);
+    add("moe_few_q8_0", "gemm", 7, 5, OJH_Q8_0, 2, check_moe_mm, shape_moe_mm);
+    add("moe_few_iq4nl", "gemm", 7, 5, OJH_IQ4_NL, 2, check_moe_mm, shape_moe_mm);
+    add("moe_few_iq4xs", "gemm", 7, 5, OJH_IQ4_XS, 2, check_moe_mm, shape_moe_mm);
     add("moe_act_half", "gemm", 3, 1, 0, 1, check_moe_mm, shape_moe_mm);
     add("copy_f32_half", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);
     add("copy_f32_bf16", "glue", 2, 1, (4u << 8) | 2u, 0, check_elementwise, shape_elementwise);

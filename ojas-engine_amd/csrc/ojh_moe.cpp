@@ -3,6 +3,7 @@
 // graph_decode.rs:441-499, prefill graph_chunk.rs:564-628; CPU crates/ojas-cpu/src/cpu_glm.rs:519-597):
 // router -> group assignments by expert -> gate/up (+SiLU*mul) -> quantize -> down -> weighted sum.
 #include "ojh_internal.h"
+#include <cstring>
 #include <string>
 
 static int ensure(ojh_device *dev, const char *family) {
@@ -163,12 +164,20 @@ extern "C" int ojh_moe_ffn(ojh_device *dev, const ojh_buf *x, uint32_t T, uint32
             uint32_t gc[3] = {(n_x / 8 + 255) / 256 + 1, 1, 1};
             if ((rc = ojh_launch(dev, "copy_f32_half", {x->ptr, xh->ptr}, {n_x}, gc, b256))) return rc;
             uint32_t tiles = (T + 127) / 128;
-            uint32_t gg[3] = {(n_ff + 127) / 128, tiles, 2 * E};
+            // experts that received a few dozen tokens: 32 assignments per pass on the few-token kernel, 64 rows per
+            // workgroup (two passes in the grid, the rest by its loop)
+            const bool few_gu = dev->moe_few && (uint64_t)NA8 <= (uint64_t)dev->moe_few * E && d % 128 == 0 && !strncmp(tile_gu, "moe_mm_", 7) && strcmp(tile_gu, "moe_mm_f16");
+            const bool few_dn = dev->moe_few && (uint64_t)NA8 <= (uint64_t)dev->moe_few * E && n_ff % 128 == 0 && !strncmp(tile_dn, "moe_mm_", 7) && strcmp(tile_dn, "moe_mm_f16");
+            const std::string few_gu_name = std::string("moe_few_") + (tile_gu + 7), few_dn_name = std::string("moe_few_") + (tile_dn + 7);
+            if (few_gu) tile_gu = few_gu_name.c_str();
+            if (few_dn) tile_dn = few_dn_name.c_str();
+            const uint32_t passes = T < 32 ? 1u : 2u;
+            uint32_t gg[3] = {few_gu ? (n_ff + 63) / 64 : (n_ff + 127) / 128, few_gu ? passes : tiles, 2 * E};
             if ((rc = ojh_launch(dev, tile_gu, {xh->ptr, wg, wu, gv->ptr, uv->ptr, offsets, list}, {d, n_ff, NA8, E, ksel}, gg, b256)))
                 return rc;
             uint32_t ga[3] = {(n_a / 8 + 255) / 256 + 1, 1, 1};
             if ((rc = ojh_launch(dev, "moe_act_half", {gv->ptr, uv->ptr, a16->ptr}, {n_a}, ga, b256))) return rc;
-            uint32_t gd[3] = {(d + 127) / 128, tiles, E};
+            uint32_t gd[3] = {few_dn ? (d + 63) / 64 : (d + 127) / 128, few_dn ? passes : tiles, E};
             if ((rc = ojh_launch(dev, tile_dn, {a16->ptr, wd, nullptr, dv->ptr, nullptr, offsets, list}, {n_ff, d, NA8, E, 1u}, gd, b256)))
                 return rc;
             uint64_t n = (uint64_t)T * d;

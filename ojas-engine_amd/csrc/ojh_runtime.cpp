@@ -98,6 +98,7 @@ extern "C" int ojh_open(int ordinal, ojh_device **out) {
     if (const char *r = getenv("OJAS_HIP_IQ4_TILE")) d->iq4_tile = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_IQ4_TILE_CAP")) d->iq4_tile_cap = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_GEMM_FEW")) d->gemm_few = (uint32_t)atoi(r);
+    if (const char *r = getenv("OJAS_HIP_MOE_FEW")) d->moe_few = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_MOE_DOWN_GS")) d->moe_down_gs = (uint32_t)atoi(r);
     if (const char *r = getenv("OJAS_HIP_Q8ROW_DEC")) d->q8row_dec = atoi(r) != 0;
     if (const char *r = getenv("OJAS_HIP_Q8ROW_SPLIT")) d->q8row_split = (uint32_t)atoi(r);

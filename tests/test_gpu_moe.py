@@ -538,13 +538,15 @@ def test_q80_experts_in_batches_on_the_grouped_matrix_tile(gpu, orc, pkg, T, E, 
         assert peak_err(outs[pkg.ACT_FLOAT][t], want[0]) <= 2e-5, t
 
 
-@pytest.mark.parametrize("fmt,tile", [(Q8_0, "moe_mm_q8_0"), (IQ4_NL, "moe_mm_iq4nl"), (IQ4_XS, "moe_mm_iq4xs")])
+@pytest.mark.parametrize("fmt,tile", [(Q8_0, "moe_mm_q8_0"), (IQ4_NL, "moe_mm_iq4nl"), (IQ4_XS, "moe_mm_iq4xs"),
+                                      (Q8_0, "moe_few_q8_0"), (IQ4_NL, "moe_few_iq4nl"), (IQ4_XS, "moe_few_iq4xs")])
 def test_grouped_f16_tile_by_name(gpu, orc, pkg, fmt, tile):
     """`moe_mm_<fmt>(xh, w0, w1, y0, y1, offsets, list, K, N, NA, E, DIV)`: a pair of tensors in one launch (gate and up:
     assignment a reads token a / DIV) and a single tensor (down: DIV = 1, NULL second tensor); an empty expert; any
     number of token tiles in the grid gives the same bits; every row against the f64 product of the exact block values
     with the f16-rounded activations."""
     E, n, k, div = 3, 200, 256, 2
+    bn = 64 if tile.startswith("moe_few") else 128      # rows per workgroup (the few-token form: 32 assignments per pass)
     counts = [150, 0, 38]
     na = sum(counts)
     tokens = na // div
@@ -561,7 +563,7 @@ def test_grouped_f16_tile_by_name(gpu, orc, pkg, fmt, tile):
     for tiles in (1, 2, 5):
         y0d, y1d = (gpu.upload(np.full(na * n + n, 777.25, np.float32)) for _ in range(2))
         gpu.dispatch(gpu.begin(), tile, [(xd, 0), (w0d, 0), (w1d, 0), (y0d, 0), (y1d, 0), (od, 0), (ld, 0)],
-                     [k, n, na, E, div], [(n + 127) // 128, tiles, 2 * E], [256, 1, 1])
+                     [k, n, na, E, div], [(n + bn - 1) // bn, tiles, 2 * E], [256, 1, 1])
         g0, g1 = gpu.read(y0d, na * n + n), gpu.read(y1d, na * n + n)
         assert np.all(g0[na * n:] == np.float32(777.25)) and np.all(g1[na * n:] == np.float32(777.25))
         seen.append(np.stack([g0[:na * n], g1[:na * n]]).reshape(2, na, n).view(np.uint32).copy())
@@ -578,7 +580,7 @@ def test_grouped_f16_tile_by_name(gpu, orc, pkg, fmt, tile):
     xa = pkg.synth.normal_f32(na * k, "moemm", "xa").reshape(na, k).astype(np.float16)
     yd = gpu.upload(np.full(na * n + n, 777.25, np.float32))
     gpu.dispatch(gpu.begin(), tile, [(gpu.upload_bytes(xa.view(np.uint8)), 0), (w0d, 0), (None, 0), (yd, 0), (None, 0), (od, 0), (ld, 0)],
-                 [k, n, na, E, 1], [(n + 127) // 128, 2, E], [256, 1, 1])
+                 [k, n, na, E, 1], [(n + bn - 1) // bn, 2, E], [256, 1, 1])
     g = gpu.read(yd, na * n + n)
     assert np.all(g[na * n:] == np.float32(777.25))
     g = g[:na * n].reshape(na, n)
@@ -589,7 +591,7 @@ def test_grouped_f16_tile_by_name(gpu, orc, pkg, fmt, tile):
             assert peak_err(g[a], want) <= 1e-5, (e, a)
     with pytest.raises(pkg.OjasHipError, match="grid must be"):
         gpu.dispatch(gpu.begin(), tile, [(xd, 0), (w0d, 0), (w1d, 0), (gpu.alloc(na * n), 0), (gpu.alloc(na * n), 0), (od, 0), (ld, 0)],
-                     [k, n, na, E, div], [(n + 127) // 128, 1, E + 1], [256, 1, 1])
+                     [k, n, na, E, div], [(n + bn - 1) // bn, 1, E + 1], [256, 1, 1])
 
 
 @pytest.mark.parametrize("T,E,ksel,k,n", [(1, 8, 2, 256, 64), (3, 6, 4, 512, 224)])
