@@ -78,7 +78,7 @@ struct ojh_device {
     uint32_t iq4_tile = 5;       // OJAS_HIP_IQ4_TILE: tokens from which IQ4_NL / IQ4_XS rows run on the tile through their own loaders instead of the decode pass (0: never)
     uint32_t iq4_tile_cap = 128; // OJAS_HIP_IQ4_TILE_CAP: tokens up to which Q3_K rows take their loader
     uint32_t gemm_few = 32;      // OJAS_HIP_GEMM_FEW: tokens up to which Q8_0 / IQ4 / legacy / MXFP4 / Q2_K / Q3_K batches take `gemm_few_*` instead of the LDS-staged tile (0: never; at most 64)
-    uint32_t moe_few = 64;       // OJAS_HIP_MOE_FEW: average assignments per expert up to which the grouped products of Q8_0 / IQ4 experts run on `moe_few_*` (0: never)
+    uint32_t moe_few = 128;       // OJAS_HIP_MOE_FEW: average assignments per expert up to which the grouped products of Q8_0 / IQ4 experts run on `moe_few_*` (0: never)
     uint32_t moe_mm_tile = 1;    // OJAS_HIP_MOE_MM_TILE: assignments per expert (average) from which Q8_0 experts run on the grouped f16 matrix tile under OJH_ACT_AUTO (0: never, 1: measured default, n: n)
     uint32_t moe_down_gs = 1;    // OJAS_HIP_MOE_DOWN_GS: assignments per expert (average) from which Q5_K / Q6_K down tensors run on the int8 matrix tile (0: never, 1: measured default, n: n)
     bool q8row_dec = true;       // OJAS_HIP_Q8ROW_DEC=0: 1 to 8 tokens on the per-row kernel instead of the one that stages the tokens in LDS
